@@ -1,0 +1,135 @@
+/*
+ * jlmi.h -- C ABI of the MI355X (gfx950) quantized-weight matmul path.
+ *
+ * This is the boundary a host program binds (cgo, ctypes, dlopen): plain
+ * pointers and sizes, no C++ or framework types.  Each entry point names the
+ * interface of the reference engine it stands behind.  The library loads one
+ * gfx950 code object with hipModuleLoad and launches its kernels on HIP
+ * streams; there is no CPU fallback inside it.
+ *
+ * Result convention (the reference's device seam returns a bool, "served" or
+ * "declined, run the host path"; engine/nn/device.go:18-31):
+ *     JL_OK        served: the output is complete
+ *     JL_DECLINED  not served (unsupported type or shape); nothing was written,
+ *                  the caller runs its own path.  Never an approximation.
+ *     < 0          failure (bad argument, HIP error); jl_last_error() says what
+ *
+ * Two families of entry points:
+ *   host-pointer  (jl_matvec, jl_matmul, ...): operands are host memory, the
+ *       library owns device residency of weights keyed on the host pointer,
+ *       exactly the contract of nn.Device.MatVec.  Synchronous.
+ *   device-pointer (*_dev): operands are device memory of the context's
+ *       device, work is enqueued on the given hipStream_t (void*; NULL = the
+ *       context's own stream) and not waited for.  This is what a resident
+ *       engine and the benchmarks call: no PCIe in the loop.
+ *
+ * Weight types are ggml type numbers (format/quant/types.go:14-55).
+ * Matrices: W is [nrows][k] (k = input features, contiguous), x is [ntok][k],
+ * out is [ntok][nrows] -- the reference's layouts (engine/nn/packedmm.go:23).
+ */
+#ifndef JLMI_H
+#define JLMI_H
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define JL_OK 0
+#define JL_DECLINED 1
+#define JL_ERR_ARG (-1)
+#define JL_ERR_HIP (-2)
+#define JL_ERR_NOMEM (-3)
+
+#define JL_TYPE_Q8_0 8
+#define JL_TYPE_Q4_K 12
+#define JL_TYPE_Q6_K 14
+#define JL_TYPE_MXFP4 39
+
+typedef struct jl_ctx jl_ctx;
+
+/* Per-context options; the library reads no environment variables, like the
+ * reference's per-instance options (engine/nn/options.go:7-13). */
+typedef struct jl_options {
+    int device;              /* HIP device ordinal */
+    int act_window;          /* activation amax window: 32 or 256; 0 = 32 */
+    const char *code_object; /* path of the gfx950 code object; NULL = the file
+                                jlmi_gfx950.hsaco beside the library */
+} jl_options;
+
+/* Creates a context: selects the device, creates a stream, hipModuleLoad()s the
+ * code object and resolves every kernel.  Replaces opening a backend device
+ * (jit/gpu/hip/hipapi.go:43-114, jit/gpu/backend/backend.go:60-78). */
+int jl_ctx_create(jl_ctx **out, const jl_options *opts);
+void jl_ctx_destroy(jl_ctx *ctx);
+
+/* Name of the HIP runtime library the context calls (resolved with dlopen; a
+ * runtime the process already holds is reused), "" when none could be loaded.
+ * The reference reaches its drivers the same way (jit/gpu/hip/hipapi.go:43-72). */
+const char *jl_hip_runtime(void);
+
+/* Text of the last failure on this context (or of the last failed
+ * jl_ctx_create when ctx is NULL).  Valid until the next call. */
+const char *jl_last_error(const jl_ctx *ctx);
+
+/* nn.ActWindower.SetActWindow (engine/nn/device.go:39-44, :1566-1568): the amax
+ * window of the activation quantizer, 32 or 256 (jit/cpu/matvec.go:46-62). */
+int jl_set_act_window(jl_ctx *ctx, int window);
+
+/* The context's own stream as a hipStream_t. */
+void *jl_stream(jl_ctx *ctx);
+int jl_synchronize(jl_ctx *ctx);
+
+/* Kernel-shape overrides for measurement: key is one of "matvec.rpw",
+ * "matvec.ni", "matvec.block", "matvec.grid"; value 0 restores the built-in
+ * choice (-1 for ni).  Mirrors the reference's per-instance tuning knobs
+ * (engine/nn/options.go:67-118). */
+int jl_set_tuning(jl_ctx *ctx, const char *key, int value);
+
+/* ---- host-pointer seam ------------------------------------------------ */
+
+/* nn.Device.MatVec (engine/nn/device.go:23-31; call site engine/nn/jit.go:935-940):
+ * out[0:nrows] = W x, W = raw GGUF row-major bytes.  Residency is keyed on the
+ * pointer w: the first offer uploads, later offers of the same pointer reuse
+ * the device copy, so w must stay put and unchanged until jl_forget. */
+int jl_matvec(jl_ctx *ctx, float *out, int type, const void *w, size_t wbytes,
+              const float *x, int nrows, int k);
+
+/* nn.CopyForgetter.Forget (engine/nn/device.go:1570-1581): drop any device copy
+ * keyed inside [p, p+n).  Callable from any thread; never blocks on the GPU. */
+int jl_forget(jl_ctx *ctx, const void *p, size_t n);
+
+/* JIT.MatMul over raw GGUF bytes (engine/nn/matmul.go:27): x [ntok][k] ->
+ * out [ntok][nrows].  Each token is quantized on its own. */
+int jl_matmul(jl_ctx *ctx, float *out, int type, const void *w, size_t wbytes,
+              const float *x, int nrows, int k, int ntok);
+
+/* ---- device-pointer entry points -------------------------------------- */
+
+/* The activation quantizer (jit/gpu/kernels/elem.go:76-170, pack.go:474-525):
+ * x [ntok][k] f32 -> q [ntok][k] int8, as [ntok][k/32] f32 scales,
+ * sum16 [ntok][k/16] f32 integer sums.  k % 32 == 0; x, q 16-byte aligned. */
+int jl_quantize_act_dev(jl_ctx *ctx, const float *x, int ntok, int k, int8_t *q,
+                        float *as, float *sum16, void *stream);
+
+/* quant.Dequant32 (format/quant/dequant.go:50): n elements of GGUF blocks -> f32,
+ * bit-identical to the reference decoder. */
+int jl_dequant_dev(jl_ctx *ctx, int type, const void *src, float *dst, size_t n,
+                   void *stream);
+
+/* JIT.MatVec / MatVecPacked semantics on resident operands (engine/nn/jit.go:916,
+ * packed.go:24): quantizes x (fused into the matvec kernel) and computes
+ * out[0:nrows].  w = GGUF row-major bytes, 16-byte aligned; x 16-byte aligned. */
+int jl_matvec_dev(jl_ctx *ctx, float *out, int type, const void *w, const float *x,
+                  int nrows, int k, void *stream);
+
+/* The same matvec over activations already quantized by jl_quantize_act_dev
+ * (the reference caches them across matvecs that share x, engine/nn/packed.go:282). */
+int jl_matvec_q8_dev(jl_ctx *ctx, float *out, int type, const void *w, const int8_t *q,
+                     const float *as, const float *sum16, int nrows, int k, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,57 @@
+"""Loads the C ABI (libjlmi.so, built in-tree by csrc/Makefile) with ctypes.
+
+There is no fallback: when the library or its gfx950 code object is missing,
+loading raises, and so does every operator built on it.
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libjlmi.so")
+CODE_OBJECT_PATH = os.path.join(_HERE, "jlmi_gfx950.hsaco")
+
+OK, DECLINED = 0, 1
+
+
+class Options(C.Structure):
+    _fields_ = [("device", C.c_int), ("act_window", C.c_int), ("code_object", C.c_char_p)]
+
+
+_vp, _sz, _int = C.c_void_p, C.c_size_t, C.c_int
+
+# name -> (restype, argtypes); every symbol include/jlmi.h declares
+SIGNATURES = {
+    "jl_hip_runtime": (C.c_char_p, []),
+    "jl_ctx_create": (_int, [C.POINTER(_vp), C.POINTER(Options)]),
+    "jl_ctx_destroy": (None, [_vp]),
+    "jl_last_error": (C.c_char_p, [_vp]),
+    "jl_set_act_window": (_int, [_vp, _int]),
+    "jl_stream": (_vp, [_vp]),
+    "jl_synchronize": (_int, [_vp]),
+    "jl_set_tuning": (_int, [_vp, C.c_char_p, _int]),
+    "jl_matvec": (_int, [_vp, _vp, _int, _vp, _sz, _vp, _int, _int]),
+    "jl_forget": (_int, [_vp, _vp, _sz]),
+    "jl_matmul": (_int, [_vp, _vp, _int, _vp, _sz, _vp, _int, _int, _int]),
+    "jl_quantize_act_dev": (_int, [_vp, _vp, _int, _int, _vp, _vp, _vp, _vp]),
+    "jl_dequant_dev": (_int, [_vp, _int, _vp, _vp, _sz, _vp]),
+    "jl_matvec_dev": (_int, [_vp, _vp, _int, _vp, _vp, _int, _int, _vp]),
+    "jl_matvec_q8_dev": (_int, [_vp, _vp, _int, _vp, _vp, _vp, _vp, _int, _int, _vp]),
+}
+
+_lib = None
+
+
+def load():
+    """The loaded library with argtypes set.  Raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `make -C jitllm_amd/csrc` "
+                "(or __graft_entry__.build()); there is no fallback path")
+        lib = C.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype, fn.argtypes = res, args
+        _lib = lib
+    return _lib

@@ -1,0 +1,455 @@
+// Host side of the C ABI declared in include/jlmi.h.
+//
+// One context = one device, one stream, one gfx950 code object loaded with
+// hipModuleLoad and its kernels resolved by name.  Entry points validate
+// shapes on the host before any launch (a kernel is never started on operands
+// it does not fit), translate the reference's operator contracts into kernel
+// launches, and report served / declined / error.  There is no CPU compute path
+// here: when the code object or the device is missing, creation fails.
+#include "../../include/jlmi.h"
+
+#include <dlfcn.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "hip_api.h"
+#include "kernels/args.h"
+
+namespace {
+
+thread_local std::string g_create_error;
+const HipApi* H = nullptr;  // the process-wide HIP runtime, resolved by the first jl_ctx_create
+
+struct Tuning {
+    int rpw = 0, ni = -1, block = 0, grid = 0;
+};
+
+struct Resident {
+    void* dev = nullptr;
+    size_t bytes = 0;
+};
+
+}  // namespace
+
+struct jl_ctx {
+    int device = 0;
+    int act_window = 32;
+    hipStream_t stream = nullptr;
+    hipModule_t module = nullptr;
+    std::map<std::string, hipFunction_t> fn;
+    std::string err;
+    std::mutex mu;  // serialises the host-pointer seam (one staging area per context)
+    Tuning tune;
+    int num_cu = 0;
+    size_t lds_limit = 0;
+
+    // host-pointer seam state
+    std::map<const void*, Resident> resident;
+    void* stage_x = nullptr;    // device
+    void* stage_out = nullptr;  // device
+    size_t stage_x_bytes = 0, stage_out_bytes = 0;
+};
+
+namespace {
+
+int fail(jl_ctx* c, int code, const char* fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    if (c) c->err = buf;
+    else g_create_error = buf;
+    return code;
+}
+
+#define HIP_TRY(c, call)                                                              \
+    do {                                                                              \
+        hipError_t e_ = (call);                                                       \
+        if (e_ != hipSuccess)                                                         \
+            return fail((c), JL_ERR_HIP, "%s: %s", #call, H->GetErrorString(e_));     \
+    } while (0)
+
+std::string default_code_object() {
+    Dl_info info;
+    if (dladdr((void*)&jl_ctx_create, &info) && info.dli_fname) {
+        std::string p = info.dli_fname;
+        size_t s = p.rfind('/');
+        return (s == std::string::npos ? std::string(".") : p.substr(0, s)) + "/jlmi_gfx950.hsaco";
+    }
+    return "jlmi_gfx950.hsaco";
+}
+
+struct TypeInfo {
+    const char* tag;   // kernel-name fragment
+    int block_elems, block_bytes;
+    int slot_elems;    // elements one lane-slot of the matvec kernel covers
+};
+
+const TypeInfo* type_info(int type) {
+    static const TypeInfo q8 = {"q8_0", 32, 34, 32};
+    static const TypeInfo q4k = {"q4k", 256, 144, 64};
+    static const TypeInfo q6k = {"q6k", 256, 210, 64};
+    switch (type) {
+    case JL_TYPE_Q8_0: return &q8;
+    case JL_TYPE_Q4_K: return &q4k;
+    case JL_TYPE_Q6_K: return &q6k;
+    }
+    return nullptr;
+}
+
+bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+
+// Kernel shapes that exist in the code object (kernels/jlmi_kernels.hip).
+bool matvec_shape_exists(int type, int rpw, int ni) {
+    switch (type) {
+    case JL_TYPE_Q4_K:
+        return (ni == 0 && (rpw == 1 || rpw == 2 || rpw == 4)) ||
+               (ni == 1 && (rpw == 1 || rpw == 2 || rpw == 4)) || (ni == 2 && (rpw == 1 || rpw == 2));
+    case JL_TYPE_Q8_0:
+        return (ni == 0 && (rpw == 1 || rpw == 2 || rpw == 4)) ||
+               (ni == 1 && (rpw == 1 || rpw == 2 || rpw == 4)) ||
+               (ni == 2 && (rpw == 1 || rpw == 2)) || (ni == 4 && rpw == 1);
+    case JL_TYPE_Q6_K:
+        return (ni == 0 && (rpw == 1 || rpw == 2)) || (ni == 1 && (rpw == 1 || rpw == 2 || rpw == 4));
+    }
+    return false;
+}
+
+hipStream_t pick_stream(jl_ctx* c, void* s) { return s ? (hipStream_t)s : c->stream; }
+
+int launch(jl_ctx* c, const char* name, unsigned gx, unsigned gy, unsigned block, unsigned lds,
+           hipStream_t st, void** params) {
+    auto it = c->fn.find(name);
+    if (it == c->fn.end()) return fail(c, JL_ERR_ARG, "kernel %s is not in the code object", name);
+    HIP_TRY(c, H->ModuleLaunchKernel(it->second, gx, gy, 1, block, 1, 1, lds, st, params, nullptr));
+    return JL_OK;
+}
+
+// Shape checks shared by every matvec entry point.  Returns JL_OK, JL_DECLINED or an error.
+int matvec_check(jl_ctx* c, int type, int nrows, int k, const TypeInfo** ti_out) {
+    const TypeInfo* ti = type_info(type);
+    if (!ti) return JL_DECLINED;
+    if (nrows <= 0 || k <= 0) return fail(c, JL_ERR_ARG, "matvec: nrows=%d k=%d", nrows, k);
+    if (k % ti->block_elems != 0) return JL_DECLINED;
+    size_t lds = (size_t)k + (size_t)(k / 32) * 4 + (size_t)(k / 16) * 4;
+    if (lds > c->lds_limit) return JL_DECLINED;  // activation does not fit LDS
+    if ((size_t)(k / ti->block_elems) * ti->block_bytes > 0x7fffffffu) return JL_DECLINED;
+    *ti_out = ti;
+    return JL_OK;
+}
+
+int matvec_launch(jl_ctx* c, float* out, int type, const void* w, const float* x, const int8_t* q,
+                  const float* as, const float* s16, int nrows, int k, hipStream_t st) {
+    const TypeInfo* ti = nullptr;
+    int rc = matvec_check(c, type, nrows, k, &ti);
+    if (rc != JL_OK) return rc;
+    if (!out || !w) return fail(c, JL_ERR_ARG, "matvec: null operand");
+    if (x && !aligned16(x)) return JL_DECLINED;
+    if (!x && (!q || !as || !s16)) return fail(c, JL_ERR_ARG, "matvec: no activation");
+    if (q && !aligned16(q)) return JL_DECLINED;
+    if (type == JL_TYPE_Q4_K && !aligned16(w)) return JL_DECLINED;
+    if (((uintptr_t)w & 1) != 0) return JL_DECLINED;
+
+    const int nslots = k / ti->slot_elems;
+    const int iters = (nslots + 63) / 64;
+
+    // Shape choice.  Small matrices: one row per wavefront with every load of the
+    // row unrolled, 16 wavefronts per workgroup so a CU quantizes x once.  Larger
+    // ones: more rows per wavefront (activation registers are reused) and a grid
+    // that covers the chip a few times over.
+    int ni = c->tune.ni, rpw = c->tune.rpw, block = c->tune.block;
+    if (ni < 0) ni = iters <= 2 ? iters : 0;
+    if (ni > 0 && ni < iters) ni = 0;  // an unrolled shape must cover the whole row
+    if (rpw <= 0) {
+        rpw = 1;
+        long waves = nrows;
+        if (waves >= 4L * c->num_cu * 16) rpw = 2;
+    }
+    while (!matvec_shape_exists(type, rpw, ni)) {
+        if (rpw > 1) rpw >>= 1;
+        else if (ni != 0) ni = 0;
+        else return fail(c, JL_ERR_ARG, "matvec: no kernel shape");
+    }
+    if (block <= 0) block = 1024;
+    if (block % 64 != 0 || block > 1024) return fail(c, JL_ERR_ARG, "matvec: block=%d", block);
+    const int rows_per_block = (block / 64) * rpw;
+    long groups = ((long)nrows + rows_per_block - 1) / rows_per_block;
+    long grid = c->tune.grid > 0 ? c->tune.grid : groups;
+    if (grid > groups) grid = groups;
+    if (grid < 1) grid = 1;
+
+    MatVecArgs a;
+    a.out = out;
+    a.w = (const uint8_t*)w;
+    a.x = x;
+    a.q = q;
+    a.as = as;
+    a.s16 = s16;
+    a.nrows = nrows;
+    a.k = k;
+    a.row_bytes = (k / ti->block_elems) * ti->block_bytes;
+    a.per = c->act_window / 32;
+    char name[64];
+    snprintf(name, sizeof name, "jl_matvec_%s_r%d_n%d", ti->tag, rpw, ni);
+    void* params[] = {&a};
+    unsigned lds = (unsigned)((size_t)k + (size_t)(k / 32) * 4 + (size_t)(k / 16) * 4);
+    return launch(c, name, (unsigned)grid, 1, (unsigned)block, lds, st, params);
+}
+
+int ensure_stage(jl_ctx* c, void** buf, size_t* have, size_t need) {
+    if (*have >= need) return JL_OK;
+    if (*buf) HIP_TRY(c, H->Free(*buf));
+    *buf = nullptr;
+    *have = 0;
+    HIP_TRY(c, H->Malloc(buf, need));
+    *have = need;
+    return JL_OK;
+}
+
+// Device copy of host weight bytes, keyed on the host pointer.
+int resident_weight(jl_ctx* c, const void* w, size_t bytes, void** dev) {
+    auto it = c->resident.find(w);
+    if (it != c->resident.end() && it->second.bytes == bytes) {
+        *dev = it->second.dev;
+        return JL_OK;
+    }
+    if (it != c->resident.end()) {
+        HIP_TRY(c, H->Free(it->second.dev));
+        c->resident.erase(it);
+    }
+    void* d = nullptr;
+    HIP_TRY(c, H->Malloc(&d, bytes));
+    hipError_t e = H->Memcpy(d, w, bytes, hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+        (void)H->Free(d);
+        return fail(c, JL_ERR_HIP, "weight upload: %s", H->GetErrorString(e));
+    }
+    c->resident[w] = Resident{d, bytes};
+    *dev = d;
+    return JL_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
+    if (!out) return fail(nullptr, JL_ERR_ARG, "jl_ctx_create: null out");
+    *out = nullptr;
+    if (!H) {
+        std::string why;
+        H = hip_api(&why);
+        if (!H) return fail(nullptr, JL_ERR_HIP, "%s", why.c_str());
+    }
+    jl_ctx* c = new (std::nothrow) jl_ctx;
+    if (!c) return fail(nullptr, JL_ERR_NOMEM, "out of memory");
+    c->device = opts ? opts->device : 0;
+    c->act_window = (opts && opts->act_window) ? opts->act_window : 32;
+    std::string path = (opts && opts->code_object) ? opts->code_object : default_code_object();
+
+    auto bail = [&](int code, const std::string& msg) {
+        g_create_error = msg;
+        jl_ctx_destroy(c);
+        return code;
+    };
+    if (c->act_window != 32 && c->act_window != 64 && c->act_window != 128 && c->act_window != 256)
+        return bail(JL_ERR_ARG, "act_window must be 32, 64, 128 or 256");
+    hipError_t e = H->SetDevice(c->device);
+    if (e != hipSuccess) return bail(JL_ERR_HIP, std::string("hipSetDevice: ") + H->GetErrorString(e));
+    hipDeviceProp_t prop;
+    e = H->GetDeviceProperties(&prop, c->device);
+    if (e != hipSuccess) return bail(JL_ERR_HIP, std::string("hipGetDeviceProperties: ") + H->GetErrorString(e));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return bail(JL_ERR_HIP, std::string("device is ") + prop.gcnArchName + ", this library is gfx950 only");
+    c->num_cu = prop.multiProcessorCount;
+    c->lds_limit = prop.sharedMemPerBlock;
+    e = H->StreamCreate(&c->stream);
+    if (e != hipSuccess) return bail(JL_ERR_HIP, std::string("hipStreamCreate: ") + H->GetErrorString(e));
+    e = H->ModuleLoad(&c->module, path.c_str());
+    if (e != hipSuccess)
+        return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
+
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant"};
+    const int types[] = {JL_TYPE_Q4_K, JL_TYPE_Q8_0, JL_TYPE_Q6_K};
+    for (int t : types)
+        for (int rpw : {1, 2, 4})
+            for (int ni : {0, 1, 2, 4})
+                if (matvec_shape_exists(t, rpw, ni)) {
+                    char nm[64];
+                    snprintf(nm, sizeof nm, "jl_matvec_%s_r%d_n%d", type_info(t)->tag, rpw, ni);
+                    names.push_back(nm);
+                }
+    for (const auto& n : names) {
+        hipFunction_t f;
+        e = H->ModuleGetFunction(&f, c->module, n.c_str());
+        if (e != hipSuccess)
+            return bail(JL_ERR_HIP, "hipModuleGetFunction(" + n + "): " + H->GetErrorString(e));
+        c->fn[n] = f;
+    }
+    *out = c;
+    return JL_OK;
+}
+
+const char* jl_hip_runtime(void) {
+    std::string why;
+    const HipApi* h = hip_api(&why);
+    return h ? h->path.c_str() : "";
+}
+
+void jl_ctx_destroy(jl_ctx* c) {
+    if (!c) return;
+    (void)H->SetDevice(c->device);
+    if (c->stream) (void)H->StreamSynchronize(c->stream);
+    for (auto& kv : c->resident) (void)H->Free(kv.second.dev);
+    if (c->stage_x) (void)H->Free(c->stage_x);
+    if (c->stage_out) (void)H->Free(c->stage_out);
+    if (c->module) (void)H->ModuleUnload(c->module);
+    if (c->stream) (void)H->StreamDestroy(c->stream);
+    delete c;
+}
+
+const char* jl_last_error(const jl_ctx* c) { return c ? c->err.c_str() : g_create_error.c_str(); }
+
+int jl_set_act_window(jl_ctx* c, int window) {
+    if (!c) return JL_ERR_ARG;
+    if (window != 32 && window != 64 && window != 128 && window != 256)
+        return fail(c, JL_ERR_ARG, "act_window must be 32, 64, 128 or 256, not %d", window);
+    c->act_window = window;
+    return JL_OK;
+}
+
+void* jl_stream(jl_ctx* c) { return c ? (void*)c->stream : nullptr; }
+
+int jl_synchronize(jl_ctx* c) {
+    if (!c) return JL_ERR_ARG;
+    HIP_TRY(c, H->SetDevice(c->device));
+    HIP_TRY(c, H->StreamSynchronize(c->stream));
+    return JL_OK;
+}
+
+int jl_set_tuning(jl_ctx* c, const char* key, int value) {
+    if (!c || !key) return JL_ERR_ARG;
+    if (!strcmp(key, "matvec.rpw")) c->tune.rpw = value;
+    else if (!strcmp(key, "matvec.ni")) c->tune.ni = value;
+    else if (!strcmp(key, "matvec.block")) c->tune.block = value;
+    else if (!strcmp(key, "matvec.grid")) c->tune.grid = value;
+    else return fail(c, JL_ERR_ARG, "unknown tuning key %s", key);
+    return JL_OK;
+}
+
+/* ------------------------------------------------ device-pointer entry points */
+
+int jl_quantize_act_dev(jl_ctx* c, const float* x, int ntok, int k, int8_t* q, float* as,
+                        float* sum16, void* stream) {
+    if (!c) return JL_ERR_ARG;
+    if (!x || !q || !as || !sum16 || ntok <= 0 || k <= 0)
+        return fail(c, JL_ERR_ARG, "quantize_act: bad operand");
+    if (k % 32 != 0 || !aligned16(x) || !aligned16(q)) return JL_DECLINED;
+    if (ntok > 65535) return JL_DECLINED;
+    HIP_TRY(c, H->SetDevice(c->device));
+    int per = c->act_window / 32;
+    void* params[] = {(void*)&x, (void*)&q, (void*)&as, (void*)&sum16, (void*)&k, (void*)&per};
+    unsigned gx = (unsigned)((k / 16 + 255) / 256);
+    return launch(c, "jl_quantize_act", gx, (unsigned)ntok, 256, 0, pick_stream(c, stream), params);
+}
+
+int jl_dequant_dev(jl_ctx* c, int type, const void* src, float* dst, size_t n, void* stream) {
+    if (!c) return JL_ERR_ARG;
+    int be;
+    switch (type) {
+    case JL_TYPE_Q8_0: case JL_TYPE_MXFP4: be = 32; break;
+    case JL_TYPE_Q4_K: case JL_TYPE_Q6_K: be = 256; break;
+    default: return JL_DECLINED;
+    }
+    if (!src || !dst) return fail(c, JL_ERR_ARG, "dequant: null operand");
+    if (n == 0 || n % (size_t)be != 0) return fail(c, JL_ERR_ARG, "dequant: %zu elements is not whole blocks", n);
+    if (type == JL_TYPE_Q4_K && ((uintptr_t)src & 3) != 0) return JL_DECLINED;
+    if (type != JL_TYPE_MXFP4 && ((uintptr_t)src & 1) != 0) return JL_DECLINED;
+    size_t blocks = (n + 255) / 256;
+    if (blocks > 0x7fffffffu) return JL_DECLINED;
+    HIP_TRY(c, H->SetDevice(c->device));
+    void* params[] = {(void*)&src, (void*)&dst, (void*)&n, (void*)&type};
+    return launch(c, "jl_dequant", (unsigned)blocks, 1, 256, 0, pick_stream(c, stream), params);
+}
+
+int jl_matvec_dev(jl_ctx* c, float* out, int type, const void* w, const float* x, int nrows, int k,
+                  void* stream) {
+    if (!c) return JL_ERR_ARG;
+    if (!x) return fail(c, JL_ERR_ARG, "matvec: null x");
+    HIP_TRY(c, H->SetDevice(c->device));
+    return matvec_launch(c, out, type, w, x, nullptr, nullptr, nullptr, nrows, k, pick_stream(c, stream));
+}
+
+int jl_matvec_q8_dev(jl_ctx* c, float* out, int type, const void* w, const int8_t* q,
+                     const float* as, const float* sum16, int nrows, int k, void* stream) {
+    if (!c) return JL_ERR_ARG;
+    HIP_TRY(c, H->SetDevice(c->device));
+    return matvec_launch(c, out, type, w, nullptr, q, as, sum16, nrows, k, pick_stream(c, stream));
+}
+
+/* ------------------------------------------------------- host-pointer seam */
+
+int jl_matvec(jl_ctx* c, float* out, int type, const void* w, size_t wbytes, const float* x,
+              int nrows, int k) {
+    return jl_matmul(c, out, type, w, wbytes, x, nrows, k, 1);
+}
+
+int jl_matmul(jl_ctx* c, float* out, int type, const void* w, size_t wbytes, const float* x,
+              int nrows, int k, int ntok) {
+    if (!c) return JL_ERR_ARG;
+    std::lock_guard<std::mutex> lock(c->mu);
+    const TypeInfo* ti = nullptr;
+    int rc = matvec_check(c, type, nrows, k, &ti);
+    if (rc != JL_OK) return rc;
+    if (!out || !w || !x || ntok <= 0) return fail(c, JL_ERR_ARG, "matmul: bad operand");
+    size_t need = (size_t)nrows * (size_t)(k / ti->block_elems) * ti->block_bytes;
+    if (wbytes < need)
+        return fail(c, JL_ERR_ARG, "matmul: weight has %zu bytes, %dx%d needs %zu", wbytes, nrows, k, need);
+    HIP_TRY(c, H->SetDevice(c->device));
+    void* wd = nullptr;
+    rc = resident_weight(c, w, need, &wd);
+    if (rc != JL_OK) return rc;
+    size_t xb = (size_t)ntok * k * 4, ob = (size_t)ntok * nrows * 4;
+    if ((rc = ensure_stage(c, &c->stage_x, &c->stage_x_bytes, xb)) != JL_OK) return rc;
+    if ((rc = ensure_stage(c, &c->stage_out, &c->stage_out_bytes, ob)) != JL_OK) return rc;
+    HIP_TRY(c, H->MemcpyAsync(c->stage_x, x, xb, hipMemcpyHostToDevice, c->stream));
+    for (int t = 0; t < ntok; t++) {
+        rc = matvec_launch(c, (float*)c->stage_out + (size_t)t * nrows, type, wd,
+                           (const float*)c->stage_x + (size_t)t * k, nullptr, nullptr, nullptr,
+                           nrows, k, c->stream);
+        if (rc != JL_OK) {
+            (void)H->StreamSynchronize(c->stream);
+            return rc;
+        }
+    }
+    HIP_TRY(c, H->MemcpyAsync(out, c->stage_out, ob, hipMemcpyDeviceToHost, c->stream));
+    HIP_TRY(c, H->StreamSynchronize(c->stream));
+    return JL_OK;
+}
+
+int jl_forget(jl_ctx* c, const void* p, size_t n) {
+    if (!c) return JL_ERR_ARG;
+    std::lock_guard<std::mutex> lock(c->mu);
+    const char* lo = (const char*)p;
+    const char* hi = lo + n;
+    (void)H->SetDevice(c->device);
+    for (auto it = c->resident.begin(); it != c->resident.end();) {
+        const char* k0 = (const char*)it->first;
+        if (k0 >= lo && k0 < hi) {
+            (void)H->Free(it->second.dev);
+            it = c->resident.erase(it);
+        } else {
+            ++it;
+        }
+    }
+    return JL_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,17 @@
+// Kernel argument blocks, shared by the device code and the host launcher.
+// Plain C layouts: the host passes each struct by value as the kernel's single
+// parameter.
+#pragma once
+#include <stdint.h>
+
+struct MatVecArgs {
+    float* out;          // [nrows]
+    const uint8_t* w;    // GGUF row-major blocks
+    const float* x;      // f32 activations (fused quantize) or null
+    const int8_t* q;     // pre-quantized activations (split form) or null
+    const float* as;     // [k/32] activation scales
+    const float* s16;    // [k/16] activation sums
+    int nrows, k;
+    int row_bytes;
+    int per;             // activation window / 32 (fused form)
+};

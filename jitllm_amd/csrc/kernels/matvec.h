@@ -1,0 +1,369 @@
+// Decode matvec over row-major GGUF blocks: out[r] = sum_k W[r][k] * x[k].
+//
+// What it computes is the reference's quantized-activation form
+// (jit/gpu/kernels/matvec.go:1121-1271, jit/cpu/packedfused.go:200-362): the
+// activation is int8 with one f32 scale d_a per 32 elements, each sub-block's
+// dot product is an exact int32, and
+//     out[r] += d_a * (scale * dot - bias * sum_a)
+// with (scale, bias) = (d*sc, dmin*m) for Q4_K, (d*sc, 32*scale) for Q6_K and
+// (d, 0) for Q8_0.  Only the f32 summation order differs from the reference.
+//
+// Shape of the kernel: HBM-bound, so everything is arranged to put the whole
+// weight matrix in flight at once.  A wavefront owns RPW rows; a row is cut
+// into "slots" (one 64-element group of a Q4_K super-block, one quarter of a
+// Q6_K super-block, one Q8_0 block) and lane l takes slots l, l+64, ... so a
+// wavefront's 128-bit loads walk a row contiguously.  The int8 activations
+// live in LDS, staged once per workgroup -- either copied from a quantizer's
+// output or, in the fused form, quantized in place from f32 x while the first
+// weight loads are still in flight.  Per-row partial sums are reduced across
+// the 64 lanes with cross-lane shuffles.
+#pragma once
+#include "args.h"
+#include "common.h"
+#include "quantize.h"
+
+// Activation staging area in LDS: int8 a[k], then f32 da[k/32], then f32 s16[k/16].
+struct ActLds {
+    const uint8_t* a;
+    const float* da;
+    const float* s16;
+};
+
+__device__ __forceinline__ ActLds act_lds_views(uint8_t* smem, int k) {
+    ActLds v;
+    v.a = smem;
+    v.da = (const float*)(smem + k);
+    v.s16 = (const float*)(smem + k + (k / 32) * 4);
+    return v;
+}
+
+// Bytes of LDS the staging area needs for a k-element activation.
+#define JL_ACT_LDS_BYTES(k) ((k) + ((k) / 32) * 4 + ((k) / 16) * 4)
+
+// Stage pre-quantized activations (global) into LDS.  k % 32 == 0.
+__device__ __forceinline__ void stage_act_copy(uint8_t* smem, const int8_t* q, const float* as,
+                                               const float* s16, int k) {
+    u32* a = (u32*)smem;
+    float* da = (float*)(smem + k);
+    float* ss = (float*)(smem + k + (k / 32) * 4);
+    for (int i = threadIdx.x; i < k / 4; i += blockDim.x) a[i] = ((const u32*)q)[i];
+    for (int i = threadIdx.x; i < k / 32; i += blockDim.x) da[i] = as[i];
+    for (int i = threadIdx.x; i < k / 16; i += blockDim.x) ss[i] = s16[i];
+}
+
+// Quantize f32 x into the LDS staging area (same bits as the standalone
+// quantizer).  k % 32 == 0, blockDim.x % 64 == 0, per = window / 32.
+__device__ __forceinline__ void stage_act_quantize(uint8_t* smem, const float* x, int k, int per) {
+    u32x4* a = (u32x4*)smem;
+    float* da = (float*)(smem + k);
+    float* ss = (float*)(smem + k + (k / 32) * 4);
+    int nhb = k / 16;
+    int nhb_pad = (nhb + 15) & ~15;  // whole 16-lane rows take part in the shuffles
+    for (int hb = threadIdx.x; hb < nhb_pad; hb += blockDim.x) {
+        f32x4 v[4];
+        bool live = hb < nhb;
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            v[i] = live ? ((const f32x4*)x)[hb * 4 + i] : f32x4{0.f, 0.f, 0.f, 0.f};
+        u32 amax = window_amax(half_block_amax(v), per);
+        u32 q[4];
+        float d;
+        i32 sum;
+        quantize_half_block(v, amax, q, d, sum);
+        if (live) {
+            a[hb] = u32x4{q[0], q[1], q[2], q[3]};
+            ss[hb] = (float)sum;
+            if ((hb & 1) == 0) da[hb >> 1] = d;
+        }
+    }
+}
+
+// ---------------------------------------------------------------- Q4_K slot
+// slot = (super-block sb, group g of 64 elements): 32 bytes of nibbles whose
+// low halves are sub-block 2g and high halves sub-block 2g+1
+// (format/quant/dequant.go:367-397).
+struct SlotActQ4K {
+    u32x4 lo[2], hi[2];  // int8 activations of sub-block 2g / 2g+1
+    float da_lo, da_hi;  // their scales
+    float s_lo, s_hi;    // their integer sums
+};
+
+__device__ __forceinline__ void load_act_q4k(const ActLds& A, int slot, SlotActQ4K& s) {
+    int e0 = slot * 64;  // first element of the group
+    const u32x4* a = (const u32x4*)(A.a + e0);
+    s.lo[0] = a[0]; s.lo[1] = a[1]; s.hi[0] = a[2]; s.hi[1] = a[3];
+    s.da_lo = A.da[e0 / 32];
+    s.da_hi = A.da[e0 / 32 + 1];
+    s.s_lo = A.s16[e0 / 16] + A.s16[e0 / 16 + 1];
+    s.s_hi = A.s16[e0 / 16 + 2] + A.s16[e0 / 16 + 3];
+}
+
+struct SlotWQ4K {
+    u32x4 hdr;    // f16 d, f16 dmin, 12 scale bytes
+    u32x4 q[2];   // 32 bytes of nibbles
+};
+
+__device__ __forceinline__ void load_w_q4k(const uint8_t* row, int slot, SlotWQ4K& w) {
+    const uint8_t* blk = row + (size_t)(slot >> 2) * 144;
+    w.hdr = ld16(blk);
+    const uint8_t* qs = blk + 16 + (slot & 3) * 32;
+    w.q[0] = ld16(qs);
+    w.q[1] = ld16(qs + 16);
+}
+
+__device__ __forceinline__ float dot_q4k(const SlotWQ4K& w, int g, const SlotActQ4K& s) {
+    float d = half_bits_to_f32((uint16_t)(w.hdr.x & 0xFFFF));
+    float dmin = half_bits_to_f32((uint16_t)(w.hdr.x >> 16));
+    // 6-bit scale/min pairs of sub-blocks 2g and 2g+1, branch-free
+    int sh = 16 * (g & 1);
+    u32 A = w.hdr.y >> sh, B = w.hdr.z >> sh, C = w.hdr.w >> sh;
+    u32 sc_lo, sc_hi, m_lo, m_hi;
+    if (g < 2) {
+        sc_lo = A & 63; sc_hi = (A >> 8) & 63;
+        m_lo = B & 63;  m_hi = (B >> 8) & 63;
+    } else {
+        sc_lo = (C & 0xF) | (((A >> 6) & 3) << 4);
+        sc_hi = ((C >> 8) & 0xF) | (((A >> 14) & 3) << 4);
+        m_lo = ((C >> 4) & 0xF) | (((B >> 6) & 3) << 4);
+        m_hi = ((C >> 12) & 0xF) | (((B >> 14) & 3) << 4);
+    }
+    i32 dl = 0, dh = 0;
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        dl = dot4(w.q[i].x & 0x0F0F0F0Fu, s.lo[i].x, dl);
+        dl = dot4(w.q[i].y & 0x0F0F0F0Fu, s.lo[i].y, dl);
+        dl = dot4(w.q[i].z & 0x0F0F0F0Fu, s.lo[i].z, dl);
+        dl = dot4(w.q[i].w & 0x0F0F0F0Fu, s.lo[i].w, dl);
+        dh = dot4((w.q[i].x >> 4) & 0x0F0F0F0Fu, s.hi[i].x, dh);
+        dh = dot4((w.q[i].y >> 4) & 0x0F0F0F0Fu, s.hi[i].y, dh);
+        dh = dot4((w.q[i].z >> 4) & 0x0F0F0F0Fu, s.hi[i].z, dh);
+        dh = dot4((w.q[i].w >> 4) & 0x0F0F0F0Fu, s.hi[i].w, dh);
+    }
+    float v_lo = (float)dl * (d * (float)sc_lo) - s.s_lo * (dmin * (float)m_lo);
+    float v_hi = (float)dh * (d * (float)sc_hi) - s.s_hi * (dmin * (float)m_hi);
+    return fmaf(v_lo, s.da_lo, v_hi * s.da_hi);
+}
+
+// ---------------------------------------------------------------- Q8_0 slot
+// slot = one 34-byte block: f16 d, 32 int8 (format/quant/dequant.go:148-157).
+struct SlotActQ8 {
+    u32x4 a[2];
+    float da;
+};
+
+__device__ __forceinline__ void load_act_q8(const ActLds& A, int slot, SlotActQ8& s) {
+    const u32x4* a = (const u32x4*)(A.a + slot * 32);
+    s.a[0] = a[0]; s.a[1] = a[1];
+    s.da = A.da[slot];
+}
+
+struct SlotWQ8 {
+    u32x4 q[2];
+    uint16_t d;
+};
+
+__device__ __forceinline__ void load_w_q8(const uint8_t* row, int slot, SlotWQ8& w) {
+    const uint8_t* blk = row + (size_t)slot * 34;
+    w.d = ld2(blk);
+    w.q[0] = ld16_a2(blk + 2);
+    w.q[1] = ld16_a2(blk + 18);
+}
+
+__device__ __forceinline__ float dot_q8(const SlotWQ8& w, const SlotActQ8& s) {
+    i32 dt = 0;
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        dt = dot4(w.q[i].x, s.a[i].x, dt);
+        dt = dot4(w.q[i].y, s.a[i].y, dt);
+        dt = dot4(w.q[i].z, s.a[i].z, dt);
+        dt = dot4(w.q[i].w, s.a[i].w, dt);
+    }
+    return (float)dt * half_bits_to_f32(w.d) * s.da;
+}
+
+// ---------------------------------------------------------------- Q6_K slot
+// slot = (super-block sb, half n, 16-run j): ql[16] (low nibbles = sub-block
+// 8n+j, high = 8n+4+j), ql[32+16] (sub-blocks 8n+2+j / 8n+6+j) and qh[16] (two
+// bits for each of the four), format/quant/dequant.go:443-470.  Each of the
+// four 16-element runs is a whole sub-block with its own int8 scale.
+struct SlotActQ6K {
+    u32x4 a[4];   // runs at elements 128n + 32q + 16j, q = 0..3
+    float da[4];
+    float s[4];
+};
+
+__device__ __forceinline__ void load_act_q6k(const ActLds& A, int slot, SlotActQ6K& s) {
+    int sb = slot >> 2, n = (slot >> 1) & 1, j = slot & 1;
+    int e0 = sb * 256 + n * 128 + j * 16;
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        int e = e0 + 32 * q;
+        s.a[q] = *(const u32x4*)(A.a + e);
+        s.da[q] = A.da[e / 32];
+        s.s[q] = A.s16[e / 16];
+    }
+}
+
+struct SlotWQ6K {
+    u32x4 qla, qlb, qh;
+    u32 sc;       // four int8 scales, byte q = sub-block 8n + 2q + j
+    uint16_t d;
+};
+
+__device__ __forceinline__ void load_w_q6k(const uint8_t* row, int slot, SlotWQ6K& w) {
+    int sb = slot >> 2, n = (slot >> 1) & 1, j = slot & 1;
+    const uint8_t* blk = row + (size_t)sb * 210;
+    w.qla = ld16_a2(blk + n * 64 + j * 16);
+    w.qlb = ld16_a2(blk + n * 64 + 32 + j * 16);
+    w.qh = ld16_a2(blk + 128 + n * 32 + j * 16);
+    const uint8_t* sc = blk + 192 + n * 8 + j;
+    w.sc = (u32)sc[0] | ((u32)sc[2] << 8) | ((u32)sc[4] << 16) | ((u32)sc[6] << 24);
+    w.d = ld2(blk + 208);
+}
+
+__device__ __forceinline__ i32 dot16(u32x4 q, u32x4 a) {
+    i32 t = dot4(q.x, a.x, 0);
+    t = dot4(q.y, a.y, t);
+    t = dot4(q.z, a.z, t);
+    return dot4(q.w, a.w, t);
+}
+
+__device__ __forceinline__ float dot_q6k(const SlotWQ6K& w, const SlotActQ6K& s) {
+    const u32 M4 = 0x0F0F0F0Fu, M2 = 0x30303030u;
+    u32x4 q0 = (w.qla & M4) | ((w.qh << 4) & M2);
+    u32x4 q1 = (w.qlb & M4) | ((w.qh << 2) & M2);
+    u32x4 q2 = ((w.qla >> 4) & M4) | (w.qh & M2);
+    u32x4 q3 = ((w.qlb >> 4) & M4) | ((w.qh >> 2) & M2);
+    float d = half_bits_to_f32(w.d);
+    float acc = 0.f;
+    // value = d*sc*(q-32): the zero point goes through the activation sum
+    float t0 = (float)(dot16(q0, s.a[0])) - 32.f * s.s[0];
+    float t1 = (float)(dot16(q1, s.a[1])) - 32.f * s.s[1];
+    float t2 = (float)(dot16(q2, s.a[2])) - 32.f * s.s[2];
+    float t3 = (float)(dot16(q3, s.a[3])) - 32.f * s.s[3];
+    acc = fmaf(t0 * (d * (float)(int8_t)(w.sc & 0xFF)), s.da[0], acc);
+    acc = fmaf(t1 * (d * (float)(int8_t)((w.sc >> 8) & 0xFF)), s.da[1], acc);
+    acc = fmaf(t2 * (d * (float)(int8_t)((w.sc >> 16) & 0xFF)), s.da[2], acc);
+    acc = fmaf(t3 * (d * (float)(int8_t)(w.sc >> 24)), s.da[3], acc);
+    return acc;
+}
+
+// ------------------------------------------------------------- the kernel
+template <int TYPE> struct SlotTraits;
+template <> struct SlotTraits<JL_Q4_K> {
+    typedef SlotActQ4K Act; typedef SlotWQ4K W;
+    static constexpr int kElems = 64;
+    static __device__ __forceinline__ void load_act(const ActLds& A, int s, Act& a) { load_act_q4k(A, s, a); }
+    static __device__ __forceinline__ void load_w(const uint8_t* row, int s, W& w) { load_w_q4k(row, s, w); }
+    static __device__ __forceinline__ float dot(const W& w, int s, const Act& a) { return dot_q4k(w, s & 3, a); }
+};
+template <> struct SlotTraits<JL_Q8_0> {
+    typedef SlotActQ8 Act; typedef SlotWQ8 W;
+    static constexpr int kElems = 32;
+    static __device__ __forceinline__ void load_act(const ActLds& A, int s, Act& a) { load_act_q8(A, s, a); }
+    static __device__ __forceinline__ void load_w(const uint8_t* row, int s, W& w) { load_w_q8(row, s, w); }
+    static __device__ __forceinline__ float dot(const W& w, int, const Act& a) { return dot_q8(w, a); }
+};
+template <> struct SlotTraits<JL_Q6_K> {
+    typedef SlotActQ6K Act; typedef SlotWQ6K W;
+    static constexpr int kElems = 64;
+    static __device__ __forceinline__ void load_act(const ActLds& A, int s, Act& a) { load_act_q6k(A, s, a); }
+    static __device__ __forceinline__ void load_w(const uint8_t* row, int s, W& w) { load_w_q6k(row, s, w); }
+    static __device__ __forceinline__ float dot(const W& w, int, const Act& a) { return dot_q6k(w, a); }
+};
+
+
+// One wavefront computes RPW rows at a time; NI = slot iterations per lane
+// unrolled so that every load of a row group is issued before the first use
+// (NI == 0: generic loop for long rows).
+template <int TYPE, int RPW, int NI>
+__device__ __forceinline__ void matvec_body(const MatVecArgs& p, uint8_t* smem) {
+    typedef SlotTraits<TYPE> T;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+    const int nslots = p.k / T::kElems;
+    const int rows_per_block = nwaves * RPW;
+    const ActLds A = act_lds_views(smem, p.k);
+
+    int r0 = blockIdx.x * rows_per_block + wave * RPW;
+
+    if constexpr (NI > 0) {
+        // Issue the first row group's weight loads before staging activations,
+        // so HBM latency overlaps the quantizer.
+        typename T::W w[NI][RPW];
+#pragma unroll
+        for (int i = 0; i < NI; i++) {
+            int s = min(lane + 64 * i, nslots - 1);
+#pragma unroll
+            for (int j = 0; j < RPW; j++) {
+                int r = min(r0 + j, p.nrows - 1);
+                T::load_w(p.w + (size_t)r * p.row_bytes, s, w[i][j]);
+            }
+        }
+        if (p.x) stage_act_quantize(smem, p.x, p.k, p.per);
+        else stage_act_copy(smem, p.q, p.as, p.s16, p.k);
+        __syncthreads();
+        typename T::Act a[NI];
+#pragma unroll
+        for (int i = 0; i < NI; i++) T::load_act(A, min(lane + 64 * i, nslots - 1), a[i]);
+
+        for (;;) {
+            float acc[RPW];
+#pragma unroll
+            for (int j = 0; j < RPW; j++) acc[j] = 0.f;
+#pragma unroll
+            for (int i = 0; i < NI; i++) {
+                int s = lane + 64 * i;
+                if (s < nslots) {
+#pragma unroll
+                    for (int j = 0; j < RPW; j++) acc[j] += T::dot(w[i][j], s, a[i]);
+                }
+            }
+            int rdone = r0;
+            r0 += gridDim.x * rows_per_block;
+            bool more = r0 < p.nrows;  // uniform per wave
+            if (more) {
+#pragma unroll
+                for (int i = 0; i < NI; i++) {
+                    int s = min(lane + 64 * i, nslots - 1);
+#pragma unroll
+                    for (int j = 0; j < RPW; j++) {
+                        int r = min(r0 + j, p.nrows - 1);
+                        T::load_w(p.w + (size_t)r * p.row_bytes, s, w[i][j]);
+                    }
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < RPW; j++) {
+                float t = wave_sum(acc[j]);
+                if (lane == 0 && rdone + j < p.nrows) p.out[rdone + j] = t;
+            }
+            if (!more) break;
+        }
+    } else {
+        if (p.x) stage_act_quantize(smem, p.x, p.k, p.per);
+        else stage_act_copy(smem, p.q, p.as, p.s16, p.k);
+        __syncthreads();
+        for (; r0 < p.nrows; r0 += gridDim.x * rows_per_block) {
+            float acc[RPW];
+#pragma unroll
+            for (int j = 0; j < RPW; j++) acc[j] = 0.f;
+            for (int s = lane; s < nslots; s += 64) {
+                typename T::Act a;
+                typename T::W w[RPW];
+#pragma unroll
+                for (int j = 0; j < RPW; j++) {
+                    int r = min(r0 + j, p.nrows - 1);
+                    T::load_w(p.w + (size_t)r * p.row_bytes, s, w[j]);
+                }
+                T::load_act(A, s, a);
+#pragma unroll
+                for (int j = 0; j < RPW; j++) acc[j] += T::dot(w[j], s, a);
+            }
+#pragma unroll
+            for (int j = 0; j < RPW; j++) {
+                float t = wave_sum(acc[j]);
+                if (lane == 0 && r0 + j < p.nrows) p.out[r0 + j] = t;
+            }
+        }
+    }
+}

@@ -1,0 +1,118 @@
+"""Host-side mirror of the reference's accelerator seam over the C ABI.
+
+`Device` is the shape of nn.Device (/root/reference/engine/nn/device.go:23-31):
+MatVec(out, t, w, x, nrows, k) -> bool, False meaning "declined, run your own
+path".  The *_dev methods take device pointers (ints, e.g. tensor.data_ptr())
+and enqueue on a stream without waiting: that is the boundary a resident engine
+and the benchmarks use.  Failures (as opposed to declines) raise DeviceError,
+where the reference's entry points panic.
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import _lib, quant
+
+
+class DeviceError(RuntimeError):
+    pass
+
+
+def _ptr(a):
+    """Address of a numpy array or a raw int address."""
+    if isinstance(a, np.ndarray):
+        return a.ctypes.data
+    return int(a)
+
+
+class Device:
+    def __init__(self, device=0, act_window=32, code_object=None):
+        self._l = _lib.load()
+        self._ctx = C.c_void_p()
+        opts = _lib.Options(device, act_window,
+                            (code_object or _lib.CODE_OBJECT_PATH).encode())
+        rc = self._l.jl_ctx_create(C.byref(self._ctx), C.byref(opts))
+        if rc != _lib.OK:
+            msg = self._l.jl_last_error(None).decode()
+            self._ctx = None
+            raise DeviceError(f"jl_ctx_create failed ({rc}): {msg}")
+
+    def close(self):
+        if getattr(self, "_ctx", None):
+            self._l.jl_ctx_destroy(self._ctx)
+            self._ctx = None
+
+    def __del__(self):
+        self.close()
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    def _served(self, rc, what):
+        if rc == _lib.OK:
+            return True
+        if rc == _lib.DECLINED:
+            return False
+        raise DeviceError(f"{what} failed ({rc}): {self._l.jl_last_error(self._ctx).decode()}")
+
+    # -- configuration -------------------------------------------------------
+    def SetActWindow(self, n):
+        """nn.ActWindower.SetActWindow (/root/reference/engine/nn/device.go:1566-1568)."""
+        self._served(self._l.jl_set_act_window(self._ctx, n), "jl_set_act_window")
+
+    def set_tuning(self, **kw):
+        for k, v in kw.items():
+            key = ("matvec." + k).encode()
+            self._served(self._l.jl_set_tuning(self._ctx, key, int(v)), "jl_set_tuning")
+
+    @property
+    def stream(self):
+        return self._l.jl_stream(self._ctx)
+
+    def synchronize(self):
+        self._served(self._l.jl_synchronize(self._ctx), "jl_synchronize")
+
+    # -- host-pointer seam ---------------------------------------------------
+    def MatVec(self, out, t, w, x, nrows, k):
+        """nn.Device.MatVec: out[0:nrows] = W x over raw GGUF bytes; False = declined."""
+        if t not in quant.BLOCK:
+            return False
+        assert out.dtype == np.float32 and x.dtype == np.float32 and w.dtype == np.uint8
+        assert out.size >= nrows and x.size >= k
+        return self._served(self._l.jl_matvec(self._ctx, _ptr(out), t, _ptr(w), w.nbytes, _ptr(x),
+                                              nrows, k), "jl_matvec")
+
+    def MatMul(self, out, t, w, x, nrows, k, ntok):
+        """JIT.MatMul (/root/reference/engine/nn/matmul.go:27): x [ntok][k] -> out [ntok][nrows]."""
+        if t not in quant.BLOCK:
+            return False
+        assert out.dtype == np.float32 and x.dtype == np.float32 and w.dtype == np.uint8
+        assert out.size >= ntok * nrows and x.size >= ntok * k
+        return self._served(self._l.jl_matmul(self._ctx, _ptr(out), t, _ptr(w), w.nbytes, _ptr(x),
+                                              nrows, k, ntok), "jl_matmul")
+
+    def Forget(self, w):
+        """nn.CopyForgetter.Forget: drop the device copy keyed on this host buffer."""
+        self._served(self._l.jl_forget(self._ctx, _ptr(w), w.nbytes), "jl_forget")
+
+    # -- device-pointer entry points ------------------------------------------
+    def quantize_act_dev(self, x, ntok, k, q, a_s, sum16, stream=None):
+        return self._served(self._l.jl_quantize_act_dev(self._ctx, _ptr(x), ntok, k, _ptr(q),
+                                                        _ptr(a_s), _ptr(sum16), stream),
+                            "jl_quantize_act_dev")
+
+    def dequant_dev(self, t, src, dst, n, stream=None):
+        return self._served(self._l.jl_dequant_dev(self._ctx, t, _ptr(src), _ptr(dst), n, stream),
+                            "jl_dequant_dev")
+
+    def matvec_dev(self, out, t, w, x, nrows, k, stream=None):
+        return self._served(self._l.jl_matvec_dev(self._ctx, _ptr(out), t, _ptr(w), _ptr(x),
+                                                  nrows, k, stream), "jl_matvec_dev")
+
+    def matvec_q8_dev(self, out, t, w, q, a_s, sum16, nrows, k, stream=None):
+        return self._served(self._l.jl_matvec_q8_dev(self._ctx, _ptr(out), t, _ptr(w), _ptr(q),
+                                                     _ptr(a_s), _ptr(sum16), nrows, k, stream),
+                            "jl_matvec_q8_dev")

@@ -1,0 +1,120 @@
+"""Device memory, copies and event timing over the HIP runtime the C ABI uses.
+
+Plumbing for tests and benchmarks: buffers are plain device allocations whose
+addresses go to the *_dev entry points.  The runtime is the one libjlmi.so
+resolved (jl_hip_runtime), so a process holds exactly one.
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import _lib
+
+_H2D, _D2H, _D2D = 1, 2, 3
+_hip = None
+
+
+def hip():
+    global _hip
+    if _hip is None:
+        lib = _lib.load()
+        lib.jl_hip_runtime.restype = C.c_char_p
+        name = lib.jl_hip_runtime().decode()
+        if not name:
+            raise RuntimeError("no HIP runtime could be loaded")
+        h = C.CDLL(name)
+        h.hipGetErrorString.restype = C.c_char_p
+        h.hipGetErrorString.argtypes = [C.c_int]
+        h.hipMalloc.argtypes = [C.POINTER(C.c_void_p), C.c_size_t]
+        h.hipFree.argtypes = [C.c_void_p]
+        h.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
+        h.hipMemset.argtypes = [C.c_void_p, C.c_int, C.c_size_t]
+        h.hipEventCreate.argtypes = [C.POINTER(C.c_void_p)]
+        h.hipEventRecord.argtypes = [C.c_void_p, C.c_void_p]
+        h.hipEventSynchronize.argtypes = [C.c_void_p]
+        h.hipEventElapsedTime.argtypes = [C.POINTER(C.c_float), C.c_void_p, C.c_void_p]
+        h.hipEventDestroy.argtypes = [C.c_void_p]
+        h.hipMemGetInfo.argtypes = [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]
+        _hip = h
+    return _hip
+
+
+def check(rc, what):
+    if rc != 0:
+        raise RuntimeError(f"{what}: {hip().hipGetErrorString(rc).decode()}")
+
+
+def synchronize():
+    check(hip().hipDeviceSynchronize(), "hipDeviceSynchronize")
+
+
+def mem_info():
+    free, total = C.c_size_t(), C.c_size_t()
+    check(hip().hipMemGetInfo(C.byref(free), C.byref(total)), "hipMemGetInfo")
+    return free.value, total.value
+
+
+class DeviceArray:
+    """A device allocation shaped like a numpy array."""
+
+    def __init__(self, arr=None, shape=None, dtype=None, fill=None):
+        if arr is not None:
+            arr = np.ascontiguousarray(arr)
+            shape, dtype = arr.shape, arr.dtype
+        self.shape, self.dtype = tuple(np.atleast_1d(shape)) if np.isscalar(shape) else tuple(shape), np.dtype(dtype)
+        self.nbytes = int(np.prod(self.shape)) * self.dtype.itemsize
+        p = C.c_void_p()
+        check(hip().hipMalloc(C.byref(p), max(self.nbytes, 16)), "hipMalloc")
+        self.ptr = p.value
+        if arr is not None:
+            self.put(arr)
+        elif fill is not None:
+            self.put(np.full(self.shape, fill, self.dtype))
+
+    def put(self, arr):
+        arr = np.ascontiguousarray(arr, self.dtype)
+        assert arr.nbytes == self.nbytes
+        check(hip().hipMemcpy(self.ptr, arr.ctypes.data, self.nbytes, _H2D), "hipMemcpy H2D")
+
+    def get(self):
+        out = np.empty(self.shape, self.dtype)
+        check(hip().hipMemcpy(out.ctypes.data, self.ptr, self.nbytes, _D2H), "hipMemcpy D2H")
+        return out
+
+    def copy_from(self, other):
+        assert other.nbytes == self.nbytes
+        check(hip().hipMemcpy(self.ptr, other.ptr, self.nbytes, _D2D), "hipMemcpy D2D")
+
+    def free(self):
+        if getattr(self, "ptr", None):
+            hip().hipFree(self.ptr)
+            self.ptr = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+class Event:
+    def __init__(self):
+        self.e = C.c_void_p()
+        check(hip().hipEventCreate(C.byref(self.e)), "hipEventCreate")
+
+    def record(self, stream):
+        check(hip().hipEventRecord(self.e, stream), "hipEventRecord")
+
+    def synchronize(self):
+        check(hip().hipEventSynchronize(self.e), "hipEventSynchronize")
+
+    def elapsed_ms(self, end):
+        ms = C.c_float()
+        check(hip().hipEventElapsedTime(C.byref(ms), self.e, end.e), "hipEventElapsedTime")
+        return ms.value
+
+    def __del__(self):
+        try:
+            hip().hipEventDestroy(self.e)
+        except Exception:
+            pass
