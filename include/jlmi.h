@@ -81,9 +81,9 @@ int jl_set_act_window(jl_ctx *ctx, int window);
 void *jl_stream(jl_ctx *ctx);
 int jl_synchronize(jl_ctx *ctx);
 
-/* Kernel-shape overrides for measurement: key is one of "matvec.rpw",
- * "matvec.ni", "matvec.block", "matvec.grid"; value 0 restores the built-in
- * choice (-1 for ni).  Mirrors the reference's per-instance tuning knobs
+/* Kernel-shape overrides for measurement: key is one of "matvec.rpw" (rows per
+ * wavefront: 1, 2, 4), "matvec.block" (threads per workgroup), "matvec.grid"
+ * (workgroups); value 0 restores the built-in choice.  Mirrors the reference's per-instance tuning knobs
  * (engine/nn/options.go:67-118). */
 int jl_set_tuning(jl_ctx *ctx, const char *key, int value);
 

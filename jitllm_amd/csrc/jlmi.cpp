@@ -27,7 +27,7 @@ thread_local std::string g_create_error;
 const HipApi* H = nullptr;  // the process-wide HIP runtime, resolved by the first jl_ctx_create
 
 struct Tuning {
-    int rpw = 0, ni = -1, block = 0, grid = 0;
+    int rpw = 0, block = 0, grid = 0;
 };
 
 struct Resident {
@@ -106,20 +106,13 @@ const TypeInfo* type_info(int type) {
 
 bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
-// Kernel shapes that exist in the code object (kernels/jlmi_kernels.hip).
-bool matvec_shape_exists(int type, int rpw, int ni) {
-    switch (type) {
-    case JL_TYPE_Q4_K:
-        return (ni == 0 && (rpw == 1 || rpw == 2 || rpw == 4)) ||
-               (ni == 1 && (rpw == 1 || rpw == 2 || rpw == 4)) || (ni == 2 && (rpw == 1 || rpw == 2));
-    case JL_TYPE_Q8_0:
-        return (ni == 0 && (rpw == 1 || rpw == 2 || rpw == 4)) ||
-               (ni == 1 && (rpw == 1 || rpw == 2 || rpw == 4)) ||
-               (ni == 2 && (rpw == 1 || rpw == 2)) || (ni == 4 && rpw == 1);
-    case JL_TYPE_Q6_K:
-        return (ni == 0 && (rpw == 1 || rpw == 2)) || (ni == 1 && (rpw == 1 || rpw == 2 || rpw == 4));
-    }
-    return false;
+// Largest workgroup of the matvec variant with `rpw` rows per wavefront, 0 when the
+// code object has no such variant (kernels/jlmi_kernels.hip).
+int matvec_max_block(int type, int rpw) {
+    if (rpw == 1) return 1024;
+    if (rpw == 2) return type == JL_TYPE_Q6_K ? 512 : 1024;
+    if (rpw == 4) return type == JL_TYPE_Q8_0 ? 1024 : 512;
+    return 0;
 }
 
 hipStream_t pick_stream(jl_ctx* c, void* s) { return s ? (hipStream_t)s : c->stream; }
@@ -157,31 +150,20 @@ int matvec_launch(jl_ctx* c, float* out, int type, const void* w, const float* x
     if (type == JL_TYPE_Q4_K && !aligned16(w)) return JL_DECLINED;
     if (((uintptr_t)w & 1) != 0) return JL_DECLINED;
 
-    const int nslots = k / ti->slot_elems;
-    const int iters = (nslots + 63) / 64;
-
-    // Shape choice.  Small matrices: one row per wavefront with every load of the
-    // row unrolled, 16 wavefronts per workgroup so a CU quantizes x once.  Larger
-    // ones: more rows per wavefront (activation registers are reused) and a grid
-    // that covers the chip a few times over.
-    int ni = c->tune.ni, rpw = c->tune.rpw, block = c->tune.block;
-    if (ni < 0) ni = iters <= 2 ? iters : 0;
-    if (ni > 0 && ni < iters) ni = 0;  // an unrolled shape must cover the whole row
-    if (rpw <= 0) {
-        rpw = 1;
-        long waves = nrows;
-        if (waves >= 4L * c->num_cu * 16) rpw = 2;
-    }
-    while (!matvec_shape_exists(type, rpw, ni)) {
-        if (rpw > 1) rpw >>= 1;
-        else if (ni != 0) ni = 0;
-        else return fail(c, JL_ERR_ARG, "matvec: no kernel shape");
-    }
-    if (block <= 0) block = 1024;
+    // Shape choice, from sweeps on MI355X: one row per wavefront; a matrix with at
+    // most sixteen rows per CU runs one 16-wavefront workgroup per CU (the CU
+    // quantizes x once), larger ones a persistent grid of two 12-wavefront
+    // workgroups per CU that stride over the row groups.
+    int rpw = c->tune.rpw, block = c->tune.block;
+    if (rpw <= 0) rpw = 1;
+    if (rpw != 1 && rpw != 2 && rpw != 4) return fail(c, JL_ERR_ARG, "matvec: rpw=%d", rpw);
+    const bool small = nrows <= 16 * c->num_cu;
+    if (block <= 0) block = (small || type == JL_TYPE_Q6_K) ? 1024 : 768;
     if (block % 64 != 0 || block > 1024) return fail(c, JL_ERR_ARG, "matvec: block=%d", block);
+    if (block > matvec_max_block(type, rpw)) block = matvec_max_block(type, rpw);
     const int rows_per_block = (block / 64) * rpw;
     long groups = ((long)nrows + rows_per_block - 1) / rows_per_block;
-    long grid = c->tune.grid > 0 ? c->tune.grid : groups;
+    long grid = c->tune.grid > 0 ? c->tune.grid : (long)c->num_cu * 2;
     if (grid > groups) grid = groups;
     if (grid < 1) grid = 1;
 
@@ -197,7 +179,7 @@ int matvec_launch(jl_ctx* c, float* out, int type, const void* w, const float* x
     a.row_bytes = (k / ti->block_elems) * ti->block_bytes;
     a.per = c->act_window / 32;
     char name[64];
-    snprintf(name, sizeof name, "jl_matvec_%s_r%d_n%d", ti->tag, rpw, ni);
+    snprintf(name, sizeof name, "jl_matvec_%s_r%d", ti->tag, rpw);
     void* params[] = {&a};
     unsigned lds = (unsigned)((size_t)k + (size_t)(k / 32) * 4 + (size_t)(k / 16) * 4);
     return launch(c, name, (unsigned)grid, 1, (unsigned)block, lds, st, params);
@@ -279,13 +261,11 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     std::vector<std::string> names = {"jl_quantize_act", "jl_dequant"};
     const int types[] = {JL_TYPE_Q4_K, JL_TYPE_Q8_0, JL_TYPE_Q6_K};
     for (int t : types)
-        for (int rpw : {1, 2, 4})
-            for (int ni : {0, 1, 2, 4})
-                if (matvec_shape_exists(t, rpw, ni)) {
-                    char nm[64];
-                    snprintf(nm, sizeof nm, "jl_matvec_%s_r%d_n%d", type_info(t)->tag, rpw, ni);
-                    names.push_back(nm);
-                }
+        for (int rpw : {1, 2, 4}) {
+            char nm[64];
+            snprintf(nm, sizeof nm, "jl_matvec_%s_r%d", type_info(t)->tag, rpw);
+            names.push_back(nm);
+        }
     for (const auto& n : names) {
         hipFunction_t f;
         e = H->ModuleGetFunction(&f, c->module, n.c_str());
@@ -337,7 +317,6 @@ int jl_synchronize(jl_ctx* c) {
 int jl_set_tuning(jl_ctx* c, const char* key, int value) {
     if (!c || !key) return JL_ERR_ARG;
     if (!strcmp(key, "matvec.rpw")) c->tune.rpw = value;
-    else if (!strcmp(key, "matvec.ni")) c->tune.ni = value;
     else if (!strcmp(key, "matvec.block")) c->tune.block = value;
     else if (!strcmp(key, "matvec.grid")) c->tune.grid = value;
     else return fail(c, JL_ERR_ARG, "unknown tuning key %s", key);
@@ -356,7 +335,7 @@ int jl_quantize_act_dev(jl_ctx* c, const float* x, int ntok, int k, int8_t* q, f
     HIP_TRY(c, H->SetDevice(c->device));
     int per = c->act_window / 32;
     void* params[] = {(void*)&x, (void*)&q, (void*)&as, (void*)&sum16, (void*)&k, (void*)&per};
-    unsigned gx = (unsigned)((k / 16 + 255) / 256);
+    unsigned gx = (unsigned)((k / 4 + 255) / 256);  // one thread per four elements
     return launch(c, "jl_quantize_act", gx, (unsigned)ntok, 256, 0, pick_stream(c, stream), params);
 }
 

@@ -40,10 +40,33 @@ __device__ __forceinline__ i32 dot4(u32 a, u32 b, i32 c) {
     return __builtin_amdgcn_sdot4((i32)a, (i32)b, c, false);
 }
 
-// Sum over the 64 lanes of a wavefront; every lane gets the total.
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, JL_WAVE);
+// Data-parallel-primitive lane moves (DPP): the value of another lane of the
+// same 16-lane row, or of the previous row's last lane, with no LDS traffic.
+#define JL_DPP_QUAD_XOR1 0xB1      // quad_perm [1,0,3,2]
+#define JL_DPP_QUAD_XOR2 0x4E      // quad_perm [2,3,0,1]
+#define JL_DPP_ROW_HALF_MIRROR 0x141
+#define JL_DPP_ROW_MIRROR 0x140
+#define JL_DPP_ROW_BCAST15 0x142
+#define JL_DPP_ROW_BCAST31 0x143
+
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ i32 dpp_i32(i32 old, i32 v) {
+    return __builtin_amdgcn_update_dpp(old, v, CTRL, ROW_MASK, 0xf, false);
+}
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_f32(float v) {  // lanes outside ROW_MASK read 0
+    return __builtin_bit_cast(float, dpp_i32<CTRL, ROW_MASK>(0, __builtin_bit_cast(i32, v)));
+}
+
+// Sum over the 64 lanes of a wavefront with DPP adds; the total lands in lane 63
+// (and in every lane of the last 16-lane row).
+__device__ __forceinline__ float wave_sum_to_lane63(float v) {
+    v += dpp_f32<JL_DPP_QUAD_XOR1, 0xf>(v);
+    v += dpp_f32<JL_DPP_QUAD_XOR2, 0xf>(v);
+    v += dpp_f32<JL_DPP_ROW_HALF_MIRROR, 0xf>(v);
+    v += dpp_f32<JL_DPP_ROW_MIRROR, 0xf>(v);       // every lane: its row's sum
+    v += dpp_f32<JL_DPP_ROW_BCAST15, 0xa>(v);      // rows 1,3 += rows 0,2
+    v += dpp_f32<JL_DPP_ROW_BCAST31, 0xc>(v);      // rows 2,3 += rows 0+1
     return v;
 }
 

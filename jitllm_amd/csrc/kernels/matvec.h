@@ -51,30 +51,37 @@ __device__ __forceinline__ void stage_act_copy(uint8_t* smem, const int8_t* q, c
     for (int i = threadIdx.x; i < k / 16; i += blockDim.x) ss[i] = s16[i];
 }
 
-// Quantize f32 x into the LDS staging area (same bits as the standalone
-// quantizer).  k % 32 == 0, blockDim.x % 64 == 0, per = window / 32.
-__device__ __forceinline__ void stage_act_quantize(uint8_t* smem, const float* x, int k, int per) {
-    u32x4* a = (u32x4*)smem;
+// Quantize one float4 of x (element group g4, i.e. elements 4*g4 .. 4*g4+3) into the
+// LDS staging area; every lane of a wavefront must call it together (DPP).
+__device__ __forceinline__ void stage_quantize4(uint8_t* smem, int k, int per, int g4, f32x4 v) {
+    u32* a = (u32*)smem;
     float* da = (float*)(smem + k);
     float* ss = (float*)(smem + k + (k / 32) * 4);
-    int nhb = k / 16;
-    int nhb_pad = (nhb + 15) & ~15;  // whole 16-lane rows take part in the shuffles
-    for (int hb = threadIdx.x; hb < nhb_pad; hb += blockDim.x) {
-        f32x4 v[4];
-        bool live = hb < nhb;
-#pragma unroll
-        for (int i = 0; i < 4; i++)
-            v[i] = live ? ((const f32x4*)x)[hb * 4 + i] : f32x4{0.f, 0.f, 0.f, 0.f};
-        u32 amax = window_amax(half_block_amax(v), per);
-        u32 q[4];
-        float d;
-        i32 sum;
-        quantize_half_block(v, amax, q, d, sum);
-        if (live) {
-            a[hb] = u32x4{q[0], q[1], q[2], q[3]};
-            ss[hb] = (float)sum;
-            if ((hb & 1) == 0) da[hb >> 1] = d;
-        }
+    const bool live = g4 < k / 4;
+    u32 m = max(max(abs_bits(v.x), abs_bits(v.y)), max(abs_bits(v.z), abs_bits(v.w)));
+    u32 amax = window_amax(live ? m : 0u, per);
+    float d;
+    i32 sum;
+    u32 q = quantize4(v, amax, d, sum);
+    if (live) {
+        a[g4] = q;
+        if ((g4 & 3) == 0) ss[g4 >> 2] = (float)sum;
+        if ((g4 & 7) == 0) da[g4 >> 3] = d;
+    }
+}
+
+// Quantize f32 x into the LDS staging area (same bits as the standalone
+// quantizer).  k % 32 == 0, blockDim.x % 64 == 0, per = window / 32.  `first` is
+// this thread's first float4 of x, loaded by the caller ahead of time.
+__device__ __forceinline__ void stage_act_quantize(uint8_t* smem, const float* x, int k, int per,
+                                                   f32x4 first) {
+    const int n4 = k / 4;
+    const int n4_pad = (n4 + 63) & ~63;  // whole wavefronts take part in the lane exchanges
+    int g4 = threadIdx.x;
+    if (g4 < n4_pad) stage_quantize4(smem, k, per, g4, first);
+    for (g4 += blockDim.x; g4 < n4_pad; g4 += blockDim.x) {
+        f32x4 v = g4 < n4 ? ((const f32x4*)x)[g4] : f32x4{0.f, 0.f, 0.f, 0.f};
+        stage_quantize4(smem, k, per, g4, v);
     }
 }
 
@@ -273,97 +280,59 @@ template <> struct SlotTraits<JL_Q6_K> {
 };
 
 
-// One wavefront computes RPW rows at a time; NI = slot iterations per lane
-// unrolled so that every load of a row group is issued before the first use
-// (NI == 0: generic loop for long rows).
-template <int TYPE, int RPW, int NI>
+// One wavefront computes RPW rows at a time and strides over the row groups of
+// a persistent grid.  The first group's weight loads are issued before the
+// activation is staged, so HBM latency overlaps the quantizer; after that each
+// group is load -> dot -> cross-lane reduce, and the wavefronts of a CU (two
+// workgroups of eight, or one of sixteen) cover each other's memory latency.
+template <int TYPE, int RPW>
 __device__ __forceinline__ void matvec_body(const MatVecArgs& p, uint8_t* smem) {
     typedef SlotTraits<TYPE> T;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
     const int nslots = p.k / T::kElems;
     const int rows_per_block = nwaves * RPW;
+    const int group_stride = gridDim.x * rows_per_block;
     const ActLds A = act_lds_views(smem, p.k);
-
     int r0 = blockIdx.x * rows_per_block + wave * RPW;
 
-    if constexpr (NI > 0) {
-        // Issue the first row group's weight loads before staging activations,
-        // so HBM latency overlaps the quantizer.
-        typename T::W w[NI][RPW];
-#pragma unroll
-        for (int i = 0; i < NI; i++) {
-            int s = min(lane + 64 * i, nslots - 1);
-#pragma unroll
-            for (int j = 0; j < RPW; j++) {
-                int r = min(r0 + j, p.nrows - 1);
-                T::load_w(p.w + (size_t)r * p.row_bytes, s, w[i][j]);
-            }
-        }
-        if (p.x) stage_act_quantize(smem, p.x, p.k, p.per);
-        else stage_act_copy(smem, p.q, p.as, p.s16, p.k);
-        __syncthreads();
-        typename T::Act a[NI];
-#pragma unroll
-        for (int i = 0; i < NI; i++) T::load_act(A, min(lane + 64 * i, nslots - 1), a[i]);
+    // The activation loads go first: loads return in order, so the quantizer can
+    // start as soon as x is back while the first weight loads are still in flight.
+    f32x4 x0 = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (p.x && (int)threadIdx.x < p.k / 4) x0 = ((const f32x4*)p.x)[threadIdx.x];
 
-        for (;;) {
-            float acc[RPW];
+    typename T::W w[RPW];
+    {
+        const int s = min(lane, nslots - 1);
 #pragma unroll
-            for (int j = 0; j < RPW; j++) acc[j] = 0.f;
+        for (int j = 0; j < RPW; j++)
+            T::load_w(p.w + (size_t)min(r0 + j, p.nrows - 1) * p.row_bytes, s, w[j]);
+    }
+    if (p.x) stage_act_quantize(smem, p.x, p.k, p.per, x0);
+    else stage_act_copy(smem, p.q, p.as, p.s16, p.k);
+    __syncthreads();
+
+    bool preloaded = true;
+    for (; r0 < p.nrows; r0 += group_stride) {
+        float acc[RPW];
 #pragma unroll
-            for (int i = 0; i < NI; i++) {
-                int s = lane + 64 * i;
-                if (s < nslots) {
+        for (int j = 0; j < RPW; j++) acc[j] = 0.f;
+        for (int slot = lane; slot < nslots; slot += 64) {
+            if (!preloaded) {
 #pragma unroll
-                    for (int j = 0; j < RPW; j++) acc[j] += T::dot(w[i][j], s, a[i]);
-                }
+                for (int j = 0; j < RPW; j++)
+                    T::load_w(p.w + (size_t)min(r0 + j, p.nrows - 1) * p.row_bytes, slot, w[j]);
             }
-            int rdone = r0;
-            r0 += gridDim.x * rows_per_block;
-            bool more = r0 < p.nrows;  // uniform per wave
-            if (more) {
+            preloaded = false;
+            typename T::Act a;
+            T::load_act(A, slot, a);
 #pragma unroll
-                for (int i = 0; i < NI; i++) {
-                    int s = min(lane + 64 * i, nslots - 1);
-#pragma unroll
-                    for (int j = 0; j < RPW; j++) {
-                        int r = min(r0 + j, p.nrows - 1);
-                        T::load_w(p.w + (size_t)r * p.row_bytes, s, w[i][j]);
-                    }
-                }
-            }
-#pragma unroll
-            for (int j = 0; j < RPW; j++) {
-                float t = wave_sum(acc[j]);
-                if (lane == 0 && rdone + j < p.nrows) p.out[rdone + j] = t;
-            }
-            if (!more) break;
+            for (int j = 0; j < RPW; j++) acc[j] += T::dot(w[j], slot, a);
         }
-    } else {
-        if (p.x) stage_act_quantize(smem, p.x, p.k, p.per);
-        else stage_act_copy(smem, p.q, p.as, p.s16, p.k);
-        __syncthreads();
-        for (; r0 < p.nrows; r0 += gridDim.x * rows_per_block) {
-            float acc[RPW];
+        preloaded = false;
 #pragma unroll
-            for (int j = 0; j < RPW; j++) acc[j] = 0.f;
-            for (int s = lane; s < nslots; s += 64) {
-                typename T::Act a;
-                typename T::W w[RPW];
-#pragma unroll
-                for (int j = 0; j < RPW; j++) {
-                    int r = min(r0 + j, p.nrows - 1);
-                    T::load_w(p.w + (size_t)r * p.row_bytes, s, w[j]);
-                }
-                T::load_act(A, s, a);
-#pragma unroll
-                for (int j = 0; j < RPW; j++) acc[j] += T::dot(w[j], s, a);
-            }
-#pragma unroll
-            for (int j = 0; j < RPW; j++) {
-                float t = wave_sum(acc[j]);
-                if (lane == 0 && r0 + j < p.nrows) p.out[r0 + j] = t;
-            }
+        for (int j = 0; j < RPW; j++) {
+            float t = wave_sum_to_lane63(acc[j]);
+            if (lane == 63 && r0 + j < p.nrows) p.out[r0 + j] = t;
         }
     }
 }

@@ -7,56 +7,57 @@
 //   q = round-half-away-from-zero(f32(x * inv)),
 //   as[b] = d, sum16[h] = sum of q over 16 elements (stored as f32, exact).
 //
-// One thread owns one 16-element half-block; the window's amax is combined
-// across the 2*per lanes that share it with cross-lane xor shuffles, so a
-// window never leaves a 16-lane row.
+// One thread owns four consecutive elements.  A 16-element half-block is a
+// quad of lanes, a 32-element block eight lanes, a window 8*per lanes, so the
+// window's amax and the half-block sums are combined with DPP lane moves.
 #pragma once
 #include "common.h"
 
 #pragma clang fp contract(off)
 
 // |v| as an integer bit pattern: comparing these orders the magnitudes exactly
-// as the reference's sign-cleared integer compare does (NaNs included).
+// as the reference's sign-cleared integer compare does.
 __device__ __forceinline__ u32 abs_bits(float v) { return __float_as_uint(v) & 0x7FFFFFFFu; }
 
-// amax bits over this thread's 16 values (all zero when the half-block is past
-// the end of the vector).
-__device__ __forceinline__ u32 half_block_amax(const f32x4 v[4]) {
-    u32 m = 0;
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        m = max(m, abs_bits(v[i].x));
-        m = max(m, abs_bits(v[i].y));
-        m = max(m, abs_bits(v[i].z));
-        m = max(m, abs_bits(v[i].w));
-    }
-    return m;
+template <int CTRL>
+__device__ __forceinline__ u32 dpp_max_u32(u32 m) {
+    return max(m, (u32)dpp_i32<CTRL, 0xf>(0, (i32)m));
 }
 
-// Combine amax over the 2*per consecutive lanes of a window (per = window/32,
-// a power of two <= 8).  Lanes of one window are aligned to 2*per.
+// amax bits over the 8*per consecutive lanes of a window (per = window/32, a power
+// of two <= 8); lanes of one window are aligned to 8*per.
 __device__ __forceinline__ u32 window_amax(u32 m, int per) {
-    for (int x = 1; x < 2 * per; x <<= 1) m = max(m, (u32)__shfl_xor((int)m, x, JL_WAVE));
+    m = dpp_max_u32<JL_DPP_QUAD_XOR1>(m);
+    m = dpp_max_u32<JL_DPP_QUAD_XOR2>(m);
+    m = dpp_max_u32<JL_DPP_ROW_HALF_MIRROR>(m);  // 8 lanes = one 32-element block
+    if (per >= 2) m = dpp_max_u32<JL_DPP_ROW_MIRROR>(m);
+    if (per >= 4) m = max(m, (u32)__shfl_xor((int)m, 16, JL_WAVE));
+    if (per >= 8) m = max(m, (u32)__shfl_xor((int)m, 32, JL_WAVE));
     return m;
 }
 
-// Quantize 16 values with the window's amax.  q[4] = 16 int8 packed little
-// endian; returns the scale d and the integer sum.
-__device__ __forceinline__ void quantize_half_block(const f32x4 v[4], u32 amax_bits, u32 q[4],
-                                                    float& d_out, i32& sum_out) {
+// Round half away from zero for |p| < 2^22, exactly: adding 0.5 - 2^-25 (the
+// largest f32 below one half) cannot carry a value below n + 0.5 up to n + 1,
+// and carries every value at or above it; the conversion then truncates.
+__device__ __forceinline__ i32 round_half_away(float p) {
+    const float c = __uint_as_float(0x3EFFFFFFu);
+    return (i32)(p + __builtin_copysignf(c, p));
+}
+
+// Quantize this thread's four values with the window's amax.  Returns the four
+// int8 packed little endian, the scale d, and the sum over the 16-element
+// half-block (identical in the four lanes of the quad).
+__device__ __forceinline__ u32 quantize4(f32x4 v, u32 amax_bits, float& d_out, i32& sum16_out) {
     float amax = __uint_as_float(amax_bits);
     float d = amax / 127.0f;
     float inv = d != 0.0f ? 1.0f / d : 0.0f;
-    i32 sum = 0;
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        i32 a = (i32)__builtin_roundf(v[i].x * inv);
-        i32 b = (i32)__builtin_roundf(v[i].y * inv);
-        i32 c = (i32)__builtin_roundf(v[i].z * inv);
-        i32 e = (i32)__builtin_roundf(v[i].w * inv);
-        q[i] = (u32)(a & 0xFF) | ((u32)(b & 0xFF) << 8) | ((u32)(c & 0xFF) << 16) | ((u32)e << 24);
-        sum += a + b + c + e;
-    }
+    i32 a = round_half_away(v.x * inv), b = round_half_away(v.y * inv);
+    i32 c = round_half_away(v.z * inv), e = round_half_away(v.w * inv);
+    u32 q = (u32)(a & 0xFF) | ((u32)(b & 0xFF) << 8) | ((u32)(c & 0xFF) << 16) | ((u32)e << 24);
+    i32 s = a + b + c + e;
+    s += dpp_i32<JL_DPP_QUAD_XOR1, 0xf>(0, s);
+    s += dpp_i32<JL_DPP_QUAD_XOR2, 0xf>(0, s);
     d_out = d;
-    sum_out = sum;
+    sum16_out = s;
+    return q;
 }

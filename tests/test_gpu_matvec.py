@@ -143,7 +143,7 @@ def test_matvec_fused_vs_oracle(dev, devbuf, t, shape, weights):
 
 @pytest.mark.parametrize("t", TYPES)
 def test_matvec_every_kernel_shape(dev, devbuf, t):
-    """Each (rows per wavefront, unroll, workgroup) variant computes the same rows."""
+    """Each (rows per wavefront, workgroup, grid) variant computes the same rows."""
     window = 32
     dev.SetActWindow(window)
     for nrows, k in [(75, 2048), (530, 4096), (70, 8192)]:
@@ -152,16 +152,15 @@ def test_matvec_every_kernel_shape(dev, devbuf, t):
         want = _like_for_like(t, w, x, nrows, k, window)
         wd, xd = devbuf(w), devbuf(x)
         for rpw in (1, 2, 4):
-            for ni in (0, 1, 2, 4):
-                for block in (64, 256, 1024):
-                    for grid in (0, 3):
-                        dev.set_tuning(rpw=rpw, ni=ni, block=block, grid=grid)
-                        out = devbuf(shape=(nrows,), dtype=np.float32, fill=np.float32(-3e33))
-                        assert dev.matvec_dev(out.ptr, t, wd.ptr, xd.ptr, nrows, k)
-                        dev.synchronize()
-                        e = nmse(out.get(), want)
-                        assert e <= 1e-10, f"{nrows}x{k} rpw={rpw} ni={ni} block={block} grid={grid}: {e:.3e}"
-    dev.set_tuning(rpw=0, ni=-1, block=0, grid=0)
+            for block in (64, 256, 512, 1024):
+                for grid in (0, 1, 3):
+                    dev.set_tuning(rpw=rpw, block=block, grid=grid)
+                    out = devbuf(shape=(nrows,), dtype=np.float32, fill=np.float32(-3e33))
+                    assert dev.matvec_dev(out.ptr, t, wd.ptr, xd.ptr, nrows, k)
+                    dev.synchronize()
+                    e = nmse(out.get(), want)
+                    assert e <= 1e-10, f"{nrows}x{k} rpw={rpw} block={block} grid={grid}: {e:.3e}"
+    dev.set_tuning(rpw=0, block=0, grid=0)
 
 
 @pytest.mark.parametrize("t", TYPES)
