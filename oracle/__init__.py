@@ -258,3 +258,62 @@ def group_pairs(sel, rows, k, n_exp, unit):
     if used < 0:
         raise ValueError("group_pairs refused")
     return used, perm, col_e, pos
+
+
+# --------------------------------------------------------------- CPU baseline
+class CpuPath:
+    """The intrinsic restatement of the reference's host kernels (jl_cpu_path.c):
+    activation quantizer + fused packed matvec on a spinning worker pool."""
+
+    def __init__(self, threads):
+        lib = os.path.join(_HERE, "libjl_cpu_path.so")
+        if not os.path.exists(lib):
+            build()
+        self._l = C.CDLL(lib)
+        self._l.jlc_pool_create.restype = C.c_void_p
+        self._l.jlc_pool_create.argtypes = [C.c_int]
+        self._l.jlc_pool_destroy.argtypes = [C.c_void_p]
+        self._l.jlc_has_vnni.argtypes = [C.c_void_p]
+        self._l.jlc_matvec_packed.argtypes = [C.c_void_p, _f32p, C.c_int, _u32p, _u32p, _u32p, _f32p,
+                                              C.c_int, C.c_int, C.c_int]
+        pp = C.POINTER(_u32p)
+        self._l.jlc_time_matvec.restype = C.c_double
+        self._l.jlc_time_matvec.argtypes = [C.c_void_p, _f32p, C.c_int, pp, pp, pp, C.c_int, _f32p,
+                                            C.c_int, C.c_int, C.c_int, C.c_int]
+        self._l.jlc_membw.restype = C.c_double
+        self._l.jlc_membw.argtypes = [C.c_int, C.c_size_t, C.c_int]
+        self.threads = threads
+        self._p = self._l.jlc_pool_create(threads)
+
+    def close(self):
+        if self._p:
+            self._l.jlc_pool_destroy(self._p)
+            self._p = None
+
+    @property
+    def vnni(self):
+        return bool(self._l.jlc_has_vnni(self._p))
+
+    def matvec_packed(self, t, qs, d, sc, x, nrows, k, window):
+        qs, d, sc = _planes(t, qs, d, sc, nrows, k)
+        x = _chk(x, np.float32, k)
+        out = np.zeros(nrows, np.float32)
+        if self._l.jlc_matvec_packed(self._p, _p(out, _f32p), t, _p(qs, _u32p), _p(d, _u32p),
+                                     _p(sc, _u32p), _p(x, _f32p), nrows, k, window):
+            raise ValueError("cpu matvec refused")
+        return out
+
+    def time_matvec(self, t, copies, x, nrows, k, window, reps=5):
+        """copies: list of (qs, d, sc) distinct plane sets.  Seconds per call (best of reps)."""
+        n = len(copies)
+        arr = lambda i: (_u32p * n)(*[_p(c[i], _u32p) for c in copies])
+        x = _chk(x, np.float32, k)
+        out = np.zeros(nrows, np.float32)
+        s = self._l.jlc_time_matvec(self._p, _p(out, _f32p), t, arr(0), arr(1), arr(2), n,
+                                    _p(x, _f32p), nrows, k, window, reps)
+        if s < 0:
+            raise ValueError("cpu timing refused")
+        return s
+
+    def membw(self, nbytes=1 << 30, reps=3):
+        return self._l.jlc_membw(self.threads, nbytes, reps)
