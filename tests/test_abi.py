@@ -1,0 +1,76 @@
+"""CPU tests of the host side: the C ABI library loads and exports every symbol the
+header declares, the container reader parses the reference-written fixture, and the
+product never reaches into the oracle."""
+import os
+import re
+
+import numpy as np
+import pytest
+
+from conftest import GOLDEN, ROOT
+from jitllm_amd import _lib, jlm, quant
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "jlmi.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(jl_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    names = _declared()
+    assert len(names) >= 12
+    for n in names:
+        assert hasattr(lib, n), f"libjlmi.so lacks {n}"
+    assert sorted(_lib.SIGNATURES) == names, "the ctypes table and the header disagree"
+
+
+def test_code_object_is_built():
+    assert os.path.getsize(_lib.CODE_OBJECT_PATH) > 1000
+
+
+def test_context_creation_fails_loudly_without_a_gpu():
+    import ctypes as C
+    lib = _lib.load()
+    ctx = C.c_void_p()
+    opts = _lib.Options(0, 32, b"/nonexistent/code_object.hsaco")
+    rc = lib.jl_ctx_create(C.byref(ctx), C.byref(opts))
+    assert rc < 0 and not ctx.value           # no device here, or no such code object on a GPU box
+    assert lib.jl_last_error(None)
+
+
+def test_product_never_imports_the_oracle():
+    """The oracle is test infrastructure: nothing under jitllm_amd/ may import, load or
+    link it (the reference enforces the same for its own, internal/oracle/oracle.go:4-5)."""
+    pkg = os.path.join(ROOT, "jitllm_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".cpp", ".h", ".hip", "Makefile")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert not re.search(r"^\s*(import|from)\s+oracle\b", text, re.M), f
+                assert "jl_oracle" not in text and "libjl_cpu_path" not in text, f
+
+
+def test_act_window_rule():
+    assert quant.act_window([quant.Q4_K, quant.Q6_K]) == 256
+    assert quant.act_window([quant.Q4_K, quant.Q8_0]) == 32
+    assert quant.act_window([]) == 32
+
+
+def test_jlm_reader_on_the_reference_written_container():
+    f = jlm.File.open(os.path.join(GOLDEN, "v29.jlm.gz"))
+    assert (f.version, f.n_blocks, f.n_tensors, f.n_exp_pages) == (29, 2, 12, 8)
+    assert (f.page_size, f.exp_page_size, f.exp_data_off, f.dense_off) == (24576, 24576, 77824, 4096)
+    assert len(f.entries) == 12
+    bank = [e for e in f.entries if e.name == "exp_gate_bank" and e.block == 1][0]
+    assert (bank.k, bank.rows, bank.sheets) == (256, 16, 4)
+    t, qs, d, sc = f.planes(bank, 3)
+    assert t == quant.Q4_K and (qs.size, d.size, sc.size) == quant.packed_words(quant.Q4_K, 16, 256)
+    with pytest.raises(ValueError):
+        f.planes(bank, 4)
+    q5 = [e for e in f.entries if e.name == "attn_q"][0]
+    with pytest.raises(ValueError):
+        f.planes(q5)                       # Q5_K is not a type of this path
+    with pytest.raises(ValueError):
+        jlm.File(b"not a container" * 20)
