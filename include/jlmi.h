@@ -83,7 +83,8 @@ int jl_synchronize(jl_ctx *ctx);
 
 /* Kernel-shape overrides for measurement: key is one of "matvec.rpw" (rows per
  * wavefront: 1, 2, 4), "matvec.block" (threads per workgroup), "matvec.grid"
- * (workgroups); value 0 restores the built-in choice.  Mirrors the reference's per-instance tuning knobs
+ * (workgroups), "gemm.min_tok" (fewest tokens sent to the matrix-core GEMM);
+ * value 0 restores the built-in choice.  Mirrors the reference's per-instance tuning knobs
  * (engine/nn/options.go:67-118). */
 int jl_set_tuning(jl_ctx *ctx, const char *key, int value);
 
@@ -128,6 +129,21 @@ int jl_matvec_dev(jl_ctx *ctx, float *out, int type, const void *w, const float 
  * (the reference caches them across matvecs that share x, engine/nn/packed.go:282). */
 int jl_matvec_q8_dev(jl_ctx *ctx, float *out, int type, const void *w, const int8_t *q,
                      const float *as, const float *sum16, int nrows, int k, void *stream);
+
+/* JIT.MatMulPacked / MatMul semantics on resident operands (engine/nn/packedmm.go:23,
+ * matmul.go:27): x [ntok][k] f32 -> out [ntok][nrows], every token quantized on
+ * its own.  Q4_K with the 256 window runs the matrix-core GEMM (quantize-and-
+ * lay-out kernel, then the GEMM kernel, in a workspace the context owns); other
+ * cases run one fused matvec launch per token, which the reference also falls
+ * back to (engine/model/prefill.go:1036-1041).  The workspace grows on demand
+ * (a device allocation); jl_reserve sizes it ahead of time. */
+int jl_matmul_dev(jl_ctx *ctx, float *out, int type, const void *w, const float *x,
+                  int nrows, int k, int ntok, void *stream);
+
+/* nn.LayerDevice.Reserve(maxRows, maxK) (engine/nn/device.go:1096-1176): size the
+ * prefill workspace for up to max_tok tokens of max_k features now, so later
+ * calls allocate nothing. */
+int jl_reserve(jl_ctx *ctx, int max_tok, int max_k);
 
 #ifdef __cplusplus
 }

@@ -36,6 +36,8 @@ SIGNATURES = {
     "jl_dequant_dev": (_int, [_vp, _int, _vp, _vp, _sz, _vp]),
     "jl_matvec_dev": (_int, [_vp, _vp, _int, _vp, _vp, _int, _int, _vp]),
     "jl_matvec_q8_dev": (_int, [_vp, _vp, _int, _vp, _vp, _vp, _vp, _int, _int, _vp]),
+    "jl_matmul_dev": (_int, [_vp, _vp, _int, _vp, _vp, _int, _int, _int, _vp]),
+    "jl_reserve": (_int, [_vp, _int, _int]),
 }
 
 _lib = None

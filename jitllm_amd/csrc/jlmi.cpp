@@ -46,8 +46,13 @@ struct jl_ctx {
     std::string err;
     std::mutex mu;  // serialises the host-pointer seam (one staging area per context)
     Tuning tune;
+    int gemm_min_tok = 8;  // below this a per-token matvec loop reads the weights as cheaply
     int num_cu = 0;
     size_t lds_limit = 0;
+
+    // prefill GEMM workspace (quantized activations in stage layout), grown on demand
+    void* gemm_ws = nullptr;
+    size_t gemm_ws_bytes = 0;
 
     // host-pointer seam state
     std::map<const void*, Resident> resident;
@@ -218,6 +223,70 @@ int resident_weight(jl_ctx* c, const void* w, size_t bytes, void** dev) {
     return JL_OK;
 }
 
+constexpr int kGemmTile = 128;         // tokens and rows per workgroup (kernels/gemm_q4k.h)
+constexpr int kGemmStride = 152;       // f16 per stage row
+constexpr unsigned kGemmLdsBytes = 4u * kGemmTile * kGemmStride * 2u + 2u * 2u * kGemmTile * 4u + 2u * kGemmTile * 4u;
+
+size_t gemm_ws_need(int ntok, int k) {
+    size_t tok_pad = ((size_t)ntok + kGemmTile - 1) / kGemmTile * kGemmTile;
+    size_t nsb = (size_t)k / 256;
+    return nsb * 2 * tok_pad * kGemmStride * 2 + nsb * tok_pad * 4;
+}
+
+int gemm_ws_ensure(jl_ctx* c, size_t need) {
+    if (c->gemm_ws_bytes >= need) return JL_OK;
+    // growing frees the old workspace: wait for work that may still read it
+    HIP_TRY(c, H->StreamSynchronize(c->stream));
+    if (c->gemm_ws) HIP_TRY(c, H->Free(c->gemm_ws));
+    c->gemm_ws = nullptr;
+    c->gemm_ws_bytes = 0;
+    HIP_TRY(c, H->Malloc(&c->gemm_ws, need));
+    c->gemm_ws_bytes = need;
+    return JL_OK;
+}
+
+// Q4_K prefill GEMM on the f16 matrix cores; operands are device pointers.
+int gemm_q4k_launch(jl_ctx* c, float* out, const void* w, const float* x, int nrows, int k, int ntok,
+                    hipStream_t st) {
+    const int tok_pad = (ntok + kGemmTile - 1) / kGemmTile * kGemmTile;
+    const int nsb = k / 256;
+    int rc = gemm_ws_ensure(c, gemm_ws_need(ntok, k));
+    if (rc != JL_OK) return rc;
+    uint16_t* bq = (uint16_t*)c->gemm_ws;
+    float* da = (float*)((char*)c->gemm_ws + (size_t)nsb * 2 * tok_pad * kGemmStride * 2);
+    GemmPrepArgs pa;
+    pa.x = x; pa.bq = bq; pa.da = da; pa.ntok = ntok; pa.tok_pad = tok_pad; pa.k = k;
+    void* pp[] = {&pa};
+    rc = launch(c, "jl_gemm_prep_q4k", (unsigned)nsb, (unsigned)(tok_pad / 4), 256, 0, st, pp);
+    if (rc != JL_OK) return rc;
+    GemmArgs ga;
+    ga.out = out; ga.w = (const uint8_t*)w; ga.bq = bq; ga.da = da;
+    ga.nrows = nrows; ga.k = k; ga.ntok = ntok; ga.tok_pad = tok_pad; ga.row_bytes = nsb * 144;
+    void* gp[] = {&ga};
+    return launch(c, "jl_gemm_q4k", (unsigned)(tok_pad / kGemmTile),
+                  (unsigned)((nrows + kGemmTile - 1) / kGemmTile), 256, kGemmLdsBytes, st, gp);
+}
+
+// out [ntok][nrows] = x [ntok][k] W^T on device operands: the matrix-core GEMM where it
+// applies, else one fused matvec launch per token (same values, token by token).
+int matmul_launch(jl_ctx* c, float* out, int type, const void* w, const float* x, int nrows, int k,
+                  int ntok, hipStream_t st) {
+    const TypeInfo* ti = nullptr;
+    int rc = matvec_check(c, type, nrows, k, &ti);
+    if (rc != JL_OK) return rc;
+    if (!out || !w || !x || ntok <= 0) return fail(c, JL_ERR_ARG, "matmul: bad operand");
+    if (!aligned16(x) || (k % 4) != 0) return JL_DECLINED;
+    const bool gemm = type == JL_TYPE_Q4_K && c->act_window == 256 && ntok >= c->gemm_min_tok &&
+                      aligned16(w) && ntok <= 65535 * 4 && kGemmLdsBytes <= c->lds_limit;
+    if (gemm) return gemm_q4k_launch(c, out, w, x, nrows, k, ntok, st);
+    for (int t = 0; t < ntok; t++) {
+        rc = matvec_launch(c, out + (size_t)t * nrows, type, w, x + (size_t)t * k, nullptr, nullptr,
+                           nullptr, nrows, k, st);
+        if (rc != JL_OK) return rc;
+    }
+    return JL_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -258,7 +327,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     if (e != hipSuccess)
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
-    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant"};
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_q4k"};
     const int types[] = {JL_TYPE_Q4_K, JL_TYPE_Q8_0, JL_TYPE_Q6_K};
     for (int t : types)
         for (int rpw : {1, 2, 4}) {
@@ -288,6 +357,7 @@ void jl_ctx_destroy(jl_ctx* c) {
     (void)H->SetDevice(c->device);
     if (c->stream) (void)H->StreamSynchronize(c->stream);
     for (auto& kv : c->resident) (void)H->Free(kv.second.dev);
+    if (c->gemm_ws) (void)H->Free(c->gemm_ws);
     if (c->stage_x) (void)H->Free(c->stage_x);
     if (c->stage_out) (void)H->Free(c->stage_out);
     if (c->module) (void)H->ModuleUnload(c->module);
@@ -319,6 +389,7 @@ int jl_set_tuning(jl_ctx* c, const char* key, int value) {
     if (!strcmp(key, "matvec.rpw")) c->tune.rpw = value;
     else if (!strcmp(key, "matvec.block")) c->tune.block = value;
     else if (!strcmp(key, "matvec.grid")) c->tune.grid = value;
+    else if (!strcmp(key, "gemm.min_tok")) c->gemm_min_tok = value > 0 ? value : 8;
     else return fail(c, JL_ERR_ARG, "unknown tuning key %s", key);
     return JL_OK;
 }
@@ -373,6 +444,20 @@ int jl_matvec_q8_dev(jl_ctx* c, float* out, int type, const void* w, const int8_
     return matvec_launch(c, out, type, w, nullptr, q, as, sum16, nrows, k, pick_stream(c, stream));
 }
 
+int jl_matmul_dev(jl_ctx* c, float* out, int type, const void* w, const float* x, int nrows, int k,
+                  int ntok, void* stream) {
+    if (!c) return JL_ERR_ARG;
+    HIP_TRY(c, H->SetDevice(c->device));
+    return matmul_launch(c, out, type, w, x, nrows, k, ntok, pick_stream(c, stream));
+}
+
+int jl_reserve(jl_ctx* c, int max_tok, int max_k) {
+    if (!c) return JL_ERR_ARG;
+    if (max_tok <= 0 || max_k <= 0 || max_k % 256 != 0) return fail(c, JL_ERR_ARG, "reserve: %d x %d", max_tok, max_k);
+    HIP_TRY(c, H->SetDevice(c->device));
+    return gemm_ws_ensure(c, gemm_ws_need(max_tok, max_k));
+}
+
 /* ------------------------------------------------------- host-pointer seam */
 
 int jl_matvec(jl_ctx* c, float* out, int type, const void* w, size_t wbytes, const float* x,
@@ -399,14 +484,10 @@ int jl_matmul(jl_ctx* c, float* out, int type, const void* w, size_t wbytes, con
     if ((rc = ensure_stage(c, &c->stage_x, &c->stage_x_bytes, xb)) != JL_OK) return rc;
     if ((rc = ensure_stage(c, &c->stage_out, &c->stage_out_bytes, ob)) != JL_OK) return rc;
     HIP_TRY(c, H->MemcpyAsync(c->stage_x, x, xb, hipMemcpyHostToDevice, c->stream));
-    for (int t = 0; t < ntok; t++) {
-        rc = matvec_launch(c, (float*)c->stage_out + (size_t)t * nrows, type, wd,
-                           (const float*)c->stage_x + (size_t)t * k, nullptr, nullptr, nullptr,
-                           nrows, k, c->stream);
-        if (rc != JL_OK) {
-            (void)H->StreamSynchronize(c->stream);
-            return rc;
-        }
+    rc = matmul_launch(c, (float*)c->stage_out, type, wd, (const float*)c->stage_x, nrows, k, ntok, c->stream);
+    if (rc != JL_OK) {
+        (void)H->StreamSynchronize(c->stream);
+        return rc;
     }
     HIP_TRY(c, H->MemcpyAsync(out, c->stage_out, ob, hipMemcpyDeviceToHost, c->stream));
     HIP_TRY(c, H->StreamSynchronize(c->stream));

@@ -15,3 +15,21 @@ struct MatVecArgs {
     int row_bytes;
     int per;             // activation window / 32 (fused form)
 };
+
+// Activation preparation for the Q4_K prefill GEMM: quantize x and lay it out
+// as the GEMM's LDS stages, bq [k/256][2][tok_pad][152] f16, da [k/256][tok_pad].
+struct GemmPrepArgs {
+    const float* x;      // [ntok][k]
+    uint16_t* bq;        // f16 bits
+    float* da;
+    int ntok, tok_pad, k;
+};
+
+struct GemmArgs {
+    float* out;          // [ntok][nrows]
+    const uint8_t* w;    // GGUF row-major Q4_K
+    const uint16_t* bq;
+    const float* da;
+    int nrows, k, ntok, tok_pad;
+    int row_bytes;
+};

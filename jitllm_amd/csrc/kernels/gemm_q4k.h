@@ -1,0 +1,304 @@
+// Prefill GEMM over Q4_K weights: out[t][r] = sum_k W[r][k] * x[t][k], many tokens.
+//
+// Arithmetic (the reference's quantized-activation form with the k-quant window
+// of 256, jit/cpu/matvec.go:46-62, so one activation scale d_a per token and
+// super-block; per (token, row) it is the decode matvec's value,
+// jit/cpu/packedgemm.go:54-58):
+//
+//   out[t][r] = sum_sb d_a[t,sb] * ( d[r,sb]    * P[t,r,sb]  -  dmin[r,sb] * M[t,r,sb] )
+//   P = sum_{s,l} (sc[r,s] * q[r,s,l]) * a[t,s,l]          sub-blocks s, elements l
+//   M = sum_s      m[r,s] * A[t,s],   A[t,s] = sum_l a[t,s,l]
+//
+// P and M are sums of products of small integers, so they run EXACTLY on the
+// f16 matrix cores (v_mfma_f32_32x32x16_f16): sc*q <= 945 and |a| <= 127 are
+// f16 values, products and partial sums are exact in the f32 accumulator.  A is
+// split as 64*A_hi + A_lo so both parts and 64*m are f16 values too.  Scales
+// change every 32 weights, which would force an f32 epilogue per 32-deep MFMA
+// step on the int8 cores; folding the 6-bit sub-block scale into the f16 operand
+// moves the epilogue out to once per 256, where the matrix cores hide it.
+//
+// Layout.  A workgroup owns a 128-token x 128-row tile and walks K in half
+// super-blocks (a "stage": 128 weights, plus the 16 minimum columns in the first
+// half).  Weights are dequantized from HBM straight into an LDS stage as f16
+// (magic-number nibble unpack with packed-f16 FMAs, eight K values per 32-bit
+// word of nibbles); activations were laid out by the prep kernel in exactly the
+// stage's LDS image -- same K permutation, same padding -- so their stage is one
+// contiguous copy, issued as direct global->LDS loads.  Two stages are
+// double-buffered.  Each of the four wavefronts computes 64 tokens x 64 rows as
+// 2x2 MFMA tiles; tokens are the MFMA M dimension so a lane owns one weight row
+// (its scales are scalars) and output stores run along rows.
+#pragma once
+#include "args.h"
+#include "common.h"
+#include "quantize.h"
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+#define JL_GEMM_TILE 128          // tokens and rows per workgroup
+#define JL_GEMM_STRIDE 152        // f16 per LDS row of a stage: 144 used + 8 pad (304 B, odd multiple of 16 B)
+#define JL_GEMM_STAGE_HALFS (JL_GEMM_TILE * JL_GEMM_STRIDE)
+#define JL_GEMM_STAGE_BYTES (JL_GEMM_STAGE_HALFS * 2)
+
+// K position (within a stage's 128 weights) of nibble pair i of 32-bit word c of a
+// 64-element group: word c holds bytes 4c..4c+3; byte b's low nibble is element
+// 4c+b of the group's first sub-block, its high nibble the same element of the
+// second.  The unpack below emits, per word, the eight values
+//   (b0.lo, b2.lo, b0.hi, b2.hi, b1.lo, b3.lo, b1.hi, b3.hi)
+// and the prep kernel writes activations in the same order.
+
+// -------------------------------------------------------------------- prep
+// x [ntok][k] f32 -> bq [nsb][2][tok_pad][152] f16 and da [nsb][tok_pad] f32.
+// One wavefront per (token, super-block); lane l owns elements 4l..4l+3.
+__device__ __forceinline__ void gemm_prep_q4k_body(const GemmPrepArgs& p) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int sb = blockIdx.x;
+    const int t = blockIdx.y * 4 + wave;
+    if (t >= p.tok_pad) return;
+    f32x4 v = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (t < p.ntok) v = ((const f32x4*)(p.x + (size_t)t * p.k + (size_t)sb * 256))[lane];
+    u32 m = max(max(abs_bits(v.x), abs_bits(v.y)), max(abs_bits(v.z), abs_bits(v.w)));
+    u32 amax = window_amax(m, 8);
+    float d;
+    i32 sum16;
+    u32 q = quantize4(v, amax, d, sum16);
+    // sub-block (32 elements = 8 lanes) sum from the two half-block sums
+    i32 a32 = sum16 + dpp_i32<JL_DPP_ROW_HALF_MIRROR, 0xf>(0, sum16);
+    const int g = lane >> 4, hi = (lane >> 3) & 1, c = lane & 7;
+    _Float16* dst = (_Float16*)p.bq + ((size_t)(sb * 2 + (g >> 1)) * p.tok_pad + t) * JL_GEMM_STRIDE;
+    const int base = 8 * (8 * (g & 1) + c) + 2 * hi;
+    f16x2 p02 = {(_Float16)(float)(int8_t)(q & 0xFF), (_Float16)(float)(int8_t)((q >> 16) & 0xFF)};
+    f16x2 p13 = {(_Float16)(float)(int8_t)((q >> 8) & 0xFF), (_Float16)(float)(int8_t)(q >> 24)};
+    *(f16x2*)(dst + base) = p02;
+    *(f16x2*)(dst + base + 4) = p13;
+    if ((lane & 7) == 0) {
+        const int s = lane >> 3;
+        _Float16* aug = (_Float16*)p.bq + ((size_t)(sb * 2) * p.tok_pad + t) * JL_GEMM_STRIDE + 128;
+        aug[s] = (_Float16)(float)(a32 & 63);       // A = 64*A_hi + A_lo, 0 <= A_lo < 64
+        aug[8 + s] = (_Float16)(float)(a32 >> 6);   // arithmetic shift: floor
+    }
+    if (lane == 0) p.da[(size_t)sb * p.tok_pad + t] = d;
+}
+
+// -------------------------------------------------------------------- main
+// One stage of weights for this thread: row = tid/2, hh = tid%2 selects the
+// 64-element group (2*half + hh) of the super-block.
+struct GemmWRegs {
+    u32x4 hdr;
+    u32x4 q[2];
+};
+
+__device__ __forceinline__ void gemm_load_w(const GemmArgs& p, int row, int sb, int g, GemmWRegs& r) {
+    const uint8_t* blk = p.w + (size_t)row * p.row_bytes + (size_t)sb * 144;
+    r.hdr = ld16(blk);
+    r.q[0] = ld16(blk + 16 + 32 * g);
+    r.q[1] = ld16(blk + 32 + 32 * g);
+}
+
+// (1024 + n) as f16 for the nibble in bits 0-3 of each 16-bit half
+__device__ __forceinline__ f16x2 nib_pair(u32 w, int shift) {
+    u32 v = ((w >> shift) & 0x000F000Fu) | 0x64006400u;
+    return __builtin_bit_cast(f16x2, v);
+}
+
+// Dequantize one thread's stage share into LDS: 8 words of nibbles -> 8 K-groups
+// of eight f16 (sc*q); in the first half also the 16 minimum columns and the
+// row's (d, dmin).
+__device__ __forceinline__ void gemm_store_w(const GemmWRegs& r, int row, int hh, int half, _Float16* sw,
+                                             float* sscale) {
+    const int g = 2 * half + hh;
+    u32 sc[8], mn[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) scale_min_k4(j, r.hdr.y, r.hdr.z, r.hdr.w, sc[j], mn[j]);
+    // scales of sub-blocks 2g (low nibbles) and 2g+1 (high nibbles); g is not a
+    // compile-time constant, so select
+    u32 slo = sc[0], shi = sc[1];
+#pragma unroll
+    for (int j = 1; j < 4; j++) {
+        slo = g == j ? sc[2 * j] : slo;
+        shi = g == j ? sc[2 * j + 1] : shi;
+    }
+    const _Float16 flo = (_Float16)(float)slo, fhi = (_Float16)(float)shi;
+    const f16x2 mlo = {flo, flo}, mhi = {fhi, fhi};
+    const _Float16 nlo = (_Float16)(-1024.0f * (float)slo), nhi = (_Float16)(-1024.0f * (float)shi);
+    const f16x2 alo = {nlo, nlo}, ahi = {nhi, nhi};
+    _Float16* dst = sw + row * JL_GEMM_STRIDE + 64 * hh;
+#pragma unroll
+    for (int c = 0; c < 8; c++) {
+        const u32 w = c < 4 ? r.q[0][c] : r.q[1][c - 4];
+        // (1024+n)*sc - 1024*sc = sc*n, exact in f16 (<= 945) through the fused multiply-add
+        f16x2 p0 = __builtin_elementwise_fma(nib_pair(w, 0), mlo, alo);
+        f16x2 p1 = __builtin_elementwise_fma(nib_pair(w, 4), mhi, ahi);
+        f16x2 p2 = __builtin_elementwise_fma(nib_pair(w, 8), mlo, alo);
+        f16x2 p3 = __builtin_elementwise_fma(nib_pair(w, 12), mhi, ahi);
+        u32x4 o = {__builtin_bit_cast(u32, p0), __builtin_bit_cast(u32, p1), __builtin_bit_cast(u32, p2),
+                   __builtin_bit_cast(u32, p3)};
+        *(u32x4*)(dst + 8 * c) = o;
+    }
+    if (half == 0) {
+        // minimum columns: hh = 0 writes m_s (pairs with A_lo), hh = 1 writes 64*m_s (pairs with A_hi)
+        const float mul = hh ? 64.0f : 1.0f;
+        f16x8 mm;
+#pragma unroll
+        for (int j = 0; j < 8; j++) mm[j] = (_Float16)((float)mn[j] * mul);
+        *(f16x8*)(sw + row * JL_GEMM_STRIDE + 128 + 8 * hh) = mm;
+        if (hh == 0) {
+            sscale[2 * row] = half_bits_to_f32((uint16_t)(r.hdr.x & 0xFFFF));
+            sscale[2 * row + 1] = half_bits_to_f32((uint16_t)(r.hdr.x >> 16));
+        }
+    }
+}
+
+// Copy one activation stage (128 tokens x 304 B, contiguous in HBM) into LDS with
+// direct global->LDS loads: each wavefront instruction moves 64 lanes x 16 B to
+// 1 KiB of consecutive LDS.
+__device__ __forceinline__ void gemm_load_a_stage(const _Float16* src, _Float16* dst) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int nchunks = JL_GEMM_STAGE_BYTES / 1024;  // 38 wavefront-sized pieces
+    for (int c = wave; c < nchunks; c += 4) {
+        const uint8_t* g = (const uint8_t*)src + (size_t)c * 1024 + lane * 16;
+        uint8_t* l = (uint8_t*)dst + c * 1024;
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g,
+                                         (__attribute__((address_space(3))) void*)l, 16, 0, 0);
+    }
+}
+
+__device__ __forceinline__ void gemm_q4k_body(const GemmArgs& p, uint8_t* smem) {
+    // LDS: activation stages [2], weight stages [2], row scales [2][128][2], token scales [2][128]
+    _Float16* sA = (_Float16*)smem;
+    _Float16* sW = sA + 2 * JL_GEMM_STAGE_HALFS;
+    float* sScale = (float*)(sW + 2 * JL_GEMM_STAGE_HALFS);
+    float* sDa = sScale + 2 * 2 * JL_GEMM_TILE;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int t0 = blockIdx.x * JL_GEMM_TILE, r0 = blockIdx.y * JL_GEMM_TILE;
+    const int nsb = p.k / 256, nsteps = 2 * nsb;
+    const int wrow = min(r0 + (tid >> 1), p.nrows - 1), hh = tid & 1;
+    const int wt = (wave >> 1) * 64, wr = (wave & 1) * 64;  // this wavefront's 64x64 corner
+
+    auto a_src = [&](int step) {
+        return (const _Float16*)p.bq + ((size_t)step * p.tok_pad + t0) * JL_GEMM_STRIDE;
+    };
+
+    f32x16 out[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) out[i][j][e] = 0.f;
+
+    // prologue: stage 0 into buffer 0, stage 1's weights into registers
+    GemmWRegs wreg;
+    gemm_load_w(p, wrow, 0, hh, wreg);
+    gemm_load_a_stage(a_src(0), sA);
+    if (tid < JL_GEMM_TILE) sDa[tid] = p.da[(size_t)0 * p.tok_pad + t0 + tid];
+    gemm_store_w(wreg, tid >> 1, hh, 0, sW, sScale);
+    if (nsteps > 1) gemm_load_w(p, wrow, 0, 2 + hh, wreg);
+    // direct-to-LDS loads are tracked by the memory-load counter
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+
+    f32x16 accP[2][2];
+    for (int step = 0; step < nsteps; step++) {
+        const int buf = step & 1, half = step & 1, sb = step >> 1;
+        const _Float16* a = sA + buf * JL_GEMM_STAGE_HALFS;
+        const _Float16* w = sW + buf * JL_GEMM_STAGE_HALFS;
+        // (a) next stage: activations by direct load, weights from registers
+        if (step + 1 < nsteps) {
+            const int nb = buf ^ 1, nhalf = (step + 1) & 1, nsbi = (step + 1) >> 1;
+            gemm_load_a_stage(a_src(step + 1), sA + nb * JL_GEMM_STAGE_HALFS);
+            if (nhalf == 0 && tid < JL_GEMM_TILE)
+                sDa[(nsbi & 1) * JL_GEMM_TILE + tid] = p.da[(size_t)nsbi * p.tok_pad + t0 + tid];
+            gemm_store_w(wreg, tid >> 1, hh, nhalf, sW + nb * JL_GEMM_STAGE_HALFS,
+                         sScale + (nsbi & 1) * 2 * JL_GEMM_TILE);
+            // (b) the stage after that, into registers
+            if (step + 2 < nsteps) gemm_load_w(p, wrow, (step + 2) >> 1, 2 * ((step + 2) & 1) + hh, wreg);
+        }
+        // (c) matrix work on the current stage
+        const int arow = lane & 31, kg = lane >> 5;
+        if (half == 0) {
+            // the 16 minimum columns first: M, folded into the output at once
+            f32x16 accM[2][2];
+            f16x8 af[2], wf[2];
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                af[i] = *(const f16x8*)(a + (wt + 32 * i + arow) * JL_GEMM_STRIDE + 128 + 8 * kg);
+                wf[i] = *(const f16x8*)(w + (wr + 32 * i + arow) * JL_GEMM_STRIDE + 128 + 8 * kg);
+            }
+            const f32x16 zero = {0};
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+                    accM[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], wf[j], zero, 0, 0, 0);
+            const float* ssc = sScale + (sb & 1) * 2 * JL_GEMM_TILE;
+            const float* sda = sDa + (sb & 1) * JL_GEMM_TILE;
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                const float dmin = ssc[2 * (wr + 32 * j + arow) + 1];
+#pragma unroll
+                for (int i = 0; i < 2; i++)
+#pragma unroll
+                    for (int e = 0; e < 16; e++) {
+                        const int tk = wt + 32 * i + 8 * (e >> 2) + 4 * kg + (e & 3);
+                        out[i][j][e] -= sda[tk] * (dmin * accM[i][j][e]);
+                    }
+            }
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+#pragma unroll
+                    for (int e = 0; e < 16; e++) accP[i][j][e] = 0.f;
+        }
+#pragma unroll
+        for (int ks = 0; ks < 8; ks++) {
+            f16x8 af[2], wf[2];
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                af[i] = *(const f16x8*)(a + (wt + 32 * i + arow) * JL_GEMM_STRIDE + 16 * ks + 8 * kg);
+                wf[i] = *(const f16x8*)(w + (wr + 32 * i + arow) * JL_GEMM_STRIDE + 16 * ks + 8 * kg);
+            }
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+                    accP[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], wf[j], accP[i][j], 0, 0, 0);
+        }
+        if (half == 1) {
+            const float* ssc = sScale + (sb & 1) * 2 * JL_GEMM_TILE;
+            const float* sda = sDa + (sb & 1) * JL_GEMM_TILE;
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                const float dd = ssc[2 * (wr + 32 * j + arow)];
+#pragma unroll
+                for (int i = 0; i < 2; i++)
+#pragma unroll
+                    for (int e = 0; e < 16; e++) {
+                        const int tk = wt + 32 * i + 8 * (e >> 2) + 4 * kg + (e & 3);
+                        out[i][j][e] += sda[tk] * (dd * accP[i][j][e]);
+                    }
+            }
+        }
+        // (d) the next stage's direct loads must have landed before anyone reads it
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+    }
+
+    // store: lane = row (contiguous in memory), register = token
+    const int arow = lane & 31, kg = lane >> 5;
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        const int r = r0 + wr + 32 * j + arow;
+        if (r >= p.nrows) continue;
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
+                const int t = t0 + wt + 32 * i + 8 * (e >> 2) + 4 * kg + (e & 3);
+                if (t < p.ntok) p.out[(size_t)t * p.nrows + r] = out[i][j][e];
+            }
+    }
+}

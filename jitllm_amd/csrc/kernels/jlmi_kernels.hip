@@ -4,6 +4,7 @@
 // Entry points are extern "C" so the host can look them up by name.
 #include "common.h"
 #include "dequant.h"
+#include "gemm_q4k.h"
 #include "matvec.h"
 #include "quantize.h"
 
@@ -48,3 +49,9 @@ extern "C" __global__ __launch_bounds__(256) void jl_dequant(
 JL_MATVEC_KERNEL(q4k, JL_Q4_K, 1, 1024) JL_MATVEC_KERNEL(q4k, JL_Q4_K, 2, 1024) JL_MATVEC_KERNEL(q4k, JL_Q4_K, 4, 512)
 JL_MATVEC_KERNEL(q8_0, JL_Q8_0, 1, 1024) JL_MATVEC_KERNEL(q8_0, JL_Q8_0, 2, 1024) JL_MATVEC_KERNEL(q8_0, JL_Q8_0, 4, 1024)
 JL_MATVEC_KERNEL(q6k, JL_Q6_K, 1, 1024) JL_MATVEC_KERNEL(q6k, JL_Q6_K, 2, 512) JL_MATVEC_KERNEL(q6k, JL_Q6_K, 4, 512)
+
+// ------------------------------------------------------------ prefill GEMM
+// grid = (k/256, tok_pad/4), block = 256: one wavefront per (token, super-block)
+extern "C" __global__ __launch_bounds__(256) void jl_gemm_prep_q4k(GemmPrepArgs p) { gemm_prep_q4k_body(p); }
+// grid = (tok_pad/128, ceil(nrows/128)), block = 256, dynamic LDS = JL_GEMM_LDS_BYTES
+extern "C" __global__ __launch_bounds__(256) void jl_gemm_q4k(GemmArgs p) { gemm_q4k_body(p, jl_smem); }

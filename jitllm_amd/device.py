@@ -63,9 +63,13 @@ class Device:
         """nn.ActWindower.SetActWindow (/root/reference/engine/nn/device.go:1566-1568)."""
         self._served(self._l.jl_set_act_window(self._ctx, n), "jl_set_act_window")
 
+    def Reserve(self, max_tok, max_k):
+        """nn.LayerDevice.Reserve: size the prefill workspace ahead of time."""
+        self._served(self._l.jl_reserve(self._ctx, max_tok, max_k), "jl_reserve")
+
     def set_tuning(self, **kw):
         for k, v in kw.items():
-            key = ("matvec." + k).encode()
+            key = (k.replace("__", ".") if "__" in k else "matvec." + k).encode()
             self._served(self._l.jl_set_tuning(self._ctx, key, int(v)), "jl_set_tuning")
 
     @property
@@ -116,3 +120,8 @@ class Device:
         return self._served(self._l.jl_matvec_q8_dev(self._ctx, _ptr(out), t, _ptr(w), _ptr(q),
                                                      _ptr(a_s), _ptr(sum16), nrows, k, stream),
                             "jl_matvec_q8_dev")
+
+    def matmul_dev(self, out, t, w, x, nrows, k, ntok, stream=None):
+        """x [ntok][k] -> out [ntok][nrows] on device operands (JIT.MatMulPacked semantics)."""
+        return self._served(self._l.jl_matmul_dev(self._ctx, _ptr(out), t, _ptr(w), _ptr(x),
+                                                  nrows, k, ntok, stream), "jl_matmul_dev")
