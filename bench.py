@@ -127,6 +127,44 @@ def cpu_baseline(t, nrows, k, window, seed=0):
     }
 
 
+MFMA_F16_PEAK_TFLOPS = 2500.0
+
+
+def gemm_section(dev):
+    """Q4_K prefill GEMM (x [ntok][4096] f32 -> out [ntok][nrows]), activation quantizer and
+    layout kernel included in every step; flops = 2*nrows*k*ntok, priced against the dense
+    f16 MFMA peak (the kernel runs exact integer operands on the f16 matrix cores)."""
+    from jitllm_amd import quant, synth
+    from jitllm_amd.hipmem import DeviceArray, Event
+    t, k = quant.Q4_K, 4096
+    dev.SetActWindow(256)
+    out = {}
+    for nrows in (4096, 14336):
+        w = DeviceArray(synth.quantized_weights(t, nrows, k, seed=0))
+        for ntok in (16, 128, 512, 2048):
+            x = DeviceArray(np.random.default_rng(2).standard_normal((ntok, k), np.float32))
+            o = DeviceArray(shape=(ntok, nrows), dtype=np.float32)
+            dev.Reserve(ntok, k)
+            for _ in range(3):
+                if not dev.matmul_dev(o.ptr, t, w.ptr, x.ptr, nrows, k, ntok):
+                    raise RuntimeError("the device declined the prefill GEMM")
+            dev.synchronize()
+            e0, e1, n = Event(), Event(), 20
+            e0.record(dev.stream)
+            for _ in range(n):
+                dev.matmul_dev(o.ptr, t, w.ptr, x.ptr, nrows, k, ntok)
+            e1.record(dev.stream)
+            e1.synchronize()
+            ms = e0.elapsed_ms(e1) / n
+            tf = 2.0 * nrows * k * ntok / (ms * 1e-3) / 1e12
+            out[f"{ntok}x{k}->{nrows}"] = {"us_per_step": round(ms * 1e3, 1), "TFLOP/s": round(tf, 1),
+                                          "frac_of_f16_mfma_peak": round(tf / MFMA_F16_PEAK_TFLOPS, 4)}
+            x.free()
+            o.free()
+        w.free()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -175,6 +213,9 @@ def main():
                           "frac_of_hbm_peak": round(g / HBM_PEAK_GBS, 4), "bytes_per_step": wl.alg_bytes}
             wl.free()
         line["other_configs"] = extra
+
+    if not args.no_extra:
+        line["prefill_gemm"] = gemm_section(dev)
 
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(quant.Q4_K, 4096, 4096, 256)

@@ -264,7 +264,7 @@ int gemm_q4k_launch(jl_ctx* c, float* out, const void* w, const float* x, int nr
     ga.nrows = nrows; ga.k = k; ga.ntok = ntok; ga.tok_pad = tok_pad; ga.row_bytes = nsb * 144;
     void* gp[] = {&ga};
     return launch(c, "jl_gemm_q4k", (unsigned)(tok_pad / kGemmTile),
-                  (unsigned)((nrows + kGemmTile - 1) / kGemmTile), 256, kGemmLdsBytes, st, gp);
+                  (unsigned)((nrows + kGemmTile - 1) / kGemmTile), 512, kGemmLdsBytes, st, gp);
 }
 
 // out [ntok][nrows] = x [ntok][k] W^T on device operands: the matrix-core GEMM where it

@@ -24,13 +24,18 @@
 // word of nibbles); activations were laid out by the prep kernel in exactly the
 // stage's LDS image -- same K permutation, same padding -- so their stage is one
 // contiguous copy, issued as direct global->LDS loads.  Two stages are
-// double-buffered.  Each of the four wavefronts computes 64 tokens x 64 rows as
-// 2x2 MFMA tiles; tokens are the MFMA M dimension so a lane owns one weight row
+// double-buffered.  Four consumer wavefronts each compute 64 tokens x 64 rows as
+// 2x2 MFMA tiles while four producer wavefronts fill the next stage; tokens are the MFMA M dimension so a lane owns one weight row
 // (its scales are scalars) and output stores run along rows.
 #pragma once
 #include "args.h"
 #include "common.h"
 #include "quantize.h"
+
+// Phase marker for profiling builds; expands to nothing in the product.
+#ifndef JL_TRACE
+#define JL_TRACE(i)
+#endif
 
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
@@ -40,6 +45,15 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 #define JL_GEMM_STRIDE 152        // f16 per LDS row of a stage: 144 used + 8 pad (304 B, odd multiple of 16 B)
 #define JL_GEMM_STAGE_HALFS (JL_GEMM_TILE * JL_GEMM_STRIDE)
 #define JL_GEMM_STAGE_BYTES (JL_GEMM_STAGE_HALFS * 2)
+
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() carries a
+// release fence that also drains every outstanding global load, which would
+// throw away the register prefetch that is meant to stay in flight across it.
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
 
 // K position (within a stage's 128 weights) of nibble pair i of 32-bit word c of a
 // 64-element group: word c holds bytes 4c..4c+3; byte b's low nibble is element
@@ -74,7 +88,7 @@ __device__ __forceinline__ void gemm_prep_q4k_body(const GemmPrepArgs& p) {
     *(f16x2*)(dst + base + 4) = p13;
     if ((lane & 7) == 0) {
         const int s = lane >> 3;
-        _Float16* aug = (_Float16*)p.bq + ((size_t)(sb * 2) * p.tok_pad + t) * JL_GEMM_STRIDE + 128;
+        _Float16* aug = (_Float16*)p.bq + ((size_t)(sb * 2 + 1) * p.tok_pad + t) * JL_GEMM_STRIDE + 128;
         aug[s] = (_Float16)(float)(a32 & 63);       // A = 64*A_hi + A_lo, 0 <= A_lo < 64
         aug[8 + s] = (_Float16)(float)(a32 >> 6);   // arithmetic shift: floor
     }
@@ -136,7 +150,7 @@ __device__ __forceinline__ void gemm_store_w(const GemmWRegs& r, int row, int hh
                    __builtin_bit_cast(u32, p3)};
         *(u32x4*)(dst + 8 * c) = o;
     }
-    if (half == 0) {
+    if (half == 1) {
         // minimum columns: hh = 0 writes m_s (pairs with A_lo), hh = 1 writes 64*m_s (pairs with A_hi)
         const float mul = hh ? 64.0f : 1.0f;
         f16x8 mm;
@@ -156,7 +170,7 @@ __device__ __forceinline__ void gemm_store_w(const GemmWRegs& r, int row, int hh
 __device__ __forceinline__ void gemm_load_a_stage(const _Float16* src, _Float16* dst) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int nchunks = JL_GEMM_STAGE_BYTES / 1024;  // 38 wavefront-sized pieces
-    for (int c = wave; c < nchunks; c += 4) {
+    for (int c = wave & 3; c < nchunks; c += 4) {
         const uint8_t* g = (const uint8_t*)src + (size_t)c * 1024 + lane * 16;
         uint8_t* l = (uint8_t*)dst + c * 1024;
         __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g,
@@ -171,11 +185,17 @@ __device__ __forceinline__ void gemm_q4k_body(const GemmArgs& p, uint8_t* smem) 
     float* sScale = (float*)(sW + 2 * JL_GEMM_STAGE_HALFS);
     float* sDa = sScale + 2 * 2 * JL_GEMM_TILE;
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    // Eight wavefronts, two per SIMD: wavefronts 0-3 are consumers (LDS -> matrix cores
+    // -> epilogue, one 64x64 corner each), wavefronts 4-7 are producers (HBM -> dequantize
+    // -> LDS, and the direct activation loads).  A SIMD then always has vector work
+    // from its producer to issue under its consumer's matrix instructions.
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const bool producer = wave >= 4;
+    const int tid = threadIdx.x & 255;  // index within the role
     const int t0 = blockIdx.x * JL_GEMM_TILE, r0 = blockIdx.y * JL_GEMM_TILE;
     const int nsb = p.k / 256, nsteps = 2 * nsb;
     const int wrow = min(r0 + (tid >> 1), p.nrows - 1), hh = tid & 1;
-    const int wt = (wave >> 1) * 64, wr = (wave & 1) * 64;  // this wavefront's 64x64 corner
+    const int wt = ((wave >> 1) & 1) * 64, wr = (wave & 1) * 64;  // a consumer's 64x64 corner
 
     auto a_src = [&](int step) {
         return (const _Float16*)p.bq + ((size_t)step * p.tok_pad + t0) * JL_GEMM_STRIDE;
@@ -189,63 +209,47 @@ __device__ __forceinline__ void gemm_q4k_body(const GemmArgs& p, uint8_t* smem) 
 #pragma unroll
             for (int e = 0; e < 16; e++) out[i][j][e] = 0.f;
 
-    // prologue: stage 0 into buffer 0, stage 1's weights into registers
+    // prologue (producers): stage 0 into buffer 0; stage 1's weights and token scales
+    // into registers
     GemmWRegs wreg;
-    gemm_load_w(p, wrow, 0, hh, wreg);
-    gemm_load_a_stage(a_src(0), sA);
-    if (tid < JL_GEMM_TILE) sDa[tid] = p.da[(size_t)0 * p.tok_pad + t0 + tid];
-    gemm_store_w(wreg, tid >> 1, hh, 0, sW, sScale);
-    if (nsteps > 1) gemm_load_w(p, wrow, 0, 2 + hh, wreg);
-    // direct-to-LDS loads are tracked by the memory-load counter
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
+    float da_reg = 0.f;
+    if (producer) {
+        gemm_load_w(p, wrow, 0, hh, wreg);
+        gemm_store_w(wreg, tid >> 1, hh, 0, sW, sScale);
+        gemm_load_a_stage(a_src(0), sA);
+        gemm_load_w(p, wrow, 0, 2 + hh, wreg);
+        da_reg = p.da[t0 + (tid & (JL_GEMM_TILE - 1))];
+        asm volatile("s_waitcnt vmcnt(4)" ::: "memory");  // the direct loads; 3 weight + 1 scale load stay in flight
+    }
+    lds_barrier();
 
     f32x16 accP[2][2];
     for (int step = 0; step < nsteps; step++) {
         const int buf = step & 1, half = step & 1, sb = step >> 1;
         const _Float16* a = sA + buf * JL_GEMM_STAGE_HALFS;
         const _Float16* w = sW + buf * JL_GEMM_STAGE_HALFS;
-        // (a) next stage: activations by direct load, weights from registers
-        if (step + 1 < nsteps) {
+        JL_TRACE(0);
+        if (producer && step + 1 < nsteps) {
             const int nb = buf ^ 1, nhalf = (step + 1) & 1, nsbi = (step + 1) >> 1;
-            gemm_load_a_stage(a_src(step + 1), sA + nb * JL_GEMM_STAGE_HALFS);
-            if (nhalf == 0 && tid < JL_GEMM_TILE)
-                sDa[(nsbi & 1) * JL_GEMM_TILE + tid] = p.da[(size_t)nsbi * p.tok_pad + t0 + tid];
+            // (a) the next stage's weights: registers (loaded a step ago) -> LDS.  Nothing
+            // newer has been issued yet, so this waits for exactly those loads.  A second
+            // half also carries the super-block's row scales and token scales.
             gemm_store_w(wreg, tid >> 1, hh, nhalf, sW + nb * JL_GEMM_STAGE_HALFS,
                          sScale + (nsbi & 1) * 2 * JL_GEMM_TILE);
-            // (b) the stage after that, into registers
-            if (step + 2 < nsteps) gemm_load_w(p, wrow, (step + 2) >> 1, 2 * ((step + 2) & 1) + hh, wreg);
+            if (nhalf == 1 && tid < JL_GEMM_TILE) sDa[(nsbi & 1) * JL_GEMM_TILE + tid] = da_reg;
+            JL_TRACE(1);
+            // (b) issue, in this order: the next stage's activations (direct to LDS), then
+            // the weights and token scales of the stage after it (to registers)
+            gemm_load_a_stage(a_src(step + 1), sA + nb * JL_GEMM_STAGE_HALFS);
+            const int s2 = min(step + 2, nsteps - 1);
+            gemm_load_w(p, wrow, s2 >> 1, 2 * (s2 & 1) + hh, wreg);
+            da_reg = p.da[(size_t)(s2 >> 1) * p.tok_pad + t0 + (tid & (JL_GEMM_TILE - 1))];
         }
+        JL_TRACE(2);
         // (c) matrix work on the current stage
         const int arow = lane & 31, kg = lane >> 5;
+        if (!producer) {
         if (half == 0) {
-            // the 16 minimum columns first: M, folded into the output at once
-            f32x16 accM[2][2];
-            f16x8 af[2], wf[2];
-#pragma unroll
-            for (int i = 0; i < 2; i++) {
-                af[i] = *(const f16x8*)(a + (wt + 32 * i + arow) * JL_GEMM_STRIDE + 128 + 8 * kg);
-                wf[i] = *(const f16x8*)(w + (wr + 32 * i + arow) * JL_GEMM_STRIDE + 128 + 8 * kg);
-            }
-            const f32x16 zero = {0};
-#pragma unroll
-            for (int i = 0; i < 2; i++)
-#pragma unroll
-                for (int j = 0; j < 2; j++)
-                    accM[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], wf[j], zero, 0, 0, 0);
-            const float* ssc = sScale + (sb & 1) * 2 * JL_GEMM_TILE;
-            const float* sda = sDa + (sb & 1) * JL_GEMM_TILE;
-#pragma unroll
-            for (int j = 0; j < 2; j++) {
-                const float dmin = ssc[2 * (wr + 32 * j + arow) + 1];
-#pragma unroll
-                for (int i = 0; i < 2; i++)
-#pragma unroll
-                    for (int e = 0; e < 16; e++) {
-                        const int tk = wt + 32 * i + 8 * (e >> 2) + 4 * kg + (e & 3);
-                        out[i][j][e] -= sda[tk] * (dmin * accM[i][j][e]);
-                    }
-            }
 #pragma unroll
             for (int i = 0; i < 2; i++)
 #pragma unroll
@@ -253,41 +257,69 @@ __device__ __forceinline__ void gemm_q4k_body(const GemmArgs& p, uint8_t* smem) 
 #pragma unroll
                     for (int e = 0; e < 16; e++) accP[i][j][e] = 0.f;
         }
+        // Fragments are fetched one K-step ahead of the matrix instructions that use
+        // them; the last prefetch of a second half fetches the minimum columns.
+        const _Float16* ap0 = a + (wt + arow) * JL_GEMM_STRIDE + 8 * kg;
+        const _Float16* wp0 = w + (wr + arow) * JL_GEMM_STRIDE + 8 * kg;
+        f16x8 af[2][2], wf[2][2];
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            af[0][i] = *(const f16x8*)(ap0 + 32 * i * JL_GEMM_STRIDE);
+            wf[0][i] = *(const f16x8*)(wp0 + 32 * i * JL_GEMM_STRIDE);
+        }
 #pragma unroll
         for (int ks = 0; ks < 8; ks++) {
-            f16x8 af[2], wf[2];
+            const int cur = ks & 1, nxt = cur ^ 1;
+            if (ks < 7 || half == 1) {
 #pragma unroll
-            for (int i = 0; i < 2; i++) {
-                af[i] = *(const f16x8*)(a + (wt + 32 * i + arow) * JL_GEMM_STRIDE + 16 * ks + 8 * kg);
-                wf[i] = *(const f16x8*)(w + (wr + 32 * i + arow) * JL_GEMM_STRIDE + 16 * ks + 8 * kg);
+                for (int i = 0; i < 2; i++) {
+                    af[nxt][i] = *(const f16x8*)(ap0 + 32 * i * JL_GEMM_STRIDE + 16 * (ks + 1));
+                    wf[nxt][i] = *(const f16x8*)(wp0 + 32 * i * JL_GEMM_STRIDE + 16 * (ks + 1));
+                }
             }
 #pragma unroll
             for (int i = 0; i < 2; i++)
 #pragma unroll
                 for (int j = 0; j < 2; j++)
-                    accP[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], wf[j], accP[i][j], 0, 0, 0);
+                    accP[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[cur][i], wf[cur][j], accP[i][j], 0, 0, 0);
         }
+        JL_TRACE(3);
         if (half == 1) {
+            // the 16 minimum columns: M, then the super-block's epilogue
+            //   out += d_a * (d * P - dmin * M)
+            const f32x16 zero = {0};
             const float* ssc = sScale + (sb & 1) * 2 * JL_GEMM_TILE;
             const float* sda = sDa + (sb & 1) * JL_GEMM_TILE;
 #pragma unroll
             for (int j = 0; j < 2; j++) {
                 const float dd = ssc[2 * (wr + 32 * j + arow)];
+                const float dmin = ssc[2 * (wr + 32 * j + arow) + 1];
+                f32x16 accM[2];
+                accM[0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[0][0], wf[0][j], zero, 0, 0, 0);
+                accM[1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[0][1], wf[0][j], zero, 0, 0, 0);
 #pragma unroll
-                for (int i = 0; i < 2; i++)
+                for (int i = 0; i < 2; i++) {
 #pragma unroll
                     for (int e = 0; e < 16; e++) {
                         const int tk = wt + 32 * i + 8 * (e >> 2) + 4 * kg + (e & 3);
-                        out[i][j][e] += sda[tk] * (dd * accP[i][j][e]);
+                        const float u = fmaf(dd, accP[i][j][e], -(dmin * accM[i][e]));
+                        out[i][j][e] = fmaf(sda[tk], u, out[i][j][e]);
                     }
+                }
             }
         }
-        // (d) the next stage's direct loads must have landed before anyone reads it
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
+        }  // consumer
+        JL_TRACE(4);
+        // (d) the next stage's direct loads must have landed before anyone reads it.
+        // Loads return in order; the four register loads of (b) were issued after them
+        // and stay in flight across the barrier.
+        if (producer) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+        lds_barrier();
+        JL_TRACE(5);
     }
 
     // store: lane = row (contiguous in memory), register = token
+    if (producer) return;
     const int arow = lane & 31, kg = lane >> 5;
 #pragma unroll
     for (int j = 0; j < 2; j++) {

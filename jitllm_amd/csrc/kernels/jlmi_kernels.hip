@@ -53,5 +53,5 @@ JL_MATVEC_KERNEL(q6k, JL_Q6_K, 1, 1024) JL_MATVEC_KERNEL(q6k, JL_Q6_K, 2, 512) J
 // ------------------------------------------------------------ prefill GEMM
 // grid = (k/256, tok_pad/4), block = 256: one wavefront per (token, super-block)
 extern "C" __global__ __launch_bounds__(256) void jl_gemm_prep_q4k(GemmPrepArgs p) { gemm_prep_q4k_body(p); }
-// grid = (tok_pad/128, ceil(nrows/128)), block = 256, dynamic LDS = JL_GEMM_LDS_BYTES
-extern "C" __global__ __launch_bounds__(256) void jl_gemm_q4k(GemmArgs p) { gemm_q4k_body(p, jl_smem); }
+// grid = (tok_pad/128, ceil(nrows/128)), block = 512 (4 consumer + 4 producer wavefronts)
+extern "C" __global__ __launch_bounds__(512) void jl_gemm_q4k(GemmArgs p) { gemm_q4k_body(p, jl_smem); }
