@@ -145,6 +145,45 @@ int jl_matmul_dev(jl_ctx *ctx, float *out, int type, const void *w, const float 
  * calls allocate nothing. */
 int jl_reserve(jl_ctx *ctx, int max_tok, int max_k);
 
+/* ---- mixture of experts (device pointers) ----------------------------- */
+
+/* The grouping the device tier runs before a batched mixture (kernels.ExpertGroup*,
+ * jit/gpu/kernels/moesort.go:12-31; specification groupPairs,
+ * jit/gpu/tier/grouppairs_test.go:91-122, with unit 1): sel [rows][sel_stride] holds
+ * each row's k_used expert ids first.  Fills start [n_expert+1] (first column of each
+ * expert's run), perm [rows*k_used] (column -> row) and pos [rows*k_used]
+ * (pair r*k_used+s -> column); experts ascending, pairs in (row, slot) order. */
+int jl_moe_group_dev(jl_ctx *ctx, const uint32_t *sel, int sel_stride, int rows, int k_used,
+                     int n_expert, uint32_t *start, uint32_t *perm, uint32_t *pos, void *stream);
+
+/* MUL_MAT_ID over sorted columns (the Experts/Slots/SlotAct forms of kernels.MatVec,
+ * jit/gpu/kernels/matvec.go:330-343, :788-836; host forms MatVecPackedMulti / GatherAct,
+ * engine/nn/packedmulti.go:24,93): for every column c of expert e,
+ *   out0[c][0:nrows] = bank0 sheet e . act(c)   (and out1 / bank1 when given),
+ * act(c) = x[src[c]] (src NULL: x[c]) or silu(x[..]) * x2[..] when x2 is given.  A bank
+ * is n_expert sheets of nrows x k GGUF rows back to back.  Activations are
+ * quantized per column exactly as jl_matvec_dev does. */
+int jl_moe_matvec_dev(jl_ctx *ctx, float *out0, float *out1, int type, const void *bank0,
+                      const void *bank1, const float *x, const float *x2, const uint32_t *src,
+                      const uint32_t *start, int n_expert, int nrows, int k, void *stream);
+
+/* kernels.ExpertCombineGrouped (jit/gpu/kernels/moegroup.go:38-68) with the host path's
+ * order (engine/model/moe.go:127-134, :752-759): resid[r] += sum of wt[r][s] *
+ * y[pos[r*k_used+s]] over the row's experts in ascending expert id. */
+int jl_moe_combine_dev(jl_ctx *ctx, float *resid, const float *y, const float *wt,
+                       const uint32_t *sel, int sel_stride, const uint32_t *pos, int rows,
+                       int k_used, int n_embd, void *stream);
+
+/* One routed feed-forward block, moeBatchFrom / moeBatchExpert
+ * (engine/model/moe.go:510-761): group, gate and up in one launch, act(gate)*up fused
+ * into the down launch's quantizer, combine into resid [rows][n_embd] (accumulated).
+ * gate/up banks: n_expert sheets of n_ffn x n_embd; down bank: n_embd x n_ffn.
+ * Intermediates live in a workspace the context owns (grown on demand). */
+int jl_moe_ffn_dev(jl_ctx *ctx, float *resid, int type, const void *gate_bank,
+                   const void *up_bank, const void *down_bank, const float *x,
+                   const uint32_t *sel, int sel_stride, const float *wt, int rows, int k_used,
+                   int n_expert, int n_ffn, int n_embd, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

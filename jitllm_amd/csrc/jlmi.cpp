@@ -54,6 +54,10 @@ struct jl_ctx {
     void* gemm_ws = nullptr;
     size_t gemm_ws_bytes = 0;
 
+    // mixture-of-experts workspace (grouping tables and intermediate columns)
+    void* moe_ws = nullptr;
+    size_t moe_ws_bytes = 0;
+
     // host-pointer seam state
     std::map<const void*, Resident> resident;
     void* stage_x = nullptr;    // device
@@ -287,6 +291,57 @@ int matmul_launch(jl_ctx* c, float* out, int type, const void* w, const float* x
     return JL_OK;
 }
 
+int ws_ensure(jl_ctx* c, void** buf, size_t* have, size_t need) {
+    if (*have >= need) return JL_OK;
+    HIP_TRY(c, H->StreamSynchronize(c->stream));  // work in flight may still read the old one
+    if (*buf) HIP_TRY(c, H->Free(*buf));
+    *buf = nullptr;
+    *have = 0;
+    HIP_TRY(c, H->Malloc(buf, need));
+    *have = need;
+    return JL_OK;
+}
+
+int moe_matvec_launch(jl_ctx* c, float* out0, float* out1, int type, const void* bank0, const void* bank1,
+                      const float* x, const float* x2, const uint32_t* src, const uint32_t* start,
+                      int n_expert, int nrows, int k, hipStream_t st) {
+    const TypeInfo* ti = nullptr;
+    int rc = matvec_check(c, type, nrows, k, &ti);
+    if (rc != JL_OK) return rc;
+    if (!out0 || !bank0 || !x || !start || n_expert <= 0) return fail(c, JL_ERR_ARG, "moe matvec: bad operand");
+    if ((bank1 == nullptr) != (out1 == nullptr)) return fail(c, JL_ERR_ARG, "moe matvec: second matrix needs both bank and out");
+    if (!aligned16(x) || (x2 && !aligned16(x2)) || k % 256 != 0 || n_expert > 65535) return JL_DECLINED;
+    if (!aligned16(bank0) || (bank1 && !aligned16(bank1))) return JL_DECLINED;
+    const int row_bytes = (k / ti->block_elems) * ti->block_bytes;
+    const size_t sheet = (size_t)nrows * row_bytes;
+    if (type == JL_TYPE_Q4_K ? sheet % 16 != 0 : sheet % 2 != 0) return JL_DECLINED;
+    const int nslots = k / ti->slot_elems;
+    int lpr = 16;
+    while (lpr < 64 && lpr < nslots) lpr <<= 1;
+    const size_t act = ((size_t)k + (size_t)(k / 32) * 4 + (size_t)(k / 16) * 4 + 15) & ~(size_t)15;
+    const size_t lds = 8 * act;
+    if (lds > c->lds_limit) return JL_DECLINED;
+    MoeMatVecArgs a;
+    a.out[0] = out0; a.out[1] = out1;
+    a.bank[0] = (const uint8_t*)bank0; a.bank[1] = (const uint8_t*)bank1;
+    a.x = x; a.x2 = x2; a.src = src; a.start = start;
+    a.sheet_bytes = sheet; a.nrows = nrows; a.k = k; a.row_bytes = row_bytes; a.per = c->act_window / 32;
+    // row shares per expert: enough workgroups to cover the chip a couple of times when
+    // every expert is in use, never fewer than 64 rows a share
+    const int nmat = bank1 ? 2 : 1;
+    int shares = (2 * c->num_cu + n_expert * nmat - 1) / (n_expert * nmat);
+    if (shares < 1) shares = 1;
+    while (shares > 1 && nrows / shares < 64) shares--;
+    char name[64];
+    snprintf(name, sizeof name, "jl_moe_matvec_%s_l%d", ti->tag, lpr);
+    auto it = c->fn.find(name);
+    if (it == c->fn.end()) return fail(c, JL_ERR_ARG, "kernel %s is not in the code object", name);
+    void* params[] = {&a};
+    HIP_TRY(c, H->ModuleLaunchKernel(it->second, (unsigned)shares, (unsigned)n_expert, (unsigned)nmat, 512, 1, 1,
+                                     (unsigned)lds, st, params, nullptr));
+    return JL_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -327,7 +382,9 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     if (e != hipSuccess)
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
-    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_q4k"};
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_q4k", "jl_moe_group", "jl_moe_combine"};
+    for (const char* tag : {"q4k", "q8_0", "q6k"})
+        for (int lpr : {16, 32, 64}) names.push_back(std::string("jl_moe_matvec_") + tag + "_l" + std::to_string(lpr));
     const int types[] = {JL_TYPE_Q4_K, JL_TYPE_Q8_0, JL_TYPE_Q6_K};
     for (int t : types)
         for (int rpw : {1, 2, 4}) {
@@ -358,6 +415,7 @@ void jl_ctx_destroy(jl_ctx* c) {
     if (c->stream) (void)H->StreamSynchronize(c->stream);
     for (auto& kv : c->resident) (void)H->Free(kv.second.dev);
     if (c->gemm_ws) (void)H->Free(c->gemm_ws);
+    if (c->moe_ws) (void)H->Free(c->moe_ws);
     if (c->stage_x) (void)H->Free(c->stage_x);
     if (c->stage_out) (void)H->Free(c->stage_out);
     if (c->module) (void)H->ModuleUnload(c->module);
@@ -456,6 +514,76 @@ int jl_reserve(jl_ctx* c, int max_tok, int max_k) {
     if (max_tok <= 0 || max_k <= 0 || max_k % 256 != 0) return fail(c, JL_ERR_ARG, "reserve: %d x %d", max_tok, max_k);
     HIP_TRY(c, H->SetDevice(c->device));
     return gemm_ws_ensure(c, gemm_ws_need(max_tok, max_k));
+}
+
+int jl_moe_group_dev(jl_ctx* c, const uint32_t* sel, int sel_stride, int rows, int k_used, int n_expert,
+                     uint32_t* start, uint32_t* perm, uint32_t* pos, void* stream) {
+    if (!c) return JL_ERR_ARG;
+    if (!sel || !start || !perm || !pos || rows <= 0 || k_used <= 0 || sel_stride < k_used)
+        return fail(c, JL_ERR_ARG, "moe group: bad operand");
+    if (n_expert <= 0 || n_expert > 1024) return JL_DECLINED;
+    HIP_TRY(c, H->SetDevice(c->device));
+    MoeGroupArgs a;
+    a.sel = sel; a.start = start; a.perm = perm; a.pos = pos;
+    a.sel_stride = sel_stride; a.rows = rows; a.k_used = k_used; a.n_expert = n_expert;
+    void* params[] = {&a};
+    return launch(c, "jl_moe_group", 1, 1, 1024, 0, pick_stream(c, stream), params);
+}
+
+int jl_moe_matvec_dev(jl_ctx* c, float* out0, float* out1, int type, const void* bank0, const void* bank1,
+                      const float* x, const float* x2, const uint32_t* src, const uint32_t* start,
+                      int n_expert, int nrows, int k, void* stream) {
+    if (!c) return JL_ERR_ARG;
+    HIP_TRY(c, H->SetDevice(c->device));
+    return moe_matvec_launch(c, out0, out1, type, bank0, bank1, x, x2, src, start, n_expert, nrows, k,
+                             pick_stream(c, stream));
+}
+
+int jl_moe_combine_dev(jl_ctx* c, float* resid, const float* y, const float* wt, const uint32_t* sel,
+                       int sel_stride, const uint32_t* pos, int rows, int k_used, int n_embd, void* stream) {
+    if (!c) return JL_ERR_ARG;
+    if (!resid || !y || !wt || !sel || !pos || rows <= 0 || n_embd <= 0)
+        return fail(c, JL_ERR_ARG, "moe combine: bad operand");
+    if (k_used <= 0 || k_used > 16 || sel_stride < k_used || rows > 65535) return JL_DECLINED;
+    HIP_TRY(c, H->SetDevice(c->device));
+    MoeCombineArgs a;
+    a.resid = resid; a.y = y; a.wt = wt; a.sel = sel; a.pos = pos;
+    a.sel_stride = sel_stride; a.k_used = k_used; a.n_embd = n_embd;
+    void* params[] = {&a};
+    return launch(c, "jl_moe_combine", (unsigned)((n_embd + 255) / 256), (unsigned)rows, 256, 0,
+                  pick_stream(c, stream), params);
+}
+
+int jl_moe_ffn_dev(jl_ctx* c, float* resid, int type, const void* gate_bank, const void* up_bank,
+                   const void* down_bank, const float* x, const uint32_t* sel, int sel_stride,
+                   const float* wt, int rows, int k_used, int n_expert, int n_ffn, int n_embd, void* stream) {
+    if (!c) return JL_ERR_ARG;
+    if (rows <= 0 || k_used <= 0 || n_expert <= 0 || n_ffn <= 0 || n_embd <= 0)
+        return fail(c, JL_ERR_ARG, "moe ffn: bad shape");
+    if (n_expert > 1024 || k_used > 16 || n_ffn % 256 != 0 || n_embd % 256 != 0) return JL_DECLINED;
+    HIP_TRY(c, H->SetDevice(c->device));
+    hipStream_t st = pick_stream(c, stream);
+    const size_t ncols = (size_t)rows * k_used;
+    auto up256 = [](size_t v) { return (v + 255) & ~(size_t)255; };
+    const size_t o_start = 0, o_perm = up256((size_t)(n_expert + 1) * 4), o_pos = o_perm + up256(ncols * 4);
+    const size_t o_g = o_pos + up256(ncols * 4), o_u = o_g + up256(ncols * n_ffn * 4);
+    const size_t o_y = o_u + up256(ncols * n_ffn * 4), total = o_y + up256(ncols * n_embd * 4);
+    int rc = ws_ensure(c, &c->moe_ws, &c->moe_ws_bytes, total);
+    if (rc != JL_OK) return rc;
+    char* ws = (char*)c->moe_ws;
+    uint32_t* start = (uint32_t*)(ws + o_start);
+    uint32_t* perm = (uint32_t*)(ws + o_perm);
+    uint32_t* pos = (uint32_t*)(ws + o_pos);
+    float *g = (float*)(ws + o_g), *u = (float*)(ws + o_u), *y = (float*)(ws + o_y);
+    rc = jl_moe_group_dev(c, sel, sel_stride, rows, k_used, n_expert, start, perm, pos, st);
+    if (rc != JL_OK) return rc;
+    // gate and up: columns read the routed rows of x
+    rc = moe_matvec_launch(c, g, u, type, gate_bank, up_bank, x, nullptr, perm, start, n_expert, n_ffn, n_embd, st);
+    if (rc != JL_OK) return rc;
+    // down: the activation of column c is silu(g[c]) * u[c]
+    rc = moe_matvec_launch(c, y, nullptr, type, down_bank, nullptr, g, u, nullptr, start, n_expert, n_embd, n_ffn, st);
+    if (rc != JL_OK) return rc;
+    return jl_moe_combine_dev(c, resid, y, wt, sel, sel_stride, pos, rows, k_used, n_embd, st);
 }
 
 /* ------------------------------------------------------- host-pointer seam */

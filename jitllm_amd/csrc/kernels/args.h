@@ -33,3 +33,36 @@ struct GemmArgs {
     int nrows, k, ntok, tok_pad;
     int row_bytes;
 };
+
+// Mixture-of-experts grouping: sel [rows][sel_stride] expert ids (the first k_used of
+// each row are the selection) -> start [n_expert+1], perm [rows*k_used] (column ->
+// row), pos [rows*k_used] (pair -> column).
+struct MoeGroupArgs {
+    const uint32_t* sel;
+    uint32_t* start;
+    uint32_t* perm;
+    uint32_t* pos;
+    int sel_stride, rows, k_used, n_expert;
+};
+
+// Grouped expert matvec over columns sorted by expert: out[m][c][0:nrows] =
+// bank[m] sheet(expert of c) . act(c), act(c) = x[src(c)] or silu(x[src(c)]) * x2[src(c)].
+struct MoeMatVecArgs {
+    float* out[2];
+    const uint8_t* bank[2];
+    const float* x;
+    const float* x2;        // null: plain activation
+    const uint32_t* src;    // null: column c reads row c
+    const uint32_t* start;  // [n_expert + 1]
+    size_t sheet_bytes;
+    int nrows, k, row_bytes, per;
+};
+
+struct MoeCombineArgs {
+    float* resid;           // [rows][n_embd], accumulated into
+    const float* y;         // [ncols][n_embd]
+    const float* wt;        // [rows][k_used]
+    const uint32_t* sel;    // [rows][sel_stride]
+    const uint32_t* pos;    // [rows*k_used]
+    int sel_stride, k_used, n_embd;
+};

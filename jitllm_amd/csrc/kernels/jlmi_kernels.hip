@@ -6,6 +6,7 @@
 #include "dequant.h"
 #include "gemm_q4k.h"
 #include "matvec.h"
+#include "moe.h"
 #include "quantize.h"
 
 extern __shared__ __attribute__((aligned(16))) uint8_t jl_smem[];
@@ -55,3 +56,20 @@ JL_MATVEC_KERNEL(q6k, JL_Q6_K, 1, 1024) JL_MATVEC_KERNEL(q6k, JL_Q6_K, 2, 512) J
 extern "C" __global__ __launch_bounds__(256) void jl_gemm_prep_q4k(GemmPrepArgs p) { gemm_prep_q4k_body(p); }
 // grid = (tok_pad/128, ceil(nrows/128)), block = 512 (4 consumer + 4 producer wavefronts)
 extern "C" __global__ __launch_bounds__(512) void jl_gemm_q4k(GemmArgs p) { gemm_q4k_body(p, jl_smem); }
+
+// ------------------------------------------------------- mixture of experts
+// one workgroup of 1024; thread e owns expert e (n_expert <= 1024)
+extern "C" __global__ __launch_bounds__(1024) void jl_moe_group(MoeGroupArgs p) {
+    __shared__ u32 scount[1024];
+    moe_group_body(p, scount);
+}
+// grid = (row shares, n_expert, matrices), block = 512, dynamic LDS = 8 staged activations
+#define JL_MOE_KERNEL(T, TYPE, LPR)                                                               \
+    extern "C" __global__ __launch_bounds__(512) void jl_moe_matvec_##T##_l##LPR(MoeMatVecArgs p) { \
+        moe_matvec_body<TYPE, LPR>(p, jl_smem);                                                   \
+    }
+JL_MOE_KERNEL(q4k, JL_Q4_K, 16) JL_MOE_KERNEL(q4k, JL_Q4_K, 32) JL_MOE_KERNEL(q4k, JL_Q4_K, 64)
+JL_MOE_KERNEL(q8_0, JL_Q8_0, 16) JL_MOE_KERNEL(q8_0, JL_Q8_0, 32) JL_MOE_KERNEL(q8_0, JL_Q8_0, 64)
+JL_MOE_KERNEL(q6k, JL_Q6_K, 16) JL_MOE_KERNEL(q6k, JL_Q6_K, 32) JL_MOE_KERNEL(q6k, JL_Q6_K, 64)
+// grid = (ceil(n_embd/256), rows), block = 256
+extern "C" __global__ __launch_bounds__(256) void jl_moe_combine(MoeCombineArgs p) { moe_combine_body(p); }

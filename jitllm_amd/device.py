@@ -125,3 +125,29 @@ class Device:
         """x [ntok][k] -> out [ntok][nrows] on device operands (JIT.MatMulPacked semantics)."""
         return self._served(self._l.jl_matmul_dev(self._ctx, _ptr(out), t, _ptr(w), _ptr(x),
                                                   nrows, k, ntok, stream), "jl_matmul_dev")
+
+    # -- mixture of experts -----------------------------------------------------
+    def moe_group_dev(self, sel, sel_stride, rows, k_used, n_expert, start, perm, pos, stream=None):
+        return self._served(self._l.jl_moe_group_dev(self._ctx, _ptr(sel), sel_stride, rows, k_used,
+                                                     n_expert, _ptr(start), _ptr(perm), _ptr(pos), stream),
+                            "jl_moe_group_dev")
+
+    def moe_matvec_dev(self, out0, out1, t, bank0, bank1, x, x2, src, start, n_expert, nrows, k,
+                       stream=None):
+        opt = lambda a: None if a is None else _ptr(a)
+        return self._served(self._l.jl_moe_matvec_dev(self._ctx, _ptr(out0), opt(out1), t, _ptr(bank0),
+                                                      opt(bank1), _ptr(x), opt(x2), opt(src), _ptr(start),
+                                                      n_expert, nrows, k, stream), "jl_moe_matvec_dev")
+
+    def moe_combine_dev(self, resid, y, wt, sel, sel_stride, pos, rows, k_used, n_embd, stream=None):
+        return self._served(self._l.jl_moe_combine_dev(self._ctx, _ptr(resid), _ptr(y), _ptr(wt), _ptr(sel),
+                                                       sel_stride, _ptr(pos), rows, k_used, n_embd, stream),
+                            "jl_moe_combine_dev")
+
+    def moe_ffn_dev(self, resid, t, gate, up, down, x, sel, sel_stride, wt, rows, k_used, n_expert,
+                    n_ffn, n_embd, stream=None):
+        """One routed feed-forward block (moeBatchFrom): resid [rows][n_embd] += mixture output."""
+        return self._served(self._l.jl_moe_ffn_dev(self._ctx, _ptr(resid), t, _ptr(gate), _ptr(up),
+                                                   _ptr(down), _ptr(x), _ptr(sel), sel_stride, _ptr(wt),
+                                                   rows, k_used, n_expert, n_ffn, n_embd, stream),
+                            "jl_moe_ffn_dev")

@@ -1,0 +1,170 @@
+"""GPU parity of the grouped expert matmul (mixture-of-experts block) against the CPU
+oracle, through the C ABI.
+
+Stages are checked on their own so each is like-for-like: grouping is integer work
+(bit-exact against the oracle's groupPairs), each grouped matvec is held to NMSE
+<= 1e-10 against the f64 evaluation of the same int8 activations, the combine to the
+same sums in the same order; the whole block to rel-L2 <= 1e-3 against a pure-oracle
+evaluation (the down projection re-quantizes act(gate)*up, so a last-bit difference in
+gate/up can move an int8: the block is not a like-for-like quantity)."""
+import numpy as np
+import pytest
+
+import oracle
+from conftest import nmse, rel_l2
+from jitllm_amd import quant, synth
+
+pytestmark = pytest.mark.gpu
+
+
+def route(rows, n_expert, k_used, seed, mode="random"):
+    rng = np.random.default_rng(seed)
+    sel = np.zeros((rows, k_used + 1), np.uint32)
+    wt = np.zeros((rows, k_used), np.float32)
+    for r in range(rows):
+        logits = rng.standard_normal(n_expert).astype(np.float32)
+        if mode == "one_expert":
+            logits[:] = -30
+            logits[5:5 + k_used] = 10 + np.arange(k_used)[::-1]
+        elif mode == "mostly_empty":
+            logits[k_used + 1:] -= 40
+        s, w, _, _ = oracle.moe_route(logits, k_used)
+        sel[r, :k_used], wt[r] = s, w
+    return sel, wt
+
+
+def silu(g):
+    g = g.astype(np.float64)
+    return g / (1 + np.exp(-g))
+
+
+@pytest.mark.parametrize("mode,rows,n_expert,k_used", [("random", 12, 16, 4), ("one_expert", 9, 16, 2),
+                                                       ("mostly_empty", 7, 32, 3), ("random", 5, 8, 1),
+                                                       ("random", 64, 128, 8)])
+def test_grouping_is_bit_exact(dev, devbuf, mode, rows, n_expert, k_used):
+    sel, _ = route(rows, n_expert, k_used, 3, mode)
+    used, perm, col_e, pos = oracle.group_pairs(sel.reshape(-1), rows, k_used, n_expert, 1)
+    assert used == rows * k_used
+    want_start = np.searchsorted(col_e[:used], np.arange(n_expert + 1)).astype(np.uint32)
+    sd = devbuf(sel)
+    start = devbuf(shape=(n_expert + 1,), dtype=np.uint32, fill=99)
+    dperm = devbuf(shape=(used,), dtype=np.uint32, fill=99)
+    dpos = devbuf(shape=(used,), dtype=np.uint32, fill=99)
+    assert dev.moe_group_dev(sd.ptr, k_used + 1, rows, k_used, n_expert, start.ptr, dperm.ptr, dpos.ptr)
+    dev.synchronize()
+    assert np.array_equal(start.get(), want_start)
+    assert np.array_equal(dperm.get(), perm[:used])
+    assert np.array_equal(dpos.get(), pos)
+
+
+def _banks(t, n_expert, nrows, k, seed, planted):
+    make = synth.random_weights if planted else synth.quantized_weights
+    return np.concatenate([make(t, nrows, k, seed=seed + e) for e in range(n_expert)])
+
+
+@pytest.mark.parametrize("t,nrows,k", [(quant.Q4_K, 96, 2048), (quant.Q4_K, 200, 768), (quant.Q4_K, 40, 4096),
+                                       (quant.Q8_0, 64, 1024), (quant.Q6_K, 70, 1024)])
+def test_grouped_matvec_vs_oracle(dev, devbuf, t, nrows, k):
+    rows, n_expert, k_used, window = 13, 8, 3, 256 if t in quant.K_QUANTS else 32
+    dev.SetActWindow(window)
+    sel, _ = route(rows, n_expert, k_used, 4)
+    sel[0, :k_used] = [1, 2, 3]
+    sel[1:12, 0] = 6                      # one expert with 11+ columns: more than one pass of eight
+    sel[1:12, 1], sel[1:12, 2] = 0, 7
+    used, perm, col_e, pos = oracle.group_pairs(sel.reshape(-1), rows, k_used, n_expert, 1)
+    start = np.searchsorted(col_e[:used], np.arange(n_expert + 1)).astype(np.uint32)
+    bank0 = _banks(t, n_expert, nrows, k, 10, False)
+    bank1 = _banks(t, n_expert, nrows, k, 50, True)
+    x = np.stack([synth.activations(k, seed=200 + r) for r in range(rows)])
+    sheet = nrows * quant.row_bytes(t, k)
+    want0 = np.zeros((used, nrows))
+    want1 = np.zeros((used, nrows))
+    for c in range(used):
+        e = int(col_e[c])
+        q, a_s, _ = oracle.quantize_act(x[perm[c]], window)
+        want0[c] = oracle.matvec_q8act_f64(t, bank0[e * sheet:(e + 1) * sheet], q, a_s, nrows, k)
+        want1[c] = oracle.matvec_q8act_f64(t, bank1[e * sheet:(e + 1) * sheet], q, a_s, nrows, k)
+    b0, b1, xd = devbuf(bank0), devbuf(bank1), devbuf(x)
+    dstart, dperm = devbuf(start), devbuf(perm[:used].copy())
+    o0 = devbuf(shape=(used, nrows), dtype=np.float32, fill=np.float32(4e30))
+    o1 = devbuf(shape=(used, nrows), dtype=np.float32, fill=np.float32(4e30))
+    assert dev.moe_matvec_dev(o0.ptr, o1.ptr, t, b0.ptr, b1.ptr, xd.ptr, None, dperm.ptr, dstart.ptr,
+                              n_expert, nrows, k)
+    dev.synchronize()
+    assert nmse(o0.get(), want0) <= 1e-10 and nmse(o1.get(), want1) <= 1e-10
+    # SwiGLU form: column c reads silu(x[c]) * x2[c], no gather
+    g = np.stack([synth.activations(k, seed=300 + c) for c in range(used)])
+    u = np.stack([synth.activations(k, seed=400 + c) for c in range(used)])
+    gd, ud = devbuf(g), devbuf(u)
+    assert dev.moe_matvec_dev(o0.ptr, None, t, b0.ptr, None, gd.ptr, ud.ptr, None, dstart.ptr, n_expert, nrows, k)
+    dev.synchronize()
+    got = o0.get()
+    h = (silu(g) * u.astype(np.float64)).astype(np.float32)
+    for c in range(used):
+        e = int(col_e[c])
+        q, a_s, _ = oracle.quantize_act(h[c], window)
+        want = oracle.matvec_q8act_f64(t, bank0[e * sheet:(e + 1) * sheet], q, a_s, nrows, k)
+        assert rel_l2(got[c], want) <= 1e-3     # exp() differs in the last bits: an int8 may move
+    dev.SetActWindow(32)
+
+
+def test_combine_order_and_values(dev, devbuf):
+    rows, n_expert, k_used, n_embd = 10, 16, 4, 300
+    sel, wt = route(rows, n_expert, k_used, 8)
+    used, perm, col_e, pos = oracle.group_pairs(sel.reshape(-1), rows, k_used, n_expert, 1)
+    rng = np.random.default_rng(1)
+    y = rng.standard_normal((used, n_embd)).astype(np.float32)
+    resid = rng.standard_normal((rows, n_embd)).astype(np.float32)
+    want = resid.copy()
+    for r in range(rows):                      # ascending expert id, one f32 multiply-add at a time
+        for s in np.argsort(sel[r, :k_used], kind="stable"):
+            want[r] = (want[r] + (wt[r, s] * y[pos[r * k_used + s]]).astype(np.float32)).astype(np.float32)
+    rd, yd, wd, sd, pd = devbuf(resid), devbuf(y), devbuf(wt), devbuf(sel), devbuf(pos)
+    assert dev.moe_combine_dev(rd.ptr, yd.ptr, wd.ptr, sd.ptr, k_used + 1, pd.ptr, rows, k_used, n_embd)
+    dev.synchronize()
+    assert np.array_equal(rd.get().view(np.uint32), want.view(np.uint32))
+
+
+def _oracle_block(t, gate, up, down, x, sel, wt, n_expert, n_ffn, n_embd, window):
+    rows, k_used = wt.shape
+    out = np.zeros((rows, n_embd))
+    gs, ds = n_ffn * quant.row_bytes(t, n_embd), n_embd * quant.row_bytes(t, n_ffn)
+    for e in range(n_expert):                   # expert-major, rows ascending
+        for r in range(rows):
+            for s in range(k_used):
+                if sel[r, s] != e:
+                    continue
+                q, a_s, _ = oracle.quantize_act(x[r], window)
+                g = oracle.matvec_q8act_f64(t, gate[e * gs:(e + 1) * gs], q, a_s, n_ffn, n_embd)
+                u = oracle.matvec_q8act_f64(t, up[e * gs:(e + 1) * gs], q, a_s, n_ffn, n_embd)
+                h = (silu(g.astype(np.float32)) * u.astype(np.float32)).astype(np.float32)
+                qh, ah, _ = oracle.quantize_act(h, window)
+                y = oracle.matvec_q8act_f64(t, down[e * ds:(e + 1) * ds], qh, ah, n_embd, n_ffn)
+                out[r] += float(wt[r, s]) * y
+    return out
+
+
+@pytest.mark.parametrize("shape", [(6, 8, 2, 256, 512), (64, 128, 8, 768, 2048)],
+                         ids=["tiny", "qwen3-30b-a3b"])
+def test_moe_block_vs_oracle(dev, devbuf, shape):
+    """The whole routed feed-forward block; the second case is the Qwen3-30B-A3B shape:
+    128 experts of 768x2048 / 2048x768 in Q4_K, 64 rows routed top-8."""
+    rows, n_expert, k_used, n_ffn, n_embd = shape
+    t, window = quant.Q4_K, 256
+    dev.SetActWindow(window)
+    sel, wt = route(rows, n_expert, k_used, 11)
+    gate = _banks(t, n_expert, n_ffn, n_embd, 1000, False)
+    up = _banks(t, n_expert, n_ffn, n_embd, 2000, False)
+    down = _banks(t, n_expert, n_embd, n_ffn, 3000, False)
+    x = np.stack([synth.activations(n_embd, seed=500 + r) for r in range(rows)])
+    want = _oracle_block(t, gate, up, down, x, sel, wt, n_expert, n_ffn, n_embd, window)
+    gd, ud, dd, xd, sd, wd = devbuf(gate), devbuf(up), devbuf(down), devbuf(x), devbuf(sel), devbuf(wt)
+    resid = devbuf(shape=(rows, n_embd), dtype=np.float32, fill=0)
+    for call in range(2):
+        resid.put(np.zeros((rows, n_embd), np.float32))
+        assert dev.moe_ffn_dev(resid.ptr, t, gd.ptr, ud.ptr, dd.ptr, xd.ptr, sd.ptr, k_used + 1, wd.ptr,
+                               rows, k_used, n_expert, n_ffn, n_embd)
+        dev.synchronize()
+        got = resid.get()
+        assert rel_l2(got, want) <= 1e-3, f"call {call}: rel-L2 {rel_l2(got, want):.3e}"
+    dev.SetActWindow(32)
