@@ -145,6 +145,15 @@ int jl_matmul_dev(jl_ctx *ctx, float *out, int type, const void *w, const float 
  * calls allocate nothing. */
 int jl_reserve(jl_ctx *ctx, int max_tok, int max_k);
 
+/* MXFP4 weights (GGUF type 39: 32 e2m1 codes + one E8M0 exponent per block) against
+ * bf16 activations with f32 accumulation: x [ntok][k] bf16 -> out [ntok][nrows] f32.
+ * The value is the reference's Dequant32 (format/quant/dequant.go:159-174) followed by
+ * an f32 matmul: dequantized MXFP4 weights are exact in bf16, so only the f32
+ * summation order differs.  The reference's own device path instead feeds e2m1 codes
+ * to its int8 kernels through a code table (jit/gpu/kernels/matvec.go:137-175). */
+int jl_matmul_mxfp4_bf16_dev(jl_ctx *ctx, float *out, const void *w, const uint16_t *x,
+                             int nrows, int k, int ntok, void *stream);
+
 /* ---- mixture of experts (device pointers) ----------------------------- */
 
 /* The grouping the device tier runs before a batched mixture (kernels.ExpertGroup*,

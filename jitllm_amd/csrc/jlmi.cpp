@@ -382,7 +382,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     if (e != hipSuccess)
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
-    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_q4k", "jl_moe_group", "jl_moe_combine"};
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_q4k", "jl_moe_group", "jl_moe_combine", "jl_mxfp4_gemm", "jl_mxfp4_matvec"};
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int lpr : {16, 32, 64}) names.push_back(std::string("jl_moe_matvec_") + tag + "_l" + std::to_string(lpr));
     const int types[] = {JL_TYPE_Q4_K, JL_TYPE_Q8_0, JL_TYPE_Q6_K};
@@ -584,6 +584,27 @@ int jl_moe_ffn_dev(jl_ctx* c, float* resid, int type, const void* gate_bank, con
     rc = moe_matvec_launch(c, y, nullptr, type, down_bank, nullptr, g, u, nullptr, start, n_expert, n_embd, n_ffn, st);
     if (rc != JL_OK) return rc;
     return jl_moe_combine_dev(c, resid, y, wt, sel, sel_stride, pos, rows, k_used, n_embd, st);
+}
+
+int jl_matmul_mxfp4_bf16_dev(jl_ctx* c, float* out, const void* w, const uint16_t* x, int nrows, int k,
+                             int ntok, void* stream) {
+    if (!c) return JL_ERR_ARG;
+    if (!out || !w || !x || nrows <= 0 || k <= 0 || ntok <= 0)
+        return fail(c, JL_ERR_ARG, "mxfp4 matmul: bad operand");
+    if (k % 32 != 0 || k < 32 || !aligned16(x) || (k % 8) != 0) return JL_DECLINED;
+    if ((size_t)(k / 32) * 17 > 0x7fffffffu || ntok > 65535 * 128) return JL_DECLINED;
+    HIP_TRY(c, H->SetDevice(c->device));
+    MxGemmArgs a;
+    a.out = out; a.w = (const uint8_t*)w; a.x = x;
+    a.nrows = nrows; a.k = k; a.ntok = ntok; a.row_bytes = (k / 32) * 17;
+    void* params[] = {&a};
+    hipStream_t st = pick_stream(c, stream);
+    if (ntok <= 8)  // a handful of tokens: stream the rows once, no tile to fill
+        return launch(c, "jl_mxfp4_matvec", (unsigned)((nrows + 3) / 4), 1, 256, 0, st, params);
+    const unsigned lds = 4u * 128u * 136u * 2u;
+    if (lds > c->lds_limit) return JL_DECLINED;
+    return launch(c, "jl_mxfp4_gemm", (unsigned)((ntok + 127) / 128), (unsigned)((nrows + 127) / 128), 256,
+                  lds, st, params);
 }
 
 /* ------------------------------------------------------- host-pointer seam */

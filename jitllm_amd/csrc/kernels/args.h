@@ -66,3 +66,12 @@ struct MoeCombineArgs {
     const uint32_t* pos;    // [rows*k_used]
     int sel_stride, k_used, n_embd;
 };
+
+// MXFP4 weights x bf16 activations: out [ntok][nrows] f32.
+struct MxGemmArgs {
+    float* out;
+    const uint8_t* w;     // GGUF row-major MXFP4 blocks (17 bytes per 32)
+    const uint16_t* x;    // bf16 bits, [ntok][k]
+    int nrows, k, ntok;
+    int row_bytes;
+};

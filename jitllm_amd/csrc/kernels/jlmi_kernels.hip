@@ -7,6 +7,7 @@
 #include "gemm_q4k.h"
 #include "matvec.h"
 #include "moe.h"
+#include "mxfp4.h"
 #include "quantize.h"
 
 extern __shared__ __attribute__((aligned(16))) uint8_t jl_smem[];
@@ -73,3 +74,9 @@ JL_MOE_KERNEL(q8_0, JL_Q8_0, 16) JL_MOE_KERNEL(q8_0, JL_Q8_0, 32) JL_MOE_KERNEL(
 JL_MOE_KERNEL(q6k, JL_Q6_K, 16) JL_MOE_KERNEL(q6k, JL_Q6_K, 32) JL_MOE_KERNEL(q6k, JL_Q6_K, 64)
 // grid = (ceil(n_embd/256), rows), block = 256
 extern "C" __global__ __launch_bounds__(256) void jl_moe_combine(MoeCombineArgs p) { moe_combine_body(p); }
+
+// ------------------------------------------------------------------- MXFP4
+// grid = (ceil(ntok/128), ceil(nrows/128)), block = 256, dynamic LDS = 4 stages of 128 x 272 B
+extern "C" __global__ __launch_bounds__(256) void jl_mxfp4_gemm(MxGemmArgs p) { mx_gemm_body(p, jl_smem); }
+// grid = ceil(nrows/4), block = 256: one wavefront per row, ntok <= 8
+extern "C" __global__ __launch_bounds__(256) void jl_mxfp4_matvec(MxGemmArgs p) { mx_matvec_body(p); }

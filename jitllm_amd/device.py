@@ -151,3 +151,9 @@ class Device:
                                                    _ptr(down), _ptr(x), _ptr(sel), sel_stride, _ptr(wt),
                                                    rows, k_used, n_expert, n_ffn, n_embd, stream),
                             "jl_moe_ffn_dev")
+
+    def matmul_mxfp4_bf16_dev(self, out, w, x, nrows, k, ntok, stream=None):
+        """MXFP4 weights x bf16 activations (bits as uint16) -> f32 out [ntok][nrows]."""
+        return self._served(self._l.jl_matmul_mxfp4_bf16_dev(self._ctx, _ptr(out), _ptr(w), _ptr(x),
+                                                             nrows, k, ntok, stream),
+                            "jl_matmul_mxfp4_bf16_dev")
