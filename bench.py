@@ -165,6 +165,89 @@ def gemm_section(dev):
     return out
 
 
+def moe_section(dev):
+    """Qwen3-30B-A3B routed feed-forward block: 128 experts (gate/up 768x2048, down 2048x768,
+    Q4_K), 64 rows routed top-8 by softmax over N(0,1) logits (seeded); one step = group +
+    gate/up + down + combine.  Bytes = the touched experts' three sheets + x in + resid out."""
+    from jitllm_amd import quant, synth
+    from jitllm_amd.hipmem import DeviceArray, Event
+    t, rows, n_expert, k_used, n_ffn, n_embd = quant.Q4_K, 64, 128, 8, 768, 2048
+    dev.SetActWindow(256)
+    rng = np.random.default_rng(0)
+    logits = rng.standard_normal((rows, n_expert)).astype(np.float32)
+    p = np.exp(logits - logits.max(axis=1, keepdims=True))
+    p = (p / p.sum(axis=1, keepdims=True)).astype(np.float32)
+    sel = np.zeros((rows, k_used + 1), np.uint32)
+    # top-k by (score desc, index asc): a stable sort of the negated scores
+    order = np.argsort(-p, axis=1, kind="stable")[:, :k_used]
+    sel[:, :k_used] = order
+    wt = np.take_along_axis(p, order, axis=1)
+    wt = (wt / (wt.sum(axis=1, keepdims=True) + np.float32(1e-20))).astype(np.float32)
+    touched = len(np.unique(order))
+    gs = n_ffn * quant.row_bytes(t, n_embd)
+    ds = n_embd * quant.row_bytes(t, n_ffn)
+    banks = []
+    for i, (r, k) in enumerate([(n_ffn, n_embd), (n_ffn, n_embd), (n_embd, n_ffn)]):
+        banks.append(DeviceArray(synth.quantized_weights(t, r * n_expert, k, seed=10 + i)))
+    x = DeviceArray(rng.standard_normal((rows, n_embd)).astype(np.float32))
+    sd, wd = DeviceArray(sel), DeviceArray(wt)
+    resid = DeviceArray(shape=(rows, n_embd), dtype=np.float32, fill=0)
+    run = lambda: dev.moe_ffn_dev(resid.ptr, t, banks[0].ptr, banks[1].ptr, banks[2].ptr, x.ptr, sd.ptr,
+                                  k_used + 1, wd.ptr, rows, k_used, n_expert, n_ffn, n_embd)
+    for _ in range(3):
+        if not run():
+            raise RuntimeError("the device declined the mixture block")
+    dev.synchronize()
+    e0, e1, n = Event(), Event(), 20
+    e0.record(dev.stream)
+    for _ in range(n):
+        run()
+    e1.record(dev.stream)
+    e1.synchronize()
+    ms = e0.elapsed_ms(e1) / n
+    nbytes = touched * (2 * gs + ds) + 2 * rows * n_embd * 4
+    for b in banks + [x, sd, wd, resid]:
+        b.free()
+    return {"us_per_step": round(ms * 1e3, 1), "experts_touched": touched, "bytes_per_step": nbytes,
+            "GB/s": round(nbytes / (ms * 1e-3) / 1e9, 1),
+            "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+            "TFLOP/s": round(rows * k_used * 3 * 2.0 * n_ffn * n_embd / (ms * 1e-3) / 1e12, 2)}
+
+
+def mxfp4_section(dev):
+    """gpt-oss-20B expert shape: MXFP4 2880x2880, bf16 activations, tokens 1 / 64 / 1024."""
+    from jitllm_amd import quant, synth
+    from jitllm_amd.hipmem import DeviceArray, Event
+    nrows = k = 2880
+    w = DeviceArray(synth.quantized_weights(quant.MXFP4, nrows, k, seed=0))
+    out = {}
+    for ntok in (1, 64, 1024):
+        xf = np.random.default_rng(3).standard_normal((ntok, k)).astype(np.float32)
+        xb = (xf.view(np.uint32) >> 16).astype(np.uint16)
+        x = DeviceArray(xb)
+        o = DeviceArray(shape=(ntok, nrows), dtype=np.float32)
+        for _ in range(3):
+            if not dev.matmul_mxfp4_bf16_dev(o.ptr, w.ptr, x.ptr, nrows, k, ntok):
+                raise RuntimeError("the device declined the MXFP4 matmul")
+        dev.synchronize()
+        e0, e1, n = Event(), Event(), 50
+        e0.record(dev.stream)
+        for _ in range(n):
+            dev.matmul_mxfp4_bf16_dev(o.ptr, w.ptr, x.ptr, nrows, k, ntok)
+        e1.record(dev.stream)
+        e1.synchronize()
+        ms = e0.elapsed_ms(e1) / n
+        nbytes = nrows * (k // 32) * 17 + ntok * k * 2 + ntok * nrows * 4
+        tf = 2.0 * nrows * k * ntok / (ms * 1e-3) / 1e12
+        out[f"{ntok} tokens"] = {"us_per_step": round(ms * 1e3, 1), "TFLOP/s": round(tf, 2),
+                                 "frac_of_bf16_mfma_peak": round(tf / MFMA_F16_PEAK_TFLOPS, 4),
+                                 "GB/s": round(nbytes / (ms * 1e-3) / 1e9, 1), "weights": "single copy (cache resident)"}
+        x.free()
+        o.free()
+    w.free()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -216,6 +299,8 @@ def main():
 
     if not args.no_extra:
         line["prefill_gemm"] = gemm_section(dev)
+        line["moe_block"] = moe_section(dev)
+        line["mxfp4_gemm"] = mxfp4_section(dev)
 
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(quant.Q4_K, 4096, 4096, 256)
