@@ -83,7 +83,9 @@ int jl_synchronize(jl_ctx *ctx);
 
 /* Kernel-shape overrides for measurement: key is one of "matvec.rpw" (rows per
  * wavefront: 1, 2, 4), "matvec.block" (threads per workgroup), "matvec.grid"
- * (workgroups), "gemm.min_tok" (fewest tokens sent to the matrix-core GEMM);
+ * (workgroups), "gemm.min_tok" (fewest tokens sent to the matrix-core GEMM),
+ * "packed.rw" (rows per wavefront of the packed-plane matvec: 16, 32, 64),
+ * "packed.block" (its threads per workgroup);
  * value 0 restores the built-in choice.  Mirrors the reference's per-instance tuning knobs
  * (engine/nn/options.go:67-118). */
 int jl_set_tuning(jl_ctx *ctx, const char *key, int value);
@@ -105,6 +107,24 @@ int jl_forget(jl_ctx *ctx, const void *p, size_t n);
  * out [ntok][nrows].  Each token is quantized on its own. */
 int jl_matmul(jl_ctx *ctx, float *out, int type, const void *w, size_t wbytes,
               const float *x, int nrows, int k, int ntok);
+
+/* ---- packed planes, host pointers ------------------------------------- */
+
+/* kernels.PackedWords (jit/gpu/kernels/pack.go:580-621): u32 words of the QS, D and
+ * SC planes of an nrows x k matrix.  Pure host arithmetic; JL_DECLINED for a type
+ * or k the planes are not defined for. */
+int jl_packed_words(int type, int nrows, int k, size_t *nq, size_t *nd, size_t *nsc);
+
+/* JIT.MatVecPacked (engine/nn/packed.go:24): rows row .. row+nrows of planes that
+ * hold `stride` rows (nn.Packed{QS,D,SC,Row,Stride}, engine/nn/device.go:70-80).
+ * Residency of the three planes is keyed on the pointer qs, as for jl_matvec. */
+int jl_matvec_packed(jl_ctx *ctx, float *out, int type, const uint32_t *qs, const uint32_t *d,
+                     const uint32_t *sc, int row, int stride, const float *x, int nrows, int k);
+
+/* JIT.MatMulPacked (engine/nn/packedmm.go:23): x [ntok][k] -> out [ntok][nrows]. */
+int jl_matmul_packed(jl_ctx *ctx, float *out, int type, const uint32_t *qs, const uint32_t *d,
+                     const uint32_t *sc, int row, int stride, const float *x, int nrows, int k,
+                     int ntok);
 
 /* ---- device-pointer entry points -------------------------------------- */
 
@@ -144,6 +164,42 @@ int jl_matmul_dev(jl_ctx *ctx, float *out, int type, const void *w, const float 
  * prefill workspace for up to max_tok tokens of max_k features now, so later
  * calls allocate nothing. */
 int jl_reserve(jl_ctx *ctx, int max_tok, int max_k);
+
+/* kernels.PackWeightsInto (jit/gpu/kernels/pack.go:52-199) on the device: GGUF
+ * row-major blocks -> the three planes [unit][row] (sizes from jl_packed_words; sc may
+ * be NULL for Q8_0).  Q4_K, Q6_K and Q8_0; the result is byte for byte the
+ * reference's.  src 4-byte aligned for Q4_K, 2-byte for the others. */
+int jl_pack_weights_dev(jl_ctx *ctx, int type, const void *src, int nrows, int k, uint32_t *qs,
+                        uint32_t *d, uint32_t *sc, void *stream);
+
+/* The inverse permutation for Q4_K: rows row .. row+nrows of the planes back to GGUF
+ * super-blocks in dst (nrows * k/256 * 144 bytes, 4-byte aligned), bit for bit. */
+int jl_unpack_weights_dev(jl_ctx *ctx, int type, const uint32_t *qs, const uint32_t *d,
+                          const uint32_t *sc, int row, int stride, int nrows, int k, void *dst,
+                          void *stream);
+
+/* JIT.MatVecPacked on resident planes (engine/nn/packed.go:24-198; device twin
+ * jit/gpu/kernels/matvec.go:1121-1271): quantizes x inside the kernel and computes
+ * out[0:nrows] for rows row .. row+nrows of planes holding `stride` rows.  An expert
+ * sheet of a bank is its own set of planes (format/jlm/write.go:123-140): pass the
+ * sheet's plane pointers with row 0. */
+int jl_matvec_packed_dev(jl_ctx *ctx, float *out, int type, const uint32_t *qs, const uint32_t *d,
+                         const uint32_t *sc, int row, int stride, const float *x, int nrows,
+                         int k, void *stream);
+
+/* The same over activations already quantized by jl_quantize_act_dev. */
+int jl_matvec_packed_q8_dev(jl_ctx *ctx, float *out, int type, const uint32_t *qs,
+                            const uint32_t *d, const uint32_t *sc, int row, int stride,
+                            const int8_t *q, const float *as, const float *sum16, int nrows,
+                            int k, void *stream);
+
+/* JIT.MatMulPacked on resident planes (engine/nn/packedmm.go:23-139).  Q4_K with the
+ * 256 window and enough tokens restores the row range to GGUF order in a workspace the
+ * context owns and runs the matrix-core GEMM on it; other cases run one packed matvec
+ * launch per token. */
+int jl_matmul_packed_dev(jl_ctx *ctx, float *out, int type, const uint32_t *qs, const uint32_t *d,
+                         const uint32_t *sc, int row, int stride, const float *x, int nrows,
+                         int k, int ntok, void *stream);
 
 /* MXFP4 weights (GGUF type 39: 32 e2m1 codes + one E8M0 exponent per block) against
  * bf16 activations with f32 accumulation: x [ntok][k] bf16 -> out [ntok][nrows] f32.

@@ -38,6 +38,16 @@ SIGNATURES = {
     "jl_matvec_q8_dev": (_int, [_vp, _vp, _int, _vp, _vp, _vp, _vp, _int, _int, _vp]),
     "jl_matmul_dev": (_int, [_vp, _vp, _int, _vp, _vp, _int, _int, _int, _vp]),
     "jl_reserve": (_int, [_vp, _int, _int]),
+    "jl_packed_words": (_int, [_int, _int, _int, C.POINTER(_sz), C.POINTER(_sz), C.POINTER(_sz)]),
+    "jl_matvec_packed": (_int, [_vp, _vp, _int, _vp, _vp, _vp, _int, _int, _vp, _int, _int]),
+    "jl_matmul_packed": (_int, [_vp, _vp, _int, _vp, _vp, _vp, _int, _int, _vp, _int, _int, _int]),
+    "jl_pack_weights_dev": (_int, [_vp, _int, _vp, _int, _int, _vp, _vp, _vp, _vp]),
+    "jl_unpack_weights_dev": (_int, [_vp, _int, _vp, _vp, _vp, _int, _int, _int, _int, _vp, _vp]),
+    "jl_matvec_packed_dev": (_int, [_vp, _vp, _int, _vp, _vp, _vp, _int, _int, _vp, _int, _int, _vp]),
+    "jl_matvec_packed_q8_dev": (_int, [_vp, _vp, _int, _vp, _vp, _vp, _int, _int, _vp, _vp, _vp, _int,
+                                       _int, _vp]),
+    "jl_matmul_packed_dev": (_int, [_vp, _vp, _int, _vp, _vp, _vp, _int, _int, _vp, _int, _int, _int,
+                                    _vp]),
     "jl_matmul_mxfp4_bf16_dev": (_int, [_vp, _vp, _vp, _vp, _int, _int, _int, _vp]),
     "jl_moe_group_dev": (_int, [_vp, _vp, _int, _int, _int, _int, _vp, _vp, _vp, _vp]),
     "jl_moe_matvec_dev": (_int, [_vp, _vp, _vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp]),

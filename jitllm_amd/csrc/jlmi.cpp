@@ -28,6 +28,7 @@ const HipApi* H = nullptr;  // the process-wide HIP runtime, resolved by the fir
 
 struct Tuning {
     int rpw = 0, block = 0, grid = 0;
+    int packed_rw = 0, packed_block = 0;
 };
 
 struct Resident {
@@ -53,6 +54,10 @@ struct jl_ctx {
     // prefill GEMM workspace (quantized activations in stage layout), grown on demand
     void* gemm_ws = nullptr;
     size_t gemm_ws_bytes = 0;
+
+    // rows restored to GGUF order for the GEMM over packed planes
+    void* unpack_ws = nullptr;
+    size_t unpack_ws_bytes = 0;
 
     // mixture-of-experts workspace (grouping tables and intermediate columns)
     void* moe_ws = nullptr;
@@ -302,6 +307,108 @@ int ws_ensure(jl_ctx* c, void** buf, size_t* have, size_t need) {
     return JL_OK;
 }
 
+// Words of the three planes of an nrows x k matrix (jit/gpu/kernels/pack.go:580-621).
+bool packed_words(int type, size_t nrows, int k, size_t* nq, size_t* nd, size_t* nsc) {
+    if (k <= 0 || nrows == 0) return false;
+    switch (type) {
+    case JL_TYPE_Q4_K:
+        if (k % 256) return false;
+        *nq = nrows * (size_t)(k / 32) * 4; *nd = nrows * (size_t)(k / 256); *nsc = *nd * 3;
+        return true;
+    case JL_TYPE_Q6_K:
+        if (k % 256) return false;
+        *nq = nrows * (size_t)(k / 16) * 3; *nd = nrows * (size_t)(k / 256); *nsc = nrows * (size_t)(k / 64);
+        return true;
+    case JL_TYPE_Q8_0:
+        if (k % 32) return false;
+        *nq = nrows * (size_t)(k / 32) * 8; *nd = (size_t)(k / 32) * ((nrows + 1) / 2); *nsc = 0;
+        return true;
+    }
+    return false;
+}
+
+struct PlaneRef {
+    const uint32_t *qs, *d, *sc;
+    int row, stride;
+};
+
+int packed_check(jl_ctx* c, int type, const PlaneRef& pl, int nrows, int k, const TypeInfo** ti) {
+    *ti = type_info(type);
+    if (!*ti) return JL_DECLINED;
+    if (nrows <= 0 || k <= 0 || pl.row < 0 || pl.stride <= 0)
+        return fail(c, JL_ERR_ARG, "packed: nrows=%d k=%d row=%d stride=%d", nrows, k, pl.row, pl.stride);
+    if ((long)pl.row + nrows > pl.stride)
+        return fail(c, JL_ERR_ARG, "packed: rows %d..%d outside a buffer of %d rows", pl.row, pl.row + nrows, pl.stride);
+    if (k % (*ti)->block_elems != 0) return JL_DECLINED;
+    if (!pl.qs || !pl.d || (type != JL_TYPE_Q8_0 && !pl.sc)) return fail(c, JL_ERR_ARG, "packed: null plane");
+    if (((uintptr_t)pl.qs | (uintptr_t)pl.d | (uintptr_t)pl.sc) & 3) return JL_DECLINED;
+    return JL_OK;
+}
+
+int packed_matvec_launch(jl_ctx* c, float* out, int type, const PlaneRef& pl, const float* x,
+                         const int8_t* q, const float* as, const float* s16, int nrows, int k,
+                         hipStream_t st) {
+    const TypeInfo* ti = nullptr;
+    int rc = packed_check(c, type, pl, nrows, k, &ti);
+    if (rc != JL_OK) return rc;
+    if (!out) return fail(c, JL_ERR_ARG, "packed matvec: null out");
+    if (x && !aligned16(x)) return JL_DECLINED;
+    if (!x && (!q || !as || !s16)) return fail(c, JL_ERR_ARG, "packed matvec: no activation");
+    if (q && ((uintptr_t)q & 3)) return JL_DECLINED;
+    // Rows per wavefront: the widest run that still gives every CU a workgroup.
+    int rw = c->tune.packed_rw;
+    if (rw <= 0) {
+        rw = 64;
+        while (rw > 16 && (nrows + rw - 1) / rw < c->num_cu) rw >>= 1;
+    }
+    if (rw != 16 && rw != 32 && rw != 64) return fail(c, JL_ERR_ARG, "packed matvec: rw=%d", rw);
+    const int nchunks = (k + 255) / 256;
+    int nw = c->tune.packed_block > 0 ? c->tune.packed_block / 64 : 16;
+    if (nw > nchunks) nw = nchunks;
+    if (nw < 1 || nw > 16) return fail(c, JL_ERR_ARG, "packed matvec: block=%d", nw * 64);
+    PackedMatVecArgs a;
+    a.out = out; a.qs = pl.qs; a.d = pl.d; a.sc = pl.sc;
+    a.x = x; a.q = q; a.as = as; a.s16 = s16;
+    a.nrows = nrows; a.k = k; a.row0 = pl.row; a.stride = pl.stride; a.per = c->act_window / 32;
+    char name[64];
+    snprintf(name, sizeof name, "jl_matvec_packed_%s_w%d", ti->tag, rw);
+    void* params[] = {&a};
+    return launch(c, name, (unsigned)((nrows + rw - 1) / rw), 1, (unsigned)(nw * 64),
+                  (unsigned)(nw * (384 + 256)), st, params);
+}
+
+int unpack_launch(jl_ctx* c, const PlaneRef& pl, int nrows, int k, void* dst, hipStream_t st) {
+    UnpackArgs a;
+    a.dst = (uint8_t*)dst; a.qs = pl.qs; a.d = pl.d; a.sc = pl.sc;
+    a.nrows = nrows; a.k = k; a.row0 = pl.row; a.stride = pl.stride;
+    void* params[] = {&a};
+    return launch(c, "jl_unpack_q4k", (unsigned)((nrows + 255) / 256), (unsigned)(k / 256), 256, 0, st, params);
+}
+
+int packed_matmul_launch(jl_ctx* c, float* out, int type, const PlaneRef& pl, const float* x, int nrows,
+                         int k, int ntok, hipStream_t st) {
+    const TypeInfo* ti = nullptr;
+    int rc = packed_check(c, type, pl, nrows, k, &ti);
+    if (rc != JL_OK) return rc;
+    if (!out || !x || ntok <= 0) return fail(c, JL_ERR_ARG, "packed matmul: bad operand");
+    if (!aligned16(x) || (k % 4) != 0) return JL_DECLINED;
+    const bool gemm = type == JL_TYPE_Q4_K && c->act_window == 256 && ntok >= c->gemm_min_tok &&
+                      ntok <= 65535 * 4 && kGemmLdsBytes <= c->lds_limit && k / 256 <= 65535;
+    if (gemm) {
+        rc = ws_ensure(c, &c->unpack_ws, &c->unpack_ws_bytes, (size_t)nrows * (size_t)(k / 256) * 144);
+        if (rc != JL_OK) return rc;
+        rc = unpack_launch(c, pl, nrows, k, c->unpack_ws, st);
+        if (rc != JL_OK) return rc;
+        return gemm_q4k_launch(c, out, c->unpack_ws, x, nrows, k, ntok, st);
+    }
+    for (int t = 0; t < ntok; t++) {
+        rc = packed_matvec_launch(c, out + (size_t)t * nrows, type, pl, x + (size_t)t * k, nullptr, nullptr,
+                                  nullptr, nrows, k, st);
+        if (rc != JL_OK) return rc;
+    }
+    return JL_OK;
+}
+
 int moe_matvec_launch(jl_ctx* c, float* out0, float* out1, int type, const void* bank0, const void* bank1,
                       const float* x, const float* x2, const uint32_t* src, const uint32_t* start,
                       int n_expert, int nrows, int k, hipStream_t st) {
@@ -382,7 +489,10 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     if (e != hipSuccess)
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
-    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_q4k", "jl_moe_group", "jl_moe_combine", "jl_mxfp4_gemm", "jl_mxfp4_matvec"};
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_q4k", "jl_moe_group", "jl_moe_combine", "jl_mxfp4_gemm", "jl_mxfp4_matvec",
+                                      "jl_pack_weights", "jl_unpack_q4k"};
+    for (const char* tag : {"q4k", "q8_0", "q6k"})
+        for (int rw : {16, 32, 64}) names.push_back(std::string("jl_matvec_packed_") + tag + "_w" + std::to_string(rw));
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int lpr : {16, 32, 64}) names.push_back(std::string("jl_moe_matvec_") + tag + "_l" + std::to_string(lpr));
     const int types[] = {JL_TYPE_Q4_K, JL_TYPE_Q8_0, JL_TYPE_Q6_K};
@@ -416,6 +526,7 @@ void jl_ctx_destroy(jl_ctx* c) {
     for (auto& kv : c->resident) (void)H->Free(kv.second.dev);
     if (c->gemm_ws) (void)H->Free(c->gemm_ws);
     if (c->moe_ws) (void)H->Free(c->moe_ws);
+    if (c->unpack_ws) (void)H->Free(c->unpack_ws);
     if (c->stage_x) (void)H->Free(c->stage_x);
     if (c->stage_out) (void)H->Free(c->stage_out);
     if (c->module) (void)H->ModuleUnload(c->module);
@@ -447,6 +558,8 @@ int jl_set_tuning(jl_ctx* c, const char* key, int value) {
     if (!strcmp(key, "matvec.rpw")) c->tune.rpw = value;
     else if (!strcmp(key, "matvec.block")) c->tune.block = value;
     else if (!strcmp(key, "matvec.grid")) c->tune.grid = value;
+    else if (!strcmp(key, "packed.rw")) c->tune.packed_rw = value;
+    else if (!strcmp(key, "packed.block")) c->tune.packed_block = value;
     else if (!strcmp(key, "gemm.min_tok")) c->gemm_min_tok = value > 0 ? value : 8;
     else return fail(c, JL_ERR_ARG, "unknown tuning key %s", key);
     return JL_OK;
@@ -507,6 +620,71 @@ int jl_matmul_dev(jl_ctx* c, float* out, int type, const void* w, const float* x
     if (!c) return JL_ERR_ARG;
     HIP_TRY(c, H->SetDevice(c->device));
     return matmul_launch(c, out, type, w, x, nrows, k, ntok, pick_stream(c, stream));
+}
+
+int jl_packed_words(int type, int nrows, int k, size_t* nq, size_t* nd, size_t* nsc) {
+    if (!nq || !nd || !nsc || nrows <= 0) return JL_ERR_ARG;
+    return packed_words(type, (size_t)nrows, k, nq, nd, nsc) ? JL_OK : JL_DECLINED;
+}
+
+int jl_pack_weights_dev(jl_ctx* c, int type, const void* src, int nrows, int k, uint32_t* qs, uint32_t* d,
+                        uint32_t* sc, void* stream) {
+    if (!c) return JL_ERR_ARG;
+    size_t nq, nd, nsc;
+    if (nrows <= 0 || !packed_words(type, (size_t)nrows, k, &nq, &nd, &nsc)) return JL_DECLINED;
+    if (!src || !qs || !d || (nsc && !sc)) return fail(c, JL_ERR_ARG, "pack: null operand");
+    if ((uintptr_t)src & (type == JL_TYPE_Q4_K ? 3 : 1)) return JL_DECLINED;
+    if (((uintptr_t)qs | (uintptr_t)d | (uintptr_t)sc) & 3) return JL_DECLINED;
+    const int units = type == JL_TYPE_Q8_0 ? k / 32 : k / 256;
+    if (units > 65535) return JL_DECLINED;
+    HIP_TRY(c, H->SetDevice(c->device));
+    PackArgs a;
+    a.src = (const uint8_t*)src; a.qs = qs; a.d = d; a.sc = sc; a.nrows = nrows; a.k = k; a.type = type;
+    void* params[] = {&a};
+    return launch(c, "jl_pack_weights", (unsigned)((nrows + 255) / 256), (unsigned)units, 256, 0,
+                  pick_stream(c, stream), params);
+}
+
+int jl_unpack_weights_dev(jl_ctx* c, int type, const uint32_t* qs, const uint32_t* d, const uint32_t* sc,
+                          int row, int stride, int nrows, int k, void* dst, void* stream) {
+    if (!c) return JL_ERR_ARG;
+    if (type != JL_TYPE_Q4_K) return JL_DECLINED;
+    const PlaneRef pl = {qs, d, sc, row, stride};
+    const TypeInfo* ti = nullptr;
+    int rc = packed_check(c, type, pl, nrows, k, &ti);
+    if (rc != JL_OK) return rc;
+    if (!dst) return fail(c, JL_ERR_ARG, "unpack: null dst");
+    if (((uintptr_t)dst & 3) || k / 256 > 65535) return JL_DECLINED;
+    HIP_TRY(c, H->SetDevice(c->device));
+    return unpack_launch(c, pl, nrows, k, dst, pick_stream(c, stream));
+}
+
+int jl_matvec_packed_dev(jl_ctx* c, float* out, int type, const uint32_t* qs, const uint32_t* d,
+                         const uint32_t* sc, int row, int stride, const float* x, int nrows, int k,
+                         void* stream) {
+    if (!c) return JL_ERR_ARG;
+    if (!x) return fail(c, JL_ERR_ARG, "packed matvec: null x");
+    HIP_TRY(c, H->SetDevice(c->device));
+    const PlaneRef pl = {qs, d, sc, row, stride};
+    return packed_matvec_launch(c, out, type, pl, x, nullptr, nullptr, nullptr, nrows, k, pick_stream(c, stream));
+}
+
+int jl_matvec_packed_q8_dev(jl_ctx* c, float* out, int type, const uint32_t* qs, const uint32_t* d,
+                            const uint32_t* sc, int row, int stride, const int8_t* q, const float* as,
+                            const float* sum16, int nrows, int k, void* stream) {
+    if (!c) return JL_ERR_ARG;
+    HIP_TRY(c, H->SetDevice(c->device));
+    const PlaneRef pl = {qs, d, sc, row, stride};
+    return packed_matvec_launch(c, out, type, pl, nullptr, q, as, sum16, nrows, k, pick_stream(c, stream));
+}
+
+int jl_matmul_packed_dev(jl_ctx* c, float* out, int type, const uint32_t* qs, const uint32_t* d,
+                         const uint32_t* sc, int row, int stride, const float* x, int nrows, int k,
+                         int ntok, void* stream) {
+    if (!c) return JL_ERR_ARG;
+    HIP_TRY(c, H->SetDevice(c->device));
+    const PlaneRef pl = {qs, d, sc, row, stride};
+    return packed_matmul_launch(c, out, type, pl, x, nrows, k, ntok, pick_stream(c, stream));
 }
 
 int jl_reserve(jl_ctx* c, int max_tok, int max_k) {
@@ -634,6 +812,64 @@ int jl_matmul(jl_ctx* c, float* out, int type, const void* w, size_t wbytes, con
     if ((rc = ensure_stage(c, &c->stage_out, &c->stage_out_bytes, ob)) != JL_OK) return rc;
     HIP_TRY(c, H->MemcpyAsync(c->stage_x, x, xb, hipMemcpyHostToDevice, c->stream));
     rc = matmul_launch(c, (float*)c->stage_out, type, wd, (const float*)c->stage_x, nrows, k, ntok, c->stream);
+    if (rc != JL_OK) {
+        (void)H->StreamSynchronize(c->stream);
+        return rc;
+    }
+    HIP_TRY(c, H->MemcpyAsync(out, c->stage_out, ob, hipMemcpyDeviceToHost, c->stream));
+    HIP_TRY(c, H->StreamSynchronize(c->stream));
+    return JL_OK;
+}
+
+int jl_matvec_packed(jl_ctx* c, float* out, int type, const uint32_t* qs, const uint32_t* d,
+                     const uint32_t* sc, int row, int stride, const float* x, int nrows, int k) {
+    return jl_matmul_packed(c, out, type, qs, d, sc, row, stride, x, nrows, k, 1);
+}
+
+int jl_matmul_packed(jl_ctx* c, float* out, int type, const uint32_t* qs, const uint32_t* d,
+                     const uint32_t* sc, int row, int stride, const float* x, int nrows, int k, int ntok) {
+    if (!c) return JL_ERR_ARG;
+    std::lock_guard<std::mutex> lock(c->mu);
+    const PlaneRef host = {qs, d, sc, row, stride};
+    const TypeInfo* ti = nullptr;
+    int rc = packed_check(c, type, host, nrows, k, &ti);
+    if (rc != JL_OK) return rc;
+    if (!out || !x || ntok <= 0) return fail(c, JL_ERR_ARG, "packed matmul: bad operand");
+    size_t nq, nd, nsc;
+    if (!packed_words(type, (size_t)stride, k, &nq, &nd, &nsc)) return JL_DECLINED;
+    HIP_TRY(c, H->SetDevice(c->device));
+    // the three planes live in one device allocation keyed on the QS pointer
+    auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
+    const size_t o_d = up(nq * 4), o_sc = o_d + up(nd * 4), total = o_sc + up(nsc * 4);
+    void* dev = nullptr;
+    auto it = c->resident.find(qs);
+    if (it != c->resident.end() && it->second.bytes == total) {
+        dev = it->second.dev;
+    } else {
+        if (it != c->resident.end()) {
+            HIP_TRY(c, H->Free(it->second.dev));
+            c->resident.erase(it);
+        }
+        HIP_TRY(c, H->Malloc(&dev, total));
+        hipError_t e = H->Memcpy(dev, qs, nq * 4, hipMemcpyHostToDevice);
+        if (e == hipSuccess) e = H->Memcpy((char*)dev + o_d, d, nd * 4, hipMemcpyHostToDevice);
+        if (e == hipSuccess && nsc) e = H->Memcpy((char*)dev + o_sc, sc, nsc * 4, hipMemcpyHostToDevice);
+        if (e != hipSuccess) {
+            (void)H->Free(dev);
+            return fail(c, JL_ERR_HIP, "plane upload: %s", H->GetErrorString(e));
+        }
+        c->resident[qs] = Resident{dev, total};
+    }
+    const PlaneRef pl = {(const uint32_t*)dev, (const uint32_t*)((char*)dev + o_d),
+                         (const uint32_t*)((char*)dev + o_sc), row, stride};
+    size_t xb = (size_t)ntok * k * 4, ob = (size_t)ntok * nrows * 4;
+    if ((rc = ensure_stage(c, &c->stage_x, &c->stage_x_bytes, xb)) != JL_OK) return rc;
+    if ((rc = ensure_stage(c, &c->stage_out, &c->stage_out_bytes, ob)) != JL_OK) return rc;
+    HIP_TRY(c, H->MemcpyAsync(c->stage_x, x, xb, hipMemcpyHostToDevice, c->stream));
+    rc = ntok == 1 ? packed_matvec_launch(c, (float*)c->stage_out, type, pl, (const float*)c->stage_x, nullptr,
+                                          nullptr, nullptr, nrows, k, c->stream)
+                   : packed_matmul_launch(c, (float*)c->stage_out, type, pl, (const float*)c->stage_x, nrows, k,
+                                          ntok, c->stream);
     if (rc != JL_OK) {
         (void)H->StreamSynchronize(c->stream);
         return rc;

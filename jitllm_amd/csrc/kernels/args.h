@@ -75,3 +75,34 @@ struct MxGemmArgs {
     int nrows, k, ntok;
     int row_bytes;
 };
+
+// GGUF row-major blocks -> the reference's device planes (and back, for Q4_K).
+struct PackArgs {
+    const uint8_t* src;   // [nrows][k / block] GGUF blocks
+    uint32_t* qs;
+    uint32_t* d;
+    uint32_t* sc;         // null for formats without a scale plane
+    int nrows, k, type;
+};
+
+struct UnpackArgs {
+    uint8_t* dst;         // [nrows][k/256] Q4_K super-blocks
+    const uint32_t* qs;
+    const uint32_t* d;
+    const uint32_t* sc;
+    int nrows, k, row0, stride;
+};
+
+// Decode matvec over the planes: rows row0 .. row0+nrows of a buffer of `stride` rows.
+struct PackedMatVecArgs {
+    float* out;           // [nrows]
+    const uint32_t* qs;
+    const uint32_t* d;
+    const uint32_t* sc;
+    const float* x;       // f32 activations (fused quantize) or null
+    const int8_t* q;      // pre-quantized activations or null
+    const float* as;
+    const float* s16;
+    int nrows, k, row0, stride;
+    int per;              // activation window / 32
+};

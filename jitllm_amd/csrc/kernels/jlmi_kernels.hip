@@ -8,6 +8,7 @@
 #include "matvec.h"
 #include "moe.h"
 #include "mxfp4.h"
+#include "packed.h"
 #include "quantize.h"
 
 extern __shared__ __attribute__((aligned(16))) uint8_t jl_smem[];
@@ -51,6 +52,19 @@ extern "C" __global__ __launch_bounds__(256) void jl_dequant(
 JL_MATVEC_KERNEL(q4k, JL_Q4_K, 1, 1024) JL_MATVEC_KERNEL(q4k, JL_Q4_K, 2, 1024) JL_MATVEC_KERNEL(q4k, JL_Q4_K, 4, 512)
 JL_MATVEC_KERNEL(q8_0, JL_Q8_0, 1, 1024) JL_MATVEC_KERNEL(q8_0, JL_Q8_0, 2, 1024) JL_MATVEC_KERNEL(q8_0, JL_Q8_0, 4, 1024)
 JL_MATVEC_KERNEL(q6k, JL_Q6_K, 1, 1024) JL_MATVEC_KERNEL(q6k, JL_Q6_K, 2, 512) JL_MATVEC_KERNEL(q6k, JL_Q6_K, 4, 512)
+
+// ---------------------------------------------------------- packed planes
+// grid = (ceil(nrows/256), k/256 or k/32 for Q8_0), block = 256
+extern "C" __global__ __launch_bounds__(256) void jl_pack_weights(PackArgs p) { pack_weights_body(p); }
+extern "C" __global__ __launch_bounds__(256) void jl_unpack_q4k(UnpackArgs p) { unpack_q4k_body(p); }
+// jl_matvec_packed_<type>_w<rows per wavefront>: grid = ceil(nrows/RW), block = 64..1024
+#define JL_PACKED_KERNEL(T, TYPE, RW)                                                                     \
+    extern "C" __global__ __launch_bounds__(1024) void jl_matvec_packed_##T##_w##RW(PackedMatVecArgs p) { \
+        packed_matvec_body<TYPE, RW>(p, jl_smem);                                                         \
+    }
+JL_PACKED_KERNEL(q4k, JL_Q4_K, 64) JL_PACKED_KERNEL(q4k, JL_Q4_K, 32) JL_PACKED_KERNEL(q4k, JL_Q4_K, 16)
+JL_PACKED_KERNEL(q8_0, JL_Q8_0, 64) JL_PACKED_KERNEL(q8_0, JL_Q8_0, 32) JL_PACKED_KERNEL(q8_0, JL_Q8_0, 16)
+JL_PACKED_KERNEL(q6k, JL_Q6_K, 64) JL_PACKED_KERNEL(q6k, JL_Q6_K, 32) JL_PACKED_KERNEL(q6k, JL_Q6_K, 16)
 
 // ------------------------------------------------------------ prefill GEMM
 // grid = (k/256, tok_pad/4), block = 256: one wavefront per (token, super-block)

@@ -1,0 +1,387 @@
+// The reference's device weight layout ("packed planes") and the decode matvec
+// over it.
+//
+// Layout (jit/gpu/kernels/pack.go:52-386, matvec.go:137-166, scstream.go:8-42):
+// three planes of u32 words, each [unit][row] with the row index fastest, so the
+// word a row needs for one unit sits beside the same word of the next row:
+//   QS  per sub-block `pw` primary words (4-bit: byte b of word w = element 4w+b
+//       in the low nibble and element 4w+b+sub/2 in the high nibble; 8-bit: raw
+//       bytes), then `hw` secondary words (Q6_K: byte j holds the top two bits of
+//       elements j, 4+j, 8+j, 12+j at bits 0,2,4,6);
+//   D   one word per (super-block, row) = d | dmin<<16 for the k-quants; Q8_0
+//       keeps two rows' f16 in one word (index super*ceil(rows/2) + row/2);
+//   SC  Q4_K: three words per (super-block, row) holding sixteen 6-bit fields
+//       sc0,m0,sc1,m1,... as one 96-bit little-endian stream; Q6_K: one byte
+//       per 16-element sub-block, int8 scale + 128, four to a word.
+// A matrix may be a row range of a larger buffer: `stride` is the buffer's row
+// count and `row0` the first row (engine/nn/device.go:70-80).
+//
+// The matvec puts rows on lanes: a wavefront takes RW rows (64, 32 or 16) and one
+// 256-element chunk of k at a time, the 64/RW lane groups splitting the chunk's
+// sub-blocks, so every load is a run of RW consecutive words and no cross-lane
+// reduction is needed for the dot products.  Each wavefront quantizes just its
+// own 256 activations (a whole quantization window) into a private corner of LDS
+// while its weight loads are in flight; the only workgroup barrier is the one
+// before the final sum over the wavefronts' partial results.
+#pragma once
+#include "args.h"
+#include "common.h"
+#include "quantize.h"
+
+#pragma clang fp contract(off)
+
+// ------------------------------------------------------------------ pack
+// One thread per (row, super-block); Q8_0's "super-block" is its 32-element block.
+// grid = (ceil(nrows/256), k/unit), block = 256.
+
+__device__ __forceinline__ void sc_stream_put(u32 ws[3], int field, u32 v) {
+    const int bit = field * 6, w = bit >> 5, b = bit & 31;
+    ws[w] |= v << b;
+    if (b > 26) ws[w + 1] |= v >> (32 - b);
+}
+
+__device__ __forceinline__ void pack_q4k(const PackArgs& p, int r, int sb) {
+    const int nsb = p.k / 256;
+    const u32* blk = (const u32*)(p.src + ((size_t)r * nsb + sb) * 144);
+    const size_t n = (size_t)p.nrows;
+    p.d[(size_t)sb * n + r] = blk[0];
+    const u32 s0 = blk[1], s1 = blk[2], s2 = blk[3];
+    u32 ws[3] = {0u, 0u, 0u};
+#pragma unroll
+    for (int s = 0; s < 8; s++) {
+        u32 sc, m;
+        scale_min_k4(s, s0, s1, s2, sc, m);
+        sc_stream_put(ws, 2 * s, sc);
+        sc_stream_put(ws, 2 * s + 1, m);
+    }
+#pragma unroll
+    for (int w = 0; w < 3; w++) p.sc[((size_t)sb * 3 + w) * n + r] = ws[w];
+    const u32 M = 0x0F0F0F0Fu;
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+        u32 G[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) G[j] = blk[4 + g * 8 + j];
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            const size_t even = ((size_t)(sb * 8 + 2 * g) * 4 + w) * n + r;
+            const size_t odd = ((size_t)(sb * 8 + 2 * g + 1) * 4 + w) * n + r;
+            p.qs[even] = (G[w] & M) | ((G[w + 4] & M) << 4);
+            p.qs[odd] = ((G[w] >> 4) & M) | (G[w + 4] & ~M);
+        }
+    }
+}
+
+__device__ __forceinline__ void pack_q6k(const PackArgs& p, int r, int sb) {
+    const int nsb = p.k / 256;
+    const uint8_t* blk = p.src + ((size_t)r * nsb + sb) * 210;
+    const size_t n = (size_t)p.nrows;
+    p.d[(size_t)sb * n + r] = (u32)ld2(blk + 208);
+    for (int j = 0; j < 4; j++) {
+        u32 v = 0;
+        for (int b = 0; b < 4; b++) v |= (u32)(uint8_t)((int)(int8_t)blk[192 + 4 * j + b] + 128) << (8 * b);
+        p.sc[((size_t)sb * 4 + j) * n + r] = v;
+    }
+    for (int s = 0; s < 16; s++) {
+        const int half = s >> 3, grp = (s & 7) >> 1, run = s & 1;
+        const uint8_t* ql = blk + half * 64 + (grp & 1) * 32 + run * 16;
+        const uint8_t* qh = blk + 128 + half * 32 + run * 16;
+        uint8_t nib[16], top[16];
+        for (int l = 0; l < 16; l++) {
+            nib[l] = grp >= 2 ? (uint8_t)(ql[l] >> 4) : (uint8_t)(ql[l] & 0xF);
+            top[l] = (uint8_t)((qh[l] >> (2 * grp)) & 3);
+        }
+        u32 w0 = 0, w1 = 0, h = 0;
+        for (int j = 0; j < 4; j++) {
+            w0 |= (u32)(nib[j] | (nib[j + 8] << 4)) << (8 * j);
+            w1 |= (u32)(nib[4 + j] | (nib[12 + j] << 4)) << (8 * j);
+            h |= (u32)(top[j] | (top[4 + j] << 2) | (top[8 + j] << 4) | (top[12 + j] << 6)) << (8 * j);
+        }
+        const size_t base = ((size_t)(sb * 16 + s) * 3) * n + r;
+        p.qs[base] = w0;
+        p.qs[base + n] = w1;
+        p.qs[base + 2 * n] = h;
+    }
+}
+
+__device__ __forceinline__ void pack_q8_0(const PackArgs& p, int r, int b) {
+    const int nb = p.k / 32;
+    const uint8_t* blk = p.src + ((size_t)r * nb + b) * 34;
+    const size_t n = (size_t)p.nrows;
+#pragma unroll
+    for (int w = 0; w < 8; w++) p.qs[((size_t)b * 8 + w) * n + r] = ld4_a2(blk + 2 + 4 * w);
+    if ((r & 1) == 0) {  // two rows share a word of the D plane
+        u32 v = (u32)ld2(blk);
+        if (r + 1 < p.nrows) v |= (u32)ld2(blk + (size_t)nb * 34) << 16;
+        p.d[(size_t)b * ((n + 1) / 2) + (r >> 1)] = v;
+    }
+}
+
+__device__ __forceinline__ void pack_weights_body(const PackArgs& p) {
+    const int r = blockIdx.x * 256 + threadIdx.x, u = blockIdx.y;
+    if (r >= p.nrows) return;
+    if (p.type == JL_Q4_K) pack_q4k(p, r, u);
+    else if (p.type == JL_Q6_K) pack_q6k(p, r, u);
+    else pack_q8_0(p, r, u);
+}
+
+// The inverse for Q4_K: planes (row range row0.. of a buffer of `stride` rows) back
+// to GGUF row-major super-blocks, bit for bit.  The 12 scale bytes are the sixteen
+// 6-bit values in ggml's arrangement (format/quant/dequant.go:360-365).
+__device__ __forceinline__ void unpack_q4k_body(const UnpackArgs& p) {
+    const int rl = blockIdx.x * 256 + threadIdx.x, sb = blockIdx.y;
+    if (rl >= p.nrows) return;
+    const size_t n = (size_t)p.stride, r = (size_t)p.row0 + rl;
+    const int nsb = p.k / 256;
+    u32* blk = (u32*)(p.dst + ((size_t)rl * nsb + sb) * 144);
+    blk[0] = p.d[(size_t)sb * n + r];
+    u32 ws[3];
+#pragma unroll
+    for (int w = 0; w < 3; w++) ws[w] = p.sc[((size_t)sb * 3 + w) * n + r];
+    const uint64_t lo = ws[0] | ((uint64_t)ws[1] << 32), hi = ws[1] | ((uint64_t)ws[2] << 32);
+    u32 sc[8], m[8];
+#pragma unroll
+    for (int s = 0; s < 8; s++) {
+        const int bit = 12 * s;
+        const u32 f = bit < 32 ? (u32)(lo >> bit) : (u32)(hi >> (bit - 32));
+        sc[s] = f & 63;
+        m[s] = (f >> 6) & 63;
+    }
+    u32 s0 = 0, s1 = 0, s2 = 0;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        s0 |= (sc[j] | ((sc[j + 4] >> 4) << 6)) << (8 * j);
+        s1 |= (m[j] | ((m[j + 4] >> 4) << 6)) << (8 * j);
+        s2 |= ((sc[j + 4] & 0xF) | ((m[j + 4] & 0xF) << 4)) << (8 * j);
+    }
+    blk[1] = s0; blk[2] = s1; blk[3] = s2;
+    const u32 M = 0x0F0F0F0Fu;
+#pragma unroll
+    for (int g = 0; g < 4; g++)
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            const u32 e = p.qs[((size_t)(sb * 8 + 2 * g) * 4 + w) * n + r];
+            const u32 o = p.qs[((size_t)(sb * 8 + 2 * g + 1) * 4 + w) * n + r];
+            blk[4 + g * 8 + w] = (e & M) | ((o & M) << 4);
+            blk[4 + g * 8 + 4 + w] = ((e >> 4) & M) | (o & ~M);
+        }
+}
+
+// ---------------------------------------------------------------- matvec
+
+// A wavefront's private LDS: 256 int8 activations, 8 scales, 16 half-block sums.
+#define JL_PK_WAVE_LDS 384
+// Dynamic LDS of a workgroup of `nw` wavefronts: the private areas, then the
+// partial sums [nw][64].
+#define JL_PK_LDS_BYTES(nw) ((nw) * (JL_PK_WAVE_LDS + 256))
+
+struct PkAct {
+    const u32x4* a;    // int8 activations of the chunk, 16 per vector
+    const float* da;   // [8]
+    const float* ss;   // [16]
+};
+
+// NB = 32-element blocks of the chunk one lane covers (8, 4 or 2).
+template <int NB> struct PkWQ4K { u32 q[NB][4]; u32 d; u32 sc[3]; };
+template <int NB> struct PkWQ8 { u32 q[NB][8]; u32 d[NB]; };
+template <int NB> struct PkWQ6K { u32 q[2 * NB][3]; u32 sc[(2 * NB + 3) / 4]; u32 d; };
+
+template <int NB>
+__device__ __forceinline__ void pk_load(const PackedMatVecArgs& p, int c, int b0, int row, PkWQ4K<NB>& w) {
+    const size_t st = (size_t)p.stride;
+    w.d = p.d[(size_t)c * st + row];
+#pragma unroll
+    for (int j = 0; j < 3; j++) w.sc[j] = p.sc[((size_t)c * 3 + j) * st + row];
+    const u32* qs = p.qs + (size_t)(c * 8 + b0) * 4 * st + row;
+#pragma unroll
+    for (int i = 0; i < NB; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) w.q[i][j] = qs[(size_t)(i * 4 + j) * st];
+}
+
+template <int NB>
+__device__ __forceinline__ float pk_dot(const PackedMatVecArgs&, const PkWQ4K<NB>& w, int, int b0, int,
+                                        const PkAct& A) {
+    const u32 M = 0x0F0F0F0Fu;
+    const float d = half_bits_to_f32((uint16_t)(w.d & 0xFFFF));
+    const float dmin = half_bits_to_f32((uint16_t)(w.d >> 16));
+    const uint64_t lo = w.sc[0] | ((uint64_t)w.sc[1] << 32), hi = w.sc[1] | ((uint64_t)w.sc[2] << 32);
+    float acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < NB; i++) {
+        const int s = b0 + i, bit = 12 * s;
+        const u32 f = bit < 32 ? (u32)(lo >> bit) : (u32)(hi >> (bit - 32));
+        const u32 sc = f & 63, m = (f >> 6) & 63;
+        const u32x4 a0 = A.a[2 * s], a1 = A.a[2 * s + 1];
+        i32 dt = dot4(w.q[i][0] & M, a0.x, 0);
+        dt = dot4(w.q[i][1] & M, a0.y, dt);
+        dt = dot4(w.q[i][2] & M, a0.z, dt);
+        dt = dot4(w.q[i][3] & M, a0.w, dt);
+        dt = dot4((w.q[i][0] >> 4) & M, a1.x, dt);
+        dt = dot4((w.q[i][1] >> 4) & M, a1.y, dt);
+        dt = dot4((w.q[i][2] >> 4) & M, a1.z, dt);
+        dt = dot4((w.q[i][3] >> 4) & M, a1.w, dt);
+        const float sa = A.ss[2 * s] + A.ss[2 * s + 1];
+        const float v = (float)dt * (d * (float)sc) - sa * (dmin * (float)m);
+        acc = fmaf(v, A.da[s], acc);
+    }
+    return acc;
+}
+
+template <int NB>
+__device__ __forceinline__ void pk_load(const PackedMatVecArgs& p, int c, int b0, int row, PkWQ8<NB>& w) {
+    const size_t st = (size_t)p.stride, dst = (st + 1) / 2;
+    const int nb = p.k / 32;
+#pragma unroll
+    for (int i = 0; i < NB; i++) {
+        const int B = min(c * 8 + b0 + i, nb - 1);
+        w.d[i] = p.d[(size_t)B * dst + (row >> 1)];
+        const u32* qs = p.qs + (size_t)B * 8 * st + row;
+#pragma unroll
+        for (int j = 0; j < 8; j++) w.q[i][j] = qs[(size_t)j * st];
+    }
+}
+
+template <int NB>
+__device__ __forceinline__ float pk_dot(const PackedMatVecArgs& p, const PkWQ8<NB>& w, int c, int b0, int row,
+                                        const PkAct& A) {
+    const int nb = p.k / 32;
+    float acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < NB; i++) {
+        const int s = b0 + i;
+        const u32x4 a0 = A.a[2 * s], a1 = A.a[2 * s + 1];
+        i32 dt = dot4(w.q[i][0], a0.x, 0);
+        dt = dot4(w.q[i][1], a0.y, dt);
+        dt = dot4(w.q[i][2], a0.z, dt);
+        dt = dot4(w.q[i][3], a0.w, dt);
+        dt = dot4(w.q[i][4], a1.x, dt);
+        dt = dot4(w.q[i][5], a1.y, dt);
+        dt = dot4(w.q[i][6], a1.z, dt);
+        dt = dot4(w.q[i][7], a1.w, dt);
+        const float d = half_bits_to_f32((uint16_t)(w.d[i] >> (16 * (row & 1))));
+        const float v = (float)dt * d * A.da[s];
+        if (c * 8 + s < nb) acc += v;   // a short last chunk has fewer blocks
+    }
+    return acc;
+}
+
+template <int NB>
+__device__ __forceinline__ void pk_load(const PackedMatVecArgs& p, int c, int b0, int row, PkWQ6K<NB>& w) {
+    const size_t st = (size_t)p.stride;
+    const int s0 = 2 * b0;   // first 16-element sub-block of this lane's share
+    w.d = p.d[(size_t)c * st + row];
+#pragma unroll
+    for (int j = 0; j < (2 * NB + 3) / 4; j++) w.sc[j] = p.sc[((size_t)(c * 16 + s0) / 4 + j) * st + row];
+    const u32* qs = p.qs + (size_t)(c * 16 + s0) * 3 * st + row;
+#pragma unroll
+    for (int i = 0; i < 2 * NB; i++)
+#pragma unroll
+        for (int j = 0; j < 3; j++) w.q[i][j] = qs[(size_t)(i * 3 + j) * st];
+}
+
+template <int NB>
+__device__ __forceinline__ float pk_dot(const PackedMatVecArgs&, const PkWQ6K<NB>& w, int, int b0, int,
+                                        const PkAct& A) {
+    const u32 M4 = 0x0F0F0F0Fu, M2 = 0x30303030u;
+    const float d = half_bits_to_f32((uint16_t)(w.d & 0xFFFF));
+    float acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < 2 * NB; i++) {
+        const int s = 2 * b0 + i;
+        const u32x4 a = A.a[s];
+        const u32 w0 = w.q[i][0], w1 = w.q[i][1], h = w.q[i][2];
+        i32 dt = dot4((w0 & M4) | ((h << 4) & M2), a.x, 0);
+        dt = dot4((w1 & M4) | ((h << 2) & M2), a.y, dt);
+        dt = dot4(((w0 >> 4) & M4) | (h & M2), a.z, dt);
+        dt = dot4(((w1 >> 4) & M4) | ((h >> 2) & M2), a.w, dt);
+        // value = d*sc*(q-32): the zero point goes through the activation sum
+        const float t = (float)dt - 32.f * A.ss[s];
+        const i32 sc = (i32)((w.sc[i >> 2] >> (8 * (i & 3))) & 0xFF) - 128;
+        acc = fmaf(t * (d * (float)sc), A.da[s >> 1], acc);
+    }
+    return acc;
+}
+
+template <int TYPE, int NB> struct PkTraits;
+template <int NB> struct PkTraits<JL_Q4_K, NB> { typedef PkWQ4K<NB> W; };
+template <int NB> struct PkTraits<JL_Q8_0, NB> { typedef PkWQ8<NB> W; };
+template <int NB> struct PkTraits<JL_Q6_K, NB> { typedef PkWQ6K<NB> W; };
+
+// grid = ceil(nrows / RW) workgroups of 64..1024 threads; dynamic LDS =
+// JL_PK_LDS_BYTES(wavefronts).  Needs k % 32 == 0 (k % 256 == 0 for the k-quants).
+template <int TYPE, int RW>
+__device__ __forceinline__ void packed_matvec_body(const PackedMatVecArgs& p, uint8_t* smem) {
+    constexpr int KP = 64 / RW, NB = 8 / KP;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+    // Workgroups are dealt to the eight XCDs round robin; give each XCD a contiguous
+    // range of row groups so neighbouring row runs meet in one L2.
+    int g = blockIdx.x;
+    const int ng = gridDim.x;
+    if ((ng & 7) == 0) g = (g & 7) * (ng >> 3) + (g >> 3);
+    const int rl = lane % RW, part = lane / RW, b0 = part * NB;
+    const int row = p.row0 + min(g * RW + rl, p.nrows - 1);
+
+    uint8_t* my = smem + wave * JL_PK_WAVE_LDS;
+    u32* a_w = (u32*)my;
+    float* da_w = (float*)(my + 256);
+    float* ss_w = (float*)(my + 288);
+    PkAct A;
+    A.a = (const u32x4*)my;
+    A.da = da_w;
+    A.ss = ss_w;
+
+    const int n4 = p.k / 4, nchunks = (p.k + 255) / 256;
+    float acc = 0.f;
+    for (int c = wave; c < nchunks; c += nwaves) {
+        // activation of this chunk first: loads come back in order
+        const int g4 = c * 64 + lane;
+        f32x4 xv = f32x4{0.f, 0.f, 0.f, 0.f};
+        u32 qv = 0;
+        float dv = 0.f, sv = 0.f;
+        if (p.x) {
+            if (g4 < n4) xv = ((const f32x4*)p.x)[g4];
+        } else {
+            if (g4 < n4) qv = ((const u32*)p.q)[g4];
+            if (lane < 8 && c * 8 + lane < p.k / 32) dv = p.as[c * 8 + lane];
+            if (lane < 16 && c * 16 + lane < p.k / 16) sv = p.s16[c * 16 + lane];
+        }
+        typename PkTraits<TYPE, NB>::W w;
+        pk_load<NB>(p, c, b0, row, w);
+
+        if (p.x) {
+            u32 m = max(max(abs_bits(xv.x), abs_bits(xv.y)), max(abs_bits(xv.z), abs_bits(xv.w)));
+            u32 amax = window_amax(m, p.per);
+            float d;
+            i32 sum;
+            qv = quantize4(xv, amax, d, sum);
+            a_w[lane] = qv;
+            if ((lane & 3) == 0) ss_w[lane >> 2] = (float)sum;
+            if ((lane & 7) == 0) da_w[lane >> 3] = d;
+        } else {
+            a_w[lane] = qv;
+            if (lane < 8) da_w[lane] = dv;
+            if (lane < 16) ss_w[lane] = sv;
+        }
+        // The area is private to this wavefront, whose LDS operations complete in
+        // order: only the compiler has to be kept from moving reads above the writes.
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        acc += pk_dot<NB>(p, w, c, b0, row, A);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    }
+
+    float* red = (float*)(smem + nwaves * JL_PK_WAVE_LDS);
+    red[wave * 64 + lane] = acc;
+    __syncthreads();
+    if ((int)threadIdx.x < RW) {
+        float t = 0.f;
+        for (int wv = 0; wv < nwaves; wv++)
+#pragma unroll
+            for (int q = 0; q < KP; q++) t += red[wv * 64 + q * RW + threadIdx.x];
+        const int r = g * RW + threadIdx.x;
+        if (r < p.nrows) p.out[r] = t;
+    }
+}

@@ -25,6 +25,18 @@ def _ptr(a):
     return int(a)
 
 
+def _opt(a):
+    return None if a is None else _ptr(a)
+
+
+class Packed:
+    """nn.Packed (/root/reference/engine/nn/device.go:70-80): the three planes of a weight,
+    and which rows of them a matrix is.  Planes are numpy uint32 arrays or device addresses."""
+
+    def __init__(self, qs, d, sc, row=0, stride=0):
+        self.qs, self.d, self.sc, self.row, self.stride = qs, d, sc, row, stride
+
+
 class Device:
     def __init__(self, device=0, act_window=32, code_object=None):
         self._l = _lib.load()
@@ -102,7 +114,57 @@ class Device:
         """nn.CopyForgetter.Forget: drop the device copy keyed on this host buffer."""
         self._served(self._l.jl_forget(self._ctx, _ptr(w), w.nbytes), "jl_forget")
 
+    # -- packed planes, host pointers -----------------------------------------
+    def packed_words(self, t, nrows, k):
+        """kernels.PackedWords: (QS, D, SC) plane sizes in u32 words, or None if undefined."""
+        nq, nd, nsc = C.c_size_t(), C.c_size_t(), C.c_size_t()
+        rc = self._l.jl_packed_words(t, nrows, k, C.byref(nq), C.byref(nd), C.byref(nsc))
+        return (nq.value, nd.value, nsc.value) if rc == _lib.OK else None
+
+    def MatVecPacked(self, out, t, p, x, nrows, k):
+        """JIT.MatVecPacked (/root/reference/engine/nn/packed.go:24); p = Packed(qs, d, sc, row, stride)."""
+        assert out.dtype == np.float32 and x.dtype == np.float32
+        return self._served(self._l.jl_matvec_packed(self._ctx, _ptr(out), t, _ptr(p.qs), _ptr(p.d),
+                                                     _opt(p.sc), p.row, p.stride, _ptr(x), nrows, k),
+                            "jl_matvec_packed")
+
+    def MatMulPacked(self, out, t, p, x, nrows, k, ntok):
+        """JIT.MatMulPacked (/root/reference/engine/nn/packedmm.go:23)."""
+        assert out.dtype == np.float32 and x.dtype == np.float32
+        return self._served(self._l.jl_matmul_packed(self._ctx, _ptr(out), t, _ptr(p.qs), _ptr(p.d),
+                                                     _opt(p.sc), p.row, p.stride, _ptr(x), nrows, k, ntok),
+                            "jl_matmul_packed")
+
+    def ForgetPacked(self, p):
+        self._served(self._l.jl_forget(self._ctx, _ptr(p.qs), 4), "jl_forget")
+
     # -- device-pointer entry points ------------------------------------------
+    def pack_weights_dev(self, t, src, nrows, k, qs, d, sc, stream=None):
+        """kernels.PackWeightsInto on the device: GGUF rows -> planes."""
+        return self._served(self._l.jl_pack_weights_dev(self._ctx, t, _ptr(src), nrows, k, _ptr(qs), _ptr(d),
+                                                        _opt(sc), stream), "jl_pack_weights_dev")
+
+    def unpack_weights_dev(self, t, p, nrows, k, dst, stream=None):
+        return self._served(self._l.jl_unpack_weights_dev(self._ctx, t, _ptr(p.qs), _ptr(p.d), _opt(p.sc),
+                                                          p.row, p.stride, nrows, k, _ptr(dst), stream),
+                            "jl_unpack_weights_dev")
+
+    def matvec_packed_dev(self, out, t, p, x, nrows, k, stream=None):
+        return self._served(self._l.jl_matvec_packed_dev(self._ctx, _ptr(out), t, _ptr(p.qs), _ptr(p.d),
+                                                         _opt(p.sc), p.row, p.stride, _ptr(x), nrows, k,
+                                                         stream), "jl_matvec_packed_dev")
+
+    def matvec_packed_q8_dev(self, out, t, p, q, a_s, sum16, nrows, k, stream=None):
+        return self._served(self._l.jl_matvec_packed_q8_dev(self._ctx, _ptr(out), t, _ptr(p.qs), _ptr(p.d),
+                                                            _opt(p.sc), p.row, p.stride, _ptr(q), _ptr(a_s),
+                                                            _ptr(sum16), nrows, k, stream),
+                            "jl_matvec_packed_q8_dev")
+
+    def matmul_packed_dev(self, out, t, p, x, nrows, k, ntok, stream=None):
+        return self._served(self._l.jl_matmul_packed_dev(self._ctx, _ptr(out), t, _ptr(p.qs), _ptr(p.d),
+                                                         _opt(p.sc), p.row, p.stride, _ptr(x), nrows, k,
+                                                         ntok, stream), "jl_matmul_packed_dev")
+
     def quantize_act_dev(self, x, ntok, k, q, a_s, sum16, stream=None):
         return self._served(self._l.jl_quantize_act_dev(self._ctx, _ptr(x), ntok, k, _ptr(q),
                                                         _ptr(a_s), _ptr(sum16), stream),

@@ -1,0 +1,264 @@
+"""GPU parity of the packed-plane path (the reference's device weight layout) against
+the CPU oracle, through the C ABI.
+
+Bars:
+  * device pack (kernels.PackWeightsInto, /root/reference/jit/gpu/kernels/pack.go:52-199):
+    byte for byte the oracle's planes, which the reference-written v29 container pins
+    for Q4_K; the inverse permutation restores the GGUF bytes exactly
+  * matvec / matmul over planes vs the f64 evaluation of the same int8 activations:
+    NMSE <= 1e-10 (/root/reference/engine/nn/packed_test.go:140-147), rel-L2 <= 1e-3
+  * planes of the reference-written container (tests/golden/v29.jlm.gz) fed straight to
+    the kernel, expert sheets included
+"""
+import gzip
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+from conftest import GOLDEN, nmse, rel_l2
+from jitllm_amd import jlm, quant, synth
+from jitllm_amd.device import Packed
+
+pytestmark = pytest.mark.gpu
+
+TYPES = [quant.Q4_K, quant.Q8_0, quant.Q6_K]
+
+
+def _window(t):
+    return 256 if t in quant.K_QUANTS else 32
+
+
+def _like_for_like(t, w, x, nrows, k, window):
+    q, a_s, _ = oracle.quantize_act(x, window)
+    return oracle.matvec_q8act_f64(t, w, q, a_s, nrows, k)
+
+
+def _dev_planes(devbuf, qs, d, sc, row=0, stride=None):
+    qd, dd = devbuf(qs), devbuf(d)
+    sd = devbuf(sc) if sc is not None and sc.size else None
+    p = Packed(qd.ptr, dd.ptr, sd.ptr if sd else None, row, stride)
+    p.keep = (qd, dd, sd)
+    return p
+
+
+@pytest.mark.parametrize("t", TYPES)
+@pytest.mark.parametrize("shape", [(1, 256), (9, 512), (300, 512), (257, 1024), (64, 4096)],
+                         ids=lambda s: f"{s[0]}x{s[1]}")
+def test_pack_on_device_is_byte_exact(dev, devbuf, t, shape):
+    nrows, k = shape
+    src = synth.random_weights(t, nrows, k, seed=nrows * 7 + k)
+    wq, wd, wsc = oracle.pack_weights(t, src, nrows, k)
+    assert dev.packed_words(t, nrows, k) == (wq.size, wd.size, wsc.size)
+    sd = devbuf(src)
+    qs = devbuf(shape=(wq.size,), dtype=np.uint32, fill=0xDEADBEEF)
+    d = devbuf(shape=(wd.size,), dtype=np.uint32, fill=0xDEADBEEF)
+    sc = devbuf(shape=(max(wsc.size, 1),), dtype=np.uint32, fill=0xDEADBEEF)
+    assert dev.pack_weights_dev(t, sd.ptr, nrows, k, qs.ptr, d.ptr, sc.ptr if wsc.size else None)
+    dev.synchronize()
+    assert np.array_equal(qs.get(), wq)
+    assert np.array_equal(d.get(), wd)
+    if wsc.size:
+        assert np.array_equal(sc.get(), wsc)
+    if t == quant.Q4_K:
+        back = devbuf(shape=(src.size,), dtype=np.uint8, fill=0x5A)
+        assert dev.unpack_weights_dev(t, Packed(qs.ptr, d.ptr, sc.ptr, 0, nrows), nrows, k, back.ptr)
+        dev.synchronize()
+        assert np.array_equal(back.get(), src)
+
+
+def test_packed_words_closed_form(dev):
+    """kernels.PackedWords (/root/reference/jit/gpu/kernels/pack.go:580-621) against the oracle's."""
+    for t in TYPES:
+        for nrows, k in [(1, 256), (7, 512), (300, 4096), (4096, 14336)]:
+            assert dev.packed_words(t, nrows, k) == tuple(oracle.packed_words(t, nrows, k))
+    assert dev.packed_words(quant.Q4_K, 8, 288) is None
+    assert dev.packed_words(quant.Q8_0, 8, 288) is not None
+
+
+SHAPES = [(1, 256), (9, 512), (300, 512), (37, 1024), (64, 2048), (1000, 4096), (129, 14336), (4096, 768)]
+
+
+@pytest.mark.parametrize("t", TYPES)
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: f"{s[0]}x{s[1]}")
+@pytest.mark.parametrize("weights", ["normal", "planted"])
+def test_matvec_packed_vs_oracle(dev, devbuf, t, shape, weights):
+    nrows, k = shape
+    window = _window(t)
+    dev.SetActWindow(window)
+    if weights == "normal":
+        w = synth.quantized_weights(t, nrows, k, seed=nrows + k)
+    else:
+        w = synth.random_weights(t, nrows, k, seed=nrows)
+    x = synth.activations(k, seed=k)
+    want = _like_for_like(t, w, x, nrows, k, window)
+    p = _dev_planes(devbuf, *oracle.pack_weights(t, w, nrows, k), stride=nrows)
+    xd = devbuf(x)
+    for rw in (0, 16, 32, 64):
+        dev.set_tuning(packed__rw=rw)
+        out = devbuf(shape=(nrows + 8,), dtype=np.float32, fill=np.float32(7e30))
+        assert dev.matvec_packed_dev(out.ptr, t, p, xd.ptr, nrows, k)
+        dev.synchronize()
+        got = out.get()
+        assert np.all(got[nrows:] == np.float32(7e30)), "wrote past nrows"
+        e = nmse(got[:nrows], want)
+        assert e <= 1e-10, f"rw={rw}: NMSE {e:.3e} vs like-for-like f64"
+        assert rel_l2(got[:nrows], want) <= 1e-3
+    dev.set_tuning(packed__rw=0)
+    if weights == "normal" and nrows >= 64:
+        ref32 = oracle.matvec_packed_rows(t, *oracle.pack_weights(t, w, nrows, k), x, nrows, k)
+        assert nmse(got[:nrows], ref32) <= 1e-3, "vs the f32-activation plane reader"
+    dev.SetActWindow(32)
+
+
+@pytest.mark.parametrize("t", TYPES)
+def test_matvec_packed_window_32_and_block_shapes(dev, devbuf, t):
+    """The 32 window (one scale per block) and every workgroup size give the same rows."""
+    nrows, k = 203, 2304 if t == quant.Q8_0 else 2048
+    if t == quant.Q8_0:
+        k = 2304 + 32   # not a whole 256-element chunk: the last chunk is short
+    dev.SetActWindow(32)
+    w = synth.random_weights(t, nrows, k, seed=11)
+    x = synth.activations(k, seed=12)
+    want = _like_for_like(t, w, x, nrows, k, 32)
+    p = _dev_planes(devbuf, *oracle.pack_weights(t, w, nrows, k), stride=nrows)
+    xd = devbuf(x)
+    for block in (64, 192, 512, 1024):
+        for rw in (16, 32, 64):
+            dev.set_tuning(packed__rw=rw, packed__block=block)
+            out = devbuf(shape=(nrows,), dtype=np.float32, fill=np.float32(-3e33))
+            assert dev.matvec_packed_dev(out.ptr, t, p, xd.ptr, nrows, k)
+            dev.synchronize()
+            e = nmse(out.get(), want)
+            assert e <= 1e-10, f"block={block} rw={rw}: {e:.3e}"
+    dev.set_tuning(packed__rw=0, packed__block=0)
+
+
+@pytest.mark.parametrize("t", TYPES)
+def test_matvec_packed_row_range_of_a_larger_buffer(dev, devbuf, t):
+    """nn.Packed.Row / Stride: a matrix that is rows 40..140 of planes holding 203 rows."""
+    stride, k, row, nrows = 203, 1024, 41, 100
+    window = _window(t)
+    dev.SetActWindow(window)
+    w = synth.random_weights(t, stride, k, seed=21)
+    x = synth.activations(k, seed=22)
+    want = _like_for_like(t, w, x, stride, k, window)[row:row + nrows]
+    p = _dev_planes(devbuf, *oracle.pack_weights(t, w, stride, k), row=row, stride=stride)
+    xd = devbuf(x)
+    out = devbuf(shape=(nrows,), dtype=np.float32, fill=np.float32(5e30))
+    assert dev.matvec_packed_dev(out.ptr, t, p, xd.ptr, nrows, k)
+    dev.synchronize()
+    assert nmse(out.get(), want) <= 1e-10
+    # rows outside the buffer are a contract violation, not a decline
+    from jitllm_amd.device import DeviceError
+    with pytest.raises(DeviceError):
+        dev.matvec_packed_dev(out.ptr, t, Packed(p.qs, p.d, p.sc, stride - 10, stride), xd.ptr, nrows, k)
+    dev.SetActWindow(32)
+
+
+@pytest.mark.parametrize("t", TYPES)
+def test_matvec_packed_split_equals_fused(dev, devbuf, t):
+    """Quantizer kernel + packed matvec over its output == the fused kernel, bit for bit."""
+    nrows, k, window = 200, 4096, _window(t)
+    dev.SetActWindow(window)
+    w = synth.quantized_weights(t, nrows, k, seed=9)
+    x = synth.activations(k, seed=10)
+    p = _dev_planes(devbuf, *oracle.pack_weights(t, w, nrows, k), stride=nrows)
+    xd = devbuf(x)
+    q = devbuf(shape=(k,), dtype=np.int8)
+    a_s = devbuf(shape=(k // 32,), dtype=np.float32)
+    s16 = devbuf(shape=(k // 16,), dtype=np.float32)
+    o1 = devbuf(shape=(nrows,), dtype=np.float32, fill=1.0)
+    o2 = devbuf(shape=(nrows,), dtype=np.float32, fill=2.0)
+    assert dev.quantize_act_dev(xd.ptr, 1, k, q.ptr, a_s.ptr, s16.ptr)
+    assert dev.matvec_packed_q8_dev(o1.ptr, t, p, q.ptr, a_s.ptr, s16.ptr, nrows, k)
+    assert dev.matvec_packed_dev(o2.ptr, t, p, xd.ptr, nrows, k)
+    dev.synchronize()
+    assert np.array_equal(o1.get().view(np.uint32), o2.get().view(np.uint32))
+    dev.SetActWindow(32)
+
+
+def _container():
+    return jlm.File(gzip.open(os.path.join(GOLDEN, "v29.jlm.gz")).read())
+
+
+def test_container_planes_fed_to_the_kernel(dev, devbuf):
+    """Q4_K planes written by the reference's own converter (format/jlm/testdata/old/v29.jlm.gz),
+    expert sheets included, go to the kernel as they lie in the file."""
+    f = _container()
+    dev.SetActWindow(256)
+    seen = 0
+    for e in f.entries:
+        if jlm.TYPE_TO_QUANT.get(e.type) != quant.Q4_K:
+            continue
+        for sheet in range(e.sheets):
+            _, qs, d, sc = f.planes(e, sheet)
+            rows, k = e.rows, e.k
+            x = synth.activations(k, seed=100 + seen)
+            want = oracle.matvec_packed_rows(quant.Q4_K, qs, d, sc, x, rows, k)
+            p = _dev_planes(devbuf, np.ascontiguousarray(qs), np.ascontiguousarray(d),
+                            np.ascontiguousarray(sc), stride=rows)
+            xd = devbuf(x)
+            out = devbuf(shape=(rows,), dtype=np.float32, fill=np.float32(1e30))
+            assert dev.matvec_packed_dev(out.ptr, quant.Q4_K, p, xd.ptr, rows, k)
+            dev.synchronize()
+            # the plane reader multiplies f32 activations; the kernel quantizes them
+            assert nmse(out.get(), want) <= 2e-3, e.name
+            # like for like: dequantize the planes row by row and evaluate in f64
+            q8, a_s, _ = oracle.quantize_act(x, 256)
+            deq = np.stack([oracle.row_packed(quant.Q4_K, qs, d, sc, r, rows, k) for r in range(rows)])
+            xa = (q8.astype(np.float64).reshape(-1, 32) * a_s.astype(np.float64)[:, None]).reshape(-1)
+            assert nmse(out.get(), deq.astype(np.float64) @ xa) <= 1e-10, e.name
+            seen += 1
+    assert seen >= 3
+    dev.SetActWindow(32)
+
+
+@pytest.mark.parametrize("t", TYPES)
+@pytest.mark.parametrize("ntok", [1, 3, 16, 130])
+def test_matmul_packed_vs_oracle(dev, devbuf, t, ntok):
+    """JIT.MatMulPacked: every token quantized on its own; the GEMM form (Q4_K, 256 window,
+    enough tokens) and the per-token form give the like-for-like values."""
+    nrows, k = 300, 1024
+    window = _window(t)
+    dev.SetActWindow(window)
+    w = synth.quantized_weights(t, nrows, k, seed=31)
+    x = synth.activations(ntok * k, seed=32).reshape(ntok, k)
+    want = oracle.matmul_q8act_f64(t, w, x, nrows, k, ntok, window)
+    p = _dev_planes(devbuf, *oracle.pack_weights(t, w, nrows, k), stride=nrows)
+    xd = devbuf(x)
+    out = devbuf(shape=(ntok, nrows), dtype=np.float32, fill=np.float32(3e30))
+    assert dev.matmul_packed_dev(out.ptr, t, p, xd.ptr, nrows, k, ntok)
+    dev.synchronize()
+    got = out.get()
+    assert nmse(got, want) <= 1e-10
+    assert rel_l2(got, want) <= 1e-3
+    dev.SetActWindow(32)
+
+
+def test_packed_host_pointer_seam(dev):
+    """JIT.MatVecPacked / MatMulPacked over host planes: residency keyed on the QS pointer."""
+    t, nrows, k = quant.Q4_K, 96, 1024
+    dev.SetActWindow(256)
+    w = synth.quantized_weights(t, nrows, k, seed=1)
+    qs, d, sc = oracle.pack_weights(t, w, nrows, k)
+    p = Packed(qs, d, sc, 0, nrows)
+    x = synth.activations(k, seed=2)
+    out = np.full(nrows, np.float32(9e9))
+    assert dev.MatVecPacked(out, t, p, x, nrows, k) is True
+    assert nmse(out, _like_for_like(t, w, x, nrows, k, 256)) <= 1e-10
+    x3 = synth.activations(3 * k, seed=4).reshape(3, k)
+    out3 = np.full((3, nrows), np.float32(9e9))
+    assert dev.MatMulPacked(out3, t, p, x3, nrows, k, 3) is True
+    assert nmse(out3, oracle.matmul_q8act_f64(t, w, x3, nrows, k, 3, 256)) <= 1e-10
+    # a sub-range of the same resident planes
+    sub = Packed(qs, d, sc, 16, nrows)
+    out16 = np.full(32, np.float32(9e9))
+    assert dev.MatVecPacked(out16, t, sub, x, 32, k) is True
+    assert nmse(out16, _like_for_like(t, w, x, nrows, k, 256)[16:48]) <= 1e-10
+    dev.ForgetPacked(p)
+    # declines: a type with no planes here, k that is not whole super-blocks
+    assert dev.MatVecPacked(out, quant.MXFP4, p, x, nrows, k) is False
+    assert dev.MatVecPacked(out, t, p, x, nrows, k - 32) is False
+    dev.SetActWindow(32)
