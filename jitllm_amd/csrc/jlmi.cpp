@@ -192,6 +192,8 @@ int matvec_launch(jl_ctx* c, float* out, int type, const void* w, const float* x
     a.k = k;
     a.row_bytes = (k / ti->block_elems) * ti->block_bytes;
     a.per = c->act_window / 32;
+    a.nwaves = block / 64;
+    a.ngroups = (int)grid;
     char name[64];
     snprintf(name, sizeof name, "jl_matvec_%s_r%d", ti->tag, rpw);
     void* params[] = {&a};
@@ -370,11 +372,12 @@ int packed_matvec_launch(jl_ctx* c, float* out, int type, const PlaneRef& pl, co
     a.out = out; a.qs = pl.qs; a.d = pl.d; a.sc = pl.sc;
     a.x = x; a.q = q; a.as = as; a.s16 = s16;
     a.nrows = nrows; a.k = k; a.row0 = pl.row; a.stride = pl.stride; a.per = c->act_window / 32;
+    a.nwaves = nw; a.ngroups = (nrows + rw - 1) / rw;
     char name[64];
-    snprintf(name, sizeof name, "jl_matvec_packed_%s_w%d", ti->tag, rw);
+    snprintf(name, sizeof name, "jl_matvec_packed_%s%s_w%d", x ? "" : "q8_", ti->tag, rw);
     void* params[] = {&a};
     return launch(c, name, (unsigned)((nrows + rw - 1) / rw), 1, (unsigned)(nw * 64),
-                  (unsigned)(nw * (384 + 256)), st, params);
+                  (unsigned)(nw * (384 + 65 * 4)), st, params);  // JL_PK_LDS_BYTES
 }
 
 int unpack_launch(jl_ctx* c, const PlaneRef& pl, int nrows, int k, void* dst, hipStream_t st) {
@@ -492,7 +495,9 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_q4k", "jl_moe_group", "jl_moe_combine", "jl_mxfp4_gemm", "jl_mxfp4_matvec",
                                       "jl_pack_weights", "jl_unpack_q4k"};
     for (const char* tag : {"q4k", "q8_0", "q6k"})
-        for (int rw : {16, 32, 64}) names.push_back(std::string("jl_matvec_packed_") + tag + "_w" + std::to_string(rw));
+        for (int rw : {16, 32, 64})
+            for (const char* form : {"", "q8_"})
+                names.push_back(std::string("jl_matvec_packed_") + form + tag + "_w" + std::to_string(rw));
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int lpr : {16, 32, 64}) names.push_back(std::string("jl_moe_matvec_") + tag + "_l" + std::to_string(lpr));
     const int types[] = {JL_TYPE_Q4_K, JL_TYPE_Q8_0, JL_TYPE_Q6_K};

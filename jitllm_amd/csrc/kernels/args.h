@@ -14,6 +14,8 @@ struct MatVecArgs {
     int nrows, k;
     int row_bytes;
     int per;             // activation window / 32 (fused form)
+    int nwaves;          // wavefronts per workgroup (the launch's block / 64)
+    int ngroups;         // workgroups (the launch's grid)
 };
 
 // Activation preparation for the Q4_K prefill GEMM: quantize x and lay it out
@@ -105,4 +107,6 @@ struct PackedMatVecArgs {
     const float* s16;
     int nrows, k, row0, stride;
     int per;              // activation window / 32
+    int nwaves;           // wavefronts per workgroup (the launch's block / 64)
+    int ngroups;          // workgroups (the launch's grid)
 };

@@ -58,13 +58,19 @@ JL_MATVEC_KERNEL(q6k, JL_Q6_K, 1, 1024) JL_MATVEC_KERNEL(q6k, JL_Q6_K, 2, 512) J
 extern "C" __global__ __launch_bounds__(256) void jl_pack_weights(PackArgs p) { pack_weights_body(p); }
 extern "C" __global__ __launch_bounds__(256) void jl_unpack_q4k(UnpackArgs p) { unpack_q4k_body(p); }
 // jl_matvec_packed_<type>_w<rows per wavefront>: grid = ceil(nrows/RW), block = 64..1024
-#define JL_PACKED_KERNEL(T, TYPE, RW)                                                                     \
-    extern "C" __global__ __launch_bounds__(1024) void jl_matvec_packed_##T##_w##RW(PackedMatVecArgs p) { \
-        packed_matvec_body<TYPE, RW>(p, jl_smem);                                                         \
+// XPRE = chunks whose activation loads go out ahead of the weights (register budget).
+// jl_matvec_packed_<type>_w<RW> quantizes f32 x itself; jl_matvec_packed_q8_<type>_w<RW>
+// takes activations already quantized.
+#define JL_PACKED_KERNEL(T, TYPE, RW, XPRE)                                                                  \
+    extern "C" __global__ __launch_bounds__(1024) void jl_matvec_packed_##T##_w##RW(PackedMatVecArgs p) {    \
+        packed_matvec_body<TYPE, RW, XPRE, true>(p, jl_smem);                                                \
+    }                                                                                                        \
+    extern "C" __global__ __launch_bounds__(1024) void jl_matvec_packed_q8_##T##_w##RW(PackedMatVecArgs p) { \
+        packed_matvec_body<TYPE, RW, XPRE, false>(p, jl_smem);                                               \
     }
-JL_PACKED_KERNEL(q4k, JL_Q4_K, 64) JL_PACKED_KERNEL(q4k, JL_Q4_K, 32) JL_PACKED_KERNEL(q4k, JL_Q4_K, 16)
-JL_PACKED_KERNEL(q8_0, JL_Q8_0, 64) JL_PACKED_KERNEL(q8_0, JL_Q8_0, 32) JL_PACKED_KERNEL(q8_0, JL_Q8_0, 16)
-JL_PACKED_KERNEL(q6k, JL_Q6_K, 64) JL_PACKED_KERNEL(q6k, JL_Q6_K, 32) JL_PACKED_KERNEL(q6k, JL_Q6_K, 16)
+JL_PACKED_KERNEL(q4k, JL_Q4_K, 64, 4) JL_PACKED_KERNEL(q4k, JL_Q4_K, 32, 4) JL_PACKED_KERNEL(q4k, JL_Q4_K, 16, 4)
+JL_PACKED_KERNEL(q8_0, JL_Q8_0, 64, 2) JL_PACKED_KERNEL(q8_0, JL_Q8_0, 32, 4) JL_PACKED_KERNEL(q8_0, JL_Q8_0, 16, 4)
+JL_PACKED_KERNEL(q6k, JL_Q6_K, 64, 4) JL_PACKED_KERNEL(q6k, JL_Q6_K, 32, 4) JL_PACKED_KERNEL(q6k, JL_Q6_K, 16, 4)
 
 // ------------------------------------------------------------ prefill GEMM
 // grid = (k/256, tok_pad/4), block = 256: one wavefront per (token, super-block)

@@ -42,13 +42,13 @@ __device__ __forceinline__ ActLds act_lds_views(uint8_t* smem, int k) {
 
 // Stage pre-quantized activations (global) into LDS.  k % 32 == 0.
 __device__ __forceinline__ void stage_act_copy(uint8_t* smem, const int8_t* q, const float* as,
-                                               const float* s16, int k) {
+                                               const float* s16, int k, int nthreads) {
     u32* a = (u32*)smem;
     float* da = (float*)(smem + k);
     float* ss = (float*)(smem + k + (k / 32) * 4);
-    for (int i = threadIdx.x; i < k / 4; i += blockDim.x) a[i] = ((const u32*)q)[i];
-    for (int i = threadIdx.x; i < k / 32; i += blockDim.x) da[i] = as[i];
-    for (int i = threadIdx.x; i < k / 16; i += blockDim.x) ss[i] = s16[i];
+    for (int i = threadIdx.x; i < k / 4; i += nthreads) a[i] = ((const u32*)q)[i];
+    for (int i = threadIdx.x; i < k / 32; i += nthreads) da[i] = as[i];
+    for (int i = threadIdx.x; i < k / 16; i += nthreads) ss[i] = s16[i];
 }
 
 // Quantize one float4 of x (element group g4, i.e. elements 4*g4 .. 4*g4+3) into the
@@ -74,12 +74,12 @@ __device__ __forceinline__ void stage_quantize4(uint8_t* smem, int k, int per, i
 // quantizer).  k % 32 == 0, blockDim.x % 64 == 0, per = window / 32.  `first` is
 // this thread's first float4 of x, loaded by the caller ahead of time.
 __device__ __forceinline__ void stage_act_quantize(uint8_t* smem, const float* x, int k, int per,
-                                                   f32x4 first) {
+                                                   f32x4 first, int nthreads) {
     const int n4 = k / 4;
     const int n4_pad = (n4 + 63) & ~63;  // whole wavefronts take part in the lane exchanges
     int g4 = threadIdx.x;
     if (g4 < n4_pad) stage_quantize4(smem, k, per, g4, first);
-    for (g4 += blockDim.x; g4 < n4_pad; g4 += blockDim.x) {
+    for (g4 += nthreads; g4 < n4_pad; g4 += nthreads) {
         f32x4 v = g4 < n4 ? ((const f32x4*)x)[g4] : f32x4{0.f, 0.f, 0.f, 0.f};
         stage_quantize4(smem, k, per, g4, v);
     }
@@ -288,10 +288,10 @@ template <> struct SlotTraits<JL_Q6_K> {
 template <int TYPE, int RPW>
 __device__ __forceinline__ void matvec_body(const MatVecArgs& p, uint8_t* smem) {
     typedef SlotTraits<TYPE> T;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = p.nwaves;
     const int nslots = p.k / T::kElems;
     const int rows_per_block = nwaves * RPW;
-    const int group_stride = gridDim.x * rows_per_block;
+    const int group_stride = p.ngroups * rows_per_block;
     const ActLds A = act_lds_views(smem, p.k);
     int r0 = blockIdx.x * rows_per_block + wave * RPW;
 
@@ -307,8 +307,8 @@ __device__ __forceinline__ void matvec_body(const MatVecArgs& p, uint8_t* smem) 
         for (int j = 0; j < RPW; j++)
             T::load_w(p.w + (size_t)min(r0 + j, p.nrows - 1) * p.row_bytes, s, w[j]);
     }
-    if (p.x) stage_act_quantize(smem, p.x, p.k, p.per, x0);
-    else stage_act_copy(smem, p.q, p.as, p.s16, p.k);
+    if (p.x) stage_act_quantize(smem, p.x, p.k, p.per, x0, nwaves * 64);
+    else stage_act_copy(smem, p.q, p.as, p.s16, p.k, nwaves * 64);
     __syncthreads();
 
     bool preloaded = true;

@@ -172,8 +172,9 @@ __device__ __forceinline__ void unpack_q4k_body(const UnpackArgs& p) {
 // A wavefront's private LDS: 256 int8 activations, 8 scales, 16 half-block sums.
 #define JL_PK_WAVE_LDS 384
 // Dynamic LDS of a workgroup of `nw` wavefronts: the private areas, then the
-// partial sums [nw][64].
-#define JL_PK_LDS_BYTES(nw) ((nw) * (JL_PK_WAVE_LDS + 256))
+// partial sums [nw][64], rows one word apart in banks.
+#define JL_PK_RED_STRIDE 65
+#define JL_PK_LDS_BYTES(nw) ((nw) * (JL_PK_WAVE_LDS + JL_PK_RED_STRIDE * 4))
 
 struct PkAct {
     const u32x4* a;    // int8 activations of the chunk, 16 per vector
@@ -308,80 +309,139 @@ template <int NB> struct PkTraits<JL_Q4_K, NB> { typedef PkWQ4K<NB> W; };
 template <int NB> struct PkTraits<JL_Q8_0, NB> { typedef PkWQ8<NB> W; };
 template <int NB> struct PkTraits<JL_Q6_K, NB> { typedef PkWQ6K<NB> W; };
 
+// The whole-wavefront (256-element window) amax without LDS traffic: DPP maxima
+// within and across the 16-lane rows, then lane 63's value read back as a scalar.
+__device__ __forceinline__ u32 wave_amax_256(u32 m) {
+    m = dpp_max_u32<JL_DPP_QUAD_XOR1>(m);
+    m = dpp_max_u32<JL_DPP_QUAD_XOR2>(m);
+    m = dpp_max_u32<JL_DPP_ROW_HALF_MIRROR>(m);
+    m = dpp_max_u32<JL_DPP_ROW_MIRROR>(m);
+    m = max(m, (u32)dpp_i32<JL_DPP_ROW_BCAST15, 0xa>(0, (i32)m));
+    m = max(m, (u32)dpp_i32<JL_DPP_ROW_BCAST31, 0xc>(0, (i32)m));
+    return (u32)__builtin_amdgcn_readlane((i32)m, 63);
+}
+
+// A chunk's activation as the lane holds it between the load and the staging: four
+// f32 values (fused form), or in the split form four int8 in .x, a scale in .y (lanes
+// 0-7) and a half-block sum in .z (lanes 0-15).  Loads are unconditional at clamped
+// addresses, so nothing between them makes the compiler wait for data; what lies past
+// the end of the vector is zeroed when the chunk is staged.
+typedef f32x4 PkX;
+
+template <bool FUSED>
+__device__ __forceinline__ void pk_load_x(const PackedMatVecArgs& p, int c, int lane, PkX& X) {
+    const int g4 = min(c * 64 + lane, p.k / 4 - 1);
+    if (FUSED) {
+        X = ((const f32x4*)p.x)[g4];
+    } else {
+        X.x = __uint_as_float(((const u32*)p.q)[g4]);
+        X.y = p.as[min(c * 8 + (lane & 7), p.k / 32 - 1)];
+        X.z = p.s16[min(c * 16 + (lane & 15), p.k / 16 - 1)];
+        X.w = 0.f;
+    }
+}
+
+// Quantize (or copy) the chunk's activation into the wavefront's private LDS area.
+template <bool FUSED>
+__device__ __forceinline__ void pk_stage_x(const PackedMatVecArgs& p, int c, int lane, const PkX& X, uint8_t* my) {
+    u32* a_w = (u32*)my;
+    float* da_w = (float*)(my + 256);
+    float* ss_w = (float*)(my + 288);
+    const bool live = c * 64 + lane < p.k / 4;
+    if (FUSED) {
+        const f32x4 xv = live ? X : f32x4{0.f, 0.f, 0.f, 0.f};
+        u32 m = max(max(abs_bits(xv.x), abs_bits(xv.y)), max(abs_bits(xv.z), abs_bits(xv.w)));
+        const u32 amax = p.per == 8 ? wave_amax_256(m) : window_amax(m, p.per);
+        float d;
+        i32 sum;
+        const u32 qv = quantize4(xv, amax, d, sum);
+        a_w[lane] = qv;
+        if ((lane & 3) == 0) ss_w[lane >> 2] = (float)sum;
+        if ((lane & 7) == 0) da_w[lane >> 3] = d;
+    } else {
+        a_w[lane] = live ? __float_as_uint(X.x) : 0u;
+        if (lane < 8) da_w[lane] = X.y;
+        if (lane < 16) ss_w[lane] = X.z;
+    }
+    // The area is private to this wavefront, whose LDS operations complete in
+    // order: only the compiler has to be kept from moving reads above the writes.
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 // grid = ceil(nrows / RW) workgroups of 64..1024 threads; dynamic LDS =
 // JL_PK_LDS_BYTES(wavefronts).  Needs k % 32 == 0 (k % 256 == 0 for the k-quants).
-template <int TYPE, int RW>
+//
+// Order of the memory requests: a CU's vector loads are served in the order they were
+// issued, whichever wavefront issued them, so an activation load that goes out after
+// another wavefront's weight loads comes back behind them.  Every wavefront therefore
+// issues the activation loads of its first XPRE chunks (as many as registers allow),
+// the workgroup meets at a barrier that waits for no data, and only then do the weight
+// loads go out: the small activation comes back first and is quantized while the
+// weights stream in.
+//
+// The partial sums [wavefront][lane] are added up by RW*16 threads at once: thread
+// (row r, j) takes wavefront j's KP partials of row r, and the sixteen j of a row sit
+// in one 16-lane DPP row, so the sum over wavefronts is four lane-exchange adds.
+template <int TYPE, int RW, int XPRE, bool FUSED>
 __device__ __forceinline__ void packed_matvec_body(const PackedMatVecArgs& p, uint8_t* smem) {
     constexpr int KP = 64 / RW, NB = 8 / KP;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = p.nwaves;
     // Workgroups are dealt to the eight XCDs round robin; give each XCD a contiguous
     // range of row groups so neighbouring row runs meet in one L2.
     int g = blockIdx.x;
-    const int ng = gridDim.x;
+    const int ng = p.ngroups;
     if ((ng & 7) == 0) g = (g & 7) * (ng >> 3) + (g >> 3);
     const int rl = lane % RW, part = lane / RW, b0 = part * NB;
     const int row = p.row0 + min(g * RW + rl, p.nrows - 1);
 
     uint8_t* my = smem + wave * JL_PK_WAVE_LDS;
-    u32* a_w = (u32*)my;
-    float* da_w = (float*)(my + 256);
-    float* ss_w = (float*)(my + 288);
     PkAct A;
     A.a = (const u32x4*)my;
-    A.da = da_w;
-    A.ss = ss_w;
+    A.da = (const float*)(my + 256);
+    A.ss = (const float*)(my + 288);
 
-    const int n4 = p.k / 4, nchunks = (p.k + 255) / 256;
+    const int nchunks = (p.k + 255) / 256;
+    PkX X[XPRE];
+#pragma unroll
+    for (int i = 0; i < XPRE; i++) pk_load_x<FUSED>(p, wave + i * nwaves, lane, X[i]);
+    __builtin_amdgcn_s_barrier();
+
     float acc = 0.f;
-    for (int c = wave; c < nchunks; c += nwaves) {
-        // activation of this chunk first: loads come back in order
-        const int g4 = c * 64 + lane;
-        f32x4 xv = f32x4{0.f, 0.f, 0.f, 0.f};
-        u32 qv = 0;
-        float dv = 0.f, sv = 0.f;
-        if (p.x) {
-            if (g4 < n4) xv = ((const f32x4*)p.x)[g4];
-        } else {
-            if (g4 < n4) qv = ((const u32*)p.q)[g4];
-            if (lane < 8 && c * 8 + lane < p.k / 32) dv = p.as[c * 8 + lane];
-            if (lane < 16 && c * 16 + lane < p.k / 16) sv = p.s16[c * 16 + lane];
-        }
+    auto chunk = [&](int c, const PkX& Xc) {
         typename PkTraits<TYPE, NB>::W w;
         pk_load<NB>(p, c, b0, row, w);
-
-        if (p.x) {
-            u32 m = max(max(abs_bits(xv.x), abs_bits(xv.y)), max(abs_bits(xv.z), abs_bits(xv.w)));
-            u32 amax = window_amax(m, p.per);
-            float d;
-            i32 sum;
-            qv = quantize4(xv, amax, d, sum);
-            a_w[lane] = qv;
-            if ((lane & 3) == 0) ss_w[lane >> 2] = (float)sum;
-            if ((lane & 7) == 0) da_w[lane >> 3] = d;
-        } else {
-            a_w[lane] = qv;
-            if (lane < 8) da_w[lane] = dv;
-            if (lane < 16) ss_w[lane] = sv;
-        }
-        // The area is private to this wavefront, whose LDS operations complete in
-        // order: only the compiler has to be kept from moving reads above the writes.
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        pk_stage_x<FUSED>(p, c, lane, Xc, my);
         acc += pk_dot<NB>(p, w, c, b0, row, A);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
+    };
+#pragma unroll
+    for (int i = 0; i < XPRE; i++) {
+        const int c = wave + i * nwaves;
+        if (c < nchunks) chunk(c, X[i]);
+    }
+    for (int c = wave + XPRE * nwaves; c < nchunks; c += nwaves) {
+        PkX Xc;
+        pk_load_x<FUSED>(p, c, lane, Xc);
+        chunk(c, Xc);
     }
 
     float* red = (float*)(smem + nwaves * JL_PK_WAVE_LDS);
-    red[wave * 64 + lane] = acc;
+    red[wave * JL_PK_RED_STRIDE + lane] = acc;
     __syncthreads();
-    if ((int)threadIdx.x < RW) {
+    const int j = threadIdx.x & 15;
+    for (int r = threadIdx.x >> 4; r < RW; r += nwaves * 4) {
         float t = 0.f;
-        for (int wv = 0; wv < nwaves; wv++)
+        if (j < nwaves) {
 #pragma unroll
-            for (int q = 0; q < KP; q++) t += red[wv * 64 + q * RW + threadIdx.x];
-        const int r = g * RW + threadIdx.x;
-        if (r < p.nrows) p.out[r] = t;
+            for (int q = 0; q < KP; q++) t += red[j * JL_PK_RED_STRIDE + q * RW + r];
+        }
+        t += dpp_f32<JL_DPP_QUAD_XOR1, 0xf>(t);
+        t += dpp_f32<JL_DPP_QUAD_XOR2, 0xf>(t);
+        t += dpp_f32<JL_DPP_ROW_HALF_MIRROR, 0xf>(t);
+        t += dpp_f32<JL_DPP_ROW_MIRROR, 0xf>(t);
+        if (j == 0 && g * RW + r < p.nrows) p.out[g * RW + r] = t;
     }
 }
