@@ -43,27 +43,52 @@ def matvec_bytes(t, nrows, k):
 class Workload:
     """A weight matrix replicated into rotating device copies plus x and out."""
 
-    def __init__(self, dev, t, nrows, k, window, seed=0):
+    def __init__(self, dev, t, nrows, k, window, seed=0, packed=False):
+        """packed=False: GGUF row-major bytes (jl_matvec_dev); packed=True: the reference's
+        QS/D/SC planes, packed on the device from the same bytes (jl_matvec_packed_dev)."""
         from jitllm_amd import quant, synth
+        from jitllm_amd.device import Packed
         from jitllm_amd.hipmem import DeviceArray, check, hip
         self.dev, self.t, self.nrows, self.k, self.window = dev, t, nrows, k, window
+        self.packed = packed
         self.name = f"{quant.NAMES[t]} matvec {nrows}x{k} batch 1"
         self.w_host = synth.quantized_weights(t, nrows, k, seed=seed)
         self.x_host = synth.activations(k, seed=seed + 1)
-        self.wbytes = self.w_host.nbytes
+        one = DeviceArray(self.w_host)
+        if packed:
+            nq, nd, nsc = dev.packed_words(t, nrows, k)
+            up = lambda v: (v + 255) & ~255
+            o_d = up(nq * 4)
+            o_sc = o_d + up(nd * 4)
+            self.wbytes = o_sc + up(nsc * 4)
+            self.alg_bytes = (nq + nd + nsc) * 4 + 4 * k + 4 * nrows
+        else:
+            self.wbytes = self.w_host.nbytes
+            self.alg_bytes = matvec_bytes(t, nrows, k)
         self.ncopies = max(2, min(128, (2 * CACHE_BYTES + 64 * (1 << 20)) // self.wbytes + 1))
         self.pool = DeviceArray(shape=(self.ncopies * self.wbytes,), dtype=np.uint8)
-        one = DeviceArray(self.w_host)
+        self.planes = []
         for i in range(self.ncopies):
-            check(hip().hipMemcpy(self.pool.ptr + i * self.wbytes, one.ptr, self.wbytes, 3), "copy")
+            base = self.pool.ptr + i * self.wbytes
+            if packed:
+                pl = Packed(base, base + o_d, base + o_sc if nsc else None, 0, nrows)
+                if not dev.pack_weights_dev(t, one.ptr, nrows, k, pl.qs, pl.d, pl.sc):
+                    raise RuntimeError(f"{self.name}: the device declined to pack")
+                self.planes.append(pl)
+            else:
+                check(hip().hipMemcpy(base, one.ptr, self.wbytes, 3), "copy")
+        dev.synchronize()
         one.free()
         self.x = DeviceArray(self.x_host)
         self.out = DeviceArray(shape=(nrows,), dtype=np.float32, fill=0)
-        self.alg_bytes = matvec_bytes(t, nrows, k)
 
     def step(self, i):
-        ok = self.dev.matvec_dev(self.out.ptr, self.t, self.pool.ptr + (i % self.ncopies) * self.wbytes,
-                                 self.x.ptr, self.nrows, self.k)
+        if self.packed:
+            ok = self.dev.matvec_packed_dev(self.out.ptr, self.t, self.planes[i % self.ncopies], self.x.ptr,
+                                            self.nrows, self.k)
+        else:
+            ok = self.dev.matvec_dev(self.out.ptr, self.t, self.pool.ptr + (i % self.ncopies) * self.wbytes,
+                                     self.x.ptr, self.nrows, self.k)
         if not ok:
             raise RuntimeError(f"{self.name}: the device declined")
 
@@ -284,17 +309,23 @@ def main():
     head.free()
 
     if not args.no_extra:
+        # the other decode matvecs, over GGUF rows and over the reference's packed planes
         extra = {}
-        for key, t, nrows, k, window in [("q8_0_14336x4096", quant.Q8_0, 14336, 4096, 32),
+        for key, t, nrows, k, window in [("q4_k_4096x4096", quant.Q4_K, 4096, 4096, 256),
+                                         ("q8_0_14336x4096", quant.Q8_0, 14336, 4096, 32),
                                          ("q6_k_4096x14336", quant.Q6_K, 4096, 14336, 32),
                                          ("q4_k_14336x4096", quant.Q4_K, 14336, 4096, 256)]:
-            wl = Workload(dev, t, nrows, k, window)
-            ems, _ = wl.timed(max(50, args.steps // 10), max(10, args.warmup // 10))
-            wl.check()
-            g = wl.alg_bytes / (ems * 1e-3) / 1e9
-            extra[key] = {"us_per_step": round(ems * 1e3, 2), "GB/s": round(g, 1),
-                          "frac_of_hbm_peak": round(g / HBM_PEAK_GBS, 4), "bytes_per_step": wl.alg_bytes}
-            wl.free()
+            for layout, packed in (("gguf_rows", False), ("packed_planes", True)):
+                if key == "q4_k_4096x4096" and not packed:
+                    continue  # the headline above
+                wl = Workload(dev, t, nrows, k, window, packed=packed)
+                ems, _ = wl.timed(max(50, args.steps // 10), max(10, args.warmup // 10))
+                wl.check()
+                g = wl.alg_bytes / (ems * 1e-3) / 1e9
+                extra.setdefault(key, {})[layout] = {
+                    "us_per_step": round(ems * 1e3, 2), "GB/s": round(g, 1),
+                    "frac_of_hbm_peak": round(g / HBM_PEAK_GBS, 4), "bytes_per_step": wl.alg_bytes}
+                wl.free()
         line["other_configs"] = extra
 
     if not args.no_extra:

@@ -357,11 +357,12 @@ int packed_matvec_launch(jl_ctx* c, float* out, int type, const PlaneRef& pl, co
     if (x && !aligned16(x)) return JL_DECLINED;
     if (!x && (!q || !as || !s16)) return fail(c, JL_ERR_ARG, "packed matvec: no activation");
     if (q && ((uintptr_t)q & 3)) return JL_DECLINED;
-    // Rows per wavefront: the widest run that still gives every CU a workgroup.
+    // Rows per wavefront: the widest run that still gives three CUs in four a
+    // workgroup (from sweeps: 224 workgroups of 64-row runs beat 448 of 32-row runs).
     int rw = c->tune.packed_rw;
     if (rw <= 0) {
         rw = 64;
-        while (rw > 16 && (nrows + rw - 1) / rw < c->num_cu) rw >>= 1;
+        while (rw > 16 && (nrows + rw - 1) / rw < c->num_cu * 3 / 4) rw >>= 1;
     }
     if (rw != 16 && rw != 32 && rw != 64) return fail(c, JL_ERR_ARG, "packed matvec: rw=%d", rw);
     const int nchunks = (k + 255) / 256;

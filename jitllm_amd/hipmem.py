@@ -35,6 +35,12 @@ def hip():
         h.hipEventElapsedTime.argtypes = [C.POINTER(C.c_float), C.c_void_p, C.c_void_p]
         h.hipEventDestroy.argtypes = [C.c_void_p]
         h.hipMemGetInfo.argtypes = [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]
+        h.hipStreamBeginCapture.argtypes = [C.c_void_p, C.c_int]
+        h.hipStreamEndCapture.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
+        h.hipGraphInstantiate.argtypes = [C.POINTER(C.c_void_p), C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]
+        h.hipGraphLaunch.argtypes = [C.c_void_p, C.c_void_p]
+        h.hipGraphExecDestroy.argtypes = [C.c_void_p]
+        h.hipGraphDestroy.argtypes = [C.c_void_p]
         _hip = h
     return _hip
 
@@ -116,5 +122,42 @@ class Event:
     def __del__(self):
         try:
             hip().hipEventDestroy(self.e)
+        except Exception:
+            pass
+
+
+class Graph:
+    """A HIP graph captured from a stream: `with Graph.capture(stream) as g: <enqueue work>`,
+    then g.launch(stream) replays the recorded launches with one submission."""
+
+    _THREAD_LOCAL = 1  # hipStreamCaptureModeThreadLocal
+
+    def __init__(self, stream):
+        self.stream, self.graph, self.exe = stream, C.c_void_p(), C.c_void_p()
+
+    @classmethod
+    def capture(cls, stream):
+        return cls(stream)
+
+    def __enter__(self):
+        check(hip().hipStreamBeginCapture(self.stream, self._THREAD_LOCAL), "hipStreamBeginCapture")
+        return self
+
+    def __exit__(self, exc_type, exc, tb):
+        rc = hip().hipStreamEndCapture(self.stream, C.byref(self.graph))
+        if exc_type is None:
+            check(rc, "hipStreamEndCapture")
+            check(hip().hipGraphInstantiate(C.byref(self.exe), self.graph, None, None, 0), "hipGraphInstantiate")
+        return False
+
+    def launch(self, stream=None):
+        check(hip().hipGraphLaunch(self.exe, stream if stream is not None else self.stream), "hipGraphLaunch")
+
+    def __del__(self):
+        try:
+            if self.exe:
+                hip().hipGraphExecDestroy(self.exe)
+            if self.graph:
+                hip().hipGraphDestroy(self.graph)
         except Exception:
             pass
