@@ -85,7 +85,8 @@ int jl_synchronize(jl_ctx *ctx);
  * wavefront: 1, 2, 4), "matvec.block" (threads per workgroup), "matvec.grid"
  * (workgroups), "gemm.min_tok" (fewest tokens sent to the matrix-core GEMM),
  * "packed.rw" (rows per wavefront of the packed-plane matvec: 16, 32, 64),
- * "packed.block" (its threads per workgroup);
+ * "packed.block" (its threads per workgroup), "moe.shares" (row shares an expert's
+ * matrix is split into);
  * value 0 restores the built-in choice.  Mirrors the reference's per-instance tuning knobs
  * (engine/nn/options.go:67-118). */
 int jl_set_tuning(jl_ctx *ctx, const char *key, int value);
@@ -226,11 +227,13 @@ int jl_moe_group_dev(jl_ctx *ctx, const uint32_t *sel, int sel_stride, int rows,
  * engine/nn/packedmulti.go:24,93): for every column c of expert e,
  *   out0[c][0:nrows] = bank0 sheet e . act(c)   (and out1 / bank1 when given),
  * act(c) = x[src[c]] (src NULL: x[c]) or silu(x[..]) * x2[..] when x2 is given.  A bank
- * is n_expert sheets of nrows x k GGUF rows back to back.  Activations are
- * quantized per column exactly as jl_matvec_dev does. */
+ * is n_expert sheets of nrows x k GGUF rows back to back.  ncols = start[n_expert], the
+ * number of columns (rows * k_used).  Activations are quantized per column exactly as
+ * jl_matvec_dev does, once, into a workspace the context owns (grown on demand). */
 int jl_moe_matvec_dev(jl_ctx *ctx, float *out0, float *out1, int type, const void *bank0,
                       const void *bank1, const float *x, const float *x2, const uint32_t *src,
-                      const uint32_t *start, int n_expert, int nrows, int k, void *stream);
+                      const uint32_t *start, int n_expert, int ncols, int nrows, int k,
+                      void *stream);
 
 /* kernels.ExpertCombineGrouped (jit/gpu/kernels/moegroup.go:38-68) with the host path's
  * order (engine/model/moe.go:127-134, :752-759): resid[r] += sum of wt[r][s] *

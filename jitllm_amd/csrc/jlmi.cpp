@@ -29,6 +29,7 @@ const HipApi* H = nullptr;  // the process-wide HIP runtime, resolved by the fir
 struct Tuning {
     int rpw = 0, block = 0, grid = 0;
     int packed_rw = 0, packed_block = 0;
+    int moe_shares = 0;
 };
 
 struct Resident {
@@ -54,6 +55,9 @@ struct jl_ctx {
     // prefill GEMM workspace (quantized activations in stage layout), grown on demand
     void* gemm_ws = nullptr;
     size_t gemm_ws_bytes = 0;
+
+    void* moe_q_ws = nullptr;   // quantized column activations of a mixture pass
+    size_t moe_q_ws_bytes = 0;
 
     // rows restored to GGUF order for the GEMM over packed planes
     void* unpack_ws = nullptr;
@@ -415,13 +419,14 @@ int packed_matmul_launch(jl_ctx* c, float* out, int type, const PlaneRef& pl, co
 
 int moe_matvec_launch(jl_ctx* c, float* out0, float* out1, int type, const void* bank0, const void* bank1,
                       const float* x, const float* x2, const uint32_t* src, const uint32_t* start,
-                      int n_expert, int nrows, int k, hipStream_t st) {
+                      int n_expert, int ncols, int nrows, int k, hipStream_t st) {
     const TypeInfo* ti = nullptr;
     int rc = matvec_check(c, type, nrows, k, &ti);
     if (rc != JL_OK) return rc;
-    if (!out0 || !bank0 || !x || !start || n_expert <= 0) return fail(c, JL_ERR_ARG, "moe matvec: bad operand");
+    if (!out0 || !bank0 || !x || !start || n_expert <= 0 || ncols <= 0)
+        return fail(c, JL_ERR_ARG, "moe matvec: bad operand");
     if ((bank1 == nullptr) != (out1 == nullptr)) return fail(c, JL_ERR_ARG, "moe matvec: second matrix needs both bank and out");
-    if (!aligned16(x) || (x2 && !aligned16(x2)) || k % 256 != 0 || n_expert > 65535) return JL_DECLINED;
+    if (!aligned16(x) || (x2 && !aligned16(x2)) || k % 256 != 0 || n_expert > 65535 || ncols > 65535) return JL_DECLINED;
     if (!aligned16(bank0) || (bank1 && !aligned16(bank1))) return JL_DECLINED;
     const int row_bytes = (k / ti->block_elems) * ti->block_bytes;
     const size_t sheet = (size_t)nrows * row_bytes;
@@ -432,23 +437,46 @@ int moe_matvec_launch(jl_ctx* c, float* out0, float* out1, int type, const void*
     const size_t act = ((size_t)k + (size_t)(k / 32) * 4 + (size_t)(k / 16) * 4 + 15) & ~(size_t)15;
     const size_t lds = 8 * act;
     if (lds > c->lds_limit) return JL_DECLINED;
+
+    // every column's activation, quantized once: q [ncols][k], as [ncols][k/32], s16 [ncols][k/16]
+    auto up256 = [](size_t v) { return (v + 255) & ~(size_t)255; };
+    const size_t o_as = up256((size_t)ncols * k), o_s16 = o_as + up256((size_t)ncols * (k / 32) * 4);
+    rc = ws_ensure(c, &c->moe_q_ws, &c->moe_q_ws_bytes, o_s16 + up256((size_t)ncols * (k / 16) * 4));
+    if (rc != JL_OK) return rc;
+    char* qws = (char*)c->moe_q_ws;
+    MoeQuantArgs qa;
+    qa.x = x; qa.x2 = x2; qa.src = src;
+    qa.q = (int8_t*)qws; qa.as = (float*)(qws + o_as); qa.s16 = (float*)(qws + o_s16);
+    qa.k = k; qa.per = c->act_window / 32;
+    void* qparams[] = {&qa};
+    rc = launch(c, "jl_moe_quant", (unsigned)((k / 4 + 255) / 256), (unsigned)ncols, 256, 0, st, qparams);
+    if (rc != JL_OK) return rc;
+
     MoeMatVecArgs a;
     a.out[0] = out0; a.out[1] = out1;
     a.bank[0] = (const uint8_t*)bank0; a.bank[1] = (const uint8_t*)bank1;
-    a.x = x; a.x2 = x2; a.src = src; a.start = start;
-    a.sheet_bytes = sheet; a.nrows = nrows; a.k = k; a.row_bytes = row_bytes; a.per = c->act_window / 32;
-    // row shares per expert: enough workgroups to cover the chip a couple of times when
-    // every expert is in use, never fewer than 64 rows a share
-    const int nmat = bank1 ? 2 : 1;
-    int shares = (2 * c->num_cu + n_expert * nmat - 1) / (n_expert * nmat);
+    a.q = qa.q; a.as = qa.as; a.s16 = qa.s16; a.start = start;
+    a.sheet_bytes = sheet; a.nrows = nrows; a.k = k; a.row_bytes = row_bytes;
+    // A workgroup of eight wavefronts covers 8 * 2 * (64 / lpr) rows per step.  Row shares:
+    // about six workgroups per CU when every expert is in use (from sweeps at the
+    // 128-expert, 64-row shape), each share at least one step.
+    const int nmat = bank1 ? 2 : 1, nwaves = 8;
+    const int rows_per_step = nwaves * 2 * (64 / lpr);  // JL_MOE_U row groups per wavefront step
+    int shares = c->tune.moe_shares;
+    if (shares <= 0) {
+        shares = (6 * c->num_cu + n_expert * nmat - 1) / (n_expert * nmat);
+        const int most = (nrows + rows_per_step - 1) / rows_per_step;
+        if (shares > most) shares = most;
+    }
     if (shares < 1) shares = 1;
-    while (shares > 1 && nrows / shares < 64) shares--;
+    if (shares > 65535) shares = 65535;
+    a.nwaves = nwaves; a.shares = shares;
     char name[64];
     snprintf(name, sizeof name, "jl_moe_matvec_%s_l%d", ti->tag, lpr);
     auto it = c->fn.find(name);
     if (it == c->fn.end()) return fail(c, JL_ERR_ARG, "kernel %s is not in the code object", name);
     void* params[] = {&a};
-    HIP_TRY(c, H->ModuleLaunchKernel(it->second, (unsigned)shares, (unsigned)n_expert, (unsigned)nmat, 512, 1, 1,
+    HIP_TRY(c, H->ModuleLaunchKernel(it->second, (unsigned)shares, (unsigned)n_expert, (unsigned)nmat, nwaves * 64, 1, 1,
                                      (unsigned)lds, st, params, nullptr));
     return JL_OK;
 }
@@ -493,7 +521,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     if (e != hipSuccess)
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
-    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_q4k", "jl_moe_group", "jl_moe_combine", "jl_mxfp4_gemm", "jl_mxfp4_matvec",
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_q4k", "jl_moe_group", "jl_moe_quant", "jl_moe_combine", "jl_mxfp4_gemm", "jl_mxfp4_matvec",
                                       "jl_pack_weights", "jl_unpack_q4k"};
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int rw : {16, 32, 64})
@@ -533,6 +561,7 @@ void jl_ctx_destroy(jl_ctx* c) {
     if (c->gemm_ws) (void)H->Free(c->gemm_ws);
     if (c->moe_ws) (void)H->Free(c->moe_ws);
     if (c->unpack_ws) (void)H->Free(c->unpack_ws);
+    if (c->moe_q_ws) (void)H->Free(c->moe_q_ws);
     if (c->stage_x) (void)H->Free(c->stage_x);
     if (c->stage_out) (void)H->Free(c->stage_out);
     if (c->module) (void)H->ModuleUnload(c->module);
@@ -566,6 +595,7 @@ int jl_set_tuning(jl_ctx* c, const char* key, int value) {
     else if (!strcmp(key, "matvec.grid")) c->tune.grid = value;
     else if (!strcmp(key, "packed.rw")) c->tune.packed_rw = value;
     else if (!strcmp(key, "packed.block")) c->tune.packed_block = value;
+    else if (!strcmp(key, "moe.shares")) c->tune.moe_shares = value;
     else if (!strcmp(key, "gemm.min_tok")) c->gemm_min_tok = value > 0 ? value : 8;
     else return fail(c, JL_ERR_ARG, "unknown tuning key %s", key);
     return JL_OK;
@@ -716,10 +746,10 @@ int jl_moe_group_dev(jl_ctx* c, const uint32_t* sel, int sel_stride, int rows, i
 
 int jl_moe_matvec_dev(jl_ctx* c, float* out0, float* out1, int type, const void* bank0, const void* bank1,
                       const float* x, const float* x2, const uint32_t* src, const uint32_t* start,
-                      int n_expert, int nrows, int k, void* stream) {
+                      int n_expert, int ncols, int nrows, int k, void* stream) {
     if (!c) return JL_ERR_ARG;
     HIP_TRY(c, H->SetDevice(c->device));
-    return moe_matvec_launch(c, out0, out1, type, bank0, bank1, x, x2, src, start, n_expert, nrows, k,
+    return moe_matvec_launch(c, out0, out1, type, bank0, bank1, x, x2, src, start, n_expert, ncols, nrows, k,
                              pick_stream(c, stream));
 }
 
@@ -762,10 +792,10 @@ int jl_moe_ffn_dev(jl_ctx* c, float* resid, int type, const void* gate_bank, con
     rc = jl_moe_group_dev(c, sel, sel_stride, rows, k_used, n_expert, start, perm, pos, st);
     if (rc != JL_OK) return rc;
     // gate and up: columns read the routed rows of x
-    rc = moe_matvec_launch(c, g, u, type, gate_bank, up_bank, x, nullptr, perm, start, n_expert, n_ffn, n_embd, st);
+    rc = moe_matvec_launch(c, g, u, type, gate_bank, up_bank, x, nullptr, perm, start, n_expert, (int)ncols, n_ffn, n_embd, st);
     if (rc != JL_OK) return rc;
     // down: the activation of column c is silu(g[c]) * u[c]
-    rc = moe_matvec_launch(c, y, nullptr, type, down_bank, nullptr, g, u, nullptr, start, n_expert, n_embd, n_ffn, st);
+    rc = moe_matvec_launch(c, y, nullptr, type, down_bank, nullptr, g, u, nullptr, start, n_expert, (int)ncols, n_embd, n_ffn, st);
     if (rc != JL_OK) return rc;
     return jl_moe_combine_dev(c, resid, y, wt, sel, sel_stride, pos, rows, k_used, n_embd, st);
 }

@@ -47,17 +47,32 @@ struct MoeGroupArgs {
     int sel_stride, rows, k_used, n_expert;
 };
 
-// Grouped expert matvec over columns sorted by expert: out[m][c][0:nrows] =
-// bank[m] sheet(expert of c) . act(c), act(c) = x[src(c)] or silu(x[src(c)]) * x2[src(c)].
-struct MoeMatVecArgs {
-    float* out[2];
-    const uint8_t* bank[2];
+// Column activations of a mixture pass: column c reads x[src(c)] (or silu(x[src(c)]) *
+// x2[src(c)]) and is quantized like any activation vector: q [ncols][k] int8,
+// as [ncols][k/32], s16 [ncols][k/16].
+struct MoeQuantArgs {
     const float* x;
     const float* x2;        // null: plain activation
     const uint32_t* src;    // null: column c reads row c
+    int8_t* q;
+    float* as;
+    float* s16;
+    int k, per;
+};
+
+// Grouped expert matvec over columns sorted by expert: out[m][c][0:nrows] =
+// bank[m] sheet(expert of c) . column c, columns already quantized (MoeQuantArgs).
+struct MoeMatVecArgs {
+    float* out[2];
+    const uint8_t* bank[2];
+    const int8_t* q;
+    const float* as;
+    const float* s16;
     const uint32_t* start;  // [n_expert + 1]
     size_t sheet_bytes;
-    int nrows, k, row_bytes, per;
+    int nrows, k, row_bytes;
+    int nwaves;             // wavefronts per workgroup
+    int shares;             // workgroups one (expert, matrix) is split into, by rows
 };
 
 struct MoeCombineArgs {

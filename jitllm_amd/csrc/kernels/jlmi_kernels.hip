@@ -79,12 +79,15 @@ extern "C" __global__ __launch_bounds__(256) void jl_gemm_prep_q4k(GemmPrepArgs 
 extern "C" __global__ __launch_bounds__(512) void jl_gemm_q4k(GemmArgs p) { gemm_q4k_body(p, jl_smem); }
 
 // ------------------------------------------------------- mixture of experts
-// one workgroup of 1024; thread e owns expert e (n_expert <= 1024)
+// one workgroup of 1024 threads (n_expert <= 1024)
 extern "C" __global__ __launch_bounds__(1024) void jl_moe_group(MoeGroupArgs p) {
-    __shared__ u32 scount[1024];
-    moe_group_body(p, scount);
+    __shared__ u32 scount[2048];
+    __shared__ __attribute__((aligned(16))) uint16_t skeys[JL_MOE_GROUP_KEYS];
+    moe_group_body(p, scount, skeys);
 }
-// grid = (row shares, n_expert, matrices), block = 512, dynamic LDS = 8 staged activations
+// grid = (ceil(k/4/256), ncols), block = 256
+extern "C" __global__ __launch_bounds__(256) void jl_moe_quant(MoeQuantArgs p) { moe_quant_body(p); }
+// grid = (row shares, n_expert, matrices), block = 512, dynamic LDS = 8 staged columns
 #define JL_MOE_KERNEL(T, TYPE, LPR)                                                               \
     extern "C" __global__ __launch_bounds__(512) void jl_moe_matvec_##T##_l##LPR(MoeMatVecArgs p) { \
         moe_matvec_body<TYPE, LPR>(p, jl_smem);                                                   \

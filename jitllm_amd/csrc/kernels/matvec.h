@@ -118,7 +118,15 @@ __device__ __forceinline__ void load_w_q4k(const uint8_t* row, int slot, SlotWQ4
     w.q[1] = ld16(qs + 16);
 }
 
-__device__ __forceinline__ float dot_q4k(const SlotWQ4K& w, int g, const SlotActQ4K& s) {
+// A slot's weights with the scale arithmetic done: what stays the same when the
+// slot meets several activations (the columns of a mixture-of-experts pass).
+struct PrepQ4K {
+    u32x4 lo[2], hi[2];    // nibbles of sub-blocks 2g / 2g+1 as bytes
+    float dsc_lo, dsc_hi;  // d * sc of sub-blocks 2g, 2g+1
+    float dm_lo, dm_hi;    // dmin * m
+};
+
+__device__ __forceinline__ void prep_q4k(const SlotWQ4K& w, int g, PrepQ4K& P) {
     float d = half_bits_to_f32((uint16_t)(w.hdr.x & 0xFFFF));
     float dmin = half_bits_to_f32((uint16_t)(w.hdr.x >> 16));
     // 6-bit scale/min pairs of sub-blocks 2g and 2g+1, branch-free
@@ -134,21 +142,37 @@ __device__ __forceinline__ float dot_q4k(const SlotWQ4K& w, int g, const SlotAct
         m_lo = ((C >> 4) & 0xF) | (((B >> 6) & 3) << 4);
         m_hi = ((C >> 12) & 0xF) | (((B >> 14) & 3) << 4);
     }
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        P.lo[i] = w.q[i] & 0x0F0F0F0Fu;
+        P.hi[i] = (w.q[i] >> 4) & 0x0F0F0F0Fu;
+    }
+    P.dsc_lo = d * (float)sc_lo; P.dsc_hi = d * (float)sc_hi;
+    P.dm_lo = dmin * (float)m_lo; P.dm_hi = dmin * (float)m_hi;
+}
+
+__device__ __forceinline__ float dotp_q4k(const PrepQ4K& w, const SlotActQ4K& s) {
     i32 dl = 0, dh = 0;
 #pragma unroll
     for (int i = 0; i < 2; i++) {
-        dl = dot4(w.q[i].x & 0x0F0F0F0Fu, s.lo[i].x, dl);
-        dl = dot4(w.q[i].y & 0x0F0F0F0Fu, s.lo[i].y, dl);
-        dl = dot4(w.q[i].z & 0x0F0F0F0Fu, s.lo[i].z, dl);
-        dl = dot4(w.q[i].w & 0x0F0F0F0Fu, s.lo[i].w, dl);
-        dh = dot4((w.q[i].x >> 4) & 0x0F0F0F0Fu, s.hi[i].x, dh);
-        dh = dot4((w.q[i].y >> 4) & 0x0F0F0F0Fu, s.hi[i].y, dh);
-        dh = dot4((w.q[i].z >> 4) & 0x0F0F0F0Fu, s.hi[i].z, dh);
-        dh = dot4((w.q[i].w >> 4) & 0x0F0F0F0Fu, s.hi[i].w, dh);
+        dl = dot4(w.lo[i].x, s.lo[i].x, dl);
+        dl = dot4(w.lo[i].y, s.lo[i].y, dl);
+        dl = dot4(w.lo[i].z, s.lo[i].z, dl);
+        dl = dot4(w.lo[i].w, s.lo[i].w, dl);
+        dh = dot4(w.hi[i].x, s.hi[i].x, dh);
+        dh = dot4(w.hi[i].y, s.hi[i].y, dh);
+        dh = dot4(w.hi[i].z, s.hi[i].z, dh);
+        dh = dot4(w.hi[i].w, s.hi[i].w, dh);
     }
-    float v_lo = (float)dl * (d * (float)sc_lo) - s.s_lo * (dmin * (float)m_lo);
-    float v_hi = (float)dh * (d * (float)sc_hi) - s.s_hi * (dmin * (float)m_hi);
+    float v_lo = (float)dl * w.dsc_lo - s.s_lo * w.dm_lo;
+    float v_hi = (float)dh * w.dsc_hi - s.s_hi * w.dm_hi;
     return fmaf(v_lo, s.da_lo, v_hi * s.da_hi);
+}
+
+__device__ __forceinline__ float dot_q4k(const SlotWQ4K& w, int g, const SlotActQ4K& s) {
+    PrepQ4K P;
+    prep_q4k(w, g, P);
+    return dotp_q4k(P, s);
 }
 
 // ---------------------------------------------------------------- Q8_0 slot
@@ -176,7 +200,17 @@ __device__ __forceinline__ void load_w_q8(const uint8_t* row, int slot, SlotWQ8&
     w.q[1] = ld16_a2(blk + 18);
 }
 
-__device__ __forceinline__ float dot_q8(const SlotWQ8& w, const SlotActQ8& s) {
+struct PrepQ8 {
+    u32x4 q[2];
+    float d;
+};
+
+__device__ __forceinline__ void prep_q8(const SlotWQ8& w, PrepQ8& P) {
+    P.q[0] = w.q[0]; P.q[1] = w.q[1];
+    P.d = half_bits_to_f32(w.d);
+}
+
+__device__ __forceinline__ float dotp_q8(const PrepQ8& w, const SlotActQ8& s) {
     i32 dt = 0;
 #pragma unroll
     for (int i = 0; i < 2; i++) {
@@ -185,7 +219,13 @@ __device__ __forceinline__ float dot_q8(const SlotWQ8& w, const SlotActQ8& s) {
         dt = dot4(w.q[i].z, s.a[i].z, dt);
         dt = dot4(w.q[i].w, s.a[i].w, dt);
     }
-    return (float)dt * half_bits_to_f32(w.d) * s.da;
+    return (float)dt * w.d * s.da;
+}
+
+__device__ __forceinline__ float dot_q8(const SlotWQ8& w, const SlotActQ8& s) {
+    PrepQ8 P;
+    prep_q8(w, P);
+    return dotp_q8(P, s);
 }
 
 // ---------------------------------------------------------------- Q6_K slot
@@ -235,24 +275,39 @@ __device__ __forceinline__ i32 dot16(u32x4 q, u32x4 a) {
     return dot4(q.w, a.w, t);
 }
 
-__device__ __forceinline__ float dot_q6k(const SlotWQ6K& w, const SlotActQ6K& s) {
+struct PrepQ6K {
+    u32x4 q[4];   // the four 16-element runs as bytes 0..63
+    float sc[4];  // d * int8 scale of each run
+};
+
+__device__ __forceinline__ void prep_q6k(const SlotWQ6K& w, PrepQ6K& P) {
     const u32 M4 = 0x0F0F0F0Fu, M2 = 0x30303030u;
-    u32x4 q0 = (w.qla & M4) | ((w.qh << 4) & M2);
-    u32x4 q1 = (w.qlb & M4) | ((w.qh << 2) & M2);
-    u32x4 q2 = ((w.qla >> 4) & M4) | (w.qh & M2);
-    u32x4 q3 = ((w.qlb >> 4) & M4) | ((w.qh >> 2) & M2);
+    P.q[0] = (w.qla & M4) | ((w.qh << 4) & M2);
+    P.q[1] = (w.qlb & M4) | ((w.qh << 2) & M2);
+    P.q[2] = ((w.qla >> 4) & M4) | (w.qh & M2);
+    P.q[3] = ((w.qlb >> 4) & M4) | ((w.qh >> 2) & M2);
     float d = half_bits_to_f32(w.d);
+    P.sc[0] = d * (float)(int8_t)(w.sc & 0xFF);
+    P.sc[1] = d * (float)(int8_t)((w.sc >> 8) & 0xFF);
+    P.sc[2] = d * (float)(int8_t)((w.sc >> 16) & 0xFF);
+    P.sc[3] = d * (float)(int8_t)(w.sc >> 24);
+}
+
+__device__ __forceinline__ float dotp_q6k(const PrepQ6K& w, const SlotActQ6K& s) {
     float acc = 0.f;
     // value = d*sc*(q-32): the zero point goes through the activation sum
-    float t0 = (float)(dot16(q0, s.a[0])) - 32.f * s.s[0];
-    float t1 = (float)(dot16(q1, s.a[1])) - 32.f * s.s[1];
-    float t2 = (float)(dot16(q2, s.a[2])) - 32.f * s.s[2];
-    float t3 = (float)(dot16(q3, s.a[3])) - 32.f * s.s[3];
-    acc = fmaf(t0 * (d * (float)(int8_t)(w.sc & 0xFF)), s.da[0], acc);
-    acc = fmaf(t1 * (d * (float)(int8_t)((w.sc >> 8) & 0xFF)), s.da[1], acc);
-    acc = fmaf(t2 * (d * (float)(int8_t)((w.sc >> 16) & 0xFF)), s.da[2], acc);
-    acc = fmaf(t3 * (d * (float)(int8_t)(w.sc >> 24)), s.da[3], acc);
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        float t = (float)(dot16(w.q[j], s.a[j])) - 32.f * s.s[j];
+        acc = fmaf(t * w.sc[j], s.da[j], acc);
+    }
     return acc;
+}
+
+__device__ __forceinline__ float dot_q6k(const SlotWQ6K& w, const SlotActQ6K& s) {
+    PrepQ6K P;
+    prep_q6k(w, P);
+    return dotp_q6k(P, s);
 }
 
 // ------------------------------------------------------------- the kernel
@@ -263,6 +318,9 @@ template <> struct SlotTraits<JL_Q4_K> {
     static __device__ __forceinline__ void load_act(const ActLds& A, int s, Act& a) { load_act_q4k(A, s, a); }
     static __device__ __forceinline__ void load_w(const uint8_t* row, int s, W& w) { load_w_q4k(row, s, w); }
     static __device__ __forceinline__ float dot(const W& w, int s, const Act& a) { return dot_q4k(w, s & 3, a); }
+    typedef PrepQ4K Prep;
+    static __device__ __forceinline__ void prep(const W& w, int s, Prep& P) { prep_q4k(w, s & 3, P); }
+    static __device__ __forceinline__ float dotp(const Prep& P, const Act& a) { return dotp_q4k(P, a); }
 };
 template <> struct SlotTraits<JL_Q8_0> {
     typedef SlotActQ8 Act; typedef SlotWQ8 W;
@@ -270,6 +328,9 @@ template <> struct SlotTraits<JL_Q8_0> {
     static __device__ __forceinline__ void load_act(const ActLds& A, int s, Act& a) { load_act_q8(A, s, a); }
     static __device__ __forceinline__ void load_w(const uint8_t* row, int s, W& w) { load_w_q8(row, s, w); }
     static __device__ __forceinline__ float dot(const W& w, int, const Act& a) { return dot_q8(w, a); }
+    typedef PrepQ8 Prep;
+    static __device__ __forceinline__ void prep(const W& w, int, Prep& P) { prep_q8(w, P); }
+    static __device__ __forceinline__ float dotp(const Prep& P, const Act& a) { return dotp_q8(P, a); }
 };
 template <> struct SlotTraits<JL_Q6_K> {
     typedef SlotActQ6K Act; typedef SlotWQ6K W;
@@ -277,6 +338,9 @@ template <> struct SlotTraits<JL_Q6_K> {
     static __device__ __forceinline__ void load_act(const ActLds& A, int s, Act& a) { load_act_q6k(A, s, a); }
     static __device__ __forceinline__ void load_w(const uint8_t* row, int s, W& w) { load_w_q6k(row, s, w); }
     static __device__ __forceinline__ float dot(const W& w, int, const Act& a) { return dot_q6k(w, a); }
+    typedef PrepQ6K Prep;
+    static __device__ __forceinline__ void prep(const W& w, int, Prep& P) { prep_q6k(w, P); }
+    static __device__ __forceinline__ float dotp(const Prep& P, const Act& a) { return dotp_q6k(P, a); }
 };
 
 

@@ -10,12 +10,14 @@
 //   moe_group      (row, slot) pairs -> columns sorted by expert, pairs in
 //                  (row, slot) order inside an expert: start[e], perm[col],
 //                  pos[pair]  (jit/gpu/tier/grouppairs_test.go:91-122, unit 1)
-//   moe_matvec     for every column c of expert e: out[c] = W_e . x[src(c)], the
+//   moe_quant      every column's activation, x[src(c)] or act(gate)*up, quantized
+//                  once like any activation vector
+//   moe_matvec     for every column c of expert e: out[c] = W_e . column c, the
 //                  decode matvec's arithmetic per column.  One workgroup owns
-//                  (expert, row share): it quantizes the expert's activations
-//                  into LDS once (optionally act(gate)*up first) and streams the
-//                  expert's weight rows once for up to eight columns at a time,
-//                  so a sheet is read from HBM once however many rows chose it.
+//                  (expert, row share): it stages up to eight of the expert's
+//                  quantized columns in LDS and streams the expert's weight rows
+//                  once for all of them, so a sheet is read from HBM once however
+//                  many rows chose it.
 //   moe_combine    resid[r] += sum_s w[r][s] * y[pos[r][s]], experts in ascending
 //                  id order as the host path adds them (engine/model/moe.go:127-134)
 //
@@ -27,32 +29,87 @@
 #include "common.h"
 #include "matvec.h"
 
+// Phase marker for profiling builds; expands to nothing in the product.
+#ifndef JL_MOE_TRACE
+#define JL_MOE_TRACE(i)
+#endif
+
 #define JL_MOE_TB 8  // columns of one expert processed per pass over its rows
+#define JL_MOE_U 2   // row groups of 64/LPR rows a wavefront step covers
+#define JL_MOE_GROUP_KEYS 16384  // (row, slot) pairs the grouping kernel holds in LDS
 
 // ------------------------------------------------------------------ grouping
-// One workgroup; thread e owns expert e and scans the pairs in order, which makes
-// the within-expert order (row, slot) with no atomics.
-__device__ __forceinline__ void moe_group_body(const MoeGroupArgs& p, u32* scount) {
-    const int e = threadIdx.x;
+// A stable counting sort of the (row, slot) pairs by expert in one workgroup of 1024
+// threads.  The threads form NSEG segments x NEXP experts (NEXP = n_expert rounded up
+// to a power of two): thread (seg, e) counts expert e's pairs in its contiguous segment
+// of the pair list, a prefix over (e, seg) turns counts into first columns, and the
+// same thread then walks its segment again handing out columns in order.  No atomics,
+// so inside an expert the order is (row, slot).
+__device__ __forceinline__ void moe_group_body(const MoeGroupArgs& p, u32* scount, uint16_t* skeys) {
     const int npairs = p.rows * p.k_used;
+    int nexp = 1;
+    while (nexp < p.n_expert) nexp <<= 1;
+    const int nseg = 1024 / nexp;
+    const int e = threadIdx.x & (nexp - 1), seg = threadIdx.x / nexp;
+    // segments are whole groups of eight pairs so the staged keys are read eight at a time
+    const int per_seg = ((npairs + nseg - 1) / nseg + 7) & ~7;
+    const int lo = min(seg * per_seg, npairs), hi = min(lo + per_seg, npairs);
+    auto key_global = [&](int i) { return p.sel[(i / p.k_used) * p.sel_stride + i % p.k_used]; };
+    // the pair list is walked twice by every segment: keep it in LDS when it fits
+    // (padded to a multiple of eight with an id no expert has)
+    const bool staged = npairs <= JL_MOE_GROUP_KEYS;
+    if (staged) {
+        const int padded = (npairs + 7) & ~7;
+        for (int i = threadIdx.x; i < padded; i += 1024)
+            skeys[i] = i < npairs ? (uint16_t)min(key_global(i), 0xFFFFu) : (uint16_t)0xFFFF;
+        __syncthreads();
+    }
+    typedef uint16_t u16x8 __attribute__((ext_vector_type(8)));
     u32 cnt = 0;
-    if (e < p.n_expert)
-        for (int i = 0; i < npairs; i++) cnt += p.sel[(i / p.k_used) * p.sel_stride + i % p.k_used] == (u32)e;
-    scount[e] = e < p.n_expert ? cnt : 0;
-    __syncthreads();
     if (e < p.n_expert) {
-        u32 start = 0;
-        for (int j = 0; j < e; j++) start += scount[j];
-        p.start[e] = start;
-        if (e == p.n_expert - 1) p.start[p.n_expert] = start + cnt;
-        u32 col = start;
-        for (int i = 0; i < npairs; i++) {
-            const int r = i / p.k_used, s = i % p.k_used;
-            if (p.sel[r * p.sel_stride + s] == (u32)e) {
-                p.perm[col] = (u32)r;
-                p.pos[i] = col;
-                col++;
+        if (staged) {
+            for (int i = lo; i < hi; i += 8) {
+                const u16x8 v = *(const u16x8*)(skeys + i);
+#pragma unroll
+                for (int b = 0; b < 8; b++) cnt += v[b] == (uint16_t)e;
             }
+        } else {
+            for (int i = lo; i < hi; i++) cnt += key_global(i) == (u32)e;
+        }
+    }
+    // Inclusive scan of the 1024 counts laid out expert-major (so a running sum is the
+    // column order): ten doubling steps between two LDS buffers.
+    const int me = e * nseg + seg;
+    u32* src = scount;
+    u32* dst = scount + 1024;
+    src[me] = cnt;
+    __syncthreads();
+    for (int off = 1; off < 1024; off <<= 1) {
+        const int i = threadIdx.x;
+        dst[i] = src[i] + (i >= off ? src[i - off] : 0u);
+        __syncthreads();
+        u32* t = src; src = dst; dst = t;
+    }
+    const u32 before = src[me] - cnt;
+    if (e < p.n_expert) {
+        if (seg == 0) p.start[e] = before;
+        if (e == p.n_expert - 1 && seg == nseg - 1) p.start[p.n_expert] = before + cnt;
+        u32 col = before;
+        auto place = [&](int i) {
+            p.perm[col] = (u32)(i / p.k_used);
+            p.pos[i] = col;
+            col++;
+        };
+        if (staged) {
+            for (int i = lo; i < hi; i += 8) {
+                const u16x8 v = *(const u16x8*)(skeys + i);
+#pragma unroll
+                for (int b = 0; b < 8; b++)
+                    if (v[b] == (uint16_t)e) place(i + b);
+            }
+        } else {
+            for (int i = lo; i < hi; i++)
+                if (key_global(i) == (u32)e) place(i);
         }
     }
 }
@@ -72,90 +129,149 @@ __device__ __forceinline__ float group_sum(float v) {
 
 __device__ __forceinline__ float silu_f32(float g) { return g / (1.0f + __expf(-g)); }
 
-// Quantize one column's activation (k floats, optionally silu(x)*x2) into the LDS
-// staging area `smem`; called by whole wavefronts, n4_pad a multiple of 64.
-__device__ __forceinline__ void moe_stage_column(uint8_t* smem, const float* x, const float* x2, int k,
-                                                 int per, int tid, int nthreads) {
-    const int n4 = k / 4, n4_pad = (n4 + 63) & ~63;
-    for (int g4 = tid; g4 < n4_pad; g4 += nthreads) {
-        f32x4 v = f32x4{0.f, 0.f, 0.f, 0.f};
-        if (g4 < n4) {
-            v = ((const f32x4*)x)[g4];
-            if (x2) {
-                f32x4 u = ((const f32x4*)x2)[g4];
-                v = f32x4{silu_f32(v.x) * u.x, silu_f32(v.y) * u.y, silu_f32(v.z) * u.z, silu_f32(v.w) * u.w};
-            }
+// --------------------------------------------------------- column activations
+// grid = (ceil(k/4/256), ncols), block = 256: one thread per four elements of a column.
+__device__ __forceinline__ void moe_quant_body(const MoeQuantArgs& p) {
+    const size_t c = blockIdx.y;
+    const size_t src = p.src ? p.src[c] : c;
+    const int g4 = blockIdx.x * 256 + threadIdx.x;
+    const bool live = g4 < p.k / 4;
+    f32x4 v = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (live) {
+        v = ((const f32x4*)(p.x + src * (size_t)p.k))[g4];
+        if (p.x2) {
+            f32x4 u = ((const f32x4*)(p.x2 + src * (size_t)p.k))[g4];
+            v = f32x4{silu_f32(v.x) * u.x, silu_f32(v.y) * u.y, silu_f32(v.z) * u.z, silu_f32(v.w) * u.w};
         }
-        stage_quantize4(smem, k, per, g4, v);
+    }
+    u32 m = max(max(abs_bits(v.x), abs_bits(v.y)), max(abs_bits(v.z), abs_bits(v.w)));
+    u32 amax = window_amax(live ? m : 0u, p.per);
+    float d;
+    i32 sum;
+    u32 qq = quantize4(v, amax, d, sum);
+    if (live) {
+        ((u32*)(p.q + c * (size_t)p.k))[g4] = qq;
+        if ((g4 & 3) == 0) p.s16[c * (size_t)(p.k / 16) + (g4 >> 2)] = (float)sum;
+        if ((g4 & 7) == 0) p.as[c * (size_t)(p.k / 32) + (g4 >> 3)] = d;
     }
 }
 
+// ------------------------------------------------------------- grouped matvec
+// grid = (shares, n_expert, matrices), block = nwaves * 64, dynamic LDS = JL_MOE_TB
+// staged columns.  A workgroup owns (expert, matrix, row share).  It copies up to eight
+// of the expert's quantized columns into LDS and streams its rows once for all of them.
+// A wavefront works in steps of 64/LPR rows (one slot per lane): it decodes the step's
+// scales and nibbles once, meets every staged column with them, and has the next step's
+// loads in flight meanwhile.  The first step is requested before the columns are staged,
+// so the copy overlaps HBM latency.  k % 256 == 0.
 template <int TYPE, int LPR>
 __device__ __forceinline__ void moe_matvec_body(const MoeMatVecArgs& p, uint8_t* smem) {
     typedef SlotTraits<TYPE> T;
-    constexpr int RW = 64 / LPR;  // weight rows per wavefront step
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+    constexpr int RW = 64 / LPR, U = JL_MOE_U;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = p.nwaves;
+    const int nthreads = nwaves * 64;
     const int e = blockIdx.y, mat = blockIdx.z;
+    JL_MOE_TRACE(0);
     const u32 c_lo = p.start[e], c_hi = p.start[e + 1];
     if (c_lo == c_hi) return;  // nobody chose this expert (uniform across the workgroup)
+    JL_MOE_TRACE(1);
     const int nslots = p.k / T::kElems;
     const int slot = lane % LPR, rw = lane / LPR;
-    const bool live = slot < nslots;
-    // this workgroup's share of the rows
-    const int share = (p.nrows + gridDim.x - 1) / gridDim.x;
+    const int share = (p.nrows + p.shares - 1) / p.shares;
     const int row_lo = blockIdx.x * share, row_hi = min(row_lo + share, p.nrows);
+    if (row_lo >= row_hi) return;
     const uint8_t* sheet = p.bank[mat] + (size_t)e * p.sheet_bytes;
     float* out = p.out[mat];
     const int act_bytes = (JL_ACT_LDS_BYTES(p.k) + 15) & ~15;
+    // steps of this wavefront: row groups (U * RW rows, stride nwaves of them) x slot groups
+    const int nsl = (nslots + LPR - 1) / LPR;
+    const int ngroups = (row_hi - row_lo - wave * U * RW + nwaves * U * RW - 1) / (nwaves * U * RW);  // may be <= 0
+    const int nsteps = max(ngroups, 0) * nsl;
+    auto step_row = [&](int it, int u) { return row_lo + (wave + (it / nsl) * nwaves) * U * RW + u * RW + rw; };
+    auto step_slot = [&](int it) { return slot + (it % nsl) * LPR; };
+    auto load_step = [&](int it, typename T::W (&w)[U]) {
+        const int s = min(step_slot(it), nslots - 1);
+#pragma unroll
+        for (int u = 0; u < U; u++)
+            T::load_w(sheet + (size_t)min(step_row(it, u), row_hi - 1) * p.row_bytes, s, w[u]);
+    };
+
+    typename T::W w_next[U];
+    if (nsteps > 0) load_step(0, w_next);
 
     for (u32 c0 = c_lo; c0 < c_hi; c0 += JL_MOE_TB) {
         const int ncol = min((u32)JL_MOE_TB, c_hi - c0);
-        // stage the pass's columns: two wavefront groups of 512 threads work on two columns at a time
+        // stage the pass's columns: int8 values, scales and sums, 16 bytes at a time
         {
-            const int half = threadIdx.x >= 512 ? 1 : 0, nth = blockDim.x >= 1024 ? 512 : blockDim.x;
-            const int ngroups = blockDim.x >= 1024 ? 2 : 1;
-            for (int j = (ngroups == 2 ? half : 0); j < ncol; j += ngroups) {
-                const u32 c = c0 + j;
-                const size_t src = p.src ? p.src[c] : c;
-                moe_stage_column(smem + (size_t)j * act_bytes, p.x + src * p.k,
-                                 p.x2 ? p.x2 + src * p.k : nullptr, p.k, p.per,
-                                 ngroups == 2 ? (int)threadIdx.x - 512 * half : (int)threadIdx.x, nth);
+            const int nq = p.k / 16, na = p.k / 128, ns = p.k / 64, per_col = nq + na + ns;
+            for (int i = threadIdx.x; i < ncol * per_col; i += nthreads) {
+                const int j = i / per_col, o = i - j * per_col;
+                const size_t c = c0 + j;
+                u32x4* dst = (u32x4*)(smem + (size_t)j * act_bytes);
+                if (o < nq) {
+                    dst[o] = ((const u32x4*)(p.q + c * (size_t)p.k))[o];
+                } else if (o < nq + na) {
+                    ((u32x4*)((uint8_t*)dst + p.k))[o - nq] = ((const u32x4*)(p.as + c * (size_t)(p.k / 32)))[o - nq];
+                } else {
+                    ((u32x4*)((uint8_t*)dst + p.k + (p.k / 32) * 4))[o - nq - na] =
+                        ((const u32x4*)(p.s16 + c * (size_t)(p.k / 16)))[o - nq - na];
+                }
             }
         }
         __syncthreads();
-        for (int r0 = row_lo + wave * RW; r0 < row_hi; r0 += nwaves * RW) {
-            const int r = min(r0 + rw, row_hi - 1);
-            float acc[JL_MOE_TB];
+        JL_MOE_TRACE(2);
+        if (c0 != c_lo && nsteps > 0) load_step(0, w_next);  // a further pass starts over
+        float acc[JL_MOE_TB][U];
 #pragma unroll
-            for (int j = 0; j < JL_MOE_TB; j++) acc[j] = 0.f;
-            for (int s = slot; s < nslots; s += LPR) {
-                typename T::W w;
-                T::load_w(sheet + (size_t)r * p.row_bytes, s, w);
+        for (int j = 0; j < JL_MOE_TB; j++)
 #pragma unroll
-                for (int j = 0; j < JL_MOE_TB; j++) {
-                    if (j < ncol) {
-                        typename T::Act a;
-                        T::load_act(act_lds_views(smem + (size_t)j * act_bytes, p.k), s, a);
-                        acc[j] += T::dot(w, s, a);
-                    }
-                }
-            }
+            for (int u = 0; u < U; u++) acc[j][u] = 0.f;
+        for (int it = 0; it < nsteps; it++) {
+            typename T::Prep P[U];
+            const int s = step_slot(it), sc = min(s, nslots - 1);
+            const bool live = s < nslots;
+#pragma unroll
+            for (int u = 0; u < U; u++) T::prep(w_next[u], sc, P[u]);
+            if (it + 1 < nsteps) load_step(it + 1, w_next);
 #pragma unroll
             for (int j = 0; j < JL_MOE_TB; j++) {
                 if (j < ncol) {
-                    float t = group_sum<LPR>(live ? acc[j] : 0.f);
-                    if (slot == LPR - 1 && r0 + rw < row_hi) out[(size_t)(c0 + j) * p.nrows + r0 + rw] = t;
+                    typename T::Act a;
+                    T::load_act(act_lds_views(smem + (size_t)j * act_bytes, p.k), sc, a);
+#pragma unroll
+                    for (int u = 0; u < U; u++) {
+                        const float v = T::dotp(P[u], a);
+                        acc[j][u] += live ? v : 0.f;
+                    }
                 }
+                // one column's activation in registers at a time
+                asm volatile("" ::: "memory");
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (it % nsl == nsl - 1) {  // the rows' last slot group: reduce and store
+#pragma unroll
+                for (int j = 0; j < JL_MOE_TB; j++)
+#pragma unroll
+                    for (int u = 0; u < U; u++) {
+                        if (j < ncol) {
+                            const int r = step_row(it, u);
+                            float t = group_sum<LPR>(acc[j][u]);
+                            if (slot == LPR - 1 && r < row_hi) out[(size_t)(c0 + j) * p.nrows + r] = t;
+                        }
+                        acc[j][u] = 0.f;
+                    }
             }
         }
+        JL_MOE_TRACE(3);
         __syncthreads();
     }
+    JL_MOE_TRACE(4);
 }
 
 // resid[r][n] += sum over the row's k_used experts, ascending expert id, of
 // wt[r][s] * y[pos[r*k_used+s]][n].  One thread per (row, n).
 __device__ __forceinline__ void moe_combine_body(const MoeCombineArgs& p) {
-    const int n = blockIdx.x * blockDim.x + threadIdx.x;
+    const int n = blockIdx.x * 256 + threadIdx.x;
     const int r = blockIdx.y;
     if (n >= p.n_embd) return;
     // order the row's slots by expert id (k_used is small: insertion sort in registers)

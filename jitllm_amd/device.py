@@ -194,12 +194,12 @@ class Device:
                                                      n_expert, _ptr(start), _ptr(perm), _ptr(pos), stream),
                             "jl_moe_group_dev")
 
-    def moe_matvec_dev(self, out0, out1, t, bank0, bank1, x, x2, src, start, n_expert, nrows, k,
+    def moe_matvec_dev(self, out0, out1, t, bank0, bank1, x, x2, src, start, n_expert, ncols, nrows, k,
                        stream=None):
         opt = lambda a: None if a is None else _ptr(a)
         return self._served(self._l.jl_moe_matvec_dev(self._ctx, _ptr(out0), opt(out1), t, _ptr(bank0),
                                                       opt(bank1), _ptr(x), opt(x2), opt(src), _ptr(start),
-                                                      n_expert, nrows, k, stream), "jl_moe_matvec_dev")
+                                                      n_expert, ncols, nrows, k, stream), "jl_moe_matvec_dev")
 
     def moe_combine_dev(self, resid, y, wt, sel, sel_stride, pos, rows, k_used, n_embd, stream=None):
         return self._served(self._l.jl_moe_combine_dev(self._ctx, _ptr(resid), _ptr(y), _ptr(wt), _ptr(sel),

@@ -89,14 +89,14 @@ def test_grouped_matvec_vs_oracle(dev, devbuf, t, nrows, k):
     o0 = devbuf(shape=(used, nrows), dtype=np.float32, fill=np.float32(4e30))
     o1 = devbuf(shape=(used, nrows), dtype=np.float32, fill=np.float32(4e30))
     assert dev.moe_matvec_dev(o0.ptr, o1.ptr, t, b0.ptr, b1.ptr, xd.ptr, None, dperm.ptr, dstart.ptr,
-                              n_expert, nrows, k)
+                              n_expert, used, nrows, k)
     dev.synchronize()
     assert nmse(o0.get(), want0) <= 1e-10 and nmse(o1.get(), want1) <= 1e-10
     # SwiGLU form: column c reads silu(x[c]) * x2[c], no gather
     g = np.stack([synth.activations(k, seed=300 + c) for c in range(used)])
     u = np.stack([synth.activations(k, seed=400 + c) for c in range(used)])
     gd, ud = devbuf(g), devbuf(u)
-    assert dev.moe_matvec_dev(o0.ptr, None, t, b0.ptr, None, gd.ptr, ud.ptr, None, dstart.ptr, n_expert, nrows, k)
+    assert dev.moe_matvec_dev(o0.ptr, None, t, b0.ptr, None, gd.ptr, ud.ptr, None, dstart.ptr, n_expert, used, nrows, k)
     dev.synchronize()
     got = o0.get()
     h = (silu(g) * u.astype(np.float64)).astype(np.float32)
