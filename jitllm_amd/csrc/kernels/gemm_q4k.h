@@ -23,8 +23,7 @@
 // (magic-number nibble unpack with packed-f16 FMAs, eight K values per 32-bit
 // word of nibbles); activations were laid out by the prep kernel in exactly the
 // stage's LDS image -- same K permutation, same padding -- so their stage is one
-// contiguous copy, issued as direct global->LDS loads.  Two stages are
-// double-buffered.  Four consumer wavefronts each compute 64 tokens x 64 rows as
+// contiguous copy.  Two stages are double-buffered.  Four consumer wavefronts each compute 64 tokens x 64 rows as
 // 2x2 MFMA tiles while four producer wavefronts fill the next stage; tokens are the MFMA M dimension so a lane owns one weight row
 // (its scales are scalars) and output stores run along rows.
 #pragma once
@@ -35,6 +34,10 @@
 // Phase marker for profiling builds; expands to nothing in the product.
 #ifndef JL_TRACE
 #define JL_TRACE(i)
+#endif
+#ifndef JL_GEMM_SKIP_PRODUCER
+#define JL_GEMM_SKIP_PRODUCER 0
+#define JL_GEMM_SKIP_CONSUMER 0
 #endif
 
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
@@ -122,16 +125,19 @@ __device__ __forceinline__ f16x2 nib_pair(u32 w, int shift) {
 __device__ __forceinline__ void gemm_store_w(const GemmWRegs& r, int row, int hh, int half, _Float16* sw,
                                              float* sscale) {
     const int g = 2 * half + hh;
-    u32 sc[8], mn[8];
-#pragma unroll
-    for (int j = 0; j < 8; j++) scale_min_k4(j, r.hdr.y, r.hdr.z, r.hdr.w, sc[j], mn[j]);
-    // scales of sub-blocks 2g (low nibbles) and 2g+1 (high nibbles); g is not a
-    // compile-time constant, so select
-    u32 slo = sc[0], shi = sc[1];
-#pragma unroll
-    for (int j = 1; j < 4; j++) {
-        slo = g == j ? sc[2 * j] : slo;
-        shi = g == j ? sc[2 * j + 1] : shi;
+    // scales of sub-blocks 2g (low nibbles) and 2g+1 (high nibbles), straight from the
+    // packed bytes (format/quant/dequant.go:360-365)
+    u32 slo, shi;
+    {
+        const int sh = 16 * (g & 1);
+        const u32 A = r.hdr.y >> sh, C = r.hdr.w >> sh;
+        if (half == 0) {
+            slo = A & 63;
+            shi = (A >> 8) & 63;
+        } else {
+            slo = (C & 0xF) | (((A >> 6) & 3) << 4);
+            shi = ((C >> 8) & 0xF) | (((A >> 14) & 3) << 4);
+        }
     }
     const _Float16 flo = (_Float16)(float)slo, fhi = (_Float16)(float)shi;
     const f16x2 mlo = {flo, flo}, mhi = {fhi, fhi};
@@ -155,7 +161,11 @@ __device__ __forceinline__ void gemm_store_w(const GemmWRegs& r, int row, int hh
         const float mul = hh ? 64.0f : 1.0f;
         f16x8 mm;
 #pragma unroll
-        for (int j = 0; j < 8; j++) mm[j] = (_Float16)((float)mn[j] * mul);
+        for (int j = 0; j < 8; j++) {
+            u32 scj, mnj;
+            scale_min_k4(j, r.hdr.y, r.hdr.z, r.hdr.w, scj, mnj);
+            mm[j] = (_Float16)((float)mnj * mul);
+        }
         *(f16x8*)(sw + row * JL_GEMM_STRIDE + 128 + 8 * hh) = mm;
         if (hh == 0) {
             sscale[2 * row] = half_bits_to_f32((uint16_t)(r.hdr.x & 0xFFFF));
@@ -164,163 +174,192 @@ __device__ __forceinline__ void gemm_store_w(const GemmWRegs& r, int row, int hh
     }
 }
 
-// Copy one activation stage (128 tokens x 304 B, contiguous in HBM) into LDS with
-// direct global->LDS loads: each wavefront instruction moves 64 lanes x 16 B to
-// 1 KiB of consecutive LDS.
-__device__ __forceinline__ void gemm_load_a_stage(const _Float16* src, _Float16* dst) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int nchunks = JL_GEMM_STAGE_BYTES / 1024;  // 38 wavefront-sized pieces
-    for (int c = wave & 3; c < nchunks; c += 4) {
-        const uint8_t* g = (const uint8_t*)src + (size_t)c * 1024 + lane * 16;
-        uint8_t* l = (uint8_t*)dst + c * 1024;
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g,
-                                         (__attribute__((address_space(3))) void*)l, 16, 0, 0);
+// One activation stage is 128 tokens x 304 B, contiguous in HBM in exactly its LDS
+// image: 2432 vectors of 16 B.  All 512 threads carry it through registers, loaded one
+// step ahead -- the 256 consumer threads four vectors each (their registers are nearly
+// all accumulators), the 256 producer threads the other 1408.  Plain vector loads issue
+// in a few cycles each, where the direct global->LDS form costs the issuing wavefront
+// about 150 cycles an instruction, and spread over every wavefront the copy hides under
+// the consumers' matrix instructions.
+#define JL_GEMM_STAGE_VECS (JL_GEMM_STAGE_BYTES / 16)
+template <int N, int FIRST>
+struct GemmARegs {
+    u32x4 v[N];
+    // tid = index within the role (0..255)
+    __device__ __forceinline__ void load(const _Float16* src, int tid) {
+        const u32x4* s = (const u32x4*)src;
+#pragma unroll
+        for (int i = 0; i < N; i++) v[i] = s[min(FIRST + tid + 256 * i, JL_GEMM_STAGE_VECS - 1)];
     }
-}
+    __device__ __forceinline__ void store(_Float16* dst, int tid) const {
+        u32x4* d = (u32x4*)dst;
+#pragma unroll
+        for (int i = 0; i < N; i++)
+            if (FIRST + 256 * (i + 1) <= JL_GEMM_STAGE_VECS || FIRST + tid + 256 * i < JL_GEMM_STAGE_VECS)
+                d[FIRST + tid + 256 * i] = v[i];
+    }
+};
+typedef GemmARegs<4, 0> GemmARegsConsumer;      // vectors 0 .. 1023
+typedef GemmARegs<6, 1024> GemmARegsProducer;   // vectors 1024 .. 2431
 
-__device__ __forceinline__ void gemm_q4k_body(const GemmArgs& p, uint8_t* smem) {
-    // LDS: activation stages [2], weight stages [2], row scales [2][128][2], token scales [2][128]
-    _Float16* sA = (_Float16*)smem;
-    _Float16* sW = sA + 2 * JL_GEMM_STAGE_HALFS;
-    float* sScale = (float*)(sW + 2 * JL_GEMM_STAGE_HALFS);
-    float* sDa = sScale + 2 * 2 * JL_GEMM_TILE;
-
-    // Eight wavefronts, two per SIMD: wavefronts 0-3 are consumers (LDS -> matrix cores
-    // -> epilogue, one 64x64 corner each), wavefronts 4-7 are producers (HBM -> dequantize
-    // -> LDS, and the direct activation loads).  A SIMD then always has vector work
-    // from its producer to issue under its consumer's matrix instructions.
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const bool producer = wave >= 4;
-    const int tid = threadIdx.x & 255;  // index within the role
-    const int t0 = blockIdx.x * JL_GEMM_TILE, r0 = blockIdx.y * JL_GEMM_TILE;
-    const int nsb = p.k / 256, nsteps = 2 * nsb;
+// Producer wavefronts (four): HBM -> registers -> (dequantize) -> LDS, one stage ahead
+// of the consumers, with the stage after that in flight in registers.
+__device__ __forceinline__ void gemm_producer(const GemmArgs& p, _Float16* sA, _Float16* sW, float* sScale,
+                                              float* sDa, int tid, int t0, int r0, int nsteps) {
     const int wrow = min(r0 + (tid >> 1), p.nrows - 1), hh = tid & 1;
-    const int wt = ((wave >> 1) & 1) * 64, wr = (wave & 1) * 64;  // a consumer's 64x64 corner
-
     auto a_src = [&](int step) {
         return (const _Float16*)p.bq + ((size_t)step * p.tok_pad + t0) * JL_GEMM_STRIDE;
     };
+    GemmWRegs wreg;
+    GemmARegsProducer areg;
+    areg.load(a_src(0), tid);
+    gemm_load_w(p, wrow, 0, hh, wreg);
+    areg.store(sA, tid);
+    gemm_store_w(wreg, tid >> 1, hh, 0, sW, sScale);
+    areg.load(a_src(min(1, nsteps - 1)), tid);
+    gemm_load_w(p, wrow, 0, 2 + hh, wreg);
+    float da_reg = p.da[t0 + (tid & (JL_GEMM_TILE - 1))];
+    lds_barrier();
+    for (int step = 0; step < nsteps; step++) {
+        JL_TRACE(0);
+        if (step + 1 < nsteps && !JL_GEMM_SKIP_PRODUCER) {
+            const int nb = (step & 1) ^ 1, nhalf = (step + 1) & 1, nsbi = (step + 1) >> 1;
+            // (a) the next stage, loaded into registers a step ago, goes to LDS.  A second
+            // half also carries the super-block's row scales and token scales.
+#ifdef JL_TRACE_PRODUCER
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            JL_TRACE(1);
+#endif
+            areg.store(sA + nb * JL_GEMM_STAGE_HALFS, tid);
+#ifdef JL_TRACE_PRODUCER
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            JL_TRACE(2);
+#endif
+            gemm_store_w(wreg, tid >> 1, hh, nhalf, sW + nb * JL_GEMM_STAGE_HALFS,
+                         sScale + (nsbi & 1) * 2 * JL_GEMM_TILE);
+            if (nhalf == 1 && tid < JL_GEMM_TILE) sDa[(nsbi & 1) * JL_GEMM_TILE + tid] = da_reg;
+#ifdef JL_TRACE_PRODUCER
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            JL_TRACE(3);
+#else
+            JL_TRACE(1);
+#endif
+            // (b) issue the loads of the stage after it
+            const int s2 = min(step + 2, nsteps - 1);
+            areg.load(a_src(s2), tid);
+            gemm_load_w(p, wrow, s2 >> 1, 2 * (s2 & 1) + hh, wreg);
+            da_reg = p.da[(size_t)(s2 >> 1) * p.tok_pad + t0 + (tid & (JL_GEMM_TILE - 1))];
+        }
+#ifndef JL_TRACE_PRODUCER
+        JL_TRACE(2);
+        JL_TRACE(3);
+#endif
+        JL_TRACE(4);
+        // the next stage is complete in LDS once every producer has passed here; the
+        // register loads of (b) stay in flight across the barrier
+        lds_barrier();
+        JL_TRACE(5);
+    }
+}
 
-    f32x16 out[2][2];
+// Consumer wavefronts (four, one 64-token x 64-row corner each): LDS -> matrix cores,
+// fragments fetched a K-step ahead of the instructions that use them; once per
+// super-block the minimum columns and the epilogue  out += d_a * (d * P - dmin * M).
+__device__ __forceinline__ void gemm_consumer(const GemmArgs& p, _Float16* sA, const _Float16* sW,
+                                              const float* sScale, const float* sDa, int wave, int lane,
+                                              int t0, int r0, int nsteps) {
+    const int wt = ((wave >> 1) & 1) * 64, wr = (wave & 1) * 64;
+    const int arow = lane & 31, kg = lane >> 5;
+    f32x16 out[2][2], accP[2][2];
 #pragma unroll
     for (int i = 0; i < 2; i++)
 #pragma unroll
         for (int j = 0; j < 2; j++)
 #pragma unroll
             for (int e = 0; e < 16; e++) out[i][j][e] = 0.f;
-
-    // prologue (producers): stage 0 into buffer 0; stage 1's weights and token scales
-    // into registers
-    GemmWRegs wreg;
-    float da_reg = 0.f;
-    if (producer) {
-        gemm_load_w(p, wrow, 0, hh, wreg);
-        gemm_store_w(wreg, tid >> 1, hh, 0, sW, sScale);
-        gemm_load_a_stage(a_src(0), sA);
-        gemm_load_w(p, wrow, 0, 2 + hh, wreg);
-        da_reg = p.da[t0 + (tid & (JL_GEMM_TILE - 1))];
-        asm volatile("s_waitcnt vmcnt(4)" ::: "memory");  // the direct loads; 3 weight + 1 scale load stay in flight
-    }
+    // this wavefront's share of the activation copy
+    const int atid = threadIdx.x;  // consumers are threads 0..255
+    auto a_src = [&](int step) {
+        return (const _Float16*)p.bq + ((size_t)step * p.tok_pad + t0) * JL_GEMM_STRIDE;
+    };
+    GemmARegsConsumer areg;
+    areg.load(a_src(0), atid);
+    areg.store(sA, atid);
+    areg.load(a_src(min(1, nsteps - 1)), atid);
     lds_barrier();
-
-    f32x16 accP[2][2];
     for (int step = 0; step < nsteps; step++) {
         const int buf = step & 1, half = step & 1, sb = step >> 1;
         const _Float16* a = sA + buf * JL_GEMM_STAGE_HALFS;
         const _Float16* w = sW + buf * JL_GEMM_STAGE_HALFS;
         JL_TRACE(0);
-        if (producer && step + 1 < nsteps) {
-            const int nb = buf ^ 1, nhalf = (step + 1) & 1, nsbi = (step + 1) >> 1;
-            // (a) the next stage's weights: registers (loaded a step ago) -> LDS.  Nothing
-            // newer has been issued yet, so this waits for exactly those loads.  A second
-            // half also carries the super-block's row scales and token scales.
-            gemm_store_w(wreg, tid >> 1, hh, nhalf, sW + nb * JL_GEMM_STAGE_HALFS,
-                         sScale + (nsbi & 1) * 2 * JL_GEMM_TILE);
-            if (nhalf == 1 && tid < JL_GEMM_TILE) sDa[(nsbi & 1) * JL_GEMM_TILE + tid] = da_reg;
-            JL_TRACE(1);
-            // (b) issue, in this order: the next stage's activations (direct to LDS), then
-            // the weights and token scales of the stage after it (to registers)
-            gemm_load_a_stage(a_src(step + 1), sA + nb * JL_GEMM_STAGE_HALFS);
-            const int s2 = min(step + 2, nsteps - 1);
-            gemm_load_w(p, wrow, s2 >> 1, 2 * (s2 & 1) + hh, wreg);
-            da_reg = p.da[(size_t)(s2 >> 1) * p.tok_pad + t0 + (tid & (JL_GEMM_TILE - 1))];
+        if (step + 1 < nsteps) {
+            areg.store(sA + (buf ^ 1) * JL_GEMM_STAGE_HALFS, atid);
+            areg.load(a_src(min(step + 2, nsteps - 1)), atid);
         }
+        JL_TRACE(1);
         JL_TRACE(2);
-        // (c) matrix work on the current stage
-        const int arow = lane & 31, kg = lane >> 5;
-        if (!producer) {
-        if (half == 0) {
+        if (!JL_GEMM_SKIP_CONSUMER) {
+            if (half == 0) {
 #pragma unroll
-            for (int i = 0; i < 2; i++)
+                for (int i = 0; i < 2; i++)
 #pragma unroll
-                for (int j = 0; j < 2; j++)
+                    for (int j = 0; j < 2; j++)
 #pragma unroll
-                    for (int e = 0; e < 16; e++) accP[i][j][e] = 0.f;
-        }
-        // Fragments are fetched one K-step ahead of the matrix instructions that use
-        // them; the last prefetch of a second half fetches the minimum columns.
-        const _Float16* ap0 = a + (wt + arow) * JL_GEMM_STRIDE + 8 * kg;
-        const _Float16* wp0 = w + (wr + arow) * JL_GEMM_STRIDE + 8 * kg;
-        f16x8 af[2][2], wf[2][2];
-#pragma unroll
-        for (int i = 0; i < 2; i++) {
-            af[0][i] = *(const f16x8*)(ap0 + 32 * i * JL_GEMM_STRIDE);
-            wf[0][i] = *(const f16x8*)(wp0 + 32 * i * JL_GEMM_STRIDE);
-        }
-#pragma unroll
-        for (int ks = 0; ks < 8; ks++) {
-            const int cur = ks & 1, nxt = cur ^ 1;
-            if (ks < 7 || half == 1) {
-#pragma unroll
-                for (int i = 0; i < 2; i++) {
-                    af[nxt][i] = *(const f16x8*)(ap0 + 32 * i * JL_GEMM_STRIDE + 16 * (ks + 1));
-                    wf[nxt][i] = *(const f16x8*)(wp0 + 32 * i * JL_GEMM_STRIDE + 16 * (ks + 1));
-                }
+                        for (int e = 0; e < 16; e++) accP[i][j][e] = 0.f;
             }
-#pragma unroll
-            for (int i = 0; i < 2; i++)
-#pragma unroll
-                for (int j = 0; j < 2; j++)
-                    accP[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[cur][i], wf[cur][j], accP[i][j], 0, 0, 0);
-        }
-        JL_TRACE(3);
-        if (half == 1) {
-            // the 16 minimum columns: M, then the super-block's epilogue
-            //   out += d_a * (d * P - dmin * M)
-            const f32x16 zero = {0};
-            const float* ssc = sScale + (sb & 1) * 2 * JL_GEMM_TILE;
-            const float* sda = sDa + (sb & 1) * JL_GEMM_TILE;
-#pragma unroll
-            for (int j = 0; j < 2; j++) {
-                const float dd = ssc[2 * (wr + 32 * j + arow)];
-                const float dmin = ssc[2 * (wr + 32 * j + arow) + 1];
-                f32x16 accM[2];
-                accM[0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[0][0], wf[0][j], zero, 0, 0, 0);
-                accM[1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[0][1], wf[0][j], zero, 0, 0, 0);
+            const _Float16* ap0 = a + (wt + arow) * JL_GEMM_STRIDE + 8 * kg;
+            const _Float16* wp0 = w + (wr + arow) * JL_GEMM_STRIDE + 8 * kg;
+            f16x8 af[2][2], wf[2][2];
+            auto fetch = [&](int slot, int ks) {
 #pragma unroll
                 for (int i = 0; i < 2; i++) {
+                    af[slot][i] = *(const f16x8*)(ap0 + 32 * i * JL_GEMM_STRIDE + 16 * ks);
+                    wf[slot][i] = *(const f16x8*)(wp0 + 32 * i * JL_GEMM_STRIDE + 16 * ks);
+                }
+            };
+            fetch(0, 0);
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                    for (int e = 0; e < 16; e++) {
-                        const int tk = wt + 32 * i + 8 * (e >> 2) + 4 * kg + (e & 3);
-                        const float u = fmaf(dd, accP[i][j][e], -(dmin * accM[i][e]));
-                        out[i][j][e] = fmaf(sda[tk], u, out[i][j][e]);
+            for (int ks = 0; ks < 8; ks++) {
+                // K-step 8 of a second half is the sixteen minimum columns
+                // (the scheduling fences keep the fetch a K-step ahead of its use; left
+                // alone the compiler re-reads fragments right before the instruction needing them)
+                if (ks + 1 < 8 || half == 1) fetch((ks + 1) & 1, ks + 1);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int i = 0; i < 2; i++)
+#pragma unroll
+                    for (int j = 0; j < 2; j++)
+                        accP[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[ks & 1][i], wf[ks & 1][j], accP[i][j], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            JL_TRACE(3);
+            if (half == 1) {
+                const f32x16 zero = {0};
+                const float* ssc = sScale + (sb & 1) * 2 * JL_GEMM_TILE;
+                const float* sda = sDa + (sb & 1) * JL_GEMM_TILE;
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    const float dd = ssc[2 * (wr + 32 * j + arow)];
+                    const float dmin = ssc[2 * (wr + 32 * j + arow) + 1];
+#pragma unroll
+                    for (int i = 0; i < 2; i++) {
+                        const f32x16 accM = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[0][i], wf[0][j], zero, 0, 0, 0);
+#pragma unroll
+                        for (int e = 0; e < 16; e++) {
+                            const int tk = wt + 32 * i + 8 * (e >> 2) + 4 * kg + (e & 3);
+                            const float u = fmaf(dd, accP[i][j][e], -(dmin * accM[e]));
+                            out[i][j][e] = fmaf(sda[tk], u, out[i][j][e]);
+                        }
                     }
                 }
             }
         }
-        }  // consumer
         JL_TRACE(4);
-        // (d) the next stage's direct loads must have landed before anyone reads it.
-        // Loads return in order; the four register loads of (b) were issued after them
-        // and stay in flight across the barrier.
-        if (producer) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
         lds_barrier();
         JL_TRACE(5);
     }
-
     // store: lane = row (contiguous in memory), register = token
-    if (producer) return;
-    const int arow = lane & 31, kg = lane >> 5;
 #pragma unroll
     for (int j = 0; j < 2; j++) {
         const int r = r0 + wr + 32 * j + arow;
@@ -333,4 +372,21 @@ __device__ __forceinline__ void gemm_q4k_body(const GemmArgs& p, uint8_t* smem) 
                 if (t < p.ntok) p.out[(size_t)t * p.nrows + r] = out[i][j][e];
             }
     }
+}
+
+__device__ __forceinline__ void gemm_q4k_body(const GemmArgs& p, uint8_t* smem) {
+    // LDS: activation stages [2], weight stages [2], row scales [2][128][2], token scales [2][128]
+    _Float16* sA = (_Float16*)smem;
+    _Float16* sW = sA + 2 * JL_GEMM_STAGE_HALFS;
+    float* sScale = (float*)(sW + 2 * JL_GEMM_STAGE_HALFS);
+    float* sDa = sScale + 2 * 2 * JL_GEMM_TILE;
+    // Eight wavefronts, two per SIMD: wavefronts 0-3 are consumers, 4-7 producers, so a
+    // SIMD always has vector work from its producer to issue under its consumer's matrix
+    // instructions.  The two roles are separate loops (their registers never coexist) that
+    // meet at the same barriers: one after the prologue, one per stage.
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int t0 = blockIdx.x * JL_GEMM_TILE, r0 = blockIdx.y * JL_GEMM_TILE;
+    const int nsteps = 2 * (p.k / 256);
+    if (wave >= 4) gemm_producer(p, sA, sW, sScale, sDa, threadIdx.x & 255, t0, r0, nsteps);
+    else gemm_consumer(p, sA, sW, sScale, sDa, wave, lane, t0, r0, nsteps);
 }
