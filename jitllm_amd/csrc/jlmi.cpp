@@ -240,12 +240,13 @@ int resident_weight(jl_ctx* c, const void* w, size_t bytes, void** dev) {
 
 constexpr int kGemmTile = 128;         // tokens and rows per workgroup (kernels/gemm_q4k.h)
 constexpr int kGemmStride = 152;       // f16 per stage row
-constexpr unsigned kGemmLdsBytes = 4u * kGemmTile * kGemmStride * 2u + 2u * 2u * kGemmTile * 4u + 2u * kGemmTile * 4u;
+constexpr unsigned kGemmLdsBytes = 2u * kGemmTile * kGemmStride * 2u + 2u * 2u * kGemmTile * 4u + 2u * kGemmTile * 4u;
+constexpr size_t kGemmAStageBytes = 9 * 1024;  // per 32 tokens and stage: nine fragments of 64 lanes x 16 B
 
 size_t gemm_ws_need(int ntok, int k) {
     size_t tok_pad = ((size_t)ntok + kGemmTile - 1) / kGemmTile * kGemmTile;
     size_t nsb = (size_t)k / 256;
-    return nsb * 2 * tok_pad * kGemmStride * 2 + nsb * tok_pad * 4;
+    return nsb * 2 * (tok_pad / 32) * kGemmAStageBytes + nsb * tok_pad * 4;
 }
 
 int gemm_ws_ensure(jl_ctx* c, size_t need) {
@@ -268,7 +269,7 @@ int gemm_q4k_launch(jl_ctx* c, float* out, const void* w, const float* x, int nr
     int rc = gemm_ws_ensure(c, gemm_ws_need(ntok, k));
     if (rc != JL_OK) return rc;
     uint16_t* bq = (uint16_t*)c->gemm_ws;
-    float* da = (float*)((char*)c->gemm_ws + (size_t)nsb * 2 * tok_pad * kGemmStride * 2);
+    float* da = (float*)((char*)c->gemm_ws + (size_t)nsb * 2 * (tok_pad / 32) * kGemmAStageBytes);
     GemmPrepArgs pa;
     pa.x = x; pa.bq = bq; pa.da = da; pa.ntok = ntok; pa.tok_pad = tok_pad; pa.k = k;
     void* pp[] = {&pa};

@@ -19,7 +19,7 @@ struct MatVecArgs {
 };
 
 // Activation preparation for the Q4_K prefill GEMM: quantize x and lay it out
-// as the GEMM's LDS stages, bq [k/256][2][tok_pad][152] f16, da [k/256][tok_pad].
+// in matrix-fragment order, bq [k/128 stages][tok_pad/32][9][64][8] f16, da [k/256][tok_pad].
 struct GemmPrepArgs {
     const float* x;      // [ntok][k]
     uint16_t* bq;        // f16 bits

@@ -75,7 +75,7 @@ JL_PACKED_KERNEL(q6k, JL_Q6_K, 64, 4) JL_PACKED_KERNEL(q6k, JL_Q6_K, 32, 4) JL_P
 // ------------------------------------------------------------ prefill GEMM
 // grid = (k/256, tok_pad/4), block = 256: one wavefront per (token, super-block)
 extern "C" __global__ __launch_bounds__(256) void jl_gemm_prep_q4k(GemmPrepArgs p) { gemm_prep_q4k_body(p); }
-// grid = (tok_pad/128, ceil(nrows/128)), block = 512 (4 consumer + 4 producer wavefronts)
+// grid = (tok_pad/128, ceil(nrows/128)), block = 512 (two wavefronts per SIMD)
 extern "C" __global__ __launch_bounds__(512) void jl_gemm_q4k(GemmArgs p) { gemm_q4k_body(p, jl_smem); }
 
 // ------------------------------------------------------- mixture of experts
