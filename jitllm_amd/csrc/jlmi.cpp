@@ -30,6 +30,7 @@ struct Tuning {
     int rpw = 0, block = 0, grid = 0;
     int packed_rw = 0, packed_block = 0;
     int moe_shares = 0;
+    int gemm_rows = 0;
 };
 
 struct Resident {
@@ -240,7 +241,10 @@ int resident_weight(jl_ctx* c, const void* w, size_t bytes, void** dev) {
 
 constexpr int kGemmTile = 128;         // tokens and rows per workgroup (kernels/gemm_q4k.h)
 constexpr int kGemmStride = 152;       // f16 per stage row
-constexpr unsigned kGemmLdsBytes = 2u * kGemmTile * kGemmStride * 2u + 2u * 2u * kGemmTile * 4u + 2u * kGemmTile * 4u;
+constexpr unsigned gemm_lds_bytes(int rows) {   // two weight stages, row scales, token scales
+    return 2u * rows * kGemmStride * 2u + 2u * 2u * rows * 4u + 2u * kGemmTile * 4u;
+}
+constexpr unsigned kGemmLdsBytes = gemm_lds_bytes(128);
 constexpr size_t kGemmAStageBytes = 9 * 1024;  // per 32 tokens and stage: nine fragments of 64 lanes x 16 B
 
 size_t gemm_ws_need(int ntok, int k) {
@@ -279,8 +283,10 @@ int gemm_q4k_launch(jl_ctx* c, float* out, const void* w, const float* x, int nr
     ga.out = out; ga.w = (const uint8_t*)w; ga.bq = bq; ga.da = da;
     ga.nrows = nrows; ga.k = k; ga.ntok = ntok; ga.tok_pad = tok_pad; ga.row_bytes = nsb * 144;
     void* gp[] = {&ga};
-    return launch(c, "jl_gemm_q4k", (unsigned)(tok_pad / kGemmTile),
-                  (unsigned)((nrows + kGemmTile - 1) / kGemmTile), 512, kGemmLdsBytes, st, gp);
+    // 64-row workgroups, two to a CU, unless asked for the 128-row form
+    const int rows = c->tune.gemm_rows == 128 ? 128 : 64;
+    return launch(c, rows == 128 ? "jl_gemm_q4k_r128" : "jl_gemm_q4k_r64", (unsigned)(tok_pad / kGemmTile),
+                  (unsigned)((nrows + rows - 1) / rows), rows == 128 ? 512 : 256, gemm_lds_bytes(rows), st, gp);
 }
 
 // out [ntok][nrows] = x [ntok][k] W^T on device operands: the matrix-core GEMM where it
@@ -522,7 +528,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     if (e != hipSuccess)
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
-    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_q4k", "jl_moe_group", "jl_moe_quant", "jl_moe_combine", "jl_mxfp4_gemm", "jl_mxfp4_matvec",
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_q4k_r64", "jl_gemm_q4k_r128", "jl_moe_group", "jl_moe_quant", "jl_moe_combine", "jl_mxfp4_gemm", "jl_mxfp4_matvec",
                                       "jl_pack_weights", "jl_unpack_q4k"};
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int rw : {16, 32, 64})
@@ -597,6 +603,7 @@ int jl_set_tuning(jl_ctx* c, const char* key, int value) {
     else if (!strcmp(key, "packed.rw")) c->tune.packed_rw = value;
     else if (!strcmp(key, "packed.block")) c->tune.packed_block = value;
     else if (!strcmp(key, "moe.shares")) c->tune.moe_shares = value;
+    else if (!strcmp(key, "gemm.rows")) c->tune.gemm_rows = value;
     else if (!strcmp(key, "gemm.min_tok")) c->gemm_min_tok = value > 0 ? value : 8;
     else return fail(c, JL_ERR_ARG, "unknown tuning key %s", key);
     return JL_OK;

@@ -43,18 +43,13 @@
 #ifndef JL_TRACE
 #define JL_TRACE(i)
 #endif
-#ifndef JL_X_NO_EPI
-#define JL_X_NO_EPI 0
-#endif
 
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-#define JL_GEMM_TILE 128          // tokens and rows per workgroup
+#define JL_GEMM_TILE 128          // tokens per workgroup (rows: 64 per group of four wavefronts)
 #define JL_GEMM_STRIDE 152        // f16 per LDS row of a stage: 144 used + 8 pad (304 B, odd multiple of 16 B)
-#define JL_GEMM_STAGE_HALFS (JL_GEMM_TILE * JL_GEMM_STRIDE)
-#define JL_GEMM_STAGE_BYTES (JL_GEMM_STAGE_HALFS * 2)
 // Activation fragments: 64 lanes x 8 f16 each; nine per (stage, 32 tokens): eight
 // K-steps and the minimum columns (used in second halves only).
 #define JL_GEMM_AFRAG_HALFS 512
@@ -208,16 +203,22 @@ __device__ __forceinline__ void gemm_w_mins(const GemmWRegs& r, int row, int hh,
     }
 }
 
-// grid = (tok_pad/128, ceil(nrows/128)), block = 512 (eight wavefronts), dynamic LDS =
-// two weight stages + row scales [2][128][2] + token scales [2][128].
+// RH = groups of four wavefronts in the workgroup, each group 64 rows: RH = 2 is the
+// 128 x 128 tile on eight wavefronts; RH = 1 a 128-token x 64-row tile on four, of which
+// two workgroups share a CU -- they drift apart, so one's vector phases (dequantization,
+// epilogue) fall under the other's matrix instructions.
+// grid = (tok_pad/128, ceil(nrows/(64*RH))), block = 256*RH, dynamic LDS = two weight
+// stages [64*RH][152] f16 + row scales [2][64*RH][2] + token scales [2][128].
+template <int RH>
 __device__ __forceinline__ void gemm_q4k_body(const GemmArgs& p, uint8_t* smem) {
+    constexpr int ROWS = 64 * RH, JL_GEMM_STAGE_HALFS = ROWS * JL_GEMM_STRIDE;
     _Float16* sW = (_Float16*)smem;
     float* sScale = (float*)(sW + 2 * JL_GEMM_STAGE_HALFS);
-    float* sDa = sScale + 2 * 2 * JL_GEMM_TILE;
+    float* sDa = sScale + 2 * 2 * ROWS;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int tg = wave & 3, rh = wave >> 2;   // this wavefront: tokens 32*tg.., rows 64*rh..
-    const int t0 = blockIdx.x * JL_GEMM_TILE, r0 = blockIdx.y * JL_GEMM_TILE;
+    const int t0 = blockIdx.x * JL_GEMM_TILE, r0 = blockIdx.y * ROWS;
     const int nsteps = 2 * (p.k / 256);
     // this thread's share of a weight stage
     const int srow = tid >> 2, hh = (tid >> 1) & 1, wq = tid & 1;
@@ -296,26 +297,17 @@ __device__ __forceinline__ void gemm_q4k_body(const GemmArgs& p, uint8_t* smem) 
             __builtin_amdgcn_sched_barrier(0);
             // (a super-block's first instruction starts from a zero accumulator operand)
             const f32x16 czero = {0};
-#ifndef JL_X_NO_MFMA
 #pragma unroll
             for (int j = 0; j < 2; j++)
                 accP[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aring[ks], wf[ks & 1][j],
                                                                  (half == 0 && ks == 0) ? czero : accP[j], 0, 0, 0);
-#else
-            if (half == 0 && ks == 0) { accP[0] = czero; accP[1] = czero; }
-            accP[0][0] += (float)aring[ks][0] * (float)wf[ks & 1][0][0] + (float)wf[ks & 1][1][0];
-#endif
-#ifndef JL_X_NO_ALOAD
             aring[ks] = a_frag(nstep, ks);
             if (ks == 0 && nhalf == 1) aaug = a_frag(nstep, 8);
-#endif
-#ifndef JL_X_NO_DEQ
             if (has_next && (ks & 1)) gemm_w_word(wcur, wsc, ks >> 1);
-#endif
             __builtin_amdgcn_sched_barrier(0);
         }
         if (has_next && nhalf == 1) {
-            if (wq == 0) gemm_w_mins(wcur, srow, hh, wnext, sScale + (nsbi & 1) * 2 * JL_GEMM_TILE);
+            if (wq == 0) gemm_w_mins(wcur, srow, hh, wnext, sScale + (nsbi & 1) * 2 * ROWS);
             if (tid < JL_GEMM_TILE) sDa[(nsbi & 1) * JL_GEMM_TILE + tid] = da_reg;
         }
         if (half == 1) {
@@ -324,11 +316,11 @@ __device__ __forceinline__ void gemm_q4k_body(const GemmArgs& p, uint8_t* smem) 
             da_reg = p.da[(size_t)sb2 * p.tok_pad + t0 + (tid & (JL_GEMM_TILE - 1))];
         }
         JL_TRACE(3);
-        if (half == 1 && !JL_X_NO_EPI) {
+        if (half == 1) {
             // the 16 minimum columns: M, then the super-block's epilogue
             //   out += d_a * (d * P - dmin * M)
             const f32x16 zero = {0};
-            const float* ssc = sScale + (sb & 1) * 2 * JL_GEMM_TILE + 2 * 64 * rh;
+            const float* ssc = sScale + (sb & 1) * 2 * ROWS + 2 * 64 * rh;
             const float* sda = sDa + (sb & 1) * JL_GEMM_TILE + 32 * tg;
 #pragma unroll
             for (int j = 0; j < 2; j++) {

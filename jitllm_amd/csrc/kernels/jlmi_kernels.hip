@@ -75,8 +75,10 @@ JL_PACKED_KERNEL(q6k, JL_Q6_K, 64, 4) JL_PACKED_KERNEL(q6k, JL_Q6_K, 32, 4) JL_P
 // ------------------------------------------------------------ prefill GEMM
 // grid = (k/256, tok_pad/4), block = 256: one wavefront per (token, super-block)
 extern "C" __global__ __launch_bounds__(256) void jl_gemm_prep_q4k(GemmPrepArgs p) { gemm_prep_q4k_body(p); }
-// grid = (tok_pad/128, ceil(nrows/128)), block = 512 (two wavefronts per SIMD)
-extern "C" __global__ __launch_bounds__(512) void jl_gemm_q4k(GemmArgs p) { gemm_q4k_body(p, jl_smem); }
+// grid = (tok_pad/128, ceil(nrows/64)), block = 256, two workgroups per CU; and the
+// 128-row form on 512 threads
+extern "C" __global__ __launch_bounds__(256, 2) void jl_gemm_q4k_r64(GemmArgs p) { gemm_q4k_body<1>(p, jl_smem); }
+extern "C" __global__ __launch_bounds__(512) void jl_gemm_q4k_r128(GemmArgs p) { gemm_q4k_body<2>(p, jl_smem); }
 
 // ------------------------------------------------------- mixture of experts
 // one workgroup of 1024 threads (n_expert <= 1024)
