@@ -86,7 +86,8 @@ int jl_synchronize(jl_ctx *ctx);
  * (workgroups), "gemm.min_tok" (fewest tokens sent to the matrix-core GEMM),
  * "packed.rw" (rows per wavefront of the packed-plane matvec: 16, 32, 64),
  * "packed.block" (its threads per workgroup), "moe.shares" (row shares an expert's
- * matrix is split into), "gemm.rows" (rows per workgroup of the GEMM: 64 or 128);
+ * matrix is split into), "gemm.rows" (rows per workgroup of the GEMM: 64 or 128), "mxfp4.split" (workgroups along
+ * K of the MXFP4 matmul);
  * value 0 restores the built-in choice.  Mirrors the reference's per-instance tuning knobs
  * (engine/nn/options.go:67-118). */
 int jl_set_tuning(jl_ctx *ctx, const char *key, int value);

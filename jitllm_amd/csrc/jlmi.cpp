@@ -31,6 +31,7 @@ struct Tuning {
     int packed_rw = 0, packed_block = 0;
     int moe_shares = 0;
     int gemm_rows = 0;
+    int mx_split = 0;
 };
 
 struct Resident {
@@ -57,6 +58,8 @@ struct jl_ctx {
     void* gemm_ws = nullptr;
     size_t gemm_ws_bytes = 0;
 
+    void* mx_ws = nullptr;      // partial sums of a K-split MXFP4 matmul
+    size_t mx_ws_bytes = 0;
     void* moe_q_ws = nullptr;   // quantized column activations of a mixture pass
     size_t moe_q_ws_bytes = 0;
 
@@ -528,7 +531,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     if (e != hipSuccess)
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
-    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_q4k_r64", "jl_gemm_q4k_r128", "jl_moe_group", "jl_moe_quant", "jl_moe_combine", "jl_mxfp4_gemm", "jl_mxfp4_matvec",
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_q4k_r64", "jl_gemm_q4k_r128", "jl_moe_group", "jl_moe_quant", "jl_moe_combine", "jl_mxfp4_gemm", "jl_mxfp4_matvec", "jl_sum_parts",
                                       "jl_pack_weights", "jl_unpack_q4k"};
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int rw : {16, 32, 64})
@@ -569,6 +572,7 @@ void jl_ctx_destroy(jl_ctx* c) {
     if (c->moe_ws) (void)H->Free(c->moe_ws);
     if (c->unpack_ws) (void)H->Free(c->unpack_ws);
     if (c->moe_q_ws) (void)H->Free(c->moe_q_ws);
+    if (c->mx_ws) (void)H->Free(c->mx_ws);
     if (c->stage_x) (void)H->Free(c->stage_x);
     if (c->stage_out) (void)H->Free(c->stage_out);
     if (c->module) (void)H->ModuleUnload(c->module);
@@ -604,6 +608,7 @@ int jl_set_tuning(jl_ctx* c, const char* key, int value) {
     else if (!strcmp(key, "packed.block")) c->tune.packed_block = value;
     else if (!strcmp(key, "moe.shares")) c->tune.moe_shares = value;
     else if (!strcmp(key, "gemm.rows")) c->tune.gemm_rows = value;
+    else if (!strcmp(key, "mxfp4.split")) c->tune.mx_split = value;
     else if (!strcmp(key, "gemm.min_tok")) c->gemm_min_tok = value > 0 ? value : 8;
     else return fail(c, JL_ERR_ARG, "unknown tuning key %s", key);
     return JL_OK;
@@ -819,12 +824,36 @@ int jl_matmul_mxfp4_bf16_dev(jl_ctx* c, float* out, const void* w, const uint16_
     MxGemmArgs a;
     a.out = out; a.w = (const uint8_t*)w; a.x = x;
     a.nrows = nrows; a.k = k; a.ntok = ntok; a.row_bytes = (k / 32) * 17;
+    a.nsplit = 1; a.part = nullptr;
     void* params[] = {&a};
     hipStream_t st = pick_stream(c, stream);
     if (ntok <= 8)  // a handful of tokens: stream the rows once, no tile to fill
         return launch(c, "jl_mxfp4_matvec", (unsigned)((nrows + 3) / 4), 1, 256, 0, st, params);
     const unsigned lds = 4u * 128u * 136u * 2u;
     if (lds > c->lds_limit) return JL_DECLINED;
+    // A grid that leaves most CUs idle is widened along K: each split writes partial sums
+    // to a workspace slab and a second kernel adds the slabs in order.
+    const int tiles = ((ntok + 127) / 128) * ((nrows + 127) / 128), stages = (k + 127) / 128;
+    int nsplit = c->tune.mx_split > 0 ? c->tune.mx_split : (tiles * 2 <= c->num_cu ? c->num_cu / tiles : 1);
+    if (nsplit > 8) nsplit = 8;
+    if (nsplit > stages) nsplit = stages;
+    if (nsplit > 1) {
+        const int per = (stages + nsplit - 1) / nsplit;
+        nsplit = (stages + per - 1) / per;   // no empty split
+    }
+    if (nsplit > 1) {
+        const size_t n = (size_t)ntok * nrows;
+        int rc = ws_ensure(c, &c->mx_ws, &c->mx_ws_bytes, n * nsplit * 4);
+        if (rc != JL_OK) return rc;
+        a.nsplit = nsplit; a.part = (float*)c->mx_ws;
+        HIP_TRY(c, H->ModuleLaunchKernel(c->fn["jl_mxfp4_gemm"], (unsigned)((ntok + 127) / 128),
+                                         (unsigned)((nrows + 127) / 128), (unsigned)nsplit, 256, 1, 1, lds, st,
+                                         params, nullptr));
+        SumPartsArgs sa;
+        sa.out = out; sa.part = a.part; sa.n = n; sa.nsplit = nsplit;
+        void* sp[] = {&sa};
+        return launch(c, "jl_sum_parts", (unsigned)((n + 255) / 256), 1, 256, 0, st, sp);
+    }
     return launch(c, "jl_mxfp4_gemm", (unsigned)((ntok + 127) / 128), (unsigned)((nrows + 127) / 128), 256,
                   lds, st, params);
 }

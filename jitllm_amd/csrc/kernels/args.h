@@ -91,6 +91,16 @@ struct MxGemmArgs {
     const uint16_t* x;    // bf16 bits, [ntok][k]
     int nrows, k, ntok;
     int row_bytes;
+    int nsplit;           // workgroups along K (grid z); > 1: partial sums go to part
+    float* part;          // [nsplit][ntok][nrows], summed by jl_sum_parts
+};
+
+// out[i] = part[0][i] + part[1][i] + ... in that order.
+struct SumPartsArgs {
+    float* out;
+    const float* part;
+    size_t n;
+    int nsplit;
 };
 
 // GGUF row-major blocks -> the reference's device planes (and back, for Q4_K).

@@ -118,7 +118,13 @@ __device__ __forceinline__ void mx_gemm_body(const MxGemmArgs& p, uint8_t* smem)
     __bf16* sW = sA + 2 * JL_MX_STAGE_ELEMS;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int t0 = blockIdx.x * JL_MX_TILE, r0 = blockIdx.y * JL_MX_TILE;
-    const int nstages = (p.k + JL_MX_KSTAGE - 1) / JL_MX_KSTAGE;
+    // a small grid is widened along K: workgroup z takes a contiguous run of the K
+    // stages and writes its partial sums to its own slab, summed afterwards in order
+    const int all_stages = (p.k + JL_MX_KSTAGE - 1) / JL_MX_KSTAGE;
+    const int per_split = (all_stages + p.nsplit - 1) / p.nsplit;
+    const int s_lo = min((int)blockIdx.z * per_split, all_stages), s_hi = min(s_lo + per_split, all_stages);
+    const int nstages = s_hi - s_lo;
+    float* outp = p.nsplit > 1 ? p.part + (size_t)blockIdx.z * p.ntok * p.nrows : p.out;
     const int wrow = min(r0 + (tid >> 1), p.nrows - 1), pr = tid & 1;
     const int wt = (wave >> 1) * 64, wr = (wave & 1) * 64;
     const int arow = lane & 31, kg = lane >> 5;
@@ -133,13 +139,15 @@ __device__ __forceinline__ void mx_gemm_body(const MxGemmArgs& p, uint8_t* smem)
 
     MxWRegs wreg;
     MxARegs areg;
-    mx_load_w(p, wrow, 0, pr, wreg);
-    mx_load_a(p, t0, 0, tid, areg);
-    mx_store_w(wreg, tid >> 1, pr, sW);
-    mx_store_a(areg, tid, sA);
+    if (nstages > 0) {
+        mx_load_w(p, wrow, s_lo, pr, wreg);
+        mx_load_a(p, t0, s_lo, tid, areg);
+        mx_store_w(wreg, tid >> 1, pr, sW);
+        mx_store_a(areg, tid, sA);
+    }
     if (nstages > 1) {
-        mx_load_w(p, wrow, 1, pr, wreg);
-        mx_load_a(p, t0, 1, tid, areg);
+        mx_load_w(p, wrow, s_lo + 1, pr, wreg);
+        mx_load_a(p, t0, s_lo + 1, tid, areg);
     }
     mx_lds_barrier();
 
@@ -151,8 +159,8 @@ __device__ __forceinline__ void mx_gemm_body(const MxGemmArgs& p, uint8_t* smem)
             mx_store_w(wreg, tid >> 1, pr, sW + (buf ^ 1) * JL_MX_STAGE_ELEMS);
             mx_store_a(areg, tid, sA + (buf ^ 1) * JL_MX_STAGE_ELEMS);
             if (st + 2 < nstages) {
-                mx_load_w(p, wrow, st + 2, pr, wreg);
-                mx_load_a(p, t0, st + 2, tid, areg);
+                mx_load_w(p, wrow, s_lo + st + 2, pr, wreg);
+                mx_load_a(p, t0, s_lo + st + 2, tid, areg);
             }
         }
 #pragma unroll
@@ -180,7 +188,7 @@ __device__ __forceinline__ void mx_gemm_body(const MxGemmArgs& p, uint8_t* smem)
 #pragma unroll
             for (int e = 0; e < 16; e++) {
                 const int t = t0 + wt + 32 * i + 8 * (e >> 2) + 4 * kg + (e & 3);
-                if (t < p.ntok) p.out[(size_t)t * p.nrows + r] = acc[i][j][e];
+                if (t < p.ntok) outp[(size_t)t * p.nrows + r] = acc[i][j][e];
             }
     }
 }
@@ -240,4 +248,13 @@ __device__ __forceinline__ void mx_matvec_body(const MxGemmArgs& p) {
             if (lane == 63) p.out[(size_t)t * p.nrows + row] = v;
         }
     }
+}
+
+// grid = ceil(n / 256), block = 256
+__device__ __forceinline__ void sum_parts_body(const SumPartsArgs& p) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= p.n) return;
+    float s = p.part[i];
+    for (int z = 1; z < p.nsplit; z++) s += p.part[(size_t)z * p.n + i];
+    p.out[i] = s;
 }

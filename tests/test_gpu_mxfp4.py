@@ -51,3 +51,21 @@ def test_mxfp4_declines_what_it_cannot_serve(dev, devbuf):
     x = devbuf(np.zeros(64, np.uint16))
     out = devbuf(shape=(4,), dtype=np.float32)
     assert dev.matmul_mxfp4_bf16_dev(out.ptr, w.ptr, x.ptr, 4, 48, 1) is False   # k not whole blocks
+
+
+def test_mxfp4_k_split_forms_agree(dev, devbuf):
+    """A small grid is widened along K (partial sums per split, added in order); every
+    split count gives the same matrix up to f32 summation order."""
+    ntok, nrows, k = 40, 300, 1504   # 1504 = 11.75 K stages: a short last stage
+    t = quant.MXFP4
+    w = synth.quantized_weights(t, nrows, k, seed=3)
+    xb, xf = to_bf16(np.stack([synth.activations(k, seed=70 + i) for i in range(ntok)]))
+    want = xf.astype(np.float64) @ oracle.dequant(t, w, nrows * k).reshape(nrows, k).astype(np.float64).T
+    dw, dx = devbuf(w), devbuf(xb)
+    for split in (1, 2, 3, 5, 8, 0):
+        dev.set_tuning(mxfp4__split=split)
+        out = devbuf(shape=(ntok, nrows), dtype=np.float32, fill=np.float32(-5e30))
+        assert dev.matmul_mxfp4_bf16_dev(out.ptr, dw.ptr, dx.ptr, nrows, k, ntok)
+        dev.synchronize()
+        assert nmse(out.get(), want) <= 1e-10, f"split {split}"
+    dev.set_tuning(mxfp4__split=0)
