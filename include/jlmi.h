@@ -214,6 +214,15 @@ int jl_matmul_mxfp4_bf16_dev(jl_ctx *ctx, float *out, const void *w, const uint1
 
 /* ---- mixture of experts (device pointers) ----------------------------- */
 
+/* The router (kernels.ExpertRoute, jit/gpu/kernels/moe.go:562; specification
+ * oracle.MoERouter, internal/oracle/moe.go:197-327, with Softmax32, oracle.go:244-265):
+ * per row, softmax over all n_expert logits (f64 exp and sum, scores narrowed to f32), the
+ * k_used largest by (score descending, index ascending), weights = score / (sum of the
+ * selected scores in selection order + 1e-20).  Fills sel [rows][sel_stride] (first k_used
+ * of each row) and wt [rows][k_used].  n_expert <= 1024, k_used <= 16. */
+int jl_moe_route_dev(jl_ctx *ctx, const float *logits, int rows, int n_expert, int k_used,
+                     uint32_t *sel, int sel_stride, float *wt, void *stream);
+
 /* The grouping the device tier runs before a batched mixture (kernels.ExpertGroup*,
  * jit/gpu/kernels/moesort.go:12-31; specification groupPairs,
  * jit/gpu/tier/grouppairs_test.go:91-122, with unit 1): sel [rows][sel_stride] holds

@@ -49,6 +49,7 @@ SIGNATURES = {
     "jl_matmul_packed_dev": (_int, [_vp, _vp, _int, _vp, _vp, _vp, _int, _int, _vp, _int, _int, _int,
                                     _vp]),
     "jl_matmul_mxfp4_bf16_dev": (_int, [_vp, _vp, _vp, _vp, _int, _int, _int, _vp]),
+    "jl_moe_route_dev": (_int, [_vp, _vp, _int, _int, _int, _vp, _int, _vp, _vp]),
     "jl_moe_group_dev": (_int, [_vp, _vp, _int, _int, _int, _int, _vp, _vp, _vp, _vp]),
     "jl_moe_matvec_dev": (_int, [_vp, _vp, _vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp]),
     "jl_moe_combine_dev": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _vp, _int, _int, _int, _vp]),

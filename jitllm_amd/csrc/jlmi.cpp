@@ -531,7 +531,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     if (e != hipSuccess)
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
-    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_q4k_r64", "jl_gemm_q4k_r128", "jl_moe_group", "jl_moe_quant", "jl_moe_combine", "jl_mxfp4_gemm", "jl_mxfp4_matvec", "jl_sum_parts",
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_q4k_r64", "jl_gemm_q4k_r128", "jl_moe_route", "jl_moe_group", "jl_moe_quant", "jl_moe_combine", "jl_mxfp4_gemm", "jl_mxfp4_matvec", "jl_sum_parts",
                                       "jl_pack_weights", "jl_unpack_q4k"};
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int rw : {16, 32, 64})
@@ -741,6 +741,19 @@ int jl_reserve(jl_ctx* c, int max_tok, int max_k) {
     if (max_tok <= 0 || max_k <= 0 || max_k % 256 != 0) return fail(c, JL_ERR_ARG, "reserve: %d x %d", max_tok, max_k);
     HIP_TRY(c, H->SetDevice(c->device));
     return gemm_ws_ensure(c, gemm_ws_need(max_tok, max_k));
+}
+
+int jl_moe_route_dev(jl_ctx* c, const float* logits, int rows, int n_expert, int k_used, uint32_t* sel,
+                     int sel_stride, float* wt, void* stream) {
+    if (!c) return JL_ERR_ARG;
+    if (!logits || !sel || !wt || rows <= 0 || n_expert <= 0 || k_used <= 0 || sel_stride < k_used)
+        return fail(c, JL_ERR_ARG, "moe route: bad operand");
+    if (n_expert > 1024 || k_used > 16 || k_used > n_expert) return JL_DECLINED;
+    HIP_TRY(c, H->SetDevice(c->device));
+    MoeRouteArgs a;
+    a.logits = logits; a.sel = sel; a.wt = wt; a.n_expert = n_expert; a.k_used = k_used; a.sel_stride = sel_stride;
+    void* params[] = {&a};
+    return launch(c, "jl_moe_route", (unsigned)rows, 1, 64, 0, pick_stream(c, stream), params);
 }
 
 int jl_moe_group_dev(jl_ctx* c, const uint32_t* sel, int sel_stride, int rows, int k_used, int n_expert,

@@ -47,6 +47,16 @@ struct MoeGroupArgs {
     int sel_stride, rows, k_used, n_expert;
 };
 
+// Router: softmax over all experts, the k largest by (score descending, index ascending),
+// weights = selected scores over their sum.  sel [rows][sel_stride] (first k_used filled),
+// wt [rows][k_used].
+struct MoeRouteArgs {
+    const float* logits;    // [rows][n_expert]
+    uint32_t* sel;
+    float* wt;
+    int n_expert, k_used, sel_stride;
+};
+
 // Column activations of a mixture pass: column c reads x[src(c)] (or silu(x[src(c)]) *
 // x2[src(c)]) and is quantized like any activation vector: q [ncols][k] int8,
 // as [ncols][k/32], s16 [ncols][k/16].

@@ -81,6 +81,8 @@ extern "C" __global__ __launch_bounds__(256, 2) void jl_gemm_q4k_r64(GemmArgs p)
 extern "C" __global__ __launch_bounds__(512) void jl_gemm_q4k_r128(GemmArgs p) { gemm_q4k_body<2>(p, jl_smem); }
 
 // ------------------------------------------------------- mixture of experts
+// grid = rows, block = 64
+extern "C" __global__ __launch_bounds__(64) void jl_moe_route(MoeRouteArgs p) { moe_route_body(p); }
 // one workgroup of 1024 threads (n_expert <= 1024)
 extern "C" __global__ __launch_bounds__(1024) void jl_moe_group(MoeGroupArgs p) {
     __shared__ u32 scount[2048];

@@ -38,6 +38,83 @@
 #define JL_MOE_U 2   // row groups of 64/LPR rows a wavefront step covers
 #define JL_MOE_GROUP_KEYS 16384  // (row, slot) pairs the grouping kernel holds in LDS
 
+// ------------------------------------------------------------------- routing
+// One wavefront per row (n_expert <= 1024: sixteen experts a lane).  The reference's
+// router (internal/oracle/oracle.go:244-265 Softmax32, moe.go:197-327 with Norm, no bias,
+// no groups): exp and the sum in f64, scores narrowed to f32, then k rounds of "largest
+// score not yet taken, lowest index on a tie", weights = score / (sum in selection order
+// + 1e-20).  The f64 sum is taken as a butterfly over the lanes, so it can differ from the
+// reference's sequential sum in its last bit; after narrowing to f32 that moves a score
+// only when it sits on a rounding boundary.
+__device__ __forceinline__ double wave_sum_f64(double v) {
+#pragma unroll
+    for (int m = 1; m < 64; m <<= 1) v += __shfl_xor(v, m, 64);
+    return v;
+}
+
+__device__ __forceinline__ void moe_route_body(const MoeRouteArgs& p) {
+    const int lane = threadIdx.x & 63, n = p.n_expert;
+    const size_t row = blockIdx.x;
+    const float* lg = p.logits + row * (size_t)n;
+    float v[16];
+    float mx = -__builtin_inff();
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        const int e = lane + 64 * i;
+        v[i] = e < n ? lg[e] : -__builtin_inff();
+        if (v[i] > mx) mx = v[i];
+    }
+#pragma unroll
+    for (int m = 1; m < 64; m <<= 1) mx = fmaxf(mx, __shfl_xor(mx, m, 64));
+    double sum = 0.0;
+    float sc[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        const int e = lane + 64 * i;
+        double ex = e < n ? exp((double)v[i] - (double)mx) : 0.0;
+        sc[i] = (float)ex;
+        sum += ex;
+    }
+    sum = wave_sum_f64(sum);
+    const double inv = 1.0 / sum;
+#pragma unroll
+    for (int i = 0; i < 16; i++) sc[i] = (float)((double)sc[i] * inv);
+
+    float prev_val = 0.f, total = 0.f;
+    int prev_idx = -1;
+    float chosen[16];
+    int found = 0;
+    for (int r = 0; r < p.k_used && r < 16; r++) {
+        // this lane's best eligible score (index ascending within a lane, so the first
+        // of equal values is kept)
+        float bv = -1.f;
+        int bi = 0x7fffffff;
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const int e = lane + 64 * i;
+            const float x = sc[i];
+            const bool ok = e < n && x == x && (r == 0 || x < prev_val || (x == prev_val && e > prev_idx));
+            if (ok && (x > bv)) { bv = x; bi = e; }
+        }
+#pragma unroll
+        for (int m = 1; m < 64; m <<= 1) {
+            const float ov = __shfl_xor(bv, m, 64);
+            const int oi = __shfl_xor(bi, m, 64);
+            if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+        }
+        if (bi == 0x7fffffff) break;
+        if (lane == 0) p.sel[row * p.sel_stride + r] = (u32)bi;
+        chosen[r] = bv;
+        prev_val = bv;
+        prev_idx = bi;
+        found = r + 1;
+    }
+    for (int r = 0; r < found; r++) total = total + chosen[r];
+    total = total + 1e-20f;
+    if (lane == 0)
+        for (int r = 0; r < found; r++) p.wt[row * p.k_used + r] = chosen[r] / total;
+}
+
 // ------------------------------------------------------------------ grouping
 // A stable counting sort of the (row, slot) pairs by expert in one workgroup of 1024
 // threads.  The threads form NSEG segments x NEXP experts (NEXP = n_expert rounded up

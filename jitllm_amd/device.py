@@ -189,6 +189,12 @@ class Device:
                                                   nrows, k, ntok, stream), "jl_matmul_dev")
 
     # -- mixture of experts -----------------------------------------------------
+    def moe_route_dev(self, logits, rows, n_expert, k_used, sel, sel_stride, wt, stream=None):
+        """oracle.MoERouter on the device: softmax, lexicographic top-k, renormalised weights."""
+        return self._served(self._l.jl_moe_route_dev(self._ctx, _ptr(logits), rows, n_expert, k_used,
+                                                     _ptr(sel), sel_stride, _ptr(wt), stream),
+                            "jl_moe_route_dev")
+
     def moe_group_dev(self, sel, sel_stride, rows, k_used, n_expert, start, perm, pos, stream=None):
         return self._served(self._l.jl_moe_group_dev(self._ctx, _ptr(sel), sel_stride, rows, k_used,
                                                      n_expert, _ptr(start), _ptr(perm), _ptr(pos), stream),

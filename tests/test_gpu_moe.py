@@ -168,3 +168,36 @@ def test_moe_block_vs_oracle(dev, devbuf, shape):
         got = resid.get()
         assert rel_l2(got, want) <= 1e-3, f"call {call}: rel-L2 {rel_l2(got, want):.3e}"
     dev.SetActWindow(32)
+
+
+@pytest.mark.parametrize("case", [(64, 128, 8), (7, 16, 1), (33, 1000, 16), (5, 8, 8), (20, 130, 4)],
+                         ids=lambda c: "x".join(map(str, c)))
+def test_router_vs_oracle(dev, devbuf, case):
+    """The device router against oracle.MoERouter's restatement: the selection (integer work)
+    is exact, ties go to the lower index, weights are the same f32 arithmetic on the same
+    scores (a score can differ in its last bit only if the f64 sum's last bit differs AND the
+    narrowed value sits on a rounding boundary; the test holds exact equality of the weights
+    on these seeds)."""
+    rows, n_expert, k_used = case
+    rng = np.random.default_rng(rows + n_expert)
+    logits = rng.standard_normal((rows, n_expert)).astype(np.float32) * 3
+    logits[0, :] = 0.25                       # every score equal: indices 0..k-1 in order
+    if rows > 2:
+        logits[1, ::2] = logits[1, 0]         # many exact ties
+        logits[2, :] = -80; logits[2, n_expert - 1] = 5   # one dominant expert, the rest underflow towards zero
+    want_sel = np.zeros((rows, k_used), np.uint32)
+    want_wt = np.zeros((rows, k_used), np.float32)
+    for r in range(rows):
+        s, w, _, _ = oracle.moe_route(logits[r], k_used)
+        want_sel[r], want_wt[r] = s, w
+    ld = devbuf(logits)
+    sel = devbuf(shape=(rows, k_used + 1), dtype=np.uint32, fill=0xFFFFFFFF)
+    wt = devbuf(shape=(rows, k_used), dtype=np.float32, fill=np.float32(-1))
+    assert dev.moe_route_dev(ld.ptr, rows, n_expert, k_used, sel.ptr, k_used + 1, wt.ptr)
+    dev.synchronize()
+    got_sel, got_wt = sel.get(), wt.get()
+    assert np.array_equal(got_sel[:, :k_used], want_sel)
+    assert np.all(got_sel[:, k_used] == 0xFFFFFFFF), "wrote past the selection"
+    assert np.array_equal(got_wt.view(np.uint32), want_wt.view(np.uint32))
+    # declines
+    assert dev.moe_route_dev(ld.ptr, rows, 2000, k_used, sel.ptr, k_used + 1, wt.ptr) is False
