@@ -70,6 +70,15 @@ __device__ __forceinline__ float wave_sum_to_lane63(float v) {
     return v;
 }
 
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() carries a
+// release fence that also drains every outstanding global load, which would
+// throw away the register prefetch that is meant to stay in flight across it.
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
 // Q4_K / Q5_K 6-bit scale and minimum of sub-block j from the 12 packed bytes,
 // given as three little-endian words (format/quant/dequant.go:360-365).
 __device__ __forceinline__ void scale_min_k4(int j, u32 s0, u32 s1, u32 s2, u32& sc, u32& m) {

@@ -55,15 +55,6 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 #define JL_GEMM_AFRAG_HALFS 512
 #define JL_GEMM_ASTAGE_FRAGS 9
 
-// Workgroup barrier that orders LDS traffic only.  __syncthreads() carries a
-// release fence that also drains every outstanding global load, which would
-// throw away the register prefetch that is meant to stay in flight across it.
-__device__ __forceinline__ void lds_barrier() {
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-}
-
 // K position (within a stage's 128 weights) of nibble pair i of 32-bit word c of a
 // 64-element group: word c holds bytes 4c..4c+3; byte b's low nibble is element
 // 4c+b of the group's first sub-block, its high nibble the same element of the

@@ -59,7 +59,7 @@ __device__ __forceinline__ void stage_quantize4(uint8_t* smem, int k, int per, i
     float* ss = (float*)(smem + k + (k / 32) * 4);
     const bool live = g4 < k / 4;
     u32 m = max(max(abs_bits(v.x), abs_bits(v.y)), max(abs_bits(v.z), abs_bits(v.w)));
-    u32 amax = window_amax(live ? m : 0u, per);
+    u32 amax = per == 8 ? wave_amax_256(live ? m : 0u) : window_amax(live ? m : 0u, per);
     float d;
     i32 sum;
     u32 q = quantize4(v, amax, d, sum);
@@ -359,10 +359,16 @@ __device__ __forceinline__ void matvec_body(const MatVecArgs& p, uint8_t* smem) 
     const ActLds A = act_lds_views(smem, p.k);
     int r0 = blockIdx.x * rows_per_block + wave * RPW;
 
-    // The activation loads go first: loads return in order, so the quantizer can
-    // start as soon as x is back while the first weight loads are still in flight.
+    // The activation loads go first, for the whole workgroup: a CU serves its vector
+    // loads in the order they were issued whichever wavefront issued them, so every
+    // wavefront issues its x load, the workgroup meets at a barrier that waits for no
+    // data, and only then do the weight loads go out.  The quantizer starts as soon as x
+    // is back while the first weight loads are still in flight.
     f32x4 x0 = f32x4{0.f, 0.f, 0.f, 0.f};
-    if (p.x && (int)threadIdx.x < p.k / 4) x0 = ((const f32x4*)p.x)[threadIdx.x];
+    if (p.x) {
+        x0 = ((const f32x4*)p.x)[min((int)threadIdx.x, p.k / 4 - 1)];
+        __builtin_amdgcn_s_barrier();
+    }
 
     typename T::W w[RPW];
     {
@@ -373,7 +379,7 @@ __device__ __forceinline__ void matvec_body(const MatVecArgs& p, uint8_t* smem) 
     }
     if (p.x) stage_act_quantize(smem, p.x, p.k, p.per, x0, nwaves * 64);
     else stage_act_copy(smem, p.q, p.as, p.s16, p.k, nwaves * 64);
-    __syncthreads();
+    lds_barrier();   // orders the LDS staging only: the weight loads stay in flight
 
     bool preloaded = true;
     for (; r0 < p.nrows; r0 += group_stride) {

@@ -309,18 +309,6 @@ template <int NB> struct PkTraits<JL_Q4_K, NB> { typedef PkWQ4K<NB> W; };
 template <int NB> struct PkTraits<JL_Q8_0, NB> { typedef PkWQ8<NB> W; };
 template <int NB> struct PkTraits<JL_Q6_K, NB> { typedef PkWQ6K<NB> W; };
 
-// The whole-wavefront (256-element window) amax without LDS traffic: DPP maxima
-// within and across the 16-lane rows, then lane 63's value read back as a scalar.
-__device__ __forceinline__ u32 wave_amax_256(u32 m) {
-    m = dpp_max_u32<JL_DPP_QUAD_XOR1>(m);
-    m = dpp_max_u32<JL_DPP_QUAD_XOR2>(m);
-    m = dpp_max_u32<JL_DPP_ROW_HALF_MIRROR>(m);
-    m = dpp_max_u32<JL_DPP_ROW_MIRROR>(m);
-    m = max(m, (u32)dpp_i32<JL_DPP_ROW_BCAST15, 0xa>(0, (i32)m));
-    m = max(m, (u32)dpp_i32<JL_DPP_ROW_BCAST31, 0xc>(0, (i32)m));
-    return (u32)__builtin_amdgcn_readlane((i32)m, 63);
-}
-
 // A chunk's activation as the lane holds it between the load and the staging: four
 // f32 values (fused form), or in the split form four int8 in .x, a scale in .y (lanes
 // 0-7) and a half-block sum in .z (lanes 0-15).  Loads are unconditional at clamped

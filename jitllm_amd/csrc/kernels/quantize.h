@@ -36,6 +36,18 @@ __device__ __forceinline__ u32 window_amax(u32 m, int per) {
     return m;
 }
 
+// The whole-wavefront (256-element window) amax without LDS traffic: DPP maxima
+// within and across the 16-lane rows, then lane 63's value read back as a scalar.
+__device__ __forceinline__ u32 wave_amax_256(u32 m) {
+    m = dpp_max_u32<JL_DPP_QUAD_XOR1>(m);
+    m = dpp_max_u32<JL_DPP_QUAD_XOR2>(m);
+    m = dpp_max_u32<JL_DPP_ROW_HALF_MIRROR>(m);
+    m = dpp_max_u32<JL_DPP_ROW_MIRROR>(m);
+    m = max(m, (u32)dpp_i32<JL_DPP_ROW_BCAST15, 0xa>(0, (i32)m));
+    m = max(m, (u32)dpp_i32<JL_DPP_ROW_BCAST31, 0xc>(0, (i32)m));
+    return (u32)__builtin_amdgcn_readlane((i32)m, 63);
+}
+
 // Round half away from zero for |p| < 2^22, exactly: adding 0.5 - 2^-25 (the
 // largest f32 below one half) cannot carry a value below n + 0.5 up to n + 1,
 // and carries every value at or above it; the conversion then truncates.
