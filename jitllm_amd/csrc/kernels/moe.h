@@ -239,8 +239,7 @@ __device__ __forceinline__ void moe_quant_body(const MoeQuantArgs& p) {
 // of the expert's quantized columns into LDS and streams its rows once for all of them.
 // A wavefront works in steps of 64/LPR rows (one slot per lane): it decodes the step's
 // scales and nibbles once, meets every staged column with them, and has the next step's
-// loads in flight meanwhile.  The first step is requested before the columns are staged,
-// so the copy overlaps HBM latency.  k % 256 == 0.
+// loads in flight meanwhile.  k % 256 == 0.
 template <int TYPE, int LPR>
 __device__ __forceinline__ void moe_matvec_body(const MoeMatVecArgs& p, uint8_t* smem) {
     typedef SlotTraits<TYPE> T;
@@ -274,7 +273,6 @@ __device__ __forceinline__ void moe_matvec_body(const MoeMatVecArgs& p, uint8_t*
     };
 
     typename T::W w_next[U];
-    if (nsteps > 0) load_step(0, w_next);
 
     for (u32 c0 = c_lo; c0 < c_hi; c0 += JL_MOE_TB) {
         const int ncol = min((u32)JL_MOE_TB, c_hi - c0);
@@ -295,9 +293,11 @@ __device__ __forceinline__ void moe_matvec_body(const MoeMatVecArgs& p, uint8_t*
                 }
             }
         }
-        __syncthreads();
+        // the first step's weights are requested behind the staging loads (loads are served
+        // in order) and stay in flight across the barrier, which orders LDS only
+        if (nsteps > 0) load_step(0, w_next);
+        lds_barrier();
         JL_MOE_TRACE(2);
-        if (c0 != c_lo && nsteps > 0) load_step(0, w_next);  // a further pass starts over
         float acc[JL_MOE_TB][U];
 #pragma unroll
         for (int j = 0; j < JL_MOE_TB; j++)
