@@ -155,18 +155,20 @@ def cpu_baseline(t, nrows, k, window, seed=0):
 MFMA_F16_PEAK_TFLOPS = 2500.0
 
 
-def gemm_section(dev):
+def gemm_section(dev, shapes=None):
     """Q4_K prefill GEMM (x [ntok][4096] f32 -> out [ntok][nrows]), activation quantizer and
     layout kernel included in every step; flops = 2*nrows*k*ntok, priced against the dense
-    f16 MFMA peak (the kernel runs exact integer operands on the f16 matrix cores)."""
+    f16 MFMA peak (the kernel runs exact integer operands on the f16 matrix cores).
+    shapes: {nrows: [ntok, ...]}; default = the baseline's prefill configurations."""
     from jitllm_amd import quant, synth
     from jitllm_amd.hipmem import DeviceArray, Event
     t, k = quant.Q4_K, 4096
     dev.SetActWindow(256)
     out = {}
-    for nrows in (4096, 14336):
+    shapes = shapes or {4096: (16, 128, 512, 2048), 14336: (16, 128, 512, 2048)}
+    for nrows, toks in shapes.items():
         w = DeviceArray(synth.quantized_weights(t, nrows, k, seed=0))
-        for ntok in (16, 128, 512, 2048):
+        for ntok in toks:
             x = DeviceArray(np.random.default_rng(2).standard_normal((ntok, k), np.float32))
             o = DeviceArray(shape=(ntok, nrows), dtype=np.float32)
             dev.Reserve(ntok, k)
@@ -281,6 +283,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="headline workload only")
+    ap.add_argument("--gemm", metavar="NTOK,NROWS", help="only the prefill GEMM of this shape (k = 4096), "
+                    "for profiling one kernel; prints its section alone")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this path runs on one GPU (no sharding, no collectives); use --gpus 1")
@@ -289,6 +293,11 @@ def main():
     from jitllm_amd.device import Device
 
     dev = Device(device=0, act_window=256)
+    if args.gemm:
+        ntok, nrows = (int(v) for v in args.gemm.split(","))
+        print(json.dumps({"prefill_gemm": gemm_section(dev, {nrows: (ntok,)})}), flush=True)
+        dev.close()
+        return
     head = Workload(dev, quant.Q4_K, 4096, 4096, window=256)
     ms, ms_host = head.timed(args.steps, args.warmup)
     head.check()
