@@ -192,6 +192,55 @@ def gemm_section(dev, shapes=None):
     return out
 
 
+def ffn_section(dev):
+    """A gated feed-forward block at decode, the baseline's second configuration: gate and up
+    (Q8_0 14336x4096) as one grouped launch, then down (Q6_K 4096x14336) over silu(gate) * up
+    formed inside its quantizer with the residual add riding on the launch: two launches per
+    block.  Four rotating sets of the three matrices (692 MiB) keep every step out of cache."""
+    from jitllm_amd import quant, synth
+    from jitllm_amd.hipmem import DeviceArray, Event, check, hip
+    n_embd, n_ffn = 4096, 14336
+    dev.SetActWindow(32)
+    wg = synth.quantized_weights(quant.Q8_0, n_ffn, n_embd, seed=0)
+    wd = synth.quantized_weights(quant.Q6_K, n_embd, n_ffn, seed=1)
+    sets = []
+    for i in range(4):
+        g, u, d = DeviceArray(wg), DeviceArray(wg), DeviceArray(wd)
+        sets.append((g, u, d))
+    x = DeviceArray(synth.activations(n_embd, seed=2))
+    gate = DeviceArray(shape=(n_ffn,), dtype=np.float32, fill=0)
+    up = DeviceArray(shape=(n_ffn,), dtype=np.float32, fill=0)
+    y = DeviceArray(shape=(n_embd,), dtype=np.float32, fill=0)
+    resid = DeviceArray(shape=(n_embd,), dtype=np.float32, fill=0)
+
+    def run(i):
+        g, u, d = sets[i % len(sets)]
+        ok = dev.matvec_group_dev([gate.ptr, up.ptr], [quant.Q8_0, quant.Q8_0], [g.ptr, u.ptr], [n_ffn, n_ffn],
+                                  x.ptr, n_embd)
+        ok = ok and dev.matvec_group_dev([y.ptr], [quant.Q6_K], [d.ptr], [n_embd], gate.ptr, n_ffn, act_up=up.ptr,
+                                         resid=resid.ptr, alpha=1.0)
+        if not ok:
+            raise RuntimeError("the device declined the feed-forward block")
+    for i in range(8):
+        run(i)
+    dev.synchronize()
+    e0, e1, n = Event(), Event(), 100
+    e0.record(dev.stream)
+    for i in range(n):
+        run(i)
+    e1.record(dev.stream)
+    e1.synchronize()
+    ms = e0.elapsed_ms(e1) / n
+    nbytes = 2 * wg.nbytes + wd.nbytes + 4 * (n_embd + 2 * n_ffn) + 4 * (2 * n_ffn + 2 * n_embd)
+    for g, u, d in sets:
+        g.free(); u.free(); d.free()
+    for b in (x, gate, up, y, resid):
+        b.free()
+    return {"us_per_step": round(ms * 1e3, 2), "launches_per_step": 2, "bytes_per_step": nbytes,
+            "GB/s": round(nbytes / (ms * 1e-3) / 1e9, 1),
+            "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+
+
 def moe_section(dev):
     """Qwen3-30B-A3B routed feed-forward block: 128 experts (gate/up 768x2048, down 2048x768,
     Q4_K), 64 rows routed top-8 by softmax over N(0,1) logits (seeded); one step = group +
@@ -339,6 +388,7 @@ def main():
         line["other_configs"] = extra
 
     if not args.no_extra:
+        line["ffn_block_decode"] = ffn_section(dev)
         line["prefill_gemm"] = gemm_section(dev)
         line["moe_block"] = moe_section(dev)
         line["mxfp4_gemm"] = mxfp4_section(dev)

@@ -152,6 +152,42 @@ int jl_matvec_dev(jl_ctx *ctx, float *out, int type, const void *w, const float 
 int jl_matvec_q8_dev(jl_ctx *ctx, float *out, int type, const void *w, const int8_t *q,
                      const float *as, const float *sum16, int nrows, int k, void *stream);
 
+/* Several decode matvecs in one launch -- on this machine a launch costs as much as
+ * streaming 10 MB, so a block's projections belong together.
+ *
+ * jl_matvec_group_dev is JIT.MatVecPackedGroup (engine/nn/packedgroup.go:13-51) over GGUF
+ * row-major weights: n <= JL_MAX_GROUP matrices (a block's q, k, v; its gate and up; a
+ * single projection) read ONE activation x[0:k]; out[i] gets rows[i] rows of w[i] (type
+ * type[i]).  act_up, when set, makes the activation silu(x) * act_up, formed on the way
+ * into the quantizer (x is left as it was).  resid, when set, takes matrix 0's rows as
+ * they are made: resid[r] += alpha * out[0][r].  Matrices of one type share a launch. */
+#define JL_MAX_GROUP 4
+typedef struct jl_mv_group {
+    int n;
+    float *out[JL_MAX_GROUP];
+    int type[JL_MAX_GROUP];
+    const void *w[JL_MAX_GROUP];
+    int rows[JL_MAX_GROUP];
+    const float *x;
+    int k;
+    const float *act_up;
+    float *resid;
+    float alpha;
+} jl_mv_group;
+int jl_matvec_group_dev(jl_ctx *ctx, const jl_mv_group *g, void *stream);
+
+/* JIT.MatVecPackedMulti (engine/nn/packedmulti.go:24): m <= 16 matrices of one type and
+ * shape sharing one activation (a mixture's experts' gate and up at decode). */
+int jl_matvec_multi_dev(jl_ctx *ctx, float *const *outs, int type, const void *const *ws,
+                        const float *x, int nrows, int k, int m, void *stream);
+
+/* JIT.MatVecPackedGather / GatherAct (engine/nn/packedmulti.go:84,93): m <= 16 matrices,
+ * matrix j with its own activation x[j*xstride : j*xstride+k] (a mixture's down
+ * projections); up, when given, makes it silu(x_j) * up[j*xstride : ...]. */
+int jl_matvec_gather_dev(jl_ctx *ctx, float *const *outs, int type, const void *const *ws,
+                         const float *x, size_t xstride, const float *up, int nrows, int k,
+                         int m, void *stream);
+
 /* JIT.MatMulPacked / MatMul semantics on resident operands (engine/nn/packedmm.go:23,
  * matmul.go:27): x [ntok][k] f32 -> out [ntok][nrows], every token quantized on
  * its own.  Q4_K with the 256 window runs the matrix-core GEMM (quantize-and-

@@ -19,6 +19,16 @@ class Options(C.Structure):
 
 _vp, _sz, _int = C.c_void_p, C.c_size_t, C.c_int
 
+MAX_GROUP = 4
+
+
+class MVGroup(C.Structure):
+    """jl_mv_group: the reference's nn.MVGroup over device pointers."""
+    _fields_ = [("n", C.c_int), ("out", C.c_void_p * MAX_GROUP), ("type", C.c_int * MAX_GROUP),
+                ("w", C.c_void_p * MAX_GROUP), ("rows", C.c_int * MAX_GROUP), ("x", C.c_void_p),
+                ("k", C.c_int), ("act_up", C.c_void_p), ("resid", C.c_void_p), ("alpha", C.c_float)]
+
+
 # name -> (restype, argtypes); every symbol include/jlmi.h declares
 SIGNATURES = {
     "jl_hip_runtime": (C.c_char_p, []),
@@ -36,6 +46,10 @@ SIGNATURES = {
     "jl_dequant_dev": (_int, [_vp, _int, _vp, _vp, _sz, _vp]),
     "jl_matvec_dev": (_int, [_vp, _vp, _int, _vp, _vp, _int, _int, _vp]),
     "jl_matvec_q8_dev": (_int, [_vp, _vp, _int, _vp, _vp, _vp, _vp, _int, _int, _vp]),
+    "jl_matvec_group_dev": (_int, [_vp, C.POINTER(MVGroup), _vp]),
+    "jl_matvec_multi_dev": (_int, [_vp, C.POINTER(_vp), _int, C.POINTER(_vp), _vp, _int, _int, _int, _vp]),
+    "jl_matvec_gather_dev": (_int, [_vp, C.POINTER(_vp), _int, C.POINTER(_vp), _vp, _sz, _vp, _int, _int, _int,
+                                    _vp]),
     "jl_matmul_dev": (_int, [_vp, _vp, _int, _vp, _vp, _int, _int, _int, _vp]),
     "jl_reserve": (_int, [_vp, _int, _int]),
     "jl_packed_words": (_int, [_int, _int, _int, C.POINTER(_sz), C.POINTER(_sz), C.POINTER(_sz)]),

@@ -209,6 +209,46 @@ int matvec_launch(jl_ctx* c, float* out, int type, const void* w, const float* x
     return launch(c, name, (unsigned)grid, 1, (unsigned)block, lds, st, params);
 }
 
+// m matrices of one type in one launch (kernels/matvec.h, matvec_multi_body).
+int matvec_multi_launch(jl_ctx* c, int type, int m, float* const* outs, const void* const* ws, const int* rows,
+                        const float* x, size_t xstride, const float* x2, float* resid, float alpha, int k,
+                        hipStream_t st) {
+    if (m < 1 || m > JL_MAX_MULTI) return fail(c, JL_ERR_ARG, "matvec multi: %d matrices", m);
+    const TypeInfo* ti = nullptr;
+    int max_rows = 0;
+    for (int i = 0; i < m; i++) {
+        int rc = matvec_check(c, type, rows[i], k, &ti);
+        if (rc != JL_OK) return rc;
+        if (!outs[i] || !ws[i]) return fail(c, JL_ERR_ARG, "matvec multi: null operand");
+        if (type == JL_TYPE_Q4_K && !aligned16(ws[i])) return JL_DECLINED;
+        if (((uintptr_t)ws[i] & 1) != 0) return JL_DECLINED;
+        if (rows[i] > max_rows) max_rows = rows[i];
+    }
+    if (!x || !aligned16(x) || (x2 && !aligned16(x2)) || (xstride % 4) != 0) return JL_DECLINED;
+    MatVecMultiArgs a;
+    memset(&a, 0, sizeof a);
+    for (int i = 0; i < m; i++) {
+        a.out[i] = outs[i];
+        a.w[i] = (const uint8_t*)ws[i];
+        a.nrows[i] = rows[i];
+    }
+    a.x = x; a.x2 = x2; a.resid = resid; a.alpha = alpha; a.xstride = xstride;
+    a.k = k; a.row_bytes = (k / ti->block_elems) * ti->block_bytes; a.per = c->act_window / 32;
+    // sixteen wavefronts a workgroup, one row each; about two workgroups per CU over all
+    // the matrices, never more row groups than the tallest matrix has
+    const int nwaves = 16;
+    long groups = ((long)max_rows + nwaves - 1) / nwaves;
+    long gx = (2L * c->num_cu + m - 1) / m;
+    if (gx > groups) gx = groups;
+    if (gx < 1) gx = 1;
+    a.nwaves = nwaves; a.ngroups = (int)gx;
+    char name[64];
+    snprintf(name, sizeof name, "jl_matvec_multi_%s", ti->tag);
+    void* params[] = {&a};
+    unsigned lds = (unsigned)((size_t)k + (size_t)(k / 32) * 4 + (size_t)(k / 16) * 4);
+    return launch(c, name, (unsigned)gx, (unsigned)m, nwaves * 64, lds, st, params);
+}
+
 int ensure_stage(jl_ctx* c, void** buf, size_t* have, size_t need) {
     if (*have >= need) return JL_OK;
     if (*buf) HIP_TRY(c, H->Free(*buf));
@@ -546,6 +586,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
             snprintf(nm, sizeof nm, "jl_matvec_%s_r%d", type_info(t)->tag, rpw);
             names.push_back(nm);
         }
+    for (const char* tag : {"q4k", "q8_0", "q6k"}) names.push_back(std::string("jl_matvec_multi_") + tag);
     for (const auto& n : names) {
         hipFunction_t f;
         e = H->ModuleGetFunction(&f, c->module, n.c_str());
@@ -662,6 +703,55 @@ int jl_matvec_q8_dev(jl_ctx* c, float* out, int type, const void* w, const int8_
     if (!c) return JL_ERR_ARG;
     HIP_TRY(c, H->SetDevice(c->device));
     return matvec_launch(c, out, type, w, nullptr, q, as, sum16, nrows, k, pick_stream(c, stream));
+}
+
+int jl_matvec_group_dev(jl_ctx* c, const jl_mv_group* g, void* stream) {
+    if (!c) return JL_ERR_ARG;
+    if (!g || g->n < 1 || g->n > JL_MAX_GROUP || !g->x || g->k <= 0) return fail(c, JL_ERR_ARG, "matvec group: bad group");
+    HIP_TRY(c, H->SetDevice(c->device));
+    hipStream_t st = pick_stream(c, stream);
+    // everything is checked before the first launch: a group is served whole or not at all
+    for (int i = 0; i < g->n; i++) {
+        const TypeInfo* ti = nullptr;
+        int rc = matvec_check(c, g->type[i], g->rows[i], g->k, &ti);
+        if (rc != JL_OK) return rc;
+        if (!g->out[i] || !g->w[i]) return fail(c, JL_ERR_ARG, "matvec group: null operand");
+        if ((g->type[i] == JL_TYPE_Q4_K && !aligned16(g->w[i])) || ((uintptr_t)g->w[i] & 1)) return JL_DECLINED;
+    }
+    if (!aligned16(g->x) || (g->act_up && !aligned16(g->act_up))) return JL_DECLINED;
+    // matrices of one type share a launch; matrix 0 leads its launch so that the residual rides on it
+    bool done[JL_MAX_GROUP] = {false, false, false, false};
+    for (int i = 0; i < g->n; i++) {
+        if (done[i]) continue;
+        float* outs[JL_MAX_GROUP];
+        const void* ws[JL_MAX_GROUP];
+        int rows[JL_MAX_GROUP], m = 0;
+        for (int j = i; j < g->n; j++)
+            if (!done[j] && g->type[j] == g->type[i]) {
+                outs[m] = g->out[j]; ws[m] = g->w[j]; rows[m] = g->rows[j]; m++;
+                done[j] = true;
+            }
+        int rc = matvec_multi_launch(c, g->type[i], m, outs, ws, rows, g->x, 0, g->act_up,
+                                     i == 0 ? g->resid : nullptr, g->alpha, g->k, st);
+        if (rc != JL_OK) return rc;
+    }
+    return JL_OK;
+}
+
+int jl_matvec_multi_dev(jl_ctx* c, float* const* outs, int type, const void* const* ws, const float* x,
+                        int nrows, int k, int m, void* stream) {
+    return jl_matvec_gather_dev(c, outs, type, ws, x, 0, nullptr, nrows, k, m, stream);
+}
+
+int jl_matvec_gather_dev(jl_ctx* c, float* const* outs, int type, const void* const* ws, const float* x,
+                         size_t xstride, const float* up, int nrows, int k, int m, void* stream) {
+    if (!c) return JL_ERR_ARG;
+    if (!outs || !ws || m < 1) return fail(c, JL_ERR_ARG, "matvec multi: bad operand");
+    if (m > JL_MAX_MULTI) return JL_DECLINED;
+    HIP_TRY(c, H->SetDevice(c->device));
+    int rows[JL_MAX_MULTI];
+    for (int i = 0; i < m; i++) rows[i] = nrows;
+    return matvec_multi_launch(c, type, m, outs, ws, rows, x, xstride, up, nullptr, 0.f, k, pick_stream(c, stream));
 }
 
 int jl_matmul_dev(jl_ctx* c, float* out, int type, const void* w, const float* x, int nrows, int k,

@@ -18,6 +18,23 @@ struct MatVecArgs {
     int ngroups;         // workgroups (the launch's grid)
 };
 
+// Several decode matvecs of one type in one launch (grid y = matrix): matrix i computes
+// out[i][0:nrows[i]] = w[i] . act(i), act(i) = x + i*xstride (xstride 0: one shared
+// activation), optionally silu(x) * (x2 + i*xstride); matrix 0 may also add
+// alpha * out[0] into resid.
+#define JL_MAX_MULTI 16
+struct MatVecMultiArgs {
+    float* out[JL_MAX_MULTI];
+    const uint8_t* w[JL_MAX_MULTI];
+    int nrows[JL_MAX_MULTI];
+    const float* x;
+    const float* x2;     // null: plain activation
+    float* resid;        // null: none
+    float alpha;
+    size_t xstride;      // elements
+    int k, row_bytes, per, nwaves, ngroups;
+};
+
 // Activation preparation for the Q4_K prefill GEMM: quantize x and lay it out
 // in matrix-fragment order, bq [k/128 stages][tok_pad/32][9][64][8] f16, da [k/256][tok_pad].
 struct GemmPrepArgs {

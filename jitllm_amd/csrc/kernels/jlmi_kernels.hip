@@ -53,6 +53,13 @@ JL_MATVEC_KERNEL(q4k, JL_Q4_K, 1, 1024) JL_MATVEC_KERNEL(q4k, JL_Q4_K, 2, 1024) 
 JL_MATVEC_KERNEL(q8_0, JL_Q8_0, 1, 1024) JL_MATVEC_KERNEL(q8_0, JL_Q8_0, 2, 1024) JL_MATVEC_KERNEL(q8_0, JL_Q8_0, 4, 1024)
 JL_MATVEC_KERNEL(q6k, JL_Q6_K, 1, 1024) JL_MATVEC_KERNEL(q6k, JL_Q6_K, 2, 512) JL_MATVEC_KERNEL(q6k, JL_Q6_K, 4, 512)
 
+// grid = (row groups, matrices), block = 64..1024
+#define JL_MATVEC_MULTI_KERNEL(T, TYPE)                                                                \
+    extern "C" __global__ __launch_bounds__(1024) void jl_matvec_multi_##T(MatVecMultiArgs p) {        \
+        matvec_multi_body<TYPE>(p, jl_smem);                                                           \
+    }
+JL_MATVEC_MULTI_KERNEL(q4k, JL_Q4_K) JL_MATVEC_MULTI_KERNEL(q8_0, JL_Q8_0) JL_MATVEC_MULTI_KERNEL(q6k, JL_Q6_K)
+
 // ---------------------------------------------------------- packed planes
 // grid = (ceil(nrows/256), k/256 or k/32 for Q8_0), block = 256
 extern "C" __global__ __launch_bounds__(256) void jl_pack_weights(PackArgs p) { pack_weights_body(p); }

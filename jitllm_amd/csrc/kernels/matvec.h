@@ -406,3 +406,62 @@ __device__ __forceinline__ void matvec_body(const MatVecArgs& p, uint8_t* smem) 
         }
     }
 }
+
+// Several matvecs of one type in one launch: grid = (row groups, matrices).  Each
+// workgroup stages its matrix's activation (shared, or its own at xstride; optionally
+// silu(x) * x2 formed on the way into the quantizer) and then is the single-matrix
+// kernel with one row per wavefront.  The reference runs such sets as one pool region:
+// q/k/v or gate/up of a block (MatVecPackedGroup, engine/nn/packedgroup.go:13-51), a
+// mixture's experts at decode (MatVecPackedMulti / MatVecPackedGatherAct,
+// engine/nn/packedmulti.go:24,84,93); on this machine the saving is the per-launch cost.
+template <int TYPE>
+__device__ __forceinline__ void matvec_multi_body(const MatVecMultiArgs& p, uint8_t* smem) {
+    typedef SlotTraits<TYPE> T;
+    const int y = blockIdx.y;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = p.nwaves;
+    const int nthreads = nwaves * 64;
+    const int nrows = p.nrows[y];
+    const int nslots = p.k / T::kElems;
+    const int group_stride = p.ngroups * nwaves;
+    const ActLds A = act_lds_views(smem, p.k);
+    int r0 = blockIdx.x * nwaves + wave;
+    if ((int)blockIdx.x * nwaves >= nrows) return;   // uniform: this matrix has fewer row groups
+    const uint8_t* w0 = p.w[y];
+    const float* x = p.x + (size_t)y * p.xstride;
+    const float* x2 = p.x2 ? p.x2 + (size_t)y * p.xstride : nullptr;
+
+    const int n4 = p.k / 4, n4_pad = (n4 + 63) & ~63;
+    f32x4 x0 = ((const f32x4*)x)[min((int)threadIdx.x, n4 - 1)];
+    f32x4 u0 = x2 ? ((const f32x4*)x2)[min((int)threadIdx.x, n4 - 1)] : f32x4{1.f, 1.f, 1.f, 1.f};
+    __builtin_amdgcn_s_barrier();   // activation loads of the whole workgroup go out first
+    typename T::W w;
+    T::load_w(w0 + (size_t)min(r0, nrows - 1) * p.row_bytes, min(lane, nslots - 1), w);
+    for (int g4 = threadIdx.x; g4 < n4_pad; g4 += nthreads) {
+        f32x4 v = x0, u = u0;
+        if (g4 != (int)threadIdx.x) {
+            v = ((const f32x4*)x)[min(g4, n4 - 1)];
+            if (x2) u = ((const f32x4*)x2)[min(g4, n4 - 1)];
+        }
+        if (x2) v = f32x4{silu_f32(v.x) * u.x, silu_f32(v.y) * u.y, silu_f32(v.z) * u.z, silu_f32(v.w) * u.w};
+        stage_quantize4(smem, p.k, p.per, g4, v);
+    }
+    lds_barrier();
+
+    bool preloaded = true;
+    for (; r0 < nrows; r0 += group_stride) {
+        float acc = 0.f;
+        for (int slot = lane; slot < nslots; slot += 64) {
+            if (!preloaded) T::load_w(w0 + (size_t)r0 * p.row_bytes, slot, w);
+            preloaded = false;
+            typename T::Act a;
+            T::load_act(A, slot, a);
+            acc += T::dot(w, slot, a);
+        }
+        preloaded = false;
+        const float t = wave_sum_to_lane63(acc);
+        if (lane == 63) {
+            p.out[y][r0] = t;
+            if (y == 0 && p.resid) p.resid[r0] += p.alpha * t;
+        }
+    }
+}

@@ -204,8 +204,6 @@ __device__ __forceinline__ float group_sum(float v) {
     return v;
 }
 
-__device__ __forceinline__ float silu_f32(float g) { return g / (1.0f + __expf(-g)); }
-
 // --------------------------------------------------------- column activations
 // grid = (ceil(k/4/256), ncols), block = 256: one thread per four elements of a column.
 __device__ __forceinline__ void moe_quant_body(const MoeQuantArgs& p) {

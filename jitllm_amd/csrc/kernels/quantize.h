@@ -48,6 +48,9 @@ __device__ __forceinline__ u32 wave_amax_256(u32 m) {
     return (u32)__builtin_amdgcn_readlane((i32)m, 63);
 }
 
+// The gated activation of a feed-forward block, silu(g) = g / (1 + e^-g).
+__device__ __forceinline__ float silu_f32(float g) { return g / (1.0f + __expf(-g)); }
+
 // Round half away from zero for |p| < 2^22, exactly: adding 0.5 - 2^-25 (the
 // largest f32 below one half) cannot carry a value below n + 0.5 up to n + 1,
 // and carries every value at or above it; the conversion then truncates.

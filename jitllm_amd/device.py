@@ -183,6 +183,24 @@ class Device:
                                                      _ptr(a_s), _ptr(sum16), nrows, k, stream),
                             "jl_matvec_q8_dev")
 
+    def matvec_group_dev(self, outs, types, ws, rows, x, k, act_up=None, resid=None, alpha=0.0, stream=None):
+        """JIT.MatVecPackedGroup: up to four matvecs reading one activation, optional
+        silu(x) * act_up and resid += alpha * out[0], in one launch per weight type."""
+        g = _lib.MVGroup()
+        g.n = len(outs)
+        for i in range(g.n):
+            g.out[i], g.type[i], g.w[i], g.rows[i] = _ptr(outs[i]), types[i], _ptr(ws[i]), rows[i]
+        g.x, g.k, g.act_up, g.resid, g.alpha = _ptr(x), k, _opt(act_up), _opt(resid), alpha
+        return self._served(self._l.jl_matvec_group_dev(self._ctx, C.byref(g), stream), "jl_matvec_group_dev")
+
+    def matvec_gather_dev(self, outs, t, ws, x, xstride, up, nrows, k, stream=None):
+        """JIT.MatVecPackedGather[Act] (xstride > 0) / MatVecPackedMulti (xstride 0, up None)."""
+        m = len(outs)
+        po = (C.c_void_p * m)(*[_ptr(o) for o in outs])
+        pw = (C.c_void_p * m)(*[_ptr(w) for w in ws])
+        return self._served(self._l.jl_matvec_gather_dev(self._ctx, po, t, pw, _ptr(x), xstride, _opt(up),
+                                                         nrows, k, m, stream), "jl_matvec_gather_dev")
+
     def matmul_dev(self, out, t, w, x, nrows, k, ntok, stream=None):
         """x [ntok][k] -> out [ntok][nrows] on device operands (JIT.MatMulPacked semantics)."""
         return self._served(self._l.jl_matmul_dev(self._ctx, _ptr(out), t, _ptr(w), _ptr(x),

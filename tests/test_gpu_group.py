@@ -1,0 +1,112 @@
+"""GPU parity of the grouped decode matvecs (several matrices, one launch) against the
+oracle, through the C ABI.  Each matrix of a group is the decode matvec on it: the bar is
+the matvec's, NMSE <= 1e-10 against the f64 evaluation of the same int8 activations; the
+gated form (silu(x) * up inside the quantizer) is held to rel-L2 <= 1e-3 because exp()
+differs from numpy's in its last bits and can move an int8."""
+import numpy as np
+import pytest
+
+import oracle
+from conftest import nmse, rel_l2
+from jitllm_amd import quant, synth
+
+pytestmark = pytest.mark.gpu
+
+
+def _want(t, w, x, nrows, k, window):
+    q, a_s, _ = oracle.quantize_act(x, window)
+    return oracle.matvec_q8act_f64(t, w, q, a_s, nrows, k)
+
+
+def silu(g):
+    g = g.astype(np.float64)
+    return g / (1 + np.exp(-g))
+
+
+def test_group_qkv_mixed_types_one_activation(dev, devbuf):
+    """MatVecPackedGroup (/root/reference/engine/nn/packedgroup.go:13-51): q, k, v of a block."""
+    k, window = 2048, 32
+    dev.SetActWindow(window)
+    spec = [(quant.Q4_K, 520), (quant.Q4_K, 128), (quant.Q6_K, 130), (quant.Q8_0, 7)]
+    ws = [synth.quantized_weights(t, r, k, seed=i + 1) for i, (t, r) in enumerate(spec)]
+    x = synth.activations(k, seed=9)
+    dws, dx = [devbuf(w) for w in ws], devbuf(x)
+    outs = [devbuf(shape=(r + 4,), dtype=np.float32, fill=np.float32(6e30)) for _, r in spec]
+    assert dev.matvec_group_dev([o.ptr for o in outs], [t for t, _ in spec], [w.ptr for w in dws],
+                                [r for _, r in spec], dx.ptr, k)
+    dev.synchronize()
+    for (t, r), w, o in zip(spec, ws, outs):
+        got = o.get()
+        assert np.all(got[r:] == np.float32(6e30)), "wrote past the matrix's rows"
+        assert nmse(got[:r], _want(t, w, x, r, k, window)) <= 1e-10
+
+
+def test_group_gate_up_then_gated_down_with_residual(dev, devbuf):
+    """A gated feed-forward block as two groups: (gate, up) sharing x, then down over
+    silu(gate) * up with the residual add riding on the launch."""
+    n_embd, n_ffn, window = 1024, 2816, 32
+    dev.SetActWindow(window)
+    t_gu, t_d = quant.Q8_0, quant.Q6_K
+    wg = synth.quantized_weights(t_gu, n_ffn, n_embd, seed=1)
+    wu = synth.quantized_weights(t_gu, n_ffn, n_embd, seed=2)
+    wdn = synth.quantized_weights(t_d, n_embd, n_ffn, seed=3)
+    x = synth.activations(n_embd, seed=4)
+    dwg, dwu, dwd, dx = devbuf(wg), devbuf(wu), devbuf(wdn), devbuf(x)
+    g = devbuf(shape=(n_ffn,), dtype=np.float32, fill=0)
+    u = devbuf(shape=(n_ffn,), dtype=np.float32, fill=0)
+    assert dev.matvec_group_dev([g.ptr, u.ptr], [t_gu, t_gu], [dwg.ptr, dwu.ptr], [n_ffn, n_ffn], dx.ptr, n_embd)
+    dev.synchronize()
+    gh, uh = g.get(), u.get()
+    assert nmse(gh, _want(t_gu, wg, x, n_ffn, n_embd, window)) <= 1e-10
+    assert nmse(uh, _want(t_gu, wu, x, n_ffn, n_embd, window)) <= 1e-10
+    resid0 = synth.activations(n_embd, seed=5)
+    resid = devbuf(resid0)
+    y = devbuf(shape=(n_embd,), dtype=np.float32, fill=0)
+    alpha = np.float32(0.75)
+    assert dev.matvec_group_dev([y.ptr], [t_d], [dwd.ptr], [n_embd], g.ptr, n_ffn, act_up=u.ptr,
+                                resid=resid.ptr, alpha=float(alpha))
+    dev.synchronize()
+    yh = y.get()
+    h = (silu(gh) * uh.astype(np.float64)).astype(np.float32)
+    assert rel_l2(yh, _want(t_d, wdn, h, n_embd, n_ffn, window)) <= 1e-3
+    assert np.array_equal(resid.get(), (resid0 + (alpha * yh).astype(np.float32)).astype(np.float32))
+    assert np.array_equal(g.get(), gh), "the activation operand must be left as it was"
+    dev.SetActWindow(32)
+
+
+@pytest.mark.parametrize("t", [quant.Q4_K, quant.Q8_0, quant.Q6_K])
+def test_multi_and_gather(dev, devbuf, t):
+    """MatVecPackedMulti (one activation, a mixture's gate and up at decode) and
+    MatVecPackedGather / GatherAct (each matrix its own activation at a stride)."""
+    m, nrows, k = 16, 96, 1024
+    window = 256 if t in quant.K_QUANTS else 32
+    dev.SetActWindow(window)
+    ws = [synth.quantized_weights(t, nrows, k, seed=10 + i) for i in range(m)]
+    dws = [devbuf(w) for w in ws]
+    x = synth.activations(k, seed=1)
+    dx = devbuf(x)
+    outs = [devbuf(shape=(nrows,), dtype=np.float32, fill=np.float32(1e30)) for _ in range(m)]
+    assert dev.matvec_gather_dev([o.ptr for o in outs], t, [w.ptr for w in dws], dx.ptr, 0, None, nrows, k)
+    dev.synchronize()
+    for w, o in zip(ws, outs):
+        assert nmse(o.get(), _want(t, w, x, nrows, k, window)) <= 1e-10
+    # each matrix its own activation, stride k + 64 elements
+    stride = k + 64
+    xs = np.stack([np.concatenate([synth.activations(k, seed=30 + j), np.full(64, np.float32(9e9))]) for j in range(m)])
+    ups = np.stack([np.concatenate([synth.activations(k, seed=60 + j), np.full(64, np.float32(9e9))]) for j in range(m)])
+    dxs, dups = devbuf(xs), devbuf(ups)
+    assert dev.matvec_gather_dev([o.ptr for o in outs[:8]], t, [w.ptr for w in dws[:8]], dxs.ptr, stride, None,
+                                 nrows, k)
+    dev.synchronize()
+    for j in range(8):
+        assert nmse(outs[j].get(), _want(t, ws[j], xs[j, :k], nrows, k, window)) <= 1e-10
+    assert dev.matvec_gather_dev([o.ptr for o in outs[:8]], t, [w.ptr for w in dws[:8]], dxs.ptr, stride, dups.ptr,
+                                 nrows, k)
+    dev.synchronize()
+    for j in range(8):
+        h = (silu(xs[j, :k]) * ups[j, :k].astype(np.float64)).astype(np.float32)
+        assert rel_l2(outs[j].get(), _want(t, ws[j], h, nrows, k, window)) <= 1e-3
+    # more than sixteen matrices is a decline, not an error
+    many = [outs[0].ptr] * 17
+    assert dev.matvec_gather_dev(many, t, [dws[0].ptr] * 17, dx.ptr, 0, None, nrows, k) is False
+    dev.SetActWindow(32)
