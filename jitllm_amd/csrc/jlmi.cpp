@@ -31,6 +31,7 @@ struct Tuning {
     int packed_rw = 0, packed_block = 0;
     int moe_shares = 0;
     int gemm_rows = 0;
+    int gemm_form = 0;
     int mx_split = 0;
 };
 
@@ -57,6 +58,8 @@ struct jl_ctx {
     // prefill GEMM workspace (quantized activations in stage layout), grown on demand
     void* gemm_ws = nullptr;
     size_t gemm_ws_bytes = 0;
+    void* w16_ws = nullptr;   // expanded weights of the two-pass GEMM
+    size_t w16_ws_bytes = 0;
 
     void* mx_ws = nullptr;      // partial sums of a K-split MXFP4 matmul
     size_t mx_ws_bytes = 0;
@@ -291,7 +294,7 @@ constexpr unsigned kGemmLdsBytes = gemm_lds_bytes(128);
 constexpr size_t kGemmAStageBytes = 9 * 1024;  // per 32 tokens and stage: nine fragments of 64 lanes x 16 B
 
 size_t gemm_ws_need(int ntok, int k) {
-    size_t tok_pad = ((size_t)ntok + kGemmTile - 1) / kGemmTile * kGemmTile;
+    size_t tok_pad = ((size_t)ntok + 255) / 256 * 256;   // the widest token tile of any form
     size_t nsb = (size_t)k / 256;
     return nsb * 2 * (tok_pad / 32) * kGemmAStageBytes + nsb * tok_pad * 4;
 }
@@ -308,24 +311,77 @@ int gemm_ws_ensure(jl_ctx* c, size_t need) {
     return JL_OK;
 }
 
-// Q4_K prefill GEMM on the f16 matrix cores; operands are device pointers.
+constexpr size_t kGemmW16StageVecs = 1152;   // JL_GEMM_W16_STAGE_VECS
+constexpr unsigned kGemmW16LdsBytes = 2u * 1152u * 16u + 2u * kGemmTile * 4u;
+
+// Two-pass form: expand the weights into f16 fragments once, then the matrix kernel.
+int gemm_q4k_w16_launch(jl_ctx* c, float* out, const void* w, const uint16_t* bq, const float* da, int nrows,
+                        int k, int ntok, int tok_pad, hipStream_t st) {
+    const int nsb = k / 256;
+    const int nrt = (nrows + 63) / 64, nrows_pad = nrt * 64, ntt = tok_pad / kGemmTile;
+    const size_t w16_bytes = (size_t)nrt * 2 * nsb * kGemmW16StageVecs * 16;
+    const size_t need = w16_bytes + (size_t)nsb * nrows_pad * 8;
+    if (c->w16_ws_bytes < need) {
+        HIP_TRY(c, H->StreamSynchronize(c->stream));
+        if (st != c->stream) HIP_TRY(c, H->StreamSynchronize(st));
+        if (c->w16_ws) HIP_TRY(c, H->Free(c->w16_ws));
+        c->w16_ws = nullptr;
+        c->w16_ws_bytes = 0;
+        HIP_TRY(c, H->Malloc(&c->w16_ws, need));
+        c->w16_ws_bytes = need;
+    }
+    float* wsc = (float*)((char*)c->w16_ws + w16_bytes);
+    GemmW16PrepArgs pa;
+    pa.w = (const uint8_t*)w; pa.w16 = c->w16_ws; pa.wsc = wsc;
+    pa.nrows = nrows; pa.nrows_pad = nrows_pad; pa.k = k; pa.row_bytes = nsb * 144;
+    void* pp[] = {&pa};
+    int rc = launch(c, "jl_gemm_w16_prep_q4k", (unsigned)nsb, (unsigned)(nrows_pad / 32), 256, 0, st, pp);
+    if (rc != JL_OK) return rc;
+    GemmW16Args ga;
+    ga.out = out; ga.w16 = c->w16_ws; ga.wsc = wsc; ga.bq = bq; ga.da = da;
+    ga.nrows = nrows; ga.nrows_pad = nrows_pad; ga.k = k; ga.ntok = ntok; ga.tok_pad = tok_pad;
+    ga.ntt = ntt; ga.nrt = nrt;
+    void* gp[] = {&ga};
+    const unsigned groups = (unsigned)((nrt + 7) / 8 * 8) * (unsigned)ntt;
+    return launch(c, "jl_gemm_q4k_w16", groups, 1, 256, kGemmW16LdsBytes, st, gp);
+}
+
+// Q4_K prefill GEMM on the f16 matrix cores; operands are device pointers.  Forms (tuning
+// key "gemm.form", 0 = choose): 1 = 128-token x 64-row tiles, weights dequantized in the
+// kernel; 2 = 256-token x 128-row tiles, a wavefront across all 128 rows (least L1 traffic
+// per matrix instruction, for grids that still fill the chip); 3 = weights expanded once
+// per call into f16 fragments, then 128 x 64 tiles.
+constexpr int kGemmWideTok = 256;
+constexpr unsigned kGemmWideLdsBytes = 2u * 128u * 136u * 2u + 2u * 128u * 24u * 2u + 2u * 128u * 2u * 4u + 2u * kGemmWideTok * 4u;   // JL_GEMM_WIDE_LDS_BYTES
+
 int gemm_q4k_launch(jl_ctx* c, float* out, const void* w, const float* x, int nrows, int k, int ntok,
                     hipStream_t st) {
-    const int tok_pad = (ntok + kGemmTile - 1) / kGemmTile * kGemmTile;
+    int form = c->tune.gemm_form;
+    if (form == 0) {
+        const long wide_groups = (long)((ntok + kGemmWideTok - 1) / kGemmWideTok) * ((nrows + 127) / 128);
+        form = wide_groups >= c->num_cu ? 2 : 1;
+    }
+    if (form == 2 && kGemmWideLdsBytes > c->lds_limit) form = 1;
+    const int tile = form == 2 ? kGemmWideTok : kGemmTile;
+    const int tok_pad = (ntok + tile - 1) / tile * tile;
     const int nsb = k / 256;
-    int rc = gemm_ws_ensure(c, gemm_ws_need(ntok, k));
+    int rc = gemm_ws_ensure(c, gemm_ws_need(tok_pad, k));
     if (rc != JL_OK) return rc;
     uint16_t* bq = (uint16_t*)c->gemm_ws;
     float* da = (float*)((char*)c->gemm_ws + (size_t)nsb * 2 * (tok_pad / 32) * kGemmAStageBytes);
     GemmPrepArgs pa;
     pa.x = x; pa.bq = bq; pa.da = da; pa.ntok = ntok; pa.tok_pad = tok_pad; pa.k = k;
     void* pp[] = {&pa};
-    rc = launch(c, "jl_gemm_prep_q4k", (unsigned)nsb, (unsigned)(tok_pad / 4), 256, 0, st, pp);
+    rc = launch(c, "jl_gemm_prep_q4k", (unsigned)nsb, (unsigned)(tok_pad / 32), 256, 0, st, pp);
     if (rc != JL_OK) return rc;
+    if (form == 3) return gemm_q4k_w16_launch(c, out, w, bq, da, nrows, k, ntok, tok_pad, st);
     GemmArgs ga;
     ga.out = out; ga.w = (const uint8_t*)w; ga.bq = bq; ga.da = da;
     ga.nrows = nrows; ga.k = k; ga.ntok = ntok; ga.tok_pad = tok_pad; ga.row_bytes = nsb * 144;
     void* gp[] = {&ga};
+    if (form == 2)
+        return launch(c, "jl_gemm_q4k_wide", (unsigned)(tok_pad / kGemmWideTok), (unsigned)((nrows + 127) / 128),
+                      512, kGemmWideLdsBytes, st, gp);
     // 64-row workgroups, two to a CU, unless asked for the 128-row form
     const int rows = c->tune.gemm_rows == 128 ? 128 : 64;
     return launch(c, rows == 128 ? "jl_gemm_q4k_r128" : "jl_gemm_q4k_r64", (unsigned)(tok_pad / kGemmTile),
@@ -571,7 +627,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     if (e != hipSuccess)
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
-    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_q4k_r64", "jl_gemm_q4k_r128", "jl_moe_route", "jl_moe_group", "jl_moe_quant", "jl_moe_combine", "jl_mxfp4_gemm", "jl_mxfp4_matvec", "jl_sum_parts",
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_q4k_r64", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_moe_route", "jl_moe_group", "jl_moe_quant", "jl_moe_combine", "jl_mxfp4_gemm", "jl_mxfp4_matvec", "jl_sum_parts",
                                       "jl_pack_weights", "jl_unpack_q4k"};
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int rw : {16, 32, 64})
@@ -610,6 +666,7 @@ void jl_ctx_destroy(jl_ctx* c) {
     if (c->stream) (void)H->StreamSynchronize(c->stream);
     for (auto& kv : c->resident) (void)H->Free(kv.second.dev);
     if (c->gemm_ws) (void)H->Free(c->gemm_ws);
+    if (c->w16_ws) (void)H->Free(c->w16_ws);
     if (c->moe_ws) (void)H->Free(c->moe_ws);
     if (c->unpack_ws) (void)H->Free(c->unpack_ws);
     if (c->moe_q_ws) (void)H->Free(c->moe_q_ws);
@@ -650,6 +707,7 @@ int jl_set_tuning(jl_ctx* c, const char* key, int value) {
     else if (!strcmp(key, "moe.shares")) c->tune.moe_shares = value;
     else if (!strcmp(key, "gemm.rows")) c->tune.gemm_rows = value;
     else if (!strcmp(key, "mxfp4.split")) c->tune.mx_split = value;
+    else if (!strcmp(key, "gemm.form")) c->tune.gemm_form = value;
     else if (!strcmp(key, "gemm.min_tok")) c->gemm_min_tok = value > 0 ? value : 8;
     else return fail(c, JL_ERR_ARG, "unknown tuning key %s", key);
     return JL_OK;

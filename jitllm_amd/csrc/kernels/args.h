@@ -53,6 +53,28 @@ struct GemmArgs {
     int row_bytes;
 };
 
+// Two-pass form of the Q4_K prefill GEMM.  Pass one expands the weights once per call into
+// f16 matrix fragments, w16 [ceil(nrows/64)][k/128 stages][18 fragments][64 lanes] 16-byte
+// vectors (fragment 2*ks+g: K-step ks of the tile's row group g; 16+g: the minimum columns,
+// meaningful in second halves) and wsc [k/256][nrows_pad] (d, dmin); pass two is the matrix
+// kernel with nothing left to dequantize.
+struct GemmW16PrepArgs {
+    const uint8_t* w;    // GGUF row-major Q4_K
+    void* w16;           // 16-byte vectors
+    float* wsc;          // pairs (d, dmin)
+    int nrows, nrows_pad, k, row_bytes;
+};
+
+struct GemmW16Args {
+    float* out;          // [ntok][nrows]
+    const void* w16;
+    const float* wsc;
+    const uint16_t* bq;
+    const float* da;
+    int nrows, nrows_pad, k, ntok, tok_pad;
+    int ntt, nrt;        // token tiles (128) and row tiles (64)
+};
+
 // Mixture-of-experts grouping: sel [rows][sel_stride] expert ids (the first k_used of
 // each row are the selection) -> start [n_expert+1], perm [rows*k_used] (column ->
 // row), pos [rows*k_used] (pair -> column).

@@ -67,43 +67,79 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 // da [nsb][tok_pad] f32.  Position pos (0..143) of token t in a stage is K-step pos/16,
 // lane 32*((pos/8)%2) + t%32, element pos%8: positions 0..127 are the stage's weights in
 // the order the unpack emits them, 128..135 the sub-block sums' low parts, 136..143
-// their high parts.  One wavefront per (token, super-block); lane l owns elements 4l..4l+3.
-__device__ __forceinline__ _Float16* gemm_a_pos(_Float16* bq, int stage, int t, int tok_pad, int pos) {
-    const size_t frag = ((size_t)stage * (tok_pad >> 5) + (t >> 5)) * JL_GEMM_ASTAGE_FRAGS + (pos >> 4);
-    return bq + frag * JL_GEMM_AFRAG_HALFS + (32 * ((pos >> 3) & 1) + (t & 31)) * 8 + (pos & 7);
-}
-
-__device__ __forceinline__ void gemm_prep_q4k_body(const GemmPrepArgs& p) {
+// their high parts.
+// grid = (k/256, tok_pad/32), block = 256: 32 tokens of one super-block.  Each wavefront
+// quantizes eight tokens (lane l owns elements 4l..4l+3) into LDS; then every wavefront
+// assembles whole fragments, 16 bytes a lane and 1 KiB contiguous a store.
+#define JL_GEMM_PREP_LDS_WORDS (32 * 65 + 32 * 8)
+__device__ __forceinline__ void gemm_prep_q4k_body(const GemmPrepArgs& p, u32* lds) {
+    u32* sq = lds;                       // [32 tokens][65]: 64 words of int8 + 1 pad (bank spread)
+    i32* sA = (i32*)(lds + 32 * 65);     // [32 tokens][8 sub-block sums]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int sb = blockIdx.x;
-    const int t = blockIdx.y * 4 + wave;
-    if (t >= p.tok_pad) return;
-    f32x4 v = f32x4{0.f, 0.f, 0.f, 0.f};
-    if (t < p.ntok) v = ((const f32x4*)(p.x + (size_t)t * p.k + (size_t)sb * 256))[lane];
-    u32 m = max(max(abs_bits(v.x), abs_bits(v.y)), max(abs_bits(v.z), abs_bits(v.w)));
-    u32 amax = window_amax(m, 8);
-    float d;
-    i32 sum16;
-    u32 q = quantize4(v, amax, d, sum16);
-    // sub-block (32 elements = 8 lanes) sum from the two half-block sums
-    i32 a32 = sum16 + dpp_i32<JL_DPP_ROW_HALF_MIRROR, 0xf>(0, sum16);
-    const int g = lane >> 4, hi = (lane >> 3) & 1, c = lane & 7;
-    const int base = 8 * (8 * (g & 1) + c) + 2 * hi;
-    _Float16* bq = (_Float16*)p.bq;
-    f16x2 p02 = {(_Float16)(float)(int8_t)(q & 0xFF), (_Float16)(float)(int8_t)((q >> 16) & 0xFF)};
-    f16x2 p13 = {(_Float16)(float)(int8_t)((q >> 8) & 0xFF), (_Float16)(float)(int8_t)(q >> 24)};
-    *(f16x2*)gemm_a_pos(bq, sb * 2 + (g >> 1), t, p.tok_pad, base) = p02;
-    *(f16x2*)gemm_a_pos(bq, sb * 2 + (g >> 1), t, p.tok_pad, base + 4) = p13;
-    if ((lane & 7) == 0) {
-        const int s = lane >> 3;
-        *gemm_a_pos(bq, sb * 2 + 1, t, p.tok_pad, 128 + s) = (_Float16)(float)(a32 & 63);  // A = 64*A_hi + A_lo, 0 <= A_lo < 64
-        *gemm_a_pos(bq, sb * 2 + 1, t, p.tok_pad, 136 + s) = (_Float16)(float)(a32 >> 6);  // arithmetic shift: floor
+    const int sb = blockIdx.x, grp = blockIdx.y;
+    f32x4 v[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const int t = grp * 32 + wave * 8 + i;
+        v[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (t < p.ntok) v[i] = ((const f32x4*)(p.x + (size_t)t * p.k + (size_t)sb * 256))[lane];
     }
-    if (lane == 0) p.da[(size_t)sb * p.tok_pad + t] = d;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const int tl = wave * 8 + i;
+        const u32 m = max(max(abs_bits(v[i].x), abs_bits(v[i].y)), max(abs_bits(v[i].z), abs_bits(v[i].w)));
+        const u32 amax = wave_amax_256(m);
+        float d;
+        i32 sum16;
+        const u32 q = quantize4(v[i], amax, d, sum16);
+        // sub-block (32 elements = 8 lanes) sum from the two half-block sums
+        const i32 a32 = sum16 + dpp_i32<JL_DPP_ROW_HALF_MIRROR, 0xf>(0, sum16);
+        sq[tl * 65 + lane] = q;
+        if ((lane & 7) == 0) sA[tl * 8 + (lane >> 3)] = a32;
+        if (lane == 0) p.da[(size_t)sb * p.tok_pad + grp * 32 + tl] = d;
+    }
+    __syncthreads();
+    const int tl = lane & 31, kg = lane >> 5;
+    u32x4* dst = (u32x4*)p.bq;
+    const size_t ngrp = (size_t)(p.tok_pad >> 5);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int pi = wave * 4 + i, h = pi >> 3, ks = pi & 7;
+        // vector (group g, word c): low nibbles' partners are elements 4c.. of sub-block 2g,
+        // high nibbles' partners the same elements of sub-block 2g+1
+        const int g = 2 * h + (ks >> 2), c = 2 * (ks & 3) + kg;
+        const u32 lo = sq[tl * 65 + 16 * g + c], hi = sq[tl * 65 + 16 * g + 8 + c];
+        auto f = [](u32 w, int b) { return (_Float16)(float)(int8_t)(w >> (8 * b)); };
+        const f16x8 o = {f(lo, 0), f(lo, 2), f(hi, 0), f(hi, 2), f(lo, 1), f(lo, 3), f(hi, 1), f(hi, 3)};
+        dst[(((size_t)(2 * sb + h) * ngrp + grp) * JL_GEMM_ASTAGE_FRAGS + ks) * 64 + lane] =
+            __builtin_bit_cast(u32x4, o);
+    }
+    if (wave == 0) {
+        // A = 64*A_hi + A_lo with 0 <= A_lo < 64 (arithmetic shift: floor); lanes 0-31 carry
+        // the low parts, lanes 32-63 the high parts
+        f16x8 o;
+#pragma unroll
+        for (int s8 = 0; s8 < 8; s8++) {
+            const i32 a32 = sA[tl * 8 + s8];
+            o[s8] = (_Float16)(float)(kg ? (a32 >> 6) : (a32 & 63));
+        }
+        dst[(((size_t)(2 * sb + 1) * ngrp + grp) * JL_GEMM_ASTAGE_FRAGS + 8) * 64 + lane] =
+            __builtin_bit_cast(u32x4, o);
+    }
 }
 
 // -------------------------------------------------------------------- main
 template <int V> struct GemmIntC { static constexpr int value = V; };
+
+// f(GemmIntC<I>{}) for I = 0..N-1 with I a compile-time constant inside f: register arrays
+// indexed by it stay in registers.
+template <int I, int N, class F>
+__device__ __forceinline__ void gemm_static_for(F&& f) {
+    if constexpr (I < N) {
+        f(GemmIntC<I>{});
+        gemm_static_for<I + 1, N>(f);
+    }
+}
 
 // One stage of weights for a thread: row = tid/4, hh = (tid/2)%2 selects the 64-element
 // group (2*half + hh) of the super-block, wq = tid%2 the half of its 32 nibble bytes
@@ -340,6 +376,499 @@ __device__ __forceinline__ void gemm_q4k_body(const GemmArgs& p, uint8_t* smem) 
 #pragma unroll
     for (int j = 0; j < 2; j++) {
         const int r = r0 + 64 * rh + 32 * j + arow;
+        if (r >= p.nrows) continue;
+#pragma unroll
+        for (int e = 0; e < 16; e++) {
+            const int t = t0 + 32 * tg + 8 * (e >> 2) + 4 * kg + (e & 3);
+            if (t < p.ntok) p.out[(size_t)t * p.nrows + r] = out[j][e];
+        }
+    }
+}
+
+// ------------------------------------------------------------- wide form
+// What bounds the tiles above, measured: (1) the vector L1 path of a CU moves 64 bytes a
+// clock, a quarter of what LDS reads deliver, and carries the activation fragments; a
+// wavefront that owns 64 rows uses each fragment for only two matrix instructions.  (2) A
+// matrix instruction hides about four vector instructions issued beside it and nothing
+// more, and wavefronts that meet at a barrier every stage run their vector phases (scale
+// decode, minimum columns, the super-block epilogue) together, with the matrix cores idle.
+//
+// Here a wavefront owns 32 tokens x ALL 128 rows of the workgroup's tile, so a fragment
+// feeds four matrix instructions, and the eight wavefronts of a workgroup share one
+// dequantization of the weights over 256 tokens.  A stage is cut into 16 slots of two
+// matrix instructions (tile pair jh = slot/8, K-step ks = slot%8) and ALL vector work is
+// dealt out over the slots, a dozen instructions each:
+//   * the epilogue of a super-block runs one quarter tile per slot: tiles 0,1 under the
+//     second half's matrix instructions for tiles 2,3, and tiles 2,3 under the NEXT
+//     super-block's first-half instructions for tiles 0,1 (its accumulators are not
+//     restarted before slot 8); minimum columns and scales are kept per super-block parity
+//     so the deferred half still finds them;
+//   * the next stage's weights are dequantized in the other eight slots: scales in the
+//     first, a word of nibbles in every odd one, the minimum columns in the even ones.
+// grid = (tok_pad/256, ceil(nrows/128)), block = 512 (one workgroup per CU, two wavefronts
+// per SIMD), dynamic LDS = JL_GEMM_WIDE_LDS_BYTES.  tok_pad is a multiple of 256.
+#define JL_GEMM_WIDE_TOK 256
+#define JL_GEMM_WROW 136   // f16 per weight row of a stage: 128 + 8 (272 B: rows advance four banks)
+#define JL_GEMM_MROW 24    // f16 per row of minimum columns: 16 + 8
+#define JL_GEMM_WIDE_LDS_BYTES (2 * 128 * JL_GEMM_WROW * 2 + 2 * 128 * JL_GEMM_MROW * 2 + 2 * 128 * 2 * 4 + 2 * 256 * 4)
+
+// The 16 six-bit scales and minimums of a Q4_K super-block as bytes of four words
+// (format/quant/dequant.go:360-365, four at a time).
+struct GemmScaleBytes {
+    u32 sc_lo, sc_hi, mn_lo, mn_hi;   // sub-blocks 0-3 and 4-7
+};
+__device__ __forceinline__ GemmScaleBytes gemm_scale_bytes(u32 s0, u32 s1, u32 s2) {
+    GemmScaleBytes r;
+    r.sc_lo = s0 & 0x3F3F3F3Fu;
+    r.mn_lo = s1 & 0x3F3F3F3Fu;
+    r.sc_hi = (s2 & 0x0F0F0F0Fu) | ((s0 >> 2) & 0x30303030u);
+    r.mn_hi = ((s2 >> 4) & 0x0F0F0F0Fu) | ((s1 >> 2) & 0x30303030u);
+    return r;
+}
+
+// Multipliers and addends that turn the magic-number nibbles into sc*q: low nibbles read
+// (1024 + q), high nibbles are left in place and read (1024 + 16 q), so their multiplier
+// is sc/16 and their addend -64 sc; every product and sum is exact in f16.
+struct GemmWideScale {
+    f16x2 mlo, alo, mhi, ahi;
+    _Float16* dst;
+};
+__device__ __forceinline__ void gemm_wide_scale(const u32x4& hdr, int hh, int half, GemmWideScale& k) {
+    // sub-blocks 2g (low nibbles) and 2g+1 (high nibbles), g = 2*half + hh
+    const u32 word = half ? ((hdr.w & 0x0F0F0F0Fu) | ((hdr.y >> 2) & 0x30303030u)) : (hdr.y & 0x3F3F3F3Fu);
+    const u32 pair = word >> (16 * hh);
+    const float flo = (float)(pair & 0xFF), fhi = (float)((pair >> 8) & 0xFF);
+    const _Float16 hlo = (_Float16)flo, hhi16 = (_Float16)(fhi * 0.0625f);
+    const _Float16 nlo = (_Float16)(-1024.0f * flo), nhi = (_Float16)(-64.0f * fhi);
+    k.mlo = f16x2{hlo, hlo};
+    k.alo = f16x2{nlo, nlo};
+    k.mhi = f16x2{hhi16, hhi16};
+    k.ahi = f16x2{nhi, nhi};
+}
+__device__ __forceinline__ void gemm_wide_word(u32 w, const GemmWideScale& k, int c, u32 mask_lo, u32 mask_hi,
+                                               u32 magic) {
+    const u32 w8 = w >> 8;
+    auto nib = [&](u32 v, u32 mask) { return __builtin_bit_cast(f16x2, (v & mask) | magic); };
+    // (b0.lo, b2.lo), (b0.hi, b2.hi), (b1.lo, b3.lo), (b1.hi, b3.hi)
+    const f16x2 p0 = __builtin_elementwise_fma(nib(w, mask_lo), k.mlo, k.alo);
+    const f16x2 p1 = __builtin_elementwise_fma(nib(w, mask_hi), k.mhi, k.ahi);
+    const f16x2 p2 = __builtin_elementwise_fma(nib(w8, mask_lo), k.mlo, k.alo);
+    const f16x2 p3 = __builtin_elementwise_fma(nib(w8, mask_hi), k.mhi, k.ahi);
+    const u32x4 o = {__builtin_bit_cast(u32, p0), __builtin_bit_cast(u32, p1), __builtin_bit_cast(u32, p2),
+                     __builtin_bit_cast(u32, p3)};
+    *(u32x4*)(k.dst + 8 * c) = o;
+}
+
+__device__ __forceinline__ void gemm_q4k_wide_body(const GemmArgs& p, uint8_t* smem) {
+    constexpr int ROWS = 128, TOK = JL_GEMM_WIDE_TOK, STAGE_HALFS = ROWS * JL_GEMM_WROW;
+    constexpr int MIN_HALFS = ROWS * JL_GEMM_MROW;
+    _Float16* sW = (_Float16*)smem;                 // [2 stages][128][136]
+    _Float16* sMin = sW + 2 * STAGE_HALFS;          // [2 super-block parities][128][24]
+    float* sScale = (float*)(sMin + 2 * MIN_HALFS); // [2][128][2]  (d, dmin)
+    float* sDa = sScale + 2 * 2 * ROWS;             // [2][256]
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int tg = __builtin_amdgcn_readfirstlane(tid >> 6);   // wavefront tg: tokens 32*tg..
+    const int t0 = blockIdx.x * TOK, r0 = blockIdx.y * ROWS;
+    const int nsteps = 2 * (p.k / 256);
+    const int srow = tid >> 2, hh = (tid >> 1) & 1, wq = tid & 1;
+    const int arow = lane & 31, kg = lane >> 5;
+    // Addresses are a uniform 64-bit base (scalar registers) plus a 32-bit lane offset.
+    // Activation fragment (step, ks) of this wavefront's 32 tokens:
+    const size_t astride = (size_t)(p.tok_pad >> 5) * (JL_GEMM_ASTAGE_FRAGS * 1024);   // bytes per stage
+    const char* abase = (const char*)p.bq + ((size_t)(t0 >> 5) + tg) * (JL_GEMM_ASTAGE_FRAGS * 1024);
+    const unsigned aoff = lane * 16;
+    auto a_frag = [&](int step, int ks) {
+        return *(const f16x8*)(abase + (size_t)step * astride + ks * 1024 + aoff);
+    };
+    // This thread's share of a weight stage: 16 bytes of nibbles and the block header.
+    const uint8_t* wbase = p.w + (size_t)r0 * p.row_bytes;
+    const unsigned woff = (unsigned)(min(r0 + srow, p.nrows - 1) - r0) * (unsigned)p.row_bytes;
+    const unsigned wqoff = woff + 16 + 32 * hh + 16 * wq;
+    auto load_w = [&](int step, GemmWRegs& r) {
+        const uint8_t* blk = wbase + (size_t)(step >> 1) * 144 + 64 * (step & 1);
+        r.hdr = ld16(blk - 64 * (step & 1) + woff);
+        r.q = ld16(blk + wqoff);
+    };
+    u32 mask_lo = 0x000F000Fu, mask_hi = 0x00F000F0u, magic = 0x64006400u;
+    asm volatile("" : "+v"(mask_lo), "+v"(mask_hi), "+v"(magic));   // keep them in vector registers
+    const int wdst = srow * JL_GEMM_WROW + 64 * hh + 32 * wq;
+
+    f32x16 out[4], accP[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+#pragma unroll
+        for (int e = 0; e < 16; e++) out[j][e] = 0.f;
+
+    // prologue: stage 0 of the weights into LDS, stage 1 into registers, the first
+    // activation fragments into the ring
+    GemmWRegs wa, wb;
+    load_w(0, wa);
+    f16x8 aring[8], aaug;
+#pragma unroll
+    for (int ks = 0; ks < 8; ks++) aring[ks] = a_frag(0, ks);
+    aaug = a_frag(min(1, nsteps - 1), 8);
+    {
+        GemmWideScale k0;
+        gemm_wide_scale(wa.hdr, hh, 0, k0);
+        k0.dst = sW + wdst;
+#pragma unroll
+        for (int c = 0; c < 4; c++) gemm_wide_word(wa.q[c], k0, c, mask_lo, mask_hi, magic);
+    }
+    load_w(min(1, nsteps - 1), wa);
+    float da_reg = p.da[t0 + (tid & (TOK - 1))];
+    lds_barrier();
+
+    // One quarter (four tokens per lane) of tile `tile`'s epilogue, out += d_a * (d * P - dmin * M),
+    // with the scales of super-block parity eb.
+    f32x16 accM;
+    float2 esc;   // (d, dmin) of the tile's row
+    auto ep_quarter = [&](auto TILE, auto I, const f32x4& dav) __attribute__((always_inline)) {
+        constexpr int tile = decltype(TILE)::value, i = decltype(I)::value;
+#pragma unroll
+        for (int e4 = 0; e4 < 4; e4++) {
+            const int e = 4 * i + e4;
+            const float u = fmaf(esc.x, accP[tile][e], -(esc.y * accM[e]));
+            out[tile][e] = fmaf(dav[e4], u, out[tile][e]);
+        }
+    };
+
+    auto stage = [&](auto HALF, auto FIRST, int step, GemmWRegs& wcur, GemmWRegs& wnxt) {
+        constexpr int half = decltype(HALF)::value;
+        constexpr bool first = decltype(FIRST)::value != 0;
+        constexpr int nhalf = half ^ 1;
+        constexpr int ep_jh = half;            // tile pair whose slots carry the epilogue
+        constexpr bool has_ep = half == 1 || !first;
+        constexpr int ej0 = half ? 0 : 2;      // its tiles: 0,1 of this super-block / 2,3 of the last
+        const int sb = step >> 1;
+        const int eb = (half ? sb : sb - 1) & 1;
+        const _Float16* w = sW + half * STAGE_HALFS;
+        _Float16* wnext = sW + nhalf * STAGE_HALFS;
+        const int nstep = min(step + 1, nsteps - 1);
+        load_w(min(step + 2, nsteps - 1), wnxt);
+        const _Float16* wp0 = w + arow * JL_GEMM_WROW + 8 * kg;
+        const _Float16* mp0 = sMin + eb * MIN_HALFS + arow * JL_GEMM_MROW + 8 * kg;
+        const float* scp = sScale + eb * 2 * ROWS + 2 * arow;
+        const float* dap = sDa + eb * TOK + 32 * tg + 4 * kg;
+        auto w_frag = [&](int slot, int j) {
+            return *(const f16x8*)(wp0 + 32 * (2 * (slot >> 3) + j) * JL_GEMM_WROW + 16 * (slot & 7));
+        };
+        f16x8 wf[2][2], wm;
+        f32x4 dav;
+        GemmWideScale wsc;
+        wsc.dst = wnext + wdst;
+#pragma unroll
+        for (int j = 0; j < 2; j++) wf[0][j] = w_frag(0, j);
+        if (has_ep && ep_jh == 0) {
+            wm = *(const f16x8*)(mp0 + 32 * ej0 * JL_GEMM_MROW);
+            esc = *(const float2*)(scp + 2 * 32 * ej0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        gemm_static_for<0, 16>([&](auto SLOT) __attribute__((always_inline)) {
+            constexpr int slot = decltype(SLOT)::value, jh = slot >> 3, ks = slot & 7;
+            constexpr bool ep = has_ep && jh == ep_jh;
+            if (slot + 1 < 16) {
+#pragma unroll
+                for (int j = 0; j < 2; j++) wf[(slot + 1) & 1][j] = w_frag(slot + 1, j);
+            }
+            // operands of the epilogue a slot ahead: the next quarter's token scales, and
+            // before a tile's first quarter its minimum columns and row scales
+            // operands of the epilogue: this slot's token scales (the matrix instructions
+            // below cover the read), and a slot ahead of a tile's first quarter its minimum
+            // columns
+            if (ep) dav = *(const f32x4*)(dap + 8 * (ks & 3));
+            if (has_ep && ep_jh == 1 && slot == 7) {
+                wm = *(const f16x8*)(mp0 + 32 * ej0 * JL_GEMM_MROW);
+                esc = *(const float2*)(scp + 2 * 32 * ej0);
+            }
+            if (ep && ks == 3) wm = *(const f16x8*)(mp0 + 32 * (ej0 + 1) * JL_GEMM_MROW);   // (the first tile's M is done with it)
+            if (ep && ks == 4) esc = *(const float2*)(scp + 2 * 32 * (ej0 + 1));
+            __builtin_amdgcn_sched_barrier(0);
+            const f32x16 czero = {0};
+            if (ep && (ks & 3) == 0) {
+                // the tile's M = sum m_s A_s, ahead of this slot's instructions so that it is
+                // ready when the vector work below asks for it
+                accM = __builtin_amdgcn_mfma_f32_32x32x16_f16(aaug, wm, czero, 0, 0, 0);
+            }
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+                accP[2 * jh + j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                    aring[ks], wf[slot & 1][j], (half == 0 && ks == 0) ? czero : accP[2 * jh + j], 0, 0, 0);
+            if (jh == 1) {
+                aring[ks] = a_frag(nstep, ks);
+                if (ks == 0 && nhalf == 1) aaug = a_frag(nstep, 8);
+            }
+            if (ep) {
+                ep_quarter(GemmIntC<ej0 + (ks >> 2)>{}, GemmIntC<(ks & 3)>{}, dav);
+            } else if (jh != ep_jh) {
+                // the next stage's weights: wcur -> f16 -> LDS
+                if (ks == 0) gemm_wide_scale(wcur.hdr, hh, nhalf, wsc);
+                if (ks & 1) gemm_wide_word(wcur.q[ks >> 1], wsc, ks >> 1, mask_lo, mask_hi, magic);
+                if (nhalf == 1) {
+                    // a first half also lays down its super-block's minimum columns and scales
+                    // (no branches on the lane here: the four threads of a row that share an
+                    // address write the same value, which costs nothing and keeps the slot
+                    // one basic block)
+                    if (ks == 4) {
+                        const GemmScaleBytes sbytes = gemm_scale_bytes(wcur.hdr.y, wcur.hdr.z, wcur.hdr.w);
+                        // hh = 0 writes m_s (pairs with A_lo), hh = 1 writes 64*m_s (pairs with A_hi)
+                        const float mul = hh ? 64.0f : 1.0f;
+                        f16x8 mm;
+#pragma unroll
+                        for (int b = 0; b < 4; b++) {
+                            mm[b] = (_Float16)((float)((sbytes.mn_lo >> (8 * b)) & 0xFF) * mul);
+                            mm[4 + b] = (_Float16)((float)((sbytes.mn_hi >> (8 * b)) & 0xFF) * mul);
+                        }
+                        *(f16x8*)(sMin + (sb & 1) * MIN_HALFS + srow * JL_GEMM_MROW + 8 * hh) = mm;
+                    }
+                    if (ks == 6) {
+                        float2 dd = {half_bits_to_f32((uint16_t)(wcur.hdr.x & 0xFFFF)),
+                                     half_bits_to_f32((uint16_t)(wcur.hdr.x >> 16))};
+                        *(float2*)(sScale + (sb & 1) * 2 * ROWS + 2 * srow) = dd;
+                        sDa[(sb & 1) * TOK + (tid & (TOK - 1))] = da_reg;
+                    }
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        if (half == 1) {
+            const int sb2 = min(sb + 1, p.k / 256 - 1);
+            da_reg = p.da[(size_t)sb2 * p.tok_pad + t0 + (tid & (TOK - 1))];
+        }
+        lds_barrier();
+    };
+    stage(GemmIntC<0>{}, GemmIntC<1>{}, 0, wa, wb);
+    stage(GemmIntC<1>{}, GemmIntC<0>{}, 1, wb, wa);
+    for (int step = 2; step < nsteps; step += 2) {
+        stage(GemmIntC<0>{}, GemmIntC<0>{}, step, wa, wb);
+        stage(GemmIntC<1>{}, GemmIntC<0>{}, step + 1, wb, wa);
+    }
+    // tiles 2,3 of the last super-block
+    {
+        const int eb = (p.k / 256 - 1) & 1;
+        const f32x16 czero = {0};
+        gemm_static_for<2, 4>([&](auto TILE) __attribute__((always_inline)) {
+            constexpr int tile = decltype(TILE)::value;
+            const f16x8 wm = *(const f16x8*)(sMin + eb * MIN_HALFS + (32 * tile + arow) * JL_GEMM_MROW + 8 * kg);
+            esc = *(const float2*)(sScale + eb * 2 * ROWS + 2 * (32 * tile + arow));
+            accM = __builtin_amdgcn_mfma_f32_32x32x16_f16(aaug, wm, czero, 0, 0, 0);
+            gemm_static_for<0, 4>([&](auto I) __attribute__((always_inline)) {
+                constexpr int i = decltype(I)::value;
+                ep_quarter(TILE, I, *(const f32x4*)(sDa + eb * TOK + 32 * tg + 4 * kg + 8 * i));
+            });
+        });
+    }
+
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int r = r0 + 32 * j + arow;
+        if (r >= p.nrows) continue;
+#pragma unroll
+        for (int e = 0; e < 16; e++) {
+            const int t = t0 + 32 * tg + 8 * (e >> 2) + 4 * kg + (e & 3);
+            if (t < p.ntok) p.out[(size_t)t * p.nrows + r] = out[j][e];
+        }
+    }
+}
+
+// ------------------------------------------------------------- two-pass form
+// With several token tiles per weight tile the dequantization above is repeated for every
+// one of them, and it is vector work that the matrix cores wait for (an MFMA hides about
+// half of the vector instructions issued beside it, and the fused kernel issues nine per
+// MFMA).  From a few hundred tokens on it is cheaper to expand the weights ONCE per call
+// into f16 fragments in a workspace (2 bytes per weight, written and re-read at HBM/L2
+// speed) and run a matrix kernel whose only vector work is the super-block epilogue.
+// The values are the same integers either way, so both forms give the same sums.
+#define JL_GEMM_W16_STAGE_VECS 1152   // 16-byte vectors per (64 rows, stage): 16 weight fragments + 2 of minimums
+
+// grid = (k/256, nrows_pad/32), block = 256: 32 rows of one super-block.  The blocks are
+// read coalesced into LDS, then thread (row = tid%32, c = tid/32) expands word c of each of
+// the four 64-element groups: one 16-byte vector each, 1 KiB contiguous per wavefront.
+__device__ __forceinline__ void gemm_w16_prep_q4k_body(const GemmW16PrepArgs& p, u32* raw) {
+    const int tid = threadIdx.x, sb = blockIdx.x, tile32 = blockIdx.y;
+    const int nst = 2 * (p.k / 256);
+    for (int idx = tid; idx < 32 * 9; idx += 256) {
+        const int rl = idx / 9, v = idx - 9 * rl;
+        const int row = min(tile32 * 32 + rl, p.nrows - 1);
+        const u32x4 t = ld16(p.w + (size_t)row * p.row_bytes + (size_t)sb * 144 + 16 * v);
+        u32* d = raw + rl * 37 + 4 * v;   // 37-word rows: lanes of a wavefront hit distinct banks
+        d[0] = t.x; d[1] = t.y; d[2] = t.z; d[3] = t.w;
+    }
+    __syncthreads();
+    const int rl = tid & 31, c = tid >> 5;
+    const u32* rr = raw + rl * 37;
+    const u32 s0 = rr[1], s1 = rr[2], s2 = rr[3];
+    const int rg = tile32 & 1;
+    u32x4* dst = (u32x4*)p.w16 + ((size_t)(tile32 >> 1) * nst + 2 * sb) * JL_GEMM_W16_STAGE_VECS;
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+        u32 sclo, schi, mlo, mhi;
+        scale_min_k4(2 * g, s0, s1, s2, sclo, mlo);
+        scale_min_k4(2 * g + 1, s0, s1, s2, schi, mhi);
+        const u32 w = rr[4 + 8 * g + c];
+        // the order gemm_w_word emits: (b0.lo, b2.lo, b0.hi, b2.hi, b1.lo, b3.lo, b1.hi, b3.hi)
+        f16x8 v;
+        v[0] = (_Float16)(float)(sclo * (w & 15));
+        v[1] = (_Float16)(float)(sclo * ((w >> 16) & 15));
+        v[2] = (_Float16)(float)(schi * ((w >> 4) & 15));
+        v[3] = (_Float16)(float)(schi * ((w >> 20) & 15));
+        v[4] = (_Float16)(float)(sclo * ((w >> 8) & 15));
+        v[5] = (_Float16)(float)(sclo * ((w >> 24) & 15));
+        v[6] = (_Float16)(float)(schi * ((w >> 12) & 15));
+        v[7] = (_Float16)(float)(schi * (w >> 28));
+        const int ks = 4 * (g & 1) + (c >> 1);
+        dst[(size_t)(g >> 1) * JL_GEMM_W16_STAGE_VECS + (2 * ks + rg) * 64 + 32 * (c & 1) + rl] =
+            __builtin_bit_cast(u32x4, v);
+    }
+    if (c < 2) {   // c = 0: m_s (pairs with A_lo), c = 1: 64*m_s (pairs with A_hi)
+        const float mul = c ? 64.0f : 1.0f;
+        f16x8 mm;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            u32 scj, mnj;
+            scale_min_k4(j, s0, s1, s2, scj, mnj);
+            mm[j] = (_Float16)((float)mnj * mul);
+        }
+        dst[JL_GEMM_W16_STAGE_VECS + (16 + rg) * 64 + 32 * c + rl] = __builtin_bit_cast(u32x4, mm);
+    } else if (c == 2) {
+        float* o = p.wsc + 2 * ((size_t)sb * p.nrows_pad + tile32 * 32 + rl);
+        o[0] = half_bits_to_f32((uint16_t)(rr[0] & 0xFFFF));
+        o[1] = half_bits_to_f32((uint16_t)(rr[0] >> 16));
+    }
+}
+
+// grid = 8 * ceil(nrt/8) * ntt workgroups of 256 threads, dynamic LDS = two weight stages
+// of 1152 vectors + token scales [2][128].  Workgroups are dealt to the eight XCDs in turn,
+// so workgroup L takes row tile 8*(L/8/ntt) + L%8 and token tile (L/8)%ntt: all token tiles
+// of a row tile run on one XCD and its L2 fetches the expanded weights once.
+// A wavefront computes 32 tokens x 64 rows exactly as in the fused kernel; a weight stage
+// is a plain copy, global -> registers (a stage ahead) -> LDS in fragment order, four
+// vectors per thread spread between the K-steps.
+__device__ __forceinline__ void gemm_q4k_w16_body(const GemmW16Args& p, uint8_t* smem) {
+    u32x4* sW = (u32x4*)smem;
+    float* sDa = (float*)(sW + 2 * JL_GEMM_W16_STAGE_VECS);
+    const int tid = threadIdx.x, lane = tid & 63, tg = tid >> 6;
+    const int L = blockIdx.x, idx = L >> 3;
+    const int tt = idx % p.ntt, rt = (idx / p.ntt) * 8 + (L & 7);
+    if (rt >= p.nrt) return;
+    const int t0 = tt * JL_GEMM_TILE, r0 = rt * 64;
+    const int nsteps = 2 * (p.k / 256);
+    const u32x4* wsrc = (const u32x4*)p.w16 + (size_t)rt * nsteps * JL_GEMM_W16_STAGE_VECS;
+    const int arow = lane & 31, kg = lane >> 5;
+    const size_t ngrp = (size_t)(p.tok_pad >> 5), mygrp = (size_t)(t0 >> 5) + tg;
+    auto a_frag = [&](int step, int ks) {
+        return ((const f16x8*)p.bq)[(((size_t)step * ngrp + mygrp) * JL_GEMM_ASTAGE_FRAGS + ks) * 64 + lane];
+    };
+
+    f32x16 out[2], accP[2];
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+        for (int e = 0; e < 16; e++) out[j][e] = 0.f;
+
+    // prologue: stage 0 into LDS, stage 1 into registers, the first activation fragments
+    u32x4 wv[4], wvaug;
+#pragma unroll
+    for (int i = 0; i < 4; i++) wv[i] = wsrc[tid + 256 * i];
+    f16x8 aring[8], aaug;
+#pragma unroll
+    for (int ks = 0; ks < 8; ks++) aring[ks] = a_frag(0, ks);
+    aaug = aring[0];
+#pragma unroll
+    for (int i = 0; i < 4; i++) sW[tid + 256 * i] = wv[i];
+    {
+        const int s1 = min(1, nsteps - 1);
+#pragma unroll
+        for (int i = 0; i < 4; i++) wv[i] = wsrc[(size_t)s1 * JL_GEMM_W16_STAGE_VECS + tid + 256 * i];
+        wvaug = wsrc[(size_t)s1 * JL_GEMM_W16_STAGE_VECS + 1024 + (tid & 127)];
+    }
+    float da_reg = p.da[t0 + (tid & (JL_GEMM_TILE - 1))];
+    lds_barrier();
+
+    auto stage = [&](auto HALF, int step) {
+        constexpr int half = decltype(HALF)::value;
+        constexpr int nhalf = half ^ 1;
+        const int sb = step >> 1;
+        const u32x4* cur = sW + half * JL_GEMM_W16_STAGE_VECS;
+        u32x4* nxt = sW + nhalf * JL_GEMM_W16_STAGE_VECS;
+        const int nstep = min(step + 1, nsteps - 1);
+        const u32x4* w2 = wsrc + (size_t)min(step + 2, nsteps - 1) * JL_GEMM_W16_STAGE_VECS;
+        JL_TRACE(0);
+        float sc2[2][2];
+        if (half == 1) {
+            // the rows' (d, dmin) for this super-block's epilogue
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                const float* s = p.wsc + 2 * ((size_t)sb * p.nrows_pad + r0 + 32 * j + arow);
+                sc2[j][0] = s[0];
+                sc2[j][1] = s[1];
+            }
+        }
+        f16x8 wf[2][2];
+#pragma unroll
+        for (int j = 0; j < 2; j++) wf[0][j] = __builtin_bit_cast(f16x8, cur[j * 64 + lane]);
+        __builtin_amdgcn_sched_barrier(0);
+        JL_TRACE(2);
+#pragma unroll
+        for (int ks = 0; ks < 8; ks++) {
+            if (ks + 1 < 8) {
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+                    wf[(ks + 1) & 1][j] = __builtin_bit_cast(f16x8, cur[(2 * (ks + 1) + j) * 64 + lane]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            const f32x16 czero = {0};
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+                accP[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aring[ks], wf[ks & 1][j],
+                                                                 (half == 0 && ks == 0) ? czero : accP[j], 0, 0, 0);
+            aring[ks] = a_frag(nstep, ks);
+            if (ks == 0 && nhalf == 1) aaug = a_frag(nstep, 8);
+            if (ks & 1) {
+                // one vector of the next stage into LDS, its register refilled for the stage after
+                const int i = ks >> 1;
+                nxt[tid + 256 * i] = wv[i];
+                wv[i] = w2[tid + 256 * i];
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (nhalf == 1) {
+            // the next stage is a second half: its minimum columns and the token scales
+            if (tid < 128) nxt[1024 + tid] = wvaug;
+            if (tid < JL_GEMM_TILE) sDa[(sb & 1) * JL_GEMM_TILE + tid] = da_reg;
+        } else {
+            wvaug = w2[1024 + (tid & 127)];
+            const int sb2 = min(sb + 1, p.k / 256 - 1);
+            da_reg = p.da[(size_t)sb2 * p.tok_pad + t0 + (tid & (JL_GEMM_TILE - 1))];
+        }
+        JL_TRACE(3);
+        if (half == 1) {
+            const f32x16 zero = {0};
+            const float* sda = sDa + (sb & 1) * JL_GEMM_TILE + 32 * tg;
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                const f16x8 wm = __builtin_bit_cast(f16x8, cur[(16 + j) * 64 + lane]);
+                const f32x16 accM = __builtin_amdgcn_mfma_f32_32x32x16_f16(aaug, wm, zero, 0, 0, 0);
+#pragma unroll
+                for (int e = 0; e < 16; e++) {
+                    const int tk = 8 * (e >> 2) + 4 * kg + (e & 3);
+                    const float u = fmaf(sc2[j][0], accP[j][e], -(sc2[j][1] * accM[e]));
+                    out[j][e] = fmaf(sda[tk], u, out[j][e]);
+                }
+            }
+        }
+        JL_TRACE(4);
+        lds_barrier();
+        JL_TRACE(5);
+    };
+    for (int step = 0; step < nsteps; step += 2) {
+        stage(GemmIntC<0>{}, step);
+        stage(GemmIntC<1>{}, step + 1);
+    }
+
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        const int r = r0 + 32 * j + arow;
         if (r >= p.nrows) continue;
 #pragma unroll
         for (int e = 0; e < 16; e++) {

@@ -81,11 +81,20 @@ JL_PACKED_KERNEL(q6k, JL_Q6_K, 64, 4) JL_PACKED_KERNEL(q6k, JL_Q6_K, 32, 4) JL_P
 
 // ------------------------------------------------------------ prefill GEMM
 // grid = (k/256, tok_pad/4), block = 256: one wavefront per (token, super-block)
-extern "C" __global__ __launch_bounds__(256) void jl_gemm_prep_q4k(GemmPrepArgs p) { gemm_prep_q4k_body(p); }
+extern "C" __global__ __launch_bounds__(256) void jl_gemm_prep_q4k(GemmPrepArgs p) {
+    __shared__ u32 lds[JL_GEMM_PREP_LDS_WORDS];
+    gemm_prep_q4k_body(p, lds);
+}
 // grid = (tok_pad/128, ceil(nrows/64)), block = 256, two workgroups per CU; and the
 // 128-row form on 512 threads
 extern "C" __global__ __launch_bounds__(256, 2) void jl_gemm_q4k_r64(GemmArgs p) { gemm_q4k_body<1>(p, jl_smem); }
 extern "C" __global__ __launch_bounds__(512) void jl_gemm_q4k_r128(GemmArgs p) { gemm_q4k_body<2>(p, jl_smem); }
+extern "C" __global__ __launch_bounds__(512) void jl_gemm_q4k_wide(GemmArgs p) { gemm_q4k_wide_body(p, jl_smem); }
+extern "C" __global__ __launch_bounds__(256) void jl_gemm_w16_prep_q4k(GemmW16PrepArgs p) {
+    __shared__ u32 raw[32 * 37];
+    gemm_w16_prep_q4k_body(p, raw);
+}
+extern "C" __global__ __launch_bounds__(256, 2) void jl_gemm_q4k_w16(GemmW16Args p) { gemm_q4k_w16_body(p, jl_smem); }
 
 // ------------------------------------------------------- mixture of experts
 // grid = rows, block = 64

@@ -22,10 +22,14 @@ def _oracle_matmul(t, w, x, nrows, k, ntok, window):
 @pytest.mark.parametrize("shape", [(16, 128, 256), (130, 200, 512), (8, 37, 1024), (512, 300, 1024),
                                    (129, 129, 4096)], ids=lambda s: "x".join(map(str, s)))
 @pytest.mark.parametrize("weights", ["normal", "planted"])
-def test_gemm_q4k_vs_oracle(dev, devbuf, shape, weights):
+@pytest.mark.parametrize("form", [1, 2, 3], ids=["tile128x64", "tile256x128", "two_pass"])
+def test_gemm_q4k_vs_oracle(dev, devbuf, shape, weights, form):
+    """Every form of the kernel: weights dequantized inside the matrix kernel on 128 x 64 and
+    on 256 x 128 tiles, and weights expanded once per call into f16 fragments."""
     ntok, nrows, k = shape
     t = quant.Q4_K
     dev.SetActWindow(256)
+    dev.set_tuning(gemm__form=form)
     w = (synth.quantized_weights(t, nrows, k, seed=ntok) if weights == "normal"
          else synth.random_weights(t, nrows, k, seed=ntok))
     x = np.stack([synth.activations(k, seed=100 + i) * np.float32(1 + i % 7) for i in range(ntok)])
@@ -45,6 +49,30 @@ def test_gemm_q4k_vs_oracle(dev, devbuf, shape, weights):
         assert worst <= 1e-9, f"worst token NMSE {worst:.3e}"
         assert np.all(got[ntok // 2] == 0)
         assert rel_l2(got, want) <= 1e-3
+    dev.SetActWindow(32)
+    dev.set_tuning(gemm__form=0)
+
+
+def test_gemm_forms_agree_bit_for_bit(dev, devbuf):
+    """The matrix cores sum the same integers in both forms and the f32 epilogue is the
+    same instruction sequence, so all forms must return identical bits; a second
+    weight of another shape reuses (and regrows) the expanded-weight workspace."""
+    dev.SetActWindow(256)
+    t = quant.Q4_K
+    for ntok, nrows, k in [(200, 300, 1536), (130, 70, 512), (384, 1000, 2048)]:
+        w = synth.random_weights(t, nrows, k, seed=nrows)
+        x = np.stack([synth.activations(k, seed=500 + i) for i in range(ntok)])
+        wd, xd = devbuf(w), devbuf(x)
+        outs = []
+        for form in (1, 2, 3):
+            dev.set_tuning(gemm__form=form)
+            out = devbuf(shape=(ntok, nrows), dtype=np.float32, fill=np.float32(-7e30))
+            assert dev.matmul_dev(out.ptr, t, wd.ptr, xd.ptr, nrows, k, ntok)
+            dev.synchronize()
+            outs.append(out.get())
+        for o in outs[1:]:
+            assert np.array_equal(outs[0].view(np.uint32), o.view(np.uint32)), (ntok, nrows, k)
+    dev.set_tuning(gemm__form=0)
     dev.SetActWindow(32)
 
 
