@@ -378,14 +378,29 @@ int gemm_q4k_launch(jl_ctx* c, float* out, const void* w, const float* x, int nr
     GemmArgs ga;
     ga.out = out; ga.w = (const uint8_t*)w; ga.bq = bq; ga.da = da;
     ga.nrows = nrows; ga.k = k; ga.ntok = ntok; ga.tok_pad = tok_pad; ga.row_bytes = nsb * 144;
+    ga.out_stride = nrows;
     void* gp[] = {&ga};
-    if (form == 2)
-        return launch(c, "jl_gemm_q4k_wide", (unsigned)(tok_pad / kGemmWideTok), (unsigned)((nrows + 127) / 128),
-                      512, kGemmWideLdsBytes, st, gp);
+    int rows_left = nrows;
+    if (form == 2) {
+        // One workgroup per CU: a grid of f full rounds and a last round at most half full
+        // leaves half the chip idle for a whole round.  The rows of that last round go to the
+        // 128 x 64 tiles instead (two workgroups per CU), which fill the chip once more.
+        const long ntt = tok_pad / kGemmWideTok, nrt = (nrows + 127) / 128;
+        const long full = ntt * nrt / c->num_cu, rem = ntt * nrt - full * c->num_cu;
+        long nrt_wide = nrt;
+        if (c->tune.gemm_form == 0 && full >= 1 && rem > 0 && 2 * rem <= c->num_cu) nrt_wide = full * c->num_cu / ntt;
+        ga.nrows = nrt_wide == nrt ? nrows : (int)(nrt_wide * 128);
+        rc = launch(c, "jl_gemm_q4k_wide", (unsigned)ntt, (unsigned)nrt_wide, 512, kGemmWideLdsBytes, st, gp);
+        rows_left = nrows - ga.nrows;
+        if (rc != JL_OK || rows_left == 0) return rc;
+        ga.w += (size_t)ga.nrows * ga.row_bytes;
+        ga.out += ga.nrows;
+        ga.nrows = rows_left;
+    }
     // 64-row workgroups, two to a CU, unless asked for the 128-row form
     const int rows = c->tune.gemm_rows == 128 ? 128 : 64;
     return launch(c, rows == 128 ? "jl_gemm_q4k_r128" : "jl_gemm_q4k_r64", (unsigned)(tok_pad / kGemmTile),
-                  (unsigned)((nrows + rows - 1) / rows), rows == 128 ? 512 : 256, gemm_lds_bytes(rows), st, gp);
+                  (unsigned)((rows_left + rows - 1) / rows), rows == 128 ? 512 : 256, gemm_lds_bytes(rows), st, gp);
 }
 
 // out [ntok][nrows] = x [ntok][k] W^T on device operands: the matrix-core GEMM where it

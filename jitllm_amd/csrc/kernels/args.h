@@ -45,12 +45,13 @@ struct GemmPrepArgs {
 };
 
 struct GemmArgs {
-    float* out;          // [ntok][nrows]
-    const uint8_t* w;    // GGUF row-major Q4_K
+    float* out;          // [ntok][out_stride]; a launch may cover a slice of the rows
+    const uint8_t* w;    // GGUF row-major Q4_K (of the slice)
     const uint16_t* bq;
     const float* da;
-    int nrows, k, ntok, tok_pad;
+    int nrows, k, ntok, tok_pad;   // nrows of the slice
     int row_bytes;
+    int out_stride;      // floats between tokens in out
 };
 
 // Two-pass form of the Q4_K prefill GEMM.  Pass one expands the weights once per call into

@@ -380,7 +380,7 @@ __device__ __forceinline__ void gemm_q4k_body(const GemmArgs& p, uint8_t* smem) 
 #pragma unroll
         for (int e = 0; e < 16; e++) {
             const int t = t0 + 32 * tg + 8 * (e >> 2) + 4 * kg + (e & 3);
-            if (t < p.ntok) p.out[(size_t)t * p.nrows + r] = out[j][e];
+            if (t < p.ntok) p.out[(size_t)t * p.out_stride + r] = out[j][e];
         }
     }
 }
@@ -666,7 +666,7 @@ __device__ __forceinline__ void gemm_q4k_wide_body(const GemmArgs& p, uint8_t* s
 #pragma unroll
         for (int e = 0; e < 16; e++) {
             const int t = t0 + 32 * tg + 8 * (e >> 2) + 4 * kg + (e & 3);
-            if (t < p.ntok) p.out[(size_t)t * p.nrows + r] = out[j][e];
+            if (t < p.ntok) p.out[(size_t)t * p.out_stride + r] = out[j][e];
         }
     }
 }

@@ -76,6 +76,31 @@ def test_gemm_forms_agree_bit_for_bit(dev, devbuf):
     dev.SetActWindow(32)
 
 
+def test_gemm_split_grid_agrees_with_single_form(dev, devbuf):
+    """A grid of whole rounds plus a last round at most half full is cut: the last round's
+    rows go to the 64-row tiles.  1.25 rounds of 256-token x 128-row tiles on 256 CUs
+    (and a ragged last tile) against the single-form result, bit for bit; a spot check of
+    one token against the oracle."""
+    dev.SetActWindow(256)
+    t, ntok, k = quant.Q4_K, 256, 256
+    nrows = 128 * (256 + 64) + 37
+    w = synth.random_weights(t, nrows, k, seed=9)
+    x = np.stack([synth.activations(k, seed=900 + i) for i in range(ntok)])
+    wd, xd = devbuf(w), devbuf(x)
+    outs = []
+    for form in (0, 1):
+        dev.set_tuning(gemm__form=form)
+        out = devbuf(shape=(ntok, nrows), dtype=np.float32, fill=np.float32(-7e30))
+        assert dev.matmul_dev(out.ptr, t, wd.ptr, xd.ptr, nrows, k, ntok)
+        dev.synchronize()
+        outs.append(out.get())
+    dev.set_tuning(gemm__form=0)
+    assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))
+    want = _oracle_matmul(t, w, x[5:6], nrows, k, 1, 256)
+    assert nmse(outs[0][5:6], want) <= 1e-10
+    dev.SetActWindow(32)
+
+
 def test_gemm_token_equals_decode_matvec(dev, devbuf):
     ntok, nrows, k, t = 40, 256, 2048, quant.Q4_K
     dev.SetActWindow(256)
