@@ -32,6 +32,7 @@ struct Tuning {
     int moe_shares = 0;
     int gemm_rows = 0;
     int gemm_form = 0;
+    int gemm_split = 0;
     int mx_split = 0;
 };
 
@@ -61,7 +62,7 @@ struct jl_ctx {
     void* w16_ws = nullptr;   // expanded weights of the two-pass GEMM
     size_t w16_ws_bytes = 0;
 
-    void* mx_ws = nullptr;      // partial sums of a K-split MXFP4 matmul
+    void* mx_ws = nullptr;      // partial sums of a K-split matmul (MXFP4, Q4_K)
     size_t mx_ws_bytes = 0;
     void* moe_q_ws = nullptr;   // quantized column activations of a mixture pass
     size_t moe_q_ws_bytes = 0;
@@ -285,6 +286,8 @@ int resident_weight(jl_ctx* c, const void* w, size_t bytes, void** dev) {
     return JL_OK;
 }
 
+int ws_ensure(jl_ctx* c, void** buf, size_t* have, size_t need);
+
 constexpr int kGemmTile = 128;         // tokens and rows per workgroup (kernels/gemm_q4k.h)
 constexpr int kGemmStride = 152;       // f16 per stage row
 constexpr unsigned gemm_lds_bytes(int rows) {   // two weight stages, row scales, token scales
@@ -378,7 +381,7 @@ int gemm_q4k_launch(jl_ctx* c, float* out, const void* w, const float* x, int nr
     GemmArgs ga;
     ga.out = out; ga.w = (const uint8_t*)w; ga.bq = bq; ga.da = da;
     ga.nrows = nrows; ga.k = k; ga.ntok = ntok; ga.tok_pad = tok_pad; ga.row_bytes = nsb * 144;
-    ga.out_stride = nrows;
+    ga.out_stride = nrows; ga.sb_per = 0;
     void* gp[] = {&ga};
     int rows_left = nrows;
     if (form == 2) {
@@ -399,6 +402,29 @@ int gemm_q4k_launch(jl_ctx* c, float* out, const void* w, const float* x, int nr
     }
     // 64-row workgroups, two to a CU, unless asked for the 128-row form
     const int rows = c->tune.gemm_rows == 128 ? 128 : 64;
+    if (rows == 64 && rows_left == nrows) {
+        // a grid that leaves most of the chip idle (few tokens) is widened along K
+        const long groups = (long)(tok_pad / kGemmTile) * ((nrows + 63) / 64);
+        int nsplit = c->tune.gemm_split > 0 ? c->tune.gemm_split
+                     : (c->tune.gemm_form == 0 && groups <= c->num_cu ? (int)(2 * c->num_cu / groups) : 1);
+        if (nsplit > 8) nsplit = 8;
+        if (nsplit > nsb) nsplit = nsb;
+        if (nsplit > 1) {
+            const int per = (nsb + nsplit - 1) / nsplit;
+            nsplit = (nsb + per - 1) / per;   // no empty split
+            const size_t n = (size_t)ntok * nrows;
+            rc = ws_ensure(c, &c->mx_ws, &c->mx_ws_bytes, n * nsplit * 4);
+            if (rc != JL_OK) return rc;
+            ga.out = (float*)c->mx_ws; ga.sb_per = per;
+            HIP_TRY(c, H->ModuleLaunchKernel(c->fn["jl_gemm_q4k_r64"], (unsigned)(tok_pad / kGemmTile),
+                                             (unsigned)((nrows + 63) / 64), (unsigned)nsplit, 256, 1, 1,
+                                             gemm_lds_bytes(64), st, gp, nullptr));
+            SumPartsArgs sa;
+            sa.out = out; sa.part = (const float*)c->mx_ws; sa.n = n; sa.nsplit = nsplit;
+            void* sp[] = {&sa};
+            return launch(c, "jl_sum_parts", (unsigned)((n + 255) / 256), 1, 256, 0, st, sp);
+        }
+    }
     return launch(c, rows == 128 ? "jl_gemm_q4k_r128" : "jl_gemm_q4k_r64", (unsigned)(tok_pad / kGemmTile),
                   (unsigned)((rows_left + rows - 1) / rows), rows == 128 ? 512 : 256, gemm_lds_bytes(rows), st, gp);
 }
@@ -723,6 +749,7 @@ int jl_set_tuning(jl_ctx* c, const char* key, int value) {
     else if (!strcmp(key, "gemm.rows")) c->tune.gemm_rows = value;
     else if (!strcmp(key, "mxfp4.split")) c->tune.mx_split = value;
     else if (!strcmp(key, "gemm.form")) c->tune.gemm_form = value;
+    else if (!strcmp(key, "gemm.split")) c->tune.gemm_split = value;
     else if (!strcmp(key, "gemm.min_tok")) c->gemm_min_tok = value > 0 ? value : 8;
     else return fail(c, JL_ERR_ARG, "unknown tuning key %s", key);
     return JL_OK;

@@ -52,6 +52,7 @@ struct GemmArgs {
     int nrows, k, ntok, tok_pad;   // nrows of the slice
     int row_bytes;
     int out_stride;      // floats between tokens in out
+    int sb_per;          // K split: super-blocks per blockIdx.z (0 = whole K), out = slab z of [gridDim.z][ntok][out_stride]
 };
 
 // Two-pass form of the Q4_K prefill GEMM.  Pass one expands the weights once per call into

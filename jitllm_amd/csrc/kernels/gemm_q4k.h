@@ -230,6 +230,19 @@ __device__ __forceinline__ void gemm_w_mins(const GemmWRegs& r, int row, int hh,
     }
 }
 
+// A grid too small for the chip is widened along K: workgroup z takes sb_per super-blocks
+// and writes its partial sums to slab z; the slabs are added in order afterwards.
+__device__ __forceinline__ void gemm_split_slice(GemmArgs& p) {
+    if (p.sb_per == 0) return;
+    const int sb0 = blockIdx.z * p.sb_per;
+    const int n = min(p.sb_per, p.k / 256 - sb0);
+    p.w += (size_t)sb0 * 144;
+    p.bq += (size_t)2 * sb0 * (p.tok_pad >> 5) * (JL_GEMM_ASTAGE_FRAGS * JL_GEMM_AFRAG_HALFS);
+    p.da += (size_t)sb0 * p.tok_pad;
+    p.k = 256 * n;
+    p.out += (size_t)blockIdx.z * p.ntok * p.out_stride;
+}
+
 // RH = groups of four wavefronts in the workgroup, each group 64 rows: RH = 2 is the
 // 128 x 128 tile on eight wavefronts; RH = 1 a 128-token x 64-row tile on four, of which
 // two workgroups share a CU -- they drift apart, so one's vector phases (dequantization,

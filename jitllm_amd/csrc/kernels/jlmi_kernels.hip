@@ -87,7 +87,10 @@ extern "C" __global__ __launch_bounds__(256) void jl_gemm_prep_q4k(GemmPrepArgs 
 }
 // grid = (tok_pad/128, ceil(nrows/64)), block = 256, two workgroups per CU; and the
 // 128-row form on 512 threads
-extern "C" __global__ __launch_bounds__(256, 2) void jl_gemm_q4k_r64(GemmArgs p) { gemm_q4k_body<1>(p, jl_smem); }
+extern "C" __global__ __launch_bounds__(256, 2) void jl_gemm_q4k_r64(GemmArgs p) {
+    gemm_split_slice(p);
+    gemm_q4k_body<1>(p, jl_smem);
+}
 extern "C" __global__ __launch_bounds__(512) void jl_gemm_q4k_r128(GemmArgs p) { gemm_q4k_body<2>(p, jl_smem); }
 extern "C" __global__ __launch_bounds__(512) void jl_gemm_q4k_wide(GemmArgs p) { gemm_q4k_wide_body(p, jl_smem); }
 extern "C" __global__ __launch_bounds__(256) void jl_gemm_w16_prep_q4k(GemmW16PrepArgs p) {

@@ -101,6 +101,28 @@ def test_gemm_split_grid_agrees_with_single_form(dev, devbuf):
     dev.SetActWindow(32)
 
 
+@pytest.mark.parametrize("split", [0, 2, 3, 8])
+def test_gemm_k_split_vs_oracle(dev, devbuf, split):
+    """Few tokens leave most of the chip idle, so K is cut across workgroups and the partial
+    sums are added in a fixed order; every split count meets the same bar."""
+    dev.SetActWindow(256)
+    t, ntok, nrows, k = quant.Q4_K, 20, 150, 2816   # 11 super-blocks: a short last split
+    w = synth.random_weights(t, nrows, k, seed=split)
+    x = np.stack([synth.activations(k, seed=300 + i) for i in range(ntok)])
+    want = _oracle_matmul(t, w, x, nrows, k, ntok, 256)
+    wd, xd = devbuf(w), devbuf(x)
+    dev.set_tuning(gemm__split=split)
+    for call in range(2):
+        out = devbuf(shape=(ntok * nrows + 8,), dtype=np.float32, fill=np.float32(4e30))
+        assert dev.matmul_dev(out.ptr, t, wd.ptr, xd.ptr, nrows, k, ntok)
+        dev.synchronize()
+        got = out.get()
+        assert np.all(got[ntok * nrows:] == np.float32(4e30))
+        assert nmse(got[:ntok * nrows].reshape(ntok, nrows), want) <= 1e-10
+    dev.set_tuning(gemm__split=0)
+    dev.SetActWindow(32)
+
+
 def test_gemm_token_equals_decode_matvec(dev, devbuf):
     ntok, nrows, k, t = 40, 256, 2048, quant.Q4_K
     dev.SetActWindow(256)
