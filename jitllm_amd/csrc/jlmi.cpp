@@ -362,7 +362,7 @@ int gemm_q4k_launch(jl_ctx* c, float* out, const void* w, const float* x, int nr
     int form = c->tune.gemm_form;
     if (form == 0) {
         const long wide_groups = (long)((ntok + kGemmWideTok - 1) / kGemmWideTok) * ((nrows + 127) / 128);
-        form = wide_groups >= c->num_cu ? 2 : 1;
+        form = 4 * wide_groups >= 3 * (long)c->num_cu ? 2 : 1;   // one round at least three quarters full
     }
     if (form == 2 && kGemmWideLdsBytes > c->lds_limit) form = 1;
     const int tile = form == 2 ? kGemmWideTok : kGemmTile;
