@@ -334,6 +334,8 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="headline workload only")
     ap.add_argument("--gemm", metavar="NTOK,NROWS", help="only the prefill GEMM of this shape (k = 4096), "
                     "for profiling one kernel; prints its section alone")
+    ap.add_argument("--section", choices=["mxfp4", "moe", "ffn"], help="only this section of the default run, for "
+                    "profiling its kernels; prints the section alone")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this path runs on one GPU (no sharding, no collectives); use --gpus 1")
@@ -345,6 +347,11 @@ def main():
     if args.gemm:
         ntok, nrows = (int(v) for v in args.gemm.split(","))
         print(json.dumps({"prefill_gemm": gemm_section(dev, {nrows: (ntok,)})}), flush=True)
+        dev.close()
+        return
+    if args.section:
+        fn = {"mxfp4": mxfp4_section, "moe": moe_section, "ffn": ffn_section}[args.section]
+        print(json.dumps({args.section: fn(dev)}), flush=True)
         dev.close()
         return
     head = Workload(dev, quant.Q4_K, 4096, 4096, window=256)

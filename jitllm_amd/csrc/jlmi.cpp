@@ -668,7 +668,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     if (e != hipSuccess)
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
-    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_q4k_r64", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_moe_route", "jl_moe_group", "jl_moe_quant", "jl_moe_combine", "jl_mxfp4_gemm", "jl_mxfp4_matvec", "jl_sum_parts",
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_q4k_r64", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_moe_route", "jl_moe_group", "jl_moe_quant", "jl_moe_combine", "jl_mxfp4_prep", "jl_mxfp4_gemm", "jl_mxfp4_matvec", "jl_sum_parts",
                                       "jl_pack_weights", "jl_unpack_q4k"};
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int rw : {16, 32, 64})
@@ -1027,16 +1027,26 @@ int jl_matmul_mxfp4_bf16_dev(jl_ctx* c, float* out, const void* w, const uint16_
     MxGemmArgs a;
     a.out = out; a.w = (const uint8_t*)w; a.x = x;
     a.nrows = nrows; a.k = k; a.ntok = ntok; a.row_bytes = (k / 32) * 17;
-    a.nsplit = 1; a.part = nullptr;
+    a.nsplit = 1; a.part = nullptr; a.tok_pad = 0;
     void* params[] = {&a};
     hipStream_t st = pick_stream(c, stream);
     if (ntok <= 8)  // a handful of tokens: stream the rows once, no tile to fill
         return launch(c, "jl_mxfp4_matvec", (unsigned)((nrows + 3) / 4), 1, 256, 0, st, params);
-    const unsigned lds = 4u * 128u * 136u * 2u;
+    const unsigned lds = 2u * 128u * 264u * 2u;   // two weight stages [128][264] bf16
     if (lds > c->lds_limit) return JL_DECLINED;
+    // activations into matrix-fragment order (tokens padded to whole tiles, K to whole stages)
+    const int tok_pad = (ntok + 127) / 128 * 128, stages = (k + 255) / 256;
+    int rc = gemm_ws_ensure(c, (size_t)stages * (tok_pad / 32) * 16 * 1024);
+    if (rc != JL_OK) return rc;
+    MxPrepArgs pa;
+    pa.x = x; pa.xf = (uint16_t*)c->gemm_ws; pa.ntok = ntok; pa.tok_pad = tok_pad; pa.k = k;
+    void* pp[] = {&pa};
+    rc = launch(c, "jl_mxfp4_prep", (unsigned)stages, (unsigned)(tok_pad / 32), 256, 0, st, pp);
+    if (rc != JL_OK) return rc;
+    a.x = (const uint16_t*)c->gemm_ws; a.tok_pad = tok_pad;
     // A grid that leaves most CUs idle is widened along K: each split writes partial sums
     // to a workspace slab and a second kernel adds the slabs in order.
-    const int tiles = ((ntok + 127) / 128) * ((nrows + 127) / 128), stages = (k + 127) / 128;
+    const int tiles = (tok_pad / 128) * ((nrows + 127) / 128);
     int nsplit = c->tune.mx_split > 0 ? c->tune.mx_split : (tiles * 2 <= c->num_cu ? c->num_cu / tiles : 1);
     if (nsplit > 8) nsplit = 8;
     if (nsplit > stages) nsplit = stages;
@@ -1046,18 +1056,18 @@ int jl_matmul_mxfp4_bf16_dev(jl_ctx* c, float* out, const void* w, const uint16_
     }
     if (nsplit > 1) {
         const size_t n = (size_t)ntok * nrows;
-        int rc = ws_ensure(c, &c->mx_ws, &c->mx_ws_bytes, n * nsplit * 4);
+        rc = ws_ensure(c, &c->mx_ws, &c->mx_ws_bytes, n * nsplit * 4);
         if (rc != JL_OK) return rc;
         a.nsplit = nsplit; a.part = (float*)c->mx_ws;
-        HIP_TRY(c, H->ModuleLaunchKernel(c->fn["jl_mxfp4_gemm"], (unsigned)((ntok + 127) / 128),
-                                         (unsigned)((nrows + 127) / 128), (unsigned)nsplit, 256, 1, 1, lds, st,
+        HIP_TRY(c, H->ModuleLaunchKernel(c->fn["jl_mxfp4_gemm"], (unsigned)(tok_pad / 128),
+                                         (unsigned)((nrows + 127) / 128), (unsigned)nsplit, 512, 1, 1, lds, st,
                                          params, nullptr));
         SumPartsArgs sa;
         sa.out = out; sa.part = a.part; sa.n = n; sa.nsplit = nsplit;
         void* sp[] = {&sa};
         return launch(c, "jl_sum_parts", (unsigned)((n + 255) / 256), 1, 256, 0, st, sp);
     }
-    return launch(c, "jl_mxfp4_gemm", (unsigned)((ntok + 127) / 128), (unsigned)((nrows + 127) / 128), 256,
+    return launch(c, "jl_mxfp4_gemm", (unsigned)((ntok + 127) / 128), (unsigned)((nrows + 127) / 128), 512,
                   lds, st, params);
 }
 

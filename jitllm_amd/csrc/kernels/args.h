@@ -136,10 +136,20 @@ struct MoeCombineArgs {
 };
 
 // MXFP4 weights x bf16 activations: out [ntok][nrows] f32.
+// bf16 activations x [ntok][k] -> matrix fragments xf [ceil(k/256) stages][tok_pad/32][16]
+// [64 lanes][8 bf16]: fragment ks of a stage holds, for lane 32*kg + t%32, the eight values
+// x[t][256*stage + 16*ks + 8*kg ..]; tokens past ntok and K past k are zero.
+struct MxPrepArgs {
+    const uint16_t* x;
+    uint16_t* xf;
+    int ntok, tok_pad, k;
+};
+
 struct MxGemmArgs {
     float* out;
     const uint8_t* w;     // GGUF row-major MXFP4 blocks (17 bytes per 32)
-    const uint16_t* x;    // bf16 bits, [ntok][k]
+    const uint16_t* x;    // bf16 bits: [ntok][k] for the matvec, fragment order (MxPrepArgs) for the GEMM
+    int tok_pad;          // GEMM: tokens padded to whole tiles of 128
     int nrows, k, ntok;
     int row_bytes;
     int nsplit;           // workgroups along K (grid z); > 1: partial sums go to part

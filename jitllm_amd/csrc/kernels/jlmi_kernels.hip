@@ -123,7 +123,11 @@ extern "C" __global__ __launch_bounds__(256) void jl_moe_combine(MoeCombineArgs 
 
 // ------------------------------------------------------------------- MXFP4
 // grid = (ceil(ntok/128), ceil(nrows/128), K splits), block = 256, dynamic LDS = 4 stages of 128 x 272 B
-extern "C" __global__ __launch_bounds__(256) void jl_mxfp4_gemm(MxGemmArgs p) { mx_gemm_body(p, jl_smem); }
+extern "C" __global__ __launch_bounds__(256) void jl_mxfp4_prep(MxPrepArgs p) {
+    __shared__ u32x4 lds[32 * 33];
+    mx_prep_body(p, lds);
+}
+extern "C" __global__ __launch_bounds__(512) void jl_mxfp4_gemm(MxGemmArgs p) { mx_gemm_body(p, jl_smem); }
 extern "C" __global__ __launch_bounds__(256) void jl_sum_parts(SumPartsArgs p) { sum_parts_body(p); }
 // grid = ceil(nrows/4), block = 256: one wavefront per row, ntok <= 8
 extern "C" __global__ __launch_bounds__(256) void jl_mxfp4_matvec(MxGemmArgs p) { mx_matvec_body(p); }

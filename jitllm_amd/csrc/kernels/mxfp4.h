@@ -9,9 +9,10 @@
 // hardware's scaled fp4 -> bf16 conversion does the decode, two codes an
 // instruction; the block scale is its power-of-two scale operand.
 //
-// GEMM: 128 tokens x 128 rows per workgroup, K in stages of 128 (four blocks a
-// row), both operands staged through double-buffered LDS with a register
-// prefetch one stage ahead.  A short-row matvec serves a handful of tokens.
+// GEMM: 128 tokens x 128 rows per workgroup, K in stages of 256 (eight blocks a
+// row); weights are decoded through double-buffered LDS, activations are laid out
+// in matrix-fragment order by a prep kernel and go straight into registers.  A
+// short-row matvec serves a handful of tokens.
 #pragma once
 #include "args.h"
 #include "common.h"
@@ -21,10 +22,8 @@ typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
 
-#define JL_MX_TILE 128
-#define JL_MX_KSTAGE 128
-#define JL_MX_STRIDE 136  // bf16 per LDS row: 128 + 8 pad (272 B, an odd multiple of 16 B)
-#define JL_MX_STAGE_ELEMS (JL_MX_TILE * JL_MX_STRIDE)
+template <int V> struct MxIntC { static constexpr int value = V; };
+
 
 struct __attribute__((packed, aligned(1))) u32x4_a1 { u32x4 v; };
 __device__ __forceinline__ u32x4 ld16_a1(const uint8_t* p) { return ((const u32x4_a1*)p)->v; }
@@ -35,75 +34,22 @@ __device__ __forceinline__ float mx_scale(uint8_t e) {
     return e ? __uint_as_float((u32)e << 23) : __uint_as_float(0x00400000u);
 }
 
-// One block: 16 bytes of codes (byte j = element j in the low nibble, element j+16
-// in the high) -> 32 bf16 in element order, as four 16-byte groups.
-__device__ __forceinline__ void mx_dequant_block(u32x4 q, float scale, u32x4 out[4]) {
+// Half a block: words (2h, 2h+1) of the 16 code bytes (byte j = element j in the low
+// nibble, element j+16 in the high) -> elements 8h..8h+7 and 16+8h..16+8h+7 as bf16, two
+// 16-byte groups.
+__device__ __forceinline__ void mx_dequant_half(u32 q0, u32 q1, float scale, u32x4& lo, u32x4& hi) {
+    const u32 q[2] = {q0, q1};
 #pragma unroll
-    for (int w = 0; w < 4; w++) {
-        // bytes 4w..4w+3: pair i = (element 4w+i, element 4w+i+16)
+    for (int w = 0; w < 2; w++) {
+        // bytes 4w..4w+3 of the half: pair i = (element 4w+i, element 4w+i+16)
         u32 p0 = __builtin_bit_cast(u32, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(q[w], scale, 0));
         u32 p1 = __builtin_bit_cast(u32, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(q[w], scale, 1));
         u32 p2 = __builtin_bit_cast(u32, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(q[w], scale, 2));
         u32 p3 = __builtin_bit_cast(u32, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(q[w], scale, 3));
-        // low halves = elements 4w..4w+3, high halves = elements 4w+16..4w+19
-        u32 lo01 = __builtin_amdgcn_perm(p1, p0, 0x05040100u), lo23 = __builtin_amdgcn_perm(p3, p2, 0x05040100u);
-        u32 hi01 = __builtin_amdgcn_perm(p1, p0, 0x07060302u), hi23 = __builtin_amdgcn_perm(p3, p2, 0x07060302u);
-        // group g holds elements 8g..8g+7: w = 0,1 fill groups 0 (low) and 2 (high); w = 2,3 groups 1 and 3
-        const int g = w >> 1, h = (w & 1) * 2;
-        out[g][h] = lo01; out[g][h + 1] = lo23;
-        out[g + 2][h] = hi01; out[g + 2][h + 1] = hi23;
-    }
-}
-
-struct MxWRegs {
-    u32x4 q[2];
-    uint8_t e[2];
-};
-
-__device__ __forceinline__ void mx_load_w(const MxGemmArgs& p, int row, int stage, int pr, MxWRegs& r) {
-    const int nblk = p.k / 32;
-#pragma unroll
-    for (int i = 0; i < 2; i++) {
-        const int b = stage * 4 + 2 * pr + i;
-        const uint8_t* blk = p.w + (size_t)row * p.row_bytes + (size_t)min(b, nblk - 1) * 17;
-        r.e[i] = blk[0];
-        r.q[i] = ld16_a1(blk + 1);
-        if (b >= nblk) r.q[i] = u32x4{0, 0, 0, 0};  // past the end of K: zero codes
-    }
-}
-
-__device__ __forceinline__ void mx_store_w(const MxWRegs& r, int row, int pr, __bf16* sw) {
-#pragma unroll
-    for (int i = 0; i < 2; i++) {
-        u32x4 o[4];
-        mx_dequant_block(r.q[i], mx_scale(r.e[i]), o);
-        __bf16* dst = sw + row * JL_MX_STRIDE + (2 * pr + i) * 32;
-#pragma unroll
-        for (int g = 0; g < 4; g++) *(u32x4*)(dst + 8 * g) = o[g];
-    }
-}
-
-struct MxARegs {
-    u32x4 c[8];
-};
-
-__device__ __forceinline__ void mx_load_a(const MxGemmArgs& p, int t0, int stage, int tid, MxARegs& r) {
-#pragma unroll
-    for (int i = 0; i < 8; i++) {
-        const int c = tid + 256 * i, tok = c >> 4, ch = c & 15;
-        const int kk = stage * JL_MX_KSTAGE + ch * 8;
-        const bool ok = t0 + tok < p.ntok && kk < p.k;
-        const uint16_t* src = p.x + (size_t)min(t0 + tok, p.ntok - 1) * p.k + min(kk, p.k - 8);
-        u32x4 v = *(const u32x4*)src;
-        r.c[i] = ok ? v : u32x4{0, 0, 0, 0};
-    }
-}
-
-__device__ __forceinline__ void mx_store_a(const MxARegs& r, int tid, __bf16* sa) {
-#pragma unroll
-    for (int i = 0; i < 8; i++) {
-        const int c = tid + 256 * i, tok = c >> 4, ch = c & 15;
-        *(u32x4*)(sa + tok * JL_MX_STRIDE + ch * 8) = r.c[i];
+        lo[2 * w] = __builtin_amdgcn_perm(p1, p0, 0x05040100u);
+        lo[2 * w + 1] = __builtin_amdgcn_perm(p3, p2, 0x05040100u);
+        hi[2 * w] = __builtin_amdgcn_perm(p1, p0, 0x07060302u);
+        hi[2 * w + 1] = __builtin_amdgcn_perm(p3, p2, 0x07060302u);
     }
 }
 
@@ -113,83 +59,180 @@ __device__ __forceinline__ void mx_lds_barrier() {
     asm volatile("" ::: "memory");
 }
 
+#define JL_MX_TILE 128
+#define JL_MX_KSTAGE 256   // eight blocks a row
+#define JL_MX_STRIDE 264   // bf16 per LDS row: 256 + 8 pad (528 B: rows advance four banks)
+#define JL_MX_STAGE_ELEMS (JL_MX_TILE * JL_MX_STRIDE)
+
+// ---------------------------------------------------------------- activation prep
+// grid = (ceil(k/256), tok_pad/32), block = 256: 32 tokens of one K stage.  Rows are read
+// coalesced (32 lanes cover a token's 512 bytes), turned through LDS, and written as whole
+// fragments, 1 KiB contiguous a wavefront.
+__device__ __forceinline__ void mx_prep_body(const MxPrepArgs& p, u32x4* lds) {
+    const int tid = threadIdx.x, st = blockIdx.x, grp = blockIdx.y;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int c = tid + 256 * i, tl = c >> 5, ch = c & 31;   // token, 16-byte chunk of its 512 bytes
+        const int t = grp * 32 + tl, kk = st * JL_MX_KSTAGE + 8 * ch;
+        u32x4 v = {0, 0, 0, 0};
+        if (t < p.ntok && kk < p.k) v = *(const u32x4*)(p.x + (size_t)t * p.k + kk);
+        lds[tl * 33 + ch] = v;   // 33-vector rows: the turned reads below spread over the banks
+    }
+    __syncthreads();
+    u32x4* dst = (u32x4*)p.xf + ((size_t)st * (p.tok_pad >> 5) + grp) * (16 * 64);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int f = (tid >> 6) * 4 + i, lane = tid & 63;       // fragment ks = f, lane = 32*kg + token
+        dst[f * 64 + lane] = lds[(lane & 31) * 33 + 2 * f + (lane >> 5)];
+    }
+}
+
+// ---------------------------------------------------------------- GEMM
+// One stage of weights for a thread: two blocks (rows 8*i + lane/8 of its wavefront's 16,
+// block lane%8 of the row's eight): a wavefront's load covers eight rows x 136 contiguous
+// bytes, sixteen cache lines instead of one per lane.
+struct MxWRegs {
+    u32x4 q[2];
+    uint8_t e[2];
+};
+
+__device__ __forceinline__ void mx_load_w(const MxGemmArgs& p, int r0, int wave, int lane, int stage, MxWRegs& r) {
+    const int nblk = p.k / 32;
+    const int b = stage * 8 + (lane & 7);
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const int row = min(r0 + wave * 16 + 8 * i + (lane >> 3), p.nrows - 1);
+        const uint8_t* blk = p.w + (size_t)row * p.row_bytes + (size_t)min(b, nblk - 1) * 17;
+        r.e[i] = blk[0];
+        r.q[i] = ld16_a1(blk + 1);
+        if (b >= nblk) r.q[i] = u32x4{0, 0, 0, 0};  // past the end of K: zero codes
+    }
+}
+
+// grid = (tok_pad/128, ceil(nrows/128), nsplit), block = 512, dynamic LDS = two weight
+// stages [128][264] bf16.  The shape this serves (a few thousand rows, a thousand tokens)
+// gives fewer 128 x 128 tiles than the chip has CUs, so a tile gets EIGHT wavefronts, two
+// per SIMD to cover each other's waits: wavefront (tg, kh) owns 32 tokens x all 128 rows
+// (four 32 x 32 accumulators) over the K-steps of parity kh, and the two parities are
+// added through LDS at the end, kh = 0 first.  Activation fragments come from the prepared
+// workspace into a register ring a stage ahead (1 KiB coalesced loads), each feeding four
+// matrix instructions; all eight wavefronts share one decode of the weights through LDS.
+// A stage (256 K) is 16 slots of two matrix instructions per wavefront with the weight
+// fragments fetched three slots ahead and the next stage's weights decoded half a block
+// at a time in between, their registers loaded two stages ahead.
 __device__ __forceinline__ void mx_gemm_body(const MxGemmArgs& p, uint8_t* smem) {
-    __bf16* sA = (__bf16*)smem;
-    __bf16* sW = sA + 2 * JL_MX_STAGE_ELEMS;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    __bf16* sW = (__bf16*)smem;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int tg = wave & 3, kh = wave >> 2;
     const int t0 = blockIdx.x * JL_MX_TILE, r0 = blockIdx.y * JL_MX_TILE;
     // a small grid is widened along K: workgroup z takes a contiguous run of the K
     // stages and writes its partial sums to its own slab, summed afterwards in order
     const int all_stages = (p.k + JL_MX_KSTAGE - 1) / JL_MX_KSTAGE;
     const int per_split = (all_stages + p.nsplit - 1) / p.nsplit;
     const int s_lo = min((int)blockIdx.z * per_split, all_stages), s_hi = min(s_lo + per_split, all_stages);
-    const int nstages = s_hi - s_lo;
     float* outp = p.nsplit > 1 ? p.part + (size_t)blockIdx.z * p.ntok * p.nrows : p.out;
-    const int wrow = min(r0 + (tid >> 1), p.nrows - 1), pr = tid & 1;
-    const int wt = (wave >> 1) * 64, wr = (wave & 1) * 64;
     const int arow = lane & 31, kg = lane >> 5;
+    // activation fragment (stage, K-step 2*ks2 + kh) of this wavefront's 32 tokens: uniform base + lane
+    const size_t astride = (size_t)(p.tok_pad >> 5) * (16 * 1024);
+    const char* abase = (const char*)p.x + ((size_t)(t0 >> 5) + tg) * (16 * 1024) + kh * 1024;
+    const unsigned aoff = lane * 16;
+    auto a_frag = [&](int stage, int ks2) {
+        return *(const bf16x8*)(abase + (size_t)stage * astride + ks2 * 2048 + aoff);
+    };
+    // where this thread's decoded blocks go in a stage buffer
+    const int wdst = (wave * 16 + (lane >> 3)) * JL_MX_STRIDE + (lane & 7) * 32;
 
-    f32x16_t acc[2][2];
+    f32x16_t acc[4];
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int j = 0; j < 4; j++)
 #pragma unroll
-        for (int j = 0; j < 2; j++)
-#pragma unroll
-            for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
+        for (int e = 0; e < 16; e++) acc[j][e] = 0.f;
 
-    MxWRegs wreg;
-    MxARegs areg;
-    if (nstages > 0) {
-        mx_load_w(p, wrow, s_lo, pr, wreg);
-        mx_load_a(p, t0, s_lo, tid, areg);
-        mx_store_w(wreg, tid >> 1, pr, sW);
-        mx_store_a(areg, tid, sA);
+    auto decode_half = [&](const MxWRegs& r, int i, int h, __bf16* buf) {
+        // block i of the thread's two, words (2h, 2h+1): elements 8h.. and 16+8h..
+        u32x4 lo, hi;
+        mx_dequant_half(r.q[i][2 * h], r.q[i][2 * h + 1], mx_scale(r.e[i]), lo, hi);
+        __bf16* dst = buf + wdst + 8 * i * JL_MX_STRIDE + 8 * h;
+        *(u32x4*)dst = lo;
+        *(u32x4*)(dst + 16) = hi;
+    };
+
+    MxWRegs wa, wb;
+    bf16x8 aring[8];
+    const int last = max(s_hi - 1, s_lo);
+    mx_load_w(p, r0, wave, lane, s_lo, wa);
+#pragma unroll
+    for (int ks2 = 0; ks2 < 8; ks2++) aring[ks2] = a_frag(s_lo, ks2);
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        decode_half(wa, i, 0, sW);
+        decode_half(wa, i, 1, sW);
     }
-    if (nstages > 1) {
-        mx_load_w(p, wrow, s_lo + 1, pr, wreg);
-        mx_load_a(p, t0, s_lo + 1, tid, areg);
-    }
+    mx_load_w(p, r0, wave, lane, min(s_lo + 1, last), wa);
     mx_lds_barrier();
 
-    for (int st = 0; st < nstages; st++) {
-        const int buf = st & 1;
-        const __bf16* a = sA + buf * JL_MX_STAGE_ELEMS;
+    auto stage = [&](auto BUF, int st, MxWRegs& wcur, MxWRegs& wnxt) {
+        constexpr int buf = decltype(BUF)::value;
         const __bf16* w = sW + buf * JL_MX_STAGE_ELEMS;
-        if (st + 1 < nstages) {
-            mx_store_w(wreg, tid >> 1, pr, sW + (buf ^ 1) * JL_MX_STAGE_ELEMS);
-            mx_store_a(areg, tid, sA + (buf ^ 1) * JL_MX_STAGE_ELEMS);
-            if (st + 2 < nstages) {
-                mx_load_w(p, wrow, s_lo + st + 2, pr, wreg);
-                mx_load_a(p, t0, s_lo + st + 2, tid, areg);
+        __bf16* wnext = sW + (buf ^ 1) * JL_MX_STAGE_ELEMS;
+        const int nst = min(st + 1, last);
+        mx_load_w(p, r0, wave, lane, min(st + 2, last), wnxt);
+        const __bf16* wp0 = w + arow * JL_MX_STRIDE + 8 * kg + 16 * kh;
+        auto w_frag = [&](int slot, int j) {
+            return *(const bf16x8*)(wp0 + 32 * (2 * (slot & 1) + j) * JL_MX_STRIDE + 32 * (slot >> 1));
+        };
+        bf16x8 wf[4][2];
+#pragma unroll
+        for (int s3 = 0; s3 < 3; s3++)
+#pragma unroll
+            for (int j = 0; j < 2; j++) wf[s3][j] = w_frag(s3, j);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int slot = 0; slot < 16; slot++) {
+            const int ks2 = slot >> 1, jh = slot & 1;
+            if (slot + 3 < 16) {
+#pragma unroll
+                for (int j = 0; j < 2; j++) wf[(slot + 3) & 3][j] = w_frag(slot + 3, j);
             }
-        }
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int ks = 0; ks < JL_MX_KSTAGE / 16; ks++) {
-            bf16x8 af[2], wf[2];
-#pragma unroll
-            for (int i = 0; i < 2; i++) {
-                af[i] = *(const bf16x8*)(a + (wt + 32 * i + arow) * JL_MX_STRIDE + 16 * ks + 8 * kg);
-                wf[i] = *(const bf16x8*)(w + (wr + 32 * i + arow) * JL_MX_STRIDE + 16 * ks + 8 * kg);
+            for (int j = 0; j < 2; j++)
+                acc[2 * jh + j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aring[ks2], wf[slot & 3][j],
+                                                                         acc[2 * jh + j], 0, 0, 0);
+            if (jh == 1) {
+                aring[ks2] = a_frag(nst, ks2);
+                // half a block of the next stage's weights in every second K-step
+                if (ks2 & 1) decode_half(wcur, ks2 >> 2, (ks2 >> 1) & 1, wnext);
             }
-#pragma unroll
-            for (int i = 0; i < 2; i++)
-#pragma unroll
-                for (int j = 0; j < 2; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], wf[j], acc[i][j], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
         }
         mx_lds_barrier();
+    };
+    for (int st = s_lo; st < s_hi; st += 2) {
+        stage(MxIntC<0>{}, st, wa, wb);
+        if (st + 1 < s_hi) stage(MxIntC<1>{}, st + 1, wb, wa);
     }
+
+    // the two K parities meet in LDS (the weight stages are done with): [tg][tile][16][64] f32
+    float* sAcc = (float*)smem + (size_t)tg * (4 * 16 * 64) + lane;
+    if (kh == 1) {
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
-        const int r = r0 + wr + 32 * j + arow;
-        if (r >= p.nrows) continue;
+        for (int j = 0; j < 4; j++)
 #pragma unroll
-        for (int i = 0; i < 2; i++)
+            for (int e = 0; e < 16; e++) sAcc[(j * 16 + e) * 64] = acc[j][e];
+    }
+    __syncthreads();
+    if (kh == 1) return;
 #pragma unroll
-            for (int e = 0; e < 16; e++) {
-                const int t = t0 + wt + 32 * i + 8 * (e >> 2) + 4 * kg + (e & 3);
-                if (t < p.ntok) outp[(size_t)t * p.nrows + r] = acc[i][j][e];
-            }
+    for (int j = 0; j < 4; j++) {
+        const int r = r0 + 32 * j + arow;
+#pragma unroll
+        for (int e = 0; e < 16; e++) {
+            const float v = acc[j][e] + sAcc[(j * 16 + e) * 64];
+            const int t = t0 + 32 * tg + 8 * (e >> 2) + 4 * kg + (e & 3);
+            if (r < p.nrows && t < p.ntok) outp[(size_t)t * p.nrows + r] = v;
+        }
     }
 }
 
