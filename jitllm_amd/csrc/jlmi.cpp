@@ -33,6 +33,7 @@ struct Tuning {
     int gemm_rows = 0;
     int gemm_form = 0;
     int gemm_split = 0;
+    int moe_form = 0;
     int mx_split = 0;
 };
 
@@ -566,7 +567,7 @@ int packed_matmul_launch(jl_ctx* c, float* out, int type, const PlaneRef& pl, co
 
 int moe_matvec_launch(jl_ctx* c, float* out0, float* out1, int type, const void* bank0, const void* bank1,
                       const float* x, const float* x2, const uint32_t* src, const uint32_t* start,
-                      int n_expert, int ncols, int nrows, int k, hipStream_t st) {
+                      int n_expert, int ncols, int max_cols, int nrows, int k, hipStream_t st) {
     const TypeInfo* ti = nullptr;
     int rc = matvec_check(c, type, nrows, k, &ti);
     if (rc != JL_OK) return rc;
@@ -578,6 +579,39 @@ int moe_matvec_launch(jl_ctx* c, float* out0, float* out1, int type, const void*
     const int row_bytes = (k / ti->block_elems) * ti->block_bytes;
     const size_t sheet = (size_t)nrows * row_bytes;
     if (type == JL_TYPE_Q4_K ? sheet % 16 != 0 : sheet % 2 != 0) return JL_DECLINED;
+    // Q4_K with the k-quant activation window can also run as groups of 32 columns on the
+    // matrix cores (tuning "moe.form" = 2).  Its vector work does not grow with the number of
+    // columns, but with a handful of columns per expert it is bound by the latency of the
+    // load -> dequantize -> LDS -> matrix chain at two wavefronts per SIMD and is the slower
+    // form (gate+up 145 us against 107 us at the 128-expert, 64-row shape), so it is not the
+    // default.
+    if (type == JL_TYPE_Q4_K && c->act_window == 256 && c->tune.moe_form == 2 &&
+        4u * 19968u <= c->lds_limit) {   // JL_MOEG_WAVE_LDS
+        if (max_cols <= 0 || max_cols > ncols) max_cols = ncols;
+        const int gmax = (max_cols + 31) / 32, nslots = ncols / 32 + n_expert + 1, nsb = k / 256;
+        if ((long)n_expert * gmax > 65535) return JL_DECLINED;
+        const size_t bq_bytes = (size_t)2 * nsb * nslots * kGemmAStageBytes;
+        rc = ws_ensure(c, &c->moe_q_ws, &c->moe_q_ws_bytes, bq_bytes + (size_t)nsb * nslots * 32 * 4);
+        if (rc != JL_OK) return rc;
+        MoeGemmPrepArgs pa;
+        pa.x = x; pa.x2 = x2; pa.src = src; pa.start = start;
+        pa.bq = (uint16_t*)c->moe_q_ws; pa.da = (float*)((char*)c->moe_q_ws + bq_bytes);
+        pa.k = k; pa.gmax = gmax; pa.nslots = nslots;
+        void* pp[] = {&pa};
+        rc = launch(c, "jl_moe_gemm_prep", (unsigned)nsb, (unsigned)(n_expert * gmax), 256, 0, st, pp);
+        if (rc != JL_OK) return rc;
+        MoeGemmArgs ga;
+        ga.out[0] = out0; ga.out[1] = out1;
+        ga.bank[0] = (const uint8_t*)bank0; ga.bank[1] = (const uint8_t*)bank1;
+        ga.bq = pa.bq; ga.da = pa.da; ga.start = start;
+        ga.sheet_bytes = sheet; ga.nrows = nrows; ga.k = k; ga.row_bytes = row_bytes;
+        ga.gmax = gmax; ga.nslots = nslots;
+        void* gp[] = {&ga};
+        HIP_TRY(c, H->ModuleLaunchKernel(c->fn["jl_moe_gemm_q4k"], (unsigned)((nrows + 255) / 256),
+                                         (unsigned)(n_expert * gmax), bank1 ? 2u : 1u, 256, 1, 1, 4u * 19968u, st,
+                                         gp, nullptr));
+        return JL_OK;
+    }
     const int nslots = k / ti->slot_elems;
     int lpr = 16;
     while (lpr < 64 && lpr < nslots) lpr <<= 1;
@@ -668,7 +702,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     if (e != hipSuccess)
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
-    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_q4k_r64", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_moe_route", "jl_moe_group", "jl_moe_quant", "jl_moe_combine", "jl_mxfp4_prep", "jl_mxfp4_gemm", "jl_mxfp4_matvec", "jl_sum_parts",
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_q4k_r64", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_moe_route", "jl_moe_group", "jl_moe_quant", "jl_moe_combine", "jl_moe_gemm_prep", "jl_moe_gemm_q4k", "jl_mxfp4_prep", "jl_mxfp4_gemm", "jl_mxfp4_matvec", "jl_sum_parts",
                                       "jl_pack_weights", "jl_unpack_q4k"};
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int rw : {16, 32, 64})
@@ -746,6 +780,7 @@ int jl_set_tuning(jl_ctx* c, const char* key, int value) {
     else if (!strcmp(key, "packed.rw")) c->tune.packed_rw = value;
     else if (!strcmp(key, "packed.block")) c->tune.packed_block = value;
     else if (!strcmp(key, "moe.shares")) c->tune.moe_shares = value;
+    else if (!strcmp(key, "moe.form")) c->tune.moe_form = value;
     else if (!strcmp(key, "gemm.rows")) c->tune.gemm_rows = value;
     else if (!strcmp(key, "mxfp4.split")) c->tune.mx_split = value;
     else if (!strcmp(key, "gemm.form")) c->tune.gemm_form = value;
@@ -965,7 +1000,7 @@ int jl_moe_matvec_dev(jl_ctx* c, float* out0, float* out1, int type, const void*
                       int n_expert, int ncols, int nrows, int k, void* stream) {
     if (!c) return JL_ERR_ARG;
     HIP_TRY(c, H->SetDevice(c->device));
-    return moe_matvec_launch(c, out0, out1, type, bank0, bank1, x, x2, src, start, n_expert, ncols, nrows, k,
+    return moe_matvec_launch(c, out0, out1, type, bank0, bank1, x, x2, src, start, n_expert, ncols, 0, nrows, k,
                              pick_stream(c, stream));
 }
 
@@ -1008,10 +1043,10 @@ int jl_moe_ffn_dev(jl_ctx* c, float* resid, int type, const void* gate_bank, con
     rc = jl_moe_group_dev(c, sel, sel_stride, rows, k_used, n_expert, start, perm, pos, st);
     if (rc != JL_OK) return rc;
     // gate and up: columns read the routed rows of x
-    rc = moe_matvec_launch(c, g, u, type, gate_bank, up_bank, x, nullptr, perm, start, n_expert, (int)ncols, n_ffn, n_embd, st);
+    rc = moe_matvec_launch(c, g, u, type, gate_bank, up_bank, x, nullptr, perm, start, n_expert, (int)ncols, rows, n_ffn, n_embd, st);
     if (rc != JL_OK) return rc;
     // down: the activation of column c is silu(g[c]) * u[c]
-    rc = moe_matvec_launch(c, y, nullptr, type, down_bank, nullptr, g, u, nullptr, start, n_expert, (int)ncols, n_embd, n_ffn, st);
+    rc = moe_matvec_launch(c, y, nullptr, type, down_bank, nullptr, g, u, nullptr, start, n_expert, (int)ncols, rows, n_embd, n_ffn, st);
     if (rc != JL_OK) return rc;
     return jl_moe_combine_dev(c, resid, y, wt, sel, sel_stride, pos, rows, k_used, n_embd, st);
 }

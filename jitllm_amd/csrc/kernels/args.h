@@ -55,6 +55,32 @@ struct GemmArgs {
     int sb_per;          // K split: super-blocks per blockIdx.z (0 = whole K), out = slab z of [gridDim.z][ntok][out_stride]
 };
 
+// Mixture block on the matrix cores (Q4_K, activation window 256).  An expert's columns are
+// cut into groups of 32; group g of expert e has the workspace slot start[e]/32 + e + g
+// (distinct for distinct groups, below ncols/32 + n_expert + 1 = nslots).  The prep kernel
+// gathers, quantizes and lays out the groups' activations as the prefill GEMM's fragments,
+// bq [k/128 stages][nslots][9][64 lanes][8] f16 and da [k/256][32*nslots]; the matrix kernel
+// meets them with the expert's sheet, out[mat][column][nrows].
+struct MoeGemmPrepArgs {
+    const float* x;       // [.][k]
+    const float* x2;      // optional: activation is silu(x) * x2
+    const uint32_t* src;  // optional: column -> row of x (identity when null)
+    const uint32_t* start;
+    uint16_t* bq;
+    float* da;
+    int k, gmax, nslots;
+};
+
+struct MoeGemmArgs {
+    float* out[2];
+    const uint8_t* bank[2];
+    const uint16_t* bq;
+    const float* da;
+    const uint32_t* start;
+    size_t sheet_bytes;
+    int nrows, k, row_bytes, gmax, nslots;
+};
+
 // Two-pass form of the Q4_K prefill GEMM.  Pass one expands the weights once per call into
 // f16 matrix fragments, w16 [ceil(nrows/64)][k/128 stages][18 fragments][64 lanes] 16-byte
 // vectors (fragment 2*ks+g: K-step ks of the tile's row group g; 16+g: the minimum columns,

@@ -72,18 +72,18 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 // quantizes eight tokens (lane l owns elements 4l..4l+3) into LDS; then every wavefront
 // assembles whole fragments, 16 bytes a lane and 1 KiB contiguous a store.
 #define JL_GEMM_PREP_LDS_WORDS (32 * 65 + 32 * 8)
-__device__ __forceinline__ void gemm_prep_q4k_body(const GemmPrepArgs& p, u32* lds) {
+// One group of 32 tokens, one super-block: load(tl) returns this lane's four elements
+// (4*lane .. 4*lane+3 of the super-block) of token tl of the group, zeros for a token that
+// does not exist.  grp of ngrp groups; da is laid [nsb][32*ngrp].
+template <class Load>
+__device__ __forceinline__ void gemm_prep_group(u32* lds, int sb, int grp, int ngrp, uint16_t* bqp, float* dap,
+                                                Load load) {
     u32* sq = lds;                       // [32 tokens][65]: 64 words of int8 + 1 pad (bank spread)
     i32* sA = (i32*)(lds + 32 * 65);     // [32 tokens][8 sub-block sums]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int sb = blockIdx.x, grp = blockIdx.y;
     f32x4 v[8];
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-        const int t = grp * 32 + wave * 8 + i;
-        v[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-        if (t < p.ntok) v[i] = ((const f32x4*)(p.x + (size_t)t * p.k + (size_t)sb * 256))[lane];
-    }
+    for (int i = 0; i < 8; i++) v[i] = load(wave * 8 + i);
 #pragma unroll
     for (int i = 0; i < 8; i++) {
         const int tl = wave * 8 + i;
@@ -96,12 +96,11 @@ __device__ __forceinline__ void gemm_prep_q4k_body(const GemmPrepArgs& p, u32* l
         const i32 a32 = sum16 + dpp_i32<JL_DPP_ROW_HALF_MIRROR, 0xf>(0, sum16);
         sq[tl * 65 + lane] = q;
         if ((lane & 7) == 0) sA[tl * 8 + (lane >> 3)] = a32;
-        if (lane == 0) p.da[(size_t)sb * p.tok_pad + grp * 32 + tl] = d;
+        if (lane == 0) dap[(size_t)sb * (32 * ngrp) + grp * 32 + tl] = d;
     }
     __syncthreads();
     const int tl = lane & 31, kg = lane >> 5;
-    u32x4* dst = (u32x4*)p.bq;
-    const size_t ngrp = (size_t)(p.tok_pad >> 5);
+    u32x4* dst = (u32x4*)bqp;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
         const int pi = wave * 4 + i, h = pi >> 3, ks = pi & 7;
@@ -126,6 +125,17 @@ __device__ __forceinline__ void gemm_prep_q4k_body(const GemmPrepArgs& p, u32* l
         dst[(((size_t)(2 * sb + 1) * ngrp + grp) * JL_GEMM_ASTAGE_FRAGS + 8) * 64 + lane] =
             __builtin_bit_cast(u32x4, o);
     }
+}
+
+__device__ __forceinline__ void gemm_prep_q4k_body(const GemmPrepArgs& p, u32* lds) {
+    const int lane = threadIdx.x & 63;
+    const int sb = blockIdx.x, grp = blockIdx.y;
+    gemm_prep_group(lds, sb, grp, p.tok_pad >> 5, p.bq, p.da, [&](int tl) {
+        const int t = grp * 32 + tl;
+        f32x4 v = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (t < p.ntok) v = ((const f32x4*)(p.x + (size_t)t * p.k + (size_t)sb * 256))[lane];
+        return v;
+    });
 }
 
 // -------------------------------------------------------------------- main

@@ -127,6 +127,11 @@ extern "C" __global__ __launch_bounds__(256) void jl_mxfp4_prep(MxPrepArgs p) {
     __shared__ u32x4 lds[32 * 33];
     mx_prep_body(p, lds);
 }
+extern "C" __global__ __launch_bounds__(256) void jl_moe_gemm_prep(MoeGemmPrepArgs p) {
+    __shared__ u32 lds[JL_GEMM_PREP_LDS_WORDS];
+    moe_gemm_prep_body(p, lds);
+}
+extern "C" __global__ __launch_bounds__(256, 2) void jl_moe_gemm_q4k(MoeGemmArgs p) { moe_gemm_q4k_body(p, jl_smem); }
 extern "C" __global__ __launch_bounds__(512) void jl_mxfp4_gemm(MxGemmArgs p) { mx_gemm_body(p, jl_smem); }
 extern "C" __global__ __launch_bounds__(256) void jl_sum_parts(SumPartsArgs p) { sum_parts_body(p); }
 // grid = ceil(nrows/4), block = 256: one wavefront per row, ntok <= 8

@@ -28,6 +28,7 @@
 #include "args.h"
 #include "common.h"
 #include "matvec.h"
+#include "gemm_q4k.h"
 
 // Phase marker for profiling builds; expands to nothing in the product.
 #ifndef JL_MOE_TRACE
@@ -341,6 +342,209 @@ __device__ __forceinline__ void moe_matvec_body(const MoeMatVecArgs& p, uint8_t*
         __syncthreads();
     }
     JL_MOE_TRACE(4);
+}
+
+// ------------------------------------------------- grouped matmul on the matrix cores
+// The dot-product kernel above pays for every (weight, column) pair in vector instructions.
+// With Q4_K weights and the k-quant activation window the prefill GEMM's exact f16
+// arithmetic applies (gemm_q4k.h): a group of up to 32 of an expert's columns is one
+// matrix operand, and the vector work is the dequantization alone, whatever the group holds.
+//
+// Activation prep: grid = (k/256, n_expert * gmax), block = 256: group g of expert e, one
+// super-block; tokens past the expert's last column are zeros.
+__device__ __forceinline__ void moe_gemm_prep_body(const MoeGemmPrepArgs& p, u32* lds) {
+    const int lane = threadIdx.x & 63;
+    const int sb = blockIdx.x, e = blockIdx.y / p.gmax, g = blockIdx.y - e * p.gmax;
+    const u32 c_lo = p.start[e], c_hi = p.start[e + 1];
+    const u32 c0 = c_lo + 32 * g;
+    if (c0 >= c_hi) return;   // uniform across the workgroup
+    const int slot = (int)(c_lo >> 5) + e + g;
+    gemm_prep_group(lds, sb, slot, p.nslots, p.bq, p.da, [&](int tl) {
+        f32x4 v = f32x4{0.f, 0.f, 0.f, 0.f};
+        const u32 c = c0 + tl;
+        if (c < c_hi) {
+            const size_t row = p.src ? p.src[c] : c;
+            v = ((const f32x4*)(p.x + row * (size_t)p.k + (size_t)sb * 256))[lane];
+            if (p.x2) {
+                const f32x4 u = ((const f32x4*)(p.x2 + row * (size_t)p.k + (size_t)sb * 256))[lane];
+                v = f32x4{silu_f32(v.x) * u.x, silu_f32(v.y) * u.y, silu_f32(v.z) * u.z, silu_f32(v.w) * u.w};
+            }
+        }
+        return v;
+    });
+}
+
+// Matrix kernel: grid = (ceil(nrows/256), n_expert * gmax, matrices), block = 256, dynamic
+// LDS = 4 * JL_MOEG_WAVE_LDS.  A wavefront owns 32 columns x 64 rows and shares nothing
+// with its neighbours -- the columns are the same for the whole workgroup, the rows are its
+// own -- so it keeps a private LDS buffer to turn its dequantized weights into matrix
+// fragments and no workgroup barrier is needed: LDS operations of one wavefront execute in
+// order.  Per stage (half a super-block) it dequantizes 64 rows x 128 weights (lane =
+// (row%16, 16-byte chunk), four rows a lane), then runs 16 matrix instructions against the
+// group's activation fragments, which come from the workspace into a register ring a stage
+// ahead; the weights of the next stage are in flight in registers meanwhile.  Two
+// workgroups share a CU and cover each other's vector phases.
+#define JL_MOEG_WROW 136   // f16 per weight row: 128 + 8 (272 B: rows advance four banks)
+#define JL_MOEG_MROW 16    // f16 per row of minimum columns
+#define JL_MOEG_WAVE_LDS (64 * JL_MOEG_WROW * 2 + 64 * JL_MOEG_MROW * 2 + 64 * 2 * 4)
+
+__device__ __forceinline__ void moe_gemm_q4k_body(const MoeGemmArgs& p, uint8_t* smem) {
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int e = blockIdx.y / p.gmax, g = blockIdx.y - e * p.gmax, mat = blockIdx.z;
+    const u32 c_lo = p.start[e], c_hi = p.start[e + 1];
+    const u32 c0 = c_lo + 32 * g;
+    if (c0 >= c_hi) return;
+    const int ncol = min(32, (int)(c_hi - c0));
+    const int slot = (int)(c_lo >> 5) + e + g;
+    const int r0 = blockIdx.x * 256 + wave * 64;
+    if (r0 >= p.nrows) return;   // (no workgroup barrier below)
+    _Float16* sW = (_Float16*)(smem + (size_t)wave * JL_MOEG_WAVE_LDS);
+    _Float16* sMin = sW + 64 * JL_MOEG_WROW;
+    float* sSc = (float*)(sMin + 64 * JL_MOEG_MROW);
+
+    const int nsb = p.k / 256, nsteps = 2 * nsb;
+    const int arow = lane & 31, kg = lane >> 5;
+    const int drow = lane >> 2, chunk = lane & 3, hh = chunk >> 1, wq_ = chunk & 1;
+    // weights: uniform base + 32-bit lane offsets, rows clamped to the sheet
+    const uint8_t* sheet = p.bank[mat] + (size_t)e * p.sheet_bytes;
+    unsigned woff[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) woff[i] = (unsigned)min(r0 + 16 * i + drow, p.nrows - 1) * (unsigned)p.row_bytes;
+    // activation fragment (step, ks) of the group: uniform base + lane
+    const size_t astride = (size_t)p.nslots * (JL_GEMM_ASTAGE_FRAGS * 1024);
+    const char* abase = (const char*)p.bq + (size_t)slot * (JL_GEMM_ASTAGE_FRAGS * 1024);
+    const unsigned aoff = lane * 16;
+    auto a_frag = [&](int step, int ks) {
+        return *(const f16x8*)(abase + (size_t)step * astride + ks * 1024 + aoff);
+    };
+    const float* dabase = p.da + (size_t)slot * 32 + 4 * kg;
+    u32 mask_lo = 0x000F000Fu, mask_hi = 0x00F000F0u, magic = 0x64006400u;
+    asm volatile("" : "+v"(mask_lo), "+v"(mask_hi), "+v"(magic));
+
+    f32x16 out[2], accP[2];
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+        for (int el = 0; el < 16; el++) out[j][el] = 0.f;
+
+    // Weights are streamed once from HBM and a stage is short, so their loads run three
+    // stages ahead (four register sets in rotation) and the block headers a whole
+    // super-block ahead: one stage of lookahead is less than the memory latency under load.
+    u32x4 hdr[2][4], wq[4][4];
+    f16x8 aring[8], aaug;
+    auto load_hdr = [&](int sb, u32x4 (&h)[4]) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) h[i] = ld16(sheet + (size_t)sb * 144 + woff[i]);
+    };
+    auto load_q = [&](int step, u32x4 (&q)[4]) {
+        const uint8_t* b = sheet + (size_t)(step >> 1) * 144 + 16 + 64 * (step & 1) + 16 * chunk;
+#pragma unroll
+        for (int i = 0; i < 4; i++) q[i] = ld16(b + woff[i]);
+    };
+    load_hdr(0, hdr[0]);
+    load_q(0, wq[0]);
+    load_q(min(1, nsteps - 1), wq[1]);
+    load_q(min(2, nsteps - 1), wq[2]);
+    load_hdr(min(1, nsb - 1), hdr[1]);
+#pragma unroll
+    for (int ks = 0; ks < 8; ks++) aring[ks] = a_frag(0, ks);
+    aaug = a_frag(1, 8);
+
+    // STEP4 = step % 4 names the register sets: weights wq[STEP4], headers hdr[(STEP4 / 2)]
+    auto stage = [&](auto STEP4, int step) {
+        constexpr int s4 = decltype(STEP4)::value, half = s4 & 1, hs = s4 >> 1;
+        const int sb = step >> 1;
+        const int nstep = min(step + 1, nsteps - 1);
+        load_q(min(step + 3, nsteps - 1), wq[(s4 + 3) & 3]);
+        // dequantize this stage into the wavefront's buffer
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            GemmWideScale sc;
+            gemm_wide_scale(hdr[hs][i], hh, half, sc);
+            sc.dst = sW + (16 * i + drow) * JL_MOEG_WROW + 64 * hh + 32 * wq_;
+#pragma unroll
+            for (int c = 0; c < 4; c++) gemm_wide_word(wq[s4][i][c], sc, c, mask_lo, mask_hi, magic);
+            if (half == 0) {
+                // the super-block's minimum columns (even chunks: m_s, odd: 64 m_s) and (d, dmin);
+                // lanes that share an address store the same value
+                const GemmScaleBytes sbytes = gemm_scale_bytes(hdr[hs][i].y, hdr[hs][i].z, hdr[hs][i].w);
+                const float mul = wq_ ? 64.0f : 1.0f;
+                f16x8 mm;
+#pragma unroll
+                for (int b = 0; b < 4; b++) {
+                    mm[b] = (_Float16)((float)((sbytes.mn_lo >> (8 * b)) & 0xFF) * mul);
+                    mm[4 + b] = (_Float16)((float)((sbytes.mn_hi >> (8 * b)) & 0xFF) * mul);
+                }
+                *(f16x8*)(sMin + (16 * i + drow) * JL_MOEG_MROW + 8 * wq_) = mm;
+                float2 dd = {half_bits_to_f32((uint16_t)(hdr[hs][i].x & 0xFFFF)),
+                             half_bits_to_f32((uint16_t)(hdr[hs][i].x >> 16))};
+                *(float2*)(sSc + 2 * (16 * i + drow)) = dd;
+            }
+        }
+        // this super-block's headers are done with after its second half: fetch those of the
+        // super-block after next into their place
+        if (half == 1) load_hdr(min(sb + 2, nsb - 1), hdr[hs]);
+        // matrix work: fragments a K-step ahead; the ring slot is refilled for the next stage
+        f32x4 dav[4];
+        if (half == 1) {   // the group's token scales, for the epilogue below
+#pragma unroll
+            for (int i = 0; i < 4; i++) dav[i] = *(const f32x4*)(dabase + (size_t)sb * (32 * p.nslots) + 8 * i);
+        }
+        const _Float16* wp0 = sW + arow * JL_MOEG_WROW + 8 * kg;
+        f16x8 wf[2][2];
+#pragma unroll
+        for (int j = 0; j < 2; j++) wf[0][j] = *(const f16x8*)(wp0 + 32 * j * JL_MOEG_WROW);
+#pragma unroll
+        for (int ks = 0; ks < 8; ks++) {
+            if (ks + 1 < 8) {
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+                    wf[(ks + 1) & 1][j] = *(const f16x8*)(wp0 + 32 * j * JL_MOEG_WROW + 16 * (ks + 1));
+            }
+            const f32x16 czero = {0};
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+                accP[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aring[ks], wf[ks & 1][j],
+                                                                 (half == 0 && ks == 0) ? czero : accP[j], 0, 0, 0);
+            aring[ks] = a_frag(nstep, ks);
+        }
+        if (half == 1) {
+            // out += d_a * (d * P - dmin * M) for the super-block
+            const f32x16 czero = {0};
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                const f16x8 wm = *(const f16x8*)(sMin + (32 * j + arow) * JL_MOEG_MROW + 8 * kg);
+                const float2 esc = *(const float2*)(sSc + 2 * (32 * j + arow));
+                const f32x16 accM = __builtin_amdgcn_mfma_f32_32x32x16_f16(aaug, wm, czero, 0, 0, 0);
+#pragma unroll
+                for (int el = 0; el < 16; el++) {
+                    const float u = fmaf(esc.x, accP[j][el], -(esc.y * accM[el]));
+                    out[j][el] = fmaf(dav[el >> 2][el & 3], u, out[j][el]);
+                }
+            }
+            aaug = a_frag(min(step + 2, nsteps - 1), 8);
+        }
+    };
+    for (int step = 0; step < nsteps; step += 4) {
+        stage(GemmIntC<0>{}, step);
+        stage(GemmIntC<1>{}, step + 1);
+        if (step + 2 < nsteps) {   // uniform
+            stage(GemmIntC<2>{}, step + 2);
+            stage(GemmIntC<3>{}, step + 3);
+        }
+    }
+
+    float* outm = p.out[mat];
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        const int r = r0 + 32 * j + arow;
+#pragma unroll
+        for (int el = 0; el < 16; el++) {
+            const int t = 8 * (el >> 2) + 4 * kg + (el & 3);
+            if (r < p.nrows && t < ncol) outm[(size_t)(c0 + t) * p.nrows + r] = out[j][el];
+        }
+    }
 }
 
 // resid[r][n] += sum over the row's k_used experts, ascending expert id, of

@@ -62,11 +62,16 @@ def _banks(t, n_expert, nrows, k, seed, planted):
     return np.concatenate([make(t, nrows, k, seed=seed + e) for e in range(n_expert)])
 
 
-@pytest.mark.parametrize("t,nrows,k", [(quant.Q4_K, 96, 2048), (quant.Q4_K, 200, 768), (quant.Q4_K, 40, 4096),
-                                       (quant.Q8_0, 64, 1024), (quant.Q6_K, 70, 1024)])
-def test_grouped_matvec_vs_oracle(dev, devbuf, t, nrows, k):
+@pytest.mark.parametrize("t,nrows,k,form", [(quant.Q4_K, 96, 2048, 1), (quant.Q4_K, 200, 768, 1),
+                                            (quant.Q4_K, 40, 4096, 1), (quant.Q4_K, 96, 2048, 2),
+                                            (quant.Q4_K, 300, 768, 2), (quant.Q4_K, 40, 4096, 2),
+                                            (quant.Q8_0, 64, 1024, 0), (quant.Q6_K, 70, 1024, 0)])
+def test_grouped_matvec_vs_oracle(dev, devbuf, t, nrows, k, form):
+    """form 1 = the dot-product kernel, 2 = groups of 32 columns on the matrix cores (Q4_K with
+    the k-quant window), 0 = what the library picks."""
     rows, n_expert, k_used, window = 13, 8, 3, 256 if t in quant.K_QUANTS else 32
     dev.SetActWindow(window)
+    dev.set_tuning(moe__form=form)
     sel, _ = route(rows, n_expert, k_used, 4)
     sel[0, :k_used] = [1, 2, 3]
     sel[1:12, 0] = 6                      # one expert with 11+ columns: more than one pass of eight
@@ -105,6 +110,40 @@ def test_grouped_matvec_vs_oracle(dev, devbuf, t, nrows, k):
         q, a_s, _ = oracle.quantize_act(h[c], window)
         want = oracle.matvec_q8act_f64(t, bank0[e * sheet:(e + 1) * sheet], q, a_s, nrows, k)
         assert rel_l2(got[c], want) <= 1e-3     # exp() differs in the last bits: an int8 may move
+    dev.SetActWindow(32)
+    dev.set_tuning(moe__form=0)
+
+
+def test_grouped_matmul_more_than_one_group_of_columns(dev, devbuf):
+    """An expert chosen by 70 rows has three groups of 32 columns (the last one ragged);
+    another gets one column, most get none.  Both forms against the oracle."""
+    t, nrows, k, window = quant.Q4_K, 130, 512, 256
+    rows, n_expert, k_used = 70, 6, 2
+    dev.SetActWindow(window)
+    sel = np.zeros((rows, k_used + 1), np.uint32)
+    sel[:, 0], sel[:, 1] = 4, 1
+    sel[3, 1] = 5
+    used, perm, col_e, pos = oracle.group_pairs(sel.reshape(-1), rows, k_used, n_expert, 1)
+    start = np.searchsorted(col_e[:used], np.arange(n_expert + 1)).astype(np.uint32)
+    bank = _banks(t, n_expert, nrows, k, 77, True)
+    x = np.stack([synth.activations(k, seed=600 + r) * np.float32(1 + r % 5) for r in range(rows)])
+    sheet = nrows * quant.row_bytes(t, k)
+    want = np.zeros((used, nrows))
+    for c in range(used):
+        e = int(col_e[c])
+        q, a_s, _ = oracle.quantize_act(x[perm[c]], window)
+        want[c] = oracle.matvec_q8act_f64(t, bank[e * sheet:(e + 1) * sheet], q, a_s, nrows, k)
+    b, xd, dstart, dperm = devbuf(bank), devbuf(x), devbuf(start), devbuf(perm[:used].copy())
+    for form in (1, 2):
+        dev.set_tuning(moe__form=form)
+        o = devbuf(shape=(used * nrows + 8,), dtype=np.float32, fill=np.float32(4e30))
+        assert dev.moe_matvec_dev(o.ptr, None, t, b.ptr, None, xd.ptr, None, dperm.ptr, dstart.ptr, n_expert, used,
+                                  nrows, k)
+        dev.synchronize()
+        got = o.get()
+        assert np.all(got[used * nrows:] == np.float32(4e30))
+        assert nmse(got[:used * nrows].reshape(used, nrows), want) <= 1e-10, form
+    dev.set_tuning(moe__form=0)
     dev.SetActWindow(32)
 
 
