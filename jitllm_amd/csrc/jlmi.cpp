@@ -34,6 +34,7 @@ struct Tuning {
     int gemm_form = 0;
     int gemm_split = 0;
     int moe_form = 0;
+    int moe_waves = 0;
     int mx_split = 0;
 };
 
@@ -638,14 +639,16 @@ int moe_matvec_launch(jl_ctx* c, float* out0, float* out1, int type, const void*
     a.bank[0] = (const uint8_t*)bank0; a.bank[1] = (const uint8_t*)bank1;
     a.q = qa.q; a.as = qa.as; a.s16 = qa.s16; a.start = start;
     a.sheet_bytes = sheet; a.nrows = nrows; a.k = k; a.row_bytes = row_bytes;
-    // A workgroup of eight wavefronts covers 8 * 2 * (64 / lpr) rows per step.  Row shares:
-    // about six workgroups per CU when every expert is in use (from sweeps at the
-    // 128-expert, 64-row shape), each share at least one step.
-    const int nmat = bank1 ? 2 : 1, nwaves = 8;
+    // A workgroup of four wavefronts covers 4 * 2 * (64 / lpr) rows per step; at the kernel's
+    // ~150 registers three such workgroups fill a CU's twelve wavefront slots, where one of
+    // eight wavefronts leaves four empty (sweeps at the 128-expert, 64-row shape: 210 -> 150 us
+    // for the block).  Row shares: about twelve workgroups per CU when every expert is in use,
+    // each share at least one step.
+    const int nmat = bank1 ? 2 : 1, nwaves = c->tune.moe_waves > 0 && c->tune.moe_waves <= 8 ? c->tune.moe_waves : 4;
     const int rows_per_step = nwaves * 2 * (64 / lpr);  // JL_MOE_U row groups per wavefront step
     int shares = c->tune.moe_shares;
     if (shares <= 0) {
-        shares = (6 * c->num_cu + n_expert * nmat - 1) / (n_expert * nmat);
+        shares = (12 * c->num_cu + n_expert * nmat - 1) / (n_expert * nmat);
         const int most = (nrows + rows_per_step - 1) / rows_per_step;
         if (shares > most) shares = most;
     }
@@ -781,6 +784,7 @@ int jl_set_tuning(jl_ctx* c, const char* key, int value) {
     else if (!strcmp(key, "packed.block")) c->tune.packed_block = value;
     else if (!strcmp(key, "moe.shares")) c->tune.moe_shares = value;
     else if (!strcmp(key, "moe.form")) c->tune.moe_form = value;
+    else if (!strcmp(key, "moe.waves")) c->tune.moe_waves = value;
     else if (!strcmp(key, "gemm.rows")) c->tune.gemm_rows = value;
     else if (!strcmp(key, "mxfp4.split")) c->tune.mx_split = value;
     else if (!strcmp(key, "gemm.form")) c->tune.gemm_form = value;
