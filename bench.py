@@ -193,10 +193,11 @@ def gemm_section(dev, shapes=None):
 
 
 def ffn_section(dev):
-    """A gated feed-forward block at decode, the baseline's second configuration: gate and up
-    (Q8_0 14336x4096) as one grouped launch, then down (Q6_K 4096x14336) over silu(gate) * up
-    formed inside its quantizer with the residual add riding on the launch: two launches per
-    block.  Four rotating sets of the three matrices (692 MiB) keep every step out of cache."""
+    """A gated feed-forward block at decode, the baseline's second configuration: RMSNorm folded
+    into the quantizer of gate and up (Q8_0 14336x4096), one grouped launch; then down (Q6_K
+    4096x14336) over silu(gate) * up formed inside its quantizer with the residual add riding
+    on the launch: two launches per block.  Four rotating sets of the three matrices
+    (692 MiB) keep every step out of cache."""
     from jitllm_amd import quant, synth
     from jitllm_amd.hipmem import DeviceArray, Event, check, hip
     n_embd, n_ffn = 4096, 14336
@@ -208,6 +209,7 @@ def ffn_section(dev):
         g, u, d = DeviceArray(wg), DeviceArray(wg), DeviceArray(wd)
         sets.append((g, u, d))
     x = DeviceArray(synth.activations(n_embd, seed=2))
+    norm_w = DeviceArray(np.ones(n_embd, np.float32))
     gate = DeviceArray(shape=(n_ffn,), dtype=np.float32, fill=0)
     up = DeviceArray(shape=(n_ffn,), dtype=np.float32, fill=0)
     y = DeviceArray(shape=(n_embd,), dtype=np.float32, fill=0)
@@ -216,7 +218,7 @@ def ffn_section(dev):
     def run(i):
         g, u, d = sets[i % len(sets)]
         ok = dev.matvec_group_dev([gate.ptr, up.ptr], [quant.Q8_0, quant.Q8_0], [g.ptr, u.ptr], [n_ffn, n_ffn],
-                                  x.ptr, n_embd)
+                                  x.ptr, n_embd, norm_w=norm_w.ptr, norm_eps=1e-5)
         ok = ok and dev.matvec_group_dev([y.ptr], [quant.Q6_K], [d.ptr], [n_embd], gate.ptr, n_ffn, act_up=up.ptr,
                                          resid=resid.ptr, alpha=1.0)
         if not ok:
@@ -234,7 +236,7 @@ def ffn_section(dev):
     nbytes = 2 * wg.nbytes + wd.nbytes + 4 * (n_embd + 2 * n_ffn) + 4 * (2 * n_ffn + 2 * n_embd)
     for g, u, d in sets:
         g.free(); u.free(); d.free()
-    for b in (x, gate, up, y, resid):
+    for b in (x, norm_w, gate, up, y, resid):
         b.free()
     return {"us_per_step": round(ms * 1e3, 2), "launches_per_step": 2, "bytes_per_step": nbytes,
             "GB/s": round(nbytes / (ms * 1e-3) / 1e9, 1),

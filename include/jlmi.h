@@ -160,7 +160,11 @@ int jl_matvec_q8_dev(jl_ctx *ctx, float *out, int type, const void *w, const int
  * single projection) read ONE activation x[0:k]; out[i] gets rows[i] rows of w[i] (type
  * type[i]).  act_up, when set, makes the activation silu(x) * act_up, formed on the way
  * into the quantizer (x is left as it was).  resid, when set, takes matrix 0's rows as
- * they are made: resid[r] += alpha * out[0][r].  Matrices of one type share a launch. */
+ * they are made: resid[r] += alpha * out[0][r].  norm_w, when set, puts an RMSNorm in
+ * front of everything, the reference's RMSNormQuantRows (jit/gpu/kernels/elem.go:252-267)
+ * with the arithmetic of its host form (internal/oracle/oracle.go:230-240): the activation
+ * is f32(f64(x) * 1/sqrt(mean(x^2) + norm_eps) * f64(norm_w)), mean in f64; norm_out, when
+ * set, receives that normed vector.  Matrices of one type share a launch. */
 #define JL_MAX_GROUP 4
 typedef struct jl_mv_group {
     int n;
@@ -173,6 +177,9 @@ typedef struct jl_mv_group {
     const float *act_up;
     float *resid;
     float alpha;
+    const float *norm_w;
+    float norm_eps;
+    float *norm_out;
 } jl_mv_group;
 int jl_matvec_group_dev(jl_ctx *ctx, const jl_mv_group *g, void *stream);
 

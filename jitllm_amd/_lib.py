@@ -26,7 +26,8 @@ class MVGroup(C.Structure):
     """jl_mv_group: the reference's nn.MVGroup over device pointers."""
     _fields_ = [("n", C.c_int), ("out", C.c_void_p * MAX_GROUP), ("type", C.c_int * MAX_GROUP),
                 ("w", C.c_void_p * MAX_GROUP), ("rows", C.c_int * MAX_GROUP), ("x", C.c_void_p),
-                ("k", C.c_int), ("act_up", C.c_void_p), ("resid", C.c_void_p), ("alpha", C.c_float)]
+                ("k", C.c_int), ("act_up", C.c_void_p), ("resid", C.c_void_p), ("alpha", C.c_float),
+                ("norm_w", C.c_void_p), ("norm_eps", C.c_float), ("norm_out", C.c_void_p)]
 
 
 # name -> (restype, argtypes); every symbol include/jlmi.h declares

@@ -218,7 +218,8 @@ int matvec_launch(jl_ctx* c, float* out, int type, const void* w, const float* x
 // m matrices of one type in one launch (kernels/matvec.h, matvec_multi_body).
 int matvec_multi_launch(jl_ctx* c, int type, int m, float* const* outs, const void* const* ws, const int* rows,
                         const float* x, size_t xstride, const float* x2, float* resid, float alpha, int k,
-                        hipStream_t st) {
+                        hipStream_t st, const float* norm_w = nullptr, float norm_eps = 0.f,
+                        float* norm_out = nullptr) {
     if (m < 1 || m > JL_MAX_MULTI) return fail(c, JL_ERR_ARG, "matvec multi: %d matrices", m);
     const TypeInfo* ti = nullptr;
     int max_rows = 0;
@@ -231,6 +232,7 @@ int matvec_multi_launch(jl_ctx* c, int type, int m, float* const* outs, const vo
         if (rows[i] > max_rows) max_rows = rows[i];
     }
     if (!x || !aligned16(x) || (x2 && !aligned16(x2)) || (xstride % 4) != 0) return JL_DECLINED;
+    if ((norm_w && !aligned16(norm_w)) || (norm_out && !aligned16(norm_out))) return JL_DECLINED;
     MatVecMultiArgs a;
     memset(&a, 0, sizeof a);
     for (int i = 0; i < m; i++) {
@@ -239,6 +241,7 @@ int matvec_multi_launch(jl_ctx* c, int type, int m, float* const* outs, const vo
         a.nrows[i] = rows[i];
     }
     a.x = x; a.x2 = x2; a.resid = resid; a.alpha = alpha; a.xstride = xstride;
+    a.norm_w = norm_w; a.norm_eps = norm_eps; a.norm_out = norm_out;
     a.k = k; a.row_bytes = (k / ti->block_elems) * ti->block_bytes; a.per = c->act_window / 32;
     // sixteen wavefronts a workgroup, one row each; about two workgroups per CU over all
     // the matrices, never more row groups than the tallest matrix has
@@ -858,6 +861,7 @@ int jl_matvec_group_dev(jl_ctx* c, const jl_mv_group* g, void* stream) {
         if ((g->type[i] == JL_TYPE_Q4_K && !aligned16(g->w[i])) || ((uintptr_t)g->w[i] & 1)) return JL_DECLINED;
     }
     if (!aligned16(g->x) || (g->act_up && !aligned16(g->act_up))) return JL_DECLINED;
+    if ((g->norm_w && !aligned16(g->norm_w)) || (g->norm_out && (!g->norm_w || !aligned16(g->norm_out)))) return JL_DECLINED;
     // matrices of one type share a launch; matrix 0 leads its launch so that the residual rides on it
     bool done[JL_MAX_GROUP] = {false, false, false, false};
     for (int i = 0; i < g->n; i++) {
@@ -871,7 +875,8 @@ int jl_matvec_group_dev(jl_ctx* c, const jl_mv_group* g, void* stream) {
                 done[j] = true;
             }
         int rc = matvec_multi_launch(c, g->type[i], m, outs, ws, rows, g->x, 0, g->act_up,
-                                     i == 0 ? g->resid : nullptr, g->alpha, g->k, st);
+                                     i == 0 ? g->resid : nullptr, g->alpha, g->k, st, g->norm_w, g->norm_eps,
+                                     i == 0 ? g->norm_out : nullptr);
         if (rc != JL_OK) return rc;
     }
     return JL_OK;

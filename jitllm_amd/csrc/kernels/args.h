@@ -33,6 +33,9 @@ struct MatVecMultiArgs {
     float alpha;
     size_t xstride;      // elements
     int k, row_bytes, per, nwaves, ngroups;
+    const float* norm_w; // null: none; else the activation is RMSNorm(x) * norm_w first
+    float* norm_out;     // optional: the normed activation, written once
+    float norm_eps;
 };
 
 // Activation preparation for the Q4_K prefill GEMM: quantize x and lay it out

@@ -414,6 +414,13 @@ __device__ __forceinline__ void matvec_body(const MatVecArgs& p, uint8_t* smem) 
 // q/k/v or gate/up of a block (MatVecPackedGroup, engine/nn/packedgroup.go:13-51), a
 // mixture's experts at decode (MatVecPackedMulti / MatVecPackedGatherAct,
 // engine/nn/packedmulti.go:24,84,93); on this machine the saving is the per-launch cost.
+// Sum over the 64 lanes in f64, butterfly order (every lane gets the sum).
+__device__ __forceinline__ double wave_sum_f64(double v) {
+#pragma unroll
+    for (int m = 1; m < 64; m <<= 1) v += __shfl_xor(v, m, 64);
+    return v;
+}
+
 template <int TYPE>
 __device__ __forceinline__ void matvec_multi_body(const MatVecMultiArgs& p, uint8_t* smem) {
     typedef SlotTraits<TYPE> T;
@@ -436,11 +443,37 @@ __device__ __forceinline__ void matvec_multi_body(const MatVecMultiArgs& p, uint
     __builtin_amdgcn_s_barrier();   // activation loads of the whole workgroup go out first
     typename T::W w;
     T::load_w(w0 + (size_t)min(r0, nrows - 1) * p.row_bytes, min(lane, nslots - 1), w);
+    // RMSNorm ahead of the quantizer (the reference's RMSNormQuantRows, jit/gpu/kernels/
+    // elem.go:252-267, with its host arithmetic, internal/oracle/oracle.go:230-240): the sum
+    // of squares in f64, scale = 1/sqrt(sum/k + eps), y = f32(f64(x) * scale * f64(w)).
+    // Every workgroup forms the sum itself: k floats are cheaper than a launch.
+    double nscale = 0.0;
+    if (p.norm_w) {
+        double ss = 0.0;
+        for (int g4 = threadIdx.x; g4 < n4; g4 += nthreads) {
+            const f32x4 v = g4 == (int)threadIdx.x ? x0 : ((const f32x4*)x)[g4];
+            ss += (double)v.x * v.x + (double)v.y * v.y + (double)v.z * v.z + (double)v.w * v.w;
+        }
+        ss = wave_sum_f64(ss);
+        double* red = (double*)smem;   // the staging area is not in use yet
+        if (lane == 0) red[wave] = ss;
+        __syncthreads();
+        double tot = 0.0;
+        for (int i = 0; i < nwaves; i++) tot += red[i];
+        __syncthreads();               // everyone has read before the quantizer writes
+        nscale = 1.0 / __builtin_sqrt(tot / (double)p.k + (double)p.norm_eps);
+    }
     for (int g4 = threadIdx.x; g4 < n4_pad; g4 += nthreads) {
         f32x4 v = x0, u = u0;
         if (g4 != (int)threadIdx.x) {
             v = ((const f32x4*)x)[min(g4, n4 - 1)];
             if (x2) u = ((const f32x4*)x2)[min(g4, n4 - 1)];
+        }
+        if (p.norm_w) {
+            const f32x4 nw = ((const f32x4*)p.norm_w)[min(g4, n4 - 1)];
+            v = f32x4{(float)((double)v.x * nscale * (double)nw.x), (float)((double)v.y * nscale * (double)nw.y),
+                      (float)((double)v.z * nscale * (double)nw.z), (float)((double)v.w * nscale * (double)nw.w)};
+            if (p.norm_out && blockIdx.x == 0 && y == 0 && g4 < n4) ((f32x4*)p.norm_out)[g4] = v;
         }
         if (x2) v = f32x4{silu_f32(v.x) * u.x, silu_f32(v.y) * u.y, silu_f32(v.z) * u.z, silu_f32(v.w) * u.w};
         stage_quantize4(smem, p.k, p.per, g4, v);

@@ -47,12 +47,6 @@
 // + 1e-20).  The f64 sum is taken as a butterfly over the lanes, so it can differ from the
 // reference's sequential sum in its last bit; after narrowing to f32 that moves a score
 // only when it sits on a rounding boundary.
-__device__ __forceinline__ double wave_sum_f64(double v) {
-#pragma unroll
-    for (int m = 1; m < 64; m <<= 1) v += __shfl_xor(v, m, 64);
-    return v;
-}
-
 __device__ __forceinline__ void moe_route_body(const MoeRouteArgs& p) {
     const int lane = threadIdx.x & 63, n = p.n_expert;
     const size_t row = blockIdx.x;

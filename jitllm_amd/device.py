@@ -183,14 +183,17 @@ class Device:
                                                      _ptr(a_s), _ptr(sum16), nrows, k, stream),
                             "jl_matvec_q8_dev")
 
-    def matvec_group_dev(self, outs, types, ws, rows, x, k, act_up=None, resid=None, alpha=0.0, stream=None):
+    def matvec_group_dev(self, outs, types, ws, rows, x, k, act_up=None, resid=None, alpha=0.0, stream=None,
+                         norm_w=None, norm_eps=0.0, norm_out=None):
         """JIT.MatVecPackedGroup: up to four matvecs reading one activation, optional
-        silu(x) * act_up and resid += alpha * out[0], in one launch per weight type."""
+        RMSNorm(x) * norm_w first, optional silu(x) * act_up and resid += alpha * out[0], in
+        one launch per weight type."""
         g = _lib.MVGroup()
         g.n = len(outs)
         for i in range(g.n):
             g.out[i], g.type[i], g.w[i], g.rows[i] = _ptr(outs[i]), types[i], _ptr(ws[i]), rows[i]
         g.x, g.k, g.act_up, g.resid, g.alpha = _ptr(x), k, _opt(act_up), _opt(resid), alpha
+        g.norm_w, g.norm_eps, g.norm_out = _opt(norm_w), norm_eps, _opt(norm_out)
         return self._served(self._l.jl_matvec_group_dev(self._ctx, C.byref(g), stream), "jl_matvec_group_dev")
 
     def matvec_gather_dev(self, outs, t, ws, x, xstride, up, nrows, k, stream=None):

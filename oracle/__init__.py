@@ -70,6 +70,8 @@ _l.jlo_bias_c.restype = C.c_double
 _l.jlo_bias_c.argtypes = [C.c_int]
 _l.jlo_matvec_q8act_f64.argtypes = [_f64p, C.c_int, _u8p, _i8p, _f32p, C.c_int, C.c_int]
 _l.jlo_matvec_q8act_f32.argtypes = [_f32p, C.c_int, _u8p, _i8p, _f32p, _f32p, C.c_int, C.c_int]
+_l.jlo_rmsnorm32.restype = None
+_l.jlo_rmsnorm32.argtypes = [_f32p, _f32p, _f32p, C.c_int, C.c_double]
 _l.jlo_moe_route.argtypes = [_f32p, C.c_int, C.c_int, _i32p, _f32p, _i32p, _f32p]
 _l.jlo_group_pairs.argtypes = [_u32p, C.c_int, C.c_int, C.c_int, C.c_int, _u32p, _u32p, _u32p,
                                C.c_int]
@@ -230,6 +232,14 @@ def matmul_q8act_f64(t, w, x, nrows, k, ntok, window):
         q, a_s, _ = quantize_act(x[i], window)
         out[i] = matvec_q8act_f64(t, w, q, a_s, nrows, k)
     return out
+
+
+def rmsnorm32(x, w, eps):
+    """RMSNorm over an f32 vector with f64 accumulation (oracle.RMSNorm32)."""
+    x, w = _chk(x, np.float32), _chk(w, np.float32, np.asarray(x).size)
+    y = np.empty(x.size, np.float32)
+    _l.jlo_rmsnorm32(_p(y, _f32p), _p(x, _f32p), _p(w, _f32p), x.size, float(eps))
+    return y
 
 
 def moe_route(logits, k):

@@ -810,6 +810,15 @@ static int lex_topk(const float *v, int n, int k, int32_t *out) {
     return found;
 }
 
+/* internal/oracle/oracle.go:230-240 (RMSNorm32): the sum of squares and the scale in f64,
+ * in element order; y[i] = f32(f64(x[i]) * scale * f64(w[i])). */
+void jlo_rmsnorm32(float *y, const float *x, const float *w, int n, double eps) {
+    double sum = 0;
+    for (int i = 0; i < n; i++) sum += (double)x[i] * (double)x[i];
+    double scale = 1 / sqrt(sum / (double)n + eps);
+    for (int i = 0; i < n; i++) y[i] = (float)((double)x[i] * scale * (double)w[i]);
+}
+
 /* internal/oracle/oracle.go:244-265 (Softmax32) then internal/oracle/moe.go:197-327
  * with Norm = true, Scale = 1, no bias, no groups, no expert scales. */
 int jlo_moe_route(const float *logits, int n, int k, int32_t *sel, float *wt, int32_t *ord,

@@ -41,6 +41,39 @@ def test_group_qkv_mixed_types_one_activation(dev, devbuf):
         assert nmse(got[:r], _want(t, w, x, r, k, window)) <= 1e-10
 
 
+@pytest.mark.parametrize("k,window", [(2048, 32), (4096, 256), (5120, 32)])
+def test_group_with_rmsnorm_in_front(dev, devbuf, k, window):
+    """RMSNorm folded into the group's quantizer (the reference's RMSNormQuantRows,
+    /root/reference/jit/gpu/kernels/elem.go:252-267): the normed vector must equal the
+    oracle's RMSNorm32 up to the order of the f64 sum (one f32 ulp at most, normally none),
+    and the matvecs must be the matvecs of THAT vector -- checked on the vector the device
+    wrote, so a moved int8 cannot hide an error."""
+    dev.SetActWindow(window)
+    types = (quant.Q4_K, quant.Q4_K, quant.Q6_K) if window == 32 else (quant.Q4_K, quant.Q4_K, quant.Q4_K)
+    spec = list(zip(types, (300, 64, 130)))
+    ws = [synth.quantized_weights(t, r, k, seed=i + 20) for i, (t, r) in enumerate(spec)]
+    x = synth.activations(k, seed=31) * np.float32(3.5)
+    nw = (1 + 0.1 * np.random.default_rng(8).standard_normal(k)).astype(np.float32)
+    eps = 1e-5
+    dws, dx, dnw = [devbuf(w) for w in ws], devbuf(x), devbuf(nw)
+    dn = devbuf(shape=(k + 4,), dtype=np.float32, fill=np.float32(-3e30))
+    outs = [devbuf(shape=(r,), dtype=np.float32, fill=np.float32(6e30)) for _, r in spec]
+    for call in range(2):
+        assert dev.matvec_group_dev([o.ptr for o in outs], [t for t, _ in spec], [w.ptr for w in dws],
+                                    [r for _, r in spec], dx.ptr, k, norm_w=dnw.ptr, norm_eps=eps, norm_out=dn.ptr)
+        dev.synchronize()
+        normed = dn.get()
+        assert np.all(normed[k:] == np.float32(-3e30))
+        normed = normed[:k]
+        want_n = oracle.rmsnorm32(x, nw, eps)
+        ulp = np.abs(normed.view(np.int32).astype(np.int64) - want_n.view(np.int32).astype(np.int64))
+        assert ulp.max() <= 1 and np.mean(ulp != 0) <= 0.01
+        for (t, r), w, o in zip(spec, ws, outs):
+            assert nmse(o.get(), _want(t, w, normed, r, k, window)) <= 1e-10
+            assert rel_l2(o.get(), _want(t, w, want_n, r, k, window)) <= 1e-3
+    dev.SetActWindow(32)
+
+
 def test_group_gate_up_then_gated_down_with_residual(dev, devbuf):
     """A gated feed-forward block as two groups: (gate, up) sharing x, then down over
     silu(gate) * up with the residual add riding on the launch."""

@@ -314,6 +314,32 @@ def test_cpu_baseline_restatement(t, window):
 
 
 # ------------------------------------------------------------------------- MoE
+def test_rmsnorm32_known_answers_and_invariants():
+    """RMSNorm32 (/root/reference/internal/oracle/oracle.go:230-240) pinned without retyping
+    it: a hand-computed case, exact rational arithmetic on a small vector, unit mean square
+    of the output for w = 1 and eps = 0, bit-identical output when x is scaled by a power of
+    two (eps = 0), and the large-eps limit x * w / sqrt(eps)."""
+    from fractions import Fraction
+    import math
+    y = oracle.rmsnorm32(np.array([3, 4], np.float32), np.array([1, 1], np.float32), 0.0)
+    assert np.array_equal(y, np.array([3 / math.sqrt(12.5), 4 / math.sqrt(12.5)], np.float64).astype(np.float32))
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal(37).astype(np.float32)
+    w = rng.standard_normal(37).astype(np.float32)
+    eps = 1e-6
+    mean = sum(Fraction(float(v)) ** 2 for v in x) / 37 + Fraction(eps)     # exact
+    want = np.array([float(Fraction(float(v)) * Fraction(float(u))) / math.sqrt(float(mean)) for v, u in zip(x, w)])
+    got = oracle.rmsnorm32(x, w, eps)
+    assert np.max(np.abs(got - want) / np.maximum(np.abs(want), 1e-30)) <= 2.0 ** -23   # one f32 rounding
+    x = rng.standard_normal(4096).astype(np.float32)
+    ones = np.ones(4096, np.float32)
+    y = oracle.rmsnorm32(x, ones, 0.0)
+    assert abs(np.sum(y.astype(np.float64) ** 2) / 4096 - 1) <= 1e-6
+    assert np.array_equal(oracle.rmsnorm32(x * np.float32(1024), ones, 0.0), y)
+    big = oracle.rmsnorm32(x, w := rng.standard_normal(4096).astype(np.float32), 1e12)
+    assert np.allclose(big, x.astype(np.float64) * w / 1e6, rtol=1e-5, atol=0)
+
+
 def test_moe_route_against_brute_force():
     rng = np.random.default_rng(0)
     for n, k in [(128, 8), (16, 2), (8, 1), (4, 4)]:
