@@ -195,6 +195,18 @@ int jl_matvec_gather_dev(jl_ctx *ctx, float *const *outs, int type, const void *
                          const float *x, size_t xstride, const float *up, int nrows, int k,
                          int m, void *stream);
 
+/* The same three operations over packed planes, as the reference runs them
+ * (engine/nn/packedmulti.go:24,84,93 take []*Packed): matrix j reads planes qs[j], d[j],
+ * sc[j] (sc may be null for Q8_0) from row row0[j] of a buffer of `stride` rows -- an
+ * expert's sheet inside its bank's pages is the bank's plane pointers with row0 =
+ * expert * nrows (device.go:70-80, format/jlm/write.go:165-180) -- and the activation
+ * x[j*xstride : j*xstride+k] (xstride 0: one shared activation); up, when given, makes it
+ * silu(x_j) * up_j.  m <= 16, one launch. */
+int jl_matvec_packed_multi_dev(jl_ctx *ctx, float *const *outs, int type, const uint32_t *const *qs,
+                               const uint32_t *const *d, const uint32_t *const *sc, const int *row0,
+                               int stride, const float *x, size_t xstride, const float *up, int nrows,
+                               int k, int m, void *stream);
+
 /* JIT.MatMulPacked / MatMul semantics on resident operands (engine/nn/packedmm.go:23,
  * matmul.go:27): x [ntok][k] f32 -> out [ntok][nrows], every token quantized on
  * its own.  Q4_K with the 256 window runs the matrix-core GEMM (quantize-and-

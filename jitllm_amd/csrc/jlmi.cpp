@@ -537,6 +537,47 @@ int packed_matvec_launch(jl_ctx* c, float* out, int type, const PlaneRef& pl, co
                   (unsigned)(nw * (384 + 65 * 4)), st, params);  // JL_PK_LDS_BYTES
 }
 
+// m packed matvecs of one type and shape in one launch (grid.y = matrix): each with its
+// own planes and first row, reading x + j * xstride; up gates the activation.
+int packed_matvec_multi_launch(jl_ctx* c, int type, int m, float* const* outs, const PlaneRef* pls,
+                               const float* x, size_t xstride, const float* up, int nrows, int k,
+                               hipStream_t st) {
+    if (m < 1 || m > JL_MAX_MULTI) return fail(c, JL_ERR_ARG, "packed multi: %d matrices", m);
+    const TypeInfo* ti = nullptr;
+    for (int j = 0; j < m; j++) {
+        int rc = packed_check(c, type, pls[j], nrows, k, &ti);
+        if (rc != JL_OK) return rc;
+        if (!outs[j]) return fail(c, JL_ERR_ARG, "packed multi: null out");
+        if (pls[j].stride != pls[0].stride) return JL_DECLINED;
+    }
+    if (!x || !aligned16(x) || (up && !aligned16(up)) || (xstride % 4) != 0) return JL_DECLINED;
+    // rows per wavefront: the widest run that still gives three CUs in four a workgroup,
+    // counting every matrix's row groups
+    int rw = c->tune.packed_rw;
+    if (rw <= 0) {
+        rw = 64;
+        while (rw > 16 && (long)m * ((nrows + rw - 1) / rw) < c->num_cu * 3 / 4) rw >>= 1;
+    }
+    if (rw != 16 && rw != 32 && rw != 64) return fail(c, JL_ERR_ARG, "packed multi: rw=%d", rw);
+    const int nchunks = (k + 255) / 256;
+    int nw = c->tune.packed_block > 0 ? c->tune.packed_block / 64 : 16;
+    if (nw > nchunks) nw = nchunks;
+    if (nw < 1 || nw > 16) return fail(c, JL_ERR_ARG, "packed multi: block=%d", nw * 64);
+    PackedMultiArgs a;
+    memset(&a, 0, sizeof a);
+    for (int j = 0; j < m; j++) {
+        a.out[j] = outs[j]; a.qs[j] = pls[j].qs; a.d[j] = pls[j].d; a.sc[j] = pls[j].sc; a.row0[j] = pls[j].row;
+    }
+    a.x = x; a.x2 = up; a.xstride = xstride;
+    a.nrows = nrows; a.k = k; a.stride = pls[0].stride; a.per = c->act_window / 32;
+    a.nwaves = nw; a.ngroups = (nrows + rw - 1) / rw;
+    char name[64];
+    snprintf(name, sizeof name, "jl_matvec_packed_multi_%s%s_w%d", up ? "act_" : "", ti->tag, rw);
+    void* params[] = {&a};
+    return launch(c, name, (unsigned)a.ngroups, (unsigned)m, (unsigned)(nw * 64), (unsigned)(nw * (384 + 65 * 4)), st,
+                  params);   // JL_PK_LDS_BYTES
+}
+
 int unpack_launch(jl_ctx* c, const PlaneRef& pl, int nrows, int k, void* dst, hipStream_t st) {
     UnpackArgs a;
     a.dst = (uint8_t*)dst; a.qs = pl.qs; a.d = pl.d; a.sc = pl.sc;
@@ -724,6 +765,10 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
             names.push_back(nm);
         }
     for (const char* tag : {"q4k", "q8_0", "q6k"}) names.push_back(std::string("jl_matvec_multi_") + tag);
+    for (const char* tag : {"q4k", "q8_0", "q6k"})
+        for (int rw : {16, 32, 64})
+            for (const char* form : {"", "act_"})
+                names.push_back(std::string("jl_matvec_packed_multi_") + form + tag + "_w" + std::to_string(rw));
     for (const auto& n : names) {
         hipFunction_t f;
         e = H->ModuleGetFunction(&f, c->module, n.c_str());
@@ -880,6 +925,22 @@ int jl_matvec_group_dev(jl_ctx* c, const jl_mv_group* g, void* stream) {
         if (rc != JL_OK) return rc;
     }
     return JL_OK;
+}
+
+int jl_matvec_packed_multi_dev(jl_ctx* c, float* const* outs, int type, const uint32_t* const* qs,
+                               const uint32_t* const* d, const uint32_t* const* sc, const int* row0, int stride,
+                               const float* x, size_t xstride, const float* up, int nrows, int k, int m,
+                               void* stream) {
+    if (!c) return JL_ERR_ARG;
+    if (!outs || !qs || !d || !row0 || m < 1) return fail(c, JL_ERR_ARG, "packed multi: bad operand");
+    if (m > JL_MAX_MULTI) return JL_DECLINED;
+    HIP_TRY(c, H->SetDevice(c->device));
+    PlaneRef pls[JL_MAX_MULTI];
+    for (int j = 0; j < m; j++) {
+        pls[j].qs = qs[j]; pls[j].d = d[j]; pls[j].sc = sc ? sc[j] : nullptr;
+        pls[j].row = row0[j]; pls[j].stride = stride;
+    }
+    return packed_matvec_multi_launch(c, type, m, outs, pls, x, xstride, up, nrows, k, pick_stream(c, stream));
 }
 
 int jl_matvec_multi_dev(jl_ctx* c, float* const* outs, int type, const void* const* ws, const float* x,

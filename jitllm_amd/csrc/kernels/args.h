@@ -223,5 +223,21 @@ struct PackedMatVecArgs {
     int nrows, k, row0, stride;
     int per;              // activation window / 32
     int nwaves;           // wavefronts per workgroup (the launch's block / 64)
-    int ngroups;          // workgroups (the launch's grid)
+    int ngroups;          // workgroups (the launch's grid.x)
+    const float* x2;      // gated kernels only: the activation is silu(x) * x2
+};
+
+// Several packed matvecs of one type and shape in one launch, grid = (row groups,
+// matrices): matrix y has its own planes and first row (an expert's sheet inside its bank's
+// planes: the same plane pointers, row0 = expert * rows) and reads x + y * xstride.
+struct PackedMultiArgs {
+    float* out[JL_MAX_MULTI];
+    const uint32_t* qs[JL_MAX_MULTI];
+    const uint32_t* d[JL_MAX_MULTI];
+    const uint32_t* sc[JL_MAX_MULTI];
+    int row0[JL_MAX_MULTI];
+    const float* x;
+    const float* x2;      // null: plain activation
+    size_t xstride;       // elements
+    int nrows, k, stride, per, nwaves, ngroups;
 };

@@ -314,30 +314,37 @@ template <int NB> struct PkTraits<JL_Q6_K, NB> { typedef PkWQ6K<NB> W; };
 // 0-7) and a half-block sum in .z (lanes 0-15).  Loads are unconditional at clamped
 // addresses, so nothing between them makes the compiler wait for data; what lies past
 // the end of the vector is zeroed when the chunk is staged.
-typedef f32x4 PkX;
+// The gated form carries the gate's partner beside it.
+template <bool GATED> struct PkX { f32x4 v; };
+template <> struct PkX<true> { f32x4 v, u; };
 
-template <bool FUSED>
-__device__ __forceinline__ void pk_load_x(const PackedMatVecArgs& p, int c, int lane, PkX& X) {
+template <bool FUSED, bool GATED>
+__device__ __forceinline__ void pk_load_x(const PackedMatVecArgs& p, int c, int lane, PkX<GATED>& X) {
     const int g4 = min(c * 64 + lane, p.k / 4 - 1);
     if (FUSED) {
-        X = ((const f32x4*)p.x)[g4];
+        X.v = ((const f32x4*)p.x)[g4];
+        if constexpr (GATED) X.u = ((const f32x4*)p.x2)[g4];
     } else {
-        X.x = __uint_as_float(((const u32*)p.q)[g4]);
-        X.y = p.as[min(c * 8 + (lane & 7), p.k / 32 - 1)];
-        X.z = p.s16[min(c * 16 + (lane & 15), p.k / 16 - 1)];
-        X.w = 0.f;
+        X.v.x = __uint_as_float(((const u32*)p.q)[g4]);
+        X.v.y = p.as[min(c * 8 + (lane & 7), p.k / 32 - 1)];
+        X.v.z = p.s16[min(c * 16 + (lane & 15), p.k / 16 - 1)];
+        X.v.w = 0.f;
     }
 }
 
 // Quantize (or copy) the chunk's activation into the wavefront's private LDS area.
-template <bool FUSED>
-__device__ __forceinline__ void pk_stage_x(const PackedMatVecArgs& p, int c, int lane, const PkX& X, uint8_t* my) {
+template <bool FUSED, bool GATED>
+__device__ __forceinline__ void pk_stage_x(const PackedMatVecArgs& p, int c, int lane, const PkX<GATED>& X, uint8_t* my) {
     u32* a_w = (u32*)my;
     float* da_w = (float*)(my + 256);
     float* ss_w = (float*)(my + 288);
     const bool live = c * 64 + lane < p.k / 4;
     if (FUSED) {
-        const f32x4 xv = live ? X : f32x4{0.f, 0.f, 0.f, 0.f};
+        f32x4 xv = live ? X.v : f32x4{0.f, 0.f, 0.f, 0.f};
+        if constexpr (GATED) {
+            const f32x4 u = live ? X.u : f32x4{0.f, 0.f, 0.f, 0.f};
+            xv = f32x4{silu_f32(xv.x) * u.x, silu_f32(xv.y) * u.y, silu_f32(xv.z) * u.z, silu_f32(xv.w) * u.w};
+        }
         u32 m = max(max(abs_bits(xv.x), abs_bits(xv.y)), max(abs_bits(xv.z), abs_bits(xv.w)));
         const u32 amax = p.per == 8 ? wave_amax_256(m) : window_amax(m, p.per);
         float d;
@@ -347,9 +354,9 @@ __device__ __forceinline__ void pk_stage_x(const PackedMatVecArgs& p, int c, int
         if ((lane & 3) == 0) ss_w[lane >> 2] = (float)sum;
         if ((lane & 7) == 0) da_w[lane >> 3] = d;
     } else {
-        a_w[lane] = live ? __float_as_uint(X.x) : 0u;
-        if (lane < 8) da_w[lane] = X.y;
-        if (lane < 16) ss_w[lane] = X.z;
+        a_w[lane] = live ? __float_as_uint(X.v.x) : 0u;
+        if (lane < 8) da_w[lane] = X.v.y;
+        if (lane < 16) ss_w[lane] = X.v.z;
     }
     // The area is private to this wavefront, whose LDS operations complete in
     // order: only the compiler has to be kept from moving reads above the writes.
@@ -372,7 +379,7 @@ __device__ __forceinline__ void pk_stage_x(const PackedMatVecArgs& p, int c, int
 // The partial sums [wavefront][lane] are added up by RW*16 threads at once: thread
 // (row r, j) takes wavefront j's KP partials of row r, and the sixteen j of a row sit
 // in one 16-lane DPP row, so the sum over wavefronts is four lane-exchange adds.
-template <int TYPE, int RW, int XPRE, bool FUSED>
+template <int TYPE, int RW, int XPRE, bool FUSED, bool GATED = false>
 __device__ __forceinline__ void packed_matvec_body(const PackedMatVecArgs& p, uint8_t* smem) {
     constexpr int KP = 64 / RW, NB = 8 / KP;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = p.nwaves;
@@ -391,16 +398,16 @@ __device__ __forceinline__ void packed_matvec_body(const PackedMatVecArgs& p, ui
     A.ss = (const float*)(my + 288);
 
     const int nchunks = (p.k + 255) / 256;
-    PkX X[XPRE];
+    PkX<GATED> X[XPRE];
 #pragma unroll
-    for (int i = 0; i < XPRE; i++) pk_load_x<FUSED>(p, wave + i * nwaves, lane, X[i]);
+    for (int i = 0; i < XPRE; i++) pk_load_x<FUSED, GATED>(p, wave + i * nwaves, lane, X[i]);
     __builtin_amdgcn_s_barrier();
 
     float acc = 0.f;
-    auto chunk = [&](int c, const PkX& Xc) {
+    auto chunk = [&](int c, const PkX<GATED>& Xc) {
         typename PkTraits<TYPE, NB>::W w;
         pk_load<NB>(p, c, b0, row, w);
-        pk_stage_x<FUSED>(p, c, lane, Xc, my);
+        pk_stage_x<FUSED, GATED>(p, c, lane, Xc, my);
         acc += pk_dot<NB>(p, w, c, b0, row, A);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -411,8 +418,8 @@ __device__ __forceinline__ void packed_matvec_body(const PackedMatVecArgs& p, ui
         if (c < nchunks) chunk(c, X[i]);
     }
     for (int c = wave + XPRE * nwaves; c < nchunks; c += nwaves) {
-        PkX Xc;
-        pk_load_x<FUSED>(p, c, lane, Xc);
+        PkX<GATED> Xc;
+        pk_load_x<FUSED, GATED>(p, c, lane, Xc);
         chunk(c, Xc);
     }
 
@@ -432,4 +439,18 @@ __device__ __forceinline__ void packed_matvec_body(const PackedMatVecArgs& p, ui
         t += dpp_f32<JL_DPP_ROW_MIRROR, 0xf>(t);
         if (j == 0 && g * RW + r < p.nrows) p.out[g * RW + r] = t;
     }
+}
+
+// Matrix blockIdx.y of a multi launch as a single packed matvec.
+template <int TYPE, int RW, int XPRE, bool GATED>
+__device__ __forceinline__ void packed_matvec_multi_body(const PackedMultiArgs& m, uint8_t* smem) {
+    const int y = blockIdx.y;
+    PackedMatVecArgs p;
+    p.out = m.out[y]; p.qs = m.qs[y]; p.d = m.d[y]; p.sc = m.sc[y];
+    p.x = m.x + (size_t)y * m.xstride;
+    p.x2 = GATED ? m.x2 + (size_t)y * m.xstride : nullptr;
+    p.q = nullptr; p.as = nullptr; p.s16 = nullptr;
+    p.nrows = m.nrows; p.k = m.k; p.row0 = m.row0[y]; p.stride = m.stride;
+    p.per = m.per; p.nwaves = m.nwaves; p.ngroups = m.ngroups;
+    packed_matvec_body<TYPE, RW, XPRE, true, GATED>(p, smem);
 }

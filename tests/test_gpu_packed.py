@@ -158,6 +158,47 @@ def test_matvec_packed_row_range_of_a_larger_buffer(dev, devbuf, t):
 
 
 @pytest.mark.parametrize("t", TYPES)
+@pytest.mark.parametrize("form", ["multi", "gather", "gather_act"])
+def test_matvec_packed_multi_over_expert_sheets(dev, devbuf, t, form):
+    """MatVecPackedMulti / Gather / GatherAct (/root/reference/engine/nn/packedmulti.go:24,84,93)
+    over the sheets of an expert bank packed as ONE set of planes: every matrix has the bank's
+    plane pointers and row0 = expert * rows, the addressing of an expert page
+    (/root/reference/engine/nn/device.go:70-80).  One launch; each matrix is the packed matvec."""
+    n_expert, nrows, k, window = 6, 90, 1024, _window(t)
+    experts = [4, 0, 5, 2]
+    dev.SetActWindow(window)
+    bank = synth.random_weights(t, n_expert * nrows, k, seed=31)
+    planes = _dev_planes(devbuf, *oracle.pack_weights(t, bank, n_expert * nrows, k), stride=n_expert * nrows)
+    m = len(experts)
+    xs = np.stack([synth.activations(k, seed=60 + j) for j in range(m)])
+    ups = np.stack([synth.activations(k, seed=80 + j) for j in range(m)])
+    if form == "multi":
+        xs = np.repeat(xs[:1], m, axis=0)
+    xd, ud = devbuf(xs), devbuf(ups)
+    outs = [devbuf(shape=(nrows + 2,), dtype=np.float32, fill=np.float32(9e30)) for _ in range(m)]
+    rb = quant.row_bytes(t, k)
+    for rw in (0, 16, 64):
+        dev.set_tuning(packed__rw=rw)
+        assert dev.matvec_packed_multi_dev([o.ptr for o in outs], t, [(planes.qs, planes.d, planes.sc)] * m,
+                                           [e * nrows for e in experts], n_expert * nrows, xd.ptr,
+                                           0 if form == "multi" else k, ud.ptr if form == "gather_act" else None,
+                                           nrows, k)
+        dev.synchronize()
+        for j, e in enumerate(experts):
+            w = bank[e * nrows * rb:(e + 1) * nrows * rb]
+            got = outs[j].get()
+            assert np.all(got[nrows:] == np.float32(9e30))
+            if form == "gather_act":
+                g = xs[j].astype(np.float64)
+                h = (g / (1 + np.exp(-g)) * ups[j].astype(np.float64)).astype(np.float32)
+                assert rel_l2(got[:nrows], _like_for_like(t, w, h, nrows, k, window)) <= 1e-3
+            else:
+                assert nmse(got[:nrows], _like_for_like(t, w, xs[j], nrows, k, window)) <= 1e-10
+    dev.set_tuning(packed__rw=0)
+    dev.SetActWindow(32)
+
+
+@pytest.mark.parametrize("t", TYPES)
 def test_matvec_packed_split_equals_fused(dev, devbuf, t):
     """Quantizer kernel + packed matvec over its output == the fused kernel, bit for bit."""
     nrows, k, window = 200, 4096, _window(t)
