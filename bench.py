@@ -293,6 +293,70 @@ def moe_section(dev):
             "TFLOP/s": round(rows * k_used * 3 * 2.0 * n_ffn * n_embd / (ms * 1e-3) / 1e12, 2)}
 
 
+def moe_decode_section(dev):
+    """The same mixture at decode: one token, its eight experts.  The three banks are packed
+    planes on the device (one set per bank, as a .jlm file holds them); gate and up of the eight
+    experts are ONE launch of sixteen packed matvecs sharing x, the eight down projections one
+    launch over silu(gate) * up.  Every step takes another eight experts, so the sheets come
+    from memory.  Bytes = 24 sheets + activations."""
+    from jitllm_amd import quant, synth
+    from jitllm_amd.hipmem import DeviceArray, Event
+    t, n_expert, k_used, n_ffn, n_embd = quant.Q4_K, 128, 8, 768, 2048
+    dev.SetActWindow(256)
+    planes = []
+    for i, (r, k) in enumerate([(n_ffn, n_embd), (n_ffn, n_embd), (n_embd, n_ffn)]):
+        src = DeviceArray(synth.quantized_weights(t, r * n_expert, k, seed=10 + i))
+        nq, nd, nsc = dev.packed_words(t, r * n_expert, k)
+        pl = [DeviceArray(shape=(n,), dtype=np.uint32, fill=0) for n in (nq, nd, nsc)]
+        if not dev.pack_weights_dev(t, src.ptr, r * n_expert, k, pl[0].ptr, pl[1].ptr, pl[2].ptr):
+            raise RuntimeError("the device declined to pack a bank")
+        dev.synchronize()
+        src.free()
+        planes.append(pl)
+    x = DeviceArray(synth.activations(n_embd, seed=4))
+    gu = [DeviceArray(shape=(n_ffn,), dtype=np.float32, fill=0) for _ in range(2 * k_used)]   # gate 0..7, up 8..15
+    g = DeviceArray(shape=(k_used, n_ffn), dtype=np.float32, fill=0)
+    u = DeviceArray(shape=(k_used, n_ffn), dtype=np.float32, fill=0)
+    ys = [DeviceArray(shape=(n_embd,), dtype=np.float32, fill=0) for _ in range(k_used)]
+    rng = np.random.default_rng(1)
+    picks = [sorted(rng.choice(n_expert, k_used, replace=False).tolist()) for _ in range(32)]
+    gp = [(planes[0][0].ptr, planes[0][1].ptr, planes[0][2].ptr)] * k_used + \
+         [(planes[1][0].ptr, planes[1][1].ptr, planes[1][2].ptr)] * k_used
+    dp = [(planes[2][0].ptr, planes[2][1].ptr, planes[2][2].ptr)] * k_used
+    gouts = [g.ptr + j * n_ffn * 4 for j in range(k_used)] + [u.ptr + j * n_ffn * 4 for j in range(k_used)]
+
+    # argument blocks are built once per expert set: the timed loop is two library calls a step
+    calls = [(dev.packed_multi_args(gouts, t, gp, [e * n_ffn for e in ex] * 2, n_expert * n_ffn, x.ptr, 0, None,
+                                    n_ffn, n_embd),
+              dev.packed_multi_args([y.ptr for y in ys], t, dp, [e * n_embd for e in ex], n_expert * n_embd,
+                                    g.ptr, n_ffn, u.ptr, n_embd, n_ffn)) for ex in picks]
+
+    def run(i):
+        a, b = calls[i % len(calls)]
+        if not (dev.packed_multi_call(a) and dev.packed_multi_call(b)):
+            raise RuntimeError("the device declined the decode mixture")
+    for i in range(4):
+        run(i)
+    dev.synchronize()
+    e0, e1, n = Event(), Event(), 64
+    e0.record(dev.stream)
+    for i in range(n):
+        run(i)
+    e1.record(dev.stream)
+    e1.synchronize()
+    ms = e0.elapsed_ms(e1) / n
+    sheet = n_ffn * quant.row_bytes(t, n_embd)
+    nbytes = 3 * k_used * sheet + 4 * n_embd + 4 * (4 * k_used * n_ffn) + 4 * k_used * n_embd
+    for pl in planes:
+        for b in pl:
+            b.free()
+    for b in [x, g, u] + gu + ys:
+        b.free()
+    return {"us_per_step": round(ms * 1e3, 2), "launches_per_step": 2, "bytes_per_step": nbytes,
+            "GB/s": round(nbytes / (ms * 1e-3) / 1e9, 1),
+            "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+
+
 def mxfp4_section(dev):
     """gpt-oss-20B expert shape: MXFP4 2880x2880, bf16 activations, tokens 1 / 64 / 1024."""
     from jitllm_amd import quant, synth
@@ -336,7 +400,7 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="headline workload only")
     ap.add_argument("--gemm", metavar="NTOK,NROWS", help="only the prefill GEMM of this shape (k = 4096), "
                     "for profiling one kernel; prints its section alone")
-    ap.add_argument("--section", choices=["mxfp4", "moe", "ffn"], help="only this section of the default run, for "
+    ap.add_argument("--section", choices=["mxfp4", "moe", "moe_decode", "ffn"], help="only this section of the default run, for "
                     "profiling its kernels; prints the section alone")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -352,7 +416,7 @@ def main():
         dev.close()
         return
     if args.section:
-        fn = {"mxfp4": mxfp4_section, "moe": moe_section, "ffn": ffn_section}[args.section]
+        fn = {"mxfp4": mxfp4_section, "moe": moe_section, "moe_decode": moe_decode_section, "ffn": ffn_section}[args.section]
         print(json.dumps({args.section: fn(dev)}), flush=True)
         dev.close()
         return
@@ -400,6 +464,7 @@ def main():
         line["ffn_block_decode"] = ffn_section(dev)
         line["prefill_gemm"] = gemm_section(dev)
         line["moe_block"] = moe_section(dev)
+        line["moe_decode"] = moe_decode_section(dev)
         line["mxfp4_gemm"] = mxfp4_section(dev)
 
     if not args.no_cpu:

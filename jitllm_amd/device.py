@@ -207,14 +207,21 @@ class Device:
     def matvec_packed_multi_dev(self, outs, t, planes, row0, stride, x, xstride, up, nrows, k, stream=None):
         """MatVecPackedMulti / Gather / GatherAct over packed planes: planes is a list of
         (qs, d, sc) device pointers, row0 the first row of each matrix in its buffer."""
+        return self.packed_multi_call(self.packed_multi_args(outs, t, planes, row0, stride, x, xstride, up,
+                                                             nrows, k), stream)
+
+    def packed_multi_args(self, outs, t, planes, row0, stride, x, xstride, up, nrows, k):
+        """The argument block of a packed multi call, built once by a caller that repeats it."""
         m = len(outs)
         po = (C.c_void_p * m)(*[_ptr(o) for o in outs])
         pq = (C.c_void_p * m)(*[_ptr(p[0]) for p in planes])
         pd = (C.c_void_p * m)(*[_ptr(p[1]) for p in planes])
         ps = (C.c_void_p * m)(*[_opt(p[2]) for p in planes])
         pr = (C.c_int * m)(*row0)
-        return self._served(self._l.jl_matvec_packed_multi_dev(self._ctx, po, t, pq, pd, ps, pr, stride, _ptr(x),
-                                                               xstride, _opt(up), nrows, k, m, stream),
+        return (po, t, pq, pd, ps, pr, stride, _ptr(x), xstride, _opt(up), nrows, k, m)
+
+    def packed_multi_call(self, args, stream=None):
+        return self._served(self._l.jl_matvec_packed_multi_dev(self._ctx, *args, stream),
                             "jl_matvec_packed_multi_dev")
 
     def matmul_dev(self, out, t, w, x, nrows, k, ntok, stream=None):
