@@ -47,6 +47,50 @@
 // + 1e-20).  The f64 sum is taken as a butterfly over the lanes, so it can differ from the
 // reference's sequential sum in its last bit; after narrowing to f32 that moves a score
 // only when it sits on a rounding boundary.
+// Reductions over the 64 lanes by DPP lane moves (a shuffle through the LDS crossbar costs
+// ~100 cycles and the router is a chain of them): quad swaps, the two row mirrors, then
+// row broadcasts; lane 63 ends up with the result and it is read back as a scalar.
+#define JL_ROUTE_STEPS(STEP)                                                                         \
+    STEP(JL_DPP_QUAD_XOR1, 0xf) STEP(JL_DPP_QUAD_XOR2, 0xf) STEP(JL_DPP_ROW_HALF_MIRROR, 0xf)        \
+    STEP(JL_DPP_ROW_MIRROR, 0xf) STEP(JL_DPP_ROW_BCAST15, 0xa) STEP(JL_DPP_ROW_BCAST31, 0xc)
+
+__device__ __forceinline__ float route_wave_max(float v) {
+    const i32 ninf = __builtin_bit_cast(i32, -__builtin_inff());
+#define STEP(C, M) v = fmaxf(v, __builtin_bit_cast(float, dpp_i32<C, M>(ninf, __builtin_bit_cast(i32, v))));
+    JL_ROUTE_STEPS(STEP)
+#undef STEP
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(i32, v), 63));
+}
+
+__device__ __forceinline__ double route_wave_sum(double v) {
+#define STEP(C, M)                                                                                   \
+    {                                                                                                \
+        const uint64_t b = __builtin_bit_cast(uint64_t, v);                                                    \
+        const u32 lo = (u32)dpp_i32<C, M>(0, (i32)(u32)b), hi = (u32)dpp_i32<C, M>(0, (i32)(u32)(b >> 32)); \
+        v += __builtin_bit_cast(double, ((uint64_t)hi << 32) | lo);                                       \
+    }
+    JL_ROUTE_STEPS(STEP)
+#undef STEP
+    const uint64_t b = __builtin_bit_cast(uint64_t, v);
+    const u32 lo = (u32)__builtin_amdgcn_readlane((i32)(u32)b, 63), hi = (u32)__builtin_amdgcn_readlane((i32)(u32)(b >> 32), 63);
+    return __builtin_bit_cast(double, ((uint64_t)hi << 32) | lo);
+}
+
+// (key, index) of the largest key, lowest index on a tie; key = -1 where a lane has none.
+__device__ __forceinline__ void route_wave_argmax(i32& key, i32& idx) {
+#define STEP(C, M)                                                                                   \
+    {                                                                                                \
+        const i32 ok = dpp_i32<C, M>(-1, key), oi = dpp_i32<C, M>(0x7fffffff, idx);                  \
+        const bool take = ok > key || (ok == key && oi < idx);                                       \
+        key = take ? ok : key;                                                                       \
+        idx = take ? oi : idx;                                                                       \
+    }
+    JL_ROUTE_STEPS(STEP)
+#undef STEP
+    key = __builtin_amdgcn_readlane(key, 63);
+    idx = __builtin_amdgcn_readlane(idx, 63);
+}
+
 __device__ __forceinline__ void moe_route_body(const MoeRouteArgs& p) {
     const int lane = threadIdx.x & 63, n = p.n_expert;
     const size_t row = blockIdx.x;
@@ -56,58 +100,55 @@ __device__ __forceinline__ void moe_route_body(const MoeRouteArgs& p) {
 #pragma unroll
     for (int i = 0; i < 16; i++) {
         const int e = lane + 64 * i;
-        v[i] = e < n ? lg[e] : -__builtin_inff();
+        v[i] = e < n ? lg[min(e, n - 1)] : -__builtin_inff();
         if (v[i] > mx) mx = v[i];
     }
-#pragma unroll
-    for (int m = 1; m < 64; m <<= 1) mx = fmaxf(mx, __shfl_xor(mx, m, 64));
+    mx = route_wave_max(mx);
     double sum = 0.0;
     float sc[16];
 #pragma unroll
     for (int i = 0; i < 16; i++) {
         const int e = lane + 64 * i;
-        double ex = e < n ? exp((double)v[i] - (double)mx) : 0.0;
+        double ex = 0.0;
+        if (64 * i < n) ex = e < n ? exp((double)v[i] - (double)mx) : 0.0;   // (uniform: whole groups of 64 past n are skipped)
         sc[i] = (float)ex;
         sum += ex;
     }
-    sum = wave_sum_f64(sum);
+    sum = route_wave_sum(sum);
     const double inv = 1.0 / sum;
 #pragma unroll
     for (int i = 0; i < 16; i++) sc[i] = (float)((double)sc[i] * inv);
 
-    float prev_val = 0.f, total = 0.f;
-    int prev_idx = -1;
-    float chosen[16];
+    // Scores are >= 0, so their bit patterns order as integers; -1 marks "none".
+    i32 prev_key = 0, prev_idx = -1;
+    float total = 0.f;
+    float chosen = 0.f;   // lane r keeps the r-th selected score
     int found = 0;
     for (int r = 0; r < p.k_used && r < 16; r++) {
         // this lane's best eligible score (index ascending within a lane, so the first
         // of equal values is kept)
-        float bv = -1.f;
-        int bi = 0x7fffffff;
+        i32 bk = -1, bi = 0x7fffffff;
 #pragma unroll
         for (int i = 0; i < 16; i++) {
+            if (64 * i >= n) continue;   // uniform
             const int e = lane + 64 * i;
             const float x = sc[i];
-            const bool ok = e < n && x == x && (r == 0 || x < prev_val || (x == prev_val && e > prev_idx));
-            if (ok && (x > bv)) { bv = x; bi = e; }
+            const i32 xk = __builtin_bit_cast(i32, x);
+            const bool ok = e < n && x == x && (r == 0 || xk < prev_key || (xk == prev_key && e > prev_idx));
+            if (ok && xk > bk) { bk = xk; bi = e; }
         }
-#pragma unroll
-        for (int m = 1; m < 64; m <<= 1) {
-            const float ov = __shfl_xor(bv, m, 64);
-            const int oi = __shfl_xor(bi, m, 64);
-            if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
-        }
+        route_wave_argmax(bk, bi);
         if (bi == 0x7fffffff) break;
         if (lane == 0) p.sel[row * p.sel_stride + r] = (u32)bi;
-        chosen[r] = bv;
-        prev_val = bv;
+        const float bv = __builtin_bit_cast(float, bk);
+        if (lane == r) chosen = bv;
+        total = total + bv;          // selection order, as the reference adds them
+        prev_key = bk;
         prev_idx = bi;
         found = r + 1;
     }
-    for (int r = 0; r < found; r++) total = total + chosen[r];
     total = total + 1e-20f;
-    if (lane == 0)
-        for (int r = 0; r < found; r++) p.wt[row * p.k_used + r] = chosen[r] / total;
+    if (lane < found) p.wt[row * p.k_used + lane] = chosen / total;
 }
 
 // ------------------------------------------------------------------ grouping
