@@ -35,6 +35,7 @@ struct Tuning {
     int gemm_split = 0;
     int moe_form = 0;
     int moe_waves = 0;
+    int moe_lpr = 0;
     int mx_split = 0;
 };
 
@@ -658,8 +659,20 @@ int moe_matvec_launch(jl_ctx* c, float* out0, float* out1, int type, const void*
         return JL_OK;
     }
     const int nslots = k / ti->slot_elems;
-    int lpr = 16;
-    while (lpr < 64 && lpr < nslots) lpr <<= 1;
+    // lanes per row: the width that leaves the fewest lanes without a slot (a row of 12 slots
+    // on 16 lanes idles a quarter of them; on 4 lanes, three slots each, none); among equals
+    // eight lanes, several slots a lane, measured best (sweeps at the 128-expert shape);
+    // tuning "moe.lpr" overrides
+    int lpr = 64, waste = 1 << 30;
+    for (int cand : {8, 16, 4, 32, 64}) {
+        const int w = (nslots + cand - 1) / cand * cand - nslots;
+        if (w < waste) { waste = w; lpr = cand; }
+    }
+    {
+        // (100 * a + b: a for rows of more than 16 slots, b for shorter ones)
+        const int tl = c->tune.moe_lpr > 64 ? (nslots > 16 ? c->tune.moe_lpr / 100 : c->tune.moe_lpr % 100) : c->tune.moe_lpr;
+        if (tl == 4 || tl == 8 || tl == 16 || tl == 32 || tl == 64) lpr = tl;
+    }
     const size_t act = ((size_t)k + (size_t)(k / 32) * 4 + (size_t)(k / 16) * 4 + 15) & ~(size_t)15;
     const size_t lds = 8 * act;
     if (lds > c->lds_limit) return JL_DECLINED;
@@ -756,7 +769,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
             for (const char* form : {"", "q8_"})
                 names.push_back(std::string("jl_matvec_packed_") + form + tag + "_w" + std::to_string(rw));
     for (const char* tag : {"q4k", "q8_0", "q6k"})
-        for (int lpr : {16, 32, 64}) names.push_back(std::string("jl_moe_matvec_") + tag + "_l" + std::to_string(lpr));
+        for (int lpr : {4, 8, 16, 32, 64}) names.push_back(std::string("jl_moe_matvec_") + tag + "_l" + std::to_string(lpr));
     const int types[] = {JL_TYPE_Q4_K, JL_TYPE_Q8_0, JL_TYPE_Q6_K};
     for (int t : types)
         for (int rpw : {1, 2, 4}) {
@@ -833,6 +846,7 @@ int jl_set_tuning(jl_ctx* c, const char* key, int value) {
     else if (!strcmp(key, "moe.shares")) c->tune.moe_shares = value;
     else if (!strcmp(key, "moe.form")) c->tune.moe_form = value;
     else if (!strcmp(key, "moe.waves")) c->tune.moe_waves = value;
+    else if (!strcmp(key, "moe.lpr")) c->tune.moe_lpr = value;
     else if (!strcmp(key, "gemm.rows")) c->tune.gemm_rows = value;
     else if (!strcmp(key, "mxfp4.split")) c->tune.mx_split = value;
     else if (!strcmp(key, "gemm.form")) c->tune.gemm_form = value;

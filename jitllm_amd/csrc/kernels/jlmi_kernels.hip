@@ -126,8 +126,11 @@ extern "C" __global__ __launch_bounds__(256) void jl_moe_quant(MoeQuantArgs p) {
     extern "C" __global__ __launch_bounds__(512) void jl_moe_matvec_##T##_l##LPR(MoeMatVecArgs p) { \
         moe_matvec_body<TYPE, LPR>(p, jl_smem);                                                   \
     }
+JL_MOE_KERNEL(q4k, JL_Q4_K, 4) JL_MOE_KERNEL(q4k, JL_Q4_K, 8)
 JL_MOE_KERNEL(q4k, JL_Q4_K, 16) JL_MOE_KERNEL(q4k, JL_Q4_K, 32) JL_MOE_KERNEL(q4k, JL_Q4_K, 64)
+JL_MOE_KERNEL(q8_0, JL_Q8_0, 4) JL_MOE_KERNEL(q8_0, JL_Q8_0, 8)
 JL_MOE_KERNEL(q8_0, JL_Q8_0, 16) JL_MOE_KERNEL(q8_0, JL_Q8_0, 32) JL_MOE_KERNEL(q8_0, JL_Q8_0, 64)
+JL_MOE_KERNEL(q6k, JL_Q6_K, 4) JL_MOE_KERNEL(q6k, JL_Q6_K, 8)
 JL_MOE_KERNEL(q6k, JL_Q6_K, 16) JL_MOE_KERNEL(q6k, JL_Q6_K, 32) JL_MOE_KERNEL(q6k, JL_Q6_K, 64)
 // grid = (ceil(n_embd/256), rows), block = 256
 extern "C" __global__ __launch_bounds__(256) void jl_moe_combine(MoeCombineArgs p) { moe_combine_body(p); }

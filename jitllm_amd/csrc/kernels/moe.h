@@ -233,8 +233,8 @@ template <int LPR>
 __device__ __forceinline__ float group_sum(float v) {
     v += dpp_f32<JL_DPP_QUAD_XOR1, 0xf>(v);
     v += dpp_f32<JL_DPP_QUAD_XOR2, 0xf>(v);
-    v += dpp_f32<JL_DPP_ROW_HALF_MIRROR, 0xf>(v);
-    v += dpp_f32<JL_DPP_ROW_MIRROR, 0xf>(v);
+    if (LPR >= 8) v += dpp_f32<JL_DPP_ROW_HALF_MIRROR, 0xf>(v);
+    if (LPR >= 16) v += dpp_f32<JL_DPP_ROW_MIRROR, 0xf>(v);
     if (LPR >= 32) v += dpp_f32<JL_DPP_ROW_BCAST15, 0xa>(v);
     if (LPR >= 64) v += dpp_f32<JL_DPP_ROW_BCAST31, 0xc>(v);
     return v;

@@ -93,10 +93,13 @@ def test_grouped_matvec_vs_oracle(dev, devbuf, t, nrows, k, form):
     dstart, dperm = devbuf(start), devbuf(perm[:used].copy())
     o0 = devbuf(shape=(used, nrows), dtype=np.float32, fill=np.float32(4e30))
     o1 = devbuf(shape=(used, nrows), dtype=np.float32, fill=np.float32(4e30))
-    assert dev.moe_matvec_dev(o0.ptr, o1.ptr, t, b0.ptr, b1.ptr, xd.ptr, None, dperm.ptr, dstart.ptr,
-                              n_expert, used, nrows, k)
-    dev.synchronize()
-    assert nmse(o0.get(), want0) <= 1e-10 and nmse(o1.get(), want1) <= 1e-10
+    for lpr in (0, 4, 16, 32, 64):     # lanes per row: the library's pick, then every other width
+        dev.set_tuning(moe__lpr=lpr)
+        assert dev.moe_matvec_dev(o0.ptr, o1.ptr, t, b0.ptr, b1.ptr, xd.ptr, None, dperm.ptr, dstart.ptr,
+                                  n_expert, used, nrows, k)
+        dev.synchronize()
+        assert nmse(o0.get(), want0) <= 1e-10 and nmse(o1.get(), want1) <= 1e-10, lpr
+    dev.set_tuning(moe__lpr=0)
     # SwiGLU form: column c reads silu(x[c]) * x2[c], no gather
     g = np.stack([synth.activations(k, seed=300 + c) for c in range(used)])
     u = np.stack([synth.activations(k, seed=400 + c) for c in range(used)])
