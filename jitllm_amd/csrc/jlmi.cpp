@@ -36,6 +36,7 @@ struct Tuning {
     int moe_form = 0;
     int moe_waves = 0;
     int moe_lpr = 0;
+    int mx_rows = 0;
     int mx_split = 0;
 };
 
@@ -762,7 +763,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     if (e != hipSuccess)
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
-    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_q4k_r64", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_moe_route", "jl_moe_group", "jl_moe_quant", "jl_moe_combine", "jl_moe_gemm_prep", "jl_moe_gemm_q4k", "jl_mxfp4_prep", "jl_mxfp4_gemm", "jl_mxfp4_matvec", "jl_sum_parts",
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_q4k_r64", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_moe_route", "jl_moe_group", "jl_moe_quant", "jl_moe_combine", "jl_moe_gemm_prep", "jl_moe_gemm_q4k", "jl_mxfp4_prep", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_sum_parts",
                                       "jl_pack_weights", "jl_unpack_q4k"};
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int rw : {16, 32, 64})
@@ -849,6 +850,7 @@ int jl_set_tuning(jl_ctx* c, const char* key, int value) {
     else if (!strcmp(key, "moe.lpr")) c->tune.moe_lpr = value;
     else if (!strcmp(key, "gemm.rows")) c->tune.gemm_rows = value;
     else if (!strcmp(key, "mxfp4.split")) c->tune.mx_split = value;
+    else if (!strcmp(key, "mxfp4.rows")) c->tune.mx_rows = value;
     else if (!strcmp(key, "gemm.form")) c->tune.gemm_form = value;
     else if (!strcmp(key, "gemm.split")) c->tune.gemm_split = value;
     else if (!strcmp(key, "gemm.min_tok")) c->gemm_min_tok = value > 0 ? value : 8;
@@ -1165,7 +1167,16 @@ int jl_matmul_mxfp4_bf16_dev(jl_ctx* c, float* out, const void* w, const uint16_
     a.x = (const uint16_t*)c->gemm_ws; a.tok_pad = tok_pad;
     // A grid that leaves most CUs idle is widened along K: each split writes partial sums
     // to a workspace slab and a second kernel adds the slabs in order.
-    const int tiles = (tok_pad / 128) * ((nrows + 127) / 128);
+    // rows per tile: 128, or 96 where that takes fewer rounds x rows (2880 rows x 1024 tokens:
+    // 184 tiles of 128 rows leave 72 CUs idle for a whole tile, 240 of 96 rows do not)
+    auto cost = [&](int rows) {
+        const long t = (long)(tok_pad / 128) * ((nrows + rows - 1) / rows);
+        return ((t + c->num_cu - 1) / c->num_cu) * rows;
+    };
+    const int trows = c->tune.mx_rows == 96 || c->tune.mx_rows == 128 ? c->tune.mx_rows
+                      : (cost(96) < cost(128) ? 96 : 128);
+    const char* gemm_name = trows == 96 ? "jl_mxfp4_gemm_r96" : "jl_mxfp4_gemm";
+    const int tiles = (tok_pad / 128) * ((nrows + trows - 1) / trows);
     int nsplit = c->tune.mx_split > 0 ? c->tune.mx_split : (tiles * 2 <= c->num_cu ? c->num_cu / tiles : 1);
     if (nsplit > 8) nsplit = 8;
     if (nsplit > stages) nsplit = stages;
@@ -1178,15 +1189,15 @@ int jl_matmul_mxfp4_bf16_dev(jl_ctx* c, float* out, const void* w, const uint16_
         rc = ws_ensure(c, &c->mx_ws, &c->mx_ws_bytes, n * nsplit * 4);
         if (rc != JL_OK) return rc;
         a.nsplit = nsplit; a.part = (float*)c->mx_ws;
-        HIP_TRY(c, H->ModuleLaunchKernel(c->fn["jl_mxfp4_gemm"], (unsigned)(tok_pad / 128),
-                                         (unsigned)((nrows + 127) / 128), (unsigned)nsplit, 512, 1, 1, lds, st,
+        HIP_TRY(c, H->ModuleLaunchKernel(c->fn[gemm_name], (unsigned)(tok_pad / 128),
+                                         (unsigned)((nrows + trows - 1) / trows), (unsigned)nsplit, 512, 1, 1, lds, st,
                                          params, nullptr));
         SumPartsArgs sa;
         sa.out = out; sa.part = a.part; sa.n = n; sa.nsplit = nsplit;
         void* sp[] = {&sa};
         return launch(c, "jl_sum_parts", (unsigned)((n + 255) / 256), 1, 256, 0, st, sp);
     }
-    return launch(c, "jl_mxfp4_gemm", (unsigned)((ntok + 127) / 128), (unsigned)((nrows + 127) / 128), 512,
+    return launch(c, gemm_name, (unsigned)(tok_pad / 128), (unsigned)((nrows + trows - 1) / trows), 512,
                   lds, st, params);
 }
 

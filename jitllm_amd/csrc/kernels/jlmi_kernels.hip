@@ -146,7 +146,8 @@ extern "C" __global__ __launch_bounds__(256) void jl_moe_gemm_prep(MoeGemmPrepAr
     moe_gemm_prep_body(p, lds);
 }
 extern "C" __global__ __launch_bounds__(256, 2) void jl_moe_gemm_q4k(MoeGemmArgs p) { moe_gemm_q4k_body(p, jl_smem); }
-extern "C" __global__ __launch_bounds__(512) void jl_mxfp4_gemm(MxGemmArgs p) { mx_gemm_body(p, jl_smem); }
+extern "C" __global__ __launch_bounds__(512) void jl_mxfp4_gemm(MxGemmArgs p) { mx_gemm_body<4>(p, jl_smem); }
+extern "C" __global__ __launch_bounds__(512) void jl_mxfp4_gemm_r96(MxGemmArgs p) { mx_gemm_body<3>(p, jl_smem); }
 extern "C" __global__ __launch_bounds__(256) void jl_sum_parts(SumPartsArgs p) { sum_parts_body(p); }
 // grid = ceil(nrows/4), block = 256: one wavefront per row, ntok <= 8
 extern "C" __global__ __launch_bounds__(256) void jl_mxfp4_matvec(MxGemmArgs p) { mx_matvec_body(p); }

@@ -109,23 +109,27 @@ __device__ __forceinline__ void mx_load_w(const MxGemmArgs& p, int r0, int wave,
     }
 }
 
-// grid = (tok_pad/128, ceil(nrows/128), nsplit), block = 512, dynamic LDS = two weight
-// stages [128][264] bf16.  The shape this serves (a few thousand rows, a thousand tokens)
-// gives fewer 128 x 128 tiles than the chip has CUs, so a tile gets EIGHT wavefronts, two
-// per SIMD to cover each other's waits: wavefront (tg, kh) owns 32 tokens x all 128 rows
-// (four 32 x 32 accumulators) over the K-steps of parity kh, and the two parities are
-// added through LDS at the end, kh = 0 first.  Activation fragments come from the prepared
-// workspace into a register ring a stage ahead (1 KiB coalesced loads), each feeding four
-// matrix instructions; all eight wavefronts share one decode of the weights through LDS.
-// A stage (256 K) is 16 slots of two matrix instructions per wavefront with the weight
-// fragments fetched three slots ahead and the next stage's weights decoded half a block
-// at a time in between, their registers loaded two stages ahead.
+// grid = (tok_pad/128, ceil(nrows/(32*NJ)), nsplit), block = 512, dynamic LDS = two weight
+// stages [128][264] bf16.  NJ = 4: 128 tokens x 128 rows a workgroup; NJ = 3: 128 x 96, for
+// shapes whose 128-row tiles would leave a quarter of the CUs without one (2880 rows x 1024
+// tokens: 184 tiles of 128 rows, 240 of 96).  The shape this serves gives about as many
+// tiles as the chip has CUs, so a tile gets EIGHT wavefronts, two per SIMD to cover each
+// other's waits: wavefront (tg, kh) owns 32 tokens x all 32*NJ rows (NJ 32 x 32
+// accumulators) over the K-steps of parity kh, and the two parities are added through LDS
+// at the end, kh = 0 first.  Activation fragments come from the prepared workspace into a
+// register ring a stage ahead (1 KiB coalesced loads), each feeding NJ matrix
+// instructions; all eight wavefronts share one decode of the weights through LDS.  A stage
+// (256 K) is 8*NJ matrix instructions per wavefront with their weight fragments fetched six
+// instructions ahead and the next stage's weights decoded half a block at a time in
+// between, their registers loaded two stages ahead.
+template <int NJ>
 __device__ __forceinline__ void mx_gemm_body(const MxGemmArgs& p, uint8_t* smem) {
+    constexpr int ROWS = 32 * NJ, UNITS = 8 * NJ, AHEAD = 6;
     __bf16* sW = (__bf16*)smem;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int tg = wave & 3, kh = wave >> 2;
-    const int t0 = blockIdx.x * JL_MX_TILE, r0 = blockIdx.y * JL_MX_TILE;
+    const int t0 = blockIdx.x * JL_MX_TILE, r0 = blockIdx.y * ROWS;
     // a small grid is widened along K: workgroup z takes a contiguous run of the K
     // stages and writes its partial sums to its own slab, summed afterwards in order
     const int all_stages = (p.k + JL_MX_KSTAGE - 1) / JL_MX_KSTAGE;
@@ -140,12 +144,13 @@ __device__ __forceinline__ void mx_gemm_body(const MxGemmArgs& p, uint8_t* smem)
     auto a_frag = [&](int stage, int ks2) {
         return *(const bf16x8*)(abase + (size_t)stage * astride + ks2 * 2048 + aoff);
     };
-    // where this thread's decoded blocks go in a stage buffer
+    // this wavefront decodes rows 16*wave .. 16*wave+15 of the tile (none if the tile is shorter)
+    const bool decodes = wave * 16 < ROWS;   // uniform
     const int wdst = (wave * 16 + (lane >> 3)) * JL_MX_STRIDE + (lane & 7) * 32;
 
-    f32x16_t acc[4];
+    f32x16_t acc[NJ];
 #pragma unroll
-    for (int j = 0; j < 4; j++)
+    for (int j = 0; j < NJ; j++)
 #pragma unroll
         for (int e = 0; e < 16; e++) acc[j][e] = 0.f;
 
@@ -161,15 +166,17 @@ __device__ __forceinline__ void mx_gemm_body(const MxGemmArgs& p, uint8_t* smem)
     MxWRegs wa, wb;
     bf16x8 aring[8];
     const int last = max(s_hi - 1, s_lo);
-    mx_load_w(p, r0, wave, lane, s_lo, wa);
+    if (decodes) mx_load_w(p, r0, wave, lane, s_lo, wa);
 #pragma unroll
     for (int ks2 = 0; ks2 < 8; ks2++) aring[ks2] = a_frag(s_lo, ks2);
+    if (decodes) {
 #pragma unroll
-    for (int i = 0; i < 2; i++) {
-        decode_half(wa, i, 0, sW);
-        decode_half(wa, i, 1, sW);
+        for (int i = 0; i < 2; i++) {
+            decode_half(wa, i, 0, sW);
+            decode_half(wa, i, 1, sW);
+        }
+        mx_load_w(p, r0, wave, lane, min(s_lo + 1, last), wa);
     }
-    mx_load_w(p, r0, wave, lane, min(s_lo + 1, last), wa);
     mx_lds_barrier();
 
     auto stage = [&](auto BUF, int st, MxWRegs& wcur, MxWRegs& wnxt) {
@@ -177,33 +184,26 @@ __device__ __forceinline__ void mx_gemm_body(const MxGemmArgs& p, uint8_t* smem)
         const __bf16* w = sW + buf * JL_MX_STAGE_ELEMS;
         __bf16* wnext = sW + (buf ^ 1) * JL_MX_STAGE_ELEMS;
         const int nst = min(st + 1, last);
-        mx_load_w(p, r0, wave, lane, min(st + 2, last), wnxt);
+        if (decodes) mx_load_w(p, r0, wave, lane, min(st + 2, last), wnxt);
         const __bf16* wp0 = w + arow * JL_MX_STRIDE + 8 * kg + 16 * kh;
-        auto w_frag = [&](int slot, int j) {
-            return *(const bf16x8*)(wp0 + 32 * (2 * (slot & 1) + j) * JL_MX_STRIDE + 32 * (slot >> 1));
+        // unit u = matrix instruction (K-step u / NJ, row tile u % NJ)
+        auto w_frag = [&](int u) {
+            return *(const bf16x8*)(wp0 + 32 * (u % NJ) * JL_MX_STRIDE + 32 * (u / NJ));
         };
-        bf16x8 wf[4][2];
+        bf16x8 wf[8];
 #pragma unroll
-        for (int s3 = 0; s3 < 3; s3++)
-#pragma unroll
-            for (int j = 0; j < 2; j++) wf[s3][j] = w_frag(s3, j);
+        for (int u = 0; u < AHEAD; u++) wf[u] = w_frag(u);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int slot = 0; slot < 16; slot++) {
-            const int ks2 = slot >> 1, jh = slot & 1;
-            if (slot + 3 < 16) {
-#pragma unroll
-                for (int j = 0; j < 2; j++) wf[(slot + 3) & 3][j] = w_frag(slot + 3, j);
-            }
+        for (int u = 0; u < UNITS; u++) {
+            const int ks2 = u / NJ, j = u % NJ;
+            if (u + AHEAD < UNITS) wf[(u + AHEAD) & 7] = w_frag(u + AHEAD);
             __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int j = 0; j < 2; j++)
-                acc[2 * jh + j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aring[ks2], wf[slot & 3][j],
-                                                                         acc[2 * jh + j], 0, 0, 0);
-            if (jh == 1) {
+            acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aring[ks2], wf[u & 7], acc[j], 0, 0, 0);
+            if (j == NJ - 1) {
                 aring[ks2] = a_frag(nst, ks2);
                 // half a block of the next stage's weights in every second K-step
-                if (ks2 & 1) decode_half(wcur, ks2 >> 2, (ks2 >> 1) & 1, wnext);
+                if (decodes && (ks2 & 1)) decode_half(wcur, ks2 >> 2, (ks2 >> 1) & 1, wnext);
             }
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -215,17 +215,17 @@ __device__ __forceinline__ void mx_gemm_body(const MxGemmArgs& p, uint8_t* smem)
     }
 
     // the two K parities meet in LDS (the weight stages are done with): [tg][tile][16][64] f32
-    float* sAcc = (float*)smem + (size_t)tg * (4 * 16 * 64) + lane;
+    float* sAcc = (float*)smem + (size_t)tg * (NJ * 16 * 64) + lane;
     if (kh == 1) {
 #pragma unroll
-        for (int j = 0; j < 4; j++)
+        for (int j = 0; j < NJ; j++)
 #pragma unroll
             for (int e = 0; e < 16; e++) sAcc[(j * 16 + e) * 64] = acc[j][e];
     }
     __syncthreads();
     if (kh == 1) return;
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
+    for (int j = 0; j < NJ; j++) {
         const int r = r0 + 32 * j + arow;
 #pragma unroll
         for (int e = 0; e < 16; e++) {

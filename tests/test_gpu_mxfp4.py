@@ -24,8 +24,11 @@ def to_bf16(x):
                                    (130, 200, 224), (1024, 2880, 2880), (9, 129, 2880)],
                          ids=lambda s: "x".join(map(str, s)))
 @pytest.mark.parametrize("weights", ["normal", "planted"])
-def test_mxfp4_bf16_matmul_vs_dequant_f32(dev, devbuf, shape, weights):
+@pytest.mark.parametrize("rows", [96, 128])
+def test_mxfp4_bf16_matmul_vs_dequant_f32(dev, devbuf, shape, weights, rows):
+    """rows = rows per workgroup tile (the library picks per shape; both are held to the bar)."""
     ntok, nrows, k = shape
+    dev.set_tuning(mxfp4__rows=rows)
     if weights == "planted" and ntok * nrows * k > 3e8:
         pytest.skip("the full-size case runs once, on quantized N(0, 0.02) weights")
     t = quant.MXFP4
@@ -44,6 +47,7 @@ def test_mxfp4_bf16_matmul_vs_dequant_f32(dev, devbuf, shape, weights):
         got = got[:ntok * nrows].reshape(ntok, nrows)
         assert nmse(got, want) <= 1e-10, f"call {call}: NMSE {nmse(got, want):.3e}"
         assert rel_l2(got, want) <= 1e-3
+    dev.set_tuning(mxfp4__rows=0)
 
 
 def test_mxfp4_declines_what_it_cannot_serve(dev, devbuf):
