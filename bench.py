@@ -243,6 +243,66 @@ def ffn_section(dev):
             "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
 
 
+def ffn_packed_section(dev):
+    """The same gated feed-forward block over packed planes, the layout a .jlm file holds:
+    gate and up (Q8_0 14336x4096) one launch of two packed matvecs sharing x, down (Q6_K
+    4096x14336) one launch over silu(gate) * up with the residual add riding on it; the
+    RMSNorm in front of gate and up is folded into their quantizer.  Four rotating sets of
+    planes keep every step out of cache."""
+    from jitllm_amd import quant, synth
+    from jitllm_amd.hipmem import DeviceArray, Event
+    n_embd, n_ffn = 4096, 14336
+    dev.SetActWindow(32)
+
+    def planes_of(t, nrows, k, seed):
+        src = DeviceArray(synth.quantized_weights(t, nrows, k, seed=seed))
+        pl = [DeviceArray(shape=(max(n, 1),), dtype=np.uint32, fill=0) for n in dev.packed_words(t, nrows, k)]
+        if not dev.pack_weights_dev(t, src.ptr, nrows, k, pl[0].ptr, pl[1].ptr, pl[2].ptr):
+            raise RuntimeError("the device declined to pack a matrix")
+        dev.synchronize()
+        src.free()
+        return pl
+    sets = [(planes_of(quant.Q8_0, n_ffn, n_embd, 0), planes_of(quant.Q8_0, n_ffn, n_embd, 0),
+             planes_of(quant.Q6_K, n_embd, n_ffn, 1)) for _ in range(4)]
+    x = DeviceArray(synth.activations(n_embd, seed=2))
+    gate = DeviceArray(shape=(n_ffn,), dtype=np.float32, fill=0)
+    up = DeviceArray(shape=(n_ffn,), dtype=np.float32, fill=0)
+    y = DeviceArray(shape=(n_embd,), dtype=np.float32, fill=0)
+    resid = DeviceArray(shape=(n_embd,), dtype=np.float32, fill=0)
+    norm_w = DeviceArray(np.ones(n_embd, np.float32))
+    tri = lambda pl: (pl[0].ptr, pl[1].ptr, pl[2].ptr)
+    calls = [(dev.packed_multi_args([gate.ptr, up.ptr], quant.Q8_0, [tri(g), tri(u)], [0, 0], n_ffn, x.ptr, 0, None,
+                                    n_ffn, n_embd, norm_w=norm_w.ptr, norm_eps=1e-5),
+              dev.packed_multi_args([y.ptr], quant.Q6_K, [tri(d)], [0], n_embd, gate.ptr, 0, up.ptr, n_embd, n_ffn,
+                                    resid=resid.ptr, alpha=1.0)) for g, u, d in sets]
+
+    def run(i):
+        a, b = calls[i % len(calls)]
+        if not (dev.packed_multi_call(a) and dev.packed_multi_call(b)):
+            raise RuntimeError("the device declined the packed feed-forward block")
+    for i in range(8):
+        run(i)
+    dev.synchronize()
+    e0, e1, n = Event(), Event(), 100
+    e0.record(dev.stream)
+    for i in range(n):
+        run(i)
+    e1.record(dev.stream)
+    e1.synchronize()
+    ms = e0.elapsed_ms(e1) / n
+    nbytes = 2 * n_ffn * quant.row_bytes(quant.Q8_0, n_embd) + n_embd * quant.row_bytes(quant.Q6_K, n_ffn) \
+        + 4 * (n_embd + 2 * n_ffn) + 4 * (2 * n_ffn + 2 * n_embd)
+    for st in sets:
+        for pl in st:
+            for b in pl:
+                b.free()
+    for b in (x, gate, up, y, resid, norm_w):
+        b.free()
+    return {"us_per_step": round(ms * 1e3, 2), "launches_per_step": 2, "bytes_per_step": nbytes,
+            "GB/s": round(nbytes / (ms * 1e-3) / 1e9, 1),
+            "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+
+
 def moe_section(dev):
     """Qwen3-30B-A3B routed feed-forward block: 128 experts (gate/up 768x2048, down 2048x768,
     Q4_K), 64 rows routed top-8 by softmax over N(0,1) logits (seeded); one step = group +
@@ -400,7 +460,7 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="headline workload only")
     ap.add_argument("--gemm", metavar="NTOK,NROWS", help="only the prefill GEMM of this shape (k = 4096), "
                     "for profiling one kernel; prints its section alone")
-    ap.add_argument("--section", choices=["mxfp4", "moe", "moe_decode", "ffn"], help="only this section of the default run, for "
+    ap.add_argument("--section", choices=["mxfp4", "moe", "moe_decode", "ffn", "ffn_packed"], help="only this section of the default run, for "
                     "profiling its kernels; prints the section alone")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -416,7 +476,8 @@ def main():
         dev.close()
         return
     if args.section:
-        fn = {"mxfp4": mxfp4_section, "moe": moe_section, "moe_decode": moe_decode_section, "ffn": ffn_section}[args.section]
+        fn = {"mxfp4": mxfp4_section, "moe": moe_section, "moe_decode": moe_decode_section, "ffn": ffn_section,
+              "ffn_packed": ffn_packed_section}[args.section]
         print(json.dumps({args.section: fn(dev)}), flush=True)
         dev.close()
         return
@@ -462,6 +523,7 @@ def main():
 
     if not args.no_extra:
         line["ffn_block_decode"] = ffn_section(dev)
+        line["ffn_block_decode_packed"] = ffn_packed_section(dev)
         line["prefill_gemm"] = gemm_section(dev)
         line["moe_block"] = moe_section(dev)
         line["moe_decode"] = moe_decode_section(dev)

@@ -201,11 +201,17 @@ int jl_matvec_gather_dev(jl_ctx *ctx, float *const *outs, int type, const void *
  * expert's sheet inside its bank's pages is the bank's plane pointers with row0 =
  * expert * nrows (device.go:70-80, format/jlm/write.go:165-180) -- and the activation
  * x[j*xstride : j*xstride+k] (xstride 0: one shared activation); up, when given, makes it
- * silu(x_j) * up_j.  m <= 16, one launch. */
+ * silu(x_j) * up_j; resid, when given, takes matrix 0's rows as they are made,
+ * resid[r] += alpha * out[0][r] (MVGroup.Resid, engine/nn/packedgroup.go:32-36); norm_w,
+ * when given (never together with up: JL_DECLINED), puts RMSNorm(x_j, norm_w, norm_eps) in
+ * front of the quantizer (RMSNormQuantRows, jit/gpu/kernels/elem.go:252-267, with the host
+ * arithmetic of internal/oracle/oracle.go:230-240) and norm_out, if not null, receives
+ * matrix 0's normed activation.  m <= 16, one launch. */
 int jl_matvec_packed_multi_dev(jl_ctx *ctx, float *const *outs, int type, const uint32_t *const *qs,
                                const uint32_t *const *d, const uint32_t *const *sc, const int *row0,
-                               int stride, const float *x, size_t xstride, const float *up, int nrows,
-                               int k, int m, void *stream);
+                               int stride, const float *x, size_t xstride, const float *up, float *resid,
+                               float alpha, const float *norm_w, float norm_eps, float *norm_out,
+                               int nrows, int k, int m, void *stream);
 
 /* JIT.MatMulPacked / MatMul semantics on resident operands (engine/nn/packedmm.go:23,
  * matmul.go:27): x [ntok][k] f32 -> out [ntok][nrows], every token quantized on

@@ -532,6 +532,7 @@ int packed_matvec_launch(jl_ctx* c, float* out, int type, const PlaneRef& pl, co
     a.x = x; a.q = q; a.as = as; a.s16 = s16;
     a.nrows = nrows; a.k = k; a.row0 = pl.row; a.stride = pl.stride; a.per = c->act_window / 32;
     a.nwaves = nw; a.ngroups = (nrows + rw - 1) / rw;
+    a.x2 = nullptr; a.resid = nullptr; a.alpha = 0.f; a.norm_out = nullptr; a.norm_eps = 0.f;
     char name[64];
     snprintf(name, sizeof name, "jl_matvec_packed_%s%s_w%d", x ? "" : "q8_", ti->tag, rw);
     void* params[] = {&a};
@@ -542,9 +543,12 @@ int packed_matvec_launch(jl_ctx* c, float* out, int type, const PlaneRef& pl, co
 // m packed matvecs of one type and shape in one launch (grid.y = matrix): each with its
 // own planes and first row, reading x + j * xstride; up gates the activation.
 int packed_matvec_multi_launch(jl_ctx* c, int type, int m, float* const* outs, const PlaneRef* pls,
-                               const float* x, size_t xstride, const float* up, int nrows, int k,
+                               const float* x, size_t xstride, const float* up, float* resid, float alpha,
+                               const float* norm_w, float norm_eps, float* norm_out, int nrows, int k,
                                hipStream_t st) {
     if (m < 1 || m > JL_MAX_MULTI) return fail(c, JL_ERR_ARG, "packed multi: %d matrices", m);
+    // the norm precedes gate and up, the gated activation precedes down: never both
+    if (norm_w && (up || !aligned16(norm_w) || (norm_out && !aligned16(norm_out)))) return JL_DECLINED;
     const TypeInfo* ti = nullptr;
     for (int j = 0; j < m; j++) {
         int rc = packed_check(c, type, pls[j], nrows, k, &ti);
@@ -570,11 +574,12 @@ int packed_matvec_multi_launch(jl_ctx* c, int type, int m, float* const* outs, c
     for (int j = 0; j < m; j++) {
         a.out[j] = outs[j]; a.qs[j] = pls[j].qs; a.d[j] = pls[j].d; a.sc[j] = pls[j].sc; a.row0[j] = pls[j].row;
     }
-    a.x = x; a.x2 = up; a.xstride = xstride;
+    a.x = x; a.x2 = up; a.xstride = xstride; a.resid = resid; a.alpha = alpha;
+    a.norm_w = norm_w; a.norm_eps = norm_eps; a.norm_out = norm_w ? norm_out : nullptr;
     a.nrows = nrows; a.k = k; a.stride = pls[0].stride; a.per = c->act_window / 32;
     a.nwaves = nw; a.ngroups = (nrows + rw - 1) / rw;
     char name[64];
-    snprintf(name, sizeof name, "jl_matvec_packed_multi_%s%s_w%d", up ? "act_" : "", ti->tag, rw);
+    snprintf(name, sizeof name, "jl_matvec_packed_multi_%s%s_w%d", up ? "act_" : norm_w ? "norm_" : "", ti->tag, rw);
     void* params[] = {&a};
     return launch(c, name, (unsigned)a.ngroups, (unsigned)m, (unsigned)(nw * 64), (unsigned)(nw * (384 + 65 * 4)), st,
                   params);   // JL_PK_LDS_BYTES
@@ -781,7 +786,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     for (const char* tag : {"q4k", "q8_0", "q6k"}) names.push_back(std::string("jl_matvec_multi_") + tag);
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int rw : {16, 32, 64})
-            for (const char* form : {"", "act_"})
+            for (const char* form : {"", "act_", "norm_"})
                 names.push_back(std::string("jl_matvec_packed_multi_") + form + tag + "_w" + std::to_string(rw));
     for (const auto& n : names) {
         hipFunction_t f;
@@ -945,7 +950,8 @@ int jl_matvec_group_dev(jl_ctx* c, const jl_mv_group* g, void* stream) {
 
 int jl_matvec_packed_multi_dev(jl_ctx* c, float* const* outs, int type, const uint32_t* const* qs,
                                const uint32_t* const* d, const uint32_t* const* sc, const int* row0, int stride,
-                               const float* x, size_t xstride, const float* up, int nrows, int k, int m,
+                               const float* x, size_t xstride, const float* up, float* resid, float alpha,
+                               const float* norm_w, float norm_eps, float* norm_out, int nrows, int k, int m,
                                void* stream) {
     if (!c) return JL_ERR_ARG;
     if (!outs || !qs || !d || !row0 || m < 1) return fail(c, JL_ERR_ARG, "packed multi: bad operand");
@@ -956,7 +962,8 @@ int jl_matvec_packed_multi_dev(jl_ctx* c, float* const* outs, int type, const ui
         pls[j].qs = qs[j]; pls[j].d = d[j]; pls[j].sc = sc ? sc[j] : nullptr;
         pls[j].row = row0[j]; pls[j].stride = stride;
     }
-    return packed_matvec_multi_launch(c, type, m, outs, pls, x, xstride, up, nrows, k, pick_stream(c, stream));
+    return packed_matvec_multi_launch(c, type, m, outs, pls, x, xstride, up, resid, alpha, norm_w, norm_eps,
+                                      norm_out, nrows, k, pick_stream(c, stream));
 }
 
 int jl_matvec_multi_dev(jl_ctx* c, float* const* outs, int type, const void* const* ws, const float* x,

@@ -225,6 +225,10 @@ struct PackedMatVecArgs {
     int nwaves;           // wavefronts per workgroup (the launch's block / 64)
     int ngroups;          // workgroups (the launch's grid.x)
     const float* x2;      // gated kernels only: the activation is silu(x) * x2
+    float* resid;         // null: none; else resid[r] += alpha * out[r]
+    float alpha;
+    float* norm_out;      // norm kernels only: null, or where the normed activation goes
+    float norm_eps;
 };
 
 // Several packed matvecs of one type and shape in one launch, grid = (row groups,
@@ -240,4 +244,9 @@ struct PackedMultiArgs {
     const float* x2;      // null: plain activation
     size_t xstride;       // elements
     int nrows, k, stride, per, nwaves, ngroups;
+    float* resid;         // null: none; else resid[r] += alpha * out[0][r] (matrix 0 only)
+    float alpha;
+    const float* norm_w;  // norm kernels only: RMSNorm weights [k]; every x_j is normed ahead of its quantizer
+    float* norm_out;      // null, or where matrix 0's normed activation goes
+    float norm_eps;
 };

@@ -78,13 +78,16 @@ extern "C" __global__ __launch_bounds__(256) void jl_unpack_q4k(UnpackArgs p) { 
 JL_PACKED_KERNEL(q4k, JL_Q4_K, 64, 4) JL_PACKED_KERNEL(q4k, JL_Q4_K, 32, 4) JL_PACKED_KERNEL(q4k, JL_Q4_K, 16, 4)
 JL_PACKED_KERNEL(q8_0, JL_Q8_0, 64, 2) JL_PACKED_KERNEL(q8_0, JL_Q8_0, 32, 4) JL_PACKED_KERNEL(q8_0, JL_Q8_0, 16, 4)
 JL_PACKED_KERNEL(q6k, JL_Q6_K, 64, 4) JL_PACKED_KERNEL(q6k, JL_Q6_K, 32, 4) JL_PACKED_KERNEL(q6k, JL_Q6_K, 16, 4)
-// jl_matvec_packed_multi[_act]_<type>_w<RW>: grid = (ceil(nrows/RW), matrices)
+// jl_matvec_packed_multi[_act|_norm]_<type>_w<RW>: grid = (ceil(nrows/RW), matrices)
 #define JL_PACKED_MULTI_KERNEL(T, TYPE, RW, XPRE)                                                               \
     extern "C" __global__ __launch_bounds__(1024) void jl_matvec_packed_multi_##T##_w##RW(PackedMultiArgs p) {  \
         packed_matvec_multi_body<TYPE, RW, XPRE, false>(p, jl_smem);                                            \
     }                                                                                                           \
     extern "C" __global__ __launch_bounds__(1024) void jl_matvec_packed_multi_act_##T##_w##RW(PackedMultiArgs p) { \
         packed_matvec_multi_body<TYPE, RW, 2, true>(p, jl_smem);                                                \
+    }                                                                                                           \
+    extern "C" __global__ __launch_bounds__(1024) void jl_matvec_packed_multi_norm_##T##_w##RW(PackedMultiArgs p) { \
+        packed_matvec_multi_body<TYPE, RW, 2, true, true>(p, jl_smem);                                          \
     }
 JL_PACKED_MULTI_KERNEL(q4k, JL_Q4_K, 64, 4) JL_PACKED_MULTI_KERNEL(q4k, JL_Q4_K, 32, 4) JL_PACKED_MULTI_KERNEL(q4k, JL_Q4_K, 16, 4)
 JL_PACKED_MULTI_KERNEL(q8_0, JL_Q8_0, 64, 2) JL_PACKED_MULTI_KERNEL(q8_0, JL_Q8_0, 32, 4) JL_PACKED_MULTI_KERNEL(q8_0, JL_Q8_0, 16, 4)

@@ -323,7 +323,7 @@ __device__ __forceinline__ void pk_load_x(const PackedMatVecArgs& p, int c, int 
     const int g4 = min(c * 64 + lane, p.k / 4 - 1);
     if (FUSED) {
         X.v = ((const f32x4*)p.x)[g4];
-        if constexpr (GATED) X.u = ((const f32x4*)p.x2)[g4];
+        if constexpr (GATED) X.u = ((const f32x4*)p.x2)[g4];   // the gate's partner, or the norm's weights
     } else {
         X.v.x = __uint_as_float(((const u32*)p.q)[g4]);
         X.v.y = p.as[min(c * 8 + (lane & 7), p.k / 32 - 1)];
@@ -333,15 +333,24 @@ __device__ __forceinline__ void pk_load_x(const PackedMatVecArgs& p, int c, int 
 }
 
 // Quantize (or copy) the chunk's activation into the wavefront's private LDS area.
-template <bool FUSED, bool GATED>
-__device__ __forceinline__ void pk_stage_x(const PackedMatVecArgs& p, int c, int lane, const PkX<GATED>& X, uint8_t* my) {
+// NORM: the second operand is the RMSNorm weight and nscale the row's 1/rms; the normed
+// value is f32(f64(x) * nscale * f64(w)), the reference's host arithmetic
+// (internal/oracle/oracle.go:230-240).
+template <bool FUSED, bool GATED, bool NORM = false>
+__device__ __forceinline__ void pk_stage_x(const PackedMatVecArgs& p, int c, int lane, const PkX<GATED>& X, uint8_t* my,
+                                           double nscale = 0.0, bool write_norm = false) {
     u32* a_w = (u32*)my;
     float* da_w = (float*)(my + 256);
     float* ss_w = (float*)(my + 288);
     const bool live = c * 64 + lane < p.k / 4;
     if (FUSED) {
         f32x4 xv = live ? X.v : f32x4{0.f, 0.f, 0.f, 0.f};
-        if constexpr (GATED) {
+        if constexpr (NORM) {
+            const f32x4 nw = X.u;
+            xv = f32x4{(float)((double)xv.x * nscale * (double)nw.x), (float)((double)xv.y * nscale * (double)nw.y),
+                       (float)((double)xv.z * nscale * (double)nw.z), (float)((double)xv.w * nscale * (double)nw.w)};
+            if (write_norm && live) ((f32x4*)p.norm_out)[c * 64 + lane] = xv;
+        } else if constexpr (GATED) {
             const f32x4 u = live ? X.u : f32x4{0.f, 0.f, 0.f, 0.f};
             xv = f32x4{silu_f32(xv.x) * u.x, silu_f32(xv.y) * u.y, silu_f32(xv.z) * u.z, silu_f32(xv.w) * u.w};
         }
@@ -379,8 +388,14 @@ __device__ __forceinline__ void pk_stage_x(const PackedMatVecArgs& p, int c, int
 // The partial sums [wavefront][lane] are added up by RW*16 threads at once: thread
 // (row r, j) takes wavefront j's KP partials of row r, and the sixteen j of a row sit
 // in one 16-lane DPP row, so the sum over wavefronts is four lane-exchange adds.
-template <int TYPE, int RW, int XPRE, bool FUSED, bool GATED = false>
+//
+// NORM (an RMSNorm in front of the quantizer, the reference's RMSNormQuantRows,
+// jit/gpu/kernels/elem.go:252-267): every workgroup forms the row's sum of squares itself,
+// in f64, before anything else; k floats from L2 are cheaper than a launch.  The norm's
+// weights ride in the gate partner's registers (p.x2), so NORM implies the two-operand load.
+template <int TYPE, int RW, int XPRE, bool FUSED, bool GATED = false, bool NORM = false>
 __device__ __forceinline__ void packed_matvec_body(const PackedMatVecArgs& p, uint8_t* smem) {
+    static_assert(!NORM || (FUSED && GATED), "the norm's weights ride in the second operand");
     constexpr int KP = 64 / RW, NB = 8 / KP;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = p.nwaves;
     // Workgroups are dealt to the eight XCDs round robin; give each XCD a contiguous
@@ -401,13 +416,37 @@ __device__ __forceinline__ void packed_matvec_body(const PackedMatVecArgs& p, ui
     PkX<GATED> X[XPRE];
 #pragma unroll
     for (int i = 0; i < XPRE; i++) pk_load_x<FUSED, GATED>(p, wave + i * nwaves, lane, X[i]);
-    __builtin_amdgcn_s_barrier();
+    double nscale = 0.0;
+    bool write_norm = false;
+    if constexpr (NORM) {
+        const int n4 = p.k / 4, nthreads = nwaves * 64;
+        double ss = 0.0;
+        auto sq = [&](const f32x4& v) {
+            ss += (double)v.x * v.x + (double)v.y * v.y + (double)v.z * v.z + (double)v.w * v.w;
+        };
+        // chunk wave + i * nwaves of lane `lane` is element threadIdx.x + i * nthreads
+#pragma unroll
+        for (int i = 0; i < XPRE; i++)
+            if ((int)threadIdx.x + i * nthreads < n4) sq(X[i].v);
+        for (int g4 = threadIdx.x + XPRE * nthreads; g4 < n4; g4 += nthreads) sq(((const f32x4*)p.x)[g4]);
+        ss = wave_sum_f64(ss);
+        double* nred = (double*)(smem + nwaves * JL_PK_WAVE_LDS);   // the partial-sum area, not in use yet
+        if (lane == 0) nred[wave] = ss;
+        __syncthreads();
+        double tot = 0.0;
+        for (int i = 0; i < nwaves; i++) tot += nred[i];
+        __syncthreads();                                            // all have read before the area is reused
+        nscale = 1.0 / __builtin_sqrt(tot / (double)p.k + (double)p.norm_eps);
+        write_norm = p.norm_out != nullptr && blockIdx.x == 0;
+    } else {
+        __builtin_amdgcn_s_barrier();
+    }
 
     float acc = 0.f;
     auto chunk = [&](int c, const PkX<GATED>& Xc) {
         typename PkTraits<TYPE, NB>::W w;
         pk_load<NB>(p, c, b0, row, w);
-        pk_stage_x<FUSED, GATED>(p, c, lane, Xc, my);
+        pk_stage_x<FUSED, GATED, NORM>(p, c, lane, Xc, my, nscale, write_norm);
         acc += pk_dot<NB>(p, w, c, b0, row, A);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -437,20 +476,25 @@ __device__ __forceinline__ void packed_matvec_body(const PackedMatVecArgs& p, ui
         t += dpp_f32<JL_DPP_QUAD_XOR2, 0xf>(t);
         t += dpp_f32<JL_DPP_ROW_HALF_MIRROR, 0xf>(t);
         t += dpp_f32<JL_DPP_ROW_MIRROR, 0xf>(t);
-        if (j == 0 && g * RW + r < p.nrows) p.out[g * RW + r] = t;
+        if (j == 0 && g * RW + r < p.nrows) {
+            p.out[g * RW + r] = t;
+            if (p.resid) p.resid[g * RW + r] += p.alpha * t;
+        }
     }
 }
 
 // Matrix blockIdx.y of a multi launch as a single packed matvec.
-template <int TYPE, int RW, int XPRE, bool GATED>
+template <int TYPE, int RW, int XPRE, bool GATED, bool NORM = false>
 __device__ __forceinline__ void packed_matvec_multi_body(const PackedMultiArgs& m, uint8_t* smem) {
     const int y = blockIdx.y;
     PackedMatVecArgs p;
     p.out = m.out[y]; p.qs = m.qs[y]; p.d = m.d[y]; p.sc = m.sc[y];
     p.x = m.x + (size_t)y * m.xstride;
-    p.x2 = GATED ? m.x2 + (size_t)y * m.xstride : nullptr;
+    p.x2 = NORM ? m.norm_w : GATED ? m.x2 + (size_t)y * m.xstride : nullptr;
+    p.norm_out = NORM && y == 0 ? m.norm_out : nullptr; p.norm_eps = m.norm_eps;
     p.q = nullptr; p.as = nullptr; p.s16 = nullptr;
     p.nrows = m.nrows; p.k = m.k; p.row0 = m.row0[y]; p.stride = m.stride;
     p.per = m.per; p.nwaves = m.nwaves; p.ngroups = m.ngroups;
-    packed_matvec_body<TYPE, RW, XPRE, true, GATED>(p, smem);
+    p.resid = y == 0 ? m.resid : nullptr; p.alpha = m.alpha;
+    packed_matvec_body<TYPE, RW, XPRE, true, GATED, NORM>(p, smem);
 }

@@ -204,13 +204,18 @@ class Device:
         return self._served(self._l.jl_matvec_gather_dev(self._ctx, po, t, pw, _ptr(x), xstride, _opt(up),
                                                          nrows, k, m, stream), "jl_matvec_gather_dev")
 
-    def matvec_packed_multi_dev(self, outs, t, planes, row0, stride, x, xstride, up, nrows, k, stream=None):
+    def matvec_packed_multi_dev(self, outs, t, planes, row0, stride, x, xstride, up, nrows, k, stream=None,
+                                resid=None, alpha=0.0, norm_w=None, norm_eps=0.0, norm_out=None):
         """MatVecPackedMulti / Gather / GatherAct over packed planes: planes is a list of
-        (qs, d, sc) device pointers, row0 the first row of each matrix in its buffer."""
+        (qs, d, sc) device pointers, row0 the first row of each matrix in its buffer;
+        resid += alpha * out[0] rides on the launch when given, and norm_w puts an RMSNorm
+        in front of the quantizer (not together with up)."""
         return self.packed_multi_call(self.packed_multi_args(outs, t, planes, row0, stride, x, xstride, up,
-                                                             nrows, k), stream)
+                                                             nrows, k, resid, alpha, norm_w, norm_eps, norm_out),
+                                      stream)
 
-    def packed_multi_args(self, outs, t, planes, row0, stride, x, xstride, up, nrows, k):
+    def packed_multi_args(self, outs, t, planes, row0, stride, x, xstride, up, nrows, k, resid=None, alpha=0.0,
+                          norm_w=None, norm_eps=0.0, norm_out=None):
         """The argument block of a packed multi call, built once by a caller that repeats it."""
         m = len(outs)
         po = (C.c_void_p * m)(*[_ptr(o) for o in outs])
@@ -218,7 +223,8 @@ class Device:
         pd = (C.c_void_p * m)(*[_ptr(p[1]) for p in planes])
         ps = (C.c_void_p * m)(*[_opt(p[2]) for p in planes])
         pr = (C.c_int * m)(*row0)
-        return (po, t, pq, pd, ps, pr, stride, _ptr(x), xstride, _opt(up), nrows, k, m)
+        return (po, t, pq, pd, ps, pr, stride, _ptr(x), xstride, _opt(up), _opt(resid), alpha, _opt(norm_w), norm_eps,
+                _opt(norm_out), nrows, k, m)
 
     def packed_multi_call(self, args, stream=None):
         return self._served(self._l.jl_matvec_packed_multi_dev(self._ctx, *args, stream),

@@ -194,7 +194,58 @@ def test_matvec_packed_multi_over_expert_sheets(dev, devbuf, t, form):
                 assert rel_l2(got[:nrows], _like_for_like(t, w, h, nrows, k, window)) <= 1e-3
             else:
                 assert nmse(got[:nrows], _like_for_like(t, w, xs[j], nrows, k, window)) <= 1e-10
+    # the residual add rides on matrix 0 alone: resid += alpha * out[0], nothing else moves
     dev.set_tuning(packed__rw=0)
+    resid0 = synth.activations(nrows + 2, seed=77)
+    resid = devbuf(resid0)
+    alpha = np.float32(-0.625)
+    assert dev.matvec_packed_multi_dev([o.ptr for o in outs], t, [(planes.qs, planes.d, planes.sc)] * m,
+                                       [e * nrows for e in experts], n_expert * nrows, xd.ptr,
+                                       0 if form == "multi" else k, ud.ptr if form == "gather_act" else None,
+                                       nrows, k, resid=resid.ptr, alpha=float(alpha))
+    dev.synchronize()
+    y0 = outs[0].get()[:nrows]
+    want_r = resid0.copy()
+    want_r[:nrows] = (resid0[:nrows] + (alpha * y0).astype(np.float32)).astype(np.float32)
+    assert np.array_equal(resid.get(), want_r)
+    dev.SetActWindow(32)
+
+
+@pytest.mark.parametrize("t,k,window", [(quant.Q8_0, 1056, 32), (quant.Q4_K, 4096, 256), (quant.Q6_K, 5120, 32)])
+def test_matvec_packed_multi_with_rmsnorm_in_front(dev, devbuf, t, k, window):
+    """RMSNorm folded into the packed kernels' quantizer (the reference's RMSNormQuantRows,
+    /root/reference/jit/gpu/kernels/elem.go:252-267): the normed vector the device writes
+    must be the oracle's RMSNorm32 up to the order of the f64 sum (one f32 ulp at most,
+    normally none), and every matrix's result the packed matvec of THAT vector.  Together
+    with a gated activation the call is declined."""
+    dev.SetActWindow(window)
+    m, nrows = 3, 150
+    ws = [synth.quantized_weights(t, nrows, k, seed=40 + j) for j in range(m)]
+    pls = [_dev_planes(devbuf, *oracle.pack_weights(t, w, nrows, k), stride=nrows) for w in ws]
+    x = synth.activations(k, seed=5) * np.float32(2.5)
+    nw = (1 + 0.1 * np.random.default_rng(3).standard_normal(k)).astype(np.float32)
+    eps = 1e-6
+    xd, nwd = devbuf(x), devbuf(nw)
+    dn = devbuf(shape=(k + 4,), dtype=np.float32, fill=np.float32(-3e30))
+    outs = [devbuf(shape=(nrows,), dtype=np.float32, fill=np.float32(9e30)) for _ in range(m)]
+    tri = [(p.qs, p.d, p.sc) for p in pls]
+    for rw in (0, 16, 64):
+        dev.set_tuning(packed__rw=rw)
+        assert dev.matvec_packed_multi_dev([o.ptr for o in outs], t, tri, [0] * m, nrows, xd.ptr, 0, None, nrows, k,
+                                           norm_w=nwd.ptr, norm_eps=eps, norm_out=dn.ptr)
+        dev.synchronize()
+        normed = dn.get()
+        assert np.all(normed[k:] == np.float32(-3e30))
+        normed = normed[:k]
+        want_n = oracle.rmsnorm32(x, nw, eps)
+        ulp = np.abs(normed.view(np.int32).astype(np.int64) - want_n.view(np.int32).astype(np.int64))
+        assert ulp.max() <= 1 and np.mean(ulp != 0) <= 0.01
+        for w, o in zip(ws, outs):
+            assert nmse(o.get(), _like_for_like(t, w, normed, nrows, k, window)) <= 1e-10
+            assert rel_l2(o.get(), _like_for_like(t, w, want_n, nrows, k, window)) <= 1e-3
+    dev.set_tuning(packed__rw=0)
+    assert dev.matvec_packed_multi_dev([o.ptr for o in outs], t, tri, [0] * m, nrows, xd.ptr, 0, xd.ptr, nrows, k,
+                                       norm_w=nwd.ptr, norm_eps=eps) is False
     dev.SetActWindow(32)
 
 
