@@ -305,19 +305,21 @@ def ffn_packed_section(dev):
 
 def moe_section(dev):
     """Qwen3-30B-A3B routed feed-forward block: 128 experts (gate/up 768x2048, down 2048x768,
-    Q4_K), 64 rows routed top-8 by softmax over N(0,1) logits (seeded); one step = group +
-    gate/up + down + combine, the router included.  Bytes = the touched experts' three sheets + x in + resid out."""
+    Q4_K), 64 rows routed top-8; one step = router logits (f32 router matrix, rows ~ N(0, 1/k)
+    so the logits are ~ N(0,1)) + softmax/top-8 + group + gate/up + down + combine, all on the
+    device.  Bytes = the touched experts' three sheets + router matrix + x in + resid out."""
     from jitllm_amd import quant, synth
     from jitllm_amd.hipmem import DeviceArray, Event
     t, rows, n_expert, k_used, n_ffn, n_embd = quant.Q4_K, 64, 128, 8, 768, 2048
     dev.SetActWindow(256)
     rng = np.random.default_rng(0)
-    logits = rng.standard_normal((rows, n_expert)).astype(np.float32)
-    # routing runs on the device inside the step (softmax, top-8 lowest-index ties, weights)
-    ld = DeviceArray(logits)
+    x = DeviceArray(rng.standard_normal((rows, n_embd)).astype(np.float32))
+    router = DeviceArray((rng.standard_normal((n_expert, n_embd)) / np.sqrt(n_embd)).astype(np.float32))
+    ld = DeviceArray(shape=(rows, n_expert), dtype=np.float32, fill=0)
     sd = DeviceArray(shape=(rows, k_used + 1), dtype=np.uint32, fill=0)
     wd = DeviceArray(shape=(rows, k_used), dtype=np.float32, fill=0)
-    if not dev.moe_route_dev(ld.ptr, rows, n_expert, k_used, sd.ptr, k_used + 1, wd.ptr):
+    if not (dev.moe_logits_dev(ld.ptr, 0, router.ptr, x.ptr, n_expert, n_embd, rows) and
+            dev.moe_route_dev(ld.ptr, rows, n_expert, k_used, sd.ptr, k_used + 1, wd.ptr)):
         raise RuntimeError("the device declined the router")
     dev.synchronize()
     touched = len(np.unique(sd.get()[:, :k_used]))
@@ -326,11 +328,11 @@ def moe_section(dev):
     banks = []
     for i, (r, k) in enumerate([(n_ffn, n_embd), (n_ffn, n_embd), (n_embd, n_ffn)]):
         banks.append(DeviceArray(synth.quantized_weights(t, r * n_expert, k, seed=10 + i)))
-    x = DeviceArray(rng.standard_normal((rows, n_embd)).astype(np.float32))
     resid = DeviceArray(shape=(rows, n_embd), dtype=np.float32, fill=0)
 
     def run():
-        return (dev.moe_route_dev(ld.ptr, rows, n_expert, k_used, sd.ptr, k_used + 1, wd.ptr) and
+        return (dev.moe_logits_dev(ld.ptr, 0, router.ptr, x.ptr, n_expert, n_embd, rows) and
+                dev.moe_route_dev(ld.ptr, rows, n_expert, k_used, sd.ptr, k_used + 1, wd.ptr) and
                 dev.moe_ffn_dev(resid.ptr, t, banks[0].ptr, banks[1].ptr, banks[2].ptr, x.ptr, sd.ptr,
                                 k_used + 1, wd.ptr, rows, k_used, n_expert, n_ffn, n_embd))
     for _ in range(3):
@@ -344,8 +346,8 @@ def moe_section(dev):
     e1.record(dev.stream)
     e1.synchronize()
     ms = e0.elapsed_ms(e1) / n
-    nbytes = touched * (2 * gs + ds) + 2 * rows * n_embd * 4
-    for b in banks + [x, sd, wd, resid, ld]:
+    nbytes = touched * (2 * gs + ds) + 2 * rows * n_embd * 4 + n_expert * n_embd * 4
+    for b in banks + [x, sd, wd, resid, ld, router]:
         b.free()
     return {"us_per_step": round(ms * 1e3, 1), "experts_touched": touched, "bytes_per_step": nbytes,
             "GB/s": round(nbytes / (ms * 1e-3) / 1e9, 1),

@@ -42,6 +42,8 @@ extern "C" {
 #define JL_ERR_HIP (-2)
 #define JL_ERR_NOMEM (-3)
 
+#define JL_TYPE_F32 0   /* router weights only (jl_moe_logits_dev) */
+#define JL_TYPE_F16 1
 #define JL_TYPE_Q8_0 8
 #define JL_TYPE_Q4_K 12
 #define JL_TYPE_Q6_K 14
@@ -91,6 +93,11 @@ int jl_synchronize(jl_ctx *ctx);
  * value 0 restores the built-in choice.  Mirrors the reference's per-instance tuning knobs
  * (engine/nn/options.go:67-118). */
 int jl_set_tuning(jl_ctx *ctx, const char *key, int value);
+
+/* Kernels this context has launched so far: how callers and tests check that a grouped
+ * call was one launch, the point of the reference's grouped forms
+ * (engine/nn/packedgroup.go:13-20). */
+unsigned long long jl_launch_count(const jl_ctx *ctx);
 
 /* ---- host-pointer seam ------------------------------------------------ */
 
@@ -164,7 +171,8 @@ int jl_matvec_q8_dev(jl_ctx *ctx, float *out, int type, const void *w, const int
  * front of everything, the reference's RMSNormQuantRows (jit/gpu/kernels/elem.go:252-267)
  * with the arithmetic of its host form (internal/oracle/oracle.go:230-240): the activation
  * is f32(f64(x) * 1/sqrt(mean(x^2) + norm_eps) * f64(norm_w)), mean in f64; norm_out, when
- * set, receives that normed vector.  Matrices of one type share a launch. */
+ * set, receives that normed vector.  One launch, whatever the mix of types (the reference's
+ * MatVecSegments, jit/gpu/kernels/matvec.go:1411-1431). */
 #define JL_MAX_GROUP 4
 typedef struct jl_mv_group {
     int n;
@@ -274,6 +282,14 @@ int jl_matmul_mxfp4_bf16_dev(jl_ctx *ctx, float *out, const void *w, const uint1
                              int nrows, int k, int ntok, void *stream);
 
 /* ---- mixture of experts (device pointers) ----------------------------- */
+
+/* The router's logits (kernels.RouterMatVecTok, jit/gpu/kernels/moe.go:820-917):
+ * logits[t][r] = sum_i W[r][i] * x[t][i], W [n_expert][k] in f32 (JL_TYPE_F32) or f16
+ * (JL_TYPE_F16, Mixtral's ffn_gate_inp), the one matrix of a mixture block that is not
+ * quantized.  f32 arithmetic in that kernel's order (128 strided partial sums, then a
+ * binary tree), so the logits are bit for bit what the reference's device path routes on. */
+int jl_moe_logits_dev(jl_ctx *ctx, float *logits, int wtype, const void *w, const float *x,
+                      int n_expert, int k, int ntok, void *stream);
 
 /* The router (kernels.ExpertRoute, jit/gpu/kernels/moe.go:562; specification
  * oracle.MoERouter, internal/oracle/moe.go:197-327, with Softmax32, oracle.go:244-265):

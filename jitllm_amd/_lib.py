@@ -34,6 +34,7 @@ class MVGroup(C.Structure):
 SIGNATURES = {
     "jl_hip_runtime": (C.c_char_p, []),
     "jl_ctx_create": (_int, [C.POINTER(_vp), C.POINTER(Options)]),
+    "jl_launch_count": (C.c_ulonglong, [_vp]),
     "jl_ctx_destroy": (None, [_vp]),
     "jl_last_error": (C.c_char_p, [_vp]),
     "jl_set_act_window": (_int, [_vp, _int]),
@@ -66,6 +67,7 @@ SIGNATURES = {
     "jl_matmul_packed_dev": (_int, [_vp, _vp, _int, _vp, _vp, _vp, _int, _int, _vp, _int, _int, _int,
                                     _vp]),
     "jl_matmul_mxfp4_bf16_dev": (_int, [_vp, _vp, _vp, _vp, _int, _int, _int, _vp]),
+    "jl_moe_logits_dev": (_int, [_vp, _vp, _int, _vp, _vp, _int, _int, _int, _vp]),
     "jl_moe_route_dev": (_int, [_vp, _vp, _int, _int, _int, _vp, _int, _vp, _vp]),
     "jl_moe_group_dev": (_int, [_vp, _vp, _int, _int, _int, _int, _vp, _vp, _vp, _vp]),
     "jl_moe_matvec_dev": (_int, [_vp, _vp, _vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp]),

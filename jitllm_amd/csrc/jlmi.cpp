@@ -59,6 +59,7 @@ struct jl_ctx {
     int gemm_min_tok = 8;  // below this a per-token matvec loop reads the weights as cheaply
     int num_cu = 0;
     size_t lds_limit = 0;
+    unsigned long long launches = 0;   // kernels launched so far (jl_launch_count)
 
     // prefill GEMM workspace (quantized activations in stage layout), grown on demand
     void* gemm_ws = nullptr;
@@ -152,6 +153,7 @@ int launch(jl_ctx* c, const char* name, unsigned gx, unsigned gy, unsigned block
     auto it = c->fn.find(name);
     if (it == c->fn.end()) return fail(c, JL_ERR_ARG, "kernel %s is not in the code object", name);
     HIP_TRY(c, H->ModuleLaunchKernel(it->second, gx, gy, 1, block, 1, 1, lds, st, params, nullptr));
+    c->launches++;
     return JL_OK;
 }
 
@@ -218,18 +220,22 @@ int matvec_launch(jl_ctx* c, float* out, int type, const void* w, const float* x
 }
 
 // m matrices of one type in one launch (kernels/matvec.h, matvec_multi_body).
+// types: null when every matrix is of `type`; else the type of each (the mixed-type kernel).
 int matvec_multi_launch(jl_ctx* c, int type, int m, float* const* outs, const void* const* ws, const int* rows,
                         const float* x, size_t xstride, const float* x2, float* resid, float alpha, int k,
                         hipStream_t st, const float* norm_w = nullptr, float norm_eps = 0.f,
-                        float* norm_out = nullptr) {
+                        float* norm_out = nullptr, const int* types = nullptr) {
     if (m < 1 || m > JL_MAX_MULTI) return fail(c, JL_ERR_ARG, "matvec multi: %d matrices", m);
     const TypeInfo* ti = nullptr;
+    const TypeInfo* tis[JL_MAX_MULTI];
     int max_rows = 0;
     for (int i = 0; i < m; i++) {
-        int rc = matvec_check(c, type, rows[i], k, &ti);
+        const int t = types ? types[i] : type;
+        int rc = matvec_check(c, t, rows[i], k, &ti);
         if (rc != JL_OK) return rc;
+        tis[i] = ti;
         if (!outs[i] || !ws[i]) return fail(c, JL_ERR_ARG, "matvec multi: null operand");
-        if (type == JL_TYPE_Q4_K && !aligned16(ws[i])) return JL_DECLINED;
+        if (t == JL_TYPE_Q4_K && !aligned16(ws[i])) return JL_DECLINED;
         if (((uintptr_t)ws[i] & 1) != 0) return JL_DECLINED;
         if (rows[i] > max_rows) max_rows = rows[i];
     }
@@ -241,6 +247,8 @@ int matvec_multi_launch(jl_ctx* c, int type, int m, float* const* outs, const vo
         a.out[i] = outs[i];
         a.w[i] = (const uint8_t*)ws[i];
         a.nrows[i] = rows[i];
+        a.type[i] = types ? types[i] : type;
+        a.row_bytes_of[i] = (k / tis[i]->block_elems) * tis[i]->block_bytes;
     }
     a.x = x; a.x2 = x2; a.resid = resid; a.alpha = alpha; a.xstride = xstride;
     a.norm_w = norm_w; a.norm_eps = norm_eps; a.norm_out = norm_out;
@@ -254,7 +262,8 @@ int matvec_multi_launch(jl_ctx* c, int type, int m, float* const* outs, const vo
     if (gx < 1) gx = 1;
     a.nwaves = nwaves; a.ngroups = (int)gx;
     char name[64];
-    snprintf(name, sizeof name, "jl_matvec_multi_%s", ti->tag);
+    if (types) snprintf(name, sizeof name, "jl_matvec_segments");
+    else snprintf(name, sizeof name, "jl_matvec_multi_%s", ti->tag);
     void* params[] = {&a};
     unsigned lds = (unsigned)((size_t)k + (size_t)(k / 32) * 4 + (size_t)(k / 16) * 4);
     return launch(c, name, (unsigned)gx, (unsigned)m, nwaves * 64, lds, st, params);
@@ -768,7 +777,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     if (e != hipSuccess)
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
-    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_q4k_r64", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_moe_route", "jl_moe_group", "jl_moe_quant", "jl_moe_combine", "jl_moe_gemm_prep", "jl_moe_gemm_q4k", "jl_mxfp4_prep", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_sum_parts",
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_q4k_r64", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_moe_route", "jl_moe_logits", "jl_moe_group", "jl_moe_quant", "jl_moe_combine", "jl_moe_gemm_prep", "jl_moe_gemm_q4k", "jl_mxfp4_prep", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_sum_parts",
                                       "jl_pack_weights", "jl_unpack_q4k"};
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int rw : {16, 32, 64})
@@ -784,6 +793,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
             names.push_back(nm);
         }
     for (const char* tag : {"q4k", "q8_0", "q6k"}) names.push_back(std::string("jl_matvec_multi_") + tag);
+    names.push_back("jl_matvec_segments");
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int rw : {16, 32, 64})
             for (const char* form : {"", "act_", "norm_"})
@@ -841,6 +851,8 @@ int jl_synchronize(jl_ctx* c) {
     HIP_TRY(c, H->StreamSynchronize(c->stream));
     return JL_OK;
 }
+
+unsigned long long jl_launch_count(const jl_ctx* c) { return c ? c->launches : 0; }
 
 int jl_set_tuning(jl_ctx* c, const char* key, int value) {
     if (!c || !key) return JL_ERR_ARG;
@@ -928,24 +940,12 @@ int jl_matvec_group_dev(jl_ctx* c, const jl_mv_group* g, void* stream) {
     }
     if (!aligned16(g->x) || (g->act_up && !aligned16(g->act_up))) return JL_DECLINED;
     if ((g->norm_w && !aligned16(g->norm_w)) || (g->norm_out && (!g->norm_w || !aligned16(g->norm_out)))) return JL_DECLINED;
-    // matrices of one type share a launch; matrix 0 leads its launch so that the residual rides on it
-    bool done[JL_MAX_GROUP] = {false, false, false, false};
-    for (int i = 0; i < g->n; i++) {
-        if (done[i]) continue;
-        float* outs[JL_MAX_GROUP];
-        const void* ws[JL_MAX_GROUP];
-        int rows[JL_MAX_GROUP], m = 0;
-        for (int j = i; j < g->n; j++)
-            if (!done[j] && g->type[j] == g->type[i]) {
-                outs[m] = g->out[j]; ws[m] = g->w[j]; rows[m] = g->rows[j]; m++;
-                done[j] = true;
-            }
-        int rc = matvec_multi_launch(c, g->type[i], m, outs, ws, rows, g->x, 0, g->act_up,
-                                     i == 0 ? g->resid : nullptr, g->alpha, g->k, st, g->norm_w, g->norm_eps,
-                                     i == 0 ? g->norm_out : nullptr);
-        if (rc != JL_OK) return rc;
-    }
-    return JL_OK;
+    // one launch: the single-type kernel, or the mixed-type one when the formats differ
+    // (the reference's MatVecSegments, jit/gpu/kernels/matvec.go:1411-1431)
+    bool mixed = false;
+    for (int i = 1; i < g->n; i++) mixed = mixed || g->type[i] != g->type[0];
+    return matvec_multi_launch(c, g->type[0], g->n, g->out, g->w, g->rows, g->x, 0, g->act_up, g->resid, g->alpha,
+                               g->k, st, g->norm_w, g->norm_eps, g->norm_out, mixed ? g->type : nullptr);
 }
 
 int jl_matvec_packed_multi_dev(jl_ctx* c, float* const* outs, int type, const uint32_t* const* qs,
@@ -1072,6 +1072,23 @@ int jl_moe_route_dev(jl_ctx* c, const float* logits, int rows, int n_expert, int
     a.logits = logits; a.sel = sel; a.wt = wt; a.n_expert = n_expert; a.k_used = k_used; a.sel_stride = sel_stride;
     void* params[] = {&a};
     return launch(c, "jl_moe_route", (unsigned)rows, 1, 64, 0, pick_stream(c, stream), params);
+}
+
+int jl_moe_logits_dev(jl_ctx* c, float* logits, int wtype, const void* w, const float* x, int n_expert, int k,
+                      int ntok, void* stream) {
+    if (!c) return JL_ERR_ARG;
+    if (!logits || !w || !x || n_expert <= 0 || k <= 0 || ntok <= 0)
+        return fail(c, JL_ERR_ARG, "moe logits: bad operand");
+    if (wtype != JL_TYPE_F32 && wtype != JL_TYPE_F16) return JL_DECLINED;
+    if (((uintptr_t)w & (wtype == JL_TYPE_F32 ? 3 : 1)) || ((uintptr_t)x & 3)) return JL_DECLINED;
+    if (n_expert > 65535 || (ntok + 7) / 8 > 65535) return JL_DECLINED;
+    HIP_TRY(c, H->SetDevice(c->device));
+    MoeLogitsArgs a;
+    a.w = w; a.x = x; a.logits = logits; a.n_expert = n_expert; a.k = k; a.ntok = ntok;
+    a.f16 = wtype == JL_TYPE_F16;
+    void* params[] = {&a};
+    return launch(c, "jl_moe_logits", (unsigned)n_expert, (unsigned)((ntok + 7) / 8), 128, 0,   // JL_LOGITS_TOK
+                  pick_stream(c, stream), params);
 }
 
 int jl_moe_group_dev(jl_ctx* c, const uint32_t* sel, int sel_stride, int rows, int k_used, int n_expert,

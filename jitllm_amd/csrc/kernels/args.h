@@ -33,6 +33,9 @@ struct MatVecMultiArgs {
     float alpha;
     size_t xstride;      // elements
     int k, row_bytes, per, nwaves, ngroups;
+    // the mixed-type kernel only: each matrix's type (JL_TYPE_*) and bytes per row
+    int type[JL_MAX_MULTI];
+    int row_bytes_of[JL_MAX_MULTI];
     const float* norm_w; // null: none; else the activation is RMSNorm(x) * norm_w first
     float* norm_out;     // optional: the normed activation, written once
     float norm_eps;
@@ -125,6 +128,15 @@ struct MoeRouteArgs {
     uint32_t* sel;
     float* wt;
     int n_expert, k_used, sel_stride;
+};
+
+// Router logits: logits[t][r] = sum_i W[r][i] * x[t][i], W f32 or f16 (the one matrix of a
+// mixture block that is not quantized).
+struct MoeLogitsArgs {
+    const void* w;          // [n_expert][k], f32 or f16
+    const float* x;         // [ntok][k]
+    float* logits;          // [ntok][n_expert]
+    int n_expert, k, ntok, f16;
 };
 
 // Column activations of a mixture pass: column c reads x[src(c)] (or silu(x[src(c)]) *

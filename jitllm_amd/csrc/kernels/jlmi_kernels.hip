@@ -56,9 +56,21 @@ JL_MATVEC_KERNEL(q6k, JL_Q6_K, 1, 1024) JL_MATVEC_KERNEL(q6k, JL_Q6_K, 2, 512) J
 // grid = (row groups, matrices), block = 64..1024
 #define JL_MATVEC_MULTI_KERNEL(T, TYPE)                                                                \
     extern "C" __global__ __launch_bounds__(1024) void jl_matvec_multi_##T(MatVecMultiArgs p) {        \
-        matvec_multi_body<TYPE>(p, jl_smem);                                                           \
+        matvec_multi_body<TYPE>(p, jl_smem, p.row_bytes);                                              \
     }
 JL_MATVEC_MULTI_KERNEL(q4k, JL_Q4_K) JL_MATVEC_MULTI_KERNEL(q8_0, JL_Q8_0) JL_MATVEC_MULTI_KERNEL(q6k, JL_Q6_K)
+// The same grid over matrices of different types (the reference's MatVecSegments,
+// jit/gpu/kernels/matvec.go:1411-1431: a block's q, k and v in one launch whatever their
+// formats): the type is uniform per workgroup, so the switch is a scalar branch into the
+// single-type body.
+extern "C" __global__ __launch_bounds__(1024) void jl_matvec_segments(MatVecMultiArgs p) {
+    const int y = blockIdx.y;
+    switch (p.type[y]) {
+    case JL_Q4_K: matvec_multi_body<JL_Q4_K>(p, jl_smem, p.row_bytes_of[y]); break;
+    case JL_Q8_0: matvec_multi_body<JL_Q8_0>(p, jl_smem, p.row_bytes_of[y]); break;
+    case JL_Q6_K: matvec_multi_body<JL_Q6_K>(p, jl_smem, p.row_bytes_of[y]); break;
+    }
+}
 
 // ---------------------------------------------------------- packed planes
 // grid = (ceil(nrows/256), k/256 or k/32 for Q8_0), block = 256
@@ -116,6 +128,11 @@ extern "C" __global__ __launch_bounds__(256, 2) void jl_gemm_q4k_w16(GemmW16Args
 // ------------------------------------------------------- mixture of experts
 // grid = rows, block = 64
 extern "C" __global__ __launch_bounds__(64) void jl_moe_route(MoeRouteArgs p) { moe_route_body(p); }
+// grid = (experts, ceil(tokens / JL_LOGITS_TOK)), block = 128
+extern "C" __global__ __launch_bounds__(128) void jl_moe_logits(MoeLogitsArgs p) {
+    __shared__ float part[JL_LOGITS_TOK * 128];
+    moe_logits_body(p, part);
+}
 // one workgroup of 1024 threads (n_expert <= 1024)
 extern "C" __global__ __launch_bounds__(1024) void jl_moe_group(MoeGroupArgs p) {
     __shared__ u32 scount[2048];

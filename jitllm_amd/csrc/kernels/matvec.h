@@ -422,7 +422,7 @@ __device__ __forceinline__ double wave_sum_f64(double v) {
 }
 
 template <int TYPE>
-__device__ __forceinline__ void matvec_multi_body(const MatVecMultiArgs& p, uint8_t* smem) {
+__device__ __forceinline__ void matvec_multi_body(const MatVecMultiArgs& p, uint8_t* smem, int row_bytes) {
     typedef SlotTraits<TYPE> T;
     const int y = blockIdx.y;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = p.nwaves;
@@ -442,7 +442,7 @@ __device__ __forceinline__ void matvec_multi_body(const MatVecMultiArgs& p, uint
     f32x4 u0 = x2 ? ((const f32x4*)x2)[min((int)threadIdx.x, n4 - 1)] : f32x4{1.f, 1.f, 1.f, 1.f};
     __builtin_amdgcn_s_barrier();   // activation loads of the whole workgroup go out first
     typename T::W w;
-    T::load_w(w0 + (size_t)min(r0, nrows - 1) * p.row_bytes, min(lane, nslots - 1), w);
+    T::load_w(w0 + (size_t)min(r0, nrows - 1) * row_bytes, min(lane, nslots - 1), w);
     // RMSNorm ahead of the quantizer (the reference's RMSNormQuantRows, jit/gpu/kernels/
     // elem.go:252-267, with its host arithmetic, internal/oracle/oracle.go:230-240): the sum
     // of squares in f64, scale = 1/sqrt(sum/k + eps), y = f32(f64(x) * scale * f64(w)).
@@ -484,7 +484,7 @@ __device__ __forceinline__ void matvec_multi_body(const MatVecMultiArgs& p, uint
     for (; r0 < nrows; r0 += group_stride) {
         float acc = 0.f;
         for (int slot = lane; slot < nslots; slot += 64) {
-            if (!preloaded) T::load_w(w0 + (size_t)r0 * p.row_bytes, slot, w);
+            if (!preloaded) T::load_w(w0 + (size_t)r0 * row_bytes, slot, w);
             preloaded = false;
             typename T::Act a;
             T::load_act(A, slot, a);

@@ -603,3 +603,51 @@ __device__ __forceinline__ void moe_combine_body(const MoeCombineArgs& p) {
     }
     p.resid[(size_t)r * p.n_embd + n] = acc;
 }
+
+// ---------------------------------------------------------------- router logits
+// logits[t][r] = sum_i W[r][i] * x[t][i] in f32, with the summation order of the reference's
+// device kernel (jit/gpu/kernels/moe.go:843-917) so that the bits are its bits: thread j of
+// 128 adds the products of i = j, j + 128, ... one after the other (product rounded, then
+// the sum; a ragged tail adds +0), and the 128 partial sums meet in a binary tree, thread j
+// taking thread j + s at s = 64, 32, ..., 1.  One workgroup per expert row and group of
+// JL_LOGITS_TOK tokens: the row is read once for all of them.
+#define JL_LOGITS_TOK 8
+__device__ __forceinline__ void moe_logits_body(const MoeLogitsArgs& p, float* part) {
+    const int r = blockIdx.x, t0 = blockIdx.y * JL_LOGITS_TOK, tid = threadIdx.x;
+    const int nt = min(JL_LOGITS_TOK, p.ntok - t0), k = p.k;
+    float acc[JL_LOGITS_TOK];
+#pragma unroll
+    for (int t = 0; t < JL_LOGITS_TOK; t++) acc[t] = 0.f;
+    const float* wf = (const float*)p.w + (size_t)r * k;
+    const uint16_t* wh = (const uint16_t*)p.w + (size_t)r * k;
+    // unrolled so that the loads of eight trips are in flight together; the sums stay in order
+#pragma unroll 8
+    for (int i0 = 0; i0 < k; i0 += 128) {
+        const int i = i0 + tid, ic = min(i, k - 1);
+        const float w = p.f16 ? half_bits_to_f32(wh[ic]) : wf[ic];
+#pragma unroll
+        for (int t = 0; t < JL_LOGITS_TOK; t++) {
+            const float xv = p.x[(size_t)(t0 + min(t, nt - 1)) * k + ic];
+            const float prod = w * xv;
+            acc[t] = acc[t] + (i < k ? prod : 0.f);
+        }
+    }
+    // part [token][128]
+#pragma unroll
+    for (int t = 0; t < JL_LOGITS_TOK; t++) part[t * 128 + tid] = acc[t];
+    __syncthreads();
+    // The tree, one token per 16 lanes: lane j of a token's row takes the partial sums the
+    // tree would bring to thread j by s = 16 (levels 64, 32, 16: seven adds in tree order),
+    // then levels 8..1 are lane moves inside the 16-lane row (lane j reads lane j + s).
+    static_assert(JL_LOGITS_TOK == 8, "eight tokens x sixteen lanes = the workgroup");
+    const int tk = tid >> 4, j = tid & 15;
+    const float* q = part + tk * 128 + j;
+    const float a0 = q[0] + q[64], a32 = q[32] + q[96], a16 = q[16] + q[80], a48 = q[48] + q[112];
+    const float b0 = a0 + a32, b16 = a16 + a48;
+    float v = b0 + b16;
+    v = v + dpp_f32<0x108, 0xf>(v);   // row_shl:8
+    v = v + dpp_f32<0x104, 0xf>(v);   // row_shl:4
+    v = v + dpp_f32<0x102, 0xf>(v);   // row_shl:2
+    v = v + dpp_f32<0x101, 0xf>(v);   // row_shl:1
+    if (j == 0 && tk < nt) p.logits[(size_t)(t0 + tk) * p.n_expert + r] = v;
+}

@@ -49,6 +49,10 @@ class Device:
             self._ctx = None
             raise DeviceError(f"jl_ctx_create failed ({rc}): {msg}")
 
+    def launch_count(self):
+        """Kernels launched so far by this device."""
+        return int(self._l.jl_launch_count(self._ctx))
+
     def close(self):
         if getattr(self, "_ctx", None):
             self._l.jl_ctx_destroy(self._ctx)
@@ -236,6 +240,12 @@ class Device:
                                                   nrows, k, ntok, stream), "jl_matmul_dev")
 
     # -- mixture of experts -----------------------------------------------------
+    def moe_logits_dev(self, logits, wtype, w, x, n_expert, k, ntok, stream=None):
+        """Router logits [ntok][n_expert] = x [ntok][k] . W^T, W f32 (wtype 0) or f16 (1), in the
+        reference device kernel's summation order (kernels.RouterMatVecTok)."""
+        return self._served(self._l.jl_moe_logits_dev(self._ctx, _ptr(logits), wtype, _ptr(w), _ptr(x),
+                                                      n_expert, k, ntok, stream), "jl_moe_logits_dev")
+
     def moe_route_dev(self, logits, rows, n_expert, k_used, sel, sel_stride, wt, stream=None):
         """oracle.MoERouter on the device: softmax, lexicographic top-k, renormalised weights."""
         return self._served(self._l.jl_moe_route_dev(self._ctx, _ptr(logits), rows, n_expert, k_used,

@@ -72,6 +72,8 @@ _l.jlo_matvec_q8act_f64.argtypes = [_f64p, C.c_int, _u8p, _i8p, _f32p, C.c_int, 
 _l.jlo_matvec_q8act_f32.argtypes = [_f32p, C.c_int, _u8p, _i8p, _f32p, _f32p, C.c_int, C.c_int]
 _l.jlo_rmsnorm32.restype = None
 _l.jlo_rmsnorm32.argtypes = [_f32p, _f32p, _f32p, C.c_int, C.c_double]
+_l.jlo_router_logits.restype = None
+_l.jlo_router_logits.argtypes = [_f32p, C.c_void_p, C.c_int, _f32p, C.c_int, C.c_int, C.c_int]
 _l.jlo_moe_route.argtypes = [_f32p, C.c_int, C.c_int, _i32p, _f32p, _i32p, _f32p]
 _l.jlo_group_pairs.argtypes = [_u32p, C.c_int, C.c_int, C.c_int, C.c_int, _u32p, _u32p, _u32p,
                                C.c_int]
@@ -240,6 +242,21 @@ def rmsnorm32(x, w, eps):
     y = np.empty(x.size, np.float32)
     _l.jlo_rmsnorm32(_p(y, _f32p), _p(x, _f32p), _p(w, _f32p), x.size, float(eps))
     return y
+
+
+def router_logits(w, x, rows, k, ntok=1):
+    """Router logits [ntok][rows] in the reference device kernel's summation order
+    (kernels.RouterMatVecTok); w is f32 [rows][k], or f16 bits (uint16) of the same shape."""
+    w = np.ascontiguousarray(w)
+    f16 = w.dtype == np.uint16
+    if not f16:
+        w = _chk(w, np.float32, rows * k)
+    elif w.size != rows * k:
+        raise ValueError("router_logits: weight size")
+    x = _chk(x, np.float32, ntok * k)
+    out = np.empty((ntok, rows), np.float32)
+    _l.jlo_router_logits(_p(out, _f32p), w.ctypes.data_as(C.c_void_p), int(f16), _p(x, _f32p), rows, k, ntok)
+    return out
 
 
 def moe_route(logits, k):

@@ -819,6 +819,36 @@ void jlo_rmsnorm32(float *y, const float *x, const float *w, int n, double eps) 
     for (int i = 0; i < n; i++) y[i] = (float)((double)x[i] * scale * (double)w[i]);
 }
 
+/* jit/gpu/kernels/moe.go:843-917 (routerMatVec): the router's logits, out[t][r] = sum_i
+ * W[r][i] * x[t][i] in f32 in the device kernel's order.  128 threads a row: thread j adds
+ * the products of i = j, j + 128, ... one after the other over ceil(k/128) trips (product
+ * rounded, then added; a trip past k adds +0), then the partial sums meet in a binary
+ * tree, thread j taking thread j + s at s = 64, 32, ..., 1.  W is f32, or f16 when f16 != 0
+ * (decoded exactly).  No golden vector of the reference covers the order; the tests pin it
+ * with crafted cancellation cases whose answer under this order is known by hand. */
+void jlo_router_logits(float *out, const void *w, int f16, const float *x, int rows, int k, int ntok) {
+    const float *wf = (const float *)w;
+    const uint16_t *wh = (const uint16_t *)w;
+    for (int t = 0; t < ntok; t++)
+        for (int r = 0; r < rows; r++) {
+            float part[128];
+            for (int j = 0; j < 128; j++) {
+                float acc = 0.f;
+                for (int i0 = 0; i0 < k; i0 += 128) {
+                    int i = i0 + j, ic = i < k ? i : k - 1;
+                    size_t e = (size_t)r * k + ic;
+                    float wv = f16 ? jlo_half_to_f32(wh[e]) : wf[e];
+                    float prod = wv * x[(size_t)t * k + ic];
+                    acc = acc + (i < k ? prod : 0.f);
+                }
+                part[j] = acc;
+            }
+            for (int s = 64; s >= 1; s >>= 1)
+                for (int j = 0; j < s; j++) part[j] = part[j] + part[j + s];
+            out[(size_t)t * rows + r] = part[0];
+        }
+}
+
 /* internal/oracle/oracle.go:244-265 (Softmax32) then internal/oracle/moe.go:197-327
  * with Norm = true, Scale = 1, no bias, no groups, no expert scales. */
 int jlo_moe_route(const float *logits, int n, int k, int32_t *sel, float *wt, int32_t *ord,

@@ -89,6 +89,7 @@ int jlo_matvec_q8act_f32(float *out, int type, const uint8_t *w, const int8_t *q
  * logits[n] -> softmax -> top-k (score desc, index asc) -> renormalised weights.
  * sel[k], wt[k] in selection order; ord[k], owt[k] ascending expert id. */
 void jlo_rmsnorm32(float *y, const float *x, const float *w, int n, double eps);
+void jlo_router_logits(float *out, const void *w, int f16, const float *x, int rows, int k, int ntok);
 int jlo_moe_route(const float *logits, int n, int k, int32_t *sel, float *wt,
                   int32_t *ord, float *owt);
 /* jit/gpu/tier/grouppairs_test.go:91-122 (groupPairs); returns used columns */

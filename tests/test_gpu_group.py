@@ -32,8 +32,12 @@ def test_group_qkv_mixed_types_one_activation(dev, devbuf):
     x = synth.activations(k, seed=9)
     dws, dx = [devbuf(w) for w in ws], devbuf(x)
     outs = [devbuf(shape=(r + 4,), dtype=np.float32, fill=np.float32(6e30)) for _, r in spec]
+    before = dev.launch_count()
     assert dev.matvec_group_dev([o.ptr for o in outs], [t for t, _ in spec], [w.ptr for w in dws],
                                 [r for _, r in spec], dx.ptr, k)
+    # three formats, one launch (the reference's MatVecSegments,
+    # /root/reference/jit/gpu/kernels/matvec.go:1411-1431)
+    assert dev.launch_count() == before + 1
     dev.synchronize()
     for (t, r), w, o in zip(spec, ws, outs):
         got = o.get()

@@ -243,3 +243,42 @@ def test_router_vs_oracle(dev, devbuf, case):
     assert np.array_equal(got_wt.view(np.uint32), want_wt.view(np.uint32))
     # declines
     assert dev.moe_route_dev(ld.ptr, rows, 2000, k_used, sel.ptr, k_used + 1, wt.ptr) is False
+
+
+@pytest.mark.parametrize("case", [(64, 128, 2048, "f32"), (1, 128, 2048, "f16"), (13, 8, 4096, "f16"),
+                                  (9, 16, 130, "f32"), (3, 5, 100, "f32")], ids=lambda c: "x".join(map(str, c)))
+def test_router_logits_bit_exact_then_route(dev, devbuf, case):
+    """The router's own matrix product on the device (kernels.RouterMatVecTok,
+    /root/reference/jit/gpu/kernels/moe.go:820-917): f32 arithmetic in that kernel's
+    summation order, so the logits must be the oracle's BITS (ragged k, f16 weights and a
+    token count that is no multiple of the kernel's token group included); routing the device's logits on
+    the device then gives the oracle's routing of the oracle's logits: the mixture block
+    needs no host step from x to the selected experts."""
+    ntok, n_expert, k, wdt = case
+    rng = np.random.default_rng(ntok * 7 + n_expert)
+    w = rng.standard_normal((n_expert, k)).astype(np.float32) * np.float32(0.05)
+    x = rng.standard_normal((ntok, k)).astype(np.float32)
+    if wdt == "f16":
+        wh = w.astype(np.float16).view(np.uint16)
+        wd, wtype, want = devbuf(wh), 1, oracle.router_logits(wh, x, n_expert, k, ntok)
+    else:
+        wd, wtype, want = devbuf(w), 0, oracle.router_logits(w, x, n_expert, k, ntok)
+    xd = devbuf(x)
+    ld = devbuf(shape=(ntok * n_expert + 3,), dtype=np.float32, fill=np.float32(7e30))
+    assert dev.moe_logits_dev(ld.ptr, wtype, wd.ptr, xd.ptr, n_expert, k, ntok)
+    dev.synchronize()
+    got = ld.get()
+    assert np.all(got[ntok * n_expert:] == np.float32(7e30)), "wrote past the logits"
+    got = got[:ntok * n_expert].reshape(ntok, n_expert)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    k_used = min(4, n_expert)
+    sel = devbuf(shape=(ntok, k_used + 1), dtype=np.uint32, fill=0)
+    wt = devbuf(shape=(ntok, k_used), dtype=np.float32, fill=0)
+    assert dev.moe_route_dev(ld.ptr, ntok, n_expert, k_used, sel.ptr, k_used + 1, wt.ptr)
+    dev.synchronize()
+    for t in range(ntok):
+        s, wgt, _, _ = oracle.moe_route(want[t], k_used)
+        assert np.array_equal(sel.get()[t, :k_used], s.astype(np.uint32))
+        assert np.array_equal(wt.get()[t].view(np.uint32), wgt.view(np.uint32))
+    # only f32 and f16 router weights are served
+    assert dev.moe_logits_dev(ld.ptr, 8, wd.ptr, xd.ptr, n_expert, k, ntok) is False

@@ -340,6 +340,43 @@ def test_rmsnorm32_known_answers_and_invariants():
     assert np.allclose(big, x.astype(np.float64) * w / 1e6, rtol=1e-5, atol=0)
 
 
+def test_router_logits_order_pinned_by_cancellation_cases():
+    """The router's logits (/root/reference/jit/gpu/kernels/moe.go:843-917) are an f32 sum in
+    a stated order: 128 strided partial sums, then a binary tree that pairs thread j with
+    j + 64, j + 32, ...  The order only shows in roundings, so it is pinned by cases built
+    to round differently under other orders: 2^24 absorbs a lone +1 but not a +2.
+    Answers are worked out by hand from the stated order, not computed by the same code."""
+    big = np.float32(2.0 ** 24)
+    def one(places, k=256):
+        w = np.zeros((1, k), np.float32)
+        w[0, 0] = big
+        for i in places:
+            w[0, i] = 1
+        return float(oracle.router_logits(w, np.ones(k, np.float32), 1, k)[0, 0])
+    assert one([128]) == 2.0 ** 24            # same thread as the big term: added one by one, lost
+    assert one([128, 129]) == 2.0 ** 24       # threads 0 and 1; thread 1's lone 1 meets 2^24 at the last step
+    assert one([64, 192]) == 2.0 ** 24 + 2    # both in thread 64: 1 + 1 = 2 survives meeting 2^24 at s = 64
+    assert one([32, 96]) == 2.0 ** 24 + 2     # threads 32 and 96 meet each other (s = 64) before the big term (s = 32)
+    assert one([32, 64]) == 2.0 ** 24         # thread 64 meets the big term alone (s = 64), thread 32 alone (s = 32)
+    assert one([1, 2, 3]) == 2.0 ** 24 + 2    # s = 2: threads 1 and 3 make 2, thread 2's lone 1 is lost to 2^24; s = 1: 2^24 + 2
+    # a sequential sum would give 2^24 for every one of these, an f64 sum 2^24 + 2 or + 4
+    # values: against f64 on random data, ragged k (tail trips add +0), f16 weights exact
+    rng = np.random.default_rng(3)
+    for rows, k, ntok in [(5, 2048, 3), (3, 130, 2), (2, 100, 1), (4, 4097, 2)]:
+        w = rng.standard_normal((rows, k)).astype(np.float32)
+        x = rng.standard_normal((ntok, k)).astype(np.float32)
+        got = oracle.router_logits(w, x, rows, k, ntok)
+        want = x.astype(np.float64) @ w.astype(np.float64).T
+        assert np.max(np.abs(got - want)) <= 1e-5 * np.sqrt(k)
+        wh = w.astype(np.float16)
+        got16 = oracle.router_logits(wh.view(np.uint16), x, rows, k, ntok)
+        assert np.array_equal(got16, oracle.router_logits(wh.astype(np.float32), x, rows, k, ntok))
+    # small integers are exact in any order: the plain dot product
+    w = rng.integers(-8, 9, (6, 300)).astype(np.float32)
+    x = rng.integers(-8, 9, (2, 300)).astype(np.float32)
+    assert np.array_equal(oracle.router_logits(w, x, 6, 300, 2), (x.astype(np.int64) @ w.astype(np.int64).T).astype(np.float32))
+
+
 def test_moe_route_against_brute_force():
     rng = np.random.default_rng(0)
     for n, k in [(128, 8), (16, 2), (8, 1), (4, 4)]:
