@@ -167,7 +167,11 @@ int jl_matvec_q8_dev(jl_ctx *ctx, float *out, int type, const void *w, const int
  * single projection) read ONE activation x[0:k]; out[i] gets rows[i] rows of w[i] (type
  * type[i]).  act_up, when set, makes the activation silu(x) * act_up, formed on the way
  * into the quantizer (x is left as it was).  resid, when set, takes matrix 0's rows as
- * they are made: resid[r] += alpha * out[0][r].  norm_w, when set, puts an RMSNorm in
+ * they are made: resid[r] += alpha * out[0][r]; resid_gate, when set, points at one logit in
+ * device memory and the weight becomes alpha * sigmoid(*resid_gate) -- a shared expert's
+ * contribution (engine/model/moe.go:401-497; sigma in f64 narrowed once,
+ * internal/oracle/moe.go:361-370; the logit is jl_moe_logits_dev with one expert row).
+ * norm_w, when set, puts an RMSNorm in
  * front of everything, the reference's RMSNormQuantRows (jit/gpu/kernels/elem.go:252-267)
  * with the arithmetic of its host form (internal/oracle/oracle.go:230-240): the activation
  * is f32(f64(x) * 1/sqrt(mean(x^2) + norm_eps) * f64(norm_w)), mean in f64; norm_out, when
@@ -185,6 +189,7 @@ typedef struct jl_mv_group {
     const float *act_up;
     float *resid;
     float alpha;
+    const float *resid_gate;
     const float *norm_w;
     float norm_eps;
     float *norm_out;
@@ -210,7 +215,8 @@ int jl_matvec_gather_dev(jl_ctx *ctx, float *const *outs, int type, const void *
  * expert * nrows (device.go:70-80, format/jlm/write.go:165-180) -- and the activation
  * x[j*xstride : j*xstride+k] (xstride 0: one shared activation); up, when given, makes it
  * silu(x_j) * up_j; resid, when given, takes matrix 0's rows as they are made,
- * resid[r] += alpha * out[0][r] (MVGroup.Resid, engine/nn/packedgroup.go:32-36); norm_w,
+ * resid[r] += alpha * out[0][r] (MVGroup.Resid, engine/nn/packedgroup.go:32-36), alpha
+ * times sigmoid(*resid_gate) when resid_gate is given, as in jl_matvec_group_dev; norm_w,
  * when given (never together with up: JL_DECLINED), puts RMSNorm(x_j, norm_w, norm_eps) in
  * front of the quantizer (RMSNormQuantRows, jit/gpu/kernels/elem.go:252-267, with the host
  * arithmetic of internal/oracle/oracle.go:230-240) and norm_out, if not null, receives
@@ -218,8 +224,8 @@ int jl_matvec_gather_dev(jl_ctx *ctx, float *const *outs, int type, const void *
 int jl_matvec_packed_multi_dev(jl_ctx *ctx, float *const *outs, int type, const uint32_t *const *qs,
                                const uint32_t *const *d, const uint32_t *const *sc, const int *row0,
                                int stride, const float *x, size_t xstride, const float *up, float *resid,
-                               float alpha, const float *norm_w, float norm_eps, float *norm_out,
-                               int nrows, int k, int m, void *stream);
+                               float alpha, const float *resid_gate, const float *norm_w, float norm_eps,
+                               float *norm_out, int nrows, int k, int m, void *stream);
 
 /* JIT.MatMulPacked / MatMul semantics on resident operands (engine/nn/packedmm.go:23,
  * matmul.go:27): x [ntok][k] f32 -> out [ntok][nrows], every token quantized on

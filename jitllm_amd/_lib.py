@@ -27,7 +27,7 @@ class MVGroup(C.Structure):
     _fields_ = [("n", C.c_int), ("out", C.c_void_p * MAX_GROUP), ("type", C.c_int * MAX_GROUP),
                 ("w", C.c_void_p * MAX_GROUP), ("rows", C.c_int * MAX_GROUP), ("x", C.c_void_p),
                 ("k", C.c_int), ("act_up", C.c_void_p), ("resid", C.c_void_p), ("alpha", C.c_float),
-                ("norm_w", C.c_void_p), ("norm_eps", C.c_float), ("norm_out", C.c_void_p)]
+                ("resid_gate", C.c_void_p), ("norm_w", C.c_void_p), ("norm_eps", C.c_float), ("norm_out", C.c_void_p)]
 
 
 # name -> (restype, argtypes); every symbol include/jlmi.h declares
@@ -53,7 +53,7 @@ SIGNATURES = {
     "jl_matvec_gather_dev": (_int, [_vp, C.POINTER(_vp), _int, C.POINTER(_vp), _vp, _sz, _vp, _int, _int, _int,
                                     _vp]),
     "jl_matvec_packed_multi_dev": (_int, [_vp, _vp, _int, _vp, _vp, _vp, C.POINTER(C.c_int), _int, _vp, C.c_size_t,
-                                          _vp, _vp, C.c_float, _vp, C.c_float, _vp, _int, _int, _int, _vp]),
+                                          _vp, _vp, C.c_float, _vp, _vp, C.c_float, _vp, _int, _int, _int, _vp]),
     "jl_matmul_dev": (_int, [_vp, _vp, _int, _vp, _vp, _int, _int, _int, _vp]),
     "jl_reserve": (_int, [_vp, _int, _int]),
     "jl_packed_words": (_int, [_int, _int, _int, C.POINTER(_sz), C.POINTER(_sz), C.POINTER(_sz)]),

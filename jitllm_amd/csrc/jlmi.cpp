@@ -224,7 +224,7 @@ int matvec_launch(jl_ctx* c, float* out, int type, const void* w, const float* x
 int matvec_multi_launch(jl_ctx* c, int type, int m, float* const* outs, const void* const* ws, const int* rows,
                         const float* x, size_t xstride, const float* x2, float* resid, float alpha, int k,
                         hipStream_t st, const float* norm_w = nullptr, float norm_eps = 0.f,
-                        float* norm_out = nullptr, const int* types = nullptr) {
+                        float* norm_out = nullptr, const int* types = nullptr, const float* resid_gate = nullptr) {
     if (m < 1 || m > JL_MAX_MULTI) return fail(c, JL_ERR_ARG, "matvec multi: %d matrices", m);
     const TypeInfo* ti = nullptr;
     const TypeInfo* tis[JL_MAX_MULTI];
@@ -250,7 +250,8 @@ int matvec_multi_launch(jl_ctx* c, int type, int m, float* const* outs, const vo
         a.type[i] = types ? types[i] : type;
         a.row_bytes_of[i] = (k / tis[i]->block_elems) * tis[i]->block_bytes;
     }
-    a.x = x; a.x2 = x2; a.resid = resid; a.alpha = alpha; a.xstride = xstride;
+    a.x = x; a.x2 = x2; a.resid = resid; a.alpha = alpha; a.resid_gate = resid ? resid_gate : nullptr;
+    a.xstride = xstride;
     a.norm_w = norm_w; a.norm_eps = norm_eps; a.norm_out = norm_out;
     a.k = k; a.row_bytes = (k / ti->block_elems) * ti->block_bytes; a.per = c->act_window / 32;
     // sixteen wavefronts a workgroup, one row each; about two workgroups per CU over all
@@ -553,8 +554,8 @@ int packed_matvec_launch(jl_ctx* c, float* out, int type, const PlaneRef& pl, co
 // own planes and first row, reading x + j * xstride; up gates the activation.
 int packed_matvec_multi_launch(jl_ctx* c, int type, int m, float* const* outs, const PlaneRef* pls,
                                const float* x, size_t xstride, const float* up, float* resid, float alpha,
-                               const float* norm_w, float norm_eps, float* norm_out, int nrows, int k,
-                               hipStream_t st) {
+                               const float* resid_gate, const float* norm_w, float norm_eps, float* norm_out,
+                               int nrows, int k, hipStream_t st) {
     if (m < 1 || m > JL_MAX_MULTI) return fail(c, JL_ERR_ARG, "packed multi: %d matrices", m);
     // the norm precedes gate and up, the gated activation precedes down: never both
     if (norm_w && (up || !aligned16(norm_w) || (norm_out && !aligned16(norm_out)))) return JL_DECLINED;
@@ -584,6 +585,7 @@ int packed_matvec_multi_launch(jl_ctx* c, int type, int m, float* const* outs, c
         a.out[j] = outs[j]; a.qs[j] = pls[j].qs; a.d[j] = pls[j].d; a.sc[j] = pls[j].sc; a.row0[j] = pls[j].row;
     }
     a.x = x; a.x2 = up; a.xstride = xstride; a.resid = resid; a.alpha = alpha;
+    a.resid_gate = resid ? resid_gate : nullptr;
     a.norm_w = norm_w; a.norm_eps = norm_eps; a.norm_out = norm_w ? norm_out : nullptr;
     a.nrows = nrows; a.k = k; a.stride = pls[0].stride; a.per = c->act_window / 32;
     a.nwaves = nw; a.ngroups = (nrows + rw - 1) / rw;
@@ -945,14 +947,15 @@ int jl_matvec_group_dev(jl_ctx* c, const jl_mv_group* g, void* stream) {
     bool mixed = false;
     for (int i = 1; i < g->n; i++) mixed = mixed || g->type[i] != g->type[0];
     return matvec_multi_launch(c, g->type[0], g->n, g->out, g->w, g->rows, g->x, 0, g->act_up, g->resid, g->alpha,
-                               g->k, st, g->norm_w, g->norm_eps, g->norm_out, mixed ? g->type : nullptr);
+                               g->k, st, g->norm_w, g->norm_eps, g->norm_out, mixed ? g->type : nullptr,
+                               g->resid_gate);
 }
 
 int jl_matvec_packed_multi_dev(jl_ctx* c, float* const* outs, int type, const uint32_t* const* qs,
                                const uint32_t* const* d, const uint32_t* const* sc, const int* row0, int stride,
                                const float* x, size_t xstride, const float* up, float* resid, float alpha,
-                               const float* norm_w, float norm_eps, float* norm_out, int nrows, int k, int m,
-                               void* stream) {
+                               const float* resid_gate, const float* norm_w, float norm_eps, float* norm_out,
+                               int nrows, int k, int m, void* stream) {
     if (!c) return JL_ERR_ARG;
     if (!outs || !qs || !d || !row0 || m < 1) return fail(c, JL_ERR_ARG, "packed multi: bad operand");
     if (m > JL_MAX_MULTI) return JL_DECLINED;
@@ -962,8 +965,8 @@ int jl_matvec_packed_multi_dev(jl_ctx* c, float* const* outs, int type, const ui
         pls[j].qs = qs[j]; pls[j].d = d[j]; pls[j].sc = sc ? sc[j] : nullptr;
         pls[j].row = row0[j]; pls[j].stride = stride;
     }
-    return packed_matvec_multi_launch(c, type, m, outs, pls, x, xstride, up, resid, alpha, norm_w, norm_eps,
-                                      norm_out, nrows, k, pick_stream(c, stream));
+    return packed_matvec_multi_launch(c, type, m, outs, pls, x, xstride, up, resid, alpha, resid_gate, norm_w,
+                                      norm_eps, norm_out, nrows, k, pick_stream(c, stream));
 }
 
 int jl_matvec_multi_dev(jl_ctx* c, float* const* outs, int type, const void* const* ws, const float* x,

@@ -31,6 +31,7 @@ struct MatVecMultiArgs {
     const float* x2;     // null: plain activation
     float* resid;        // null: none
     float alpha;
+    const float* resid_gate;   // null, or one logit: the residual weight is alpha * sigmoid(*resid_gate)
     size_t xstride;      // elements
     int k, row_bytes, per, nwaves, ngroups;
     // the mixed-type kernel only: each matrix's type (JL_TYPE_*) and bytes per row
@@ -258,6 +259,7 @@ struct PackedMultiArgs {
     int nrows, k, stride, per, nwaves, ngroups;
     float* resid;         // null: none; else resid[r] += alpha * out[0][r] (matrix 0 only)
     float alpha;
+    const float* resid_gate;    // null, or one logit: the residual weight is alpha * sigmoid(*resid_gate)
     const float* norm_w;  // norm kernels only: RMSNorm weights [k]; every x_j is normed ahead of its quantizer
     float* norm_out;      // null, or where matrix 0's normed activation goes
     float norm_eps;

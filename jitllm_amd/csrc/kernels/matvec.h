@@ -421,6 +421,14 @@ __device__ __forceinline__ double wave_sum_f64(double v) {
     return v;
 }
 
+// Weight of a residual add: alpha, or alpha * sigmoid(logit) when the add is gated by a
+// logit in device memory (a shared expert's contribution, engine/model/moe.go:401-497;
+// sigma(x) = 1/(1+exp(-x)) in f64, narrowed once, internal/oracle/moe.go:361-370).
+__device__ __forceinline__ float resid_weight(float alpha, const float* gate) {
+    if (!gate) return alpha;
+    return alpha * (float)(1.0 / (1.0 + exp(-(double)*gate)));
+}
+
 template <int TYPE>
 __device__ __forceinline__ void matvec_multi_body(const MatVecMultiArgs& p, uint8_t* smem, int row_bytes) {
     typedef SlotTraits<TYPE> T;
@@ -494,7 +502,7 @@ __device__ __forceinline__ void matvec_multi_body(const MatVecMultiArgs& p, uint
         const float t = wave_sum_to_lane63(acc);
         if (lane == 63) {
             p.out[y][r0] = t;
-            if (y == 0 && p.resid) p.resid[r0] += p.alpha * t;
+            if (y == 0 && p.resid) p.resid[r0] += resid_weight(p.alpha, p.resid_gate) * t;
         }
     }
 }

@@ -495,6 +495,7 @@ __device__ __forceinline__ void packed_matvec_multi_body(const PackedMultiArgs& 
     p.q = nullptr; p.as = nullptr; p.s16 = nullptr;
     p.nrows = m.nrows; p.k = m.k; p.row0 = m.row0[y]; p.stride = m.stride;
     p.per = m.per; p.nwaves = m.nwaves; p.ngroups = m.ngroups;
-    p.resid = y == 0 ? m.resid : nullptr; p.alpha = m.alpha;
+    p.resid = y == 0 ? m.resid : nullptr;
+    p.alpha = y == 0 && m.resid ? resid_weight(m.alpha, m.resid_gate) : 0.f;
     packed_matvec_body<TYPE, RW, XPRE, true, GATED, NORM>(p, smem);
 }

@@ -188,16 +188,16 @@ class Device:
                             "jl_matvec_q8_dev")
 
     def matvec_group_dev(self, outs, types, ws, rows, x, k, act_up=None, resid=None, alpha=0.0, stream=None,
-                         norm_w=None, norm_eps=0.0, norm_out=None):
+                         norm_w=None, norm_eps=0.0, norm_out=None, resid_gate=None):
         """JIT.MatVecPackedGroup: up to four matvecs reading one activation, optional
-        RMSNorm(x) * norm_w first, optional silu(x) * act_up and resid += alpha * out[0], in
-        one launch per weight type."""
+        RMSNorm(x) * norm_w first, optional silu(x) * act_up and resid += alpha * out[0]
+        (alpha * sigmoid(*resid_gate) when a device logit gates the add), in one launch."""
         g = _lib.MVGroup()
         g.n = len(outs)
         for i in range(g.n):
             g.out[i], g.type[i], g.w[i], g.rows[i] = _ptr(outs[i]), types[i], _ptr(ws[i]), rows[i]
         g.x, g.k, g.act_up, g.resid, g.alpha = _ptr(x), k, _opt(act_up), _opt(resid), alpha
-        g.norm_w, g.norm_eps, g.norm_out = _opt(norm_w), norm_eps, _opt(norm_out)
+        g.norm_w, g.norm_eps, g.norm_out, g.resid_gate = _opt(norm_w), norm_eps, _opt(norm_out), _opt(resid_gate)
         return self._served(self._l.jl_matvec_group_dev(self._ctx, C.byref(g), stream), "jl_matvec_group_dev")
 
     def matvec_gather_dev(self, outs, t, ws, x, xstride, up, nrows, k, stream=None):
@@ -209,17 +209,17 @@ class Device:
                                                          nrows, k, m, stream), "jl_matvec_gather_dev")
 
     def matvec_packed_multi_dev(self, outs, t, planes, row0, stride, x, xstride, up, nrows, k, stream=None,
-                                resid=None, alpha=0.0, norm_w=None, norm_eps=0.0, norm_out=None):
+                                resid=None, alpha=0.0, norm_w=None, norm_eps=0.0, norm_out=None, resid_gate=None):
         """MatVecPackedMulti / Gather / GatherAct over packed planes: planes is a list of
         (qs, d, sc) device pointers, row0 the first row of each matrix in its buffer;
         resid += alpha * out[0] rides on the launch when given, and norm_w puts an RMSNorm
         in front of the quantizer (not together with up)."""
         return self.packed_multi_call(self.packed_multi_args(outs, t, planes, row0, stride, x, xstride, up,
-                                                             nrows, k, resid, alpha, norm_w, norm_eps, norm_out),
-                                      stream)
+                                                             nrows, k, resid, alpha, norm_w, norm_eps, norm_out,
+                                                             resid_gate), stream)
 
     def packed_multi_args(self, outs, t, planes, row0, stride, x, xstride, up, nrows, k, resid=None, alpha=0.0,
-                          norm_w=None, norm_eps=0.0, norm_out=None):
+                          norm_w=None, norm_eps=0.0, norm_out=None, resid_gate=None):
         """The argument block of a packed multi call, built once by a caller that repeats it."""
         m = len(outs)
         po = (C.c_void_p * m)(*[_ptr(o) for o in outs])
@@ -227,7 +227,7 @@ class Device:
         pd = (C.c_void_p * m)(*[_ptr(p[1]) for p in planes])
         ps = (C.c_void_p * m)(*[_opt(p[2]) for p in planes])
         pr = (C.c_int * m)(*row0)
-        return (po, t, pq, pd, ps, pr, stride, _ptr(x), xstride, _opt(up), _opt(resid), alpha, _opt(norm_w), norm_eps,
+        return (po, t, pq, pd, ps, pr, stride, _ptr(x), xstride, _opt(up), _opt(resid), alpha, _opt(resid_gate), _opt(norm_w), norm_eps,
                 _opt(norm_out), nrows, k, m)
 
     def packed_multi_call(self, args, stream=None):

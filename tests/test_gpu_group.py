@@ -147,3 +147,45 @@ def test_multi_and_gather(dev, devbuf, t):
     many = [outs[0].ptr] * 17
     assert dev.matvec_gather_dev(many, t, [dws[0].ptr] * 17, dx.ptr, 0, None, nrows, k) is False
     dev.SetActWindow(32)
+
+
+@pytest.mark.parametrize("layout", ["rows", "packed"])
+def test_shared_expert_add_gated_by_a_device_logit(dev, devbuf, layout):
+    """A shared expert's contribution (/root/reference/engine/model/moe.go:401-497): the gate
+    logit is a one-row router product on the device, the down projection adds
+    scale * sigmoid(logit) * out into the residual on its own launch, sigma in f64 narrowed
+    once (/root/reference/internal/oracle/moe.go:361-370).  The matvec is the plain matvec
+    (checked on the out it wrote), the add is exact f32 arithmetic on that out."""
+    n_embd, n_ffn, window, t = 1024, 512, 32, quant.Q8_0
+    dev.SetActWindow(window)
+    w = synth.quantized_weights(t, n_embd, n_ffn, seed=3)
+    h = synth.activations(n_ffn, seed=4)
+    xin = synth.activations(n_embd, seed=5)
+    shr = (np.random.default_rng(6).standard_normal(n_embd) * 0.05).astype(np.float32)
+    resid0 = synth.activations(n_embd, seed=7)
+    hd, xd, shd, resid = devbuf(h), devbuf(xin), devbuf(shr), devbuf(resid0)
+    logit = devbuf(shape=(1,), dtype=np.float32, fill=0)
+    y = devbuf(shape=(n_embd,), dtype=np.float32, fill=0)
+    assert dev.moe_logits_dev(logit.ptr, 0, shd.ptr, xd.ptr, 1, n_embd, 1)
+    scale = np.float32(0.75)
+    if layout == "rows":
+        wd = devbuf(w)
+        assert dev.matvec_group_dev([y.ptr], [t], [wd.ptr], [n_embd], hd.ptr, n_ffn, resid=resid.ptr,
+                                    alpha=float(scale), resid_gate=logit.ptr)
+    else:
+        qs, d, sc = oracle.pack_weights(t, w, n_embd, n_ffn)
+        pq, pd = devbuf(qs), devbuf(d)
+        assert dev.matvec_packed_multi_dev([y.ptr], t, [(pq.ptr, pd.ptr, None)], [0], n_embd, hd.ptr, 0, None,
+                                           n_embd, n_ffn, resid=resid.ptr, alpha=float(scale), resid_gate=logit.ptr)
+    dev.synchronize()
+    lg = logit.get()[0]
+    assert lg.view(np.uint32) == oracle.router_logits(shr, xin, 1, n_embd)[0, 0].view(np.uint32)
+    yh = y.get()
+    assert nmse(yh, _want(t, w, h, n_embd, n_ffn, window)) <= 1e-10
+    sig = np.float32(1.0 / (1.0 + np.exp(-np.float64(lg))))
+    wgt = np.float32(scale * sig)
+    want = (resid0 + (wgt * yh).astype(np.float32)).astype(np.float32)
+    got = resid.get()
+    # the device's f64 exp may differ from numpy's in its last bit, which can move the f32 weight by one ulp
+    assert np.max(np.abs(got - want)) <= 2.0 ** -22 * np.max(np.abs(yh))
+    dev.SetActWindow(32)
