@@ -56,7 +56,7 @@ struct jl_ctx {
     std::string err;
     std::mutex mu;  // serialises the host-pointer seam (one staging area per context)
     Tuning tune;
-    int gemm_min_tok = 8;  // below this a per-token matvec loop reads the weights as cheaply
+    int gemm_min_tok = 3;  // below this a per-token matvec loop is as fast (3.8 us a token against 8.9 us for up to 16)
     int num_cu = 0;
     size_t lds_limit = 0;
     unsigned long long launches = 0;   // kernels launched so far (jl_launch_count)
@@ -377,6 +377,29 @@ constexpr unsigned kGemmWideLdsBytes = 2u * 128u * 136u * 2u + 2u * 128u * 24u *
 int gemm_q4k_launch(jl_ctx* c, float* out, const void* w, const float* x, int nrows, int k, int ntok,
                     hipStream_t st) {
     int form = c->tune.gemm_form;
+    if ((form == 0 || form == 4) && ntok <= 64 && (size_t)nrows * (size_t)(k / 256) * 144 < ((size_t)1 << 32)) {
+        // few tokens: 16-row workgroups that split K over their wavefronts, one launch after
+        // the activation prep (kernels/gemm_q4k.h, "few tokens")
+        const int tok_pad = (ntok + 31) / 32 * 32, nsb = k / 256, nt = (ntok + 15) / 16;
+        int rc = gemm_ws_ensure(c, gemm_ws_need(tok_pad, k));
+        if (rc != JL_OK) return rc;
+        uint16_t* bq = (uint16_t*)c->gemm_ws;
+        float* da = (float*)((char*)c->gemm_ws + (size_t)nsb * 2 * (tok_pad / 32) * kGemmAStageBytes);
+        GemmPrepArgs pa;
+        pa.x = x; pa.bq = bq; pa.da = da; pa.ntok = ntok; pa.tok_pad = tok_pad; pa.k = k;
+        void* pp[] = {&pa};
+        rc = launch(c, "jl_gemm_prep_q4k_w16", (unsigned)nsb, (unsigned)(tok_pad / 32), 1024, 0, st, pp);
+        if (rc != JL_OK) return rc;
+        GemmArgs ga;
+        ga.out = out; ga.w = (const uint8_t*)w; ga.bq = bq; ga.da = da;
+        ga.nrows = nrows; ga.k = k; ga.ntok = ntok; ga.tok_pad = tok_pad; ga.row_bytes = nsb * 144;
+        ga.out_stride = nrows; ga.sb_per = 0;
+        void* gp[] = {&ga};
+        char name[32];
+        snprintf(name, sizeof name, "jl_gemm_q4k_few_t%d", nt);
+        return launch(c, name, (unsigned)((nrows + 15) / 16), 1, 512, 0, st, gp);
+    }
+    if (form == 4) form = 0;   // more tokens than the few-token form takes
     if (form == 0) {
         const long wide_groups = (long)((ntok + kGemmWideTok - 1) / kGemmWideTok) * ((nrows + 127) / 128);
         form = 4 * wide_groups >= 3 * (long)c->num_cu ? 2 : 1;   // one round at least three quarters full
@@ -779,7 +802,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     if (e != hipSuccess)
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
-    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_q4k_r64", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_moe_route", "jl_moe_logits", "jl_moe_group", "jl_moe_quant", "jl_moe_combine", "jl_moe_gemm_prep", "jl_moe_gemm_q4k", "jl_mxfp4_prep", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_sum_parts",
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_moe_route", "jl_moe_logits", "jl_moe_group", "jl_moe_quant", "jl_moe_combine", "jl_moe_gemm_prep", "jl_moe_gemm_q4k", "jl_mxfp4_prep", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_sum_parts",
                                       "jl_pack_weights", "jl_unpack_q4k"};
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int rw : {16, 32, 64})
@@ -872,7 +895,7 @@ int jl_set_tuning(jl_ctx* c, const char* key, int value) {
     else if (!strcmp(key, "mxfp4.rows")) c->tune.mx_rows = value;
     else if (!strcmp(key, "gemm.form")) c->tune.gemm_form = value;
     else if (!strcmp(key, "gemm.split")) c->tune.gemm_split = value;
-    else if (!strcmp(key, "gemm.min_tok")) c->gemm_min_tok = value > 0 ? value : 8;
+    else if (!strcmp(key, "gemm.min_tok")) c->gemm_min_tok = value > 0 ? value : 3;
     else return fail(c, JL_ERR_ARG, "unknown tuning key %s", key);
     return JL_OK;
 }

@@ -68,25 +68,28 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 // lane 32*((pos/8)%2) + t%32, element pos%8: positions 0..127 are the stage's weights in
 // the order the unpack emits them, 128..135 the sub-block sums' low parts, 136..143
 // their high parts.
-// grid = (k/256, tok_pad/32), block = 256: 32 tokens of one super-block.  Each wavefront
-// quantizes eight tokens (lane l owns elements 4l..4l+3) into LDS; then every wavefront
+// grid = (k/256, tok_pad/32), block = 256 (or 1024): 32 tokens of one super-block.  Each wavefront
+// quantizes eight (two) tokens (lane l owns elements 4l..4l+3) into LDS; then every wavefront
 // assembles whole fragments, 16 bytes a lane and 1 KiB contiguous a store.
 #define JL_GEMM_PREP_LDS_WORDS (32 * 65 + 32 * 8)
 // One group of 32 tokens, one super-block: load(tl) returns this lane's four elements
 // (4*lane .. 4*lane+3 of the super-block) of token tl of the group, zeros for a token that
 // does not exist.  grp of ngrp groups; da is laid [nsb][32*ngrp].
-template <class Load>
+// NW wavefronts a workgroup (4, or 16 where few tokens make the grid small and the chain of
+// tokens a wavefront quantizes one after the other is the kernel's length).
+template <int NW, class Load>
 __device__ __forceinline__ void gemm_prep_group(u32* lds, int sb, int grp, int ngrp, uint16_t* bqp, float* dap,
                                                 Load load) {
+    constexpr int TPW = 32 / NW, FPW = 16 / NW;   // tokens and fragments per wavefront
     u32* sq = lds;                       // [32 tokens][65]: 64 words of int8 + 1 pad (bank spread)
     i32* sA = (i32*)(lds + 32 * 65);     // [32 tokens][8 sub-block sums]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    f32x4 v[8];
+    f32x4 v[TPW];
 #pragma unroll
-    for (int i = 0; i < 8; i++) v[i] = load(wave * 8 + i);
+    for (int i = 0; i < TPW; i++) v[i] = load(wave * TPW + i);
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-        const int tl = wave * 8 + i;
+    for (int i = 0; i < TPW; i++) {
+        const int tl = wave * TPW + i;
         const u32 m = max(max(abs_bits(v[i].x), abs_bits(v[i].y)), max(abs_bits(v[i].z), abs_bits(v[i].w)));
         const u32 amax = wave_amax_256(m);
         float d;
@@ -102,8 +105,8 @@ __device__ __forceinline__ void gemm_prep_group(u32* lds, int sb, int grp, int n
     const int tl = lane & 31, kg = lane >> 5;
     u32x4* dst = (u32x4*)bqp;
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const int pi = wave * 4 + i, h = pi >> 3, ks = pi & 7;
+    for (int i = 0; i < FPW; i++) {
+        const int pi = wave * FPW + i, h = pi >> 3, ks = pi & 7;
         // vector (group g, word c): low nibbles' partners are elements 4c.. of sub-block 2g,
         // high nibbles' partners the same elements of sub-block 2g+1
         const int g = 2 * h + (ks >> 2), c = 2 * (ks & 3) + kg;
@@ -127,10 +130,11 @@ __device__ __forceinline__ void gemm_prep_group(u32* lds, int sb, int grp, int n
     }
 }
 
+template <int NW>
 __device__ __forceinline__ void gemm_prep_q4k_body(const GemmPrepArgs& p, u32* lds) {
     const int lane = threadIdx.x & 63;
     const int sb = blockIdx.x, grp = blockIdx.y;
-    gemm_prep_group(lds, sb, grp, p.tok_pad >> 5, p.bq, p.da, [&](int tl) {
+    gemm_prep_group<NW>(lds, sb, grp, p.tok_pad >> 5, p.bq, p.da, [&](int tl) {
         const int t = grp * 32 + tl;
         f32x4 v = f32x4{0.f, 0.f, 0.f, 0.f};
         if (t < p.ntok) v = ((const f32x4*)(p.x + (size_t)t * p.k + (size_t)sb * 256))[lane];
@@ -897,6 +901,176 @@ __device__ __forceinline__ void gemm_q4k_w16_body(const GemmW16Args& p, uint8_t*
         for (int e = 0; e < 16; e++) {
             const int t = t0 + 32 * tg + 8 * (e >> 2) + 4 * kg + (e & 3);
             if (t < p.ntok) p.out[(size_t)t * p.nrows + r] = out[j][e];
+        }
+    }
+}
+
+// ------------------------------------------------------------- few tokens
+// Up to 64 tokens (speculative decoding, small batches, the first tokens of a prompt): the
+// weights are read once at the decode matvec's pace and nothing else should cost anything.
+// The tiles above stage weights through LDS behind workgroup barriers, need a K split with a
+// second launch to fill the chip, and idle most of a 32- or 128-token tile.  Here:
+//   * the matrix instruction is v_mfma_f32_16x16x32_f16: 16 tokens x 16 rows, K = 32; a
+//     workgroup owns 16 rows and ALL tokens, so 4096 rows are 256 workgroups;
+//   * its eight wavefronts split K (wavefront w takes super-blocks w, w + 8, ...), each with
+//     its own accumulators; the eight partial tiles meet in LDS at the end and are added in
+//     wavefront order: one launch, no atomics, no second pass;
+//   * weights go from memory straight into the operand registers: lane (row r = lane % 16,
+//     kq = lane / 16) loads the 16 bytes at 16 + 64 G + 16 kq of its row's block (G = 0, 1:
+//     the super-block's halves), four 32-bit words, and word j is its operand for the
+//     half's K-step j after the usual unpack (eight nibbles -> eight f16 values sc * q);
+//   * the activations are the prefill GEMM's fragments, read where they lie: word j of lane
+//     kq is word c = 4 (kq % 2) + j of the 64-element group g = 2 G + kq / 2, whose partner
+//     values sit in fragment ks = 4 (kq / 2) + c / 2, lane-half c % 2 of stage 2 sb + G.
+// The arithmetic per super-block is the other forms': out += d_a * (d * P - dmin * M), P and M
+// exact on the matrix cores (M through one 16x16x16 instruction over the sixteen minimum
+// columns).  grid = ceil(nrows / 16), block = 512, static LDS = 8 x NT x 1 KiB.
+// Measured and not kept: two 16-row groups a workgroup (an activation operand then feeds two
+// instructions: no faster at 14336 rows, slower at 4096 where it halves the grid), and
+// copying the rows' blocks into LDS with coalesced loads first (slower by a microsecond).
+// Every load is a buffer load: a descriptor on the operand's base, a per-lane byte offset
+// formed once (the lane's row, its quarter of a K-step) and a scalar offset for everything
+// that moves (super-block, half, K-step, token tile), so the address arithmetic runs on the
+// scalar unit: at sixteen tokens the vector unit is the busiest part of this kernel.  The
+// host declines matrices of 4 GiB and more.
+template <int NT>   // NT tiles of 16 tokens: tok_pad = 32 * ceil(NT / 2) covers them
+__device__ __forceinline__ void gemm_q4k_few_body(const GemmArgs& p, float* part) {
+    typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+    typedef unsigned bl4 __attribute__((__vector_size__(16)));
+    typedef unsigned bl2 __attribute__((__vector_size__(8)));
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r16 = lane & 15, kq = lane >> 4;
+    const int r0 = blockIdx.x * 16;
+    const int nsb = p.k / 256;
+    const u32 ngrp = (u32)(p.tok_pad >> 5);
+    const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc((void*)p.w, 0, -1, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc((void*)p.bq, 0, -1, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rd = __builtin_amdgcn_make_buffer_rsrc((void*)p.da, 0, -1, 0x00020000);
+    const u32 vrow = (u32)min(r0 + r16, p.nrows - 1) * (u32)p.row_bytes;   // this lane's row
+    const u32 vq = vrow + 16u + 16u * (u32)kq;                               // its 16 bytes of a half
+    // its operand in a fragment: K-steps 4 (kq/2) + 2 (kq%2) + j/2, lane 32 (j%2) + 16 (tile%2) + r16
+    const u32 va = ((u32)(4 * (kq >> 1) + 2 * (kq & 1)) * 64u + (u32)r16) * 16u;
+    const u32 vm = ((u32)(32 * (kq >> 1) + r16)) * 16u + 8u * (u32)(kq & 1);   // in the sums' fragment
+    const u32 vd = 16u * (u32)kq;                                             // its four tokens' scales
+
+    f32x4 out[NT];
+#pragma unroll
+    for (int t = 0; t < NT; t++) out[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    struct W { u32x4 hdr, q[2]; };
+    auto load_w = [&](int sb, W& w) {
+        const u32 so = (u32)sb * 144u;
+        w.hdr = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rw, vrow, so, 0));
+        w.q[0] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rw, vq, so, 0));
+        w.q[1] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rw, vq + 64u, so, 0));
+    };
+    // activation operands of half G of super-block sb: [K-step j][token tile]
+    auto load_a = [&](int sb, int G, f16x8* af) {
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
+                const u32 so = ((((u32)(2 * sb + G) * ngrp + (u32)(t >> 1)) * JL_GEMM_ASTAGE_FRAGS + (u32)(j >> 1)) * 64u +
+                                32u * (u32)(j & 1) + 16u * (u32)(t & 1)) * 16u;
+                af[j * NT + t] = __builtin_bit_cast(f16x8, __builtin_amdgcn_raw_buffer_load_b128(rb, va, so, 0));
+            }
+    };
+    u32 mask = 0x000F000Fu, magic = 0x64006400u;
+    asm volatile("" : "+v"(mask), "+v"(magic));
+
+    W wcur, wnxt;
+    if (wave < nsb) load_w(wave, wcur);
+    for (int sb = wave; sb < nsb; sb += 8) {
+        if (sb + 8 < nsb) load_w(sb + 8, wnxt);
+        f32x4 accP[NT];
+#pragma unroll
+        for (int t = 0; t < NT; t++) accP[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int G = 0; G < 2; G++) {
+            f16x8 af[4 * NT];
+            load_a(sb, G, af);
+            // scales of sub-blocks 2s (low nibbles) and 2s+1 (high nibbles), s = 2G + kq/2,
+            // straight from the packed bytes (format/quant/dequant.go:360-365)
+            const int sh = 16 * (kq >> 1);
+            const u32 A = wcur.hdr.y >> sh, C = wcur.hdr.w >> sh;
+            u32 slo, shi;
+            if (G == 0) {
+                slo = A & 63;
+                shi = (A >> 8) & 63;
+            } else {
+                slo = (C & 0xF) | (((A >> 6) & 3) << 4);
+                shi = ((C >> 8) & 0xF) | (((A >> 14) & 3) << 4);
+            }
+            const _Float16 flo = (_Float16)(float)slo, fhi = (_Float16)(float)shi;
+            const _Float16 nlo = (_Float16)(-1024.0f * (float)slo), nhi = (_Float16)(-1024.0f * (float)shi);
+            const f16x2 mlo = {flo, flo}, mhi = {fhi, fhi}, alo = {nlo, nlo}, ahi = {nhi, nhi};
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const u32 w = wcur.q[G][j];
+                // (1024+n)*sc - 1024*sc = sc*n, exact in f16 (<= 945) through the fused multiply-add
+                const f16x2 p0 = __builtin_elementwise_fma(nib_pair(w, 0, mask, magic), mlo, alo);
+                const f16x2 p1 = __builtin_elementwise_fma(nib_pair(w, 4, mask, magic), mhi, ahi);
+                const f16x2 p2 = __builtin_elementwise_fma(nib_pair(w, 8, mask, magic), mlo, alo);
+                const f16x2 p3 = __builtin_elementwise_fma(nib_pair(w, 12, mask, magic), mhi, ahi);
+                const f16x8 wf = {p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
+#pragma unroll
+                for (int t = 0; t < NT; t++)
+                    accP[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[j * NT + t], wf, accP[t], 0, 0, 0);
+            }
+        }
+        // minimum columns: K = 16 = (m_0..m_7 against the sums' low parts, 64 m_0..m_7 against
+        // their high parts); lane kq holds columns 4 kq .. 4 kq + 3
+        f16x4 wm;
+        {
+            const float mul = (kq >> 1) ? 64.0f : 1.0f;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                u32 scj, mnj;
+                scale_min_k4(4 * (kq & 1) + i, wcur.hdr.y, wcur.hdr.z, wcur.hdr.w, scj, mnj);
+                wm[i] = (_Float16)((float)mnj * mul);
+            }
+        }
+        const float dd = half_bits_to_f32((uint16_t)(wcur.hdr.x & 0xFFFF));
+        const float dmin = half_bits_to_f32((uint16_t)(wcur.hdr.x >> 16));
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            // the sums' fragment (index 8 of the super-block's second stage): lanes 0-31 low
+            // parts, 32-63 high parts, eight sub-blocks each
+            const u32 som = ((((u32)(2 * sb + 1) * ngrp + (u32)(t >> 1)) * JL_GEMM_ASTAGE_FRAGS + 8u) * 64u +
+                             16u * (u32)(t & 1)) * 16u;
+            const f16x4 am = __builtin_bit_cast(f16x4, __builtin_amdgcn_raw_buffer_load_b64(rb, vm, som, 0));
+            const f32x4 accM = __builtin_amdgcn_mfma_f32_16x16x16f16(am, wm, f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+            // this lane's four tokens: 16 t + 4 kq + i
+            const f32x4 da = __builtin_bit_cast(
+                f32x4, __builtin_amdgcn_raw_buffer_load_b128(rd, vd, ((u32)sb * (u32)p.tok_pad + 16u * (u32)t) * 4u, 0));
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const float u = fmaf(dd, accP[t][i], -(dmin * accM[i]));
+                out[t][i] = fmaf(da[i], u, out[t][i]);
+            }
+        }
+        wcur = wnxt;
+    }
+
+    // the eight K shares, added in wavefront order; part [wave][tile][lane] of four floats
+    f32x4* pv = (f32x4*)part;
+#pragma unroll
+    for (int t = 0; t < NT; t++) pv[(wave * NT + t) * 64 + lane] = out[t];
+    __syncthreads();
+    for (int o = tid; o < NT * 64; o += 512) {
+        f32x4 s = pv[o];
+#pragma unroll
+        for (int w = 1; w < 8; w++) {
+            const f32x4 v = pv[w * NT * 64 + o];
+            s = f32x4{s.x + v.x, s.y + v.y, s.z + v.z, s.w + v.w};
+        }
+        const int t = o >> 6, l = o & 63, r = r0 + (l & 15);
+        if (r < p.nrows) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int tok = 16 * t + 4 * (l >> 4) + i;
+                if (tok < p.ntok) p.out[(size_t)tok * p.out_stride + r] = s[i];
+            }
         }
     }
 }

@@ -107,9 +107,21 @@ JL_PACKED_MULTI_KERNEL(q6k, JL_Q6_K, 64, 4) JL_PACKED_MULTI_KERNEL(q6k, JL_Q6_K,
 
 // ------------------------------------------------------------ prefill GEMM
 // grid = (k/256, tok_pad/4), block = 256: one wavefront per (token, super-block)
+// few tokens: grid = ceil(nrows / 16), block = 512; _t<NT>: up to 16 NT tokens
+#define JL_GEMM_FEW_KERNEL(NT)                                                                     \
+    extern "C" __global__ __launch_bounds__(512) void jl_gemm_q4k_few_t##NT(GemmArgs p) {          \
+        __shared__ __attribute__((aligned(16))) float part[8 * NT * 256];                          \
+        gemm_q4k_few_body<NT>(p, part);                                                            \
+    }
+JL_GEMM_FEW_KERNEL(1) JL_GEMM_FEW_KERNEL(2) JL_GEMM_FEW_KERNEL(3) JL_GEMM_FEW_KERNEL(4)
 extern "C" __global__ __launch_bounds__(256) void jl_gemm_prep_q4k(GemmPrepArgs p) {
     __shared__ u32 lds[JL_GEMM_PREP_LDS_WORDS];
-    gemm_prep_q4k_body(p, lds);
+    gemm_prep_q4k_body<4>(p, lds);
+}
+// the same with sixteen wavefronts a workgroup (few tokens): block = 1024
+extern "C" __global__ __launch_bounds__(1024) void jl_gemm_prep_q4k_w16(GemmPrepArgs p) {
+    __shared__ u32 lds[JL_GEMM_PREP_LDS_WORDS];
+    gemm_prep_q4k_body<16>(p, lds);
 }
 // grid = (tok_pad/128, ceil(nrows/64)), block = 256, two workgroups per CU; and the
 // 128-row form on 512 threads

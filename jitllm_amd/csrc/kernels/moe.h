@@ -394,7 +394,7 @@ __device__ __forceinline__ void moe_gemm_prep_body(const MoeGemmPrepArgs& p, u32
     const u32 c0 = c_lo + 32 * g;
     if (c0 >= c_hi) return;   // uniform across the workgroup
     const int slot = (int)(c_lo >> 5) + e + g;
-    gemm_prep_group(lds, sb, slot, p.nslots, p.bq, p.da, [&](int tl) {
+    gemm_prep_group<4>(lds, sb, slot, p.nslots, p.bq, p.da, [&](int tl) {
         f32x4 v = f32x4{0.f, 0.f, 0.f, 0.f};
         const u32 c = c0 + tl;
         if (c < c_hi) {

@@ -154,3 +154,44 @@ def test_matmul_fallback_is_the_per_token_loop(dev, devbuf, t, window, ntok):
     dev.synchronize()
     assert nmse(out.get(), want) <= 1e-10
     dev.SetActWindow(32)
+
+
+@pytest.mark.parametrize("shape", [(16, 4096, 4096), (1, 48, 256), (8, 130, 512), (17, 64, 2304), (33, 200, 1024),
+                                   (48, 16, 4096), (64, 1000, 2048), (5, 15, 256)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_gemm_few_tokens_vs_oracle(dev, devbuf, shape):
+    """Up to 64 tokens: 16-row workgroups on 16x16x32 matrix instructions, K split over the
+    eight wavefronts of a workgroup and summed in LDS, weights straight from memory into the
+    operand registers.  The inner sums are the same exact integers as in every other form;
+    only the order in which super-blocks are added differs (wavefront shares), so the bar is
+    the like-for-like one, NMSE <= 1e-10 against the f64 evaluation of the same int8
+    activations.  Ragged rows (not a multiple of 16), fewer super-blocks than wavefronts and
+    every token-tile count are covered; nothing is written past a token's rows."""
+    ntok, nrows, k = shape
+    dev.SetActWindow(256)
+    dev.set_tuning(gemm__form=4, gemm__min_tok=1)   # also the token counts a matvec loop would take
+    w = synth.quantized_weights(quant.Q4_K, nrows, k, seed=ntok + nrows)
+    x = np.stack([synth.activations(k, seed=50 + t) for t in range(ntok)])
+    x[0, :min(k, 512)] = 0                    # a window of zeros
+    if ntok > 2:
+        x[2] *= np.float32(37.5)              # tokens of different scale
+    wd, xd = devbuf(w), devbuf(x)
+    out = devbuf(shape=(ntok * nrows + 5,), dtype=np.float32, fill=np.float32(3e30))
+    assert dev.matmul_dev(out.ptr, quant.Q4_K, wd.ptr, xd.ptr, nrows, k, ntok)
+    dev.synchronize()
+    got = out.get()
+    assert np.all(got[ntok * nrows:] == np.float32(3e30)), "wrote past the output"
+    got = got[:ntok * nrows].reshape(ntok, nrows)
+    want = oracle.matmul_q8act_f64(quant.Q4_K, w, x, nrows, k, ntok, 256)
+    assert nmse(got, want) <= 1e-10
+    for t in (0, ntok - 1):
+        assert rel_l2(got[t], oracle.matvec_f64(quant.Q4_K, w, x[t], nrows, k)) <= 1e-2 or np.all(x[t] == 0)
+    # the tiled form on the same operands: the same integers, another order of the f32 adds
+    if ntok >= 8:
+        dev.set_tuning(gemm__form=1, gemm__rows=0)
+        out2 = devbuf(shape=(ntok * nrows,), dtype=np.float32, fill=0)
+        assert dev.matmul_dev(out2.ptr, quant.Q4_K, wd.ptr, xd.ptr, nrows, k, ntok)
+        dev.synchronize()
+        assert nmse(got, out2.get().reshape(ntok, nrows)) <= 1e-12
+    dev.set_tuning(gemm__form=0, gemm__min_tok=0)
+    dev.SetActWindow(32)
