@@ -28,7 +28,7 @@ const HipApi* H = nullptr;  // the process-wide HIP runtime, resolved by the fir
 
 struct Tuning {
     int rpw = 0, block = 0, grid = 0;
-    int packed_rw = 0, packed_block = 0;
+    int packed_rw = 0, packed_block = 0, moe_group = 0;
     int moe_shares = 0;
     int gemm_rows = 0;
     int gemm_form = 0;
@@ -802,7 +802,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     if (e != hipSuccess)
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
-    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_moe_route", "jl_moe_logits", "jl_moe_group", "jl_moe_quant", "jl_moe_combine", "jl_moe_gemm_prep", "jl_moe_gemm_q4k", "jl_mxfp4_prep", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_sum_parts",
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_moe_route", "jl_moe_logits", "jl_moe_group", "jl_moe_group2", "jl_moe_quant", "jl_moe_combine", "jl_moe_gemm_prep", "jl_moe_gemm_q4k", "jl_mxfp4_prep", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_sum_parts",
                                       "jl_pack_weights", "jl_unpack_q4k"};
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int rw : {16, 32, 64})
@@ -886,6 +886,7 @@ int jl_set_tuning(jl_ctx* c, const char* key, int value) {
     else if (!strcmp(key, "matvec.grid")) c->tune.grid = value;
     else if (!strcmp(key, "packed.rw")) c->tune.packed_rw = value;
     else if (!strcmp(key, "packed.block")) c->tune.packed_block = value;
+    else if (!strcmp(key, "moe.group")) c->tune.moe_group = value;
     else if (!strcmp(key, "moe.shares")) c->tune.moe_shares = value;
     else if (!strcmp(key, "moe.form")) c->tune.moe_form = value;
     else if (!strcmp(key, "moe.waves")) c->tune.moe_waves = value;
@@ -1128,6 +1129,12 @@ int jl_moe_group_dev(jl_ctx* c, const uint32_t* sel, int sel_stride, int rows, i
     a.sel = sel; a.start = start; a.perm = perm; a.pos = pos;
     a.sel_stride = sel_stride; a.rows = rows; a.k_used = k_used; a.n_expert = n_expert;
     void* params[] = {&a};
+    // the linear-time form where its tables fit LDS (moe.group = 1 / 2 forces a form)
+    const size_t npairs = (size_t)rows * k_used, nruns = (npairs + 63) / 64;
+    const size_t lds2 = nruns * 64 * 4 + nruns * (size_t)n_expert * 2 + ((size_t)n_expert + 32) * 4;   // JL_MOE_GROUP2_LDS
+    if (c->tune.moe_group != 1 && lds2 <= 64 * 1024)
+        return launch(c, "jl_moe_group2", 1, 1, 1024, (unsigned)lds2, pick_stream(c, stream), params);
+    if (c->tune.moe_group == 2) return fail(c, JL_ERR_ARG, "moe group: %zu pairs x %d experts do not fit the linear form", npairs, n_expert);
     return launch(c, "jl_moe_group", 1, 1, 1024, 0, pick_stream(c, stream), params);
 }
 
@@ -1146,12 +1153,13 @@ int jl_moe_combine_dev(jl_ctx* c, float* resid, const float* y, const float* wt,
     if (!resid || !y || !wt || !sel || !pos || rows <= 0 || n_embd <= 0)
         return fail(c, JL_ERR_ARG, "moe combine: bad operand");
     if (k_used <= 0 || k_used > 16 || sel_stride < k_used || rows > 65535) return JL_DECLINED;
+    if (n_embd % 4 != 0 || !aligned16(resid) || !aligned16(y)) return JL_DECLINED;   // four columns a thread
     HIP_TRY(c, H->SetDevice(c->device));
     MoeCombineArgs a;
     a.resid = resid; a.y = y; a.wt = wt; a.sel = sel; a.pos = pos;
     a.sel_stride = sel_stride; a.k_used = k_used; a.n_embd = n_embd;
     void* params[] = {&a};
-    return launch(c, "jl_moe_combine", (unsigned)((n_embd + 255) / 256), (unsigned)rows, 256, 0,
+    return launch(c, "jl_moe_combine", (unsigned)((n_embd / 4 + 255) / 256), (unsigned)rows, 256, 0,
                   pick_stream(c, stream), params);
 }
 

@@ -151,6 +151,8 @@ extern "C" __global__ __launch_bounds__(1024) void jl_moe_group(MoeGroupArgs p) 
     __shared__ __attribute__((aligned(16))) uint16_t skeys[JL_MOE_GROUP_KEYS];
     moe_group_body(p, scount, skeys);
 }
+// the linear-time form: one workgroup of 1024 threads, dynamic LDS = JL_MOE_GROUP2_LDS(pairs, experts)
+extern "C" __global__ __launch_bounds__(1024) void jl_moe_group2(MoeGroupArgs p) { moe_group2_body(p, jl_smem); }
 // grid = (ceil(k/4/256), ncols), block = 256
 extern "C" __global__ __launch_bounds__(256) void jl_moe_quant(MoeQuantArgs p) { moe_quant_body(p); }
 // grid = (row shares, n_expert, matrices), block = 512, dynamic LDS = 8 staged columns
@@ -165,7 +167,11 @@ JL_MOE_KERNEL(q8_0, JL_Q8_0, 16) JL_MOE_KERNEL(q8_0, JL_Q8_0, 32) JL_MOE_KERNEL(
 JL_MOE_KERNEL(q6k, JL_Q6_K, 4) JL_MOE_KERNEL(q6k, JL_Q6_K, 8)
 JL_MOE_KERNEL(q6k, JL_Q6_K, 16) JL_MOE_KERNEL(q6k, JL_Q6_K, 32) JL_MOE_KERNEL(q6k, JL_Q6_K, 64)
 // grid = (ceil(n_embd/256), rows), block = 256
-extern "C" __global__ __launch_bounds__(256) void jl_moe_combine(MoeCombineArgs p) { moe_combine_body(p); }
+extern "C" __global__ __launch_bounds__(256) void jl_moe_combine(MoeCombineArgs p) {
+    __shared__ float swt[16];
+    __shared__ u32 spos[16];
+    moe_combine_body(p, swt, spos);
+}
 
 // ------------------------------------------------------------------- MXFP4
 // grid = (ceil(ntok/128), ceil(nrows/128), K splits), block = 256, dynamic LDS = 4 stages of 128 x 272 B

@@ -191,18 +191,25 @@ __device__ __forceinline__ void moe_group_body(const MoeGroupArgs& p, u32* scoun
         }
     }
     // Inclusive scan of the 1024 counts laid out expert-major (so a running sum is the
-    // column order): ten doubling steps between two LDS buffers.
+    // column order): the counts change places through LDS, every wavefront scans its 64 with
+    // lane moves, and the sixteen wavefront totals are added up by whoever needs them.
     const int me = e * nseg + seg;
-    u32* src = scount;
-    u32* dst = scount + 1024;
+    u32* src = scount;            // [1024] counts in scan order, then the scanned values
+    u32* tot = scount + 1024;     // [16] wavefront totals
     src[me] = cnt;
     __syncthreads();
-    for (int off = 1; off < 1024; off <<= 1) {
-        const int i = threadIdx.x;
-        dst[i] = src[i] + (i >= off ? src[i - off] : 0u);
-        __syncthreads();
-        u32* t = src; src = dst; dst = t;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    u32 v = src[threadIdx.x];
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const u32 o = __shfl_up(v, off, 64);
+        if (lane >= off) v += o;
     }
+    if (lane == 63) tot[wave] = v;
+    __syncthreads();
+    for (int w = 0; w < wave; w++) v += tot[w];
+    src[threadIdx.x] = v;
+    __syncthreads();
     const u32 before = src[me] - cnt;
     if (e < p.n_expert) {
         if (seg == 0) p.start[e] = before;
@@ -224,6 +231,83 @@ __device__ __forceinline__ void moe_group_body(const MoeGroupArgs& p, u32* scoun
             for (int i = lo; i < hi; i++)
                 if (key_global(i) == (u32)e) place(i);
         }
+    }
+}
+
+// The same sort in time linear in the pairs, for pair lists that fit LDS with a count table
+// beside them (the form above compares every pair with every expert, all on one CU: 11 us
+// at 512 pairs and 128 experts, and growing with both).  Pairs are cut into runs of 64, one
+// per wavefront pass.  Inside a run a lane's rank among the lanes with its expert comes from
+// ballots (one round per distinct expert of the run) and the first lane of each expert notes
+// the run's count; a thread per expert then turns the counts of successive runs into running
+// sums, the expert totals are scanned, and a pair's column is its expert's first column +
+// the expert's pairs in earlier runs + its rank in its own run: (row, slot) order inside an
+// expert, no atomics.  LDS: keys and ranks [npairs] u16, counts [runs][nexp] u16, totals.
+// grid = 1, block = 1024, dynamic LDS = JL_MOE_GROUP2_LDS(npairs, nexp).
+#define JL_MOE_GROUP2_LDS(npairs, nexp) \
+    ((((npairs) + 63) / 64 * 64) * 4 + (((npairs) + 63) / 64) * (nexp) * 2 + ((nexp) + 32) * 4)
+__device__ __forceinline__ void moe_group2_body(const MoeGroupArgs& p, uint8_t* smem) {
+    const int npairs = p.rows * p.k_used, nexp = p.n_expert;
+    const int nruns = (npairs + 63) / 64, padded = nruns * 64;
+    uint16_t* skey = (uint16_t*)smem;                 // [padded]
+    uint16_t* srank = skey + padded;                  // [padded]
+    uint16_t* scnt = srank + padded;                  // [nruns][nexp], then running sums
+    u32* sstart = (u32*)(scnt + (size_t)nruns * nexp + ((nruns * nexp) & 1));   // [nexp + 1], then [16] wavefront totals
+    u32* stot = sstart + nexp + 1;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    for (int i = tid; i < nruns * nexp; i += 1024) scnt[i] = 0;
+    __syncthreads();
+    const uint64_t lt = lane ? (~0ull >> (64 - lane)) : 0ull;   // lanes below this one
+    for (int run = wave; run < nruns; run += 16) {
+        const int i = run * 64 + lane;
+        const bool valid = i < npairs;
+        u32 e = 0xFFFFu;
+        if (valid) e = min(p.sel[(i / p.k_used) * p.sel_stride + i % p.k_used], 0xFFFFu);
+        uint64_t todo = __ballot(valid && e < (u32)nexp);
+        u32 rank = 0;
+        while (todo) {
+            const int l0 = __builtin_ctzll(todo);
+            const u32 e0 = __builtin_amdgcn_readlane(e, l0);
+            const uint64_t m = __ballot(e == e0) & todo;
+            if (e == e0) rank = (u32)__builtin_popcountll(m & lt);
+            if (lane == l0) scnt[run * nexp + e0] = (uint16_t)__builtin_popcountll(m);
+            todo &= ~m;
+        }
+        skey[i] = (uint16_t)e;
+        srank[i] = (uint16_t)rank;
+    }
+    __syncthreads();
+    // per expert: counts of successive runs -> pairs in earlier runs; the total goes to the scan
+    u32 total = 0;
+    if (tid < nexp) {
+        for (int run = 0; run < nruns; run++) {
+            const u32 c = scnt[run * nexp + tid];
+            scnt[run * nexp + tid] = (uint16_t)total;
+            total += c;
+        }
+    }
+    // exclusive scan of the totals over experts (thread = expert; nexp <= 1024)
+    u32 v = total;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const u32 o = __shfl_up(v, off, 64);
+        if (lane >= off) v += o;
+    }
+    if (lane == 63) stot[wave] = v;
+    __syncthreads();
+    for (int w = 0; w < wave; w++) v += stot[w];
+    if (tid < nexp) {
+        sstart[tid] = v - total;
+        p.start[tid] = v - total;
+        if (tid == nexp - 1) p.start[nexp] = v;
+    }
+    __syncthreads();
+    for (int i = tid; i < npairs; i += 1024) {
+        const u32 e = skey[i];
+        if (e >= (u32)nexp) continue;   // an id no expert has: the pair is left out, as in the form above
+        const u32 col = sstart[e] + scnt[(i >> 6) * nexp + e] + srank[i];
+        p.perm[col] = (u32)(i / p.k_used);
+        p.pos[i] = col;
     }
 }
 
@@ -583,25 +667,30 @@ __device__ __forceinline__ void moe_gemm_q4k_body(const MoeGemmArgs& p, uint8_t*
 }
 
 // resid[r][n] += sum over the row's k_used experts, ascending expert id, of
-// wt[r][s] * y[pos[r*k_used+s]][n].  One thread per (row, n).
-__device__ __forceinline__ void moe_combine_body(const MoeCombineArgs& p) {
-    const int n = blockIdx.x * 256 + threadIdx.x;
-    const int r = blockIdx.y;
-    if (n >= p.n_embd) return;
-    // order the row's slots by expert id (k_used is small: insertion sort in registers)
-    int order[16];
-    const int ku = p.k_used;
-    for (int s = 0; s < ku; s++) order[s] = s;
-    for (int i = 1; i < ku; i++)
-        for (int j = i; j > 0 && p.sel[r * p.sel_stride + order[j]] < p.sel[r * p.sel_stride + order[j - 1]]; j--) {
-            int t = order[j]; order[j] = order[j - 1]; order[j - 1] = t;
-        }
-    float acc = p.resid[(size_t)r * p.n_embd + n];
-    for (int i = 0; i < ku; i++) {
-        const int s = order[i];
-        acc += p.wt[r * ku + s] * p.y[(size_t)p.pos[r * ku + s] * p.n_embd + n];
+// wt[r][s] * y[pos[r*k_used+s]][n].  grid = (ceil(n_embd/4/256), rows): a thread owns four
+// columns of a row.  The first k_used threads rank the row's slots by expert id (ids of a row
+// are distinct) and lay weights and positions out in that order in LDS, so every thread adds
+// in the reference's order without sorting anything itself.
+__device__ __forceinline__ void moe_combine_body(const MoeCombineArgs& p, float* swt, u32* spos) {
+    const int r = blockIdx.y, ku = p.k_used, tid = threadIdx.x;
+    if (tid < ku) {
+        const u32 mine = p.sel[r * p.sel_stride + tid];
+        int rank = 0;
+        for (int j = 0; j < ku; j++) rank += p.sel[r * p.sel_stride + j] < mine;
+        swt[rank] = p.wt[r * ku + tid];
+        spos[rank] = p.pos[r * ku + tid];
     }
-    p.resid[(size_t)r * p.n_embd + n] = acc;
+    __syncthreads();
+    const int n4 = p.n_embd >> 2, n = blockIdx.x * 256 + tid;
+    if (n >= n4) return;
+    f32x4* res = (f32x4*)(p.resid + (size_t)r * p.n_embd) + n;
+    f32x4 acc = *res;
+    for (int i = 0; i < ku; i++) {
+        const float w = swt[i];
+        const f32x4 y = ((const f32x4*)(p.y + (size_t)spos[i] * p.n_embd))[n];
+        acc = f32x4{acc.x + w * y.x, acc.y + w * y.y, acc.z + w * y.z, acc.w + w * y.w};
+    }
+    *res = acc;
 }
 
 // ---------------------------------------------------------------- router logits

@@ -38,10 +38,16 @@ def silu(g):
     return g / (1 + np.exp(-g))
 
 
+@pytest.mark.parametrize("form", [1, 2], ids=["every_pair_every_expert", "linear"])
 @pytest.mark.parametrize("mode,rows,n_expert,k_used", [("random", 12, 16, 4), ("one_expert", 9, 16, 2),
                                                        ("mostly_empty", 7, 32, 3), ("random", 5, 8, 1),
-                                                       ("random", 64, 128, 8)])
-def test_grouping_is_bit_exact(dev, devbuf, mode, rows, n_expert, k_used):
+                                                       ("random", 64, 128, 8), ("random", 300, 60, 6),
+                                                       ("random", 1, 1000, 16), ("one_expert", 129, 16, 2)])
+def test_grouping_is_bit_exact(dev, devbuf, mode, rows, n_expert, k_used, form):
+    """Both forms of the grouping kernel against the oracle's groupPairs: integer work, exact.
+    Runs of 64 pairs that end inside a row, more runs than wavefronts (300 x 6 pairs), more
+    experts than pairs and every pair on a handful of experts are among the cases."""
+    dev.set_tuning(moe__group=form)
     sel, _ = route(rows, n_expert, k_used, 3, mode)
     used, perm, col_e, pos = oracle.group_pairs(sel.reshape(-1), rows, k_used, n_expert, 1)
     assert used == rows * k_used
@@ -55,6 +61,7 @@ def test_grouping_is_bit_exact(dev, devbuf, mode, rows, n_expert, k_used):
     assert np.array_equal(start.get(), want_start)
     assert np.array_equal(dperm.get(), perm[:used])
     assert np.array_equal(dpos.get(), pos)
+    dev.set_tuning(moe__group=0)
 
 
 def _banks(t, n_expert, nrows, k, seed, planted):
