@@ -399,7 +399,31 @@ int gemm_q4k_launch(jl_ctx* c, float* out, const void* w, const float* x, int nr
         snprintf(name, sizeof name, "jl_gemm_q4k_few_t%d", nt);
         return launch(c, name, (unsigned)((nrows + 15) / 16), 1, 512, 0, st, gp);
     }
-    if (form == 4) form = 0;   // more tokens than the few-token form takes
+    const long few32_groups = (long)((nrows + 31) / 32) * ((ntok + 63) / 64);
+    if (((form == 0 && 2 * few32_groups <= 3L * c->num_cu) || (form == 5 && ntok <= 1024)) && ntok > 64 &&
+        (size_t)nrows * (size_t)(k / 256) * 144 < ((size_t)1 << 32)) {
+        // some more tokens, few enough rows: the same scheme on 32-row x 64-token workgroups,
+        // one to a CU, while the grid is at most a round and a half (4096 rows: up to 192
+        // tokens; measured against the tiled forms, 128 tokens x 4096 rows 24.6 -> 16.5 us;
+        // at 14336 rows the tiled forms win)
+        const int tok_pad = (ntok + 63) / 64 * 64, nsb = k / 256;
+        int rc = gemm_ws_ensure(c, gemm_ws_need(tok_pad, k));
+        if (rc != JL_OK) return rc;
+        uint16_t* bq = (uint16_t*)c->gemm_ws;
+        float* da = (float*)((char*)c->gemm_ws + (size_t)nsb * 2 * (tok_pad / 32) * kGemmAStageBytes);
+        GemmPrepArgs pa;
+        pa.x = x; pa.bq = bq; pa.da = da; pa.ntok = ntok; pa.tok_pad = tok_pad; pa.k = k;
+        void* pp[] = {&pa};
+        rc = launch(c, "jl_gemm_prep_q4k_w16", (unsigned)nsb, (unsigned)(tok_pad / 32), 1024, 0, st, pp);
+        if (rc != JL_OK) return rc;
+        GemmArgs ga;
+        ga.out = out; ga.w = (const uint8_t*)w; ga.bq = bq; ga.da = da;
+        ga.nrows = nrows; ga.k = k; ga.ntok = ntok; ga.tok_pad = tok_pad; ga.row_bytes = nsb * 144;
+        ga.out_stride = nrows; ga.sb_per = 0;
+        void* gp[] = {&ga};
+        return launch(c, "jl_gemm_q4k_few32", (unsigned)((nrows + 31) / 32), (unsigned)(tok_pad / 64), 512, 0, st, gp);
+    }
+    if (form == 4 || form == 5) form = 0;   // outside the few-token forms' range
     if (form == 0) {
         const long wide_groups = (long)((ntok + kGemmWideTok - 1) / kGemmWideTok) * ((nrows + 127) / 128);
         form = 4 * wide_groups >= 3 * (long)c->num_cu ? 2 : 1;   // one round at least three quarters full
@@ -802,7 +826,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     if (e != hipSuccess)
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
-    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_moe_route", "jl_moe_logits", "jl_moe_group", "jl_moe_group2", "jl_moe_quant", "jl_moe_combine", "jl_moe_gemm_prep", "jl_moe_gemm_q4k", "jl_mxfp4_prep", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_sum_parts",
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_group", "jl_moe_group2", "jl_moe_quant", "jl_moe_combine", "jl_moe_gemm_prep", "jl_moe_gemm_q4k", "jl_mxfp4_prep", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_sum_parts",
                                       "jl_pack_weights", "jl_unpack_q4k"};
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int rw : {16, 32, 64})

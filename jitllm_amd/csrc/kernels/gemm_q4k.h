@@ -1074,3 +1074,149 @@ __device__ __forceinline__ void gemm_q4k_few_body(const GemmArgs& p, float* part
         }
     }
 }
+
+// The same scheme on v_mfma_f32_32x32x16_f16 for 65..128 tokens, where the tiled forms still
+// need a K split with a second launch: a workgroup owns 32 rows and 64 tokens (NT tiles of
+// 32; grid.y = groups of 64 tokens, which read the weights again from L2), its eight
+// wavefronts split K.  Lane (row r = lane % 32, half = lane / 32) loads the 16 bytes at
+// 16 + 32 g + 16 half of its row's block for each 64-element group g: words c = 4 half + j,
+// and word j is its operand for the group's K-step j; the partner activations sit in
+// fragment ks = 4 (g % 2) + 2 half + j / 2, lane-half j % 2 of stage 2 sb + g / 2.
+// grid = (ceil(nrows / 32), ceil(ntok / 64)), block = 512, static LDS = 8 x NT x 4 KiB.
+// The kernel takes ~150 registers, one workgroup a CU; a build held to 128 (operands loaded a
+// K-step at a time, no weight prefetch) spilled and ran 1.5x slower, so the host sends only
+// grids of at most one and a half workgroups a CU here.
+template <int NT>
+__device__ __forceinline__ void gemm_q4k_few32_body(const GemmArgs& p, float* part) {
+    typedef unsigned bl4 __attribute__((__vector_size__(16)));
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r32 = lane & 31, half = lane >> 5;
+    const int r0 = blockIdx.x * 32, t0 = blockIdx.y * 64;
+    const int nsb = p.k / 256;
+    const u32 ngrp = (u32)(p.tok_pad >> 5), grp0 = (u32)(t0 >> 5);
+    const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc((void*)p.w, 0, -1, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc((void*)p.bq, 0, -1, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rd = __builtin_amdgcn_make_buffer_rsrc((void*)p.da, 0, -1, 0x00020000);
+    const u32 vrow = (u32)min(r0 + r32, p.nrows - 1) * (u32)p.row_bytes;
+    const u32 vq = vrow + 16u + 16u * (u32)half;
+    const u32 va = ((u32)(2 * half) * 64u + (u32)r32) * 16u;   // fragment 2 half (+ j / 2), lane r32 (+ 32 (j % 2))
+    const u32 vm = (u32)lane * 16u;                            // the sums' fragment as it lies
+    const u32 vd = 16u * (u32)half;                            // tokens 4 half .. 4 half + 3 of each eight
+
+    f32x16 out[NT];
+#pragma unroll
+    for (int t = 0; t < NT; t++)
+#pragma unroll
+        for (int e = 0; e < 16; e++) out[t][e] = 0.f;
+
+    struct W { u32x4 hdr, q[4]; };
+    auto load_w = [&](int sb, W& w) {
+        const u32 so = (u32)sb * 144u;
+        w.hdr = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rw, vrow, so, 0));
+#pragma unroll
+        for (int g = 0; g < 4; g++)
+            w.q[g] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rw, vq + 32u * (u32)g, so, 0));
+    };
+    u32 mask = 0x000F000Fu, magic = 0x64006400u;
+    asm volatile("" : "+v"(mask), "+v"(magic));
+
+    W wcur, wnxt;
+    if (wave < nsb) load_w(wave, wcur);
+    for (int sb = wave; sb < nsb; sb += 8) {
+        if (sb + 8 < nsb) load_w(sb + 8, wnxt);
+        f32x16 accP[NT];
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            // activation operands of the group: [K-step j][token tile]
+            f16x8 af[4 * NT];
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+#pragma unroll
+                for (int t = 0; t < NT; t++) {
+                    const u32 so = ((((u32)(2 * sb + (g >> 1)) * ngrp + grp0 + (u32)t) * JL_GEMM_ASTAGE_FRAGS +
+                                     (u32)(4 * (g & 1) + (j >> 1))) * 64u + 32u * (u32)(j & 1)) * 16u;
+                    af[j * NT + t] = __builtin_bit_cast(f16x8, __builtin_amdgcn_raw_buffer_load_b128(rb, va, so, 0));
+                }
+            // scales of sub-blocks 2g (low nibbles) and 2g+1 (high nibbles), straight from the
+            // packed bytes (format/quant/dequant.go:360-365)
+            const int sh = 16 * (g & 1);
+            const u32 A = wcur.hdr.y >> sh, C = wcur.hdr.w >> sh;
+            u32 slo, shi;
+            if ((g >> 1) == 0) {
+                slo = A & 63;
+                shi = (A >> 8) & 63;
+            } else {
+                slo = (C & 0xF) | (((A >> 6) & 3) << 4);
+                shi = ((C >> 8) & 0xF) | (((A >> 14) & 3) << 4);
+            }
+            const _Float16 flo = (_Float16)(float)slo, fhi = (_Float16)(float)shi;
+            const _Float16 nlo = (_Float16)(-1024.0f * (float)slo), nhi = (_Float16)(-1024.0f * (float)shi);
+            const f16x2 mlo = {flo, flo}, mhi = {fhi, fhi}, alo = {nlo, nlo}, ahi = {nhi, nhi};
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const u32 w = wcur.q[g][j];
+                // (1024+n)*sc - 1024*sc = sc*n, exact in f16 (<= 945) through the fused multiply-add
+                const f16x2 p0 = __builtin_elementwise_fma(nib_pair(w, 0, mask, magic), mlo, alo);
+                const f16x2 p1 = __builtin_elementwise_fma(nib_pair(w, 4, mask, magic), mhi, ahi);
+                const f16x2 p2 = __builtin_elementwise_fma(nib_pair(w, 8, mask, magic), mlo, alo);
+                const f16x2 p3 = __builtin_elementwise_fma(nib_pair(w, 12, mask, magic), mhi, ahi);
+                const f16x8 wf = {p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
+                const f32x16 czero = {0};
+#pragma unroll
+                for (int t = 0; t < NT; t++)
+                    accP[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[j * NT + t], wf, (g == 0 && j == 0) ? czero : accP[t],
+                                                                     0, 0, 0);
+            }
+        }
+        // minimum columns: lanes 0-31 hold m_0..m_7 (against the sums' low parts), lanes 32-63
+        // 64 m_0..m_7 (against their high parts)
+        f16x8 wm;
+        {
+            const float mul = half ? 64.0f : 1.0f;
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                u32 scj, mnj;
+                scale_min_k4(j, wcur.hdr.y, wcur.hdr.z, wcur.hdr.w, scj, mnj);
+                wm[j] = (_Float16)((float)mnj * mul);
+            }
+        }
+        const float dd = half_bits_to_f32((uint16_t)(wcur.hdr.x & 0xFFFF));
+        const float dmin = half_bits_to_f32((uint16_t)(wcur.hdr.x >> 16));
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            const u32 som = ((((u32)(2 * sb + 1) * ngrp + grp0 + (u32)t) * JL_GEMM_ASTAGE_FRAGS + 8u) * 64u) * 16u;
+            const f16x8 am = __builtin_bit_cast(f16x8, __builtin_amdgcn_raw_buffer_load_b128(rb, vm, som, 0));
+            const f32x16 zero = {0};
+            const f32x16 accM = __builtin_amdgcn_mfma_f32_32x32x16_f16(am, wm, zero, 0, 0, 0);
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                // tokens 8 q + 4 half + i of the tile
+                const f32x4 da = __builtin_bit_cast(
+                    f32x4, __builtin_amdgcn_raw_buffer_load_b128(
+                               rd, vd, ((u32)sb * (u32)p.tok_pad + (u32)t0 + 32u * (u32)t + 8u * (u32)q) * 4u, 0));
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int e = 4 * q + i;
+                    const float u = fmaf(dd, accP[t][e], -(dmin * accM[e]));
+                    out[t][e] = fmaf(da[i], u, out[t][e]);
+                }
+            }
+        }
+        wcur = wnxt;
+    }
+
+    // the eight K shares, added in wavefront order; part [wave][tile][register][lane]
+#pragma unroll
+    for (int t = 0; t < NT; t++)
+#pragma unroll
+        for (int e = 0; e < 16; e++) part[((wave * NT + t) * 16 + e) * 64 + lane] = out[t][e];
+    __syncthreads();
+    for (int o = tid; o < NT * 1024; o += 512) {
+        float s = part[o];
+#pragma unroll
+        for (int w = 1; w < 8; w++) s += part[w * NT * 1024 + o];
+        const int t = o >> 10, e = (o >> 6) & 15, l = o & 63, r = r0 + (l & 31);
+        const int tok = t0 + 32 * t + 8 * (e >> 2) + 4 * (l >> 5) + (e & 3);
+        if (r < p.nrows && tok < p.ntok) p.out[(size_t)tok * p.out_stride + r] = s;
+    }
+}

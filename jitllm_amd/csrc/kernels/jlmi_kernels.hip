@@ -114,6 +114,11 @@ JL_PACKED_MULTI_KERNEL(q6k, JL_Q6_K, 64, 4) JL_PACKED_MULTI_KERNEL(q6k, JL_Q6_K,
         gemm_q4k_few_body<NT>(p, part);                                                            \
     }
 JL_GEMM_FEW_KERNEL(1) JL_GEMM_FEW_KERNEL(2) JL_GEMM_FEW_KERNEL(3) JL_GEMM_FEW_KERNEL(4)
+// some more tokens: grid = (ceil(nrows / 32), ceil(ntok / 64)), block = 512
+extern "C" __global__ __launch_bounds__(512) void jl_gemm_q4k_few32(GemmArgs p) {
+    __shared__ __attribute__((aligned(16))) float part[8 * 2 * 1024];
+    gemm_q4k_few32_body<2>(p, part);
+}
 extern "C" __global__ __launch_bounds__(256) void jl_gemm_prep_q4k(GemmPrepArgs p) {
     __shared__ u32 lds[JL_GEMM_PREP_LDS_WORDS];
     gemm_prep_q4k_body<4>(p, lds);

@@ -195,3 +195,36 @@ def test_gemm_few_tokens_vs_oracle(dev, devbuf, shape):
         assert nmse(got, out2.get().reshape(ntok, nrows)) <= 1e-12
     dev.set_tuning(gemm__form=0, gemm__min_tok=0)
     dev.SetActWindow(32)
+
+
+@pytest.mark.parametrize("shape", [(128, 4096, 4096), (65, 33, 512), (100, 200, 1024), (300, 64, 768), (128, 31, 256)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_gemm_65_to_128_tokens_vs_oracle(dev, devbuf, shape):
+    """The few-token scheme on 32x32x16 matrix instructions: 32-row x 64-token workgroups, K
+    split over the wavefronts, one launch after the prep.  Chosen when the grid stays small
+    (4096 rows: 65..192 tokens); forced here (gemm.form = 5), also for 300 tokens, which
+    makes five token groups with a ragged last one.  Same bar as every form: NMSE <= 1e-10 against the f64 evaluation of the same int8
+    activations, nothing written past the output, and agreement with the tiled form."""
+    ntok, nrows, k = shape
+    dev.SetActWindow(256)
+    dev.set_tuning(gemm__form=5)
+    w = synth.quantized_weights(quant.Q4_K, nrows, k, seed=ntok + nrows)
+    x = np.stack([synth.activations(k, seed=70 + t) * np.float32(1 + t % 5) for t in range(ntok)])
+    x[ntok // 3] = 0
+    wd, xd = devbuf(w), devbuf(x)
+    out = devbuf(shape=(ntok * nrows + 5,), dtype=np.float32, fill=np.float32(3e30))
+    assert dev.matmul_dev(out.ptr, quant.Q4_K, wd.ptr, xd.ptr, nrows, k, ntok)
+    dev.synchronize()
+    got = out.get()
+    assert np.all(got[ntok * nrows:] == np.float32(3e30)), "wrote past the output"
+    got = got[:ntok * nrows].reshape(ntok, nrows)
+    want = oracle.matmul_q8act_f64(quant.Q4_K, w, x, nrows, k, ntok, 256)
+    assert nmse(got, want) <= 1e-10
+    assert np.all(got[ntok // 3] == 0)
+    dev.set_tuning(gemm__form=1)
+    out2 = devbuf(shape=(ntok * nrows,), dtype=np.float32, fill=0)
+    assert dev.matmul_dev(out2.ptr, quant.Q4_K, wd.ptr, xd.ptr, nrows, k, ntok)
+    dev.synchronize()
+    assert nmse(got, out2.get().reshape(ntok, nrows)) <= 1e-12
+    dev.set_tuning(gemm__form=0)
+    dev.SetActWindow(32)
