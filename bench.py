@@ -111,13 +111,44 @@ class Workload:
         t1 = time.perf_counter()
         return e0.elapsed_ms(e1) / steps, (t1 - t0) * 1e3 / steps
 
+    def timed_hot(self, steps):
+        """ms per step over copy 0 alone (weights cache resident)."""
+        from jitllm_amd.hipmem import Event
+        self.dev.SetActWindow(self.window)
+        for _ in range(20):
+            self.step(0)
+        self.dev.synchronize()
+        e0, e1 = Event(), Event()
+        e0.record(self.dev.stream)
+        for _ in range(steps):
+            self.step(0)
+        e1.record(self.dev.stream)
+        e1.synchronize()
+        return e0.elapsed_ms(e1) / steps
+
     def check(self):
-        """The last step's output against a dequant + f64 dot of a few rows."""
+        """The last step's output: finite everywhere, and the first rows within 2 % (of the
+        rows' RMS) of dequantize (on the device) + f64 dot with the f32 activation; the int8
+        activation accounts for a few parts in a thousand.  A sanity gate on what was
+        timed, not the parity test."""
         from jitllm_amd import quant
+        from jitllm_amd.hipmem import DeviceArray
         got = self.out.get()
         if not np.all(np.isfinite(got)):
             raise RuntimeError(f"{self.name}: non-finite output")
-        return float(np.abs(got).mean())
+        nr = min(16, self.nrows)
+        src = DeviceArray(self.w_host[:nr * quant.row_bytes(self.t, self.k)])
+        dst = DeviceArray(shape=(nr * self.k,), dtype=np.float32, fill=0)
+        if not self.dev.dequant_dev(self.t, src.ptr, dst.ptr, nr * self.k):
+            raise RuntimeError(f"{self.name}: the device declined to dequantize")
+        self.dev.synchronize()
+        want = dst.get().reshape(nr, self.k).astype(np.float64) @ self.x_host.astype(np.float64)
+        src.free()
+        dst.free()
+        err = float(np.sqrt(np.mean((got[:nr] - want) ** 2)) / max(np.sqrt(np.mean(want ** 2)), 1e-30))
+        if err > 2e-2:
+            raise RuntimeError(f"{self.name}: output differs from dequantize + dot by {err:.3e}")
+        return err
 
     def free(self):
         self.pool.free()
@@ -501,6 +532,11 @@ def main():
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get("c1"),
                      "kernel": "jl_matvec_q4k_r1", "pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2)},
     }
+    # the same launch over ONE copy of the weights (cache resident): what the memory side costs
+    head_hot = head.timed_hot(max(200, args.steps // 4))
+    line["headline_single_copy"] = {"us_per_step": round(head_hot * 1e3, 2),
+                                    "GB/s": round(head.alg_bytes / (head_hot * 1e-3) / 1e9, 1),
+                                    "weights": "single copy (cache resident); not the metric"}
     head.free()
 
     if not args.no_extra:
