@@ -826,7 +826,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     if (e != hipSuccess)
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
-    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_group", "jl_moe_group2", "jl_moe_quant", "jl_moe_combine", "jl_moe_gemm_prep", "jl_moe_gemm_q4k", "jl_mxfp4_prep", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_sum_parts",
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_group", "jl_moe_group2", "jl_moe_quant", "jl_moe_combine", "jl_moe_gemm_prep", "jl_moe_gemm_q4k", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_sum_parts",
                                       "jl_pack_weights", "jl_unpack_q4k"};
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int rw : {16, 32, 64})
@@ -1235,6 +1235,22 @@ int jl_matmul_mxfp4_bf16_dev(jl_ctx* c, float* out, const void* w, const uint16_
     hipStream_t st = pick_stream(c, stream);
     if (ntok <= 8)  // a handful of tokens: stream the rows once, no tile to fill
         return launch(c, "jl_mxfp4_matvec", (unsigned)((nrows + 3) / 4), 1, 256, 0, st, params);
+    if (ntok <= 64 && c->tune.mx_rows != 96 && c->tune.mx_rows != 128) {
+        // few tokens: 16-row workgroups whose wavefronts split K, one launch after a prep
+        // that lays the activations out in the order the block decode produces
+        const int nt = (ntok + 15) / 16, groups = (k + 127) / 128;
+        int rc = gemm_ws_ensure(c, (size_t)groups * 4 * nt * 1024);
+        if (rc != JL_OK) return rc;
+        MxPrepArgs pa;
+        pa.x = x; pa.xf = (uint16_t*)c->gemm_ws; pa.ntok = ntok; pa.tok_pad = 16 * nt; pa.k = k;
+        void* pp[] = {&pa};
+        rc = launch(c, "jl_mxfp4_prep_few", (unsigned)groups, (unsigned)nt, 256, 0, st, pp);
+        if (rc != JL_OK) return rc;
+        a.x = (const uint16_t*)c->gemm_ws; a.tok_pad = 16 * nt;
+        char name[32];
+        snprintf(name, sizeof name, "jl_mxfp4_few_t%d", nt);
+        return launch(c, name, (unsigned)((nrows + 15) / 16), 1, 512, 0, st, params);
+    }
     const unsigned lds = 2u * 128u * 264u * 2u;   // two weight stages [128][264] bf16
     if (lds > c->lds_limit) return JL_DECLINED;
     // activations into matrix-fragment order (tokens padded to whole tiles, K to whole stages)

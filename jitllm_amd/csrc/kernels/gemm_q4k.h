@@ -987,8 +987,11 @@ __device__ __forceinline__ void gemm_q4k_few_body(const GemmArgs& p, float* part
         for (int t = 0; t < NT; t++) accP[t] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int G = 0; G < 2; G++) {
+            // the half's operands go out together; left to itself the scheduler sinks each load
+            // next to its use and the loop becomes a chain of waits
             f16x8 af[4 * NT];
             load_a(sb, G, af);
+            __builtin_amdgcn_sched_barrier(0);
             // scales of sub-blocks 2s (low nibbles) and 2s+1 (high nibbles), s = 2G + kq/2,
             // straight from the packed bytes (format/quant/dequant.go:360-365)
             const int sh = 16 * (kq >> 1);

@@ -194,3 +194,12 @@ extern "C" __global__ __launch_bounds__(512) void jl_mxfp4_gemm_r96(MxGemmArgs p
 extern "C" __global__ __launch_bounds__(256) void jl_sum_parts(SumPartsArgs p) { sum_parts_body(p); }
 // grid = ceil(nrows/4), block = 256: one wavefront per row, ntok <= 8
 extern "C" __global__ __launch_bounds__(256) void jl_mxfp4_matvec(MxGemmArgs p) { mx_matvec_body(p); }
+// 9..64 tokens: prep grid = (ceil(k/128), tiles of 16 tokens), block = 256; kernel grid =
+// ceil(nrows/16), block = 512; _t<NT>: up to 16 NT tokens
+extern "C" __global__ __launch_bounds__(256) void jl_mxfp4_prep_few(MxPrepArgs p) { mx_prep_few_body(p); }
+#define JL_MX_FEW_KERNEL(NT)                                                                   \
+    extern "C" __global__ __launch_bounds__(512) void jl_mxfp4_few_t##NT(MxGemmArgs p) {       \
+        __shared__ __attribute__((aligned(16))) float part[8 * NT * 256];                      \
+        mx_few_body<NT>(p, part);                                                              \
+    }
+JL_MX_FEW_KERNEL(1) JL_MX_FEW_KERNEL(2) JL_MX_FEW_KERNEL(3) JL_MX_FEW_KERNEL(4)

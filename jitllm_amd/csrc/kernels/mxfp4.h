@@ -301,3 +301,107 @@ __device__ __forceinline__ void sum_parts_body(const SumPartsArgs& p) {
     for (int z = 1; z < p.nsplit; z++) s += p.part[(size_t)z * p.n + i];
     p.out[i] = s;
 }
+
+// ---------------------------------------------------------------- few tokens
+// 9..64 tokens: the weights (4.4 MB at 2880 x 2880) should be read once and nothing else
+// should cost; the tiled GEMM above needs a K split with a second launch there.  The scheme
+// of the Q4_K few-token kernel: v_mfma_f32_16x16x32_bf16 (16 tokens x 16 rows, K = 32), a
+// workgroup owns 16 rows and all tokens, its eight wavefronts split K and meet in LDS.
+// K is walked in groups of four blocks (128 weights).  Lane (row r = lane % 16, kq = lane / 16)
+// loads block 4 G + kq of its row whole (16 code bytes + the exponent) and K-step j of the
+// group takes code word j of every lane: a step mixes four blocks, each lane converting its
+// word with its own block's scale (the hardware conversion takes the scale per lane).  Word
+// j, byte i decodes to elements 4j+i and 16+4j+i of the block, so the lane's operand is
+//   (e[4j], e[16+4j], e[4j+1], e[16+4j+1], e[4j+2], e[16+4j+2], e[4j+3], e[16+4j+3])
+// and the prep kernel below lays the activations out in exactly that order.
+//
+// prep: x bf16 [ntok][k] -> xf [ceil(k/128) groups][4 steps][ntiles][64 lanes][8] bf16;
+// grid = (ceil(k/128), ntiles), block = 256 (thread = step j, lane); zeros past ntok and k.
+__device__ __forceinline__ void mx_prep_few_body(const MxPrepArgs& p) {
+    const int G = blockIdx.x, tile = blockIdx.y, ntiles = gridDim.y;
+    const int j = threadIdx.x >> 6, lane = threadIdx.x & 63, t = tile * 16 + (lane & 15), kq = lane >> 4;
+    const int k0 = 128 * G + 32 * kq + 4 * j;   // elements k0..k0+3 and k0+16..k0+19
+    typedef uint16_t u16x4 __attribute__((ext_vector_type(4)));
+    u16x4 lo = {0, 0, 0, 0}, hi = {0, 0, 0, 0};
+    if (t < p.ntok && k0 < p.k) {   // k % 32 == 0: a block is inside K or outside it
+        const uint16_t* src = p.x + (size_t)t * p.k + k0;
+        lo = *(const u16x4*)src;
+        hi = *(const u16x4*)(src + 16);
+    }
+    typedef uint16_t u16x8 __attribute__((ext_vector_type(8)));
+    const u16x8 o = {lo[0], hi[0], lo[1], hi[1], lo[2], hi[2], lo[3], hi[3]};
+    ((u16x8*)p.xf)[(((size_t)G * 4 + j) * ntiles + tile) * 64 + lane] = o;
+}
+
+// grid = ceil(nrows / 16), block = 512, static LDS = 8 x NT x 1 KiB; p.x is the prep's
+// workspace, p.tok_pad = 16 * NT.
+template <int NT>
+__device__ __forceinline__ void mx_few_body(const MxGemmArgs& p, float* part) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r16 = lane & 15, kq = lane >> 4;
+    const int r0 = blockIdx.x * 16;
+    const int nblk = p.k / 32, ngroups = (nblk + 3) / 4;
+    const uint8_t* wrow = p.w + (size_t)min(r0 + r16, p.nrows - 1) * p.row_bytes;
+    const u32x4* xf = (const u32x4*)p.x;
+
+    f32x4 out[NT];
+#pragma unroll
+    for (int t = 0; t < NT; t++) out[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    struct W { u32x4 q; u32 e; };
+    auto load_w = [&](int G, W& w) {
+        const int b = 4 * G + kq;
+        const uint8_t* blk = wrow + (size_t)min(b, nblk - 1) * 17;
+        w.e = blk[0];
+        w.q = ld16_a1(blk + 1);
+        if (b >= nblk) w.q = u32x4{0, 0, 0, 0};   // past the end of K: zero codes
+    };
+    W wcur, wnxt;
+    if (wave < ngroups) load_w(wave, wcur);
+    for (int G = wave; G < ngroups; G += 8) {
+        if (G + 8 < ngroups) load_w(G + 8, wnxt);
+        // the group's sixteen NT activation operands go out together; left to itself the
+        // scheduler sinks each load next to its use and the loop becomes a chain of waits
+        bf16x8 af[4 * NT];
+#pragma unroll
+        for (int i = 0; i < 4 * NT; i++)
+            af[i] = __builtin_bit_cast(bf16x8, xf[((size_t)G * 4 * NT + i) * 64 + lane]);
+        __builtin_amdgcn_sched_barrier(0);
+        const float scale = mx_scale((uint8_t)wcur.e);
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const u32 q = wcur.q[j];
+            const u32x4 wv = {__builtin_bit_cast(u32, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(q, scale, 0)),
+                              __builtin_bit_cast(u32, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(q, scale, 1)),
+                              __builtin_bit_cast(u32, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(q, scale, 2)),
+                              __builtin_bit_cast(u32, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(q, scale, 3))};
+            const bf16x8 wf = __builtin_bit_cast(bf16x8, wv);
+#pragma unroll
+            for (int t = 0; t < NT; t++)
+                out[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[j * NT + t], wf, out[t], 0, 0, 0);
+        }
+        wcur = wnxt;
+    }
+
+    // the eight K shares, added in wavefront order; part [wave][tile][lane] of four floats
+    f32x4* pv = (f32x4*)part;
+#pragma unroll
+    for (int t = 0; t < NT; t++) pv[(wave * NT + t) * 64 + lane] = out[t];
+    __syncthreads();
+    for (int o = tid; o < NT * 64; o += 512) {
+        f32x4 s = pv[o];
+#pragma unroll
+        for (int w = 1; w < 8; w++) {
+            const f32x4 v = pv[w * NT * 64 + o];
+            s = f32x4{s.x + v.x, s.y + v.y, s.z + v.z, s.w + v.w};
+        }
+        const int t = o >> 6, l = o & 63, r = r0 + (l & 15);
+        if (r < p.nrows) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int tok = 16 * t + 4 * (l >> 4) + i;
+                if (tok < p.ntok) p.out[(size_t)tok * p.nrows + r] = s[i];
+            }
+        }
+    }
+}
