@@ -1140,6 +1140,7 @@ __device__ __forceinline__ void gemm_q4k_few32_body(const GemmArgs& p, float* pa
                                      (u32)(4 * (g & 1) + (j >> 1))) * 64u + 32u * (u32)(j & 1)) * 16u;
                     af[j * NT + t] = __builtin_bit_cast(f16x8, __builtin_amdgcn_raw_buffer_load_b128(rb, va, so, 0));
                 }
+            __builtin_amdgcn_sched_barrier(0);   // the group's loads go out together, not one before each use
             // scales of sub-blocks 2g (low nibbles) and 2g+1 (high nibbles), straight from the
             // packed bytes (format/quant/dequant.go:360-365)
             const int sh = 16 * (g & 1);
