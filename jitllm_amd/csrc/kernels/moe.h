@@ -668,15 +668,18 @@ __device__ __forceinline__ void moe_gemm_q4k_body(const MoeGemmArgs& p, uint8_t*
 
 // resid[r][n] += sum over the row's k_used experts, ascending expert id, of
 // wt[r][s] * y[pos[r*k_used+s]][n].  grid = (ceil(n_embd/4/256), rows): a thread owns four
-// columns of a row.  The first k_used threads rank the row's slots by expert id (ids of a row
-// are distinct) and lay weights and positions out in that order in LDS, so every thread adds
-// in the reference's order without sorting anything itself.
+// columns of a row.  The first k_used threads rank the row's slots by expert id and lay weights
+// and positions out in that order in LDS, so every thread adds in the reference's order
+// without sorting anything itself.
 __device__ __forceinline__ void moe_combine_body(const MoeCombineArgs& p, float* swt, u32* spos) {
     const int r = blockIdx.y, ku = p.k_used, tid = threadIdx.x;
     if (tid < ku) {
         const u32 mine = p.sel[r * p.sel_stride + tid];
-        int rank = 0;
-        for (int j = 0; j < ku; j++) rank += p.sel[r * p.sel_stride + j] < mine;
+        int rank = 0;   // a stable rank: equal ids (not a valid routing) keep their slot order
+        for (int j = 0; j < ku; j++) {
+            const u32 other = p.sel[r * p.sel_stride + j];
+            rank += other < mine || (other == mine && j < tid);
+        }
         swt[rank] = p.wt[r * ku + tid];
         spos[rank] = p.pos[r * ku + tid];
     }
