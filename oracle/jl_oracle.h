@@ -21,6 +21,12 @@
  *                      the three independent forms (f32 dequant + Neumaier,
  *                      packed reader, int8-activation f64 form)
  *   MoE router / group brute force on tiny cases, edge cases of the reference
+ *   RMSNorm32          a hand-computed case, exact rational arithmetic, unit mean
+ *                      square, power-of-two scaling, the large-eps limit
+ *   router logits      the ORDER of the f32 sum by cancellation cases worked out
+ *                      by hand (2^24 absorbs a lone +1, not a +2); the VALUE
+ *                      against f64, exact small integers, f16 == f32 weights;
+ *                      the reference holds no golden vector for the order
  *   weight quantizers  NOT an oracle function: the reference has none for
  *                      Q4_K/Q6_K/MXFP4 ("parity unpinned" for the quantizer;
  *                      matmul parity is measured on the quantized bytes)
