@@ -334,14 +334,14 @@ def ffn_packed_section(dev):
             "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
 
 
-def moe_section(dev):
+def moe_section(dev, rows=64):
     """Qwen3-30B-A3B routed feed-forward block: 128 experts (gate/up 768x2048, down 2048x768,
     Q4_K), 64 rows routed top-8; one step = router logits (f32 router matrix, rows ~ N(0, 1/k)
     so the logits are ~ N(0,1)) + softmax/top-8 + group + gate/up + down + combine, all on the
     device.  Bytes = the touched experts' three sheets + router matrix + x in + resid out."""
     from jitllm_amd import quant, synth
     from jitllm_amd.hipmem import DeviceArray, Event
-    t, rows, n_expert, k_used, n_ffn, n_embd = quant.Q4_K, 64, 128, 8, 768, 2048
+    t, n_expert, k_used, n_ffn, n_embd = quant.Q4_K, 128, 8, 768, 2048
     dev.SetActWindow(256)
     rng = np.random.default_rng(0)
     x = DeviceArray(rng.standard_normal((rows, n_embd)).astype(np.float32))

@@ -677,7 +677,7 @@ int packed_matmul_launch(jl_ctx* c, float* out, int type, const PlaneRef& pl, co
 
 int moe_matvec_launch(jl_ctx* c, float* out0, float* out1, int type, const void* bank0, const void* bank1,
                       const float* x, const float* x2, const uint32_t* src, const uint32_t* start,
-                      int n_expert, int ncols, int max_cols, int nrows, int k, hipStream_t st) {
+                      int n_expert, int ncols, int nrows, int k, hipStream_t st) {
     const TypeInfo* ti = nullptr;
     int rc = matvec_check(c, type, nrows, k, &ti);
     if (rc != JL_OK) return rc;
@@ -689,37 +689,62 @@ int moe_matvec_launch(jl_ctx* c, float* out0, float* out1, int type, const void*
     const int row_bytes = (k / ti->block_elems) * ti->block_bytes;
     const size_t sheet = (size_t)nrows * row_bytes;
     if (type == JL_TYPE_Q4_K ? sheet % 16 != 0 : sheet % 2 != 0) return JL_DECLINED;
-    // Q4_K with the k-quant activation window can also run as groups of 32 columns on the
-    // matrix cores (tuning "moe.form" = 2).  Its vector work does not grow with the number of
-    // columns, but with a handful of columns per expert it is bound by the latency of the
-    // load -> dequantize -> LDS -> matrix chain at two wavefronts per SIMD and is the slower
-    // form (gate+up 145 us against 107 us at the 128-expert, 64-row shape), so it is not the
-    // default.
-    if (type == JL_TYPE_Q4_K && c->act_window == 256 && c->tune.moe_form == 2 &&
+    // Q4_K with the k-quant activation window can also run on the matrix cores (tuning
+    // "moe.form" = 2: groups of 32 columns, a wavefront to itself; 4: the prefill GEMM's tile).
+    // Their vector work does not grow with the number of columns, but with a handful of
+    // columns per expert form 2 is bound by the latency of the load -> dequantize -> LDS ->
+    // matrix chain at two wavefronts per SIMD and the dot-product kernel is the faster one.
+    // Measured at the 128-expert shape, top-8 (gate+up+down, whole block, us; forms 1 / 2 / 4):
+    //   64 rows 142 / 215 / 319    128 rows 214 / 227 / 337    160 rows 244 / 235 / 349
+    //   256 rows 366 / 243 / 352   512 rows 630 / 330 / 388    768 rows 916 / 416 / 429
+    //   1024 rows 1180 / 496 / 463                             2048 rows 2177 / 815 / 720
+    // so form 2 takes over from ten columns an expert on average and form 4 from 56.
+    const bool many_cols = c->tune.moe_form == 0 && (long)ncols >= 10L * n_expert;
+    if (type == JL_TYPE_Q4_K && c->act_window == 256 && (c->tune.moe_form == 2 || c->tune.moe_form == 4 || many_cols) &&
         4u * 19968u <= c->lds_limit) {   // JL_MOEG_WAVE_LDS
-        if (max_cols <= 0 || max_cols > ncols) max_cols = ncols;
-        const int gmax = (max_cols + 31) / 32, nslots = ncols / 32 + n_expert + 1, nsb = k / 256;
-        if ((long)n_expert * gmax > 65535) return JL_DECLINED;
+        const int nslots = ncols / 32 + n_expert + 1, nsb = k / 256;
+        const int tiles_max = ncols / 128 + n_expert;
+        if (nslots > 65535) return JL_DECLINED;
+        auto up256 = [](size_t v) { return (v + 255) & ~(size_t)255; };
         const size_t bq_bytes = (size_t)2 * nsb * nslots * kGemmAStageBytes;
-        rc = ws_ensure(c, &c->moe_q_ws, &c->moe_q_ws_bytes, bq_bytes + (size_t)nsb * nslots * 32 * 4);
+        const size_t o_wl = bq_bytes + up256((size_t)nsb * nslots * 32 * 4);
+        rc = ws_ensure(c, &c->moe_q_ws, &c->moe_q_ws_bytes, o_wl + (size_t)(4 + nslots + tiles_max) * 4);
+        if (rc != JL_OK) return rc;
+        // the work list of groups and tiles, from start[]
+        MoeWorklistArgs wa;
+        wa.start = start; wa.wl = (uint32_t*)((char*)c->moe_q_ws + o_wl);
+        wa.n_expert = n_expert; wa.nslots = nslots;
+        void* wp[] = {&wa};
+        rc = launch(c, "jl_moe_worklist", 1, 1, 1024, 0, st, wp);
         if (rc != JL_OK) return rc;
         MoeGemmPrepArgs pa;
-        pa.x = x; pa.x2 = x2; pa.src = src; pa.start = start;
+        pa.x = x; pa.x2 = x2; pa.src = src; pa.start = start; pa.wl = wa.wl;
         pa.bq = (uint16_t*)c->moe_q_ws; pa.da = (float*)((char*)c->moe_q_ws + bq_bytes);
-        pa.k = k; pa.gmax = gmax; pa.nslots = nslots;
+        pa.k = k; pa.nslots = nslots;
         void* pp[] = {&pa};
-        rc = launch(c, "jl_moe_gemm_prep", (unsigned)nsb, (unsigned)(n_expert * gmax), 256, 0, st, pp);
+        rc = launch(c, "jl_moe_gemm_prep", (unsigned)nsb, (unsigned)nslots, 256, 0, st, pp);
         if (rc != JL_OK) return rc;
         MoeGemmArgs ga;
         ga.out[0] = out0; ga.out[1] = out1;
         ga.bank[0] = (const uint8_t*)bank0; ga.bank[1] = (const uint8_t*)bank1;
-        ga.bq = pa.bq; ga.da = pa.da; ga.start = start;
+        ga.bq = pa.bq; ga.da = pa.da; ga.start = start; ga.wl = wa.wl;
         ga.sheet_bytes = sheet; ga.nrows = nrows; ga.k = k; ga.row_bytes = row_bytes;
-        ga.gmax = gmax; ga.nslots = nslots;
+        ga.nslots = nslots; ga.nmat = bank1 ? 2 : 1;
         void* gp[] = {&ga};
+        const long rtiles = (nrows + 63) / 64;
+        if ((c->tune.moe_form == 4 || (c->tune.moe_form == 0 && (long)ncols >= 56L * n_expert)) &&
+            kGemmLdsBytes <= c->lds_limit && n_expert <= 65535 && (long)tiles_max * rtiles * ga.nmat < (1L << 31)) {
+            const long work = (long)tiles_max * rtiles * ga.nmat;
+            const unsigned grid = (unsigned)std::min<long>(work, 2L * c->num_cu);
+            HIP_TRY(c, H->ModuleLaunchKernel(c->fn["jl_moe_gemm_r64"], grid, 1, 1, 256, 1, 1,
+                                             gemm_lds_bytes(64), st, gp, nullptr));
+            c->launches++;
+            return JL_OK;
+        }
         HIP_TRY(c, H->ModuleLaunchKernel(c->fn["jl_moe_gemm_q4k"], (unsigned)((nrows + 255) / 256),
-                                         (unsigned)(n_expert * gmax), bank1 ? 2u : 1u, 256, 1, 1, 4u * 19968u, st,
+                                         (unsigned)nslots, (unsigned)ga.nmat, 256, 1, 1, 4u * 19968u, st,
                                          gp, nullptr));
+        c->launches++;
         return JL_OK;
     }
     const int nslots = k / ti->slot_elems;
@@ -826,7 +851,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     if (e != hipSuccess)
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
-    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_group", "jl_moe_group2", "jl_moe_quant", "jl_moe_combine", "jl_moe_gemm_prep", "jl_moe_gemm_q4k", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_sum_parts",
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_group", "jl_moe_group2", "jl_moe_quant", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_q4k", "jl_moe_gemm_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_sum_parts",
                                       "jl_pack_weights", "jl_unpack_q4k"};
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int rw : {16, 32, 64})
@@ -1153,12 +1178,12 @@ int jl_moe_group_dev(jl_ctx* c, const uint32_t* sel, int sel_stride, int rows, i
     a.sel = sel; a.start = start; a.perm = perm; a.pos = pos;
     a.sel_stride = sel_stride; a.rows = rows; a.k_used = k_used; a.n_expert = n_expert;
     void* params[] = {&a};
-    // the linear-time form where its tables fit LDS (moe.group = 1 / 2 forces a form)
-    const size_t npairs = (size_t)rows * k_used, nruns = (npairs + 63) / 64;
-    const size_t lds2 = nruns * 64 * 4 + nruns * (size_t)n_expert * 2 + ((size_t)n_expert + 32) * 4;   // JL_MOE_GROUP2_LDS
-    if (c->tune.moe_group != 1 && lds2 <= 64 * 1024)
+    // the linear-time form (moe.group = 1 forces the one that compares every pair with every
+    // expert); a wavefront's share of the pairs is counted in 16 bits
+    const size_t npairs = (size_t)rows * k_used;
+    const size_t lds2 = 16 * (size_t)n_expert * 2 + ((size_t)n_expert + 17) * 4;   // JL_MOE_GROUP2_LDS
+    if (c->tune.moe_group != 1 && lds2 <= c->lds_limit && npairs <= 16 * 65535)
         return launch(c, "jl_moe_group2", 1, 1, 1024, (unsigned)lds2, pick_stream(c, stream), params);
-    if (c->tune.moe_group == 2) return fail(c, JL_ERR_ARG, "moe group: %zu pairs x %d experts do not fit the linear form", npairs, n_expert);
     return launch(c, "jl_moe_group", 1, 1, 1024, 0, pick_stream(c, stream), params);
 }
 
@@ -1167,7 +1192,7 @@ int jl_moe_matvec_dev(jl_ctx* c, float* out0, float* out1, int type, const void*
                       int n_expert, int ncols, int nrows, int k, void* stream) {
     if (!c) return JL_ERR_ARG;
     HIP_TRY(c, H->SetDevice(c->device));
-    return moe_matvec_launch(c, out0, out1, type, bank0, bank1, x, x2, src, start, n_expert, ncols, 0, nrows, k,
+    return moe_matvec_launch(c, out0, out1, type, bank0, bank1, x, x2, src, start, n_expert, ncols, nrows, k,
                              pick_stream(c, stream));
 }
 
@@ -1211,10 +1236,10 @@ int jl_moe_ffn_dev(jl_ctx* c, float* resid, int type, const void* gate_bank, con
     rc = jl_moe_group_dev(c, sel, sel_stride, rows, k_used, n_expert, start, perm, pos, st);
     if (rc != JL_OK) return rc;
     // gate and up: columns read the routed rows of x
-    rc = moe_matvec_launch(c, g, u, type, gate_bank, up_bank, x, nullptr, perm, start, n_expert, (int)ncols, rows, n_ffn, n_embd, st);
+    rc = moe_matvec_launch(c, g, u, type, gate_bank, up_bank, x, nullptr, perm, start, n_expert, (int)ncols, n_ffn, n_embd, st);
     if (rc != JL_OK) return rc;
     // down: the activation of column c is silu(g[c]) * u[c]
-    rc = moe_matvec_launch(c, y, nullptr, type, down_bank, nullptr, g, u, nullptr, start, n_expert, (int)ncols, rows, n_embd, n_ffn, st);
+    rc = moe_matvec_launch(c, y, nullptr, type, down_bank, nullptr, g, u, nullptr, start, n_expert, (int)ncols, n_embd, n_ffn, st);
     if (rc != JL_OK) return rc;
     return jl_moe_combine_dev(c, resid, y, wt, sel, sel_stride, pos, rows, k_used, n_embd, st);
 }

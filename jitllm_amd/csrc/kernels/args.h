@@ -68,14 +68,26 @@ struct GemmArgs {
 // gathers, quantizes and lays out the groups' activations as the prefill GEMM's fragments,
 // bq [k/128 stages][nslots][9][64 lanes][8] f16 and da [k/256][32*nslots]; the matrix kernel
 // meets them with the expert's sheet, out[mat][column][nrows].
+//
+// Most (expert, group) pairs of a grid sized for the fullest expert are empty, and an empty
+// workgroup still costs its dispatch, so the kernels walk a work list instead, written by
+// jl_moe_worklist from start[]: wl[0] = number of 128-column tiles, wl[4 + s] = expert of
+// slot s (all ones: unused), wl[4 + nslots + t] = tile t as expert | (tile of the expert << 16).
+struct MoeWorklistArgs {
+    const uint32_t* start;
+    uint32_t* wl;
+    int n_expert, nslots;
+};
+
 struct MoeGemmPrepArgs {
     const float* x;       // [.][k]
     const float* x2;      // optional: activation is silu(x) * x2
     const uint32_t* src;  // optional: column -> row of x (identity when null)
     const uint32_t* start;
+    const uint32_t* wl;
     uint16_t* bq;
     float* da;
-    int k, gmax, nslots;
+    int k, nslots;
 };
 
 struct MoeGemmArgs {
@@ -84,8 +96,9 @@ struct MoeGemmArgs {
     const uint16_t* bq;
     const float* da;
     const uint32_t* start;
+    const uint32_t* wl;
     size_t sheet_bytes;
-    int nrows, k, row_bytes, gmax, nslots;
+    int nrows, k, row_bytes, nslots, nmat;
 };
 
 // Two-pass form of the Q4_K prefill GEMM.  Pass one expands the weights once per call into

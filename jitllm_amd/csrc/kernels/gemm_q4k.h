@@ -263,8 +263,9 @@ __device__ __forceinline__ void gemm_split_slice(GemmArgs& p) {
 // epilogue) fall under the other's matrix instructions.
 // grid = (tok_pad/128, ceil(nrows/(64*RH))), block = 256*RH, dynamic LDS = two weight
 // stages [64*RH][152] f16 + row scales [2][64*RH][2] + token scales [2][128].
+// t0, r0: the tile's first token and row (a grouped launch places tiles per expert).
 template <int RH>
-__device__ __forceinline__ void gemm_q4k_body(const GemmArgs& p, uint8_t* smem) {
+__device__ __forceinline__ void gemm_q4k_body(const GemmArgs& p, uint8_t* smem, int t0, int r0) {
     constexpr int ROWS = 64 * RH, JL_GEMM_STAGE_HALFS = ROWS * JL_GEMM_STRIDE;
     _Float16* sW = (_Float16*)smem;
     float* sScale = (float*)(sW + 2 * JL_GEMM_STAGE_HALFS);
@@ -272,14 +273,14 @@ __device__ __forceinline__ void gemm_q4k_body(const GemmArgs& p, uint8_t* smem) 
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int tg = wave & 3, rh = wave >> 2;   // this wavefront: tokens 32*tg.., rows 64*rh..
-    const int t0 = blockIdx.x * JL_GEMM_TILE, r0 = blockIdx.y * ROWS;
     const int nsteps = 2 * (p.k / 256);
     // this thread's share of a weight stage
     const int srow = tid >> 2, hh = (tid >> 1) & 1, wq = tid & 1;
     const int wrow = min(r0 + srow, p.nrows - 1);
     const int arow = lane & 31, kg = lane >> 5;
     // fragment (step, ks) of this wavefront's 32 tokens
-    const size_t ngrp = (size_t)(p.tok_pad >> 5), mygrp = (size_t)(t0 >> 5) + tg;
+    // (a tile may reach past the last group of the workspace: such tokens are never stored)
+    const size_t ngrp = (size_t)(p.tok_pad >> 5), mygrp = min((size_t)(t0 >> 5) + tg, ngrp - 1);
     auto a_frag = [&](int step, int ks) {
         return ((const f16x8*)p.bq)[(((size_t)step * ngrp + mygrp) * JL_GEMM_ASTAGE_FRAGS + ks) * 64 + lane];
     };
@@ -305,7 +306,8 @@ __device__ __forceinline__ void gemm_q4k_body(const GemmArgs& p, uint8_t* smem) 
         for (int c = 0; c < 4; c++) gemm_w_word(wa, k0, c);
     }
     gemm_load_w(p, wrow, 0, 2 + hh, wq, wa);
-    float da_reg = p.da[t0 + (tid & (JL_GEMM_TILE - 1))];
+    const int da_tok = min(t0 + (tid & (JL_GEMM_TILE - 1)), p.tok_pad - 1);
+    float da_reg = p.da[da_tok];
     lds_barrier();
 
     // One stage.  HALF is the stage's half of its super-block; wcur holds the next
@@ -367,7 +369,7 @@ __device__ __forceinline__ void gemm_q4k_body(const GemmArgs& p, uint8_t* smem) 
         if (half == 1) {
             // the token scales of the next super-block (written to LDS during its first half)
             const int sb2 = min(sb + 1, p.k / 256 - 1);
-            da_reg = p.da[(size_t)sb2 * p.tok_pad + t0 + (tid & (JL_GEMM_TILE - 1))];
+            da_reg = p.da[(size_t)sb2 * p.tok_pad + da_tok];
         }
         JL_TRACE(3);
         if (half == 1) {
@@ -782,7 +784,8 @@ __device__ __forceinline__ void gemm_q4k_w16_body(const GemmW16Args& p, uint8_t*
     const int nsteps = 2 * (p.k / 256);
     const u32x4* wsrc = (const u32x4*)p.w16 + (size_t)rt * nsteps * JL_GEMM_W16_STAGE_VECS;
     const int arow = lane & 31, kg = lane >> 5;
-    const size_t ngrp = (size_t)(p.tok_pad >> 5), mygrp = (size_t)(t0 >> 5) + tg;
+    // (a tile may reach past the last group of the workspace: such tokens are never stored)
+    const size_t ngrp = (size_t)(p.tok_pad >> 5), mygrp = min((size_t)(t0 >> 5) + tg, ngrp - 1);
     auto a_frag = [&](int step, int ks) {
         return ((const f16x8*)p.bq)[(((size_t)step * ngrp + mygrp) * JL_GEMM_ASTAGE_FRAGS + ks) * 64 + lane];
     };
@@ -809,7 +812,8 @@ __device__ __forceinline__ void gemm_q4k_w16_body(const GemmW16Args& p, uint8_t*
         for (int i = 0; i < 4; i++) wv[i] = wsrc[(size_t)s1 * JL_GEMM_W16_STAGE_VECS + tid + 256 * i];
         wvaug = wsrc[(size_t)s1 * JL_GEMM_W16_STAGE_VECS + 1024 + (tid & 127)];
     }
-    float da_reg = p.da[t0 + (tid & (JL_GEMM_TILE - 1))];
+    const int da_tok = min(t0 + (tid & (JL_GEMM_TILE - 1)), p.tok_pad - 1);
+    float da_reg = p.da[da_tok];
     lds_barrier();
 
     auto stage = [&](auto HALF, int step) {
@@ -866,7 +870,7 @@ __device__ __forceinline__ void gemm_q4k_w16_body(const GemmW16Args& p, uint8_t*
         } else {
             wvaug = w2[1024 + (tid & 127)];
             const int sb2 = min(sb + 1, p.k / 256 - 1);
-            da_reg = p.da[(size_t)sb2 * p.tok_pad + t0 + (tid & (JL_GEMM_TILE - 1))];
+            da_reg = p.da[(size_t)sb2 * p.tok_pad + da_tok];
         }
         JL_TRACE(3);
         if (half == 1) {

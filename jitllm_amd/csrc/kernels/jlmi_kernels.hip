@@ -132,9 +132,11 @@ extern "C" __global__ __launch_bounds__(1024) void jl_gemm_prep_q4k_w16(GemmPrep
 // 128-row form on 512 threads
 extern "C" __global__ __launch_bounds__(256, 2) void jl_gemm_q4k_r64(GemmArgs p) {
     gemm_split_slice(p);
-    gemm_q4k_body<1>(p, jl_smem);
+    gemm_q4k_body<1>(p, jl_smem, blockIdx.x * JL_GEMM_TILE, blockIdx.y * 64);
 }
-extern "C" __global__ __launch_bounds__(512) void jl_gemm_q4k_r128(GemmArgs p) { gemm_q4k_body<2>(p, jl_smem); }
+extern "C" __global__ __launch_bounds__(512) void jl_gemm_q4k_r128(GemmArgs p) {
+    gemm_q4k_body<2>(p, jl_smem, blockIdx.x * JL_GEMM_TILE, blockIdx.y * 128);
+}
 extern "C" __global__ __launch_bounds__(512) void jl_gemm_q4k_wide(GemmArgs p) { gemm_q4k_wide_body(p, jl_smem); }
 extern "C" __global__ __launch_bounds__(256) void jl_gemm_w16_prep_q4k(GemmW16PrepArgs p) {
     __shared__ u32 raw[32 * 37];
@@ -156,7 +158,7 @@ extern "C" __global__ __launch_bounds__(1024) void jl_moe_group(MoeGroupArgs p) 
     __shared__ __attribute__((aligned(16))) uint16_t skeys[JL_MOE_GROUP_KEYS];
     moe_group_body(p, scount, skeys);
 }
-// the linear-time form: one workgroup of 1024 threads, dynamic LDS = JL_MOE_GROUP2_LDS(pairs, experts)
+// the linear-time form: one workgroup of 1024 threads, dynamic LDS = JL_MOE_GROUP2_LDS(experts)
 extern "C" __global__ __launch_bounds__(1024) void jl_moe_group2(MoeGroupArgs p) { moe_group2_body(p, jl_smem); }
 // grid = (ceil(k/4/256), ncols), block = 256
 extern "C" __global__ __launch_bounds__(256) void jl_moe_quant(MoeQuantArgs p) { moe_quant_body(p); }
@@ -189,6 +191,40 @@ extern "C" __global__ __launch_bounds__(256) void jl_moe_gemm_prep(MoeGemmPrepAr
     moe_gemm_prep_body(p, lds);
 }
 extern "C" __global__ __launch_bounds__(256, 2) void jl_moe_gemm_q4k(MoeGemmArgs p) { moe_gemm_q4k_body(p, jl_smem); }
+// Experts with many columns: the prefill GEMM's 128-token x 64-row tile placed per expert.  An
+// expert's column groups are consecutive slots of the prepared workspace, so to the tile they
+// are a token range; columns past the expert's last are computed and not stored.  The
+// workgroups stride over (row tile, column tile of the work list, matrix), so none is empty.
+// grid = up to two workgroups a CU, block = 256, dynamic LDS as jl_gemm_q4k_r64.
+extern "C" __global__ __launch_bounds__(256, 2) void jl_moe_gemm_r64(MoeGemmArgs p) {
+    const u32 rtiles = (u32)(p.nrows + 63) / 64;
+    const u32 ntiles = p.wl[0];
+    const u32 per_mat = ntiles * rtiles, total = per_mat * (u32)p.nmat;
+    for (u32 idx = blockIdx.x; idx < total; idx += gridDim.x) {   // uniform across the workgroup
+        const u32 mat = idx / per_mat, rem = idx - mat * per_mat;
+        const u32 t = rem / rtiles, rt = rem - t * rtiles;
+        const u32 ent = p.wl[4 + p.nslots + t];
+        const int e = (int)(ent & 0xFFFFu), ctile = (int)(ent >> 16);
+        const u32 c_lo = p.start[e], c_hi = p.start[e + 1];
+        const int ncol = (int)(c_hi - c_lo);
+        const int slot0 = (int)(c_lo >> 5) + e;
+        GemmArgs g;
+        g.w = p.bank[mat] + (size_t)e * p.sheet_bytes;
+        g.bq = p.bq; g.da = p.da;
+        g.nrows = p.nrows; g.k = p.k; g.row_bytes = p.row_bytes;
+        g.tok_pad = 32 * p.nslots;
+        g.ntok = 32 * slot0 + ncol;                  // tokens are positions in the workspace
+        g.out_stride = p.nrows; g.sb_per = 0;
+        g.out = p.out[mat] + ((ptrdiff_t)c_lo - (ptrdiff_t)32 * slot0) * p.nrows;   // workspace position -> column
+        gemm_q4k_body<1>(g, jl_smem, 32 * slot0 + 128 * ctile, (int)rt * 64);
+        __syncthreads();   // the tile's LDS is free for the next one
+    }
+}
+// grid = 1, block = 1024
+extern "C" __global__ __launch_bounds__(1024) void jl_moe_worklist(MoeWorklistArgs p) {
+    __shared__ u32 tot[16];
+    moe_worklist_body(p, tot);
+}
 extern "C" __global__ __launch_bounds__(512) void jl_mxfp4_gemm(MxGemmArgs p) { mx_gemm_body<4>(p, jl_smem); }
 extern "C" __global__ __launch_bounds__(512) void jl_mxfp4_gemm_r96(MxGemmArgs p) { mx_gemm_body<3>(p, jl_smem); }
 extern "C" __global__ __launch_bounds__(256) void jl_sum_parts(SumPartsArgs p) { sum_parts_body(p); }

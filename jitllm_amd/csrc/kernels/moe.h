@@ -234,55 +234,61 @@ __device__ __forceinline__ void moe_group_body(const MoeGroupArgs& p, u32* scoun
     }
 }
 
-// The same sort in time linear in the pairs, for pair lists that fit LDS with a count table
-// beside them (the form above compares every pair with every expert, all on one CU: 11 us
-// at 512 pairs and 128 experts, and growing with both).  Pairs are cut into runs of 64, one
-// per wavefront pass.  Inside a run a lane's rank among the lanes with its expert comes from
-// ballots (one round per distinct expert of the run) and the first lane of each expert notes
-// the run's count; a thread per expert then turns the counts of successive runs into running
-// sums, the expert totals are scanned, and a pair's column is its expert's first column +
-// the expert's pairs in earlier runs + its rank in its own run: (row, slot) order inside an
-// expert, no atomics.  LDS: keys and ranks [npairs] u16, counts [runs][nexp] u16, totals.
-// grid = 1, block = 1024, dynamic LDS = JL_MOE_GROUP2_LDS(npairs, nexp).
-#define JL_MOE_GROUP2_LDS(npairs, nexp) \
-    ((((npairs) + 63) / 64 * 64) * 4 + (((npairs) + 63) / 64) * (nexp) * 2 + ((nexp) + 32) * 4)
+// The same sort in time linear in the pairs (the form above compares every pair with every
+// expert, all on one CU: 11 us at 512 pairs and 128 experts, 234 us at 16,384 pairs).  The
+// pair list is cut into sixteen contiguous shares, one per wavefront, walked in runs of 64.
+// Inside a run every lane finds the lanes that hold its expert with one ballot per bit of the
+// expert id, which gives its rank among them and their number; the share's running count of
+// the expert (an LDS table the wavefront owns, so its accesses execute in order) gives the
+// pairs before the run.  A thread per expert then turns the sixteen share counts into offsets,
+// the expert totals are scanned, and a pair's column is its expert's first column + the
+// expert's pairs in earlier shares + its rank in its own share: (row, slot) order inside an
+// expert, no atomics.  The rank waits in pos[] between the passes (the same thread writes
+// and reads it).  grid = 1, block = 1024, dynamic LDS = JL_MOE_GROUP2_LDS(nexp).
+#define JL_MOE_GROUP2_LDS(nexp) (16 * (nexp) * 2 + ((nexp) + 1 + 16) * 4)
 __device__ __forceinline__ void moe_group2_body(const MoeGroupArgs& p, uint8_t* smem) {
     const int npairs = p.rows * p.k_used, nexp = p.n_expert;
-    const int nruns = (npairs + 63) / 64, padded = nruns * 64;
-    uint16_t* skey = (uint16_t*)smem;                 // [padded]
-    uint16_t* srank = skey + padded;                  // [padded]
-    uint16_t* scnt = srank + padded;                  // [nruns][nexp], then running sums
-    u32* sstart = (u32*)(scnt + (size_t)nruns * nexp + ((nruns * nexp) & 1));   // [nexp + 1], then [16] wavefront totals
-    u32* stot = sstart + nexp + 1;
+    const int nruns = (npairs + 63) / 64, runs_per = (nruns + 15) / 16;
+    uint16_t* scnt = (uint16_t*)smem;                                  // [16][nexp]
+    u32* sstart = (u32*)(scnt + 16 * nexp);                            // [nexp + 1]
+    u32* stot = sstart + nexp + 1;                                     // [16] wavefront totals
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    for (int i = tid; i < nruns * nexp; i += 1024) scnt[i] = 0;
+    int nbits = 0;
+    while ((1 << nbits) < nexp) nbits++;
+    for (int i = tid; i < 16 * nexp; i += 1024) scnt[i] = 0;
     __syncthreads();
     const uint64_t lt = lane ? (~0ull >> (64 - lane)) : 0ull;   // lanes below this one
-    for (int run = wave; run < nruns; run += 16) {
+    uint16_t* mine = scnt + wave * nexp;
+    const int run_lo = min(wave * runs_per, nruns), run_hi = min(run_lo + runs_per, nruns);
+    auto key_of = [&](int i) { return p.sel[(i / p.k_used) * p.sel_stride + i % p.k_used]; };
+    for (int run = run_lo; run < run_hi; run++) {
         const int i = run * 64 + lane;
-        const bool valid = i < npairs;
-        u32 e = 0xFFFFu;
-        if (valid) e = min(p.sel[(i / p.k_used) * p.sel_stride + i % p.k_used], 0xFFFFu);
-        uint64_t todo = __ballot(valid && e < (u32)nexp);
-        u32 rank = 0;
-        while (todo) {
-            const int l0 = __builtin_ctzll(todo);
-            const u32 e0 = __builtin_amdgcn_readlane(e, l0);
-            const uint64_t m = __ballot(e == e0) & todo;
-            if (e == e0) rank = (u32)__builtin_popcountll(m & lt);
-            if (lane == l0) scnt[run * nexp + e0] = (uint16_t)__builtin_popcountll(m);
-            todo &= ~m;
+        u32 e = 0;
+        bool valid = i < npairs;
+        if (valid) {
+            e = key_of(i);
+            valid = e < (u32)nexp;   // an id no expert has: the pair is left out, as in the form above
         }
-        skey[i] = (uint16_t)e;
-        srank[i] = (uint16_t)rank;
+        uint64_t m = __ballot(valid);
+        for (int b = 0; b < nbits; b++) {
+            const bool bit = (e >> b) & 1;
+            const uint64_t bal = __ballot(bit);
+            m &= bit ? bal : ~bal;
+        }
+        if (valid) {
+            const u32 before = mine[e];
+            p.pos[i] = before + (u32)__builtin_popcountll(m & lt);
+            if ((m & lt) == 0) mine[e] = (uint16_t)(before + (u32)__builtin_popcountll(m));
+        }
     }
     __syncthreads();
-    // per expert: counts of successive runs -> pairs in earlier runs; the total goes to the scan
+    // per expert: counts of successive shares -> pairs in earlier shares; the total goes to the scan
     u32 total = 0;
     if (tid < nexp) {
-        for (int run = 0; run < nruns; run++) {
-            const u32 c = scnt[run * nexp + tid];
-            scnt[run * nexp + tid] = (uint16_t)total;
+#pragma unroll
+        for (int w = 0; w < 16; w++) {
+            const u32 c = scnt[w * nexp + tid];
+            scnt[w * nexp + tid] = (uint16_t)total;
             total += c;
         }
     }
@@ -302,10 +308,12 @@ __device__ __forceinline__ void moe_group2_body(const MoeGroupArgs& p, uint8_t* 
         if (tid == nexp - 1) p.start[nexp] = v;
     }
     __syncthreads();
-    for (int i = tid; i < npairs; i += 1024) {
-        const u32 e = skey[i];
-        if (e >= (u32)nexp) continue;   // an id no expert has: the pair is left out, as in the form above
-        const u32 col = sstart[e] + scnt[(i >> 6) * nexp + e] + srank[i];
+    for (int run = run_lo; run < run_hi; run++) {
+        const int i = run * 64 + lane;
+        if (i >= npairs) continue;
+        const u32 e = key_of(i);
+        if (e >= (u32)nexp) continue;
+        const u32 col = sstart[e] + mine[e] + p.pos[i];
         p.perm[col] = (u32)(i / p.k_used);
         p.pos[i] = col;
     }
@@ -469,15 +477,58 @@ __device__ __forceinline__ void moe_matvec_body(const MoeMatVecArgs& p, uint8_t*
 // arithmetic applies (gemm_q4k.h): a group of up to 32 of an expert's columns is one
 // matrix operand, and the vector work is the dequantization alone, whatever the group holds.
 //
-// Activation prep: grid = (k/256, n_expert * gmax), block = 256: group g of expert e, one
+// Work list: grid = 1, block = 1024.  Expert e owns the slots from start[e]/32 + e up to the
+// next expert's first; the leading ceil(columns / 32) of them are its groups, the rest stay
+// unused, so every slot is written exactly once.  The 128-column tiles are numbered by a
+// running sum over the experts (wavefront scans, wavefront totals through LDS).
+__device__ __forceinline__ void moe_worklist_body(const MoeWorklistArgs& p, u32* tot) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    u32* slot_e = p.wl + 4;
+    u32* tiles = p.wl + 4 + p.nslots;
+    u32 base = 0;
+    for (int e0 = 0; e0 < p.n_expert; e0 += 1024) {
+        const int e = e0 + (int)threadIdx.x;
+        u32 nt = 0, c_lo = 0, ncol = 0;
+        if (e < p.n_expert) {
+            c_lo = p.start[e];
+            const u32 c_hi = p.start[e + 1];
+            ncol = c_hi - c_lo;
+            nt = (ncol + 127) >> 7;
+            const u32 s0 = (c_lo >> 5) + (u32)e, ng = (ncol + 31) >> 5;
+            const u32 s1 = e + 1 < p.n_expert ? (c_hi >> 5) + (u32)e + 1 : (u32)p.nslots;
+            for (u32 s = s0; s < s1; s++) slot_e[s] = s - s0 < ng ? (u32)e : 0xFFFFFFFFu;
+        }
+        u32 v = nt;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const u32 o = __shfl_up(v, off, 64);
+            if (lane >= off) v += o;
+        }
+        __syncthreads();   // the totals of the previous round have been read
+        if (lane == 63) tot[wave] = v;
+        __syncthreads();
+        u32 round = 0;
+        for (int w = 0; w < 16; w++) {
+            if (w < wave) v += tot[w];
+            round += tot[w];
+        }
+        const u32 first = base + v - nt;
+        for (u32 j = 0; j < nt; j++) tiles[first + j] = (u32)e | (j << 16);
+        base += round;
+    }
+    if (threadIdx.x == 0) p.wl[0] = base;
+}
+
+// Activation prep: grid = (k/256, nslots), block = 256: one group of 32 columns, one
 // super-block; tokens past the expert's last column are zeros.
 __device__ __forceinline__ void moe_gemm_prep_body(const MoeGemmPrepArgs& p, u32* lds) {
     const int lane = threadIdx.x & 63;
-    const int sb = blockIdx.x, e = blockIdx.y / p.gmax, g = blockIdx.y - e * p.gmax;
+    const int sb = blockIdx.x, slot = blockIdx.y;
+    const u32 eu = p.wl[4 + slot];
+    if (eu == 0xFFFFFFFFu) return;   // uniform across the workgroup
+    const int e = (int)eu;
     const u32 c_lo = p.start[e], c_hi = p.start[e + 1];
-    const u32 c0 = c_lo + 32 * g;
-    if (c0 >= c_hi) return;   // uniform across the workgroup
-    const int slot = (int)(c_lo >> 5) + e + g;
+    const u32 c0 = c_lo + 32 * (u32)(slot - ((int)(c_lo >> 5) + e));
     gemm_prep_group<4>(lds, sb, slot, p.nslots, p.bq, p.da, [&](int tl) {
         f32x4 v = f32x4{0.f, 0.f, 0.f, 0.f};
         const u32 c = c0 + tl;
@@ -493,7 +544,7 @@ __device__ __forceinline__ void moe_gemm_prep_body(const MoeGemmPrepArgs& p, u32
     });
 }
 
-// Matrix kernel: grid = (ceil(nrows/256), n_expert * gmax, matrices), block = 256, dynamic
+// Matrix kernel: grid = (ceil(nrows/256), nslots, matrices), block = 256, dynamic
 // LDS = 4 * JL_MOEG_WAVE_LDS.  A wavefront owns 32 columns x 64 rows and shares nothing
 // with its neighbours -- the columns are the same for the whole workgroup, the rows are its
 // own -- so it keeps a private LDS buffer to turn its dequantized weights into matrix
@@ -510,12 +561,13 @@ __device__ __forceinline__ void moe_gemm_prep_body(const MoeGemmPrepArgs& p, u32
 __device__ __forceinline__ void moe_gemm_q4k_body(const MoeGemmArgs& p, uint8_t* smem) {
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int e = blockIdx.y / p.gmax, g = blockIdx.y - e * p.gmax, mat = blockIdx.z;
+    const int slot = blockIdx.y, mat = blockIdx.z;
+    const u32 eu = p.wl[4 + slot];
+    if (eu == 0xFFFFFFFFu) return;
+    const int e = (int)eu;
     const u32 c_lo = p.start[e], c_hi = p.start[e + 1];
-    const u32 c0 = c_lo + 32 * g;
-    if (c0 >= c_hi) return;
+    const u32 c0 = c_lo + 32 * (u32)(slot - ((int)(c_lo >> 5) + e));
     const int ncol = min(32, (int)(c_hi - c0));
-    const int slot = (int)(c_lo >> 5) + e + g;
     const int r0 = blockIdx.x * 256 + wave * 64;
     if (r0 >= p.nrows) return;   // (no workgroup barrier below)
     _Float16* sW = (_Float16*)(smem + (size_t)wave * JL_MOEG_WAVE_LDS);

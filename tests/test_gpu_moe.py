@@ -42,11 +42,14 @@ def silu(g):
 @pytest.mark.parametrize("mode,rows,n_expert,k_used", [("random", 12, 16, 4), ("one_expert", 9, 16, 2),
                                                        ("mostly_empty", 7, 32, 3), ("random", 5, 8, 1),
                                                        ("random", 64, 128, 8), ("random", 300, 60, 6),
-                                                       ("random", 1, 1000, 16), ("one_expert", 129, 16, 2)])
+                                                       ("random", 1, 1000, 16), ("one_expert", 129, 16, 2),
+                                                       ("random", 2048, 128, 8), ("random", 700, 1000, 16),
+                                                       ("one_expert", 2100, 7, 2)])
 def test_grouping_is_bit_exact(dev, devbuf, mode, rows, n_expert, k_used, form):
     """Both forms of the grouping kernel against the oracle's groupPairs: integer work, exact.
     Runs of 64 pairs that end inside a row, more runs than wavefronts (300 x 6 pairs), more
-    experts than pairs and every pair on a handful of experts are among the cases."""
+    experts than pairs, every pair on a handful of experts and pair lists of many runs a
+    wavefront (16,384 pairs) are among the cases."""
     dev.set_tuning(moe__group=form)
     sel, _ = route(rows, n_expert, k_used, 3, mode)
     used, perm, col_e, pos = oracle.group_pairs(sel.reshape(-1), rows, k_used, n_expert, 1)
@@ -72,10 +75,13 @@ def _banks(t, n_expert, nrows, k, seed, planted):
 @pytest.mark.parametrize("t,nrows,k,form", [(quant.Q4_K, 96, 2048, 1), (quant.Q4_K, 200, 768, 1),
                                             (quant.Q4_K, 40, 4096, 1), (quant.Q4_K, 96, 2048, 2),
                                             (quant.Q4_K, 300, 768, 2), (quant.Q4_K, 40, 4096, 2),
+                                            (quant.Q4_K, 96, 2048, 4), (quant.Q4_K, 300, 768, 4),
+                                            (quant.Q4_K, 40, 4096, 4), (quant.Q4_K, 129, 256, 4),
                                             (quant.Q8_0, 64, 1024, 0), (quant.Q6_K, 70, 1024, 0)])
 def test_grouped_matvec_vs_oracle(dev, devbuf, t, nrows, k, form):
     """form 1 = the dot-product kernel, 2 = groups of 32 columns on the matrix cores (Q4_K with
-    the k-quant window), 0 = what the library picks."""
+    the k-quant window), 4 = the prefill GEMM's 128-column x 64-row tile placed per expert,
+    0 = what the library picks."""
     rows, n_expert, k_used, window = 13, 8, 3, 256 if t in quant.K_QUANTS else 32
     dev.SetActWindow(window)
     dev.set_tuning(moe__form=form)
@@ -124,11 +130,13 @@ def test_grouped_matvec_vs_oracle(dev, devbuf, t, nrows, k, form):
     dev.set_tuning(moe__form=0)
 
 
-def test_grouped_matmul_more_than_one_group_of_columns(dev, devbuf):
-    """An expert chosen by 70 rows has three groups of 32 columns (the last one ragged);
-    another gets one column, most get none.  Both forms against the oracle."""
+@pytest.mark.parametrize("rows", [70, 150])
+def test_grouped_matmul_more_than_one_group_of_columns(dev, devbuf, rows):
+    """An expert chosen by 70 rows has three groups of 32 columns (the last one ragged), by 150
+    rows five groups and two tiles of 128 columns; another gets one column, most get none.
+    Every form against the oracle."""
     t, nrows, k, window = quant.Q4_K, 130, 512, 256
-    rows, n_expert, k_used = 70, 6, 2
+    n_expert, k_used = 6, 2
     dev.SetActWindow(window)
     sel = np.zeros((rows, k_used + 1), np.uint32)
     sel[:, 0], sel[:, 1] = 4, 1
@@ -144,7 +152,7 @@ def test_grouped_matmul_more_than_one_group_of_columns(dev, devbuf):
         q, a_s, _ = oracle.quantize_act(x[perm[c]], window)
         want[c] = oracle.matvec_q8act_f64(t, bank[e * sheet:(e + 1) * sheet], q, a_s, nrows, k)
     b, xd, dstart, dperm = devbuf(bank), devbuf(x), devbuf(start), devbuf(perm[:used].copy())
-    for form in (1, 2):
+    for form in (1, 2, 4):
         dev.set_tuning(moe__form=form)
         o = devbuf(shape=(used * nrows + 8,), dtype=np.float32, fill=np.float32(4e30))
         assert dev.moe_matvec_dev(o.ptr, None, t, b.ptr, None, xd.ptr, None, dperm.ptr, dstart.ptr, n_expert, used,
@@ -153,6 +161,39 @@ def test_grouped_matmul_more_than_one_group_of_columns(dev, devbuf):
         got = o.get()
         assert np.all(got[used * nrows:] == np.float32(4e30))
         assert nmse(got[:used * nrows].reshape(used, nrows), want) <= 1e-10, form
+    dev.set_tuning(moe__form=0)
+    dev.SetActWindow(32)
+
+
+def test_grouped_matmul_more_experts_than_one_work_list_round(dev, devbuf):
+    """The work list of groups and tiles is written 1024 experts a round: 1100 experts, columns
+    on five of them across the rounds' border, one with two tiles of 128 columns."""
+    t, nrows, k, window = quant.Q4_K, 64, 256, 256
+    n_expert, k_used, rows = 1100, 2, 140
+    dev.SetActWindow(window)
+    sel = np.zeros((rows, k_used + 1), np.uint32)
+    sel[:, 0], sel[:, 1] = 1023, 1024
+    sel[:5, 0], sel[5:9, 1], sel[9, 0] = 3, 1099, 1025
+    used, perm, col_e, pos = oracle.group_pairs(sel.reshape(-1), rows, k_used, n_expert, 1)
+    start = np.searchsorted(col_e[:used], np.arange(n_expert + 1)).astype(np.uint32)
+    bank = np.tile(synth.random_weights(t, nrows, k, seed=9), n_expert)
+    sheet = nrows * quant.row_bytes(t, k)
+    for e in (3, 1023, 1024, 1025, 1099):   # the sheets in use differ from one another
+        bank[e * sheet:(e + 1) * sheet] = synth.random_weights(t, nrows, k, seed=100 + e)
+    x = np.stack([synth.activations(k, seed=900 + r) for r in range(rows)])
+    want = np.zeros((used, nrows))
+    for c in range(used):
+        e = int(col_e[c])
+        q, a_s, _ = oracle.quantize_act(x[perm[c]], window)
+        want[c] = oracle.matvec_q8act_f64(t, bank[e * sheet:(e + 1) * sheet], q, a_s, nrows, k)
+    b, xd, dstart, dperm = devbuf(bank), devbuf(x), devbuf(start), devbuf(perm[:used].copy())
+    for form in (1, 2, 4):
+        dev.set_tuning(moe__form=form)
+        o = devbuf(shape=(used, nrows), dtype=np.float32, fill=np.float32(4e30))
+        assert dev.moe_matvec_dev(o.ptr, None, t, b.ptr, None, xd.ptr, None, dperm.ptr, dstart.ptr, n_expert, used,
+                                  nrows, k)
+        dev.synchronize()
+        assert nmse(o.get(), want) <= 1e-10, form
     dev.set_tuning(moe__form=0)
     dev.SetActWindow(32)
 
