@@ -264,7 +264,9 @@ __device__ __forceinline__ void gemm_split_slice(GemmArgs& p) {
 // grid = (tok_pad/128, ceil(nrows/(64*RH))), block = 256*RH, dynamic LDS = two weight
 // stages [64*RH][152] f16 + row scales [2][64*RH][2] + token scales [2][128].
 // t0, r0: the tile's first token and row (a grouped launch places tiles per expert).
-template <int RH>
+// SKIP: a wavefront whose 32 tokens all lie past ntok takes its share of the dequantization
+// and the barriers and leaves the matrix work out (ragged tiles of a grouped launch).
+template <int RH, bool SKIP = false>
 __device__ __forceinline__ void gemm_q4k_body(const GemmArgs& p, uint8_t* smem, int t0, int r0) {
     constexpr int ROWS = 64 * RH, JL_GEMM_STAGE_HALFS = ROWS * JL_GEMM_STRIDE;
     _Float16* sW = (_Float16*)smem;
@@ -273,6 +275,7 @@ __device__ __forceinline__ void gemm_q4k_body(const GemmArgs& p, uint8_t* smem, 
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int tg = wave & 3, rh = wave >> 2;   // this wavefront: tokens 32*tg.., rows 64*rh..
+    const bool live = !SKIP || t0 + 32 * (__builtin_amdgcn_readfirstlane(wave) & 3) < p.ntok;   // wavefront-uniform
     const int nsteps = 2 * (p.k / 256);
     // this thread's share of a weight stage
     const int srow = tid >> 2, hh = (tid >> 1) & 1, wq = tid & 1;
@@ -339,26 +342,30 @@ __device__ __forceinline__ void gemm_q4k_body(const GemmArgs& p, uint8_t* smem, 
         const _Float16* wp0 = w + (64 * rh + arow) * JL_GEMM_STRIDE + 8 * kg;
         const int nstep = min(step + 1, nsteps - 1);
         f16x8 wf[2][2];
+        if (live) {
 #pragma unroll
-        for (int j = 0; j < 2; j++) wf[0][j] = *(const f16x8*)(wp0 + 32 * j * JL_GEMM_STRIDE);
+            for (int j = 0; j < 2; j++) wf[0][j] = *(const f16x8*)(wp0 + 32 * j * JL_GEMM_STRIDE);
+        }
         __builtin_amdgcn_sched_barrier(0);
         JL_TRACE(2);
 #pragma unroll
         for (int ks = 0; ks < 8; ks++) {
-            if (ks + 1 < 8) {
+            if (live) {
+                if (ks + 1 < 8) {
+#pragma unroll
+                    for (int j = 0; j < 2; j++)
+                        wf[(ks + 1) & 1][j] = *(const f16x8*)(wp0 + 32 * j * JL_GEMM_STRIDE + 16 * (ks + 1));
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                // (a super-block's first instruction starts from a zero accumulator operand)
+                const f32x16 czero = {0};
 #pragma unroll
                 for (int j = 0; j < 2; j++)
-                    wf[(ks + 1) & 1][j] = *(const f16x8*)(wp0 + 32 * j * JL_GEMM_STRIDE + 16 * (ks + 1));
+                    accP[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aring[ks], wf[ks & 1][j],
+                                                                     (half == 0 && ks == 0) ? czero : accP[j], 0, 0, 0);
+                aring[ks] = a_frag(nstep, ks);
+                if (ks == 0 && nhalf == 1) aaug = a_frag(nstep, 8);
             }
-            __builtin_amdgcn_sched_barrier(0);
-            // (a super-block's first instruction starts from a zero accumulator operand)
-            const f32x16 czero = {0};
-#pragma unroll
-            for (int j = 0; j < 2; j++)
-                accP[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aring[ks], wf[ks & 1][j],
-                                                                 (half == 0 && ks == 0) ? czero : accP[j], 0, 0, 0);
-            aring[ks] = a_frag(nstep, ks);
-            if (ks == 0 && nhalf == 1) aaug = a_frag(nstep, 8);
             if (has_next && (ks & 1)) gemm_w_word(wcur, wsc, ks >> 1);
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -372,7 +379,7 @@ __device__ __forceinline__ void gemm_q4k_body(const GemmArgs& p, uint8_t* smem, 
             da_reg = p.da[(size_t)sb2 * p.tok_pad + da_tok];
         }
         JL_TRACE(3);
-        if (half == 1) {
+        if (half == 1 && live) {
             // the 16 minimum columns: M, then the super-block's epilogue
             //   out += d_a * (d * P - dmin * M)
             const f32x16 zero = {0};

@@ -150,7 +150,12 @@ extern "C" __global__ __launch_bounds__(64) void jl_moe_route(MoeRouteArgs p) { 
 // grid = (experts, ceil(tokens / JL_LOGITS_TOK)), block = 128
 extern "C" __global__ __launch_bounds__(128) void jl_moe_logits(MoeLogitsArgs p) {
     __shared__ float part[JL_LOGITS_TOK * 128];
-    moe_logits_body(p, part);
+    moe_logits_body<1>(p, part);
+}
+// many tokens: grid = (ceil(experts / 8), ceil(tokens / JL_LOGITS_TOK)), block = 128
+extern "C" __global__ __launch_bounds__(128) void jl_moe_logits_e8(MoeLogitsArgs p) {
+    __shared__ float part[JL_LOGITS_TOK * 128];
+    moe_logits_body<8>(p, part);
 }
 // one workgroup of 1024 threads (n_expert <= 1024)
 extern "C" __global__ __launch_bounds__(1024) void jl_moe_group(MoeGroupArgs p) {
@@ -216,7 +221,7 @@ extern "C" __global__ __launch_bounds__(256, 2) void jl_moe_gemm_r64(MoeGemmArgs
         g.ntok = 32 * slot0 + ncol;                  // tokens are positions in the workspace
         g.out_stride = p.nrows; g.sb_per = 0;
         g.out = p.out[mat] + ((ptrdiff_t)c_lo - (ptrdiff_t)32 * slot0) * p.nrows;   // workspace position -> column
-        gemm_q4k_body<1>(g, jl_smem, 32 * slot0 + 128 * ctile, (int)rt * 64);
+        gemm_q4k_body<1, true>(g, jl_smem, 32 * slot0 + 128 * ctile, (int)rt * 64);
         __syncthreads();   // the tile's LDS is free for the next one
     }
 }

@@ -755,43 +755,60 @@ __device__ __forceinline__ void moe_combine_body(const MoeCombineArgs& p, float*
 // the sum; a ragged tail adds +0), and the 128 partial sums meet in a binary tree, thread j
 // taking thread j + s at s = 64, 32, ..., 1.  One workgroup per expert row and group of
 // JL_LOGITS_TOK tokens: the row is read once for all of them.
+// With many tokens the launch is bound by re-reading x from L2 for every expert row (2048
+// tokens x 128 experts x k = 2048: 114 us), so there a workgroup takes EB = 8 expert rows
+// for its eight tokens and every x value loaded meets eight weights (grid.x = ceil(rows/EB)).
 #define JL_LOGITS_TOK 8
+template <int EB>
 __device__ __forceinline__ void moe_logits_body(const MoeLogitsArgs& p, float* part) {
-    const int r = blockIdx.x, t0 = blockIdx.y * JL_LOGITS_TOK, tid = threadIdx.x;
+    const int r0 = blockIdx.x * EB, t0 = blockIdx.y * JL_LOGITS_TOK, tid = threadIdx.x;
     const int nt = min(JL_LOGITS_TOK, p.ntok - t0), k = p.k;
-    float acc[JL_LOGITS_TOK];
+    float acc[EB][JL_LOGITS_TOK];
 #pragma unroll
-    for (int t = 0; t < JL_LOGITS_TOK; t++) acc[t] = 0.f;
-    const float* wf = (const float*)p.w + (size_t)r * k;
-    const uint16_t* wh = (const uint16_t*)p.w + (size_t)r * k;
-    // unrolled so that the loads of eight trips are in flight together; the sums stay in order
-#pragma unroll 8
+    for (int e = 0; e < EB; e++)
+#pragma unroll
+        for (int t = 0; t < JL_LOGITS_TOK; t++) acc[e][t] = 0.f;
+    // unrolled so that the loads of several trips are in flight together; the sums stay in order
+#pragma unroll EB == 1 ? 8 : 2
     for (int i0 = 0; i0 < k; i0 += 128) {
         const int i = i0 + tid, ic = min(i, k - 1);
-        const float w = p.f16 ? half_bits_to_f32(wh[ic]) : wf[ic];
+        float w[EB], xv[JL_LOGITS_TOK];
 #pragma unroll
-        for (int t = 0; t < JL_LOGITS_TOK; t++) {
-            const float xv = p.x[(size_t)(t0 + min(t, nt - 1)) * k + ic];
-            const float prod = w * xv;
-            acc[t] = acc[t] + (i < k ? prod : 0.f);
+        for (int e = 0; e < EB; e++) {
+            const size_t at = (size_t)min(r0 + e, p.n_expert - 1) * k + ic;
+            w[e] = p.f16 ? half_bits_to_f32(((const uint16_t*)p.w)[at]) : ((const float*)p.w)[at];
         }
-    }
-    // part [token][128]
 #pragma unroll
-    for (int t = 0; t < JL_LOGITS_TOK; t++) part[t * 128 + tid] = acc[t];
-    __syncthreads();
+        for (int t = 0; t < JL_LOGITS_TOK; t++) xv[t] = p.x[(size_t)(t0 + min(t, nt - 1)) * k + ic];
+#pragma unroll
+        for (int e = 0; e < EB; e++)
+#pragma unroll
+            for (int t = 0; t < JL_LOGITS_TOK; t++) {
+                const float prod = w[e] * xv[t];
+                acc[e][t] = acc[e][t] + (i < k ? prod : 0.f);
+            }
+    }
     // The tree, one token per 16 lanes: lane j of a token's row takes the partial sums the
     // tree would bring to thread j by s = 16 (levels 64, 32, 16: seven adds in tree order),
     // then levels 8..1 are lane moves inside the 16-lane row (lane j reads lane j + s).
+    // One expert row at a time through part [token][128] (a buffer per row would cost the
+    // eight-row form its wavefronts per CU).
     static_assert(JL_LOGITS_TOK == 8, "eight tokens x sixteen lanes = the workgroup");
     const int tk = tid >> 4, j = tid & 15;
-    const float* q = part + tk * 128 + j;
-    const float a0 = q[0] + q[64], a32 = q[32] + q[96], a16 = q[16] + q[80], a48 = q[48] + q[112];
-    const float b0 = a0 + a32, b16 = a16 + a48;
-    float v = b0 + b16;
-    v = v + dpp_f32<0x108, 0xf>(v);   // row_shl:8
-    v = v + dpp_f32<0x104, 0xf>(v);   // row_shl:4
-    v = v + dpp_f32<0x102, 0xf>(v);   // row_shl:2
-    v = v + dpp_f32<0x101, 0xf>(v);   // row_shl:1
-    if (j == 0 && tk < nt) p.logits[(size_t)(t0 + tk) * p.n_expert + r] = v;
+#pragma unroll
+    for (int e = 0; e < EB; e++) {
+        if (e) __syncthreads();
+#pragma unroll
+        for (int t = 0; t < JL_LOGITS_TOK; t++) part[t * 128 + tid] = acc[e][t];
+        __syncthreads();
+        const float* q = part + tk * 128 + j;
+        const float a0 = q[0] + q[64], a32 = q[32] + q[96], a16 = q[16] + q[80], a48 = q[48] + q[112];
+        const float b0 = a0 + a32, b16 = a16 + a48;
+        float v = b0 + b16;
+        v = v + dpp_f32<0x108, 0xf>(v);   // row_shl:8
+        v = v + dpp_f32<0x104, 0xf>(v);   // row_shl:4
+        v = v + dpp_f32<0x102, 0xf>(v);   // row_shl:2
+        v = v + dpp_f32<0x101, 0xf>(v);   // row_shl:1
+        if (j == 0 && tk < nt && r0 + e < p.n_expert) p.logits[(size_t)(t0 + tk) * p.n_expert + r0 + e] = v;
+    }
 }

@@ -293,9 +293,11 @@ def test_router_vs_oracle(dev, devbuf, case):
     assert dev.moe_route_dev(ld.ptr, rows, 2000, k_used, sel.ptr, k_used + 1, wt.ptr) is False
 
 
+@pytest.mark.parametrize("form", [1, 8, 0], ids=["row_a_workgroup", "eight_rows_a_workgroup", "auto"])
 @pytest.mark.parametrize("case", [(64, 128, 2048, "f32"), (1, 128, 2048, "f16"), (13, 8, 4096, "f16"),
-                                  (9, 16, 130, "f32"), (3, 5, 100, "f32")], ids=lambda c: "x".join(map(str, c)))
-def test_router_logits_bit_exact_then_route(dev, devbuf, case):
+                                  (9, 16, 130, "f32"), (3, 5, 100, "f32"), (300, 130, 1000, "f16"),
+                                  (515, 128, 2048, "f32")], ids=lambda c: "x".join(map(str, c)))
+def test_router_logits_bit_exact_then_route(dev, devbuf, case, form):
     """The router's own matrix product on the device (kernels.RouterMatVecTok,
     /root/reference/jit/gpu/kernels/moe.go:820-917): f32 arithmetic in that kernel's
     summation order, so the logits must be the oracle's BITS (ragged k, f16 weights and a
@@ -303,6 +305,7 @@ def test_router_logits_bit_exact_then_route(dev, devbuf, case):
     the device then gives the oracle's routing of the oracle's logits: the mixture block
     needs no host step from x to the selected experts."""
     ntok, n_expert, k, wdt = case
+    dev.set_tuning(moe__logits=form)
     rng = np.random.default_rng(ntok * 7 + n_expert)
     w = rng.standard_normal((n_expert, k)).astype(np.float32) * np.float32(0.05)
     x = rng.standard_normal((ntok, k)).astype(np.float32)
@@ -330,3 +333,4 @@ def test_router_logits_bit_exact_then_route(dev, devbuf, case):
         assert np.array_equal(wt.get()[t].view(np.uint32), wgt.view(np.uint32))
     # only f32 and f16 router weights are served
     assert dev.moe_logits_dev(ld.ptr, 8, wd.ptr, xd.ptr, n_expert, k, ntok) is False
+    dev.set_tuning(moe__logits=0)
