@@ -149,10 +149,10 @@ int matvec_max_block(int type, int rpw) {
 hipStream_t pick_stream(jl_ctx* c, void* s) { return s ? (hipStream_t)s : c->stream; }
 
 int launch(jl_ctx* c, const char* name, unsigned gx, unsigned gy, unsigned block, unsigned lds,
-           hipStream_t st, void** params) {
+           hipStream_t st, void** params, unsigned gz = 1) {
     auto it = c->fn.find(name);
     if (it == c->fn.end()) return fail(c, JL_ERR_ARG, "kernel %s is not in the code object", name);
-    HIP_TRY(c, H->ModuleLaunchKernel(it->second, gx, gy, 1, block, 1, 1, lds, st, params, nullptr));
+    HIP_TRY(c, H->ModuleLaunchKernel(it->second, gx, gy, gz, block, 1, 1, lds, st, params, nullptr));
     c->launches++;
     return JL_OK;
 }
@@ -493,6 +493,51 @@ int gemm_q4k_launch(jl_ctx* c, float* out, const void* w, const float* x, int nr
                   (unsigned)((rows_left + rows - 1) / rows), rows == 128 ? 512 : 256, gemm_lds_bytes(rows), st, gp);
 }
 
+// Q6_K prefill GEMM on the f16 matrix cores (kernels/gemm_q6k.h): 128-token x 64-row tiles,
+// the Q4_K form's activation prep; a grid that leaves most of the chip idle is widened along
+// K and the partial slabs are added in order.
+constexpr unsigned kGemm6LdsBytes = 2u * 64u * kGemmStride * 2u;   // JL_GEMM6_LDS_BYTES
+
+int gemm_q6k_launch(jl_ctx* c, float* out, const void* w, const float* x, int nrows, int k, int ntok,
+                    hipStream_t st) {
+    const int tok_pad = (ntok + kGemmTile - 1) / kGemmTile * kGemmTile, nsb = k / 256;
+    int rc = gemm_ws_ensure(c, gemm_ws_need(tok_pad, k));
+    if (rc != JL_OK) return rc;
+    uint16_t* bq = (uint16_t*)c->gemm_ws;
+    float* da = (float*)((char*)c->gemm_ws + (size_t)nsb * 2 * (tok_pad / 32) * kGemmAStageBytes);
+    GemmPrepArgs pa;
+    pa.x = x; pa.bq = bq; pa.da = da; pa.ntok = ntok; pa.tok_pad = tok_pad; pa.k = k;
+    void* pp[] = {&pa};
+    rc = launch(c, "jl_gemm_prep_q4k", (unsigned)nsb, (unsigned)(tok_pad / 32), 256, 0, st, pp);
+    if (rc != JL_OK) return rc;
+    GemmArgs ga;
+    ga.out = out; ga.w = (const uint8_t*)w; ga.bq = bq; ga.da = da;
+    ga.nrows = nrows; ga.k = k; ga.ntok = ntok; ga.tok_pad = tok_pad; ga.row_bytes = nsb * 210;
+    ga.out_stride = nrows; ga.sb_per = 0;
+    void* gp[] = {&ga};
+    const long groups = (long)(tok_pad / kGemmTile) * ((nrows + 63) / 64);
+    int nsplit = c->tune.gemm_split > 0 ? c->tune.gemm_split : (groups <= c->num_cu ? (int)(2 * c->num_cu / groups) : 1);
+    if (nsplit > 8) nsplit = 8;
+    if (nsplit > nsb) nsplit = nsb;
+    if (nsplit > 1) {
+        const int per = (nsb + nsplit - 1) / nsplit;
+        nsplit = (nsb + per - 1) / per;   // no empty split
+        const size_t n = (size_t)ntok * nrows;
+        rc = ws_ensure(c, &c->mx_ws, &c->mx_ws_bytes, n * nsplit * 4);
+        if (rc != JL_OK) return rc;
+        ga.out = (float*)c->mx_ws; ga.sb_per = per;
+        rc = launch(c, "jl_gemm_q6k_r64", (unsigned)(tok_pad / kGemmTile), (unsigned)((nrows + 63) / 64),
+                    256, kGemm6LdsBytes, st, gp, (unsigned)nsplit);
+        if (rc != JL_OK) return rc;
+        SumPartsArgs sa;
+        sa.out = out; sa.part = (const float*)c->mx_ws; sa.n = n; sa.nsplit = nsplit;
+        void* sp[] = {&sa};
+        return launch(c, "jl_sum_parts", (unsigned)((n + 255) / 256), 1, 256, 0, st, sp);
+    }
+    return launch(c, "jl_gemm_q6k_r64", (unsigned)(tok_pad / kGemmTile), (unsigned)((nrows + 63) / 64), 256,
+                  kGemm6LdsBytes, st, gp);
+}
+
 // out [ntok][nrows] = x [ntok][k] W^T on device operands: the matrix-core GEMM where it
 // applies, else one fused matvec launch per token (same values, token by token).
 int matmul_launch(jl_ctx* c, float* out, int type, const void* w, const float* x, int nrows, int k,
@@ -505,6 +550,9 @@ int matmul_launch(jl_ctx* c, float* out, int type, const void* w, const float* x
     const bool gemm = type == JL_TYPE_Q4_K && c->act_window == 256 && ntok >= c->gemm_min_tok &&
                       aligned16(w) && ntok <= 65535 * 4 && kGemmLdsBytes <= c->lds_limit;
     if (gemm) return gemm_q4k_launch(c, out, w, x, nrows, k, ntok, st);
+    if (type == JL_TYPE_Q6_K && c->act_window == 256 && ntok >= c->gemm_min_tok && c->tune.gemm_form != 9 &&
+        ((uintptr_t)w & 1) == 0 && ntok <= 65535 * 4 && (nrows + 63) / 64 <= 65535 && kGemm6LdsBytes <= c->lds_limit)
+        return gemm_q6k_launch(c, out, w, x, nrows, k, ntok, st);   // ("gemm.form" = 9: token by token)
     for (int t = 0; t < ntok; t++) {
         rc = matvec_launch(c, out + (size_t)t * nrows, type, w, x + (size_t)t * k, nullptr, nullptr,
                            nullptr, nrows, k, st);
@@ -851,7 +899,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     if (e != hipSuccess)
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
-    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_quant", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_q4k", "jl_moe_gemm_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_sum_parts",
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_quant", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_q4k", "jl_moe_gemm_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_sum_parts",
                                       "jl_pack_weights", "jl_unpack_q4k"};
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int rw : {16, 32, 64})

@@ -5,6 +5,7 @@
 #include "common.h"
 #include "dequant.h"
 #include "gemm_q4k.h"
+#include "gemm_q6k.h"
 #include "matvec.h"
 #include "moe.h"
 #include "mxfp4.h"
@@ -134,6 +135,9 @@ extern "C" __global__ __launch_bounds__(256, 2) void jl_gemm_q4k_r64(GemmArgs p)
     gemm_split_slice(p);
     gemm_q4k_body<1>(p, jl_smem, blockIdx.x * JL_GEMM_TILE, blockIdx.y * 64);
 }
+// Q6_K with the k-quant window: grid = (tok_pad/128, ceil(nrows/64), K splits), block = 256,
+// dynamic LDS = JL_GEMM6_LDS_BYTES; the activation prep is jl_gemm_prep_q4k
+extern "C" __global__ __launch_bounds__(256, 2) void jl_gemm_q6k_r64(GemmArgs p) { gemm_q6k_body(p, jl_smem); }
 extern "C" __global__ __launch_bounds__(512) void jl_gemm_q4k_r128(GemmArgs p) {
     gemm_q4k_body<2>(p, jl_smem, blockIdx.x * JL_GEMM_TILE, blockIdx.y * 128);
 }
