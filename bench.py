@@ -186,14 +186,15 @@ def cpu_baseline(t, nrows, k, window, seed=0):
 MFMA_F16_PEAK_TFLOPS = 2500.0
 
 
-def gemm_section(dev, shapes=None):
+def gemm_section(dev, shapes=None, t=None, k=4096):
     """Q4_K prefill GEMM (x [ntok][4096] f32 -> out [ntok][nrows]), activation quantizer and
     layout kernel included in every step; flops = 2*nrows*k*ntok, priced against the dense
     f16 MFMA peak (the kernel runs exact integer operands on the f16 matrix cores).
-    shapes: {nrows: [ntok, ...]}; default = the baseline's prefill configurations."""
+    shapes: {nrows: [ntok, ...]}; default = the baseline's prefill configurations.
+    t = Q6_K: the same model's Q6_K tensors (a weight is two matrix operands there)."""
     from jitllm_amd import quant, synth
     from jitllm_amd.hipmem import DeviceArray, Event
-    t, k = quant.Q4_K, 4096
+    t = quant.Q4_K if t is None else t
     dev.SetActWindow(256)
     out = {}
     shapes = shapes or {4096: (16, 128, 512, 2048), 14336: (16, 128, 512, 2048)}
@@ -563,6 +564,8 @@ def main():
         line["ffn_block_decode"] = ffn_section(dev)
         line["ffn_block_decode_packed"] = ffn_packed_section(dev)
         line["prefill_gemm"] = gemm_section(dev)
+        from jitllm_amd import quant as _quant
+        line["prefill_gemm_q6k"] = gemm_section(dev, {4096: (512, 2048)}, _quant.Q6_K, 14336)
         line["moe_block"] = moe_section(dev)
         line["moe_decode"] = moe_decode_section(dev)
         line["mxfp4_gemm"] = mxfp4_section(dev)
