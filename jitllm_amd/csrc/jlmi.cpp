@@ -691,12 +691,13 @@ int packed_matvec_multi_launch(jl_ctx* c, int type, int m, float* const* outs, c
                   params);   // JL_PK_LDS_BYTES
 }
 
-int unpack_launch(jl_ctx* c, const PlaneRef& pl, int nrows, int k, void* dst, hipStream_t st) {
+int unpack_launch(jl_ctx* c, int type, const PlaneRef& pl, int nrows, int k, void* dst, hipStream_t st) {
     UnpackArgs a;
     a.dst = (uint8_t*)dst; a.qs = pl.qs; a.d = pl.d; a.sc = pl.sc;
     a.nrows = nrows; a.k = k; a.row0 = pl.row; a.stride = pl.stride;
     void* params[] = {&a};
-    return launch(c, "jl_unpack_q4k", (unsigned)((nrows + 255) / 256), (unsigned)(k / 256), 256, 0, st, params);
+    return launch(c, type == JL_TYPE_Q6_K ? "jl_unpack_q6k" : "jl_unpack_q4k", (unsigned)((nrows + 255) / 256),
+                  (unsigned)(k / 256), 256, 0, st, params);
 }
 
 int packed_matmul_launch(jl_ctx* c, float* out, int type, const PlaneRef& pl, const float* x, int nrows,
@@ -706,14 +707,19 @@ int packed_matmul_launch(jl_ctx* c, float* out, int type, const PlaneRef& pl, co
     if (rc != JL_OK) return rc;
     if (!out || !x || ntok <= 0) return fail(c, JL_ERR_ARG, "packed matmul: bad operand");
     if (!aligned16(x) || (k % 4) != 0) return JL_DECLINED;
+    // the matrix-core forms read GGUF rows: the planes are turned back into rows in a workspace
     const bool gemm = type == JL_TYPE_Q4_K && c->act_window == 256 && ntok >= c->gemm_min_tok &&
                       ntok <= 65535 * 4 && kGemmLdsBytes <= c->lds_limit && k / 256 <= 65535;
-    if (gemm) {
-        rc = ws_ensure(c, &c->unpack_ws, &c->unpack_ws_bytes, (size_t)nrows * (size_t)(k / 256) * 144);
+    const bool gemm6 = type == JL_TYPE_Q6_K && c->act_window == 256 && ntok >= c->gemm_min_tok &&
+                       c->tune.gemm_form != 9 && ntok <= 65535 * 4 && (nrows + 63) / 64 <= 65535 &&
+                       kGemm6LdsBytes <= c->lds_limit && k / 256 <= 65535;
+    if (gemm || gemm6) {
+        rc = ws_ensure(c, &c->unpack_ws, &c->unpack_ws_bytes, (size_t)nrows * (size_t)(k / 256) * (gemm ? 144 : 210));
         if (rc != JL_OK) return rc;
-        rc = unpack_launch(c, pl, nrows, k, c->unpack_ws, st);
+        rc = unpack_launch(c, type, pl, nrows, k, c->unpack_ws, st);
         if (rc != JL_OK) return rc;
-        return gemm_q4k_launch(c, out, c->unpack_ws, x, nrows, k, ntok, st);
+        return gemm ? gemm_q4k_launch(c, out, c->unpack_ws, x, nrows, k, ntok, st)
+                    : gemm_q6k_launch(c, out, c->unpack_ws, x, nrows, k, ntok, st);
     }
     for (int t = 0; t < ntok; t++) {
         rc = packed_matvec_launch(c, out + (size_t)t * nrows, type, pl, x + (size_t)t * k, nullptr, nullptr,
@@ -900,7 +906,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
     std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_quant", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_q4k", "jl_moe_gemm_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_sum_parts",
-                                      "jl_pack_weights", "jl_unpack_q4k"};
+                                      "jl_pack_weights", "jl_unpack_q4k", "jl_unpack_q6k"};
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int rw : {16, 32, 64})
             for (const char* form : {"", "q8_"})
@@ -1140,15 +1146,15 @@ int jl_pack_weights_dev(jl_ctx* c, int type, const void* src, int nrows, int k, 
 int jl_unpack_weights_dev(jl_ctx* c, int type, const uint32_t* qs, const uint32_t* d, const uint32_t* sc,
                           int row, int stride, int nrows, int k, void* dst, void* stream) {
     if (!c) return JL_ERR_ARG;
-    if (type != JL_TYPE_Q4_K) return JL_DECLINED;
+    if (type != JL_TYPE_Q4_K && type != JL_TYPE_Q6_K) return JL_DECLINED;
     const PlaneRef pl = {qs, d, sc, row, stride};
     const TypeInfo* ti = nullptr;
     int rc = packed_check(c, type, pl, nrows, k, &ti);
     if (rc != JL_OK) return rc;
     if (!dst) return fail(c, JL_ERR_ARG, "unpack: null dst");
-    if (((uintptr_t)dst & 3) || k / 256 > 65535) return JL_DECLINED;
+    if (((uintptr_t)dst & (type == JL_TYPE_Q4_K ? 3 : 1)) || k / 256 > 65535) return JL_DECLINED;
     HIP_TRY(c, H->SetDevice(c->device));
-    return unpack_launch(c, pl, nrows, k, dst, pick_stream(c, stream));
+    return unpack_launch(c, type, pl, nrows, k, dst, pick_stream(c, stream));
 }
 
 int jl_matvec_packed_dev(jl_ctx* c, float* out, int type, const uint32_t* qs, const uint32_t* d,

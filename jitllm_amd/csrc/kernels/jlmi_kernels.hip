@@ -77,6 +77,7 @@ extern "C" __global__ __launch_bounds__(1024) void jl_matvec_segments(MatVecMult
 // grid = (ceil(nrows/256), k/256 or k/32 for Q8_0), block = 256
 extern "C" __global__ __launch_bounds__(256) void jl_pack_weights(PackArgs p) { pack_weights_body(p); }
 extern "C" __global__ __launch_bounds__(256) void jl_unpack_q4k(UnpackArgs p) { unpack_q4k_body(p); }
+extern "C" __global__ __launch_bounds__(256) void jl_unpack_q6k(UnpackArgs p) { unpack_q6k_body(p); }
 // jl_matvec_packed_<type>_w<rows per wavefront>: grid = ceil(nrows/RW), block = 64..1024
 // XPRE = chunks whose activation loads go out ahead of the weights (register budget).
 // jl_matvec_packed_<type>_w<RW> quantizes f32 x itself; jl_matvec_packed_q8_<type>_w<RW>

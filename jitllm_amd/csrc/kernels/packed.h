@@ -167,6 +167,49 @@ __device__ __forceinline__ void unpack_q4k_body(const UnpackArgs& p) {
         }
 }
 
+// The inverse for Q6_K (pack_q6k above): one thread per (row, super-block).  Per (half, run)
+// the four sub-blocks 8*half + 2*grp + run share sixteen ql bytes pairwise (grp and grp + 2:
+// low and high nibbles) and sixteen qh bytes all four (two bits each); a plane word holds the
+// nibbles of elements j and j + 8 (w0) or 4 + j and 12 + j (w1) in byte j, the bit-pair word
+// the top bits of elements j, 4 + j, 8 + j, 12 + j.  Blocks are 210 bytes: 2-byte aligned stores.
+__device__ __forceinline__ void st4_a2(uint8_t* p, u32 v) { ((u32_a2*)p)->v = v; }
+
+__device__ __forceinline__ void unpack_q6k_body(const UnpackArgs& p) {
+    const int rl = blockIdx.x * 256 + threadIdx.x, sb = blockIdx.y;
+    if (rl >= p.nrows) return;
+    const size_t n = (size_t)p.stride, r = (size_t)p.row0 + rl;
+    const int nsb = p.k / 256;
+    uint8_t* blk = p.dst + ((size_t)rl * nsb + sb) * 210;
+    *(uint16_t*)(blk + 208) = (uint16_t)p.d[(size_t)sb * n + r];
+#pragma unroll
+    for (int j = 0; j < 4; j++)   // int8 scales are stored + 128
+        st4_a2(blk + 192 + 4 * j, p.sc[((size_t)sb * 4 + j) * n + r] ^ 0x80808080u);
+    const u32 M = 0x0F0F0F0Fu, T = 0x03030303u;
+#pragma unroll
+    for (int half = 0; half < 2; half++)
+#pragma unroll
+        for (int run = 0; run < 2; run++) {
+            u32 N[4][4], H[4];   // [grp][four elements] nibbles in bytes; bit-pair words
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const size_t base = ((size_t)(sb * 16 + half * 8 + 2 * g + run) * 3) * n + r;
+                const u32 w0 = p.qs[base], w1 = p.qs[base + n];
+                H[g] = p.qs[base + 2 * n];
+                N[g][0] = w0 & M; N[g][2] = (w0 >> 4) & M;
+                N[g][1] = w1 & M; N[g][3] = (w1 >> 4) & M;
+            }
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                st4_a2(blk + half * 64 + run * 16 + 4 * i, N[0][i] | (N[2][i] << 4));
+                st4_a2(blk + half * 64 + 32 + run * 16 + 4 * i, N[1][i] | (N[3][i] << 4));
+                u32 q = 0;
+#pragma unroll
+                for (int g = 0; g < 4; g++) q |= ((H[g] >> (2 * i)) & T) << (2 * g);
+                st4_a2(blk + 128 + half * 32 + run * 16 + 4 * i, q);
+            }
+        }
+}
+
 // ---------------------------------------------------------------- matvec
 
 // A wavefront's private LDS: 256 int8 activations, 8 scales, 16 half-block sums.

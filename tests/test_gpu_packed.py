@@ -61,11 +61,19 @@ def test_pack_on_device_is_byte_exact(dev, devbuf, t, shape):
     assert np.array_equal(d.get(), wd)
     if wsc.size:
         assert np.array_equal(sc.get(), wsc)
-    if t == quant.Q4_K:
-        back = devbuf(shape=(src.size,), dtype=np.uint8, fill=0x5A)
+    if t in (quant.Q4_K, quant.Q6_K):
+        back = devbuf(shape=(src.size + 4,), dtype=np.uint8, fill=0x5A)
         assert dev.unpack_weights_dev(t, Packed(qs.ptr, d.ptr, sc.ptr, 0, nrows), nrows, k, back.ptr)
         dev.synchronize()
-        assert np.array_equal(back.get(), src)
+        assert np.array_equal(back.get()[:src.size], src)
+        assert np.all(back.get()[src.size:] == 0x5A), "wrote past the rows"
+        if nrows > 4:     # a row range inside the planes
+            lo, n = nrows // 3, nrows // 2
+            rb = quant.row_bytes(t, k)
+            part = devbuf(shape=(n * rb,), dtype=np.uint8, fill=0x5A)
+            assert dev.unpack_weights_dev(t, Packed(qs.ptr, d.ptr, sc.ptr, lo, nrows), n, k, part.ptr)
+            dev.synchronize()
+            assert np.array_equal(part.get(), src[lo * rb:(lo + n) * rb])
 
 
 def test_packed_words_closed_form(dev):
