@@ -538,6 +538,52 @@ int gemm_q6k_launch(jl_ctx* c, float* out, const void* w, const float* x, int nr
                   kGemm6LdsBytes, st, gp);
 }
 
+// Q8_0 prefill GEMM with the activation window of 32 (kernels/gemm_w32.h): its own prep
+// (fragments in the order of the byte unpack, a token scale per 32), 128-token x 64-row tiles,
+// K split in stages of 128 for small grids.
+constexpr unsigned kGemm32LdsBytes = 64u * kGemmStride * 2u + 64u * 4u * 4u + 4u * kGemmTile * 4u;   // JL_GEMM32_LDS_BYTES
+
+int gemm_q8_0_w32_launch(jl_ctx* c, float* out, const void* w, const float* x, int nrows, int k, int ntok,
+                         hipStream_t st) {
+    const int tok_pad = (ntok + kGemmTile - 1) / kGemmTile * kGemmTile, nstage = k / 128;
+    const size_t bq_bytes = (size_t)nstage * (tok_pad / 32) * 8 * 1024;
+    int rc = gemm_ws_ensure(c, bq_bytes + (size_t)(k / 32) * tok_pad * 4);
+    if (rc != JL_OK) return rc;
+    uint16_t* bq = (uint16_t*)c->gemm_ws;
+    float* da = (float*)((char*)c->gemm_ws + bq_bytes);
+    GemmPrepArgs pa;
+    pa.x = x; pa.bq = bq; pa.da = da; pa.ntok = ntok; pa.tok_pad = tok_pad; pa.k = k;
+    void* pp[] = {&pa};
+    rc = launch(c, "jl_gemm_prep_w32", (unsigned)((k + 255) / 256), (unsigned)(tok_pad / 32), 256, 0, st, pp);
+    if (rc != JL_OK) return rc;
+    GemmArgs ga;
+    ga.out = out; ga.w = (const uint8_t*)w; ga.bq = bq; ga.da = da;
+    ga.nrows = nrows; ga.k = k; ga.ntok = ntok; ga.tok_pad = tok_pad; ga.row_bytes = (k / 32) * 34;
+    ga.out_stride = nrows; ga.sb_per = 0;
+    void* gp[] = {&ga};
+    const long groups = (long)(tok_pad / kGemmTile) * ((nrows + 63) / 64);
+    int nsplit = c->tune.gemm_split > 0 ? c->tune.gemm_split : (groups <= c->num_cu ? (int)(2 * c->num_cu / groups) : 1);
+    if (nsplit > 8) nsplit = 8;
+    if (nsplit > nstage) nsplit = nstage;
+    if (nsplit > 1) {
+        const int per = (nstage + nsplit - 1) / nsplit;
+        nsplit = (nstage + per - 1) / per;   // no empty split
+        const size_t n = (size_t)ntok * nrows;
+        rc = ws_ensure(c, &c->mx_ws, &c->mx_ws_bytes, n * nsplit * 4);
+        if (rc != JL_OK) return rc;
+        ga.out = (float*)c->mx_ws; ga.sb_per = per;
+        rc = launch(c, "jl_gemm_q8_0_w32", (unsigned)(tok_pad / kGemmTile), (unsigned)((nrows + 63) / 64), 256,
+                    kGemm32LdsBytes, st, gp, (unsigned)nsplit);
+        if (rc != JL_OK) return rc;
+        SumPartsArgs sa;
+        sa.out = out; sa.part = (const float*)c->mx_ws; sa.n = n; sa.nsplit = nsplit;
+        void* sp[] = {&sa};
+        return launch(c, "jl_sum_parts", (unsigned)((n + 255) / 256), 1, 256, 0, st, sp);
+    }
+    return launch(c, "jl_gemm_q8_0_w32", (unsigned)(tok_pad / kGemmTile), (unsigned)((nrows + 63) / 64), 256,
+                  kGemm32LdsBytes, st, gp);
+}
+
 // out [ntok][nrows] = x [ntok][k] W^T on device operands: the matrix-core GEMM where it
 // applies, else one fused matvec launch per token (same values, token by token).
 int matmul_launch(jl_ctx* c, float* out, int type, const void* w, const float* x, int nrows, int k,
@@ -553,6 +599,10 @@ int matmul_launch(jl_ctx* c, float* out, int type, const void* w, const float* x
     if (type == JL_TYPE_Q6_K && c->act_window == 256 && ntok >= c->gemm_min_tok && c->tune.gemm_form != 9 &&
         ((uintptr_t)w & 1) == 0 && ntok <= 65535 * 4 && (nrows + 63) / 64 <= 65535 && kGemm6LdsBytes <= c->lds_limit)
         return gemm_q6k_launch(c, out, w, x, nrows, k, ntok, st);   // ("gemm.form" = 9: token by token)
+    if (type == JL_TYPE_Q8_0 && c->act_window == 32 && ntok >= c->gemm_min_tok && c->tune.gemm_form != 9 &&
+        k % 128 == 0 && ((uintptr_t)w & 1) == 0 && ntok <= 65535 * 4 && (nrows + 63) / 64 <= 65535 &&
+        kGemm32LdsBytes <= c->lds_limit)
+        return gemm_q8_0_w32_launch(c, out, w, x, nrows, k, ntok, st);
     for (int t = 0; t < ntok; t++) {
         rc = matvec_launch(c, out + (size_t)t * nrows, type, w, x + (size_t)t * k, nullptr, nullptr,
                            nullptr, nrows, k, st);
@@ -905,7 +955,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     if (e != hipSuccess)
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
-    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_quant", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_q4k", "jl_moe_gemm_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_sum_parts",
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_quant", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_q4k", "jl_moe_gemm_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_sum_parts",
                                       "jl_pack_weights", "jl_unpack_q4k", "jl_unpack_q6k"};
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int rw : {16, 32, 64})

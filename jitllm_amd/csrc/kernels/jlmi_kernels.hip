@@ -6,6 +6,7 @@
 #include "dequant.h"
 #include "gemm_q4k.h"
 #include "gemm_q6k.h"
+#include "gemm_w32.h"
 #include "matvec.h"
 #include "moe.h"
 #include "mxfp4.h"
@@ -139,6 +140,14 @@ extern "C" __global__ __launch_bounds__(256, 2) void jl_gemm_q4k_r64(GemmArgs p)
 // Q6_K with the k-quant window: grid = (tok_pad/128, ceil(nrows/64), K splits), block = 256,
 // dynamic LDS = JL_GEMM6_LDS_BYTES; the activation prep is jl_gemm_prep_q4k
 extern "C" __global__ __launch_bounds__(256, 2) void jl_gemm_q6k_r64(GemmArgs p) { gemm_q6k_body(p, jl_smem); }
+// Q8_0 with the activation window of 32: prep grid = (ceil(k/256), tok_pad/32), block = 256;
+// matrix kernel grid = (tok_pad/128, ceil(nrows/64), K splits), block = 256, dynamic LDS =
+// JL_GEMM32_LDS_BYTES
+extern "C" __global__ __launch_bounds__(256) void jl_gemm_prep_w32(GemmPrepArgs p) {
+    __shared__ u32 sq[32 * 65];
+    gemm_prep_w32_body(p, sq);
+}
+extern "C" __global__ __launch_bounds__(256, 2) void jl_gemm_q8_0_w32(GemmArgs p) { gemm_q8_0_w32_body(p, jl_smem); }
 extern "C" __global__ __launch_bounds__(512) void jl_gemm_q4k_r128(GemmArgs p) {
     gemm_q4k_body<2>(p, jl_smem, blockIdx.x * JL_GEMM_TILE, blockIdx.y * 128);
 }

@@ -291,3 +291,64 @@ def test_gemm_q6k_k_split_and_token_loop_agree(dev, devbuf, split):
     assert nmse(got, loop.get()) <= 1e-10
     dev.set_tuning(gemm__form=0)
     dev.SetActWindow(32)
+
+
+@pytest.mark.parametrize("shape", [(16, 128, 128), (130, 200, 512), (8, 37, 1024), (512, 300, 1024),
+                                   (129, 129, 4096), (3, 64, 2816), (40, 70, 384)], ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("weights", ["normal", "planted"])
+def test_gemm_q8_0_window32_vs_oracle(dev, devbuf, shape, weights):
+    """Q8_0 with the activation window of 32 on the matrix cores: the int8 products are exact
+    f16 integers and both scales enter once per block, so the sums are the oracle's.  Token
+    counts that leave wavefronts of a tile without a token, rows that end inside a tile, K of
+    one stage, K that is no multiple of 256 and grids widened along K are among the shapes."""
+    ntok, nrows, k = shape
+    t = quant.Q8_0
+    dev.SetActWindow(32)
+    w = (synth.quantized_weights(t, nrows, k, seed=ntok) if weights == "normal"
+         else synth.random_weights(t, nrows, k, seed=ntok))
+    x = np.stack([synth.activations(k, seed=100 + i) * np.float32(1 + i % 7) for i in range(ntok)])
+    x[ntok // 2] = 0                       # an all-zero token: scale 0, inverse 0
+    x[0, 32:64] = 0                        # an all-zero window inside a token
+    want = _oracle_matmul(t, w, x, nrows, k, ntok, 32)
+    wd, xd = devbuf(w), devbuf(x)
+    out = devbuf(shape=(ntok * nrows + 16,), dtype=np.float32, fill=np.float32(3e30))
+    n0 = dev.launch_count()
+    for call in range(2):
+        assert dev.matmul_dev(out.ptr, t, wd.ptr, xd.ptr, nrows, k, ntok)
+        dev.synchronize()
+        got = out.get()
+        assert np.all(got[ntok * nrows:] == np.float32(3e30)), "wrote past the output"
+        got = got[:ntok * nrows].reshape(ntok, nrows)
+        e = nmse(got, want)
+        assert e <= 1e-10, f"call {call}: NMSE {e:.3e}"
+        worst = max(nmse(got[i], want[i]) for i in range(ntok) if np.any(want[i]))
+        assert worst <= 1e-9, f"worst token NMSE {worst:.3e}"
+        assert np.all(got[ntok // 2] == 0)
+        assert rel_l2(got, want) <= 1e-3
+    assert dev.launch_count() - n0 <= 6, "the matrix kernel, not a launch per token"
+
+
+@pytest.mark.parametrize("split", [1, 2, 3, 8])
+def test_gemm_q8_0_k_split_and_token_loop_agree(dev, devbuf, split):
+    """Every K split meets the bar, and the matrix kernel's token t is the decode matvec of
+    token t (the per-token loop, tuning gemm.form = 9) to the same bar."""
+    dev.SetActWindow(32)
+    t, ntok, nrows, k = quant.Q8_0, 20, 150, 1408   # 11 stages: a short last split
+    w = synth.random_weights(t, nrows, k, seed=split)
+    x = np.stack([synth.activations(k, seed=300 + i) for i in range(ntok)])
+    want = _oracle_matmul(t, w, x, nrows, k, ntok, 32)
+    wd, xd = devbuf(w), devbuf(x)
+    dev.set_tuning(gemm__split=split)
+    out = devbuf(shape=(ntok * nrows + 8,), dtype=np.float32, fill=np.float32(4e30))
+    assert dev.matmul_dev(out.ptr, t, wd.ptr, xd.ptr, nrows, k, ntok)
+    dev.synchronize()
+    got = out.get()
+    assert np.all(got[ntok * nrows:] == np.float32(4e30))
+    got = got[:ntok * nrows].reshape(ntok, nrows)
+    assert nmse(got, want) <= 1e-10
+    dev.set_tuning(gemm__split=0, gemm__form=9)
+    loop = devbuf(shape=(ntok, nrows), dtype=np.float32, fill=1.0)
+    assert dev.matmul_dev(loop.ptr, t, wd.ptr, xd.ptr, nrows, k, ntok)
+    dev.synchronize()
+    assert nmse(got, loop.get()) <= 1e-10
+    dev.set_tuning(gemm__form=0)
