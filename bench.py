@@ -186,7 +186,7 @@ def cpu_baseline(t, nrows, k, window, seed=0):
 MFMA_F16_PEAK_TFLOPS = 2500.0
 
 
-def gemm_section(dev, shapes=None, t=None, k=4096):
+def gemm_section(dev, shapes=None, t=None, k=4096, window=256):
     """Q4_K prefill GEMM (x [ntok][4096] f32 -> out [ntok][nrows]), activation quantizer and
     layout kernel included in every step; flops = 2*nrows*k*ntok, priced against the dense
     f16 MFMA peak (the kernel runs exact integer operands on the f16 matrix cores).
@@ -195,7 +195,7 @@ def gemm_section(dev, shapes=None, t=None, k=4096):
     from jitllm_amd import quant, synth
     from jitllm_amd.hipmem import DeviceArray, Event
     t = quant.Q4_K if t is None else t
-    dev.SetActWindow(256)
+    dev.SetActWindow(window)
     out = {}
     shapes = shapes or {4096: (16, 128, 512, 2048), 14336: (16, 128, 512, 2048)}
     for nrows, toks in shapes.items():
@@ -566,6 +566,10 @@ def main():
         line["prefill_gemm"] = gemm_section(dev)
         from jitllm_amd import quant as _quant
         line["prefill_gemm_q6k"] = gemm_section(dev, {4096: (512, 2048)}, _quant.Q6_K, 14336)
+        # the second configuration's matrices at prefill: the activation window is 32 there
+        line["prefill_gemm_window32"] = {
+            "q8_0": gemm_section(dev, {14336: (512, 2048)}, _quant.Q8_0, 4096, 32),
+            "q6_k": gemm_section(dev, {4096: (512, 2048)}, _quant.Q6_K, 14336, 32)}
         line["moe_block"] = moe_section(dev)
         line["moe_decode"] = moe_decode_section(dev)
         line["mxfp4_gemm"] = mxfp4_section(dev)

@@ -249,9 +249,9 @@ int jl_reserve(jl_ctx *ctx, int max_tok, int max_k);
 int jl_pack_weights_dev(jl_ctx *ctx, int type, const void *src, int nrows, int k, uint32_t *qs,
                         uint32_t *d, uint32_t *sc, void *stream);
 
-/* The inverse permutation for Q4_K and Q6_K: rows row .. row+nrows of the planes back to
- * GGUF super-blocks in dst (nrows * k/256 * 144 bytes, 4-byte aligned; Q6_K 210 bytes a
- * super-block, 2-byte aligned), bit for bit. */
+/* The inverse permutation for Q4_K, Q6_K and Q8_0: rows row .. row+nrows of the planes back
+ * to GGUF blocks in dst (nrows * k/256 * 144 bytes, 4-byte aligned; Q6_K 210 bytes a
+ * super-block, Q8_0 34 bytes a block of 32, 2-byte aligned), bit for bit. */
 int jl_unpack_weights_dev(jl_ctx *ctx, int type, const uint32_t *qs, const uint32_t *d,
                           const uint32_t *sc, int row, int stride, int nrows, int k, void *dst,
                           void *stream);

@@ -538,13 +538,18 @@ int gemm_q6k_launch(jl_ctx* c, float* out, const void* w, const float* x, int nr
                   kGemm6LdsBytes, st, gp);
 }
 
-// Q8_0 prefill GEMM with the activation window of 32 (kernels/gemm_w32.h): its own prep
-// (fragments in the order of the byte unpack, a token scale per 32), 128-token x 64-row tiles,
-// K split in stages of 128 for small grids.
-constexpr unsigned kGemm32LdsBytes = 64u * kGemmStride * 2u + 64u * 4u * 4u + 4u * kGemmTile * 4u;   // JL_GEMM32_LDS_BYTES
+// Q8_0 and Q6_K prefill GEMM with the activation window of 32 (kernels/gemm_w32.h): its own
+// prep (fragments in the order of the byte unpack, a token scale per 32), 128-token x 64-row
+// tiles, K split in stages of 128 (Q6_K: whole super-blocks) for small grids.
+constexpr unsigned gemm32_lds_bytes(int planes) {   // JL_GEMM32_LDS_BYTES
+    return (unsigned)planes * 64u * kGemmStride * 2u + 64u * 4u * 4u + 4u * kGemmTile * 4u;
+}
 
-int gemm_q8_0_w32_launch(jl_ctx* c, float* out, const void* w, const float* x, int nrows, int k, int ntok,
-                         hipStream_t st) {
+int gemm_w32_launch(jl_ctx* c, float* out, int type, const void* w, const float* x, int nrows, int k, int ntok,
+                    hipStream_t st) {
+    const bool q6 = type == JL_TYPE_Q6_K;
+    const char* kernel = q6 ? "jl_gemm_q6k_w32" : "jl_gemm_q8_0_w32";
+    const unsigned lds = gemm32_lds_bytes(q6 ? 2 : 1);
     const int tok_pad = (ntok + kGemmTile - 1) / kGemmTile * kGemmTile, nstage = k / 128;
     const size_t bq_bytes = (size_t)nstage * (tok_pad / 32) * 8 * 1024;
     int rc = gemm_ws_ensure(c, bq_bytes + (size_t)(k / 32) * tok_pad * 4);
@@ -558,30 +563,31 @@ int gemm_q8_0_w32_launch(jl_ctx* c, float* out, const void* w, const float* x, i
     if (rc != JL_OK) return rc;
     GemmArgs ga;
     ga.out = out; ga.w = (const uint8_t*)w; ga.bq = bq; ga.da = da;
-    ga.nrows = nrows; ga.k = k; ga.ntok = ntok; ga.tok_pad = tok_pad; ga.row_bytes = (k / 32) * 34;
+    ga.nrows = nrows; ga.k = k; ga.ntok = ntok; ga.tok_pad = tok_pad;
+    ga.row_bytes = q6 ? (k / 256) * 210 : (k / 32) * 34;
     ga.out_stride = nrows; ga.sb_per = 0;
     void* gp[] = {&ga};
     const long groups = (long)(tok_pad / kGemmTile) * ((nrows + 63) / 64);
+    const int unit = q6 ? 2 : 1, nunit = nstage / unit;   // stages a split is made of
     int nsplit = c->tune.gemm_split > 0 ? c->tune.gemm_split : (groups <= c->num_cu ? (int)(2 * c->num_cu / groups) : 1);
     if (nsplit > 8) nsplit = 8;
-    if (nsplit > nstage) nsplit = nstage;
+    if (nsplit > nunit) nsplit = nunit;
     if (nsplit > 1) {
-        const int per = (nstage + nsplit - 1) / nsplit;
-        nsplit = (nstage + per - 1) / per;   // no empty split
+        const int per = (nunit + nsplit - 1) / nsplit;
+        nsplit = (nunit + per - 1) / per;   // no empty split
         const size_t n = (size_t)ntok * nrows;
         rc = ws_ensure(c, &c->mx_ws, &c->mx_ws_bytes, n * nsplit * 4);
         if (rc != JL_OK) return rc;
-        ga.out = (float*)c->mx_ws; ga.sb_per = per;
-        rc = launch(c, "jl_gemm_q8_0_w32", (unsigned)(tok_pad / kGemmTile), (unsigned)((nrows + 63) / 64), 256,
-                    kGemm32LdsBytes, st, gp, (unsigned)nsplit);
+        ga.out = (float*)c->mx_ws; ga.sb_per = per * unit;
+        rc = launch(c, kernel, (unsigned)(tok_pad / kGemmTile), (unsigned)((nrows + 63) / 64), 256, lds, st, gp,
+                    (unsigned)nsplit);
         if (rc != JL_OK) return rc;
         SumPartsArgs sa;
         sa.out = out; sa.part = (const float*)c->mx_ws; sa.n = n; sa.nsplit = nsplit;
         void* sp[] = {&sa};
         return launch(c, "jl_sum_parts", (unsigned)((n + 255) / 256), 1, 256, 0, st, sp);
     }
-    return launch(c, "jl_gemm_q8_0_w32", (unsigned)(tok_pad / kGemmTile), (unsigned)((nrows + 63) / 64), 256,
-                  kGemm32LdsBytes, st, gp);
+    return launch(c, kernel, (unsigned)(tok_pad / kGemmTile), (unsigned)((nrows + 63) / 64), 256, lds, st, gp);
 }
 
 // out [ntok][nrows] = x [ntok][k] W^T on device operands: the matrix-core GEMM where it
@@ -599,10 +605,10 @@ int matmul_launch(jl_ctx* c, float* out, int type, const void* w, const float* x
     if (type == JL_TYPE_Q6_K && c->act_window == 256 && ntok >= c->gemm_min_tok && c->tune.gemm_form != 9 &&
         ((uintptr_t)w & 1) == 0 && ntok <= 65535 * 4 && (nrows + 63) / 64 <= 65535 && kGemm6LdsBytes <= c->lds_limit)
         return gemm_q6k_launch(c, out, w, x, nrows, k, ntok, st);   // ("gemm.form" = 9: token by token)
-    if (type == JL_TYPE_Q8_0 && c->act_window == 32 && ntok >= c->gemm_min_tok && c->tune.gemm_form != 9 &&
-        k % 128 == 0 && ((uintptr_t)w & 1) == 0 && ntok <= 65535 * 4 && (nrows + 63) / 64 <= 65535 &&
-        kGemm32LdsBytes <= c->lds_limit)
-        return gemm_q8_0_w32_launch(c, out, w, x, nrows, k, ntok, st);
+    if ((type == JL_TYPE_Q8_0 || type == JL_TYPE_Q6_K) && c->act_window == 32 && ntok >= c->gemm_min_tok &&
+        c->tune.gemm_form != 9 && k % 128 == 0 && ((uintptr_t)w & 1) == 0 && ntok <= 65535 * 4 &&
+        (nrows + 63) / 64 <= 65535 && gemm32_lds_bytes(2) <= c->lds_limit)
+        return gemm_w32_launch(c, out, type, w, x, nrows, k, ntok, st);
     for (int t = 0; t < ntok; t++) {
         rc = matvec_launch(c, out + (size_t)t * nrows, type, w, x + (size_t)t * k, nullptr, nullptr,
                            nullptr, nrows, k, st);
@@ -746,6 +752,8 @@ int unpack_launch(jl_ctx* c, int type, const PlaneRef& pl, int nrows, int k, voi
     a.dst = (uint8_t*)dst; a.qs = pl.qs; a.d = pl.d; a.sc = pl.sc;
     a.nrows = nrows; a.k = k; a.row0 = pl.row; a.stride = pl.stride;
     void* params[] = {&a};
+    if (type == JL_TYPE_Q8_0)
+        return launch(c, "jl_unpack_q8_0", (unsigned)((nrows + 255) / 256), (unsigned)(k / 32), 256, 0, st, params);
     return launch(c, type == JL_TYPE_Q6_K ? "jl_unpack_q6k" : "jl_unpack_q4k", (unsigned)((nrows + 255) / 256),
                   (unsigned)(k / 256), 256, 0, st, params);
 }
@@ -763,11 +771,15 @@ int packed_matmul_launch(jl_ctx* c, float* out, int type, const PlaneRef& pl, co
     const bool gemm6 = type == JL_TYPE_Q6_K && c->act_window == 256 && ntok >= c->gemm_min_tok &&
                        c->tune.gemm_form != 9 && ntok <= 65535 * 4 && (nrows + 63) / 64 <= 65535 &&
                        kGemm6LdsBytes <= c->lds_limit && k / 256 <= 65535;
-    if (gemm || gemm6) {
-        rc = ws_ensure(c, &c->unpack_ws, &c->unpack_ws_bytes, (size_t)nrows * (size_t)(k / 256) * (gemm ? 144 : 210));
+    const bool gemm32 = (type == JL_TYPE_Q8_0 || type == JL_TYPE_Q6_K) && c->act_window == 32 &&
+                        ntok >= c->gemm_min_tok && c->tune.gemm_form != 9 && k % 128 == 0 && ntok <= 65535 * 4 &&
+                        (nrows + 63) / 64 <= 65535 && gemm32_lds_bytes(2) <= c->lds_limit && k / 32 <= 65535;
+    if (gemm || gemm6 || gemm32) {
+        rc = ws_ensure(c, &c->unpack_ws, &c->unpack_ws_bytes, (size_t)nrows * (size_t)(k / ti->block_elems) * ti->block_bytes);
         if (rc != JL_OK) return rc;
         rc = unpack_launch(c, type, pl, nrows, k, c->unpack_ws, st);
         if (rc != JL_OK) return rc;
+        if (gemm32) return gemm_w32_launch(c, out, type, c->unpack_ws, x, nrows, k, ntok, st);
         return gemm ? gemm_q4k_launch(c, out, c->unpack_ws, x, nrows, k, ntok, st)
                     : gemm_q6k_launch(c, out, c->unpack_ws, x, nrows, k, ntok, st);
     }
@@ -955,8 +967,8 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     if (e != hipSuccess)
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
-    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_quant", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_q4k", "jl_moe_gemm_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_sum_parts",
-                                      "jl_pack_weights", "jl_unpack_q4k", "jl_unpack_q6k"};
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_quant", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_q4k", "jl_moe_gemm_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_sum_parts",
+                                      "jl_pack_weights", "jl_unpack_q4k", "jl_unpack_q6k", "jl_unpack_q8_0"};
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int rw : {16, 32, 64})
             for (const char* form : {"", "q8_"})
@@ -1196,13 +1208,13 @@ int jl_pack_weights_dev(jl_ctx* c, int type, const void* src, int nrows, int k, 
 int jl_unpack_weights_dev(jl_ctx* c, int type, const uint32_t* qs, const uint32_t* d, const uint32_t* sc,
                           int row, int stride, int nrows, int k, void* dst, void* stream) {
     if (!c) return JL_ERR_ARG;
-    if (type != JL_TYPE_Q4_K && type != JL_TYPE_Q6_K) return JL_DECLINED;
+    if (type != JL_TYPE_Q4_K && type != JL_TYPE_Q6_K && type != JL_TYPE_Q8_0) return JL_DECLINED;
     const PlaneRef pl = {qs, d, sc, row, stride};
     const TypeInfo* ti = nullptr;
     int rc = packed_check(c, type, pl, nrows, k, &ti);
     if (rc != JL_OK) return rc;
     if (!dst) return fail(c, JL_ERR_ARG, "unpack: null dst");
-    if (((uintptr_t)dst & (type == JL_TYPE_Q4_K ? 3 : 1)) || k / 256 > 65535) return JL_DECLINED;
+    if (((uintptr_t)dst & (type == JL_TYPE_Q4_K ? 3 : 1)) || k / ti->block_elems > 65535) return JL_DECLINED;
     HIP_TRY(c, H->SetDevice(c->device));
     return unpack_launch(c, type, pl, nrows, k, dst, pick_stream(c, stream));
 }

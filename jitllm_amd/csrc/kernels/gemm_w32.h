@@ -1,7 +1,7 @@
 // Prefill GEMM with the activation window of 32 (the window of a model that holds a type
-// with 32-element blocks, jit/cpu/matvec.go:46-62), Q8_0 weights.  Per (token, row) it is the
-// decode matvec's value (format/quant/dequant.go:148-157 for the weights,
-// jit/cpu/packedgemm.go:54-58 for the identity with the matvec):
+// with 32-element blocks, jit/cpu/matvec.go:46-62), Q8_0 and Q6_K weights.  Per (token, row)
+// it is the decode matvec's value (format/quant/dequant.go:148-157 and :443-470 for the
+// weights, jit/cpu/packedgemm.go:54-58 for the identity with the matvec):
 //
 //   out[t][r] = sum_b d[r,b] * d_a[t,b] * P[t,r,b],   P = sum_{l<32} q[r,b,l] * a[t,b,l]
 //
@@ -9,6 +9,9 @@
 // (v_mfma_f32_32x32x16_f16, two K-steps a block); both scales change every 32 weights, so
 // the f32 epilogue runs once per block: two vector instructions an output element per two
 // matrix instructions, which is what bounds the kernel (the matrix cores wait).
+// Q6_K: q is sc * (q6 - 32) with the int8 sub-block scale split into two exact f16 operands
+// as in gemm_q6k.h (two planes in LDS, four matrix instructions a K-step pair and tile), d
+// the super-block's.
 //
 // Activation prep (gemm_prep_w32_body): x [ntok][k] f32 -> bq [k/128 stages][tok_pad/32]
 // [8 K-steps][64 lanes][8] f16 and da [k/32][tok_pad] f32.  Lane (t = lane%32, kg = lane/32)
@@ -20,14 +23,16 @@
 // tokens x 64 rows.  Per stage (128 weights = four blocks a row) the 256 threads turn 64 rows
 // into f16 in LDS (thread = row, block: 32 bytes, xor 0x80 and the 1024 + byte trick), with
 // the rows' block scales and the tile's token scales beside them; then every wavefront runs
-// its sixteen matrix instructions, the block epilogue after every second K-step.  Three
-// workgroups share a CU and cover each other's vector phases.
-// grid = (tok_pad/128, ceil(nrows/64), K splits), block = 256, dynamic LDS = JL_GEMM32_LDS_BYTES.
+// its sixteen matrix instructions, the block epilogue after every second K-step.  Workgroups
+// that share a CU cover each other's vector phases.  Q6_K: thread = row, 32-element run of the
+// half super-block (ql nibbles + two qh bits, two sub-block scales).
+// grid = (tok_pad/128, ceil(nrows/64), K splits), block = 256, dynamic LDS =
+// JL_GEMM32_LDS_BYTES(planes), planes = 1 (Q8_0) or 2 (Q6_K).
 #pragma once
 #include "gemm_q4k.h"
 
 #define JL_GEMM32_FRAGS 8
-#define JL_GEMM32_LDS_BYTES (64 * JL_GEMM_STRIDE * 2 + 64 * 4 * 4 + 4 * JL_GEMM_TILE * 4)
+#define JL_GEMM32_LDS_BYTES(planes) ((planes) * 64 * JL_GEMM_STRIDE * 2 + 64 * 4 * 4 + 4 * JL_GEMM_TILE * 4)
 
 __device__ __forceinline__ void gemm_prep_w32_body(const GemmPrepArgs& p, u32* sq) {
     // sq [32 tokens][65]: 64 words of int8 + 1 pad (bank spread)
@@ -69,61 +74,110 @@ __device__ __forceinline__ void gemm_prep_w32_body(const GemmPrepArgs& p, u32* s
 }
 
 struct Gemm32Raw {
-    u32x4 q0, q1;   // the block's 32 int8
-    uint16_t d;
+    u32x4 q0, q1;   // Q8_0: the block's 32 int8; Q6_K: the run's 32 ql bytes
+    u32x4 h0, h1;   // Q6_K: the half's 32 qh bytes
+    u32 d;          // Q8_0: the block's f16 scale; Q6_K: d | the run's two int8 scales << 16
     float da[2];    // two of the stage's 4 x 128 token scales
 };
 
-__device__ __forceinline__ void gemm_q8_0_w32_body(const GemmArgs& p0, uint8_t* smem) {
+template <int TYPE>
+__device__ __forceinline__ void gemm_w32_body(const GemmArgs& p0, uint8_t* smem) {
+    constexpr bool Q6 = TYPE == JL_Q6_K;
+    constexpr int NPL = Q6 ? 2 : 1;
+    constexpr int STAGE_BYTES = Q6 ? 105 : 4 * 34;   // 128 weights; a Q6_K half super-block shares its block
     GemmArgs p = p0;
-    if (p.sb_per) {   // K split: sb_per stages to a workgroup, partial sums to slab z
+    if (p.sb_per) {   // K split: sb_per stages to a workgroup (Q6_K: an even number), partial sums to slab z
         const int s0 = blockIdx.z * p.sb_per;
         const int n = min(p.sb_per, p.k / 128 - s0);
-        p.w += (size_t)s0 * 4 * 34;
+        p.w += Q6 ? (size_t)(s0 / 2) * 210 : (size_t)s0 * STAGE_BYTES;
         p.bq += (size_t)s0 * (p.tok_pad >> 5) * (JL_GEMM32_FRAGS * JL_GEMM_AFRAG_HALFS);
         p.da += (size_t)s0 * 4 * p.tok_pad;
         p.k = 128 * n;
         p.out += (size_t)blockIdx.z * p.ntok * p.out_stride;
     }
     const int t0 = blockIdx.x * JL_GEMM_TILE, r0 = blockIdx.y * 64;
-    _Float16* sW = (_Float16*)smem;                      // [64][JL_GEMM_STRIDE]
-    float* sD = (float*)(sW + 64 * JL_GEMM_STRIDE);      // [64 rows][4 blocks]
-    float* sDa = sD + 64 * 4;                            // [4 blocks][128 tokens]
+    _Float16* sW = (_Float16*)smem;                            // [planes][64][JL_GEMM_STRIDE]
+    float* sD = (float*)(sW + NPL * 64 * JL_GEMM_STRIDE);      // [64 rows][4 blocks]
+    float* sDa = sD + 64 * 4;                                  // [4 blocks][128 tokens]
     const int tid = threadIdx.x, lane = tid & 63;
     const int tg = __builtin_amdgcn_readfirstlane(tid >> 6);   // this wavefront: tokens 32*tg..
     const bool live = t0 + 32 * tg < p.ntok;                   // else no token of its 32 exists
     const int arow = lane & 31, kg = lane >> 5;
     const int nsteps = p.k / 128;
-    // this thread's share of a weight stage: one block of one row
+    // this thread's share of a weight stage: one block (run) of one row
     const int srow = tid >> 2, qb = tid & 3;
     const uint8_t* wrow = p.w + (size_t)min(r0 + srow, p.nrows - 1) * p.row_bytes;
     const float* dsrc = p.da + (size_t)(tid >> 7) * p.tok_pad + t0 + (tid & 127);   // blocks tid/128 and + 2
     auto load_raw = [&](int step, Gemm32Raw& r) {
-        const uint8_t* blk = wrow + (size_t)(4 * step + qb) * 34;
-        r.d = ld2(blk);
-        r.q0 = ld16_a2(blk + 2);
-        r.q1 = ld16_a2(blk + 18);
+        if constexpr (Q6) {
+            const uint8_t* blk = wrow + (size_t)(step >> 1) * 210;
+            const int n = step & 1;
+            r.q0 = ld16_a2(blk + 64 * n + 32 * (qb & 1));
+            r.q1 = ld16_a2(blk + 64 * n + 32 * (qb & 1) + 16);
+            r.h0 = ld16_a2(blk + 128 + 32 * n);
+            r.h1 = ld16_a2(blk + 128 + 32 * n + 16);
+            r.d = (u32)ld2(blk + 208) | ((u32)ld2(blk + 192 + 8 * n + 2 * qb) << 16);
+        } else {
+            const uint8_t* blk = wrow + (size_t)(4 * step + qb) * 34;
+            r.d = ld2(blk);
+            r.q0 = ld16_a2(blk + 2);
+            r.q1 = ld16_a2(blk + 18);
+        }
         r.da[0] = dsrc[(size_t)(4 * step) * p.tok_pad];
         r.da[1] = dsrc[(size_t)(4 * step + 2) * p.tok_pad];
     };
-    u32 m8 = 0x00FF00FFu, magic = 0x64006400u;
-    asm volatile("" : "+v"(m8), "+v"(magic));   // keep them in vector registers
+    u32 m8 = Q6 ? 0x000F000Fu : 0x00FF00FFu, m2 = 0x00300030u, magic = 0x64006400u;
+    asm volatile("" : "+v"(m8), "+v"(m2), "+v"(magic));   // keep them in vector registers
     _Float16* dst = sW + srow * JL_GEMM_STRIDE + 32 * qb;
     auto dequant = [&](const Gemm32Raw& r) {
-        const f16x2 off = {(_Float16)-1152.0f, (_Float16)-1152.0f};
-        // bytes (b0, b2) and (b1, b3) of a word as 1024 + (q + 128), then q: exact
-        auto pair = [&](u32 w) {
-            const u32 v = (w & m8) | magic;
-            return __builtin_bit_cast(u32, __builtin_bit_cast(f16x2, v) + off);
-        };
+        auto word = [](f16x2 v) { return __builtin_bit_cast(u32, v); };
+        if constexpr (Q6) {
+            // run qb of the half: nibble qb/2 of the ql bytes, qh bits 2*qb; elements 0-15 and
+            // 16-31 are sub-blocks with their own scale, each split as 2 * (sc >> 1) + (sc & 1)
+            const f16x2 off = {(_Float16)-1056.0f, (_Float16)-1056.0f};
+            const int nsh = 4 * (qb >> 1), hsh = 2 * qb;
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const u32 wa = (i < 2 ? r.q0[2 * i] : r.q1[2 * i - 4]) ^ 0x80808080u;
-            const u32 wb = (i < 2 ? r.q0[2 * i + 1] : r.q1[2 * i - 3]) ^ 0x80808080u;
-            const u32x4 o = {pair(wa), pair(wa >> 8), pair(wb), pair(wb >> 8)};
-            *(u32x4*)(dst + 8 * i) = o;
+            for (int half = 0; half < 2; half++) {
+                const i32 sc = (i32)(int8_t)(r.d >> (16 + 8 * half));
+                const _Float16 s2 = (_Float16)(float)(2 * (sc >> 1)), s0 = (_Float16)(float)(sc & 1);
+                const f16x2 S2 = {s2, s2}, S0 = {s0, s0};
+                const u32x4 ql = half ? r.q1 : r.q0, qh = half ? r.h1 : r.h0;
+#pragma unroll
+                for (int i = 0; i < 2; i++) {
+                    f16x2 t[4];
+#pragma unroll
+                    for (int c = 0; c < 2; c++) {
+                        const u32 wn = ql[2 * i + c] >> nsh;
+                        // the two high bits of an element at bits 4-5 of its 16-bit half
+                        const u32 wh = (qh[2 * i + c] >> hsh) << 4;
+                        const u32 v02 = (wh & m2) | ((wn & m8) | magic);
+                        const u32 v13 = ((wh >> 8) & m2) | (((wn >> 8) & m8) | magic);
+                        t[2 * c] = __builtin_bit_cast(f16x2, v02) + off;      // (1024 + q) - 1056: exact
+                        t[2 * c + 1] = __builtin_bit_cast(f16x2, v13) + off;
+                    }
+                    const u32x4 oa = {word(t[0] * S2), word(t[1] * S2), word(t[2] * S2), word(t[3] * S2)};
+                    const u32x4 ob = {word(t[0] * S0), word(t[1] * S0), word(t[2] * S0), word(t[3] * S0)};
+                    *(u32x4*)(dst + 16 * half + 8 * i) = oa;
+                    *(u32x4*)(dst + 64 * JL_GEMM_STRIDE + 16 * half + 8 * i) = ob;
+                }
+            }
+            sD[srow * 4 + qb] = half_bits_to_f32((uint16_t)(r.d & 0xFFFF));
+        } else {
+            const f16x2 off = {(_Float16)-1152.0f, (_Float16)-1152.0f};
+            // bytes (b0, b2) and (b1, b3) of a word as 1024 + (q + 128), then q: exact
+            auto pair = [&](u32 w) {
+                const u32 v = (w & m8) | magic;
+                return word(__builtin_bit_cast(f16x2, v) + off);
+            };
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const u32 wa = (i < 2 ? r.q0[2 * i] : r.q1[2 * i - 4]) ^ 0x80808080u;
+                const u32 wb = (i < 2 ? r.q0[2 * i + 1] : r.q1[2 * i - 3]) ^ 0x80808080u;
+                const u32x4 o = {pair(wa), pair(wa >> 8), pair(wb), pair(wb >> 8)};
+                *(u32x4*)(dst + 8 * i) = o;
+            }
+            sD[srow * 4 + qb] = half_bits_to_f32((uint16_t)r.d);
         }
-        sD[srow * 4 + qb] = half_bits_to_f32(r.d);
         sDa[tid] = r.da[0];
         sDa[256 + tid] = r.da[1];
     };
@@ -159,12 +213,17 @@ __device__ __forceinline__ void gemm_q8_0_w32_body(const GemmArgs& p0, uint8_t* 
 #pragma unroll
                 for (int h = 0; h < 2; h++) {
                     const int ks = 2 * b + h;
-                    f16x8 wf[2];
+                    f16x8 wf[NPL][2];
 #pragma unroll
-                    for (int j = 0; j < 2; j++) wf[j] = *(const f16x8*)(w0 + 32 * j * JL_GEMM_STRIDE + 16 * ks);
+                    for (int pl = 0; pl < NPL; pl++)
 #pragma unroll
-                    for (int j = 0; j < 2; j++)
-                        acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aring[ks], wf[j], h ? acc[j] : czero, 0, 0, 0);
+                        for (int j = 0; j < 2; j++)
+                            wf[pl][j] = *(const f16x8*)(w0 + (pl * 64 + 32 * j) * JL_GEMM_STRIDE + 16 * ks);
+#pragma unroll
+                    for (int j = 0; j < 2; j++) {
+                        acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aring[ks], wf[0][j], h ? acc[j] : czero, 0, 0, 0);
+                        if constexpr (Q6) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aring[ks], wf[1][j], acc[j], 0, 0, 0);
+                    }
                     aring[ks] = a_frag(nstep, ks);
                 }
                 // out += d_a * (d * P) for the block

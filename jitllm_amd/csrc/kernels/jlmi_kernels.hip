@@ -79,6 +79,8 @@ extern "C" __global__ __launch_bounds__(1024) void jl_matvec_segments(MatVecMult
 extern "C" __global__ __launch_bounds__(256) void jl_pack_weights(PackArgs p) { pack_weights_body(p); }
 extern "C" __global__ __launch_bounds__(256) void jl_unpack_q4k(UnpackArgs p) { unpack_q4k_body(p); }
 extern "C" __global__ __launch_bounds__(256) void jl_unpack_q6k(UnpackArgs p) { unpack_q6k_body(p); }
+// grid = (ceil(nrows/256), k/32)
+extern "C" __global__ __launch_bounds__(256) void jl_unpack_q8_0(UnpackArgs p) { unpack_q8_0_body(p); }
 // jl_matvec_packed_<type>_w<rows per wavefront>: grid = ceil(nrows/RW), block = 64..1024
 // XPRE = chunks whose activation loads go out ahead of the weights (register budget).
 // jl_matvec_packed_<type>_w<RW> quantizes f32 x itself; jl_matvec_packed_q8_<type>_w<RW>
@@ -140,14 +142,15 @@ extern "C" __global__ __launch_bounds__(256, 2) void jl_gemm_q4k_r64(GemmArgs p)
 // Q6_K with the k-quant window: grid = (tok_pad/128, ceil(nrows/64), K splits), block = 256,
 // dynamic LDS = JL_GEMM6_LDS_BYTES; the activation prep is jl_gemm_prep_q4k
 extern "C" __global__ __launch_bounds__(256, 2) void jl_gemm_q6k_r64(GemmArgs p) { gemm_q6k_body(p, jl_smem); }
-// Q8_0 with the activation window of 32: prep grid = (ceil(k/256), tok_pad/32), block = 256;
+// Q8_0 and Q6_K with the activation window of 32: prep grid = (ceil(k/256), tok_pad/32), block = 256;
 // matrix kernel grid = (tok_pad/128, ceil(nrows/64), K splits), block = 256, dynamic LDS =
-// JL_GEMM32_LDS_BYTES
+// JL_GEMM32_LDS_BYTES(planes)
 extern "C" __global__ __launch_bounds__(256) void jl_gemm_prep_w32(GemmPrepArgs p) {
     __shared__ u32 sq[32 * 65];
     gemm_prep_w32_body(p, sq);
 }
-extern "C" __global__ __launch_bounds__(256, 2) void jl_gemm_q8_0_w32(GemmArgs p) { gemm_q8_0_w32_body(p, jl_smem); }
+extern "C" __global__ __launch_bounds__(256, 2) void jl_gemm_q8_0_w32(GemmArgs p) { gemm_w32_body<JL_Q8_0>(p, jl_smem); }
+extern "C" __global__ __launch_bounds__(256, 2) void jl_gemm_q6k_w32(GemmArgs p) { gemm_w32_body<JL_Q6_K>(p, jl_smem); }
 extern "C" __global__ __launch_bounds__(512) void jl_gemm_q4k_r128(GemmArgs p) {
     gemm_q4k_body<2>(p, jl_smem, blockIdx.x * JL_GEMM_TILE, blockIdx.y * 128);
 }

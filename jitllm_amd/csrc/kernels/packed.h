@@ -210,6 +210,20 @@ __device__ __forceinline__ void unpack_q6k_body(const UnpackArgs& p) {
         }
 }
 
+// The inverse for Q8_0 (pack_q8_0 above): one thread per (row, block); two rows share a word
+// of the D plane.
+__device__ __forceinline__ void unpack_q8_0_body(const UnpackArgs& p) {
+    const int rl = blockIdx.x * 256 + threadIdx.x, b = blockIdx.y;
+    if (rl >= p.nrows) return;
+    const size_t n = (size_t)p.stride, r = (size_t)p.row0 + rl;
+    const int nb = p.k / 32;
+    uint8_t* blk = p.dst + ((size_t)rl * nb + b) * 34;
+    const u32 dd = p.d[(size_t)b * ((n + 1) / 2) + (r >> 1)];
+    *(uint16_t*)blk = (uint16_t)(r & 1 ? dd >> 16 : dd);
+#pragma unroll
+    for (int w = 0; w < 8; w++) st4_a2(blk + 2 + 4 * w, p.qs[((size_t)b * 8 + w) * n + r]);
+}
+
 // ---------------------------------------------------------------- matvec
 
 // A wavefront's private LDS: 256 int8 activations, 8 scales, 16 half-block sums.

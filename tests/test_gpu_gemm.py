@@ -139,7 +139,7 @@ def test_gemm_token_equals_decode_matvec(dev, devbuf):
     dev.SetActWindow(32)
 
 
-@pytest.mark.parametrize("t,window,ntok", [(quant.Q8_0, 32, 5), (quant.Q6_K, 32, 3), (quant.Q4_K, 32, 9),
+@pytest.mark.parametrize("t,window,ntok", [(quant.Q8_0, 32, 2), (quant.Q6_K, 32, 2), (quant.Q4_K, 32, 9),
                                            (quant.Q4_K, 256, 3)])
 def test_matmul_fallback_is_the_per_token_loop(dev, devbuf, t, window, ntok):
     """Types, windows and token counts the GEMM does not take still return the right values."""
@@ -296,13 +296,16 @@ def test_gemm_q6k_k_split_and_token_loop_agree(dev, devbuf, split):
 @pytest.mark.parametrize("shape", [(16, 128, 128), (130, 200, 512), (8, 37, 1024), (512, 300, 1024),
                                    (129, 129, 4096), (3, 64, 2816), (40, 70, 384)], ids=lambda s: "x".join(map(str, s)))
 @pytest.mark.parametrize("weights", ["normal", "planted"])
-def test_gemm_q8_0_window32_vs_oracle(dev, devbuf, shape, weights):
-    """Q8_0 with the activation window of 32 on the matrix cores: the int8 products are exact
-    f16 integers and both scales enter once per block, so the sums are the oracle's.  Token
-    counts that leave wavefronts of a tile without a token, rows that end inside a tile, K of
-    one stage, K that is no multiple of 256 and grids widened along K are among the shapes."""
+@pytest.mark.parametrize("t", [quant.Q8_0, quant.Q6_K], ids=["q8_0", "q6_k"])
+def test_gemm_window32_vs_oracle(dev, devbuf, shape, weights, t):
+    """Q8_0 and Q6_K with the activation window of 32 on the matrix cores: the int8 products
+    are exact f16 integers (Q6_K: the sub-block scale split over two operands) and the scales
+    enter once per block of 32, so the sums are the oracle's.  Token counts that leave
+    wavefronts of a tile without a token, rows that end inside a tile, K of one stage, K that
+    is no multiple of 256 and grids widened along K are among the shapes."""
     ntok, nrows, k = shape
-    t = quant.Q8_0
+    if k % quant.block_elems(t):
+        pytest.skip("K is not a whole number of this type's blocks")
     dev.SetActWindow(32)
     w = (synth.quantized_weights(t, nrows, k, seed=ntok) if weights == "normal"
          else synth.random_weights(t, nrows, k, seed=ntok))
@@ -329,11 +332,13 @@ def test_gemm_q8_0_window32_vs_oracle(dev, devbuf, shape, weights):
 
 
 @pytest.mark.parametrize("split", [1, 2, 3, 8])
-def test_gemm_q8_0_k_split_and_token_loop_agree(dev, devbuf, split):
+@pytest.mark.parametrize("t", [quant.Q8_0, quant.Q6_K], ids=["q8_0", "q6_k"])
+def test_gemm_window32_k_split_and_token_loop_agree(dev, devbuf, split, t):
     """Every K split meets the bar, and the matrix kernel's token t is the decode matvec of
     token t (the per-token loop, tuning gemm.form = 9) to the same bar."""
     dev.SetActWindow(32)
-    t, ntok, nrows, k = quant.Q8_0, 20, 150, 1408   # 11 stages: a short last split
+    ntok, nrows = 20, 150
+    k = 1408 if t == quant.Q8_0 else 2816   # 11 stages / 11 super-blocks: a short last split
     w = synth.random_weights(t, nrows, k, seed=split)
     x = np.stack([synth.activations(k, seed=300 + i) for i in range(ntok)])
     want = _oracle_matmul(t, w, x, nrows, k, ntok, 32)

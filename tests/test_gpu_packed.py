@@ -61,9 +61,9 @@ def test_pack_on_device_is_byte_exact(dev, devbuf, t, shape):
     assert np.array_equal(d.get(), wd)
     if wsc.size:
         assert np.array_equal(sc.get(), wsc)
-    if t in (quant.Q4_K, quant.Q6_K):
+    if t in (quant.Q4_K, quant.Q6_K, quant.Q8_0):
         back = devbuf(shape=(src.size + 4,), dtype=np.uint8, fill=0x5A)
-        assert dev.unpack_weights_dev(t, Packed(qs.ptr, d.ptr, sc.ptr, 0, nrows), nrows, k, back.ptr)
+        assert dev.unpack_weights_dev(t, Packed(qs.ptr, d.ptr, sc.ptr if wsc.size else None, 0, nrows), nrows, k, back.ptr)
         dev.synchronize()
         assert np.array_equal(back.get()[:src.size], src)
         assert np.all(back.get()[src.size:] == 0x5A), "wrote past the rows"
@@ -71,7 +71,7 @@ def test_pack_on_device_is_byte_exact(dev, devbuf, t, shape):
             lo, n = nrows // 3, nrows // 2
             rb = quant.row_bytes(t, k)
             part = devbuf(shape=(n * rb,), dtype=np.uint8, fill=0x5A)
-            assert dev.unpack_weights_dev(t, Packed(qs.ptr, d.ptr, sc.ptr, lo, nrows), n, k, part.ptr)
+            assert dev.unpack_weights_dev(t, Packed(qs.ptr, d.ptr, sc.ptr if wsc.size else None, lo, nrows), n, k, part.ptr)
             dev.synchronize()
             assert np.array_equal(part.get(), src[lo * rb:(lo + n) * rb])
 
@@ -335,6 +335,25 @@ def test_matmul_packed_vs_oracle(dev, devbuf, t, ntok):
     assert nmse(got, want) <= 1e-10
     assert rel_l2(got, want) <= 1e-3
     dev.SetActWindow(32)
+
+
+def test_matmul_packed_q6k_planes_window32(dev, devbuf):
+    """Q6_K planes in a model whose window is 32 (a Q8_0 tensor beside them): unpacked into rows,
+    then the window-32 matrix kernel; a row range of a larger plane set."""
+    t, nrows, k, ntok, stride, row0 = quant.Q6_K, 200, 1024, 40, 300, 60
+    dev.SetActWindow(32)
+    w = synth.random_weights(t, stride, k, seed=5)
+    rb = quant.row_bytes(t, k)
+    x = synth.activations(ntok * k, seed=6).reshape(ntok, k)
+    want = oracle.matmul_q8act_f64(t, w[row0 * rb:(row0 + nrows) * rb], x, nrows, k, ntok, 32)
+    p = _dev_planes(devbuf, *oracle.pack_weights(t, w, stride, k), row=row0, stride=stride)
+    xd = devbuf(x)
+    out = devbuf(shape=(ntok, nrows), dtype=np.float32, fill=np.float32(3e30))
+    n0 = dev.launch_count()
+    assert dev.matmul_packed_dev(out.ptr, t, p, xd.ptr, nrows, k, ntok)
+    dev.synchronize()
+    assert dev.launch_count() - n0 <= 5
+    assert nmse(out.get(), want) <= 1e-10
 
 
 def test_packed_host_pointer_seam(dev):
