@@ -571,6 +571,7 @@ def main():
             "q8_0": gemm_section(dev, {14336: (512, 2048)}, _quant.Q8_0, 4096, 32),
             "q6_k": gemm_section(dev, {4096: (512, 2048)}, _quant.Q6_K, 14336, 32)}
         line["moe_block"] = moe_section(dev)
+        line["moe_block_prefill_1024_rows"] = moe_section(dev, 1024)   # matrix-core tiles per expert
         line["moe_decode"] = moe_decode_section(dev)
         line["mxfp4_gemm"] = mxfp4_section(dev)
 
