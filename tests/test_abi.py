@@ -74,3 +74,16 @@ def test_jlm_reader_on_the_reference_written_container():
         f.planes(q5)                       # Q5_K is not a type of this path
     with pytest.raises(ValueError):
         jlm.File(b"not a container" * 20)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """The bench runs on one GPU: asking for more ends with a message, before anything
+    touches a device."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True,
+                       text=True, timeout=120)
+    assert r.returncode != 0
+    assert "one GPU" in r.stderr
+    assert r.stdout.strip() == ""
