@@ -149,8 +149,8 @@ extern "C" __global__ __launch_bounds__(256) void jl_gemm_prep_w32(GemmPrepArgs 
     __shared__ u32 sq[32 * 65];
     gemm_prep_w32_body(p, sq);
 }
-extern "C" __global__ __launch_bounds__(256, 2) void jl_gemm_q8_0_w32(GemmArgs p) { gemm_w32_body<JL_Q8_0>(p, jl_smem); }
-extern "C" __global__ __launch_bounds__(256, 2) void jl_gemm_q6k_w32(GemmArgs p) { gemm_w32_body<JL_Q6_K>(p, jl_smem); }
+extern "C" __global__ __launch_bounds__(256, 3) void jl_gemm_q8_0_w32(GemmArgs p) { gemm_w32_body<JL_Q8_0>(p, jl_smem); }
+extern "C" __global__ __launch_bounds__(256, 3) void jl_gemm_q6k_w32(GemmArgs p) { gemm_w32_body<JL_Q6_K>(p, jl_smem); }
 extern "C" __global__ __launch_bounds__(512) void jl_gemm_q4k_r128(GemmArgs p) {
     gemm_q4k_body<2>(p, jl_smem, blockIdx.x * JL_GEMM_TILE, blockIdx.y * 128);
 }
