@@ -139,7 +139,7 @@ def test_gemm_token_equals_decode_matvec(dev, devbuf):
     dev.SetActWindow(32)
 
 
-@pytest.mark.parametrize("t,window,ntok", [(quant.Q8_0, 32, 2), (quant.Q6_K, 32, 2), (quant.Q4_K, 32, 9),
+@pytest.mark.parametrize("t,window,ntok", [(quant.Q8_0, 32, 2), (quant.Q8_0, 32, 1), (quant.Q6_K, 32, 2), (quant.Q4_K, 32, 9),
                                            (quant.Q4_K, 256, 3)])
 def test_matmul_fallback_is_the_per_token_loop(dev, devbuf, t, window, ntok):
     """Types, windows and token counts the GEMM does not take still return the right values."""
