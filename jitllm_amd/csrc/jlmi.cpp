@@ -28,7 +28,7 @@ const HipApi* H = nullptr;  // the process-wide HIP runtime, resolved by the fir
 
 struct Tuning {
     int rpw = 0, block = 0, grid = 0;
-    int packed_rw = 0, packed_block = 0, moe_group = 0, moe_logits = 0;
+    int packed_rw = 0, packed_block = 0, moe_group = 0, moe_logits = 0, moe_q6k_cols = 0;
     int moe_shares = 0;
     int gemm_rows = 0;
     int gemm_form = 0;
@@ -829,8 +829,14 @@ int moe_matvec_launch(jl_ctx* c, float* out0, float* out1, int type, const void*
     //   256 rows 366 / 243 / 352   512 rows 630 / 330 / 388    768 rows 916 / 416 / 429
     //   1024 rows 1180 / 496 / 463                             2048 rows 2177 / 815 / 720
     // so form 2 takes over from ten columns an expert on average and form 4 from 56.
-    const bool many_cols = c->tune.moe_form == 0 && (long)ncols >= 10L * n_expert;
-    if (type == JL_TYPE_Q4_K && c->act_window == 256 && (c->tune.moe_form == 2 || c->tune.moe_form == 4 || many_cols) &&
+    // Q6_K sheets (the down projections of a model whose other experts are Q4_K) have form 4
+    // alone, with the Q6_K GEMM's tile; the dot-product kernel is slower for that type, so the
+    // tile takes over earlier ("moe.q6k_cols": columns an expert on average, default 12).
+    const bool q6 = type == JL_TYPE_Q6_K;
+    const long q6_cols = c->tune.moe_q6k_cols > 0 ? c->tune.moe_q6k_cols : 12;
+    const bool many_cols = c->tune.moe_form == 0 && (long)ncols >= (q6 ? q6_cols : 10L) * n_expert;
+    if ((type == JL_TYPE_Q4_K || q6) && c->act_window == 256 &&
+        (c->tune.moe_form == 4 || many_cols || (!q6 && c->tune.moe_form == 2)) &&
         4u * 19968u <= c->lds_limit) {   // JL_MOEG_WAVE_LDS
         const int nslots = ncols / 32 + n_expert + 1, nsb = k / 256;
         const int tiles_max = ncols / 128 + n_expert;
@@ -862,15 +868,16 @@ int moe_matvec_launch(jl_ctx* c, float* out0, float* out1, int type, const void*
         ga.nslots = nslots; ga.nmat = bank1 ? 2 : 1;
         void* gp[] = {&ga};
         const long rtiles = (nrows + 63) / 64;
-        if ((c->tune.moe_form == 4 || (c->tune.moe_form == 0 && (long)ncols >= 56L * n_expert)) &&
+        if ((q6 || c->tune.moe_form == 4 || (c->tune.moe_form == 0 && (long)ncols >= 56L * n_expert)) &&
             kGemmLdsBytes <= c->lds_limit && n_expert <= 65535 && (long)tiles_max * rtiles * ga.nmat < (1L << 31)) {
             const long work = (long)tiles_max * rtiles * ga.nmat;
-            const unsigned grid = (unsigned)std::min<long>(work, 2L * c->num_cu);
-            HIP_TRY(c, H->ModuleLaunchKernel(c->fn["jl_moe_gemm_r64"], grid, 1, 1, 256, 1, 1,
-                                             gemm_lds_bytes(64), st, gp, nullptr));
+            const unsigned grid = (unsigned)std::min<long>(work, (q6 ? 3L : 2L) * c->num_cu);
+            HIP_TRY(c, H->ModuleLaunchKernel(c->fn[q6 ? "jl_moe_gemm_q6k_r64" : "jl_moe_gemm_r64"], grid, 1, 1, 256, 1, 1,
+                                             q6 ? kGemm6LdsBytes : gemm_lds_bytes(64), st, gp, nullptr));
             c->launches++;
             return JL_OK;
         }
+        if (q6) return fail(c, JL_ERR_ARG, "moe matvec: %d experts x %ld row tiles do not fit the tile form", n_expert, rtiles);
         HIP_TRY(c, H->ModuleLaunchKernel(c->fn["jl_moe_gemm_q4k"], (unsigned)((nrows + 255) / 256),
                                          (unsigned)nslots, (unsigned)ga.nmat, 256, 1, 1, 4u * 19968u, st,
                                          gp, nullptr));
@@ -981,7 +988,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     if (e != hipSuccess)
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
-    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_quant", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_q4k", "jl_moe_gemm_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_sum_parts",
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_quant", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_q4k", "jl_moe_gemm_r64", "jl_moe_gemm_q6k_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_sum_parts",
                                       "jl_pack_weights", "jl_unpack_q4k", "jl_unpack_q6k", "jl_unpack_q8_0"};
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int rw : {16, 32, 64})
@@ -1075,6 +1082,7 @@ int jl_set_tuning(jl_ctx* c, const char* key, int value) {
     else if (!strcmp(key, "packed.block")) c->tune.packed_block = value;
     else if (!strcmp(key, "moe.group")) c->tune.moe_group = value;
     else if (!strcmp(key, "moe.logits")) c->tune.moe_logits = value;
+    else if (!strcmp(key, "moe.q6k_cols")) c->tune.moe_q6k_cols = value;
     else if (!strcmp(key, "moe.shares")) c->tune.moe_shares = value;
     else if (!strcmp(key, "moe.form")) c->tune.moe_form = value;
     else if (!strcmp(key, "moe.waves")) c->tune.moe_waves = value;

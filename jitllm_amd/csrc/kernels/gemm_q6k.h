@@ -38,18 +38,21 @@ struct Gemm6Raw {
     u32 sc;   // the four int8 scales 8n + 4hh .. + 3
 };
 
-__device__ __forceinline__ void gemm_q6k_body(const GemmArgs& p0, uint8_t* smem) {
-    GemmArgs p = p0;
-    if (p.sb_per) {   // K split: this workgroup's super-blocks, partial sums to slab z
-        const int sb0 = blockIdx.z * p.sb_per;
-        const int n = min(p.sb_per, p.k / 256 - sb0);
-        p.w += (size_t)sb0 * 210;
-        p.bq += (size_t)2 * sb0 * (p.tok_pad >> 5) * (JL_GEMM_ASTAGE_FRAGS * JL_GEMM_AFRAG_HALFS);
-        p.da += (size_t)sb0 * p.tok_pad;
-        p.k = 256 * n;
-        p.out += (size_t)blockIdx.z * p.ntok * p.out_stride;
-    }
-    const int t0 = blockIdx.x * JL_GEMM_TILE, r0 = blockIdx.y * 64;
+// K split: workgroup z takes sb_per super-blocks and writes its partial sums to slab z
+__device__ __forceinline__ void gemm_q6k_split_slice(GemmArgs& p) {
+    if (p.sb_per == 0) return;
+    const int sb0 = blockIdx.z * p.sb_per;
+    const int n = min(p.sb_per, p.k / 256 - sb0);
+    p.w += (size_t)sb0 * 210;
+    p.bq += (size_t)2 * sb0 * (p.tok_pad >> 5) * (JL_GEMM_ASTAGE_FRAGS * JL_GEMM_AFRAG_HALFS);
+    p.da += (size_t)sb0 * p.tok_pad;
+    p.k = 256 * n;
+    p.out += (size_t)blockIdx.z * p.ntok * p.out_stride;
+}
+
+// t0, r0: the tile's first token and row (a grouped launch places tiles per expert; a
+// wavefront whose tokens lie past ntok loads and computes nothing)
+__device__ __forceinline__ void gemm_q6k_body(const GemmArgs& p, uint8_t* smem, int t0, int r0) {
     _Float16* sA = (_Float16*)smem;                 // [64][JL_GEMM_STRIDE]: 2 * (sc >> 1) * (q - 32)
     _Float16* sB = sA + 64 * JL_GEMM_STRIDE;        // (sc & 1) * (q - 32)
     const int tid = threadIdx.x, lane = tid & 63;

@@ -141,7 +141,10 @@ extern "C" __global__ __launch_bounds__(256, 2) void jl_gemm_q4k_r64(GemmArgs p)
 }
 // Q6_K with the k-quant window: grid = (tok_pad/128, ceil(nrows/64), K splits), block = 256,
 // dynamic LDS = JL_GEMM6_LDS_BYTES; the activation prep is jl_gemm_prep_q4k
-extern "C" __global__ __launch_bounds__(256, 2) void jl_gemm_q6k_r64(GemmArgs p) { gemm_q6k_body(p, jl_smem); }
+extern "C" __global__ __launch_bounds__(256, 2) void jl_gemm_q6k_r64(GemmArgs p) {
+    gemm_q6k_split_slice(p);
+    gemm_q6k_body(p, jl_smem, blockIdx.x * JL_GEMM_TILE, blockIdx.y * 64);
+}
 // Q8_0 and Q6_K with the activation window of 32: prep grid = (ceil(k/256), tok_pad/32), block = 256;
 // matrix kernel grid = (tok_pad/128, ceil(nrows/64), K splits), block = 256, dynamic LDS =
 // JL_GEMM32_LDS_BYTES(planes)
@@ -218,7 +221,8 @@ extern "C" __global__ __launch_bounds__(256, 2) void jl_moe_gemm_q4k(MoeGemmArgs
 // are a token range; columns past the expert's last are computed and not stored.  The
 // workgroups stride over (row tile, column tile of the work list, matrix), so none is empty.
 // grid = up to two workgroups a CU, block = 256, dynamic LDS as jl_gemm_q4k_r64.
-extern "C" __global__ __launch_bounds__(256, 2) void jl_moe_gemm_r64(MoeGemmArgs p) {
+template <int TYPE>
+__device__ __forceinline__ void moe_gemm_tiles(const MoeGemmArgs& p) {
     const u32 rtiles = (u32)(p.nrows + 63) / 64;
     const u32 ntiles = p.wl[0];
     const u32 per_mat = ntiles * rtiles, total = per_mat * (u32)p.nmat;
@@ -238,10 +242,14 @@ extern "C" __global__ __launch_bounds__(256, 2) void jl_moe_gemm_r64(MoeGemmArgs
         g.ntok = 32 * slot0 + ncol;                  // tokens are positions in the workspace
         g.out_stride = p.nrows; g.sb_per = 0;
         g.out = p.out[mat] + ((ptrdiff_t)c_lo - (ptrdiff_t)32 * slot0) * p.nrows;   // workspace position -> column
-        gemm_q4k_body<1, true>(g, jl_smem, 32 * slot0 + 128 * ctile, (int)rt * 64);
+        if constexpr (TYPE == JL_Q6_K) gemm_q6k_body(g, jl_smem, 32 * slot0 + 128 * ctile, (int)rt * 64);
+        else gemm_q4k_body<1, true>(g, jl_smem, 32 * slot0 + 128 * ctile, (int)rt * 64);
         __syncthreads();   // the tile's LDS is free for the next one
     }
 }
+extern "C" __global__ __launch_bounds__(256, 2) void jl_moe_gemm_r64(MoeGemmArgs p) { moe_gemm_tiles<JL_Q4_K>(p); }
+// Q6_K sheets: dynamic LDS = JL_GEMM6_LDS_BYTES
+extern "C" __global__ __launch_bounds__(256, 2) void jl_moe_gemm_q6k_r64(MoeGemmArgs p) { moe_gemm_tiles<JL_Q6_K>(p); }
 // grid = 1, block = 1024
 extern "C" __global__ __launch_bounds__(1024) void jl_moe_worklist(MoeWorklistArgs p) {
     __shared__ u32 tot[16];

@@ -77,7 +77,9 @@ def _banks(t, n_expert, nrows, k, seed, planted):
                                             (quant.Q4_K, 300, 768, 2), (quant.Q4_K, 40, 4096, 2),
                                             (quant.Q4_K, 96, 2048, 4), (quant.Q4_K, 300, 768, 4),
                                             (quant.Q4_K, 40, 4096, 4), (quant.Q4_K, 129, 256, 4),
-                                            (quant.Q8_0, 64, 1024, 0), (quant.Q6_K, 70, 1024, 0)])
+                                            (quant.Q8_0, 64, 1024, 0), (quant.Q6_K, 70, 1024, 0),
+                                            (quant.Q6_K, 96, 2048, 4), (quant.Q6_K, 300, 768, 4),
+                                            (quant.Q6_K, 129, 256, 4)])
 def test_grouped_matvec_vs_oracle(dev, devbuf, t, nrows, k, form):
     """form 1 = the dot-product kernel, 2 = groups of 32 columns on the matrix cores (Q4_K with
     the k-quant window), 4 = the prefill GEMM's 128-column x 64-row tile placed per expert,
@@ -130,12 +132,14 @@ def test_grouped_matvec_vs_oracle(dev, devbuf, t, nrows, k, form):
     dev.set_tuning(moe__form=0)
 
 
+@pytest.mark.parametrize("t", [quant.Q4_K, quant.Q6_K], ids=["q4_k", "q6_k"])
 @pytest.mark.parametrize("rows", [70, 150])
-def test_grouped_matmul_more_than_one_group_of_columns(dev, devbuf, rows):
+def test_grouped_matmul_more_than_one_group_of_columns(dev, devbuf, rows, t):
     """An expert chosen by 70 rows has three groups of 32 columns (the last one ragged), by 150
     rows five groups and two tiles of 128 columns; another gets one column, most get none.
-    Every form against the oracle."""
-    t, nrows, k, window = quant.Q4_K, 130, 512, 256
+    Every form against the oracle (Q6_K sheets: the dot-product kernel, the tile, the
+    library's pick)."""
+    nrows, k, window = 130, 512, 256
     n_expert, k_used = 6, 2
     dev.SetActWindow(window)
     sel = np.zeros((rows, k_used + 1), np.uint32)
@@ -152,7 +156,7 @@ def test_grouped_matmul_more_than_one_group_of_columns(dev, devbuf, rows):
         q, a_s, _ = oracle.quantize_act(x[perm[c]], window)
         want[c] = oracle.matvec_q8act_f64(t, bank[e * sheet:(e + 1) * sheet], q, a_s, nrows, k)
     b, xd, dstart, dperm = devbuf(bank), devbuf(x), devbuf(start), devbuf(perm[:used].copy())
-    for form in (1, 2, 4):
+    for form in ((1, 2, 4) if t == quant.Q4_K else (1, 4, 0)):
         dev.set_tuning(moe__form=form)
         o = devbuf(shape=(used * nrows + 8,), dtype=np.float32, fill=np.float32(4e30))
         assert dev.moe_matvec_dev(o.ptr, None, t, b.ptr, None, xd.ptr, None, dperm.ptr, dstart.ptr, n_expert, used,
