@@ -346,6 +346,14 @@ int jl_moe_ffn_dev(jl_ctx *ctx, float *resid, int type, const void *gate_bank,
                    const uint32_t *sel, int sel_stride, const float *wt, int rows, int k_used,
                    int n_expert, int n_ffn, int n_embd, void *stream);
 
+/* The same block with the down bank in a type of its own: every expert tensor carries its
+ * own quant.Type in the reference (nn.Weight.T, engine/nn/device.go:47-58; a Q4_K_M file
+ * holds Q4_K gate and up sheets beside Q6_K down sheets). */
+int jl_moe_ffn_types_dev(jl_ctx *ctx, float *resid, int type, int down_type, const void *gate_bank,
+                         const void *up_bank, const void *down_bank, const float *x,
+                         const uint32_t *sel, int sel_stride, const float *wt, int rows,
+                         int k_used, int n_expert, int n_ffn, int n_embd, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -74,6 +74,8 @@ SIGNATURES = {
     "jl_moe_combine_dev": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _vp, _int, _int, _int, _vp]),
     "jl_moe_ffn_dev": (_int, [_vp, _vp, _int, _vp, _vp, _vp, _vp, _vp, _int, _vp, _int, _int, _int, _int,
                               _int, _vp]),
+    "jl_moe_ffn_types_dev": (_int, [_vp, _vp, _int, _int, _vp, _vp, _vp, _vp, _vp, _int, _vp, _int, _int, _int,
+                                    _int, _int, _vp]),
 }
 
 _lib = None

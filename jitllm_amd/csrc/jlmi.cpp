@@ -1366,8 +1366,8 @@ int jl_moe_combine_dev(jl_ctx* c, float* resid, const float* y, const float* wt,
                   pick_stream(c, stream), params);
 }
 
-int jl_moe_ffn_dev(jl_ctx* c, float* resid, int type, const void* gate_bank, const void* up_bank,
-                   const void* down_bank, const float* x, const uint32_t* sel, int sel_stride,
+int jl_moe_ffn_types_dev(jl_ctx* c, float* resid, int type, int down_type, const void* gate_bank, const void* up_bank,
+                         const void* down_bank, const float* x, const uint32_t* sel, int sel_stride,
                    const float* wt, int rows, int k_used, int n_expert, int n_ffn, int n_embd, void* stream) {
     if (!c) return JL_ERR_ARG;
     if (rows <= 0 || k_used <= 0 || n_expert <= 0 || n_ffn <= 0 || n_embd <= 0)
@@ -1393,9 +1393,16 @@ int jl_moe_ffn_dev(jl_ctx* c, float* resid, int type, const void* gate_bank, con
     rc = moe_matvec_launch(c, g, u, type, gate_bank, up_bank, x, nullptr, perm, start, n_expert, (int)ncols, n_ffn, n_embd, st);
     if (rc != JL_OK) return rc;
     // down: the activation of column c is silu(g[c]) * u[c]
-    rc = moe_matvec_launch(c, y, nullptr, type, down_bank, nullptr, g, u, nullptr, start, n_expert, (int)ncols, n_embd, n_ffn, st);
+    rc = moe_matvec_launch(c, y, nullptr, down_type, down_bank, nullptr, g, u, nullptr, start, n_expert, (int)ncols, n_embd, n_ffn, st);
     if (rc != JL_OK) return rc;
     return jl_moe_combine_dev(c, resid, y, wt, sel, sel_stride, pos, rows, k_used, n_embd, st);
+}
+
+int jl_moe_ffn_dev(jl_ctx* c, float* resid, int type, const void* gate_bank, const void* up_bank,
+                   const void* down_bank, const float* x, const uint32_t* sel, int sel_stride,
+                   const float* wt, int rows, int k_used, int n_expert, int n_ffn, int n_embd, void* stream) {
+    return jl_moe_ffn_types_dev(c, resid, type, type, gate_bank, up_bank, down_bank, x, sel, sel_stride, wt, rows,
+                                k_used, n_expert, n_ffn, n_embd, stream);
 }
 
 int jl_matmul_mxfp4_bf16_dev(jl_ctx* c, float* out, const void* w, const uint16_t* x, int nrows, int k,

@@ -270,12 +270,14 @@ class Device:
                             "jl_moe_combine_dev")
 
     def moe_ffn_dev(self, resid, t, gate, up, down, x, sel, sel_stride, wt, rows, k_used, n_expert,
-                    n_ffn, n_embd, stream=None):
-        """One routed feed-forward block (moeBatchFrom): resid [rows][n_embd] += mixture output."""
-        return self._served(self._l.jl_moe_ffn_dev(self._ctx, _ptr(resid), t, _ptr(gate), _ptr(up),
-                                                   _ptr(down), _ptr(x), _ptr(sel), sel_stride, _ptr(wt),
-                                                   rows, k_used, n_expert, n_ffn, n_embd, stream),
-                            "jl_moe_ffn_dev")
+                    n_ffn, n_embd, stream=None, down_type=None):
+        """One routed feed-forward block (moeBatchFrom): resid [rows][n_embd] += mixture output.
+        down_type: the down bank's type where it differs from gate and up."""
+        return self._served(self._l.jl_moe_ffn_types_dev(self._ctx, _ptr(resid), t, t if down_type is None else down_type,
+                                                         _ptr(gate), _ptr(up), _ptr(down), _ptr(x), _ptr(sel),
+                                                         sel_stride, _ptr(wt), rows, k_used, n_expert, n_ffn, n_embd,
+                                                         stream),
+                            "jl_moe_ffn_types_dev")
 
     def matmul_mxfp4_bf16_dev(self, out, w, x, nrows, k, ntok, stream=None):
         """MXFP4 weights x bf16 activations (bits as uint16) -> f32 out [ntok][nrows]."""

@@ -219,10 +219,11 @@ def test_combine_order_and_values(dev, devbuf):
     assert np.array_equal(rd.get().view(np.uint32), want.view(np.uint32))
 
 
-def _oracle_block(t, gate, up, down, x, sel, wt, n_expert, n_ffn, n_embd, window):
+def _oracle_block(t, gate, up, down, x, sel, wt, n_expert, n_ffn, n_embd, window, td=None):
     rows, k_used = wt.shape
     out = np.zeros((rows, n_embd))
-    gs, ds = n_ffn * quant.row_bytes(t, n_embd), n_embd * quant.row_bytes(t, n_ffn)
+    td = t if td is None else td
+    gs, ds = n_ffn * quant.row_bytes(t, n_embd), n_embd * quant.row_bytes(td, n_ffn)
     for e in range(n_expert):                   # expert-major, rows ascending
         for r in range(rows):
             for s in range(k_used):
@@ -233,7 +234,7 @@ def _oracle_block(t, gate, up, down, x, sel, wt, n_expert, n_ffn, n_embd, window
                 u = oracle.matvec_q8act_f64(t, up[e * gs:(e + 1) * gs], q, a_s, n_ffn, n_embd)
                 h = (silu(g.astype(np.float32)) * u.astype(np.float32)).astype(np.float32)
                 qh, ah, _ = oracle.quantize_act(h, window)
-                y = oracle.matvec_q8act_f64(t, down[e * ds:(e + 1) * ds], qh, ah, n_embd, n_ffn)
+                y = oracle.matvec_q8act_f64(td, down[e * ds:(e + 1) * ds], qh, ah, n_embd, n_ffn)
                 out[r] += float(wt[r, s]) * y
     return out
 
@@ -261,6 +262,27 @@ def test_moe_block_vs_oracle(dev, devbuf, shape):
         dev.synchronize()
         got = resid.get()
         assert rel_l2(got, want) <= 1e-3, f"call {call}: rel-L2 {rel_l2(got, want):.3e}"
+    dev.SetActWindow(32)
+
+
+@pytest.mark.parametrize("rows", [6, 70])
+def test_moe_block_q6k_down_sheets_vs_oracle(dev, devbuf, rows):
+    """Gate and up in Q4_K, down in Q6_K (the mix of a Q4_K_M file), few columns an expert (the
+    dot-product kernels) and many (matrix-core tiles of both types)."""
+    n_expert, k_used, n_ffn, n_embd, window = 4, 2, 256, 512, 256
+    dev.SetActWindow(window)
+    sel, wt = route(rows, n_expert, k_used, 21)
+    gate = _banks(quant.Q4_K, n_expert, n_ffn, n_embd, 1100, False)
+    up = _banks(quant.Q4_K, n_expert, n_ffn, n_embd, 2100, False)
+    down = _banks(quant.Q6_K, n_expert, n_embd, n_ffn, 3100, False)
+    x = np.stack([synth.activations(n_embd, seed=700 + r) for r in range(rows)])
+    want = _oracle_block(quant.Q4_K, gate, up, down, x, sel, wt, n_expert, n_ffn, n_embd, window, quant.Q6_K)
+    gd, ud, dd, xd, sd, wd = devbuf(gate), devbuf(up), devbuf(down), devbuf(x), devbuf(sel), devbuf(wt)
+    resid = devbuf(shape=(rows, n_embd), dtype=np.float32, fill=0)
+    assert dev.moe_ffn_dev(resid.ptr, quant.Q4_K, gd.ptr, ud.ptr, dd.ptr, xd.ptr, sd.ptr, k_used + 1, wd.ptr,
+                           rows, k_used, n_expert, n_ffn, n_embd, down_type=quant.Q6_K)
+    dev.synchronize()
+    assert rel_l2(resid.get(), want) <= 1e-3
     dev.SetActWindow(32)
 
 
