@@ -542,37 +542,38 @@ int gemm_q6k_launch(jl_ctx* c, float* out, const void* w, const float* x, int nr
                   kGemm6LdsBytes, st, gp);
 }
 
-// Q8_0 and Q6_K prefill GEMM with the activation window of 32 (kernels/gemm_w32.h): its own
+// Q8_0, Q6_K and Q4_K prefill GEMM with the activation window of 32 (kernels/gemm_w32.h): its own
 // prep (fragments in the order of the byte unpack, a token scale per 32), 128-token x 64-row
 // tiles, K split in stages of 128 (Q6_K: whole super-blocks) for small grids.
 constexpr unsigned gemm32_lds_bytes(int planes) {   // JL_GEMM32_LDS_BYTES
-    return (unsigned)planes * 64u * kGemmStride * 2u + 64u * 4u * 4u + 4u * kGemmTile * 4u;
+    return (unsigned)planes * 64u * kGemmStride * 2u + 2u * 64u * 4u * 4u + 2u * 4u * kGemmTile * 4u;
 }
 
 int gemm_w32_launch(jl_ctx* c, float* out, int type, const void* w, const float* x, int nrows, int k, int ntok,
                     hipStream_t st) {
-    const bool q6 = type == JL_TYPE_Q6_K;
-    const char* kernel = q6 ? "jl_gemm_q6k_w32" : "jl_gemm_q8_0_w32";
+    const bool q6 = type == JL_TYPE_Q6_K, q4 = type == JL_TYPE_Q4_K;
+    const char* kernel = q6 ? "jl_gemm_q6k_w32" : q4 ? "jl_gemm_q4k_w32" : "jl_gemm_q8_0_w32";
     const unsigned lds = gemm32_lds_bytes(q6 ? 2 : 1);
     const int tok_pad = (ntok + kGemmTile - 1) / kGemmTile * kGemmTile, nstage = k / 128;
-    const size_t bq_bytes = (size_t)nstage * (tok_pad / 32) * 8 * 1024;
-    int rc = gemm_ws_ensure(c, bq_bytes + (size_t)(k / 32) * tok_pad * 4);
+    const size_t bq_bytes = (size_t)nstage * (tok_pad / 32) * 8 * 1024, da_bytes = (size_t)(k / 32) * tok_pad * 4;
+    int rc = gemm_ws_ensure(c, bq_bytes + (q4 ? 2 : 1) * da_bytes);
     if (rc != JL_OK) return rc;
     uint16_t* bq = (uint16_t*)c->gemm_ws;
     float* da = (float*)((char*)c->gemm_ws + bq_bytes);
     GemmPrepArgs pa;
     pa.x = x; pa.bq = bq; pa.da = da; pa.ntok = ntok; pa.tok_pad = tok_pad; pa.k = k;
+    if (q4) pa.dsum = (float*)((char*)da + da_bytes);   // the minimums meet d_a * block sums
     void* pp[] = {&pa};
     rc = launch(c, "jl_gemm_prep_w32", (unsigned)((k + 255) / 256), (unsigned)(tok_pad / 32), 256, 0, st, pp);
     if (rc != JL_OK) return rc;
     GemmArgs ga;
     ga.out = out; ga.w = (const uint8_t*)w; ga.bq = bq; ga.da = da;
     ga.nrows = nrows; ga.k = k; ga.ntok = ntok; ga.tok_pad = tok_pad;
-    ga.row_bytes = q6 ? (k / 256) * 210 : (k / 32) * 34;
-    ga.out_stride = nrows; ga.sb_per = 0;
+    ga.row_bytes = q6 ? (k / 256) * 210 : q4 ? (k / 256) * 144 : (k / 32) * 34;
+    ga.out_stride = nrows; ga.sb_per = 0; ga.dsum = pa.dsum;
     void* gp[] = {&ga};
     const long groups = (long)(tok_pad / kGemmTile) * ((nrows + 63) / 64);
-    const int unit = q6 ? 2 : 1, nunit = nstage / unit;   // stages a split is made of
+    const int unit = q6 || q4 ? 2 : 1, nunit = nstage / unit;   // stages a split is made of
     int nsplit = c->tune.gemm_split > 0 ? c->tune.gemm_split : (groups <= c->num_cu ? (int)(2 * c->num_cu / groups) : 1);
     if (nsplit > 8) nsplit = 8;
     if (nsplit > nunit) nsplit = nunit;
@@ -619,8 +620,8 @@ int matmul_launch(jl_ctx* c, float* out, int type, const void* w, const float* x
                                nrows, k, st);
         if (rc != JL_DECLINED) return rc;
     }
-    if ((type == JL_TYPE_Q8_0 || type == JL_TYPE_Q6_K) && c->act_window == 32 && ntok >= c->gemm_min_tok &&
-        c->tune.gemm_form != 9 && k % 128 == 0 && ((uintptr_t)w & 1) == 0 && ntok <= 65535 * 4 &&
+    if ((type == JL_TYPE_Q8_0 || type == JL_TYPE_Q6_K || type == JL_TYPE_Q4_K) && c->act_window == 32 &&
+        ntok >= c->gemm_min_tok && c->tune.gemm_form != 9 && k % 128 == 0 && ((uintptr_t)w & 1) == 0 && ntok <= 65535 * 4 &&
         (nrows + 63) / 64 <= 65535 && gemm32_lds_bytes(2) <= c->lds_limit)
         return gemm_w32_launch(c, out, type, w, x, nrows, k, ntok, st);
     for (int t = 0; t < ntok; t++) {
@@ -785,7 +786,7 @@ int packed_matmul_launch(jl_ctx* c, float* out, int type, const PlaneRef& pl, co
     const bool gemm6 = type == JL_TYPE_Q6_K && c->act_window == 256 && ntok >= c->gemm_min_tok &&
                        c->tune.gemm_form != 9 && ntok <= 65535 * 4 && (nrows + 63) / 64 <= 65535 &&
                        kGemm6LdsBytes <= c->lds_limit && k / 256 <= 65535;
-    const bool gemm32 = (type == JL_TYPE_Q8_0 || type == JL_TYPE_Q6_K) && c->act_window == 32 &&
+    const bool gemm32 = (type == JL_TYPE_Q8_0 || type == JL_TYPE_Q6_K || type == JL_TYPE_Q4_K) && c->act_window == 32 &&
                         ntok >= c->gemm_min_tok && c->tune.gemm_form != 9 && k % 128 == 0 && ntok <= 65535 * 4 &&
                         (nrows + 63) / 64 <= 65535 && gemm32_lds_bytes(2) <= c->lds_limit && k / 32 <= 65535;
     if (gemm || gemm6 || gemm32) {
@@ -988,7 +989,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     if (e != hipSuccess)
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
-    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_quant", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_q4k", "jl_moe_gemm_r64", "jl_moe_gemm_q6k_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_sum_parts",
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_quant", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_q4k", "jl_moe_gemm_r64", "jl_moe_gemm_q6k_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_sum_parts",
                                       "jl_pack_weights", "jl_unpack_q4k", "jl_unpack_q6k", "jl_unpack_q8_0"};
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int rw : {16, 32, 64})

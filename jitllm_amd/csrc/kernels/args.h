@@ -49,6 +49,7 @@ struct GemmPrepArgs {
     uint16_t* bq;        // f16 bits
     float* da;
     int ntok, tok_pad, k;
+    float* dsum = nullptr;   // window 32, optional: d_a * (sum of the block's int8) [k/32][tok_pad]
 };
 
 struct GemmArgs {
@@ -60,6 +61,7 @@ struct GemmArgs {
     int row_bytes;
     int out_stride;      // floats between tokens in out
     int sb_per;          // K split: super-blocks per blockIdx.z (0 = whole K), out = slab z of [gridDim.z][ntok][out_stride]
+    const float* dsum = nullptr;   // window 32, Q4_K: the prep's d_a * block sums
 };
 
 // Mixture block on the matrix cores (Q4_K, activation window 256).  An expert's columns are

@@ -1,7 +1,7 @@
 // Prefill GEMM with the activation window of 32 (the window of a model that holds a type
-// with 32-element blocks, jit/cpu/matvec.go:46-62), Q8_0 and Q6_K weights.  Per (token, row)
-// it is the decode matvec's value (format/quant/dequant.go:148-157 and :443-470 for the
-// weights, jit/cpu/packedgemm.go:54-58 for the identity with the matvec):
+// with 32-element blocks, jit/cpu/matvec.go:46-62), Q8_0, Q6_K and Q4_K weights.  Per (token,
+// row) it is the decode matvec's value (format/quant/dequant.go:148-157, :443-470 and :360-397
+// for the weights, jit/cpu/packedgemm.go:54-58 for the identity with the matvec):
 //
 //   out[t][r] = sum_b d[r,b] * d_a[t,b] * P[t,r,b],   P = sum_{l<32} q[r,b,l] * a[t,b,l]
 //
@@ -12,6 +12,9 @@
 // Q6_K: q is sc * (q6 - 32) with the int8 sub-block scale split into two exact f16 operands
 // as in gemm_q6k.h (two planes in LDS, four matrix instructions a K-step pair and tile), d
 // the super-block's.
+// Q4_K: q is the nibble, d the product d * sc of the 32-element sub-block, and the minimum
+// joins as  - (dmin * m) * (d_a * sum of the block's activations), the second factor from
+// the prep: a third vector instruction an element.
 //
 // Activation prep (gemm_prep_w32_body): x [ntok][k] f32 -> bq [k/128 stages][tok_pad/32]
 // [8 K-steps][64 lanes][8] f16 and da [k/32][tok_pad] f32.  Lane (t = lane%32, kg = lane/32)
@@ -27,12 +30,12 @@
 // that share a CU cover each other's vector phases.  Q6_K: thread = row, 32-element run of the
 // half super-block (ql nibbles + two qh bits, two sub-block scales).
 // grid = (tok_pad/128, ceil(nrows/64), K splits), block = 256, dynamic LDS =
-// JL_GEMM32_LDS_BYTES(planes), planes = 1 (Q8_0) or 2 (Q6_K).
+// JL_GEMM32_LDS_BYTES(planes), planes = 1 (Q8_0, Q4_K) or 2 (Q6_K).
 #pragma once
 #include "gemm_q4k.h"
 
 #define JL_GEMM32_FRAGS 8
-#define JL_GEMM32_LDS_BYTES(planes) ((planes) * 64 * JL_GEMM_STRIDE * 2 + 64 * 4 * 4 + 4 * JL_GEMM_TILE * 4)
+#define JL_GEMM32_LDS_BYTES(planes) ((planes) * 64 * JL_GEMM_STRIDE * 2 + 2 * 64 * 4 * 4 + 2 * 4 * JL_GEMM_TILE * 4)
 
 __device__ __forceinline__ void gemm_prep_w32_body(const GemmPrepArgs& p, u32* sq) {
     // sq [32 tokens][65]: 64 words of int8 + 1 pad (bank spread)
@@ -54,7 +57,13 @@ __device__ __forceinline__ void gemm_prep_w32_body(const GemmPrepArgs& p, u32* s
         float d;
         i32 sum16;
         sq[tl * 65 + lane] = quantize4(v[i], amax, d, sum16);
-        if ((lane & 7) == 0 && e0 < p.k) p.da[(size_t)(ch * 8 + (lane >> 3)) * p.tok_pad + grp * 32 + tl] = d;
+        // the block's sum from its two half-block sums (eight lanes a block)
+        const i32 a32 = sum16 + dpp_i32<JL_DPP_ROW_HALF_MIRROR, 0xf>(0, sum16);
+        if ((lane & 7) == 0 && e0 < p.k) {
+            const size_t at = (size_t)(ch * 8 + (lane >> 3)) * p.tok_pad + grp * 32 + tl;
+            p.da[at] = d;
+            if (p.dsum) p.dsum[at] = d * (float)a32;
+        }
     }
     __syncthreads();
     const int tl = lane & 31, kg = lane >> 5;
@@ -78,18 +87,20 @@ struct Gemm32Raw {
     u32x4 h0, h1;   // Q6_K: the half's 32 qh bytes
     u32 d;          // Q8_0: the block's f16 scale; Q6_K: d | the run's two int8 scales << 16
     float da[2];    // two of the stage's 4 x 128 token scales
+    float ds[2];    // Q4_K: and of its d_a * block sums
 };
 
 template <int TYPE>
 __device__ __forceinline__ void gemm_w32_body(const GemmArgs& p0, uint8_t* smem) {
-    constexpr bool Q6 = TYPE == JL_Q6_K;
+    constexpr bool Q6 = TYPE == JL_Q6_K, Q4 = TYPE == JL_Q4_K;
     constexpr int NPL = Q6 ? 2 : 1;
-    constexpr int STAGE_BYTES = Q6 ? 105 : 4 * 34;   // 128 weights; a Q6_K half super-block shares its block
+    constexpr int SB_BYTES = Q6 ? 210 : 144;   // k-quants: a stage is half a super-block
     GemmArgs p = p0;
-    if (p.sb_per) {   // K split: sb_per stages to a workgroup (Q6_K: an even number), partial sums to slab z
+    if (p.sb_per) {   // K split: sb_per stages to a workgroup (k-quants: an even number), partial sums to slab z
         const int s0 = blockIdx.z * p.sb_per;
         const int n = min(p.sb_per, p.k / 128 - s0);
-        p.w += Q6 ? (size_t)(s0 / 2) * 210 : (size_t)s0 * STAGE_BYTES;
+        p.w += Q6 || Q4 ? (size_t)(s0 / 2) * SB_BYTES : (size_t)s0 * 4 * 34;
+        if (Q4) p.dsum += (size_t)s0 * 4 * p.tok_pad;
         p.bq += (size_t)s0 * (p.tok_pad >> 5) * (JL_GEMM32_FRAGS * JL_GEMM_AFRAG_HALFS);
         p.da += (size_t)s0 * 4 * p.tok_pad;
         p.k = 128 * n;
@@ -98,7 +109,9 @@ __device__ __forceinline__ void gemm_w32_body(const GemmArgs& p0, uint8_t* smem)
     const int t0 = blockIdx.x * JL_GEMM_TILE, r0 = blockIdx.y * 64;
     _Float16* sW = (_Float16*)smem;                            // [planes][64][JL_GEMM_STRIDE]
     float* sD = (float*)(sW + NPL * 64 * JL_GEMM_STRIDE);      // [64 rows][4 blocks]
-    float* sDa = sD + 64 * 4;                                  // [4 blocks][128 tokens]
+    float* sD2 = sD + 64 * 4;                                  // Q4_K: dmin * m, [64 rows][4 blocks]
+    float* sDa = sD2 + 64 * 4;                                 // [4 blocks][128 tokens]
+    float* sDs = sDa + 4 * JL_GEMM_TILE;                       // Q4_K: d_a * block sum, [4 blocks][128 tokens]
     const int tid = threadIdx.x, lane = tid & 63;
     const int tg = __builtin_amdgcn_readfirstlane(tid >> 6);   // this wavefront: tokens 32*tg..
     const bool live = t0 + 32 * tg < p.ntok;                   // else no token of its 32 exists
@@ -117,6 +130,16 @@ __device__ __forceinline__ void gemm_w32_body(const GemmArgs& p0, uint8_t* smem)
             r.h0 = ld16_a2(blk + 128 + 32 * n);
             r.h1 = ld16_a2(blk + 128 + 32 * n + 16);
             r.d = (u32)ld2(blk + 208) | ((u32)ld2(blk + 192 + 8 * n + 2 * qb) << 16);
+        } else if constexpr (Q4) {
+            // sub-block 4 * n + qb: nibble qb % 2 of the 32 bytes of group 2 * n + qb / 2
+            const uint8_t* blk = wrow + (size_t)(step >> 1) * 144;
+            const int g = 2 * (step & 1) + (qb >> 1);
+            r.h0 = ld16_a2(blk);
+            r.q0 = ld16_a2(blk + 16 + 32 * g);
+            r.q1 = ld16_a2(blk + 32 + 32 * g);
+            r.d = (u32)(4 * (step & 1) + qb);
+            r.ds[0] = (p.dsum + (dsrc - p.da))[(size_t)(4 * step) * p.tok_pad];
+            r.ds[1] = (p.dsum + (dsrc - p.da))[(size_t)(4 * step + 2) * p.tok_pad];
         } else {
             const uint8_t* blk = wrow + (size_t)(4 * step + qb) * 34;
             r.d = ld2(blk);
@@ -126,7 +149,7 @@ __device__ __forceinline__ void gemm_w32_body(const GemmArgs& p0, uint8_t* smem)
         r.da[0] = dsrc[(size_t)(4 * step) * p.tok_pad];
         r.da[1] = dsrc[(size_t)(4 * step + 2) * p.tok_pad];
     };
-    u32 m8 = Q6 ? 0x000F000Fu : 0x00FF00FFu, m2 = 0x00300030u, magic = 0x64006400u;
+    u32 m8 = Q6 || Q4 ? 0x000F000Fu : 0x00FF00FFu, m2 = 0x00300030u, magic = 0x64006400u;
     asm volatile("" : "+v"(m8), "+v"(m2), "+v"(magic));   // keep them in vector registers
     _Float16* dst = sW + srow * JL_GEMM_STRIDE + 32 * qb;
     auto dequant = [&](const Gemm32Raw& r) {
@@ -162,6 +185,27 @@ __device__ __forceinline__ void gemm_w32_body(const GemmArgs& p0, uint8_t* smem)
                 }
             }
             sD[srow * 4 + qb] = half_bits_to_f32((uint16_t)(r.d & 0xFFFF));
+        } else if constexpr (Q4) {
+            const f16x2 off = {(_Float16)-1024.0f, (_Float16)-1024.0f};
+            const int nsh = 4 * (qb & 1);
+            // nibbles of bytes (b0, b2) and (b1, b3) of a word as 1024 + q, then q: exact
+            auto pair = [&](u32 w) {
+                const u32 v = (w & m8) | magic;
+                return word(__builtin_bit_cast(f16x2, v) + off);
+            };
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const u32 wa = (i < 2 ? r.q0[2 * i] : r.q1[2 * i - 4]) >> nsh;
+                const u32 wb = (i < 2 ? r.q0[2 * i + 1] : r.q1[2 * i - 3]) >> nsh;
+                const u32x4 o = {pair(wa), pair(wa >> 8), pair(wb), pair(wb >> 8)};
+                *(u32x4*)(dst + 8 * i) = o;
+            }
+            u32 sc, mn;
+            scale_min_k4((int)r.d, r.h0.y, r.h0.z, r.h0.w, sc, mn);
+            sD[srow * 4 + qb] = half_bits_to_f32((uint16_t)(r.h0.x & 0xFFFF)) * (float)sc;
+            sD2[srow * 4 + qb] = half_bits_to_f32((uint16_t)(r.h0.x >> 16)) * (float)mn;
+            sDs[tid] = r.ds[0];
+            sDs[256 + tid] = r.ds[1];
         } else {
             const f16x2 off = {(_Float16)-1152.0f, (_Float16)-1152.0f};
             // bytes (b0, b2) and (b1, b3) of a word as 1024 + (q + 128), then q: exact
@@ -235,6 +279,17 @@ __device__ __forceinline__ void gemm_w32_body(const GemmArgs& p0, uint8_t* smem)
                     const float dd = sD[(32 * j + arow) * 4 + b];
 #pragma unroll
                     for (int e = 0; e < 16; e++) out[j][e] = fmaf(dav[e >> 2][e & 3], dd * acc[j][e], out[j][e]);
+                }
+                if constexpr (Q4) {
+                    f32x4 dsv[4];
+#pragma unroll
+                    for (int i = 0; i < 4; i++) dsv[i] = *(const f32x4*)(sDs + b * JL_GEMM_TILE + 32 * tg + 8 * i + 4 * kg);
+#pragma unroll
+                    for (int j = 0; j < 2; j++) {
+                        const float nm = -sD2[(32 * j + arow) * 4 + b];
+#pragma unroll
+                        for (int e = 0; e < 16; e++) out[j][e] = fmaf(dsv[e >> 2][e & 3], nm, out[j][e]);
+                    }
                 }
             }
         }

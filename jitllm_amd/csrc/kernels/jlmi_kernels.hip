@@ -145,7 +145,7 @@ extern "C" __global__ __launch_bounds__(256, 2) void jl_gemm_q6k_r64(GemmArgs p)
     gemm_q6k_split_slice(p);
     gemm_q6k_body(p, jl_smem, blockIdx.x * JL_GEMM_TILE, blockIdx.y * 64);
 }
-// Q8_0 and Q6_K with the activation window of 32: prep grid = (ceil(k/256), tok_pad/32), block = 256;
+// Q8_0, Q6_K and Q4_K with the activation window of 32: prep grid = (ceil(k/256), tok_pad/32), block = 256;
 // matrix kernel grid = (tok_pad/128, ceil(nrows/64), K splits), block = 256, dynamic LDS =
 // JL_GEMM32_LDS_BYTES(planes)
 extern "C" __global__ __launch_bounds__(256) void jl_gemm_prep_w32(GemmPrepArgs p) {
@@ -154,6 +154,7 @@ extern "C" __global__ __launch_bounds__(256) void jl_gemm_prep_w32(GemmPrepArgs 
 }
 extern "C" __global__ __launch_bounds__(256, 3) void jl_gemm_q8_0_w32(GemmArgs p) { gemm_w32_body<JL_Q8_0>(p, jl_smem); }
 extern "C" __global__ __launch_bounds__(256, 3) void jl_gemm_q6k_w32(GemmArgs p) { gemm_w32_body<JL_Q6_K>(p, jl_smem); }
+extern "C" __global__ __launch_bounds__(256, 3) void jl_gemm_q4k_w32(GemmArgs p) { gemm_w32_body<JL_Q4_K>(p, jl_smem); }
 extern "C" __global__ __launch_bounds__(512) void jl_gemm_q4k_r128(GemmArgs p) {
     gemm_q4k_body<2>(p, jl_smem, blockIdx.x * JL_GEMM_TILE, blockIdx.y * 128);
 }

@@ -139,7 +139,7 @@ def test_gemm_token_equals_decode_matvec(dev, devbuf):
     dev.SetActWindow(32)
 
 
-@pytest.mark.parametrize("t,window,ntok", [(quant.Q8_0, 32, 2), (quant.Q8_0, 32, 1), (quant.Q6_K, 32, 2), (quant.Q4_K, 32, 9),
+@pytest.mark.parametrize("t,window,ntok", [(quant.Q8_0, 32, 2), (quant.Q8_0, 32, 1), (quant.Q6_K, 32, 2), (quant.Q4_K, 32, 2),
                                            (quant.Q4_K, 256, 3)])
 def test_matmul_fallback_is_the_per_token_loop(dev, devbuf, t, window, ntok):
     """Types, windows and token counts the GEMM does not take still return the right values."""
@@ -296,11 +296,12 @@ def test_gemm_q6k_k_split_and_token_loop_agree(dev, devbuf, split):
 @pytest.mark.parametrize("shape", [(16, 128, 128), (130, 200, 512), (8, 37, 1024), (512, 300, 1024),
                                    (129, 129, 4096), (3, 64, 2816), (40, 70, 384)], ids=lambda s: "x".join(map(str, s)))
 @pytest.mark.parametrize("weights", ["normal", "planted"])
-@pytest.mark.parametrize("t", [quant.Q8_0, quant.Q6_K], ids=["q8_0", "q6_k"])
+@pytest.mark.parametrize("t", [quant.Q8_0, quant.Q6_K, quant.Q4_K], ids=["q8_0", "q6_k", "q4_k"])
 def test_gemm_window32_vs_oracle(dev, devbuf, shape, weights, t):
-    """Q8_0 and Q6_K with the activation window of 32 on the matrix cores: the int8 products
-    are exact f16 integers (Q6_K: the sub-block scale split over two operands) and the scales
-    enter once per block of 32, so the sums are the oracle's.  Token counts that leave
+    """Q8_0, Q6_K and Q4_K with the activation window of 32 on the matrix cores: the int8
+    products are exact f16 integers (Q6_K: the sub-block scale split over two operands; Q4_K:
+    the minimums against the prep's block sums) and the scales enter once per block of 32, so
+    the sums are the oracle's.  Token counts that leave
     wavefronts of a tile without a token, rows that end inside a tile, K of one stage, K that
     is no multiple of 256 and grids widened along K are among the shapes."""
     ntok, nrows, k = shape
@@ -332,7 +333,7 @@ def test_gemm_window32_vs_oracle(dev, devbuf, shape, weights, t):
 
 
 @pytest.mark.parametrize("split", [1, 2, 3, 8])
-@pytest.mark.parametrize("t", [quant.Q8_0, quant.Q6_K], ids=["q8_0", "q6_k"])
+@pytest.mark.parametrize("t", [quant.Q8_0, quant.Q6_K, quant.Q4_K], ids=["q8_0", "q6_k", "q4_k"])
 def test_gemm_window32_k_split_and_token_loop_agree(dev, devbuf, split, t):
     """Every K split meets the bar, and the matrix kernel's token t is the decode matvec of
     token t (the per-token loop, tuning gemm.form = 9) to the same bar."""

@@ -98,16 +98,16 @@ def test_mxfp4_any_token_count(dev, devbuf, seed):
 
 @pytest.mark.parametrize("seed", range(4))
 def test_q6k_q8_0_matmul_any_token_count(dev, devbuf, seed):
-    """Q6_K with either activation window and Q8_0 with the window of 32, library's own
+    """Q6_K with either activation window, Q8_0 and Q4_K with the window of 32, library's own
     choice of form (per-token loop, grouped dot-product kernel, 128-token tiles with and
     without a K split): token counts on both sides of every threshold, ragged rows, K of one
     stage up, K that is no multiple of 256 for Q8_0."""
     rng = np.random.default_rng(300 + seed)
     for ntok in rng.permutation([1, 2, 3, 8, 9, 17, 33, 64, 100, 128, 129, 260])[:6]:
         ntok = int(ntok)
-        t, window = [(quant.Q6_K, 256), (quant.Q6_K, 32), (quant.Q8_0, 32)][int(rng.integers(0, 3))]
+        t, window = [(quant.Q6_K, 256), (quant.Q6_K, 32), (quant.Q8_0, 32), (quant.Q4_K, 32)][int(rng.integers(0, 4))]
         nrows = int(rng.integers(1, 400))
-        k = 256 * int(rng.integers(1, 9)) if t == quant.Q6_K else 128 * int(rng.integers(1, 17))
+        k = 256 * int(rng.integers(1, 9)) if t != quant.Q8_0 else 128 * int(rng.integers(1, 17))
         dev.SetActWindow(window)
         w = synth.random_weights(t, nrows, k, seed=seed * 89 + ntok) if rng.random() < 0.5 \
             else synth.quantized_weights(t, nrows, k, seed=seed * 89 + ntok)
