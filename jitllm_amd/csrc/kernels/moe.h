@@ -389,13 +389,13 @@ __device__ __forceinline__ void moe_matvec_body(const MoeMatVecArgs& p, uint8_t*
     const int nsl = (nslots + LPR - 1) / LPR;
     const int ngroups = (row_hi - row_lo - wave * U * RW + nwaves * U * RW - 1) / (nwaves * U * RW);  // may be <= 0
     const int nsteps = max(ngroups, 0) * nsl;
-    auto step_row = [&](int it, int u) { return row_lo + (wave + (it / nsl) * nwaves) * U * RW + u * RW + rw; };
-    auto step_slot = [&](int it) { return slot + (it % nsl) * LPR; };
-    auto load_step = [&](int it, typename T::W (&w)[U]) {
-        const int s = min(step_slot(it), nslots - 1);
+    // step it = (row group it / nsl, slot group it % nsl); the pair is carried along the loop
+    const int row_first = row_lo + wave * U * RW + rw, row_stride = nwaves * U * RW;
+    auto load_step = [&](int row0, int sg, typename T::W (&w)[U]) {
+        const int s = min(slot + sg * LPR, nslots - 1);
 #pragma unroll
         for (int u = 0; u < U; u++)
-            T::load_w(sheet + (size_t)min(step_row(it, u), row_hi - 1) * p.row_bytes, s, w[u]);
+            T::load_w(sheet + (size_t)min(row0 + u * RW, row_hi - 1) * p.row_bytes, s, w[u]);
     };
 
     typename T::W w_next[U];
@@ -421,7 +421,7 @@ __device__ __forceinline__ void moe_matvec_body(const MoeMatVecArgs& p, uint8_t*
         }
         // the first step's weights are requested behind the staging loads (loads are served
         // in order) and stay in flight across the barrier, which orders LDS only
-        if (nsteps > 0) load_step(0, w_next);
+        if (nsteps > 0) load_step(row_first, 0, w_next);
         lds_barrier();
         JL_MOE_TRACE(2);
         float acc[JL_MOE_TB][U];
@@ -429,13 +429,16 @@ __device__ __forceinline__ void moe_matvec_body(const MoeMatVecArgs& p, uint8_t*
         for (int j = 0; j < JL_MOE_TB; j++)
 #pragma unroll
             for (int u = 0; u < U; u++) acc[j][u] = 0.f;
+        int row0 = row_first, sg = 0;   // this step's first row of the lane and its slot group
         for (int it = 0; it < nsteps; it++) {
             typename T::Prep P[U];
-            const int s = step_slot(it), sc = min(s, nslots - 1);
+            const int s = slot + sg * LPR, sc = min(s, nslots - 1);
             const bool live = s < nslots;
+            const bool last_sg = sg == nsl - 1;
+            const int row_n = last_sg ? row0 + row_stride : row0, sg_n = last_sg ? 0 : sg + 1;
 #pragma unroll
             for (int u = 0; u < U; u++) T::prep(w_next[u], sc, P[u]);
-            if (it + 1 < nsteps) load_step(it + 1, w_next);
+            if (it + 1 < nsteps) load_step(row_n, sg_n, w_next);
 #pragma unroll
             for (int j = 0; j < JL_MOE_TB; j++) {
                 if (j < ncol) {
@@ -451,19 +454,21 @@ __device__ __forceinline__ void moe_matvec_body(const MoeMatVecArgs& p, uint8_t*
                 asm volatile("" ::: "memory");
                 __builtin_amdgcn_sched_barrier(0);
             }
-            if (it % nsl == nsl - 1) {  // the rows' last slot group: reduce and store
+            if (last_sg) {  // the rows' last slot group: reduce and store
 #pragma unroll
                 for (int j = 0; j < JL_MOE_TB; j++)
 #pragma unroll
                     for (int u = 0; u < U; u++) {
                         if (j < ncol) {
-                            const int r = step_row(it, u);
+                            const int r = row0 + u * RW;
                             float t = group_sum<LPR>(acc[j][u]);
                             if (slot == LPR - 1 && r < row_hi) out[(size_t)(c0 + j) * p.nrows + r] = t;
                         }
                         acc[j][u] = 0.f;
                     }
             }
+            row0 = row_n;
+            sg = sg_n;
         }
         JL_MOE_TRACE(3);
         __syncthreads();
