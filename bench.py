@@ -9,9 +9,17 @@ Weights rotate through enough distinct device copies to exceed twice the
 256 MB Infinity Cache, so no launch is served from cache (same file,
 :184-189, :246-253).  Inputs are resident in HBM before the timed region.
 
+Timing protocol (the reference's: warm calls, then the median of nine timed
+runs, perbyte_test.go:131-144): at least 200 untimed launches, then NINE timed
+windows of exactly --steps launches each, each window bracketed by HIP events
+on the launch stream; the reported step time is the median window's.  Every
+window is enqueued behind a fill of a scratch buffer, so its launches are
+already queued when the first one starts and a short window measures the
+device, not the host's launch rate.  Every section checks the output it timed
+against dequantize (on the device) + an f64 product on rows spread over the grid.
+
 Prints ONE JSON line.  `value` is algorithmic bytes per second (weight bytes +
-x + out per launch) over the timed region, timed with HIP events on the stream
-the kernels run on; `roofline` prices the same figure against the 8 TB/s HBM
+x + out per launch), `roofline` prices the same figure against the 8 TB/s HBM
 peak; `cpu_baseline` is the intrinsic restatement of the reference's host
 kernels timed on this box's cores (a reported baseline, not a target).
 """
@@ -38,6 +46,53 @@ MEASURED_TRAFFIC = {"c1": 9643571}
 def matvec_bytes(t, nrows, k):
     from jitllm_amd import quant
     return nrows * quant.row_bytes(t, k) + 4 * k + 4 * nrows
+
+
+def spread_rows(nrows, n):
+    """About n row indices: the first and last eight and the rest evenly over the matrix."""
+    picks = set(range(min(8, nrows))) | set(range(max(0, nrows - 8), nrows))
+    picks |= set(int(v) for v in np.linspace(0, nrows - 1, n))
+    return np.array(sorted(picks))
+
+
+def dequant_rows(dev, t, w_host, rows, k):
+    """Rows of a GGUF weight dequantized ON THE DEVICE (jl_dequant_dev) -> f64 [len(rows)][k]."""
+    from jitllm_amd import quant
+    from jitllm_amd.hipmem import DeviceArray
+    rb = quant.row_bytes(t, k)
+    rows = np.asarray(rows)
+    if len(rows) > 1 and np.all(np.diff(rows) == 1):      # a contiguous range (an expert's sheet)
+        src = DeviceArray(w_host[int(rows[0]) * rb:(int(rows[-1]) + 1) * rb])
+    else:
+        src = DeviceArray(np.concatenate([w_host[r * rb:(r + 1) * rb] for r in rows]))
+    dst = DeviceArray(shape=(len(rows) * k,), dtype=np.float32, fill=0)
+    if not dev.dequant_dev(t, src.ptr, dst.ptr, len(rows) * k):
+        raise RuntimeError("the device declined to dequantize")
+    dev.synchronize()
+    out = dst.get().reshape(len(rows), k).astype(np.float64)
+    src.free()
+    dst.free()
+    return out
+
+
+def rel_err(got, want, what, bar=2e-2):
+    got = np.asarray(got, np.float64)
+    if not np.all(np.isfinite(got)):
+        raise RuntimeError(f"{what}: non-finite output")
+    err = float(np.sqrt(np.mean((got - want) ** 2)) / max(np.sqrt(np.mean(want ** 2)), 1e-30))
+    if not err <= bar:
+        raise RuntimeError(f"{what}: output differs from dequantize + f64 product by {err:.3e}")
+    return err
+
+
+def measure(dev, run, steps, gate, warm=3, windows=9, gate_bytes=256 << 20):
+    """warm untimed calls of run(i), then the median over nine windows of `steps` calls."""
+    from jitllm_amd.hipmem import timed_windows
+    for i in range(warm):
+        run(i)
+    dev.synchronize()
+    ms, _ = timed_windows(run, steps, dev.stream, windows, gate, gate_bytes)
+    return ms
 
 
 class Workload:
@@ -92,63 +147,47 @@ class Workload:
         if not ok:
             raise RuntimeError(f"{self.name}: the device declined")
 
-    def timed(self, steps, warmup):
-        """(ms per step by HIP events on the launch stream, ms per step by host clock)."""
-        from jitllm_amd.hipmem import Event, synchronize
+    def timed(self, steps, warmup, gate=None):
+        """(ms per step of the median of nine windows of `steps` launches, by HIP events on the
+        launch stream; every window's ms per step; host microseconds to enqueue one launch)."""
+        from jitllm_amd.hipmem import synchronize, timed_windows
         self.dev.SetActWindow(self.window)
-        for i in range(warmup):
+        for i in range(max(warmup, 200)):
             self.step(i)
         self.dev.synchronize()
         synchronize()
-        e0, e1 = Event(), Event()
         t0 = time.perf_counter()
-        e0.record(self.dev.stream)
-        for i in range(steps):
-            self.step(warmup + i)
-        e1.record(self.dev.stream)
-        e1.synchronize()
+        for i in range(64):
+            self.step(i)
+        host_us = (time.perf_counter() - t0) * 1e6 / 64
+        self.dev.synchronize()
+        # the gate covers the host's enqueue time of a window, up to ~1 GiB of fill
+        gate_bytes = min(1 << 30, max(64 << 20, int(steps * host_us * 1.5 * 3e6)))
+        ms, per = timed_windows(self.step, steps, self.dev.stream, 9, gate, gate_bytes)
         synchronize()
-        t1 = time.perf_counter()
-        return e0.elapsed_ms(e1) / steps, (t1 - t0) * 1e3 / steps
+        return ms, per, host_us
 
-    def timed_hot(self, steps):
+    def timed_hot(self, steps, gate=None):
         """ms per step over copy 0 alone (weights cache resident)."""
-        from jitllm_amd.hipmem import Event
+        from jitllm_amd.hipmem import timed_windows
         self.dev.SetActWindow(self.window)
-        for _ in range(20):
+        for _ in range(50):
             self.step(0)
         self.dev.synchronize()
-        e0, e1 = Event(), Event()
-        e0.record(self.dev.stream)
-        for _ in range(steps):
-            self.step(0)
-        e1.record(self.dev.stream)
-        e1.synchronize()
-        return e0.elapsed_ms(e1) / steps
+        ms, _ = timed_windows(lambda i: self.step(0), steps, self.dev.stream, 9, gate, 64 << 20)
+        return ms
 
     def check(self):
-        """The last step's output: finite everywhere, and the first rows within 2 % (of the
-        rows' RMS) of dequantize (on the device) + f64 dot with the f32 activation; the int8
-        activation accounts for a few parts in a thousand.  A sanity gate on what was
-        timed, not the parity test."""
-        from jitllm_amd import quant
-        from jitllm_amd.hipmem import DeviceArray
+        """The last step's output: every row finite, and 96 rows spread over the whole grid
+        (first, last, and evenly between) within 2 % (of the rows' RMS) of dequantize (on the
+        device) + f64 dot with the f32 activation; the int8 activation accounts for a few parts
+        in a thousand.  A sanity gate on what was timed, not the parity test."""
         got = self.out.get()
         if not np.all(np.isfinite(got)):
             raise RuntimeError(f"{self.name}: non-finite output")
-        nr = min(16, self.nrows)
-        src = DeviceArray(self.w_host[:nr * quant.row_bytes(self.t, self.k)])
-        dst = DeviceArray(shape=(nr * self.k,), dtype=np.float32, fill=0)
-        if not self.dev.dequant_dev(self.t, src.ptr, dst.ptr, nr * self.k):
-            raise RuntimeError(f"{self.name}: the device declined to dequantize")
-        self.dev.synchronize()
-        want = dst.get().reshape(nr, self.k).astype(np.float64) @ self.x_host.astype(np.float64)
-        src.free()
-        dst.free()
-        err = float(np.sqrt(np.mean((got[:nr] - want) ** 2)) / max(np.sqrt(np.mean(want ** 2)), 1e-30))
-        if err > 2e-2:
-            raise RuntimeError(f"{self.name}: output differs from dequantize + dot by {err:.3e}")
-        return err
+        rows = spread_rows(self.nrows, 96)
+        want = dequant_rows(self.dev, self.t, self.w_host, rows, self.k) @ self.x_host.astype(np.float64)
+        return rel_err(got[rows], want, self.name)
 
     def free(self):
         self.pool.free()
@@ -186,52 +225,91 @@ def cpu_baseline(t, nrows, k, window, seed=0):
 MFMA_F16_PEAK_TFLOPS = 2500.0
 
 
-def gemm_section(dev, shapes=None, t=None, k=4096, window=256):
-    """Q4_K prefill GEMM (x [ntok][4096] f32 -> out [ntok][nrows]), activation quantizer and
-    layout kernel included in every step; flops = 2*nrows*k*ntok, priced against the dense
-    f16 MFMA peak (the kernel runs exact integer operands on the f16 matrix cores).
+def gemm_section(dev, gate, shapes=None, t=None, k=4096, window=256, packed=False):
+    """Prefill GEMM (x [ntok][k] f32 -> out [ntok][nrows]), activation quantizer and layout
+    kernel included in every step; flops = 2*nrows*k*ntok, priced against the dense f16 MFMA
+    peak (the kernel runs exact integer operands on the f16 matrix cores).
     shapes: {nrows: [ntok, ...]}; default = the baseline's prefill configurations.
-    t = Q6_K: the same model's Q6_K tensors (a weight is two matrix operands there)."""
+    t = Q6_K / Q8_0: the same model's other tensors.  packed: the weights as packed planes
+    (jl_matmul_packed_dev).  Output check: 96 rows spread over the matrix x every token."""
     from jitllm_amd import quant, synth
-    from jitllm_amd.hipmem import DeviceArray, Event
+    from jitllm_amd.device import Packed
+    from jitllm_amd.hipmem import DeviceArray
     t = quant.Q4_K if t is None else t
     dev.SetActWindow(window)
     out = {}
     shapes = shapes or {4096: (16, 128, 512, 2048), 14336: (16, 128, 512, 2048)}
     for nrows, toks in shapes.items():
-        w = DeviceArray(synth.quantized_weights(t, nrows, k, seed=0))
-        for ntok in toks:
-            x = DeviceArray(np.random.default_rng(2).standard_normal((ntok, k), np.float32))
-            o = DeviceArray(shape=(ntok, nrows), dtype=np.float32)
-            dev.Reserve(ntok, k)
-            for _ in range(3):
-                if not dev.matmul_dev(o.ptr, t, w.ptr, x.ptr, nrows, k, ntok):
-                    raise RuntimeError("the device declined the prefill GEMM")
+        w_host = synth.quantized_weights(t, nrows, k, seed=0)
+        w = DeviceArray(w_host)
+        rows = spread_rows(nrows, 96)
+        wrows = dequant_rows(dev, t, w_host, rows, k)
+        pl = None
+        if packed:
+            bufs = [DeviceArray(shape=(max(n, 1),), dtype=np.uint32, fill=0) for n in dev.packed_words(t, nrows, k)]
+            if not dev.pack_weights_dev(t, w.ptr, nrows, k, bufs[0].ptr, bufs[1].ptr, bufs[2].ptr):
+                raise RuntimeError("the device declined to pack")
             dev.synchronize()
-            e0, e1, n = Event(), Event(), 20
-            e0.record(dev.stream)
-            for _ in range(n):
-                dev.matmul_dev(o.ptr, t, w.ptr, x.ptr, nrows, k, ntok)
-            e1.record(dev.stream)
-            e1.synchronize()
-            ms = e0.elapsed_ms(e1) / n
+            pl = Packed(bufs[0].ptr, bufs[1].ptr, bufs[2].ptr, 0, nrows)
+        for ntok in toks:
+            x_host = np.random.default_rng(2).standard_normal((ntok, k), np.float32)
+            x = DeviceArray(x_host)
+            o = DeviceArray(shape=(ntok, nrows), dtype=np.float32, fill=np.float32(np.nan))
+            if not dev.reserve_shape(t, nrows, k, ntok, packed):
+                raise RuntimeError("the device declined the prefill GEMM's shape")
+
+            def run(_):
+                ok = (dev.matmul_packed_dev(o.ptr, t, pl, x.ptr, nrows, k, ntok) if packed
+                      else dev.matmul_dev(o.ptr, t, w.ptr, x.ptr, nrows, k, ntok))
+                if not ok:
+                    raise RuntimeError("the device declined the prefill GEMM")
+            ms = measure(dev, run, 20, gate)
+            got = o.get()
+            if not np.all(np.isfinite(got)):
+                raise RuntimeError(f"prefill GEMM {ntok}x{k}->{nrows}: non-finite or unwritten output")
+            err = rel_err(got[:, rows], x_host.astype(np.float64) @ wrows.T, f"prefill GEMM {ntok}x{k}->{nrows}")
             tf = 2.0 * nrows * k * ntok / (ms * 1e-3) / 1e12
             out[f"{ntok}x{k}->{nrows}"] = {"us_per_step": round(ms * 1e3, 1), "TFLOP/s": round(tf, 1),
-                                          "frac_of_f16_mfma_peak": round(tf / MFMA_F16_PEAK_TFLOPS, 4)}
+                                          "frac_of_f16_mfma_peak": round(tf / MFMA_F16_PEAK_TFLOPS, 4),
+                                          "checked_rel_err": float(f"{err:.2e}")}
             x.free()
             o.free()
         w.free()
+        if packed:
+            for b in bufs:
+                b.free()
     return out
 
 
-def ffn_section(dev):
+def _silu(v):
+    return v / (1.0 + np.exp(-v))
+
+
+def _ffn_check(dev, quant, wg, wd, x_host, gate, up, y, resid, n_embd, n_ffn, what):
+    """gate / up rows against dequantize + f64 dot of the normed x (norm weight 1), and y rows
+    against dequantize + f64 dot of silu(gate) * up taken from the device's own gate and up."""
+    g, u, yy, r = gate.get(), up.get(), y.get(), resid.get()
+    xn = x_host.astype(np.float64)
+    xn = xn / np.sqrt(np.mean(xn * xn) + 1e-5)
+    rows = spread_rows(n_ffn, 64)
+    want = dequant_rows(dev, quant.Q8_0, wg, rows, n_embd) @ xn
+    e1 = rel_err(g[rows], want, what + " gate")
+    rel_err(u[rows], want, what + " up")
+    rows = spread_rows(n_embd, 64)
+    h = _silu(g.astype(np.float64)) * u.astype(np.float64)
+    e2 = rel_err(yy[rows], dequant_rows(dev, quant.Q6_K, wd, rows, n_ffn) @ h, what + " down")
+    rel_err(r[rows], yy[rows].astype(np.float64), what + " residual add", 1e-5)
+    return max(e1, e2)
+
+
+def ffn_section(dev, gate_):
     """A gated feed-forward block at decode, the baseline's second configuration: RMSNorm folded
     into the quantizer of gate and up (Q8_0 14336x4096), one grouped launch; then down (Q6_K
     4096x14336) over silu(gate) * up formed inside its quantizer with the residual add riding
     on the launch: two launches per block.  Four rotating sets of the three matrices
     (692 MiB) keep every step out of cache."""
     from jitllm_amd import quant, synth
-    from jitllm_amd.hipmem import DeviceArray, Event, check, hip
+    from jitllm_amd.hipmem import DeviceArray
     n_embd, n_ffn = 4096, 14336
     dev.SetActWindow(32)
     wg = synth.quantized_weights(quant.Q8_0, n_ffn, n_embd, seed=0)
@@ -240,7 +318,8 @@ def ffn_section(dev):
     for i in range(4):
         g, u, d = DeviceArray(wg), DeviceArray(wg), DeviceArray(wd)
         sets.append((g, u, d))
-    x = DeviceArray(synth.activations(n_embd, seed=2))
+    x_host = synth.activations(n_embd, seed=2)
+    x = DeviceArray(x_host)
     norm_w = DeviceArray(np.ones(n_embd, np.float32))
     gate = DeviceArray(shape=(n_ffn,), dtype=np.float32, fill=0)
     up = DeviceArray(shape=(n_ffn,), dtype=np.float32, fill=0)
@@ -255,16 +334,11 @@ def ffn_section(dev):
                                          resid=resid.ptr, alpha=1.0)
         if not ok:
             raise RuntimeError("the device declined the feed-forward block")
-    for i in range(8):
-        run(i)
+    ms = measure(dev, run, 20, gate_, warm=8)
+    resid.zero()
+    run(0)
     dev.synchronize()
-    e0, e1, n = Event(), Event(), 100
-    e0.record(dev.stream)
-    for i in range(n):
-        run(i)
-    e1.record(dev.stream)
-    e1.synchronize()
-    ms = e0.elapsed_ms(e1) / n
+    err = _ffn_check(dev, quant, wg, wd, x_host, gate, up, y, resid, n_embd, n_ffn, "feed-forward block")
     nbytes = 2 * wg.nbytes + wd.nbytes + 4 * (n_embd + 2 * n_ffn) + 4 * (2 * n_ffn + 2 * n_embd)
     for g, u, d in sets:
         g.free(); u.free(); d.free()
@@ -272,31 +346,35 @@ def ffn_section(dev):
         b.free()
     return {"us_per_step": round(ms * 1e3, 2), "launches_per_step": 2, "bytes_per_step": nbytes,
             "GB/s": round(nbytes / (ms * 1e-3) / 1e9, 1),
-            "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+            "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+            "checked_rel_err": float(f"{err:.2e}")}
 
 
-def ffn_packed_section(dev):
+def ffn_packed_section(dev, gate_):
     """The same gated feed-forward block over packed planes, the layout a .jlm file holds:
     gate and up (Q8_0 14336x4096) one launch of two packed matvecs sharing x, down (Q6_K
     4096x14336) one launch over silu(gate) * up with the residual add riding on it; the
     RMSNorm in front of gate and up is folded into their quantizer.  Four rotating sets of
     planes keep every step out of cache."""
     from jitllm_amd import quant, synth
-    from jitllm_amd.hipmem import DeviceArray, Event
+    from jitllm_amd.hipmem import DeviceArray
     n_embd, n_ffn = 4096, 14336
     dev.SetActWindow(32)
+    wg = synth.quantized_weights(quant.Q8_0, n_ffn, n_embd, seed=0)
+    wd = synth.quantized_weights(quant.Q6_K, n_embd, n_ffn, seed=1)
 
-    def planes_of(t, nrows, k, seed):
-        src = DeviceArray(synth.quantized_weights(t, nrows, k, seed=seed))
+    def planes_of(t, w_host, nrows, k):
+        src = DeviceArray(w_host)
         pl = [DeviceArray(shape=(max(n, 1),), dtype=np.uint32, fill=0) for n in dev.packed_words(t, nrows, k)]
         if not dev.pack_weights_dev(t, src.ptr, nrows, k, pl[0].ptr, pl[1].ptr, pl[2].ptr):
             raise RuntimeError("the device declined to pack a matrix")
         dev.synchronize()
         src.free()
         return pl
-    sets = [(planes_of(quant.Q8_0, n_ffn, n_embd, 0), planes_of(quant.Q8_0, n_ffn, n_embd, 0),
-             planes_of(quant.Q6_K, n_embd, n_ffn, 1)) for _ in range(4)]
-    x = DeviceArray(synth.activations(n_embd, seed=2))
+    sets = [(planes_of(quant.Q8_0, wg, n_ffn, n_embd), planes_of(quant.Q8_0, wg, n_ffn, n_embd),
+             planes_of(quant.Q6_K, wd, n_embd, n_ffn)) for _ in range(4)]
+    x_host = synth.activations(n_embd, seed=2)
+    x = DeviceArray(x_host)
     gate = DeviceArray(shape=(n_ffn,), dtype=np.float32, fill=0)
     up = DeviceArray(shape=(n_ffn,), dtype=np.float32, fill=0)
     y = DeviceArray(shape=(n_embd,), dtype=np.float32, fill=0)
@@ -312,16 +390,11 @@ def ffn_packed_section(dev):
         a, b = calls[i % len(calls)]
         if not (dev.packed_multi_call(a) and dev.packed_multi_call(b)):
             raise RuntimeError("the device declined the packed feed-forward block")
-    for i in range(8):
-        run(i)
+    ms = measure(dev, run, 20, gate_, warm=8)
+    resid.zero()
+    run(0)
     dev.synchronize()
-    e0, e1, n = Event(), Event(), 100
-    e0.record(dev.stream)
-    for i in range(n):
-        run(i)
-    e1.record(dev.stream)
-    e1.synchronize()
-    ms = e0.elapsed_ms(e1) / n
+    err = _ffn_check(dev, quant, wg, wd, x_host, gate, up, y, resid, n_embd, n_ffn, "packed feed-forward block")
     nbytes = 2 * n_ffn * quant.row_bytes(quant.Q8_0, n_embd) + n_embd * quant.row_bytes(quant.Q6_K, n_ffn) \
         + 4 * (n_embd + 2 * n_ffn) + 4 * (2 * n_ffn + 2 * n_embd)
     for st in sets:
@@ -332,20 +405,24 @@ def ffn_packed_section(dev):
         b.free()
     return {"us_per_step": round(ms * 1e3, 2), "launches_per_step": 2, "bytes_per_step": nbytes,
             "GB/s": round(nbytes / (ms * 1e-3) / 1e9, 1),
-            "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+            "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+            "checked_rel_err": float(f"{err:.2e}")}
 
 
-def moe_section(dev, rows=64):
+def moe_section(dev, gate_, rows=64):
     """Qwen3-30B-A3B routed feed-forward block: 128 experts (gate/up 768x2048, down 2048x768,
     Q4_K), 64 rows routed top-8; one step = router logits (f32 router matrix, rows ~ N(0, 1/k)
     so the logits are ~ N(0,1)) + softmax/top-8 + group + gate/up + down + combine, all on the
-    device.  Bytes = the touched experts' three sheets + router matrix + x in + resid out."""
+    device.  Bytes = the touched experts' three sheets + router matrix + x in + resid out.
+    Output check: three rows of the block recomputed in f64 from sheets dequantized on the
+    device, with the device's own selection and weights."""
     from jitllm_amd import quant, synth
-    from jitllm_amd.hipmem import DeviceArray, Event
+    from jitllm_amd.hipmem import DeviceArray
     t, n_expert, k_used, n_ffn, n_embd = quant.Q4_K, 128, 8, 768, 2048
     dev.SetActWindow(256)
     rng = np.random.default_rng(0)
-    x = DeviceArray(rng.standard_normal((rows, n_embd)).astype(np.float32))
+    x_host = rng.standard_normal((rows, n_embd)).astype(np.float32)
+    x = DeviceArray(x_host)
     router = DeviceArray((rng.standard_normal((n_expert, n_embd)) / np.sqrt(n_embd)).astype(np.float32))
     ld = DeviceArray(shape=(rows, n_expert), dtype=np.float32, fill=0)
     sd = DeviceArray(shape=(rows, k_used + 1), dtype=np.uint32, fill=0)
@@ -357,49 +434,61 @@ def moe_section(dev, rows=64):
     touched = len(np.unique(sd.get()[:, :k_used]))
     gs = n_ffn * quant.row_bytes(t, n_embd)
     ds = n_embd * quant.row_bytes(t, n_ffn)
-    banks = []
+    banks, hosts = [], []
     for i, (r, k) in enumerate([(n_ffn, n_embd), (n_ffn, n_embd), (n_embd, n_ffn)]):
-        banks.append(DeviceArray(synth.quantized_weights(t, r * n_expert, k, seed=10 + i)))
+        hosts.append(synth.quantized_weights(t, r * n_expert, k, seed=10 + i))
+        banks.append(DeviceArray(hosts[-1]))
     resid = DeviceArray(shape=(rows, n_embd), dtype=np.float32, fill=0)
 
-    def run():
-        return (dev.moe_logits_dev(ld.ptr, 0, router.ptr, x.ptr, n_expert, n_embd, rows) and
+    def run(_):
+        if not (dev.moe_logits_dev(ld.ptr, 0, router.ptr, x.ptr, n_expert, n_embd, rows) and
                 dev.moe_route_dev(ld.ptr, rows, n_expert, k_used, sd.ptr, k_used + 1, wd.ptr) and
                 dev.moe_ffn_dev(resid.ptr, t, banks[0].ptr, banks[1].ptr, banks[2].ptr, x.ptr, sd.ptr,
-                                k_used + 1, wd.ptr, rows, k_used, n_expert, n_ffn, n_embd))
-    for _ in range(3):
-        if not run():
+                                k_used + 1, wd.ptr, rows, k_used, n_expert, n_ffn, n_embd)):
             raise RuntimeError("the device declined the mixture block")
+    ms = measure(dev, run, 20, gate_)
+    resid.zero()
+    run(0)
     dev.synchronize()
-    e0, e1, n = Event(), Event(), 20
-    e0.record(dev.stream)
-    for _ in range(n):
-        run()
-    e1.record(dev.stream)
-    e1.synchronize()
-    ms = e0.elapsed_ms(e1) / n
+    got, sel, wt = resid.get(), sd.get(), wd.get()
+    if not np.all(np.isfinite(got)):
+        raise RuntimeError("mixture block: non-finite output")
+    err = 0.0
+    for r in (0, rows // 2, rows - 1):
+        want = np.zeros(n_embd)
+        xr = x_host[r].astype(np.float64)
+        for s_ in range(k_used):
+            e = int(sel[r, s_])
+            g = dequant_rows(dev, t, hosts[0], np.arange(e * n_ffn, (e + 1) * n_ffn), n_embd) @ xr
+            u = dequant_rows(dev, t, hosts[1], np.arange(e * n_ffn, (e + 1) * n_ffn), n_embd) @ xr
+            want += float(wt[r, s_]) * (dequant_rows(dev, t, hosts[2], np.arange(e * n_embd, (e + 1) * n_embd), n_ffn)
+                                        @ (_silu(g) * u))
+        err = max(err, rel_err(got[r], want, f"mixture block row {r}", 3e-2))
     nbytes = touched * (2 * gs + ds) + 2 * rows * n_embd * 4 + n_expert * n_embd * 4
     for b in banks + [x, sd, wd, resid, ld, router]:
         b.free()
     return {"us_per_step": round(ms * 1e3, 1), "experts_touched": touched, "bytes_per_step": nbytes,
             "GB/s": round(nbytes / (ms * 1e-3) / 1e9, 1),
             "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-            "TFLOP/s": round(rows * k_used * 3 * 2.0 * n_ffn * n_embd / (ms * 1e-3) / 1e12, 2)}
+            "TFLOP/s": round(rows * k_used * 3 * 2.0 * n_ffn * n_embd / (ms * 1e-3) / 1e12, 2),
+            "checked_rel_err": float(f"{err:.2e}")}
 
 
-def moe_decode_section(dev):
+def moe_decode_section(dev, gate_):
     """The same mixture at decode: one token, its eight experts.  The three banks are packed
     planes on the device (one set per bank, as a .jlm file holds them); gate and up of the eight
     experts are ONE launch of sixteen packed matvecs sharing x, the eight down projections one
     launch over silu(gate) * up.  Every step takes another eight experts, so the sheets come
-    from memory.  Bytes = 24 sheets + activations."""
+    from memory.  Bytes = 24 sheets + activations.  Output check: the last step's first and
+    last expert recomputed in f64 from their sheets dequantized on the device."""
     from jitllm_amd import quant, synth
-    from jitllm_amd.hipmem import DeviceArray, Event
+    from jitllm_amd.hipmem import DeviceArray
     t, n_expert, k_used, n_ffn, n_embd = quant.Q4_K, 128, 8, 768, 2048
     dev.SetActWindow(256)
-    planes = []
+    planes, hosts = [], []
     for i, (r, k) in enumerate([(n_ffn, n_embd), (n_ffn, n_embd), (n_embd, n_ffn)]):
-        src = DeviceArray(synth.quantized_weights(t, r * n_expert, k, seed=10 + i))
+        hosts.append(synth.quantized_weights(t, r * n_expert, k, seed=10 + i))
+        src = DeviceArray(hosts[-1])
         nq, nd, nsc = dev.packed_words(t, r * n_expert, k)
         pl = [DeviceArray(shape=(n,), dtype=np.uint32, fill=0) for n in (nq, nd, nsc)]
         if not dev.pack_weights_dev(t, src.ptr, r * n_expert, k, pl[0].ptr, pl[1].ptr, pl[2].ptr):
@@ -407,8 +496,8 @@ def moe_decode_section(dev):
         dev.synchronize()
         src.free()
         planes.append(pl)
-    x = DeviceArray(synth.activations(n_embd, seed=4))
-    gu = [DeviceArray(shape=(n_ffn,), dtype=np.float32, fill=0) for _ in range(2 * k_used)]   # gate 0..7, up 8..15
+    x_host = synth.activations(n_embd, seed=4)
+    x = DeviceArray(x_host)
     g = DeviceArray(shape=(k_used, n_ffn), dtype=np.float32, fill=0)
     u = DeviceArray(shape=(k_used, n_ffn), dtype=np.float32, fill=0)
     ys = [DeviceArray(shape=(n_embd,), dtype=np.float32, fill=0) for _ in range(k_used)]
@@ -429,59 +518,109 @@ def moe_decode_section(dev):
         a, b = calls[i % len(calls)]
         if not (dev.packed_multi_call(a) and dev.packed_multi_call(b)):
             raise RuntimeError("the device declined the decode mixture")
-    for i in range(4):
-        run(i)
+    ms = measure(dev, run, 32, gate_, warm=4)
+    run(5)
     dev.synchronize()
-    e0, e1, n = Event(), Event(), 64
-    e0.record(dev.stream)
-    for i in range(n):
-        run(i)
-    e1.record(dev.stream)
-    e1.synchronize()
-    ms = e0.elapsed_ms(e1) / n
+    err, xr = 0.0, x_host.astype(np.float64)
+    for j in (0, k_used - 1):
+        e = picks[5][j]
+        gg = dequant_rows(dev, t, hosts[0], np.arange(e * n_ffn, (e + 1) * n_ffn), n_embd) @ xr
+        uu = dequant_rows(dev, t, hosts[1], np.arange(e * n_ffn, (e + 1) * n_ffn), n_embd) @ xr
+        err = max(err, rel_err(g.get()[j], gg, "decode mixture gate"), rel_err(u.get()[j], uu, "decode mixture up"))
+        want = dequant_rows(dev, t, hosts[2], np.arange(e * n_embd, (e + 1) * n_embd), n_ffn) @ (_silu(gg) * uu)
+        err = max(err, rel_err(ys[j].get(), want, "decode mixture down", 3e-2))
     sheet = n_ffn * quant.row_bytes(t, n_embd)
     nbytes = 3 * k_used * sheet + 4 * n_embd + 4 * (4 * k_used * n_ffn) + 4 * k_used * n_embd
     for pl in planes:
         for b in pl:
             b.free()
-    for b in [x, g, u] + gu + ys:
+    for b in [x, g, u] + ys:
         b.free()
     return {"us_per_step": round(ms * 1e3, 2), "launches_per_step": 2, "bytes_per_step": nbytes,
             "GB/s": round(nbytes / (ms * 1e-3) / 1e9, 1),
-            "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+            "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+            "checked_rel_err": float(f"{err:.2e}")}
 
 
-def mxfp4_section(dev):
-    """gpt-oss-20B expert shape: MXFP4 2880x2880, bf16 activations, tokens 1 / 64 / 1024."""
+def mxfp4_section(dev, gate_):
+    """gpt-oss-20B expert shape: MXFP4 2880x2880, bf16 activations, tokens 1 / 64 / 1024.  The
+    1- and 64-token cases are bound by the weight stream, so they rotate through enough
+    distinct weight copies to exceed twice the Infinity Cache, like the headline; 1024 tokens
+    is bound by the matrix cores and reads one copy.  Output check: rows spread over the matrix
+    against dequantize (on the device) + f64 dot with the bf16 activations (exact inputs, so
+    the bar is 1e-5)."""
     from jitllm_amd import quant, synth
-    from jitllm_amd.hipmem import DeviceArray, Event
+    from jitllm_amd.hipmem import DeviceArray, check, hip
     nrows = k = 2880
-    w = DeviceArray(synth.quantized_weights(quant.MXFP4, nrows, k, seed=0))
+    w_host = synth.quantized_weights(quant.MXFP4, nrows, k, seed=0)
+    wbytes = (w_host.nbytes + 255) & ~255
+    ncopies = (2 * CACHE_BYTES + (64 << 20)) // wbytes + 1
+    one = DeviceArray(w_host)
+    pool = DeviceArray(shape=(ncopies * wbytes,), dtype=np.uint8)
+    for i in range(ncopies):
+        check(hip().hipMemcpy(pool.ptr + i * wbytes, one.ptr, w_host.nbytes, 3), "copy")
+    rows = spread_rows(nrows, 96)
+    wrows = dequant_rows(dev, quant.MXFP4, w_host, rows, k)
     out = {}
     for ntok in (1, 64, 1024):
         xf = np.random.default_rng(3).standard_normal((ntok, k)).astype(np.float32)
         xb = (xf.view(np.uint32) >> 16).astype(np.uint16)
         x = DeviceArray(xb)
-        o = DeviceArray(shape=(ntok, nrows), dtype=np.float32)
-        for _ in range(3):
-            if not dev.matmul_mxfp4_bf16_dev(o.ptr, w.ptr, x.ptr, nrows, k, ntok):
+        o = DeviceArray(shape=(ntok, nrows), dtype=np.float32, fill=np.float32(np.nan))
+        rotate = ntok <= 64
+        if not dev.reserve_shape(quant.MXFP4, nrows, k, ntok):
+            raise RuntimeError("the device declined the MXFP4 shape")
+
+        def run(i):
+            wp = pool.ptr + (i % ncopies) * wbytes if rotate else one.ptr
+            if not dev.matmul_mxfp4_bf16_dev(o.ptr, wp, x.ptr, nrows, k, ntok):
                 raise RuntimeError("the device declined the MXFP4 matmul")
-        dev.synchronize()
-        e0, e1, n = Event(), Event(), 50
-        e0.record(dev.stream)
-        for _ in range(n):
-            dev.matmul_mxfp4_bf16_dev(o.ptr, w.ptr, x.ptr, nrows, k, ntok)
-        e1.record(dev.stream)
-        e1.synchronize()
-        ms = e0.elapsed_ms(e1) / n
+        ms = measure(dev, run, 40, gate_, warm=20)
+        got = o.get()
+        if not np.all(np.isfinite(got)):
+            raise RuntimeError(f"MXFP4 {ntok} tokens: non-finite or unwritten output")
+        xe = (xb.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+        err = rel_err(got[:, rows], xe @ wrows.T, f"MXFP4 {ntok} tokens", 1e-5)
         nbytes = nrows * (k // 32) * 17 + ntok * k * 2 + ntok * nrows * 4
         tf = 2.0 * nrows * k * ntok / (ms * 1e-3) / 1e12
         out[f"{ntok} tokens"] = {"us_per_step": round(ms * 1e3, 1), "TFLOP/s": round(tf, 2),
                                  "frac_of_bf16_mfma_peak": round(tf / MFMA_F16_PEAK_TFLOPS, 4),
-                                 "GB/s": round(nbytes / (ms * 1e-3) / 1e9, 1), "weights": "single copy (cache resident)"}
+                                 "GB/s": round(nbytes / (ms * 1e-3) / 1e9, 1),
+                                 "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                                 "weights": f"{ncopies} rotating copies" if rotate else "single copy (cache resident)",
+                                 "checked_rel_err": float(f"{err:.2e}")}
         x.free()
         o.free()
-    w.free()
+    one.free()
+    pool.free()
+    return out
+
+
+def ceiling_section(dev, gate_):
+    """What a single launch costs on this machine before any arithmetic, beside the kernels it
+    bounds: back-to-back empty kernels, and a kernel that only READS n bytes (every thread
+    keeps eight 128-bit loads in flight; nothing is stored), over rotating buffers that exceed
+    twice the Infinity Cache, at the sizes of the decode matvecs.  Median of nine windows."""
+    from jitllm_amd.hipmem import DeviceArray
+    out = {}
+    ms = measure(dev, lambda i: dev.probe_dev(0, None, 0, 512, 1024), 200, gate_, warm=50)
+    out["empty_kernel"] = {"us_per_launch": round(ms * 1e3, 3), "grid": 512, "block": 1024}
+    pool = DeviceArray(np.random.default_rng(0).integers(0, 1 << 32, (640 << 20) // 4, dtype=np.uint32))
+    for name, nbytes in [("9.4 MB (Q4_K 4096x4096)", 9437184), ("33 MB (Q4_K 14336x4096)", 33030144),
+                         ("48 MB (Q6_K 4096x14336)", 48168960), ("62 MB (Q8_0 14336x4096)", 62390272)]:
+        stride = (nbytes + 4095) & ~4095
+        ncopies = pool.nbytes // stride
+        best = None
+        for grid, block in [(256, 1024), (512, 1024), (1024, 512), (2048, 256), (512, 768)]:
+            ms = measure(dev, lambda i: dev.probe_dev(1, pool.ptr + (i % ncopies) * stride, nbytes, grid, block),
+                         100, gate_, warm=20)
+            if best is None or ms < best[0]:
+                best = (ms, grid, block)
+        ms, grid, block = best
+        out[name] = {"us_per_launch": round(ms * 1e3, 3), "GB/s": round(nbytes / (ms * 1e-3) / 1e9, 1),
+                     "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                     "grid": grid, "block": block, "copies": ncopies}
+    pool.free()
     return out
 
 
@@ -494,47 +633,71 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="headline workload only")
     ap.add_argument("--gemm", metavar="NTOK,NROWS", help="only the prefill GEMM of this shape (k = 4096), "
                     "for profiling one kernel; prints its section alone")
-    ap.add_argument("--section", choices=["mxfp4", "moe", "moe_decode", "ffn", "ffn_packed"], help="only this section of the default run, for "
-                    "profiling its kernels; prints the section alone")
+    ap.add_argument("--matvec", metavar="TYPE,NROWS,K[,packed][,w32]", help="only this decode matvec (TYPE q4_k, q6_k or "
+                    "q8_0; packed = packed planes; w32 = activation window 32), for profiling one kernel; "
+                    "prints its section alone")
+    ap.add_argument("--section", choices=["mxfp4", "moe", "moe_decode", "ffn", "ffn_packed", "ceiling", "gemm_packed"],
+                    help="only this section of the default run, for profiling its kernels; prints the section alone")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this path runs on one GPU (no sharding, no collectives); use --gpus 1")
 
     from jitllm_amd import quant
     from jitllm_amd.device import Device
+    from jitllm_amd.hipmem import Gate
 
     dev = Device(device=0, act_window=256)
+    gate = Gate()
     if args.gemm:
         ntok, nrows = (int(v) for v in args.gemm.split(","))
-        print(json.dumps({"prefill_gemm": gemm_section(dev, {nrows: (ntok,)})}), flush=True)
+        print(json.dumps({"prefill_gemm": gemm_section(dev, gate, {nrows: (ntok,)})}), flush=True)
+        dev.close()
+        return
+    if args.matvec:
+        f = args.matvec.split(",")
+        t = {"q4_k": quant.Q4_K, "q6_k": quant.Q6_K, "q8_0": quant.Q8_0}[f[0]]
+        wl = Workload(dev, t, int(f[1]), int(f[2]), 32 if t == quant.Q8_0 or "w32" in f else 256,
+                      packed="packed" in f)
+        ms, per, host_us = wl.timed(args.steps, args.warmup, gate)
+        wl.check()
+        g = wl.alg_bytes / (ms * 1e-3) / 1e9
+        print(json.dumps({"matvec": wl.name, "packed": wl.packed, "us_per_step": round(ms * 1e3, 3),
+                          "GB/s": round(g, 1), "frac_of_hbm_peak": round(g / HBM_PEAK_GBS, 4),
+                          "bytes_per_step": wl.alg_bytes}), flush=True)
         dev.close()
         return
     if args.section:
         fn = {"mxfp4": mxfp4_section, "moe": moe_section, "moe_decode": moe_decode_section, "ffn": ffn_section,
-              "ffn_packed": ffn_packed_section}[args.section]
-        print(json.dumps({args.section: fn(dev)}), flush=True)
+              "ffn_packed": ffn_packed_section, "ceiling": ceiling_section,
+              "gemm_packed": lambda d, g: gemm_section(d, g, {4096: (512,), 14336: (512,)}, packed=True)}[args.section]
+        print(json.dumps({args.section: fn(dev, gate)}), flush=True)
         dev.close()
         return
     head = Workload(dev, quant.Q4_K, 4096, 4096, window=256)
-    ms, ms_host = head.timed(args.steps, args.warmup)
+    ms, per, host_us = head.timed(args.steps, args.warmup, gate)
     head.check()
     gbs = head.alg_bytes / (ms * 1e-3) / 1e9
     line = {
         "metric": "Q4_K matvec GB/s (% of HBM peak)",
         "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms, 6), "ms_per_step_host_clock": round(ms_host, 6),
+        "ms_per_step": round(ms, 6),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "i8 dot, f32 accumulate", "data": "synthetic",
         "config": {"workload": head.name + ", weights N(0,0.02) seed 0 quantized to Q4_K, x N(0,1); "
                                f"activation quantizer (window 256) fused into the launch; "
                                f"{head.ncopies} rotating weight copies ({head.ncopies * head.wbytes >> 20} MiB)",
                    "bytes_per_step": head.alg_bytes},
+        "timing": {"protocol": f">= 200 untimed launches, then 9 timed windows of {args.steps} launches each, HIP events "
+                               "on the launch stream, each window enqueued behind a fill of a scratch buffer; "
+                               "ms_per_step is the median window",
+                   "windows_us_per_step": [round(v * 1e3, 3) for v in per],
+                   "host_enqueue_us_per_launch": round(host_us, 2)},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get("c1"),
                      "kernel": "jl_matvec_q4k_r1", "pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2)},
     }
     # the same launch over ONE copy of the weights (cache resident): what the memory side costs
-    head_hot = head.timed_hot(max(200, args.steps // 4))
+    head_hot = head.timed_hot(max(200, args.steps // 4), gate)
     line["headline_single_copy"] = {"us_per_step": round(head_hot * 1e3, 2),
                                     "GB/s": round(head.alg_bytes / (head_hot * 1e-3) / 1e9, 1),
                                     "weights": "single copy (cache resident); not the metric"}
@@ -551,32 +714,37 @@ def main():
                 if key == "q4_k_4096x4096" and not packed:
                     continue  # the headline above
                 wl = Workload(dev, t, nrows, k, window, packed=packed)
-                ems, _ = wl.timed(max(50, args.steps // 10), max(10, args.warmup // 10))
-                wl.check()
+                ems, _, _ = wl.timed(max(50, min(args.steps, 200)), args.warmup, gate)
+                err = wl.check()
                 g = wl.alg_bytes / (ems * 1e-3) / 1e9
                 extra.setdefault(key, {})[layout] = {
                     "us_per_step": round(ems * 1e3, 2), "GB/s": round(g, 1),
-                    "frac_of_hbm_peak": round(g / HBM_PEAK_GBS, 4), "bytes_per_step": wl.alg_bytes}
+                    "frac_of_hbm_peak": round(g / HBM_PEAK_GBS, 4), "bytes_per_step": wl.alg_bytes,
+                    "checked_rel_err": float(f"{err:.2e}")}
                 wl.free()
         line["other_configs"] = extra
-
-    if not args.no_extra:
-        line["ffn_block_decode"] = ffn_section(dev)
-        line["ffn_block_decode_packed"] = ffn_packed_section(dev)
-        line["prefill_gemm"] = gemm_section(dev)
-        from jitllm_amd import quant as _quant
-        line["prefill_gemm_q6k"] = gemm_section(dev, {4096: (512, 2048)}, _quant.Q6_K, 14336)
+        line["launch_ceiling"] = ceiling_section(dev, gate)
+        line["ffn_block_decode"] = ffn_section(dev, gate)
+        line["ffn_block_decode_packed"] = ffn_packed_section(dev, gate)
+        line["prefill_gemm"] = gemm_section(dev, gate)
+        g512 = line["prefill_gemm"]["512x4096->4096"]
+        line["roofline_prefill_gemm"] = {"bound": "mfma", "achieved": g512["TFLOP/s"], "peak": MFMA_F16_PEAK_TFLOPS,
+                                         "unit": "TFLOP/s", "frac": g512["frac_of_f16_mfma_peak"], "traffic": None,
+                                         "workload": "Q4_K prefill GEMM 512 tokens x 4096 -> 4096, prep + GEMM per step"}
+        line["prefill_gemm_packed_planes"] = gemm_section(dev, gate, {4096: (512,), 14336: (512,)}, packed=True)
+        line["prefill_gemm_q6k"] = gemm_section(dev, gate, {4096: (512, 2048)}, quant.Q6_K, 14336)
         # the second configuration's matrices at prefill: the activation window is 32 there
         line["prefill_gemm_window32"] = {
-            "q8_0": gemm_section(dev, {14336: (512, 2048)}, _quant.Q8_0, 4096, 32),
-            "q6_k": gemm_section(dev, {4096: (512, 2048)}, _quant.Q6_K, 14336, 32)}
-        line["moe_block"] = moe_section(dev)
-        line["moe_block_prefill_1024_rows"] = moe_section(dev, 1024)   # matrix-core tiles per expert
-        line["moe_decode"] = moe_decode_section(dev)
-        line["mxfp4_gemm"] = mxfp4_section(dev)
+            "q8_0": gemm_section(dev, gate, {14336: (512, 2048)}, quant.Q8_0, 4096, 32),
+            "q6_k": gemm_section(dev, gate, {4096: (512, 2048)}, quant.Q6_K, 14336, 32)}
+        line["moe_block"] = moe_section(dev, gate)
+        line["moe_block_prefill_1024_rows"] = moe_section(dev, gate, 1024)   # matrix-core tiles per expert
+        line["moe_decode"] = moe_decode_section(dev, gate)
+        line["mxfp4_gemm"] = mxfp4_section(dev, gate)
 
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(quant.Q4_K, 4096, 4096, 256)
+    gate.free()
     dev.close()
     print(json.dumps(line), flush=True)
 

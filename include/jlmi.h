@@ -54,7 +54,10 @@ typedef struct jl_ctx jl_ctx;
 /* Per-context options; the library reads no environment variables, like the
  * reference's per-instance options (engine/nn/options.go:7-13). */
 typedef struct jl_options {
-    int device;              /* HIP device ordinal */
+    int device;              /* HIP device ordinal; < 0: a context bound to no device --
+                                its host-side bookkeeping works (residency keys, the
+                                forget queue, the lock), every entry point that needs
+                                the GPU fails with JL_ERR_HIP */
     int act_window;          /* activation amax window: 32 or 256; 0 = 32 */
     const char *code_object; /* path of the gfx950 code object; NULL = the file
                                 jlmi_gfx950.hsaco beside the library */
@@ -99,6 +102,14 @@ int jl_set_tuning(jl_ctx *ctx, const char *key, int value);
  * (engine/nn/packedgroup.go:13-20). */
 unsigned long long jl_launch_count(const jl_ctx *ctx);
 
+/* Measurement only; no counterpart in the reference.  What a single launch costs on this
+ * machine before any arithmetic, so a kernel's time can be set beside it: kind 0 launches
+ * an empty kernel, kind 1 a kernel that only reads nbytes of device memory at src (16-byte
+ * aligned; every thread keeps eight 128-bit loads in flight) and stores nothing.  grid and
+ * block <= 0 pick two 1024-thread workgroups per CU. */
+int jl_probe_dev(jl_ctx *ctx, int kind, const void *src, size_t nbytes, int grid, int block,
+                 void *stream);
+
 /* ---- host-pointer seam ------------------------------------------------ */
 
 /* nn.Device.MatVec (engine/nn/device.go:23-31; call site engine/nn/jit.go:935-940):
@@ -109,8 +120,25 @@ int jl_matvec(jl_ctx *ctx, float *out, int type, const void *w, size_t wbytes,
               const float *x, int nrows, int k);
 
 /* nn.CopyForgetter.Forget (engine/nn/device.go:1570-1581): drop any device copy
- * keyed inside [p, p+n).  Callable from any thread; never blocks on the GPU. */
+ * keyed inside [p, p+n).  Callable from any thread, also from inside a page-in that
+ * this context's own upload started: it only queues the range under a lock of its own
+ * -- no HIP call, no lock that a launch or an upload holds (the reference queues the
+ * range the same way when its device is busy, jit/gpu/tier/forget.go:20-40).  The
+ * next host-pointer call on the context unlinks and frees the matching copies before
+ * it looks its weight up; jl_ctx_destroy frees what is left. */
 int jl_forget(jl_ctx *ctx, const void *p, size_t n);
+
+/* The lock the host-pointer entry points hold for their whole synchronous run (the
+ * reference's tier serialises the same way, jit/gpu/tier/tier.go:2831-2843), for a
+ * caller that needs several of them to run as one.  Not recursive: a host-pointer call
+ * between lock and unlock on the same thread deadlocks; *_dev calls and jl_forget take
+ * no such lock. */
+int jl_ctx_lock(jl_ctx *ctx);
+int jl_ctx_unlock(jl_ctx *ctx);
+
+/* Device copies the context holds for the host-pointer seam, after applying queued
+ * forgets (takes the context lock). */
+size_t jl_resident_count(jl_ctx *ctx);
 
 /* JIT.MatMul over raw GGUF bytes (engine/nn/matmul.go:27): x [ntok][k] ->
  * out [ntok][nrows].  Each token is quantized on its own. */
@@ -241,6 +269,14 @@ int jl_matmul_dev(jl_ctx *ctx, float *out, int type, const void *w, const float 
  * prefill workspace for up to max_tok tokens of max_k features now, so later
  * calls allocate nothing. */
 int jl_reserve(jl_ctx *ctx, int max_tok, int max_k);
+
+/* The same for one call shape, exactly: walks the launch path of jl_matmul_dev
+ * (packed = 0), jl_matmul_packed_dev (packed = 1) or jl_matmul_mxfp4_bf16_dev (type
+ * MXFP4) for this type, shape and the context's current activation window with
+ * launching switched off, so every workspace that call would grow -- activation
+ * fragments, rows restored from planes, K-split partial sums -- has its size
+ * afterwards and the call itself allocates nothing.  Returns what the call would. */
+int jl_reserve_shape(jl_ctx *ctx, int type, int nrows, int k, int ntok, int packed);
 
 /* kernels.PackWeightsInto (jit/gpu/kernels/pack.go:52-199) on the device: GGUF
  * row-major blocks -> the three planes [unit][row] (sizes from jl_packed_words; sc may

@@ -43,6 +43,11 @@ SIGNATURES = {
     "jl_set_tuning": (_int, [_vp, C.c_char_p, _int]),
     "jl_matvec": (_int, [_vp, _vp, _int, _vp, _sz, _vp, _int, _int]),
     "jl_forget": (_int, [_vp, _vp, _sz]),
+    "jl_probe_dev": (_int, [_vp, _int, _vp, _sz, _int, _int, _vp]),
+    "jl_ctx_lock": (_int, [_vp]),
+    "jl_ctx_unlock": (_int, [_vp]),
+    "jl_resident_count": (_sz, [_vp]),
+    "jl_reserve_shape": (_int, [_vp, _int, _int, _int, _int, _int]),
     "jl_matmul": (_int, [_vp, _vp, _int, _vp, _sz, _vp, _int, _int, _int]),
     "jl_quantize_act_dev": (_int, [_vp, _vp, _int, _int, _vp, _vp, _vp, _vp]),
     "jl_dequant_dev": (_int, [_vp, _int, _vp, _vp, _sz, _vp]),

@@ -19,6 +19,7 @@ struct HipApi {
     hipError_t (*StreamCreate)(hipStream_t*) = nullptr;
     hipError_t (*StreamDestroy)(hipStream_t) = nullptr;
     hipError_t (*StreamSynchronize)(hipStream_t) = nullptr;
+    hipError_t (*DeviceSynchronize)() = nullptr;
     hipError_t (*ModuleLoad)(hipModule_t*, const char*) = nullptr;
     hipError_t (*ModuleUnload)(hipModule_t) = nullptr;
     hipError_t (*ModuleGetFunction)(hipFunction_t*, hipModule_t, const char*) = nullptr;
@@ -65,6 +66,7 @@ inline const HipApi* hip_api(std::string* why) {
             JL_SYM(StreamCreate, "hipStreamCreate");
             JL_SYM(StreamDestroy, "hipStreamDestroy");
             JL_SYM(StreamSynchronize, "hipStreamSynchronize");
+            JL_SYM(DeviceSynchronize, "hipDeviceSynchronize");
             JL_SYM(ModuleLoad, "hipModuleLoad");
             JL_SYM(ModuleUnload, "hipModuleUnload");
             JL_SYM(ModuleGetFunction, "hipModuleGetFunction");

@@ -10,6 +10,7 @@
 
 #include <dlfcn.h>
 
+#include <algorithm>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -55,6 +56,12 @@ struct jl_ctx {
     std::map<std::string, hipFunction_t> fn;
     std::string err;
     std::mutex mu;  // serialises the host-pointer seam (one staging area per context)
+    // jl_forget only queues its range here, under a lock no launch or upload path holds; the
+    // host-pointer calls apply the queue (unlink + hipFree) before their residency lookup
+    std::mutex forget_mu;
+    std::vector<std::pair<uintptr_t, uintptr_t>> pending_forget;
+    bool no_device = false;   // created with device < 0: host-side bookkeeping only
+    bool dry_run = false;     // jl_reserve_shape: size the workspaces, launch nothing
     Tuning tune;
     int gemm_min_tok = 3;  // below this a per-token matvec loop is as fast (3.8 us a token against 8.9 us for up to 16)
     int num_cu = 0;
@@ -153,8 +160,26 @@ int launch(jl_ctx* c, const char* name, unsigned gx, unsigned gy, unsigned block
            hipStream_t st, void** params, unsigned gz = 1) {
     auto it = c->fn.find(name);
     if (it == c->fn.end()) return fail(c, JL_ERR_ARG, "kernel %s is not in the code object", name);
+    if (c->dry_run) return JL_OK;
     HIP_TRY(c, H->ModuleLaunchKernel(it->second, gx, gy, gz, block, 1, 1, lds, st, params, nullptr));
     c->launches++;
+    return JL_OK;
+}
+
+// Grows a context-owned device buffer.  Growing frees the old one, which kernels enqueued by
+// earlier calls -- on the context's stream or on any stream a caller passed -- may still
+// read, so the whole device is waited for first.  Never reached once the buffer is large
+// enough (jl_reserve, jl_reserve_shape).
+int grow(jl_ctx* c, void** buf, size_t* have, size_t need) {
+    if (*have >= need) return JL_OK;
+    if (*buf) {
+        HIP_TRY(c, H->DeviceSynchronize());
+        HIP_TRY(c, H->Free(*buf));
+    }
+    *buf = nullptr;
+    *have = 0;
+    HIP_TRY(c, H->Malloc(buf, need));
+    *have = need;
     return JL_OK;
 }
 
@@ -271,14 +296,26 @@ int matvec_multi_launch(jl_ctx* c, int type, int m, float* const* outs, const vo
     return launch(c, name, (unsigned)gx, (unsigned)m, nwaves * 64, lds, st, params);
 }
 
-int ensure_stage(jl_ctx* c, void** buf, size_t* have, size_t need) {
-    if (*have >= need) return JL_OK;
-    if (*buf) HIP_TRY(c, H->Free(*buf));
-    *buf = nullptr;
-    *have = 0;
-    HIP_TRY(c, H->Malloc(buf, need));
-    *have = need;
-    return JL_OK;
+int ensure_stage(jl_ctx* c, void** buf, size_t* have, size_t need) { return grow(c, buf, have, need); }
+
+// Applies the ranges jl_forget queued: every device copy keyed inside one of them is
+// unlinked and freed.  Called with c->mu held, before a residency lookup.
+void drain_forget(jl_ctx* c) {
+    std::vector<std::pair<uintptr_t, uintptr_t>> todo;
+    {
+        std::lock_guard<std::mutex> g(c->forget_mu);
+        todo.swap(c->pending_forget);
+    }
+    for (const auto& r : todo)
+        for (auto it = c->resident.begin(); it != c->resident.end();) {
+            const uintptr_t k0 = (uintptr_t)it->first;
+            if (k0 >= r.first && k0 < r.second) {
+                if (!c->no_device) (void)H->Free(it->second.dev);
+                it = c->resident.erase(it);
+            } else {
+                ++it;
+            }
+        }
 }
 
 // Device copy of host weight bytes, keyed on the host pointer.
@@ -323,17 +360,7 @@ size_t gemm_ws_need(int ntok, int k) {
     return nsb * 2 * (tok_pad / 32) * kGemmAStageBytes + nsb * tok_pad * 4;
 }
 
-int gemm_ws_ensure(jl_ctx* c, size_t need) {
-    if (c->gemm_ws_bytes >= need) return JL_OK;
-    // growing frees the old workspace: wait for work that may still read it
-    HIP_TRY(c, H->StreamSynchronize(c->stream));
-    if (c->gemm_ws) HIP_TRY(c, H->Free(c->gemm_ws));
-    c->gemm_ws = nullptr;
-    c->gemm_ws_bytes = 0;
-    HIP_TRY(c, H->Malloc(&c->gemm_ws, need));
-    c->gemm_ws_bytes = need;
-    return JL_OK;
-}
+int gemm_ws_ensure(jl_ctx* c, size_t need) { return grow(c, &c->gemm_ws, &c->gemm_ws_bytes, need); }
 
 constexpr size_t kGemmW16StageVecs = 1152;   // JL_GEMM_W16_STAGE_VECS
 constexpr unsigned kGemmW16LdsBytes = 2u * 1152u * 16u + 2u * kGemmTile * 4u;
@@ -345,15 +372,8 @@ int gemm_q4k_w16_launch(jl_ctx* c, float* out, const void* w, const uint16_t* bq
     const int nrt = (nrows + 63) / 64, nrows_pad = nrt * 64, ntt = tok_pad / kGemmTile;
     const size_t w16_bytes = (size_t)nrt * 2 * nsb * kGemmW16StageVecs * 16;
     const size_t need = w16_bytes + (size_t)nsb * nrows_pad * 8;
-    if (c->w16_ws_bytes < need) {
-        HIP_TRY(c, H->StreamSynchronize(c->stream));
-        if (st != c->stream) HIP_TRY(c, H->StreamSynchronize(st));
-        if (c->w16_ws) HIP_TRY(c, H->Free(c->w16_ws));
-        c->w16_ws = nullptr;
-        c->w16_ws_bytes = 0;
-        HIP_TRY(c, H->Malloc(&c->w16_ws, need));
-        c->w16_ws_bytes = need;
-    }
+    int rcw = grow(c, &c->w16_ws, &c->w16_ws_bytes, need);
+    if (rcw != JL_OK) return rcw;
     float* wsc = (float*)((char*)c->w16_ws + w16_bytes);
     GemmW16PrepArgs pa;
     pa.w = (const uint8_t*)w; pa.w16 = c->w16_ws; pa.wsc = wsc;
@@ -484,9 +504,9 @@ int gemm_q4k_launch(jl_ctx* c, float* out, const void* w, const float* x, int nr
             rc = ws_ensure(c, &c->mx_ws, &c->mx_ws_bytes, n * nsplit * 4);
             if (rc != JL_OK) return rc;
             ga.out = (float*)c->mx_ws; ga.sb_per = per;
-            HIP_TRY(c, H->ModuleLaunchKernel(c->fn["jl_gemm_q4k_r64"], (unsigned)(tok_pad / kGemmTile),
-                                             (unsigned)((nrows + 63) / 64), (unsigned)nsplit, 256, 1, 1,
-                                             gemm_lds_bytes(64), st, gp, nullptr));
+            rc = launch(c, "jl_gemm_q4k_r64", (unsigned)(tok_pad / kGemmTile), (unsigned)((nrows + 63) / 64), 256,
+                        gemm_lds_bytes(64), st, gp, (unsigned)nsplit);
+            if (rc != JL_OK) return rc;
             SumPartsArgs sa;
             sa.out = out; sa.part = (const float*)c->mx_ws; sa.n = n; sa.nsplit = nsplit;
             void* sp[] = {&sa};
@@ -632,16 +652,7 @@ int matmul_launch(jl_ctx* c, float* out, int type, const void* w, const float* x
     return JL_OK;
 }
 
-int ws_ensure(jl_ctx* c, void** buf, size_t* have, size_t need) {
-    if (*have >= need) return JL_OK;
-    HIP_TRY(c, H->StreamSynchronize(c->stream));  // work in flight may still read the old one
-    if (*buf) HIP_TRY(c, H->Free(*buf));
-    *buf = nullptr;
-    *have = 0;
-    HIP_TRY(c, H->Malloc(buf, need));
-    *have = need;
-    return JL_OK;
-}
+int ws_ensure(jl_ctx* c, void** buf, size_t* have, size_t need) { return grow(c, buf, have, need); }
 
 // Words of the three planes of an nrows x k matrix (jit/gpu/kernels/pack.go:580-621).
 bool packed_words(int type, size_t nrows, int k, size_t* nq, size_t* nd, size_t* nsc) {
@@ -873,17 +884,12 @@ int moe_matvec_launch(jl_ctx* c, float* out0, float* out1, int type, const void*
             kGemmLdsBytes <= c->lds_limit && n_expert <= 65535 && (long)tiles_max * rtiles * ga.nmat < (1L << 31)) {
             const long work = (long)tiles_max * rtiles * ga.nmat;
             const unsigned grid = (unsigned)std::min<long>(work, (q6 ? 3L : 2L) * c->num_cu);
-            HIP_TRY(c, H->ModuleLaunchKernel(c->fn[q6 ? "jl_moe_gemm_q6k_r64" : "jl_moe_gemm_r64"], grid, 1, 1, 256, 1, 1,
-                                             q6 ? kGemm6LdsBytes : gemm_lds_bytes(64), st, gp, nullptr));
-            c->launches++;
-            return JL_OK;
+            return launch(c, q6 ? "jl_moe_gemm_q6k_r64" : "jl_moe_gemm_r64", grid, 1, 256,
+                          q6 ? kGemm6LdsBytes : gemm_lds_bytes(64), st, gp);
         }
         if (q6) return fail(c, JL_ERR_ARG, "moe matvec: %d experts x %ld row tiles do not fit the tile form", n_expert, rtiles);
-        HIP_TRY(c, H->ModuleLaunchKernel(c->fn["jl_moe_gemm_q4k"], (unsigned)((nrows + 255) / 256),
-                                         (unsigned)nslots, (unsigned)ga.nmat, 256, 1, 1, 4u * 19968u, st,
-                                         gp, nullptr));
-        c->launches++;
-        return JL_OK;
+        return launch(c, "jl_moe_gemm_q4k", (unsigned)((nrows + 255) / 256), (unsigned)nslots, 256, 4u * 19968u, st, gp,
+                      (unsigned)ga.nmat);
     }
     const int nslots = k / ti->slot_elems;
     // lanes per row: the width that leaves the fewest lanes without a slot (a row of 12 slots
@@ -941,12 +947,8 @@ int moe_matvec_launch(jl_ctx* c, float* out0, float* out1, int type, const void*
     a.nwaves = nwaves; a.shares = shares;
     char name[64];
     snprintf(name, sizeof name, "jl_moe_matvec_%s_l%d", ti->tag, lpr);
-    auto it = c->fn.find(name);
-    if (it == c->fn.end()) return fail(c, JL_ERR_ARG, "kernel %s is not in the code object", name);
     void* params[] = {&a};
-    HIP_TRY(c, H->ModuleLaunchKernel(it->second, (unsigned)shares, (unsigned)n_expert, (unsigned)nmat, nwaves * 64, 1, 1,
-                                     (unsigned)lds, st, params, nullptr));
-    return JL_OK;
+    return launch(c, name, (unsigned)shares, (unsigned)n_expert, nwaves * 64, (unsigned)lds, st, params, (unsigned)nmat);
 }
 
 }  // namespace
@@ -974,6 +976,13 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     };
     if (c->act_window != 32 && c->act_window != 64 && c->act_window != 128 && c->act_window != 256)
         return bail(JL_ERR_ARG, "act_window must be 32, 64, 128 or 256");
+    if (c->device < 0) {
+        // no device: the host-side bookkeeping (residency keys, the forget queue, the lock)
+        // works, every entry point that needs the GPU fails at its hipSetDevice
+        c->no_device = true;
+        *out = c;
+        return JL_OK;
+    }
     hipError_t e = H->SetDevice(c->device);
     if (e != hipSuccess) return bail(JL_ERR_HIP, std::string("hipSetDevice: ") + H->GetErrorString(e));
     hipDeviceProp_t prop;
@@ -989,7 +998,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     if (e != hipSuccess)
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
-    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_quant", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_q4k", "jl_moe_gemm_r64", "jl_moe_gemm_q6k_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_sum_parts",
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_group2_wide", "jl_moe_quant", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_q4k", "jl_moe_gemm_r64", "jl_moe_gemm_q6k_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_sum_parts", "jl_probe_read", "jl_probe_empty",
                                       "jl_pack_weights", "jl_unpack_q4k", "jl_unpack_q6k", "jl_unpack_q8_0"};
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int rw : {16, 32, 64})
@@ -1036,8 +1045,13 @@ const char* jl_hip_runtime(void) {
 
 void jl_ctx_destroy(jl_ctx* c) {
     if (!c) return;
+    if (c->no_device) {
+        delete c;
+        return;
+    }
     (void)H->SetDevice(c->device);
     if (c->stream) (void)H->StreamSynchronize(c->stream);
+    (void)H->DeviceSynchronize();   // callers' streams may still read the workspaces
     for (auto& kv : c->resident) (void)H->Free(kv.second.dev);
     if (c->gemm_ws) (void)H->Free(c->gemm_ws);
     if (c->w16_ws) (void)H->Free(c->w16_ws);
@@ -1282,7 +1296,33 @@ int jl_reserve(jl_ctx* c, int max_tok, int max_k) {
     if (!c) return JL_ERR_ARG;
     if (max_tok <= 0 || max_k <= 0 || max_k % 256 != 0) return fail(c, JL_ERR_ARG, "reserve: %d x %d", max_tok, max_k);
     HIP_TRY(c, H->SetDevice(c->device));
-    return gemm_ws_ensure(c, gemm_ws_need(max_tok, max_k));
+    // the k-quant prep's layout and the window-32 prep's (fragments + two scale planes)
+    const size_t tok_pad = ((size_t)max_tok + 255) / 256 * 256;
+    const size_t w32 = (size_t)(max_k / 128) * (tok_pad / 32) * 8 * 1024 + 2 * (size_t)(max_k / 32) * tok_pad * 4;
+    return gemm_ws_ensure(c, std::max(gemm_ws_need(max_tok, max_k), w32));
+}
+
+int jl_reserve_shape(jl_ctx* c, int type, int nrows, int k, int ntok, int packed) {
+    if (!c) return JL_ERR_ARG;
+    if (nrows <= 0 || k <= 0 || ntok <= 0) return fail(c, JL_ERR_ARG, "reserve shape: %d x %d, %d tokens", nrows, k, ntok);
+    HIP_TRY(c, H->SetDevice(c->device));
+    // Walk the call's own launch path with launching switched off: every workspace the path
+    // would grow is grown now, by the code that sizes it for the real call.
+    float* const out = (float*)(uintptr_t)4096;
+    const float* const x = (const float*)(uintptr_t)4096;
+    const void* const w = (const void*)(uintptr_t)4096;
+    c->dry_run = true;
+    int rc;
+    if (type == JL_TYPE_MXFP4) {
+        rc = packed ? JL_DECLINED : jl_matmul_mxfp4_bf16_dev(c, out, w, (const uint16_t*)w, nrows, k, ntok, nullptr);
+    } else if (packed) {
+        const PlaneRef pl = {(const uint32_t*)w, (const uint32_t*)w, (const uint32_t*)w, 0, nrows};
+        rc = packed_matmul_launch(c, out, type, pl, x, nrows, k, ntok, c->stream);
+    } else {
+        rc = matmul_launch(c, out, type, w, x, nrows, k, ntok, c->stream);
+    }
+    c->dry_run = false;
+    return rc;
 }
 
 int jl_moe_route_dev(jl_ctx* c, const float* logits, int rows, int n_expert, int k_used, uint32_t* sel,
@@ -1337,8 +1377,13 @@ int jl_moe_group_dev(jl_ctx* c, const uint32_t* sel, int sel_stride, int rows, i
     // expert); a wavefront's share of the pairs is counted in 16 bits
     const size_t npairs = (size_t)rows * k_used;
     const size_t lds2 = 16 * (size_t)n_expert * 2 + ((size_t)n_expert + 17) * 4;   // JL_MOE_GROUP2_LDS
-    if (c->tune.moe_group != 1 && lds2 <= c->lds_limit && npairs <= 16 * 65535)
+    // (an expert's running count, over all shares, is kept in 16 bits up to 65535 pairs and
+    // in 32 bits above)
+    if (c->tune.moe_group != 1 && lds2 <= c->lds_limit && npairs <= 65535)
         return launch(c, "jl_moe_group2", 1, 1, 1024, (unsigned)lds2, pick_stream(c, stream), params);
+    const size_t lds2w = 16 * (size_t)n_expert * 4 + ((size_t)n_expert + 17) * 4;
+    if (c->tune.moe_group != 1 && lds2w <= c->lds_limit && npairs <= 0x7fffffffu)
+        return launch(c, "jl_moe_group2_wide", 1, 1, 1024, (unsigned)lds2w, pick_stream(c, stream), params);
     return launch(c, "jl_moe_group", 1, 1, 1024, 0, pick_stream(c, stream), params);
 }
 
@@ -1474,9 +1519,9 @@ int jl_matmul_mxfp4_bf16_dev(jl_ctx* c, float* out, const void* w, const uint16_
         rc = ws_ensure(c, &c->mx_ws, &c->mx_ws_bytes, n * nsplit * 4);
         if (rc != JL_OK) return rc;
         a.nsplit = nsplit; a.part = (float*)c->mx_ws;
-        HIP_TRY(c, H->ModuleLaunchKernel(c->fn[gemm_name], (unsigned)(tok_pad / 128),
-                                         (unsigned)((nrows + trows - 1) / trows), (unsigned)nsplit, 512, 1, 1, lds, st,
-                                         params, nullptr));
+        rc = launch(c, gemm_name, (unsigned)(tok_pad / 128), (unsigned)((nrows + trows - 1) / trows), 512, lds, st,
+                    params, (unsigned)nsplit);
+        if (rc != JL_OK) return rc;
         SumPartsArgs sa;
         sa.out = out; sa.part = a.part; sa.n = n; sa.nsplit = nsplit;
         void* sp[] = {&sa};
@@ -1497,6 +1542,8 @@ int jl_matmul(jl_ctx* c, float* out, int type, const void* w, size_t wbytes, con
               int nrows, int k, int ntok) {
     if (!c) return JL_ERR_ARG;
     std::lock_guard<std::mutex> lock(c->mu);
+    drain_forget(c);
+    if (c->no_device) return fail(c, JL_ERR_HIP, "this context is bound to no device");
     const TypeInfo* ti = nullptr;
     int rc = matvec_check(c, type, nrows, k, &ti);
     if (rc != JL_OK) return rc;
@@ -1531,6 +1578,8 @@ int jl_matmul_packed(jl_ctx* c, float* out, int type, const uint32_t* qs, const 
                      const uint32_t* sc, int row, int stride, const float* x, int nrows, int k, int ntok) {
     if (!c) return JL_ERR_ARG;
     std::lock_guard<std::mutex> lock(c->mu);
+    drain_forget(c);
+    if (c->no_device) return fail(c, JL_ERR_HIP, "this context is bound to no device");
     const PlaneRef host = {qs, d, sc, row, stride};
     const TypeInfo* ti = nullptr;
     int rc = packed_check(c, type, host, nrows, k, &ti);
@@ -1582,20 +1631,48 @@ int jl_matmul_packed(jl_ctx* c, float* out, int type, const uint32_t* qs, const 
 
 int jl_forget(jl_ctx* c, const void* p, size_t n) {
     if (!c) return JL_ERR_ARG;
-    std::lock_guard<std::mutex> lock(c->mu);
-    const char* lo = (const char*)p;
-    const char* hi = lo + n;
-    (void)H->SetDevice(c->device);
-    for (auto it = c->resident.begin(); it != c->resident.end();) {
-        const char* k0 = (const char*)it->first;
-        if (k0 >= lo && k0 < hi) {
-            (void)H->Free(it->second.dev);
-            it = c->resident.erase(it);
-        } else {
-            ++it;
-        }
-    }
+    if (!p || n == 0) return JL_OK;
+    // Only queue the range: no HIP call, and no lock that a launch or an upload holds, so this
+    // returns at once from any thread -- also from inside a page-in that this context's own
+    // weight upload started.  The next host-pointer call applies the queue before it looks a
+    // pointer up; jl_ctx_destroy frees whatever is left.
+    std::lock_guard<std::mutex> g(c->forget_mu);
+    c->pending_forget.emplace_back((uintptr_t)p, (uintptr_t)p + n);
     return JL_OK;
+}
+
+int jl_probe_dev(jl_ctx* c, int kind, const void* src, size_t nbytes, int grid, int block, void* stream) {
+    if (!c) return JL_ERR_ARG;
+    if (kind != 0 && kind != 1) return fail(c, JL_ERR_ARG, "probe: kind %d", kind);
+    if (grid <= 0) grid = 2 * c->num_cu;
+    if (block <= 0) block = 1024;
+    if (block % 64 != 0 || block > 1024) return fail(c, JL_ERR_ARG, "probe: block=%d", block);
+    if (kind == 1 && (!src || !aligned16(src))) return fail(c, JL_ERR_ARG, "probe: src");
+    HIP_TRY(c, H->SetDevice(c->device));
+    size_t nvec = nbytes / 16;
+    void* sink = nullptr;
+    void* params[] = {(void*)&src, (void*)&nvec, (void*)&sink};
+    return launch(c, kind ? "jl_probe_read" : "jl_probe_empty", (unsigned)grid, 1, (unsigned)block, 0,
+                  pick_stream(c, stream), params);
+}
+
+int jl_ctx_lock(jl_ctx* c) {
+    if (!c) return JL_ERR_ARG;
+    c->mu.lock();
+    return JL_OK;
+}
+
+int jl_ctx_unlock(jl_ctx* c) {
+    if (!c) return JL_ERR_ARG;
+    c->mu.unlock();
+    return JL_OK;
+}
+
+size_t jl_resident_count(jl_ctx* c) {
+    if (!c) return 0;
+    std::lock_guard<std::mutex> lock(c->mu);
+    drain_forget(c);
+    return c->resident.size();
 }
 
 }  // extern "C"

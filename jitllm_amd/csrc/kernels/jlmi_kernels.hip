@@ -185,7 +185,9 @@ extern "C" __global__ __launch_bounds__(1024) void jl_moe_group(MoeGroupArgs p) 
     moe_group_body(p, scount, skeys);
 }
 // the linear-time form: one workgroup of 1024 threads, dynamic LDS = JL_MOE_GROUP2_LDS(experts)
-extern "C" __global__ __launch_bounds__(1024) void jl_moe_group2(MoeGroupArgs p) { moe_group2_body(p, jl_smem); }
+extern "C" __global__ __launch_bounds__(1024) void jl_moe_group2(MoeGroupArgs p) { moe_group2_body<uint16_t>(p, jl_smem); }
+// more than 65535 pairs: 32-bit counts, dynamic LDS = 16 * experts * 4 + (experts + 17) * 4
+extern "C" __global__ __launch_bounds__(1024) void jl_moe_group2_wide(MoeGroupArgs p) { moe_group2_body<u32>(p, jl_smem); }
 // grid = (ceil(k/4/256), ncols), block = 256
 extern "C" __global__ __launch_bounds__(256) void jl_moe_quant(MoeQuantArgs p) { moe_quant_body(p); }
 // grid = (row shares, n_expert, matrices), block = 512, dynamic LDS = 8 staged columns
@@ -270,3 +272,25 @@ extern "C" __global__ __launch_bounds__(256) void jl_mxfp4_prep_few(MxPrepArgs p
         mx_few_body<NT>(p, part);                                                              \
     }
 JL_MX_FEW_KERNEL(1) JL_MX_FEW_KERNEL(2) JL_MX_FEW_KERNEL(3) JL_MX_FEW_KERNEL(4)
+
+// ------------------------------------------------------------------ probes
+// What one launch costs on this machine before any arithmetic: jl_probe_read streams nvec
+// 16-byte vectors with every thread keeping eight loads in flight and folds them into a word
+// that is stored only if it matches a value random data never gives; jl_probe_empty returns
+// at once.  Timed by the benchmark beside the kernels they bound.  grid and block are free.
+extern "C" __global__ __launch_bounds__(1024) void jl_probe_read(const u32x4* __restrict__ src, size_t nvec,
+                                                                  u32* __restrict__ sink) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    u32x4 acc = u32x4{0u, 0u, 0u, 0u};
+    for (; i + 7 * stride < nvec; i += 8 * stride) {
+        u32x4 v[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) v[j] = __builtin_nontemporal_load(src + i + j * stride);
+#pragma unroll
+        for (int j = 0; j < 8; j++) acc ^= v[j];
+    }
+    for (; i < nvec; i += stride) acc ^= __builtin_nontemporal_load(src + i);
+    if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x9e3779b9u && sink) sink[0] = acc.x;
+}
+extern "C" __global__ __launch_bounds__(1024) void jl_probe_empty(const u32x4* __restrict__, size_t, u32* __restrict__) {}

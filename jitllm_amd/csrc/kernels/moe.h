@@ -246,10 +246,14 @@ __device__ __forceinline__ void moe_group_body(const MoeGroupArgs& p, u32* scoun
 // expert, no atomics.  The rank waits in pos[] between the passes (the same thread writes
 // and reads it).  grid = 1, block = 1024, dynamic LDS = JL_MOE_GROUP2_LDS(nexp).
 #define JL_MOE_GROUP2_LDS(nexp) (16 * (nexp) * 2 + ((nexp) + 1 + 16) * 4)
+// CNT: the type of a share's per-expert counts and of their running sums over the sixteen
+// shares: uint16_t while the whole pair list has at most 65535 pairs (no sum can pass that),
+// u32 above.  Dynamic LDS = 16 * nexp * sizeof(CNT) + (nexp + 17) * 4.
+template <typename CNT>
 __device__ __forceinline__ void moe_group2_body(const MoeGroupArgs& p, uint8_t* smem) {
     const int npairs = p.rows * p.k_used, nexp = p.n_expert;
     const int nruns = (npairs + 63) / 64, runs_per = (nruns + 15) / 16;
-    uint16_t* scnt = (uint16_t*)smem;                                  // [16][nexp]
+    CNT* scnt = (CNT*)smem;                                            // [16][nexp]
     u32* sstart = (u32*)(scnt + 16 * nexp);                            // [nexp + 1]
     u32* stot = sstart + nexp + 1;                                     // [16] wavefront totals
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -258,7 +262,7 @@ __device__ __forceinline__ void moe_group2_body(const MoeGroupArgs& p, uint8_t* 
     for (int i = tid; i < 16 * nexp; i += 1024) scnt[i] = 0;
     __syncthreads();
     const uint64_t lt = lane ? (~0ull >> (64 - lane)) : 0ull;   // lanes below this one
-    uint16_t* mine = scnt + wave * nexp;
+    CNT* mine = scnt + wave * nexp;
     const int run_lo = min(wave * runs_per, nruns), run_hi = min(run_lo + runs_per, nruns);
     auto key_of = [&](int i) { return p.sel[(i / p.k_used) * p.sel_stride + i % p.k_used]; };
     for (int run = run_lo; run < run_hi; run++) {
@@ -278,7 +282,7 @@ __device__ __forceinline__ void moe_group2_body(const MoeGroupArgs& p, uint8_t* 
         if (valid) {
             const u32 before = mine[e];
             p.pos[i] = before + (u32)__builtin_popcountll(m & lt);
-            if ((m & lt) == 0) mine[e] = (uint16_t)(before + (u32)__builtin_popcountll(m));
+            if ((m & lt) == 0) mine[e] = (CNT)(before + (u32)__builtin_popcountll(m));
         }
     }
     __syncthreads();
@@ -288,7 +292,7 @@ __device__ __forceinline__ void moe_group2_body(const MoeGroupArgs& p, uint8_t* 
 #pragma unroll
         for (int w = 0; w < 16; w++) {
             const u32 c = scnt[w * nexp + tid];
-            scnt[w * nexp + tid] = (uint16_t)total;
+            scnt[w * nexp + tid] = (CNT)total;
             total += c;
         }
     }

@@ -83,6 +83,27 @@ class Device:
         """nn.LayerDevice.Reserve: size the prefill workspace ahead of time."""
         self._served(self._l.jl_reserve(self._ctx, max_tok, max_k), "jl_reserve")
 
+    def reserve_shape(self, t, nrows, k, ntok, packed=False):
+        """Grow every workspace a matmul of this shape would grow, launching nothing."""
+        return self._served(self._l.jl_reserve_shape(self._ctx, t, nrows, k, ntok, int(packed)), "jl_reserve_shape")
+
+    def probe_dev(self, kind, src, nbytes, grid=0, block=0, stream=None):
+        """An empty kernel (kind 0) or a kernel that only reads nbytes at src (kind 1)."""
+        return self._served(self._l.jl_probe_dev(self._ctx, kind, src, nbytes, grid, block, stream), "jl_probe_dev")
+
+    def lock(self):
+        """The lock host-pointer calls hold while they run (jl_ctx_lock)."""
+        self._served(self._l.jl_ctx_lock(self._ctx), "jl_ctx_lock")
+
+    def unlock(self):
+        self._served(self._l.jl_ctx_unlock(self._ctx), "jl_ctx_unlock")
+
+    def resident_count(self):
+        return int(self._l.jl_resident_count(self._ctx))
+
+    def forget_range(self, address, nbytes):
+        self._served(self._l.jl_forget(self._ctx, int(address), int(nbytes)), "jl_forget")
+
     def set_tuning(self, **kw):
         for k, v in kw.items():
             key = (k.replace("__", ".") if "__" in k else "matvec." + k).encode()

@@ -29,6 +29,7 @@ def hip():
         h.hipFree.argtypes = [C.c_void_p]
         h.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
         h.hipMemset.argtypes = [C.c_void_p, C.c_int, C.c_size_t]
+        h.hipMemsetAsync.argtypes = [C.c_void_p, C.c_int, C.c_size_t, C.c_void_p]
         h.hipEventCreate.argtypes = [C.POINTER(C.c_void_p)]
         h.hipEventRecord.argtypes = [C.c_void_p, C.c_void_p]
         h.hipEventSynchronize.argtypes = [C.c_void_p]
@@ -91,6 +92,9 @@ class DeviceArray:
         assert other.nbytes == self.nbytes
         check(hip().hipMemcpy(self.ptr, other.ptr, self.nbytes, _D2D), "hipMemcpy D2D")
 
+    def zero(self):
+        check(hip().hipMemset(self.ptr, 0, self.nbytes), "hipMemset")
+
     def free(self):
         if getattr(self, "ptr", None):
             hip().hipFree(self.ptr)
@@ -124,6 +128,42 @@ class Event:
             hip().hipEventDestroy(self.e)
         except Exception:
             pass
+
+
+class Gate:
+    """Work that keeps a stream busy for a while: a fill of a large scratch buffer.  Launches
+    enqueued behind it pile up in the queue while it runs and then execute back to back, so a
+    short timed window measures the device and not the host's launch rate."""
+
+    def __init__(self, nbytes=1 << 30):
+        self.buf = DeviceArray(shape=(nbytes,), dtype=np.uint8)
+
+    def hold(self, stream, nbytes=None):
+        n = self.buf.nbytes if nbytes is None else min(int(nbytes), self.buf.nbytes)
+        check(hip().hipMemsetAsync(self.buf.ptr, 0, n, stream), "hipMemsetAsync")
+
+    def free(self):
+        self.buf.free()
+
+
+def timed_windows(enqueue, steps, stream, windows=9, gate=None, gate_bytes=None):
+    """Median over `windows` timed windows of `steps` launches each: (ms per step of the median
+    window, every window's ms per step).  enqueue(i) enqueues step i on `stream`; the window is
+    bracketed by HIP events recorded on that stream, behind `gate` when one is given."""
+    per = []
+    i = 0
+    for _ in range(windows):
+        e0, e1 = Event(), Event()
+        if gate is not None:
+            gate.hold(stream, gate_bytes)
+        e0.record(stream)
+        for _ in range(steps):
+            enqueue(i)
+            i += 1
+        e1.record(stream)
+        e1.synchronize()
+        per.append(e0.elapsed_ms(e1) / steps)
+    return float(np.median(per)), per
 
 
 class Graph:

@@ -87,3 +87,50 @@ def test_bench_refuses_more_than_one_gpu():
     assert r.returncode != 0
     assert "one GPU" in r.stderr
     assert r.stdout.strip() == ""
+
+
+def test_forget_returns_while_another_thread_holds_the_context_lock():
+    """nn.CopyForgetter.Forget "must not block on the device's own work" and may be called
+    from inside a page-in the device started (/root/reference/engine/nn/device.go:1570-1581).
+    The host-pointer entry points hold the context lock for their whole synchronous run; a
+    context bound to no device lets this be shown without a GPU: while another thread sits on
+    that lock, jl_forget returns at once, and the lock holder itself may call it too."""
+    import ctypes as C
+    import threading
+    import time
+    lib = _lib.load()
+    ctx = C.c_void_p()
+    opts = _lib.Options(-1, 32, None)
+    assert lib.jl_ctx_create(C.byref(ctx), C.byref(opts)) == _lib.OK and ctx.value
+    held, release, done = threading.Event(), threading.Event(), threading.Event()
+
+    def holder():
+        assert lib.jl_ctx_lock(ctx) == _lib.OK
+        buf = np.zeros(64, np.uint8)
+        assert lib.jl_forget(ctx, buf.ctypes.data, buf.nbytes) == _lib.OK   # same thread, lock held
+        held.set()
+        release.wait(30)
+        assert lib.jl_ctx_unlock(ctx) == _lib.OK
+        done.set()
+
+    th = threading.Thread(target=holder)
+    th.start()
+    assert held.wait(30)
+    buf = np.zeros(4096, np.uint8)
+    t0 = time.perf_counter()
+    for _ in range(1000):
+        assert lib.jl_forget(ctx, buf.ctypes.data, buf.nbytes) == _lib.OK
+    dt = time.perf_counter() - t0
+    assert not done.is_set(), "the holder released before the forgets returned"
+    assert dt < 1.0, f"1000 forgets took {dt:.3f} s with the context lock held elsewhere"
+    release.set()
+    th.join(30)
+    assert done.is_set()
+    assert lib.jl_resident_count(ctx) == 0        # takes the lock itself: free again, queue applied
+    # a context without a device fails every compute entry point loudly
+    out = np.zeros(4, np.float32)
+    w = np.zeros(144, np.uint8)
+    x = np.zeros(256, np.float32)
+    rc = lib.jl_matvec(ctx, out.ctypes.data, quant.Q4_K, w.ctypes.data, w.nbytes, x.ctypes.data, 1, 256)
+    assert rc < 0 and lib.jl_last_error(ctx)
+    lib.jl_ctx_destroy(ctx)
