@@ -13,9 +13,9 @@ Timing protocol (the reference's: warm calls, then the median of nine timed
 runs, perbyte_test.go:131-144): at least 200 untimed launches, then NINE timed
 windows of exactly --steps launches each, each window bracketed by HIP events
 on the launch stream; the reported step time is the median window's.  Every
-window is enqueued behind a fill of a scratch buffer, so its launches are
-already queued when the first one starts and a short window measures the
-device, not the host's launch rate.  Every section checks the output it timed
+window is enqueued behind a wait kernel (one wavefront watching the clock, no
+memory traffic), so its launches are already queued when the first one starts
+and a short window measures the device, not the host's launch rate.  Every section checks the output it timed
 against dequantize (on the device) + an f64 product on rows spread over the grid.
 
 Prints ONE JSON line.  `value` is algorithmic bytes per second (weight bytes +
@@ -85,13 +85,14 @@ def rel_err(got, want, what, bar=2e-2):
     return err
 
 
-def measure(dev, run, steps, gate, warm=3, windows=9, gate_bytes=256 << 20):
-    """warm untimed calls of run(i), then the median over nine windows of `steps` calls."""
+def measure(dev, run, steps, gate, warm=3, windows=9):
+    """warm untimed calls of run(i), then the median over nine windows of `steps` calls, each
+    window enqueued behind the gate."""
     from jitllm_amd.hipmem import timed_windows
     for i in range(warm):
         run(i)
     dev.synchronize()
-    ms, _ = timed_windows(run, steps, dev.stream, windows, gate, gate_bytes)
+    ms, _ = timed_windows(run, steps, dev.stream, windows, gate)
     return ms
 
 
@@ -161,9 +162,7 @@ class Workload:
             self.step(i)
         host_us = (time.perf_counter() - t0) * 1e6 / 64
         self.dev.synchronize()
-        # the gate covers the host's enqueue time of a window, up to ~1 GiB of fill
-        gate_bytes = min(1 << 30, max(64 << 20, int(steps * host_us * 1.5 * 3e6)))
-        ms, per = timed_windows(self.step, steps, self.dev.stream, 9, gate, gate_bytes)
+        ms, per = timed_windows(self.step, steps, self.dev.stream, 9, gate, host_us)
         synchronize()
         return ms, per, host_us
 
@@ -174,7 +173,7 @@ class Workload:
         for _ in range(50):
             self.step(0)
         self.dev.synchronize()
-        ms, _ = timed_windows(lambda i: self.step(0), steps, self.dev.stream, 9, gate, 64 << 20)
+        ms, _ = timed_windows(lambda i: self.step(0), steps, self.dev.stream, 9, gate)
         return ms
 
     def check(self):
@@ -647,7 +646,7 @@ def main():
     from jitllm_amd.hipmem import Gate
 
     dev = Device(device=0, act_window=256)
-    gate = Gate()
+    gate = Gate(dev)
     if args.gemm:
         ntok, nrows = (int(v) for v in args.gemm.split(","))
         print(json.dumps({"prefill_gemm": gemm_section(dev, gate, {nrows: (ntok,)})}), flush=True)
@@ -688,8 +687,9 @@ def main():
                                f"{head.ncopies} rotating weight copies ({head.ncopies * head.wbytes >> 20} MiB)",
                    "bytes_per_step": head.alg_bytes},
         "timing": {"protocol": f">= 200 untimed launches, then 9 timed windows of {args.steps} launches each, HIP events "
-                               "on the launch stream, each window enqueued behind a fill of a scratch buffer; "
-                               "ms_per_step is the median window",
+                               "on the launch stream, each window enqueued behind a wait kernel (one wavefront, no memory "
+                               "traffic) that lasts 1.5 x the host's enqueue time of the window, so the launches "
+                               "run back to back; ms_per_step is the median window",
                    "windows_us_per_step": [round(v * 1e3, 3) for v in per],
                    "host_enqueue_us_per_launch": round(host_us, 2)},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",

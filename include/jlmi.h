@@ -105,8 +105,11 @@ unsigned long long jl_launch_count(const jl_ctx *ctx);
 /* Measurement only; no counterpart in the reference.  What a single launch costs on this
  * machine before any arithmetic, so a kernel's time can be set beside it: kind 0 launches
  * an empty kernel, kind 1 a kernel that only reads nbytes of device memory at src (16-byte
- * aligned; every thread keeps eight 128-bit loads in flight) and stores nothing.  grid and
- * block <= 0 pick two 1024-thread workgroups per CU. */
+ * aligned; every thread keeps eight 128-bit loads in flight) and stores nothing; kind 2
+ * holds the stream for nbytes MICROSECONDS (<= 100000) on one wavefront that touches no
+ * memory -- a benchmark enqueues it in front of a timed window so that the window's
+ * launches are all queued before the first starts.  grid and block <= 0 pick two
+ * 1024-thread workgroups per CU (kinds 0 and 1). */
 int jl_probe_dev(jl_ctx *ctx, int kind, const void *src, size_t nbytes, int grid, int block,
                  void *stream);
 

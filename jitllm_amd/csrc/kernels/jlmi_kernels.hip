@@ -294,3 +294,10 @@ extern "C" __global__ __launch_bounds__(1024) void jl_probe_read(const u32x4* __
     if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x9e3779b9u && sink) sink[0] = acc.x;
 }
 extern "C" __global__ __launch_bounds__(1024) void jl_probe_empty(const u32x4* __restrict__, size_t, u32* __restrict__) {}
+// Holds the stream for `ticks` ticks of the 100 MHz constant clock and touches no memory: what a
+// benchmark enqueues in front of a timed window so that the window's launches are all queued
+// before the first one starts.  One wavefront; the wait is bounded by the clock, so it always ends.
+extern "C" __global__ __launch_bounds__(64) void jl_probe_wait(const u32x4* __restrict__, size_t ticks, u32* __restrict__) {
+    const uint64_t t0 = wall_clock64();
+    while (wall_clock64() - t0 < ticks) __builtin_amdgcn_s_sleep(8);
+}

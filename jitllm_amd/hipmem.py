@@ -33,6 +33,7 @@ def hip():
         h.hipEventCreate.argtypes = [C.POINTER(C.c_void_p)]
         h.hipEventRecord.argtypes = [C.c_void_p, C.c_void_p]
         h.hipEventSynchronize.argtypes = [C.c_void_p]
+        h.hipStreamSynchronize.argtypes = [C.c_void_p]
         h.hipEventElapsedTime.argtypes = [C.POINTER(C.c_float), C.c_void_p, C.c_void_p]
         h.hipEventDestroy.argtypes = [C.c_void_p]
         h.hipMemGetInfo.argtypes = [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]
@@ -131,31 +132,46 @@ class Event:
 
 
 class Gate:
-    """Work that keeps a stream busy for a while: a fill of a large scratch buffer.  Launches
-    enqueued behind it pile up in the queue while it runs and then execute back to back, so a
-    short timed window measures the device and not the host's launch rate."""
+    """Keeps a stream busy for a chosen time with the library's wait kernel (one wavefront
+    watching the constant clock, no memory traffic).  Launches enqueued behind it pile up in the
+    queue while it runs and then execute back to back, so a timed window measures the device
+    and not the host's launch rate."""
 
-    def __init__(self, nbytes=1 << 30):
-        self.buf = DeviceArray(shape=(nbytes,), dtype=np.uint8)
+    def __init__(self, dev):
+        self.dev = dev
 
-    def hold(self, stream, nbytes=None):
-        n = self.buf.nbytes if nbytes is None else min(int(nbytes), self.buf.nbytes)
-        check(hip().hipMemsetAsync(self.buf.ptr, 0, n, stream), "hipMemsetAsync")
+    def hold(self, stream, us):
+        """Keep `stream` busy for at least `us` microseconds."""
+        us = int(us) + 1
+        while us > 0:
+            self.dev.probe_dev(2, None, min(us, 100000), stream=stream)
+            us -= 100000
 
     def free(self):
-        self.buf.free()
+        pass
 
 
-def timed_windows(enqueue, steps, stream, windows=9, gate=None, gate_bytes=None):
+def timed_windows(enqueue, steps, stream, windows=9, gate=None, host_us=None):
     """Median over `windows` timed windows of `steps` launches each: (ms per step of the median
     window, every window's ms per step).  enqueue(i) enqueues step i on `stream`; the window is
-    bracketed by HIP events recorded on that stream, behind `gate` when one is given."""
-    per = []
+    bracketed by HIP events recorded on that stream.  With a gate, the window is enqueued
+    behind work that lasts 1.5 x the host's time to enqueue it (host_us per step, measured
+    here over 32 untimed steps when not given) plus 100 us, so the whole window is queued
+    before its first launch starts."""
+    import time
     i = 0
+    if gate is not None and host_us is None:
+        t0 = time.perf_counter()
+        for _ in range(32):
+            enqueue(i)
+            i += 1
+        host_us = (time.perf_counter() - t0) * 1e6 / 32
+        check(hip().hipStreamSynchronize(stream), "hipStreamSynchronize")
+    per = []
     for _ in range(windows):
         e0, e1 = Event(), Event()
         if gate is not None:
-            gate.hold(stream, gate_bytes)
+            gate.hold(stream, 1.5 * steps * host_us + 100.0)
         e0.record(stream)
         for _ in range(steps):
             enqueue(i)
