@@ -281,6 +281,21 @@ int jl_reserve(jl_ctx *ctx, int max_tok, int max_k);
  * afterwards and the call itself allocates nothing.  Returns what the call would. */
 int jl_reserve_shape(jl_ctx *ctx, int type, int nrows, int k, int ntok, int packed);
 
+/* jl_matmul_dev for callers that cannot allocate.  It has no counterpart in the reference:
+ * it exists for code under HIP graph capture, tight serving loops and harnesses that forbid
+ * hipMalloc.  Same operands, same values, same launches as jl_matmul_dev, but every
+ * workspace the call needs (activation fragments, K-split partial sums) is carved from ONE
+ * static device array of jl_static_scratch_bytes() bytes (32 MiB) that each GPU holds from
+ * library load to process exit; the call allocates nothing, frees nothing and waits for
+ * nothing.  A shape whose workspaces do not fit is refused with JL_ERR_NOMEM before
+ * anything is launched (jl_last_error says how many bytes it needed).  Every call on a GPU
+ * shares that GPU's array, which keeps the last call's contents: the kernels write all they
+ * read, so nothing needs clearing, but calls that OVERLAP on one GPU (two streams, two
+ * contexts, two threads) race on it -- order them on one stream. */
+int jl_matmul_static_dev(jl_ctx *ctx, float *out, int type, const void *w, const float *x,
+                         int nrows, int k, int ntok, void *stream);
+size_t jl_static_scratch_bytes(void);
+
 /* kernels.PackWeightsInto (jit/gpu/kernels/pack.go:52-199) on the device: GGUF
  * row-major blocks -> the three planes [unit][row] (sizes from jl_packed_words; sc may
  * be NULL for Q8_0).  Q4_K, Q6_K and Q8_0; the result is byte for byte the

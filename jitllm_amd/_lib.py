@@ -60,6 +60,8 @@ SIGNATURES = {
     "jl_matvec_packed_multi_dev": (_int, [_vp, _vp, _int, _vp, _vp, _vp, C.POINTER(C.c_int), _int, _vp, C.c_size_t,
                                           _vp, _vp, C.c_float, _vp, _vp, C.c_float, _vp, _int, _int, _int, _vp]),
     "jl_matmul_dev": (_int, [_vp, _vp, _int, _vp, _vp, _int, _int, _int, _vp]),
+    "jl_matmul_static_dev": (_int, [_vp, _vp, _int, _vp, _vp, _int, _int, _int, _vp]),
+    "jl_static_scratch_bytes": (_sz, []),
     "jl_reserve": (_int, [_vp, _int, _int]),
     "jl_packed_words": (_int, [_int, _int, _int, C.POINTER(_sz), C.POINTER(_sz), C.POINTER(_sz)]),
     "jl_matvec_packed": (_int, [_vp, _vp, _int, _vp, _vp, _vp, _int, _int, _vp, _int, _int]),

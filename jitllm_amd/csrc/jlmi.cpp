@@ -21,6 +21,7 @@
 
 #include "hip_api.h"
 #include "kernels/args.h"
+#include "scratch.h"
 
 namespace {
 
@@ -62,6 +63,13 @@ struct jl_ctx {
     std::vector<std::pair<uintptr_t, uintptr_t>> pending_forget;
     bool no_device = false;   // created with device < 0: host-side bookkeeping only
     bool dry_run = false;     // jl_reserve_shape: size the workspaces, launch nothing
+    // the static device array of scratch.hip on this context's device (null: the lookup
+    // failed and static_err says why), and the state of a call that lives on it
+    void* static_scratch = nullptr;
+    size_t static_scratch_bytes = 0;
+    std::string static_err;
+    bool no_alloc = false;    // jl_matmul_static_dev: workspaces are carved from the array
+    size_t static_used = 0;
     Tuning tune;
     int gemm_min_tok = 3;  // below this a per-token matvec loop is as fast (3.8 us a token against 8.9 us for up to 16)
     int num_cu = 0;
@@ -172,6 +180,17 @@ int launch(jl_ctx* c, const char* name, unsigned gx, unsigned gy, unsigned block
 // enough (jl_reserve, jl_reserve_shape).
 int grow(jl_ctx* c, void** buf, size_t* have, size_t need) {
     if (*have >= need) return JL_OK;
+    if (c->no_alloc) {
+        // a call that must not allocate: the next piece of the static array, or an error
+        const size_t off = (c->static_used + 255) & ~(size_t)255;
+        if (*have != 0 || off + need > c->static_scratch_bytes)
+            return fail(c, JL_ERR_NOMEM, "this shape needs %zu bytes of workspace beyond the %zu already taken; the static "
+                        "scratch holds %zu", need, off, c->static_scratch_bytes);
+        *buf = (char*)c->static_scratch + off;
+        *have = need;
+        c->static_used = off + need;
+        return JL_OK;
+    }
     if (*buf) {
         HIP_TRY(c, H->DeviceSynchronize());
         HIP_TRY(c, H->Free(*buf));
@@ -992,6 +1011,16 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
         return bail(JL_ERR_HIP, std::string("device is ") + prop.gcnArchName + ", this library is gfx950 only");
     c->num_cu = prop.multiProcessorCount;
     c->lds_limit = prop.sharedMemPerBlock;
+    {
+        // the static workspace's address on this device, looked up once per device with the
+        // device current; a failure only disables the entry point that lives on it
+        const char* why = "";
+        if (jl_static_scratch_get(c->device, &c->static_scratch, &c->static_scratch_bytes, &why) != 0) {
+            c->static_scratch = nullptr;
+            c->static_scratch_bytes = 0;
+            c->static_err = why;
+        }
+    }
     e = H->StreamCreate(&c->stream);
     if (e != hipSuccess) return bail(JL_ERR_HIP, std::string("hipStreamCreate: ") + H->GetErrorString(e));
     e = H->ModuleLoad(&c->module, path.c_str());
@@ -1226,6 +1255,38 @@ int jl_matmul_dev(jl_ctx* c, float* out, int type, const void* w, const float* x
     HIP_TRY(c, H->SetDevice(c->device));
     return matmul_launch(c, out, type, w, x, nrows, k, ntok, pick_stream(c, stream));
 }
+
+int jl_matmul_static_dev(jl_ctx* c, float* out, int type, const void* w, const float* x, int nrows, int k,
+                         int ntok, void* stream) {
+    if (!c) return JL_ERR_ARG;
+    HIP_TRY(c, H->SetDevice(c->device));
+    if (!c->static_scratch) return fail(c, JL_ERR_HIP, "the static scratch is not available: %s", c->static_err.c_str());
+    // The call runs jl_matmul_dev's own launch path with every context workspace set aside:
+    // whatever the path asks for is carved, in order, from the static array (grow() above), and
+    // a shape that needs more than the array holds is an error before anything is launched
+    // that would use the missing piece.  No hipMalloc, no hipFree, no synchronisation.
+    struct Saved { void** buf; size_t* have; void* b; size_t h; };
+    Saved saved[] = {{&c->gemm_ws, &c->gemm_ws_bytes, nullptr, 0}, {&c->w16_ws, &c->w16_ws_bytes, nullptr, 0},
+                     {&c->mx_ws, &c->mx_ws_bytes, nullptr, 0},     {&c->moe_q_ws, &c->moe_q_ws_bytes, nullptr, 0},
+                     {&c->unpack_ws, &c->unpack_ws_bytes, nullptr, 0}};
+    for (auto& s : saved) { s.b = *s.buf; s.h = *s.have; *s.buf = nullptr; *s.have = 0; }
+    // a dry run first: the sizes are checked against the array before the first real launch
+    c->no_alloc = true;
+    c->static_used = 0;
+    c->dry_run = true;
+    int rc = matmul_launch(c, out, type, w, x, nrows, k, ntok, pick_stream(c, stream));
+    c->dry_run = false;
+    if (rc == JL_OK) {
+        for (auto& s : saved) { *s.buf = nullptr; *s.have = 0; }
+        c->static_used = 0;
+        rc = matmul_launch(c, out, type, w, x, nrows, k, ntok, pick_stream(c, stream));
+    }
+    c->no_alloc = false;
+    for (auto& s : saved) { *s.buf = s.b; *s.have = s.h; }
+    return rc;
+}
+
+size_t jl_static_scratch_bytes(void) { return JL_STATIC_SCRATCH_BYTES; }
 
 int jl_packed_words(int type, int nrows, int k, size_t* nq, size_t* nd, size_t* nsc) {
     if (!nq || !nd || !nsc || nrows <= 0) return JL_ERR_ARG;

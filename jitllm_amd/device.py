@@ -260,6 +260,11 @@ class Device:
         return self._served(self._l.jl_matmul_dev(self._ctx, _ptr(out), t, _ptr(w), _ptr(x),
                                                   nrows, k, ntok, stream), "jl_matmul_dev")
 
+    def matmul_static_dev(self, out, t, w, x, nrows, k, ntok, stream=None):
+        """jl_matmul_dev on the library's static device workspace: allocates nothing."""
+        return self._served(self._l.jl_matmul_static_dev(self._ctx, _ptr(out), t, _ptr(w), _ptr(x),
+                                                         nrows, k, ntok, stream), "jl_matmul_static_dev")
+
     # -- mixture of experts -----------------------------------------------------
     def moe_logits_dev(self, logits, wtype, w, x, n_expert, k, ntok, stream=None):
         """Router logits [ntok][n_expert] = x [ntok][k] . W^T, W f32 (wtype 0) or f16 (1), in the
