@@ -18,6 +18,7 @@ int jlo_block_elems(int type) {
     switch (type) {
     case JLO_Q8_0: return 32;
     case JLO_Q4_K: return 256;
+    case JLO_Q5_K: return 256;
     case JLO_Q6_K: return 256;
     case JLO_MXFP4: return 32;
     }
@@ -27,6 +28,7 @@ int jlo_block_bytes(int type) {
     switch (type) {
     case JLO_Q8_0: return 34;
     case JLO_Q4_K: return 144;
+    case JLO_Q5_K: return 176;
     case JLO_Q6_K: return 210;
     case JLO_MXFP4: return 17;
     }
@@ -140,6 +142,43 @@ static void dequant_q4_k(const uint8_t *src, float *dst, size_t blocks) {
     }
 }
 
+/* format/quant/dequant.go:399-441.  Q4_K's scales; the fifth bit of element l of 64-group g
+ * is bit 2g (first half) / 2g+1 (second half) of qh[l]: the same 32 bytes serve all four
+ * groups.  Not a type of the matmul path: it is here because it is the one format with a
+ * secondary (high-bit) plane whose packed bytes the reference wrote into a fixture. */
+static void dequant_q5_k(const uint8_t *src, float *dst, size_t blocks) {
+    for (size_t b = 0; b < blocks; b++) {
+        const uint8_t *blk = src + b * 176;
+        float d = jlo_half_to_f32(rd16(blk));
+        float dmin = jlo_half_to_f32(rd16(blk + 2));
+        const uint8_t *scales = blk + 4, *qh = blk + 16, *qs = blk + 48;
+        float *out = dst + b * 256;
+        int o = 0, is = 0;
+        uint8_t u1 = 1, u2 = 2;
+        for (int j = 0; j < 256; j += 64) {
+            const uint8_t *ql = qs + j / 2;
+            uint8_t sc1, m1, sc2, m2;
+            scale_min_k4(is, scales, &sc1, &m1);
+            scale_min_k4(is + 1, scales, &sc2, &m2);
+            volatile float d1 = d * (float)sc1, min1 = dmin * (float)m1;
+            volatile float d2 = d * (float)sc2, min2 = dmin * (float)m2;
+            for (int l = 0; l < 32; l++) {
+                int32_t v = (ql[l] & 0xF) + ((qh[l] & u1) ? 16 : 0);
+                volatile float p = d1 * (float)v;
+                out[o++] = p - min1;
+            }
+            for (int l = 0; l < 32; l++) {
+                int32_t v = (ql[l] >> 4) + ((qh[l] & u2) ? 16 : 0);
+                volatile float p = d2 * (float)v;
+                out[o++] = p - min2;
+            }
+            is += 2;
+            u1 = (uint8_t)(u1 << 2);
+            u2 = (uint8_t)(u2 << 2);
+        }
+    }
+}
+
 /* format/quant/dequant.go:443-470.  (d*sc)*q, left to right in f32. */
 static void dequant_q6_k(const uint8_t *src, float *dst, size_t blocks) {
     for (size_t b = 0; b < blocks; b++) {
@@ -175,6 +214,7 @@ int jlo_dequant(int type, const uint8_t *src, float *dst, size_t n) {
     switch (type) {
     case JLO_Q8_0: dequant_q8_0(src, dst, blocks); return 0;
     case JLO_Q4_K: dequant_q4_k(src, dst, blocks); return 0;
+    case JLO_Q5_K: dequant_q5_k(src, dst, blocks); return 0;
     case JLO_Q6_K: dequant_q6_k(src, dst, blocks); return 0;
     case JLO_MXFP4: dequant_mxfp4(src, dst, blocks); return 0;
     }
@@ -198,6 +238,9 @@ static int qinfo_of(int type, qinfo *qi) {
         qi->signed_q = 1; return 0;
     case JLO_Q4_K:
         qi->bits = 4; qi->sub = 32; qi->bias_array = 1; qi->block_b = 144; qi->block_e = 256;
+        qi->per_super = 8; return 0;
+    case JLO_Q5_K:   /* a 4-bit primary plane plus a one-bit secondary plane, the two-plane form Q6_K uses */
+        qi->bits = 4; qi->hi = 1; qi->sub = 32; qi->bias_array = 1; qi->block_b = 176; qi->block_e = 256;
         qi->per_super = 8; return 0;
     case JLO_Q6_K:
         qi->bits = 4; qi->hi = 2; qi->sub = 16; qi->bias_k = 32; qi->block_b = 210;
@@ -295,6 +338,18 @@ static void extract(int type, const uint8_t *blk, int s, int32_t *q, uint16_t *d
         scale_min_k4(s, blk + 4, sc, m);
         const uint8_t *grp = blk + 16 + (s / 2) * 32;
         for (int l = 0; l < 32; l++) q[l] = (s % 2 == 0) ? (grp[l] & 0xF) : (grp[l] >> 4);
+        *dbits = rd16(blk);
+        *dminbits = rd16(blk + 2);
+        return;
+    }
+    case JLO_Q5_K: {   /* pack.go:332-349 */
+        scale_min_k4(s, blk + 4, sc, m);
+        const uint8_t *qh = blk + 16, *ql = blk + 48 + (s / 2) * 32;
+        for (int l = 0; l < 32; l++) {
+            int32_t v = (s % 2 == 1) ? (ql[l] >> 4) : (ql[l] & 0xF);
+            if (qh[l] & (1u << s)) v += 16;
+            q[l] = v;
+        }
         *dbits = rd16(blk);
         *dminbits = rd16(blk + 2);
         return;

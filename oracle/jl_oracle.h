@@ -10,12 +10,19 @@
  *   half codecs        all 65,536 patterns vs numpy float16
  *   dequant            libggml / gguf-py golden vectors held by the reference's
  *                      own tests (Q4_K, Q6_K, Q8_0, MXFP4), uint32 equality
- *   pack (Q4_K)        byte equality with planes written by the reference's
- *                      container writer (v29 fixture, k = 256)
+ *   pack (Q4_K, Q5_K)  byte equality with planes written by the reference's
+ *                      container writer (v29 fixture, k = 256): Q4_K pins the primary
+ *                      nibble plane, the D word and the 96-bit SC stream; Q5_K (kept in
+ *                      the oracle for this purpose only) pins the SECONDARY plane half of
+ *                      packSub -- byte pw*4 + (g/lanes)*4 + l%4, shift hi*(g%lanes) --
+ *                      which Q6_K shares with hi = 2, and its reader (RowPacked of the
+ *                      packed q5_k_tiny blocks == the libggml golden values)
  *   pack (Q6_K, Q8_0,  round trip RowPacked(pack(src)) == dequant(src) on the
  *         MXFP4)       golden blocks, an independently written numpy reader,
- *                      closed-form plane sizes; golden plane bytes do not
- *                      exist for these formats
+ *                      closed-form plane sizes.  What stays "parity unpinned"
+ *                      (held by reading pack.go only, no bytes the reference wrote):
+ *                      Q6_K's SC bytes (int8 + 128, four a word), Q8_0's D pairing
+ *                      (two rows' f16 a word), MXFP4's D bytes (e - 1, four rows a word)
  *   act quantizer      numpy float32 brute force incl. rounding-boundary cases
  *   matvec evaluators  brute force on hand-decoded blocks; agreement between
  *                      the three independent forms (f32 dequant + Neumaier,
@@ -41,7 +48,9 @@ extern "C" {
 #endif
 
 /* ggml type numbers, format/quant/types.go:14-55 */
-enum { JLO_Q8_0 = 8, JLO_Q4_K = 12, JLO_Q6_K = 14, JLO_MXFP4 = 39 };
+/* (Q5_K is not a type of the matmul path; it is here to pin the secondary-plane half of the
+ * packer against bytes the reference wrote, see the pinning table above) */
+enum { JLO_Q8_0 = 8, JLO_Q4_K = 12, JLO_Q5_K = 13, JLO_Q6_K = 14, JLO_MXFP4 = 39 };
 
 /* format/quant/types.go:61-85 */
 int jlo_block_elems(int type);

@@ -92,6 +92,73 @@ def test_pack_q4k_matches_planes_written_by_the_reference_writer():
     assert checked == 11  # token_embd, 2 attn_k, 2 banks x 4 sheets
 
 
+Q5_K = 13   # not a type of the matmul path: the one format whose secondary plane the reference wrote into a fixture
+
+
+def test_dequant_q5k_matches_libggml_golden():
+    """testdata/golden/dequant/q5_k_tiny of the reference (libggml on real weights): the oracle's
+    Q5_K decoder is only the yardstick for the packed reader below."""
+    src = np.fromfile(os.path.join(GOLDEN, "q5_k_tiny.in"), np.uint8)
+    want = np.fromfile(os.path.join(GOLDEN, "q5_k_tiny.f32"), np.uint32)
+    assert src.size == 32 * 176 and want.size == 8192
+    assert np.array_equal(oracle.dequant(Q5_K, src, want.size).view(np.uint32), want)
+
+
+def test_pack_q5k_secondary_plane_matches_planes_written_by_the_reference_writer():
+    """The secondary (high-bit) plane half of packSub
+    (/root/reference/jit/gpu/kernels/pack.go:229-235), which Q6_K shares with two bits a
+    weight, against bytes the reference's own writer produced: both attn_q tensors and the
+    eight exp_down_bank sheets of v29.jlm.gz are Q5_K (4-bit primary + 1-bit secondary plane,
+    D word, 96-bit SC stream) and must re-pack to the same bytes."""
+    from v29_source import source_tensors
+    from jitllm_amd import jlm
+    f = jlm.File.open(os.path.join(GOLDEN, "v29.jlm.gz"))
+    src = {(n, b): (kind, p) for n, b, kind, p in source_tensors()}
+    checked = 0
+    for e in f.entries:
+        kind, payload = src[(e.name, e.block)]
+        if kind != "q5k":
+            continue
+        assert e.type == 7                      # Q5S, /root/reference/format/jlm/schema.go:25-58
+        nq, nd, nsc = oracle.packed_words(Q5_K, e.rows, e.k)
+        assert (nq, nd, nsc) == (e.rows * 8 * 5, e.rows, e.rows * 3)
+        rb = e.rows * oracle.row_bytes(Q5_K, e.k)
+        for x in range(e.sheets):
+            x0 = x * f.exp_page_size if e.sheets > 1 else 0
+            qs = np.frombuffer(f.data, np.uint32, nq, e.qs_off + x0)
+            d = np.frombuffer(f.data, np.uint32, nd, e.d_off + x0)
+            sc = np.frombuffer(f.data, np.uint32, nsc, e.sc_off + x0)
+            mq, md, msc = oracle.pack_weights(Q5_K, payload[x * rb:(x + 1) * rb], e.rows, e.k)
+            assert np.array_equal(md, d) and np.array_equal(msc, sc)
+            # primary words 0..3 and the secondary word 4 of every sub-block, separately
+            mq5, qs5 = mq.reshape(-1, 5, e.rows), qs.reshape(-1, 5, e.rows)
+            assert np.array_equal(mq5[:, :4], qs5[:, :4]), "primary plane"
+            assert np.array_equal(mq5[:, 4], qs5[:, 4]), "secondary plane"
+            assert np.any(qs5[:, 4] != 0)
+            # and the reader of the secondary plane: the reference-written planes read back
+            # to what Dequant32 gives for the source blocks
+            for r in (0, e.rows - 1):
+                got = oracle.row_packed(Q5_K, qs, d, sc, r, e.rows, e.k)
+                want = oracle.dequant(Q5_K, payload[x * rb:(x + 1) * rb], e.rows * e.k)[r * e.k:(r + 1) * e.k]
+                assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+            checked += 1
+    assert checked == 10  # 2 attn_q, 2 banks x 4 sheets
+
+
+def test_row_packed_q5k_reads_the_golden_values_back():
+    """pack -> RowPacked over the libggml golden blocks (k = 512: two super-blocks a row, so the
+    cross-super strides the k = 256 fixture cannot show are exercised) gives the golden bits:
+    writer and reader of the secondary plane agree with each other AND with libggml."""
+    src = np.fromfile(os.path.join(GOLDEN, "q5_k_tiny.in"), np.uint8)
+    want = np.fromfile(os.path.join(GOLDEN, "q5_k_tiny.f32"), np.uint32)
+    for k in (256, 512, 2048):
+        nrows = 8192 // k
+        qs, d, sc = oracle.pack_weights(Q5_K, src, nrows, k)
+        for r in range(nrows):
+            got = oracle.row_packed(Q5_K, qs, d, sc, r, nrows, k)
+            assert np.array_equal(got.view(np.uint32), want[r * k:(r + 1) * k]), (k, r)
+
+
 def test_packed_words_closed_form():
     """Bytes per 256 weights: Q4_K 144 (= GGUF), Q6_K 212, Q8_0 8*34, MXFP4 8*17
     (/root/reference/internal/oracle/packed_test.go:177-213)."""
