@@ -88,7 +88,7 @@ int jl_synchronize(jl_ctx *ctx);
 
 /* Kernel-shape overrides for measurement: key is one of "matvec.rpw" (rows per
  * wavefront: 1, 2, 4), "matvec.block" (threads per workgroup), "matvec.grid"
- * (workgroups), "gemm.min_tok" (fewest tokens sent to the matrix-core GEMM),
+ * (workgroups), "matvec.pipe" (1: the row loop as a two-deep load pipeline), "gemm.min_tok" (fewest tokens sent to the matrix-core GEMM),
  * "packed.rw" (rows per wavefront of the packed-plane matvec: 16, 32, 64),
  * "packed.block" (its threads per workgroup), "moe.shares" (row shares an expert's
  * matrix is split into), "gemm.rows" (rows per workgroup of the GEMM: 64 or 128), "mxfp4.split" (workgroups along

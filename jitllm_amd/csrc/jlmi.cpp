@@ -29,7 +29,7 @@ thread_local std::string g_create_error;
 const HipApi* H = nullptr;  // the process-wide HIP runtime, resolved by the first jl_ctx_create
 
 struct Tuning {
-    int rpw = 0, block = 0, grid = 0;
+    int rpw = 0, block = 0, grid = 0, pipe = 0;
     int packed_rw = 0, packed_block = 0, moe_group = 0, moe_logits = 0, moe_q6k_cols = 0;
     int moe_shares = 0;
     int gemm_rows = 0;
@@ -235,12 +235,14 @@ int matvec_launch(jl_ctx* c, float* out, int type, const void* w, const float* x
     if (rpw <= 0) rpw = 1;
     if (rpw != 1 && rpw != 2 && rpw != 4) return fail(c, JL_ERR_ARG, "matvec: rpw=%d", rpw);
     const bool small = nrows <= 16 * c->num_cu;
-    if (block <= 0) block = (small || type == JL_TYPE_Q6_K) ? 1024 : 768;
+    // (Q4_K 14336 x 4096: one 16-wavefront workgroup a CU 8.1 us, two of twelve 8.6)
+    const bool one_per_cu = small || type == JL_TYPE_Q6_K || type == JL_TYPE_Q4_K;
+    if (block <= 0) block = one_per_cu ? 1024 : 768;
     if (block % 64 != 0 || block > 1024) return fail(c, JL_ERR_ARG, "matvec: block=%d", block);
     if (block > matvec_max_block(type, rpw)) block = matvec_max_block(type, rpw);
     const int rows_per_block = (block / 64) * rpw;
     long groups = ((long)nrows + rows_per_block - 1) / rows_per_block;
-    long grid = c->tune.grid > 0 ? c->tune.grid : (long)c->num_cu * 2;
+    long grid = c->tune.grid > 0 ? c->tune.grid : (long)c->num_cu * (type == JL_TYPE_Q4_K && !small ? 1 : 2);
     if (grid > groups) grid = groups;
     if (grid < 1) grid = 1;
 
@@ -257,6 +259,10 @@ int matvec_launch(jl_ctx* c, float* out, int type, const void* w, const float* x
     a.per = c->act_window / 32;
     a.nwaves = block / 64;
     a.ngroups = (int)grid;
+    // the two-deep pipeline of the row loop ("matvec.pipe" = 1) measured slower than the plain
+    // loop on this machine (Q8_0 14336 x 4096: 17.4 against 15.7 us; Q6_K 4096 x 14336: 15.1
+    // against 14.2), so it stays off unless asked for
+    a.pipe = c->tune.pipe == 1 ? 1 : 2;
     char name[64];
     snprintf(name, sizeof name, "jl_matvec_%s_r%d", ti->tag, rpw);
     void* params[] = {&a};
@@ -1122,6 +1128,7 @@ int jl_set_tuning(jl_ctx* c, const char* key, int value) {
     if (!strcmp(key, "matvec.rpw")) c->tune.rpw = value;
     else if (!strcmp(key, "matvec.block")) c->tune.block = value;
     else if (!strcmp(key, "matvec.grid")) c->tune.grid = value;
+    else if (!strcmp(key, "matvec.pipe")) c->tune.pipe = value;
     else if (!strcmp(key, "packed.rw")) c->tune.packed_rw = value;
     else if (!strcmp(key, "packed.block")) c->tune.packed_block = value;
     else if (!strcmp(key, "moe.group")) c->tune.moe_group = value;

@@ -16,6 +16,7 @@ struct MatVecArgs {
     int per;             // activation window / 32 (fused form)
     int nwaves;          // wavefronts per workgroup (the launch's block / 64)
     int ngroups;         // workgroups (the launch's grid)
+    int pipe;            // 2: the plain row loop; else the two-deep pipeline where a wavefront has several steps
 };
 
 // Several decode matvecs of one type in one launch (grid y = matrix): matrix i computes

@@ -263,8 +263,10 @@ __device__ __forceinline__ void load_w_q6k(const uint8_t* row, int slot, SlotWQ6
     w.qla = ld16_a2(blk + n * 64 + j * 16);
     w.qlb = ld16_a2(blk + n * 64 + 32 + j * 16);
     w.qh = ld16_a2(blk + 128 + n * 32 + j * 16);
-    const uint8_t* sc = blk + 192 + n * 8 + j;
-    w.sc = (u32)sc[0] | ((u32)sc[2] << 8) | ((u32)sc[4] << 16) | ((u32)sc[6] << 24);
+    // the half's eight int8 scales in one load; bytes j, j+2, j+4, j+6 are this slot's
+    const u32x2 s8 = ld8_a2(blk + 192 + n * 8);
+    const u32 lo = (s8.x >> (8 * j)) & 0x00FF00FFu, hi = (s8.y >> (8 * j)) & 0x00FF00FFu;
+    w.sc = (lo & 0xFF) | ((lo >> 8) & 0xFF00) | ((hi & 0xFF) << 16) | ((hi >> 16) << 24);
     w.d = ld2(blk + 208);
 }
 
@@ -344,6 +346,94 @@ template <> struct SlotTraits<JL_Q6_K> {
 };
 
 
+// The row loop of one wavefront: rows r0, r0 + group_stride, ... (RPW at a time), each row's
+// slots dealt to the lanes in chunks of 64.  w holds the first step's weights, loaded by the
+// caller before the activation was staged.  Two forms: the plain loop (each step's loads are
+// issued when the step begins; the dozen or so wavefronts of a CU cover each other's
+// latency), and a two-deep pipeline (`pipe`: the next step's weight loads are issued BEFORE
+// the current step's dot products, into the other of two register sets; unconditional loads
+// with clamped addresses, so the compiler's wait counts stay exact).  On MI355X the plain
+// loop measured faster for every type but Q4_K, where they tie: more loads in flight per
+// wavefront do not help a kernel that is not waiting on latency.
+// store(row, total) receives a finished row in lane 63.
+template <int TYPE, int RPW, class Store>
+__device__ __forceinline__ void matvec_rows(const uint8_t* w0, int row_bytes, const ActLds& A, int nrows, int r0,
+                                            int group_stride, int nslots, int lane,
+                                            typename SlotTraits<TYPE>::W (&w)[RPW], Store store, bool pipe) {
+    typedef SlotTraits<TYPE> T;
+    if (r0 >= nrows) return;   // wavefront-uniform
+    const int nper = (nslots + 63) >> 6;                             // steps per row group
+    const int ngrp = (nrows - r0 + group_stride - 1) / group_stride;   // row groups of this wavefront
+    float acc[RPW];
+#pragma unroll
+    for (int j = 0; j < RPW; j++) acc[j] = 0.f;
+    if (ngrp * nper == 1 || !pipe) {
+        // a single step (a matrix that fits the grid, every row one chunk): nothing to overlap;
+        // or the plain loop, each step's loads issued when the step begins
+        bool preloaded = true;
+        for (; r0 < nrows; r0 += group_stride) {
+            for (int slot = lane; slot < nslots; slot += 64) {
+                if (!preloaded) {
+#pragma unroll
+                    for (int j = 0; j < RPW; j++)
+                        T::load_w(w0 + (size_t)min(r0 + j, nrows - 1) * row_bytes, slot, w[j]);
+                }
+                preloaded = false;
+                typename T::Act a;
+                T::load_act(A, slot, a);
+#pragma unroll
+                for (int j = 0; j < RPW; j++) acc[j] += T::dot(w[j], slot, a);
+            }
+            preloaded = false;
+#pragma unroll
+            for (int j = 0; j < RPW; j++) {
+                const float t = wave_sum_to_lane63(acc[j]);
+                if (lane == 63 && r0 + j < nrows) store(r0 + j, t);
+                acc[j] = 0.f;
+            }
+        }
+        return;
+    }
+    typename T::W wb[RPW];
+    int g = 0, sidx = 0;   // the current step: row group g of this wavefront, chunk sidx of its slots
+    auto step = [&](typename T::W (&wc)[RPW], typename T::W (&wn)[RPW]) __attribute__((always_inline)) {
+        int gn = g, sn = sidx + 1;
+        if (sn == nper) { sn = 0; gn++; }
+        {
+            const int rn = r0 + min(gn, ngrp - 1) * group_stride;
+            const int slot_n = min(lane + 64 * sn, nslots - 1);
+#pragma unroll
+            for (int j = 0; j < RPW; j++) T::load_w(w0 + (size_t)min(rn + j, nrows - 1) * row_bytes, slot_n, wn[j]);
+        }
+        const int slot = lane + 64 * sidx;
+        const bool live = slot < nslots;
+        const int sl = min(slot, nslots - 1);
+        typename T::Act a;
+        T::load_act(A, sl, a);
+#pragma unroll
+        for (int j = 0; j < RPW; j++) {
+            const float v = T::dot(wc[j], sl, a);
+            acc[j] += live ? v : 0.f;
+        }
+        if (sn == 0) {   // the row group's last chunk
+            const int r = r0 + g * group_stride;
+#pragma unroll
+            for (int j = 0; j < RPW; j++) {
+                const float t = wave_sum_to_lane63(acc[j]);
+                if (lane == 63 && r + j < nrows) store(r + j, t);
+                acc[j] = 0.f;
+            }
+        }
+        g = gn;
+        sidx = sn;
+    };
+    const int nsteps = ngrp * nper;
+    for (int i = 0; i < nsteps; i += 2) {
+        step(w, wb);
+        if (i + 1 < nsteps) step(wb, w);
+    }
+}
+
 // One wavefront computes RPW rows at a time and strides over the row groups of
 // a persistent grid.  The first group's weight loads are issued before the
 // activation is staged, so HBM latency overlaps the quantizer; after that each
@@ -381,30 +471,8 @@ __device__ __forceinline__ void matvec_body(const MatVecArgs& p, uint8_t* smem) 
     else stage_act_copy(smem, p.q, p.as, p.s16, p.k, nwaves * 64);
     lds_barrier();   // orders the LDS staging only: the weight loads stay in flight
 
-    bool preloaded = true;
-    for (; r0 < p.nrows; r0 += group_stride) {
-        float acc[RPW];
-#pragma unroll
-        for (int j = 0; j < RPW; j++) acc[j] = 0.f;
-        for (int slot = lane; slot < nslots; slot += 64) {
-            if (!preloaded) {
-#pragma unroll
-                for (int j = 0; j < RPW; j++)
-                    T::load_w(p.w + (size_t)min(r0 + j, p.nrows - 1) * p.row_bytes, slot, w[j]);
-            }
-            preloaded = false;
-            typename T::Act a;
-            T::load_act(A, slot, a);
-#pragma unroll
-            for (int j = 0; j < RPW; j++) acc[j] += T::dot(w[j], slot, a);
-        }
-        preloaded = false;
-#pragma unroll
-        for (int j = 0; j < RPW; j++) {
-            float t = wave_sum_to_lane63(acc[j]);
-            if (lane == 63 && r0 + j < p.nrows) p.out[r0 + j] = t;
-        }
-    }
+    matvec_rows<TYPE, RPW>(p.w, p.row_bytes, A, p.nrows, r0, group_stride, nslots, lane, w,
+                           [&](int r, float t) { p.out[r] = t; }, p.pipe != 2);
 }
 
 // Several matvecs of one type in one launch: grid = (row groups, matrices).  Each
@@ -449,8 +517,8 @@ __device__ __forceinline__ void matvec_multi_body(const MatVecMultiArgs& p, uint
     f32x4 x0 = ((const f32x4*)x)[min((int)threadIdx.x, n4 - 1)];
     f32x4 u0 = x2 ? ((const f32x4*)x2)[min((int)threadIdx.x, n4 - 1)] : f32x4{1.f, 1.f, 1.f, 1.f};
     __builtin_amdgcn_s_barrier();   // activation loads of the whole workgroup go out first
-    typename T::W w;
-    T::load_w(w0 + (size_t)min(r0, nrows - 1) * row_bytes, min(lane, nslots - 1), w);
+    typename T::W w[1];
+    T::load_w(w0 + (size_t)min(r0, nrows - 1) * row_bytes, min(lane, nslots - 1), w[0]);
     // RMSNorm ahead of the quantizer (the reference's RMSNormQuantRows, jit/gpu/kernels/
     // elem.go:252-267, with its host arithmetic, internal/oracle/oracle.go:230-240): the sum
     // of squares in f64, scale = 1/sqrt(sum/k + eps), y = f32(f64(x) * scale * f64(w)).
@@ -488,21 +556,10 @@ __device__ __forceinline__ void matvec_multi_body(const MatVecMultiArgs& p, uint
     }
     lds_barrier();
 
-    bool preloaded = true;
-    for (; r0 < nrows; r0 += group_stride) {
-        float acc = 0.f;
-        for (int slot = lane; slot < nslots; slot += 64) {
-            if (!preloaded) T::load_w(w0 + (size_t)r0 * row_bytes, slot, w);
-            preloaded = false;
-            typename T::Act a;
-            T::load_act(A, slot, a);
-            acc += T::dot(w, slot, a);
-        }
-        preloaded = false;
-        const float t = wave_sum_to_lane63(acc);
-        if (lane == 63) {
-            p.out[y][r0] = t;
-            if (y == 0 && p.resid) p.resid[r0] += resid_weight(p.alpha, p.resid_gate) * t;
-        }
-    }
+    float* const outp = p.out[y];
+    float* const resid = y == 0 ? p.resid : nullptr;
+    matvec_rows<TYPE, 1>(w0, row_bytes, A, nrows, r0, group_stride, nslots, lane, w, [&](int r, float t) {
+        outp[r] = t;
+        if (resid) resid[r] += resid_weight(p.alpha, p.resid_gate) * t;
+    }, false);
 }
