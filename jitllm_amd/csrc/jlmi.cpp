@@ -36,6 +36,7 @@ struct Tuning {
     int gemm_form = 0;
     int gemm_split = 0;
     int gemm_prep = 0;
+    int gemm_planes = 0;
     int moe_form = 0;
     int moe_waves = 0;
     int moe_lpr = 0;
@@ -421,13 +422,31 @@ int gemm_q4k_w16_launch(jl_ctx* c, float* out, const void* w, const uint16_t* bq
 // kernel; 2 = 256-token x 128-row tiles, a wavefront across all 128 rows (least L1 traffic
 // per matrix instruction, for grids that still fill the chip); 3 = weights expanded once
 // per call into f16 fragments, then 128 x 64 tiles.
+struct PlaneRef {
+    const uint32_t *qs, *d, *sc;
+    int row, stride;
+};
+
 constexpr int kGemmWideTok = 256;
 constexpr unsigned kGemmWideLdsBytes = 2u * 128u * 136u * 2u + 2u * 128u * 24u * 2u + 2u * 128u * 2u * 4u + 2u * kGemmWideTok * 4u;   // JL_GEMM_WIDE_LDS_BYTES
 
+// Few tokens, or a grid of at most a round and a half of 32-row workgroups: the forms that
+// take a lane's operand words straight from GGUF rows (no plane form of them exists).
+bool gemm_q4k_few_applies(const jl_ctx* c, int nrows, int k, int ntok) {
+    const int form = c->tune.gemm_form;
+    if ((size_t)nrows * (size_t)(k / 256) * 144 >= ((size_t)1 << 32)) return false;
+    if ((form == 0 || form == 4) && ntok <= 64) return true;
+    const long few32_groups = (long)((nrows + 31) / 32) * ((ntok + 63) / 64);
+    return ((form == 0 && 2 * few32_groups <= 3L * c->num_cu) || (form == 5 && ntok <= 1024)) && ntok > 64;
+}
+
+// pl: the weights as packed planes (w unused): the tiled forms read them where they lie.  The
+// caller has checked that gemm_q4k_few_applies() is false.
 int gemm_q4k_launch(jl_ctx* c, float* out, const void* w, const float* x, int nrows, int k, int ntok,
-                    hipStream_t st) {
+                    hipStream_t st, const PlaneRef* pl = nullptr) {
     int form = c->tune.gemm_form;
-    if ((form == 0 || form == 4) && ntok <= 64 && (size_t)nrows * (size_t)(k / 256) * 144 < ((size_t)1 << 32)) {
+    if (pl && form == 3) form = 0;
+    if (!pl && (form == 0 || form == 4) && ntok <= 64 && (size_t)nrows * (size_t)(k / 256) * 144 < ((size_t)1 << 32)) {
         // few tokens: 16-row workgroups that split K over their wavefronts, one launch after
         // the activation prep (kernels/gemm_q4k.h, "few tokens")
         const int tok_pad = (ntok + 31) / 32 * 32, nsb = k / 256, nt = (ntok + 15) / 16;
@@ -450,7 +469,7 @@ int gemm_q4k_launch(jl_ctx* c, float* out, const void* w, const float* x, int nr
         return launch(c, name, (unsigned)((nrows + 15) / 16), 1, 512, 0, st, gp);
     }
     const long few32_groups = (long)((nrows + 31) / 32) * ((ntok + 63) / 64);
-    if (((form == 0 && 2 * few32_groups <= 3L * c->num_cu) || (form == 5 && ntok <= 1024)) && ntok > 64 &&
+    if (!pl && ((form == 0 && 2 * few32_groups <= 3L * c->num_cu) || (form == 5 && ntok <= 1024)) && ntok > 64 &&
         (size_t)nrows * (size_t)(k / 256) * 144 < ((size_t)1 << 32)) {
         // some more tokens, few enough rows: the same scheme on 32-row x 64-token workgroups,
         // one to a CU, while the grid is at most a round and a half (4096 rows: up to 192
@@ -493,11 +512,13 @@ int gemm_q4k_launch(jl_ctx* c, float* out, const void* w, const float* x, int nr
     // is the kernel's length (whole matmul, 512 tokens x 4096 rows: 41.0 -> 39.7 us; 2048 tokens:
     // 87.1 -> 83.4; "gemm.prep" = 4 asks for four wavefronts)
     const bool prep16 = c->tune.gemm_prep != 4;
-    rc = launch(c, prep16 ? "jl_gemm_prep_q4k_w16" : "jl_gemm_prep_q4k", (unsigned)nsb, (unsigned)(tok_pad / 32),
-                prep16 ? 1024 : 256, 0, st, pp);
+    // (the plane kernels take the activations in the planes' K order: their own prep)
+    rc = launch(c, pl ? "jl_gemm_prep_q4k_planes" : prep16 ? "jl_gemm_prep_q4k_w16" : "jl_gemm_prep_q4k", (unsigned)nsb,
+                (unsigned)(tok_pad / 32), pl || prep16 ? 1024 : 256, 0, st, pp);
     if (rc != JL_OK) return rc;
     if (form == 3) return gemm_q4k_w16_launch(c, out, w, bq, da, nrows, k, ntok, tok_pad, st);
     GemmArgs ga;
+    if (pl) { ga.pqs = pl->qs; ga.pd = pl->d; ga.psc = pl->sc; ga.prow0 = pl->row; ga.pstride = pl->stride; }
     ga.out = out; ga.w = (const uint8_t*)w; ga.bq = bq; ga.da = da;
     ga.nrows = nrows; ga.k = k; ga.ntok = ntok; ga.tok_pad = tok_pad; ga.row_bytes = nsb * 144;
     ga.out_stride = nrows; ga.sb_per = 0;
@@ -512,15 +533,18 @@ int gemm_q4k_launch(jl_ctx* c, float* out, const void* w, const float* x, int nr
         long nrt_wide = nrt;
         if (c->tune.gemm_form == 0 && full >= 1 && rem > 0 && 2 * rem <= c->num_cu) nrt_wide = full * c->num_cu / ntt;
         ga.nrows = nrt_wide == nrt ? nrows : (int)(nrt_wide * 128);
-        rc = launch(c, "jl_gemm_q4k_wide", (unsigned)ntt, (unsigned)nrt_wide, 512, kGemmWideLdsBytes, st, gp);
+        rc = launch(c, pl ? "jl_gemm_q4k_wide_planes" : "jl_gemm_q4k_wide", (unsigned)ntt, (unsigned)nrt_wide, 512,
+                    kGemmWideLdsBytes, st, gp);
         rows_left = nrows - ga.nrows;
         if (rc != JL_OK || rows_left == 0) return rc;
-        ga.w += (size_t)ga.nrows * ga.row_bytes;
+        if (pl) ga.prow0 += ga.nrows;
+        else ga.w += (size_t)ga.nrows * ga.row_bytes;
         ga.out += ga.nrows;
         ga.nrows = rows_left;
     }
     // 64-row workgroups, two to a CU, unless asked for the 128-row form
-    const int rows = c->tune.gemm_rows == 128 ? 128 : 64;
+    const int rows = c->tune.gemm_rows == 128 && !pl ? 128 : 64;
+    const char* const r64 = pl ? "jl_gemm_q4k_r64_planes" : "jl_gemm_q4k_r64";
     if (rows == 64 && rows_left == nrows) {
         // a grid that leaves most of the chip idle (few tokens) is widened along K
         const long groups = (long)(tok_pad / kGemmTile) * ((nrows + 63) / 64);
@@ -535,7 +559,7 @@ int gemm_q4k_launch(jl_ctx* c, float* out, const void* w, const float* x, int nr
             rc = ws_ensure(c, &c->mx_ws, &c->mx_ws_bytes, n * nsplit * 4);
             if (rc != JL_OK) return rc;
             ga.out = (float*)c->mx_ws; ga.sb_per = per;
-            rc = launch(c, "jl_gemm_q4k_r64", (unsigned)(tok_pad / kGemmTile), (unsigned)((nrows + 63) / 64), 256,
+            rc = launch(c, r64, (unsigned)(tok_pad / kGemmTile), (unsigned)((nrows + 63) / 64), 256,
                         gemm_lds_bytes(64), st, gp, (unsigned)nsplit);
             if (rc != JL_OK) return rc;
             SumPartsArgs sa;
@@ -544,7 +568,7 @@ int gemm_q4k_launch(jl_ctx* c, float* out, const void* w, const float* x, int nr
             return launch(c, "jl_sum_parts", (unsigned)((n + 255) / 256), 1, 256, 0, st, sp);
         }
     }
-    return launch(c, rows == 128 ? "jl_gemm_q4k_r128" : "jl_gemm_q4k_r64", (unsigned)(tok_pad / kGemmTile),
+    return launch(c, rows == 128 ? "jl_gemm_q4k_r128" : r64, (unsigned)(tok_pad / kGemmTile),
                   (unsigned)((rows_left + rows - 1) / rows), rows == 128 ? 512 : 256, gemm_lds_bytes(rows), st, gp);
 }
 
@@ -705,11 +729,6 @@ bool packed_words(int type, size_t nrows, int k, size_t* nq, size_t* nd, size_t*
     return false;
 }
 
-struct PlaneRef {
-    const uint32_t *qs, *d, *sc;
-    int row, stride;
-};
-
 int packed_check(jl_ctx* c, int type, const PlaneRef& pl, int nrows, int k, const TypeInfo** ti) {
     *ti = type_info(type);
     if (!*ti) return JL_DECLINED;
@@ -831,6 +850,10 @@ int packed_matmul_launch(jl_ctx* c, float* out, int type, const PlaneRef& pl, co
     const bool gemm32 = (type == JL_TYPE_Q8_0 || type == JL_TYPE_Q6_K || type == JL_TYPE_Q4_K) && c->act_window == 32 &&
                         ntok >= c->gemm_min_tok && c->tune.gemm_form != 9 && k % 128 == 0 && ntok <= 65535 * 4 &&
                         (nrows + 63) / 64 <= 65535 && gemm32_lds_bytes(2) <= c->lds_limit && k / 32 <= 65535;
+    // Q4_K with the k-quant window: the tiled forms read the planes where they lie; only the
+    // few-token forms, which take a lane's operand words straight from GGUF rows, restore rows first
+    if (gemm && c->tune.gemm_planes != 2 && !gemm_q4k_few_applies(c, nrows, k, ntok) && (size_t)pl.stride * 4 < ((size_t)1 << 31))
+        return gemm_q4k_launch(c, out, nullptr, x, nrows, k, ntok, st, &pl);
     if (gemm || gemm6 || gemm32) {
         rc = ws_ensure(c, &c->unpack_ws, &c->unpack_ws_bytes, (size_t)nrows * (size_t)(k / ti->block_elems) * ti->block_bytes);
         if (rc != JL_OK) return rc;
@@ -1039,7 +1062,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     if (e != hipSuccess)
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
-    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_group2_wide", "jl_moe_quant", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_q4k", "jl_moe_gemm_r64", "jl_moe_gemm_q6k_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_sum_parts", "jl_probe_read", "jl_probe_empty", "jl_probe_wait",
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_prep_q4k_planes", "jl_gemm_q4k_r64_planes", "jl_gemm_q4k_wide_planes", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_group2_wide", "jl_moe_quant", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_q4k", "jl_moe_gemm_r64", "jl_moe_gemm_q6k_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_sum_parts", "jl_probe_read", "jl_probe_empty", "jl_probe_wait",
                                       "jl_pack_weights", "jl_unpack_q4k", "jl_unpack_q6k", "jl_unpack_q8_0"};
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int rw : {16, 32, 64})
@@ -1150,6 +1173,7 @@ int jl_set_tuning(jl_ctx* c, const char* key, int value) {
     else if (!strcmp(key, "gemm.form")) c->tune.gemm_form = value;
     else if (!strcmp(key, "gemm.split")) c->tune.gemm_split = value;
     else if (!strcmp(key, "gemm.prep")) c->tune.gemm_prep = value;
+    else if (!strcmp(key, "gemm.planes")) c->tune.gemm_planes = value;
     else if (!strcmp(key, "gemm.min_tok")) c->gemm_min_tok = value > 0 ? value : 3;
     else return fail(c, JL_ERR_ARG, "unknown tuning key %s", key);
     return JL_OK;

@@ -63,6 +63,13 @@ struct GemmArgs {
     int out_stride;      // floats between tokens in out
     int sb_per;          // K split: super-blocks per blockIdx.z (0 = whole K), out = slab z of [gridDim.z][ntok][out_stride]
     const float* dsum = nullptr;   // window 32, Q4_K: the prep's d_a * block sums
+    // the weights as packed planes (the kernels' plane forms; w is unused then): QS, D and SC
+    // planes of a buffer of pstride rows, this launch's first row at prow0 (nrows counted from
+    // it), its first super-block psb0 (a K split moves it)
+    const uint32_t* pqs = nullptr;
+    const uint32_t* pd = nullptr;
+    const uint32_t* psc = nullptr;
+    int prow0 = 0, pstride = 0, psb0 = 0;
 };
 
 // Mixture block on the matrix cores (Q4_K, activation window 256).  An expert's columns are

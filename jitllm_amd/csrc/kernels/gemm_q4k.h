@@ -77,7 +77,12 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 // does not exist.  grp of ngrp groups; da is laid [nsb][32*ngrp].
 // NW wavefronts a workgroup (4, or 16 where few tokens make the grid small and the chain of
 // tokens a wavefront quantizes one after the other is the kernel's length).
-template <int NW, class Load>
+// PL: the K order of the plane-reading kernels.  There a 32-bit word of nibbles holds eight
+// weights of ONE sub-block (byte b of word w: element 4w+b in the low nibble, element 4w+b+16
+// in the high nibble, jit/gpu/kernels/pack.go:210-239), so vector v = 2*ks + kg of a stage is
+// word v%4 of the stage's sub-block v/4, and its eight values pair with the activations of
+// elements 4w + (0, 2, 16, 18, 1, 3, 17, 19) of that sub-block.
+template <int NW, bool PL = false, class Load>
 __device__ __forceinline__ void gemm_prep_group(u32* lds, int sb, int grp, int ngrp, uint16_t* bqp, float* dap,
                                                 Load load) {
     constexpr int TPW = 32 / NW, FPW = 16 / NW;   // tokens and fragments per wavefront
@@ -109,8 +114,16 @@ __device__ __forceinline__ void gemm_prep_group(u32* lds, int sb, int grp, int n
         const int pi = wave * FPW + i, h = pi >> 3, ks = pi & 7;
         // vector (group g, word c): low nibbles' partners are elements 4c.. of sub-block 2g,
         // high nibbles' partners the same elements of sub-block 2g+1
-        const int g = 2 * h + (ks >> 2), c = 2 * (ks & 3) + kg;
-        const u32 lo = sq[tl * 65 + 16 * g + c], hi = sq[tl * 65 + 16 * g + 8 + c];
+        u32 lo, hi;
+        if (PL) {
+            const int v = 2 * ks + kg, sub = 4 * h + (v >> 2), w = v & 3;
+            lo = sq[tl * 65 + 8 * sub + w];
+            hi = sq[tl * 65 + 8 * sub + 4 + w];
+        } else {
+            const int g = 2 * h + (ks >> 2), c = 2 * (ks & 3) + kg;
+            lo = sq[tl * 65 + 16 * g + c];
+            hi = sq[tl * 65 + 16 * g + 8 + c];
+        }
         auto f = [](u32 w, int b) { return (_Float16)(float)(int8_t)(w >> (8 * b)); };
         const f16x8 o = {f(lo, 0), f(lo, 2), f(hi, 0), f(hi, 2), f(lo, 1), f(lo, 3), f(hi, 1), f(hi, 3)};
         dst[(((size_t)(2 * sb + h) * ngrp + grp) * JL_GEMM_ASTAGE_FRAGS + ks) * 64 + lane] =
@@ -130,11 +143,11 @@ __device__ __forceinline__ void gemm_prep_group(u32* lds, int sb, int grp, int n
     }
 }
 
-template <int NW>
+template <int NW, bool PL = false>
 __device__ __forceinline__ void gemm_prep_q4k_body(const GemmPrepArgs& p, u32* lds) {
     const int lane = threadIdx.x & 63;
     const int sb = blockIdx.x, grp = blockIdx.y;
-    gemm_prep_group<NW>(lds, sb, grp, p.tok_pad >> 5, p.bq, p.da, [&](int tl) {
+    gemm_prep_group<NW, PL>(lds, sb, grp, p.tok_pad >> 5, p.bq, p.da, [&](int tl) {
         const int t = grp * 32 + tl;
         f32x4 v = f32x4{0.f, 0.f, 0.f, 0.f};
         if (t < p.ntok) v = ((const f32x4*)(p.x + (size_t)t * p.k + (size_t)sb * 256))[lane];
@@ -167,6 +180,29 @@ __device__ __forceinline__ void gemm_load_w(const GemmArgs& p, int row, int sb, 
     const uint8_t* blk = p.w + (size_t)row * p.row_bytes + (size_t)sb * 144;
     r.hdr = ld16(blk);
     r.q = ld16(blk + 16 + 32 * g + 16 * wq);
+}
+
+// The same registers from packed planes (jit/gpu/kernels/pack.go:52-247): thread = (row, sub-block
+// of the stage).  hdr = (d | dmin << 16, the three words of the 96-bit stream of 6-bit scales
+// and minimums: scale of sub-block j at bit 12 j, its minimum at bit 12 j + 6); q = the four
+// words of the sub-block's nibbles.  Every load is a 32-bit word a lane, consecutive rows in
+// consecutive lanes: 256 contiguous bytes an instruction.  row: relative to the launch's first.
+__device__ __forceinline__ void gemm_load_w_planes(const GemmArgs& p, int row, int sb, int sub, GemmWRegs& r) {
+    const size_t st = (size_t)p.pstride;
+    const size_t sup = (size_t)(p.psb0 + sb);
+    const u32* d = p.pd + sup * st + p.prow0;
+    const u32* sc = p.psc + sup * 3 * st + p.prow0;
+    const u32* q = p.pqs + (sup * 8 + sub) * 4 * st + p.prow0;
+    r.hdr = u32x4{d[row], sc[row], sc[st + row], sc[2 * st + row]};
+    r.q = u32x4{q[row], q[st + row], q[2 * st + row], q[3 * st + row]};
+}
+
+// Field f (six bits at bit 6 f) of the 96-bit stream in hdr.y, hdr.z, hdr.w (scstream.go:32-52).
+__device__ __forceinline__ u32 gemm_stream_field(const u32x4& hdr, int f) {
+    const int b = 6 * f, wi = b >> 5, sh = b & 31;
+    const u32 lo = wi == 0 ? hdr.y : wi == 1 ? hdr.z : hdr.w;
+    const u32 hi = wi == 0 ? hdr.z : wi == 1 ? hdr.w : 0u;
+    return __builtin_amdgcn_alignbit(hi, lo, sh) & 63u;
 }
 
 // (1024 + n) as f16 for the nibble in bits 0-3 of each 16-bit half.  mask and magic
@@ -213,6 +249,19 @@ __device__ __forceinline__ void gemm_w_scale(const GemmWRegs& r, int row, int hh
     k.dst = sw + row * JL_GEMM_STRIDE + 64 * hh + 32 * wq;
 }
 
+// the same for a thread of the plane form: all eight nibbles of a word belong to sub-block
+// `sub` of the super-block, the row's K positions 32 * (sub % 4) .. of the stage
+__device__ __forceinline__ void gemm_w_scale_planes(const GemmWRegs& r, int row, int sub, _Float16* sw, GemmWScale& k) {
+    const u32 sc = gemm_stream_field(r.hdr, 2 * sub);
+    const _Float16 f = (_Float16)(float)sc, n = (_Float16)(-1024.0f * (float)sc);
+    k.mlo = k.mhi = f16x2{f, f};
+    k.alo = k.ahi = f16x2{n, n};
+    k.mask = 0x000F000Fu;
+    k.magic = 0x64006400u;
+    asm volatile("" : "+v"(k.mask), "+v"(k.magic));
+    k.dst = sw + row * JL_GEMM_STRIDE + 32 * (sub & 3);
+}
+
 // word c (0..3) of the thread's four
 __device__ __forceinline__ void gemm_w_word(const GemmWRegs& r, const GemmWScale& k, int c) {
     const u32 w = r.q[c];
@@ -244,6 +293,19 @@ __device__ __forceinline__ void gemm_w_mins(const GemmWRegs& r, int row, int hh,
     }
 }
 
+// plane form: sub-block threads 0 (m_s, and the row's d and dmin) and 1 (64 * m_s) of a row
+__device__ __forceinline__ void gemm_w_mins_planes(const GemmWRegs& r, int row, int hh, _Float16* sw, float* sscale) {
+    const float mul = hh ? 64.0f : 1.0f;
+    f16x8 mm;
+#pragma unroll
+    for (int j = 0; j < 8; j++) mm[j] = (_Float16)((float)gemm_stream_field(r.hdr, 2 * j + 1) * mul);
+    *(f16x8*)(sw + row * JL_GEMM_STRIDE + 128 + 8 * hh) = mm;
+    if (hh == 0) {
+        sscale[2 * row] = half_bits_to_f32((uint16_t)(r.hdr.x & 0xFFFF));
+        sscale[2 * row + 1] = half_bits_to_f32((uint16_t)(r.hdr.x >> 16));
+    }
+}
+
 // A grid too small for the chip is widened along K: workgroup z takes sb_per super-blocks
 // and writes its partial sums to slab z; the slabs are added in order afterwards.
 __device__ __forceinline__ void gemm_split_slice(GemmArgs& p) {
@@ -251,6 +313,7 @@ __device__ __forceinline__ void gemm_split_slice(GemmArgs& p) {
     const int sb0 = blockIdx.z * p.sb_per;
     const int n = min(p.sb_per, p.k / 256 - sb0);
     p.w += (size_t)sb0 * 144;
+    p.psb0 += sb0;
     p.bq += (size_t)2 * sb0 * (p.tok_pad >> 5) * (JL_GEMM_ASTAGE_FRAGS * JL_GEMM_AFRAG_HALFS);
     p.da += (size_t)sb0 * p.tok_pad;
     p.k = 256 * n;
@@ -266,8 +329,12 @@ __device__ __forceinline__ void gemm_split_slice(GemmArgs& p) {
 // t0, r0: the tile's first token and row (a grouped launch places tiles per expert).
 // SKIP: a wavefront whose 32 tokens all lie past ntok takes its share of the dequantization
 // and the barriers and leaves the matrix work out (ragged tiles of a grouped launch).
-template <int RH, bool SKIP = false>
+// PL (RH = 1 only): the weights come from packed planes.  Thread = (row = lane, sub-block of the
+// stage = wavefront); the stage's K order is the planes' (the prep kernel's PL order), the rest
+// of the kernel is the same.
+template <int RH, bool SKIP = false, bool PL = false>
 __device__ __forceinline__ void gemm_q4k_body(const GemmArgs& p, uint8_t* smem, int t0, int r0) {
+    static_assert(!PL || RH == 1, "the plane form is the four-wavefront tile");
     constexpr int ROWS = 64 * RH, JL_GEMM_STAGE_HALFS = ROWS * JL_GEMM_STRIDE;
     _Float16* sW = (_Float16*)smem;
     float* sScale = (float*)(sW + 2 * JL_GEMM_STAGE_HALFS);
@@ -278,8 +345,17 @@ __device__ __forceinline__ void gemm_q4k_body(const GemmArgs& p, uint8_t* smem, 
     const bool live = !SKIP || t0 + 32 * (__builtin_amdgcn_readfirstlane(wave) & 3) < p.ntok;   // wavefront-uniform
     const int nsteps = 2 * (p.k / 256);
     // this thread's share of a weight stage
-    const int srow = tid >> 2, hh = (tid >> 1) & 1, wq = tid & 1;
+    const int srow = PL ? lane : tid >> 2, hh = PL ? (wave & 1) : (tid >> 1) & 1, wq = tid & 1;
+    const int psub = __builtin_amdgcn_readfirstlane(wave) & 3;   // plane form: its sub-block of a stage
     const int wrow = min(r0 + srow, p.nrows - 1);
+    auto load_w = [&](int sb, int half, GemmWRegs& r) {
+        if (PL) gemm_load_w_planes(p, wrow, sb, 4 * half + psub, r);
+        else gemm_load_w(p, wrow, sb, 2 * half + hh, wq, r);
+    };
+    auto w_scale = [&](const GemmWRegs& r, int half, _Float16* sw, GemmWScale& k) {
+        if (PL) gemm_w_scale_planes(r, srow, 4 * half + psub, sw, k);
+        else gemm_w_scale(r, srow, hh, wq, half, sw, k);
+    };
     const int arow = lane & 31, kg = lane >> 5;
     // fragment (step, ks) of this wavefront's 32 tokens
     // (a tile may reach past the last group of the workspace: such tokens are never stored)
@@ -297,18 +373,18 @@ __device__ __forceinline__ void gemm_q4k_body(const GemmArgs& p, uint8_t* smem, 
     // prologue: stage 0 of the weights into LDS, stage 1 into registers; the first
     // stage's activation fragments into the ring
     GemmWRegs wa, wb;   // stages alternate between the two register sets
-    gemm_load_w(p, wrow, 0, hh, wq, wa);
+    load_w(0, 0, wa);
     f16x8 aring[8], aaug;
 #pragma unroll
     for (int ks = 0; ks < 8; ks++) aring[ks] = a_frag(0, ks);
     aaug = aring[0];
     {
         GemmWScale k0;
-        gemm_w_scale(wa, srow, hh, wq, 0, sW, k0);
+        w_scale(wa, 0, sW, k0);
 #pragma unroll
         for (int c = 0; c < 4; c++) gemm_w_word(wa, k0, c);
     }
-    gemm_load_w(p, wrow, 0, 2 + hh, wq, wa);
+    load_w(0, 1, wa);
     const int da_tok = min(t0 + (tid & (JL_GEMM_TILE - 1)), p.tok_pad - 1);
     float da_reg = p.da[da_tok];
     lds_barrier();
@@ -328,13 +404,13 @@ __device__ __forceinline__ void gemm_q4k_body(const GemmArgs& p, uint8_t* smem, 
         // covers their latency (that stage has this stage's half)
         {
             const int s2 = min(step + 2, nsteps - 1);
-            gemm_load_w(p, wrow, s2 >> 1, 2 * half + hh, wq, wnxt);
+            load_w(s2 >> 1, half, wnxt);
         }
         // The next weight stage sits in registers; its dequantization into LDS is spread
         // over this stage's K-steps, one word after every second K-step's matrix
         // instructions, so the vector work runs under the matrix core.
         GemmWScale wsc;
-        gemm_w_scale(wcur, srow, hh, wq, nhalf, wnext, wsc);
+        w_scale(wcur, nhalf, wnext, wsc);
         JL_TRACE(1);
         // matrix work: per K-step one activation fragment (already in the ring) against
         // the two row groups' weight fragments, fetched from LDS a K-step ahead; the ring
@@ -370,7 +446,11 @@ __device__ __forceinline__ void gemm_q4k_body(const GemmArgs& p, uint8_t* smem, 
             __builtin_amdgcn_sched_barrier(0);
         }
         if (has_next && nhalf == 1) {
-            if (wq == 0) gemm_w_mins(wcur, srow, hh, wnext, sScale + (nsbi & 1) * 2 * ROWS);
+            if (PL) {
+                if (psub < 2) gemm_w_mins_planes(wcur, srow, psub, wnext, sScale + (nsbi & 1) * 2 * ROWS);
+            } else if (wq == 0) {
+                gemm_w_mins(wcur, srow, hh, wnext, sScale + (nsbi & 1) * 2 * ROWS);
+            }
             if (tid < JL_GEMM_TILE) sDa[(nsbi & 1) * JL_GEMM_TILE + tid] = da_reg;
         }
         if (half == 1) {
@@ -481,6 +561,16 @@ __device__ __forceinline__ void gemm_wide_scale(const u32x4& hdr, int hh, int ha
     k.mhi = f16x2{hhi16, hhi16};
     k.ahi = f16x2{nhi, nhi};
 }
+// plane form: all eight nibbles of a word belong to sub-block `sub` of the super-block
+__device__ __forceinline__ void gemm_wide_scale_planes(const u32x4& hdr, int sub, GemmWideScale& k) {
+    const float f = (float)gemm_stream_field(hdr, 2 * sub);
+    const _Float16 hlo = (_Float16)f, hhi16 = (_Float16)(f * 0.0625f);
+    const _Float16 nlo = (_Float16)(-1024.0f * f), nhi = (_Float16)(-64.0f * f);
+    k.mlo = f16x2{hlo, hlo};
+    k.alo = f16x2{nlo, nlo};
+    k.mhi = f16x2{hhi16, hhi16};
+    k.ahi = f16x2{nhi, nhi};
+}
 __device__ __forceinline__ void gemm_wide_word(u32 w, const GemmWideScale& k, int c, u32 mask_lo, u32 mask_hi,
                                                u32 magic) {
     const u32 w8 = w >> 8;
@@ -495,6 +585,9 @@ __device__ __forceinline__ void gemm_wide_word(u32 w, const GemmWideScale& k, in
     *(u32x4*)(k.dst + 8 * c) = o;
 }
 
+// PL: the weights come from packed planes; thread = (row = 64 * (wavefront % 2) + lane, sub-block
+// of the stage = wavefront / 2), the stage's K order is the planes' (the prep kernel's PL order).
+template <bool PL = false>
 __device__ __forceinline__ void gemm_q4k_wide_body(const GemmArgs& p, uint8_t* smem) {
     constexpr int ROWS = 128, TOK = JL_GEMM_WIDE_TOK, STAGE_HALFS = ROWS * JL_GEMM_WROW;
     constexpr int MIN_HALFS = ROWS * JL_GEMM_MROW;
@@ -507,7 +600,8 @@ __device__ __forceinline__ void gemm_q4k_wide_body(const GemmArgs& p, uint8_t* s
     const int tg = __builtin_amdgcn_readfirstlane(tid >> 6);   // wavefront tg: tokens 32*tg..
     const int t0 = blockIdx.x * TOK, r0 = blockIdx.y * ROWS;
     const int nsteps = 2 * (p.k / 256);
-    const int srow = tid >> 2, hh = (tid >> 1) & 1, wq = tid & 1;
+    const int psub = tg >> 1;   // plane form: this thread's sub-block of a stage
+    const int srow = PL ? 64 * (tg & 1) + lane : tid >> 2, hh = PL ? (psub & 1) : (tid >> 1) & 1, wq = tid & 1;
     const int arow = lane & 31, kg = lane >> 5;
     // Addresses are a uniform 64-bit base (scalar registers) plus a 32-bit lane offset.
     // Activation fragment (step, ks) of this wavefront's 32 tokens:
@@ -521,14 +615,19 @@ __device__ __forceinline__ void gemm_q4k_wide_body(const GemmArgs& p, uint8_t* s
     const uint8_t* wbase = p.w + (size_t)r0 * p.row_bytes;
     const unsigned woff = (unsigned)(min(r0 + srow, p.nrows - 1) - r0) * (unsigned)p.row_bytes;
     const unsigned wqoff = woff + 16 + 32 * hh + 16 * wq;
+    const int prow = min(r0 + srow, p.nrows - 1);
     auto load_w = [&](int step, GemmWRegs& r) {
-        const uint8_t* blk = wbase + (size_t)(step >> 1) * 144 + 64 * (step & 1);
-        r.hdr = ld16(blk - 64 * (step & 1) + woff);
-        r.q = ld16(blk + wqoff);
+        if (PL) {
+            gemm_load_w_planes(p, prow, step >> 1, 4 * (step & 1) + psub, r);
+        } else {
+            const uint8_t* blk = wbase + (size_t)(step >> 1) * 144 + 64 * (step & 1);
+            r.hdr = ld16(blk - 64 * (step & 1) + woff);
+            r.q = ld16(blk + wqoff);
+        }
     };
     u32 mask_lo = 0x000F000Fu, mask_hi = 0x00F000F0u, magic = 0x64006400u;
     asm volatile("" : "+v"(mask_lo), "+v"(mask_hi), "+v"(magic));   // keep them in vector registers
-    const int wdst = srow * JL_GEMM_WROW + 64 * hh + 32 * wq;
+    const int wdst = PL ? srow * JL_GEMM_WROW + 32 * psub : srow * JL_GEMM_WROW + 64 * hh + 32 * wq;
 
     f32x16 out[4], accP[4];
 #pragma unroll
@@ -546,7 +645,8 @@ __device__ __forceinline__ void gemm_q4k_wide_body(const GemmArgs& p, uint8_t* s
     aaug = a_frag(min(1, nsteps - 1), 8);
     {
         GemmWideScale k0;
-        gemm_wide_scale(wa.hdr, hh, 0, k0);
+        if (PL) gemm_wide_scale_planes(wa.hdr, psub, k0);
+        else gemm_wide_scale(wa.hdr, hh, 0, k0);
         k0.dst = sW + wdst;
 #pragma unroll
         for (int c = 0; c < 4; c++) gemm_wide_word(wa.q[c], k0, c, mask_lo, mask_hi, magic);
@@ -638,7 +738,10 @@ __device__ __forceinline__ void gemm_q4k_wide_body(const GemmArgs& p, uint8_t* s
                 ep_quarter(GemmIntC<ej0 + (ks >> 2)>{}, GemmIntC<(ks & 3)>{}, dav);
             } else if (jh != ep_jh) {
                 // the next stage's weights: wcur -> f16 -> LDS
-                if (ks == 0) gemm_wide_scale(wcur.hdr, hh, nhalf, wsc);
+                if (ks == 0) {
+                    if (PL) gemm_wide_scale_planes(wcur.hdr, 4 * nhalf + psub, wsc);
+                    else gemm_wide_scale(wcur.hdr, hh, nhalf, wsc);
+                }
                 if (ks & 1) gemm_wide_word(wcur.q[ks >> 1], wsc, ks >> 1, mask_lo, mask_hi, magic);
                 if (nhalf == 1) {
                     // a first half also lays down its super-block's minimum columns and scales
@@ -646,14 +749,20 @@ __device__ __forceinline__ void gemm_q4k_wide_body(const GemmArgs& p, uint8_t* s
                     // address write the same value, which costs nothing and keeps the slot
                     // one basic block)
                     if (ks == 4) {
-                        const GemmScaleBytes sbytes = gemm_scale_bytes(wcur.hdr.y, wcur.hdr.z, wcur.hdr.w);
                         // hh = 0 writes m_s (pairs with A_lo), hh = 1 writes 64*m_s (pairs with A_hi)
                         const float mul = hh ? 64.0f : 1.0f;
                         f16x8 mm;
+                        if (PL) {
 #pragma unroll
-                        for (int b = 0; b < 4; b++) {
-                            mm[b] = (_Float16)((float)((sbytes.mn_lo >> (8 * b)) & 0xFF) * mul);
-                            mm[4 + b] = (_Float16)((float)((sbytes.mn_hi >> (8 * b)) & 0xFF) * mul);
+                            for (int j = 0; j < 8; j++)
+                                mm[j] = (_Float16)((float)gemm_stream_field(wcur.hdr, 2 * j + 1) * mul);
+                        } else {
+                            const GemmScaleBytes sbytes = gemm_scale_bytes(wcur.hdr.y, wcur.hdr.z, wcur.hdr.w);
+#pragma unroll
+                            for (int b = 0; b < 4; b++) {
+                                mm[b] = (_Float16)((float)((sbytes.mn_lo >> (8 * b)) & 0xFF) * mul);
+                                mm[4 + b] = (_Float16)((float)((sbytes.mn_hi >> (8 * b)) & 0xFF) * mul);
+                            }
                         }
                         *(f16x8*)(sMin + (sb & 1) * MIN_HALFS + srow * JL_GEMM_MROW + 8 * hh) = mm;
                     }

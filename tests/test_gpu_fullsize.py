@@ -178,6 +178,21 @@ def test_prefill_gemm_full_size(dev, devbuf, shape):
         assert nmse(outs[0], outs[1].astype(np.float64)) <= 1e-12, "K-split form vs 128 x 64 tiles"
     else:
         assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32)), "automatic form != 128 x 64 tiles"
+    # the same weights as packed planes: the tiled forms read them where they lie (no rows are
+    # restored first), the same integers and the same epilogue, so the same bits
+    pl = [devbuf(shape=(max(n, 1),), dtype=np.uint32, fill=0) for n in dev.packed_words(t, nrows, k)]
+    assert dev.pack_weights_dev(t, wd.ptr, nrows, k, pl[0].ptr, pl[1].ptr, pl[2].ptr)
+    assert dev.reserve_shape(t, nrows, k, ntok, packed=True)
+    outp = devbuf(shape=(ntok * nrows + 16,), dtype=np.float32, fill=POISON)
+    n0 = dev.launch_count()
+    assert dev.matmul_packed_dev(outp.ptr, t, Packed(pl[0].ptr, pl[1].ptr, pl[2].ptr, 0, nrows), xd.ptr, nrows, k, ntok)
+    assert dev.launch_count() - n0 <= 3, "a launch restored rows in front of the GEMM"
+    dev.synchronize()
+    gotp = outp.get()
+    assert np.all(gotp[ntok * nrows:] == POISON)
+    assert np.array_equal(gotp[:ntok * nrows].view(np.uint32), outs[0].reshape(-1).view(np.uint32)), "planes != rows"
+    for b_ in pl + [outp]:
+        b_.free()
     # token t of the GEMM == the decode matvec of token t, every row
     mv = devbuf(shape=(nrows,), dtype=np.float32, fill=POISON)
     for tok in (0, ntok // 2 + 1, ntok - 1):

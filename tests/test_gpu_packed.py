@@ -381,3 +381,57 @@ def test_packed_host_pointer_seam(dev):
     assert dev.MatVecPacked(out, quant.MXFP4, p, x, nrows, k) is False
     assert dev.MatVecPacked(out, t, p, x, nrows, k - 32) is False
     dev.SetActWindow(32)
+
+
+@pytest.mark.parametrize("shape", [(130, 300, 1024, 0, 300), (512, 260, 2048, 90, 400), (256, 700, 512, 0, 700),
+                                   (96, 150, 2816, 37, 200), (200, 33000, 256, 0, 33000)],
+                         ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("form", [0, 1, 2], ids=["auto", "tile128x64", "tile256x128"])
+def test_matmul_packed_q4k_reads_planes_where_they_lie(dev, devbuf, shape, form):
+    """JIT.MatMulPacked (/root/reference/engine/nn/packedmm.go:23-139) never re-lays weights per
+    call: the tiled GEMM forms read the QS / D / SC planes directly (their own activation prep in
+    the planes' K order), with no row-restoring launch in front.  A row range inside a larger plane
+    set (an expert's sheet inside its bank), a K split (few tokens, 11 super-blocks), the split of
+    a grid between the two tiles (33000 rows); against the oracle, and bit for bit against the
+    GEMM over the same weights as GGUF rows (the same integers, the same f32 epilogue)."""
+    ntok, nrows, k, row0, stride = shape
+    t = quant.Q4_K
+    dev.SetActWindow(256)
+    w = synth.random_weights(t, stride, k, seed=ntok + nrows)
+    rb = quant.row_bytes(t, k)
+    wsub = w[row0 * rb:(row0 + nrows) * rb]
+    x = np.stack([synth.activations(k, seed=700 + i) * np.float32(1 + i % 3) for i in range(ntok)])
+    x[ntok // 2] = 0
+    p = _dev_planes(devbuf, *oracle.pack_weights(t, w, stride, k), row=row0, stride=stride)
+    xd, wd = devbuf(x), devbuf(np.ascontiguousarray(wsub))
+    dev.set_tuning(gemm__form=form)
+    out = devbuf(shape=(ntok * nrows + 16,), dtype=np.float32, fill=np.float32(3e30))
+    ref = devbuf(shape=(ntok * nrows + 16,), dtype=np.float32, fill=np.float32(3e30))
+    n0 = dev.launch_count()
+    assert dev.matmul_packed_dev(out.ptr, t, p, xd.ptr, nrows, k, ntok)
+    launches = dev.launch_count() - n0
+    assert dev.matmul_dev(ref.ptr, t, wd.ptr, xd.ptr, nrows, k, ntok)
+    dev.synchronize()
+    dev.set_tuning(gemm__form=0)
+    got, same = out.get(), ref.get()
+    assert np.all(got[ntok * nrows:] == np.float32(3e30)), "wrote past the output"
+    got = got[:ntok * nrows].reshape(ntok, nrows)
+    assert np.all(np.abs(got) < 1e30), "elements left unwritten"
+    if nrows <= 1000:
+        want = oracle.matmul_q8act_f64(t, wsub, x, nrows, k, ntok, 256)
+    else:   # the oracle on a sample of rows: first, last, and around the tiles' boundary
+        rows = np.unique(np.concatenate([np.arange(0, 40), np.arange(nrows - 40, nrows),
+                                         np.arange(32768 - 20, 32768 + 20)]))
+        want = oracle.matmul_q8act_f64(t, np.concatenate([wsub[r * rb:(r + 1) * rb] for r in rows]), x, len(rows), k,
+                                       ntok, 256)
+        got = got[:, rows]
+    assert nmse(got, want) <= 1e-10
+    assert np.all(got[ntok // 2] == 0)
+    # no launch restores rows: prep + one or two tile kernels (+ the slab sum of a K split)
+    assert launches <= 3, launches
+    few32 = form == 0 and ntok > 64 and 2 * ((nrows + 31) // 32) * ((ntok + 63) // 64) <= 3 * 256
+    if not few32 and form != 0:   # the same form on both sides: the same bits
+        assert np.array_equal(out.get()[:ntok * nrows].view(np.uint32), same[:ntok * nrows].view(np.uint32))
+    else:
+        assert nmse(out.get()[:ntok * nrows], same[:ntok * nrows].astype(np.float64)) <= 1e-12
+    dev.SetActWindow(32)
