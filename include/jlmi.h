@@ -400,6 +400,36 @@ int jl_moe_ffn_dev(jl_ctx *ctx, float *resid, int type, const void *gate_bank,
                    const uint32_t *sel, int sel_stride, const float *wt, int rows, int k_used,
                    int n_expert, int n_ffn, int n_embd, void *stream);
 
+/* A mixture's bank as packed planes, the way a container holds it (nn.Packed.Sheet / Sheets,
+ * engine/nn/device.go:70-80; format/jlm/write.go:123-180, read.go:447-469): qs, d, sc are
+ * expert 0's planes in device memory.
+ *   sheet_bytes > 0: every expert's sheet was packed on its own and expert e's three planes
+ *       start sheet_bytes * e bytes after expert 0's (a container's expert page size; a
+ *       sheet holds `stride` rows, normally the expert's own row count);
+ *   sheet_bytes == 0: the bank is ONE plane set of `stride` rows and expert e is rows
+ *       e * nrows .. of it (Packed.Row / Stride). */
+typedef struct jl_packed_bank {
+    const uint32_t *qs, *d, *sc;
+    size_t sheet_bytes;
+    int stride;
+} jl_packed_bank;
+
+/* jl_moe_matvec_dev over banks of packed planes: the per-expert matrix-core tile reads every
+ * sheet where it lies (Q4_K with the activation window of 256; anything else JL_DECLINED).
+ * bank1 / out1 may be null; both banks must share one layout (sheet_bytes, stride). */
+int jl_moe_matvec_packed_dev(jl_ctx *ctx, float *out0, float *out1, int type,
+                             const jl_packed_bank *bank0, const jl_packed_bank *bank1, const float *x,
+                             const float *x2, const uint32_t *src, const uint32_t *start, int n_expert,
+                             int ncols, int nrows, int k, void *stream);
+
+/* jl_moe_ffn_dev over banks of packed planes (moeBatchFrom over a container's expert pages,
+ * engine/model/moe.go:510-761): gate and up banks hold n_ffn x n_embd sheets, the down bank
+ * n_embd x n_ffn sheets. */
+int jl_moe_ffn_packed_dev(jl_ctx *ctx, float *resid, int type, const jl_packed_bank *gate,
+                          const jl_packed_bank *up, const jl_packed_bank *down, const float *x,
+                          const uint32_t *sel, int sel_stride, const float *wt, int rows, int k_used,
+                          int n_expert, int n_ffn, int n_embd, void *stream);
+
 /* The same block with the down bank in a type of its own: every expert tensor carries its
  * own quant.Type in the reference (nn.Weight.T, engine/nn/device.go:47-58; a Q4_K_M file
  * holds Q4_K gate and up sheets beside Q6_K down sheets). */

@@ -30,6 +30,12 @@ class MVGroup(C.Structure):
                 ("resid_gate", C.c_void_p), ("norm_w", C.c_void_p), ("norm_eps", C.c_float), ("norm_out", C.c_void_p)]
 
 
+class PackedBank(C.Structure):
+    """jl_packed_bank: a mixture's bank as packed planes (device addresses)."""
+    _fields_ = [("qs", C.c_void_p), ("d", C.c_void_p), ("sc", C.c_void_p), ("sheet_bytes", C.c_size_t),
+                ("stride", C.c_int)]
+
+
 # name -> (restype, argtypes); every symbol include/jlmi.h declares
 SIGNATURES = {
     "jl_hip_runtime": (C.c_char_p, []),
@@ -78,6 +84,10 @@ SIGNATURES = {
     "jl_moe_route_dev": (_int, [_vp, _vp, _int, _int, _int, _vp, _int, _vp, _vp]),
     "jl_moe_group_dev": (_int, [_vp, _vp, _int, _int, _int, _int, _vp, _vp, _vp, _vp]),
     "jl_moe_matvec_dev": (_int, [_vp, _vp, _vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp]),
+    "jl_moe_matvec_packed_dev": (_int, [_vp, _vp, _vp, _int, C.POINTER(PackedBank), C.POINTER(PackedBank), _vp, _vp, _vp,
+                                        _vp, _int, _int, _int, _int, _vp]),
+    "jl_moe_ffn_packed_dev": (_int, [_vp, _vp, _int, C.POINTER(PackedBank), C.POINTER(PackedBank), C.POINTER(PackedBank),
+                                     _vp, _vp, _int, _vp, _int, _int, _int, _int, _int, _vp]),
     "jl_moe_combine_dev": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _vp, _int, _int, _int, _vp]),
     "jl_moe_ffn_dev": (_int, [_vp, _vp, _int, _vp, _vp, _vp, _vp, _vp, _int, _vp, _int, _int, _int, _int,
                               _int, _vp]),

@@ -371,7 +371,8 @@ int resident_weight(jl_ctx* c, const void* w, size_t bytes, void** dev) {
 int ws_ensure(jl_ctx* c, void** buf, size_t* have, size_t need);
 int moe_matvec_launch(jl_ctx* c, float* out0, float* out1, int type, const void* bank0, const void* bank1,
                       const float* x, const float* x2, const uint32_t* src, const uint32_t* start,
-                      int n_expert, int ncols, int nrows, int k, hipStream_t st);
+                      int n_expert, int ncols, int nrows, int k, hipStream_t st,
+                      const jl_packed_bank* pb0 = nullptr, const jl_packed_bank* pb1 = nullptr);
 
 constexpr int kGemmTile = 128;         // tokens and rows per workgroup (kernels/gemm_q4k.h)
 constexpr int kGemmStride = 152;       // f16 per stage row
@@ -871,17 +872,38 @@ int packed_matmul_launch(jl_ctx* c, float* out, int type, const PlaneRef& pl, co
     return JL_OK;
 }
 
+// pb0 / pb1: the banks as packed planes (bank0 / bank1 unused then): the per-expert tile kernel
+// reads an expert's sheet where it lies in the bank's pages.
 int moe_matvec_launch(jl_ctx* c, float* out0, float* out1, int type, const void* bank0, const void* bank1,
                       const float* x, const float* x2, const uint32_t* src, const uint32_t* start,
-                      int n_expert, int ncols, int nrows, int k, hipStream_t st) {
+                      int n_expert, int ncols, int nrows, int k, hipStream_t st, const jl_packed_bank* pb0,
+                      const jl_packed_bank* pb1) {
     const TypeInfo* ti = nullptr;
     int rc = matvec_check(c, type, nrows, k, &ti);
     if (rc != JL_OK) return rc;
-    if (!out0 || !bank0 || !x || !start || n_expert <= 0 || ncols <= 0)
+    const bool planes = pb0 != nullptr;
+    if (!out0 || (!planes && !bank0) || !x || !start || n_expert <= 0 || ncols <= 0)
         return fail(c, JL_ERR_ARG, "moe matvec: bad operand");
-    if ((bank1 == nullptr) != (out1 == nullptr)) return fail(c, JL_ERR_ARG, "moe matvec: second matrix needs both bank and out");
+    if (planes) {
+        if ((pb1 == nullptr) != (out1 == nullptr)) return fail(c, JL_ERR_ARG, "moe matvec: second matrix needs both bank and out");
+        for (const jl_packed_bank* b : {pb0, pb1}) {
+            if (!b) continue;
+            if (!b->qs || !b->d || !b->sc || b->stride <= 0) return fail(c, JL_ERR_ARG, "moe matvec: null plane");
+            if ((((uintptr_t)b->qs | (uintptr_t)b->d | (uintptr_t)b->sc) & 3) || (b->sheet_bytes & 3)) return JL_DECLINED;
+            // an expert's rows must lie inside a plane set: its own sheet, or its range of the bank's
+            if (b->sheet_bytes ? b->stride < nrows : (long)b->stride < (long)n_expert * nrows)
+                return fail(c, JL_ERR_ARG, "moe matvec: plane sets of %d rows do not hold %d experts x %d rows", b->stride,
+                            n_expert, nrows);
+            if (b->sheet_bytes != pb0->sheet_bytes || b->stride != pb0->stride) return JL_DECLINED;   // one layout a launch
+        }
+        // plane sheets are served by the tile form (Q4_K, the k-quant window)
+        if (type != JL_TYPE_Q4_K || c->act_window != 256) return JL_DECLINED;
+        if ((size_t)pb0->stride * 4 >= ((size_t)1 << 31)) return JL_DECLINED;
+    } else if ((bank1 == nullptr) != (out1 == nullptr)) {
+        return fail(c, JL_ERR_ARG, "moe matvec: second matrix needs both bank and out");
+    }
     if (!aligned16(x) || (x2 && !aligned16(x2)) || k % 256 != 0 || n_expert > 65535 || ncols > 65535) return JL_DECLINED;
-    if (!aligned16(bank0) || (bank1 && !aligned16(bank1))) return JL_DECLINED;
+    if (!planes && (!aligned16(bank0) || (bank1 && !aligned16(bank1)))) return JL_DECLINED;
     const int row_bytes = (k / ti->block_elems) * ti->block_bytes;
     const size_t sheet = (size_t)nrows * row_bytes;
     if (type == JL_TYPE_Q4_K ? sheet % 16 != 0 : sheet % 2 != 0) return JL_DECLINED;
@@ -902,7 +924,7 @@ int moe_matvec_launch(jl_ctx* c, float* out0, float* out1, int type, const void*
     const long q6_cols = c->tune.moe_q6k_cols > 0 ? c->tune.moe_q6k_cols : 12;
     const bool many_cols = c->tune.moe_form == 0 && (long)ncols >= (q6 ? q6_cols : 10L) * n_expert;
     if ((type == JL_TYPE_Q4_K || q6) && c->act_window == 256 &&
-        (c->tune.moe_form == 4 || many_cols || (!q6 && c->tune.moe_form == 2)) &&
+        (planes || c->tune.moe_form == 4 || many_cols || (!q6 && c->tune.moe_form == 2)) &&
         4u * 19968u <= c->lds_limit) {   // JL_MOEG_WAVE_LDS
         const int nslots = ncols / 32 + n_expert + 1, nsb = k / 256;
         const int tiles_max = ncols / 128 + n_expert;
@@ -924,16 +946,29 @@ int moe_matvec_launch(jl_ctx* c, float* out0, float* out1, int type, const void*
         pa.bq = (uint16_t*)c->moe_q_ws; pa.da = (float*)((char*)c->moe_q_ws + bq_bytes);
         pa.k = k; pa.nslots = nslots;
         void* pp[] = {&pa};
-        rc = launch(c, "jl_moe_gemm_prep", (unsigned)nsb, (unsigned)nslots, 256, 0, st, pp);
+        rc = launch(c, planes ? "jl_moe_gemm_prep_planes" : "jl_moe_gemm_prep", (unsigned)nsb, (unsigned)nslots, 256, 0, st, pp);
         if (rc != JL_OK) return rc;
         MoeGemmArgs ga;
         ga.out[0] = out0; ga.out[1] = out1;
         ga.bank[0] = (const uint8_t*)bank0; ga.bank[1] = (const uint8_t*)bank1;
         ga.bq = pa.bq; ga.da = pa.da; ga.start = start; ga.wl = wa.wl;
         ga.sheet_bytes = sheet; ga.nrows = nrows; ga.k = k; ga.row_bytes = row_bytes;
-        ga.nslots = nslots; ga.nmat = bank1 ? 2 : 1;
+        ga.nslots = nslots; ga.nmat = (planes ? pb1 != nullptr : bank1 != nullptr) ? 2 : 1;
+        if (planes) {
+            const jl_packed_bank* pbs[2] = {pb0, pb1};
+            for (int m = 0; m < ga.nmat; m++) { ga.pqs[m] = pbs[m]->qs; ga.pd[m] = pbs[m]->d; ga.psc[m] = pbs[m]->sc; }
+            ga.sheet_words = pb0->sheet_bytes / 4;
+            ga.row_step = pb0->sheet_bytes ? 0 : nrows;
+            ga.pstride = pb0->stride;
+        }
         void* gp[] = {&ga};
         const long rtiles = (nrows + 63) / 64;
+        if (planes) {
+            if (kGemmLdsBytes > c->lds_limit || (long)tiles_max * rtiles * ga.nmat >= (1L << 31)) return JL_DECLINED;
+            const long work = (long)tiles_max * rtiles * ga.nmat;
+            return launch(c, "jl_moe_gemm_r64_planes", (unsigned)std::min<long>(work, 2L * c->num_cu), 1, 256,
+                          gemm_lds_bytes(64), st, gp);
+        }
         if ((q6 || c->tune.moe_form == 4 || (c->tune.moe_form == 0 && (long)ncols >= 56L * n_expert)) &&
             kGemmLdsBytes <= c->lds_limit && n_expert <= 65535 && (long)tiles_max * rtiles * ga.nmat < (1L << 31)) {
             const long work = (long)tiles_max * rtiles * ga.nmat;
@@ -945,6 +980,7 @@ int moe_matvec_launch(jl_ctx* c, float* out0, float* out1, int type, const void*
         return launch(c, "jl_moe_gemm_q4k", (unsigned)((nrows + 255) / 256), (unsigned)nslots, 256, 4u * 19968u, st, gp,
                       (unsigned)ga.nmat);
     }
+    if (planes) return JL_DECLINED;   // (no LDS for the tile form on this device)
     const int nslots = k / ti->slot_elems;
     // lanes per row: the width that leaves the fewest lanes without a slot (a row of 12 slots
     // on 16 lanes idles a quarter of them; on 4 lanes, three slots each, none); among equals
@@ -1062,7 +1098,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     if (e != hipSuccess)
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
-    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_prep_q4k_planes", "jl_gemm_q4k_r64_planes", "jl_gemm_q4k_wide_planes", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_group2_wide", "jl_moe_quant", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_q4k", "jl_moe_gemm_r64", "jl_moe_gemm_q6k_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_sum_parts", "jl_probe_read", "jl_probe_empty", "jl_probe_wait",
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_prep_q4k_planes", "jl_gemm_q4k_r64_planes", "jl_gemm_q4k_wide_planes", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_group2_wide", "jl_moe_quant", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_prep_planes", "jl_moe_gemm_q4k", "jl_moe_gemm_r64", "jl_moe_gemm_r64_planes", "jl_moe_gemm_q6k_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_sum_parts", "jl_probe_read", "jl_probe_empty", "jl_probe_wait",
                                       "jl_pack_weights", "jl_unpack_q4k", "jl_unpack_q6k", "jl_unpack_q8_0"};
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int rw : {16, 32, 64})
@@ -1495,6 +1531,16 @@ int jl_moe_matvec_dev(jl_ctx* c, float* out0, float* out1, int type, const void*
                              pick_stream(c, stream));
 }
 
+int jl_moe_matvec_packed_dev(jl_ctx* c, float* out0, float* out1, int type, const jl_packed_bank* bank0,
+                             const jl_packed_bank* bank1, const float* x, const float* x2, const uint32_t* src,
+                             const uint32_t* start, int n_expert, int ncols, int nrows, int k, void* stream) {
+    if (!c) return JL_ERR_ARG;
+    if (!bank0) return fail(c, JL_ERR_ARG, "moe matvec: null bank");
+    HIP_TRY(c, H->SetDevice(c->device));
+    return moe_matvec_launch(c, out0, out1, type, nullptr, nullptr, x, x2, src, start, n_expert, ncols, nrows, k,
+                             pick_stream(c, stream), bank0, bank1);
+}
+
 int jl_moe_combine_dev(jl_ctx* c, float* resid, const float* y, const float* wt, const uint32_t* sel,
                        int sel_stride, const uint32_t* pos, int rows, int k_used, int n_embd, void* stream) {
     if (!c) return JL_ERR_ARG;
@@ -1511,9 +1557,11 @@ int jl_moe_combine_dev(jl_ctx* c, float* resid, const float* y, const float* wt,
                   pick_stream(c, stream), params);
 }
 
-int jl_moe_ffn_types_dev(jl_ctx* c, float* resid, int type, int down_type, const void* gate_bank, const void* up_bank,
-                         const void* down_bank, const float* x, const uint32_t* sel, int sel_stride,
-                   const float* wt, int rows, int k_used, int n_expert, int n_ffn, int n_embd, void* stream) {
+namespace {
+int moe_ffn(jl_ctx* c, float* resid, int type, int down_type, const void* gate_bank, const void* up_bank,
+            const void* down_bank, const jl_packed_bank* pg, const jl_packed_bank* pu, const jl_packed_bank* pd,
+            const float* x, const uint32_t* sel, int sel_stride, const float* wt, int rows, int k_used, int n_expert,
+            int n_ffn, int n_embd, void* stream) {
     if (!c) return JL_ERR_ARG;
     if (rows <= 0 || k_used <= 0 || n_expert <= 0 || n_ffn <= 0 || n_embd <= 0)
         return fail(c, JL_ERR_ARG, "moe ffn: bad shape");
@@ -1535,12 +1583,31 @@ int jl_moe_ffn_types_dev(jl_ctx* c, float* resid, int type, int down_type, const
     rc = jl_moe_group_dev(c, sel, sel_stride, rows, k_used, n_expert, start, perm, pos, st);
     if (rc != JL_OK) return rc;
     // gate and up: columns read the routed rows of x
-    rc = moe_matvec_launch(c, g, u, type, gate_bank, up_bank, x, nullptr, perm, start, n_expert, (int)ncols, n_ffn, n_embd, st);
+    rc = moe_matvec_launch(c, g, u, type, gate_bank, up_bank, x, nullptr, perm, start, n_expert, (int)ncols, n_ffn, n_embd, st,
+                           pg, pu);
     if (rc != JL_OK) return rc;
     // down: the activation of column c is silu(g[c]) * u[c]
-    rc = moe_matvec_launch(c, y, nullptr, down_type, down_bank, nullptr, g, u, nullptr, start, n_expert, (int)ncols, n_embd, n_ffn, st);
+    rc = moe_matvec_launch(c, y, nullptr, down_type, down_bank, nullptr, g, u, nullptr, start, n_expert, (int)ncols, n_embd, n_ffn, st,
+                           pd, nullptr);
     if (rc != JL_OK) return rc;
     return jl_moe_combine_dev(c, resid, y, wt, sel, sel_stride, pos, rows, k_used, n_embd, st);
+}
+}  // namespace
+
+int jl_moe_ffn_types_dev(jl_ctx* c, float* resid, int type, int down_type, const void* gate_bank, const void* up_bank,
+                         const void* down_bank, const float* x, const uint32_t* sel, int sel_stride,
+                         const float* wt, int rows, int k_used, int n_expert, int n_ffn, int n_embd, void* stream) {
+    return moe_ffn(c, resid, type, down_type, gate_bank, up_bank, down_bank, nullptr, nullptr, nullptr, x, sel, sel_stride, wt,
+                   rows, k_used, n_expert, n_ffn, n_embd, stream);
+}
+
+int jl_moe_ffn_packed_dev(jl_ctx* c, float* resid, int type, const jl_packed_bank* gate, const jl_packed_bank* up,
+                          const jl_packed_bank* down, const float* x, const uint32_t* sel, int sel_stride,
+                          const float* wt, int rows, int k_used, int n_expert, int n_ffn, int n_embd, void* stream) {
+    if (!c) return JL_ERR_ARG;
+    if (!gate || !up || !down) return fail(c, JL_ERR_ARG, "moe ffn: null bank");
+    return moe_ffn(c, resid, type, type, nullptr, nullptr, nullptr, gate, up, down, x, sel, sel_stride, wt, rows, k_used,
+                   n_expert, n_ffn, n_embd, stream);
 }
 
 int jl_moe_ffn_dev(jl_ctx* c, float* resid, int type, const void* gate_bank, const void* up_bank,

@@ -109,6 +109,15 @@ struct MoeGemmArgs {
     const uint32_t* wl;
     size_t sheet_bytes;
     int nrows, k, row_bytes, nslots, nmat;
+    // the banks as packed planes (plane form of the tile kernel; bank[] unused): expert e's planes
+    // are pqs / pd / psc [mat] + e * sheet_words (u32 words; 0 when the bank is ONE plane set), its
+    // first row e * row_step inside them (0 when every expert has its own sheet), pstride rows a
+    // plane set
+    const uint32_t* pqs[2] = {nullptr, nullptr};
+    const uint32_t* pd[2] = {nullptr, nullptr};
+    const uint32_t* psc[2] = {nullptr, nullptr};
+    size_t sheet_words = 0;
+    int row_step = 0, pstride = 0;
 };
 
 // Two-pass form of the Q4_K prefill GEMM.  Pass one expands the weights once per call into

@@ -227,7 +227,11 @@ extern "C" __global__ __launch_bounds__(256) void jl_mxfp4_prep(MxPrepArgs p) {
 }
 extern "C" __global__ __launch_bounds__(256) void jl_moe_gemm_prep(MoeGemmPrepArgs p) {
     __shared__ u32 lds[JL_GEMM_PREP_LDS_WORDS];
-    moe_gemm_prep_body(p, lds);
+    moe_gemm_prep_body<false>(p, lds);
+}
+extern "C" __global__ __launch_bounds__(256) void jl_moe_gemm_prep_planes(MoeGemmPrepArgs p) {
+    __shared__ u32 lds[JL_GEMM_PREP_LDS_WORDS];
+    moe_gemm_prep_body<true>(p, lds);
 }
 extern "C" __global__ __launch_bounds__(256, 2) void jl_moe_gemm_q4k(MoeGemmArgs p) { moe_gemm_q4k_body(p, jl_smem); }
 // Experts with many columns: the prefill GEMM's 128-token x 64-row tile placed per expert.  An
@@ -235,7 +239,9 @@ extern "C" __global__ __launch_bounds__(256, 2) void jl_moe_gemm_q4k(MoeGemmArgs
 // are a token range; columns past the expert's last are computed and not stored.  The
 // workgroups stride over (row tile, column tile of the work list, matrix), so none is empty.
 // grid = up to two workgroups a CU, block = 256, dynamic LDS as jl_gemm_q4k_r64.
-template <int TYPE>
+// PL (Q4_K): the banks are packed planes, an expert's sheet a plane set of its own or a row range
+// of the bank's (MoeGemmArgs.pqs ...); the tile is the plane form of the prefill GEMM's.
+template <int TYPE, bool PL = false>
 __device__ __forceinline__ void moe_gemm_tiles(const MoeGemmArgs& p) {
     const u32 rtiles = (u32)(p.nrows + 63) / 64;
     const u32 ntiles = p.wl[0];
@@ -249,7 +255,14 @@ __device__ __forceinline__ void moe_gemm_tiles(const MoeGemmArgs& p) {
         const int ncol = (int)(c_hi - c_lo);
         const int slot0 = (int)(c_lo >> 5) + e;
         GemmArgs g;
-        g.w = p.bank[mat] + (size_t)e * p.sheet_bytes;
+        if (PL) {
+            const size_t ew = (size_t)e * p.sheet_words;
+            g.pqs = p.pqs[mat] + ew; g.pd = p.pd[mat] + ew; g.psc = p.psc[mat] + ew;
+            g.prow0 = e * p.row_step; g.pstride = p.pstride; g.psb0 = 0;
+            g.w = nullptr;
+        } else {
+            g.w = p.bank[mat] + (size_t)e * p.sheet_bytes;
+        }
         g.bq = p.bq; g.da = p.da;
         g.nrows = p.nrows; g.k = p.k; g.row_bytes = p.row_bytes;
         g.tok_pad = 32 * p.nslots;
@@ -257,11 +270,12 @@ __device__ __forceinline__ void moe_gemm_tiles(const MoeGemmArgs& p) {
         g.out_stride = p.nrows; g.sb_per = 0;
         g.out = p.out[mat] + ((ptrdiff_t)c_lo - (ptrdiff_t)32 * slot0) * p.nrows;   // workspace position -> column
         if constexpr (TYPE == JL_Q6_K) gemm_q6k_body(g, jl_smem, 32 * slot0 + 128 * ctile, (int)rt * 64);
-        else gemm_q4k_body<1, true>(g, jl_smem, 32 * slot0 + 128 * ctile, (int)rt * 64);
+        else gemm_q4k_body<1, true, PL>(g, jl_smem, 32 * slot0 + 128 * ctile, (int)rt * 64);
         __syncthreads();   // the tile's LDS is free for the next one
     }
 }
 extern "C" __global__ __launch_bounds__(256, 2) void jl_moe_gemm_r64(MoeGemmArgs p) { moe_gemm_tiles<JL_Q4_K>(p); }
+extern "C" __global__ __launch_bounds__(256, 2) void jl_moe_gemm_r64_planes(MoeGemmArgs p) { moe_gemm_tiles<JL_Q4_K, true>(p); }
 // Q6_K sheets: dynamic LDS = JL_GEMM6_LDS_BYTES
 extern "C" __global__ __launch_bounds__(256, 2) void jl_moe_gemm_q6k_r64(MoeGemmArgs p) { moe_gemm_tiles<JL_Q6_K>(p); }
 // grid = 1, block = 1024

@@ -530,6 +530,8 @@ __device__ __forceinline__ void moe_worklist_body(const MoeWorklistArgs& p, u32*
 
 // Activation prep: grid = (k/256, nslots), block = 256: one group of 32 columns, one
 // super-block; tokens past the expert's last column are zeros.
+// PL: the K order of the plane-reading tile kernel (gemm_q4k.h).
+template <bool PL = false>
 __device__ __forceinline__ void moe_gemm_prep_body(const MoeGemmPrepArgs& p, u32* lds) {
     const int lane = threadIdx.x & 63;
     const int sb = blockIdx.x, slot = blockIdx.y;
@@ -538,7 +540,7 @@ __device__ __forceinline__ void moe_gemm_prep_body(const MoeGemmPrepArgs& p, u32
     const int e = (int)eu;
     const u32 c_lo = p.start[e], c_hi = p.start[e + 1];
     const u32 c0 = c_lo + 32 * (u32)(slot - ((int)(c_lo >> 5) + e));
-    gemm_prep_group<4>(lds, sb, slot, p.nslots, p.bq, p.da, [&](int tl) {
+    gemm_prep_group<4, PL>(lds, sb, slot, p.nslots, p.bq, p.da, [&](int tl) {
         f32x4 v = f32x4{0.f, 0.f, 0.f, 0.f};
         const u32 c = c0 + tl;
         if (c < c_hi) {

@@ -290,6 +290,27 @@ class Device:
                                                       opt(bank1), _ptr(x), opt(x2), opt(src), _ptr(start),
                                                       n_expert, ncols, nrows, k, stream), "jl_moe_matvec_dev")
 
+    @staticmethod
+    def packed_bank(qs, d, sc, sheet_bytes, stride):
+        """jl_packed_bank: expert 0's planes (device addresses); sheet_bytes between experts' sheets
+        (0: one plane set of `stride` rows holding every expert)."""
+        return _lib.PackedBank(_ptr(qs), _ptr(d), _ptr(sc), int(sheet_bytes), int(stride))
+
+    def moe_matvec_packed_dev(self, out0, out1, t, bank0, bank1, x, x2, src, start, n_expert, ncols, nrows, k,
+                              stream=None):
+        """jl_moe_matvec_dev over banks of packed planes (packed_bank(...))."""
+        opt = lambda a: None if a is None else _ptr(a)
+        return self._served(self._l.jl_moe_matvec_packed_dev(
+            self._ctx, _ptr(out0), opt(out1), t, C.byref(bank0), None if bank1 is None else C.byref(bank1), _ptr(x),
+            opt(x2), opt(src), _ptr(start), n_expert, ncols, nrows, k, stream), "jl_moe_matvec_packed_dev")
+
+    def moe_ffn_packed_dev(self, resid, t, gate, up, down, x, sel, sel_stride, wt, rows, k_used, n_expert, n_ffn,
+                           n_embd, stream=None):
+        """One routed feed-forward block over banks of packed planes."""
+        return self._served(self._l.jl_moe_ffn_packed_dev(
+            self._ctx, _ptr(resid), t, C.byref(gate), C.byref(up), C.byref(down), _ptr(x), _ptr(sel), sel_stride,
+            _ptr(wt), rows, k_used, n_expert, n_ffn, n_embd, stream), "jl_moe_ffn_packed_dev")
+
     def moe_combine_dev(self, resid, y, wt, sel, sel_stride, pos, rows, k_used, n_embd, stream=None):
         return self._served(self._l.jl_moe_combine_dev(self._ctx, _ptr(resid), _ptr(y), _ptr(wt), _ptr(sel),
                                                        sel_stride, _ptr(pos), rows, k_used, n_embd, stream),

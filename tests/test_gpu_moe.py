@@ -7,6 +7,8 @@ Stages are checked on their own so each is like-for-like: grouping is integer wo
 same sums in the same order; the whole block to rel-L2 <= 1e-3 against a pure-oracle
 evaluation (the down projection re-quantizes act(gate)*up, so a last-bit difference in
 gate/up can move an int8: the block is not a like-for-like quantity)."""
+import functools
+
 import numpy as np
 import pytest
 
@@ -239,6 +241,21 @@ def _oracle_block(t, gate, up, down, x, sel, wt, n_expert, n_ffn, n_embd, window
     return out
 
 
+@functools.lru_cache(maxsize=None)
+def _block_case(shape):
+    """Seeded banks, routing, activations and the oracle's value of a whole block (computed once:
+    the Qwen3 shape takes the oracle ten seconds)."""
+    rows, n_expert, k_used, n_ffn, n_embd = shape
+    t, window = quant.Q4_K, 256
+    sel, wt = route(rows, n_expert, k_used, 11)
+    gate = _banks(t, n_expert, n_ffn, n_embd, 1000, False)
+    up = _banks(t, n_expert, n_ffn, n_embd, 2000, False)
+    down = _banks(t, n_expert, n_embd, n_ffn, 3000, False)
+    x = np.stack([synth.activations(n_embd, seed=500 + r) for r in range(rows)])
+    want = _oracle_block(t, gate, up, down, x, sel, wt, n_expert, n_ffn, n_embd, window)
+    return sel, wt, gate, up, down, x, want
+
+
 @pytest.mark.parametrize("shape", [(6, 8, 2, 256, 512), (64, 128, 8, 768, 2048)],
                          ids=["tiny", "qwen3-30b-a3b"])
 def test_moe_block_vs_oracle(dev, devbuf, shape):
@@ -247,12 +264,7 @@ def test_moe_block_vs_oracle(dev, devbuf, shape):
     rows, n_expert, k_used, n_ffn, n_embd = shape
     t, window = quant.Q4_K, 256
     dev.SetActWindow(window)
-    sel, wt = route(rows, n_expert, k_used, 11)
-    gate = _banks(t, n_expert, n_ffn, n_embd, 1000, False)
-    up = _banks(t, n_expert, n_ffn, n_embd, 2000, False)
-    down = _banks(t, n_expert, n_embd, n_ffn, 3000, False)
-    x = np.stack([synth.activations(n_embd, seed=500 + r) for r in range(rows)])
-    want = _oracle_block(t, gate, up, down, x, sel, wt, n_expert, n_ffn, n_embd, window)
+    sel, wt, gate, up, down, x, want = _block_case(shape)
     gd, ud, dd, xd, sd, wd = devbuf(gate), devbuf(up), devbuf(down), devbuf(x), devbuf(sel), devbuf(wt)
     resid = devbuf(shape=(rows, n_embd), dtype=np.float32, fill=0)
     for call in range(2):
@@ -360,3 +372,151 @@ def test_router_logits_bit_exact_then_route(dev, devbuf, case, form):
     # only f32 and f16 router weights are served
     assert dev.moe_logits_dev(ld.ptr, 8, wd.ptr, xd.ptr, n_expert, k, ntok) is False
     dev.set_tuning(moe__logits=0)
+
+
+def _pack_bank(dev, devbuf, t, bank, n_expert, nrows, k, layout):
+    """A GGUF bank -> packed planes on the device.  layout "sheets": every expert's sheet packed
+    on its own, plane sets `page` bytes apart as a container's expert pages are
+    (/root/reference/format/jlm/write.go:123-180); "one": the whole bank packed as one matrix of
+    n_expert * nrows rows.  Returns (jl_packed_bank, buffers to keep alive)."""
+    sheet = nrows * quant.row_bytes(t, k)
+    if layout == "one":
+        qs, d, sc = oracle.pack_weights(t, bank, n_expert * nrows, k)
+        bufs = [devbuf(qs), devbuf(d), devbuf(sc)]
+        return dev.packed_bank(bufs[0].ptr, bufs[1].ptr, bufs[2].ptr, 0, n_expert * nrows), bufs
+    nq, nd, nsc = oracle.packed_words(t, nrows, k)
+    o_d, o_sc = 4 * nq, 4 * (nq + nd)
+    page = (4 * (nq + nd + nsc) + 4095) // 4096 * 4096 + 4096       # a page size, with slack between sheets
+    host = np.full(page * n_expert, 0xA5, np.uint8)                 # poison between the sheets
+    for e in range(n_expert):
+        qs, d, sc = oracle.pack_weights(t, bank[e * sheet:(e + 1) * sheet], nrows, k)
+        base = e * page
+        host[base:base + o_d] = qs.view(np.uint8)
+        host[base + o_d:base + o_sc] = d.view(np.uint8)
+        host[base + o_sc:base + o_sc + 4 * nsc] = sc.view(np.uint8)
+    buf = devbuf(host)
+    return dev.packed_bank(buf.ptr, buf.ptr + o_d, buf.ptr + o_sc, page, nrows), [buf]
+
+
+@pytest.mark.parametrize("layout", ["sheets", "one"])
+@pytest.mark.parametrize("nrows,k", [(96, 2048), (200, 768), (16, 256)])
+def test_grouped_matvec_over_packed_expert_sheets(dev, devbuf, layout, nrows, k):
+    """jl_moe_matvec_packed_dev: the banks as packed planes, expert sheets packed on their own a
+    page apart (a container's expert pages) or as row ranges of one plane set; against the
+    oracle over the same bytes, and bit for bit against the tile form over the GGUF banks."""
+    t, rows, n_expert, k_used, window = quant.Q4_K, 13, 8, 3, 256
+    dev.SetActWindow(window)
+    sel, _ = route(rows, n_expert, k_used, 4)
+    sel[1:12, 0], sel[1:12, 1], sel[1:12, 2] = 6, 0, 7
+    used, perm, col_e, pos = oracle.group_pairs(sel.reshape(-1), rows, k_used, n_expert, 1)
+    start = np.searchsorted(col_e[:used], np.arange(n_expert + 1)).astype(np.uint32)
+    bank0 = _banks(t, n_expert, nrows, k, 10, False)
+    bank1 = _banks(t, n_expert, nrows, k, 50, True)
+    x = np.stack([synth.activations(k, seed=200 + r) for r in range(rows)])
+    sheet = nrows * quant.row_bytes(t, k)
+    want0, want1 = np.zeros((used, nrows)), np.zeros((used, nrows))
+    for c in range(used):
+        e = int(col_e[c])
+        q, a_s, _ = oracle.quantize_act(x[perm[c]], window)
+        want0[c] = oracle.matvec_q8act_f64(t, bank0[e * sheet:(e + 1) * sheet], q, a_s, nrows, k)
+        want1[c] = oracle.matvec_q8act_f64(t, bank1[e * sheet:(e + 1) * sheet], q, a_s, nrows, k)
+    pb0, keep0 = _pack_bank(dev, devbuf, t, bank0, n_expert, nrows, k, layout)
+    pb1, keep1 = _pack_bank(dev, devbuf, t, bank1, n_expert, nrows, k, layout)
+    xd, dstart, dperm = devbuf(x), devbuf(start), devbuf(perm[:used].copy())
+    o0 = devbuf(shape=(used * nrows + 8,), dtype=np.float32, fill=np.float32(4e30))
+    o1 = devbuf(shape=(used * nrows + 8,), dtype=np.float32, fill=np.float32(4e30))
+    assert dev.moe_matvec_packed_dev(o0.ptr, o1.ptr, t, pb0, pb1, xd.ptr, None, dperm.ptr, dstart.ptr, n_expert, used,
+                                     nrows, k)
+    dev.synchronize()
+    g0, g1 = o0.get(), o1.get()
+    assert np.all(g0[used * nrows:] == np.float32(4e30)) and np.all(g1[used * nrows:] == np.float32(4e30))
+    assert nmse(g0[:used * nrows].reshape(used, nrows), want0) <= 1e-10
+    assert nmse(g1[:used * nrows].reshape(used, nrows), want1) <= 1e-10
+    # the tile form over the same weights as GGUF banks: the same integers, the same epilogue
+    b0, b1 = devbuf(bank0), devbuf(bank1)
+    r0 = devbuf(shape=(used * nrows,), dtype=np.float32, fill=0)
+    r1 = devbuf(shape=(used * nrows,), dtype=np.float32, fill=0)
+    dev.set_tuning(moe__form=4)
+    assert dev.moe_matvec_dev(r0.ptr, r1.ptr, t, b0.ptr, b1.ptr, xd.ptr, None, dperm.ptr, dstart.ptr, n_expert, used,
+                              nrows, k)
+    dev.synchronize()
+    dev.set_tuning(moe__form=0)
+    assert np.array_equal(g0[:used * nrows].view(np.uint32), r0.get().view(np.uint32))
+    assert np.array_equal(g1[:used * nrows].view(np.uint32), r1.get().view(np.uint32))
+    # what the plane form does not serve is declined, never approximated
+    dev.SetActWindow(32)
+    assert not dev.moe_matvec_packed_dev(o0.ptr, None, t, pb0, None, xd.ptr, None, dperm.ptr, dstart.ptr, n_expert,
+                                         used, nrows, k)
+    assert not dev.moe_matvec_packed_dev(o0.ptr, None, quant.Q6_K, pb0, None, xd.ptr, None, dperm.ptr, dstart.ptr,
+                                         n_expert, used, nrows, k)
+
+
+def test_grouped_matvec_over_the_expert_pages_of_the_reference_written_container(dev, devbuf):
+    """The four exp_gate_bank sheets of each block of v29.jlm.gz, uploaded as the file holds them
+    (one device copy of the container's bytes, the bank addressed by the entry's plane offsets
+    and the header's expert page size, /root/reference/format/jlm/read.go:447-469) and fed to
+    the mixture's grouped matvec; the expectation comes from the regenerated GGUF source
+    bytes, which are independent of the packing."""
+    import os
+    from conftest import GOLDEN
+    from v29_source import source_tensors
+    from jitllm_amd import jlm
+    f = jlm.File.open(os.path.join(GOLDEN, "v29.jlm.gz"))
+    src = {(n, b): p for n, b, kind, p in source_tensors() if kind == "q4k"}
+    t, window = quant.Q4_K, 256
+    dev.SetActWindow(window)
+    data = np.frombuffer(f.data, np.uint8)
+    file_d = devbuf(np.concatenate([data, np.zeros((-len(data)) % 16, np.uint8)]))
+    seen = 0
+    for e in f.entries:
+        if e.name != "exp_gate_bank":
+            continue
+        n_expert, nrows, k = e.sheets, e.rows, e.k
+        assert (n_expert, nrows, k) == (4, 16, 256)
+        pb = dev.packed_bank(file_d.ptr + e.qs_off, file_d.ptr + e.d_off, file_d.ptr + e.sc_off, f.exp_page_size, nrows)
+        rows, k_used = 9, 2
+        sel = np.zeros((rows, k_used + 1), np.uint32)
+        sel[:, 0] = np.arange(rows) % n_expert
+        sel[:, 1] = (np.arange(rows) + 1 + e.block) % n_expert
+        used, perm, col_e, pos = oracle.group_pairs(sel.reshape(-1), rows, k_used, n_expert, 1)
+        start = np.searchsorted(col_e[:used], np.arange(n_expert + 1)).astype(np.uint32)
+        x = np.stack([synth.activations(k, seed=40 + r) for r in range(rows)])
+        bank = src[(e.name, e.block)]
+        sheet = nrows * quant.row_bytes(t, k)
+        want = np.zeros((used, nrows))
+        for c in range(used):
+            q, a_s, _ = oracle.quantize_act(x[perm[c]], window)
+            ex = int(col_e[c])
+            want[c] = oracle.matvec_q8act_f64(t, bank[ex * sheet:(ex + 1) * sheet], q, a_s, nrows, k)
+        xd, dstart, dperm = devbuf(x), devbuf(start), devbuf(perm[:used].copy())
+        o = devbuf(shape=(used, nrows), dtype=np.float32, fill=np.float32(4e30))
+        assert dev.moe_matvec_packed_dev(o.ptr, None, t, pb, None, xd.ptr, None, dperm.ptr, dstart.ptr, n_expert, used,
+                                         nrows, k)
+        dev.synchronize()
+        assert nmse(o.get(), want) <= 1e-10, (e.name, e.block)
+        seen += 1
+    assert seen == 2
+    dev.SetActWindow(32)
+
+
+@pytest.mark.parametrize("layout", ["sheets", "one"])
+@pytest.mark.parametrize("shape", [(6, 8, 2, 256, 512), (64, 128, 8, 768, 2048)], ids=["tiny", "qwen3-30b-a3b"])
+def test_moe_block_over_packed_banks_vs_oracle(dev, devbuf, shape, layout):
+    """The whole routed feed-forward block with the three banks as packed planes."""
+    rows, n_expert, k_used, n_ffn, n_embd = shape
+    t, window = quant.Q4_K, 256
+    dev.SetActWindow(window)
+    sel, wt, gate, up, down, x, want = _block_case(shape)
+    pg, k0 = _pack_bank(dev, devbuf, t, gate, n_expert, n_ffn, n_embd, layout)
+    pu, k1 = _pack_bank(dev, devbuf, t, up, n_expert, n_ffn, n_embd, layout)
+    pd, k2 = _pack_bank(dev, devbuf, t, down, n_expert, n_embd, n_ffn, layout)
+    xd, sd, wd = devbuf(x), devbuf(sel), devbuf(wt)
+    resid = devbuf(shape=(rows, n_embd), dtype=np.float32, fill=0)
+    for call in range(2):
+        resid.put(np.zeros((rows, n_embd), np.float32))
+        assert dev.moe_ffn_packed_dev(resid.ptr, t, pg, pu, pd, xd.ptr, sd.ptr, k_used + 1, wd.ptr, rows, k_used,
+                                      n_expert, n_ffn, n_embd)
+        dev.synchronize()
+        got = resid.get()
+        assert rel_l2(got, want) <= 1e-3, f"call {call}: rel-L2 {rel_l2(got, want):.3e}"
+    dev.SetActWindow(32)
