@@ -374,6 +374,9 @@ int moe_matvec_launch(jl_ctx* c, float* out0, float* out1, int type, const void*
                       int n_expert, int ncols, int nrows, int k, hipStream_t st,
                       const jl_packed_bank* pb0 = nullptr, const jl_packed_bank* pb1 = nullptr);
 
+// plane banks of a mixture: from this many columns an expert (on average) the matrix-core tile
+// per expert takes over from the dot-product form ("moe.form" = 1 / 4 forces one)
+constexpr long kMoePlaneTileCols = 14;
 constexpr int kGemmTile = 128;         // tokens and rows per workgroup (kernels/gemm_q4k.h)
 constexpr int kGemmStride = 152;       // f16 per stage row
 constexpr unsigned gemm_lds_bytes(int rows) {   // two weight stages, row scales, token scales
@@ -920,6 +923,36 @@ int moe_matvec_launch(jl_ctx* c, float* out0, float* out1, int type, const void*
     // Q6_K sheets (the down projections of a model whose other experts are Q4_K) have form 4
     // alone, with the Q6_K GEMM's tile; the dot-product kernel is slower for that type, so the
     // tile takes over earlier ("moe.q6k_cols": columns an expert on average, default 12).
+    if (planes && c->tune.moe_form != 4 && (c->tune.moe_form == 1 || (long)ncols < kMoePlaneTileCols * n_expert)) {
+        // few columns an expert: the dot-product form over planes (rows on lanes, a lane's share of a
+        // chunk loaded once for all the expert's columns, the columns as scalar operands)
+        if ((size_t)ncols * (k / 256) * 88 >= ((size_t)1 << 32)) return JL_DECLINED;   // 32-bit word offsets in the kernel
+        // the columns quantized once, chunk by chunk: 88 words a (column, 256 elements)
+        rc = ws_ensure(c, &c->moe_q_ws, &c->moe_q_ws_bytes, (size_t)ncols * (k / 256) * 88 * 4);
+        if (rc != JL_OK) return rc;
+        MoeQuantArgs qa;
+        qa.x = x; qa.x2 = x2; qa.src = src;
+        qa.q = nullptr; qa.as = nullptr; qa.s16 = nullptr; qa.chunked = (uint32_t*)c->moe_q_ws;
+        qa.k = k; qa.per = c->act_window / 32;
+        void* qparams[] = {&qa};
+        rc = launch(c, "jl_moe_quant", (unsigned)((k / 4 + 255) / 256), (unsigned)ncols, 256, 0, st, qparams);
+        if (rc != JL_OK) return rc;
+        MoePlanesArgs a;
+        const jl_packed_bank* pbs[2] = {pb0, pb1};
+        const int nmat = pb1 ? 2 : 1;
+        for (int m = 0; m < 2; m++) {
+            a.out[m] = m == 0 ? out0 : out1;
+            a.pqs[m] = m < nmat ? pbs[m]->qs : nullptr; a.pd[m] = m < nmat ? pbs[m]->d : nullptr;
+            a.psc[m] = m < nmat ? pbs[m]->sc : nullptr;
+        }
+        a.chunked = qa.chunked; a.start = start;
+        a.sheet_words = pb0->sheet_bytes / 4; a.row_step = pb0->sheet_bytes ? 0 : nrows; a.pstride = pb0->stride;
+        a.nrows = nrows; a.k = k;
+        a.nwaves = std::min(8, k / 256);
+        void* params[] = {&a};
+        return launch(c, "jl_moe_matvec_planes_q4k", (unsigned)((nrows + 63) / 64), (unsigned)n_expert, (unsigned)(a.nwaves * 64),
+                      (unsigned)(a.nwaves * 8 * 256), st, params, (unsigned)nmat);   // JL_MOEP_TB columns a pass
+    }
     const bool q6 = type == JL_TYPE_Q6_K;
     const long q6_cols = c->tune.moe_q6k_cols > 0 ? c->tune.moe_q6k_cols : 12;
     const bool many_cols = c->tune.moe_form == 0 && (long)ncols >= (q6 ? q6_cols : 10L) * n_expert;
@@ -1098,7 +1131,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     if (e != hipSuccess)
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
-    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_prep_q4k_planes", "jl_gemm_q4k_r64_planes", "jl_gemm_q4k_wide_planes", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_group2_wide", "jl_moe_quant", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_prep_planes", "jl_moe_gemm_q4k", "jl_moe_gemm_r64", "jl_moe_gemm_r64_planes", "jl_moe_gemm_q6k_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_sum_parts", "jl_probe_read", "jl_probe_empty", "jl_probe_wait",
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_prep_q4k_planes", "jl_gemm_q4k_r64_planes", "jl_gemm_q4k_wide_planes", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_group2_wide", "jl_moe_quant", "jl_moe_matvec_planes_q4k", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_prep_planes", "jl_moe_gemm_q4k", "jl_moe_gemm_r64", "jl_moe_gemm_r64_planes", "jl_moe_gemm_q6k_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_sum_parts", "jl_probe_read", "jl_probe_empty", "jl_probe_wait",
                                       "jl_pack_weights", "jl_unpack_q4k", "jl_unpack_q6k", "jl_unpack_q8_0"};
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int rw : {16, 32, 64})

@@ -183,6 +183,10 @@ struct MoeQuantArgs {
     float* as;
     float* s16;
     int k, per;
+    // chunked form (q, as, s16 unused): column c's 256-element chunk i as 88 consecutive words at
+    // chunked + (c * k/256 + i) * 88 -- 64 of int8 values, 8 scales, 16 half-block sums -- so a
+    // reader addresses everything it needs of a (column, chunk) from one base
+    uint32_t* chunked = nullptr;
 };
 
 // Grouped expert matvec over columns sorted by expert: out[m][c][0:nrows] =
@@ -198,6 +202,23 @@ struct MoeMatVecArgs {
     int nrows, k, row_bytes;
     int nwaves;             // wavefronts per workgroup
     int shares;             // workgroups one (expert, matrix) is split into, by rows
+};
+
+// The same over banks of packed planes (moe_matvec_planes_body): expert e's planes are
+// pqs / pd / psc [m] + e * sheet_words (u32 words; 0 when a bank is ONE plane set), its first
+// row e * row_step inside them (0 when every expert has a sheet of its own), pstride rows a
+// plane set.
+struct MoePlanesArgs {
+    float* out[2];
+    const uint32_t* pqs[2];
+    const uint32_t* pd[2];
+    const uint32_t* psc[2];
+    const uint32_t* chunked;   // the columns, quantized in the chunked form (MoeQuantArgs.chunked)
+    const uint32_t* start;  // [n_expert + 1]
+    size_t sheet_words;
+    int row_step, pstride;
+    int nrows, k;
+    int nwaves;             // wavefronts per workgroup: they split the 256-element chunks of K
 };
 
 struct MoeCombineArgs {

@@ -212,6 +212,11 @@ JL_MOE_KERNEL(q8_0, JL_Q8_0, 4) JL_MOE_KERNEL(q8_0, JL_Q8_0, 8)
 JL_MOE_KERNEL(q8_0, JL_Q8_0, 16) JL_MOE_KERNEL(q8_0, JL_Q8_0, 32) JL_MOE_KERNEL(q8_0, JL_Q8_0, 64)
 JL_MOE_KERNEL(q6k, JL_Q6_K, 4) JL_MOE_KERNEL(q6k, JL_Q6_K, 8)
 JL_MOE_KERNEL(q6k, JL_Q6_K, 16) JL_MOE_KERNEL(q6k, JL_Q6_K, 32) JL_MOE_KERNEL(q6k, JL_Q6_K, 64)
+// banks of packed planes: grid = (ceil(nrows/64), n_expert, matrices), block = 64 * wavefronts (<= 8),
+// dynamic LDS = wavefronts * JL_MOEP_TB * 256
+extern "C" __global__ __launch_bounds__(512) void jl_moe_matvec_planes_q4k(MoePlanesArgs p) {
+    moe_matvec_planes_body(p, jl_smem);
+}
 // grid = (ceil(n_embd/256), rows), block = 256
 extern "C" __global__ __launch_bounds__(256) void jl_moe_combine(MoeCombineArgs p) {
     __shared__ float swt[16];

@@ -336,6 +336,110 @@ __device__ __forceinline__ float group_sum(float v) {
     return v;
 }
 
+// ------------------------------------------------- grouped matvec, packed planes
+// The dot-product form over banks of packed planes, for a handful of columns an expert (a small
+// prefill batch through a mixture: 64 rows top-8 of 128 experts is four columns an expert).
+// The planes put a word of one row beside the same word of the next row, so rows go on LANES:
+// a workgroup owns 64 rows of one expert's sheet, its wavefronts split K in chunks of 256
+// elements (one super-block), and a lane loads its row's share of a chunk -- 32 words of
+// nibbles, three of scales, one of (d, dmin), every load 256 contiguous bytes a wavefront --
+// exactly once, whatever the number of columns.  The chunk's scale arithmetic is done once;
+// then the expert's columns pass by, eight at a time.  A column's int8 values, scales and sums
+// are the SAME for every lane of the wavefront (all lanes work on the same chunk), so they are
+// read through the scalar cache into scalar registers and meet the weights as scalar operands
+// of the dot instructions: no LDS traffic, no staging, no barrier inside the loop.  The column
+// quantizer lays a (column, chunk) out as 88 consecutive words for this reader
+// (MoeQuantArgs.chunked), read as 32-bit words and bit-cast: the kernel stores floats, and a
+// float load that a float store might alias would not be made a scalar load.  The wavefronts'
+// partial sums meet in LDS at the end and are added in wavefront order.
+// (A form with one wavefront a workgroup walking all of K, its scalar loads pipelined by hand,
+// measured 2.1x slower at the 128-expert shape: few, long wavefronts expose every scalar
+// round trip, many short ones cover each other.)
+// Q4_K.  grid = (ceil(nrows/64), n_expert, matrices), block = 64 * nwaves (<= 8),
+// dynamic LDS = nwaves * JL_MOEP_TB * 64 * 4.
+#define JL_MOEP_TB 8   // columns a pass
+
+__device__ __forceinline__ void moe_matvec_planes_body(const MoePlanesArgs& p, uint8_t* smem) {
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), nwaves = p.nwaves;
+    const int e = blockIdx.y, mat = blockIdx.z;
+    // (the same in every lane: in scalar registers, so that what depends on them is scalar too)
+    const u32 c_lo = (u32)__builtin_amdgcn_readfirstlane((int)p.start[e]);
+    const u32 c_hi = (u32)__builtin_amdgcn_readfirstlane((int)p.start[e + 1]);
+    if (c_lo == c_hi) return;   // nobody chose this expert (uniform across the workgroup)
+    const int r_l = blockIdx.x * 64 + lane;
+    const size_t st = (size_t)p.pstride;
+    const size_t row = (size_t)e * p.row_step + min(r_l, p.nrows - 1);
+    const size_t ew = (size_t)e * p.sheet_words;
+    const u32* pqs = p.pqs[mat] + ew + row;
+    const u32* pd = p.pd[mat] + ew + row;
+    const u32* psc = p.psc[mat] + ew + row;
+    float* red = (float*)smem;   // [nwaves][JL_MOEP_TB][64]
+    const int nchunks = p.k / 256;
+    const u32 M = 0x0F0F0F0Fu;
+
+    for (u32 c0 = c_lo; c0 < c_hi; c0 += JL_MOEP_TB) {
+        const int ncol = (int)min((u32)JL_MOEP_TB, c_hi - c0);   // uniform
+        float acc[JL_MOEP_TB];
+#pragma unroll
+        for (int j = 0; j < JL_MOEP_TB; j++) acc[j] = 0.f;
+        for (int c = wave; c < nchunks; c += nwaves) {
+            // this row's chunk: (d, dmin), the 96-bit stream of 6-bit scales and minimums, 8 x 4 words
+            const u32 dw = pd[(size_t)c * st];
+            const u32 s0 = psc[(size_t)(3 * c) * st], s1 = psc[(size_t)(3 * c + 1) * st], s2 = psc[(size_t)(3 * c + 2) * st];
+            u32 wq[8][4];
+#pragma unroll
+            for (int s = 0; s < 8; s++)
+#pragma unroll
+                for (int w = 0; w < 4; w++) wq[s][w] = pqs[(size_t)((c * 8 + s) * 4 + w) * st];
+            const float d = half_bits_to_f32((uint16_t)(dw & 0xFFFF)), dmin = half_bits_to_f32((uint16_t)(dw >> 16));
+            const uint64_t lo = s0 | ((uint64_t)s1 << 32), hi = s1 | ((uint64_t)s2 << 32);
+            float dsc[8], dm[8];
+#pragma unroll
+            for (int s = 0; s < 8; s++) {
+                const int bit = 12 * s;
+                const u32 f = bit < 32 ? (u32)(lo >> bit) : (u32)(hi >> (bit - 32));
+                dsc[s] = d * (float)(f & 63);
+                dm[s] = dmin * (float)((f >> 6) & 63);
+            }
+#pragma unroll
+            for (int j = 0; j < JL_MOEP_TB; j++) {
+                if (j < ncol) {   // uniform
+                    // column c0 + j, chunk c: the same address in every lane -> scalar loads, one
+                    // base and immediate offsets
+                    const u32* cb = p.chunked + ((size_t)(c0 + j) * nchunks + c) * 88;
+                    float t = acc[j];
+#pragma unroll
+                    for (int s = 0; s < 8; s++) {
+                        i32 dt = 0;
+#pragma unroll
+                        for (int w = 0; w < 4; w++) {
+                            dt = dot4(wq[s][w] & M, cb[8 * s + w], dt);
+                            dt = dot4((wq[s][w] >> 4) & M, cb[8 * s + 4 + w], dt);
+                        }
+                        const float sa = __uint_as_float(cb[72 + 2 * s]) + __uint_as_float(cb[73 + 2 * s]);
+                        const float v = (float)dt * dsc[s] - sa * dm[s];
+                        t = fmaf(v, __uint_as_float(cb[64 + s]), t);
+                    }
+                    acc[j] = t;
+                }
+            }
+        }
+        // the wavefronts' shares of K meet in LDS and are added in wavefront order
+#pragma unroll
+        for (int j = 0; j < JL_MOEP_TB; j++) red[(wave * JL_MOEP_TB + j) * 64 + lane] = acc[j];
+        __syncthreads();
+        for (int i = threadIdx.x; i < ncol * 64; i += nwaves * 64) {
+            const int j = i >> 6, l = i & 63;
+            float sum = red[j * 64 + l];
+            for (int w = 1; w < nwaves; w++) sum += red[(w * JL_MOEP_TB + j) * 64 + l];
+            const int r = blockIdx.x * 64 + l;
+            if (r < p.nrows) p.out[mat][(size_t)(c0 + j) * p.nrows + r] = sum;
+        }
+        __syncthreads();   // red is free for the next pass
+    }
+}
+
 // --------------------------------------------------------- column activations
 // grid = (ceil(k/4/256), ncols), block = 256: one thread per four elements of a column.
 __device__ __forceinline__ void moe_quant_body(const MoeQuantArgs& p) {
@@ -356,7 +460,13 @@ __device__ __forceinline__ void moe_quant_body(const MoeQuantArgs& p) {
     float d;
     i32 sum;
     u32 qq = quantize4(v, amax, d, sum);
-    if (live) {
+    if (live && p.chunked) {
+        const int within = g4 & 63;
+        u32* cb = p.chunked + (c * (size_t)(p.k / 256) + (size_t)(g4 >> 6)) * 88;
+        cb[within] = qq;
+        if ((g4 & 3) == 0) cb[72 + (within >> 2)] = __float_as_uint((float)sum);
+        if ((g4 & 7) == 0) cb[64 + (within >> 3)] = __float_as_uint(d);
+    } else if (live) {
         ((u32*)(p.q + c * (size_t)p.k))[g4] = qq;
         if ((g4 & 3) == 0) p.s16[c * (size_t)(p.k / 16) + (g4 >> 2)] = (float)sum;
         if ((g4 & 7) == 0) p.as[c * (size_t)(p.k / 32) + (g4 >> 3)] = d;

@@ -402,8 +402,9 @@ def _pack_bank(dev, devbuf, t, bank, n_expert, nrows, k, layout):
 @pytest.mark.parametrize("nrows,k", [(96, 2048), (200, 768), (16, 256)])
 def test_grouped_matvec_over_packed_expert_sheets(dev, devbuf, layout, nrows, k):
     """jl_moe_matvec_packed_dev: the banks as packed planes, expert sheets packed on their own a
-    page apart (a container's expert pages) or as row ranges of one plane set; against the
-    oracle over the same bytes, and bit for bit against the tile form over the GGUF banks."""
+    page apart (a container's expert pages) or as row ranges of one plane set; both forms (rows
+    on lanes with the columns as scalar operands; the matrix-core tile per expert) against the
+    oracle over the same bytes, the tile also bit for bit against the tile over the GGUF banks."""
     t, rows, n_expert, k_used, window = quant.Q4_K, 13, 8, 3, 256
     dev.SetActWindow(window)
     sel, _ = route(rows, n_expert, k_used, 4)
@@ -425,13 +426,18 @@ def test_grouped_matvec_over_packed_expert_sheets(dev, devbuf, layout, nrows, k)
     xd, dstart, dperm = devbuf(x), devbuf(start), devbuf(perm[:used].copy())
     o0 = devbuf(shape=(used * nrows + 8,), dtype=np.float32, fill=np.float32(4e30))
     o1 = devbuf(shape=(used * nrows + 8,), dtype=np.float32, fill=np.float32(4e30))
-    assert dev.moe_matvec_packed_dev(o0.ptr, o1.ptr, t, pb0, pb1, xd.ptr, None, dperm.ptr, dstart.ptr, n_expert, used,
-                                     nrows, k)
-    dev.synchronize()
-    g0, g1 = o0.get(), o1.get()
-    assert np.all(g0[used * nrows:] == np.float32(4e30)) and np.all(g1[used * nrows:] == np.float32(4e30))
-    assert nmse(g0[:used * nrows].reshape(used, nrows), want0) <= 1e-10
-    assert nmse(g1[:used * nrows].reshape(used, nrows), want1) <= 1e-10
+    for form in (1, 0, 4):   # the dot-product form over planes (also the library's pick here), then the tile
+        dev.set_tuning(moe__form=form)
+        o0.put(np.full(used * nrows + 8, 4e30, np.float32))
+        o1.put(np.full(used * nrows + 8, 4e30, np.float32))
+        assert dev.moe_matvec_packed_dev(o0.ptr, o1.ptr, t, pb0, pb1, xd.ptr, None, dperm.ptr, dstart.ptr, n_expert,
+                                         used, nrows, k)
+        dev.synchronize()
+        g0, g1 = o0.get(), o1.get()
+        assert np.all(g0[used * nrows:] == np.float32(4e30)) and np.all(g1[used * nrows:] == np.float32(4e30))
+        assert nmse(g0[:used * nrows].reshape(used, nrows), want0) <= 1e-10, form
+        assert nmse(g1[:used * nrows].reshape(used, nrows), want1) <= 1e-10, form
+    dev.set_tuning(moe__form=0)
     # the tile form over the same weights as GGUF banks: the same integers, the same epilogue
     b0, b1 = devbuf(bank0), devbuf(bank1)
     r0 = devbuf(shape=(used * nrows,), dtype=np.float32, fill=0)
