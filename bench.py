@@ -590,6 +590,37 @@ def mxfp4_section(dev, gate_):
                                  "checked_rel_err": float(f"{err:.2e}")}
         x.free()
         o.free()
+    # the same matrix as packed planes (the device packer's), one token: a lane a row
+    from jitllm_amd.device import Packed
+    nq, nd, _ = dev.packed_words(quant.MXFP4, nrows, k)
+    pbytes = ((nq + nd) * 4 + 255) & ~255
+    pcopies = min(ncopies, pool.nbytes // pbytes)
+    if not dev.pack_weights_dev(quant.MXFP4, one.ptr, nrows, k, pool.ptr, pool.ptr + nq * 4, None):
+        raise RuntimeError("the device declined to pack the MXFP4 matrix")
+    dev.synchronize()
+    for i in range(1, pcopies):
+        check(hip().hipMemcpy(pool.ptr + i * pbytes, pool.ptr, (nq + nd) * 4, 3), "copy")
+    xf = np.random.default_rng(3).standard_normal((1, k)).astype(np.float32)
+    xb = (xf.view(np.uint32) >> 16).astype(np.uint16)
+    x = DeviceArray(xb)
+    o = DeviceArray(shape=(1, nrows), dtype=np.float32, fill=np.float32(np.nan))
+
+    def run_planes(i):
+        base = pool.ptr + (i % pcopies) * pbytes
+        if not dev.matmul_mxfp4_packed_bf16_dev(o.ptr, Packed(base, base + nq * 4, None, 0, nrows), x.ptr, nrows, k, 1):
+            raise RuntimeError("the device declined the packed MXFP4 matmul")
+    ms = measure(dev, run_planes, 40, gate_, warm=20)
+    got = o.get()
+    if not np.all(np.isfinite(got)):
+        raise RuntimeError("MXFP4 planes: non-finite or unwritten output")
+    xe = (xb.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+    err = rel_err(got[:, rows], xe @ wrows.T, "MXFP4 planes 1 token", 1e-5)
+    nbytes = (nq + nd) * 4 + k * 2 + nrows * 4
+    out["1 token, packed planes"] = {"us_per_step": round(ms * 1e3, 1), "GB/s": round(nbytes / (ms * 1e-3) / 1e9, 1),
+                                     "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                                     "weights": f"{pcopies} rotating copies", "checked_rel_err": float(f"{err:.2e}")}
+    x.free()
+    o.free()
     one.free()
     pool.free()
     return out

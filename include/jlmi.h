@@ -298,14 +298,19 @@ size_t jl_static_scratch_bytes(void);
 
 /* kernels.PackWeightsInto (jit/gpu/kernels/pack.go:52-199) on the device: GGUF
  * row-major blocks -> the three planes [unit][row] (sizes from jl_packed_words; sc may
- * be NULL for Q8_0).  Q4_K, Q6_K and Q8_0; the result is byte for byte the
- * reference's.  src 4-byte aligned for Q4_K, 2-byte for the others. */
+ * be NULL for Q8_0 and MXFP4).  Q4_K, Q6_K, Q8_0 and MXFP4; the result is byte for byte
+ * the reference's.  src 4-byte aligned for Q4_K, 2-byte for Q6_K and Q8_0.
+ * MXFP4 (pack.go:395-420): the D plane holds the E8M0 exponent minus one, four rows a
+ * word, and a matrix with a block of exponent 0, 1 or 255 whose codes are not all +-0 is
+ * refused as the reference's mxfp4Refuse refuses it: JL_DECLINED, the planes' contents
+ * then undefined.  To learn that, the MXFP4 call alone waits for its kernel. */
 int jl_pack_weights_dev(jl_ctx *ctx, int type, const void *src, int nrows, int k, uint32_t *qs,
                         uint32_t *d, uint32_t *sc, void *stream);
 
-/* The inverse permutation for Q4_K, Q6_K and Q8_0: rows row .. row+nrows of the planes back
- * to GGUF blocks in dst (nrows * k/256 * 144 bytes, 4-byte aligned; Q6_K 210 bytes a
- * super-block, Q8_0 34 bytes a block of 32, 2-byte aligned), bit for bit. */
+/* The inverse permutation for Q4_K, Q6_K, Q8_0 and MXFP4: rows row .. row+nrows of the
+ * planes back to GGUF blocks in dst (nrows * k/256 * 144 bytes, 4-byte aligned; Q6_K 210
+ * bytes a super-block, Q8_0 34 bytes a block of 32, 2-byte aligned; MXFP4 17 bytes a block
+ * of 32, any alignment, sc ignored), bit for bit. */
 int jl_unpack_weights_dev(jl_ctx *ctx, int type, const uint32_t *qs, const uint32_t *d,
                           const uint32_t *sc, int row, int stride, int nrows, int k, void *dst,
                           void *stream);
@@ -341,6 +346,16 @@ int jl_matmul_packed_dev(jl_ctx *ctx, float *out, int type, const uint32_t *qs, 
  * to its int8 kernels through a code table (jit/gpu/kernels/matvec.go:137-175). */
 int jl_matmul_mxfp4_bf16_dev(jl_ctx *ctx, float *out, const void *w, const uint16_t *x,
                              int nrows, int k, int ntok, void *stream);
+
+/* The same over packed MXFP4 planes (jit/gpu/kernels/pack.go:543-575: QS the code bytes
+ * four words a block, D the exponent minus one four rows a word; sizes from
+ * jl_packed_words, no SC plane): rows row .. row+nrows of planes of `stride` rows.  Up to
+ * 8 tokens read the planes where they lie, a lane a row; more tokens restore the row range
+ * to GGUF blocks in a workspace the context owns and run the matrix-core forms on it.  The
+ * value of a block is that of the GGUF block it was packed from. */
+int jl_matmul_mxfp4_packed_bf16_dev(jl_ctx *ctx, float *out, const uint32_t *qs, const uint32_t *d,
+                                    int row, int stride, const uint16_t *x, int nrows, int k,
+                                    int ntok, void *stream);
 
 /* ---- mixture of experts (device pointers) ----------------------------- */
 

@@ -80,6 +80,7 @@ SIGNATURES = {
     "jl_matmul_packed_dev": (_int, [_vp, _vp, _int, _vp, _vp, _vp, _int, _int, _vp, _int, _int, _int,
                                     _vp]),
     "jl_matmul_mxfp4_bf16_dev": (_int, [_vp, _vp, _vp, _vp, _int, _int, _int, _vp]),
+    "jl_matmul_mxfp4_packed_bf16_dev": (_int, [_vp, _vp, _vp, _vp, _int, _int, _vp, _int, _int, _int, _vp]),
     "jl_moe_logits_dev": (_int, [_vp, _vp, _int, _vp, _vp, _int, _int, _int, _vp]),
     "jl_moe_route_dev": (_int, [_vp, _vp, _int, _int, _int, _vp, _int, _vp, _vp]),
     "jl_moe_group_dev": (_int, [_vp, _vp, _int, _int, _int, _int, _vp, _vp, _vp, _vp]),

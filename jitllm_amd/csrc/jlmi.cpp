@@ -41,6 +41,7 @@ struct Tuning {
     int moe_waves = 0;
     int moe_lpr = 0;
     int mx_rows = 0;
+    int mx_planes = 0;          // packed MXFP4, a handful of tokens: 2 restores rows first; 64 / 32 / 16 rows a workgroup
     int mx_split = 0;
 };
 
@@ -93,6 +94,8 @@ struct jl_ctx {
     // rows restored to GGUF order for the GEMM over packed planes
     void* unpack_ws = nullptr;
     size_t unpack_ws_bytes = 0;
+    void* flag_ws = nullptr;    // one word the MXFP4 packer raises when it must refuse
+    size_t flag_ws_bytes = 0;
 
     // mixture-of-experts workspace (grouping tables and intermediate columns)
     void* moe_ws = nullptr;
@@ -729,6 +732,10 @@ bool packed_words(int type, size_t nrows, int k, size_t* nq, size_t* nd, size_t*
         if (k % 32) return false;
         *nq = nrows * (size_t)(k / 32) * 8; *nd = (size_t)(k / 32) * ((nrows + 1) / 2); *nsc = 0;
         return true;
+    case JL_TYPE_MXFP4:   // DSlots 4: an exponent byte a row, four rows a word (pack.go:543-575)
+        if (k % 32) return false;
+        *nq = nrows * (size_t)(k / 32) * 4; *nd = (size_t)(k / 32) * ((nrows + 3) / 4); *nsc = 0;
+        return true;
     }
     return false;
 }
@@ -827,13 +834,26 @@ int packed_matvec_multi_launch(jl_ctx* c, int type, int m, float* const* outs, c
                   params);   // JL_PK_LDS_BYTES
 }
 
+// MXFP4 planes (QS and D only): rows row .. row+nrows of a buffer of `stride` rows.
+int mx_planes_check(jl_ctx* c, const PlaneRef& pl, int nrows, int k) {
+    if (nrows <= 0 || k <= 0 || pl.row < 0 || pl.stride <= 0)
+        return fail(c, JL_ERR_ARG, "mxfp4 planes: nrows=%d k=%d row=%d stride=%d", nrows, k, pl.row, pl.stride);
+    if ((long)pl.row + nrows > pl.stride)
+        return fail(c, JL_ERR_ARG, "mxfp4 planes: rows %d..%d outside a buffer of %d rows", pl.row, pl.row + nrows,
+                    pl.stride);
+    if (!pl.qs || !pl.d) return fail(c, JL_ERR_ARG, "mxfp4 planes: null plane");
+    if (k % 32 != 0 || k / 32 > 65535 || (((uintptr_t)pl.qs | (uintptr_t)pl.d) & 3)) return JL_DECLINED;
+    return JL_OK;
+}
+
 int unpack_launch(jl_ctx* c, int type, const PlaneRef& pl, int nrows, int k, void* dst, hipStream_t st) {
     UnpackArgs a;
     a.dst = (uint8_t*)dst; a.qs = pl.qs; a.d = pl.d; a.sc = pl.sc;
     a.nrows = nrows; a.k = k; a.row0 = pl.row; a.stride = pl.stride;
     void* params[] = {&a};
-    if (type == JL_TYPE_Q8_0)
-        return launch(c, "jl_unpack_q8_0", (unsigned)((nrows + 255) / 256), (unsigned)(k / 32), 256, 0, st, params);
+    if (type == JL_TYPE_Q8_0 || type == JL_TYPE_MXFP4)
+        return launch(c, type == JL_TYPE_Q8_0 ? "jl_unpack_q8_0" : "jl_unpack_mxfp4", (unsigned)((nrows + 255) / 256),
+                      (unsigned)(k / 32), 256, 0, st, params);
     return launch(c, type == JL_TYPE_Q6_K ? "jl_unpack_q6k" : "jl_unpack_q4k", (unsigned)((nrows + 255) / 256),
                   (unsigned)(k / 256), 256, 0, st, params);
 }
@@ -1131,7 +1151,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     if (e != hipSuccess)
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
-    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_prep_q4k_planes", "jl_gemm_q4k_r64_planes", "jl_gemm_q4k_wide_planes", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_group2_wide", "jl_moe_quant", "jl_moe_matvec_planes_q4k", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_prep_planes", "jl_moe_gemm_q4k", "jl_moe_gemm_r64", "jl_moe_gemm_r64_planes", "jl_moe_gemm_q6k_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_sum_parts", "jl_probe_read", "jl_probe_empty", "jl_probe_wait",
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_prep_q4k_planes", "jl_gemm_q4k_r64_planes", "jl_gemm_q4k_wide_planes", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_group2_wide", "jl_moe_quant", "jl_moe_matvec_planes_q4k", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_prep_planes", "jl_moe_gemm_q4k", "jl_moe_gemm_r64", "jl_moe_gemm_r64_planes", "jl_moe_gemm_q6k_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_mxfp4_matvec_planes_r64", "jl_mxfp4_matvec_planes_r32", "jl_mxfp4_matvec_planes_r16", "jl_unpack_mxfp4", "jl_sum_parts", "jl_probe_read", "jl_probe_empty", "jl_probe_wait",
                                       "jl_pack_weights", "jl_unpack_q4k", "jl_unpack_q6k", "jl_unpack_q8_0"};
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int rw : {16, 32, 64})
@@ -1190,6 +1210,7 @@ void jl_ctx_destroy(jl_ctx* c) {
     if (c->w16_ws) (void)H->Free(c->w16_ws);
     if (c->moe_ws) (void)H->Free(c->moe_ws);
     if (c->unpack_ws) (void)H->Free(c->unpack_ws);
+    if (c->flag_ws) (void)H->Free(c->flag_ws);
     if (c->moe_q_ws) (void)H->Free(c->moe_q_ws);
     if (c->one_group) (void)H->Free(c->one_group);
     if (c->mx_ws) (void)H->Free(c->mx_ws);
@@ -1239,6 +1260,7 @@ int jl_set_tuning(jl_ctx* c, const char* key, int value) {
     else if (!strcmp(key, "gemm.rows")) c->tune.gemm_rows = value;
     else if (!strcmp(key, "mxfp4.split")) c->tune.mx_split = value;
     else if (!strcmp(key, "mxfp4.rows")) c->tune.mx_rows = value;
+    else if (!strcmp(key, "mxfp4.planes")) c->tune.mx_planes = value;
     else if (!strcmp(key, "gemm.form")) c->tune.gemm_form = value;
     else if (!strcmp(key, "gemm.split")) c->tune.gemm_split = value;
     else if (!strcmp(key, "gemm.prep")) c->tune.gemm_prep = value;
@@ -1406,21 +1428,44 @@ int jl_pack_weights_dev(jl_ctx* c, int type, const void* src, int nrows, int k, 
     size_t nq, nd, nsc;
     if (nrows <= 0 || !packed_words(type, (size_t)nrows, k, &nq, &nd, &nsc)) return JL_DECLINED;
     if (!src || !qs || !d || (nsc && !sc)) return fail(c, JL_ERR_ARG, "pack: null operand");
-    if ((uintptr_t)src & (type == JL_TYPE_Q4_K ? 3 : 1)) return JL_DECLINED;
+    if (type != JL_TYPE_MXFP4 && ((uintptr_t)src & (type == JL_TYPE_Q4_K ? 3 : 1))) return JL_DECLINED;
     if (((uintptr_t)qs | (uintptr_t)d | (uintptr_t)sc) & 3) return JL_DECLINED;
-    const int units = type == JL_TYPE_Q8_0 ? k / 32 : k / 256;
+    const int units = type == JL_TYPE_Q8_0 || type == JL_TYPE_MXFP4 ? k / 32 : k / 256;
     if (units > 65535) return JL_DECLINED;
     HIP_TRY(c, H->SetDevice(c->device));
+    hipStream_t st = pick_stream(c, stream);
     PackArgs a;
     a.src = (const uint8_t*)src; a.qs = qs; a.d = d; a.sc = sc; a.nrows = nrows; a.k = k; a.type = type;
+    a.flag = nullptr;
     void* params[] = {&a};
-    return launch(c, "jl_pack_weights", (unsigned)((nrows + 255) / 256), (unsigned)units, 256, 0,
-                  pick_stream(c, stream), params);
+    if (type != JL_TYPE_MXFP4)
+        return launch(c, "jl_pack_weights", (unsigned)((nrows + 255) / 256), (unsigned)units, 256, 0, st, params);
+    // MXFP4: the packer raises a flag for a block whose exponent the D plane cannot hold
+    // (mxfp4Refuse, jit/gpu/kernels/pack.go:407-420); the call waits for it, and a refused
+    // matrix leaves the planes' contents undefined.
+    int rc = ws_ensure(c, &c->flag_ws, &c->flag_ws_bytes, 256);
+    if (rc != JL_OK) return rc;
+    uint32_t flag = 0;
+    HIP_TRY(c, H->Memcpy(c->flag_ws, &flag, 4, hipMemcpyHostToDevice));
+    a.flag = (uint32_t*)c->flag_ws;
+    rc = launch(c, "jl_pack_weights", (unsigned)((nrows + 255) / 256), (unsigned)units, 256, 0, st, params);
+    if (rc != JL_OK) return rc;
+    HIP_TRY(c, H->StreamSynchronize(st));
+    HIP_TRY(c, H->Memcpy(&flag, c->flag_ws, 4, hipMemcpyDeviceToHost));
+    return flag ? JL_DECLINED : JL_OK;
 }
 
 int jl_unpack_weights_dev(jl_ctx* c, int type, const uint32_t* qs, const uint32_t* d, const uint32_t* sc,
                           int row, int stride, int nrows, int k, void* dst, void* stream) {
     if (!c) return JL_ERR_ARG;
+    if (type == JL_TYPE_MXFP4) {
+        const PlaneRef mpl = {qs, d, nullptr, row, stride};
+        int mrc = mx_planes_check(c, mpl, nrows, k);
+        if (mrc != JL_OK) return mrc;
+        if (!dst) return fail(c, JL_ERR_ARG, "unpack: null dst");
+        HIP_TRY(c, H->SetDevice(c->device));
+        return unpack_launch(c, type, mpl, nrows, k, dst, pick_stream(c, stream));
+    }
     if (type != JL_TYPE_Q4_K && type != JL_TYPE_Q6_K && type != JL_TYPE_Q8_0) return JL_DECLINED;
     const PlaneRef pl = {qs, d, sc, row, stride};
     const TypeInfo* ti = nullptr;
@@ -1728,6 +1773,40 @@ int jl_matmul_mxfp4_bf16_dev(jl_ctx* c, float* out, const void* w, const uint16_
     }
     return launch(c, gemm_name, (unsigned)(tok_pad / 128), (unsigned)((nrows + trows - 1) / trows), 512,
                   lds, st, params);
+}
+
+int jl_matmul_mxfp4_packed_bf16_dev(jl_ctx* c, float* out, const uint32_t* qs, const uint32_t* d, int row,
+                                    int stride, const uint16_t* x, int nrows, int k, int ntok, void* stream) {
+    if (!c) return JL_ERR_ARG;
+    const PlaneRef pl = {qs, d, nullptr, row, stride};
+    int rc = mx_planes_check(c, pl, nrows, k);
+    if (rc != JL_OK) return rc;
+    if (!out || !x || ntok <= 0) return fail(c, JL_ERR_ARG, "mxfp4 packed matmul: bad operand");
+    if (!aligned16(x)) return JL_DECLINED;
+    HIP_TRY(c, H->SetDevice(c->device));
+    hipStream_t st = pick_stream(c, stream);
+    if (ntok <= 8 && c->tune.mx_planes != 2) {
+        // a handful of tokens: the planes are read where they lie, a lane a row
+        MxPlanesArgs a;
+        a.out = out; a.qs = qs; a.d = d; a.x = (const uint32_t*)x;
+        a.nrows = nrows; a.k = k; a.ntok = ntok; a.row0 = row; a.stride = stride;
+        a.nwaves = k / 32 < 16 ? k / 32 : 16;
+        // rows a workgroup: 64 when that fills the CUs, else 32 or 16 (more, smaller workgroups)
+        int rl = c->tune.mx_planes == 64 || c->tune.mx_planes == 32 || c->tune.mx_planes == 16 ? c->tune.mx_planes : 0;
+        // (measured: 2880 rows 5.4 us at 16 against 6.8 at 64; 5760 rows 6.3 at 32 against 7.1 and 8.6)
+        if (!rl) rl = (nrows + 63) / 64 * 10 >= c->num_cu * 7 ? 64 : ((nrows + 31) / 32 * 10 >= c->num_cu * 7 ? 32 : 16);
+        char name[40];
+        snprintf(name, sizeof name, "jl_mxfp4_matvec_planes_r%d", rl);
+        void* params[] = {&a};
+        return launch(c, name, (unsigned)((nrows + rl - 1) / rl), 1, (unsigned)(64 * a.nwaves),
+                      (unsigned)(a.nwaves * 8 * 64 * 4), st, params);
+    }
+    // more tokens: the matrix-core forms stage GGUF blocks, so the rows are restored first
+    rc = ws_ensure(c, &c->unpack_ws, &c->unpack_ws_bytes, (size_t)nrows * (size_t)(k / 32) * 17);
+    if (rc != JL_OK) return rc;
+    rc = unpack_launch(c, JL_TYPE_MXFP4, pl, nrows, k, c->unpack_ws, st);
+    if (rc != JL_OK) return rc;
+    return jl_matmul_mxfp4_bf16_dev(c, out, c->unpack_ws, x, nrows, k, ntok, st);
 }
 
 /* ------------------------------------------------------- host-pointer seam */

@@ -251,6 +251,16 @@ struct MxGemmArgs {
     float* part;          // [nsplit][ntok][nrows], summed by jl_sum_parts
 };
 
+// MXFP4 planes x a handful of bf16 tokens: rows row0 .. row0+nrows of planes of `stride` rows.
+struct MxPlanesArgs {
+    float* out;           // [ntok][nrows]
+    const uint32_t* qs;   // [k/32][4][stride]: a block's 16 code bytes, four words
+    const uint32_t* d;    // [k/32][ceil(stride/4)]: E8M0 exponent minus one, four rows a word
+    const uint32_t* x;    // [ntok][k] bf16 bits, read two a word
+    int nrows, k, ntok, row0, stride;
+    int nwaves;           // wavefronts of a workgroup; they split the blocks of K
+};
+
 // out[i] = part[0][i] + part[1][i] + ... in that order.
 struct SumPartsArgs {
     float* out;
@@ -266,6 +276,7 @@ struct PackArgs {
     uint32_t* d;
     uint32_t* sc;         // null for formats without a scale plane
     int nrows, k, type;
+    uint32_t* flag;       // MXFP4: set to 1 when a block's exponent cannot be stored (else untouched)
 };
 
 struct UnpackArgs {

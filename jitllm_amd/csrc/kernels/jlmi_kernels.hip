@@ -81,6 +81,7 @@ extern "C" __global__ __launch_bounds__(256) void jl_unpack_q4k(UnpackArgs p) { 
 extern "C" __global__ __launch_bounds__(256) void jl_unpack_q6k(UnpackArgs p) { unpack_q6k_body(p); }
 // grid = (ceil(nrows/256), k/32)
 extern "C" __global__ __launch_bounds__(256) void jl_unpack_q8_0(UnpackArgs p) { unpack_q8_0_body(p); }
+extern "C" __global__ __launch_bounds__(256) void jl_unpack_mxfp4(UnpackArgs p) { unpack_mxfp4_body(p); }
 // jl_matvec_packed_<type>_w<rows per wavefront>: grid = ceil(nrows/RW), block = 64..1024
 // XPRE = chunks whose activation loads go out ahead of the weights (register budget).
 // jl_matvec_packed_<type>_w<RW> quantizes f32 x itself; jl_matvec_packed_q8_<type>_w<RW>
@@ -293,6 +294,17 @@ extern "C" __global__ __launch_bounds__(512) void jl_mxfp4_gemm_r96(MxGemmArgs p
 extern "C" __global__ __launch_bounds__(256) void jl_sum_parts(SumPartsArgs p) { sum_parts_body(p); }
 // grid = ceil(nrows/4), block = 256: one wavefront per row, ntok <= 8
 extern "C" __global__ __launch_bounds__(256) void jl_mxfp4_matvec(MxGemmArgs p) { mx_matvec_body(p); }
+// ntok <= 8 over packed planes, _r<rows a workgroup>: grid = ceil(nrows/R), block = 64 * nwaves,
+// LDS = nwaves * 8 * 64 floats
+extern "C" __global__ __launch_bounds__(1024) void jl_mxfp4_matvec_planes_r64(MxPlanesArgs p) {
+    mx_planes_matvec_body<64, 6>(p, (float*)jl_smem);
+}
+extern "C" __global__ __launch_bounds__(1024) void jl_mxfp4_matvec_planes_r32(MxPlanesArgs p) {
+    mx_planes_matvec_body<32, 3>(p, (float*)jl_smem);
+}
+extern "C" __global__ __launch_bounds__(1024) void jl_mxfp4_matvec_planes_r16(MxPlanesArgs p) {
+    mx_planes_matvec_body<16, 2>(p, (float*)jl_smem);
+}
 // 9..64 tokens: prep grid = (ceil(k/128), tiles of 16 tokens), block = 256; kernel grid =
 // ceil(nrows/16), block = 512; _t<NT>: up to 16 NT tokens
 extern "C" __global__ __launch_bounds__(256) void jl_mxfp4_prep_few(MxPrepArgs p) { mx_prep_few_body(p); }

@@ -293,6 +293,114 @@ __device__ __forceinline__ void mx_matvec_body(const MxGemmArgs& p) {
     }
 }
 
+// The same handful of tokens over packed planes (jit/gpu/kernels/pack.go:543-575).  A lane
+// takes a row, so the four code words and the exponent word of a block are consecutive
+// across RL lanes; the 64 / RL lane groups of a wavefront, and the wavefronts of a workgroup,
+// take the blocks of K in turn (a slice each).  RL = 64: the activations are the same for
+// every lane and come as scalar operands; RL = 32 / 16: more, smaller workgroups for a
+// matrix of few rows, the activations as vector loads a lane group shares.  The slices' sums
+// are added in a fixed order: across a wavefront's lane groups, then the wavefronts in turn
+// through LDS (red: [nwaves][8][RL] floats).
+// AHEAD blocks at a time: all their loads go out before the first is decoded, so a slice's
+// few blocks cost one trip to memory and not one each.
+// grid = ceil(nrows/RL), block = 64 * nwaves
+template <int RL, int AHEAD>
+__device__ __forceinline__ void mx_planes_matvec_body(const MxPlanesArgs& p, float* red) {
+    constexpr int G = 64 / RL;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int rlane = lane % RL;
+    const int slice = G == 1 ? wave : wave * G + lane / RL, nsl = p.nwaves * G;
+    const int rl = blockIdx.x * RL + rlane;
+    const bool live = rl < p.nrows;
+    const size_t n = (size_t)p.stride;
+    const size_t r = (size_t)p.row0 + (live ? rl : p.nrows - 1);   // idle lanes re-read the last row
+    const int nblk = p.k / 32, sh = 8 * (int)(r & 3);
+    const size_t dwords = (n + 3) / 4;
+    float acc[8];
+#pragma unroll
+    for (int t = 0; t < 8; t++) acc[t] = 0.f;
+    for (int base = 0; base < nblk; base += AHEAD * nsl) {
+        const int b0 = base + slice;
+        u32 q[AHEAD][4], dd[AHEAD];
+#pragma unroll
+        for (int u = 0; u < AHEAD; u++) {
+            const int b = b0 + u * nsl < nblk ? b0 + u * nsl : nblk - 1;
+            const u32* qp = p.qs + (size_t)b * 4 * n + r;
+#pragma unroll
+            for (int w = 0; w < 4; w++) q[u][w] = qp[(size_t)w * n];
+            dd[u] = p.d[(size_t)b * dwords + (r >> 2)];
+        }
+#pragma unroll
+        for (int u = 0; u < AHEAD; u++) {
+            const int b = b0 + u * nsl;
+            if (b < nblk) {
+                const float scale = mx_scale((uint8_t)(((dd[u] >> sh) & 0xFF) + 1));
+                float wv[32];
+#pragma unroll
+                for (int w = 0; w < 4; w++) {
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        f32x2 pr;
+                        switch (i) {
+                        case 0: pr = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(q[u][w], scale, 0); break;
+                        case 1: pr = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(q[u][w], scale, 1); break;
+                        case 2: pr = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(q[u][w], scale, 2); break;
+                        default: pr = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(q[u][w], scale, 3); break;
+                        }
+                        wv[4 * w + i] = pr.x;
+                        wv[4 * w + i + 16] = pr.y;
+                    }
+                }
+#pragma unroll
+                for (int t = 0; t < 8; t++) {
+                    if (t < p.ntok) {
+                        const u32* xt = p.x + (((size_t)t * p.k + (size_t)b * 32) >> 1);
+                        float s = 0.f;
+#pragma unroll
+                        for (int c4 = 0; c4 < 4; c4++) {
+                            u32 v[4];
+                            if constexpr (G == 1) {
+#pragma unroll
+                                for (int j = 0; j < 4; j++) v[j] = xt[4 * c4 + j];
+                            } else {
+                                const u32x4 vv = ((const u32x4*)xt)[c4];
+#pragma unroll
+                                for (int j = 0; j < 4; j++) v[j] = vv[j];
+                            }
+#pragma unroll
+                            for (int j = 0; j < 4; j++) {
+                                s = fmaf(wv[8 * c4 + 2 * j], __uint_as_float(v[j] << 16), s);
+                                s = fmaf(wv[8 * c4 + 2 * j + 1], __uint_as_float(v[j] & 0xFFFF0000u), s);
+                            }
+                        }
+                        acc[t] += s;
+                    }
+                }
+            }
+        }
+    }
+    // a wavefront's lane groups first (lanes RL apart hold the same row), then the wavefronts
+    // in order through LDS
+#pragma unroll
+    for (int t = 0; t < 8; t++) {
+        if (t < p.ntok) {
+            float s = acc[t];
+            if constexpr (G >= 2) s += __shfl_xor(s, 32);
+            if constexpr (G >= 4) s += __shfl_xor(s, 16);
+            if (lane < RL) red[(wave * 8 + t) * RL + rlane] = s;
+        }
+    }
+    __syncthreads();
+    // one thread per (token, row) adds the wavefronts' sums
+    for (int i = threadIdx.x; i < p.ntok * RL; i += blockDim.x) {
+        const int t = i / RL, rr = i % RL;
+        float s = red[t * RL + rr];
+        for (int w = 1; w < p.nwaves; w++) s += red[(w * 8 + t) * RL + rr];
+        if (blockIdx.x * RL + rr < p.nrows) p.out[(size_t)t * p.nrows + blockIdx.x * RL + rr] = s;
+    }
+}
+
 // grid = ceil(n / 256), block = 256
 __device__ __forceinline__ void sum_parts_body(const SumPartsArgs& p) {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;

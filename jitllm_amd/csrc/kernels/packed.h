@@ -117,11 +117,35 @@ __device__ __forceinline__ void pack_q8_0(const PackArgs& p, int r, int b) {
     }
 }
 
+// MXFP4 (jit/gpu/kernels/pack.go:395-420, :543-575): a block's 16 code bytes are the four QS
+// words as they lie (byte j = element j in the low nibble, element j+16 in the high); the D
+// plane holds the E8M0 exponent minus one, a byte a row, four rows a word, so that the byte
+// shifted left 23 is the f32 scale of the doubled code table.  Exponents 0, 1 and 255 have no
+// such byte: a block that carries one and a code other than +-0 raises the flag.
+__device__ __forceinline__ void pack_mxfp4(const PackArgs& p, int r, int b) {
+    const int nb = p.k / 32;
+    const size_t n = (size_t)p.nrows, step = (size_t)nb * 17;
+    const uint8_t* blk = p.src + ((size_t)r * nb + b) * 17;
+    const u32x4 q = ld16_a1(blk + 1);
+#pragma unroll
+    for (int w = 0; w < 4; w++) p.qs[((size_t)b * 4 + w) * n + r] = q[w];
+    const u32 e = blk[0];
+    if ((e < 2 || e == 255) && ((q[0] | q[1] | q[2] | q[3]) & 0x77777777u)) *p.flag = 1;
+    if ((r & 3) == 0) {
+        u32 v = (e - 1) & 0xFF;
+#pragma unroll
+        for (int i = 1; i < 4; i++)
+            if (r + i < p.nrows) v |= (((u32)blk[i * step] - 1) & 0xFF) << (8 * i);
+        p.d[(size_t)b * ((n + 3) / 4) + (r >> 2)] = v;
+    }
+}
+
 __device__ __forceinline__ void pack_weights_body(const PackArgs& p) {
     const int r = blockIdx.x * 256 + threadIdx.x, u = blockIdx.y;
     if (r >= p.nrows) return;
     if (p.type == JL_Q4_K) pack_q4k(p, r, u);
     else if (p.type == JL_Q6_K) pack_q6k(p, r, u);
+    else if (p.type == JL_MXFP4) pack_mxfp4(p, r, u);
     else pack_q8_0(p, r, u);
 }
 
@@ -222,6 +246,22 @@ __device__ __forceinline__ void unpack_q8_0_body(const UnpackArgs& p) {
     *(uint16_t*)blk = (uint16_t)(r & 1 ? dd >> 16 : dd);
 #pragma unroll
     for (int w = 0; w < 8; w++) st4_a2(blk + 2 + 4 * w, p.qs[((size_t)b * 8 + w) * n + r]);
+}
+
+// The inverse for MXFP4 (pack_mxfp4 above): one thread per (row, block).
+struct __attribute__((packed, aligned(1))) u32x4_st1 { u32x4 v; };
+__device__ __forceinline__ void unpack_mxfp4_body(const UnpackArgs& p) {
+    const int rl = blockIdx.x * 256 + threadIdx.x, b = blockIdx.y;
+    if (rl >= p.nrows) return;
+    const size_t n = (size_t)p.stride, r = (size_t)p.row0 + rl;
+    const int nb = p.k / 32;
+    uint8_t* blk = p.dst + ((size_t)rl * nb + b) * 17;
+    const u32 dd = p.d[(size_t)b * ((n + 3) / 4) + (r >> 2)];
+    blk[0] = (uint8_t)(((dd >> (8 * (r & 3))) & 0xFF) + 1);
+    u32x4 q;
+#pragma unroll
+    for (int w = 0; w < 4; w++) q[w] = p.qs[((size_t)b * 4 + w) * n + r];
+    ((u32x4_st1*)(blk + 1))->v = q;
 }
 
 // ---------------------------------------------------------------- matvec

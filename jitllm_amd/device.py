@@ -331,3 +331,9 @@ class Device:
         return self._served(self._l.jl_matmul_mxfp4_bf16_dev(self._ctx, _ptr(out), _ptr(w), _ptr(x),
                                                              nrows, k, ntok, stream),
                             "jl_matmul_mxfp4_bf16_dev")
+
+    def matmul_mxfp4_packed_bf16_dev(self, out, p, x, nrows, k, ntok, stream=None):
+        """The same over packed MXFP4 planes; p = Packed(qs, d, None, row, stride)."""
+        return self._served(self._l.jl_matmul_mxfp4_packed_bf16_dev(self._ctx, _ptr(out), _ptr(p.qs), _ptr(p.d),
+                                                                    p.row, p.stride, _ptr(x), nrows, k, ntok,
+                                                                    stream), "jl_matmul_mxfp4_packed_bf16_dev")

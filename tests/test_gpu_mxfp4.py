@@ -77,3 +77,153 @@ def test_mxfp4_k_split_forms_agree(dev, devbuf):
         dev.synchronize()
         assert nmse(out.get(), want) <= 1e-10, f"split {split}"
     dev.set_tuning(mxfp4__split=0)
+
+
+# ------------------------------------------------------------------ packed planes
+def _exponent_spread(w, seed):
+    """Give the blocks of GGUF MXFP4 bytes exponents from the whole storable range (2..254
+    keeps every block packable; the matmul tests keep them near 127 so sums stay finite)."""
+    w = w.copy()
+    rng = np.random.default_rng(seed)
+    w[0::17] = rng.integers(2, 255, w[0::17].size, dtype=np.uint8)
+    return w
+
+
+@pytest.mark.parametrize("shape", [(1, 32), (3, 64), (4, 96), (5, 2880), (130, 224), (257, 512), (2880, 2880)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_mxfp4_device_pack_is_the_reference_packer_byte_for_byte(dev, devbuf, shape):
+    """/root/reference/jit/gpu/kernels/pack.go:52-199 with e8m0Store (:395) and DSlots 4 (:543-575):
+    the device planes equal the CPU restatement's, ragged row counts (a last D word of one to
+    three rows) and every storable exponent included, and unpacking gives the GGUF bytes back."""
+    nrows, k = shape
+    t = quant.MXFP4
+    w = _exponent_spread(synth.random_weights(t, nrows, k, seed=nrows + k), seed=k)
+    want_qs, want_d, _ = oracle.pack_weights(t, w, nrows, k)
+    nq, nd, nsc = dev.packed_words(t, nrows, k)
+    assert (nq, nd, nsc) == (want_qs.size, want_d.size, 0) == oracle.packed_words(t, nrows, k)
+    dw = devbuf(w)
+    qs = devbuf(shape=(nq + 4,), dtype=np.uint32, fill=np.uint32(0xA5A5A5A5))
+    d = devbuf(shape=(nd + 4,), dtype=np.uint32, fill=np.uint32(0xA5A5A5A5))
+    assert dev.pack_weights_dev(t, dw.ptr, nrows, k, qs.ptr, d.ptr, None)
+    got_qs, got_d = qs.get(), d.get()
+    assert np.array_equal(got_qs[:nq], want_qs) and np.all(got_qs[nq:] == 0xA5A5A5A5)
+    assert np.array_equal(got_d[:nd], want_d) and np.all(got_d[nd:] == 0xA5A5A5A5)
+    # back to GGUF blocks, whole and as a row range
+    from jitllm_amd.device import Packed
+    back = devbuf(shape=(w.size + 17,), dtype=np.uint8, fill=np.uint8(0xEE))
+    assert dev.unpack_weights_dev(t, Packed(qs.ptr, d.ptr, None, 0, nrows), nrows, k, back.ptr)
+    got = back.get()
+    assert np.array_equal(got[:w.size], w) and np.all(got[w.size:] == 0xEE)
+    if nrows >= 5:
+        r0, n = nrows // 3 + 1, nrows - nrows // 3 - 2
+        rb = k // 32 * 17
+        assert dev.unpack_weights_dev(t, Packed(qs.ptr, d.ptr, None, r0, nrows), n, k, back.ptr)
+        assert np.array_equal(back.get()[:n * rb], w[r0 * rb:(r0 + n) * rb])
+
+
+def test_mxfp4_device_pack_refuses_what_the_reference_refuses(dev, devbuf):
+    """/root/reference/jit/gpu/kernels/pack.go:407-420, /root/reference/internal/oracle/packed_test.go:220-247:
+    exponents 0, 1 and 255 pass only on a block of +-0 codes; the device and the CPU restatement
+    agree case by case."""
+    t = quant.MXFP4
+    nrows, k = 3, 1024
+    base = np.zeros(17 * 32 * nrows, np.uint8)
+    base[0::17] = 127
+    base[1::17] = 0x21
+    nq, nd, _ = dev.packed_words(t, nrows, k)
+    qs, d = devbuf(shape=(nq,), dtype=np.uint32), devbuf(shape=(nd,), dtype=np.uint32)
+
+    def both(w):
+        try:
+            oracle.pack_weights(t, w, nrows, k)
+            want = True
+        except ValueError:
+            want = False
+        got = dev.pack_weights_dev(t, devbuf(w).ptr, nrows, k, qs.ptr, d.ptr, None)
+        assert got is want
+        return got
+
+    assert both(base)
+    for e in (0, 1, 255):
+        for blk in (3, 32 + 7, 17 * 32 * nrows // 17 - 1):     # first row, second row, last block
+            bad = base.copy()
+            bad[17 * blk] = e
+            assert not both(bad)                   # the block still holds 0x21 codes
+            bad[17 * blk + 1:17 * blk + 17] = 0
+            assert both(bad)                       # all-zero codes pass at any exponent
+            bad[17 * blk + 5] = 0x88
+            assert both(bad)                       # -0 codes are still zero
+            bad[17 * blk + 16] = 0x10
+            assert not both(bad)
+    assert both(base)                              # a refusal leaves nothing behind
+
+
+@pytest.mark.parametrize("shape", [(1, 2880, 2880), (1, 5760, 2880), (2, 100, 512), (8, 130, 96), (5, 64, 32),
+                                   (7, 257, 544), (64, 2880, 2880), (9, 129, 160)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_mxfp4_packed_matmul_vs_dequant_f32(dev, devbuf, shape):
+    """Planes written by the device packer, read by the plane kernel (up to 8 tokens) or restored
+    and fed to the matrix-core forms: the same bar as the GGUF-row path, and for more than 8
+    tokens the same bits, since the restored rows are the GGUF rows."""
+    from jitllm_amd.device import Packed
+    ntok, nrows, k = shape
+    t = quant.MXFP4
+    w = synth.quantized_weights(t, nrows, k, seed=ntok + 11)
+    xb, xf = to_bf16(np.stack([synth.activations(k, seed=40 + i) for i in range(ntok)]))
+    want = xf.astype(np.float64) @ oracle.dequant(t, w, nrows * k).reshape(nrows, k).astype(np.float64).T
+    nq, nd, _ = dev.packed_words(t, nrows, k)
+    dw, dx = devbuf(w), devbuf(xb)
+    qs, d = devbuf(shape=(nq,), dtype=np.uint32), devbuf(shape=(nd,), dtype=np.uint32)
+    assert dev.pack_weights_dev(t, dw.ptr, nrows, k, qs.ptr, d.ptr, None)
+    out = devbuf(shape=(ntok * nrows + 8,), dtype=np.float32, fill=np.float32(2e30))
+    forms = (0, 64, 32, 16, 2) if ntok <= 8 else (0,)   # rows a workgroup of the plane kernel; 2: restore rows
+    for form in forms:
+        dev.set_tuning(mxfp4__planes=form)
+        n0 = dev.launch_count()
+        assert dev.matmul_mxfp4_packed_bf16_dev(out.ptr, Packed(qs.ptr, d.ptr, None, 0, nrows), dx.ptr, nrows, k, ntok)
+        dev.synchronize()
+        if ntok <= 8 and form != 2:
+            assert dev.launch_count() - n0 == 1
+        got = out.get()
+        assert np.all(got[ntok * nrows:] == np.float32(2e30))
+        got = got[:ntok * nrows].reshape(ntok, nrows)
+        assert nmse(got, want) <= 1e-10 and rel_l2(got, want) <= 1e-3, f"form {form}"
+    dev.set_tuning(mxfp4__planes=0)
+    if ntok > 8:
+        ref = devbuf(shape=(ntok, nrows), dtype=np.float32)
+        assert dev.matmul_mxfp4_bf16_dev(ref.ptr, dw.ptr, dx.ptr, nrows, k, ntok)
+        dev.synchronize()
+        assert np.array_equal(ref.get(), got)
+    # a row range of the planes: rows r0 .. r0+n of the same buffer
+    if nrows >= 100:
+        r0, n = 37, nrows - 70
+        out.put(np.full(ntok * nrows + 8, np.float32(2e30)))
+        assert dev.matmul_mxfp4_packed_bf16_dev(out.ptr, Packed(qs.ptr, d.ptr, None, r0, nrows), dx.ptr, n, k, ntok)
+        dev.synchronize()
+        got = out.get()
+        assert np.all(got[ntok * n:] == np.float32(2e30))
+        assert nmse(got[:ntok * n].reshape(ntok, n), want[:, r0:r0 + n]) <= 1e-10
+
+
+def test_mxfp4_packed_matmul_every_exponent_one_token(dev, devbuf):
+    """The plane reader's scale is the stored byte plus one as an f32 exponent: blocks at both ends
+    of the storable range (2 and 254) against the f64 evaluation of the dequantized rows."""
+    from jitllm_amd.device import Packed
+    t = quant.MXFP4
+    nrows, k = 67, 64
+    w = synth.random_weights(t, nrows, k, seed=5)
+    w[0::17] = np.resize(np.array([2, 3, 64, 127, 128, 200], np.uint8), w[0::17].size)
+    x = np.zeros(k, np.float32)
+    x[::3] = 1.0
+    x[1::3] = -0.5
+    xb, xf = to_bf16(x[None, :])
+    wd = oracle.dequant(t, w, nrows * k).reshape(nrows, k).astype(np.float64)
+    want = (xf.astype(np.float64) @ wd.T).astype(np.float32)
+    nq, nd, _ = dev.packed_words(t, nrows, k)
+    qs, d = devbuf(shape=(nq,), dtype=np.uint32), devbuf(shape=(nd,), dtype=np.uint32)
+    assert dev.pack_weights_dev(t, devbuf(w).ptr, nrows, k, qs.ptr, d.ptr, None)
+    out = devbuf(shape=(nrows,), dtype=np.float32)
+    assert dev.matmul_mxfp4_packed_bf16_dev(out.ptr, Packed(qs.ptr, d.ptr, None, 0, nrows), devbuf(xb).ptr, nrows, k, 1)
+    dev.synchronize()
+    got = out.get()
+    assert np.all(np.isfinite(want)) and np.allclose(got, want, rtol=2e-6, atol=0)
