@@ -502,7 +502,9 @@ int gemm_q4k_launch(jl_ctx* c, float* out, const void* w, const float* x, int nr
     if (form == 4 || form == 5) form = 0;   // outside the few-token forms' range
     if (form == 0) {
         const long wide_groups = (long)((ntok + kGemmWideTok - 1) / kGemmWideTok) * ((nrows + 127) / 128);
-        form = 4 * wide_groups >= 3 * (long)c->num_cu ? 2 : 1;   // one round at least three quarters full
+        // from a quarter of the CUs on: a smaller grid is widened along K below (measured
+        // against the 64-row tiles: 1024 tokens x 4096 rows 56 against 62 us, 512 x 4096 38 against 40)
+        form = 4 * wide_groups >= (long)c->num_cu ? 2 : 1;
     }
     if (form == 2 && kGemmWideLdsBytes > c->lds_limit) form = 1;
     const int tile = form == 2 ? kGemmWideTok : kGemmTile;
@@ -540,6 +542,27 @@ int gemm_q4k_launch(jl_ctx* c, float* out, const void* w, const float* x, int nr
         long nrt_wide = nrt;
         if (c->tune.gemm_form == 0 && full >= 1 && rem > 0 && 2 * rem <= c->num_cu) nrt_wide = full * c->num_cu / ntt;
         ga.nrows = nrt_wide == nrt ? nrows : (int)(nrt_wide * 128);
+        // a grid of at most half the CUs is widened along K, partial slabs added in order
+        int wsplit = c->tune.gemm_split > 0 ? c->tune.gemm_split : (c->tune.gemm_form == 0 ? (int)(c->num_cu / (ntt * nrt)) : 1);
+        if (wsplit > 8) wsplit = 8;
+        if (wsplit > nsb) wsplit = nsb;
+        if (wsplit > 1) {
+            const int per = (nsb + wsplit - 1) / wsplit;
+            wsplit = (nsb + per - 1) / per;   // no empty split
+        }
+        if (wsplit > 1 && nrt_wide == nrt) {
+            const size_t n = (size_t)ntok * nrows;
+            rc = ws_ensure(c, &c->mx_ws, &c->mx_ws_bytes, n * wsplit * 4);
+            if (rc != JL_OK) return rc;
+            ga.out = (float*)c->mx_ws; ga.sb_per = (nsb + wsplit - 1) / wsplit;
+            rc = launch(c, pl ? "jl_gemm_q4k_wide_planes" : "jl_gemm_q4k_wide", (unsigned)ntt, (unsigned)nrt, 512,
+                        kGemmWideLdsBytes, st, gp, (unsigned)wsplit);
+            if (rc != JL_OK) return rc;
+            SumPartsArgs sa;
+            sa.out = out; sa.part = (const float*)c->mx_ws; sa.n = n; sa.nsplit = wsplit;
+            void* sp[] = {&sa};
+            return launch(c, "jl_sum_parts", (unsigned)((n + 255) / 256), 1, 256, 0, st, sp);
+        }
         rc = launch(c, pl ? "jl_gemm_q4k_wide_planes" : "jl_gemm_q4k_wide", (unsigned)ntt, (unsigned)nrt_wide, 512,
                     kGemmWideLdsBytes, st, gp);
         rows_left = nrows - ga.nrows;

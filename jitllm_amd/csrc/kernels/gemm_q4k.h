@@ -43,6 +43,12 @@
 #ifndef JL_TRACE
 #define JL_TRACE(i)
 #endif
+// Profiling builds only (results are then wrong): bits switch parts of the wide kernel's loop
+// off, to time what each costs.  1 epilogue, 2 dequantization, 4 activation loads, 8 weight
+// fragment reads, 16 barriers, 32 the minimum-term matrix instructions, 64 weight loads.
+#ifndef JL_ABL
+#define JL_ABL 0
+#endif
 
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
@@ -681,7 +687,7 @@ __device__ __forceinline__ void gemm_q4k_wide_body(const GemmArgs& p, uint8_t* s
         const _Float16* w = sW + half * STAGE_HALFS;
         _Float16* wnext = sW + nhalf * STAGE_HALFS;
         const int nstep = min(step + 1, nsteps - 1);
-        load_w(min(step + 2, nsteps - 1), wnxt);
+        if (!(JL_ABL & 64)) load_w(min(step + 2, nsteps - 1), wnxt);
         const _Float16* wp0 = w + arow * JL_GEMM_WROW + 8 * kg;
         const _Float16* mp0 = sMin + eb * MIN_HALFS + arow * JL_GEMM_MROW + 8 * kg;
         const float* scp = sScale + eb * 2 * ROWS + 2 * arow;
@@ -690,12 +696,13 @@ __device__ __forceinline__ void gemm_q4k_wide_body(const GemmArgs& p, uint8_t* s
             return *(const f16x8*)(wp0 + 32 * (2 * (slot >> 3) + j) * JL_GEMM_WROW + 16 * (slot & 7));
         };
         f16x8 wf[2][2], wm;
-        f32x4 dav;
+        f32x4 dav[2];   // token scales of an epilogue slot, read from LDS a slot ahead
         GemmWideScale wsc;
         wsc.dst = wnext + wdst;
 #pragma unroll
         for (int j = 0; j < 2; j++) wf[0][j] = w_frag(0, j);
         if (has_ep && ep_jh == 0) {
+            dav[0] = *(const f32x4*)dap;
             wm = *(const f16x8*)(mp0 + 32 * ej0 * JL_GEMM_MROW);
             esc = *(const float2*)(scp + 2 * 32 * ej0);
         }
@@ -703,16 +710,15 @@ __device__ __forceinline__ void gemm_q4k_wide_body(const GemmArgs& p, uint8_t* s
         gemm_static_for<0, 16>([&](auto SLOT) __attribute__((always_inline)) {
             constexpr int slot = decltype(SLOT)::value, jh = slot >> 3, ks = slot & 7;
             constexpr bool ep = has_ep && jh == ep_jh;
-            if (slot + 1 < 16) {
+            constexpr bool ep_next = has_ep && slot + 1 < 16 && ((slot + 1) >> 3) == ep_jh;
+            // the next slot's token scales first: the wait that guards them then leaves the
+            // weight fragments (read after them, used a slot later) in flight
+            if (ep_next) dav[(slot + 1) & 1] = *(const f32x4*)(dap + 8 * ((ks + 1) & 3));
+            if (slot + 1 < 16 && !(JL_ABL & 8)) {
 #pragma unroll
                 for (int j = 0; j < 2; j++) wf[(slot + 1) & 1][j] = w_frag(slot + 1, j);
             }
-            // operands of the epilogue a slot ahead: the next quarter's token scales, and
-            // before a tile's first quarter its minimum columns and row scales
-            // operands of the epilogue: this slot's token scales (the matrix instructions
-            // below cover the read), and a slot ahead of a tile's first quarter its minimum
-            // columns
-            if (ep) dav = *(const f32x4*)(dap + 8 * (ks & 3));
+            // a slot ahead of a tile's first quarter: its minimum columns and row scales
             if (has_ep && ep_jh == 1 && slot == 7) {
                 wm = *(const f16x8*)(mp0 + 32 * ej0 * JL_GEMM_MROW);
                 esc = *(const float2*)(scp + 2 * 32 * ej0);
@@ -721,7 +727,7 @@ __device__ __forceinline__ void gemm_q4k_wide_body(const GemmArgs& p, uint8_t* s
             if (ep && ks == 4) esc = *(const float2*)(scp + 2 * 32 * (ej0 + 1));
             __builtin_amdgcn_sched_barrier(0);
             const f32x16 czero = {0};
-            if (ep && (ks & 3) == 0) {
+            if (ep && (ks & 3) == 0 && !(JL_ABL & 32)) {
                 // the tile's M = sum m_s A_s, ahead of this slot's instructions so that it is
                 // ready when the vector work below asks for it
                 accM = __builtin_amdgcn_mfma_f32_32x32x16_f16(aaug, wm, czero, 0, 0, 0);
@@ -730,13 +736,13 @@ __device__ __forceinline__ void gemm_q4k_wide_body(const GemmArgs& p, uint8_t* s
             for (int j = 0; j < 2; j++)
                 accP[2 * jh + j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
                     aring[ks], wf[slot & 1][j], (half == 0 && ks == 0) ? czero : accP[2 * jh + j], 0, 0, 0);
-            if (jh == 1) {
+            if (jh == 1 && !(JL_ABL & 4)) {
                 aring[ks] = a_frag(nstep, ks);
                 if (ks == 0 && nhalf == 1) aaug = a_frag(nstep, 8);
             }
             if (ep) {
-                ep_quarter(GemmIntC<ej0 + (ks >> 2)>{}, GemmIntC<(ks & 3)>{}, dav);
-            } else if (jh != ep_jh) {
+                if (!(JL_ABL & 1)) ep_quarter(GemmIntC<ej0 + (ks >> 2)>{}, GemmIntC<(ks & 3)>{}, dav[slot & 1]);
+            } else if (jh != ep_jh && !(JL_ABL & 2)) {
                 // the next stage's weights: wcur -> f16 -> LDS
                 if (ks == 0) {
                     if (PL) gemm_wide_scale_planes(wcur.hdr, 4 * nhalf + psub, wsc);
@@ -774,13 +780,26 @@ __device__ __forceinline__ void gemm_q4k_wide_body(const GemmArgs& p, uint8_t* s
                     }
                 }
             }
+            // Issue order inside the slot.  A wavefront issues in order, and a matrix
+            // instruction waits at issue until the one before it has left the matrix core: two
+            // in a row park the vector work behind the second for its whole length, and vector
+            // work ahead of them that waits on an LDS read parks the matrix core.  So: a matrix
+            // instruction, half of the vector work under it, the second, the rest.
+            if (ep && (ks & 3) == 0) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 3, 0);   // M first: the vector work reads it
+            } else {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            }
+            __builtin_amdgcn_sched_group_barrier(0x002, 48, 0);
             __builtin_amdgcn_sched_barrier(0);
         });
         if (half == 1) {
             const int sb2 = min(sb + 1, p.k / 256 - 1);
             da_reg = p.da[(size_t)sb2 * p.tok_pad + t0 + (tid & (TOK - 1))];
         }
-        lds_barrier();
+        if (!(JL_ABL & 16)) lds_barrier();
     };
     stage(GemmIntC<0>{}, GemmIntC<1>{}, 0, wa, wb);
     stage(GemmIntC<1>{}, GemmIntC<0>{}, 1, wb, wa);

@@ -159,7 +159,10 @@ extern "C" __global__ __launch_bounds__(256, 3) void jl_gemm_q4k_w32(GemmArgs p)
 extern "C" __global__ __launch_bounds__(512) void jl_gemm_q4k_r128(GemmArgs p) {
     gemm_q4k_body<2>(p, jl_smem, blockIdx.x * JL_GEMM_TILE, blockIdx.y * 128);
 }
-extern "C" __global__ __launch_bounds__(512) void jl_gemm_q4k_wide(GemmArgs p) { gemm_q4k_wide_body<false>(p, jl_smem); }
+extern "C" __global__ __launch_bounds__(512) void jl_gemm_q4k_wide(GemmArgs p) {
+    gemm_split_slice(p);
+    gemm_q4k_wide_body<false>(p, jl_smem);
+}
 // The same two tiles reading the weights from packed planes (GemmArgs.pqs / pd / psc), after the
 // prep in the planes' K order: no rows are restored first.
 extern "C" __global__ __launch_bounds__(1024) void jl_gemm_prep_q4k_planes(GemmPrepArgs p) {
@@ -170,7 +173,10 @@ extern "C" __global__ __launch_bounds__(256, 2) void jl_gemm_q4k_r64_planes(Gemm
     gemm_split_slice(p);
     gemm_q4k_body<1, false, true>(p, jl_smem, blockIdx.x * JL_GEMM_TILE, blockIdx.y * 64);
 }
-extern "C" __global__ __launch_bounds__(512) void jl_gemm_q4k_wide_planes(GemmArgs p) { gemm_q4k_wide_body<true>(p, jl_smem); }
+extern "C" __global__ __launch_bounds__(512) void jl_gemm_q4k_wide_planes(GemmArgs p) {
+    gemm_split_slice(p);
+    gemm_q4k_wide_body<true>(p, jl_smem);
+}
 extern "C" __global__ __launch_bounds__(256) void jl_gemm_w16_prep_q4k(GemmW16PrepArgs p) {
     __shared__ u32 raw[32 * 37];
     gemm_w16_prep_q4k_body(p, raw);
