@@ -635,6 +635,15 @@ def ceiling_section(dev, gate_):
     out = {}
     ms = measure(dev, lambda i: dev.probe_dev(0, None, 0, 512, 1024), 200, gate_, warm=50)
     out["empty_kernel"] = {"us_per_launch": round(ms * 1e3, 3), "grid": 512, "block": 1024}
+    # the matrix cores with nothing to wait for: 8 wavefronts a CU, 2000 rounds of four
+    # 32x32x16 f16 matrix instructions each; then the same with five vector instructions
+    # after each matrix instruction, the prefill GEMM loop's share
+    rounds, ncu = 2000, 256   # one 512-thread workgroup for each of the MI355X's 256 CUs
+    for key, kind in [("matrix_cores_f16", 3), ("matrix_cores_f16_with_5_vector_instructions_each", 4)]:
+        ms = measure(dev, lambda i: dev.probe_dev(kind, None, rounds, ncu, 512), 5, gate_, warm=2)
+        tf = ncu * 8 * rounds * 4 * 32768.0 / (ms * 1e-3) / 1e12
+        out[key] = {"TFLOP/s": round(tf, 1), "frac_of_f16_mfma_peak": round(tf / MFMA_F16_PEAK_TFLOPS, 4),
+                    "us_per_launch": round(ms * 1e3, 1)}
     pool = DeviceArray(np.random.default_rng(0).integers(0, 1 << 32, (640 << 20) // 4, dtype=np.uint32))
     for name, nbytes in [("9.4 MB (Q4_K 4096x4096)", 9437184), ("33 MB (Q4_K 14336x4096)", 33030144),
                          ("48 MB (Q6_K 4096x14336)", 48168960), ("62 MB (Q8_0 14336x4096)", 62390272)]:

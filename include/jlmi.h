@@ -108,8 +108,12 @@ unsigned long long jl_launch_count(const jl_ctx *ctx);
  * aligned; every thread keeps eight 128-bit loads in flight) and stores nothing; kind 2
  * holds the stream for nbytes MICROSECONDS (<= 100000) on one wavefront that touches no
  * memory -- a benchmark enqueues it in front of a timed window so that the window's
- * launches are all queued before the first starts.  grid and block <= 0 pick two
- * 1024-thread workgroups per CU (kinds 0 and 1). */
+ * launches are all queued before the first starts; kinds 3 and 4 price the matrix cores:
+ * every wavefront issues nbytes ROUNDS (<= 1000000) of four independent 32x32x16 f16 matrix
+ * instructions on registers, kind 4 with five f32 multiply-adds after each (the vector load
+ * of the prefill GEMM's loop) -- 4 * 32768 flops a round a wavefront.  grid and block <= 0
+ * pick two 1024-thread workgroups per CU (kinds 0 and 1), one 512-thread workgroup per CU
+ * (kinds 3 and 4). */
 int jl_probe_dev(jl_ctx *ctx, int kind, const void *src, size_t nbytes, int grid, int block,
                  void *stream);
 

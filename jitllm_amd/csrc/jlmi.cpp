@@ -1174,7 +1174,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     if (e != hipSuccess)
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
-    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_prep_q4k_planes", "jl_gemm_q4k_r64_planes", "jl_gemm_q4k_wide_planes", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_group2_wide", "jl_moe_quant", "jl_moe_matvec_planes_q4k", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_prep_planes", "jl_moe_gemm_q4k", "jl_moe_gemm_r64", "jl_moe_gemm_r64_planes", "jl_moe_gemm_q6k_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_mxfp4_matvec_planes_r64", "jl_mxfp4_matvec_planes_r32", "jl_mxfp4_matvec_planes_r16", "jl_unpack_mxfp4", "jl_sum_parts", "jl_probe_read", "jl_probe_empty", "jl_probe_wait",
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_prep_q4k_planes", "jl_gemm_q4k_r64_planes", "jl_gemm_q4k_wide_planes", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_group2_wide", "jl_moe_quant", "jl_moe_matvec_planes_q4k", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_prep_planes", "jl_moe_gemm_q4k", "jl_moe_gemm_r64", "jl_moe_gemm_r64_planes", "jl_moe_gemm_q6k_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_mxfp4_matvec_planes_r64", "jl_mxfp4_matvec_planes_r32", "jl_mxfp4_matvec_planes_r16", "jl_unpack_mxfp4", "jl_sum_parts", "jl_probe_read", "jl_probe_empty", "jl_probe_wait", "jl_probe_mfma", "jl_probe_mfma_v5",
                                       "jl_pack_weights", "jl_unpack_q4k", "jl_unpack_q6k", "jl_unpack_q8_0"};
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int rw : {16, 32, 64})
@@ -1952,6 +1952,18 @@ int jl_probe_dev(jl_ctx* c, int kind, const void* src, size_t nbytes, int grid, 
         void* none = nullptr;
         void* wp[] = {(void*)&none, (void*)&ticks, (void*)&none};
         return launch(c, "jl_probe_wait", 1, 1, 64, 0, pick_stream(c, stream), wp);
+    }
+    if (kind == 3 || kind == 4) {
+        // matrix-core ceiling: nbytes is the rounds of four matrix instructions a wavefront issues
+        if (nbytes == 0 || nbytes > 1000000) return fail(c, JL_ERR_ARG, "probe: %zu rounds", nbytes);
+        if (grid <= 0) grid = c->num_cu;
+        if (block <= 0) block = 512;
+        if (block % 64 != 0 || block > 1024) return fail(c, JL_ERR_ARG, "probe: block=%d", block);
+        HIP_TRY(c, H->SetDevice(c->device));
+        void* none = nullptr;
+        void* mp[] = {(void*)&none, (void*)&nbytes, (void*)&none};
+        return launch(c, kind == 3 ? "jl_probe_mfma" : "jl_probe_mfma_v5", (unsigned)grid, 1, (unsigned)block, 0,
+                      pick_stream(c, stream), mp);
     }
     if (kind != 0 && kind != 1) return fail(c, JL_ERR_ARG, "probe: kind %d", kind);
     if (grid <= 0) grid = 2 * c->num_cu;

@@ -341,6 +341,51 @@ extern "C" __global__ __launch_bounds__(1024) void jl_probe_read(const u32x4* __
     for (; i < nvec; i += stride) acc ^= __builtin_nontemporal_load(src + i);
     if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x9e3779b9u && sink) sink[0] = acc.x;
 }
+// What the matrix cores deliver with nothing to wait for: every wavefront issues `iters` rounds
+// of four independent 32x32x16 f16 matrix instructions on registers (jl_probe_mfma), and the
+// same with five f32 multiply-adds issued after each of them (jl_probe_mfma_v5, the vector load
+// of the prefill GEMM's loop).  2 * 32 * 32 * 16 flops an instruction.
+template <int V>
+__device__ __forceinline__ void probe_mfma_body(size_t iters, u32* sink) {
+    typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+    typedef float f16v __attribute__((ext_vector_type(16)));
+    h8 a, b;
+#pragma unroll
+    for (int i = 0; i < 8; i++) { a[i] = (_Float16)(int)(threadIdx.x & 3); b[i] = (_Float16)(int)(threadIdx.x & 1); }
+    f16v acc[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+#pragma unroll
+        for (int e = 0; e < 16; e++) acc[j][e] = 0.f;
+    float v[5];
+#pragma unroll
+    for (int i = 0; i < 5; i++) v[i] = (float)threadIdx.x + (float)i;
+    const float c = __uint_as_float(0x3f7ff000u + (threadIdx.x & 1)), d = 0.5f;
+    for (size_t it = 0; it < iters; it++) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc[j], 0, 0, 0);
+#pragma unroll
+            for (int i = 0; i < V; i++) v[i] = fmaf(v[i], c, d);
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if (V > 0) __builtin_amdgcn_sched_group_barrier(0x002, V, 0);
+        }
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+#pragma unroll
+        for (int e = 0; e < 16; e++) s += acc[j][e];
+#pragma unroll
+    for (int i = 0; i < 5; i++) s += v[i];
+    if (sink && __float_as_uint(s) == 0x9e3779b9u) sink[0] = 1;
+}
+extern "C" __global__ __launch_bounds__(1024) void jl_probe_mfma(const u32x4* __restrict__, size_t iters, u32* __restrict__ sink) {
+    probe_mfma_body<0>(iters, sink);
+}
+extern "C" __global__ __launch_bounds__(1024) void jl_probe_mfma_v5(const u32x4* __restrict__, size_t iters, u32* __restrict__ sink) {
+    probe_mfma_body<5>(iters, sink);
+}
 extern "C" __global__ __launch_bounds__(1024) void jl_probe_empty(const u32x4* __restrict__, size_t, u32* __restrict__) {}
 // Holds the stream for `ticks` ticks of the 100 MHz constant clock and touches no memory: what a
 // benchmark enqueues in front of a timed window so that the window's launches are all queued
