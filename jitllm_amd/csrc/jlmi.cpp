@@ -41,6 +41,7 @@ struct Tuning {
     int moe_waves = 0;
     int moe_lpr = 0;
     int mx_rows = 0;
+    int mx_scaled = 0;          // 1: packed MXFP4 matmul on the block-scaled fp8 x fp4 matrix instruction (lossy)
     int mx_planes = 0;          // packed MXFP4, a handful of tokens: 2 restores rows first; 64 / 32 / 16 rows a workgroup
     int mx_split = 0;
 };
@@ -1174,7 +1175,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     if (e != hipSuccess)
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
-    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_prep_q4k_planes", "jl_gemm_q4k_r64_planes", "jl_gemm_q4k_wide_planes", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_group2_wide", "jl_moe_quant", "jl_moe_matvec_planes_q4k", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_prep_planes", "jl_moe_gemm_q4k", "jl_moe_gemm_r64", "jl_moe_gemm_r64_planes", "jl_moe_gemm_q6k_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_mxfp4_matvec_planes_r64", "jl_mxfp4_matvec_planes_r32", "jl_mxfp4_matvec_planes_r16", "jl_unpack_mxfp4", "jl_sum_parts", "jl_probe_read", "jl_probe_empty", "jl_probe_wait", "jl_probe_mfma", "jl_probe_mfma_v5",
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_prep_q4k_planes", "jl_gemm_q4k_r64_planes", "jl_gemm_q4k_wide_planes", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_group2_wide", "jl_moe_quant", "jl_moe_matvec_planes_q4k", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_prep_planes", "jl_moe_gemm_q4k", "jl_moe_gemm_r64", "jl_moe_gemm_r64_planes", "jl_moe_gemm_q6k_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_mxfp4_scaled_prep", "jl_mxfp4_scaled_gemm", "jl_mxfp4_matvec_planes_r64", "jl_mxfp4_matvec_planes_r32", "jl_mxfp4_matvec_planes_r16", "jl_unpack_mxfp4", "jl_sum_parts", "jl_probe_read", "jl_probe_empty", "jl_probe_wait", "jl_probe_mfma", "jl_probe_mfma_v5",
                                       "jl_pack_weights", "jl_unpack_q4k", "jl_unpack_q6k", "jl_unpack_q8_0"};
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int rw : {16, 32, 64})
@@ -1284,6 +1285,7 @@ int jl_set_tuning(jl_ctx* c, const char* key, int value) {
     else if (!strcmp(key, "mxfp4.split")) c->tune.mx_split = value;
     else if (!strcmp(key, "mxfp4.rows")) c->tune.mx_rows = value;
     else if (!strcmp(key, "mxfp4.planes")) c->tune.mx_planes = value;
+    else if (!strcmp(key, "mxfp4.scaled")) c->tune.mx_scaled = value;
     else if (!strcmp(key, "gemm.form")) c->tune.gemm_form = value;
     else if (!strcmp(key, "gemm.split")) c->tune.gemm_split = value;
     else if (!strcmp(key, "gemm.prep")) c->tune.gemm_prep = value;
@@ -1808,6 +1810,27 @@ int jl_matmul_mxfp4_packed_bf16_dev(jl_ctx* c, float* out, const uint32_t* qs, c
     if (!aligned16(x)) return JL_DECLINED;
     HIP_TRY(c, H->SetDevice(c->device));
     hipStream_t st = pick_stream(c, stream);
+    if (c->tune.mx_scaled == 1) {
+        // opt-in: activations to MX fp8, the planes' codes and exponents straight into the
+        // block-scaled matrix instruction (about three bits of every activation are lost)
+        if (ntok > 65535 * 32 || k % 8 != 0) return JL_DECLINED;
+        const int tok_pad = (ntok + 127) / 128 * 128, nks = (k + 63) / 64, ntt = tok_pad / 32;
+        const size_t xa_bytes = (size_t)nks * ntt * 64 * 32;
+        rc = gemm_ws_ensure(c, xa_bytes + (size_t)nks * ntt * 64);
+        if (rc != JL_OK) return rc;
+        MxScaledPrepArgs pa;
+        pa.x = x; pa.xa = (uint32_t*)c->gemm_ws; pa.xs = (uint8_t*)c->gemm_ws + xa_bytes;
+        pa.ntok = ntok; pa.tok_pad = tok_pad; pa.k = k;
+        void* pp[] = {&pa};
+        rc = launch(c, "jl_mxfp4_scaled_prep", (unsigned)((nks + 3) / 4), (unsigned)ntt, 256, 0, st, pp);
+        if (rc != JL_OK) return rc;
+        MxScaledGemmArgs ga;
+        ga.out = out; ga.qs = qs; ga.d = d; ga.xa = pa.xa; ga.xs = pa.xs;
+        ga.nrows = nrows; ga.k = k; ga.ntok = ntok; ga.tok_pad = tok_pad; ga.row0 = row; ga.stride = stride;
+        void* gp[] = {&ga};
+        if (65536u > c->lds_limit) return JL_DECLINED;
+        return launch(c, "jl_mxfp4_scaled_gemm", (unsigned)(tok_pad / 64), (unsigned)((nrows + 63) / 64), 256, 65536, st, gp);
+    }
     if (ntok <= 8 && c->tune.mx_planes != 2) {
         // a handful of tokens: the planes are read where they lie, a lane a row
         MxPlanesArgs a;

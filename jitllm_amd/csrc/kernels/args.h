@@ -261,6 +261,24 @@ struct MxPlanesArgs {
     int nwaves;           // wavefronts of a workgroup; they split the blocks of K
 };
 
+// The opt-in block-scaled form: activations as MX fp8 (e4m3 codes, one E8M0 scale a token and
+// block of 32) in the operand order of the 32x32x64 scaled matrix instruction.
+struct MxScaledPrepArgs {
+    const uint16_t* x;    // [ntok][k] bf16 bits
+    uint32_t* xa;         // [K-step][token tile][64 lanes][8 words]
+    uint8_t* xs;          // [K-step][token tile][64 lanes]
+    int ntok, tok_pad, k;
+};
+
+struct MxScaledGemmArgs {
+    float* out;           // [ntok][nrows]
+    const uint32_t* qs;   // MXFP4 planes, rows row0 .. row0+nrows of `stride`
+    const uint32_t* d;
+    const uint32_t* xa;
+    const uint8_t* xs;
+    int nrows, k, ntok, tok_pad, row0, stride;
+};
+
 // out[i] = part[0][i] + part[1][i] + ... in that order.
 struct SumPartsArgs {
     float* out;

@@ -311,6 +311,12 @@ extern "C" __global__ __launch_bounds__(1024) void jl_mxfp4_matvec_planes_r32(Mx
 extern "C" __global__ __launch_bounds__(1024) void jl_mxfp4_matvec_planes_r16(MxPlanesArgs p) {
     mx_planes_matvec_body<16, 2>(p, (float*)jl_smem);
 }
+// the opt-in block-scaled form over packed planes: prep grid = (ceil(ceil(k/64) / 4), tok_pad/32),
+// block = 256; GEMM grid = (tok_pad/64, ceil(nrows/64)), block = 256, dynamic LDS = 64 KiB
+extern "C" __global__ __launch_bounds__(256) void jl_mxfp4_scaled_prep(MxScaledPrepArgs p) { mx_scaled_prep_body(p); }
+extern "C" __global__ __launch_bounds__(256, 2) void jl_mxfp4_scaled_gemm(MxScaledGemmArgs p) {
+    mx_scaled_gemm_body(p, (float*)jl_smem);
+}
 // 9..64 tokens: prep grid = (ceil(k/128), tiles of 16 tokens), block = 256; kernel grid =
 // ceil(nrows/16), block = 512; _t<NT>: up to 16 NT tokens
 extern "C" __global__ __launch_bounds__(256) void jl_mxfp4_prep_few(MxPrepArgs p) { mx_prep_few_body(p); }

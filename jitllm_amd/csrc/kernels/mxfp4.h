@@ -401,6 +401,154 @@ __device__ __forceinline__ void mx_planes_matvec_body(const MxPlanesArgs& p, flo
     }
 }
 
+// ------------------------------------------------- block-scaled form (opt-in)
+// v_mfma_scale_f32_32x32x64_f8f6f4 takes MXFP4 as it is stored: 32 e2m1 codes a lane (one
+// block: row = lane % 32, block of the K-step = lane / 32, position = nibble index) and the
+// block's E8M0 exponent as the lane's scale.  The other operand cannot be bf16: the activations are quantized to MX fp8
+// (e4m3, a power-of-two scale per token and block of 32, chosen so the block's largest value
+// stays below 448), which costs about three bits of every activation -- so this form is never
+// the default and reports its error beside its time.  The codes of a block are stored byte j =
+// (element j, element j + 16), so the activation block is laid out in that order too:
+// position 2j holds element j, position 2j + 1 element j + 16.
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+typedef short i16x2 __attribute__((ext_vector_type(2)));
+
+// grid = (ceil(K-steps / 4), tok_pad / 32), block = 256: a wavefront per (K-step of 64, 32 tokens)
+__device__ __forceinline__ void mx_scaled_prep_body(const MxScaledPrepArgs& p) {
+    const int lane = threadIdx.x & 63, nks = (p.k + 63) / 64, ntt = p.tok_pad / 32;
+    const int ks = blockIdx.x * 4 + (threadIdx.x >> 6), tile = blockIdx.y;
+    if (ks >= nks) return;
+    const int t = 32 * tile + (lane & 31), b = 2 * ks + (lane >> 5);
+    float v[32];
+    float amax = 0.f;
+    if (t < p.ntok && b < p.k / 32) {
+        const u32x4* src = (const u32x4*)(p.x + (size_t)t * p.k + (size_t)b * 32);
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const u32x4 w = src[c];
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                v[8 * c + 2 * j] = __uint_as_float(w[j] << 16);
+                v[8 * c + 2 * j + 1] = __uint_as_float(w[j] & 0xFFFF0000u);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 32; i++) amax = fmaxf(amax, fabsf(v[i]));
+    } else {
+#pragma unroll
+        for (int i = 0; i < 32; i++) v[i] = 0.f;
+    }
+    // scale 2^(sb - 127): the largest value lands in [224, 448]
+    const u32 bits = __float_as_uint(amax);
+    int sb = (int)((bits >> 23) & 0xFF) - 8 + ((bits & 0x7FFFFFu) > 0x600000u ? 1 : 0);
+    sb = amax == 0.f ? 127 : min(max(sb, 1), 254);
+    const float scale = __uint_as_float((u32)sb << 23);
+    u32 w[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        i16x2 r = {0, 0};
+        r = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(r, v[2 * i], v[2 * i + 16], scale, false);
+        r = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(r, v[2 * i + 1], v[2 * i + 17], scale, true);
+        w[i] = __builtin_bit_cast(u32, r);
+    }
+    // An 8-bit operand keeps, in lane (token, g), positions 16g .. 16g+15 of BOTH blocks of the
+    // K-step (first block in the low four registers); the block's scale stays with lane
+    // (token, block).  So the two lanes of a token trade half a block.
+    const int g = lane >> 5;
+    u32 got[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) got[i] = __shfl_xor(g ? w[i] : w[4 + i], 32);
+    const size_t frag = (size_t)ks * ntt + tile;
+    u32x4* dst = (u32x4*)(p.xa + (frag * 64 + lane) * 8);
+    dst[0] = g ? u32x4{got[0], got[1], got[2], got[3]} : u32x4{w[0], w[1], w[2], w[3]};
+    dst[1] = g ? u32x4{w[4], w[5], w[6], w[7]} : u32x4{got[0], got[1], got[2], got[3]};
+    p.xs[frag * 64 + lane] = (uint8_t)sb;
+}
+
+// grid = (tok_pad / 64, ceil(nrows / 64)), block = 256, LDS = 64 KiB: a workgroup owns 64 tokens x
+// 64 rows (2 x 2 tiles of 32 x 32) and its four wavefronts take the K-steps of 64 in turn --
+// many small workgroups, so that a CU holds enough wavefronts to cover the trip to memory, which
+// is all a loop of loads and matrix instructions has to hide.  Weights come straight from the
+// planes (a lane a row: coalesced), activations from the prepared fragments, both two K-steps
+// ahead of their use; the four partial tiles are added in wavefront order through LDS
+// (red: [wavefront][tile][16][64] floats), wavefront w finishing tile w.
+__device__ __forceinline__ void mx_scaled_gemm_body(const MxScaledGemmArgs& p, float* red) {
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int t0 = blockIdx.x * 64, r0 = blockIdx.y * 64;
+    const int nblk = p.k / 32, nks = (p.k + 63) / 64, ntt = p.tok_pad / 32;
+    const size_t n = (size_t)p.stride, dwords = (n + 3) / 4;
+    size_t row[2];
+    int sh[2];
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        row[j] = (size_t)p.row0 + min(r0 + 32 * j + (lane & 31), p.nrows - 1);
+        sh[j] = 8 * (int)(row[j] & 3);
+    }
+    struct Ops { i32x8 a[2]; u32 sa[2]; i32x8 b[2]; u32 sb[2]; };
+    auto load = [&](int ks, Ops& o) {
+        ks = min(ks, nks - 1);
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const size_t frag = (size_t)ks * ntt + (t0 >> 5) + i;
+            const u32x4* src = (const u32x4*)(p.xa + (frag * 64 + lane) * 8);
+            const u32x4 lo = src[0], hi = src[1];
+            o.a[i] = i32x8{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+            o.sa[i] = p.xs[frag * 64 + lane];
+        }
+        const int b = 2 * ks + (lane >> 5);
+        const bool past = b >= nblk;   // the second block of a last, half K-step
+        const size_t bc = (size_t)(past ? nblk - 1 : b);
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const u32* qp = p.qs + bc * 4 * n + row[j];
+            u32 q[4];
+#pragma unroll
+            for (int w = 0; w < 4; w++) q[w] = past ? 0u : qp[(size_t)w * n];
+            o.b[j] = i32x8{(int)q[0], (int)q[1], (int)q[2], (int)q[3], 0, 0, 0, 0};
+            o.sb[j] = ((p.d[bc * dwords + (row[j] >> 2)] >> sh[j]) + 1) & 0xFF;
+        }
+    };
+    f32x16_t acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
+    Ops o0, o1, o2;
+    load(wave, o0);
+    load(wave + 4, o1);
+    for (int ks = wave; ks < nks; ks += 4) {
+        load(ks + 8, o2);
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(o0.a[i], o0.b[j], acc[i][j], 0, 4, 0,
+                                                                             (int)o0.sa[i], 0, (int)o0.sb[j]);
+        o0 = o1;
+        o1 = o2;
+    }
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) red[((wave * 4 + 2 * i + j) * 16 + e) * 64 + lane] = acc[i][j][e];
+    __syncthreads();
+    const int i = wave >> 1, j = wave & 1, kg = lane >> 5;
+    const int r = r0 + 32 * j + (lane & 31);
+#pragma unroll
+    for (int e = 0; e < 16; e++) {
+        float s = red[((0 * 4 + wave) * 16 + e) * 64 + lane];
+#pragma unroll
+        for (int w = 1; w < 4; w++) s += red[((w * 4 + wave) * 16 + e) * 64 + lane];
+        const int t = t0 + 32 * i + 8 * (e >> 2) + 4 * kg + (e & 3);
+        if (r < p.nrows && t < p.ntok) p.out[(size_t)t * p.nrows + r] = s;
+    }
+}
+
 // grid = ceil(n / 256), block = 256
 __device__ __forceinline__ void sum_parts_body(const SumPartsArgs& p) {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;

@@ -227,3 +227,60 @@ def test_mxfp4_packed_matmul_every_exponent_one_token(dev, devbuf):
     dev.synchronize()
     got = out.get()
     assert np.all(np.isfinite(want)) and np.allclose(got, want, rtol=2e-6, atol=0)
+
+
+# ------------------------------------------------------------------ block-scaled form (opt-in)
+def mx_fp8_activations(xf):
+    """The opt-in form's activation quantizer restated in numpy: per token and block of 32 a
+    power-of-two scale that puts the block's largest magnitude in [224, 448], values rounded to
+    fp8 e4m3 (three mantissa bits, subnormals below 2^-6), nearest even.  Returns the values
+    the matrix instruction multiplies, as f64."""
+    x = xf.astype(np.float64).reshape(xf.shape[0], -1, 32)
+    amax = np.abs(x).max(axis=2, keepdims=True)
+    m, ex = np.frexp(amax)                       # amax = m * 2^ex, m in [0.5, 1)
+    e = ex - 1 - 8 + (2 * m > 1.75)              # floor(log2 amax) - 8, one more above 1.75 * 2^floor
+    scale = np.where(amax > 0, np.exp2(e.astype(np.float64)), 1.0)
+    v = x / scale
+    _, vex = np.frexp(np.abs(v))
+    step = np.exp2(np.maximum(vex - 1, -6) - 3.0)
+    q = np.round(v / step) * step                # numpy rounds halves to even
+    assert np.abs(q).max() <= 448
+    return (q * scale).reshape(xf.shape)
+
+
+@pytest.mark.parametrize("shape", [(1, 64, 64), (40, 130, 96), (128, 128, 2880), (130, 300, 160), (1024, 2880, 2880)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_mxfp4_scaled_form_is_exact_over_its_own_quantizer_and_reports_its_loss(dev, devbuf, shape):
+    """`mxfp4.scaled` = 1 (never the default): the planes' e2m1 codes and E8M0 exponents go into
+    v_mfma_scale_f32_32x32x64_f8f6f4 as they are, the activations as MX fp8.  Against the f64
+    product of the dequantized weights with the SAME fp8 activations the result differs by the
+    instruction's own accumulation (it sums a block's 32 products in less than f32: measured
+    NMSE ~1e-10, bar 1e-8, which still pins the operand layout and the scale bytes: one
+    misplaced element or exponent gives 1e-3 or more);
+    against the bf16 activations the loss is the quantizer's, a few percent rel-L2, stated here
+    and in the benchmark beside the form's time."""
+    from jitllm_amd.device import Packed
+    ntok, nrows, k = shape
+    t = quant.MXFP4
+    w = synth.quantized_weights(t, nrows, k, seed=ntok + 3)
+    xb, xf = to_bf16(np.stack([synth.activations(k, seed=90 + i) for i in range(ntok)]))
+    wd = oracle.dequant(t, w, nrows * k).reshape(nrows, k).astype(np.float64)
+    want_q = mx_fp8_activations(xf) @ wd.T
+    want = xf.astype(np.float64) @ wd.T
+    nq, nd, _ = dev.packed_words(t, nrows, k)
+    qs, d = devbuf(shape=(nq,), dtype=np.uint32), devbuf(shape=(nd,), dtype=np.uint32)
+    assert dev.pack_weights_dev(t, devbuf(w).ptr, nrows, k, qs.ptr, d.ptr, None)
+    out = devbuf(shape=(ntok * nrows + 8,), dtype=np.float32, fill=np.float32(2e30))
+    dev.set_tuning(mxfp4__scaled=1)
+    try:
+        assert dev.matmul_mxfp4_packed_bf16_dev(out.ptr, Packed(qs.ptr, d.ptr, None, 0, nrows), devbuf(xb).ptr, nrows, k, ntok)
+        dev.synchronize()
+    finally:
+        dev.set_tuning(mxfp4__scaled=0)
+    got = out.get()
+    assert np.all(got[ntok * nrows:] == np.float32(2e30))
+    got = got[:ntok * nrows].reshape(ntok, nrows)
+    assert nmse(got, want_q) <= 1e-8, f"NMSE {nmse(got, want_q):.3e} against its own quantizer"
+    loss = rel_l2(got, want)
+    print(f"block-scaled form {shape}: rel-L2 {loss:.3e} against bf16 activations")
+    assert 1e-3 < loss <= 5e-2
