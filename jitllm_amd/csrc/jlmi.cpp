@@ -505,7 +505,9 @@ int gemm_q4k_launch(jl_ctx* c, float* out, const void* w, const float* x, int nr
         const long wide_groups = (long)((ntok + kGemmWideTok - 1) / kGemmWideTok) * ((nrows + 127) / 128);
         // from a quarter of the CUs on: a smaller grid is widened along K below (measured
         // against the 64-row tiles: 1024 tokens x 4096 rows 56 against 62 us, 512 x 4096 38 against 40)
-        form = 4 * wide_groups >= (long)c->num_cu ? 2 : 1;
+        // (not for a last token tile that is mostly padding: 128 tokens x 14336 rows 40 against 45 us)
+        const bool padded = (ntok % kGemmWideTok) != 0 && (ntok % kGemmWideTok) <= kGemmWideTok / 2 && ntok < 2 * kGemmWideTok;
+        form = 4 * wide_groups >= 3 * (long)c->num_cu || (4 * wide_groups >= (long)c->num_cu && !padded) ? 2 : 1;
     }
     if (form == 2 && kGemmWideLdsBytes > c->lds_limit) form = 1;
     const int tile = form == 2 ? kGemmWideTok : kGemmTile;
