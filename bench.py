@@ -39,8 +39,8 @@ CACHE_BYTES = 256 << 20  # Infinity Cache; rotate through more than twice this
 
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # script (profiles/), scaled by the same counters over a plain copy of known
-# size (profiles/matvec_q4k_4096_hbm_traffic.md: fetch 4712.5 x 1.9950 KiB + write 16 KiB).
-MEASURED_TRAFFIC = {"c1": 9643571}
+# size (profiles/matvec_q4k_4096_hbm_traffic.md: fetch 4723.0 x 1.9950 KiB + write 16 KiB).
+MEASURED_TRAFFIC = {"c1": 9664922}
 
 
 def matvec_bytes(t, nrows, k):
