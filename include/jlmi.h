@@ -289,7 +289,7 @@ int jl_reserve_shape(jl_ctx *ctx, int type, int nrows, int k, int ntok, int pack
  * it exists for code under HIP graph capture, tight serving loops and harnesses that forbid
  * hipMalloc.  Same operands, same values, same launches as jl_matmul_dev, but every
  * workspace the call needs (activation fragments, K-split partial sums) is carved from ONE
- * static device array of jl_static_scratch_bytes() bytes (32 MiB) that each GPU holds from
+ * static device array of jl_static_scratch_bytes() bytes (64 MiB) that each GPU holds from
  * library load to process exit; the call allocates nothing, frees nothing and waits for
  * nothing.  A shape whose workspaces do not fit is refused with JL_ERR_NOMEM before
  * anything is launched (jl_last_error says how many bytes it needed).  Every call on a GPU

@@ -5,6 +5,6 @@
 // Its size: enough for every Q4_K / Q6_K / Q8_0 prefill matmul up to 512 tokens of 4096
 // features against 14336 rows (activation fragments 4.7 MiB, K-split partial sums up to 16 MiB)
 // and for 2048 tokens of 4096 features wherever no K split is needed (fragments 18.1 MiB).
-#define JL_STATIC_SCRATCH_BYTES ((size_t)32 << 20)
+#define JL_STATIC_SCRATCH_BYTES ((size_t)64 << 20)
 
 extern "C" int jl_static_scratch_get(int device, void** ptr, size_t* bytes, const char** err);

@@ -51,7 +51,7 @@ def test_static_matmul_equals_matmul_two_calls_in_a_row(dev, devbuf):
     workspaces), the wide tiles, the few-token form, and the window-32 forms of the other
     types."""
     cases = [
-        (quant.Q4_K, 256, 512, 4096, 2048),     # one round of 128 x 64 tiles cut along K: fragments + partial sums
+        (quant.Q4_K, 256, 512, 4096, 2048),     # 64 wide tiles cut four ways along K: fragments + 32 MiB of partial sums
         (quant.Q4_K, 256, 130, 300, 1024),      # smaller, ragged, over the leftovers
         (quant.Q4_K, 256, 512, 9000, 1024),     # 256 x 128 tiles
         (quant.Q4_K, 256, 16, 700, 512),        # few-token form
@@ -69,9 +69,9 @@ def test_static_matmul_equals_matmul_two_calls_in_a_row(dev, devbuf):
 def test_static_matmul_refuses_what_does_not_fit(dev, devbuf):
     """A shape whose activation fragments alone exceed the array: a clear error, and the
     output untouched."""
-    t, ntok, nrows, k = quant.Q4_K, 4096, 64, 4096      # fragments: 16 x 2 x 128 x 9 KiB = 36 MiB > 32 MiB
+    t, ntok, nrows, k = quant.Q4_K, 8192, 64, 4096      # fragments: 16 x 2 x 256 x 9 KiB = 72 MiB > 64 MiB
     dev.SetActWindow(256)
-    assert dev._l.jl_static_scratch_bytes() == 32 << 20
+    assert dev._l.jl_static_scratch_bytes() == 64 << 20
     w = synth.random_weights(t, nrows, k, seed=1)
     wd = devbuf(w)
     xd = devbuf(shape=(ntok, k), dtype=np.float32, fill=1.0)
