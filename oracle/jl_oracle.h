@@ -19,8 +19,11 @@
  *                      packed q5_k_tiny blocks == the libggml golden values)
  *   pack (Q6_K, Q8_0,  round trip RowPacked(pack(src)) == dequant(src) on the
  *         MXFP4)       golden blocks, an independently written numpy reader,
- *                      closed-form plane sizes.  What stays "parity unpinned"
- *                      (held by reading pack.go only, no bytes the reference wrote):
+ *                      closed-form plane sizes; that reader's indexing is also what
+ *                      the reference's own independent gate restates
+ *                      (jit/gpu/kernels/realpack_test.go:67-195, checkPack), so two
+ *                      texts inside the reference agree with it.  What stays "parity
+ *                      unpinned" (held by reading those texts, no bytes the reference wrote):
  *                      Q6_K's SC bytes (int8 + 128, four a word), Q8_0's D pairing
  *                      (two rows' f16 a word), MXFP4's D bytes (e - 1, four rows a word)
  *   act quantizer      numpy float32 brute force incl. rounding-boundary cases

@@ -174,7 +174,13 @@ def test_packed_words_closed_form():
 
 def _numpy_row_reader(t, qs, d, sc, r, nrows, k):
     """An independent, vectorised reader of one row of the planes, written from the layout
-    description rather than from the oracle's loops."""
+    description rather than from the oracle's loops.  Its indexing is also what the reference's
+    own independent gate restates (/root/reference/jit/gpu/kernels/realpack_test.go:67-195,
+    checkPack: "restated, not called"): the Q8_0 D word at sup*((nrows+1)/2) + r/2 with the odd
+    row in the high half (:109-116), the MXFP4 D byte r%4 of word sup*((nrows+3)/4) + r/4 shifted
+    left 23 (:101-107), the Q6_K scale byte (si%4) of word si/4 plus the offset -128 (:138-146),
+    the secondary plane's bit position (:181-187).  So the packer's text (pack.go) and a second
+    statement inside the reference both agree with what is checked here."""
     P = quant.PACKED[t]
     sub, words = P["sub"], P["words"]
     nsub = k // sub
