@@ -354,9 +354,11 @@ int jl_matmul_mxfp4_bf16_dev(jl_ctx *ctx, float *out, const void *w, const uint1
 /* The same over packed MXFP4 planes (jit/gpu/kernels/pack.go:543-575: QS the code bytes
  * four words a block, D the exponent minus one four rows a word; sizes from
  * jl_packed_words, no SC plane): rows row .. row+nrows of planes of `stride` rows.  Up to
- * 8 tokens read the planes where they lie, a lane a row; more tokens restore the row range
- * to GGUF blocks in a workspace the context owns and run the matrix-core forms on it.  The
- * value of a block is that of the GGUF block it was packed from. */
+ * 8 tokens read the planes where they lie, a lane a row; so do more tokens when tiles of
+ * 64 tokens x 64 rows give at least half the CUs a workgroup (a plane word is a lane's
+ * eight K values of the matrix instruction's weight operand); the shapes between restore
+ * the row range to GGUF blocks in a workspace the context owns and run the few-token and
+ * tiled forms on it.  The value of a block is that of the GGUF block it was packed from. */
 int jl_matmul_mxfp4_packed_bf16_dev(jl_ctx *ctx, float *out, const uint32_t *qs, const uint32_t *d,
                                     int row, int stride, const uint16_t *x, int nrows, int k,
                                     int ntok, void *stream);

@@ -42,7 +42,8 @@ struct Tuning {
     int moe_lpr = 0;
     int mx_rows = 0;
     int mx_scaled = 0;          // 1: packed MXFP4 matmul on the block-scaled fp8 x fp4 matrix instruction (lossy)
-    int mx_planes = 0;          // packed MXFP4, a handful of tokens: 2 restores rows first; 64 / 32 / 16 rows a workgroup
+    int mx_planes = 0;          // packed MXFP4: 2 restores rows first, 3 the plane GEMM whatever the grid; 64 / 32 / 16
+                                // rows a workgroup of the plane matvec
     int mx_split = 0;
 };
 
@@ -1177,7 +1178,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     if (e != hipSuccess)
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
-    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_prep_q4k_planes", "jl_gemm_q4k_r64_planes", "jl_gemm_q4k_wide_planes", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_group2_wide", "jl_moe_quant", "jl_moe_matvec_planes_q4k", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_prep_planes", "jl_moe_gemm_q4k", "jl_moe_gemm_r64", "jl_moe_gemm_r64_planes", "jl_moe_gemm_q6k_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_mxfp4_scaled_prep", "jl_mxfp4_scaled_gemm", "jl_mxfp4_matvec_planes_r64", "jl_mxfp4_matvec_planes_r32", "jl_mxfp4_matvec_planes_r16", "jl_unpack_mxfp4", "jl_sum_parts", "jl_probe_read", "jl_probe_empty", "jl_probe_wait", "jl_probe_mfma", "jl_probe_mfma_v5",
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_prep_q4k_planes", "jl_gemm_q4k_r64_planes", "jl_gemm_q4k_wide_planes", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_group2_wide", "jl_moe_quant", "jl_moe_matvec_planes_q4k", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_prep_planes", "jl_moe_gemm_q4k", "jl_moe_gemm_r64", "jl_moe_gemm_r64_planes", "jl_moe_gemm_q6k_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_mxfp4_scaled_prep", "jl_mxfp4_scaled_gemm", "jl_mxfp4_planes_prep", "jl_mxfp4_planes_gemm", "jl_mxfp4_matvec_planes_r64", "jl_mxfp4_matvec_planes_r32", "jl_mxfp4_matvec_planes_r16", "jl_unpack_mxfp4", "jl_sum_parts", "jl_probe_read", "jl_probe_empty", "jl_probe_wait", "jl_probe_mfma", "jl_probe_mfma_v5",
                                       "jl_pack_weights", "jl_unpack_q4k", "jl_unpack_q6k", "jl_unpack_q8_0"};
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int rw : {16, 32, 64})
@@ -1831,7 +1832,9 @@ int jl_matmul_mxfp4_packed_bf16_dev(jl_ctx* c, float* out, const uint32_t* qs, c
         ga.nrows = nrows; ga.k = k; ga.ntok = ntok; ga.tok_pad = tok_pad; ga.row0 = row; ga.stride = stride;
         void* gp[] = {&ga};
         if (65536u > c->lds_limit) return JL_DECLINED;
-        return launch(c, "jl_mxfp4_scaled_gemm", (unsigned)(tok_pad / 64), (unsigned)((nrows + 63) / 64), 256, 65536, st, gp);
+        const long stiles = (long)(tok_pad / 64) * ((nrows + 63) / 64);
+        if (stiles > 0x7fffffffL / 2) return JL_DECLINED;
+        return launch(c, "jl_mxfp4_scaled_gemm", (unsigned)(8 * ((stiles + 7) / 8)), 1, 256, 65536, st, gp);
     }
     if (ntok <= 8 && c->tune.mx_planes != 2) {
         // a handful of tokens: the planes are read where they lie, a lane a row
@@ -1849,7 +1852,27 @@ int jl_matmul_mxfp4_packed_bf16_dev(jl_ctx* c, float* out, const uint32_t* qs, c
         return launch(c, name, (unsigned)((nrows + rl - 1) / rl), 1, (unsigned)(64 * a.nwaves),
                       (unsigned)(a.nwaves * 8 * 64 * 4), st, params);
     }
-    // more tokens: the matrix-core forms stage GGUF blocks, so the rows are restored first
+    // a grid of 64 x 64 tiles that gives most CUs a workgroup: the planes feed the matrix
+    // instruction's weight operand as they lie (a plane word is a lane's eight K values)
+    const long tiles = (long)((ntok + 63) / 64) * ((nrows + 63) / 64);
+    if (c->tune.mx_planes != 2 && (c->tune.mx_planes == 3 || 2 * tiles >= c->num_cu) && ntok <= 65535 * 32 &&
+        k % 8 == 0 && 65536u <= c->lds_limit) {
+        const int tok_pad = (ntok + 63) / 64 * 64, nks = (k + 63) / 64, ntt = tok_pad / 32;
+        rc = gemm_ws_ensure(c, (size_t)nks * ntt * 4 * 1024);
+        if (rc != JL_OK) return rc;
+        MxPlanesPrepArgs pa;
+        pa.x = x; pa.xa = (uint32_t*)c->gemm_ws; pa.ntok = ntok; pa.tok_pad = tok_pad; pa.k = k;
+        void* pp[] = {&pa};
+        rc = launch(c, "jl_mxfp4_planes_prep", (unsigned)((nks + 3) / 4), (unsigned)ntt, 256, 0, st, pp);
+        if (rc != JL_OK) return rc;
+        MxPlanesGemmArgs ga;
+        ga.out = out; ga.qs = qs; ga.d = d; ga.xa = pa.xa;
+        ga.nrows = nrows; ga.k = k; ga.ntok = ntok; ga.tok_pad = tok_pad; ga.row0 = row; ga.stride = stride;
+        void* gp[] = {&ga};
+        if (tiles > 0x7fffffffL / 2) return JL_DECLINED;
+        return launch(c, "jl_mxfp4_planes_gemm", (unsigned)(8 * ((tiles + 7) / 8)), 1, 256, 65536, st, gp);
+    }
+    // fewer tiles: the few-token and tiled forms stage GGUF blocks, so the rows are restored first
     rc = ws_ensure(c, &c->unpack_ws, &c->unpack_ws_bytes, (size_t)nrows * (size_t)(k / 32) * 17);
     if (rc != JL_OK) return rc;
     rc = unpack_launch(c, JL_TYPE_MXFP4, pl, nrows, k, c->unpack_ws, st);

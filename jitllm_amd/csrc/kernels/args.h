@@ -261,6 +261,22 @@ struct MxPlanesArgs {
     int nwaves;           // wavefronts of a workgroup; they split the blocks of K
 };
 
+// MXFP4 planes x bf16, more than a handful of tokens, the planes read where they lie:
+// activation fragments in the planes' K order.
+struct MxPlanesPrepArgs {
+    const uint16_t* x;    // [ntok][k] bf16 bits
+    uint32_t* xa;         // [K-step of 64][token tile of 32][4 matrix K-steps][64 lanes][4 words]
+    int ntok, tok_pad, k;
+};
+
+struct MxPlanesGemmArgs {
+    float* out;           // [ntok][nrows]
+    const uint32_t* qs;   // rows row0 .. row0+nrows of planes of `stride` rows
+    const uint32_t* d;
+    const uint32_t* xa;
+    int nrows, k, ntok, tok_pad, row0, stride;
+};
+
 // The opt-in block-scaled form: activations as MX fp8 (e4m3 codes, one E8M0 scale a token and
 // block of 32) in the operand order of the 32x32x64 scaled matrix instruction.
 struct MxScaledPrepArgs {

@@ -311,8 +311,14 @@ extern "C" __global__ __launch_bounds__(1024) void jl_mxfp4_matvec_planes_r32(Mx
 extern "C" __global__ __launch_bounds__(1024) void jl_mxfp4_matvec_planes_r16(MxPlanesArgs p) {
     mx_planes_matvec_body<16, 2>(p, (float*)jl_smem);
 }
+// MXFP4 planes x bf16 beyond a handful of tokens: prep grid = (ceil(ceil(k/64) / 4), tok_pad/32),
+// block = 256; GEMM grid = 8 * ceil(tiles of 64 x 64 / 8), block = 256, dynamic LDS = 64 KiB
+extern "C" __global__ __launch_bounds__(256) void jl_mxfp4_planes_prep(MxPlanesPrepArgs p) { mx_planes_prep_body(p); }
+extern "C" __global__ __launch_bounds__(256, 2) void jl_mxfp4_planes_gemm(MxPlanesGemmArgs p) {
+    mx_planes_gemm_body(p, (float*)jl_smem);
+}
 // the opt-in block-scaled form over packed planes: prep grid = (ceil(ceil(k/64) / 4), tok_pad/32),
-// block = 256; GEMM grid = (tok_pad/64, ceil(nrows/64)), block = 256, dynamic LDS = 64 KiB
+// block = 256; GEMM grid = 8 * ceil(tiles of 64 x 64 / 8), block = 256, dynamic LDS = 64 KiB
 extern "C" __global__ __launch_bounds__(256) void jl_mxfp4_scaled_prep(MxScaledPrepArgs p) { mx_scaled_prep_body(p); }
 extern "C" __global__ __launch_bounds__(256, 2) void jl_mxfp4_scaled_gemm(MxScaledGemmArgs p) {
     mx_scaled_gemm_body(p, (float*)jl_smem);

@@ -401,6 +401,176 @@ __device__ __forceinline__ void mx_planes_matvec_body(const MxPlanesArgs& p, flo
     }
 }
 
+// ------------------------------------------------- the GEMM over packed planes
+// More than a handful of tokens over MX4 planes, nothing restored: a lane of the matrix
+// instruction's weight operand is (row = lane % 32, kg = lane / 32), and with the planes laid
+// [block][word][row] its eight K values of a 16-deep step are ONE plane word -- word 2s + kg of
+// the block for the block's step s -- read coalesced (32 consecutive rows) and decoded by four
+// conversions with the block's scale.  The word holds elements 4w..4w+3 in its low nibbles and
+// 4w+16..4w+19 in its high ones, and a conversion gives a byte's pair, so the operand's K order
+// is 4w, 4w+16, 4w+1, 4w+17, ...; the prep kernel lays the activation fragments out in that order.
+// A workgroup owns 64 tokens x 64 rows (2 x 2 tiles) and its four wavefronts take the K-steps of
+// 64 (two blocks) in turn: many small workgroups, so a CU holds enough wavefronts to cover the
+// trip to memory; the four partial tiles meet in LDS in wavefront order, wavefront w finishing
+// tile w (red: [wavefront][tile][16][64] floats).
+//
+// Tile of workgroup L in a 1-D grid of 8 * ceil(tiles / 8): the hardware deals consecutive
+// workgroups round the eight XCDs, each with an L2 of its own, so XCD x = L % 8 is given a
+// contiguous run of the token-major tile order -- its workgroups share a few token tiles, whose
+// activation fragments then stay in that L2 while the row tiles walk past.  False: no tile.
+__device__ __forceinline__ bool mx_xcd_tile(int ntt64, int nrt, int& tt, int& rt) {
+    const int tiles = ntt64 * nrt, per = (tiles + 7) / 8;
+    const int g = (int)(blockIdx.x & 7) * per + (int)(blockIdx.x >> 3);
+    if ((int)(blockIdx.x >> 3) >= per || g >= tiles) return false;
+    tt = g / nrt;
+    rt = g - tt * nrt;
+    return true;
+}
+
+// prep: grid = (ceil(K-steps / 4), tok_pad / 32), block = 256: a wavefront per (K-step, 32 tokens)
+__device__ __forceinline__ void mx_planes_prep_body(const MxPlanesPrepArgs& p) {
+    const int lane = threadIdx.x & 63, nks = (p.k + 63) / 64, ntt = p.tok_pad / 32;
+    const int ks = blockIdx.x * 4 + (threadIdx.x >> 6), tile = blockIdx.y;
+    if (ks >= nks) return;
+    const int t = 32 * tile + (lane & 31), kg = lane >> 5, nblk = p.k / 32;
+    u32x4* dst = (u32x4*)p.xa + ((size_t)ks * ntt + tile) * 4 * 64 + lane;
+#pragma unroll
+    for (int s4 = 0; s4 < 4; s4++) {
+        const int b = 2 * ks + (s4 >> 1), w = 2 * (s4 & 1) + kg;
+        u32x4 v = u32x4{0u, 0u, 0u, 0u};
+        if (t < p.ntok && b < nblk) {
+            const uint16_t* src = p.x + (size_t)t * p.k + (size_t)b * 32 + 4 * w;
+            const u32x2 lo = *(const u32x2*)src, hi = *(const u32x2*)(src + 16);
+            // elements (4w, 4w+1 | 4w+2, 4w+3) and (4w+16, 4w+17 | 4w+18, 4w+19), interleaved
+            v.x = (lo.x & 0xFFFFu) | (hi.x << 16);
+            v.y = (lo.x >> 16) | (hi.x & 0xFFFF0000u);
+            v.z = (lo.y & 0xFFFFu) | (hi.y << 16);
+            v.w = (lo.y >> 16) | (hi.y & 0xFFFF0000u);
+        }
+        dst[(size_t)s4 * 64] = v;
+    }
+}
+
+// grid = 8 * ceil(tiles / 8) (mx_xcd_tile), block = 256, dynamic LDS = 64 KiB
+__device__ __forceinline__ void mx_planes_gemm_body(const MxPlanesGemmArgs& p, float* red) {
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    int tt, rt;
+    if (!mx_xcd_tile(p.tok_pad / 64, (p.nrows + 63) / 64, tt, rt)) return;
+    const int t0 = tt * 64, r0 = rt * 64;
+    const int nblk = p.k / 32, nks = (p.k + 63) / 64, ntt = p.tok_pad / 32, kg = lane >> 5;
+    const size_t n = (size_t)p.stride, dwords = (n + 3) / 4;
+    // every load is a uniform base (scalar registers) plus a 32-bit lane offset
+    u32 qoff[2][2], doff[2];
+    int sh[2];
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        const u32 row = (u32)p.row0 + (u32)min(r0 + 32 * j + (lane & 31), p.nrows - 1);
+        sh[j] = 8 * (int)(row & 3);
+        doff[j] = row >> 2;
+#pragma unroll
+        for (int s = 0; s < 2; s++) qoff[j][s] = (u32)(2 * s + kg) * (u32)p.stride + row;
+    }
+    struct WOps { u32 q[2][4]; u32 d[2][2]; };     // [row tile][matrix K-step], [row tile][block]
+    struct AOps { u32x4 a[2][4]; };                // [token tile][matrix K-step]
+    auto load_w = [&](int ks, WOps& o) {
+        ks = min(ks, nks - 1);
+#pragma unroll
+        for (int bi = 0; bi < 2; bi++) {
+            const int b = 2 * ks + bi;
+            const bool past = b >= nblk;   // the second block of a last, half K-step (uniform)
+            const size_t bc = (size_t)(past ? nblk - 1 : b);
+            const u32* qb = p.qs + bc * 4 * n;
+            const u32* db = p.d + bc * dwords;
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+#pragma unroll
+                for (int s = 0; s < 2; s++) {
+                    const u32 v = qb[qoff[j][s]];
+                    o.q[j][2 * bi + s] = past ? 0u : v;
+                }
+                o.d[j][bi] = db[doff[j]];
+            }
+        }
+    };
+    const u32 aoff = (u32)lane * 4;
+    auto load_a = [&](int ks, AOps& o) {
+        ks = min(ks, nks - 1);
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const u32* ab = p.xa + ((size_t)ks * ntt + (t0 >> 5) + i) * (4 * 64 * 4);
+#pragma unroll
+            for (int s4 = 0; s4 < 4; s4++) o.a[i][s4] = *(const u32x4*)(ab + aoff + s4 * 256);
+        }
+    };
+    f32x16_t acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
+    auto compute = [&](const WOps& wo, const AOps& ao) {
+#pragma unroll
+        for (int s4 = 0; s4 < 4; s4++) {
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                const float scale = mx_scale((uint8_t)(((wo.d[j][s4 >> 1] >> sh[j]) & 0xFF) + 1));
+                const u32 q = wo.q[j][s4];
+                u32x4 wb;
+                wb.x = __builtin_bit_cast(u32, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(q, scale, 0));
+                wb.y = __builtin_bit_cast(u32, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(q, scale, 1));
+                wb.z = __builtin_bit_cast(u32, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(q, scale, 2));
+                wb.w = __builtin_bit_cast(u32, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(q, scale, 3));
+                const bf16x8 wf = __builtin_bit_cast(bf16x8, wb);
+#pragma unroll
+                for (int i = 0; i < 2; i++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, ao.a[i][s4]), wf,
+                                                                         acc[i][j], 0, 0, 0);
+            }
+        }
+    };
+    // Operand sets in rotation -- three of weights (from HBM: loaded two K-steps before their
+    // use), two of activations (from L2: one K-step) -- and the loop unrolled by six so that no
+    // set is ever copied (a copy would wait for the load it copies).
+    WOps w0, w1, w2;
+    AOps a0, a1;
+    load_w(wave, w0);
+    load_a(wave, a0);
+    load_w(wave + 4, w1);
+#define JL_MXP_STEP(N, WL, AL, WC, AC)                   \
+    load_w(wave + 4 * (n + (N) + 2), WL);                \
+    load_a(wave + 4 * (n + (N) + 1), AL);                \
+    if (n + (N) < my_steps) compute(WC, AC);
+    const int my_steps = (nks - wave + 3) / 4;   // K-steps wave, wave + 4, ... (uniform)
+    for (int n = 0; n < my_steps; n += 6) {
+        JL_MXP_STEP(0, w2, a1, w0, a0)
+        JL_MXP_STEP(1, w0, a0, w1, a1)
+        JL_MXP_STEP(2, w1, a1, w2, a0)
+        JL_MXP_STEP(3, w2, a0, w0, a1)
+        JL_MXP_STEP(4, w0, a1, w1, a0)
+        JL_MXP_STEP(5, w1, a0, w2, a1)
+    }
+#undef JL_MXP_STEP
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) red[((wave * 4 + 2 * i + j) * 16 + e) * 64 + lane] = acc[i][j][e];
+    __syncthreads();
+    const int i = wave >> 1, j = wave & 1;
+    const int r = r0 + 32 * j + (lane & 31);
+#pragma unroll
+    for (int e = 0; e < 16; e++) {
+        float s = red[((0 * 4 + wave) * 16 + e) * 64 + lane];
+#pragma unroll
+        for (int w = 1; w < 4; w++) s += red[((w * 4 + wave) * 16 + e) * 64 + lane];
+        const int t = t0 + 32 * i + 8 * (e >> 2) + 4 * kg + (e & 3);
+        if (r < p.nrows && t < p.ntok) p.out[(size_t)t * p.nrows + r] = s;
+    }
+}
+
 // ------------------------------------------------- block-scaled form (opt-in)
 // v_mfma_scale_f32_32x32x64_f8f6f4 takes MXFP4 as it is stored: 32 e2m1 codes a lane (one
 // block: row = lane % 32, block of the K-step = lane / 32, position = nibble index) and the
@@ -465,7 +635,7 @@ __device__ __forceinline__ void mx_scaled_prep_body(const MxScaledPrepArgs& p) {
     p.xs[frag * 64 + lane] = (uint8_t)sb;
 }
 
-// grid = (tok_pad / 64, ceil(nrows / 64)), block = 256, LDS = 64 KiB: a workgroup owns 64 tokens x
+// grid = 8 * ceil(tiles / 8) (mx_xcd_tile), block = 256, LDS = 64 KiB: a workgroup owns 64 tokens x
 // 64 rows (2 x 2 tiles of 32 x 32) and its four wavefronts take the K-steps of 64 in turn --
 // many small workgroups, so that a CU holds enough wavefronts to cover the trip to memory, which
 // is all a loop of loads and matrix instructions has to hide.  Weights come straight from the
@@ -475,7 +645,9 @@ __device__ __forceinline__ void mx_scaled_prep_body(const MxScaledPrepArgs& p) {
 __device__ __forceinline__ void mx_scaled_gemm_body(const MxScaledGemmArgs& p, float* red) {
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-    const int t0 = blockIdx.x * 64, r0 = blockIdx.y * 64;
+    int tt, rt;
+    if (!mx_xcd_tile(p.tok_pad / 64, (p.nrows + 63) / 64, tt, rt)) return;
+    const int t0 = tt * 64, r0 = rt * 64;
     const int nblk = p.k / 32, nks = (p.k + 63) / 64, ntt = p.tok_pad / 32;
     const size_t n = (size_t)p.stride, dwords = (n + 3) / 4;
     size_t row[2];
@@ -516,19 +688,28 @@ __device__ __forceinline__ void mx_scaled_gemm_body(const MxScaledGemmArgs& p, f
         for (int j = 0; j < 2; j++)
 #pragma unroll
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
-    Ops o0, o1, o2;
-    load(wave, o0);
-    load(wave + 4, o1);
-    for (int ks = wave; ks < nks; ks += 4) {
-        load(ks + 8, o2);
+    auto compute = [&](const Ops& o) {
 #pragma unroll
         for (int i = 0; i < 2; i++)
 #pragma unroll
             for (int j = 0; j < 2; j++)
-                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(o0.a[i], o0.b[j], acc[i][j], 0, 4, 0,
-                                                                             (int)o0.sa[i], 0, (int)o0.sb[j]);
-        o0 = o1;
-        o1 = o2;
+                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(o.a[i], o.b[j], acc[i][j], 0, 4, 0,
+                                                                             (int)o.sa[i], 0, (int)o.sb[j]);
+    };
+    // three operand sets in rotation, the loop unrolled by three so that no set is ever copied
+    // (a copy would wait for the load it copies)
+    Ops o0, o1, o2;
+    load(wave, o0);
+    load(wave + 4, o1);
+    for (int ks = wave; ks < nks; ks += 12) {
+        load(ks + 8, o2);
+        compute(o0);
+        if (ks + 4 >= nks) break;
+        load(ks + 12, o0);
+        compute(o1);
+        if (ks + 8 >= nks) break;
+        load(ks + 16, o1);
+        compute(o2);
     }
 #pragma unroll
     for (int i = 0; i < 2; i++)

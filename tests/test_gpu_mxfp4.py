@@ -159,7 +159,8 @@ def test_mxfp4_device_pack_refuses_what_the_reference_refuses(dev, devbuf):
 
 
 @pytest.mark.parametrize("shape", [(1, 2880, 2880), (1, 5760, 2880), (2, 100, 512), (8, 130, 96), (5, 64, 32),
-                                   (7, 257, 544), (64, 2880, 2880), (9, 129, 160)],
+                                   (7, 257, 544), (64, 2880, 2880), (9, 129, 160), (130, 200, 224), (1024, 2880, 2880),
+                                   (300, 70, 96)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_mxfp4_packed_matmul_vs_dequant_f32(dev, devbuf, shape):
     """Planes written by the device packer, read by the plane kernel (up to 8 tokens) or restored
@@ -176,24 +177,31 @@ def test_mxfp4_packed_matmul_vs_dequant_f32(dev, devbuf, shape):
     qs, d = devbuf(shape=(nq,), dtype=np.uint32), devbuf(shape=(nd,), dtype=np.uint32)
     assert dev.pack_weights_dev(t, dw.ptr, nrows, k, qs.ptr, d.ptr, None)
     out = devbuf(shape=(ntok * nrows + 8,), dtype=np.float32, fill=np.float32(2e30))
-    forms = (0, 64, 32, 16, 2) if ntok <= 8 else (0,)   # rows a workgroup of the plane kernel; 2: restore rows
+    # mxfp4.planes: up to 8 tokens 64 / 32 / 16 = rows a workgroup of the plane matvec; more tokens
+    # 3 = the plane GEMM whatever the grid; 2 = restore rows first (the GGUF path's bits)
+    forms = (0, 64, 32, 16, 2) if ntok <= 8 else (0, 3, 2)
+    got_by_form = {}
     for form in forms:
         dev.set_tuning(mxfp4__planes=form)
+        out.put(np.full(ntok * nrows + 8, np.float32(2e30)))
         n0 = dev.launch_count()
         assert dev.matmul_mxfp4_packed_bf16_dev(out.ptr, Packed(qs.ptr, d.ptr, None, 0, nrows), dx.ptr, nrows, k, ntok)
         dev.synchronize()
         if ntok <= 8 and form != 2:
             assert dev.launch_count() - n0 == 1
+        if form == 3:
+            assert dev.launch_count() - n0 == 2      # prep + the plane GEMM, nothing restored
         got = out.get()
         assert np.all(got[ntok * nrows:] == np.float32(2e30))
         got = got[:ntok * nrows].reshape(ntok, nrows)
-        assert nmse(got, want) <= 1e-10 and rel_l2(got, want) <= 1e-3, f"form {form}"
+        assert nmse(got, want) <= 1e-10 and rel_l2(got, want) <= 1e-3, f"form {form}: NMSE {nmse(got, want):.3e}"
+        got_by_form[form] = got
     dev.set_tuning(mxfp4__planes=0)
     if ntok > 8:
         ref = devbuf(shape=(ntok, nrows), dtype=np.float32)
         assert dev.matmul_mxfp4_bf16_dev(ref.ptr, dw.ptr, dx.ptr, nrows, k, ntok)
         dev.synchronize()
-        assert np.array_equal(ref.get(), got)
+        assert np.array_equal(ref.get(), got_by_form[2])
     # a row range of the planes: rows r0 .. r0+n of the same buffer
     if nrows >= 100:
         r0, n = 37, nrows - 70
