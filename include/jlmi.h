@@ -278,8 +278,9 @@ int jl_matmul_dev(jl_ctx *ctx, float *out, int type, const void *w, const float 
 int jl_reserve(jl_ctx *ctx, int max_tok, int max_k);
 
 /* The same for one call shape, exactly: walks the launch path of jl_matmul_dev
- * (packed = 0), jl_matmul_packed_dev (packed = 1) or jl_matmul_mxfp4_bf16_dev (type
- * MXFP4) for this type, shape and the context's current activation window with
+ * (packed = 0), jl_matmul_packed_dev (packed = 1) or, for type MXFP4,
+ * jl_matmul_mxfp4_bf16_dev / jl_matmul_mxfp4_packed_bf16_dev, for this type, shape and the
+ * context's current activation window (and tuning) with
  * launching switched off, so every workspace that call would grow -- activation
  * fragments, rows restored from planes, K-split partial sums -- has its size
  * afterwards and the call itself allocates nothing.  Returns what the call would. */

@@ -1555,7 +1555,9 @@ int jl_reserve_shape(jl_ctx* c, int type, int nrows, int k, int ntok, int packed
     c->dry_run = true;
     int rc;
     if (type == JL_TYPE_MXFP4) {
-        rc = packed ? JL_DECLINED : jl_matmul_mxfp4_bf16_dev(c, out, w, (const uint16_t*)w, nrows, k, ntok, nullptr);
+        rc = packed ? jl_matmul_mxfp4_packed_bf16_dev(c, out, (const uint32_t*)w, (const uint32_t*)w, 0, nrows,
+                                                      (const uint16_t*)w, nrows, k, ntok, nullptr)
+                    : jl_matmul_mxfp4_bf16_dev(c, out, w, (const uint16_t*)w, nrows, k, ntok, nullptr);
     } else if (packed) {
         const PlaneRef pl = {(const uint32_t*)w, (const uint32_t*)w, (const uint32_t*)w, 0, nrows};
         rc = packed_matmul_launch(c, out, type, pl, x, nrows, k, ntok, c->stream);

@@ -292,3 +292,33 @@ def test_mxfp4_scaled_form_is_exact_over_its_own_quantizer_and_reports_its_loss(
     loss = rel_l2(got, want)
     print(f"block-scaled form {shape}: rel-L2 {loss:.3e} against bf16 activations")
     assert 1e-3 < loss <= 5e-2
+
+
+@pytest.mark.parametrize("tuning", [{}, {"mxfp4__planes": 2}, {"mxfp4__scaled": 1}], ids=["auto", "restore", "scaled"])
+def test_mxfp4_packed_reserve_shape_leaves_nothing_to_allocate(dev, devbuf, tuning):
+    """jl_reserve_shape walks the packed MXFP4 call's own launch path (fragments of the plane GEMM,
+    restored rows, the block-scaled form's fp8 fragments): afterwards the call itself allocates
+    nothing, for shapes that grow on the one before."""
+    from jitllm_amd.device import Packed
+    from jitllm_amd.hipmem import mem_info
+    t = quant.MXFP4
+    dev.set_tuning(**tuning)
+    try:
+        for ntok, nrows, k in [(200, 640, 1024), (520, 1100, 2048), (48, 300, 4096)]:
+            w = synth.quantized_weights(t, nrows, k, seed=ntok)
+            xb, xf = to_bf16(np.stack([synth.activations(k, seed=3 + i) for i in range(ntok)]))
+            nq, nd, _ = dev.packed_words(t, nrows, k)
+            qs, d = devbuf(shape=(nq,), dtype=np.uint32), devbuf(shape=(nd,), dtype=np.uint32)
+            assert dev.pack_weights_dev(t, devbuf(w).ptr, nrows, k, qs.ptr, d.ptr, None)
+            dx = devbuf(xb)
+            out = devbuf(shape=(ntok, nrows), dtype=np.float32)
+            assert dev.reserve_shape(t, nrows, k, ntok, packed=True)
+            dev.synchronize()
+            free_before, _ = mem_info()
+            assert dev.matmul_mxfp4_packed_bf16_dev(out.ptr, Packed(qs.ptr, d.ptr, None, 0, nrows), dx.ptr, nrows, k, ntok)
+            dev.synchronize()
+            assert mem_info()[0] == free_before, f"{ntok} x {k} -> {nrows}: the call allocated"
+            want = xf.astype(np.float64) @ oracle.dequant(t, w, nrows * k).reshape(nrows, k).astype(np.float64).T
+            assert rel_l2(out.get(), want) <= (5e-2 if tuning.get("mxfp4__scaled") else 1e-3)
+    finally:
+        dev.set_tuning(**{k_: 0 for k_ in tuning})
