@@ -306,7 +306,7 @@ class CpuPath:
         pp = C.POINTER(_u32p)
         self._l.jlc_time_matvec.restype = C.c_double
         self._l.jlc_time_matvec.argtypes = [C.c_void_p, _f32p, C.c_int, pp, pp, pp, C.c_int, _f32p,
-                                            C.c_int, C.c_int, C.c_int, C.c_int]
+                                            C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
         self._l.jlc_membw.restype = C.c_double
         self._l.jlc_membw.argtypes = [C.c_int, C.c_size_t, C.c_int]
         self.threads = threads
@@ -330,14 +330,15 @@ class CpuPath:
             raise ValueError("cpu matvec refused")
         return out
 
-    def time_matvec(self, t, copies, x, nrows, k, window, reps=5):
-        """copies: list of (qs, d, sc) distinct plane sets.  Seconds per call (best of reps)."""
+    def time_matvec(self, t, copies, x, nrows, k, window, reps=9, sweeps=1):
+        """copies: list of (qs, d, sc) distinct plane sets.  Seconds per call: the median of `reps`
+        timed passes of `sweeps` sweeps over all the copies."""
         n = len(copies)
         arr = lambda i: (_u32p * n)(*[_p(c[i], _u32p) for c in copies])
         x = _chk(x, np.float32, k)
         out = np.zeros(nrows, np.float32)
         s = self._l.jlc_time_matvec(self._p, _p(out, _f32p), t, arr(0), arr(1), arr(2), n,
-                                    _p(x, _f32p), nrows, k, window, reps)
+                                    _p(x, _f32p), nrows, k, window, reps, sweeps)
         if s < 0:
             raise ValueError("cpu timing refused")
         return s

@@ -342,23 +342,32 @@ int jlc_matvec_packed(pool_t *p, float *out, int type, const uint32_t *qs, const
 /* Streams `n` distinct packed copies `reps` times and returns the best seconds per
  * call (3 warm calls first), the reference's protocol for a bandwidth-bound shape
  * (engine/nn/perbyte_test.go:184-292). */
+/* Seconds per call: 3 warm calls, then `reps` timed passes (at most 32) of `sweeps` sweeps over
+ * all the copies each; the MEDIAN pass (the reference's protocol, engine/nn/perbyte_test.go:131-144). */
 double jlc_time_matvec(pool_t *p, float *out, int type, const uint32_t *const *qs,
                        const uint32_t *const *d, const uint32_t *const *sc, int ncopies,
-                       const float *x, int nrows, int k, int window, int reps) {
+                       const float *x, int nrows, int k, int window, int reps, int sweeps) {
+    double pass[32];
+    if (reps < 1 || reps > 32 || sweeps < 1) return -1;
     for (int i = 0; i < 3; i++)
         if (jlc_matvec_packed(p, out, type, qs[i % ncopies], d[i % ncopies], sc ? sc[i % ncopies] : NULL,
                               x, nrows, k, window)) return -1;
-    double best = 1e30;
     for (int r = 0; r < reps; r++) {
         struct timespec t0, t1;
         clock_gettime(CLOCK_MONOTONIC, &t0);
-        for (int i = 0; i < ncopies; i++)
-            jlc_matvec_packed(p, out, type, qs[i], d[i], sc ? sc[i] : NULL, x, nrows, k, window);
+        for (int s = 0; s < sweeps; s++)
+            for (int i = 0; i < ncopies; i++)
+                jlc_matvec_packed(p, out, type, qs[i], d[i], sc ? sc[i] : NULL, x, nrows, k, window);
         clock_gettime(CLOCK_MONOTONIC, &t1);
-        double s = ((t1.tv_sec - t0.tv_sec) + 1e-9 * (t1.tv_nsec - t0.tv_nsec)) / ncopies;
-        if (s < best) best = s;
+        pass[r] = ((t1.tv_sec - t0.tv_sec) + 1e-9 * (t1.tv_nsec - t0.tv_nsec)) / ((double)ncopies * sweeps);
     }
-    return best;
+    for (int a = 1; a < reps; a++) {   /* insertion sort */
+        double v = pass[a];
+        int b = a - 1;
+        for (; b >= 0 && pass[b] > v; b--) pass[b + 1] = pass[b];
+        pass[b + 1] = v;
+    }
+    return reps & 1 ? pass[reps / 2] : 0.5 * (pass[reps / 2 - 1] + pass[reps / 2]);
 }
 
 /* Read-bandwidth wall of the host: every worker sums a private slice of `bytes`
