@@ -1178,7 +1178,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     if (e != hipSuccess)
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
-    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_prep_q4k_planes", "jl_gemm_q4k_r64_planes", "jl_gemm_q4k_wide_planes", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_group2_wide", "jl_moe_quant", "jl_moe_matvec_planes_q4k", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_prep_planes", "jl_moe_gemm_q4k", "jl_moe_gemm_r64", "jl_moe_gemm_r64_planes", "jl_moe_gemm_q6k_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_mxfp4_scaled_prep", "jl_mxfp4_scaled_gemm", "jl_mxfp4_planes_prep", "jl_mxfp4_planes_gemm", "jl_mxfp4_matvec_planes_r64", "jl_mxfp4_matvec_planes_r32", "jl_mxfp4_matvec_planes_r16", "jl_unpack_mxfp4", "jl_sum_parts", "jl_probe_read", "jl_probe_empty", "jl_probe_wait", "jl_probe_mfma", "jl_probe_mfma_v5",
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_prep_q4k_planes", "jl_gemm_q4k_r64_planes", "jl_gemm_q4k_wide_planes", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_group2_wide", "jl_moe_quant", "jl_moe_matvec_planes_q4k", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_prep_planes", "jl_moe_gemm_q4k", "jl_moe_gemm_r64", "jl_moe_gemm_r64_planes", "jl_moe_gemm_q6k_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_mxfp4_matvec1_b1", "jl_mxfp4_matvec1_b2", "jl_mxfp4_matvec1_b3", "jl_mxfp4_scaled_prep", "jl_mxfp4_scaled_gemm", "jl_mxfp4_planes_prep", "jl_mxfp4_planes_gemm", "jl_mxfp4_matvec_planes_r64", "jl_mxfp4_matvec_planes_r32", "jl_mxfp4_matvec_planes_r16", "jl_unpack_mxfp4", "jl_sum_parts", "jl_probe_read", "jl_probe_empty", "jl_probe_wait", "jl_probe_mfma", "jl_probe_mfma_v5",
                                       "jl_pack_weights", "jl_unpack_q4k", "jl_unpack_q6k", "jl_unpack_q8_0"};
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int rw : {16, 32, 64})
@@ -1739,6 +1739,13 @@ int jl_matmul_mxfp4_bf16_dev(jl_ctx* c, float* out, const void* w, const uint16_
     a.nsplit = 1; a.part = nullptr; a.tok_pad = 0;
     void* params[] = {&a};
     hipStream_t st = pick_stream(c, stream);
+    if (ntok == 1 && k <= 3 * 2048 && c->tune.mx_rows != 1) {
+        // one token: the activation stays in registers while a wavefront walks four rows
+        const int nbi = (k / 32 + 63) / 64;
+        char name[32];
+        snprintf(name, sizeof name, "jl_mxfp4_matvec1_b%d", nbi);
+        return launch(c, name, (unsigned)((nrows + 15) / 16), 1, 256, 0, st, params);
+    }
     if (ntok <= 8)  // a handful of tokens: stream the rows once, no tile to fill
         return launch(c, "jl_mxfp4_matvec", (unsigned)((nrows + 3) / 4), 1, 256, 0, st, params);
     if (ntok <= 64 && c->tune.mx_rows != 96 && c->tune.mx_rows != 128) {

@@ -300,6 +300,10 @@ extern "C" __global__ __launch_bounds__(512) void jl_mxfp4_gemm_r96(MxGemmArgs p
 extern "C" __global__ __launch_bounds__(256) void jl_sum_parts(SumPartsArgs p) { sum_parts_body(p); }
 // grid = ceil(nrows/4), block = 256: one wavefront per row, ntok <= 8
 extern "C" __global__ __launch_bounds__(256) void jl_mxfp4_matvec(MxGemmArgs p) { mx_matvec_body(p); }
+// one token, _b<blocks a lane holds>: grid = ceil(nrows / (4 wavefronts * 4 rows)), block = 256
+extern "C" __global__ __launch_bounds__(256) void jl_mxfp4_matvec1_b1(MxGemmArgs p) { mx_matvec1_body<1>(p); }
+extern "C" __global__ __launch_bounds__(256) void jl_mxfp4_matvec1_b2(MxGemmArgs p) { mx_matvec1_body<2>(p); }
+extern "C" __global__ __launch_bounds__(256) void jl_mxfp4_matvec1_b3(MxGemmArgs p) { mx_matvec1_body<3>(p); }
 // ntok <= 8 over packed planes, _r<rows a workgroup>: grid = ceil(nrows/R), block = 64 * nwaves,
 // LDS = nwaves * 8 * 64 floats
 extern "C" __global__ __launch_bounds__(1024) void jl_mxfp4_matvec_planes_r64(MxPlanesArgs p) {

@@ -236,8 +236,11 @@ __device__ __forceinline__ void mx_gemm_body(const MxGemmArgs& p, uint8_t* smem)
     }
 }
 
-// A few tokens (ntok <= 8): one wavefront per row, lane l takes blocks l, l+64, ...;
-// weights decode to f32 pairs, activations (bf16 in global memory) widen to f32.
+// A few tokens (ntok <= 8): one wavefront per row, lane l takes blocks l, l+64, ...
+// A conversion turns a code byte into the bf16 pair (element j, element j + 16), exact; the
+// matching activation pair is picked out of two of the block's words with one byte permute,
+// and v_dot2_f32_bf16 adds the pair's two products to the f32 sum: three vector instructions
+// for two weights per token where widening everything to f32 took five.
 __device__ __forceinline__ void mx_matvec_body(const MxGemmArgs& p) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
     const int row = blockIdx.x * nwaves + wave;
@@ -250,35 +253,30 @@ __device__ __forceinline__ void mx_matvec_body(const MxGemmArgs& p) {
         const uint8_t* blk = p.w + (size_t)row * p.row_bytes + (size_t)b * 17;
         const float scale = mx_scale(blk[0]);
         const u32x4 q = ld16_a1(blk + 1);
-        float wv[32];
+        bf16x2 wp[16];   // wp[4w + i] = (element 4w + i, element 4w + i + 16)
 #pragma unroll
         for (int w = 0; w < 4; w++) {
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                f32x2 pr;
-                switch (i) {
-                case 0: pr = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(q[w], scale, 0); break;
-                case 1: pr = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(q[w], scale, 1); break;
-                case 2: pr = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(q[w], scale, 2); break;
-                default: pr = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(q[w], scale, 3); break;
-                }
-                wv[4 * w + i] = pr.x;
-                wv[4 * w + i + 16] = pr.y;
-            }
+            wp[4 * w + 0] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(q[w], scale, 0);
+            wp[4 * w + 1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(q[w], scale, 1);
+            wp[4 * w + 2] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(q[w], scale, 2);
+            wp[4 * w + 3] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(q[w], scale, 3);
         }
 #pragma unroll
         for (int t = 0; t < 8; t++) {
             if (t < p.ntok) {
-                const uint16_t* xt = p.x + (size_t)t * p.k + (size_t)b * 32;
-                float s = 0.f;
+                const u32x4* xt = (const u32x4*)(p.x + (size_t)t * p.k + (size_t)b * 32);
+                u32 X[16];   // X[j] = (element 2j, element 2j + 1)
 #pragma unroll
                 for (int c = 0; c < 4; c++) {
-                    u32x4 v = ((const u32x4*)xt)[c];
+                    const u32x4 v = xt[c];
+                    X[4 * c] = v.x; X[4 * c + 1] = v.y; X[4 * c + 2] = v.z; X[4 * c + 3] = v.w;
+                }
+                float s = 0.f;
 #pragma unroll
-                    for (int d = 0; d < 4; d++) {
-                        s = fmaf(wv[8 * c + 2 * d], __uint_as_float(v[d] << 16), s);
-                        s = fmaf(wv[8 * c + 2 * d + 1], __uint_as_float(v[d] & 0xFFFF0000u), s);
-                    }
+                for (int e = 0; e < 16; e++) {
+                    // (x[e], x[e + 16]): the same half of words e/2 and e/2 + 8
+                    const u32 xp = __builtin_amdgcn_perm(X[e / 2 + 8], X[e / 2], (e & 1) ? 0x07060302u : 0x05040100u);
+                    s = __builtin_amdgcn_fdot2_f32_bf16(wp[e], __builtin_bit_cast(bf16x2, xp), s, false);
                 }
                 acc[t] += s;
             }
@@ -290,6 +288,67 @@ __device__ __forceinline__ void mx_matvec_body(const MxGemmArgs& p) {
             float v = wave_sum_to_lane63(acc[t]);
             if (lane == 63) p.out[(size_t)t * p.nrows + row] = v;
         }
+    }
+}
+
+// One token: the activation is the same for every row, so a lane keeps its blocks' activation
+// pairs in registers (already in the conversions' pair order) and the wavefront walks RPW rows
+// with them: the activation is read and permuted once per wavefront instead of once per row, and
+// all the rows' weight loads go out before the first row is decoded.
+// NBI = blocks a lane holds (lane l: blocks l, l + 64, ...: k <= 2048 * NBI).
+// grid = ceil(nrows / (nwaves * RPW)), block = 64 * nwaves
+#define JL_MX1_RPW 4
+template <int NBI>
+__device__ __forceinline__ void mx_matvec1_body(const MxGemmArgs& p) {
+    constexpr int RPW = JL_MX1_RPW;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+    const int row0 = (blockIdx.x * nwaves + wave) * RPW;
+    if (row0 >= p.nrows) return;
+    const int nblk = p.k / 32;
+    u32x4 q[RPW][NBI];
+    uint8_t e[RPW][NBI];
+#pragma unroll
+    for (int r = 0; r < RPW; r++) {
+        const uint8_t* wrow = p.w + (size_t)min(row0 + r, p.nrows - 1) * p.row_bytes;
+#pragma unroll
+        for (int u = 0; u < NBI; u++) {
+            const uint8_t* blk = wrow + (size_t)min(lane + 64 * u, nblk - 1) * 17;
+            e[r][u] = blk[0];
+            q[r][u] = ld16_a1(blk + 1);
+        }
+    }
+    bf16x2 xp[NBI][16];   // xp[u][e] = (x[32b + e], x[32b + e + 16]) of block b = lane + 64u
+#pragma unroll
+    for (int u = 0; u < NBI; u++) {
+        const int b = lane + 64 * u;
+        const u32x4* xt = (const u32x4*)(p.x + (size_t)min(b, nblk - 1) * 32);
+        u32 X[16];
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const u32x4 v = b < nblk ? xt[c] : u32x4{0u, 0u, 0u, 0u};   // a block past the row's end adds nothing
+            X[4 * c] = v.x; X[4 * c + 1] = v.y; X[4 * c + 2] = v.z; X[4 * c + 3] = v.w;
+        }
+#pragma unroll
+        for (int i = 0; i < 16; i++)
+            xp[u][i] = __builtin_bit_cast(bf16x2, __builtin_amdgcn_perm(X[i / 2 + 8], X[i / 2],
+                                                                         (i & 1) ? 0x07060302u : 0x05040100u));
+    }
+#pragma unroll
+    for (int r = 0; r < RPW; r++) {
+        float s = 0.f;
+#pragma unroll
+        for (int u = 0; u < NBI; u++) {
+            const float scale = mx_scale(e[r][u]);
+#pragma unroll
+            for (int w = 0; w < 4; w++) {
+                s = __builtin_amdgcn_fdot2_f32_bf16(__builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(q[r][u][w], scale, 0), xp[u][4 * w + 0], s, false);
+                s = __builtin_amdgcn_fdot2_f32_bf16(__builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(q[r][u][w], scale, 1), xp[u][4 * w + 1], s, false);
+                s = __builtin_amdgcn_fdot2_f32_bf16(__builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(q[r][u][w], scale, 2), xp[u][4 * w + 2], s, false);
+                s = __builtin_amdgcn_fdot2_f32_bf16(__builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(q[r][u][w], scale, 3), xp[u][4 * w + 3], s, false);
+            }
+        }
+        const float v = wave_sum_to_lane63(s);
+        if (lane == 63 && row0 + r < p.nrows) p.out[row0 + r] = v;
     }
 }
 

@@ -22,7 +22,7 @@ def to_bf16(x):
 
 @pytest.mark.parametrize("shape", [(1, 2880, 2880), (3, 100, 512), (8, 130, 96), (64, 2880, 2880),
                                    (130, 200, 224), (1024, 2880, 2880), (9, 129, 2880), (17, 33, 160),
-                                   (48, 16, 2880), (33, 300, 64)],
+                                   (48, 16, 2880), (33, 300, 64), (1, 100, 512), (1, 131, 4192), (1, 37, 8192)],
                          ids=lambda s: "x".join(map(str, s)))
 @pytest.mark.parametrize("weights", ["normal", "planted"])
 @pytest.mark.parametrize("rows", [0, 96, 128], ids=["auto", "tile96", "tile128"])
@@ -30,7 +30,8 @@ def test_mxfp4_bf16_matmul_vs_dequant_f32(dev, devbuf, shape, weights, rows):
     """rows = rows per workgroup tile of the tiled GEMM (the library picks per shape; both are
     held to the bar); auto also takes 9..64 tokens to the few-token kernel (16-row
     workgroups, K split over wavefronts; a last group of fewer than four blocks and ragged
-    rows are among the shapes)."""
+    rows are among the shapes) and one token to the kernel that keeps the activation in
+    registers (one, two and three blocks a lane; k = 8192 is past it and runs the general one)."""
     ntok, nrows, k = shape
     dev.set_tuning(mxfp4__rows=rows)
     if weights == "planted" and ntok * nrows * k > 3e8:
