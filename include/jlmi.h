@@ -86,15 +86,24 @@ int jl_set_act_window(jl_ctx *ctx, int window);
 void *jl_stream(jl_ctx *ctx);
 int jl_synchronize(jl_ctx *ctx);
 
-/* Kernel-shape overrides for measurement: key is one of "matvec.rpw" (rows per
- * wavefront: 1, 2, 4), "matvec.block" (threads per workgroup), "matvec.grid"
- * (workgroups), "matvec.pipe" (1: the row loop as a two-deep load pipeline), "gemm.min_tok" (fewest tokens sent to the matrix-core GEMM),
- * "packed.rw" (rows per wavefront of the packed-plane matvec: 16, 32, 64),
- * "packed.block" (its threads per workgroup), "moe.shares" (row shares an expert's
- * matrix is split into), "gemm.rows" (rows per workgroup of the GEMM: 64 or 128), "mxfp4.split" (workgroups along
- * K of the MXFP4 matmul);
- * value 0 restores the built-in choice.  Mirrors the reference's per-instance tuning knobs
- * (engine/nn/options.go:67-118). */
+/* Kernel-shape overrides for measurement and the parity tests: key is one of "matvec.rpw"
+ * (rows per wavefront: 1, 2, 4), "matvec.block" (threads per workgroup), "matvec.grid"
+ * (workgroups), "matvec.pipe" (1: the row loop as a two-deep load pipeline), "gemm.min_tok"
+ * (fewest tokens sent to the matrix-core GEMM), "gemm.form" (1: 128 x 64 tiles, 2: 256 x 128
+ * tiles, 3: two-pass, 4 / 5: the few-token forms, 9: token by token), "gemm.rows" (64 or 128),
+ * "gemm.split" (K slices), "gemm.prep" (4: the four-wavefront activation prep), "gemm.planes"
+ * (2: restore rows from planes before the GEMM), "packed.rw" (rows per wavefront of the
+ * packed-plane matvec: 16, 32, 64), "packed.block" (its threads per workgroup), "moe.shares"
+ * (row shares an expert's matrix is split into), "moe.form" / "moe.group" / "moe.logits" /
+ * "moe.q6k_cols" / "moe.waves" / "moe.lpr" (forms of the mixture block's kernels),
+ * "mxfp4.split" (K slices of the MXFP4 GEMM), "mxfp4.rows" (96 or 128 rows a tile; 1: the
+ * general decode matvec also for one token), "mxfp4.planes" (packed MXFP4: 2 restores rows
+ * first, 3 the plane GEMM whatever the grid, 64 / 32 / 16 rows a workgroup of the plane
+ * matvec); value 0 restores the built-in choice.  These change launch shapes and f32 summation
+ * order only.  One key changes values: "mxfp4.scaled" = 1 runs jl_matmul_mxfp4_packed_bf16_dev
+ * on the block-scaled fp8 x fp4 matrix instruction, which quantizes the activations to MX fp8
+ * (rel-L2 about 2.7e-2 against the bf16 activations); it is off unless set.  Mirrors the
+ * reference's per-instance tuning knobs (engine/nn/options.go:67-118). */
 int jl_set_tuning(jl_ctx *ctx, const char *key, int value);
 
 /* Kernels this context has launched so far: how callers and tests check that a grouped
