@@ -449,6 +449,11 @@ __device__ __forceinline__ void gemm_q4k_body(const GemmArgs& p, uint8_t* smem, 
                 if (ks == 0 && nhalf == 1) aaug = a_frag(nstep, 8);
             }
             if (has_next && (ks & 1)) gemm_w_word(wcur, wsc, ks >> 1);
+            // a matrix instruction, vector work under it, the second (two in a row would park
+            // the vector work behind the second for its whole length)
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
             __builtin_amdgcn_sched_barrier(0);
         }
         if (has_next && nhalf == 1) {
