@@ -890,7 +890,7 @@ __device__ __forceinline__ void moe_logits_body(const MoeLogitsArgs& p, float* p
 #pragma unroll
         for (int t = 0; t < JL_LOGITS_TOK; t++) acc[e][t] = 0.f;
     // unrolled so that the loads of several trips are in flight together; the sums stay in order
-#pragma unroll EB == 1 ? 8 : 2
+#pragma unroll EB == 1 ? 16 : 2
     for (int i0 = 0; i0 < k; i0 += 128) {
         const int i = i0 + tid, ic = min(i, k - 1);
         float w[EB], xv[JL_LOGITS_TOK];
