@@ -94,8 +94,11 @@ int jl_synchronize(jl_ctx *ctx);
  * "gemm.split" (K slices), "gemm.prep" (4: the four-wavefront activation prep), "gemm.planes"
  * (2: restore rows from planes before the GEMM), "packed.rw" (rows per wavefront of the
  * packed-plane matvec: 16, 32, 64), "packed.block" (its threads per workgroup), "moe.shares"
- * (row shares an expert's matrix is split into), "moe.form" / "moe.group" / "moe.logits" /
- * "moe.q6k_cols" / "moe.waves" / "moe.lpr" (forms of the mixture block's kernels),
+ * (row shares an expert's matrix is split into), "moe.form" (grouped matmul: 1 dot products,
+ * 2 / 3 groups of 32 / 16 columns on the matrix cores, 4 the prefill tile per expert),
+ * "moe.group16" (form 3: 1 a prep kernel quantizes the columns, 2 the matrix kernel does),
+ * "moe.group" / "moe.logits" / "moe.q6k_cols" / "moe.waves" / "moe.lpr" (forms of the mixture
+ * block's other kernels),
  * "mxfp4.split" (K slices of the MXFP4 GEMM), "mxfp4.rows" (96 or 128 rows a tile; 1: the
  * general decode matvec also for one token), "mxfp4.planes" (packed MXFP4: 2 restores rows
  * first, 3 the plane GEMM whatever the grid, 64 / 32 / 16 rows a workgroup of the plane

@@ -120,6 +120,34 @@ struct MoeGemmArgs {
     int row_step = 0, pstride = 0;
 };
 
+// Grouped expert matmul, sixteen columns a group (moe_g16_body).  Column group g of expert e is
+// slot (start[e] >> 4) + e + g of the prepared workspace; a slot holds, for every super-block,
+// JL_MOE_G16_SB_WORDS words: eight matrix fragments of 64 lanes x 16 bytes (half, K-step), the
+// sub-block sums' fragment (32 lanes x 16 bytes) and the sixteen columns' scales.
+#define JL_MOE_G16_SB_WORDS 2192
+struct MoeG16PrepArgs {
+    const float* x;
+    const float* x2;        // null: plain activation
+    const uint32_t* src;    // null: column c reads row c
+    const uint32_t* start;  // [n_expert + 1]
+    uint32_t* ws;
+    int k, n_expert;
+};
+struct MoeG16Args {
+    float* out[2];
+    const uint8_t* bank[2];
+    const uint32_t* ws;
+    const uint32_t* start;
+    size_t sheet_bytes;
+    int nrows, k, row_bytes;
+    int tiles_wg;           // tiles of sixteen rows a workgroup owns
+    int blocks, nmat, n_expert, nwaves;   // row blocks an (expert, matrix); wavefronts a workgroup
+    // fused form: the columns are quantized by the matrix kernel itself (ws unused)
+    const float* x = nullptr;
+    const float* x2 = nullptr;
+    const uint32_t* src = nullptr;
+};
+
 // Two-pass form of the Q4_K prefill GEMM.  Pass one expands the weights once per call into
 // f16 matrix fragments, w16 [ceil(nrows/64)][k/128 stages][18 fragments][64 lanes] 16-byte
 // vectors (fragment 2*ks+g: K-step ks of the tile's row group g; 16+g: the minimum columns,

@@ -839,6 +839,306 @@ __device__ __forceinline__ void moe_gemm_q4k_body(const MoeGemmArgs& p, uint8_t*
     }
 }
 
+// ------------------------------------ grouped matmul, sixteen columns a group, no weight staging
+// A handful of columns an expert (a small prefill batch through a wide mixture) is too few for
+// the 32-column tile above and too many for the dot-product kernel, which pays every (weight,
+// column) pair in vector instructions.  Here a group is up to sixteen columns and the matrix
+// instruction is the 16 x 16 x 32 one: tokens are its M, sixteen weight rows its N, and a lane
+// (row j = lane % 16, kg = lane / 16) supplies eight K values a step.  The K order of a step is
+// free as long as both operands agree, so it is chosen to be what the lane's own 32-byte load
+// of nibbles decodes to: lane (j, kg) loads group kg of the super-block of row j (32 bytes: low
+// nibbles sub-block 2 kg, high nibbles sub-block 2 kg + 1), and word ks of it, unpacked as in
+// the prefill GEMM (b0.lo, b2.lo, b0.hi, b2.hi, b1.lo, b3.lo, b1.hi, b3.hi),
+// IS the lane's operand of K-step ks.  Weights therefore go HBM -> registers -> matrix core:
+// no LDS staging, no barrier in the loop.  The prep kernel writes the columns in the matching
+// order.  The group's activation fragments for the whole of K sit in LDS (JL_MOE_G16_SB_WORDS
+// words a super-block), filled once per (workgroup, group); columns the group does not have are
+// filled with zeros, so the workspace needs none.
+//
+// Prep: grid = (ceil(k/1024), ncols), block = 256: a wavefront quantizes one super-block of one
+// column (lane l owns elements 4l..4l+3), finds the column's expert by counting the experts
+// whose first column is not after it, and writes the 32 sixteen-byte pieces of the column's
+// fragments, the two pieces of its sub-block sums (low six bits, the rest) and its scale.
+__device__ __forceinline__ void moe_g16_prep_body(const MoeG16PrepArgs& p, u32* lds) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const u32 c = blockIdx.y;
+    const int nsb = p.k / 256, sb = blockIdx.x * 4 + wave;
+    if (sb >= nsb) return;   // whole wavefronts; no workgroup barrier below
+    const size_t row = p.src ? p.src[c] : c;
+    f32x4 v = ((const f32x4*)(p.x + row * (size_t)p.k + (size_t)sb * 256))[lane];
+    f32x4 u = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (p.x2) u = ((const f32x4*)(p.x2 + row * (size_t)p.k + (size_t)sb * 256))[lane];
+    u32 cnt = 0;
+    for (int base = 0; base <= p.n_expert; base += 64) {
+        const int idx = base + lane;
+        const u32 s = idx <= p.n_expert ? p.start[idx] : 0xFFFFFFFFu;
+        cnt += (u32)__builtin_popcountll(__ballot(s <= c));
+    }
+    const int e = (int)cnt - 1;
+    const u32 c_lo = p.start[e];
+    const u32 rel = c - c_lo;
+    const size_t slot = (size_t)(c_lo >> 4) + (size_t)e + (rel >> 4);
+    const int i = (int)(rel & 15);
+    if (p.x2) v = f32x4{silu_f32(v.x) * u.x, silu_f32(v.y) * u.y, silu_f32(v.z) * u.z, silu_f32(v.w) * u.w};
+    const u32 m = max(max(abs_bits(v.x), abs_bits(v.y)), max(abs_bits(v.z), abs_bits(v.w)));
+    const u32 amax = wave_amax_256(m);
+    float d;
+    i32 sum16;
+    const u32 q = quantize4(v, amax, d, sum16);
+    const i32 a32 = sum16 + dpp_i32<JL_DPP_ROW_HALF_MIRROR, 0xf>(0, sum16);
+    u32* sq = lds + wave * 72;   // the wavefront's own: 64 words of int8, 8 sub-block sums
+    sq[lane] = q;
+    if ((lane & 7) == 0) sq[64 + (lane >> 3)] = (u32)a32;
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // LDS operations of a wavefront execute in order
+    u32* blk = p.ws + (slot * nsb + sb) * JL_MOE_G16_SB_WORDS;
+    if (lane < 32) {
+        const int ks = lane >> 2, kg = lane & 3;
+        const u32 lo = sq[16 * kg + ks], hi = sq[16 * kg + 8 + ks];
+        auto f = [](u32 w, int b) { return (_Float16)(float)(int8_t)(w >> (8 * b)); };
+        const f16x8 o = {f(lo, 0), f(lo, 2), f(hi, 0), f(hi, 2), f(lo, 1), f(lo, 3), f(hi, 1), f(hi, 3)};
+        ((u32x4*)blk)[ks * 64 + 16 * kg + i] = __builtin_bit_cast(u32x4, o);
+    } else if (lane < 34) {
+        const int kg = lane - 32;
+        f16x8 o;
+#pragma unroll
+        for (int s8 = 0; s8 < 8; s8++) {
+            const i32 a = (i32)sq[64 + s8];
+            o[s8] = (_Float16)(float)(kg ? (a >> 6) : (a & 63));
+        }
+        ((u32x4*)blk)[512 + 16 * kg + i] = __builtin_bit_cast(u32x4, o);
+    } else if (lane == 34) {
+        blk[2176 + i] = __float_as_uint(d);
+    }
+}
+
+// One 32-bit word of nibbles as a matrix operand: the prefill GEMM's unpack, kept in registers.
+__device__ __forceinline__ f16x8 moe_g16_word(u32 w, const GemmWideScale& k, u32 mask_lo, u32 mask_hi, u32 magic) {
+    const u32 w8 = w >> 8;
+    auto nib = [&](u32 v, u32 mask) { return __builtin_bit_cast(f16x2, (v & mask) | magic); };
+    const f16x2 p0 = __builtin_elementwise_fma(nib(w, mask_lo), k.mlo, k.alo);
+    const f16x2 p1 = __builtin_elementwise_fma(nib(w, mask_hi), k.mhi, k.ahi);
+    const f16x2 p2 = __builtin_elementwise_fma(nib(w8, mask_lo), k.mlo, k.alo);
+    const f16x2 p3 = __builtin_elementwise_fma(nib(w8, mask_hi), k.mhi, k.ahi);
+    const u32x4 o = {__builtin_bit_cast(u32, p0), __builtin_bit_cast(u32, p1), __builtin_bit_cast(u32, p2),
+                     __builtin_bit_cast(u32, p3)};
+    return __builtin_bit_cast(f16x8, o);
+}
+
+// Matrix kernel: grid = 8 * ceil(n_expert / 8) * blocks * matrices (one dimension), block =
+// 64 * nwaves, dynamic LDS = (k/256) * JL_MOE_G16_SB_WORDS * 4.  Workgroups go round the eight
+// XCDs in the order of their ids, so id % 8 names the XCD: expert e is worked on by XCD e % 8
+// alone, its (matrix, row block) workgroups one after the other there, and the group's fragments
+// are fetched into one L2 once.  A workgroup owns tiles_wg tiles of sixteen rows of the
+// expert's sheet and walks the expert's column groups; wavefront w takes tiles w, w + nwaves, ...
+// one after the other.  A step is (tile, chunk of CH super-blocks): CH * 144 contiguous bytes of
+// each of the tile's rows, requested in one go a whole step ahead (two register sets), so a
+// cache line is used up by the step that fetched it and only the line at a chunk's border is
+// touched twice.  Per super-block: eight K-steps, then the epilogue into the tile's four sums.
+// FUSED: no prep kernel and no workspace -- the workgroup quantizes its group's columns itself
+// (a wavefront per (column, super-block), the prep kernel's arithmetic) straight into the LDS
+// fragments, behind the first weight loads.  Every workgroup of the expert repeats that, which
+// pays while an expert has a handful of columns: two launches less a call.
+template <int CH, bool FUSED>
+__device__ __forceinline__ void moe_g16_body(const MoeG16Args& p, uint8_t* smem) {
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    JL_MOE_TRACE(0);
+    const int nwaves = p.nwaves, nthreads = 64 * nwaves;
+    const int per_e = p.blocks * p.nmat;
+    const int xcd = blockIdx.x & 7, q = blockIdx.x >> 3;
+    const int e = xcd + 8 * (q / per_e), sub = q % per_e;
+    if (e >= p.n_expert) return;
+    const int mat = sub / p.blocks, blk = sub % p.blocks;
+    const u32 c_lo = p.start[e], c_hi = p.start[e + 1];
+    if (c_lo == c_hi) return;   // nobody chose this expert (uniform across the workgroup)
+    const int nsb = p.k / 256, nch = (nsb + CH - 1) / CH;
+    const int tiles = (p.nrows + 15) >> 4;
+    const int tile0 = blk * p.tiles_wg + wave;
+    const int tile_end = min(tiles, (blk + 1) * p.tiles_wg);
+    const int ntl = tile0 < tile_end ? (tile_end - tile0 + nwaves - 1) / nwaves : 0;   // this wavefront's tiles (uniform)
+    const int nsteps = ntl * nch;
+    const int j = lane & 15, kg = lane >> 4;
+    const uint8_t* sheet = p.bank[mat] + (size_t)e * p.sheet_bytes;
+    u32 mask_lo = 0x000F000Fu, mask_hi = 0x00F000F0u, magic = 0x64006400u;
+    asm volatile("" : "+v"(mask_lo), "+v"(mask_hi), "+v"(magic));
+    u32x4* sA4 = (u32x4*)smem;
+    const float* sAf = (const float*)smem;
+    float* outm = p.out[mat];
+    constexpr int V = JL_MOE_G16_SB_WORDS / 4;   // 548 vectors a super-block
+
+    u32x4 hd[2][CH], wq[2][CH][2];
+    // step (tile number tn of this wavefront, chunk ch) into a register set
+    auto load_step = [&](int tn, int ch, u32x4 (&h)[CH], u32x4 (&q)[CH][2]) {
+        const int row = min(16 * (tile0 + nwaves * tn) + j, p.nrows - 1);
+        const uint8_t* b = sheet + (size_t)row * p.row_bytes;
+#pragma unroll
+        for (int s = 0; s < CH; s++) {
+            const uint8_t* bs = b + (size_t)min(ch * CH + s, nsb - 1) * 144;
+            h[s] = ld16(bs);
+            q[s][0] = ld16(bs + 16 + 32 * kg);
+            q[s][1] = ld16(bs + 32 + 32 * kg);
+        }
+    };
+
+    for (u32 c0 = c_lo; c0 < c_hi; c0 += 16) {
+        const int ncg = min(16, (int)(c_hi - c0));
+        const size_t slot = (size_t)(c_lo >> 4) + (size_t)e + ((c0 - c_lo) >> 4);
+        // FUSED: the group's source rows, one a lane, and the first eight (column, super-block)
+        // tasks of this wavefront requested ahead of the weights, which have the longer way and
+        // would hold them up (a wavefront's loads return in order)
+        constexpr int TB = 8;
+        const int ntask = ncg * nsb;
+        u32 rowv = 0;
+        f32x4 xv[TB], xu[TB];
+        auto issue = [&](int t0) {
+#pragma unroll
+            for (int b = 0; b < TB; b++) {
+                xu[b] = f32x4{0.f, 0.f, 0.f, 0.f};
+                const int task = min(t0 + b * nwaves, ntask - 1);
+                const int i = task / nsb, sb = task - i * nsb;
+                const size_t row = (size_t)__shfl(rowv, i, 64);
+                xv[b] = ((const f32x4*)(p.x + row * (size_t)p.k + (size_t)sb * 256))[lane];
+                if (p.x2) xu[b] = ((const f32x4*)(p.x2 + row * (size_t)p.k + (size_t)sb * 256))[lane];
+            }
+        };
+        if (FUSED) {
+            if (lane < ncg) rowv = p.src ? p.src[c0 + lane] : c0 + (u32)lane;
+            issue(wave);
+        }
+        if (nsteps > 0) load_step(0, 0, hd[0], wq[0]);
+        if (c0 != c_lo) __syncthreads();   // the previous group's fragments have been read
+        if (FUSED) {
+            // zeros where the group has no column (fragments and sums; the scales are not read there)
+            const int total = nsb * V;
+            for (int idx = tid; idx < total; idx += nthreads) {
+                const int o = idx % V;
+                if (o < 544 && (o & 15) >= ncg) sA4[idx] = u32x4{0u, 0u, 0u, 0u};
+            }
+            u32* sAw = (u32*)smem;
+            _Float16* sAh = (_Float16*)smem;
+            float* sAfw = (float*)smem;
+            for (int t0 = wave; t0 < ntask; t0 += TB * nwaves) {
+                if (t0 != wave) issue(t0);
+#pragma unroll
+                for (int b = 0; b < TB; b++) {
+                    const int task = t0 + b * nwaves;
+                    if (task < ntask) {   // uniform
+                        const int i = task / nsb, sb = task - i * nsb;
+                        f32x4 w = xv[b];
+                        if (p.x2) w = f32x4{silu_f32(w.x) * xu[b].x, silu_f32(w.y) * xu[b].y, silu_f32(w.z) * xu[b].z, silu_f32(w.w) * xu[b].w};
+                        const u32 m = max(max(abs_bits(w.x), abs_bits(w.y)), max(abs_bits(w.z), abs_bits(w.w)));
+                        const u32 amax = wave_amax_256(m);
+                        float d;
+                        i32 sum16;
+                        const u32 q = quantize4(w, amax, d, sum16);
+                        const i32 a32 = sum16 + dpp_i32<JL_DPP_ROW_HALF_MIRROR, 0xf>(0, sum16);
+                        // lane l holds word l of the super-block: sub-block l / 8 (group kg, low or
+                        // high nibbles' partner), K-step l % 8; its bytes go to two f16 pairs
+                        const int sub = lane >> 3, ks = lane & 7, kg = sub >> 1, hi = sub & 1;
+                        auto f = [](u32 x, int b2) { return (_Float16)(float)(int8_t)(x >> (8 * b2)); };
+                        const f16x2 p02 = {f(q, 0), f(q, 2)}, p13 = {f(q, 1), f(q, 3)};
+                        const int vec = sb * V + ks * 64 + 16 * kg + i;
+                        sAw[vec * 4 + hi] = __builtin_bit_cast(u32, p02);
+                        sAw[vec * 4 + 2 + hi] = __builtin_bit_cast(u32, p13);
+                        if ((lane & 7) == 0) {
+                            sAh[(sb * V + 512 + i) * 8 + sub] = (_Float16)(float)(a32 & 63);
+                            sAh[(sb * V + 512 + 16 + i) * 8 + sub] = (_Float16)(float)(a32 >> 6);
+                        }
+                        if (lane == 0) sAfw[sb * JL_MOE_G16_SB_WORDS + 2176 + i] = d;
+                    }
+                }
+            }
+        } else {
+            const u32x4* src = (const u32x4*)(p.ws + slot * nsb * JL_MOE_G16_SB_WORDS);
+            // up to eighteen loads in flight a thread (all of K = 2048 at 256 threads): the fill is
+            // one round trip to L2, not one a vector
+            constexpr int NB = 18;
+            const int total = nsb * V;
+            for (int base = tid; base < total; base += NB * nthreads) {
+                u32x4 val[NB];
+#pragma unroll
+                for (int u = 0; u < NB; u++) {
+                    const int idx = base + u * nthreads, o = idx % V;
+                    // fragments: lane = o % 64, its column o % 16; sums: (o - 512) % 16; scales: all
+                    const bool have = idx < total && (o >= 544 || (o & 15) < ncg);
+                    val[u] = u32x4{0u, 0u, 0u, 0u};
+                    if (have) val[u] = src[idx];
+                }
+#pragma unroll
+                for (int u = 0; u < NB; u++) {
+                    const int idx = base + u * nthreads;
+                    if (idx < total) sA4[idx] = val[u];
+                }
+            }
+        }
+        __syncthreads();
+        JL_MOE_TRACE(1);
+        f32x4 out = {0.f, 0.f, 0.f, 0.f};
+        int tn = 0, ch = 0;   // this step's tile and chunk
+        auto step = [&](auto PAR) {
+            constexpr int cur = decltype(PAR)::value;
+            const bool last_ch = ch == nch - 1;
+            const int tn_n = last_ch ? tn + 1 : tn, ch_n = last_ch ? 0 : ch + 1;
+            load_step(min(tn_n, ntl - 1), ch_n, hd[cur ^ 1], wq[cur ^ 1]);
+#pragma unroll
+            for (int s = 0; s < CH; s++) {
+                const int sb = ch * CH + s;
+                if (sb < nsb) {   // uniform
+                    f32x4 accP;
+                    GemmWideScale sc;
+                    gemm_wide_scale(hd[cur][s], kg & 1, kg >> 1, sc);
+#pragma unroll
+                    for (int ks = 0; ks < 8; ks++) {
+                        const f16x8 af = __builtin_bit_cast(f16x8, sA4[sb * V + ks * 64 + lane]);
+                        const f16x8 b = moe_g16_word(wq[cur][s][ks >> 2][ks & 3], sc, mask_lo, mask_hi, magic);
+                        const f32x4 czero = {0.f, 0.f, 0.f, 0.f};
+                        accP = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, b, ks == 0 ? czero : accP, 0, 0, 0);
+                    }
+                    // out += d_a * (d * P - dmin * M) for the super-block
+                    u32x4 augw = u32x4{0u, 0u, 0u, 0u};
+                    if (lane < 32) augw = sA4[sb * V + 512 + lane];
+                    const f16x8 aug = __builtin_bit_cast(f16x8, augw);
+                    const f32x4 dav = *(const f32x4*)(sAf + sb * JL_MOE_G16_SB_WORDS + 2176 + 4 * kg);
+                    const float mul = kg == 0 ? 1.0f : (kg == 1 ? 64.0f : 0.0f);
+                    const GemmScaleBytes sbytes = gemm_scale_bytes(hd[cur][s].y, hd[cur][s].z, hd[cur][s].w);
+                    f16x8 mm;
+#pragma unroll
+                    for (int b = 0; b < 4; b++) {
+                        mm[b] = (_Float16)((float)((sbytes.mn_lo >> (8 * b)) & 0xFF) * mul);
+                        mm[4 + b] = (_Float16)((float)((sbytes.mn_hi >> (8 * b)) & 0xFF) * mul);
+                    }
+                    const f32x4 czero = {0.f, 0.f, 0.f, 0.f};
+                    const f32x4 accM = __builtin_amdgcn_mfma_f32_16x16x32_f16(aug, mm, czero, 0, 0, 0);
+                    const float dd = half_bits_to_f32((uint16_t)(hd[cur][s].x & 0xFFFF));
+                    const float dmin = half_bits_to_f32((uint16_t)(hd[cur][s].x >> 16));
+#pragma unroll
+                    for (int el = 0; el < 4; el++) {
+                        const float uu = fmaf(dd, accP[el], -(dmin * accM[el]));
+                        out[el] = fmaf(dav[el], uu, out[el]);
+                    }
+                }
+            }
+            if (last_ch) {   // the tile is done: store its 16 rows x ncg columns
+                const int r = 16 * (tile0 + nwaves * tn) + j;
+#pragma unroll
+                for (int el = 0; el < 4; el++) {
+                    const int tok = 4 * kg + el;
+                    if (r < p.nrows && tok < ncg) outm[(size_t)(c0 + tok) * p.nrows + r] = out[el];
+                    out[el] = 0.f;
+                }
+            }
+            tn = tn_n;
+            ch = ch_n;
+        };
+        for (int s = 0; s < nsteps; s += 2) {
+            step(GemmIntC<0>{});
+            if (s == 0) JL_MOE_TRACE(2);
+            if (s + 1 < nsteps) step(GemmIntC<1>{});   // uniform
+        }
+        JL_MOE_TRACE(3);
+    }
+}
+
 // resid[r][n] += sum over the row's k_used experts, ascending expert id, of
 // wt[r][s] * y[pos[r*k_used+s]][n].  grid = (ceil(n_embd/4/256), rows): a thread owns four
 // columns of a row.  The first k_used threads rank the row's slots by expert id and lay weights

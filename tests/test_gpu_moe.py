@@ -79,12 +79,15 @@ def _banks(t, n_expert, nrows, k, seed, planted):
                                             (quant.Q4_K, 300, 768, 2), (quant.Q4_K, 40, 4096, 2),
                                             (quant.Q4_K, 96, 2048, 4), (quant.Q4_K, 300, 768, 4),
                                             (quant.Q4_K, 40, 4096, 4), (quant.Q4_K, 129, 256, 4),
+                                            (quant.Q4_K, 96, 2048, 3), (quant.Q4_K, 300, 768, 3),
+                                            (quant.Q4_K, 40, 4096, 3), (quant.Q4_K, 129, 256, 3),
                                             (quant.Q8_0, 64, 1024, 0), (quant.Q6_K, 70, 1024, 0),
                                             (quant.Q6_K, 96, 2048, 4), (quant.Q6_K, 300, 768, 4),
                                             (quant.Q6_K, 129, 256, 4)])
 def test_grouped_matvec_vs_oracle(dev, devbuf, t, nrows, k, form):
     """form 1 = the dot-product kernel, 2 = groups of 32 columns on the matrix cores (Q4_K with
-    the k-quant window), 4 = the prefill GEMM's 128-column x 64-row tile placed per expert,
+    the k-quant window), 3 = groups of 16 columns, the weights decoded in registers into the
+    matrix operand, 4 = the prefill GEMM's 128-column x 64-row tile placed per expert,
     0 = what the library picks."""
     rows, n_expert, k_used, window = 13, 8, 3, 256 if t in quant.K_QUANTS else 32
     dev.SetActWindow(window)
@@ -110,13 +113,18 @@ def test_grouped_matvec_vs_oracle(dev, devbuf, t, nrows, k, form):
     dstart, dperm = devbuf(start), devbuf(perm[:used].copy())
     o0 = devbuf(shape=(used, nrows), dtype=np.float32, fill=np.float32(4e30))
     o1 = devbuf(shape=(used, nrows), dtype=np.float32, fill=np.float32(4e30))
-    for lpr in (0, 4, 16, 32, 64):     # lanes per row: the library's pick, then every other width
-        dev.set_tuning(moe__lpr=lpr)
-        assert dev.moe_matvec_dev(o0.ptr, o1.ptr, t, b0.ptr, b1.ptr, xd.ptr, None, dperm.ptr, dstart.ptr,
-                                  n_expert, used, nrows, k)
-        dev.synchronize()
-        assert nmse(o0.get(), want0) <= 1e-10 and nmse(o1.get(), want1) <= 1e-10, lpr
-    dev.set_tuning(moe__lpr=0)
+    # form 1: lanes per row -- the library's pick, then every other width; form 3: the columns
+    # quantized by a prep kernel (1) or by the matrix kernel itself (2)
+    for key, values in (("moe__group16", (1, 2)),) if form == 3 else (("moe__lpr", (0, 4, 16, 32, 64)),):
+        for v in values:
+            dev.set_tuning(**{key: v})
+            o0.put(np.full((used, nrows), 4e30, np.float32))
+            o1.put(np.full((used, nrows), 4e30, np.float32))
+            assert dev.moe_matvec_dev(o0.ptr, o1.ptr, t, b0.ptr, b1.ptr, xd.ptr, None, dperm.ptr, dstart.ptr,
+                                      n_expert, used, nrows, k)
+            dev.synchronize()
+            assert nmse(o0.get(), want0) <= 1e-10 and nmse(o1.get(), want1) <= 1e-10, (key, v)
+        dev.set_tuning(**{key: 0})
     # SwiGLU form: column c reads silu(x[c]) * x2[c], no gather
     g = np.stack([synth.activations(k, seed=300 + c) for c in range(used)])
     u = np.stack([synth.activations(k, seed=400 + c) for c in range(used)])
@@ -158,8 +166,8 @@ def test_grouped_matmul_more_than_one_group_of_columns(dev, devbuf, rows, t):
         q, a_s, _ = oracle.quantize_act(x[perm[c]], window)
         want[c] = oracle.matvec_q8act_f64(t, bank[e * sheet:(e + 1) * sheet], q, a_s, nrows, k)
     b, xd, dstart, dperm = devbuf(bank), devbuf(x), devbuf(start), devbuf(perm[:used].copy())
-    for form in ((1, 2, 4) if t == quant.Q4_K else (1, 4, 0)):
-        dev.set_tuning(moe__form=form)
+    for form in ((1, 2, 3, 13, 4) if t == quant.Q4_K else (1, 4, 0)):   # 13: form 3, fused quantization
+        dev.set_tuning(moe__form=form % 10, moe__group16=2 if form == 13 else 1)
         o = devbuf(shape=(used * nrows + 8,), dtype=np.float32, fill=np.float32(4e30))
         assert dev.moe_matvec_dev(o.ptr, None, t, b.ptr, None, xd.ptr, None, dperm.ptr, dstart.ptr, n_expert, used,
                                   nrows, k)
@@ -167,7 +175,7 @@ def test_grouped_matmul_more_than_one_group_of_columns(dev, devbuf, rows, t):
         got = o.get()
         assert np.all(got[used * nrows:] == np.float32(4e30))
         assert nmse(got[:used * nrows].reshape(used, nrows), want) <= 1e-10, form
-    dev.set_tuning(moe__form=0)
+    dev.set_tuning(moe__form=0, moe__group16=0)
     dev.SetActWindow(32)
 
 
@@ -193,14 +201,14 @@ def test_grouped_matmul_more_experts_than_one_work_list_round(dev, devbuf):
         q, a_s, _ = oracle.quantize_act(x[perm[c]], window)
         want[c] = oracle.matvec_q8act_f64(t, bank[e * sheet:(e + 1) * sheet], q, a_s, nrows, k)
     b, xd, dstart, dperm = devbuf(bank), devbuf(x), devbuf(start), devbuf(perm[:used].copy())
-    for form in (1, 2, 4):
-        dev.set_tuning(moe__form=form)
+    for form in (1, 2, 3, 13, 4):
+        dev.set_tuning(moe__form=form % 10, moe__group16=2 if form == 13 else 1)
         o = devbuf(shape=(used, nrows), dtype=np.float32, fill=np.float32(4e30))
         assert dev.moe_matvec_dev(o.ptr, None, t, b.ptr, None, xd.ptr, None, dperm.ptr, dstart.ptr, n_expert, used,
                                   nrows, k)
         dev.synchronize()
         assert nmse(o.get(), want) <= 1e-10, form
-    dev.set_tuning(moe__form=0)
+    dev.set_tuning(moe__form=0, moe__group16=0)
     dev.SetActWindow(32)
 
 
@@ -269,11 +277,15 @@ def test_moe_block_vs_oracle(dev, devbuf, shape):
     resid = devbuf(shape=(rows, n_embd), dtype=np.float32, fill=0)
     for call in range(2):
         resid.put(np.zeros((rows, n_embd), np.float32))
+        before = dev.launch_count()
         assert dev.moe_ffn_dev(resid.ptr, t, gd.ptr, ud.ptr, dd.ptr, xd.ptr, sd.ptr, k_used + 1, wd.ptr,
                                rows, k_used, n_expert, n_ffn, n_embd)
         dev.synchronize()
         got = resid.get()
         assert rel_l2(got, want) <= 1e-3, f"call {call}: rel-L2 {rel_l2(got, want):.3e}"
+        # four columns an expert on average: grouping, two matrix-core launches that quantize
+        # their own columns, combine; the tiny case takes the dot-product form (two more launches)
+        assert dev.launch_count() - before == (4 if rows == 64 else 6)
     dev.SetActWindow(32)
 
 
