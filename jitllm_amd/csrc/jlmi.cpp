@@ -1007,7 +1007,7 @@ int moe_matvec_launch(jl_ctx* c, float* out0, float* out1, int type, const void*
     // fit a CU's LDS (K <= 2304); "moe.form" = 3 forces it wherever one fits.
     {
         const int nsb = k / 256;
-        const size_t lds16 = (size_t)nsb * JL_MOE_G16_SB_WORDS * 4;
+        const size_t lds16 = (size_t)nsb * JL_MOE_G16_SB_WORDS * 4 + 16;   // the fragments, the tile counter
         const size_t nslots16 = (size_t)ncols / 16 + (size_t)n_expert + 1;
         const bool can16 = !planes && type == JL_TYPE_Q4_K && c->act_window == 256 && lds16 <= c->lds_limit &&
                            (size_t)nrows * row_bytes < ((size_t)1 << 32);
@@ -1020,7 +1020,7 @@ int moe_matvec_launch(jl_ctx* c, float* out0, float* out1, int type, const void*
             MoeG16PrepArgs pa;
             pa.ws = nullptr;
             if (!fused) {
-                rc = ws_ensure(c, &c->moe_q_ws, &c->moe_q_ws_bytes, nslots16 * lds16);
+                rc = ws_ensure(c, &c->moe_q_ws, &c->moe_q_ws_bytes, nslots16 * nsb * JL_MOE_G16_SB_WORDS * 4);
                 if (rc != JL_OK) return rc;
                 pa.x = x; pa.x2 = x2; pa.src = src; pa.start = start; pa.ws = (uint32_t*)c->moe_q_ws;
                 pa.k = k; pa.n_expert = n_expert;
@@ -1034,18 +1034,21 @@ int moe_matvec_launch(jl_ctx* c, float* out0, float* out1, int type, const void*
             ga.ws = pa.ws; ga.start = start;
             if (fused) { ga.x = x; ga.x2 = x2; ga.src = src; }
             ga.sheet_bytes = sheet; ga.nrows = nrows; ga.k = k; ga.row_bytes = row_bytes;
-            // Two workgroups of four wavefronts a CU (the fragments of K = 2048 are 70 KB), so the grid
-            // runs in rounds of 2 * CUs workgroups; among the splits of the rows into blocks the one
-            // with the least rounds x tiles a wavefront, the fewest blocks among equals (every block
-            // fills LDS anew).  Experts that can have a column: at most one a column.
-            const int nmat = bank1 ? 2 : 1, tiles = (nrows + 15) / 16, nwaves = 4;
+            // One workgroup of eight wavefronts a CU (the same age on every SIMD, tiles handed out as
+            // they get to them: two younger workgroups of four measured 4 % slower), so the grid runs
+            // in rounds of CUs workgroups; among the splits of the rows into blocks the one with the
+            // least rounds x tiles a wavefront, the fewest blocks among equals (every block fills LDS
+            // anew).  Experts that can have a column: at most one a column.  "moe.waves" = 4: the
+            // two-workgroup form.
+            const int nmat = bank1 ? 2 : 1, tiles = (nrows + 15) / 16, nwaves = c->tune.moe_waves == 4 ? 4 : 8;
+            const long wgs_cu = nwaves == 4 ? 2 : 1;
             const int sets = (tiles + nwaves - 1) / nwaves;
             const long n_act = std::min<long>(n_expert, ncols);
             int best_blocks = 1;
             long best_cost = -1;
             for (int nb = 1; nb <= sets && nb <= 64; nb++) {
                 const long per_wave = (sets + nb - 1) / nb;
-                const long rounds = ((long)nb * n_act * nmat + 2L * c->num_cu - 1) / (2L * c->num_cu);
+                const long rounds = ((long)nb * n_act * nmat + wgs_cu * c->num_cu - 1) / (wgs_cu * c->num_cu);
                 const long cost = rounds * per_wave;
                 if (best_cost < 0 || cost < best_cost) { best_cost = cost; best_blocks = nb; }
             }

@@ -925,12 +925,12 @@ __device__ __forceinline__ f16x8 moe_g16_word(u32 w, const GemmWideScale& k, u32
 }
 
 // Matrix kernel: grid = 8 * ceil(n_expert / 8) * blocks * matrices (one dimension), block =
-// 64 * nwaves, dynamic LDS = (k/256) * JL_MOE_G16_SB_WORDS * 4.  Workgroups go round the eight
+// 64 * nwaves, dynamic LDS = (k/256) * JL_MOE_G16_SB_WORDS * 4 + 16.  Workgroups go round the eight
 // XCDs in the order of their ids, so id % 8 names the XCD: expert e is worked on by XCD e % 8
 // alone, its (matrix, row block) workgroups one after the other there, and the group's fragments
 // are fetched into one L2 once.  A workgroup owns tiles_wg tiles of sixteen rows of the
-// expert's sheet and walks the expert's column groups; wavefront w takes tiles w, w + nwaves, ...
-// one after the other.  A step is (tile, chunk of CH super-blocks): CH * 144 contiguous bytes of
+// expert's sheet and walks the expert's column groups; its wavefronts take the tiles one after
+// the other from a counter in LDS.  A step is (tile, chunk of CH super-blocks): CH * 144 contiguous bytes of
 // each of the tile's rows, requested in one go a whole step ahead (two register sets), so a
 // cache line is used up by the step that fetched it and only the line at a chunk's border is
 // touched twice.  Per super-block: eight K-steps, then the epilogue into the tile's four sums.
@@ -953,23 +953,22 @@ __device__ __forceinline__ void moe_g16_body(const MoeG16Args& p, uint8_t* smem)
     if (c_lo == c_hi) return;   // nobody chose this expert (uniform across the workgroup)
     const int nsb = p.k / 256, nch = (nsb + CH - 1) / CH;
     const int tiles = (p.nrows + 15) >> 4;
-    const int tile0 = blk * p.tiles_wg + wave;
-    const int tile_end = min(tiles, (blk + 1) * p.tiles_wg);
-    const int ntl = tile0 < tile_end ? (tile_end - tile0 + nwaves - 1) / nwaves : 0;   // this wavefront's tiles (uniform)
-    const int nsteps = ntl * nch;
+    const int tile_base = blk * p.tiles_wg;
+    const int ntw = min(tiles, tile_base + p.tiles_wg) - tile_base;   // tiles of this workgroup
     const int j = lane & 15, kg = lane >> 4;
     const uint8_t* sheet = p.bank[mat] + (size_t)e * p.sheet_bytes;
     u32 mask_lo = 0x000F000Fu, mask_hi = 0x00F000F0u, magic = 0x64006400u;
     asm volatile("" : "+v"(mask_lo), "+v"(mask_hi), "+v"(magic));
     u32x4* sA4 = (u32x4*)smem;
     const float* sAf = (const float*)smem;
+    u32* next_tile = (u32*)smem + (size_t)nsb * JL_MOE_G16_SB_WORDS;   // behind the fragments
     float* outm = p.out[mat];
     constexpr int V = JL_MOE_G16_SB_WORDS / 4;   // 548 vectors a super-block
 
     u32x4 hd[2][CH], wq[2][CH][2];
-    // step (tile number tn of this wavefront, chunk ch) into a register set
-    auto load_step = [&](int tn, int ch, u32x4 (&h)[CH], u32x4 (&q)[CH][2]) {
-        const int row = min(16 * (tile0 + nwaves * tn) + j, p.nrows - 1);
+    // step (tile ti of the workgroup's range, chunk ch) into a register set
+    auto load_step = [&](int ti, int ch, u32x4 (&h)[CH], u32x4 (&q)[CH][2]) {
+        const int row = min(16 * (tile_base + ti) + j, p.nrows - 1);
         const uint8_t* b = sheet + (size_t)row * p.row_bytes;
 #pragma unroll
         for (int s = 0; s < CH; s++) {
@@ -1005,8 +1004,9 @@ __device__ __forceinline__ void moe_g16_body(const MoeG16Args& p, uint8_t* smem)
             if (lane < ncg) rowv = p.src ? p.src[c0 + lane] : c0 + (u32)lane;
             issue(wave);
         }
-        if (nsteps > 0) load_step(0, 0, hd[0], wq[0]);
+        if (wave < ntw) load_step(wave, 0, hd[0], wq[0]);
         if (c0 != c_lo) __syncthreads();   // the previous group's fragments have been read
+        if (tid == 0) *next_tile = (u32)nwaves;   // tiles 0 .. nwaves - 1 are the wavefronts' first ones
         if (FUSED) {
             // zeros where the group has no column (fragments and sums; the scales are not read there)
             const int total = nsb * V;
@@ -1074,12 +1074,21 @@ __device__ __forceinline__ void moe_g16_body(const MoeG16Args& p, uint8_t* smem)
         __syncthreads();
         JL_MOE_TRACE(1);
         f32x4 out = {0.f, 0.f, 0.f, 0.f};
-        int tn = 0, ch = 0;   // this step's tile and chunk
+        // Tiles are handed out as the wavefronts get to them (a counter in LDS): the SIMD issues
+        // its oldest wavefront first, so with a fixed share each the young ones fall behind and
+        // run the last tenth of the kernel alone.  A wavefront knows its next tile a tile ahead.
+        auto take = [&]() {
+            u32 v = 0;
+            if (lane == 0) v = __hip_atomic_fetch_add(next_tile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            return (int)__builtin_amdgcn_readfirstlane(v);
+        };
+        int ti = wave, ch = 0;   // this step's tile and chunk
+        int ti_n = ti < ntw ? take() : ntw;
         auto step = [&](auto PAR) {
             constexpr int cur = decltype(PAR)::value;
             const bool last_ch = ch == nch - 1;
-            const int tn_n = last_ch ? tn + 1 : tn, ch_n = last_ch ? 0 : ch + 1;
-            load_step(min(tn_n, ntl - 1), ch_n, hd[cur ^ 1], wq[cur ^ 1]);
+            const int t_n = last_ch ? ti_n : ti, ch_n = last_ch ? 0 : ch + 1;
+            load_step(min(t_n, ntw - 1), ch_n, hd[cur ^ 1], wq[cur ^ 1]);
 #pragma unroll
             for (int s = 0; s < CH; s++) {
                 const int sb = ch * CH + s;
@@ -1119,7 +1128,7 @@ __device__ __forceinline__ void moe_g16_body(const MoeG16Args& p, uint8_t* smem)
                 }
             }
             if (last_ch) {   // the tile is done: store its 16 rows x ncg columns
-                const int r = 16 * (tile0 + nwaves * tn) + j;
+                const int r = 16 * (tile_base + ti) + j;
 #pragma unroll
                 for (int el = 0; el < 4; el++) {
                     const int tok = 4 * kg + el;
@@ -1127,13 +1136,18 @@ __device__ __forceinline__ void moe_g16_body(const MoeG16Args& p, uint8_t* smem)
                     out[el] = 0.f;
                 }
             }
-            tn = tn_n;
+            if (last_ch) {
+                ti = ti_n;
+                if (ti < ntw) ti_n = take();
+            }
             ch = ch_n;
         };
-        for (int s = 0; s < nsteps; s += 2) {
+        bool first = true;
+        while (ti < ntw) {   // uniform
             step(GemmIntC<0>{});
-            if (s == 0) JL_MOE_TRACE(2);
-            if (s + 1 < nsteps) step(GemmIntC<1>{});   // uniform
+            if (first) JL_MOE_TRACE(2);
+            first = false;
+            if (ti < ntw) step(GemmIntC<1>{});
         }
         JL_MOE_TRACE(3);
     }
