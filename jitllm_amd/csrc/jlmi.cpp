@@ -1007,7 +1007,7 @@ int moe_matvec_launch(jl_ctx* c, float* out0, float* out1, int type, const void*
     // fit a CU's LDS (K <= 2304); "moe.form" = 3 forces it wherever one fits.
     {
         const int nsb = k / 256;
-        const size_t lds16 = (size_t)nsb * JL_MOE_G16_SB_WORDS * 4 + 16;   // the fragments, the tile counter
+        const size_t lds16 = (size_t)nsb * JL_MOE_G16_LDS_WORDS * 4 + 16;   // the fragments, the tile counter
         const size_t nslots16 = (size_t)ncols / 16 + (size_t)n_expert + 1;
         const bool can16 = !planes && type == JL_TYPE_Q4_K && c->act_window == 256 && lds16 <= c->lds_limit &&
                            (size_t)nrows * row_bytes < ((size_t)1 << 32);
@@ -1040,7 +1040,7 @@ int moe_matvec_launch(jl_ctx* c, float* out0, float* out1, int type, const void*
             // least rounds x tiles a wavefront, the fewest blocks among equals (every block fills LDS
             // anew).  Experts that can have a column: at most one a column.  "moe.waves" = 4: the
             // two-workgroup form.
-            const int nmat = bank1 ? 2 : 1, tiles = (nrows + 15) / 16, nwaves = c->tune.moe_waves == 4 ? 4 : 8;
+            const int nmat = bank1 ? 2 : 1, tiles = (nrows + 15) / 16, nwaves = c->tune.moe_waves == 4 || c->tune.moe_waves == 12 ? c->tune.moe_waves : 8;
             const long wgs_cu = nwaves == 4 ? 2 : 1;
             const int sets = (tiles + nwaves - 1) / nwaves;
             const long n_act = std::min<long>(n_expert, ncols);
@@ -1053,15 +1053,16 @@ int moe_matvec_launch(jl_ctx* c, float* out0, float* out1, int type, const void*
                 if (best_cost < 0 || cost < best_cost) { best_cost = cost; best_blocks = nb; }
             }
             if (c->tune.moe_shares > 0) best_blocks = std::min(c->tune.moe_shares, sets);
-            ga.tiles_wg = nwaves * ((sets + best_blocks - 1) / best_blocks);
+            ga.tiles_wg = (tiles + best_blocks - 1) / best_blocks;   // handed out inside the workgroup as its wavefronts get to them
             ga.blocks = (tiles + ga.tiles_wg - 1) / ga.tiles_wg;
             ga.nmat = nmat; ga.n_expert = n_expert; ga.nwaves = nwaves;
             const long grid = 8L * ((n_expert + 7) / 8) * ga.blocks * nmat;
             if (grid >= (1L << 31)) return JL_DECLINED;
-            // super-blocks a step: four (576 contiguous bytes a row), or all of a short row
-            const int ch = nsb <= 4 ? nsb : (nsb % 4 == 0 ? 4 : (nsb % 3 == 0 ? 3 : 4));
+            // super-blocks a step: all of a short row, else two (288 contiguous bytes a row; four
+            // measured 10 % slower at K = 2048: twice the bytes in flight before the first step)
+            const int ch = nsb <= 3 ? nsb : 2;
             char name[32];
-            snprintf(name, sizeof name, "jl_moe_g16_%c%d", fused ? 'f' : 'c', ch);
+            snprintf(name, sizeof name, "jl_moe_g16_%c%d", fused ? (x2 ? 'g' : 'f') : 'c', ch);
             void* gp[] = {&ga};
             return launch(c, name, (unsigned)grid, 1, (unsigned)(64 * nwaves), (unsigned)lds16, st, gp);
         }
@@ -1244,7 +1245,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     if (e != hipSuccess)
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
-    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_prep_q4k_planes", "jl_gemm_q4k_r64_planes", "jl_gemm_q4k_wide_planes", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_group2_wide", "jl_moe_quant", "jl_moe_matvec_planes_q4k", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_prep_planes", "jl_moe_gemm_q4k", "jl_moe_g16_prep", "jl_moe_g16_c1", "jl_moe_g16_c2", "jl_moe_g16_c3", "jl_moe_g16_c4", "jl_moe_g16_f1", "jl_moe_g16_f2", "jl_moe_g16_f3", "jl_moe_g16_f4", "jl_moe_gemm_r64", "jl_moe_gemm_r64_planes", "jl_moe_gemm_q6k_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_mxfp4_matvec1_b1", "jl_mxfp4_matvec1_b2", "jl_mxfp4_matvec1_b3", "jl_mxfp4_scaled_prep", "jl_mxfp4_scaled_gemm", "jl_mxfp4_planes_prep", "jl_mxfp4_planes_gemm", "jl_mxfp4_matvec_planes_r64", "jl_mxfp4_matvec_planes_r32", "jl_mxfp4_matvec_planes_r16", "jl_unpack_mxfp4", "jl_sum_parts", "jl_probe_read", "jl_probe_empty", "jl_probe_wait", "jl_probe_mfma", "jl_probe_mfma_v5",
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_prep_q4k_planes", "jl_gemm_q4k_r64_planes", "jl_gemm_q4k_wide_planes", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_group2_wide", "jl_moe_quant", "jl_moe_matvec_planes_q4k", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_prep_planes", "jl_moe_gemm_q4k", "jl_moe_g16_prep", "jl_moe_g16_c1", "jl_moe_g16_c2", "jl_moe_g16_c3", "jl_moe_g16_f1", "jl_moe_g16_f2", "jl_moe_g16_f3", "jl_moe_g16_g1", "jl_moe_g16_g2", "jl_moe_g16_g3", "jl_moe_gemm_r64", "jl_moe_gemm_r64_planes", "jl_moe_gemm_q6k_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_mxfp4_matvec1_b1", "jl_mxfp4_matvec1_b2", "jl_mxfp4_matvec1_b3", "jl_mxfp4_scaled_prep", "jl_mxfp4_scaled_gemm", "jl_mxfp4_planes_prep", "jl_mxfp4_planes_gemm", "jl_mxfp4_matvec_planes_r64", "jl_mxfp4_matvec_planes_r32", "jl_mxfp4_matvec_planes_r16", "jl_unpack_mxfp4", "jl_sum_parts", "jl_probe_read", "jl_probe_empty", "jl_probe_wait", "jl_probe_mfma", "jl_probe_mfma_v5",
                                       "jl_pack_weights", "jl_unpack_q4k", "jl_unpack_q6k", "jl_unpack_q8_0"};
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int rw : {16, 32, 64})

@@ -125,6 +125,7 @@ struct MoeGemmArgs {
 // JL_MOE_G16_SB_WORDS words: eight matrix fragments of 64 lanes x 16 bytes (half, K-step), the
 // sub-block sums' fragment (32 lanes x 16 bytes) and the sixteen columns' scales.
 #define JL_MOE_G16_SB_WORDS 2192
+#define JL_MOE_G16_LDS_WORDS 2224   // the same in LDS, the fragments 65 vectors apart
 struct MoeG16PrepArgs {
     const float* x;
     const float* x2;        // null: plain activation

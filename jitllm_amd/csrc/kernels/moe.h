@@ -925,7 +925,7 @@ __device__ __forceinline__ f16x8 moe_g16_word(u32 w, const GemmWideScale& k, u32
 }
 
 // Matrix kernel: grid = 8 * ceil(n_expert / 8) * blocks * matrices (one dimension), block =
-// 64 * nwaves, dynamic LDS = (k/256) * JL_MOE_G16_SB_WORDS * 4 + 16.  Workgroups go round the eight
+// 64 * nwaves, dynamic LDS = (k/256) * JL_MOE_G16_LDS_WORDS * 4 + 16.  Workgroups go round the eight
 // XCDs in the order of their ids, so id % 8 names the XCD: expert e is worked on by XCD e % 8
 // alone, its (matrix, row block) workgroups one after the other there, and the group's fragments
 // are fetched into one L2 once.  A workgroup owns tiles_wg tiles of sixteen rows of the
@@ -937,8 +937,9 @@ __device__ __forceinline__ f16x8 moe_g16_word(u32 w, const GemmWideScale& k, u32
 // FUSED: no prep kernel and no workspace -- the workgroup quantizes its group's columns itself
 // (a wavefront per (column, super-block), the prep kernel's arithmetic) straight into the LDS
 // fragments, behind the first weight loads.  Every workgroup of the expert repeats that, which
-// pays while an expert has a handful of columns: two launches less a call.
-template <int CH, bool FUSED>
+// pays while an expert has a handful of columns: two launches less a call.  FUSED = 1: plain
+// columns, 2: silu(x) * x2.
+template <int CH, int FUSED>
 __device__ __forceinline__ void moe_g16_body(const MoeG16Args& p, uint8_t* smem) {
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -961,9 +962,12 @@ __device__ __forceinline__ void moe_g16_body(const MoeG16Args& p, uint8_t* smem)
     asm volatile("" : "+v"(mask_lo), "+v"(mask_hi), "+v"(magic));
     u32x4* sA4 = (u32x4*)smem;
     const float* sAf = (const float*)smem;
-    u32* next_tile = (u32*)smem + (size_t)nsb * JL_MOE_G16_SB_WORDS;   // behind the fragments
+    u32* next_tile = (u32*)smem + (size_t)nsb * JL_MOE_G16_LDS_WORDS;   // behind the fragments
     float* outm = p.out[mat];
-    constexpr int V = JL_MOE_G16_SB_WORDS / 4;   // 548 vectors a super-block
+    // LDS vectors a super-block: eight fragments 65 vectors apart (64 used: a column's pieces, one
+    // a fragment, then spread over sixteen banks when the fused form writes them), the sums' 32, the
+    // scales' 4; WS: vectors a super-block of the prep kernel's workspace
+    constexpr int V = JL_MOE_G16_LDS_WORDS / 4, WS = JL_MOE_G16_SB_WORDS / 4;
 
     u32x4 hd[2][CH], wq[2][CH][2];
     // step (tile ti of the workgroup's range, chunk ch) into a register set
@@ -985,19 +989,19 @@ __device__ __forceinline__ void moe_g16_body(const MoeG16Args& p, uint8_t* smem)
         // FUSED: the group's source rows, one a lane, and the first eight (column, super-block)
         // tasks of this wavefront requested ahead of the weights, which have the longer way and
         // would hold them up (a wavefront's loads return in order)
-        constexpr int TB = 8;
+        constexpr bool X2 = FUSED == 2;           // columns are silu(x) * x2 (the down projection's)
+        constexpr int TB = FUSED == 1 ? 16 : 8;   // tasks of a wavefront in flight: 128 or 64 a workgroup of eight
         const int ntask = ncg * nsb;
         u32 rowv = 0;
-        f32x4 xv[TB], xu[TB];
+        f32x4 xv[TB], xu[X2 ? TB : 1];
         auto issue = [&](int t0) {
 #pragma unroll
             for (int b = 0; b < TB; b++) {
-                xu[b] = f32x4{0.f, 0.f, 0.f, 0.f};
                 const int task = min(t0 + b * nwaves, ntask - 1);
                 const int i = task / nsb, sb = task - i * nsb;
                 const size_t row = (size_t)__shfl(rowv, i, 64);
                 xv[b] = ((const f32x4*)(p.x + row * (size_t)p.k + (size_t)sb * 256))[lane];
-                if (p.x2) xu[b] = ((const f32x4*)(p.x2 + row * (size_t)p.k + (size_t)sb * 256))[lane];
+                if (X2) xu[X2 ? b : 0] = ((const f32x4*)(p.x2 + row * (size_t)p.k + (size_t)sb * 256))[lane];
             }
         };
         if (FUSED) {
@@ -1009,10 +1013,10 @@ __device__ __forceinline__ void moe_g16_body(const MoeG16Args& p, uint8_t* smem)
         if (tid == 0) *next_tile = (u32)nwaves;   // tiles 0 .. nwaves - 1 are the wavefronts' first ones
         if (FUSED) {
             // zeros where the group has no column (fragments and sums; the scales are not read there)
-            const int total = nsb * V;
+            const int total = nsb * WS;
             for (int idx = tid; idx < total; idx += nthreads) {
-                const int o = idx % V;
-                if (o < 544 && (o & 15) >= ncg) sA4[idx] = u32x4{0u, 0u, 0u, 0u};
+                const int sb = idx / WS, o = idx - sb * WS;
+                if (o < 544 && (o & 15) >= ncg) sA4[sb * V + (o < 512 ? o + (o >> 6) : o + 8)] = u32x4{0u, 0u, 0u, 0u};
             }
             u32* sAw = (u32*)smem;
             _Float16* sAh = (_Float16*)smem;
@@ -1025,7 +1029,10 @@ __device__ __forceinline__ void moe_g16_body(const MoeG16Args& p, uint8_t* smem)
                     if (task < ntask) {   // uniform
                         const int i = task / nsb, sb = task - i * nsb;
                         f32x4 w = xv[b];
-                        if (p.x2) w = f32x4{silu_f32(w.x) * xu[b].x, silu_f32(w.y) * xu[b].y, silu_f32(w.z) * xu[b].z, silu_f32(w.w) * xu[b].w};
+                        if (X2) {
+                            const f32x4 u = xu[X2 ? b : 0];
+                            w = f32x4{silu_f32(w.x) * u.x, silu_f32(w.y) * u.y, silu_f32(w.z) * u.z, silu_f32(w.w) * u.w};
+                        }
                         const u32 m = max(max(abs_bits(w.x), abs_bits(w.y)), max(abs_bits(w.z), abs_bits(w.w)));
                         const u32 amax = wave_amax_256(m);
                         float d;
@@ -1037,28 +1044,28 @@ __device__ __forceinline__ void moe_g16_body(const MoeG16Args& p, uint8_t* smem)
                         const int sub = lane >> 3, ks = lane & 7, kg = sub >> 1, hi = sub & 1;
                         auto f = [](u32 x, int b2) { return (_Float16)(float)(int8_t)(x >> (8 * b2)); };
                         const f16x2 p02 = {f(q, 0), f(q, 2)}, p13 = {f(q, 1), f(q, 3)};
-                        const int vec = sb * V + ks * 64 + 16 * kg + i;
+                        const int vec = sb * V + ks * 65 + 16 * kg + i;
                         sAw[vec * 4 + hi] = __builtin_bit_cast(u32, p02);
                         sAw[vec * 4 + 2 + hi] = __builtin_bit_cast(u32, p13);
                         if ((lane & 7) == 0) {
-                            sAh[(sb * V + 512 + i) * 8 + sub] = (_Float16)(float)(a32 & 63);
-                            sAh[(sb * V + 512 + 16 + i) * 8 + sub] = (_Float16)(float)(a32 >> 6);
+                            sAh[(sb * V + 520 + i) * 8 + sub] = (_Float16)(float)(a32 & 63);
+                            sAh[(sb * V + 520 + 16 + i) * 8 + sub] = (_Float16)(float)(a32 >> 6);
                         }
-                        if (lane == 0) sAfw[sb * JL_MOE_G16_SB_WORDS + 2176 + i] = d;
+                        if (lane == 0) sAfw[(sb * V + 552) * 4 + i] = d;
                     }
                 }
             }
         } else {
             const u32x4* src = (const u32x4*)(p.ws + slot * nsb * JL_MOE_G16_SB_WORDS);
-            // up to eighteen loads in flight a thread (all of K = 2048 at 256 threads): the fill is
-            // one round trip to L2, not one a vector
-            constexpr int NB = 18;
-            const int total = nsb * V;
+            // twelve loads in flight a thread (all of K = 2048 at 512 threads): the fill is one round
+            // trip to L2, not one a vector
+            constexpr int NB = 12;
+            const int total = nsb * WS;
             for (int base = tid; base < total; base += NB * nthreads) {
                 u32x4 val[NB];
 #pragma unroll
                 for (int u = 0; u < NB; u++) {
-                    const int idx = base + u * nthreads, o = idx % V;
+                    const int idx = base + u * nthreads, o = idx % WS;
                     // fragments: lane = o % 64, its column o % 16; sums: (o - 512) % 16; scales: all
                     const bool have = idx < total && (o >= 544 || (o & 15) < ncg);
                     val[u] = u32x4{0u, 0u, 0u, 0u};
@@ -1066,8 +1073,8 @@ __device__ __forceinline__ void moe_g16_body(const MoeG16Args& p, uint8_t* smem)
                 }
 #pragma unroll
                 for (int u = 0; u < NB; u++) {
-                    const int idx = base + u * nthreads;
-                    if (idx < total) sA4[idx] = val[u];
+                    const int idx = base + u * nthreads, sb = idx / WS, o = idx - sb * WS;
+                    if (idx < total) sA4[sb * V + (o < 512 ? o + (o >> 6) : o + 8)] = val[u];
                 }
             }
         }
@@ -1098,16 +1105,16 @@ __device__ __forceinline__ void moe_g16_body(const MoeG16Args& p, uint8_t* smem)
                     gemm_wide_scale(hd[cur][s], kg & 1, kg >> 1, sc);
 #pragma unroll
                     for (int ks = 0; ks < 8; ks++) {
-                        const f16x8 af = __builtin_bit_cast(f16x8, sA4[sb * V + ks * 64 + lane]);
+                        const f16x8 af = __builtin_bit_cast(f16x8, sA4[sb * V + ks * 65 + lane]);
                         const f16x8 b = moe_g16_word(wq[cur][s][ks >> 2][ks & 3], sc, mask_lo, mask_hi, magic);
                         const f32x4 czero = {0.f, 0.f, 0.f, 0.f};
                         accP = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, b, ks == 0 ? czero : accP, 0, 0, 0);
                     }
                     // out += d_a * (d * P - dmin * M) for the super-block
                     u32x4 augw = u32x4{0u, 0u, 0u, 0u};
-                    if (lane < 32) augw = sA4[sb * V + 512 + lane];
+                    if (lane < 32) augw = sA4[sb * V + 520 + lane];
                     const f16x8 aug = __builtin_bit_cast(f16x8, augw);
-                    const f32x4 dav = *(const f32x4*)(sAf + sb * JL_MOE_G16_SB_WORDS + 2176 + 4 * kg);
+                    const f32x4 dav = *(const f32x4*)(sAf + (sb * V + 552) * 4 + 4 * kg);
                     const float mul = kg == 0 ? 1.0f : (kg == 1 ? 64.0f : 0.0f);
                     const GemmScaleBytes sbytes = gemm_scale_bytes(hd[cur][s].y, hd[cur][s].z, hd[cur][s].w);
                     f16x8 mm;
