@@ -413,13 +413,15 @@ def ffn_packed_section(dev, gate_):
             "checked_rel_err": float(f"{err:.2e}")}
 
 
-def moe_section(dev, gate_, rows=64):
+def moe_section(dev, gate_, rows=64, packed=False):
     """Qwen3-30B-A3B routed feed-forward block: 128 experts (gate/up 768x2048, down 2048x768,
     Q4_K), 64 rows routed top-8; one step = router logits (f32 router matrix, rows ~ N(0, 1/k)
     so the logits are ~ N(0,1)) + softmax/top-8 + group + gate/up + down + combine, all on the
     device.  Bytes = the touched experts' three sheets + router matrix + x in + resid out.
     Output check: three rows of the block recomputed in f64 from sheets dequantized on the
-    device, with the device's own selection and weights."""
+    device, with the device's own selection and weights.
+    packed: the three banks are packed planes on the device (one plane set per bank, as a .jlm
+    file holds them), read where they lie."""
     from jitllm_amd import quant, synth
     from jitllm_amd.hipmem import DeviceArray
     t, n_expert, k_used, n_ffn, n_embd = quant.Q4_K, 128, 8, 768, 2048
@@ -443,12 +445,26 @@ def moe_section(dev, gate_, rows=64):
         hosts.append(synth.quantized_weights(t, r * n_expert, k, seed=10 + i))
         banks.append(DeviceArray(hosts[-1]))
     resid = DeviceArray(shape=(rows, n_embd), dtype=np.float32, fill=0)
+    pbanks = []
+    if packed:
+        for i, (r, k) in enumerate([(n_ffn, n_embd), (n_ffn, n_embd), (n_embd, n_ffn)]):
+            nq, nd, nsc = dev.packed_words(t, r * n_expert, k)
+            pl = [DeviceArray(shape=(n,), dtype=np.uint32, fill=0) for n in (nq, nd, nsc)]
+            if not dev.pack_weights_dev(t, banks[i].ptr, r * n_expert, k, pl[0].ptr, pl[1].ptr, pl[2].ptr):
+                raise RuntimeError("the device declined to pack a bank")
+            dev.synchronize()
+            banks[i].free()
+            banks[i] = pl[0]
+            banks += pl[1:]
+            pbanks.append(dev.packed_bank(pl[0].ptr, pl[1].ptr, pl[2].ptr, 0, r * n_expert))
 
     def run(_):
         if not (dev.moe_logits_dev(ld.ptr, 0, router.ptr, x.ptr, n_expert, n_embd, rows) and
                 dev.moe_route_dev(ld.ptr, rows, n_expert, k_used, sd.ptr, k_used + 1, wd.ptr) and
-                dev.moe_ffn_dev(resid.ptr, t, banks[0].ptr, banks[1].ptr, banks[2].ptr, x.ptr, sd.ptr,
-                                k_used + 1, wd.ptr, rows, k_used, n_expert, n_ffn, n_embd)):
+                (dev.moe_ffn_packed_dev(resid.ptr, t, pbanks[0], pbanks[1], pbanks[2], x.ptr, sd.ptr, k_used + 1,
+                                        wd.ptr, rows, k_used, n_expert, n_ffn, n_embd) if packed else
+                 dev.moe_ffn_dev(resid.ptr, t, banks[0].ptr, banks[1].ptr, banks[2].ptr, x.ptr, sd.ptr,
+                                 k_used + 1, wd.ptr, rows, k_used, n_expert, n_ffn, n_embd))):
             raise RuntimeError("the device declined the mixture block")
     ms = measure(dev, run, 20, gate_)
     resid.zero()
@@ -718,7 +734,7 @@ def main():
     ap.add_argument("--matvec", metavar="TYPE,NROWS,K[,packed][,w32]", help="only this decode matvec (TYPE q4_k, q6_k or "
                     "q8_0; packed = packed planes; w32 = activation window 32), for profiling one kernel; "
                     "prints its section alone")
-    ap.add_argument("--section", choices=["mxfp4", "moe", "moe_decode", "ffn", "ffn_packed", "ceiling", "gemm_packed"],
+    ap.add_argument("--section", choices=["mxfp4", "moe", "moe_packed", "moe_decode", "ffn", "ffn_packed", "ceiling", "gemm_packed"],
                     help="only this section of the default run, for profiling its kernels; prints the section alone")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -749,7 +765,8 @@ def main():
         dev.close()
         return
     if args.section:
-        fn = {"mxfp4": mxfp4_section, "moe": moe_section, "moe_decode": moe_decode_section, "ffn": ffn_section,
+        fn = {"mxfp4": mxfp4_section, "moe": moe_section, "moe_packed": lambda d, g: moe_section(d, g, packed=True),
+              "moe_decode": moe_decode_section, "ffn": ffn_section,
               "ffn_packed": ffn_packed_section, "ceiling": ceiling_section,
               "gemm_packed": lambda d, g: gemm_section(d, g, {4096: (512,), 14336: (512,)}, packed=True)}[args.section]
         print(json.dumps({args.section: fn(dev, gate)}), flush=True)
@@ -821,6 +838,7 @@ def main():
             "q8_0": gemm_section(dev, gate, {14336: (512, 2048)}, quant.Q8_0, 4096, 32),
             "q6_k": gemm_section(dev, gate, {4096: (512, 2048)}, quant.Q6_K, 14336, 32)}
         line["moe_block"] = moe_section(dev, gate)
+        line["moe_block_packed_planes"] = moe_section(dev, gate, packed=True)
         line["moe_block_prefill_1024_rows"] = moe_section(dev, gate, 1024)   # matrix-core tiles per expert
         line["moe_decode"] = moe_decode_section(dev, gate)
         line["mxfp4_gemm"] = mxfp4_section(dev, gate)

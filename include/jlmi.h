@@ -97,6 +97,7 @@ int jl_synchronize(jl_ctx *ctx);
  * (row shares an expert's matrix is split into), "moe.form" (grouped matmul: 1 dot products,
  * 2 / 3 groups of 32 / 16 columns on the matrix cores, 4 the prefill tile per expert),
  * "moe.group16" (form 3: 1 a prep kernel quantizes the columns, 2 the matrix kernel does),
+ * "moe.chunk" (form 3: super-blocks a step, 1-3),
  * "moe.group" / "moe.logits" / "moe.q6k_cols" / "moe.waves" / "moe.lpr" (forms of the mixture
  * block's other kernels),
  * "mxfp4.split" (K slices of the MXFP4 GEMM), "mxfp4.rows" (96 or 128 rows a tile; 1: the

@@ -39,6 +39,7 @@ struct Tuning {
     int gemm_planes = 0;
     int moe_form = 0;
     int moe_g16 = 0;
+    int moe_chunk = 0;
     int moe_waves = 0;
     int moe_lpr = 0;
     int mx_rows = 0;
@@ -970,6 +971,85 @@ int moe_matvec_launch(jl_ctx* c, float* out0, float* out1, int type, const void*
     // Q6_K sheets (the down projections of a model whose other experts are Q4_K) have form 4
     // alone, with the Q6_K GEMM's tile; the dot-product kernel is slower for that type, so the
     // tile takes over earlier ("moe.q6k_cols": columns an expert on average, default 12).
+    // Form 3: groups of sixteen columns on the 16 x 16 x 32 matrix instruction, the weights decoded
+    // in registers straight into its operand (Q4_K GGUF sheets or packed planes, the k-quant window; the group's
+    // fragments for the whole of K sit in LDS).  Its steady state runs at the rate of a plain read;
+    // the library picks it from two (over planes three) columns an expert on average up to 22, while the
+    // fragments take at most half a CU's LDS (K <= 2304); "moe.form" = 3 forces it wherever they fit.
+    {
+        const int nsb = k / 256;
+        const size_t lds16 = (size_t)nsb * JL_MOE_G16_LDS_WORDS * 4 + 16;   // the fragments, the tile counter
+        const size_t nslots16 = (size_t)ncols / 16 + (size_t)n_expert + 1;
+        const bool can16 = type == JL_TYPE_Q4_K && c->act_window == 256 && lds16 <= c->lds_limit &&
+                           (size_t)nrows * row_bytes < ((size_t)1 << 32);
+        const bool pick16 = c->tune.moe_form == 0 && 2 * lds16 <= c->lds_limit && (long)ncols >= (planes ? 3L : 2L) * n_expert &&
+                            (long)ncols < 22L * n_expert;
+        if (can16 && (c->tune.moe_form == 3 || pick16)) {
+            // up to eight columns an expert the matrix kernel quantizes them itself: no prep launch,
+            // no workspace ("moe.group16" = 1 forces the prep kernel, 2 the fused form)
+            const bool fused = c->tune.moe_g16 == 2 || (c->tune.moe_g16 == 0 && (long)ncols <= 8L * n_expert);
+            MoeG16PrepArgs pa;
+            pa.ws = nullptr;
+            if (!fused) {
+                rc = ws_ensure(c, &c->moe_q_ws, &c->moe_q_ws_bytes, nslots16 * nsb * JL_MOE_G16_SB_WORDS * 4);
+                if (rc != JL_OK) return rc;
+                pa.x = x; pa.x2 = x2; pa.src = src; pa.start = start; pa.ws = (uint32_t*)c->moe_q_ws;
+                pa.k = k; pa.n_expert = n_expert;
+                void* pp[] = {&pa};
+                rc = launch(c, planes ? "jl_moe_g16_prep_planes" : "jl_moe_g16_prep", (unsigned)((nsb + 3) / 4), (unsigned)ncols, 256, 0,
+                            st, pp);
+                if (rc != JL_OK) return rc;
+            }
+            MoeG16Args ga;
+            ga.out[0] = out0; ga.out[1] = out1;
+            ga.bank[0] = (const uint8_t*)bank0; ga.bank[1] = (const uint8_t*)bank1;
+            ga.ws = pa.ws; ga.start = start;
+            if (fused) { ga.x = x; ga.x2 = x2; ga.src = src; }
+            ga.sheet_bytes = sheet; ga.nrows = nrows; ga.k = k; ga.row_bytes = row_bytes;
+            if (planes) {
+                const jl_packed_bank* pbs[2] = {pb0, pb1};
+                for (int m = 0; m < (pb1 ? 2 : 1); m++) { ga.pqs[m] = pbs[m]->qs; ga.pd[m] = pbs[m]->d; ga.psc[m] = pbs[m]->sc; }
+                ga.sheet_words = pb0->sheet_bytes / 4;
+                ga.row_step = pb0->sheet_bytes ? 0 : nrows;
+                ga.pstride = pb0->stride;
+            }
+            // One workgroup of eight wavefronts a CU (the same age on every SIMD, tiles handed out as
+            // they get to them: two younger workgroups of four measured 4 % slower), so the grid runs
+            // in rounds of CUs workgroups; among the splits of the rows into blocks the one with the
+            // least rounds x tiles a wavefront, the fewest blocks among equals (every block fills LDS
+            // anew).  Experts that can have a column: at most one a column.  "moe.waves" = 4: the
+            // two-workgroup form.
+            const int nmat = (planes ? pb1 != nullptr : bank1 != nullptr) ? 2 : 1, tiles = (nrows + 15) / 16;
+            const int nwaves = c->tune.moe_waves == 4 || (c->tune.moe_waves == 12 && !planes) ? c->tune.moe_waves : 8;
+            const long wgs_cu = nwaves == 4 ? 2 : 1;
+            const int sets = (tiles + nwaves - 1) / nwaves;
+            const long n_act = std::min<long>(n_expert, ncols);
+            int best_blocks = 1;
+            long best_cost = -1;
+            for (int nb = 1; nb <= sets && nb <= 64; nb++) {
+                const long per_wave = (sets + nb - 1) / nb;
+                const long rounds = ((long)nb * n_act * nmat + wgs_cu * c->num_cu - 1) / (wgs_cu * c->num_cu);
+                const long cost = rounds * per_wave;
+                if (best_cost < 0 || cost < best_cost) { best_cost = cost; best_blocks = nb; }
+            }
+            if (c->tune.moe_shares > 0) best_blocks = std::min(c->tune.moe_shares, sets);
+            ga.tiles_wg = (tiles + best_blocks - 1) / best_blocks;   // handed out inside the workgroup as its wavefronts get to them
+            ga.blocks = (tiles + ga.tiles_wg - 1) / ga.tiles_wg;
+            ga.nmat = nmat; ga.n_expert = n_expert; ga.nwaves = nwaves;
+            const long grid = 8L * ((n_expert + 7) / 8) * ga.blocks * nmat;
+            if (grid >= (1L << 31)) return JL_DECLINED;
+            // super-blocks a step: all of a short row, else two (288 contiguous bytes a row; four
+            // measured 10 % slower at K = 2048: twice the bytes in flight before the first step)
+            // (over planes one: a lane's twelve loads of a super-block go to twelve planes, and more
+            // of them in flight measured 5 % slower)
+            int ch = planes ? 1 : (nsb <= 3 ? nsb : 2);
+            if (c->tune.moe_chunk >= 1 && c->tune.moe_chunk <= 3) ch = std::min(c->tune.moe_chunk, nsb);
+            char name[32];
+            snprintf(name, sizeof name, "jl_moe_g16%s_%c%d", planes ? "p" : "", fused ? (x2 ? 'g' : 'f') : 'c', ch);
+            void* gp[] = {&ga};
+            return launch(c, name, (unsigned)grid, 1, (unsigned)(64 * nwaves), (unsigned)lds16, st, gp);
+        }
+    }
     if (planes && c->tune.moe_form != 4 && (c->tune.moe_form == 1 || (long)ncols < kMoePlaneTileCols * n_expert)) {
         // few columns an expert: the dot-product form over planes (rows on lanes, a lane's share of a
         // chunk loaded once for all the expert's columns, the columns as scalar operands)
@@ -999,73 +1079,6 @@ int moe_matvec_launch(jl_ctx* c, float* out0, float* out1, int type, const void*
         void* params[] = {&a};
         return launch(c, "jl_moe_matvec_planes_q4k", (unsigned)((nrows + 63) / 64), (unsigned)n_expert, (unsigned)(a.nwaves * 64),
                       (unsigned)(a.nwaves * 8 * 256), st, params, (unsigned)nmat);   // JL_MOEP_TB columns a pass
-    }
-    // Form 3: groups of sixteen columns on the 16 x 16 x 32 matrix instruction, the weights decoded
-    // in registers straight into its operand (Q4_K GGUF sheets, the k-quant window; the group's
-    // fragments for the whole of K sit in LDS).  Its steady state runs at the rate of a plain read;
-    // the library picks it from two columns an expert on average up to 22, while two workgroups
-    // fit a CU's LDS (K <= 2304); "moe.form" = 3 forces it wherever one fits.
-    {
-        const int nsb = k / 256;
-        const size_t lds16 = (size_t)nsb * JL_MOE_G16_LDS_WORDS * 4 + 16;   // the fragments, the tile counter
-        const size_t nslots16 = (size_t)ncols / 16 + (size_t)n_expert + 1;
-        const bool can16 = !planes && type == JL_TYPE_Q4_K && c->act_window == 256 && lds16 <= c->lds_limit &&
-                           (size_t)nrows * row_bytes < ((size_t)1 << 32);
-        const bool pick16 = c->tune.moe_form == 0 && 2 * lds16 <= c->lds_limit && (long)ncols >= 2L * n_expert &&
-                            (long)ncols < 22L * n_expert;
-        if (can16 && (c->tune.moe_form == 3 || pick16)) {
-            // up to eight columns an expert the matrix kernel quantizes them itself: no prep launch,
-            // no workspace ("moe.group16" = 1 forces the prep kernel, 2 the fused form)
-            const bool fused = c->tune.moe_g16 == 2 || (c->tune.moe_g16 == 0 && (long)ncols <= 8L * n_expert);
-            MoeG16PrepArgs pa;
-            pa.ws = nullptr;
-            if (!fused) {
-                rc = ws_ensure(c, &c->moe_q_ws, &c->moe_q_ws_bytes, nslots16 * nsb * JL_MOE_G16_SB_WORDS * 4);
-                if (rc != JL_OK) return rc;
-                pa.x = x; pa.x2 = x2; pa.src = src; pa.start = start; pa.ws = (uint32_t*)c->moe_q_ws;
-                pa.k = k; pa.n_expert = n_expert;
-                void* pp[] = {&pa};
-                rc = launch(c, "jl_moe_g16_prep", (unsigned)((nsb + 3) / 4), (unsigned)ncols, 256, 0, st, pp);
-                if (rc != JL_OK) return rc;
-            }
-            MoeG16Args ga;
-            ga.out[0] = out0; ga.out[1] = out1;
-            ga.bank[0] = (const uint8_t*)bank0; ga.bank[1] = (const uint8_t*)bank1;
-            ga.ws = pa.ws; ga.start = start;
-            if (fused) { ga.x = x; ga.x2 = x2; ga.src = src; }
-            ga.sheet_bytes = sheet; ga.nrows = nrows; ga.k = k; ga.row_bytes = row_bytes;
-            // One workgroup of eight wavefronts a CU (the same age on every SIMD, tiles handed out as
-            // they get to them: two younger workgroups of four measured 4 % slower), so the grid runs
-            // in rounds of CUs workgroups; among the splits of the rows into blocks the one with the
-            // least rounds x tiles a wavefront, the fewest blocks among equals (every block fills LDS
-            // anew).  Experts that can have a column: at most one a column.  "moe.waves" = 4: the
-            // two-workgroup form.
-            const int nmat = bank1 ? 2 : 1, tiles = (nrows + 15) / 16, nwaves = c->tune.moe_waves == 4 || c->tune.moe_waves == 12 ? c->tune.moe_waves : 8;
-            const long wgs_cu = nwaves == 4 ? 2 : 1;
-            const int sets = (tiles + nwaves - 1) / nwaves;
-            const long n_act = std::min<long>(n_expert, ncols);
-            int best_blocks = 1;
-            long best_cost = -1;
-            for (int nb = 1; nb <= sets && nb <= 64; nb++) {
-                const long per_wave = (sets + nb - 1) / nb;
-                const long rounds = ((long)nb * n_act * nmat + wgs_cu * c->num_cu - 1) / (wgs_cu * c->num_cu);
-                const long cost = rounds * per_wave;
-                if (best_cost < 0 || cost < best_cost) { best_cost = cost; best_blocks = nb; }
-            }
-            if (c->tune.moe_shares > 0) best_blocks = std::min(c->tune.moe_shares, sets);
-            ga.tiles_wg = (tiles + best_blocks - 1) / best_blocks;   // handed out inside the workgroup as its wavefronts get to them
-            ga.blocks = (tiles + ga.tiles_wg - 1) / ga.tiles_wg;
-            ga.nmat = nmat; ga.n_expert = n_expert; ga.nwaves = nwaves;
-            const long grid = 8L * ((n_expert + 7) / 8) * ga.blocks * nmat;
-            if (grid >= (1L << 31)) return JL_DECLINED;
-            // super-blocks a step: all of a short row, else two (288 contiguous bytes a row; four
-            // measured 10 % slower at K = 2048: twice the bytes in flight before the first step)
-            const int ch = nsb <= 3 ? nsb : 2;
-            char name[32];
-            snprintf(name, sizeof name, "jl_moe_g16_%c%d", fused ? (x2 ? 'g' : 'f') : 'c', ch);
-            void* gp[] = {&ga};
-            return launch(c, name, (unsigned)grid, 1, (unsigned)(64 * nwaves), (unsigned)lds16, st, gp);
-        }
     }
     const bool q6 = type == JL_TYPE_Q6_K;
     const long q6_cols = c->tune.moe_q6k_cols > 0 ? c->tune.moe_q6k_cols : 12;
@@ -1245,7 +1258,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     if (e != hipSuccess)
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
-    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_prep_q4k_planes", "jl_gemm_q4k_r64_planes", "jl_gemm_q4k_wide_planes", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_group2_wide", "jl_moe_quant", "jl_moe_matvec_planes_q4k", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_prep_planes", "jl_moe_gemm_q4k", "jl_moe_g16_prep", "jl_moe_g16_c1", "jl_moe_g16_c2", "jl_moe_g16_c3", "jl_moe_g16_f1", "jl_moe_g16_f2", "jl_moe_g16_f3", "jl_moe_g16_g1", "jl_moe_g16_g2", "jl_moe_g16_g3", "jl_moe_gemm_r64", "jl_moe_gemm_r64_planes", "jl_moe_gemm_q6k_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_mxfp4_matvec1_b1", "jl_mxfp4_matvec1_b2", "jl_mxfp4_matvec1_b3", "jl_mxfp4_scaled_prep", "jl_mxfp4_scaled_gemm", "jl_mxfp4_planes_prep", "jl_mxfp4_planes_gemm", "jl_mxfp4_matvec_planes_r64", "jl_mxfp4_matvec_planes_r32", "jl_mxfp4_matvec_planes_r16", "jl_unpack_mxfp4", "jl_sum_parts", "jl_probe_read", "jl_probe_empty", "jl_probe_wait", "jl_probe_mfma", "jl_probe_mfma_v5",
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_prep_q4k_planes", "jl_gemm_q4k_r64_planes", "jl_gemm_q4k_wide_planes", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_group2_wide", "jl_moe_quant", "jl_moe_matvec_planes_q4k", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_prep_planes", "jl_moe_gemm_q4k", "jl_moe_g16_prep", "jl_moe_g16_c1", "jl_moe_g16_c2", "jl_moe_g16_c3", "jl_moe_g16_f1", "jl_moe_g16_f2", "jl_moe_g16_f3", "jl_moe_g16_g1", "jl_moe_g16_g2", "jl_moe_g16_g3", "jl_moe_g16_prep_planes", "jl_moe_g16p_c1", "jl_moe_g16p_c2", "jl_moe_g16p_c3", "jl_moe_g16p_f1", "jl_moe_g16p_f2", "jl_moe_g16p_f3", "jl_moe_g16p_g1", "jl_moe_g16p_g2", "jl_moe_g16p_g3", "jl_moe_gemm_r64", "jl_moe_gemm_r64_planes", "jl_moe_gemm_q6k_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_mxfp4_matvec1_b1", "jl_mxfp4_matvec1_b2", "jl_mxfp4_matvec1_b3", "jl_mxfp4_scaled_prep", "jl_mxfp4_scaled_gemm", "jl_mxfp4_planes_prep", "jl_mxfp4_planes_gemm", "jl_mxfp4_matvec_planes_r64", "jl_mxfp4_matvec_planes_r32", "jl_mxfp4_matvec_planes_r16", "jl_unpack_mxfp4", "jl_sum_parts", "jl_probe_read", "jl_probe_empty", "jl_probe_wait", "jl_probe_mfma", "jl_probe_mfma_v5",
                                       "jl_pack_weights", "jl_unpack_q4k", "jl_unpack_q6k", "jl_unpack_q8_0"};
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int rw : {16, 32, 64})
@@ -1350,6 +1363,7 @@ int jl_set_tuning(jl_ctx* c, const char* key, int value) {
     else if (!strcmp(key, "moe.shares")) c->tune.moe_shares = value;
     else if (!strcmp(key, "moe.form")) c->tune.moe_form = value;
     else if (!strcmp(key, "moe.group16")) c->tune.moe_g16 = value;
+    else if (!strcmp(key, "moe.chunk")) c->tune.moe_chunk = value;
     else if (!strcmp(key, "moe.waves")) c->tune.moe_waves = value;
     else if (!strcmp(key, "moe.lpr")) c->tune.moe_lpr = value;
     else if (!strcmp(key, "gemm.rows")) c->tune.gemm_rows = value;

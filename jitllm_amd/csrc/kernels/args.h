@@ -143,6 +143,14 @@ struct MoeG16Args {
     int nrows, k, row_bytes;
     int tiles_wg;           // tiles of sixteen rows a workgroup owns
     int blocks, nmat, n_expert, nwaves;   // row blocks an (expert, matrix); wavefronts a workgroup
+    // the banks as packed planes (plane form; bank[] and sheet_bytes unused): expert e's planes are
+    // pqs / pd / psc [mat] + e * sheet_words (u32 words; 0 when the bank is ONE plane set), its first
+    // row e * row_step inside them (0 when every expert has its own sheet), pstride rows a plane set
+    const uint32_t* pqs[2] = {nullptr, nullptr};
+    const uint32_t* pd[2] = {nullptr, nullptr};
+    const uint32_t* psc[2] = {nullptr, nullptr};
+    size_t sheet_words = 0;
+    int row_step = 0, pstride = 0;
     // fused form: the columns are quantized by the matrix kernel itself (ws unused)
     const float* x = nullptr;
     const float* x2 = nullptr;

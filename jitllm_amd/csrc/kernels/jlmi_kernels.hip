@@ -251,14 +251,21 @@ extern "C" __global__ __launch_bounds__(256, 2) void jl_moe_gemm_q4k(MoeGemmArgs
 // block = 64 * nwaves (<= 768), dynamic LDS = (k/256) * JL_MOE_G16_SB_WORDS * 4
 extern "C" __global__ __launch_bounds__(256) void jl_moe_g16_prep(MoeG16PrepArgs p) {
     __shared__ u32 lds[4 * 72];
-    moe_g16_prep_body(p, lds);
+    moe_g16_prep_body<false>(p, lds);
+}
+extern "C" __global__ __launch_bounds__(256) void jl_moe_g16_prep_planes(MoeG16PrepArgs p) {
+    __shared__ u32 lds[4 * 72];
+    moe_g16_prep_body<true>(p, lds);
 }
 // _c: fragments from the prep kernel's workspace; _f / _g: the columns (plain / silu(x) * x2) quantized by
-// the kernel itself
+// the kernel itself; g16p: the sheets are packed planes
 #define JL_MOE_G16_KERNEL(CH)                                                                                           \
     extern "C" __global__ __launch_bounds__(768) void jl_moe_g16_c##CH(MoeG16Args p) { moe_g16_body<CH, 0>(p, jl_smem); } \
     extern "C" __global__ __launch_bounds__(768) void jl_moe_g16_f##CH(MoeG16Args p) { moe_g16_body<CH, 1>(p, jl_smem); } \
-    extern "C" __global__ __launch_bounds__(768) void jl_moe_g16_g##CH(MoeG16Args p) { moe_g16_body<CH, 2>(p, jl_smem); }
+    extern "C" __global__ __launch_bounds__(768) void jl_moe_g16_g##CH(MoeG16Args p) { moe_g16_body<CH, 2>(p, jl_smem); } \
+    extern "C" __global__ __launch_bounds__(512) void jl_moe_g16p_c##CH(MoeG16Args p) { moe_g16_body<CH, 0, true>(p, jl_smem); } \
+    extern "C" __global__ __launch_bounds__(512) void jl_moe_g16p_f##CH(MoeG16Args p) { moe_g16_body<CH, 1, true>(p, jl_smem); } \
+    extern "C" __global__ __launch_bounds__(512) void jl_moe_g16p_g##CH(MoeG16Args p) { moe_g16_body<CH, 2, true>(p, jl_smem); }
 JL_MOE_G16_KERNEL(1) JL_MOE_G16_KERNEL(2) JL_MOE_G16_KERNEL(3)
 // Experts with many columns: the prefill GEMM's 128-token x 64-row tile placed per expert.  An
 // expert's column groups are consecutive slots of the prepared workspace, so to the tile they

@@ -859,6 +859,7 @@ __device__ __forceinline__ void moe_gemm_q4k_body(const MoeGemmArgs& p, uint8_t*
 // column (lane l owns elements 4l..4l+3), finds the column's expert by counting the experts
 // whose first column is not after it, and writes the 32 sixteen-byte pieces of the column's
 // fragments, the two pieces of its sub-block sums (low six bits, the rest) and its scale.
+template <bool PL = false>
 __device__ __forceinline__ void moe_g16_prep_body(const MoeG16PrepArgs& p, u32* lds) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const u32 c = blockIdx.y;
@@ -893,7 +894,12 @@ __device__ __forceinline__ void moe_g16_prep_body(const MoeG16PrepArgs& p, u32* 
     u32* blk = p.ws + (slot * nsb + sb) * JL_MOE_G16_SB_WORDS;
     if (lane < 32) {
         const int ks = lane >> 2, kg = lane & 3;
-        const u32 lo = sq[16 * kg + ks], hi = sq[16 * kg + 8 + ks];
+        // GGUF sheets: word ks of group kg pairs elements 4 ks.. of sub-blocks 2 kg and 2 kg + 1;
+        // packed planes: K-step ks is word ks % 4 of sub-block 2 kg + ks / 4, whose low nibbles are
+        // elements 4 w.. and whose high nibbles elements 4 w + 16.. of that one sub-block
+        const int psub = 2 * kg + (ks >> 2), pw = ks & 3;
+        const u32 lo = PL ? sq[8 * psub + pw] : sq[16 * kg + ks];
+        const u32 hi = PL ? sq[8 * psub + 4 + pw] : sq[16 * kg + 8 + ks];
         auto f = [](u32 w, int b) { return (_Float16)(float)(int8_t)(w >> (8 * b)); };
         const f16x8 o = {f(lo, 0), f(lo, 2), f(hi, 0), f(hi, 2), f(lo, 1), f(lo, 3), f(hi, 1), f(hi, 3)};
         ((u32x4*)blk)[ks * 64 + 16 * kg + i] = __builtin_bit_cast(u32x4, o);
@@ -939,7 +945,7 @@ __device__ __forceinline__ f16x8 moe_g16_word(u32 w, const GemmWideScale& k, u32
 // fragments, behind the first weight loads.  Every workgroup of the expert repeats that, which
 // pays while an expert has a handful of columns: two launches less a call.  FUSED = 1: plain
 // columns, 2: silu(x) * x2.
-template <int CH, int FUSED>
+template <int CH, int FUSED, bool PL = false>
 __device__ __forceinline__ void moe_g16_body(const MoeG16Args& p, uint8_t* smem) {
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -957,7 +963,7 @@ __device__ __forceinline__ void moe_g16_body(const MoeG16Args& p, uint8_t* smem)
     const int tile_base = blk * p.tiles_wg;
     const int ntw = min(tiles, tile_base + p.tiles_wg) - tile_base;   // tiles of this workgroup
     const int j = lane & 15, kg = lane >> 4;
-    const uint8_t* sheet = p.bank[mat] + (size_t)e * p.sheet_bytes;
+    const uint8_t* sheet = PL ? nullptr : p.bank[mat] + (size_t)e * p.sheet_bytes;
     u32 mask_lo = 0x000F000Fu, mask_hi = 0x00F000F0u, magic = 0x64006400u;
     asm volatile("" : "+v"(mask_lo), "+v"(mask_hi), "+v"(magic));
     u32x4* sA4 = (u32x4*)smem;
@@ -971,8 +977,29 @@ __device__ __forceinline__ void moe_g16_body(const MoeG16Args& p, uint8_t* smem)
 
     u32x4 hd[2][CH], wq[2][CH][2];
     // step (tile ti of the workgroup's range, chunk ch) into a register set
+    // PL (packed planes): the header is the row's (d, dmin) word and its three words of 6-bit fields,
+    // the lane's eight words are sub-blocks 2 kg and 2 kg + 1 (four words each); every load
+    // instruction reads four runs of sixteen consecutive rows
+    const size_t pst = (size_t)p.pstride;
+    const u32* pl_qs = PL ? p.pqs[mat] + (size_t)e * p.sheet_words + (size_t)e * p.row_step : nullptr;
+    const u32* pl_d = PL ? p.pd[mat] + (size_t)e * p.sheet_words + (size_t)e * p.row_step : nullptr;
+    const u32* pl_sc = PL ? p.psc[mat] + (size_t)e * p.sheet_words + (size_t)e * p.row_step : nullptr;
     auto load_step = [&](int ti, int ch, u32x4 (&h)[CH], u32x4 (&q)[CH][2]) {
         const int row = min(16 * (tile_base + ti) + j, p.nrows - 1);
+        if (PL) {
+#pragma unroll
+            for (int s = 0; s < CH; s++) {
+                const size_t sbi = (size_t)min(ch * CH + s, nsb - 1);
+                h[s] = u32x4{pl_d[sbi * pst + row], pl_sc[(3 * sbi) * pst + row], pl_sc[(3 * sbi + 1) * pst + row],
+                             pl_sc[(3 * sbi + 2) * pst + row]};
+#pragma unroll
+                for (int hh = 0; hh < 2; hh++) {
+                    const u32* b = pl_qs + ((sbi * 8 + 2 * kg + hh) * 4) * pst + row;
+                    q[s][hh] = u32x4{b[0], b[pst], b[2 * pst], b[3 * pst]};
+                }
+            }
+            return;
+        }
         const uint8_t* b = sheet + (size_t)row * p.row_bytes;
 #pragma unroll
         for (int s = 0; s < CH; s++) {
@@ -1041,7 +1068,11 @@ __device__ __forceinline__ void moe_g16_body(const MoeG16Args& p, uint8_t* smem)
                         const i32 a32 = sum16 + dpp_i32<JL_DPP_ROW_HALF_MIRROR, 0xf>(0, sum16);
                         // lane l holds word l of the super-block: sub-block l / 8 (group kg, low or
                         // high nibbles' partner), K-step l % 8; its bytes go to two f16 pairs
-                        const int sub = lane >> 3, ks = lane & 7, kg = sub >> 1, hi = sub & 1;
+                        // (planes: word l % 4 of sub-block l / 8, low nibbles' partner where
+                        // l % 8 < 4; K-step 4 (sub % 2) + l % 4 of group sub / 2)
+                        const int sub = lane >> 3;
+                        const int kg = sub >> 1, ks = PL ? 4 * (sub & 1) + (lane & 3) : lane & 7;
+                        const int hi = PL ? (lane >> 2) & 1 : sub & 1;
                         auto f = [](u32 x, int b2) { return (_Float16)(float)(int8_t)(x >> (8 * b2)); };
                         const f16x2 p02 = {f(q, 0), f(q, 2)}, p13 = {f(q, 1), f(q, 3)};
                         const int vec = sb * V + ks * 65 + 16 * kg + i;
@@ -1101,12 +1132,17 @@ __device__ __forceinline__ void moe_g16_body(const MoeG16Args& p, uint8_t* smem)
                 const int sb = ch * CH + s;
                 if (sb < nsb) {   // uniform
                     f32x4 accP;
-                    GemmWideScale sc;
-                    gemm_wide_scale(hd[cur][s], kg & 1, kg >> 1, sc);
+                    GemmWideScale sc, sc1;
+                    if (PL) {
+                        gemm_wide_scale_planes(hd[cur][s], 2 * kg, sc);
+                        gemm_wide_scale_planes(hd[cur][s], 2 * kg + 1, sc1);
+                    } else {
+                        gemm_wide_scale(hd[cur][s], kg & 1, kg >> 1, sc);
+                    }
 #pragma unroll
                     for (int ks = 0; ks < 8; ks++) {
                         const f16x8 af = __builtin_bit_cast(f16x8, sA4[sb * V + ks * 65 + lane]);
-                        const f16x8 b = moe_g16_word(wq[cur][s][ks >> 2][ks & 3], sc, mask_lo, mask_hi, magic);
+                        const f16x8 b = moe_g16_word(wq[cur][s][ks >> 2][ks & 3], PL && ks >= 4 ? sc1 : sc, mask_lo, mask_hi, magic);
                         const f32x4 czero = {0.f, 0.f, 0.f, 0.f};
                         accP = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, b, ks == 0 ? czero : accP, 0, 0, 0);
                     }
@@ -1116,12 +1152,17 @@ __device__ __forceinline__ void moe_g16_body(const MoeG16Args& p, uint8_t* smem)
                     const f16x8 aug = __builtin_bit_cast(f16x8, augw);
                     const f32x4 dav = *(const f32x4*)(sAf + (sb * V + 552) * 4 + 4 * kg);
                     const float mul = kg == 0 ? 1.0f : (kg == 1 ? 64.0f : 0.0f);
-                    const GemmScaleBytes sbytes = gemm_scale_bytes(hd[cur][s].y, hd[cur][s].z, hd[cur][s].w);
                     f16x8 mm;
+                    if (PL) {
 #pragma unroll
-                    for (int b = 0; b < 4; b++) {
-                        mm[b] = (_Float16)((float)((sbytes.mn_lo >> (8 * b)) & 0xFF) * mul);
-                        mm[4 + b] = (_Float16)((float)((sbytes.mn_hi >> (8 * b)) & 0xFF) * mul);
+                        for (int b = 0; b < 8; b++) mm[b] = (_Float16)((float)gemm_stream_field(hd[cur][s], 2 * b + 1) * mul);
+                    } else {
+                        const GemmScaleBytes sbytes = gemm_scale_bytes(hd[cur][s].y, hd[cur][s].z, hd[cur][s].w);
+#pragma unroll
+                        for (int b = 0; b < 4; b++) {
+                            mm[b] = (_Float16)((float)((sbytes.mn_lo >> (8 * b)) & 0xFF) * mul);
+                            mm[4 + b] = (_Float16)((float)((sbytes.mn_hi >> (8 * b)) & 0xFF) * mul);
+                        }
                     }
                     const f32x4 czero = {0.f, 0.f, 0.f, 0.f};
                     const f32x4 accM = __builtin_amdgcn_mfma_f32_16x16x32_f16(aug, mm, czero, 0, 0, 0);

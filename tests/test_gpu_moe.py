@@ -438,8 +438,10 @@ def test_grouped_matvec_over_packed_expert_sheets(dev, devbuf, layout, nrows, k)
     xd, dstart, dperm = devbuf(x), devbuf(start), devbuf(perm[:used].copy())
     o0 = devbuf(shape=(used * nrows + 8,), dtype=np.float32, fill=np.float32(4e30))
     o1 = devbuf(shape=(used * nrows + 8,), dtype=np.float32, fill=np.float32(4e30))
-    for form in (1, 0, 4):   # the dot-product form over planes (also the library's pick here), then the tile
-        dev.set_tuning(moe__form=form)
+    # the dot-product form over planes, the library's pick, groups of sixteen columns (columns from a
+    # prep kernel, then quantized by the matrix kernel itself), then the tile
+    for form in (1, 0, 3, 13, 4):
+        dev.set_tuning(moe__form=form % 10, moe__group16=2 if form == 13 else 1 if form == 3 else 0)
         o0.put(np.full(used * nrows + 8, 4e30, np.float32))
         o1.put(np.full(used * nrows + 8, 4e30, np.float32))
         assert dev.moe_matvec_packed_dev(o0.ptr, o1.ptr, t, pb0, pb1, xd.ptr, None, dperm.ptr, dstart.ptr, n_expert,
@@ -449,7 +451,7 @@ def test_grouped_matvec_over_packed_expert_sheets(dev, devbuf, layout, nrows, k)
         assert np.all(g0[used * nrows:] == np.float32(4e30)) and np.all(g1[used * nrows:] == np.float32(4e30))
         assert nmse(g0[:used * nrows].reshape(used, nrows), want0) <= 1e-10, form
         assert nmse(g1[:used * nrows].reshape(used, nrows), want1) <= 1e-10, form
-    dev.set_tuning(moe__form=0)
+    dev.set_tuning(moe__form=0, moe__group16=0)
     # the tile form over the same weights as GGUF banks: the same integers, the same epilogue
     b0, b1 = devbuf(bank0), devbuf(bank1)
     r0 = devbuf(shape=(used * nrows,), dtype=np.float32, fill=0)
