@@ -839,7 +839,7 @@ def main():
             "q6_k": gemm_section(dev, gate, {4096: (512, 2048)}, quant.Q6_K, 14336, 32)}
         line["moe_block"] = moe_section(dev, gate)
         line["moe_block_packed_planes"] = moe_section(dev, gate, packed=True)
-        line["moe_block_prefill_1024_rows"] = moe_section(dev, gate, 1024)   # matrix-core tiles per expert
+        line["moe_block_prefill_1024_rows"] = moe_section(dev, gate, 1024)   # groups of 32 columns per expert
         line["moe_decode"] = moe_decode_section(dev, gate)
         line["mxfp4_gemm"] = mxfp4_section(dev, gate)
 

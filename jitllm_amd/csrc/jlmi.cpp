@@ -963,31 +963,37 @@ int moe_matvec_launch(jl_ctx* c, float* out0, float* out1, int type, const void*
     // "moe.form" = 2: groups of 32 columns, a wavefront to itself; 3: groups of 16, the weights
     // decoded in registers, below; 4: the prefill GEMM's tile).  Their vector work does not grow
     // with the number of columns.  Measured at the 128-expert shape, top-8 (router + gate + up +
-    // down + combine, whole block, us; forms 1 / 2 / 3 / 4):
-    //   16 rows 73 / 155 / 90 / -      32 rows 107 / 193 / 102 / -     64 rows 133 / 210 / 112 / -
-    //   128 rows 191 / 223 / 129 / -   256 rows 333 / 237 / 193 / -    384 rows - / 248 / 257 / 328
-    //   512 rows - / 302 / 291 / 353   768 rows - / 364 / 413 / 377    1024 rows - / 424 / 495 / 399
-    // so form 3 takes over from two columns an expert on average, form 2 from 22 and form 4 from 56.
+    // down + combine, whole block, us; forms 1 / 2 / 3 with groups of 16 / 3 with groups of 32 / 4):
+    //   16 rows 73 / 155 / 85 / - / -       64 rows 133 / 210 / 110 / - / -     128 rows 191 / 223 / 130 / 137 / 302
+    //   192 rows - / 232 / 171 / 147 / 309  256 rows 333 / 238 / 187 / 157 / 315  512 rows - / 301 / 281 / 243 / 352
+    //   1024 rows - / 426 / 489 / 372 / 400 1280 rows - / 501 / 577 / 475 / 435   2048 rows - / 709 / 831 / 639 / 623
+    // so form 3 takes over from two columns an expert on average (groups of 32 from ten) and form 4
+    // from 72; form 2 is left to "moe.form" = 2.
     // Q6_K sheets (the down projections of a model whose other experts are Q4_K) have form 4
     // alone, with the Q6_K GEMM's tile; the dot-product kernel is slower for that type, so the
     // tile takes over earlier ("moe.q6k_cols": columns an expert on average, default 12).
     // Form 3: groups of sixteen columns on the 16 x 16 x 32 matrix instruction, the weights decoded
     // in registers straight into its operand (Q4_K GGUF sheets or packed planes, the k-quant window; the group's
     // fragments for the whole of K sit in LDS).  Its steady state runs at the rate of a plain read;
-    // the library picks it from two (over planes three) columns an expert on average up to 22, while the
+    // the library picks it from two (over planes three) columns an expert on average up to 72, while the
     // fragments take at most half a CU's LDS (K <= 2304); "moe.form" = 3 forces it wherever they fit.
     {
         const int nsb = k / 256;
-        const size_t lds16 = (size_t)nsb * JL_MOE_G16_LDS_WORDS * 4 + 16;   // the fragments, the tile counter
+        const size_t frag16 = (size_t)nsb * JL_MOE_G16_LDS_WORDS * 4;   // a token tile's fragments
+        const size_t lds16 = frag16 + 16;                               // and the tile counter
         const size_t nslots16 = (size_t)ncols / 16 + (size_t)n_expert + 1;
         const bool can16 = type == JL_TYPE_Q4_K && c->act_window == 256 && lds16 <= c->lds_limit &&
                            (size_t)nrows * row_bytes < ((size_t)1 << 32);
         const bool pick16 = c->tune.moe_form == 0 && 2 * lds16 <= c->lds_limit && (long)ncols >= (planes ? 3L : 2L) * n_expert &&
-                            (long)ncols < 22L * n_expert;
+                            (long)ncols < 72L * n_expert;
         if (can16 && (c->tune.moe_form == 3 || pick16)) {
             // up to eight columns an expert the matrix kernel quantizes them itself: no prep launch,
             // no workspace ("moe.group16" = 1 forces the prep kernel, 2 the fused form)
             const bool fused = c->tune.moe_g16 == 2 || (c->tune.moe_g16 == 0 && (long)ncols <= 8L * n_expert);
+            // from ten columns an expert groups of 32 (two token tiles, a decoded word meets both), so
+            // that an expert of 17-32 columns reads its sheet once ("moe.group16" = 3 forces them)
+            const bool two = !fused && 2 * frag16 + 16 <= c->lds_limit &&
+                             (c->tune.moe_g16 == 3 || (c->tune.moe_g16 == 0 && (long)ncols >= 10L * n_expert));
             MoeG16PrepArgs pa;
             pa.ws = nullptr;
             if (!fused) {
@@ -1020,7 +1026,7 @@ int moe_matvec_launch(jl_ctx* c, float* out0, float* out1, int type, const void*
             // anew).  Experts that can have a column: at most one a column.  "moe.waves" = 4: the
             // two-workgroup form.
             const int nmat = (planes ? pb1 != nullptr : bank1 != nullptr) ? 2 : 1, tiles = (nrows + 15) / 16;
-            const int nwaves = c->tune.moe_waves == 4 || (c->tune.moe_waves == 12 && !planes) ? c->tune.moe_waves : 8;
+            const int nwaves = !two && c->tune.moe_waves == 4 ? 4 : 8;
             const long wgs_cu = nwaves == 4 ? 2 : 1;
             const int sets = (tiles + nwaves - 1) / nwaves;
             const long n_act = std::min<long>(n_expert, ncols);
@@ -1045,9 +1051,9 @@ int moe_matvec_launch(jl_ctx* c, float* out0, float* out1, int type, const void*
             int ch = planes ? 1 : (nsb <= 3 ? nsb : 2);
             if (c->tune.moe_chunk >= 1 && c->tune.moe_chunk <= 3) ch = std::min(c->tune.moe_chunk, nsb);
             char name[32];
-            snprintf(name, sizeof name, "jl_moe_g16%s_%c%d", planes ? "p" : "", fused ? (x2 ? 'g' : 'f') : 'c', ch);
+            snprintf(name, sizeof name, "jl_moe_g16%s_%c%d", planes ? "p" : "", fused ? (x2 ? 'g' : 'f') : two ? 'd' : 'c', ch);
             void* gp[] = {&ga};
-            return launch(c, name, (unsigned)grid, 1, (unsigned)(64 * nwaves), (unsigned)lds16, st, gp);
+            return launch(c, name, (unsigned)grid, 1, (unsigned)(64 * nwaves), (unsigned)(two ? 2 * frag16 + 16 : lds16), st, gp);
         }
     }
     if (planes && c->tune.moe_form != 4 && (c->tune.moe_form == 1 || (long)ncols < kMoePlaneTileCols * n_expert)) {
@@ -1082,7 +1088,7 @@ int moe_matvec_launch(jl_ctx* c, float* out0, float* out1, int type, const void*
     }
     const bool q6 = type == JL_TYPE_Q6_K;
     const long q6_cols = c->tune.moe_q6k_cols > 0 ? c->tune.moe_q6k_cols : 12;
-    const bool many_cols = c->tune.moe_form == 0 && (long)ncols >= (q6 ? q6_cols : 10L) * n_expert;   // (Q4_K: 22 and more get here)
+    const bool many_cols = c->tune.moe_form == 0 && (long)ncols >= (q6 ? q6_cols : 10L) * n_expert;   // (Q4_K: 72 and more get here)
     if ((type == JL_TYPE_Q4_K || q6) && c->act_window == 256 &&
         (planes || c->tune.moe_form == 4 || many_cols || (!q6 && c->tune.moe_form == 2)) &&
         4u * 19968u <= c->lds_limit) {   // JL_MOEG_WAVE_LDS
@@ -1258,7 +1264,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     if (e != hipSuccess)
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
-    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_prep_q4k_planes", "jl_gemm_q4k_r64_planes", "jl_gemm_q4k_wide_planes", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_group2_wide", "jl_moe_quant", "jl_moe_matvec_planes_q4k", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_prep_planes", "jl_moe_gemm_q4k", "jl_moe_g16_prep", "jl_moe_g16_c1", "jl_moe_g16_c2", "jl_moe_g16_c3", "jl_moe_g16_f1", "jl_moe_g16_f2", "jl_moe_g16_f3", "jl_moe_g16_g1", "jl_moe_g16_g2", "jl_moe_g16_g3", "jl_moe_g16_prep_planes", "jl_moe_g16p_c1", "jl_moe_g16p_c2", "jl_moe_g16p_c3", "jl_moe_g16p_f1", "jl_moe_g16p_f2", "jl_moe_g16p_f3", "jl_moe_g16p_g1", "jl_moe_g16p_g2", "jl_moe_g16p_g3", "jl_moe_gemm_r64", "jl_moe_gemm_r64_planes", "jl_moe_gemm_q6k_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_mxfp4_matvec1_b1", "jl_mxfp4_matvec1_b2", "jl_mxfp4_matvec1_b3", "jl_mxfp4_scaled_prep", "jl_mxfp4_scaled_gemm", "jl_mxfp4_planes_prep", "jl_mxfp4_planes_gemm", "jl_mxfp4_matvec_planes_r64", "jl_mxfp4_matvec_planes_r32", "jl_mxfp4_matvec_planes_r16", "jl_unpack_mxfp4", "jl_sum_parts", "jl_probe_read", "jl_probe_empty", "jl_probe_wait", "jl_probe_mfma", "jl_probe_mfma_v5",
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_prep_q4k_planes", "jl_gemm_q4k_r64_planes", "jl_gemm_q4k_wide_planes", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_group2_wide", "jl_moe_quant", "jl_moe_matvec_planes_q4k", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_prep_planes", "jl_moe_gemm_q4k", "jl_moe_g16_prep", "jl_moe_g16_c1", "jl_moe_g16_c2", "jl_moe_g16_c3", "jl_moe_g16_f1", "jl_moe_g16_f2", "jl_moe_g16_f3", "jl_moe_g16_g1", "jl_moe_g16_g2", "jl_moe_g16_g3", "jl_moe_g16_prep_planes", "jl_moe_g16p_c1", "jl_moe_g16p_c2", "jl_moe_g16p_c3", "jl_moe_g16p_f1", "jl_moe_g16p_f2", "jl_moe_g16p_f3", "jl_moe_g16p_g1", "jl_moe_g16p_g2", "jl_moe_g16p_g3", "jl_moe_g16_d1", "jl_moe_g16_d2", "jl_moe_g16_d3", "jl_moe_g16p_d1", "jl_moe_g16p_d2", "jl_moe_g16p_d3", "jl_moe_gemm_r64", "jl_moe_gemm_r64_planes", "jl_moe_gemm_q6k_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_mxfp4_matvec1_b1", "jl_mxfp4_matvec1_b2", "jl_mxfp4_matvec1_b3", "jl_mxfp4_scaled_prep", "jl_mxfp4_scaled_gemm", "jl_mxfp4_planes_prep", "jl_mxfp4_planes_gemm", "jl_mxfp4_matvec_planes_r64", "jl_mxfp4_matvec_planes_r32", "jl_mxfp4_matvec_planes_r16", "jl_unpack_mxfp4", "jl_sum_parts", "jl_probe_read", "jl_probe_empty", "jl_probe_wait", "jl_probe_mfma", "jl_probe_mfma_v5",
                                       "jl_pack_weights", "jl_unpack_q4k", "jl_unpack_q6k", "jl_unpack_q8_0"};
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int rw : {16, 32, 64})

@@ -248,7 +248,7 @@ extern "C" __global__ __launch_bounds__(256) void jl_moe_gemm_prep_planes(MoeGem
 extern "C" __global__ __launch_bounds__(256, 2) void jl_moe_gemm_q4k(MoeGemmArgs p) { moe_gemm_q4k_body(p, jl_smem); }
 // Sixteen columns a group, weights from HBM straight into matrix operands.
 // prep: grid = (ceil(k/1024), ncols), block = 256; main (CH super-blocks a step): grid = 8 * ceil(n_expert/8) * row blocks * matrices,
-// block = 64 * nwaves (<= 768), dynamic LDS = (k/256) * JL_MOE_G16_SB_WORDS * 4
+// block = 64 * nwaves (<= 512), dynamic LDS = (k/256) * JL_MOE_G16_SB_WORDS * 4
 extern "C" __global__ __launch_bounds__(256) void jl_moe_g16_prep(MoeG16PrepArgs p) {
     __shared__ u32 lds[4 * 72];
     moe_g16_prep_body<false>(p, lds);
@@ -258,14 +258,16 @@ extern "C" __global__ __launch_bounds__(256) void jl_moe_g16_prep_planes(MoeG16P
     moe_g16_prep_body<true>(p, lds);
 }
 // _c: fragments from the prep kernel's workspace; _f / _g: the columns (plain / silu(x) * x2) quantized by
-// the kernel itself; g16p: the sheets are packed planes
+// the kernel itself; _d: groups of 32 columns (two token tiles); g16p: the sheets are packed planes
 #define JL_MOE_G16_KERNEL(CH)                                                                                           \
-    extern "C" __global__ __launch_bounds__(768) void jl_moe_g16_c##CH(MoeG16Args p) { moe_g16_body<CH, 0>(p, jl_smem); } \
-    extern "C" __global__ __launch_bounds__(768) void jl_moe_g16_f##CH(MoeG16Args p) { moe_g16_body<CH, 1>(p, jl_smem); } \
-    extern "C" __global__ __launch_bounds__(768) void jl_moe_g16_g##CH(MoeG16Args p) { moe_g16_body<CH, 2>(p, jl_smem); } \
+    extern "C" __global__ __launch_bounds__(512) void jl_moe_g16_c##CH(MoeG16Args p) { moe_g16_body<CH, 0>(p, jl_smem); } \
+    extern "C" __global__ __launch_bounds__(512) void jl_moe_g16_f##CH(MoeG16Args p) { moe_g16_body<CH, 1>(p, jl_smem); } \
+    extern "C" __global__ __launch_bounds__(512) void jl_moe_g16_g##CH(MoeG16Args p) { moe_g16_body<CH, 2>(p, jl_smem); } \
     extern "C" __global__ __launch_bounds__(512) void jl_moe_g16p_c##CH(MoeG16Args p) { moe_g16_body<CH, 0, true>(p, jl_smem); } \
     extern "C" __global__ __launch_bounds__(512) void jl_moe_g16p_f##CH(MoeG16Args p) { moe_g16_body<CH, 1, true>(p, jl_smem); } \
-    extern "C" __global__ __launch_bounds__(512) void jl_moe_g16p_g##CH(MoeG16Args p) { moe_g16_body<CH, 2, true>(p, jl_smem); }
+    extern "C" __global__ __launch_bounds__(512) void jl_moe_g16p_g##CH(MoeG16Args p) { moe_g16_body<CH, 2, true>(p, jl_smem); } \
+    extern "C" __global__ __launch_bounds__(512) void jl_moe_g16_d##CH(MoeG16Args p) { moe_g16_body<CH, 0, false, 2>(p, jl_smem); } \
+    extern "C" __global__ __launch_bounds__(512) void jl_moe_g16p_d##CH(MoeG16Args p) { moe_g16_body<CH, 0, true, 2>(p, jl_smem); }
 JL_MOE_G16_KERNEL(1) JL_MOE_G16_KERNEL(2) JL_MOE_G16_KERNEL(3)
 // Experts with many columns: the prefill GEMM's 128-token x 64-row tile placed per expert.  An
 // expert's column groups are consecutive slots of the prepared workspace, so to the tile they

@@ -944,8 +944,10 @@ __device__ __forceinline__ f16x8 moe_g16_word(u32 w, const GemmWideScale& k, u32
 // (a wavefront per (column, super-block), the prep kernel's arithmetic) straight into the LDS
 // fragments, behind the first weight loads.  Every workgroup of the expert repeats that, which
 // pays while an expert has a handful of columns: two launches less a call.  FUSED = 1: plain
-// columns, 2: silu(x) * x2.
-template <int CH, int FUSED, bool PL = false>
+// columns, 2: silu(x) * x2.  NT = 2: a group is 32 columns, two token tiles whose fragments sit
+// in LDS one behind the other (two workspace slots), and a decoded word meets both: an expert of
+// 17-32 columns reads its sheet once.
+template <int CH, int FUSED, bool PL = false, int NT = 1>
 __device__ __forceinline__ void moe_g16_body(const MoeG16Args& p, uint8_t* smem) {
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -968,7 +970,9 @@ __device__ __forceinline__ void moe_g16_body(const MoeG16Args& p, uint8_t* smem)
     asm volatile("" : "+v"(mask_lo), "+v"(mask_hi), "+v"(magic));
     u32x4* sA4 = (u32x4*)smem;
     const float* sAf = (const float*)smem;
-    u32* next_tile = (u32*)smem + (size_t)nsb * JL_MOE_G16_LDS_WORDS;   // behind the fragments
+    static_assert(NT == 1 || FUSED == 0, "two token tiles a group take their fragments from the prep kernel");
+    u32* next_tile = (u32*)smem + (size_t)NT * nsb * JL_MOE_G16_LDS_WORDS;   // behind the fragments
+    const int RV = nsb * (JL_MOE_G16_LDS_WORDS / 4);   // vectors of one token tile's fragments (NT = 2: two regions)
     float* outm = p.out[mat];
     // LDS vectors a super-block: eight fragments 65 vectors apart (64 used: a column's pieces, one
     // a fragment, then spread over sixteen banks when the fused form writes them), the sums' 32, the
@@ -1010,8 +1014,8 @@ __device__ __forceinline__ void moe_g16_body(const MoeG16Args& p, uint8_t* smem)
         }
     };
 
-    for (u32 c0 = c_lo; c0 < c_hi; c0 += 16) {
-        const int ncg = min(16, (int)(c_hi - c0));
+    for (u32 c0 = c_lo; c0 < c_hi; c0 += 16 * NT) {
+        const int ncg = min(16 * NT, (int)(c_hi - c0));
         const size_t slot = (size_t)(c_lo >> 4) + (size_t)e + ((c0 - c_lo) >> 4);
         // FUSED: the group's source rows, one a lane, and the first eight (column, super-block)
         // tasks of this wavefront requested ahead of the weights, which have the longer way and
@@ -1087,31 +1091,37 @@ __device__ __forceinline__ void moe_g16_body(const MoeG16Args& p, uint8_t* smem)
                 }
             }
         } else {
-            const u32x4* src = (const u32x4*)(p.ws + slot * nsb * JL_MOE_G16_SB_WORDS);
             // twelve loads in flight a thread (all of K = 2048 at 512 threads): the fill is one round
             // trip to L2, not one a vector
             constexpr int NB = 12;
             const int total = nsb * WS;
-            for (int base = tid; base < total; base += NB * nthreads) {
-                u32x4 val[NB];
 #pragma unroll
-                for (int u = 0; u < NB; u++) {
-                    const int idx = base + u * nthreads, o = idx % WS;
-                    // fragments: lane = o % 64, its column o % 16; sums: (o - 512) % 16; scales: all
-                    const bool have = idx < total && (o >= 544 || (o & 15) < ncg);
-                    val[u] = u32x4{0u, 0u, 0u, 0u};
-                    if (have) val[u] = src[idx];
-                }
+            for (int r = 0; r < NT; r++) {
+                const int ncr = min(16, max(0, ncg - 16 * r));   // columns of token tile r
+                const u32x4* src = (const u32x4*)(p.ws + (slot + r) * nsb * JL_MOE_G16_SB_WORDS);
+                for (int base = tid; base < total; base += NB * nthreads) {
+                    u32x4 val[NB];
 #pragma unroll
-                for (int u = 0; u < NB; u++) {
-                    const int idx = base + u * nthreads, sb = idx / WS, o = idx - sb * WS;
-                    if (idx < total) sA4[sb * V + (o < 512 ? o + (o >> 6) : o + 8)] = val[u];
+                    for (int u = 0; u < NB; u++) {
+                        const int idx = base + u * nthreads, o = idx % WS;
+                        // fragments: lane = o % 64, its column o % 16; sums: (o - 512) % 16; scales: all
+                        const bool have = idx < total && (o >= 544 ? ncr > 0 : (o & 15) < ncr);
+                        val[u] = u32x4{0u, 0u, 0u, 0u};
+                        if (have) val[u] = src[idx];
+                    }
+#pragma unroll
+                    for (int u = 0; u < NB; u++) {
+                        const int idx = base + u * nthreads, sb = idx / WS, o = idx - sb * WS;
+                        if (idx < total) sA4[r * RV + sb * V + (o < 512 ? o + (o >> 6) : o + 8)] = val[u];
+                    }
                 }
             }
         }
         __syncthreads();
         JL_MOE_TRACE(1);
-        f32x4 out = {0.f, 0.f, 0.f, 0.f};
+        f32x4 out[NT];
+#pragma unroll
+        for (int r = 0; r < NT; r++) out[r] = f32x4{0.f, 0.f, 0.f, 0.f};
         // Tiles are handed out as the wavefronts get to them (a counter in LDS): the SIMD issues
         // its oldest wavefront first, so with a fixed share each the young ones fall behind and
         // run the last tenth of the kernel alone.  A wavefront knows its next tile a tile ahead.
@@ -1131,7 +1141,7 @@ __device__ __forceinline__ void moe_g16_body(const MoeG16Args& p, uint8_t* smem)
             for (int s = 0; s < CH; s++) {
                 const int sb = ch * CH + s;
                 if (sb < nsb) {   // uniform
-                    f32x4 accP;
+                    f32x4 accP[NT];
                     GemmWideScale sc, sc1;
                     if (PL) {
                         gemm_wide_scale_planes(hd[cur][s], 2 * kg, sc);
@@ -1141,16 +1151,15 @@ __device__ __forceinline__ void moe_g16_body(const MoeG16Args& p, uint8_t* smem)
                     }
 #pragma unroll
                     for (int ks = 0; ks < 8; ks++) {
-                        const f16x8 af = __builtin_bit_cast(f16x8, sA4[sb * V + ks * 65 + lane]);
                         const f16x8 b = moe_g16_word(wq[cur][s][ks >> 2][ks & 3], PL && ks >= 4 ? sc1 : sc, mask_lo, mask_hi, magic);
                         const f32x4 czero = {0.f, 0.f, 0.f, 0.f};
-                        accP = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, b, ks == 0 ? czero : accP, 0, 0, 0);
+#pragma unroll
+                        for (int r = 0; r < NT; r++) {
+                            const f16x8 af = __builtin_bit_cast(f16x8, sA4[r * RV + sb * V + ks * 65 + lane]);
+                            accP[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, b, ks == 0 ? czero : accP[r], 0, 0, 0);
+                        }
                     }
                     // out += d_a * (d * P - dmin * M) for the super-block
-                    u32x4 augw = u32x4{0u, 0u, 0u, 0u};
-                    if (lane < 32) augw = sA4[sb * V + 520 + lane];
-                    const f16x8 aug = __builtin_bit_cast(f16x8, augw);
-                    const f32x4 dav = *(const f32x4*)(sAf + (sb * V + 552) * 4 + 4 * kg);
                     const float mul = kg == 0 ? 1.0f : (kg == 1 ? 64.0f : 0.0f);
                     f16x8 mm;
                     if (PL) {
@@ -1164,25 +1173,34 @@ __device__ __forceinline__ void moe_g16_body(const MoeG16Args& p, uint8_t* smem)
                             mm[4 + b] = (_Float16)((float)((sbytes.mn_hi >> (8 * b)) & 0xFF) * mul);
                         }
                     }
-                    const f32x4 czero = {0.f, 0.f, 0.f, 0.f};
-                    const f32x4 accM = __builtin_amdgcn_mfma_f32_16x16x32_f16(aug, mm, czero, 0, 0, 0);
                     const float dd = half_bits_to_f32((uint16_t)(hd[cur][s].x & 0xFFFF));
                     const float dmin = half_bits_to_f32((uint16_t)(hd[cur][s].x >> 16));
 #pragma unroll
-                    for (int el = 0; el < 4; el++) {
-                        const float uu = fmaf(dd, accP[el], -(dmin * accM[el]));
-                        out[el] = fmaf(dav[el], uu, out[el]);
+                    for (int r = 0; r < NT; r++) {
+                        u32x4 augw = u32x4{0u, 0u, 0u, 0u};
+                        if (lane < 32) augw = sA4[r * RV + sb * V + 520 + lane];
+                        const f16x8 aug = __builtin_bit_cast(f16x8, augw);
+                        const f32x4 dav = *(const f32x4*)(sAf + ((size_t)r * RV + sb * V + 552) * 4 + 4 * kg);
+                        const f32x4 czero = {0.f, 0.f, 0.f, 0.f};
+                        const f32x4 accM = __builtin_amdgcn_mfma_f32_16x16x32_f16(aug, mm, czero, 0, 0, 0);
+#pragma unroll
+                        for (int el = 0; el < 4; el++) {
+                            const float uu = fmaf(dd, accP[r][el], -(dmin * accM[el]));
+                            out[r][el] = fmaf(dav[el], uu, out[r][el]);
+                        }
                     }
                 }
             }
             if (last_ch) {   // the tile is done: store its 16 rows x ncg columns
                 const int r = 16 * (tile_base + ti) + j;
 #pragma unroll
-                for (int el = 0; el < 4; el++) {
-                    const int tok = 4 * kg + el;
-                    if (r < p.nrows && tok < ncg) outm[(size_t)(c0 + tok) * p.nrows + r] = out[el];
-                    out[el] = 0.f;
-                }
+                for (int tt = 0; tt < NT; tt++)
+#pragma unroll
+                    for (int el = 0; el < 4; el++) {
+                        const int tok = 16 * tt + 4 * kg + el;
+                        if (r < p.nrows && tok < ncg) outm[(size_t)(c0 + tok) * p.nrows + r] = out[tt][el];
+                        out[tt][el] = 0.f;
+                    }
             }
             if (last_ch) {
                 ti = ti_n;

@@ -114,8 +114,8 @@ def test_grouped_matvec_vs_oracle(dev, devbuf, t, nrows, k, form):
     o0 = devbuf(shape=(used, nrows), dtype=np.float32, fill=np.float32(4e30))
     o1 = devbuf(shape=(used, nrows), dtype=np.float32, fill=np.float32(4e30))
     # form 1: lanes per row -- the library's pick, then every other width; form 3: the columns
-    # quantized by a prep kernel (1) or by the matrix kernel itself (2)
-    for key, values in (("moe__group16", (1, 2)),) if form == 3 else (("moe__lpr", (0, 4, 16, 32, 64)),):
+    # quantized by a prep kernel (1), by the matrix kernel itself (2), groups of 32 columns (3)
+    for key, values in (("moe__group16", (1, 2, 3)),) if form == 3 else (("moe__lpr", (0, 4, 16, 32, 64)),):
         for v in values:
             dev.set_tuning(**{key: v})
             o0.put(np.full((used, nrows), 4e30, np.float32))
@@ -166,8 +166,9 @@ def test_grouped_matmul_more_than_one_group_of_columns(dev, devbuf, rows, t):
         q, a_s, _ = oracle.quantize_act(x[perm[c]], window)
         want[c] = oracle.matvec_q8act_f64(t, bank[e * sheet:(e + 1) * sheet], q, a_s, nrows, k)
     b, xd, dstart, dperm = devbuf(bank), devbuf(x), devbuf(start), devbuf(perm[:used].copy())
-    for form in ((1, 2, 3, 13, 4) if t == quant.Q4_K else (1, 4, 0)):   # 13: form 3, fused quantization
-        dev.set_tuning(moe__form=form % 10, moe__group16=2 if form == 13 else 1)
+    # 13: form 3, fused quantization; 23: form 3, groups of 32 columns
+    for form in ((1, 2, 3, 13, 23, 4) if t == quant.Q4_K else (1, 4, 0)):
+        dev.set_tuning(moe__form=form % 10, moe__group16={13: 2, 23: 3}.get(form, 1))
         o = devbuf(shape=(used * nrows + 8,), dtype=np.float32, fill=np.float32(4e30))
         assert dev.moe_matvec_dev(o.ptr, None, t, b.ptr, None, xd.ptr, None, dperm.ptr, dstart.ptr, n_expert, used,
                                   nrows, k)
@@ -201,8 +202,8 @@ def test_grouped_matmul_more_experts_than_one_work_list_round(dev, devbuf):
         q, a_s, _ = oracle.quantize_act(x[perm[c]], window)
         want[c] = oracle.matvec_q8act_f64(t, bank[e * sheet:(e + 1) * sheet], q, a_s, nrows, k)
     b, xd, dstart, dperm = devbuf(bank), devbuf(x), devbuf(start), devbuf(perm[:used].copy())
-    for form in (1, 2, 3, 13, 4):
-        dev.set_tuning(moe__form=form % 10, moe__group16=2 if form == 13 else 1)
+    for form in (1, 2, 3, 13, 23, 4):
+        dev.set_tuning(moe__form=form % 10, moe__group16={13: 2, 23: 3}.get(form, 1))
         o = devbuf(shape=(used, nrows), dtype=np.float32, fill=np.float32(4e30))
         assert dev.moe_matvec_dev(o.ptr, None, t, b.ptr, None, xd.ptr, None, dperm.ptr, dstart.ptr, n_expert, used,
                                   nrows, k)
@@ -440,8 +441,8 @@ def test_grouped_matvec_over_packed_expert_sheets(dev, devbuf, layout, nrows, k)
     o1 = devbuf(shape=(used * nrows + 8,), dtype=np.float32, fill=np.float32(4e30))
     # the dot-product form over planes, the library's pick, groups of sixteen columns (columns from a
     # prep kernel, then quantized by the matrix kernel itself), then the tile
-    for form in (1, 0, 3, 13, 4):
-        dev.set_tuning(moe__form=form % 10, moe__group16=2 if form == 13 else 1 if form == 3 else 0)
+    for form in (1, 0, 3, 13, 23, 4):
+        dev.set_tuning(moe__form=form % 10, moe__group16={3: 1, 13: 2, 23: 3}.get(form, 0))
         o0.put(np.full(used * nrows + 8, 4e30, np.float32))
         o1.put(np.full(used * nrows + 8, 4e30, np.float32))
         assert dev.moe_matvec_packed_dev(o0.ptr, o1.ptr, t, pb0, pb1, xd.ptr, None, dperm.ptr, dstart.ptr, n_expert,
