@@ -96,7 +96,8 @@ int jl_synchronize(jl_ctx *ctx);
  * packed-plane matvec: 16, 32, 64), "packed.block" (its threads per workgroup), "moe.shares"
  * (row shares an expert's matrix is split into), "moe.form" (grouped matmul: 1 dot products,
  * 2 / 3 groups of 32 / 16 columns on the matrix cores, 4 the prefill tile per expert),
- * "moe.group16" (form 3: 1 a prep kernel quantizes the columns, 2 the matrix kernel does),
+ * "moe.group16" (form 3: 1 a prep kernel quantizes the columns, 2 the matrix kernel does, 3 groups
+ * of 32 columns),
  * "moe.chunk" (form 3: super-blocks a step, 1-3),
  * "moe.group" / "moe.logits" / "moe.q6k_cols" / "moe.waves" / "moe.lpr" (forms of the mixture
  * block's other kernels),
