@@ -1000,10 +1000,9 @@ int moe_matvec_launch(jl_ctx* c, float* out0, float* out1, int type, const void*
                 rc = ws_ensure(c, &c->moe_q_ws, &c->moe_q_ws_bytes, nslots16 * nsb * JL_MOE_G16_SB_WORDS * 4);
                 if (rc != JL_OK) return rc;
                 pa.x = x; pa.x2 = x2; pa.src = src; pa.start = start; pa.ws = (uint32_t*)c->moe_q_ws;
-                pa.k = k; pa.n_expert = n_expert;
+                pa.k = k; pa.n_expert = n_expert; pa.ncols = ncols;
                 void* pp[] = {&pa};
-                rc = launch(c, planes ? "jl_moe_g16_prep_planes" : "jl_moe_g16_prep", (unsigned)((nsb + 3) / 4), (unsigned)ncols, 256, 0,
-                            st, pp);
+                rc = launch(c, planes ? "jl_moe_g16_prep_planes" : "jl_moe_g16_prep", (unsigned)((ncols + 3) / 4), 1, 256, 0, st, pp);
                 if (rc != JL_OK) return rc;
             }
             MoeG16Args ga;

@@ -132,7 +132,7 @@ struct MoeG16PrepArgs {
     const uint32_t* src;    // null: column c reads row c
     const uint32_t* start;  // [n_expert + 1]
     uint32_t* ws;
-    int k, n_expert;
+    int k, n_expert, ncols;
 };
 struct MoeG16Args {
     float* out[2];

@@ -247,7 +247,7 @@ extern "C" __global__ __launch_bounds__(256) void jl_moe_gemm_prep_planes(MoeGem
 }
 extern "C" __global__ __launch_bounds__(256, 2) void jl_moe_gemm_q4k(MoeGemmArgs p) { moe_gemm_q4k_body(p, jl_smem); }
 // Sixteen columns a group, weights from HBM straight into matrix operands.
-// prep: grid = (ceil(k/1024), ncols), block = 256; main (CH super-blocks a step): grid = 8 * ceil(n_expert/8) * row blocks * matrices,
+// prep: grid = ceil(ncols/4), block = 256; main (CH super-blocks a step): grid = 8 * ceil(n_expert/8) * row blocks * matrices,
 // block = 64 * nwaves (<= 512), dynamic LDS = (k/256) * JL_MOE_G16_SB_WORDS * 4
 extern "C" __global__ __launch_bounds__(256) void jl_moe_g16_prep(MoeG16PrepArgs p) {
     __shared__ u32 lds[4 * 72];

@@ -855,65 +855,88 @@ __device__ __forceinline__ void moe_gemm_q4k_body(const MoeGemmArgs& p, uint8_t*
 // words a super-block), filled once per (workgroup, group); columns the group does not have are
 // filled with zeros, so the workspace needs none.
 //
-// Prep: grid = (ceil(k/1024), ncols), block = 256: a wavefront quantizes one super-block of one
-// column (lane l owns elements 4l..4l+3), finds the column's expert by counting the experts
-// whose first column is not after it, and writes the 32 sixteen-byte pieces of the column's
-// fragments, the two pieces of its sub-block sums (low six bits, the rest) and its scale.
+// Prep: grid = ceil(ncols / 4), block = 256: a wavefront owns one column.  It finds the column's
+// expert by counting the experts whose first column is not after it (one load of start[] a lane,
+// ballots; the expert's first column is the largest start not after the column, a lane
+// reduction, not a second trip to memory), then quantizes the column's super-blocks four at a
+// time (lane l owns elements 4l..4l+3; the four loads go out together) and writes, per
+// super-block, the 32 sixteen-byte pieces of the column's fragments, the two pieces of its
+// sub-block sums (low six bits, the rest) and its scale.  (A wavefront a super-block, 65,536
+// short wavefronts at 1024 rows, was bound by their dependent loads: 36 us where this takes 20.)
 template <bool PL = false>
 __device__ __forceinline__ void moe_g16_prep_body(const MoeG16PrepArgs& p, u32* lds) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const u32 c = blockIdx.y;
-    const int nsb = p.k / 256, sb = blockIdx.x * 4 + wave;
-    if (sb >= nsb) return;   // whole wavefronts; no workgroup barrier below
+    const u32 c = blockIdx.x * 4 + wave;
+    if (c >= (u32)p.ncols) return;   // whole wavefronts; no workgroup barrier below
+    const int nsb = p.k / 256;
     const size_t row = p.src ? p.src[c] : c;
-    f32x4 v = ((const f32x4*)(p.x + row * (size_t)p.k + (size_t)sb * 256))[lane];
-    f32x4 u = f32x4{0.f, 0.f, 0.f, 0.f};
-    if (p.x2) u = ((const f32x4*)(p.x2 + row * (size_t)p.k + (size_t)sb * 256))[lane];
-    u32 cnt = 0;
+    u32 cnt = 0, c_lo = 0;
     for (int base = 0; base <= p.n_expert; base += 64) {
         const int idx = base + lane;
         const u32 s = idx <= p.n_expert ? p.start[idx] : 0xFFFFFFFFu;
-        cnt += (u32)__builtin_popcountll(__ballot(s <= c));
+        const bool le = s <= c;
+        cnt += (u32)__builtin_popcountll(__ballot(le));
+        c_lo = max(c_lo, le ? s : 0u);
     }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) c_lo = max(c_lo, (u32)__shfl_xor((int)c_lo, off, 64));
     const int e = (int)cnt - 1;
-    const u32 c_lo = p.start[e];
     const u32 rel = c - c_lo;
     const size_t slot = (size_t)(c_lo >> 4) + (size_t)e + (rel >> 4);
     const int i = (int)(rel & 15);
-    if (p.x2) v = f32x4{silu_f32(v.x) * u.x, silu_f32(v.y) * u.y, silu_f32(v.z) * u.z, silu_f32(v.w) * u.w};
-    const u32 m = max(max(abs_bits(v.x), abs_bits(v.y)), max(abs_bits(v.z), abs_bits(v.w)));
-    const u32 amax = wave_amax_256(m);
-    float d;
-    i32 sum16;
-    const u32 q = quantize4(v, amax, d, sum16);
-    const i32 a32 = sum16 + dpp_i32<JL_DPP_ROW_HALF_MIRROR, 0xf>(0, sum16);
     u32* sq = lds + wave * 72;   // the wavefront's own: 64 words of int8, 8 sub-block sums
-    sq[lane] = q;
-    if ((lane & 7) == 0) sq[64 + (lane >> 3)] = (u32)a32;
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // LDS operations of a wavefront execute in order
-    u32* blk = p.ws + (slot * nsb + sb) * JL_MOE_G16_SB_WORDS;
-    if (lane < 32) {
-        const int ks = lane >> 2, kg = lane & 3;
-        // GGUF sheets: word ks of group kg pairs elements 4 ks.. of sub-blocks 2 kg and 2 kg + 1;
-        // packed planes: K-step ks is word ks % 4 of sub-block 2 kg + ks / 4, whose low nibbles are
-        // elements 4 w.. and whose high nibbles elements 4 w + 16.. of that one sub-block
-        const int psub = 2 * kg + (ks >> 2), pw = ks & 3;
-        const u32 lo = PL ? sq[8 * psub + pw] : sq[16 * kg + ks];
-        const u32 hi = PL ? sq[8 * psub + 4 + pw] : sq[16 * kg + 8 + ks];
-        auto f = [](u32 w, int b) { return (_Float16)(float)(int8_t)(w >> (8 * b)); };
-        const f16x8 o = {f(lo, 0), f(lo, 2), f(hi, 0), f(hi, 2), f(lo, 1), f(lo, 3), f(hi, 1), f(hi, 3)};
-        ((u32x4*)blk)[ks * 64 + 16 * kg + i] = __builtin_bit_cast(u32x4, o);
-    } else if (lane < 34) {
-        const int kg = lane - 32;
-        f16x8 o;
+    const f32x4* xr = (const f32x4*)(p.x + row * (size_t)p.k);
+    const f32x4* ur = p.x2 ? (const f32x4*)(p.x2 + row * (size_t)p.k) : nullptr;
+    for (int sb0 = 0; sb0 < nsb; sb0 += 4) {
+        f32x4 vv[4], uu[4];
 #pragma unroll
-        for (int s8 = 0; s8 < 8; s8++) {
-            const i32 a = (i32)sq[64 + s8];
-            o[s8] = (_Float16)(float)(kg ? (a >> 6) : (a & 63));
+        for (int b = 0; b < 4; b++) {
+            const int sb = min(sb0 + b, nsb - 1);
+            vv[b] = xr[sb * 64 + lane];
+            uu[b] = f32x4{0.f, 0.f, 0.f, 0.f};
+            if (ur) uu[b] = ur[sb * 64 + lane];
         }
-        ((u32x4*)blk)[512 + 16 * kg + i] = __builtin_bit_cast(u32x4, o);
-    } else if (lane == 34) {
-        blk[2176 + i] = __float_as_uint(d);
+#pragma unroll
+        for (int b = 0; b < 4; b++) {
+            const int sb = sb0 + b;
+            if (sb >= nsb) break;   // uniform
+            f32x4 v = vv[b];
+            if (ur) v = f32x4{silu_f32(v.x) * uu[b].x, silu_f32(v.y) * uu[b].y, silu_f32(v.z) * uu[b].z, silu_f32(v.w) * uu[b].w};
+            const u32 m = max(max(abs_bits(v.x), abs_bits(v.y)), max(abs_bits(v.z), abs_bits(v.w)));
+            const u32 amax = wave_amax_256(m);
+            float d;
+            i32 sum16;
+            const u32 q = quantize4(v, amax, d, sum16);
+            const i32 a32 = sum16 + dpp_i32<JL_DPP_ROW_HALF_MIRROR, 0xf>(0, sum16);
+            sq[lane] = q;
+            if ((lane & 7) == 0) sq[64 + (lane >> 3)] = (u32)a32;
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // LDS operations of a wavefront execute in order
+            u32* blk = p.ws + (slot * nsb + sb) * JL_MOE_G16_SB_WORDS;
+            if (lane < 32) {
+                const int ks = lane >> 2, kg = lane & 3;
+                // GGUF sheets: word ks of group kg pairs elements 4 ks.. of sub-blocks 2 kg and 2 kg + 1;
+                // packed planes: K-step ks is word ks % 4 of sub-block 2 kg + ks / 4, whose low nibbles
+                // are elements 4 w.. and whose high nibbles elements 4 w + 16.. of that one sub-block
+                const int psub = 2 * kg + (ks >> 2), pw = ks & 3;
+                const u32 lo = PL ? sq[8 * psub + pw] : sq[16 * kg + ks];
+                const u32 hi = PL ? sq[8 * psub + 4 + pw] : sq[16 * kg + 8 + ks];
+                auto f = [](u32 w, int b2) { return (_Float16)(float)(int8_t)(w >> (8 * b2)); };
+                const f16x8 o = {f(lo, 0), f(lo, 2), f(hi, 0), f(hi, 2), f(lo, 1), f(lo, 3), f(hi, 1), f(hi, 3)};
+                ((u32x4*)blk)[ks * 64 + 16 * kg + i] = __builtin_bit_cast(u32x4, o);
+            } else if (lane < 34) {
+                const int kg = lane - 32;
+                f16x8 o;
+#pragma unroll
+                for (int s8 = 0; s8 < 8; s8++) {
+                    const i32 a = (i32)sq[64 + s8];
+                    o[s8] = (_Float16)(float)(kg ? (a >> 6) : (a & 63));
+                }
+                ((u32x4*)blk)[512 + 16 * kg + i] = __builtin_bit_cast(u32x4, o);
+            } else if (lane == 34) {
+                blk[2176 + i] = __float_as_uint(d);
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the reads above, before the next task's writes
+        }
     }
 }
 
