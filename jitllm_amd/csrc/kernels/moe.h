@@ -862,7 +862,7 @@ __device__ __forceinline__ void moe_gemm_q4k_body(const MoeGemmArgs& p, uint8_t*
 // time (lane l owns elements 4l..4l+3; the four loads go out together) and writes, per
 // super-block, the 32 sixteen-byte pieces of the column's fragments, the two pieces of its
 // sub-block sums (low six bits, the rest) and its scale.  (A wavefront a super-block, 65,536
-// short wavefronts at 1024 rows, was bound by their dependent loads: 36 us where this takes 20.)
+// short wavefronts at 1024 rows, was bound by their dependent loads: 36 us where this takes 26.)
 template <bool PL = false>
 __device__ __forceinline__ void moe_g16_prep_body(const MoeG16PrepArgs& p, u32* lds) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
