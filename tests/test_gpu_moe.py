@@ -142,6 +142,42 @@ def test_grouped_matvec_vs_oracle(dev, devbuf, t, nrows, k, form):
     dev.set_tuning(moe__form=0)
 
 
+@pytest.mark.parametrize("nrows,k", [(100, 2048), (2048 + 24, 768), (48, 1280)])
+def test_sixteen_column_groups_launch_shapes(dev, devbuf, nrows, k):
+    """Form 3 under every launch shape its tuning keys reach: one to three super-blocks a step (K = 1280
+    has five: a ragged last chunk), workgroups of four wavefronts, more row blocks than the library
+    would take, every way of preparing the columns; ragged row counts; an expert with 19 columns."""
+    t, window, rows, n_expert, k_used = quant.Q4_K, 256, 21, 5, 2
+    dev.SetActWindow(window)
+    sel = np.zeros((rows, k_used + 1), np.uint32)
+    sel[:, 0], sel[:, 1] = 3, 1
+    sel[:2, 0], sel[19:, 1] = 0, 4
+    used, perm, col_e, pos = oracle.group_pairs(sel.reshape(-1), rows, k_used, n_expert, 1)
+    start = np.searchsorted(col_e[:used], np.arange(n_expert + 1)).astype(np.uint32)
+    bank = _banks(t, n_expert, nrows, k, 31, True)
+    x = np.stack([synth.activations(k, seed=700 + r) * np.float32(1 + r % 3) for r in range(rows)])
+    sheet = nrows * quant.row_bytes(t, k)
+    want = np.zeros((used, nrows))
+    for c in range(used):
+        e = int(col_e[c])
+        q, a_s, _ = oracle.quantize_act(x[perm[c]], window)
+        want[c] = oracle.matvec_q8act_f64(t, bank[e * sheet:(e + 1) * sheet], q, a_s, nrows, k)
+    b, xd, dstart, dperm = devbuf(bank), devbuf(x), devbuf(start), devbuf(perm[:used].copy())
+    dev.set_tuning(moe__form=3)
+    for g16 in (1, 2, 3):
+        for chunk, waves, shares in ((1, 0, 0), (2, 0, 0), (3, 0, 0), (0, 4, 0), (0, 0, 3), (2, 4, 5)):
+            dev.set_tuning(moe__group16=g16, moe__chunk=chunk, moe__waves=waves, moe__shares=shares)
+            o = devbuf(shape=(used * nrows + 8,), dtype=np.float32, fill=np.float32(4e30))
+            assert dev.moe_matvec_dev(o.ptr, None, t, b.ptr, None, xd.ptr, None, dperm.ptr, dstart.ptr, n_expert,
+                                      used, nrows, k)
+            dev.synchronize()
+            got = o.get()
+            assert np.all(got[used * nrows:] == np.float32(4e30))
+            assert nmse(got[:used * nrows].reshape(used, nrows), want) <= 1e-10, (g16, chunk, waves, shares)
+    dev.set_tuning(moe__form=0, moe__group16=0, moe__chunk=0, moe__waves=0, moe__shares=0)
+    dev.SetActWindow(32)
+
+
 @pytest.mark.parametrize("t", [quant.Q4_K, quant.Q6_K], ids=["q4_k", "q6_k"])
 @pytest.mark.parametrize("rows", [70, 150])
 def test_grouped_matmul_more_than_one_group_of_columns(dev, devbuf, rows, t):
