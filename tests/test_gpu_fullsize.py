@@ -130,7 +130,7 @@ GEMMS = [(512, 4096), (512, 14336), (2048, 4096), (2048, 14336)]
 
 @pytest.mark.parametrize("shape", GEMMS, ids=lambda s: f"{s[0]}x4096->{s[1]}")
 def test_prefill_gemm_full_size(dev, devbuf, shape):
-    """BASELINE configuration 3 at its real sizes: the library's own choice of form, then the
+    """The Q4_K prefill GEMM (512 and 2048 tokens x 4096 -> 4096 and 14336) at its real sizes: the library's own choice of form, then the
     256 x 128 and the 128 x 64 tiles forced.  Sampled rows x all tokens against the oracle;
     a few tokens whole against the decode matvec; the forms bit for bit against each other."""
     ntok, nrows = shape
