@@ -973,7 +973,7 @@ int moe_matvec_launch(jl_ctx* c, float* out0, float* out1, int type, const void*
     // alone, with the Q6_K GEMM's tile; the dot-product kernel is slower for that type, so the
     // tile takes over earlier ("moe.q6k_cols": columns an expert on average, default 12).
     // Form 3: groups of sixteen columns on the 16 x 16 x 32 matrix instruction, the weights decoded
-    // in registers straight into its operand (Q4_K GGUF sheets or packed planes, the k-quant window; the group's
+    // in registers straight into its operand (Q4_K GGUF sheets or packed planes, Q6_K GGUF sheets, the k-quant window; the group's
     // fragments for the whole of K sit in LDS).  Its steady state runs at the rate of a plain read;
     // the library picks it from two (over planes three) columns an expert on average up to 72, while the
     // fragments take at most half a CU's LDS (K <= 2304); "moe.form" = 3 forces it wherever they fit.
@@ -982,18 +982,24 @@ int moe_matvec_launch(jl_ctx* c, float* out0, float* out1, int type, const void*
         const size_t frag16 = (size_t)nsb * JL_MOE_G16_LDS_WORDS * 4;   // a token tile's fragments
         const size_t lds16 = frag16 + 16;                               // and the tile counter
         const size_t nslots16 = (size_t)ncols / 16 + (size_t)n_expert + 1;
-        const bool can16 = type == JL_TYPE_Q4_K && c->act_window == 256 && lds16 <= c->lds_limit &&
+        const bool q6k = type == JL_TYPE_Q6_K;   // (GGUF sheets only: plane sheets are Q4_K)
+        const bool can16 = (type == JL_TYPE_Q4_K || (q6k && !planes)) && c->act_window == 256 && lds16 <= c->lds_limit &&
                            (size_t)nrows * row_bytes < ((size_t)1 << 32);
-        const bool pick16 = c->tune.moe_form == 0 && 2 * lds16 <= c->lds_limit && (long)ncols >= (planes ? 3L : 2L) * n_expert &&
-                            (long)ncols < 72L * n_expert;
+        // (Q6_K sheets: the decode is 4.5 vector instructions a weight, two matrix instructions a K-step,
+        // and the kernel is bound by them: 62 us for the 2048 x 768 down projections of 128 experts at 64
+        // rows where the dot-product kernel takes 58; with two token tiles a decoded word it costs the
+        // same, so it is picked from six columns an expert, always in groups of 32: 128 rows 68 us against
+        // 97, 256 rows 71 against 139 for the tile, 1024 rows 193 against 195)
+        const bool pick16 = c->tune.moe_form == 0 && 2 * lds16 <= c->lds_limit &&
+                            (long)ncols >= (q6k ? 6L : planes ? 3L : 2L) * n_expert && (long)ncols < (q6k ? 64L : 72L) * n_expert;
         if (can16 && (c->tune.moe_form == 3 || pick16)) {
             // up to eight columns an expert the matrix kernel quantizes them itself: no prep launch,
             // no workspace ("moe.group16" = 1 forces the prep kernel, 2 the fused form)
-            const bool fused = c->tune.moe_g16 == 2 || (c->tune.moe_g16 == 0 && (long)ncols <= 8L * n_expert);
+            const bool fused = c->tune.moe_g16 == 2 || (c->tune.moe_g16 == 0 && !q6k && (long)ncols <= 8L * n_expert);
             // from ten columns an expert groups of 32 (two token tiles, a decoded word meets both), so
             // that an expert of 17-32 columns reads its sheet once ("moe.group16" = 3 forces them)
             const bool two = !fused && 2 * frag16 + 16 <= c->lds_limit &&
-                             (c->tune.moe_g16 == 3 || (c->tune.moe_g16 == 0 && (long)ncols >= 10L * n_expert));
+                             (c->tune.moe_g16 == 3 || (c->tune.moe_g16 == 0 && (q6k || (long)ncols >= 10L * n_expert)));
             MoeG16PrepArgs pa;
             pa.ws = nullptr;
             if (!fused) {
@@ -1002,7 +1008,8 @@ int moe_matvec_launch(jl_ctx* c, float* out0, float* out1, int type, const void*
                 pa.x = x; pa.x2 = x2; pa.src = src; pa.start = start; pa.ws = (uint32_t*)c->moe_q_ws;
                 pa.k = k; pa.n_expert = n_expert; pa.ncols = ncols;
                 void* pp[] = {&pa};
-                rc = launch(c, planes ? "jl_moe_g16_prep_planes" : "jl_moe_g16_prep", (unsigned)((ncols + 3) / 4), 1, 256, 0, st, pp);
+                rc = launch(c, planes ? "jl_moe_g16_prep_planes" : q6k ? "jl_moe_g16_prep_q6k" : "jl_moe_g16_prep", (unsigned)((ncols + 3) / 4), 1,
+                            256, 0, st, pp);
                 if (rc != JL_OK) return rc;
             }
             MoeG16Args ga;
@@ -1050,7 +1057,7 @@ int moe_matvec_launch(jl_ctx* c, float* out0, float* out1, int type, const void*
             int ch = planes ? 1 : (nsb <= 3 ? nsb : 2);
             if (c->tune.moe_chunk >= 1 && c->tune.moe_chunk <= 3) ch = std::min(c->tune.moe_chunk, nsb);
             char name[32];
-            snprintf(name, sizeof name, "jl_moe_g16%s_%c%d", planes ? "p" : "", fused ? (x2 ? 'g' : 'f') : two ? 'd' : 'c', ch);
+            snprintf(name, sizeof name, "jl_moe_g16%s_%c%d", planes ? "p" : q6k ? "q6" : "", fused ? (x2 ? 'g' : 'f') : two ? 'd' : 'c', ch);
             void* gp[] = {&ga};
             return launch(c, name, (unsigned)grid, 1, (unsigned)(64 * nwaves), (unsigned)(two ? 2 * frag16 + 16 : lds16), st, gp);
         }
@@ -1263,7 +1270,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     if (e != hipSuccess)
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
-    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_prep_q4k_planes", "jl_gemm_q4k_r64_planes", "jl_gemm_q4k_wide_planes", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_group2_wide", "jl_moe_quant", "jl_moe_matvec_planes_q4k", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_prep_planes", "jl_moe_gemm_q4k", "jl_moe_g16_prep", "jl_moe_g16_c1", "jl_moe_g16_c2", "jl_moe_g16_c3", "jl_moe_g16_f1", "jl_moe_g16_f2", "jl_moe_g16_f3", "jl_moe_g16_g1", "jl_moe_g16_g2", "jl_moe_g16_g3", "jl_moe_g16_prep_planes", "jl_moe_g16p_c1", "jl_moe_g16p_c2", "jl_moe_g16p_c3", "jl_moe_g16p_f1", "jl_moe_g16p_f2", "jl_moe_g16p_f3", "jl_moe_g16p_g1", "jl_moe_g16p_g2", "jl_moe_g16p_g3", "jl_moe_g16_d1", "jl_moe_g16_d2", "jl_moe_g16_d3", "jl_moe_g16p_d1", "jl_moe_g16p_d2", "jl_moe_g16p_d3", "jl_moe_gemm_r64", "jl_moe_gemm_r64_planes", "jl_moe_gemm_q6k_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_mxfp4_matvec1_b1", "jl_mxfp4_matvec1_b2", "jl_mxfp4_matvec1_b3", "jl_mxfp4_scaled_prep", "jl_mxfp4_scaled_gemm", "jl_mxfp4_planes_prep", "jl_mxfp4_planes_gemm", "jl_mxfp4_matvec_planes_r64", "jl_mxfp4_matvec_planes_r32", "jl_mxfp4_matvec_planes_r16", "jl_unpack_mxfp4", "jl_sum_parts", "jl_probe_read", "jl_probe_empty", "jl_probe_wait", "jl_probe_mfma", "jl_probe_mfma_v5",
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_prep_q4k_planes", "jl_gemm_q4k_r64_planes", "jl_gemm_q4k_wide_planes", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_group2_wide", "jl_moe_quant", "jl_moe_matvec_planes_q4k", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_prep_planes", "jl_moe_gemm_q4k", "jl_moe_g16_prep", "jl_moe_g16_prep_planes", "jl_moe_g16_prep_q6k", "jl_moe_g16_c1", "jl_moe_g16_c2", "jl_moe_g16_c3", "jl_moe_g16_f1", "jl_moe_g16_f2", "jl_moe_g16_f3", "jl_moe_g16_g1", "jl_moe_g16_g2", "jl_moe_g16_g3", "jl_moe_g16_d1", "jl_moe_g16_d2", "jl_moe_g16_d3", "jl_moe_g16p_c1", "jl_moe_g16p_c2", "jl_moe_g16p_c3", "jl_moe_g16p_f1", "jl_moe_g16p_f2", "jl_moe_g16p_f3", "jl_moe_g16p_g1", "jl_moe_g16p_g2", "jl_moe_g16p_g3", "jl_moe_g16p_d1", "jl_moe_g16p_d2", "jl_moe_g16p_d3", "jl_moe_g16q6_c1", "jl_moe_g16q6_c2", "jl_moe_g16q6_c3", "jl_moe_g16q6_f1", "jl_moe_g16q6_f2", "jl_moe_g16q6_f3", "jl_moe_g16q6_g1", "jl_moe_g16q6_g2", "jl_moe_g16q6_g3", "jl_moe_g16q6_d1", "jl_moe_g16q6_d2", "jl_moe_g16q6_d3", "jl_moe_gemm_r64", "jl_moe_gemm_r64_planes", "jl_moe_gemm_q6k_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_mxfp4_matvec1_b1", "jl_mxfp4_matvec1_b2", "jl_mxfp4_matvec1_b3", "jl_mxfp4_scaled_prep", "jl_mxfp4_scaled_gemm", "jl_mxfp4_planes_prep", "jl_mxfp4_planes_gemm", "jl_mxfp4_matvec_planes_r64", "jl_mxfp4_matvec_planes_r32", "jl_mxfp4_matvec_planes_r16", "jl_unpack_mxfp4", "jl_sum_parts", "jl_probe_read", "jl_probe_empty", "jl_probe_wait", "jl_probe_mfma", "jl_probe_mfma_v5",
                                       "jl_pack_weights", "jl_unpack_q4k", "jl_unpack_q6k", "jl_unpack_q8_0"};
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int rw : {16, 32, 64})

@@ -251,23 +251,24 @@ extern "C" __global__ __launch_bounds__(256, 2) void jl_moe_gemm_q4k(MoeGemmArgs
 // block = 64 * nwaves (<= 512), dynamic LDS = (k/256) * JL_MOE_G16_SB_WORDS * 4
 extern "C" __global__ __launch_bounds__(256) void jl_moe_g16_prep(MoeG16PrepArgs p) {
     __shared__ u32 lds[4 * 72];
-    moe_g16_prep_body<false>(p, lds);
+    moe_g16_prep_body<0>(p, lds);
 }
 extern "C" __global__ __launch_bounds__(256) void jl_moe_g16_prep_planes(MoeG16PrepArgs p) {
     __shared__ u32 lds[4 * 72];
-    moe_g16_prep_body<true>(p, lds);
+    moe_g16_prep_body<1>(p, lds);
+}
+extern "C" __global__ __launch_bounds__(256) void jl_moe_g16_prep_q6k(MoeG16PrepArgs p) {
+    __shared__ u32 lds[4 * 72];
+    moe_g16_prep_body<2>(p, lds);
 }
 // _c: fragments from the prep kernel's workspace; _f / _g: the columns (plain / silu(x) * x2) quantized by
-// the kernel itself; _d: groups of 32 columns (two token tiles); g16p: the sheets are packed planes
-#define JL_MOE_G16_KERNEL(CH)                                                                                           \
-    extern "C" __global__ __launch_bounds__(512) void jl_moe_g16_c##CH(MoeG16Args p) { moe_g16_body<CH, 0>(p, jl_smem); } \
-    extern "C" __global__ __launch_bounds__(512) void jl_moe_g16_f##CH(MoeG16Args p) { moe_g16_body<CH, 1>(p, jl_smem); } \
-    extern "C" __global__ __launch_bounds__(512) void jl_moe_g16_g##CH(MoeG16Args p) { moe_g16_body<CH, 2>(p, jl_smem); } \
-    extern "C" __global__ __launch_bounds__(512) void jl_moe_g16p_c##CH(MoeG16Args p) { moe_g16_body<CH, 0, true>(p, jl_smem); } \
-    extern "C" __global__ __launch_bounds__(512) void jl_moe_g16p_f##CH(MoeG16Args p) { moe_g16_body<CH, 1, true>(p, jl_smem); } \
-    extern "C" __global__ __launch_bounds__(512) void jl_moe_g16p_g##CH(MoeG16Args p) { moe_g16_body<CH, 2, true>(p, jl_smem); } \
-    extern "C" __global__ __launch_bounds__(512) void jl_moe_g16_d##CH(MoeG16Args p) { moe_g16_body<CH, 0, false, 2>(p, jl_smem); } \
-    extern "C" __global__ __launch_bounds__(512) void jl_moe_g16p_d##CH(MoeG16Args p) { moe_g16_body<CH, 0, true, 2>(p, jl_smem); }
+// the kernel itself; _d: groups of 32 columns (two token tiles); g16p: the sheets are packed planes; g16q6: Q6_K rows
+#define JL_MOE_G16_FORMS(NAME, KO, CH)                                                                                          \
+    extern "C" __global__ __launch_bounds__(512) void jl_moe_##NAME##_c##CH(MoeG16Args p) { moe_g16_body<CH, 0, KO>(p, jl_smem); } \
+    extern "C" __global__ __launch_bounds__(512) void jl_moe_##NAME##_f##CH(MoeG16Args p) { moe_g16_body<CH, 1, KO>(p, jl_smem); } \
+    extern "C" __global__ __launch_bounds__(512) void jl_moe_##NAME##_g##CH(MoeG16Args p) { moe_g16_body<CH, 2, KO>(p, jl_smem); } \
+    extern "C" __global__ __launch_bounds__(512) void jl_moe_##NAME##_d##CH(MoeG16Args p) { moe_g16_body<CH, 0, KO, 2>(p, jl_smem); }
+#define JL_MOE_G16_KERNEL(CH) JL_MOE_G16_FORMS(g16, 0, CH) JL_MOE_G16_FORMS(g16p, 1, CH) JL_MOE_G16_FORMS(g16q6, 2, CH)
 JL_MOE_G16_KERNEL(1) JL_MOE_G16_KERNEL(2) JL_MOE_G16_KERNEL(3)
 // Experts with many columns: the prefill GEMM's 128-token x 64-row tile placed per expert.  An
 // expert's column groups are consecutive slots of the prepared workspace, so to the tile they

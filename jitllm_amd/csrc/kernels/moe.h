@@ -863,7 +863,8 @@ __device__ __forceinline__ void moe_gemm_q4k_body(const MoeGemmArgs& p, uint8_t*
 // super-block, the 32 sixteen-byte pieces of the column's fragments, the two pieces of its
 // sub-block sums (low six bits, the rest) and its scale.  (A wavefront a super-block, 65,536
 // short wavefronts at 1024 rows, was bound by their dependent loads: 36 us where this takes 26.)
-template <bool PL = false>
+// KO: the K order of the matrix kernel's weights: 0 Q4_K GGUF rows, 1 Q4_K packed planes, 2 Q6_K GGUF rows
+template <int KO = 0>
 __device__ __forceinline__ void moe_g16_prep_body(const MoeG16PrepArgs& p, u32* lds) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const u32 c = blockIdx.x * 4 + wave;
@@ -917,9 +918,12 @@ __device__ __forceinline__ void moe_g16_prep_body(const MoeG16PrepArgs& p, u32* 
                 // GGUF sheets: word ks of group kg pairs elements 4 ks.. of sub-blocks 2 kg and 2 kg + 1;
                 // packed planes: K-step ks is word ks % 4 of sub-block 2 kg + ks / 4, whose low nibbles
                 // are elements 4 w.. and whose high nibbles elements 4 w + 16.. of that one sub-block
+                // Q6_K rows: lane group kg = (half n, half-run c), K-step ks = (nibble hh, word w): the
+                // word of the run of elements 128 n + 64 hh + 16 c + 4 w.. and of the run 32 further on
                 const int psub = 2 * kg + (ks >> 2), pw = ks & 3;
-                const u32 lo = PL ? sq[8 * psub + pw] : sq[16 * kg + ks];
-                const u32 hi = PL ? sq[8 * psub + 4 + pw] : sq[16 * kg + 8 + ks];
+                const int q6 = 32 * (kg >> 1) + 16 * (ks >> 2) + 4 * (kg & 1) + (ks & 3);
+                const u32 lo = KO == 2 ? sq[q6] : KO == 1 ? sq[8 * psub + pw] : sq[16 * kg + ks];
+                const u32 hi = KO == 2 ? sq[q6 + 8] : KO == 1 ? sq[8 * psub + 4 + pw] : sq[16 * kg + 8 + ks];
                 auto f = [](u32 w, int b2) { return (_Float16)(float)(int8_t)(w >> (8 * b2)); };
                 const f16x8 o = {f(lo, 0), f(lo, 2), f(hi, 0), f(hi, 2), f(lo, 1), f(lo, 3), f(hi, 1), f(hi, 3)};
                 ((u32x4*)blk)[ks * 64 + 16 * kg + i] = __builtin_bit_cast(u32x4, o);
@@ -970,7 +974,7 @@ __device__ __forceinline__ f16x8 moe_g16_word(u32 w, const GemmWideScale& k, u32
 // columns, 2: silu(x) * x2.  NT = 2: a group is 32 columns, two token tiles whose fragments sit
 // in LDS one behind the other (two workspace slots), and a decoded word meets both: an expert of
 // 17-32 columns reads its sheet once.
-template <int CH, int FUSED, bool PL = false, int NT = 1>
+template <int CH, int FUSED, int KO = 0, int NT = 1>
 __device__ __forceinline__ void moe_g16_body(const MoeG16Args& p, uint8_t* smem) {
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -988,6 +992,7 @@ __device__ __forceinline__ void moe_g16_body(const MoeG16Args& p, uint8_t* smem)
     const int tile_base = blk * p.tiles_wg;
     const int ntw = min(tiles, tile_base + p.tiles_wg) - tile_base;   // tiles of this workgroup
     const int j = lane & 15, kg = lane >> 4;
+    constexpr bool PL = KO == 1, Q6 = KO == 2;
     const uint8_t* sheet = PL ? nullptr : p.bank[mat] + (size_t)e * p.sheet_bytes;
     u32 mask_lo = 0x000F000Fu, mask_hi = 0x00F000F0u, magic = 0x64006400u;
     asm volatile("" : "+v"(mask_lo), "+v"(mask_hi), "+v"(magic));
@@ -1002,7 +1007,10 @@ __device__ __forceinline__ void moe_g16_body(const MoeG16Args& p, uint8_t* smem)
     // scales' 4; WS: vectors a super-block of the prep kernel's workspace
     constexpr int V = JL_MOE_G16_LDS_WORDS / 4, WS = JL_MOE_G16_SB_WORDS / 4;
 
-    u32x4 hd[2][CH], wq[2][CH][2];
+    // a step's registers: header and two vectors of nibbles a super-block (Q6_K: the scales' eight
+    // bytes and d in the header, the two runs' low nibbles, and a third vector of high bits)
+    constexpr int NQ = Q6 ? 3 : 2;
+    u32x4 hd[2][CH], wq[2][CH][NQ];
     // step (tile ti of the workgroup's range, chunk ch) into a register set
     // PL (packed planes): the header is the row's (d, dmin) word and its three words of 6-bit fields,
     // the lane's eight words are sub-blocks 2 kg and 2 kg + 1 (four words each); every load
@@ -1011,8 +1019,23 @@ __device__ __forceinline__ void moe_g16_body(const MoeG16Args& p, uint8_t* smem)
     const u32* pl_qs = PL ? p.pqs[mat] + (size_t)e * p.sheet_words + (size_t)e * p.row_step : nullptr;
     const u32* pl_d = PL ? p.pd[mat] + (size_t)e * p.sheet_words + (size_t)e * p.row_step : nullptr;
     const u32* pl_sc = PL ? p.psc[mat] + (size_t)e * p.sheet_words + (size_t)e * p.row_step : nullptr;
-    auto load_step = [&](int ti, int ch, u32x4 (&h)[CH], u32x4 (&q)[CH][2]) {
+    auto load_step = [&](int ti, int ch, u32x4 (&h)[CH], u32x4 (&q)[CH][NQ]) {
         const int row = min(16 * (tile_base + ti) + j, p.nrows - 1);
+        if (Q6) {
+            // lane (j, kg): half n = kg / 2 of the super-block, half-run c = kg % 2: sixteen bytes of each
+            // run's nibbles and of the high bits, the half's eight scales, d
+            const uint8_t* b = sheet + (size_t)row * p.row_bytes;
+            const int n = kg >> 1, c = kg & 1;
+#pragma unroll
+            for (int s = 0; s < CH; s++) {
+                const uint8_t* bs = b + (size_t)min(ch * CH + s, nsb - 1) * 210;
+                q[s][0] = ld16_a2(bs + 64 * n + 16 * c);
+                q[s][1] = ld16_a2(bs + 64 * n + 32 + 16 * c);
+                q[s][NQ - 1] = ld16_a2(bs + 128 + 32 * n + 16 * c);
+                h[s] = u32x4{ld4_a2(bs + 192 + 8 * n), ld4_a2(bs + 196 + 8 * n), (u32)ld2(bs + 208), 0u};
+            }
+            return;
+        }
         if (PL) {
 #pragma unroll
             for (int s = 0; s < CH; s++) {
@@ -1097,9 +1120,11 @@ __device__ __forceinline__ void moe_g16_body(const MoeG16Args& p, uint8_t* smem)
                         // high nibbles' partner), K-step l % 8; its bytes go to two f16 pairs
                         // (planes: word l % 4 of sub-block l / 8, low nibbles' partner where
                         // l % 8 < 4; K-step 4 (sub % 2) + l % 4 of group sub / 2)
+                        // (Q6_K: l = 32 n + 16 hh + 8 r + 4 c + w: group 2 n + c, K-step 4 hh + w, run r)
                         const int sub = lane >> 3;
-                        const int kg = sub >> 1, ks = PL ? 4 * (sub & 1) + (lane & 3) : lane & 7;
-                        const int hi = PL ? (lane >> 2) & 1 : sub & 1;
+                        const int kg = Q6 ? 2 * (lane >> 5) + ((lane >> 2) & 1) : sub >> 1;
+                        const int ks = Q6 ? 4 * ((lane >> 4) & 1) + (lane & 3) : PL ? 4 * (sub & 1) + (lane & 3) : lane & 7;
+                        const int hi = Q6 ? (lane >> 3) & 1 : PL ? (lane >> 2) & 1 : sub & 1;
                         auto f = [](u32 x, int b2) { return (_Float16)(float)(int8_t)(x >> (8 * b2)); };
                         const f16x2 p02 = {f(q, 0), f(q, 2)}, p13 = {f(q, 1), f(q, 3)};
                         const int vec = sb * V + ks * 65 + 16 * kg + i;
@@ -1165,6 +1190,53 @@ __device__ __forceinline__ void moe_g16_body(const MoeG16Args& p, uint8_t* smem)
                 const int sb = ch * CH + s;
                 if (sb < nsb) {   // uniform
                     f32x4 accP[NT];
+                    if (Q6) {
+                        // sc * (q - 32) reaches 4096 and f16 holds odd integers only up to 2048: the scale
+                        // is split, sc = 2 (sc >> 1) + (sc & 1), two operands and two matrix instructions
+                        // a K-step into the same sums (gemm_q6k.h); the zero point is inside the operand
+                        const int c = kg & 1;
+                        u32 m4 = 0x000F000Fu, m2 = 0x00300030u;
+                        asm volatile("" : "+v"(m4), "+v"(m2));
+                        const f16x2 off = {(_Float16)-1056.0f, (_Float16)-1056.0f};
+#pragma unroll
+                        for (int ks = 0; ks < 8; ks++) {
+                            const int hh = ks >> 2, w = ks & 3;
+                            // the two runs' scales: bytes c and 2 + c of the half's word hh
+                            const u32 scw = hh ? hd[cur][s].y : hd[cur][s].x;
+                            const i32 sa = (i32)(int8_t)(scw >> (8 * c)), sb_ = (i32)(int8_t)(scw >> (8 * (2 + c)));
+                            const _Float16 a2 = (_Float16)(float)(2 * (sa >> 1)), a0 = (_Float16)(float)(sa & 1);
+                            const _Float16 b2 = (_Float16)(float)(2 * (sb_ >> 1)), b0 = (_Float16)(float)(sb_ & 1);
+                            const f16x2 A2 = {a2, a2}, A0 = {a0, a0}, B2 = {b2, b2}, B0 = {b0, b0};
+                            const u32 wa = wq[cur][s][0][w] >> (4 * hh), wb = wq[cur][s][1][w] >> (4 * hh);
+                            const u32 whq = wq[cur][s][NQ - 1][w];
+                            const u32 wh = hh ? whq : whq << 4;   // an element's two high bits at bits 4-5 of its half
+                            auto val = [&](u32 nib, u32 hi2) {
+                                const u32 v = (hi2 & m2) | ((nib & m4) | magic);
+                                return __builtin_bit_cast(f16x2, v) + off;
+                            };
+                            const f16x2 ta02 = val(wa, wh), tb02 = val(wb, wh >> 2);
+                            const f16x2 ta13 = val(wa >> 8, wh >> 8), tb13 = val(wb >> 8, wh >> 10);
+                            auto word = [](f16x2 v) { return __builtin_bit_cast(u32, v); };
+                            const u32x4 oa = {word(ta02 * A2), word(tb02 * B2), word(ta13 * A2), word(tb13 * B2)};
+                            const u32x4 ob = {word(ta02 * A0), word(tb02 * B0), word(ta13 * A0), word(tb13 * B0)};
+                            const f32x4 czero = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                            for (int r = 0; r < NT; r++) {
+                                const f16x8 af = __builtin_bit_cast(f16x8, sA4[r * RV + sb * V + ks * 65 + lane]);
+                                accP[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, __builtin_bit_cast(f16x8, oa),
+                                                                                 ks == 0 ? czero : accP[r], 0, 0, 0);
+                                accP[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, __builtin_bit_cast(f16x8, ob), accP[r], 0, 0, 0);
+                            }
+                        }
+                        // out += d_a * (d * P) for the super-block
+                        const float dd = half_bits_to_f32((uint16_t)(hd[cur][s].z & 0xFFFF));
+#pragma unroll
+                        for (int r = 0; r < NT; r++) {
+                            const f32x4 dav = *(const f32x4*)(sAf + ((size_t)r * RV + sb * V + 552) * 4 + 4 * kg);
+#pragma unroll
+                            for (int el = 0; el < 4; el++) out[r][el] = fmaf(dav[el], dd * accP[r][el], out[r][el]);
+                        }
+                    } else {
                     GemmWideScale sc, sc1;
                     if (PL) {
                         gemm_wide_scale_planes(hd[cur][s], 2 * kg, sc);
@@ -1211,6 +1283,7 @@ __device__ __forceinline__ void moe_g16_body(const MoeG16Args& p, uint8_t* smem)
                             const float uu = fmaf(dd, accP[r][el], -(dmin * accM[el]));
                             out[r][el] = fmaf(dav[el], uu, out[r][el]);
                         }
+                    }
                     }
                 }
             }

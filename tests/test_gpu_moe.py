@@ -83,7 +83,8 @@ def _banks(t, n_expert, nrows, k, seed, planted):
                                             (quant.Q4_K, 40, 4096, 3), (quant.Q4_K, 129, 256, 3),
                                             (quant.Q8_0, 64, 1024, 0), (quant.Q6_K, 70, 1024, 0),
                                             (quant.Q6_K, 96, 2048, 4), (quant.Q6_K, 300, 768, 4),
-                                            (quant.Q6_K, 129, 256, 4)])
+                                            (quant.Q6_K, 129, 256, 4), (quant.Q6_K, 96, 2048, 3),
+                                            (quant.Q6_K, 300, 768, 3), (quant.Q6_K, 129, 256, 3)])
 def test_grouped_matvec_vs_oracle(dev, devbuf, t, nrows, k, form):
     """form 1 = the dot-product kernel, 2 = groups of 32 columns on the matrix cores (Q4_K with
     the k-quant window), 3 = groups of 16 columns, the weights decoded in registers into the
@@ -142,12 +143,13 @@ def test_grouped_matvec_vs_oracle(dev, devbuf, t, nrows, k, form):
     dev.set_tuning(moe__form=0)
 
 
+@pytest.mark.parametrize("t", [quant.Q4_K, quant.Q6_K], ids=["q4_k", "q6_k"])
 @pytest.mark.parametrize("nrows,k", [(100, 2048), (2048 + 24, 768), (48, 1280)])
-def test_sixteen_column_groups_launch_shapes(dev, devbuf, nrows, k):
+def test_sixteen_column_groups_launch_shapes(dev, devbuf, nrows, k, t):
     """Form 3 under every launch shape its tuning keys reach: one to three super-blocks a step (K = 1280
     has five: a ragged last chunk), workgroups of four wavefronts, more row blocks than the library
     would take, every way of preparing the columns; ragged row counts; an expert with 19 columns."""
-    t, window, rows, n_expert, k_used = quant.Q4_K, 256, 21, 5, 2
+    window, rows, n_expert, k_used = 256, 21, 5, 2
     dev.SetActWindow(window)
     sel = np.zeros((rows, k_used + 1), np.uint32)
     sel[:, 0], sel[:, 1] = 3, 1
@@ -203,7 +205,7 @@ def test_grouped_matmul_more_than_one_group_of_columns(dev, devbuf, rows, t):
         want[c] = oracle.matvec_q8act_f64(t, bank[e * sheet:(e + 1) * sheet], q, a_s, nrows, k)
     b, xd, dstart, dperm = devbuf(bank), devbuf(x), devbuf(start), devbuf(perm[:used].copy())
     # 13: form 3, fused quantization; 23: form 3, groups of 32 columns
-    for form in ((1, 2, 3, 13, 23, 4) if t == quant.Q4_K else (1, 4, 0)):
+    for form in ((1, 2, 3, 13, 23, 4) if t == quant.Q4_K else (1, 3, 13, 23, 4, 0)):
         dev.set_tuning(moe__form=form % 10, moe__group16={13: 2, 23: 3}.get(form, 1))
         o = devbuf(shape=(used * nrows + 8,), dtype=np.float32, fill=np.float32(4e30))
         assert dev.moe_matvec_dev(o.ptr, None, t, b.ptr, None, xd.ptr, None, dperm.ptr, dstart.ptr, n_expert, used,
