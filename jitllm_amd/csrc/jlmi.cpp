@@ -969,9 +969,9 @@ int moe_matvec_launch(jl_ctx* c, float* out0, float* out1, int type, const void*
     //   1024 rows - / 426 / 489 / 372 / 400 1280 rows - / 501 / 577 / 475 / 435   2048 rows - / 709 / 831 / 639 / 623
     // so form 3 takes over from two columns an expert on average (groups of 32 from ten) and form 4
     // from 72; form 2 is left to "moe.form" = 2.
-    // Q6_K sheets (the down projections of a model whose other experts are Q4_K) have form 4
-    // alone, with the Q6_K GEMM's tile; the dot-product kernel is slower for that type, so the
-    // tile takes over earlier ("moe.q6k_cols": columns an expert on average, default 12).
+    // Q6_K sheets (the down projections of a model whose other experts are Q4_K) have forms 1, 3
+    // and 4 (the Q6_K GEMM's tile); where form 3 does not apply (K too long for LDS) the tile takes
+    // over from "moe.q6k_cols" columns an expert on average, default 12.
     // Form 3: groups of sixteen columns on the 16 x 16 x 32 matrix instruction, the weights decoded
     // in registers straight into its operand (Q4_K GGUF sheets or packed planes, Q6_K GGUF sheets, the k-quant window; the group's
     // fragments for the whole of K sit in LDS).  Its steady state runs at the rate of a plain read;
