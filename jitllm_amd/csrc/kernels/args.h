@@ -124,6 +124,7 @@ struct MoeGemmArgs {
 // slot (start[e] >> 4) + e + g of the prepared workspace; a slot holds, for every super-block,
 // JL_MOE_G16_SB_WORDS words: eight matrix fragments of 64 lanes x 16 bytes (half, K-step), the
 // sub-block sums' fragment (32 lanes x 16 bytes) and the sixteen columns' scales.
+#define JL_MX1_RPW 2   // rows a wavefront of the one-token MXFP4 matvec walks (2880 x 2880: 1 / 2 / 3 / 4 rows 4.46 / 4.18 / 4.22 / 4.30 us)
 #define JL_MOE_G16_SB_WORDS 2192
 #define JL_MOE_G16_LDS_WORDS 2224   // the same in LDS, the fragments 65 vectors apart
 struct MoeG16PrepArgs {

@@ -296,8 +296,7 @@ __device__ __forceinline__ void mx_matvec_body(const MxGemmArgs& p) {
 // with them: the activation is read and permuted once per wavefront instead of once per row, and
 // all the rows' weight loads go out before the first row is decoded.
 // NBI = blocks a lane holds (lane l: blocks l, l + 64, ...: k <= 2048 * NBI).
-// grid = ceil(nrows / (nwaves * RPW)), block = 64 * nwaves
-#define JL_MX1_RPW 4
+// grid = ceil(nrows / (nwaves * RPW)), block = 64 * nwaves (the library launches one wavefront a workgroup)
 template <int NBI>
 __device__ __forceinline__ void mx_matvec1_body(const MxGemmArgs& p) {
     constexpr int RPW = JL_MX1_RPW;
