@@ -1337,10 +1337,22 @@ __device__ __forceinline__ void moe_combine_body(const MoeCombineArgs& p, float*
     if (n >= n4) return;
     f32x4* res = (f32x4*)(p.resid + (size_t)r * p.n_embd) + n;
     f32x4 acc = *res;
-    for (int i = 0; i < ku; i++) {
-        const float w = swt[i];
-        const f32x4 y = ((const f32x4*)(p.y + (size_t)spos[i] * p.n_embd))[n];
-        acc = f32x4{acc.x + w * y.x, acc.y + w * y.y, acc.z + w * y.z, acc.w + w * y.w};
+    // eight experts' rows requested together (a loop of load, add, load, ... is a chain of trips to
+    // memory), added in ascending expert order as before
+    for (int i0 = 0; i0 < ku; i0 += 8) {
+        f32x4 y[8];
+#pragma unroll
+        for (int b = 0; b < 8; b++) {
+            const int i = min(i0 + b, ku - 1);
+            y[b] = ((const f32x4*)(p.y + (size_t)spos[i] * p.n_embd))[n];
+        }
+#pragma unroll
+        for (int b = 0; b < 8; b++) {
+            if (i0 + b < ku) {   // uniform
+                const float w = swt[i0 + b];
+                acc = f32x4{acc.x + w * y[b].x, acc.y + w * y[b].y, acc.z + w * y[b].z, acc.w + w * y[b].w};
+            }
+        }
     }
     *res = acc;
 }
