@@ -1080,8 +1080,6 @@ __device__ __forceinline__ void gemm_q4k_w16_body(const GemmW16Args& p, uint8_t*
 template <int NT>   // NT tiles of 16 tokens: tok_pad = 32 * ceil(NT / 2) covers them
 __device__ __forceinline__ void gemm_q4k_few_body(const GemmArgs& p, float* part) {
     typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
-    typedef unsigned bl4 __attribute__((__vector_size__(16)));
-    typedef unsigned bl2 __attribute__((__vector_size__(8)));
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r16 = lane & 15, kq = lane >> 4;
     const int r0 = blockIdx.x * 16;
@@ -1235,7 +1233,6 @@ __device__ __forceinline__ void gemm_q4k_few_body(const GemmArgs& p, float* part
 // grids of at most one and a half workgroups a CU here.
 template <int NT>
 __device__ __forceinline__ void gemm_q4k_few32_body(const GemmArgs& p, float* part) {
-    typedef unsigned bl4 __attribute__((__vector_size__(16)));
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r32 = lane & 31, half = lane >> 5;
     const int r0 = blockIdx.x * 32, t0 = blockIdx.y * 64;

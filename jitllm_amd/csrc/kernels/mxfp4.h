@@ -455,7 +455,7 @@ __device__ __forceinline__ void mx_planes_matvec_body(const MxPlanesArgs& p, flo
         const int t = i / RL, rr = i % RL;
         float s = red[t * RL + rr];
         for (int w = 1; w < p.nwaves; w++) s += red[(w * 8 + t) * RL + rr];
-        if (blockIdx.x * RL + rr < p.nrows) p.out[(size_t)t * p.nrows + blockIdx.x * RL + rr] = s;
+        if ((int)(blockIdx.x * RL + rr) < p.nrows) p.out[(size_t)t * p.nrows + blockIdx.x * RL + rr] = s;
     }
 }
 
