@@ -736,6 +736,8 @@ def main():
                     "prints its section alone")
     ap.add_argument("--section", choices=["mxfp4", "moe", "moe_packed", "moe_decode", "ffn", "ffn_packed", "ceiling", "gemm_packed"],
                     help="only this section of the default run, for profiling its kernels; prints the section alone")
+    ap.add_argument("--tune", metavar="KEY=VALUE", action="append", default=[],
+                    help="a tuning key of the library (include/jlmi.h, jl_set_tuning), e.g. gemm.form=6; repeatable")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this path runs on one GPU (no sharding, no collectives); use --gpus 1")
@@ -746,6 +748,9 @@ def main():
 
     dev = Device(device=0, act_window=256)
     gate = Gate(dev)
+    for kv in args.tune:
+        key, value = kv.split("=")
+        dev.set_tuning(**{key.replace(".", "__"): int(value)})
     if args.gemm:
         ntok, nrows = (int(v) for v in args.gemm.split(","))
         print(json.dumps({"prefill_gemm": gemm_section(dev, gate, {nrows: (ntok,)})}), flush=True)

@@ -90,7 +90,8 @@ int jl_synchronize(jl_ctx *ctx);
  * (rows per wavefront: 1, 2, 4), "matvec.block" (threads per workgroup), "matvec.grid"
  * (workgroups), "matvec.pipe" (1: the row loop as a two-deep load pipeline), "gemm.min_tok"
  * (fewest tokens sent to the matrix-core GEMM), "gemm.form" (1: 128 x 64 tiles, 2: 256 x 128
- * tiles, 3: two-pass, 4 / 5: the few-token forms, 9: token by token), "gemm.rows" (64 or 128),
+ * tiles, 3: two-pass, 4 / 5: the few-token forms, 6: 128 x 64 tiles over the whole of K on two
+ * groups of wavefronts, 9: token by token), "gemm.rows" (64 or 128),
  * "gemm.split" (K slices), "gemm.prep" (4: the four-wavefront activation prep), "gemm.planes"
  * (2: restore rows from planes before the GEMM), "packed.rw" (rows per wavefront of the
  * packed-plane matvec: 16, 32, 64), "packed.block" (its threads per workgroup), "moe.shares"

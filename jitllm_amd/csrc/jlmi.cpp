@@ -432,13 +432,16 @@ int gemm_q4k_w16_launch(jl_ctx* c, float* out, const void* w, const uint16_t* bq
 // key "gemm.form", 0 = choose): 1 = 128-token x 64-row tiles, weights dequantized in the
 // kernel; 2 = 256-token x 128-row tiles, a wavefront across all 128 rows (least L1 traffic
 // per matrix instruction, for grids that still fill the chip); 3 = weights expanded once
-// per call into f16 fragments, then 128 x 64 tiles.
+// per call into f16 fragments, then 128 x 64 tiles; 6 = 128 x 64 tiles that walk the whole of K,
+// its halves on two groups of four wavefronts (grids of half a round up to one round of the chip).
 struct PlaneRef {
     const uint32_t *qs, *d, *sc;
     int row, stride;
 };
 
 constexpr int kGemmWideTok = 256;
+// JL_GEMM_K2_LDS_BYTES: two groups of (two weight stages, minimum columns, row scales, token scales)
+constexpr unsigned kGemmK2LdsBytes = 2u * (2u * 64u * 136u * 2u + 2u * 64u * 24u * 2u + 2u * 64u * 2u * 4u + 2u * 128u * 4u);
 constexpr unsigned kGemmWideLdsBytes = 2u * 128u * 136u * 2u + 2u * 128u * 24u * 2u + 2u * 128u * 2u * 4u + 2u * kGemmWideTok * 4u;   // JL_GEMM_WIDE_LDS_BYTES
 
 // Few tokens, or a grid of at most a round and a half of 32-row workgroups: the forms that
@@ -504,6 +507,15 @@ int gemm_q4k_launch(jl_ctx* c, float* out, const void* w, const float* x, int nr
         return launch(c, "jl_gemm_q4k_few32", (unsigned)((nrows + 31) / 32), (unsigned)(tok_pad / 64), 512, 0, st, gp);
     }
     if (form == 4 || form == 5) form = 0;   // outside the few-token forms' range
+    const bool k2_fits = (k / 256) % 4 == 0 && kGemmK2LdsBytes <= c->lds_limit;
+    if (form == 0 && k2_fits) {
+        // 128 x 64 tiles over the whole of K: from half a round of the chip up to one round nothing
+        // has to be cut along K and added afterwards (measured against the forms below, us:
+        // 512 tokens x 4096 rows 32.0 against 37.9, 384 x 4096 29.4 against 35.9, 128 x 14336
+        // 27.9 against 36.2, 256 x 4096 26.5 against 27.7; two rounds and more go to the wide tile)
+        const long k2_groups = (long)((ntok + kGemmTile - 1) / kGemmTile) * ((nrows + 63) / 64);
+        if (k2_groups <= c->num_cu && 2 * k2_groups >= c->num_cu) form = 6;
+    }
     if (form == 0) {
         const long wide_groups = (long)((ntok + kGemmWideTok - 1) / kGemmWideTok) * ((nrows + 127) / 128);
         // from a quarter of the CUs on: a smaller grid is widened along K below (measured
@@ -513,6 +525,7 @@ int gemm_q4k_launch(jl_ctx* c, float* out, const void* w, const float* x, int nr
         form = 4 * wide_groups >= 3 * (long)c->num_cu || (4 * wide_groups >= (long)c->num_cu && !padded) ? 2 : 1;
     }
     if (form == 2 && kGemmWideLdsBytes > c->lds_limit) form = 1;
+    if (form == 6 && !k2_fits) form = 1;
     const int tile = form == 2 ? kGemmWideTok : kGemmTile;
     const int tok_pad = (ntok + tile - 1) / tile * tile;
     const int nsb = k / 256;
@@ -538,6 +551,9 @@ int gemm_q4k_launch(jl_ctx* c, float* out, const void* w, const float* x, int nr
     ga.nrows = nrows; ga.k = k; ga.ntok = ntok; ga.tok_pad = tok_pad; ga.row_bytes = nsb * 144;
     ga.out_stride = nrows; ga.sb_per = 0;
     void* gp[] = {&ga};
+    if (form == 6)   // 128 x 64 tiles over the whole of K, the K halves on two groups of wavefronts
+        return launch(c, pl ? "jl_gemm_q4k_k2_planes" : "jl_gemm_q4k_k2", (unsigned)(tok_pad / kGemmTile), (unsigned)((nrows + 63) / 64), 512,
+                      kGemmK2LdsBytes, st, gp);
     int rows_left = nrows;
     if (form == 2) {
         // One workgroup per CU: a grid of f full rounds and a last round at most half full
@@ -1270,7 +1286,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     if (e != hipSuccess)
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
-    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_prep_q4k_planes", "jl_gemm_q4k_r64_planes", "jl_gemm_q4k_wide_planes", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_group2_wide", "jl_moe_quant", "jl_moe_matvec_planes_q4k", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_prep_planes", "jl_moe_gemm_q4k", "jl_moe_g16_prep", "jl_moe_g16_prep_planes", "jl_moe_g16_prep_q6k", "jl_moe_g16_c1", "jl_moe_g16_c2", "jl_moe_g16_c3", "jl_moe_g16_f1", "jl_moe_g16_f2", "jl_moe_g16_f3", "jl_moe_g16_g1", "jl_moe_g16_g2", "jl_moe_g16_g3", "jl_moe_g16_d1", "jl_moe_g16_d2", "jl_moe_g16_d3", "jl_moe_g16p_c1", "jl_moe_g16p_c2", "jl_moe_g16p_c3", "jl_moe_g16p_f1", "jl_moe_g16p_f2", "jl_moe_g16p_f3", "jl_moe_g16p_g1", "jl_moe_g16p_g2", "jl_moe_g16p_g3", "jl_moe_g16p_d1", "jl_moe_g16p_d2", "jl_moe_g16p_d3", "jl_moe_g16q6_c1", "jl_moe_g16q6_c2", "jl_moe_g16q6_c3", "jl_moe_g16q6_f1", "jl_moe_g16q6_f2", "jl_moe_g16q6_f3", "jl_moe_g16q6_g1", "jl_moe_g16q6_g2", "jl_moe_g16q6_g3", "jl_moe_g16q6_d1", "jl_moe_g16q6_d2", "jl_moe_g16q6_d3", "jl_moe_gemm_r64", "jl_moe_gemm_r64_planes", "jl_moe_gemm_q6k_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_mxfp4_matvec1_b1", "jl_mxfp4_matvec1_b2", "jl_mxfp4_matvec1_b3", "jl_mxfp4_scaled_prep", "jl_mxfp4_scaled_gemm", "jl_mxfp4_planes_prep", "jl_mxfp4_planes_gemm", "jl_mxfp4_matvec_planes_r64", "jl_mxfp4_matvec_planes_r32", "jl_mxfp4_matvec_planes_r16", "jl_unpack_mxfp4", "jl_sum_parts", "jl_probe_read", "jl_probe_empty", "jl_probe_wait", "jl_probe_mfma", "jl_probe_mfma_v5",
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_q4k_k2", "jl_gemm_q4k_k2_planes", "jl_gemm_prep_q4k_planes", "jl_gemm_q4k_r64_planes", "jl_gemm_q4k_wide_planes", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_group2_wide", "jl_moe_quant", "jl_moe_matvec_planes_q4k", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_prep_planes", "jl_moe_gemm_q4k", "jl_moe_g16_prep", "jl_moe_g16_prep_planes", "jl_moe_g16_prep_q6k", "jl_moe_g16_c1", "jl_moe_g16_c2", "jl_moe_g16_c3", "jl_moe_g16_f1", "jl_moe_g16_f2", "jl_moe_g16_f3", "jl_moe_g16_g1", "jl_moe_g16_g2", "jl_moe_g16_g3", "jl_moe_g16_d1", "jl_moe_g16_d2", "jl_moe_g16_d3", "jl_moe_g16p_c1", "jl_moe_g16p_c2", "jl_moe_g16p_c3", "jl_moe_g16p_f1", "jl_moe_g16p_f2", "jl_moe_g16p_f3", "jl_moe_g16p_g1", "jl_moe_g16p_g2", "jl_moe_g16p_g3", "jl_moe_g16p_d1", "jl_moe_g16p_d2", "jl_moe_g16p_d3", "jl_moe_g16q6_c1", "jl_moe_g16q6_c2", "jl_moe_g16q6_c3", "jl_moe_g16q6_f1", "jl_moe_g16q6_f2", "jl_moe_g16q6_f3", "jl_moe_g16q6_g1", "jl_moe_g16q6_g2", "jl_moe_g16q6_g3", "jl_moe_g16q6_d1", "jl_moe_g16q6_d2", "jl_moe_g16q6_d3", "jl_moe_gemm_r64", "jl_moe_gemm_r64_planes", "jl_moe_gemm_q6k_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_mxfp4_matvec1_b1", "jl_mxfp4_matvec1_b2", "jl_mxfp4_matvec1_b3", "jl_mxfp4_scaled_prep", "jl_mxfp4_scaled_gemm", "jl_mxfp4_planes_prep", "jl_mxfp4_planes_gemm", "jl_mxfp4_matvec_planes_r64", "jl_mxfp4_matvec_planes_r32", "jl_mxfp4_matvec_planes_r16", "jl_unpack_mxfp4", "jl_sum_parts", "jl_probe_read", "jl_probe_empty", "jl_probe_wait", "jl_probe_mfma", "jl_probe_mfma_v5",
                                       "jl_pack_weights", "jl_unpack_q4k", "jl_unpack_q6k", "jl_unpack_q8_0"};
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int rw : {16, 32, 64})

@@ -5,6 +5,7 @@
 #include "common.h"
 #include "dequant.h"
 #include "gemm_q4k.h"
+#include "gemm_q4k_k2.h"
 #include "gemm_q6k.h"
 #include "gemm_w32.h"
 #include "matvec.h"
@@ -163,6 +164,10 @@ extern "C" __global__ __launch_bounds__(512) void jl_gemm_q4k_wide(GemmArgs p) {
     gemm_split_slice(p);
     gemm_q4k_wide_body<false>(p, jl_smem);
 }
+// 128 tokens x 64 rows over the whole of K, the K halves on two groups of four wavefronts:
+// grid = (tok_pad/128, ceil(nrows/64)), block = 512, dynamic LDS = JL_GEMM_K2_LDS_BYTES
+extern "C" __global__ __launch_bounds__(512) void jl_gemm_q4k_k2(GemmArgs p) { gemm_q4k_k2_body<false>(p, jl_smem); }
+extern "C" __global__ __launch_bounds__(512) void jl_gemm_q4k_k2_planes(GemmArgs p) { gemm_q4k_k2_body<true>(p, jl_smem); }
 // The same two tiles reading the weights from packed planes (GemmArgs.pqs / pd / psc), after the
 // prep in the planes' K order: no rows are restored first.
 extern "C" __global__ __launch_bounds__(1024) void jl_gemm_prep_q4k_planes(GemmPrepArgs p) {

@@ -50,11 +50,12 @@ MATVECS = [
     (quant.Q4_K, 4096, 4096, 256, "normal"),      # the headline configuration
     (quant.Q8_0, 14336, 4096, 32, "normal"),      # gate / up: more than 16 rows a CU
     (quant.Q6_K, 4096, 14336, 32, "planted"),     # down
+    (quant.Q6_K, 4096, 14336, 32, "normal"),      # down with the N(0, 0.02) weights the configuration names
     (quant.Q4_K, 14336, 4096, 256, "planted"),
 ]
 
 
-@pytest.mark.parametrize("case", MATVECS, ids=lambda c: f"{quant.NAMES[c[0]]}_{c[1]}x{c[2]}")
+@pytest.mark.parametrize("case", MATVECS, ids=lambda c: f"{quant.NAMES[c[0]]}_{c[1]}x{c[2]}_{c[4]}")
 def test_decode_matvec_full_size_rows_and_planes(dev, devbuf, case):
     """GGUF rows with the library's own launch shape (a persistent grid of 768-thread
     workgroups once a matrix has more than sixteen rows a CU) and the packed planes of the
@@ -125,14 +126,18 @@ def _sample_rows(nrows, rng, boundaries):
     return np.array(sorted(r for r in picks if 0 <= r < nrows))
 
 
-GEMMS = [(512, 4096), (512, 14336), (2048, 4096), (2048, 14336)]
+# the baseline's sweep {16, 128, 512, 2048} tokens x {4096, 14336} rows
+GEMMS = [(16, 4096), (16, 14336), (128, 4096), (128, 14336), (512, 4096), (512, 14336), (2048, 4096), (2048, 14336)]
 
 
 @pytest.mark.parametrize("shape", GEMMS, ids=lambda s: f"{s[0]}x4096->{s[1]}")
 def test_prefill_gemm_full_size(dev, devbuf, shape):
-    """The Q4_K prefill GEMM (512 and 2048 tokens x 4096 -> 4096 and 14336) at its real sizes: the library's own choice of form, then the
-    256 x 128 and the 128 x 64 tiles forced.  Sampled rows x all tokens against the oracle;
-    a few tokens whole against the decode matvec; the forms bit for bit against each other."""
+    """The Q4_K prefill GEMM at its real sizes (every point of the baseline's sweep): the library's
+    own choice of form (the few-token forms at 16 and 128 tokens x 4096 rows, the 128 x 64 tile
+    over the whole of K where the grid is half a round to one round of the chip, the 256 x 128
+    tile beyond), then the 256 x 128 tile, the 128 x 64 tile and the whole-K tile forced.
+    Sampled rows x all tokens against the oracle; a few tokens whole against the decode
+    matvec; the forms against each other."""
     ntok, nrows = shape
     k, t, window = 4096, quant.Q4_K, 256
     dev.SetActWindow(window)
@@ -150,7 +155,7 @@ def test_prefill_gemm_full_size(dev, devbuf, shape):
     want = oracle.matmul_q8act_f64(t, w_rows, x, len(rows), k, ntok, window)
     wd, xd = devbuf(w), devbuf(x)
     outs = {}
-    for form in (0, 2, 1):
+    for form in (0, 2, 1, 6):
         dev.set_tuning(gemm__form=form)
         assert dev.reserve_shape(t, nrows, k, ntok)
         out = devbuf(shape=(ntok * nrows + 16,), dtype=np.float32, fill=POISON)
@@ -169,14 +174,14 @@ def test_prefill_gemm_full_size(dev, devbuf, shape):
         assert np.all(got[ntok // 3] == 0)
         outs[form] = got
     dev.set_tuning(gemm__form=0)
-    # every form sums the same integers and runs the same f32 epilogue, so the forms agree bit
-    # for bit -- except where the automatic choice cuts K across workgroups (a grid of at most
-    # one workgroup a CU: 512 tokens x 4096 rows), which adds the super-blocks' terms in
-    # another association
+    # every form sums the same integers and runs the same f32 epilogue, so forms that walk K in
+    # one piece agree bit for bit; a form that cuts K (across workgroups, or across the
+    # wavefronts of one) adds the super-blocks' terms in another association
     assert np.array_equal(outs[1].view(np.uint32), outs[2].view(np.uint32)), "128 x 64 tiles != 256 x 128 tiles"
-    if (ntok + 127) // 128 * ((nrows + 63) // 64) <= 256 and (ntok + 255) // 256 * ((nrows + 127) // 128) * 4 < 3 * 256:
-        assert nmse(outs[0], outs[1].astype(np.float64)) <= 1e-12, "K-split form vs 128 x 64 tiles"
-    else:
+    for form in (0, 6):
+        assert nmse(outs[form], outs[1].astype(np.float64)) <= 1e-12, f"form {form} vs 128 x 64 tiles"
+    k_cut = ntok <= 192 or (128 <= (ntok + 127) // 128 * ((nrows + 63) // 64) <= 256)
+    if not k_cut:
         assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32)), "automatic form != 128 x 64 tiles"
     # the same weights as packed planes: the tiled forms read them where they lie (no rows are
     # restored first), the same integers and the same epilogue, so the same bits
@@ -186,7 +191,8 @@ def test_prefill_gemm_full_size(dev, devbuf, shape):
     outp = devbuf(shape=(ntok * nrows + 16,), dtype=np.float32, fill=POISON)
     n0 = dev.launch_count()
     assert dev.matmul_packed_dev(outp.ptr, t, Packed(pl[0].ptr, pl[1].ptr, pl[2].ptr, 0, nrows), xd.ptr, nrows, k, ntok)
-    assert dev.launch_count() - n0 <= 3, "a launch restored rows in front of the GEMM"
+    if ntok > 192:
+        assert dev.launch_count() - n0 <= 3, "a launch restored rows in front of the GEMM"
     dev.synchronize()
     gotp = outp.get()
     assert np.all(gotp[ntok * nrows:] == POISON)
@@ -199,6 +205,59 @@ def test_prefill_gemm_full_size(dev, devbuf, shape):
         assert dev.matvec_dev(mv.ptr, t, wd.ptr, xd.ptr + tok * k * 4, nrows, k)
         dev.synchronize()
         e = nmse(outs[0][tok], mv.get().astype(np.float64))
+        assert e <= 1e-10, f"token {tok}: GEMM vs decode matvec NMSE {e:.3e}"
+    for b in (wd, xd, mv):
+        b.free()
+    dev.SetActWindow(32)
+
+
+OTHER_GEMMS = [
+    # (type, nrows, k, window, tokens): every other prefill GEMM the benchmark times
+    (quant.Q8_0, 14336, 4096, 32, 512), (quant.Q8_0, 14336, 4096, 32, 2048),
+    (quant.Q6_K, 4096, 14336, 32, 512), (quant.Q6_K, 4096, 14336, 32, 2048),
+    (quant.Q6_K, 4096, 14336, 256, 512), (quant.Q6_K, 4096, 14336, 256, 2048),
+]
+
+
+@pytest.mark.parametrize("case", OTHER_GEMMS, ids=lambda c: f"{quant.NAMES[c[0]]}_w{c[3]}_{c[4]}x{c[2]}->{c[1]}")
+def test_prefill_gemm_other_types_full_size(dev, devbuf, case):
+    """The Llama-3-8B feed-forward matrices at prefill, at their real sizes: Q8_0 gate / up
+    with the activation window of 32, Q6_K down with both windows; 512 and 2048 tokens.
+    Sampled rows x all tokens against the oracle, and a few tokens whole against the decode
+    matvec of the same token."""
+    t, nrows, k, window, ntok = case
+    dev.SetActWindow(window)
+    rng = np.random.default_rng(ntok + nrows + window)
+    w = _weights(t, nrows, k, "normal")
+    x = rng.standard_normal((ntok, k), np.float32) * (1 + np.arange(ntok, dtype=np.float32)[:, None] % 5)
+    x[ntok // 3] = 0
+    rows = _sample_rows(nrows, rng, [64, 128, nrows - 64])
+    rb = quant.row_bytes(t, k)
+    w_rows = np.concatenate([w[r * rb:(r + 1) * rb] for r in rows])
+    want = oracle.matmul_q8act_f64(t, w_rows, x, len(rows), k, ntok, window)
+    wd, xd = devbuf(w), devbuf(x)
+    assert dev.reserve_shape(t, nrows, k, ntok)
+    out = devbuf(shape=(ntok * nrows + 16,), dtype=np.float32, fill=POISON)
+    n0 = dev.launch_count()
+    assert dev.matmul_dev(out.ptr, t, wd.ptr, xd.ptr, nrows, k, ntok)
+    dev.synchronize()
+    assert dev.launch_count() - n0 <= 3, "the matrix kernel, not a launch per token"
+    got = out.get()
+    out.free()
+    assert np.all(got[ntok * nrows:] == POISON), "wrote past the output"
+    got = got[:ntok * nrows].reshape(ntok, nrows)
+    assert np.all(np.abs(got) < 1e30), "elements left unwritten"
+    sub = got[:, rows]
+    e = nmse(sub, want)
+    assert e <= 1e-10, f"NMSE {e:.3e} on the sampled rows"
+    worst = max(nmse(sub[:, j], want[:, j]) for j in range(len(rows)) if np.any(want[:, j]))
+    assert worst <= 1e-9, f"worst sampled row NMSE {worst:.3e}"
+    assert np.all(got[ntok // 3] == 0)
+    mv = devbuf(shape=(nrows,), dtype=np.float32, fill=POISON)
+    for tok in (0, ntok // 2 + 1, ntok - 1):
+        assert dev.matvec_dev(mv.ptr, t, wd.ptr, xd.ptr + tok * k * 4, nrows, k)
+        dev.synchronize()
+        e = nmse(got[tok], mv.get().astype(np.float64))
         assert e <= 1e-10, f"token {tok}: GEMM vs decode matvec NMSE {e:.3e}"
     for b in (wd, xd, mv):
         b.free()

@@ -69,6 +69,7 @@ def test_grouping_is_bit_exact(dev, devbuf, mode, rows, n_expert, k_used, form):
     dev.set_tuning(moe__group=0)
 
 
+@functools.lru_cache(maxsize=8)
 def _banks(t, n_expert, nrows, k, seed, planted):
     make = synth.random_weights if planted else synth.quantized_weights
     return np.concatenate([make(t, nrows, k, seed=seed + e) for e in range(n_expert)])
@@ -325,6 +326,39 @@ def test_moe_block_vs_oracle(dev, devbuf, shape):
         # four columns an expert on average: grouping, two matrix-core launches that quantize
         # their own columns, combine; the tiny case takes the dot-product form (two more launches)
         assert dev.launch_count() - before == (4 if rows == 64 else 6)
+    dev.SetActWindow(32)
+
+
+def test_moe_block_prefill_1024_rows_vs_oracle_on_sampled_rows(dev, devbuf):
+    """The Qwen3-30B-A3B block at a prefill batch, the size the benchmark times: 1024 rows routed
+    top-8 over 128 experts (64 columns an expert on average: the matrix-core forms with groups of
+    32 columns).  A row's output depends on that row alone, so the oracle evaluates a spread
+    sample of rows (first, last, and evenly between) through their own eight experts."""
+    rows, n_expert, k_used, n_ffn, n_embd = 1024, 128, 8, 768, 2048
+    t, window = quant.Q4_K, 256
+    dev.SetActWindow(window)
+    sel, wt = route(rows, n_expert, k_used, 12)
+    gate = _banks(t, n_expert, n_ffn, n_embd, 1000, False)
+    up = _banks(t, n_expert, n_ffn, n_embd, 2000, False)
+    down = _banks(t, n_expert, n_embd, n_ffn, 3000, False)
+    x = np.stack([synth.activations(n_embd, seed=9000 + r) for r in range(rows)])
+    sample = np.unique(np.linspace(0, rows - 1, 40).astype(int))
+    want = _oracle_block(t, gate, up, down, x[sample], sel[sample], wt[sample], n_expert, n_ffn, n_embd, window)
+    gd, ud, dd, xd, sd, wd = devbuf(gate), devbuf(up), devbuf(down), devbuf(x), devbuf(sel), devbuf(wt)
+    resid = devbuf(shape=(rows, n_embd), dtype=np.float32, fill=0)
+    for call in range(2):
+        resid.put(np.zeros((rows, n_embd), np.float32))
+        assert dev.moe_ffn_dev(resid.ptr, t, gd.ptr, ud.ptr, dd.ptr, xd.ptr, sd.ptr, k_used + 1, wd.ptr,
+                               rows, k_used, n_expert, n_ffn, n_embd)
+        dev.synchronize()
+        got = resid.get()
+        assert np.all(np.isfinite(got))
+        assert rel_l2(got[sample], want) <= 1e-3, f"call {call}: rel-L2 {rel_l2(got[sample], want):.3e}"
+        worst = max(rel_l2(got[r], want[i]) for i, r in enumerate(sample))
+        assert worst <= 2e-3, f"call {call}: worst sampled row rel-L2 {worst:.3e}"
+        # rows outside the sample: every one written, and of the size of its neighbours
+        norms = np.sqrt(np.mean(got.astype(np.float64) ** 2, axis=1))
+        assert norms.min() > 0.05 * np.median(norms) and norms.max() < 20 * np.median(norms)
     dev.SetActWindow(32)
 
 
