@@ -30,6 +30,7 @@ const HipApi* H = nullptr;  // the process-wide HIP runtime, resolved by the fir
 
 struct Tuning {
     int rpw = 0, block = 0, grid = 0, pipe = 0;
+    int q8pair = 0;             // Q8_0 rows: 2 keeps one block a lane-slot (2-byte-aligned loads)
     int packed_rw = 0, packed_block = 0, moe_group = 0, moe_logits = 0, moe_q6k_cols = 0;
     int moe_shares = 0;
     int gemm_rows = 0;
@@ -164,14 +165,25 @@ bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
 // Largest workgroup of the matvec variant with `rpw` rows per wavefront, 0 when the
 // code object has no such variant (kernels/jlmi_kernels.hip).
-int matvec_max_block(int type, int rpw) {
+int matvec_max_block(int type, int rpw, bool q8_pair = false) {
     if (rpw == 1) return 1024;
     if (rpw == 2) return type == JL_TYPE_Q6_K ? 512 : 1024;
-    if (rpw == 4) return type == JL_TYPE_Q8_0 ? 1024 : 512;
+    if (rpw == 4) return type == JL_TYPE_Q8_0 && !q8_pair ? 1024 : 512;
     return 0;
 }
 
 hipStream_t pick_stream(jl_ctx* c, void* s) { return s ? (hipStream_t)s : c->stream; }
+
+// LDS of the decode matvec: int8 activations, a scale per 32, a sum per 16
+size_t act_lds_bytes(int k) { return (size_t)k + (size_t)(k / 32) * 4 + (size_t)(k / 16) * 4; }
+
+// Q8_0 rows in the form that takes two blocks a lane-slot with every load 4-byte aligned
+// (kernels/matvec.h): rows on 4-byte boundaries, an even number of blocks a row, room in
+// LDS for the second copy of the activations.
+bool q8_pair_form(const jl_ctx* c, int type, const void* w, int k) {
+    return type == JL_TYPE_Q8_0 && c->tune.q8pair != 2 && k % 64 == 0 && ((uintptr_t)w & 3) == 0 &&
+           act_lds_bytes(k) + (size_t)k + 16 <= c->lds_limit;
+}
 
 int launch(jl_ctx* c, const char* name, unsigned gx, unsigned gy, unsigned block, unsigned lds,
            hipStream_t st, void** params, unsigned gz = 1) {
@@ -248,7 +260,8 @@ int matvec_launch(jl_ctx* c, float* out, int type, const void* w, const float* x
     const bool one_per_cu = small || type == JL_TYPE_Q6_K || type == JL_TYPE_Q4_K;
     if (block <= 0) block = one_per_cu ? 1024 : 768;
     if (block % 64 != 0 || block > 1024) return fail(c, JL_ERR_ARG, "matvec: block=%d", block);
-    if (block > matvec_max_block(type, rpw)) block = matvec_max_block(type, rpw);
+    const bool pair = q8_pair_form(c, type, w, k);
+    if (block > matvec_max_block(type, rpw, pair)) block = matvec_max_block(type, rpw, pair);
     const int rows_per_block = (block / 64) * rpw;
     long groups = ((long)nrows + rows_per_block - 1) / rows_per_block;
     long grid = c->tune.grid > 0 ? c->tune.grid : (long)c->num_cu * (type == JL_TYPE_Q4_K && !small ? 1 : 2);
@@ -273,9 +286,9 @@ int matvec_launch(jl_ctx* c, float* out, int type, const void* w, const float* x
     // against 14.2), so it stays off unless asked for
     a.pipe = c->tune.pipe == 1 ? 1 : 2;
     char name[64];
-    snprintf(name, sizeof name, "jl_matvec_%s_r%d", ti->tag, rpw);
+    snprintf(name, sizeof name, "jl_matvec_%s_r%d", pair ? "q8_0p" : ti->tag, rpw);
     void* params[] = {&a};
-    unsigned lds = (unsigned)((size_t)k + (size_t)(k / 32) * 4 + (size_t)(k / 16) * 4);
+    unsigned lds = (unsigned)(act_lds_bytes(k) + (pair ? (size_t)k + 16 : 0));
     return launch(c, name, (unsigned)grid, 1, (unsigned)block, lds, st, params);
 }
 
@@ -323,10 +336,12 @@ int matvec_multi_launch(jl_ctx* c, int type, int m, float* const* outs, const vo
     if (gx < 1) gx = 1;
     a.nwaves = nwaves; a.ngroups = (int)gx;
     char name[64];
+    bool pair = !types;
+    for (int i = 0; i < m && pair; i++) pair = q8_pair_form(c, type, ws[i], k);
     if (types) snprintf(name, sizeof name, "jl_matvec_segments");
-    else snprintf(name, sizeof name, "jl_matvec_multi_%s", ti->tag);
+    else snprintf(name, sizeof name, "jl_matvec_multi_%s", pair ? "q8_0p" : ti->tag);
     void* params[] = {&a};
-    unsigned lds = (unsigned)((size_t)k + (size_t)(k / 32) * 4 + (size_t)(k / 16) * 4);
+    unsigned lds = (unsigned)(act_lds_bytes(k) + (pair ? (size_t)k + 16 : 0));
     return launch(c, name, (unsigned)gx, (unsigned)m, nwaves * 64, lds, st, params);
 }
 
@@ -1286,7 +1301,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     if (e != hipSuccess)
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
-    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_q4k_k2", "jl_gemm_q4k_k2_planes", "jl_gemm_prep_q4k_planes", "jl_gemm_q4k_r64_planes", "jl_gemm_q4k_wide_planes", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_group2_wide", "jl_moe_quant", "jl_moe_matvec_planes_q4k", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_prep_planes", "jl_moe_gemm_q4k", "jl_moe_g16_prep", "jl_moe_g16_prep_planes", "jl_moe_g16_prep_q6k", "jl_moe_g16_c1", "jl_moe_g16_c2", "jl_moe_g16_c3", "jl_moe_g16_f1", "jl_moe_g16_f2", "jl_moe_g16_f3", "jl_moe_g16_g1", "jl_moe_g16_g2", "jl_moe_g16_g3", "jl_moe_g16_d1", "jl_moe_g16_d2", "jl_moe_g16_d3", "jl_moe_g16p_c1", "jl_moe_g16p_c2", "jl_moe_g16p_c3", "jl_moe_g16p_f1", "jl_moe_g16p_f2", "jl_moe_g16p_f3", "jl_moe_g16p_g1", "jl_moe_g16p_g2", "jl_moe_g16p_g3", "jl_moe_g16p_d1", "jl_moe_g16p_d2", "jl_moe_g16p_d3", "jl_moe_g16q6_c1", "jl_moe_g16q6_c2", "jl_moe_g16q6_c3", "jl_moe_g16q6_f1", "jl_moe_g16q6_f2", "jl_moe_g16q6_f3", "jl_moe_g16q6_g1", "jl_moe_g16q6_g2", "jl_moe_g16q6_g3", "jl_moe_g16q6_d1", "jl_moe_g16q6_d2", "jl_moe_g16q6_d3", "jl_moe_gemm_r64", "jl_moe_gemm_r64_planes", "jl_moe_gemm_q6k_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_mxfp4_matvec1_b1", "jl_mxfp4_matvec1_b2", "jl_mxfp4_matvec1_b3", "jl_mxfp4_scaled_prep", "jl_mxfp4_scaled_gemm", "jl_mxfp4_planes_prep", "jl_mxfp4_planes_gemm", "jl_mxfp4_matvec_planes_r64", "jl_mxfp4_matvec_planes_r32", "jl_mxfp4_matvec_planes_r16", "jl_unpack_mxfp4", "jl_sum_parts", "jl_probe_read", "jl_probe_empty", "jl_probe_wait", "jl_probe_mfma", "jl_probe_mfma_v5",
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_matvec_q8_0p_r1", "jl_matvec_q8_0p_r2", "jl_matvec_q8_0p_r4", "jl_matvec_multi_q8_0p", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_q4k_k2", "jl_gemm_q4k_k2_planes", "jl_gemm_prep_q4k_planes", "jl_gemm_q4k_r64_planes", "jl_gemm_q4k_wide_planes", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_group2_wide", "jl_moe_quant", "jl_moe_matvec_planes_q4k", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_prep_planes", "jl_moe_gemm_q4k", "jl_moe_g16_prep", "jl_moe_g16_prep_planes", "jl_moe_g16_prep_q6k", "jl_moe_g16_c1", "jl_moe_g16_c2", "jl_moe_g16_c3", "jl_moe_g16_f1", "jl_moe_g16_f2", "jl_moe_g16_f3", "jl_moe_g16_g1", "jl_moe_g16_g2", "jl_moe_g16_g3", "jl_moe_g16_d1", "jl_moe_g16_d2", "jl_moe_g16_d3", "jl_moe_g16p_c1", "jl_moe_g16p_c2", "jl_moe_g16p_c3", "jl_moe_g16p_f1", "jl_moe_g16p_f2", "jl_moe_g16p_f3", "jl_moe_g16p_g1", "jl_moe_g16p_g2", "jl_moe_g16p_g3", "jl_moe_g16p_d1", "jl_moe_g16p_d2", "jl_moe_g16p_d3", "jl_moe_g16q6_c1", "jl_moe_g16q6_c2", "jl_moe_g16q6_c3", "jl_moe_g16q6_f1", "jl_moe_g16q6_f2", "jl_moe_g16q6_f3", "jl_moe_g16q6_g1", "jl_moe_g16q6_g2", "jl_moe_g16q6_g3", "jl_moe_g16q6_d1", "jl_moe_g16q6_d2", "jl_moe_g16q6_d3", "jl_moe_gemm_r64", "jl_moe_gemm_r64_planes", "jl_moe_gemm_q6k_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_mxfp4_matvec1_b1", "jl_mxfp4_matvec1_b2", "jl_mxfp4_matvec1_b3", "jl_mxfp4_scaled_prep", "jl_mxfp4_scaled_gemm", "jl_mxfp4_planes_prep", "jl_mxfp4_planes_gemm", "jl_mxfp4_matvec_planes_r64", "jl_mxfp4_matvec_planes_r32", "jl_mxfp4_matvec_planes_r16", "jl_unpack_mxfp4", "jl_sum_parts", "jl_probe_read", "jl_probe_empty", "jl_probe_wait", "jl_probe_mfma", "jl_probe_mfma_v5",
                                       "jl_pack_weights", "jl_unpack_q4k", "jl_unpack_q6k", "jl_unpack_q8_0"};
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int rw : {16, 32, 64})
@@ -1399,6 +1414,7 @@ int jl_set_tuning(jl_ctx* c, const char* key, int value) {
     else if (!strcmp(key, "mxfp4.rows")) c->tune.mx_rows = value;
     else if (!strcmp(key, "mxfp4.planes")) c->tune.mx_planes = value;
     else if (!strcmp(key, "mxfp4.scaled")) c->tune.mx_scaled = value;
+    else if (!strcmp(key, "matvec.q8pair")) c->tune.q8pair = value;
     else if (!strcmp(key, "gemm.form")) c->tune.gemm_form = value;
     else if (!strcmp(key, "gemm.split")) c->tune.gemm_split = value;
     else if (!strcmp(key, "gemm.prep")) c->tune.gemm_prep = value;
@@ -2138,7 +2154,7 @@ int jl_probe_dev(jl_ctx* c, int kind, const void* src, size_t nbytes, int grid, 
     if (grid <= 0) grid = 2 * c->num_cu;
     if (block <= 0) block = 1024;
     if (block % 64 != 0 || block > 1024) return fail(c, JL_ERR_ARG, "probe: block=%d", block);
-    if (kind == 1 && (!src || !aligned16(src))) return fail(c, JL_ERR_ARG, "probe: src");
+    if (kind == 1 && (!src || ((uintptr_t)src & 1) != 0)) return fail(c, JL_ERR_ARG, "probe: src");
     HIP_TRY(c, H->SetDevice(c->device));
     size_t nvec = nbytes / 16;
     void* sink = nullptr;

@@ -55,6 +55,9 @@ extern "C" __global__ __launch_bounds__(256) void jl_dequant(
 JL_MATVEC_KERNEL(q4k, JL_Q4_K, 1, 1024) JL_MATVEC_KERNEL(q4k, JL_Q4_K, 2, 1024) JL_MATVEC_KERNEL(q4k, JL_Q4_K, 4, 512)
 JL_MATVEC_KERNEL(q8_0, JL_Q8_0, 1, 1024) JL_MATVEC_KERNEL(q8_0, JL_Q8_0, 2, 1024) JL_MATVEC_KERNEL(q8_0, JL_Q8_0, 4, 1024)
 JL_MATVEC_KERNEL(q6k, JL_Q6_K, 1, 1024) JL_MATVEC_KERNEL(q6k, JL_Q6_K, 2, 512) JL_MATVEC_KERNEL(q6k, JL_Q6_K, 4, 512)
+// Q8_0 with two blocks a lane-slot, every load 4-byte aligned (rows 4-byte aligned, k % 64 == 0);
+// dynamic LDS = JL_ACT_LDS_BYTES_SHIFTED(k)
+JL_MATVEC_KERNEL(q8_0p, JL_Q8_0P, 1, 1024) JL_MATVEC_KERNEL(q8_0p, JL_Q8_0P, 2, 1024) JL_MATVEC_KERNEL(q8_0p, JL_Q8_0P, 4, 512)
 
 // grid = (row groups, matrices), block = 64..1024
 #define JL_MATVEC_MULTI_KERNEL(T, TYPE)                                                                \
@@ -62,6 +65,7 @@ JL_MATVEC_KERNEL(q6k, JL_Q6_K, 1, 1024) JL_MATVEC_KERNEL(q6k, JL_Q6_K, 2, 512) J
         matvec_multi_body<TYPE>(p, jl_smem, p.row_bytes);                                              \
     }
 JL_MATVEC_MULTI_KERNEL(q4k, JL_Q4_K) JL_MATVEC_MULTI_KERNEL(q8_0, JL_Q8_0) JL_MATVEC_MULTI_KERNEL(q6k, JL_Q6_K)
+JL_MATVEC_MULTI_KERNEL(q8_0p, JL_Q8_0P)
 // The same grid over matrices of different types (the reference's MatVecSegments,
 // jit/gpu/kernels/matvec.go:1411-1431: a block's q, k and v in one launch whatever their
 // formats): the type is uniform per workgroup, so the switch is a scalar branch into the

@@ -27,32 +27,47 @@ struct ActLds {
     const uint8_t* a;
     const float* da;
     const float* s16;
+    const uint8_t* a2;   // the Q8_0 pair form only: a second copy of a[], two bytes further on
 };
+
+// Bytes of LDS the staging area needs for a k-element activation.
+#define JL_ACT_LDS_BYTES(k) ((k) + ((k) / 32) * 4 + ((k) / 16) * 4)
+// ... and with the second copy of the int8 values that the Q8_0 pair form reads (k % 64 == 0)
+#define JL_ACT_LDS_BYTES_SHIFTED(k) (JL_ACT_LDS_BYTES(k) + (k) + 16)
 
 __device__ __forceinline__ ActLds act_lds_views(uint8_t* smem, int k) {
     ActLds v;
     v.a = smem;
     v.da = (const float*)(smem + k);
     v.s16 = (const float*)(smem + k + (k / 32) * 4);
+    v.a2 = smem + JL_ACT_LDS_BYTES(k);   // 16-byte aligned when k % 64 == 0
     return v;
 }
 
-// Bytes of LDS the staging area needs for a k-element activation.
-#define JL_ACT_LDS_BYTES(k) ((k) + ((k) / 32) * 4 + ((k) / 16) * 4)
-
 // Stage pre-quantized activations (global) into LDS.  k % 32 == 0.
+// SH: also the copy two bytes further on (a2[i + 2] = a[i]), written as two 16-bit halves.
+template <bool SH = false>
 __device__ __forceinline__ void stage_act_copy(uint8_t* smem, const int8_t* q, const float* as,
                                                const float* s16, int k, int nthreads) {
     u32* a = (u32*)smem;
     float* da = (float*)(smem + k);
     float* ss = (float*)(smem + k + (k / 32) * 4);
-    for (int i = threadIdx.x; i < k / 4; i += nthreads) a[i] = ((const u32*)q)[i];
+    for (int i = threadIdx.x; i < k / 4; i += nthreads) {
+        const u32 v = ((const u32*)q)[i];
+        a[i] = v;
+        if (SH) {
+            uint16_t* h = (uint16_t*)(smem + JL_ACT_LDS_BYTES(k)) + 2 * i + 1;
+            h[0] = (uint16_t)v;
+            h[1] = (uint16_t)(v >> 16);
+        }
+    }
     for (int i = threadIdx.x; i < k / 32; i += nthreads) da[i] = as[i];
     for (int i = threadIdx.x; i < k / 16; i += nthreads) ss[i] = s16[i];
 }
 
 // Quantize one float4 of x (element group g4, i.e. elements 4*g4 .. 4*g4+3) into the
 // LDS staging area; every lane of a wavefront must call it together (DPP).
+template <bool SH = false>
 __device__ __forceinline__ void stage_quantize4(uint8_t* smem, int k, int per, int g4, f32x4 v) {
     u32* a = (u32*)smem;
     float* da = (float*)(smem + k);
@@ -65,6 +80,11 @@ __device__ __forceinline__ void stage_quantize4(uint8_t* smem, int k, int per, i
     u32 q = quantize4(v, amax, d, sum);
     if (live) {
         a[g4] = q;
+        if (SH) {
+            uint16_t* h = (uint16_t*)(smem + JL_ACT_LDS_BYTES(k)) + 2 * g4 + 1;
+            h[0] = (uint16_t)q;
+            h[1] = (uint16_t)(q >> 16);
+        }
         if ((g4 & 3) == 0) ss[g4 >> 2] = (float)sum;
         if ((g4 & 7) == 0) da[g4 >> 3] = d;
     }
@@ -73,15 +93,16 @@ __device__ __forceinline__ void stage_quantize4(uint8_t* smem, int k, int per, i
 // Quantize f32 x into the LDS staging area (same bits as the standalone
 // quantizer).  k % 32 == 0, blockDim.x % 64 == 0, per = window / 32.  `first` is
 // this thread's first float4 of x, loaded by the caller ahead of time.
+template <bool SH = false>
 __device__ __forceinline__ void stage_act_quantize(uint8_t* smem, const float* x, int k, int per,
                                                    f32x4 first, int nthreads) {
     const int n4 = k / 4;
     const int n4_pad = (n4 + 63) & ~63;  // whole wavefronts take part in the lane exchanges
     int g4 = threadIdx.x;
-    if (g4 < n4_pad) stage_quantize4(smem, k, per, g4, first);
+    if (g4 < n4_pad) stage_quantize4<SH>(smem, k, per, g4, first);
     for (g4 += nthreads; g4 < n4_pad; g4 += nthreads) {
         f32x4 v = g4 < n4 ? ((const f32x4*)x)[g4] : f32x4{0.f, 0.f, 0.f, 0.f};
-        stage_quantize4(smem, k, per, g4, v);
+        stage_quantize4<SH>(smem, k, per, g4, v);
     }
 }
 
@@ -228,6 +249,71 @@ __device__ __forceinline__ float dot_q8(const SlotWQ8& w, const SlotActQ8& s) {
     return dotp_q8(P, s);
 }
 
+// ------------------------------------------------- Q8_0, two blocks a slot
+// A 34-byte block leaves every second block's int8 values two bytes off a 32-bit boundary,
+// and a 16-byte load that is only 2-byte aligned is served at about three quarters of the
+// rate of one that is 4-byte aligned (a pure read of 62 MB: 14.2 against 11.2 us).  Two blocks
+// are 68 bytes, so a slot of two blocks is seventeen 4-byte-aligned words
+//   w0 = d0 | q0[0..1] << 16,  w1..w7 = q0[2..29],  w8 = q0[30..31] | d1 << 16,  w9..w16 = q1[0..31].
+// Block 1's values sit on word boundaries.  Block 0's sit two bytes into theirs: they meet a
+// second copy of the activations laid two bytes further on (ActLds.a2, so that word m of it is
+// a[4m-2 .. 4m+1]), with the scale halves of w0 and w8 masked off.
+// Rows must be 4-byte aligned and k a multiple of 64.
+#define JL_Q8_0P 1008   // (not a ggml type: the kernel form's tag)
+struct SlotActQ8P {
+    u32x4 s[2];   // a[-2 .. 29] of block 0, as the shifted copy has them
+    u32 s8;       // a[30 .. 33]
+    u32x4 a[2];   // a[0 .. 31] of block 1
+    float da0, da1;
+};
+
+__device__ __forceinline__ void load_act_q8p(const ActLds& A, int slot, SlotActQ8P& s) {
+    const u32* a2 = (const u32*)A.a2 + 16 * slot;
+    s.s[0] = *(const u32x4*)a2;
+    s.s[1] = *(const u32x4*)(a2 + 4);
+    s.s8 = a2[8];
+    const u32x4* a = (const u32x4*)(A.a + slot * 64 + 32);
+    s.a[0] = a[0]; s.a[1] = a[1];
+    s.da0 = A.da[2 * slot];
+    s.da1 = A.da[2 * slot + 1];
+}
+
+struct SlotWQ8P {
+    u32x4 q[4];
+    u32 t;
+};
+
+struct __attribute__((packed, aligned(4))) u32x4_a4 { u32x4 v; };
+__device__ __forceinline__ void load_w_q8p(const uint8_t* row, int slot, SlotWQ8P& w) {
+    const uint8_t* blk = row + (size_t)slot * 68;
+#pragma unroll
+    for (int i = 0; i < 4; i++) w.q[i] = ((const u32x4_a4*)(blk + 16 * i))->v;
+    w.t = *(const u32*)(blk + 64);
+}
+
+__device__ __forceinline__ float dot_q8p(const SlotWQ8P& w, const SlotActQ8P& s) {
+    i32 t0 = dot4(w.q[0].x & 0xFFFF0000u, s.s[0].x, 0);
+    t0 = dot4(w.q[0].y, s.s[0].y, t0);
+    t0 = dot4(w.q[0].z, s.s[0].z, t0);
+    t0 = dot4(w.q[0].w, s.s[0].w, t0);
+    t0 = dot4(w.q[1].x, s.s[1].x, t0);
+    t0 = dot4(w.q[1].y, s.s[1].y, t0);
+    t0 = dot4(w.q[1].z, s.s[1].z, t0);
+    t0 = dot4(w.q[1].w, s.s[1].w, t0);
+    t0 = dot4(w.q[2].x & 0x0000FFFFu, s.s8, t0);
+    i32 t1 = dot4(w.q[2].y, s.a[0].x, 0);
+    t1 = dot4(w.q[2].z, s.a[0].y, t1);
+    t1 = dot4(w.q[2].w, s.a[0].z, t1);
+    t1 = dot4(w.q[3].x, s.a[0].w, t1);
+    t1 = dot4(w.q[3].y, s.a[1].x, t1);
+    t1 = dot4(w.q[3].z, s.a[1].y, t1);
+    t1 = dot4(w.q[3].w, s.a[1].z, t1);
+    t1 = dot4(w.t, s.a[1].w, t1);
+    const float d0 = half_bits_to_f32((uint16_t)(w.q[0].x & 0xFFFF));
+    const float d1 = half_bits_to_f32((uint16_t)(w.q[2].x >> 16));
+    return (float)t0 * d0 * s.da0 + (float)t1 * d1 * s.da1;
+}
+
 // ---------------------------------------------------------------- Q6_K slot
 // slot = (super-block sb, half n, 16-run j): ql[16] (low nibbles = sub-block
 // 8n+j, high = 8n+4+j), ql[32+16] (sub-blocks 8n+2+j / 8n+6+j) and qh[16] (two
@@ -333,6 +419,13 @@ template <> struct SlotTraits<JL_Q8_0> {
     typedef PrepQ8 Prep;
     static __device__ __forceinline__ void prep(const W& w, int, Prep& P) { prep_q8(w, P); }
     static __device__ __forceinline__ float dotp(const Prep& P, const Act& a) { return dotp_q8(P, a); }
+};
+template <> struct SlotTraits<JL_Q8_0P> {
+    typedef SlotActQ8P Act; typedef SlotWQ8P W;
+    static constexpr int kElems = 64;
+    static __device__ __forceinline__ void load_act(const ActLds& A, int s, Act& a) { load_act_q8p(A, s, a); }
+    static __device__ __forceinline__ void load_w(const uint8_t* row, int s, W& w) { load_w_q8p(row, s, w); }
+    static __device__ __forceinline__ float dot(const W& w, int, const Act& a) { return dot_q8p(w, a); }
 };
 template <> struct SlotTraits<JL_Q6_K> {
     typedef SlotActQ6K Act; typedef SlotWQ6K W;
@@ -467,8 +560,9 @@ __device__ __forceinline__ void matvec_body(const MatVecArgs& p, uint8_t* smem) 
         for (int j = 0; j < RPW; j++)
             T::load_w(p.w + (size_t)min(r0 + j, p.nrows - 1) * p.row_bytes, s, w[j]);
     }
-    if (p.x) stage_act_quantize(smem, p.x, p.k, p.per, x0, nwaves * 64);
-    else stage_act_copy(smem, p.q, p.as, p.s16, p.k, nwaves * 64);
+    constexpr bool SH = TYPE == JL_Q8_0P;
+    if (p.x) stage_act_quantize<SH>(smem, p.x, p.k, p.per, x0, nwaves * 64);
+    else stage_act_copy<SH>(smem, p.q, p.as, p.s16, p.k, nwaves * 64);
     lds_barrier();   // orders the LDS staging only: the weight loads stay in flight
 
     matvec_rows<TYPE, RPW>(p.w, p.row_bytes, A, p.nrows, r0, group_stride, nslots, lane, w,
@@ -552,7 +646,7 @@ __device__ __forceinline__ void matvec_multi_body(const MatVecMultiArgs& p, uint
             if (p.norm_out && blockIdx.x == 0 && y == 0 && g4 < n4) ((f32x4*)p.norm_out)[g4] = v;
         }
         if (x2) v = f32x4{silu_f32(v.x) * u.x, silu_f32(v.y) * u.y, silu_f32(v.z) * u.z, silu_f32(v.w) * u.w};
-        stage_quantize4(smem, p.k, p.per, g4, v);
+        stage_quantize4<TYPE == JL_Q8_0P>(smem, p.k, p.per, g4, v);
     }
     lds_barrier();
 

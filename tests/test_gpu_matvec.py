@@ -163,6 +163,38 @@ def test_matvec_every_kernel_shape(dev, devbuf, t):
     dev.set_tuning(rpw=0, block=0, grid=0)
 
 
+@pytest.mark.parametrize("shape", [(300, 1024), (129, 14336), (70, 4160), (37, 96), (16 * 256 + 40, 2176)],
+                         ids=lambda s: f"{s[0]}x{s[1]}")
+def test_matvec_q8_0_both_row_forms(dev, devbuf, shape):
+    """Q8_0 rows in both forms of the kernel: two blocks a lane-slot with every load 4-byte
+    aligned (the library's pick when the rows are 4-byte aligned and hold an even number of
+    blocks: here every k but 96 and every base but the odd one) and one block a slot
+    (tuning matvec.q8pair = 2, also what a base that is only 2-byte aligned falls back to).
+    Each against the oracle, both windows, planted scales, every rows-per-wavefront variant."""
+    nrows, k = shape
+    t = quant.Q8_0
+    w = synth.random_weights(t, nrows, k, seed=nrows + k)
+    x = synth.activations(k, seed=k + 1)
+    wd, xd = devbuf(w), devbuf(x)
+    shifted = devbuf(shape=(w.size + 16,), dtype=np.uint8, fill=0)     # the same bytes two bytes further on
+    shifted.put(np.concatenate([np.zeros(2, np.uint8), w, np.zeros(14, np.uint8)]))
+    for window in (32, 256):
+        dev.SetActWindow(window)
+        want = _like_for_like(t, w, x, nrows, k, window)
+        for pair, base, rpw in [(0, wd.ptr, 0), (2, wd.ptr, 0), (0, shifted.ptr + 2, 0), (0, wd.ptr, 2), (0, wd.ptr, 4)]:
+            dev.set_tuning(q8pair=pair, rpw=rpw)
+            out = devbuf(shape=(nrows + 8,), dtype=np.float32, fill=np.float32(7e30))
+            assert dev.matvec_dev(out.ptr, t, base, xd.ptr, nrows, k)
+            dev.synchronize()
+            got = out.get()
+            assert np.all(got[nrows:] == np.float32(7e30)), "wrote past nrows"
+            e = nmse(got[:nrows], want)
+            assert e <= 1e-10, f"window {window} q8pair={pair} rpw={rpw} base%4={base % 4}: NMSE {e:.3e}"
+            out.free()
+    dev.set_tuning(q8pair=0, rpw=0)
+    dev.SetActWindow(32)
+
+
 @pytest.mark.parametrize("t", TYPES)
 def test_matvec_split_equals_fused(dev, devbuf, t):
     """Quantizer kernel + matvec over its output == the fused kernel, bit for bit."""
