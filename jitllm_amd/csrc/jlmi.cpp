@@ -30,6 +30,7 @@ const HipApi* H = nullptr;  // the process-wide HIP runtime, resolved by the fir
 
 struct Tuning {
     int rpw = 0, block = 0, grid = 0, pipe = 0;
+    int xpre = 0;               // decode matvec: 1 / 4 float4 groups of x a thread loads ahead of its weights
     int q8pair = 0;             // Q8_0 rows: 2 keeps one block a lane-slot (2-byte-aligned loads)
     int packed_rw = 0, packed_block = 0, moe_group = 0, moe_logits = 0, moe_q6k_cols = 0;
     int moe_shares = 0;
@@ -285,8 +286,9 @@ int matvec_launch(jl_ctx* c, float* out, int type, const void* w, const float* x
     // loop on this machine (Q8_0 14336 x 4096: 17.4 against 15.7 us; Q6_K 4096 x 14336: 15.1
     // against 14.2), so it stays off unless asked for
     a.pipe = c->tune.pipe == 1 ? 1 : 2;
+    const int xpre = c->tune.xpre == 1 || c->tune.xpre == 4 ? c->tune.xpre : (k / 4 > 2 * block ? 4 : 1);   // three groups a thread and more
     char name[64];
-    snprintf(name, sizeof name, "jl_matvec_%s_r%d", pair ? "q8_0p" : ti->tag, rpw);
+    snprintf(name, sizeof name, "jl_matvec_%s_r%d%s", pair ? "q8_0p" : ti->tag, rpw, xpre == 4 ? "_x4" : "");
     void* params[] = {&a};
     unsigned lds = (unsigned)(act_lds_bytes(k) + (pair ? (size_t)k + 16 : 0));
     return launch(c, name, (unsigned)grid, 1, (unsigned)block, lds, st, params);
@@ -335,11 +337,12 @@ int matvec_multi_launch(jl_ctx* c, int type, int m, float* const* outs, const vo
     if (gx > groups) gx = groups;
     if (gx < 1) gx = 1;
     a.nwaves = nwaves; a.ngroups = (int)gx;
+    const int xpre = c->tune.xpre == 1 || c->tune.xpre == 4 ? c->tune.xpre : (k / 4 > 2 * nwaves * 64 ? 4 : 1);
     char name[64];
     bool pair = !types;
     for (int i = 0; i < m && pair; i++) pair = q8_pair_form(c, type, ws[i], k);
     if (types) snprintf(name, sizeof name, "jl_matvec_segments");
-    else snprintf(name, sizeof name, "jl_matvec_multi_%s", pair ? "q8_0p" : ti->tag);
+    else snprintf(name, sizeof name, "jl_matvec_multi_%s%s", pair ? "q8_0p" : ti->tag, xpre == 4 ? "_x4" : "");
     void* params[] = {&a};
     unsigned lds = (unsigned)(act_lds_bytes(k) + (pair ? (size_t)k + 16 : 0));
     return launch(c, name, (unsigned)gx, (unsigned)m, nwaves * 64, lds, st, params);
@@ -1301,7 +1304,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     if (e != hipSuccess)
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
-    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_matvec_q8_0p_r1", "jl_matvec_q8_0p_r2", "jl_matvec_q8_0p_r4", "jl_matvec_multi_q8_0p", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_q4k_k2", "jl_gemm_q4k_k2_planes", "jl_gemm_prep_q4k_planes", "jl_gemm_q4k_r64_planes", "jl_gemm_q4k_wide_planes", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_group2_wide", "jl_moe_quant", "jl_moe_matvec_planes_q4k", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_prep_planes", "jl_moe_gemm_q4k", "jl_moe_g16_prep", "jl_moe_g16_prep_planes", "jl_moe_g16_prep_q6k", "jl_moe_g16_c1", "jl_moe_g16_c2", "jl_moe_g16_c3", "jl_moe_g16_f1", "jl_moe_g16_f2", "jl_moe_g16_f3", "jl_moe_g16_g1", "jl_moe_g16_g2", "jl_moe_g16_g3", "jl_moe_g16_d1", "jl_moe_g16_d2", "jl_moe_g16_d3", "jl_moe_g16p_c1", "jl_moe_g16p_c2", "jl_moe_g16p_c3", "jl_moe_g16p_f1", "jl_moe_g16p_f2", "jl_moe_g16p_f3", "jl_moe_g16p_g1", "jl_moe_g16p_g2", "jl_moe_g16p_g3", "jl_moe_g16p_d1", "jl_moe_g16p_d2", "jl_moe_g16p_d3", "jl_moe_g16q6_c1", "jl_moe_g16q6_c2", "jl_moe_g16q6_c3", "jl_moe_g16q6_f1", "jl_moe_g16q6_f2", "jl_moe_g16q6_f3", "jl_moe_g16q6_g1", "jl_moe_g16q6_g2", "jl_moe_g16q6_g3", "jl_moe_g16q6_d1", "jl_moe_g16q6_d2", "jl_moe_g16q6_d3", "jl_moe_gemm_r64", "jl_moe_gemm_r64_planes", "jl_moe_gemm_q6k_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_mxfp4_matvec1_b1", "jl_mxfp4_matvec1_b2", "jl_mxfp4_matvec1_b3", "jl_mxfp4_scaled_prep", "jl_mxfp4_scaled_gemm", "jl_mxfp4_planes_prep", "jl_mxfp4_planes_gemm", "jl_mxfp4_matvec_planes_r64", "jl_mxfp4_matvec_planes_r32", "jl_mxfp4_matvec_planes_r16", "jl_unpack_mxfp4", "jl_sum_parts", "jl_probe_read", "jl_probe_empty", "jl_probe_wait", "jl_probe_mfma", "jl_probe_mfma_v5",
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_matvec_q8_0p_r1", "jl_matvec_q8_0p_r2", "jl_matvec_q8_0p_r4", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_q4k_k2", "jl_gemm_q4k_k2_planes", "jl_gemm_prep_q4k_planes", "jl_gemm_q4k_r64_planes", "jl_gemm_q4k_wide_planes", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_group2_wide", "jl_moe_quant", "jl_moe_matvec_planes_q4k", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_prep_planes", "jl_moe_gemm_q4k", "jl_moe_g16_prep", "jl_moe_g16_prep_planes", "jl_moe_g16_prep_q6k", "jl_moe_g16_c1", "jl_moe_g16_c2", "jl_moe_g16_c3", "jl_moe_g16_f1", "jl_moe_g16_f2", "jl_moe_g16_f3", "jl_moe_g16_g1", "jl_moe_g16_g2", "jl_moe_g16_g3", "jl_moe_g16_d1", "jl_moe_g16_d2", "jl_moe_g16_d3", "jl_moe_g16p_c1", "jl_moe_g16p_c2", "jl_moe_g16p_c3", "jl_moe_g16p_f1", "jl_moe_g16p_f2", "jl_moe_g16p_f3", "jl_moe_g16p_g1", "jl_moe_g16p_g2", "jl_moe_g16p_g3", "jl_moe_g16p_d1", "jl_moe_g16p_d2", "jl_moe_g16p_d3", "jl_moe_g16q6_c1", "jl_moe_g16q6_c2", "jl_moe_g16q6_c3", "jl_moe_g16q6_f1", "jl_moe_g16q6_f2", "jl_moe_g16q6_f3", "jl_moe_g16q6_g1", "jl_moe_g16q6_g2", "jl_moe_g16q6_g3", "jl_moe_g16q6_d1", "jl_moe_g16q6_d2", "jl_moe_g16q6_d3", "jl_moe_gemm_r64", "jl_moe_gemm_r64_planes", "jl_moe_gemm_q6k_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_mxfp4_matvec1_b1", "jl_mxfp4_matvec1_b2", "jl_mxfp4_matvec1_b3", "jl_mxfp4_scaled_prep", "jl_mxfp4_scaled_gemm", "jl_mxfp4_planes_prep", "jl_mxfp4_planes_gemm", "jl_mxfp4_matvec_planes_r64", "jl_mxfp4_matvec_planes_r32", "jl_mxfp4_matvec_planes_r16", "jl_unpack_mxfp4", "jl_sum_parts", "jl_probe_read", "jl_probe_empty", "jl_probe_wait", "jl_probe_mfma", "jl_probe_mfma_v5",
                                       "jl_pack_weights", "jl_unpack_q4k", "jl_unpack_q6k", "jl_unpack_q8_0"};
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int rw : {16, 32, 64})
@@ -1315,8 +1318,13 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
             char nm[64];
             snprintf(nm, sizeof nm, "jl_matvec_%s_r%d", type_info(t)->tag, rpw);
             names.push_back(nm);
+            names.push_back(std::string(nm) + "_x4");
         }
-    for (const char* tag : {"q4k", "q8_0", "q6k"}) names.push_back(std::string("jl_matvec_multi_") + tag);
+    for (int rpw : {1, 2, 4}) names.push_back("jl_matvec_q8_0p_r" + std::to_string(rpw) + "_x4");
+    for (const char* tag : {"q4k", "q8_0", "q6k", "q8_0p"}) {
+        names.push_back(std::string("jl_matvec_multi_") + tag);
+        names.push_back(std::string("jl_matvec_multi_") + tag + "_x4");
+    }
     names.push_back("jl_matvec_segments");
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int rw : {16, 32, 64})
@@ -1415,6 +1423,7 @@ int jl_set_tuning(jl_ctx* c, const char* key, int value) {
     else if (!strcmp(key, "mxfp4.planes")) c->tune.mx_planes = value;
     else if (!strcmp(key, "mxfp4.scaled")) c->tune.mx_scaled = value;
     else if (!strcmp(key, "matvec.q8pair")) c->tune.q8pair = value;
+    else if (!strcmp(key, "matvec.xpre")) c->tune.xpre = value;
     else if (!strcmp(key, "gemm.form")) c->tune.gemm_form = value;
     else if (!strcmp(key, "gemm.split")) c->tune.gemm_split = value;
     else if (!strcmp(key, "gemm.prep")) c->tune.gemm_prep = value;

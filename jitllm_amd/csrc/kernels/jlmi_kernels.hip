@@ -48,9 +48,14 @@ extern "C" __global__ __launch_bounds__(256) void jl_dequant(
 // ---------------------------------------------------------------- matvec
 // jl_matvec_<type>_r<rows per wavefront>; the workgroup is 64..1024 threads.
 // MAXT is the largest workgroup the variant's register use allows.
+// _x4: the same for an activation longer than one float4 group a thread, whose first four
+// groups a thread loads together ahead of its weights.
 #define JL_MATVEC_KERNEL(T, TYPE, RPW, MAXT)                                                 \
     extern "C" __global__ __launch_bounds__(MAXT) void jl_matvec_##T##_r##RPW(MatVecArgs p) { \
-        matvec_body<TYPE, RPW>(p, jl_smem);                                                  \
+        matvec_body<TYPE, RPW, 1>(p, jl_smem);                                               \
+    }                                                                                        \
+    extern "C" __global__ __launch_bounds__(MAXT) void jl_matvec_##T##_r##RPW##_x4(MatVecArgs p) { \
+        matvec_body<TYPE, RPW, 4>(p, jl_smem);                                               \
     }
 JL_MATVEC_KERNEL(q4k, JL_Q4_K, 1, 1024) JL_MATVEC_KERNEL(q4k, JL_Q4_K, 2, 1024) JL_MATVEC_KERNEL(q4k, JL_Q4_K, 4, 512)
 JL_MATVEC_KERNEL(q8_0, JL_Q8_0, 1, 1024) JL_MATVEC_KERNEL(q8_0, JL_Q8_0, 2, 1024) JL_MATVEC_KERNEL(q8_0, JL_Q8_0, 4, 1024)
@@ -62,7 +67,10 @@ JL_MATVEC_KERNEL(q8_0p, JL_Q8_0P, 1, 1024) JL_MATVEC_KERNEL(q8_0p, JL_Q8_0P, 2, 
 // grid = (row groups, matrices), block = 64..1024
 #define JL_MATVEC_MULTI_KERNEL(T, TYPE)                                                                \
     extern "C" __global__ __launch_bounds__(1024) void jl_matvec_multi_##T(MatVecMultiArgs p) {        \
-        matvec_multi_body<TYPE>(p, jl_smem, p.row_bytes);                                              \
+        matvec_multi_body<TYPE, 1>(p, jl_smem, p.row_bytes);                                           \
+    }                                                                                                  \
+    extern "C" __global__ __launch_bounds__(1024) void jl_matvec_multi_##T##_x4(MatVecMultiArgs p) {   \
+        matvec_multi_body<TYPE, 4>(p, jl_smem, p.row_bytes);                                           \
     }
 JL_MATVEC_MULTI_KERNEL(q4k, JL_Q4_K) JL_MATVEC_MULTI_KERNEL(q8_0, JL_Q8_0) JL_MATVEC_MULTI_KERNEL(q6k, JL_Q6_K)
 JL_MATVEC_MULTI_KERNEL(q8_0p, JL_Q8_0P)

@@ -93,14 +93,29 @@ __device__ __forceinline__ void stage_quantize4(uint8_t* smem, int k, int per, i
 // Quantize f32 x into the LDS staging area (same bits as the standalone
 // quantizer).  k % 32 == 0, blockDim.x % 64 == 0, per = window / 32.  `first` is
 // this thread's first float4 of x, loaded by the caller ahead of time.
-template <bool SH = false>
+// This thread's first XP float4 groups of x (groups tid, tid + nthreads, ...), loaded
+// together so that their latency is paid once, under the first weight loads (a loop that
+// loads and quantizes a group at a time waits out a load per pass: at k = 14336 three and a
+// half passes, about two microseconds before the first row could start).
+// XP = 1 for a vector of at most one group a thread (no loads it has no use for go out ahead
+// of the weights), 4 for longer ones: the body is compiled for both and chosen once, at its top.
+template <int XP>
+__device__ __forceinline__ void load_x_groups(const float* x, int k, int nthreads, f32x4 (&xs)[XP]) {
+    const int n4 = k / 4;
+#pragma unroll
+    for (int i = 0; i < XP; i++) xs[i] = ((const f32x4*)x)[min((int)threadIdx.x + i * nthreads, n4 - 1)];
+}
+
+template <bool SH, int XP>
 __device__ __forceinline__ void stage_act_quantize(uint8_t* smem, const float* x, int k, int per,
-                                                   f32x4 first, int nthreads) {
+                                                   const f32x4 (&first)[XP], int nthreads) {
     const int n4 = k / 4;
     const int n4_pad = (n4 + 63) & ~63;  // whole wavefronts take part in the lane exchanges
     int g4 = threadIdx.x;
-    if (g4 < n4_pad) stage_quantize4<SH>(smem, k, per, g4, first);
-    for (g4 += nthreads; g4 < n4_pad; g4 += nthreads) {
+#pragma unroll
+    for (int i = 0; i < XP; i++, g4 += nthreads)
+        if (g4 < n4_pad) stage_quantize4<SH>(smem, k, per, g4, first[i]);   // (a group past n4 is not stored)
+    for (; g4 < n4_pad; g4 += nthreads) {
         f32x4 v = g4 < n4 ? ((const f32x4*)x)[g4] : f32x4{0.f, 0.f, 0.f, 0.f};
         stage_quantize4<SH>(smem, k, per, g4, v);
     }
@@ -532,8 +547,8 @@ __device__ __forceinline__ void matvec_rows(const uint8_t* w0, int row_bytes, co
 // activation is staged, so HBM latency overlaps the quantizer; after that each
 // group is load -> dot -> cross-lane reduce, and the wavefronts of a CU (two
 // workgroups of eight, or one of sixteen) cover each other's memory latency.
-template <int TYPE, int RPW>
-__device__ __forceinline__ void matvec_body(const MatVecArgs& p, uint8_t* smem) {
+template <int TYPE, int RPW, int XP>
+__device__ __forceinline__ void matvec_body_xp(const MatVecArgs& p, uint8_t* smem) {
     typedef SlotTraits<TYPE> T;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = p.nwaves;
     const int nslots = p.k / T::kElems;
@@ -547,9 +562,11 @@ __device__ __forceinline__ void matvec_body(const MatVecArgs& p, uint8_t* smem) 
     // wavefront issues its x load, the workgroup meets at a barrier that waits for no
     // data, and only then do the weight loads go out.  The quantizer starts as soon as x
     // is back while the first weight loads are still in flight.
-    f32x4 x0 = f32x4{0.f, 0.f, 0.f, 0.f};
+    f32x4 x0[XP];
+#pragma unroll
+    for (int i = 0; i < XP; i++) x0[i] = f32x4{0.f, 0.f, 0.f, 0.f};
     if (p.x) {
-        x0 = ((const f32x4*)p.x)[min((int)threadIdx.x, p.k / 4 - 1)];
+        load_x_groups<XP>(p.x, p.k, nwaves * 64, x0);
         __builtin_amdgcn_s_barrier();
     }
 
@@ -561,12 +578,19 @@ __device__ __forceinline__ void matvec_body(const MatVecArgs& p, uint8_t* smem) 
             T::load_w(p.w + (size_t)min(r0 + j, p.nrows - 1) * p.row_bytes, s, w[j]);
     }
     constexpr bool SH = TYPE == JL_Q8_0P;
-    if (p.x) stage_act_quantize<SH>(smem, p.x, p.k, p.per, x0, nwaves * 64);
+    if (p.x) stage_act_quantize<SH, XP>(smem, p.x, p.k, p.per, x0, nwaves * 64);
     else stage_act_copy<SH>(smem, p.q, p.as, p.s16, p.k, nwaves * 64);
     lds_barrier();   // orders the LDS staging only: the weight loads stay in flight
 
     matvec_rows<TYPE, RPW>(p.w, p.row_bytes, A, p.nrows, r0, group_stride, nslots, lane, w,
                            [&](int r, float t) { p.out[r] = t; }, p.pipe != 2);
+}
+
+// XP = 1: a vector of at most one float4 group a thread; 4: longer ones (the host picks the
+// entry point; one body compiled for both behind a branch ran the short-vector case 10 % slower).
+template <int TYPE, int RPW, int XP = 1>
+__device__ __forceinline__ void matvec_body(const MatVecArgs& p, uint8_t* smem) {
+    matvec_body_xp<TYPE, RPW, XP>(p, smem);
 }
 
 // Several matvecs of one type in one launch: grid = (row groups, matrices).  Each
@@ -591,8 +615,8 @@ __device__ __forceinline__ float resid_weight(float alpha, const float* gate) {
     return alpha * (float)(1.0 / (1.0 + exp(-(double)*gate)));
 }
 
-template <int TYPE>
-__device__ __forceinline__ void matvec_multi_body(const MatVecMultiArgs& p, uint8_t* smem, int row_bytes) {
+template <int TYPE, int XP>
+__device__ __forceinline__ void matvec_multi_body_xp(const MatVecMultiArgs& p, uint8_t* smem, int row_bytes) {
     typedef SlotTraits<TYPE> T;
     const int y = blockIdx.y;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = p.nwaves;
@@ -608,8 +632,13 @@ __device__ __forceinline__ void matvec_multi_body(const MatVecMultiArgs& p, uint
     const float* x2 = p.x2 ? p.x2 + (size_t)y * p.xstride : nullptr;
 
     const int n4 = p.k / 4, n4_pad = (n4 + 63) & ~63;
-    f32x4 x0 = ((const f32x4*)x)[min((int)threadIdx.x, n4 - 1)];
-    f32x4 u0 = x2 ? ((const f32x4*)x2)[min((int)threadIdx.x, n4 - 1)] : f32x4{1.f, 1.f, 1.f, 1.f};
+    f32x4 x0[XP], u0[XP];
+    load_x_groups<XP>(x, p.k, nthreads, x0);
+    if (x2) load_x_groups<XP>(x2, p.k, nthreads, u0);
+    else {
+#pragma unroll
+        for (int i = 0; i < XP; i++) u0[i] = f32x4{1.f, 1.f, 1.f, 1.f};
+    }
     __builtin_amdgcn_s_barrier();   // activation loads of the whole workgroup go out first
     typename T::W w[1];
     T::load_w(w0 + (size_t)min(r0, nrows - 1) * row_bytes, min(lane, nslots - 1), w[0]);
@@ -620,8 +649,14 @@ __device__ __forceinline__ void matvec_multi_body(const MatVecMultiArgs& p, uint
     double nscale = 0.0;
     if (p.norm_w) {
         double ss = 0.0;
-        for (int g4 = threadIdx.x; g4 < n4; g4 += nthreads) {
-            const f32x4 v = g4 == (int)threadIdx.x ? x0 : ((const f32x4*)x)[g4];
+        int g4 = threadIdx.x;
+#pragma unroll
+        for (int i = 0; i < XP; i++, g4 += nthreads) {
+            const f32x4 v = x0[i];
+            if (g4 < n4) ss += (double)v.x * v.x + (double)v.y * v.y + (double)v.z * v.z + (double)v.w * v.w;
+        }
+        for (; g4 < n4; g4 += nthreads) {
+            const f32x4 v = ((const f32x4*)x)[g4];
             ss += (double)v.x * v.x + (double)v.y * v.y + (double)v.z * v.z + (double)v.w * v.w;
         }
         ss = wave_sum_f64(ss);
@@ -633,12 +668,7 @@ __device__ __forceinline__ void matvec_multi_body(const MatVecMultiArgs& p, uint
         __syncthreads();               // everyone has read before the quantizer writes
         nscale = 1.0 / __builtin_sqrt(tot / (double)p.k + (double)p.norm_eps);
     }
-    for (int g4 = threadIdx.x; g4 < n4_pad; g4 += nthreads) {
-        f32x4 v = x0, u = u0;
-        if (g4 != (int)threadIdx.x) {
-            v = ((const f32x4*)x)[min(g4, n4 - 1)];
-            if (x2) u = ((const f32x4*)x2)[min(g4, n4 - 1)];
-        }
+    auto stage_group = [&](int g4, f32x4 v, f32x4 u) __attribute__((always_inline)) {
         if (p.norm_w) {
             const f32x4 nw = ((const f32x4*)p.norm_w)[min(g4, n4 - 1)];
             v = f32x4{(float)((double)v.x * nscale * (double)nw.x), (float)((double)v.y * nscale * (double)nw.y),
@@ -647,6 +677,15 @@ __device__ __forceinline__ void matvec_multi_body(const MatVecMultiArgs& p, uint
         }
         if (x2) v = f32x4{silu_f32(v.x) * u.x, silu_f32(v.y) * u.y, silu_f32(v.z) * u.z, silu_f32(v.w) * u.w};
         stage_quantize4<TYPE == JL_Q8_0P>(smem, p.k, p.per, g4, v);
+    };
+    {
+        int g4 = threadIdx.x;
+#pragma unroll
+        for (int i = 0; i < XP; i++, g4 += nthreads)
+            if (g4 < n4_pad) stage_group(g4, x0[i], u0[i]);
+        for (; g4 < n4_pad; g4 += nthreads)
+            stage_group(g4, ((const f32x4*)x)[min(g4, n4 - 1)],
+                        x2 ? ((const f32x4*)x2)[min(g4, n4 - 1)] : f32x4{1.f, 1.f, 1.f, 1.f});
     }
     lds_barrier();
 
@@ -656,4 +695,9 @@ __device__ __forceinline__ void matvec_multi_body(const MatVecMultiArgs& p, uint
         outp[r] = t;
         if (resid) resid[r] += resid_weight(p.alpha, p.resid_gate) * t;
     }, false);
+}
+
+template <int TYPE, int XP = 1>
+__device__ __forceinline__ void matvec_multi_body(const MatVecMultiArgs& p, uint8_t* smem, int row_bytes) {
+    matvec_multi_body_xp<TYPE, XP>(p, smem, row_bytes);
 }
