@@ -17,6 +17,9 @@ struct MatVecArgs {
     int nwaves;          // wavefronts per workgroup (the launch's block / 64)
     int ngroups;         // workgroups (the launch's grid)
     int pipe;            // 2: the plain row loop; else the two-deep pipeline where a wavefront has several steps
+    float* resid;        // optional: resid[r] += alpha * out[r] (times sigmoid(*resid_gate) when resid_gate is set)
+    const float* resid_gate;
+    float alpha;
 };
 
 // Several decode matvecs of one type in one launch (grid y = matrix): matrix i computes
@@ -38,6 +41,10 @@ struct MatVecMultiArgs {
     // the mixed-type kernel only: each matrix's type (JL_TYPE_*) and bytes per row
     int type[JL_MAX_MULTI];
     int row_bytes_of[JL_MAX_MULTI];
+    // the _q entry points: one activation for every matrix, quantized beforehand (x unused)
+    const int8_t* q;
+    const float* as;
+    const float* s16;
     const float* norm_w; // null: none; else the activation is RMSNorm(x) * norm_w first
     float* norm_out;     // optional: the normed activation, written once
     float norm_eps;

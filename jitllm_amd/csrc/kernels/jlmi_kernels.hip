@@ -19,13 +19,19 @@ extern __shared__ __attribute__((aligned(16))) uint8_t jl_smem[];
 // ------------------------------------------------------------- quantizer
 // x [ntok][k] f32 -> q [ntok][k] int8, as [ntok][k/32], sum16 [ntok][k/16].
 // grid = (ceil(k/4/256), ntok), block = 256: one thread per four elements.
+// x2 (may be null): the activation is silu(x) * x2, the gated feed-forward block's, formed
+// with the arithmetic of the fused matvec's own quantizer.
 extern "C" __global__ __launch_bounds__(256) void jl_quantize_act(
     const float* __restrict__ x, int8_t* __restrict__ q, float* __restrict__ as,
-    float* __restrict__ sum16, int k, int per) {
+    float* __restrict__ sum16, int k, int per, const float* __restrict__ x2) {
     const size_t tok = blockIdx.y;
     const int g4 = blockIdx.x * 256 + threadIdx.x;
     const bool live = g4 < k / 4;
     f32x4 v = live ? ((const f32x4*)(x + tok * (size_t)k))[g4] : f32x4{0.f, 0.f, 0.f, 0.f};
+    if (x2) {
+        const f32x4 u = live ? ((const f32x4*)(x2 + tok * (size_t)k))[g4] : f32x4{0.f, 0.f, 0.f, 0.f};
+        v = f32x4{silu_f32(v.x) * u.x, silu_f32(v.y) * u.y, silu_f32(v.z) * u.z, silu_f32(v.w) * u.w};
+    }
     u32 m = max(max(abs_bits(v.x), abs_bits(v.y)), max(abs_bits(v.z), abs_bits(v.w)));
     u32 amax = window_amax(live ? m : 0u, per);
     float d;
@@ -71,6 +77,9 @@ JL_MATVEC_KERNEL(q8_0p, JL_Q8_0P, 1, 1024) JL_MATVEC_KERNEL(q8_0p, JL_Q8_0P, 2, 
     }                                                                                                  \
     extern "C" __global__ __launch_bounds__(1024) void jl_matvec_multi_##T##_x4(MatVecMultiArgs p) {   \
         matvec_multi_body<TYPE, 4>(p, jl_smem, p.row_bytes);                                           \
+    }                                                                                                  \
+    extern "C" __global__ __launch_bounds__(1024) void jl_matvec_multi_##T##_q(MatVecMultiArgs p) {    \
+        matvec_multi_body<TYPE, 0>(p, jl_smem, p.row_bytes);                                           \
     }
 JL_MATVEC_MULTI_KERNEL(q4k, JL_Q4_K) JL_MATVEC_MULTI_KERNEL(q8_0, JL_Q8_0) JL_MATVEC_MULTI_KERNEL(q6k, JL_Q6_K)
 JL_MATVEC_MULTI_KERNEL(q8_0p, JL_Q8_0P)

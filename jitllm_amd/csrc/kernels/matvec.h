@@ -542,6 +542,14 @@ __device__ __forceinline__ void matvec_rows(const uint8_t* w0, int row_bytes, co
     }
 }
 
+// Weight of a residual add: alpha, or alpha * sigmoid(logit) when the add is gated by a
+// logit in device memory (a shared expert's contribution, engine/model/moe.go:401-497;
+// sigma(x) = 1/(1+exp(-x)) in f64, narrowed once, internal/oracle/moe.go:361-370).
+__device__ __forceinline__ float resid_weight(float alpha, const float* gate) {
+    if (!gate) return alpha;
+    return alpha * (float)(1.0 / (1.0 + exp(-(double)*gate)));
+}
+
 // One wavefront computes RPW rows at a time and strides over the row groups of
 // a persistent grid.  The first group's weight loads are issued before the
 // activation is staged, so HBM latency overlaps the quantizer; after that each
@@ -582,8 +590,11 @@ __device__ __forceinline__ void matvec_body_xp(const MatVecArgs& p, uint8_t* sme
     else stage_act_copy<SH>(smem, p.q, p.as, p.s16, p.k, nwaves * 64);
     lds_barrier();   // orders the LDS staging only: the weight loads stay in flight
 
-    matvec_rows<TYPE, RPW>(p.w, p.row_bytes, A, p.nrows, r0, group_stride, nslots, lane, w,
-                           [&](int r, float t) { p.out[r] = t; }, p.pipe != 2);
+    float* const resid = p.resid;
+    matvec_rows<TYPE, RPW>(p.w, p.row_bytes, A, p.nrows, r0, group_stride, nslots, lane, w, [&](int r, float t) {
+        p.out[r] = t;
+        if (resid) resid[r] += resid_weight(p.alpha, p.resid_gate) * t;
+    }, p.pipe != 2);
 }
 
 // XP = 1: a vector of at most one float4 group a thread; 4: longer ones (the host picks the
@@ -607,14 +618,10 @@ __device__ __forceinline__ double wave_sum_f64(double v) {
     return v;
 }
 
-// Weight of a residual add: alpha, or alpha * sigmoid(logit) when the add is gated by a
-// logit in device memory (a shared expert's contribution, engine/model/moe.go:401-497;
-// sigma(x) = 1/(1+exp(-x)) in f64, narrowed once, internal/oracle/moe.go:361-370).
-__device__ __forceinline__ float resid_weight(float alpha, const float* gate) {
-    if (!gate) return alpha;
-    return alpha * (float)(1.0 / (1.0 + exp(-(double)*gate)));
-}
-
+// XP = 0: the activation comes quantized (MatVecMultiArgs.q / as / s16, one for all matrices):
+// a long gated activation is formed and quantized once by the quantizer kernel instead of by
+// every workgroup (silu and its division for 14336 elements in each of 256 workgroups cost the
+// down projection of a feed-forward block 6 of its 20 us).
 template <int TYPE, int XP>
 __device__ __forceinline__ void matvec_multi_body_xp(const MatVecMultiArgs& p, uint8_t* smem, int row_bytes) {
     typedef SlotTraits<TYPE> T;
@@ -628,6 +635,19 @@ __device__ __forceinline__ void matvec_multi_body_xp(const MatVecMultiArgs& p, u
     int r0 = blockIdx.x * nwaves + wave;
     if ((int)blockIdx.x * nwaves >= nrows) return;   // uniform: this matrix has fewer row groups
     const uint8_t* w0 = p.w[y];
+    if constexpr (XP == 0) {
+        typename T::W w[1];
+        T::load_w(w0 + (size_t)min(r0, nrows - 1) * row_bytes, min(lane, nslots - 1), w[0]);
+        stage_act_copy<TYPE == JL_Q8_0P>(smem, p.q, p.as, p.s16, p.k, nthreads);
+        lds_barrier();
+        float* const outp = p.out[y];
+        float* const resid = y == 0 ? p.resid : nullptr;
+        matvec_rows<TYPE, 1>(w0, row_bytes, A, nrows, r0, group_stride, nslots, lane, w, [&](int r, float t) {
+            outp[r] = t;
+            if (resid) resid[r] += resid_weight(p.alpha, p.resid_gate) * t;
+        }, false);
+        return;
+    } else {
     const float* x = p.x + (size_t)y * p.xstride;
     const float* x2 = p.x2 ? p.x2 + (size_t)y * p.xstride : nullptr;
 
@@ -639,6 +659,10 @@ __device__ __forceinline__ void matvec_multi_body_xp(const MatVecMultiArgs& p, u
 #pragma unroll
         for (int i = 0; i < XP; i++) u0[i] = f32x4{1.f, 1.f, 1.f, 1.f};
     }
+    f32x4 nw0[XP];   // the norm weights of the same groups
+#pragma unroll
+    for (int i = 0; i < XP; i++) nw0[i] = f32x4{1.f, 1.f, 1.f, 1.f};
+    if (p.norm_w) load_x_groups<XP>(p.norm_w, p.k, nthreads, nw0);
     __builtin_amdgcn_s_barrier();   // activation loads of the whole workgroup go out first
     typename T::W w[1];
     T::load_w(w0 + (size_t)min(r0, nrows - 1) * row_bytes, min(lane, nslots - 1), w[0]);
@@ -662,15 +686,14 @@ __device__ __forceinline__ void matvec_multi_body_xp(const MatVecMultiArgs& p, u
         ss = wave_sum_f64(ss);
         double* red = (double*)smem;   // the staging area is not in use yet
         if (lane == 0) red[wave] = ss;
-        __syncthreads();
+        lds_barrier();                 // (orders LDS only: the first weight loads stay in flight)
         double tot = 0.0;
         for (int i = 0; i < nwaves; i++) tot += red[i];
-        __syncthreads();               // everyone has read before the quantizer writes
+        lds_barrier();                 // everyone has read before the quantizer writes
         nscale = 1.0 / __builtin_sqrt(tot / (double)p.k + (double)p.norm_eps);
     }
-    auto stage_group = [&](int g4, f32x4 v, f32x4 u) __attribute__((always_inline)) {
+    auto stage_group = [&](int g4, f32x4 v, f32x4 u, f32x4 nw) __attribute__((always_inline)) {
         if (p.norm_w) {
-            const f32x4 nw = ((const f32x4*)p.norm_w)[min(g4, n4 - 1)];
             v = f32x4{(float)((double)v.x * nscale * (double)nw.x), (float)((double)v.y * nscale * (double)nw.y),
                       (float)((double)v.z * nscale * (double)nw.z), (float)((double)v.w * nscale * (double)nw.w)};
             if (p.norm_out && blockIdx.x == 0 && y == 0 && g4 < n4) ((f32x4*)p.norm_out)[g4] = v;
@@ -682,19 +705,23 @@ __device__ __forceinline__ void matvec_multi_body_xp(const MatVecMultiArgs& p, u
         int g4 = threadIdx.x;
 #pragma unroll
         for (int i = 0; i < XP; i++, g4 += nthreads)
-            if (g4 < n4_pad) stage_group(g4, x0[i], u0[i]);
+            if (g4 < n4_pad) stage_group(g4, x0[i], u0[i], nw0[i]);
         for (; g4 < n4_pad; g4 += nthreads)
             stage_group(g4, ((const f32x4*)x)[min(g4, n4 - 1)],
-                        x2 ? ((const f32x4*)x2)[min(g4, n4 - 1)] : f32x4{1.f, 1.f, 1.f, 1.f});
+                        x2 ? ((const f32x4*)x2)[min(g4, n4 - 1)] : f32x4{1.f, 1.f, 1.f, 1.f},
+                        p.norm_w ? ((const f32x4*)p.norm_w)[min(g4, n4 - 1)] : f32x4{1.f, 1.f, 1.f, 1.f});
     }
     lds_barrier();
 
     float* const outp = p.out[y];
     float* const resid = y == 0 ? p.resid : nullptr;
+    // (a second step of weights requested ahead of the staging, for the launches with an RMSNorm or
+    // a gated activation in front, measured slower: gate + up 26.2 -> 32.8 us, down 14.5 -> 16.9)
     matvec_rows<TYPE, 1>(w0, row_bytes, A, nrows, r0, group_stride, nslots, lane, w, [&](int r, float t) {
         outp[r] = t;
         if (resid) resid[r] += resid_weight(p.alpha, p.resid_gate) * t;
     }, false);
+    }
 }
 
 template <int TYPE, int XP = 1>

@@ -78,6 +78,44 @@ def test_group_with_rmsnorm_in_front(dev, devbuf, k, window):
     dev.SetActWindow(32)
 
 
+@pytest.mark.parametrize("t_d,n_ffn,window", [(quant.Q6_K, 14336, 32), (quant.Q8_0, 9216, 32), (quant.Q4_K, 11008 // 256 * 256, 256)],
+                         ids=["q6_k_14336", "q8_0_9216", "q4_k_10752"])
+def test_group_long_gated_activation_quantized_once(dev, devbuf, t_d, n_ffn, window):
+    """A gated down projection with a long activation (three float4 groups a thread and more, each
+    thread's groups loaded together ahead of its weights): silu(gate) * up formed by every
+    workgroup (one launch, the default) and formed and quantized once by the quantizer kernel with
+    the matvec staging the int8 copy (two launches, matvec.act_split = 1).  Both against the
+    oracle, and bit for bit against each other; the residual add rides on either."""
+    n_embd = 200
+    dev.SetActWindow(window)
+    wdn = synth.quantized_weights(t_d, n_embd, n_ffn, seed=3)
+    gh = synth.activations(n_ffn, seed=6) * np.float32(2.0)
+    uh = synth.activations(n_ffn, seed=7)
+    h = (silu(gh) * uh.astype(np.float64)).astype(np.float32)
+    want = _want(t_d, wdn, h, n_embd, n_ffn, window)
+    dwd, g, u = devbuf(wdn), devbuf(gh), devbuf(uh)
+    resid0 = synth.activations(n_embd, seed=5)
+    got = {}
+    for split, launches in ((0, 1), (1, 2)):
+        dev.set_tuning(act_split=split)
+        resid = devbuf(resid0)
+        y = devbuf(shape=(n_embd + 4,), dtype=np.float32, fill=np.float32(5e30))
+        before = dev.launch_count()
+        assert dev.matvec_group_dev([y.ptr], [t_d], [dwd.ptr], [n_embd], g.ptr, n_ffn, act_up=u.ptr,
+                                    resid=resid.ptr, alpha=0.5)
+        assert dev.launch_count() == before + launches
+        dev.synchronize()
+        yh = y.get()
+        assert np.all(yh[n_embd:] == np.float32(5e30))
+        got[split] = yh[:n_embd]
+        assert rel_l2(got[split], want) <= 1e-3
+        assert np.array_equal(resid.get(), (resid0 + (np.float32(0.5) * got[split]).astype(np.float32)).astype(np.float32))
+        assert np.array_equal(g.get(), gh), "the activation operand must be left as it was"
+    dev.set_tuning(act_split=0)
+    assert np.array_equal(got[0].view(np.uint32), got[1].view(np.uint32)), "quantized once != quantized by every workgroup"
+    dev.SetActWindow(32)
+
+
 def test_group_gate_up_then_gated_down_with_residual(dev, devbuf):
     """A gated feed-forward block as two groups: (gate, up) sharing x, then down over
     silu(gate) * up with the residual add riding on the launch."""
