@@ -393,7 +393,8 @@ int matvec_multi_launch(jl_ctx* c, int type, int m, float* const* outs, const vo
     if (types) snprintf(name, sizeof name, "jl_matvec_segments");
     else snprintf(name, sizeof name, "jl_matvec_multi_%s%s", pair ? "q8_0p" : ti->tag, xpre == 4 ? "_x4" : "");
     void* params[] = {&a};
-    unsigned lds = (unsigned)(act_lds_bytes(k) + (pair ? (size_t)k + 16 : 0));
+    // (+ 16 to round the staging area up, + JL_NORM_LDS_BYTES for the RMSNorm's partial sums)
+    unsigned lds = (unsigned)(act_lds_bytes(k) + (pair ? (size_t)k + 16 : 0) + 16 + 160);
     return launch(c, name, (unsigned)gx, (unsigned)m, nwaves * 64, lds, st, params);
 }
 

@@ -65,7 +65,8 @@ extern "C" __global__ __launch_bounds__(256) void jl_dequant(
     }
 JL_MATVEC_KERNEL(q4k, JL_Q4_K, 1, 1024) JL_MATVEC_KERNEL(q4k, JL_Q4_K, 2, 1024) JL_MATVEC_KERNEL(q4k, JL_Q4_K, 4, 512)
 JL_MATVEC_KERNEL(q8_0, JL_Q8_0, 1, 1024) JL_MATVEC_KERNEL(q8_0, JL_Q8_0, 2, 1024) JL_MATVEC_KERNEL(q8_0, JL_Q8_0, 4, 1024)
-JL_MATVEC_KERNEL(q6k, JL_Q6_K, 1, 1024) JL_MATVEC_KERNEL(q6k, JL_Q6_K, 2, 512) JL_MATVEC_KERNEL(q6k, JL_Q6_K, 4, 512)
+// (Q6_K over the staging layout made for it: JL_STAGE_Q6K in kernels/matvec.h)
+JL_MATVEC_KERNEL(q6k, JL_Q6_KS, 1, 1024) JL_MATVEC_KERNEL(q6k, JL_Q6_KS, 2, 512) JL_MATVEC_KERNEL(q6k, JL_Q6_KS, 4, 512)
 // Q8_0 with two blocks a lane-slot, every load 4-byte aligned (rows 4-byte aligned, k % 64 == 0);
 // dynamic LDS = JL_ACT_LDS_BYTES_SHIFTED(k)
 JL_MATVEC_KERNEL(q8_0p, JL_Q8_0P, 1, 1024) JL_MATVEC_KERNEL(q8_0p, JL_Q8_0P, 2, 1024) JL_MATVEC_KERNEL(q8_0p, JL_Q8_0P, 4, 512)
@@ -81,7 +82,7 @@ JL_MATVEC_KERNEL(q8_0p, JL_Q8_0P, 1, 1024) JL_MATVEC_KERNEL(q8_0p, JL_Q8_0P, 2, 
     extern "C" __global__ __launch_bounds__(1024) void jl_matvec_multi_##T##_q(MatVecMultiArgs p) {    \
         matvec_multi_body<TYPE, 0>(p, jl_smem, p.row_bytes);                                           \
     }
-JL_MATVEC_MULTI_KERNEL(q4k, JL_Q4_K) JL_MATVEC_MULTI_KERNEL(q8_0, JL_Q8_0) JL_MATVEC_MULTI_KERNEL(q6k, JL_Q6_K)
+JL_MATVEC_MULTI_KERNEL(q4k, JL_Q4_K) JL_MATVEC_MULTI_KERNEL(q8_0, JL_Q8_0) JL_MATVEC_MULTI_KERNEL(q6k, JL_Q6_KS)
 JL_MATVEC_MULTI_KERNEL(q8_0p, JL_Q8_0P)
 // The same grid over matrices of different types (the reference's MatVecSegments,
 // jit/gpu/kernels/matvec.go:1411-1431: a block's q, k and v in one launch whatever their
@@ -92,7 +93,7 @@ extern "C" __global__ __launch_bounds__(1024) void jl_matvec_segments(MatVecMult
     switch (p.type[y]) {
     case JL_Q4_K: matvec_multi_body<JL_Q4_K>(p, jl_smem, p.row_bytes_of[y]); break;
     case JL_Q8_0: matvec_multi_body<JL_Q8_0>(p, jl_smem, p.row_bytes_of[y]); break;
-    case JL_Q6_K: matvec_multi_body<JL_Q6_K>(p, jl_smem, p.row_bytes_of[y]); break;
+    case JL_Q6_K: matvec_multi_body<JL_Q6_KS>(p, jl_smem, p.row_bytes_of[y]); break;
     }
 }
 

@@ -22,6 +22,8 @@
 #include "common.h"
 #include "quantize.h"
 
+struct __attribute__((packed, aligned(4))) u32x4_a4 { u32x4 v; };   // a 16-byte load on a 4-byte boundary
+
 // Activation staging area in LDS: int8 a[k], then f32 da[k/32], then f32 s16[k/16].
 struct ActLds {
     const uint8_t* a;
@@ -32,6 +34,8 @@ struct ActLds {
 
 // Bytes of LDS the staging area needs for a k-element activation.
 #define JL_ACT_LDS_BYTES(k) ((k) + ((k) / 32) * 4 + ((k) / 16) * 4)
+// the grouped kernels' RMSNorm: up to sixteen partial sums and the scale, behind the staging area
+#define JL_NORM_LDS_BYTES 160
 // ... and with the second copy of the int8 values that the Q8_0 pair form reads (k % 64 == 0)
 #define JL_ACT_LDS_BYTES_SHIFTED(k) (JL_ACT_LDS_BYTES(k) + (k) + 16)
 
@@ -45,8 +49,21 @@ __device__ __forceinline__ ActLds act_lds_views(uint8_t* smem, int k) {
 }
 
 // Stage pre-quantized activations (global) into LDS.  k % 32 == 0.
-// SH: also the copy two bytes further on (a2[i + 2] = a[i]), written as two 16-bit halves.
-template <bool SH = false>
+// Layouts of the staging area.  JL_STAGE_SHIFTED: also the copy two bytes further on
+// (a2[i + 2] = a[i]), written as two 16-bit halves.  JL_STAGE_Q6K: the half-block sums as the
+// Q6_K slot wants them -- the integer -32 * sum (the zero point of a 6-bit weight times the
+// sum, what its dot-product accumulator starts from), and the eight sums of a 128-element
+// half laid (j, q) -> 4 j + q for the sum of elements 32 q + 16 j .., so that the four runs of
+// a slot are one 16-byte read.
+#define JL_STAGE_PLAIN 0
+#define JL_STAGE_SHIFTED 1
+#define JL_STAGE_Q6K 2
+__device__ __forceinline__ int stage_q6k_sum_index(int h) {   // h = element / 16
+    const int p = h & 7;
+    return (h & ~7) + ((p & 1) << 2) + (p >> 1);
+}
+
+template <int SH = JL_STAGE_PLAIN>
 __device__ __forceinline__ void stage_act_copy(uint8_t* smem, const int8_t* q, const float* as,
                                                const float* s16, int k, int nthreads) {
     u32* a = (u32*)smem;
@@ -55,19 +72,22 @@ __device__ __forceinline__ void stage_act_copy(uint8_t* smem, const int8_t* q, c
     for (int i = threadIdx.x; i < k / 4; i += nthreads) {
         const u32 v = ((const u32*)q)[i];
         a[i] = v;
-        if (SH) {
+        if (SH == JL_STAGE_SHIFTED) {
             uint16_t* h = (uint16_t*)(smem + JL_ACT_LDS_BYTES(k)) + 2 * i + 1;
             h[0] = (uint16_t)v;
             h[1] = (uint16_t)(v >> 16);
         }
     }
     for (int i = threadIdx.x; i < k / 32; i += nthreads) da[i] = as[i];
-    for (int i = threadIdx.x; i < k / 16; i += nthreads) ss[i] = s16[i];
+    for (int i = threadIdx.x; i < k / 16; i += nthreads) {
+        if (SH == JL_STAGE_Q6K) ((i32*)ss)[stage_q6k_sum_index(i)] = -32 * (i32)s16[i];
+        else ss[i] = s16[i];
+    }
 }
 
 // Quantize one float4 of x (element group g4, i.e. elements 4*g4 .. 4*g4+3) into the
 // LDS staging area; every lane of a wavefront must call it together (DPP).
-template <bool SH = false>
+template <int SH = JL_STAGE_PLAIN>
 __device__ __forceinline__ void stage_quantize4(uint8_t* smem, int k, int per, int g4, f32x4 v) {
     u32* a = (u32*)smem;
     float* da = (float*)(smem + k);
@@ -80,12 +100,15 @@ __device__ __forceinline__ void stage_quantize4(uint8_t* smem, int k, int per, i
     u32 q = quantize4(v, amax, d, sum);
     if (live) {
         a[g4] = q;
-        if (SH) {
+        if (SH == JL_STAGE_SHIFTED) {
             uint16_t* h = (uint16_t*)(smem + JL_ACT_LDS_BYTES(k)) + 2 * g4 + 1;
             h[0] = (uint16_t)q;
             h[1] = (uint16_t)(q >> 16);
         }
-        if ((g4 & 3) == 0) ss[g4 >> 2] = (float)sum;
+        if ((g4 & 3) == 0) {
+            if (SH == JL_STAGE_Q6K) ((i32*)ss)[stage_q6k_sum_index(g4 >> 2)] = -32 * sum;
+            else ss[g4 >> 2] = (float)sum;
+        }
         if ((g4 & 7) == 0) da[g4 >> 3] = d;
     }
 }
@@ -106,7 +129,7 @@ __device__ __forceinline__ void load_x_groups(const float* x, int k, int nthread
     for (int i = 0; i < XP; i++) xs[i] = ((const f32x4*)x)[min((int)threadIdx.x + i * nthreads, n4 - 1)];
 }
 
-template <bool SH, int XP>
+template <int SH, int XP>
 __device__ __forceinline__ void stage_act_quantize(uint8_t* smem, const float* x, int k, int per,
                                                    const f32x4 (&first)[XP], int nthreads) {
     const int n4 = k / 4;
@@ -298,7 +321,6 @@ struct SlotWQ8P {
     u32 t;
 };
 
-struct __attribute__((packed, aligned(4))) u32x4_a4 { u32x4 v; };
 __device__ __forceinline__ void load_w_q8p(const uint8_t* row, int slot, SlotWQ8P& w) {
     const uint8_t* blk = row + (size_t)slot * 68;
 #pragma unroll
@@ -371,11 +393,57 @@ __device__ __forceinline__ void load_w_q6k(const uint8_t* row, int slot, SlotWQ6
     w.d = ld2(blk + 208);
 }
 
+// (Reading each 16-byte field as five 4-byte-aligned words moved down by a funnel shift, so
+// that no load of an odd super-block is only 2-byte aligned, measured slower: eight load
+// instructions a slot instead of five, 14.0 against 13.6 us at 4096 x 14336.)
 __device__ __forceinline__ i32 dot16(u32x4 q, u32x4 a) {
     i32 t = dot4(q.x, a.x, 0);
     t = dot4(q.y, a.y, t);
     t = dot4(q.z, a.z, t);
     return dot4(q.w, a.w, t);
+}
+
+// The same slot over the staging layout JL_STAGE_Q6K: the four runs' scales and (already
+// multiplied by the zero point) sums are one 16-byte read each, the dot products accumulate
+// onto the sums as integers, and the block scale d multiplies the slot's total once.
+#define JL_Q6_KS 1014   // (not a ggml type: the kernel form's tag)
+struct SlotActQ6KS {
+    u32x4 a[4];
+    f32x4 da;
+    u32x4 s;      // int32: -32 * sum of each run
+};
+
+__device__ __forceinline__ void load_act_q6ks(const ActLds& A, int slot, SlotActQ6KS& s) {
+    const int h = slot >> 1, j = slot & 1;   // half-super-block h = 2 sb + n
+    const u32x4* a = (const u32x4*)(A.a + h * 128 + j * 16);
+    s.a[0] = a[0]; s.a[1] = a[2]; s.a[2] = a[4]; s.a[3] = a[6];
+    s.da = *(const f32x4*)(A.da + 4 * h);
+    s.s = *(const u32x4*)((const u32*)A.s16 + 8 * h + 4 * j);
+}
+
+__device__ __forceinline__ i32 dot16_acc(u32x4 q, u32x4 a, i32 t) {
+    t = dot4(q.x, a.x, t);
+    t = dot4(q.y, a.y, t);
+    t = dot4(q.z, a.z, t);
+    return dot4(q.w, a.w, t);
+}
+
+__device__ __forceinline__ float dot_q6ks(const SlotWQ6K& w, const SlotActQ6KS& s) {
+    const u32 M4 = 0x0F0F0F0Fu, M2 = 0x30303030u;
+    const u32x4 q0 = (w.qla & M4) | ((w.qh << 4) & M2);
+    const u32x4 q1 = (w.qlb & M4) | ((w.qh << 2) & M2);
+    const u32x4 q2 = ((w.qla >> 4) & M4) | (w.qh & M2);
+    const u32x4 q3 = ((w.qlb >> 4) & M4) | ((w.qh >> 2) & M2);
+    // value = d * sc * (q - 32): the zero point is in the accumulator's start
+    const float t0 = (float)dot16_acc(q0, s.a[0], (i32)s.s.x) * (float)(int8_t)(w.sc & 0xFF);
+    const float t1 = (float)dot16_acc(q1, s.a[1], (i32)s.s.y) * (float)(int8_t)((w.sc >> 8) & 0xFF);
+    const float t2 = (float)dot16_acc(q2, s.a[2], (i32)s.s.z) * (float)(int8_t)((w.sc >> 16) & 0xFF);
+    const float t3 = (float)dot16_acc(q3, s.a[3], (i32)s.s.w) * (float)(int8_t)(w.sc >> 24);
+    float acc = t0 * s.da.x;
+    acc = fmaf(t1, s.da.y, acc);
+    acc = fmaf(t2, s.da.z, acc);
+    acc = fmaf(t3, s.da.w, acc);
+    return acc * half_bits_to_f32(w.d);
 }
 
 struct PrepQ6K {
@@ -414,6 +482,9 @@ __device__ __forceinline__ float dot_q6k(const SlotWQ6K& w, const SlotActQ6K& s)
 }
 
 // ------------------------------------------------------------- the kernel
+__device__ constexpr int stage_layout_of(int type) {
+    return type == JL_Q8_0P ? JL_STAGE_SHIFTED : type == JL_Q6_KS ? JL_STAGE_Q6K : JL_STAGE_PLAIN;
+}
 template <int TYPE> struct SlotTraits;
 template <> struct SlotTraits<JL_Q4_K> {
     typedef SlotActQ4K Act; typedef SlotWQ4K W;
@@ -441,6 +512,13 @@ template <> struct SlotTraits<JL_Q8_0P> {
     static __device__ __forceinline__ void load_act(const ActLds& A, int s, Act& a) { load_act_q8p(A, s, a); }
     static __device__ __forceinline__ void load_w(const uint8_t* row, int s, W& w) { load_w_q8p(row, s, w); }
     static __device__ __forceinline__ float dot(const W& w, int, const Act& a) { return dot_q8p(w, a); }
+};
+template <> struct SlotTraits<JL_Q6_KS> {
+    typedef SlotActQ6KS Act; typedef SlotWQ6K W;
+    static constexpr int kElems = 64;
+    static __device__ __forceinline__ void load_act(const ActLds& A, int s, Act& a) { load_act_q6ks(A, s, a); }
+    static __device__ __forceinline__ void load_w(const uint8_t* row, int s, W& w) { load_w_q6k(row, s, w); }
+    static __device__ __forceinline__ float dot(const W& w, int, const Act& a) { return dot_q6ks(w, a); }
 };
 template <> struct SlotTraits<JL_Q6_K> {
     typedef SlotActQ6K Act; typedef SlotWQ6K W;
@@ -585,7 +663,7 @@ __device__ __forceinline__ void matvec_body_xp(const MatVecArgs& p, uint8_t* sme
         for (int j = 0; j < RPW; j++)
             T::load_w(p.w + (size_t)min(r0 + j, p.nrows - 1) * p.row_bytes, s, w[j]);
     }
-    constexpr bool SH = TYPE == JL_Q8_0P;
+    constexpr int SH = stage_layout_of(TYPE);
     if (p.x) stage_act_quantize<SH, XP>(smem, p.x, p.k, p.per, x0, nwaves * 64);
     else stage_act_copy<SH>(smem, p.q, p.as, p.s16, p.k, nwaves * 64);
     lds_barrier();   // orders the LDS staging only: the weight loads stay in flight
@@ -638,7 +716,7 @@ __device__ __forceinline__ void matvec_multi_body_xp(const MatVecMultiArgs& p, u
     if constexpr (XP == 0) {
         typename T::W w[1];
         T::load_w(w0 + (size_t)min(r0, nrows - 1) * row_bytes, min(lane, nslots - 1), w[0]);
-        stage_act_copy<TYPE == JL_Q8_0P>(smem, p.q, p.as, p.s16, p.k, nthreads);
+        stage_act_copy<stage_layout_of(TYPE)>(smem, p.q, p.as, p.s16, p.k, nthreads);
         lds_barrier();
         float* const outp = p.out[y];
         float* const resid = y == 0 ? p.resid : nullptr;
@@ -684,13 +762,20 @@ __device__ __forceinline__ void matvec_multi_body_xp(const MatVecMultiArgs& p, u
             ss += (double)v.x * v.x + (double)v.y * v.y + (double)v.z * v.z + (double)v.w * v.w;
         }
         ss = wave_sum_f64(ss);
-        double* red = (double*)smem;   // the staging area is not in use yet
+        // nwaves partial sums and the scale, behind the staging area (JL_NORM_LDS_BYTES more of
+        // dynamic LDS).  One wavefront turns the sum into the scale: the f64 division and square
+        // root are a hundred dependent instructions, and sixteen wavefronts taking them side by
+        // side on four SIMDs made the launch 1.3 us longer than one taking them for all.
+        double* red = (double*)(smem + (((TYPE == JL_Q8_0P ? JL_ACT_LDS_BYTES_SHIFTED(p.k) : JL_ACT_LDS_BYTES(p.k)) + 15) & ~15));
         if (lane == 0) red[wave] = ss;
         lds_barrier();                 // (orders LDS only: the first weight loads stay in flight)
-        double tot = 0.0;
-        for (int i = 0; i < nwaves; i++) tot += red[i];
-        lds_barrier();                 // everyone has read before the quantizer writes
-        nscale = 1.0 / __builtin_sqrt(tot / (double)p.k + (double)p.norm_eps);
+        if (wave == 0) {
+            double tot = 0.0;
+            for (int i = 0; i < nwaves; i++) tot += red[i];
+            if (lane == 0) red[nwaves] = 1.0 / __builtin_sqrt(tot / (double)p.k + (double)p.norm_eps);
+        }
+        lds_barrier();
+        nscale = red[nwaves];
     }
     auto stage_group = [&](int g4, f32x4 v, f32x4 u, f32x4 nw) __attribute__((always_inline)) {
         if (p.norm_w) {
@@ -699,7 +784,7 @@ __device__ __forceinline__ void matvec_multi_body_xp(const MatVecMultiArgs& p, u
             if (p.norm_out && blockIdx.x == 0 && y == 0 && g4 < n4) ((f32x4*)p.norm_out)[g4] = v;
         }
         if (x2) v = f32x4{silu_f32(v.x) * u.x, silu_f32(v.y) * u.y, silu_f32(v.z) * u.z, silu_f32(v.w) * u.w};
-        stage_quantize4<TYPE == JL_Q8_0P>(smem, p.k, p.per, g4, v);
+        stage_quantize4<stage_layout_of(TYPE)>(smem, p.k, p.per, g4, v);
     };
     {
         int g4 = threadIdx.x;
