@@ -15,7 +15,9 @@
 #include <cstdio>
 #include <cstring>
 #include <map>
+#include <atomic>
 #include <mutex>
+#include <thread>
 #include <string>
 #include <vector>
 
@@ -67,24 +69,22 @@ struct jl_ctx {
     std::map<std::string, hipFunction_t> fn;
     std::string err;
     std::mutex mu;  // serialises the host-pointer seam (one staging area per context)
+    std::atomic<std::thread::id> mu_owner{};   // the thread inside mu (jl_forget must not try it again)
     // jl_forget only queues its range here, under a lock no launch or upload path holds; the
     // host-pointer calls apply the queue (unlink + hipFree) before their residency lookup
     std::mutex forget_mu;
     std::vector<std::pair<uintptr_t, uintptr_t>> pending_forget;
     bool no_device = false;   // created with device < 0: host-side bookkeeping only
-    bool dry_run = false;     // jl_reserve_shape: size the workspaces, launch nothing
     // the static device array of scratch.hip on this context's device (null: the lookup
     // failed and static_err says why), and the state of a call that lives on it
     void* static_scratch = nullptr;
     size_t static_scratch_bytes = 0;
     std::string static_err;
-    bool no_alloc = false;    // jl_matmul_static_dev: workspaces are carved from the array
-    size_t static_used = 0;
     Tuning tune;
     int gemm_min_tok = 3;  // below this a per-token matvec loop is as fast (3.8 us a token against 8.9 us for up to 16)
     int num_cu = 0;
     size_t lds_limit = 0;
-    unsigned long long launches = 0;   // kernels launched so far (jl_launch_count)
+    std::atomic<unsigned long long> launches{0};   // kernels launched so far (jl_launch_count)
 
     // prefill GEMM workspace (quantized activations in stage layout), grown on demand
     void* gemm_ws = nullptr;
@@ -118,6 +118,44 @@ struct jl_ctx {
 };
 
 namespace {
+
+// What a call in progress on THIS thread has switched on for its context: jl_reserve_shape
+// walks a launch path with launching off (dry_run), jl_matmul_static_dev carves workspaces
+// from the static array instead of the heap (no_alloc).  Kept per thread and tagged with the
+// context, so a launch that another thread makes on the same context meanwhile is a launch.
+struct CallState {
+    const jl_ctx* ctx = nullptr;
+    bool dry_run = false;
+    bool no_alloc = false;
+    size_t static_used = 0;
+};
+thread_local CallState g_call;
+bool call_dry_run(const jl_ctx* c) { return g_call.ctx == c && g_call.dry_run; }
+bool call_no_alloc(const jl_ctx* c) { return g_call.ctx == c && g_call.no_alloc; }
+// Switches the state on for a scope; nests (a dry run inside a no-alloc call).
+struct CallScope {
+    CallState saved;
+    CallScope(const jl_ctx* c, bool dry_run, bool no_alloc) : saved(g_call) {
+        if (g_call.ctx != c) g_call = CallState{};
+        g_call.ctx = c;
+        g_call.dry_run = g_call.dry_run || dry_run;
+        g_call.no_alloc = g_call.no_alloc || no_alloc;
+    }
+    ~CallScope() { g_call = saved; }
+};
+
+// c->mu with its owner recorded.
+struct CtxLock {
+    jl_ctx* c;
+    explicit CtxLock(jl_ctx* ctx) : c(ctx) {
+        c->mu.lock();
+        c->mu_owner.store(std::this_thread::get_id());
+    }
+    ~CtxLock() {
+        c->mu_owner.store(std::thread::id());
+        c->mu.unlock();
+    }
+};
 
 int fail(jl_ctx* c, int code, const char* fmt, ...) {
     char buf[512];
@@ -193,7 +231,7 @@ int launch(jl_ctx* c, const char* name, unsigned gx, unsigned gy, unsigned block
            hipStream_t st, void** params, unsigned gz = 1) {
     auto it = c->fn.find(name);
     if (it == c->fn.end()) return fail(c, JL_ERR_ARG, "kernel %s is not in the code object", name);
-    if (c->dry_run) return JL_OK;
+    if (call_dry_run(c)) return JL_OK;
     HIP_TRY(c, H->ModuleLaunchKernel(it->second, gx, gy, gz, block, 1, 1, lds, st, params, nullptr));
     c->launches++;
     return JL_OK;
@@ -205,15 +243,17 @@ int launch(jl_ctx* c, const char* name, unsigned gx, unsigned gy, unsigned block
 // enough (jl_reserve, jl_reserve_shape).
 int grow(jl_ctx* c, void** buf, size_t* have, size_t need) {
     if (*have >= need) return JL_OK;
-    if (c->no_alloc) {
-        // a call that must not allocate: the next piece of the static array, or an error
-        const size_t off = (c->static_used + 255) & ~(size_t)255;
-        if (*have != 0 || off + need > c->static_scratch_bytes)
-            return fail(c, JL_ERR_NOMEM, "this shape needs %zu bytes of workspace beyond the %zu already taken; the static "
+    if (call_no_alloc(c)) {
+        // a call that must not allocate: the next piece of the static array, or an error.  (A
+        // workspace asked for a second time with a larger size gets a new, larger piece: the
+        // one it had stays taken until the call ends.)
+        const size_t off = (g_call.static_used + 255) & ~(size_t)255;
+        if (off + need > c->static_scratch_bytes)
+            return fail(c, JL_ERR_NOMEM, "this shape needs %zu bytes of workspace on top of %zu already carved; the static "
                         "scratch holds %zu", need, off, c->static_scratch_bytes);
         *buf = (char*)c->static_scratch + off;
         *have = need;
-        c->static_used = off + need;
+        g_call.static_used = off + need;
         return JL_OK;
     }
     if (*buf) {
@@ -1450,7 +1490,7 @@ int jl_synchronize(jl_ctx* c) {
     return JL_OK;
 }
 
-unsigned long long jl_launch_count(const jl_ctx* c) { return c ? c->launches : 0; }
+unsigned long long jl_launch_count(const jl_ctx* c) { return c ? c->launches.load() : 0ull; }
 
 int jl_set_tuning(jl_ctx* c, const char* key, int value) {
     if (!c || !key) return JL_ERR_ARG;
@@ -1617,17 +1657,19 @@ int jl_matmul_static_dev(jl_ctx* c, float* out, int type, const void* w, const f
                      {&c->unpack_ws, &c->unpack_ws_bytes, nullptr, 0}};
     for (auto& s : saved) { s.b = *s.buf; s.h = *s.have; *s.buf = nullptr; *s.have = 0; }
     // a dry run first: the sizes are checked against the array before the first real launch
-    c->no_alloc = true;
-    c->static_used = 0;
-    c->dry_run = true;
-    int rc = matmul_launch(c, out, type, w, x, nrows, k, ntok, pick_stream(c, stream));
-    c->dry_run = false;
-    if (rc == JL_OK) {
-        for (auto& s : saved) { *s.buf = nullptr; *s.have = 0; }
-        c->static_used = 0;
-        rc = matmul_launch(c, out, type, w, x, nrows, k, ntok, pick_stream(c, stream));
+    int rc;
+    {
+        CallScope no_alloc(c, false, true);
+        {
+            CallScope dry(c, true, false);
+            rc = matmul_launch(c, out, type, w, x, nrows, k, ntok, pick_stream(c, stream));
+        }
+        if (rc == JL_OK) {
+            for (auto& s : saved) { *s.buf = nullptr; *s.have = 0; }
+            g_call.static_used = 0;
+            rc = matmul_launch(c, out, type, w, x, nrows, k, ntok, pick_stream(c, stream));
+        }
     }
-    c->no_alloc = false;
     for (auto& s : saved) { *s.buf = s.b; *s.have = s.h; }
     return rc;
 }
@@ -1741,7 +1783,7 @@ int jl_reserve_shape(jl_ctx* c, int type, int nrows, int k, int ntok, int packed
     float* const out = (float*)(uintptr_t)4096;
     const float* const x = (const float*)(uintptr_t)4096;
     const void* const w = (const void*)(uintptr_t)4096;
-    c->dry_run = true;
+    CallScope dry(c, true, false);
     int rc;
     if (type == JL_TYPE_MXFP4) {
         rc = packed ? jl_matmul_mxfp4_packed_bf16_dev(c, out, (const uint32_t*)w, (const uint32_t*)w, 0, nrows,
@@ -1753,7 +1795,6 @@ int jl_reserve_shape(jl_ctx* c, int type, int nrows, int k, int ntok, int packed
     } else {
         rc = matmul_launch(c, out, type, w, x, nrows, k, ntok, c->stream);
     }
-    c->dry_run = false;
     return rc;
 }
 
@@ -2090,7 +2131,7 @@ int jl_matvec(jl_ctx* c, float* out, int type, const void* w, size_t wbytes, con
 int jl_matmul(jl_ctx* c, float* out, int type, const void* w, size_t wbytes, const float* x,
               int nrows, int k, int ntok) {
     if (!c) return JL_ERR_ARG;
-    std::lock_guard<std::mutex> lock(c->mu);
+    CtxLock lock(c);
     drain_forget(c);
     if (c->no_device) return fail(c, JL_ERR_HIP, "this context is bound to no device");
     const TypeInfo* ti = nullptr;
@@ -2126,7 +2167,7 @@ int jl_matvec_packed(jl_ctx* c, float* out, int type, const uint32_t* qs, const 
 int jl_matmul_packed(jl_ctx* c, float* out, int type, const uint32_t* qs, const uint32_t* d,
                      const uint32_t* sc, int row, int stride, const float* x, int nrows, int k, int ntok) {
     if (!c) return JL_ERR_ARG;
-    std::lock_guard<std::mutex> lock(c->mu);
+    CtxLock lock(c);
     drain_forget(c);
     if (c->no_device) return fail(c, JL_ERR_HIP, "this context is bound to no device");
     const PlaneRef host = {qs, d, sc, row, stride};
@@ -2181,12 +2222,22 @@ int jl_matmul_packed(jl_ctx* c, float* out, int type, const uint32_t* qs, const 
 int jl_forget(jl_ctx* c, const void* p, size_t n) {
     if (!c) return JL_ERR_ARG;
     if (!p || n == 0) return JL_OK;
-    // Only queue the range: no HIP call, and no lock that a launch or an upload holds, so this
-    // returns at once from any thread -- also from inside a page-in that this context's own
-    // weight upload started.  The next host-pointer call applies the queue before it looks a
-    // pointer up; jl_ctx_destroy frees whatever is left.
-    std::lock_guard<std::mutex> g(c->forget_mu);
-    c->pending_forget.emplace_back((uintptr_t)p, (uintptr_t)p + n);
+    // Queue the range under a lock no launch or upload holds, so this returns from any thread --
+    // also from inside a page-in that this context's own weight upload started.  Then, as the
+    // reference does (jit/gpu/tier/forget.go:38-49), apply the queue at once if the context is
+    // free: the device copies go now and a caller that never makes another host-pointer call
+    // still gets its memory back.  A busy context (another thread's call, or this thread's own)
+    // applies the queue at the start of its next host-pointer call; jl_ctx_destroy frees the rest.
+    {
+        std::lock_guard<std::mutex> g(c->forget_mu);
+        c->pending_forget.emplace_back((uintptr_t)p, (uintptr_t)p + n);
+    }
+    if (c->mu_owner.load() != std::this_thread::get_id() && c->mu.try_lock()) {
+        c->mu_owner.store(std::this_thread::get_id());
+        drain_forget(c);
+        c->mu_owner.store(std::thread::id());
+        c->mu.unlock();
+    }
     return JL_OK;
 }
 
@@ -2229,18 +2280,20 @@ int jl_probe_dev(jl_ctx* c, int kind, const void* src, size_t nbytes, int grid, 
 int jl_ctx_lock(jl_ctx* c) {
     if (!c) return JL_ERR_ARG;
     c->mu.lock();
+    c->mu_owner.store(std::this_thread::get_id());
     return JL_OK;
 }
 
 int jl_ctx_unlock(jl_ctx* c) {
     if (!c) return JL_ERR_ARG;
+    c->mu_owner.store(std::thread::id());
     c->mu.unlock();
     return JL_OK;
 }
 
 size_t jl_resident_count(jl_ctx* c) {
     if (!c) return 0;
-    std::lock_guard<std::mutex> lock(c->mu);
+    CtxLock lock(c);
     drain_forget(c);
     return c->resident.size();
 }

@@ -39,16 +39,6 @@
 #include "common.h"
 #include "quantize.h"
 
-// Phase marker for profiling builds; expands to nothing in the product.
-#ifndef JL_TRACE
-#define JL_TRACE(i)
-#endif
-// Profiling builds only (results are then wrong): bits switch parts of the wide kernel's loop
-// off, to time what each costs.  1 epilogue, 2 dequantization, 4 activation loads, 8 weight
-// fragment reads, 16 barriers, 32 the minimum-term matrix instructions, 64 weight loads.
-#ifndef JL_ABL
-#define JL_ABL 0
-#endif
 
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
@@ -405,7 +395,6 @@ __device__ __forceinline__ void gemm_q4k_body(const GemmArgs& p, uint8_t* smem, 
         constexpr int nhalf = half ^ 1;
         const int nsbi = (step + 1) >> 1;
         _Float16* wnext = sW + nhalf * JL_GEMM_STAGE_HALFS;
-        JL_TRACE(0);
         // the loads of the stage after next go out first: a whole stage of matrix work
         // covers their latency (that stage has this stage's half)
         {
@@ -417,7 +406,6 @@ __device__ __forceinline__ void gemm_q4k_body(const GemmArgs& p, uint8_t* smem, 
         // instructions, so the vector work runs under the matrix core.
         GemmWScale wsc;
         w_scale(wcur, nhalf, wnext, wsc);
-        JL_TRACE(1);
         // matrix work: per K-step one activation fragment (already in the ring) against
         // the two row groups' weight fragments, fetched from LDS a K-step ahead; the ring
         // slot is refilled with the next stage's fragment as soon as it has been used
@@ -429,7 +417,6 @@ __device__ __forceinline__ void gemm_q4k_body(const GemmArgs& p, uint8_t* smem, 
             for (int j = 0; j < 2; j++) wf[0][j] = *(const f16x8*)(wp0 + 32 * j * JL_GEMM_STRIDE);
         }
         __builtin_amdgcn_sched_barrier(0);
-        JL_TRACE(2);
 #pragma unroll
         for (int ks = 0; ks < 8; ks++) {
             if (live) {
@@ -469,7 +456,6 @@ __device__ __forceinline__ void gemm_q4k_body(const GemmArgs& p, uint8_t* smem, 
             const int sb2 = min(sb + 1, p.k / 256 - 1);
             da_reg = p.da[(size_t)sb2 * p.tok_pad + da_tok];
         }
-        JL_TRACE(3);
         if (half == 1 && live) {
             // the 16 minimum columns: M, then the super-block's epilogue
             //   out += d_a * (d * P - dmin * M)
@@ -490,9 +476,7 @@ __device__ __forceinline__ void gemm_q4k_body(const GemmArgs& p, uint8_t* smem, 
                 }
             }
         }
-        JL_TRACE(4);
         lds_barrier();
-        JL_TRACE(5);
     };
     for (int step = 0; step < nsteps; step += 2) {
         stage(GemmIntC<0>{}, step, wa, wb);
@@ -692,7 +676,7 @@ __device__ __forceinline__ void gemm_q4k_wide_body(const GemmArgs& p, uint8_t* s
         const _Float16* w = sW + half * STAGE_HALFS;
         _Float16* wnext = sW + nhalf * STAGE_HALFS;
         const int nstep = min(step + 1, nsteps - 1);
-        if (!(JL_ABL & 64)) load_w(min(step + 2, nsteps - 1), wnxt);
+        load_w(min(step + 2, nsteps - 1), wnxt);
         const _Float16* wp0 = w + arow * JL_GEMM_WROW + 8 * kg;
         const _Float16* mp0 = sMin + eb * MIN_HALFS + arow * JL_GEMM_MROW + 8 * kg;
         const float* scp = sScale + eb * 2 * ROWS + 2 * arow;
@@ -719,7 +703,7 @@ __device__ __forceinline__ void gemm_q4k_wide_body(const GemmArgs& p, uint8_t* s
             // the next slot's token scales first: the wait that guards them then leaves the
             // weight fragments (read after them, used a slot later) in flight
             if (ep_next) dav[(slot + 1) & 1] = *(const f32x4*)(dap + 8 * ((ks + 1) & 3));
-            if (slot + 1 < 16 && !(JL_ABL & 8)) {
+            if (slot + 1 < 16) {
 #pragma unroll
                 for (int j = 0; j < 2; j++) wf[(slot + 1) & 1][j] = w_frag(slot + 1, j);
             }
@@ -732,7 +716,7 @@ __device__ __forceinline__ void gemm_q4k_wide_body(const GemmArgs& p, uint8_t* s
             if (ep && ks == 4) esc = *(const float2*)(scp + 2 * 32 * (ej0 + 1));
             __builtin_amdgcn_sched_barrier(0);
             const f32x16 czero = {0};
-            if (ep && (ks & 3) == 0 && !(JL_ABL & 32)) {
+            if (ep && (ks & 3) == 0) {
                 // the tile's M = sum m_s A_s, ahead of this slot's instructions so that it is
                 // ready when the vector work below asks for it
                 accM = __builtin_amdgcn_mfma_f32_32x32x16_f16(aaug, wm, czero, 0, 0, 0);
@@ -741,13 +725,13 @@ __device__ __forceinline__ void gemm_q4k_wide_body(const GemmArgs& p, uint8_t* s
             for (int j = 0; j < 2; j++)
                 accP[2 * jh + j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
                     aring[ks], wf[slot & 1][j], (half == 0 && ks == 0) ? czero : accP[2 * jh + j], 0, 0, 0);
-            if (jh == 1 && !(JL_ABL & 4)) {
+            if (jh == 1) {
                 aring[ks] = a_frag(nstep, ks);
                 if (ks == 0 && nhalf == 1) aaug = a_frag(nstep, 8);
             }
             if (ep) {
-                if (!(JL_ABL & 1)) ep_quarter(GemmIntC<ej0 + (ks >> 2)>{}, GemmIntC<(ks & 3)>{}, dav[slot & 1]);
-            } else if (jh != ep_jh && !(JL_ABL & 2)) {
+                ep_quarter(GemmIntC<ej0 + (ks >> 2)>{}, GemmIntC<(ks & 3)>{}, dav[slot & 1]);
+            } else if (jh != ep_jh) {
                 // the next stage's weights: wcur -> f16 -> LDS
                 if (ks == 0) {
                     if (PL) gemm_wide_scale_planes(wcur.hdr, 4 * nhalf + psub, wsc);
@@ -804,7 +788,7 @@ __device__ __forceinline__ void gemm_q4k_wide_body(const GemmArgs& p, uint8_t* s
             const int sb2 = min(sb + 1, p.k / 256 - 1);
             da_reg = p.da[(size_t)sb2 * p.tok_pad + t0 + (tid & (TOK - 1))];
         }
-        if (!(JL_ABL & 16)) lds_barrier();
+        lds_barrier();
     };
     stage(GemmIntC<0>{}, GemmIntC<1>{}, 0, wa, wb);
     stage(GemmIntC<1>{}, GemmIntC<0>{}, 1, wb, wa);
@@ -964,7 +948,6 @@ __device__ __forceinline__ void gemm_q4k_w16_body(const GemmW16Args& p, uint8_t*
         u32x4* nxt = sW + nhalf * JL_GEMM_W16_STAGE_VECS;
         const int nstep = min(step + 1, nsteps - 1);
         const u32x4* w2 = wsrc + (size_t)min(step + 2, nsteps - 1) * JL_GEMM_W16_STAGE_VECS;
-        JL_TRACE(0);
         float sc2[2][2];
         if (half == 1) {
             // the rows' (d, dmin) for this super-block's epilogue
@@ -979,7 +962,6 @@ __device__ __forceinline__ void gemm_q4k_w16_body(const GemmW16Args& p, uint8_t*
 #pragma unroll
         for (int j = 0; j < 2; j++) wf[0][j] = __builtin_bit_cast(f16x8, cur[j * 64 + lane]);
         __builtin_amdgcn_sched_barrier(0);
-        JL_TRACE(2);
 #pragma unroll
         for (int ks = 0; ks < 8; ks++) {
             if (ks + 1 < 8) {
@@ -1012,7 +994,6 @@ __device__ __forceinline__ void gemm_q4k_w16_body(const GemmW16Args& p, uint8_t*
             const int sb2 = min(sb + 1, p.k / 256 - 1);
             da_reg = p.da[(size_t)sb2 * p.tok_pad + da_tok];
         }
-        JL_TRACE(3);
         if (half == 1) {
             const f32x16 zero = {0};
             const float* sda = sDa + (sb & 1) * JL_GEMM_TILE + 32 * tg;
@@ -1028,9 +1009,7 @@ __device__ __forceinline__ void gemm_q4k_w16_body(const GemmW16Args& p, uint8_t*
                 }
             }
         }
-        JL_TRACE(4);
         lds_barrier();
-        JL_TRACE(5);
     };
     for (int step = 0; step < nsteps; step += 2) {
         stage(GemmIntC<0>{}, step);

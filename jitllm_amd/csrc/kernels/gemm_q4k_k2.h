@@ -37,7 +37,6 @@ __device__ __forceinline__ void gemm_q4k_k2_body(const GemmArgs& p, uint8_t* sme
     constexpr int ROWS = JL_GEMM_K2_ROWS, TOK = JL_GEMM_K2_TOK, STAGE_HALFS = ROWS * JL_GEMM_WROW;
     constexpr int MIN_HALFS = ROWS * JL_GEMM_MROW;
     const int tid = threadIdx.x, lane = tid & 63;
-    JL_TRACE(0);
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int tg = wave & 3, kh = wave >> 2;
     uint8_t* gmem = smem + kh * JL_GEMM_K2_GROUP_BYTES;
@@ -110,7 +109,6 @@ __device__ __forceinline__ void gemm_q4k_k2_body(const GemmArgs& p, uint8_t* sme
     load_w(1, wa);
     float da_reg = dag[0];
     lds_barrier();
-    JL_TRACE(1);
 
     f32x16 accM;
     float2 esc;
@@ -229,7 +227,6 @@ __device__ __forceinline__ void gemm_q4k_k2_body(const GemmArgs& p, uint8_t* sme
         stage(GemmIntC<0>{}, GemmIntC<1>{}, GemmIntC<0>{}, step + 2, wa, wb);
         stage(GemmIntC<1>{}, GemmIntC<1>{}, GemmIntC<0>{}, step + 3, wb, wa);
     }
-    JL_TRACE(2);
     // the last super-block's epilogue (its parity is 1)
     {
         const f32x16 czero = {0};
@@ -277,5 +274,4 @@ __device__ __forceinline__ void gemm_q4k_k2_body(const GemmArgs& p, uint8_t* sme
             }
         });
     }
-    JL_TRACE(3);
 }

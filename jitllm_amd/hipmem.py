@@ -37,6 +37,8 @@ def hip():
         h.hipEventElapsedTime.argtypes = [C.POINTER(C.c_float), C.c_void_p, C.c_void_p]
         h.hipEventDestroy.argtypes = [C.c_void_p]
         h.hipMemGetInfo.argtypes = [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]
+        h.hipStreamCreate.argtypes = [C.POINTER(C.c_void_p)]
+        h.hipStreamDestroy.argtypes = [C.c_void_p]
         h.hipStreamBeginCapture.argtypes = [C.c_void_p, C.c_int]
         h.hipStreamEndCapture.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
         h.hipGraphInstantiate.argtypes = [C.POINTER(C.c_void_p), C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]
@@ -129,6 +131,22 @@ class Event:
             hip().hipEventDestroy(self.e)
         except Exception:
             pass
+
+
+class Stream:
+    """A HIP stream of the caller's own (default priority), to pass where an entry point takes one."""
+
+    def __init__(self):
+        self.handle = C.c_void_p()
+        check(hip().hipStreamCreate(C.byref(self.handle)), "hipStreamCreate")
+
+    def synchronize(self):
+        check(hip().hipStreamSynchronize(self.handle), "hipStreamSynchronize")
+
+    def destroy(self):
+        if self.handle:
+            check(hip().hipStreamDestroy(self.handle), "hipStreamDestroy")
+            self.handle = C.c_void_p()
 
 
 class Gate:

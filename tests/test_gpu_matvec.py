@@ -248,3 +248,68 @@ def test_device_seam_host_pointers(dev):
     assert dev.MatVec(out, 2, w, x, nrows, k) is False          # Q4_0: not served
     assert dev.MatVec(out, t, w, x, nrows, k - 32) is False
     dev.SetActWindow(32)
+
+
+def test_forget_frees_at_once_when_the_context_is_free(dev):
+    """Forget applies at once when no call holds the context (the reference's TryLock branch,
+    /root/reference/jit/gpu/tier/forget.go:38-49): the device copy of a forgotten buffer is
+    gone -- free device memory is back -- before any other call is made."""
+    from jitllm_amd.hipmem import mem_info
+    nrows, k, t = 8192, 4096, quant.Q8_0                  # 35 MB of weights
+    dev.SetActWindow(32)
+    w = synth.random_weights(t, nrows, k, seed=5)
+    x = synth.activations(k, seed=6)
+    out = np.zeros(nrows, np.float32)
+    dev.synchronize()
+    free0, _ = mem_info()
+    assert dev.MatVec(out, t, w, x, nrows, k) is True
+    free1, _ = mem_info()
+    assert free0 - free1 >= w.nbytes, "the weights are not resident after the first call"
+    dev.Forget(w)
+    free2, _ = mem_info()
+    assert free2 - free1 >= w.nbytes, "Forget left the device copy allocated"
+    assert dev.resident_count() == 0
+
+
+def test_reserve_shape_on_one_thread_does_not_switch_off_another_threads_launches(dev, devbuf):
+    """jl_reserve_shape walks a launch path with launching switched off.  That state belongs to
+    the call, not to the context: a matvec another thread enqueues meanwhile on the same
+    context must still be launched.  One thread reserves shapes in a loop, the other runs
+    matvecs into a poisoned buffer and checks every one."""
+    import threading
+    nrows, k, t, window = 300, 1024, quant.Q4_K, 256
+    dev.SetActWindow(window)
+    w = synth.quantized_weights(t, nrows, k, seed=2)
+    x = synth.activations(k, seed=3)
+    want = _like_for_like(t, w, x, nrows, k, window)
+    wd, xd = devbuf(w), devbuf(x)
+    out = devbuf(shape=(nrows,), dtype=np.float32, fill=np.float32(7e30))
+    stop = threading.Event()
+    errors = []
+
+    def reserver():
+        i = 0
+        while not stop.is_set():
+            try:
+                assert dev.reserve_shape(t, 512 + 64 * (i % 5), 4096, 128 + (i % 7))
+            except Exception as e:      # noqa: BLE001 - reported by the main thread
+                errors.append(e)
+                return
+            i += 1
+
+    th = threading.Thread(target=reserver)
+    th.start()
+    try:
+        for _ in range(300):
+            out.put(np.full(nrows, np.float32(7e30)))
+            before = dev.launch_count()
+            assert dev.matvec_dev(out.ptr, t, wd.ptr, xd.ptr, nrows, k)
+            dev.synchronize()
+            got = out.get()
+            assert np.all(np.abs(got) < 1e30), "a matvec was swallowed by another thread's dry run"
+            assert nmse(got, want) <= 1e-10
+    finally:
+        stop.set()
+        th.join(30)
+    assert not errors, errors
+    dev.SetActWindow(32)

@@ -66,6 +66,37 @@ def test_static_matmul_equals_matmul_two_calls_in_a_row(dev, devbuf):
     dev.SetActWindow(32)
 
 
+def test_static_matmul_on_a_stream_of_the_callers(dev, devbuf):
+    """The callers this entry point is for bring their own stream (a serving loop's, one under
+    graph capture): the same bits as jl_matmul_dev, with the work enqueued on that stream (the
+    context's stream is kept busy behind a wait kernel meanwhile, so an answer can only come
+    from the caller's)."""
+    from jitllm_amd.hipmem import Gate, Stream
+    t, window, ntok, nrows, k = quant.Q4_K, 256, 300, 520, 1024
+    dev.SetActWindow(window)
+    w = synth.random_weights(t, nrows, k, seed=3)
+    x = np.stack([synth.activations(k, seed=300 + i) for i in range(ntok)])
+    wd, xd = devbuf(w), devbuf(x)
+    want = devbuf(shape=(ntok * nrows,), dtype=np.float32, fill=POISON)
+    got = devbuf(shape=(ntok * nrows,), dtype=np.float32, fill=POISON)
+    assert dev.matmul_dev(want.ptr, t, wd.ptr, xd.ptr, nrows, k, ntok)
+    dev.synchronize()
+    st = Stream()
+    free_before, _ = mem_info()
+    Gate(dev).hold(dev.stream, 20000)                      # 20 ms of nothing on the context's stream
+    assert dev.matmul_static_dev(got.ptr, t, wd.ptr, xd.ptr, nrows, k, ntok, stream=st.handle)
+    st.synchronize()
+    a = got.get()                                          # (a blocking copy: the caller's stream has finished)
+    dev.synchronize()
+    free_after, _ = mem_info()
+    assert free_after == free_before
+    assert np.array_equal(a.view(np.uint32), want.get().view(np.uint32))
+    st.destroy()
+    for buf in (wd, xd, want, got):
+        buf.free()
+    dev.SetActWindow(32)
+
+
 def test_static_matmul_refuses_what_does_not_fit(dev, devbuf):
     """A shape whose activation fragments alone exceed the array: a clear error, and the
     output untouched."""
