@@ -229,6 +229,44 @@ def cpu_baseline(t, nrows, k, window, seed=0):
 MFMA_F16_PEAK_TFLOPS = 2500.0
 
 
+def cpu_baseline_gemm(nrows, k, ntok, window=256, seed=0):
+    """The reference's weight-stationary prefill GEMM on this box's cores (restated with
+    intrinsics, oracle/jl_cpu_path.c; Q4_K planes, the activation quantizer inside every call):
+    3 warm calls, then the median of nine timed calls of the whole matmul."""
+    import oracle
+    from jitllm_amd import quant, synth
+    cores = min(16, len(os.sched_getaffinity(0)))
+    w = synth.quantized_weights(quant.Q4_K, nrows, k, seed=seed)
+    x = np.random.default_rng(2).standard_normal((ntok, k), np.float32)
+    qs, d, sc = oracle.pack_weights(quant.Q4_K, w, nrows, k)
+    cp = oracle.CpuPath(cores)
+    sec = cp.time_matmul(quant.Q4_K, qs, d, sc, x, nrows, k, ntok, window, reps=9)
+    vnni = cp.vnni
+    cp.close()
+    return {"value": round(2.0 * nrows * k * ntok / sec / 1e12, 3), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "sample": f"{ntok} tokens x {k} -> {nrows}, Q4_K planes, window {window}: 3 warm calls, median of 9 calls "
+                      f"(12 calls, {12 * sec:.2f} s); work items of 16 rows x 64 tokens handed to {cores} spinning workers; "
+                      f"{'AVX-VNNI VPDPBUSD' if vnni else 'AVX2 VPMADDUBSW'} 256-bit",
+            "ms_per_call": round(sec * 1e3, 2)}
+
+
+def cpu_baseline_moe(hosts, x_host, sel, wt, n_expert, n_ffn, n_embd, window=256):
+    """The reference's routed feed-forward block on this box's cores (oracle/jl_cpu_path.c: expert
+    by expert, gather, gate and up through the GEMM, silu(g) * u, down, the residual add), over
+    the same banks (as planes), rows, selection and weights the device block was given."""
+    import oracle
+    from jitllm_amd import quant
+    cores = min(16, len(os.sched_getaffinity(0)))
+    shapes = [(n_ffn, n_embd), (n_ffn, n_embd), (n_embd, n_ffn)]
+    planes = [oracle.pack_weights(quant.Q4_K, h, n_expert * r, k) for h, (r, k) in zip(hosts, shapes)]
+    cp = oracle.CpuPath(cores)
+    sec = cp.time_moe_block(planes[0], planes[1], planes[2], x_host, sel, wt, n_expert, n_ffn, n_embd, window, reps=9)
+    cp.close()
+    return {"us_per_step": round(sec * 1e6, 1), "cores": cores, "kind": "port",
+            "sample": f"one warm block, median of 9 blocks; selection and weights given (the router is not in the CPU "
+                      f"figure); {cores} spinning workers"}
+
+
 def gemm_section(dev, gate, shapes=None, t=None, k=4096, window=256, packed=False):
     """Prefill GEMM (x [ntok][k] f32 -> out [ntok][nrows]), activation quantizer and layout
     kernel included in every step; flops = 2*nrows*k*ntok, priced against the dense f16 MFMA
@@ -413,7 +451,7 @@ def ffn_packed_section(dev, gate_):
             "checked_rel_err": float(f"{err:.2e}")}
 
 
-def moe_section(dev, gate_, rows=64, packed=False):
+def moe_section(dev, gate_, rows=64, packed=False, cpu=False):
     """Qwen3-30B-A3B routed feed-forward block: 128 experts (gate/up 768x2048, down 2048x768,
     Q4_K), 64 rows routed top-8; one step = router logits (f32 router matrix, rows ~ N(0, 1/k)
     so the logits are ~ N(0,1)) + softmax/top-8 + group + gate/up + down + combine, all on the
@@ -487,11 +525,16 @@ def moe_section(dev, gate_, rows=64, packed=False):
     nbytes = touched * (2 * gs + ds) + 2 * rows * n_embd * 4 + n_expert * n_embd * 4
     for b in banks + [x, sd, wd, resid, ld, router]:
         b.free()
-    return {"us_per_step": round(ms * 1e3, 1), "experts_touched": touched, "bytes_per_step": nbytes,
-            "GB/s": round(nbytes / (ms * 1e-3) / 1e9, 1),
-            "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-            "TFLOP/s": round(rows * k_used * 3 * 2.0 * n_ffn * n_embd / (ms * 1e-3) / 1e12, 2),
-            "checked_rel_err": float(f"{err:.2e}")}
+    out = {"us_per_step": round(ms * 1e3, 1), "experts_touched": touched, "bytes_per_step": nbytes,
+           "GB/s": round(nbytes / (ms * 1e-3) / 1e9, 1),
+           "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+           "TFLOP/s": round(rows * k_used * 3 * 2.0 * n_ffn * n_embd / (ms * 1e-3) / 1e12, 2),
+           "checked_rel_err": float(f"{err:.2e}")}
+    if cpu:
+        base = cpu_baseline_moe(hosts, x_host, sel, wt, n_expert, n_ffn, n_embd)
+        base["GB/s"] = round(nbytes / (base["us_per_step"] * 1e-6) / 1e9, 1)
+        out["cpu_baseline"] = base
+    return out
 
 
 def moe_decode_section(dev, gate_):
@@ -836,13 +879,15 @@ def main():
         line["roofline_prefill_gemm"] = {"bound": "mfma", "achieved": g512["TFLOP/s"], "peak": MFMA_F16_PEAK_TFLOPS,
                                          "unit": "TFLOP/s", "frac": g512["frac_of_f16_mfma_peak"], "traffic": None,
                                          "workload": "Q4_K prefill GEMM 512 tokens x 4096 -> 4096, prep + GEMM per step"}
+        if not args.no_cpu:
+            line["roofline_prefill_gemm"]["cpu_baseline"] = cpu_baseline_gemm(4096, 4096, 512)
         line["prefill_gemm_packed_planes"] = gemm_section(dev, gate, {4096: (512,), 14336: (512,)}, packed=True)
         line["prefill_gemm_q6k"] = gemm_section(dev, gate, {4096: (512, 2048)}, quant.Q6_K, 14336)
         # the second configuration's matrices at prefill: the activation window is 32 there
         line["prefill_gemm_window32"] = {
             "q8_0": gemm_section(dev, gate, {14336: (512, 2048)}, quant.Q8_0, 4096, 32),
             "q6_k": gemm_section(dev, gate, {4096: (512, 2048)}, quant.Q6_K, 14336, 32)}
-        line["moe_block"] = moe_section(dev, gate)
+        line["moe_block"] = moe_section(dev, gate, cpu=not args.no_cpu)
         line["moe_block_packed_planes"] = moe_section(dev, gate, packed=True)
         line["moe_block_prefill_1024_rows"] = moe_section(dev, gate, 1024)   # groups of 32 columns per expert
         line["moe_decode"] = moe_decode_section(dev, gate)

@@ -309,6 +309,15 @@ class CpuPath:
                                             C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
         self._l.jlc_membw.restype = C.c_double
         self._l.jlc_membw.argtypes = [C.c_int, C.c_size_t, C.c_int]
+        self._l.jlc_matmul_packed.argtypes = [C.c_void_p, _f32p, C.c_int, _u32p, _u32p, _u32p, C.c_int, C.c_int,
+                                              _f32p, C.c_int, C.c_int, C.c_int, C.c_int]
+        self._l.jlc_time_matmul.restype = C.c_double
+        self._l.jlc_time_matmul.argtypes = [C.c_void_p, _f32p, C.c_int, _u32p, _u32p, _u32p, _f32p, C.c_int, C.c_int,
+                                            C.c_int, C.c_int, C.c_int]
+        moe = [C.c_void_p, _f32p, pp, pp, pp, _f32p, _u32p, C.c_int, _f32p] + [C.c_int] * 6
+        self._l.jlc_moe_block.argtypes = moe
+        self._l.jlc_time_moe_block.restype = C.c_double
+        self._l.jlc_time_moe_block.argtypes = moe + [C.c_int]
         self.threads = threads
         self._p = self._l.jlc_pool_create(threads)
 
@@ -339,6 +348,61 @@ class CpuPath:
         out = np.zeros(nrows, np.float32)
         s = self._l.jlc_time_matvec(self._p, _p(out, _f32p), t, arr(0), arr(1), arr(2), n,
                                     _p(x, _f32p), nrows, k, window, reps, sweeps)
+        if s < 0:
+            raise ValueError("cpu timing refused")
+        return s
+
+    def matmul_packed(self, t, qs, d, sc, x, nrows, k, ntok, window, row0=0, stride=None):
+        """The weight-stationary prefill GEMM over Q4_K planes (rows row0.. of planes `stride`
+        rows long): out [ntok][nrows]."""
+        stride = nrows if stride is None else stride
+        qs, d, sc = _planes(t, qs, d, sc, stride, k)
+        x = _chk(x, np.float32, ntok * k)
+        out = np.zeros((ntok, nrows), np.float32)
+        if self._l.jlc_matmul_packed(self._p, _p(out, _f32p), t, _p(qs, _u32p), _p(d, _u32p), _p(sc, _u32p),
+                                     row0, stride, _p(x, _f32p), nrows, k, ntok, window):
+            raise ValueError("cpu matmul refused")
+        return out
+
+    def time_matmul(self, t, qs, d, sc, x, nrows, k, ntok, window, reps=9):
+        """Seconds per call: 3 warm calls, then the median of `reps` timed calls."""
+        qs, d, sc = _planes(t, qs, d, sc, nrows, k)
+        x = _chk(x, np.float32, ntok * k)
+        out = np.zeros((ntok, nrows), np.float32)
+        s = self._l.jlc_time_matmul(self._p, _p(out, _f32p), t, _p(qs, _u32p), _p(d, _u32p), _p(sc, _u32p),
+                                    _p(x, _f32p), nrows, k, ntok, window, reps)
+        if s < 0:
+            raise ValueError("cpu timing refused")
+        return s
+
+    def _moe_args(self, gate, up, down, x, sel, wt, n_expert, n_ffn, n_embd):
+        rows, k_used = wt.shape
+        banks = []
+        for planes, r, kk in ((gate, n_ffn, n_embd), (up, n_ffn, n_embd), (down, n_embd, n_ffn)):
+            pl = _planes(Q4_K, planes[0], planes[1], planes[2], n_expert * r, kk)
+            banks.append((pl, (_u32p * 3)(*[_p(a, _u32p) for a in pl])))
+        x = _chk(x, np.float32, rows * n_embd)
+        sel = np.ascontiguousarray(sel, np.uint32)
+        wt = np.ascontiguousarray(wt, np.float32)
+        return banks, x, sel, wt, rows, k_used
+
+    def moe_block(self, gate, up, down, x, sel, wt, n_expert, n_ffn, n_embd, window):
+        """The routed feed-forward block over banks of Q4_K planes (each a (qs, d, sc) plane set of
+        n_expert * rows rows): resid [rows][n_embd], starting from zero."""
+        banks, x, sel, wt, rows, k_used = self._moe_args(gate, up, down, x, sel, wt, n_expert, n_ffn, n_embd)
+        resid = np.zeros((rows, n_embd), np.float32)
+        if self._l.jlc_moe_block(self._p, _p(resid, _f32p), banks[0][1], banks[1][1], banks[2][1], _p(x, _f32p),
+                                 _p(sel, _u32p), sel.shape[1], _p(wt, _f32p), rows, k_used, n_expert, n_ffn, n_embd,
+                                 window):
+            raise ValueError("cpu mixture block refused")
+        return resid
+
+    def time_moe_block(self, gate, up, down, x, sel, wt, n_expert, n_ffn, n_embd, window, reps=9):
+        banks, x, sel, wt, rows, k_used = self._moe_args(gate, up, down, x, sel, wt, n_expert, n_ffn, n_embd)
+        resid = np.zeros((rows, n_embd), np.float32)
+        s = self._l.jlc_time_moe_block(self._p, _p(resid, _f32p), banks[0][1], banks[1][1], banks[2][1], _p(x, _f32p),
+                                       _p(sel, _u32p), sel.shape[1], _p(wt, _f32p), rows, k_used, n_expert, n_ffn,
+                                       n_embd, window, reps)
         if s < 0:
             raise ValueError("cpu timing refused")
         return s

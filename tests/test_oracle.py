@@ -386,6 +386,65 @@ def test_cpu_baseline_restatement(t, window):
         assert nmse(got, want) < 1e-10
 
 
+@pytest.mark.parametrize("ntok,window", [(1, 256), (5, 256), (70, 256), (9, 32)])
+def test_cpu_baseline_gemm_restatement(ntok, window):
+    """The weight-stationary prefill GEMM of the CPU baseline (the port of
+    /root/reference/jit/cpu/packedgemm.go:37-75): token t of the GEMM is the fused matvec of
+    token t bit for bit (the reference's own gate, nn.TestMatMulPackedMatchesTheRowLoopExactly),
+    and every token meets the oracle's like-for-like bar.  Ragged token blocks (70 = 64 + 6), a
+    row count that is not a multiple of 16, an expert's sheet inside a bank's planes."""
+    t, nrows, k = Q4_K, 264, 1024
+    w = synth.random_weights(t, nrows, k, seed=3)
+    x = np.stack([synth.activations(k, seed=40 + i) * np.float32(1 + i % 3) for i in range(ntok)])
+    qs, d, sc = oracle.pack_weights(t, w, nrows, k)
+    want = oracle.matmul_q8act_f64(t, w, x, nrows, k, ntok, window)
+    for threads in (1, 3):
+        cp = oracle.CpuPath(threads)
+        got = cp.matmul_packed(t, qs, d, sc, x, nrows, k, ntok, window)
+        assert nmse(got, want) < 1e-10
+        for tok in (0, ntok - 1):
+            mv = cp.matvec_packed(t, qs, d, sc, x[tok], nrows, k, window)
+            assert np.array_equal(got[tok].view(np.uint32), mv.view(np.uint32)), "GEMM token != fused matvec"
+        # rows 64..199 of the same planes as a matrix of their own (an expert's sheet)
+        sub = cp.matmul_packed(t, qs, d, sc, x, 136, k, ntok, window, row0=64, stride=nrows)
+        assert np.array_equal(sub.view(np.uint32), got[:, 64:200].view(np.uint32))
+        cp.close()
+
+
+def test_cpu_baseline_mixture_block_restatement():
+    """The CPU baseline's routed feed-forward block (the port of moeBatchExpert,
+    /root/reference/engine/model/moe.go:697-761) against the block built from the oracle's
+    own pieces: per (row, expert) the like-for-like matvecs, silu(g) * u, the weighted sum."""
+    rows, n_expert, k_used, n_ffn, n_embd, window = 9, 6, 2, 256, 512, 256
+    rng = np.random.default_rng(3)
+    sel = np.zeros((rows, k_used + 1), np.uint32)
+    wt = np.zeros((rows, k_used), np.float32)
+    for r in range(rows):
+        s, wv, _, _ = oracle.moe_route(rng.standard_normal(n_expert).astype(np.float32), k_used)
+        sel[r, :k_used], wt[r] = s, wv
+    mk = lambda nr, kk, seed: np.concatenate([synth.quantized_weights(Q4_K, nr, kk, seed=seed + e) for e in range(n_expert)])
+    gate, up, down = mk(n_ffn, n_embd, 100), mk(n_ffn, n_embd, 200), mk(n_embd, n_ffn, 300)
+    x = np.stack([synth.activations(n_embd, seed=50 + r) for r in range(rows)])
+    gs, ds = n_ffn * quant.row_bytes(Q4_K, n_embd), n_embd * quant.row_bytes(Q4_K, n_ffn)
+    want = np.zeros((rows, n_embd))
+    for r in range(rows):
+        q, a_s, _ = oracle.quantize_act(x[r], window)
+        for s_ in range(k_used):
+            e = int(sel[r, s_])
+            g = oracle.matvec_q8act_f64(Q4_K, gate[e * gs:(e + 1) * gs], q, a_s, n_ffn, n_embd).astype(np.float32)
+            u = oracle.matvec_q8act_f64(Q4_K, up[e * gs:(e + 1) * gs], q, a_s, n_ffn, n_embd).astype(np.float32)
+            h = (g.astype(np.float64) / (1 + np.exp(-g.astype(np.float64))) * u).astype(np.float32)
+            qh, ah, _ = oracle.quantize_act(h, window)
+            want[r] += float(wt[r, s_]) * oracle.matvec_q8act_f64(Q4_K, down[e * ds:(e + 1) * ds], qh, ah, n_embd, n_ffn)
+    planes = lambda bank, nr, kk: oracle.pack_weights(Q4_K, bank, n_expert * nr, kk)
+    cp = oracle.CpuPath(3)
+    got = cp.moe_block(planes(gate, n_ffn, n_embd), planes(up, n_ffn, n_embd), planes(down, n_embd, n_ffn), x, sel, wt,
+                       n_expert, n_ffn, n_embd, window)
+    cp.close()
+    err = float(np.sqrt(np.sum((got - want) ** 2) / np.sum(want ** 2)))
+    assert err <= 1e-4, f"rel-L2 {err:.3e}"
+
+
 # ------------------------------------------------------------------------- MoE
 def test_rmsnorm32_known_answers_and_invariants():
     """RMSNorm32 (/root/reference/internal/oracle/oracle.go:230-240) pinned without retyping
