@@ -296,6 +296,59 @@ int jl_matmul_dev(jl_ctx *ctx, float *out, int type, const void *w, const float 
  * calls allocate nothing. */
 int jl_reserve(jl_ctx *ctx, int max_tok, int max_k);
 
+/* nn.LayerDevice.PrepLayer / Layers / ReleaseLayers (engine/nn/device.go:1096-1176) for the
+ * matmul part of a block: a block's feed-forward weights are handed over ONCE and the block is
+ * then run by handle, so that no weight pointer crosses the boundary per call.  (Attention,
+ * rotary tables, KV migration and the head are other parts of that interface and not of this
+ * path.)
+ *
+ * jl_prep_layer uploads block li's weights from HOST memory (LayerPlan + LayerWeights) and keeps
+ * them until jl_release_layers: JL_DECLINED when a type or shape has no kernel or the block does
+ * not fit in device memory -- the reference then runs that block and every later one on the
+ * CPU.  Preparing a block again replaces it.
+ *   kind JL_LAYER_DENSE: the gated feed-forward block  resid += W_down (silu(W_gate h) * W_up h);
+ *       gate and up of `type` [n_ffn][n_embd], down of `down_type` [n_embd][n_ffn].  norm_w, when
+ *       set, is an RMSNorm in front of gate and up (h = RMSNorm(x, norm_w, norm_eps), as in
+ *       jl_matvec_group_dev).
+ *   kind JL_LAYER_MOE: the routed block of jl_moe_ffn_types_dev behind its own router: router
+ *       f32 [n_expert][n_embd], softmax and top-k_used (jl_moe_logits_dev, jl_moe_route_dev), banks
+ *       of n_expert sheets.
+ *   packed = 0: gate / up / down point at GGUF row-major bytes (a bank: its sheets back to back);
+ *   packed = 1: they point at a jl_host_planes each, the three packed planes of the matrix (of a
+ *       bank: ONE plane set of n_expert * rows rows, an expert's sheet a row range of it).
+ *
+ * jl_layer_ffn_dev runs block li for n rows: h [n][n_embd] in, resid [n][n_embd] updated, both in
+ * device memory (they may be one buffer, as they are for a block with its norm in front: every
+ * launch that reads a row of h has been enqueued before the one that adds to it).  One row runs the
+ * decode kernels (two launches for a dense block), more rows the grouped kernels of the mixture
+ * block (a dense block is a mixture of one expert that every row selects with weight 1; with
+ * norm_w set its rows run one at a time).  The values are those of the pointer-form entry points
+ * on the same operands, bit for bit.  Workspaces are the context's (calls on one context are
+ * serialized by the caller).
+ *
+ * jl_release_layers frees blocks lo .. hi-1 (those that are prepared). */
+#define JL_LAYER_DENSE 0
+#define JL_LAYER_MOE 1
+typedef struct jl_host_planes {
+    const uint32_t *qs, *d, *sc;   /* host memory; sc may be null for Q8_0 */
+} jl_host_planes;
+typedef struct jl_layer_plan {
+    int kind;
+    int type, down_type;
+    int n_embd, n_ffn;
+    int packed;
+    const void *gate, *up, *down;
+    const float *norm_w;           /* dense only; may be null */
+    float norm_eps;
+    int n_expert, k_used;          /* mixture only */
+    const float *router;           /* mixture only */
+} jl_layer_plan;
+int jl_prep_layer(jl_ctx *ctx, int li, const jl_layer_plan *plan);
+int jl_layer_ffn_dev(jl_ctx *ctx, int li, const float *h, float *resid, int n, void *stream);
+int jl_release_layers(jl_ctx *ctx, int lo, int hi);
+/* blocks resident now */
+int jl_layer_count(jl_ctx *ctx);
+
 /* The same for one call shape, exactly: walks the launch path of jl_matmul_dev
  * (packed = 0), jl_matmul_packed_dev (packed = 1) or, for type MXFP4,
  * jl_matmul_mxfp4_bf16_dev / jl_matmul_mxfp4_packed_bf16_dev, for this type, shape and the

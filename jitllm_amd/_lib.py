@@ -36,6 +36,21 @@ class PackedBank(C.Structure):
                 ("stride", C.c_int)]
 
 
+class HostPlanes(C.Structure):
+    """jl_host_planes: a matrix's (a bank's) three packed planes in host memory."""
+    _fields_ = [("qs", C.c_void_p), ("d", C.c_void_p), ("sc", C.c_void_p)]
+
+
+class LayerPlan(C.Structure):
+    """jl_layer_plan: a block's feed-forward weights as jl_prep_layer takes them (host memory)."""
+    _fields_ = [("kind", C.c_int), ("type", C.c_int), ("down_type", C.c_int), ("n_embd", C.c_int),
+                ("n_ffn", C.c_int), ("packed", C.c_int), ("gate", C.c_void_p), ("up", C.c_void_p),
+                ("down", C.c_void_p), ("norm_w", C.c_void_p), ("norm_eps", C.c_float), ("n_expert", C.c_int),
+                ("k_used", C.c_int), ("router", C.c_void_p)]
+
+
+LAYER_DENSE, LAYER_MOE = 0, 1
+
 # name -> (restype, argtypes); every symbol include/jlmi.h declares
 SIGNATURES = {
     "jl_hip_runtime": (C.c_char_p, []),
@@ -69,6 +84,10 @@ SIGNATURES = {
     "jl_matmul_static_dev": (_int, [_vp, _vp, _int, _vp, _vp, _int, _int, _int, _vp]),
     "jl_static_scratch_bytes": (_sz, []),
     "jl_reserve": (_int, [_vp, _int, _int]),
+    "jl_prep_layer": (_int, [_vp, _int, C.POINTER(LayerPlan)]),
+    "jl_layer_ffn_dev": (_int, [_vp, _int, _vp, _vp, _int, _vp]),
+    "jl_release_layers": (_int, [_vp, _int, _int]),
+    "jl_layer_count": (_int, [_vp]),
     "jl_packed_words": (_int, [_int, _int, _int, C.POINTER(_sz), C.POINTER(_sz), C.POINTER(_sz)]),
     "jl_matvec_packed": (_int, [_vp, _vp, _int, _vp, _vp, _vp, _int, _int, _vp, _int, _int]),
     "jl_matmul_packed": (_int, [_vp, _vp, _int, _vp, _vp, _vp, _int, _int, _vp, _int, _int, _int]),

@@ -59,6 +59,19 @@ struct Resident {
     size_t bytes = 0;
 };
 
+// A block whose feed-forward weights jl_prep_layer made resident: one device allocation, the
+// pieces' addresses in it.
+struct Layer {
+    jl_layer_plan plan;          // host pointers cleared
+    void* mem = nullptr;         // the allocation
+    // packed = 0: the matrices' (banks') bytes; packed = 1: plane sets
+    const void *gate = nullptr, *up = nullptr, *down = nullptr;
+    const uint32_t *gp[3] = {nullptr, nullptr, nullptr}, *upl[3] = {nullptr, nullptr, nullptr},
+                   *dp[3] = {nullptr, nullptr, nullptr};
+    const float* norm_w = nullptr;
+    const float* router = nullptr;
+};
+
 }  // namespace
 
 struct jl_ctx {
@@ -109,6 +122,12 @@ struct jl_ctx {
     // mixture-of-experts workspace (grouping tables and intermediate columns)
     void* moe_ws = nullptr;
     size_t moe_ws_bytes = 0;
+
+    // blocks prepared by jl_prep_layer, and the workspace their runs share (router logits,
+    // selection and weights of a mixture; gate and up of a dense block at one row)
+    std::map<int, Layer> layers;
+    void* layer_ws = nullptr;
+    size_t layer_ws_bytes = 0;
 
     // host-pointer seam state
     std::map<const void*, Resident> resident;
@@ -1394,7 +1413,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     if (e != hipSuccess)
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
-    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_matvec_q8_0p_r1", "jl_matvec_q8_0p_r2", "jl_matvec_q8_0p_r4", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_q4k_k2", "jl_gemm_q4k_k2_planes", "jl_gemm_prep_q4k_planes", "jl_gemm_q4k_r64_planes", "jl_gemm_q4k_wide_planes", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_group2_wide", "jl_moe_quant", "jl_moe_matvec_planes_q4k", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_prep_planes", "jl_moe_gemm_q4k", "jl_moe_g16_prep", "jl_moe_g16_prep_planes", "jl_moe_g16_prep_q6k", "jl_moe_g16_c1", "jl_moe_g16_c2", "jl_moe_g16_c3", "jl_moe_g16_f1", "jl_moe_g16_f2", "jl_moe_g16_f3", "jl_moe_g16_g1", "jl_moe_g16_g2", "jl_moe_g16_g3", "jl_moe_g16_d1", "jl_moe_g16_d2", "jl_moe_g16_d3", "jl_moe_g16p_c1", "jl_moe_g16p_c2", "jl_moe_g16p_c3", "jl_moe_g16p_f1", "jl_moe_g16p_f2", "jl_moe_g16p_f3", "jl_moe_g16p_g1", "jl_moe_g16p_g2", "jl_moe_g16p_g3", "jl_moe_g16p_d1", "jl_moe_g16p_d2", "jl_moe_g16p_d3", "jl_moe_g16q6_c1", "jl_moe_g16q6_c2", "jl_moe_g16q6_c3", "jl_moe_g16q6_f1", "jl_moe_g16q6_f2", "jl_moe_g16q6_f3", "jl_moe_g16q6_g1", "jl_moe_g16q6_g2", "jl_moe_g16q6_g3", "jl_moe_g16q6_d1", "jl_moe_g16q6_d2", "jl_moe_g16q6_d3", "jl_moe_gemm_r64", "jl_moe_gemm_r64_planes", "jl_moe_gemm_q6k_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_mxfp4_matvec1_b1", "jl_mxfp4_matvec1_b2", "jl_mxfp4_matvec1_b3", "jl_mxfp4_scaled_prep", "jl_mxfp4_scaled_gemm", "jl_mxfp4_planes_prep", "jl_mxfp4_planes_gemm", "jl_mxfp4_matvec_planes_r64", "jl_mxfp4_matvec_planes_r32", "jl_mxfp4_matvec_planes_r16", "jl_unpack_mxfp4", "jl_sum_parts", "jl_probe_read", "jl_probe_empty", "jl_probe_wait", "jl_probe_mfma", "jl_probe_mfma_v5",
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_matvec_q8_0p_r1", "jl_matvec_q8_0p_r2", "jl_matvec_q8_0p_r4", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_q4k_k2", "jl_gemm_q4k_k2_planes", "jl_gemm_prep_q4k_planes", "jl_gemm_q4k_r64_planes", "jl_gemm_q4k_wide_planes", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_group2_wide", "jl_moe_quant", "jl_moe_matvec_planes_q4k", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_prep_planes", "jl_moe_gemm_q4k", "jl_moe_g16_prep", "jl_moe_g16_prep_planes", "jl_moe_g16_prep_q6k", "jl_moe_g16_c1", "jl_moe_g16_c2", "jl_moe_g16_c3", "jl_moe_g16_f1", "jl_moe_g16_f2", "jl_moe_g16_f3", "jl_moe_g16_g1", "jl_moe_g16_g2", "jl_moe_g16_g3", "jl_moe_g16_d1", "jl_moe_g16_d2", "jl_moe_g16_d3", "jl_moe_g16p_c1", "jl_moe_g16p_c2", "jl_moe_g16p_c3", "jl_moe_g16p_f1", "jl_moe_g16p_f2", "jl_moe_g16p_f3", "jl_moe_g16p_g1", "jl_moe_g16p_g2", "jl_moe_g16p_g3", "jl_moe_g16p_d1", "jl_moe_g16p_d2", "jl_moe_g16p_d3", "jl_moe_g16q6_c1", "jl_moe_g16q6_c2", "jl_moe_g16q6_c3", "jl_moe_g16q6_f1", "jl_moe_g16q6_f2", "jl_moe_g16q6_f3", "jl_moe_g16q6_g1", "jl_moe_g16q6_g2", "jl_moe_g16q6_g3", "jl_moe_g16q6_d1", "jl_moe_g16q6_d2", "jl_moe_g16q6_d3", "jl_moe_gemm_r64", "jl_moe_gemm_r64_planes", "jl_moe_gemm_q6k_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_mxfp4_matvec1_b1", "jl_mxfp4_matvec1_b2", "jl_mxfp4_matvec1_b3", "jl_mxfp4_scaled_prep", "jl_mxfp4_scaled_gemm", "jl_mxfp4_planes_prep", "jl_mxfp4_planes_gemm", "jl_mxfp4_matvec_planes_r64", "jl_mxfp4_matvec_planes_r32", "jl_mxfp4_matvec_planes_r16", "jl_unpack_mxfp4", "jl_sum_parts", "jl_fill_u32", "jl_probe_read", "jl_probe_empty", "jl_probe_wait", "jl_probe_mfma", "jl_probe_mfma_v5",
                                       "jl_pack_weights", "jl_unpack_q4k", "jl_unpack_q6k", "jl_unpack_q8_0"};
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int rw : {16, 32, 64})
@@ -1462,6 +1481,9 @@ void jl_ctx_destroy(jl_ctx* c) {
     if (c->flag_ws) (void)H->Free(c->flag_ws);
     if (c->moe_q_ws) (void)H->Free(c->moe_q_ws);
     if (c->act_ws) (void)H->Free(c->act_ws);
+    if (c->layer_ws) (void)H->Free(c->layer_ws);
+    for (auto& kv : c->layers)
+        if (kv.second.mem) (void)H->Free(kv.second.mem);
     if (c->one_group) (void)H->Free(c->one_group);
     if (c->mx_ws) (void)H->Free(c->mx_ws);
     if (c->stage_x) (void)H->Free(c->stage_x);
@@ -1953,6 +1975,208 @@ int jl_moe_ffn_dev(jl_ctx* c, float* resid, int type, const void* gate_bank, con
                    const float* wt, int rows, int k_used, int n_expert, int n_ffn, int n_embd, void* stream) {
     return jl_moe_ffn_types_dev(c, resid, type, type, gate_bank, up_bank, down_bank, x, sel, sel_stride, wt, rows,
                                 k_used, n_expert, n_ffn, n_embd, stream);
+}
+
+// ------------------------------------------------------------------ the block seam
+namespace {
+size_t up256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+// Bytes of one matrix (or bank of `sheets` sheets) of a plan: GGUF bytes, or its three planes
+// (each rounded up to 256 bytes so that every plane starts aligned).
+bool layer_matrix_bytes(int type, int packed, size_t nrows, int k, size_t* total, size_t plane[3]) {
+    const TypeInfo* ti = type_info(type);
+    if (!ti || k % ti->block_elems) return false;
+    if (!packed) {
+        *total = nrows * (size_t)(k / ti->block_elems) * ti->block_bytes;
+        return true;
+    }
+    size_t nq, nd, nsc;
+    if (nrows > 0x7fffffff || !packed_words(type, nrows, k, &nq, &nd, &nsc)) return false;
+    plane[0] = nq * 4; plane[1] = nd * 4; plane[2] = nsc * 4;
+    *total = up256(plane[0]) + up256(plane[1]) + up256(plane[2]);
+    return true;
+}
+}  // namespace
+
+int jl_prep_layer(jl_ctx* c, int li, const jl_layer_plan* plan) {
+    if (!c) return JL_ERR_ARG;
+    if (!plan || li < 0) return fail(c, JL_ERR_ARG, "prep layer: bad argument");
+    const jl_layer_plan& P = *plan;
+    if (P.n_embd <= 0 || P.n_ffn <= 0 || !P.gate || !P.up || !P.down)
+        return fail(c, JL_ERR_ARG, "prep layer %d: missing weights or shape", li);
+    const bool moe = P.kind == JL_LAYER_MOE;
+    if (P.kind != JL_LAYER_DENSE && !moe) return fail(c, JL_ERR_ARG, "prep layer %d: kind %d", li, P.kind);
+    if (moe && (P.n_expert < 1 || P.k_used < 1 || P.k_used > P.n_expert || !P.router))
+        return fail(c, JL_ERR_ARG, "prep layer %d: mixture without router or experts", li);
+    if (moe && (P.n_expert > 1024 || P.k_used > 16 || P.n_ffn % 256 || P.n_embd % 256)) return JL_DECLINED;
+    if (moe && P.norm_w) return JL_DECLINED;
+    if (P.packed && P.type != P.down_type && moe) return JL_DECLINED;   // packed banks: one type
+    const size_t sheets = moe ? (size_t)P.n_expert : 1;
+    size_t bg, bd, pg[3], pd[3];
+    if (!layer_matrix_bytes(P.type, P.packed, sheets * P.n_ffn, P.n_embd, &bg, pg) ||
+        !layer_matrix_bytes(P.down_type, P.packed, sheets * P.n_embd, P.n_ffn, &bd, pd))
+        return JL_DECLINED;   // a type or shape without a kernel
+    HIP_TRY(c, H->SetDevice(c->device));
+    const size_t o_gate = 0, o_up = up256(bg), o_down = o_up + up256(bg), o_norm = o_down + up256(bd);
+    const size_t o_router = o_norm + up256(P.norm_w ? (size_t)P.n_embd * 4 : 0);
+    const size_t total = o_router + up256(moe ? (size_t)P.n_expert * P.n_embd * 4 : 0);
+    jl_release_layers(c, li, li + 1);
+    void* mem = nullptr;
+    if (H->Malloc(&mem, total) != hipSuccess) {
+        (void)H->GetLastError();
+        return JL_DECLINED;   // the block does not fit: it stays on the host
+    }
+    Layer L;
+    L.plan = P;
+    L.plan.gate = L.plan.up = L.plan.down = nullptr;
+    L.plan.norm_w = L.plan.router = nullptr;
+    L.mem = mem;
+    char* base = (char*)mem;
+    auto fail_free = [&](hipError_t e, const char* what) {
+        (void)H->Free(mem);
+        return fail(c, JL_ERR_HIP, "prep layer %d: %s: %s", li, what, H->GetErrorString(e));
+    };
+    auto put = [&](size_t off, const void* src, size_t n) { return H->Memcpy(base + off, src, n, hipMemcpyHostToDevice); };
+    hipError_t e = hipSuccess;
+    if (!P.packed) {
+        if ((e = put(o_gate, P.gate, bg)) != hipSuccess || (e = put(o_up, P.up, bg)) != hipSuccess ||
+            (e = put(o_down, P.down, bd)) != hipSuccess)
+            return fail_free(e, "weight upload");
+        L.gate = base + o_gate; L.up = base + o_up; L.down = base + o_down;
+    } else {
+        auto put_planes = [&](size_t off, const void* hp, const size_t pl[3], const uint32_t* out[3]) {
+            const jl_host_planes* h = (const jl_host_planes*)hp;
+            const uint32_t* src[3] = {h->qs, h->d, h->sc};
+            for (int i = 0; i < 3; i++) {
+                out[i] = (const uint32_t*)(base + off);
+                if (pl[i]) {
+                    if (!src[i]) return hipErrorInvalidValue;
+                    hipError_t ee = put(off, src[i], pl[i]);
+                    if (ee != hipSuccess) return ee;
+                }
+                off += up256(pl[i]);
+            }
+            return hipSuccess;
+        };
+        if ((e = put_planes(o_gate, P.gate, pg, L.gp)) != hipSuccess || (e = put_planes(o_up, P.up, pg, L.upl)) != hipSuccess ||
+            (e = put_planes(o_down, P.down, pd, L.dp)) != hipSuccess)
+            return fail_free(e, "plane upload");
+    }
+    if (P.norm_w) {
+        if ((e = put(o_norm, P.norm_w, (size_t)P.n_embd * 4)) != hipSuccess) return fail_free(e, "norm upload");
+        L.norm_w = (const float*)(base + o_norm);
+    }
+    if (moe) {
+        if ((e = put(o_router, P.router, (size_t)P.n_expert * P.n_embd * 4)) != hipSuccess) return fail_free(e, "router upload");
+        L.router = (const float*)(base + o_router);
+    }
+    c->layers[li] = L;
+    return JL_OK;
+}
+
+int jl_release_layers(jl_ctx* c, int lo, int hi) {
+    if (!c) return JL_ERR_ARG;
+    bool any = false;
+    for (auto it = c->layers.lower_bound(lo); it != c->layers.end() && it->first < hi;) {
+        if (!any && !c->no_device) {
+            // kernels enqueued by earlier runs may still read the block
+            (void)H->SetDevice(c->device);
+            (void)H->DeviceSynchronize();
+            any = true;
+        }
+        if (it->second.mem) (void)H->Free(it->second.mem);
+        it = c->layers.erase(it);
+    }
+    return JL_OK;
+}
+
+int jl_layer_count(jl_ctx* c) { return c ? (int)c->layers.size() : 0; }
+
+int jl_layer_ffn_dev(jl_ctx* c, int li, const float* h, float* resid, int n, void* stream) {
+    if (!c) return JL_ERR_ARG;
+    auto it = c->layers.find(li);
+    if (it == c->layers.end()) return fail(c, JL_ERR_ARG, "layer %d is not prepared", li);
+    if (!h || !resid || n <= 0) return fail(c, JL_ERR_ARG, "layer %d: bad operand", li);
+    const Layer& L = it->second;
+    const jl_layer_plan& P = L.plan;
+    HIP_TRY(c, H->SetDevice(c->device));
+    hipStream_t st = pick_stream(c, stream);
+    const int E = P.n_embd, F = P.n_ffn;
+    jl_packed_bank bg, bu, bd;
+    if (P.packed) {
+        const int sheets = P.kind == JL_LAYER_MOE ? P.n_expert : 1;
+        bg = jl_packed_bank{L.gp[0], L.gp[1], L.gp[2], 0, sheets * F};
+        bu = jl_packed_bank{L.upl[0], L.upl[1], L.upl[2], 0, sheets * F};
+        bd = jl_packed_bank{L.dp[0], L.dp[1], L.dp[2], 0, sheets * E};
+    }
+    if (P.kind == JL_LAYER_MOE) {
+        const size_t o_sel = up256((size_t)n * P.n_expert * 4), o_wt = o_sel + up256((size_t)n * (P.k_used + 1) * 4);
+        int rc = grow(c, &c->layer_ws, &c->layer_ws_bytes, o_wt + up256((size_t)n * P.k_used * 4));
+        if (rc != JL_OK) return rc;
+        float* logits = (float*)c->layer_ws;
+        uint32_t* sel = (uint32_t*)((char*)c->layer_ws + o_sel);
+        float* wt = (float*)((char*)c->layer_ws + o_wt);
+        rc = jl_moe_logits_dev(c, logits, JL_TYPE_F32, L.router, h, P.n_expert, E, n, st);
+        if (rc != JL_OK) return rc;
+        rc = jl_moe_route_dev(c, logits, n, P.n_expert, P.k_used, sel, P.k_used + 1, wt, st);
+        if (rc != JL_OK) return rc;
+        return moe_ffn(c, resid, P.type, P.down_type, L.gate, L.up, L.down, P.packed ? &bg : nullptr,
+                       P.packed ? &bu : nullptr, P.packed ? &bd : nullptr, h, sel, P.k_used + 1, wt, n, P.k_used,
+                       P.n_expert, F, E, st);
+    }
+    // dense.  More than one row without a norm in front: the grouped kernels, the block as a
+    // mixture of one expert that every row selects with weight 1.
+    if (n > 1 && !L.norm_w && F % 256 == 0 && E % 256 == 0 && (!P.packed || P.type == P.down_type)) {
+        const size_t o_wt = up256((size_t)n * 2 * 4);
+        int rc = grow(c, &c->layer_ws, &c->layer_ws_bytes, o_wt + up256((size_t)n * 4));
+        if (rc != JL_OK) return rc;
+        uint32_t* sel = (uint32_t*)c->layer_ws;
+        float* wt = (float*)((char*)c->layer_ws + o_wt);
+        size_t n_sel = (size_t)n * 2, n_wt = (size_t)n;
+        uint32_t zero = 0, one = 0x3F800000u;
+        void* p0[] = {&sel, &n_sel, &zero};
+        rc = launch(c, "jl_fill_u32", (unsigned)((n_sel + 255) / 256), 1, 256, 0, st, p0);
+        if (rc != JL_OK) return rc;
+        void* p1[] = {&wt, &n_wt, &one};
+        rc = launch(c, "jl_fill_u32", (unsigned)((n_wt + 255) / 256), 1, 256, 0, st, p1);
+        if (rc != JL_OK) return rc;
+        rc = moe_ffn(c, resid, P.type, P.down_type, L.gate, L.up, L.down, P.packed ? &bg : nullptr, P.packed ? &bu : nullptr,
+                     P.packed ? &bd : nullptr, h, sel, 2, wt, n, 1, 1, F, E, st);
+        if (rc != JL_DECLINED) return rc;
+    }
+    // one row at a time: gate and up in one launch (the norm riding in front), down over
+    // silu(gate) * up with the residual add riding on it
+    const size_t fb = up256((size_t)F * 4);
+    int rc = grow(c, &c->layer_ws, &c->layer_ws_bytes, 2 * fb + up256((size_t)E * 4));
+    if (rc != JL_OK) return rc;
+    float* g = (float*)c->layer_ws;
+    float* u = (float*)((char*)c->layer_ws + fb);
+    float* y = (float*)((char*)c->layer_ws + 2 * fb);   // down's own rows (resid takes them as they are made)
+    for (int r = 0; r < n; r++) {
+        const float* hr = h + (size_t)r * E;
+        float* rr = resid + (size_t)r * E;
+        float* gu[2] = {g, u};
+        float* yo[1] = {y};
+        if (!P.packed) {
+            const void* wgu[2] = {L.gate, L.up};
+            const int rgu[2] = {F, F};
+            rc = matvec_multi_launch(c, P.type, 2, gu, wgu, rgu, hr, 0, nullptr, nullptr, 0.f, E, st, L.norm_w, P.norm_eps);
+            if (rc != JL_OK) return rc;
+            const void* wd[1] = {L.down};
+            const int rd[1] = {E};
+            rc = matvec_multi_launch(c, P.down_type, 1, yo, wd, rd, g, 0, u, rr, 1.0f, F, st);
+        } else {
+            PlaneRef pgu[2] = {{L.gp[0], L.gp[1], L.gp[2], 0, F}, {L.upl[0], L.upl[1], L.upl[2], 0, F}};
+            rc = packed_matvec_multi_launch(c, P.type, 2, gu, pgu, hr, 0, nullptr, nullptr, 0.f, nullptr, L.norm_w,
+                                            P.norm_eps, nullptr, F, E, st);
+            if (rc != JL_OK) return rc;
+            PlaneRef pd1[1] = {{L.dp[0], L.dp[1], L.dp[2], 0, E}};
+            rc = packed_matvec_multi_launch(c, P.down_type, 1, yo, pd1, g, 0, u, rr, 1.0f, nullptr, nullptr, 0.f, nullptr,
+                                            E, F, st);
+        }
+        if (rc != JL_OK) return rc;
+    }
+    return JL_OK;
 }
 
 int jl_matmul_mxfp4_bf16_dev(jl_ctx* c, float* out, const void* w, const uint16_t* x, int nrows, int k,

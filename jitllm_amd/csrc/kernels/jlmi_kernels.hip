@@ -388,6 +388,13 @@ extern "C" __global__ __launch_bounds__(256) void jl_mxfp4_prep_few(MxPrepArgs p
     }
 JL_MX_FEW_KERNEL(1) JL_MX_FEW_KERNEL(2) JL_MX_FEW_KERNEL(3) JL_MX_FEW_KERNEL(4)
 
+// n words of `value`: the selection and weight tables of a dense block run as a mixture of one
+// expert (a kernel, not a memset, so that a caller may capture it).  grid = ceil(n / 256), block = 256
+extern "C" __global__ __launch_bounds__(256) void jl_fill_u32(u32* __restrict__ dst, size_t n, u32 value) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) dst[i] = value;
+}
+
 // ------------------------------------------------------------------ probes
 // What one launch costs on this machine before any arithmetic: jl_probe_read streams nvec
 // 16-byte vectors with every thread keeping eight loads in flight and folds them into a word

@@ -83,6 +83,49 @@ class Device:
         """nn.LayerDevice.Reserve: size the prefill workspace ahead of time."""
         self._served(self._l.jl_reserve(self._ctx, max_tok, max_k), "jl_reserve")
 
+    def PrepLayer(self, li, kind, t, n_embd, n_ffn, gate, up, down, down_type=None, norm_w=None, norm_eps=0.0,
+                  n_expert=0, k_used=0, router=None):
+        """nn.LayerDevice.PrepLayer for a block's feed-forward weights
+        (/root/reference/engine/nn/device.go:1096-1131): uploaded once from host memory and kept until
+        ReleaseLayers.  gate / up / down are numpy arrays of GGUF bytes, or (qs, d, sc) tuples of
+        packed planes (sc None for Q8_0); router f32 [n_expert][n_embd] for a mixture.  False when
+        the block is declined (no kernel for it, or it does not fit): it then stays on the host."""
+        keep = []
+
+        def host(a):
+            if a is None:
+                return None
+            a = np.ascontiguousarray(a)
+            keep.append(a)
+            return a.ctypes.data
+
+        packed = isinstance(gate, tuple)
+        if packed:
+            def planes(m):
+                hp = _lib.HostPlanes(host(m[0]), host(m[1]), host(m[2]))
+                keep.append(hp)
+                return C.cast(C.pointer(hp), C.c_void_p).value
+            g, u, d = planes(gate), planes(up), planes(down)
+        else:
+            g, u, d = host(gate), host(up), host(down)
+        plan = _lib.LayerPlan(int(kind), int(t), int(t if down_type is None else down_type), int(n_embd), int(n_ffn),
+                              int(packed), g, u, d, host(norm_w), float(norm_eps), int(n_expert), int(k_used),
+                              host(router))
+        return self._served(self._l.jl_prep_layer(self._ctx, int(li), C.byref(plan)), "jl_prep_layer")
+
+    def layer_ffn_dev(self, li, h, resid, n, stream=None):
+        """Run prepared block li's feed-forward for n rows: resid [n][n_embd] += ffn(h [n][n_embd])."""
+        return self._served(self._l.jl_layer_ffn_dev(self._ctx, int(li), _ptr(h), _ptr(resid), int(n), stream),
+                            "jl_layer_ffn_dev")
+
+    def ReleaseLayers(self, lo, hi):
+        """nn.LayerDevice.ReleaseLayers (/root/reference/engine/nn/device.go:1160-1176)."""
+        self._served(self._l.jl_release_layers(self._ctx, int(lo), int(hi)), "jl_release_layers")
+
+    def Layers(self):
+        """nn.LayerDevice.Layers: how many blocks are resident."""
+        return int(self._l.jl_layer_count(self._ctx))
+
     def reserve_shape(self, t, nrows, k, ntok, packed=False):
         """Grow every workspace a matmul of this shape would grow, launching nothing."""
         return self._served(self._l.jl_reserve_shape(self._ctx, t, nrows, k, ntok, int(packed)), "jl_reserve_shape")
