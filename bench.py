@@ -497,12 +497,10 @@ def moe_section(dev, gate_, rows=64, packed=False, cpu=False):
             pbanks.append(dev.packed_bank(pl[0].ptr, pl[1].ptr, pl[2].ptr, 0, r * n_expert))
 
     def run(_):
-        if not (dev.moe_logits_dev(ld.ptr, 0, router.ptr, x.ptr, n_expert, n_embd, rows) and
-                dev.moe_route_dev(ld.ptr, rows, n_expert, k_used, sd.ptr, k_used + 1, wd.ptr) and
-                (dev.moe_ffn_packed_dev(resid.ptr, t, pbanks[0], pbanks[1], pbanks[2], x.ptr, sd.ptr, k_used + 1,
-                                        wd.ptr, rows, k_used, n_expert, n_ffn, n_embd) if packed else
-                 dev.moe_ffn_dev(resid.ptr, t, banks[0].ptr, banks[1].ptr, banks[2].ptr, x.ptr, sd.ptr,
-                                 k_used + 1, wd.ptr, rows, k_used, n_expert, n_ffn, n_embd))):
+        # one call: router logits, softmax + top-8, grouping, gate + up, down, combine
+        b = pbanks if packed else [bk.ptr for bk in banks[:3]]
+        if not dev.moe_block_dev(resid.ptr, t, b[0], b[1], b[2], router.ptr, x.ptr, rows, k_used, n_expert, n_ffn,
+                                 n_embd, sel=sd.ptr, wt=wd.ptr):
             raise RuntimeError("the device declined the mixture block")
     ms = measure(dev, run, 20, gate_)
     resid.zero()

@@ -532,6 +532,22 @@ int jl_moe_ffn_types_dev(jl_ctx *ctx, float *resid, int type, int down_type, con
                          const uint32_t *sel, int sel_stride, const float *wt, int rows,
                          int k_used, int n_expert, int n_ffn, int n_embd, void *stream);
 
+/* The whole mixture block for rows rows, router included (engine/model/moe.go:697-761 from the
+ * hidden state on): jl_moe_logits_dev (router f32 or f16, [n_expert][n_embd]), jl_moe_route_dev,
+ * then jl_moe_ffn_types_dev on that selection, in one call and bit for bit.  sel
+ * [rows][k_used + 1] and wt [rows][k_used] receive the routing when given (null: kept in the
+ * context's workspace, like the logits). */
+int jl_moe_block_dev(jl_ctx *ctx, float *resid, int type, int down_type, const void *gate_bank,
+                     const void *up_bank, const void *down_bank, int router_type, const void *router,
+                     const float *x, int rows, int k_used, int n_expert, int n_ffn, int n_embd,
+                     uint32_t *sel, float *wt, void *stream);
+
+/* The same over banks of packed planes (jl_moe_ffn_packed_dev behind the router). */
+int jl_moe_block_packed_dev(jl_ctx *ctx, float *resid, int type, const jl_packed_bank *gate,
+                            const jl_packed_bank *up, const jl_packed_bank *down, int router_type,
+                            const void *router, const float *x, int rows, int k_used, int n_expert,
+                            int n_ffn, int n_embd, uint32_t *sel, float *wt, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

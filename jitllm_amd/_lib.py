@@ -113,6 +113,11 @@ SIGNATURES = {
                               _int, _vp]),
     "jl_moe_ffn_types_dev": (_int, [_vp, _vp, _int, _int, _vp, _vp, _vp, _vp, _vp, _int, _vp, _int, _int, _int,
                                     _int, _int, _vp]),
+    "jl_moe_block_dev": (_int, [_vp, _vp, _int, _int, _vp, _vp, _vp, _int, _vp, _vp, _int, _int, _int, _int, _int,
+                                _vp, _vp, _vp]),
+    "jl_moe_block_packed_dev": (_int, [_vp, _vp, _int, C.POINTER(PackedBank), C.POINTER(PackedBank),
+                                       C.POINTER(PackedBank), _int, _vp, _vp, _int, _int, _int, _int, _int, _vp, _vp,
+                                       _vp]),
 }
 
 _lib = None

@@ -128,6 +128,9 @@ struct jl_ctx {
     std::map<int, Layer> layers;
     void* layer_ws = nullptr;
     size_t layer_ws_bytes = 0;
+    // a block's router logits and, when it is not handed a place for them, selection and weights
+    void* moe_route_ws = nullptr;
+    size_t moe_route_ws_bytes = 0;
 
     // host-pointer seam state
     std::map<const void*, Resident> resident;
@@ -1482,6 +1485,7 @@ void jl_ctx_destroy(jl_ctx* c) {
     if (c->moe_q_ws) (void)H->Free(c->moe_q_ws);
     if (c->act_ws) (void)H->Free(c->act_ws);
     if (c->layer_ws) (void)H->Free(c->layer_ws);
+    if (c->moe_route_ws) (void)H->Free(c->moe_route_ws);
     for (auto& kv : c->layers)
         if (kv.second.mem) (void)H->Free(kv.second.mem);
     if (c->one_group) (void)H->Free(c->one_group);
@@ -1918,6 +1922,28 @@ int jl_moe_combine_dev(jl_ctx* c, float* resid, const float* y, const float* wt,
 }
 
 namespace {
+// The routed block's workspace: first columns, row of a column, column of a pair, then gate, up
+// and down of every column.
+struct MoeWs {
+    uint32_t *start, *perm, *pos;
+    float *g, *u, *y;
+};
+int moe_ws(jl_ctx* c, int rows, int k_used, int n_expert, int n_ffn, int n_embd, MoeWs* w) {
+    const size_t ncols = (size_t)rows * k_used;
+    auto up256 = [](size_t v) { return (v + 255) & ~(size_t)255; };
+    const size_t o_start = 0, o_perm = up256((size_t)(n_expert + 1) * 4), o_pos = o_perm + up256(ncols * 4);
+    const size_t o_g = o_pos + up256(ncols * 4), o_u = o_g + up256(ncols * n_ffn * 4);
+    const size_t o_y = o_u + up256(ncols * n_ffn * 4), total = o_y + up256(ncols * n_embd * 4);
+    int rc = ws_ensure(c, &c->moe_ws, &c->moe_ws_bytes, total);
+    if (rc != JL_OK) return rc;
+    char* ws = (char*)c->moe_ws;
+    w->start = (uint32_t*)(ws + o_start);
+    w->perm = (uint32_t*)(ws + o_perm);
+    w->pos = (uint32_t*)(ws + o_pos);
+    w->g = (float*)(ws + o_g); w->u = (float*)(ws + o_u); w->y = (float*)(ws + o_y);
+    return JL_OK;
+}
+
 int moe_ffn(jl_ctx* c, float* resid, int type, int down_type, const void* gate_bank, const void* up_bank,
             const void* down_bank, const jl_packed_bank* pg, const jl_packed_bank* pu, const jl_packed_bank* pd,
             const float* x, const uint32_t* sel, int sel_stride, const float* wt, int rows, int k_used, int n_expert,
@@ -1929,17 +1955,11 @@ int moe_ffn(jl_ctx* c, float* resid, int type, int down_type, const void* gate_b
     HIP_TRY(c, H->SetDevice(c->device));
     hipStream_t st = pick_stream(c, stream);
     const size_t ncols = (size_t)rows * k_used;
-    auto up256 = [](size_t v) { return (v + 255) & ~(size_t)255; };
-    const size_t o_start = 0, o_perm = up256((size_t)(n_expert + 1) * 4), o_pos = o_perm + up256(ncols * 4);
-    const size_t o_g = o_pos + up256(ncols * 4), o_u = o_g + up256(ncols * n_ffn * 4);
-    const size_t o_y = o_u + up256(ncols * n_ffn * 4), total = o_y + up256(ncols * n_embd * 4);
-    int rc = ws_ensure(c, &c->moe_ws, &c->moe_ws_bytes, total);
+    MoeWs w;
+    int rc = moe_ws(c, rows, k_used, n_expert, n_ffn, n_embd, &w);
     if (rc != JL_OK) return rc;
-    char* ws = (char*)c->moe_ws;
-    uint32_t* start = (uint32_t*)(ws + o_start);
-    uint32_t* perm = (uint32_t*)(ws + o_perm);
-    uint32_t* pos = (uint32_t*)(ws + o_pos);
-    float *g = (float*)(ws + o_g), *u = (float*)(ws + o_u), *y = (float*)(ws + o_y);
+    uint32_t *start = w.start, *perm = w.perm, *pos = w.pos;
+    float *g = w.g, *u = w.u, *y = w.y;
     rc = jl_moe_group_dev(c, sel, sel_stride, rows, k_used, n_expert, start, perm, pos, st);
     if (rc != JL_OK) return rc;
     // gate and up: columns read the routed rows of x
@@ -1952,7 +1972,56 @@ int moe_ffn(jl_ctx* c, float* resid, int type, int down_type, const void* gate_b
     if (rc != JL_OK) return rc;
     return jl_moe_combine_dev(c, resid, y, wt, sel, sel_stride, pos, rows, k_used, n_embd, st);
 }
+
+// The whole block from the hidden state on: router logits, softmax + top-k, the routed
+// feed-forward.  (The three router steps as ONE launch -- the workgroup that stores a token
+// group's last logit routes it, the one that routes the last group sorts the pairs -- measured
+// slower than the launches it replaces, 117 us a 64-row block against 109: every hand-over inside
+// a launch is a device-scope store, an atomic and a device-scope load one after the other, which
+// costs what a launch boundary costs.)
+int moe_block(jl_ctx* c, float* resid, int type, int down_type, const void* gate_bank, const void* up_bank,
+              const void* down_bank, const jl_packed_bank* pg, const jl_packed_bank* pu, const jl_packed_bank* pd,
+              int rtype, const void* router, const float* x, int rows, int k_used, int n_expert, int n_ffn, int n_embd,
+              uint32_t* sel, float* wt, void* stream) {
+    if (rows <= 0 || k_used <= 0 || n_expert <= 0 || n_ffn <= 0 || n_embd <= 0 || !router || !x || !resid)
+        return fail(c, JL_ERR_ARG, "moe block: bad operand");
+    if (n_expert > 1024 || k_used > 16 || k_used > n_expert || n_ffn % 256 != 0 || n_embd % 256 != 0) return JL_DECLINED;
+    HIP_TRY(c, H->SetDevice(c->device));
+    hipStream_t st = pick_stream(c, stream);
+    const int sel_stride = k_used + 1;
+    auto up256 = [](size_t v) { return (v + 255) & ~(size_t)255; };
+    const size_t o_sel = up256((size_t)rows * n_expert * 4), o_wt = o_sel + up256((size_t)rows * sel_stride * 4);
+    int rc = ws_ensure(c, &c->moe_route_ws, &c->moe_route_ws_bytes, o_wt + up256((size_t)rows * k_used * 4));
+    if (rc != JL_OK) return rc;
+    float* logits = (float*)c->moe_route_ws;
+    if (!sel) sel = (uint32_t*)((char*)c->moe_route_ws + o_sel);
+    if (!wt) wt = (float*)((char*)c->moe_route_ws + o_wt);
+    rc = jl_moe_logits_dev(c, logits, rtype, router, x, n_expert, n_embd, rows, st);
+    if (rc != JL_OK) return rc;
+    rc = jl_moe_route_dev(c, logits, rows, n_expert, k_used, sel, sel_stride, wt, st);
+    if (rc != JL_OK) return rc;
+    return moe_ffn(c, resid, type, down_type, gate_bank, up_bank, down_bank, pg, pu, pd, x, sel, sel_stride, wt, rows, k_used,
+                   n_expert, n_ffn, n_embd, st);
+}
 }  // namespace
+
+int jl_moe_block_dev(jl_ctx* c, float* resid, int type, int down_type, const void* gate_bank, const void* up_bank,
+                     const void* down_bank, int router_type, const void* router, const float* x, int rows, int k_used,
+                     int n_expert, int n_ffn, int n_embd, uint32_t* sel, float* wt, void* stream) {
+    if (!c) return JL_ERR_ARG;
+    if (!gate_bank || !up_bank || !down_bank) return fail(c, JL_ERR_ARG, "moe block: null bank");
+    return moe_block(c, resid, type, down_type, gate_bank, up_bank, down_bank, nullptr, nullptr, nullptr, router_type, router,
+                     x, rows, k_used, n_expert, n_ffn, n_embd, sel, wt, stream);
+}
+
+int jl_moe_block_packed_dev(jl_ctx* c, float* resid, int type, const jl_packed_bank* gate, const jl_packed_bank* up,
+                            const jl_packed_bank* down, int router_type, const void* router, const float* x, int rows,
+                            int k_used, int n_expert, int n_ffn, int n_embd, uint32_t* sel, float* wt, void* stream) {
+    if (!c) return JL_ERR_ARG;
+    if (!gate || !up || !down) return fail(c, JL_ERR_ARG, "moe block: null bank");
+    return moe_block(c, resid, type, type, nullptr, nullptr, nullptr, gate, up, down, router_type, router, x, rows, k_used,
+                     n_expert, n_ffn, n_embd, sel, wt, stream);
+}
 
 int jl_moe_ffn_types_dev(jl_ctx* c, float* resid, int type, int down_type, const void* gate_bank, const void* up_bank,
                          const void* down_bank, const float* x, const uint32_t* sel, int sel_stride,
@@ -2110,19 +2179,8 @@ int jl_layer_ffn_dev(jl_ctx* c, int li, const float* h, float* resid, int n, voi
         bd = jl_packed_bank{L.dp[0], L.dp[1], L.dp[2], 0, sheets * E};
     }
     if (P.kind == JL_LAYER_MOE) {
-        const size_t o_sel = up256((size_t)n * P.n_expert * 4), o_wt = o_sel + up256((size_t)n * (P.k_used + 1) * 4);
-        int rc = grow(c, &c->layer_ws, &c->layer_ws_bytes, o_wt + up256((size_t)n * P.k_used * 4));
-        if (rc != JL_OK) return rc;
-        float* logits = (float*)c->layer_ws;
-        uint32_t* sel = (uint32_t*)((char*)c->layer_ws + o_sel);
-        float* wt = (float*)((char*)c->layer_ws + o_wt);
-        rc = jl_moe_logits_dev(c, logits, JL_TYPE_F32, L.router, h, P.n_expert, E, n, st);
-        if (rc != JL_OK) return rc;
-        rc = jl_moe_route_dev(c, logits, n, P.n_expert, P.k_used, sel, P.k_used + 1, wt, st);
-        if (rc != JL_OK) return rc;
-        return moe_ffn(c, resid, P.type, P.down_type, L.gate, L.up, L.down, P.packed ? &bg : nullptr,
-                       P.packed ? &bu : nullptr, P.packed ? &bd : nullptr, h, sel, P.k_used + 1, wt, n, P.k_used,
-                       P.n_expert, F, E, st);
+        return moe_block(c, resid, P.type, P.down_type, L.gate, L.up, L.down, P.packed ? &bg : nullptr, P.packed ? &bu : nullptr,
+                         P.packed ? &bd : nullptr, JL_TYPE_F32, L.router, h, n, P.k_used, P.n_expert, F, E, nullptr, nullptr, st);
     }
     // dense.  More than one row without a norm in front: the grouped kernels, the block as a
     // mixture of one expert that every row selects with weight 1.

@@ -369,6 +369,19 @@ class Device:
                                                          stream),
                             "jl_moe_ffn_types_dev")
 
+    def moe_block_dev(self, resid, t, gate, up, down, router, x, rows, k_used, n_expert, n_ffn, n_embd, sel=None,
+                      wt=None, stream=None, down_type=None, router_type=0):
+        """The whole mixture block, router included: resid [rows][n_embd] += mixture output.  gate / up /
+        down: banks of GGUF sheets (device addresses), or three packed_bank(...) structures."""
+        if isinstance(gate, _lib.PackedBank):
+            return self._served(self._l.jl_moe_block_packed_dev(
+                self._ctx, _ptr(resid), t, C.byref(gate), C.byref(up), C.byref(down), router_type, _ptr(router), _ptr(x),
+                rows, k_used, n_expert, n_ffn, n_embd, _opt(sel), _opt(wt), stream), "jl_moe_block_packed_dev")
+        return self._served(self._l.jl_moe_block_dev(
+            self._ctx, _ptr(resid), t, t if down_type is None else down_type, _ptr(gate), _ptr(up), _ptr(down),
+            router_type, _ptr(router), _ptr(x), rows, k_used, n_expert, n_ffn, n_embd, _opt(sel), _opt(wt), stream),
+            "jl_moe_block_dev")
+
     def matmul_mxfp4_bf16_dev(self, out, w, x, nrows, k, ntok, stream=None):
         """MXFP4 weights x bf16 activations (bits as uint16) -> f32 out [ntok][nrows]."""
         return self._served(self._l.jl_matmul_mxfp4_bf16_dev(self._ctx, _ptr(out), _ptr(w), _ptr(x),

@@ -613,3 +613,61 @@ def test_moe_block_over_packed_banks_vs_oracle(dev, devbuf, shape, layout):
         got = resid.get()
         assert rel_l2(got, want) <= 1e-3, f"call {call}: rel-L2 {rel_l2(got, want):.3e}"
     dev.SetActWindow(32)
+
+
+@pytest.mark.parametrize("layout", ["rows", "planes"])
+@pytest.mark.parametrize("rows", [64, 5])
+def test_block_in_one_call_is_router_then_ffn_bit_for_bit(dev, devbuf, layout, rows):
+    """jl_moe_block_dev: the logits, router and feed-forward calls in one, bit for bit."""
+    t, n_expert, k_used, n_ffn, n_embd = quant.Q4_K, 32, 4, 512, 1024
+    dev.SetActWindow(256)
+    gate, up = _banks(t, n_expert, n_ffn, n_embd, 1000, False), _banks(t, n_expert, n_ffn, n_embd, 2000, False)
+    down = _banks(t, n_expert, n_embd, n_ffn, 3000, False)
+    rng = np.random.default_rng(rows)
+    router = (rng.standard_normal((n_expert, n_embd)) / np.sqrt(n_embd)).astype(np.float32)
+    x = rng.standard_normal((rows, n_embd)).astype(np.float32)
+    resid0 = rng.standard_normal((rows, n_embd)).astype(np.float32)
+    xd, rd = devbuf(x), devbuf(router)
+    if layout == "planes":
+        keep = [_pack_bank(dev, devbuf, t, b, n_expert, r, k, "one")
+                for b, r, k in ((gate, n_ffn, n_embd), (up, n_ffn, n_embd), (down, n_embd, n_ffn))]
+        banks = [kb[0] for kb in keep]
+    else:
+        keep = [devbuf(gate), devbuf(up), devbuf(down)]
+        banks = [b.ptr for b in keep]
+    ld = devbuf(shape=(rows, n_expert), dtype=np.float32, fill=0)
+    sel = devbuf(shape=(rows, k_used + 1), dtype=np.uint32, fill=0)
+    wt = devbuf(shape=(rows, k_used), dtype=np.float32, fill=0)
+    want = devbuf(resid0)
+    try:
+        separate = dev.launch_count()
+        assert dev.moe_logits_dev(ld.ptr, 0, rd.ptr, xd.ptr, n_expert, n_embd, rows)
+        assert dev.moe_route_dev(ld.ptr, rows, n_expert, k_used, sel.ptr, k_used + 1, wt.ptr)
+        if layout == "planes":
+            assert dev.moe_ffn_packed_dev(want.ptr, t, banks[0], banks[1], banks[2], xd.ptr, sel.ptr, k_used + 1, wt.ptr,
+                                          rows, k_used, n_expert, n_ffn, n_embd)
+        else:
+            assert dev.moe_ffn_dev(want.ptr, t, banks[0], banks[1], banks[2], xd.ptr, sel.ptr, k_used + 1, wt.ptr, rows,
+                                   k_used, n_expert, n_ffn, n_embd)
+        separate = dev.launch_count() - separate
+        dev.synchronize()
+        for i in range(2):
+            got = devbuf(resid0)
+            sel2 = devbuf(shape=(rows, k_used + 1), dtype=np.uint32, fill=0)
+            wt2 = devbuf(shape=(rows, k_used), dtype=np.float32, fill=0)
+            before = dev.launch_count()
+            assert dev.moe_block_dev(got.ptr, t, banks[0], banks[1], banks[2], rd.ptr, xd.ptr, rows, k_used, n_expert,
+                                     n_ffn, n_embd, sel=sel2.ptr, wt=wt2.ptr)
+            assert dev.launch_count() == before + separate
+            dev.synchronize()
+            assert np.array_equal(sel2.get()[:, :k_used], sel.get()[:, :k_used])
+            assert np.array_equal(wt2.get().view(np.uint32), wt.get().view(np.uint32))
+            assert np.array_equal(got.get().view(np.uint32), want.get().view(np.uint32))
+        # the routing kept in the context's own workspace
+        got = devbuf(resid0)
+        assert dev.moe_block_dev(got.ptr, t, banks[0], banks[1], banks[2], rd.ptr, xd.ptr, rows, k_used, n_expert,
+                                 n_ffn, n_embd)
+        dev.synchronize()
+        assert np.array_equal(got.get().view(np.uint32), want.get().view(np.uint32))
+    finally:
+        dev.SetActWindow(32)
