@@ -63,6 +63,16 @@ extern "C" __global__ __launch_bounds__(256) void jl_dequant(
     extern "C" __global__ __launch_bounds__(MAXT) void jl_matvec_##T##_r##RPW##_x4(MatVecArgs p) { \
         matvec_body<TYPE, RPW, 4>(p, jl_smem);                                               \
     }
+// _res: one row a wavefront with resid[r] += weight * out[r] riding on the store (MatVecArgs.resid set)
+#define JL_MATVEC_RES_KERNEL(T, TYPE)                                                               \
+    extern "C" __global__ __launch_bounds__(1024) void jl_matvec_##T##_r1_res(MatVecArgs p) {       \
+        matvec_body<TYPE, 1, 1, true>(p, jl_smem);                                                  \
+    }                                                                                               \
+    extern "C" __global__ __launch_bounds__(1024) void jl_matvec_##T##_r1_x4_res(MatVecArgs p) {    \
+        matvec_body<TYPE, 1, 4, true>(p, jl_smem);                                                  \
+    }
+JL_MATVEC_RES_KERNEL(q4k, JL_Q4_K) JL_MATVEC_RES_KERNEL(q8_0, JL_Q8_0) JL_MATVEC_RES_KERNEL(q6k, JL_Q6_KS)
+JL_MATVEC_RES_KERNEL(q8_0p, JL_Q8_0P)
 JL_MATVEC_KERNEL(q4k, JL_Q4_K, 1, 1024) JL_MATVEC_KERNEL(q4k, JL_Q4_K, 2, 1024) JL_MATVEC_KERNEL(q4k, JL_Q4_K, 4, 512)
 JL_MATVEC_KERNEL(q8_0, JL_Q8_0, 1, 1024) JL_MATVEC_KERNEL(q8_0, JL_Q8_0, 2, 1024) JL_MATVEC_KERNEL(q8_0, JL_Q8_0, 4, 1024)
 // (Q6_K over the staging layout made for it: JL_STAGE_Q6K in kernels/matvec.h)
@@ -72,16 +82,18 @@ JL_MATVEC_KERNEL(q6k, JL_Q6_KS, 1, 1024) JL_MATVEC_KERNEL(q6k, JL_Q6_KS, 2, 512)
 JL_MATVEC_KERNEL(q8_0p, JL_Q8_0P, 1, 1024) JL_MATVEC_KERNEL(q8_0p, JL_Q8_0P, 2, 1024) JL_MATVEC_KERNEL(q8_0p, JL_Q8_0P, 4, 512)
 
 // grid = (row groups, matrices), block = 64..1024
-#define JL_MATVEC_MULTI_KERNEL(T, TYPE)                                                                \
-    extern "C" __global__ __launch_bounds__(1024) void jl_matvec_multi_##T(MatVecMultiArgs p) {        \
-        matvec_multi_body<TYPE, 1>(p, jl_smem, p.row_bytes);                                           \
-    }                                                                                                  \
-    extern "C" __global__ __launch_bounds__(1024) void jl_matvec_multi_##T##_x4(MatVecMultiArgs p) {   \
-        matvec_multi_body<TYPE, 4>(p, jl_smem, p.row_bytes);                                           \
-    }                                                                                                  \
-    extern "C" __global__ __launch_bounds__(1024) void jl_matvec_multi_##T##_q(MatVecMultiArgs p) {    \
-        matvec_multi_body<TYPE, 0>(p, jl_smem, p.row_bytes);                                           \
+#define JL_MATVEC_MULTI_FORMS(T, TYPE, SUF, RES)                                                               \
+    extern "C" __global__ __launch_bounds__(1024) void jl_matvec_multi_##T##SUF(MatVecMultiArgs p) {           \
+        matvec_multi_body<TYPE, 1, RES>(p, jl_smem, p.row_bytes);                                              \
+    }                                                                                                          \
+    extern "C" __global__ __launch_bounds__(1024) void jl_matvec_multi_##T##_x4##SUF(MatVecMultiArgs p) {      \
+        matvec_multi_body<TYPE, 4, RES>(p, jl_smem, p.row_bytes);                                              \
+    }                                                                                                          \
+    extern "C" __global__ __launch_bounds__(1024) void jl_matvec_multi_##T##_q##SUF(MatVecMultiArgs p) {       \
+        matvec_multi_body<TYPE, 0, RES>(p, jl_smem, p.row_bytes);                                              \
     }
+// (_res: MatVecMultiArgs.resid set)
+#define JL_MATVEC_MULTI_KERNEL(T, TYPE) JL_MATVEC_MULTI_FORMS(T, TYPE, , false) JL_MATVEC_MULTI_FORMS(T, TYPE, _res, true)
 JL_MATVEC_MULTI_KERNEL(q4k, JL_Q4_K) JL_MATVEC_MULTI_KERNEL(q8_0, JL_Q8_0) JL_MATVEC_MULTI_KERNEL(q6k, JL_Q6_KS)
 JL_MATVEC_MULTI_KERNEL(q8_0p, JL_Q8_0P)
 // The same grid over matrices of different types (the reference's MatVecSegments,

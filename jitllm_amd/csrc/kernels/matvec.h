@@ -633,7 +633,10 @@ __device__ __forceinline__ float resid_weight(float alpha, const float* gate) {
 // activation is staged, so HBM latency overlaps the quantizer; after that each
 // group is load -> dot -> cross-lane reduce, and the wavefronts of a CU (two
 // workgroups of eight, or one of sixteen) cover each other's memory latency.
-template <int TYPE, int RPW, int XP>
+// RES: the residual add rides on the store (entry points of their own: with the add and its
+// gate's f64 exponential compiled into the plain kernel behind a branch, the plain matvecs ran
+// 10-20 % slower, Q8_0 14336 x 4096 14.2 against 11.8 us).
+template <int TYPE, int RPW, int XP, bool RES>
 __device__ __forceinline__ void matvec_body_xp(const MatVecArgs& p, uint8_t* smem) {
     typedef SlotTraits<TYPE> T;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = p.nwaves;
@@ -668,18 +671,23 @@ __device__ __forceinline__ void matvec_body_xp(const MatVecArgs& p, uint8_t* sme
     else stage_act_copy<SH>(smem, p.q, p.as, p.s16, p.k, nwaves * 64);
     lds_barrier();   // orders the LDS staging only: the weight loads stay in flight
 
-    float* const resid = p.resid;
-    matvec_rows<TYPE, RPW>(p.w, p.row_bytes, A, p.nrows, r0, group_stride, nslots, lane, w, [&](int r, float t) {
-        p.out[r] = t;
-        if (resid) resid[r] += resid_weight(p.alpha, p.resid_gate) * t;
-    }, p.pipe != 2);
+    if constexpr (RES) {
+        float* const resid = p.resid;
+        matvec_rows<TYPE, RPW>(p.w, p.row_bytes, A, p.nrows, r0, group_stride, nslots, lane, w, [&](int r, float t) {
+            p.out[r] = t;
+            resid[r] += resid_weight(p.alpha, p.resid_gate) * t;
+        }, p.pipe != 2);
+    } else {
+        matvec_rows<TYPE, RPW>(p.w, p.row_bytes, A, p.nrows, r0, group_stride, nslots, lane, w,
+                               [&](int r, float t) { p.out[r] = t; }, p.pipe != 2);
+    }
 }
 
 // XP = 1: a vector of at most one float4 group a thread; 4: longer ones (the host picks the
 // entry point; one body compiled for both behind a branch ran the short-vector case 10 % slower).
-template <int TYPE, int RPW, int XP = 1>
+template <int TYPE, int RPW, int XP = 1, bool RES = false>
 __device__ __forceinline__ void matvec_body(const MatVecArgs& p, uint8_t* smem) {
-    matvec_body_xp<TYPE, RPW, XP>(p, smem);
+    matvec_body_xp<TYPE, RPW, XP, RES>(p, smem);
 }
 
 // Several matvecs of one type in one launch: grid = (row groups, matrices).  Each
@@ -700,7 +708,9 @@ __device__ __forceinline__ double wave_sum_f64(double v) {
 // a long gated activation is formed and quantized once by the quantizer kernel instead of by
 // every workgroup (silu and its division for 14336 elements in each of 256 workgroups cost the
 // down projection of a feed-forward block 6 of its 20 us).
-template <int TYPE, int XP>
+// RES: matrix 0's rows are added into the residual as they are made (entry points of their own,
+// like the single-matrix kernel's).
+template <int TYPE, int XP, bool RES>
 __device__ __forceinline__ void matvec_multi_body_xp(const MatVecMultiArgs& p, uint8_t* smem, int row_bytes) {
     typedef SlotTraits<TYPE> T;
     const int y = blockIdx.y;
@@ -719,11 +729,16 @@ __device__ __forceinline__ void matvec_multi_body_xp(const MatVecMultiArgs& p, u
         stage_act_copy<stage_layout_of(TYPE)>(smem, p.q, p.as, p.s16, p.k, nthreads);
         lds_barrier();
         float* const outp = p.out[y];
-        float* const resid = y == 0 ? p.resid : nullptr;
-        matvec_rows<TYPE, 1>(w0, row_bytes, A, nrows, r0, group_stride, nslots, lane, w, [&](int r, float t) {
-            outp[r] = t;
-            if (resid) resid[r] += resid_weight(p.alpha, p.resid_gate) * t;
-        }, false);
+        if constexpr (RES) {
+            float* const resid = y == 0 ? p.resid : nullptr;
+            matvec_rows<TYPE, 1>(w0, row_bytes, A, nrows, r0, group_stride, nslots, lane, w, [&](int r, float t) {
+                outp[r] = t;
+                if (resid) resid[r] += resid_weight(p.alpha, p.resid_gate) * t;
+            }, false);
+        } else {
+            matvec_rows<TYPE, 1>(w0, row_bytes, A, nrows, r0, group_stride, nslots, lane, w,
+                                 [&](int r, float t) { outp[r] = t; }, false);
+        }
         return;
     } else {
     const float* x = p.x + (size_t)y * p.xstride;
@@ -799,17 +814,22 @@ __device__ __forceinline__ void matvec_multi_body_xp(const MatVecMultiArgs& p, u
     lds_barrier();
 
     float* const outp = p.out[y];
-    float* const resid = y == 0 ? p.resid : nullptr;
     // (a second step of weights requested ahead of the staging, for the launches with an RMSNorm or
     // a gated activation in front, measured slower: gate + up 26.2 -> 32.8 us, down 14.5 -> 16.9)
-    matvec_rows<TYPE, 1>(w0, row_bytes, A, nrows, r0, group_stride, nslots, lane, w, [&](int r, float t) {
-        outp[r] = t;
-        if (resid) resid[r] += resid_weight(p.alpha, p.resid_gate) * t;
-    }, false);
+    if constexpr (RES) {
+        float* const resid = y == 0 ? p.resid : nullptr;
+        matvec_rows<TYPE, 1>(w0, row_bytes, A, nrows, r0, group_stride, nslots, lane, w, [&](int r, float t) {
+            outp[r] = t;
+            if (resid) resid[r] += resid_weight(p.alpha, p.resid_gate) * t;
+        }, false);
+    } else {
+        matvec_rows<TYPE, 1>(w0, row_bytes, A, nrows, r0, group_stride, nslots, lane, w,
+                             [&](int r, float t) { outp[r] = t; }, false);
+    }
     }
 }
 
-template <int TYPE, int XP = 1>
+template <int TYPE, int XP = 1, bool RES = true>
 __device__ __forceinline__ void matvec_multi_body(const MatVecMultiArgs& p, uint8_t* smem, int row_bytes) {
-    matvec_multi_body_xp<TYPE, XP>(p, smem, row_bytes);
+    matvec_multi_body_xp<TYPE, XP, RES>(p, smem, row_bytes);
 }
