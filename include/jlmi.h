@@ -88,7 +88,7 @@ int jl_synchronize(jl_ctx *ctx);
 
 /* Kernel-shape overrides for measurement and the parity tests: key is one of "matvec.rpw"
  * (rows per wavefront: 1, 2, 4), "matvec.block" (threads per workgroup), "matvec.grid"
- * (workgroups), "matvec.pipe" (1: the row loop as a two-deep load pipeline), "matvec.q8pair" (2: Q8_0
+ * (workgroups), "matvec.q8pair" (2: Q8_0
  * rows one block a lane-slot even where the two-block form with 4-byte-aligned loads applies),
  * "matvec.xpre" (1 / 4: float4 groups of the activation a thread loads ahead of its weights),
  * "matvec.act_split" (1: a group's gated activation is formed and quantized once, by a launch of

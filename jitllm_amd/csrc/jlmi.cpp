@@ -31,7 +31,7 @@ thread_local std::string g_create_error;
 const HipApi* H = nullptr;  // the process-wide HIP runtime, resolved by the first jl_ctx_create
 
 struct Tuning {
-    int rpw = 0, block = 0, grid = 0, pipe = 0;
+    int rpw = 0, block = 0, grid = 0;
     int act_split = 0;          // grouped matvec with a gated activation: 1 always quantize it in its own launch, 2 never
     int xpre = 0;               // decode matvec: 1 / 4 float4 groups of x a thread loads ahead of its weights
     int q8pair = 0;             // Q8_0 rows: 2 keeps one block a lane-slot (2-byte-aligned loads)
@@ -348,10 +348,6 @@ int matvec_launch(jl_ctx* c, float* out, int type, const void* w, const float* x
     a.per = c->act_window / 32;
     a.nwaves = block / 64;
     a.ngroups = (int)grid;
-    // the two-deep pipeline of the row loop ("matvec.pipe" = 1) measured slower than the plain
-    // loop on this machine (Q8_0 14336 x 4096: 17.4 against 15.7 us; Q6_K 4096 x 14336: 15.1
-    // against 14.2), so it stays off unless asked for
-    a.pipe = c->tune.pipe == 1 ? 1 : 2;
     a.resid = resid; a.alpha = alpha; a.resid_gate = resid ? resid_gate : nullptr;
     const int xpre = c->tune.xpre == 1 || c->tune.xpre == 4 ? c->tune.xpre : (k / 4 > 2 * block ? 4 : 1);   // three groups a thread and more
     char name[64];
@@ -1525,7 +1521,6 @@ int jl_set_tuning(jl_ctx* c, const char* key, int value) {
     if (!strcmp(key, "matvec.rpw")) c->tune.rpw = value;
     else if (!strcmp(key, "matvec.block")) c->tune.block = value;
     else if (!strcmp(key, "matvec.grid")) c->tune.grid = value;
-    else if (!strcmp(key, "matvec.pipe")) c->tune.pipe = value;
     else if (!strcmp(key, "packed.rw")) c->tune.packed_rw = value;
     else if (!strcmp(key, "packed.block")) c->tune.packed_block = value;
     else if (!strcmp(key, "moe.group")) c->tune.moe_group = value;

@@ -16,7 +16,6 @@ struct MatVecArgs {
     int per;             // activation window / 32 (fused form)
     int nwaves;          // wavefronts per workgroup (the launch's block / 64)
     int ngroups;         // workgroups (the launch's grid)
-    int pipe;            // 2: the plain row loop; else the two-deep pipeline where a wavefront has several steps
     float* resid;        // optional: resid[r] += alpha * out[r] (times sigmoid(*resid_gate) when resid_gate is set)
     const float* resid_gate;
     float alpha;

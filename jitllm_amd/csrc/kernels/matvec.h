@@ -534,89 +534,42 @@ template <> struct SlotTraits<JL_Q6_K> {
 
 // The row loop of one wavefront: rows r0, r0 + group_stride, ... (RPW at a time), each row's
 // slots dealt to the lanes in chunks of 64.  w holds the first step's weights, loaded by the
-// caller before the activation was staged.  Two forms: the plain loop (each step's loads are
-// issued when the step begins; the dozen or so wavefronts of a CU cover each other's
-// latency), and a two-deep pipeline (`pipe`: the next step's weight loads are issued BEFORE
-// the current step's dot products, into the other of two register sets; unconditional loads
-// with clamped addresses, so the compiler's wait counts stay exact).  On MI355X the plain
-// loop measured faster for every type but Q4_K, where they tie: more loads in flight per
-// wavefront do not help a kernel that is not waiting on latency.
+// caller before the activation was staged; every later step's loads are issued when the step
+// begins, and the dozen or so wavefronts of a CU cover each other's latency.  (A two-deep
+// pipeline -- the next step's weight loads issued BEFORE the current step's dot products, into
+// a second register set -- measured slower for every type but Q4_K, where they tie: more loads
+// in flight per wavefront do not help a kernel that is not waiting on latency.  Kept behind a
+// run-time switch it also cost the plain loop, so it is gone.)
 // store(row, total) receives a finished row in lane 63.
 template <int TYPE, int RPW, class Store>
 __device__ __forceinline__ void matvec_rows(const uint8_t* w0, int row_bytes, const ActLds& A, int nrows, int r0,
                                             int group_stride, int nslots, int lane,
-                                            typename SlotTraits<TYPE>::W (&w)[RPW], Store store, bool pipe) {
+                                            typename SlotTraits<TYPE>::W (&w)[RPW], Store store) {
     typedef SlotTraits<TYPE> T;
-    if (r0 >= nrows) return;   // wavefront-uniform
-    const int nper = (nslots + 63) >> 6;                             // steps per row group
-    const int ngrp = (nrows - r0 + group_stride - 1) / group_stride;   // row groups of this wavefront
     float acc[RPW];
 #pragma unroll
     for (int j = 0; j < RPW; j++) acc[j] = 0.f;
-    if (ngrp * nper == 1 || !pipe) {
-        // a single step (a matrix that fits the grid, every row one chunk): nothing to overlap;
-        // or the plain loop, each step's loads issued when the step begins
-        bool preloaded = true;
-        for (; r0 < nrows; r0 += group_stride) {
-            for (int slot = lane; slot < nslots; slot += 64) {
-                if (!preloaded) {
+    bool preloaded = true;
+    for (; r0 < nrows; r0 += group_stride) {
+        for (int slot = lane; slot < nslots; slot += 64) {
+            if (!preloaded) {
 #pragma unroll
-                    for (int j = 0; j < RPW; j++)
-                        T::load_w(w0 + (size_t)min(r0 + j, nrows - 1) * row_bytes, slot, w[j]);
-                }
-                preloaded = false;
-                typename T::Act a;
-                T::load_act(A, slot, a);
-#pragma unroll
-                for (int j = 0; j < RPW; j++) acc[j] += T::dot(w[j], slot, a);
+                for (int j = 0; j < RPW; j++)
+                    T::load_w(w0 + (size_t)min(r0 + j, nrows - 1) * row_bytes, slot, w[j]);
             }
             preloaded = false;
+            typename T::Act a;
+            T::load_act(A, slot, a);
 #pragma unroll
-            for (int j = 0; j < RPW; j++) {
-                const float t = wave_sum_to_lane63(acc[j]);
-                if (lane == 63 && r0 + j < nrows) store(r0 + j, t);
-                acc[j] = 0.f;
-            }
+            for (int j = 0; j < RPW; j++) acc[j] += T::dot(w[j], slot, a);
         }
-        return;
-    }
-    typename T::W wb[RPW];
-    int g = 0, sidx = 0;   // the current step: row group g of this wavefront, chunk sidx of its slots
-    auto step = [&](typename T::W (&wc)[RPW], typename T::W (&wn)[RPW]) __attribute__((always_inline)) {
-        int gn = g, sn = sidx + 1;
-        if (sn == nper) { sn = 0; gn++; }
-        {
-            const int rn = r0 + min(gn, ngrp - 1) * group_stride;
-            const int slot_n = min(lane + 64 * sn, nslots - 1);
-#pragma unroll
-            for (int j = 0; j < RPW; j++) T::load_w(w0 + (size_t)min(rn + j, nrows - 1) * row_bytes, slot_n, wn[j]);
-        }
-        const int slot = lane + 64 * sidx;
-        const bool live = slot < nslots;
-        const int sl = min(slot, nslots - 1);
-        typename T::Act a;
-        T::load_act(A, sl, a);
+        preloaded = false;
 #pragma unroll
         for (int j = 0; j < RPW; j++) {
-            const float v = T::dot(wc[j], sl, a);
-            acc[j] += live ? v : 0.f;
+            const float t = wave_sum_to_lane63(acc[j]);
+            if (lane == 63 && r0 + j < nrows) store(r0 + j, t);
+            acc[j] = 0.f;
         }
-        if (sn == 0) {   // the row group's last chunk
-            const int r = r0 + g * group_stride;
-#pragma unroll
-            for (int j = 0; j < RPW; j++) {
-                const float t = wave_sum_to_lane63(acc[j]);
-                if (lane == 63 && r + j < nrows) store(r + j, t);
-                acc[j] = 0.f;
-            }
-        }
-        g = gn;
-        sidx = sn;
-    };
-    const int nsteps = ngrp * nper;
-    for (int i = 0; i < nsteps; i += 2) {
-        step(w, wb);
-        if (i + 1 < nsteps) step(wb, w);
     }
 }
 
@@ -676,10 +629,10 @@ __device__ __forceinline__ void matvec_body_xp(const MatVecArgs& p, uint8_t* sme
         matvec_rows<TYPE, RPW>(p.w, p.row_bytes, A, p.nrows, r0, group_stride, nslots, lane, w, [&](int r, float t) {
             p.out[r] = t;
             resid[r] += resid_weight(p.alpha, p.resid_gate) * t;
-        }, p.pipe != 2);
+        });
     } else {
         matvec_rows<TYPE, RPW>(p.w, p.row_bytes, A, p.nrows, r0, group_stride, nslots, lane, w,
-                               [&](int r, float t) { p.out[r] = t; }, p.pipe != 2);
+                               [&](int r, float t) { p.out[r] = t; });
     }
 }
 
@@ -734,10 +687,10 @@ __device__ __forceinline__ void matvec_multi_body_xp(const MatVecMultiArgs& p, u
             matvec_rows<TYPE, 1>(w0, row_bytes, A, nrows, r0, group_stride, nslots, lane, w, [&](int r, float t) {
                 outp[r] = t;
                 if (resid) resid[r] += resid_weight(p.alpha, p.resid_gate) * t;
-            }, false);
+            });
         } else {
             matvec_rows<TYPE, 1>(w0, row_bytes, A, nrows, r0, group_stride, nslots, lane, w,
-                                 [&](int r, float t) { outp[r] = t; }, false);
+                                 [&](int r, float t) { outp[r] = t; });
         }
         return;
     } else {
@@ -821,10 +774,10 @@ __device__ __forceinline__ void matvec_multi_body_xp(const MatVecMultiArgs& p, u
         matvec_rows<TYPE, 1>(w0, row_bytes, A, nrows, r0, group_stride, nslots, lane, w, [&](int r, float t) {
             outp[r] = t;
             if (resid) resid[r] += resid_weight(p.alpha, p.resid_gate) * t;
-        }, false);
+        });
     } else {
         matvec_rows<TYPE, 1>(w0, row_bytes, A, nrows, r0, group_stride, nslots, lane, w,
-                             [&](int r, float t) { outp[r] = t; }, false);
+                             [&](int r, float t) { outp[r] = t; });
     }
     }
 }

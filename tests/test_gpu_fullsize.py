@@ -91,8 +91,8 @@ def test_decode_matvec_full_size_rows_and_planes(dev, devbuf, case):
 @pytest.mark.parametrize("t", [quant.Q4_K, quant.Q8_0, quant.Q6_K])
 def test_matvec_persistent_grid_shapes(dev, devbuf, t):
     """More rows than sixteen a CU (so the default is the persistent grid) and the 768-thread
-    workgroup forced beside the others, the row loop plain and as a two-deep load pipeline
-    (odd and even step counts, several chunks a row), on a matrix short enough in K to be cheap."""
+    workgroup forced beside the others (odd and even step counts, several chunks a row), on a
+    matrix short enough in K to be cheap."""
     window = 32
     dev.SetActWindow(window)
     nrows, k = 16 * 256 + 200, 2176 if t == quant.Q8_0 else 4352    # 68 slots a row: two chunks, the second ragged
@@ -100,17 +100,17 @@ def test_matvec_persistent_grid_shapes(dev, devbuf, t):
     x = synth.activations(k, seed=4)
     want = _like_for_like(t, w, x, nrows, k, window)
     wd, xd = devbuf(w), devbuf(x)
-    for rpw, block, grid, pipe in [(0, 0, 0, 0), (1, 768, 0, 0), (2, 768, 0, 0), (1, 768, 7, 0), (1, 768, 512, 0),
-                                   (4, 512, 0, 0), (0, 0, 0, 1), (2, 768, 7, 1), (1, 1024, 3, 1), (4, 512, 0, 1)]:
-        dev.set_tuning(rpw=rpw, block=block, grid=grid, pipe=pipe)
+    for rpw, block, grid in [(0, 0, 0), (1, 768, 0), (2, 768, 0), (1, 768, 7), (1, 768, 512), (4, 512, 0),
+                             (2, 768, 7), (1, 1024, 3)]:
+        dev.set_tuning(rpw=rpw, block=block, grid=grid)
         out = devbuf(shape=(nrows + 8,), dtype=np.float32, fill=POISON)
         assert dev.matvec_dev(out.ptr, t, wd.ptr, xd.ptr, nrows, k)
         dev.synchronize()
         got = out.get()
         assert np.all(got[nrows:] == POISON)
-        _check_rows(got[:nrows], want, f"rpw={rpw} block={block} grid={grid} pipe={pipe}")
+        _check_rows(got[:nrows], want, f"rpw={rpw} block={block} grid={grid}")
         out.free()
-    dev.set_tuning(rpw=0, block=0, grid=0, pipe=0)
+    dev.set_tuning(rpw=0, block=0, grid=0)
 
 
 def _sample_rows(nrows, rng, boundaries):
