@@ -320,7 +320,7 @@ int matvec_launch(jl_ctx* c, float* out, int type, const void* w, const float* x
     // quantizes x once), larger ones a persistent grid of two 12-wavefront
     // workgroups per CU that stride over the row groups.
     int rpw = c->tune.rpw, block = c->tune.block;
-    if (rpw <= 0 || resid) rpw = 1;   // (the kernels with the residual add: one row a wavefront)
+    if (rpw <= 0 || resid || !x) rpw = 1;   // (the kernels with the residual add or a quantized activation: one row a wavefront)
     if (rpw != 1 && rpw != 2 && rpw != 4) return fail(c, JL_ERR_ARG, "matvec: rpw=%d", rpw);
     const bool small = nrows <= 16 * c->num_cu;
     // (Q4_K 14336 x 4096: one 16-wavefront workgroup a CU 8.1 us, two of twelve 8.6)
@@ -351,7 +351,7 @@ int matvec_launch(jl_ctx* c, float* out, int type, const void* w, const float* x
     a.resid = resid; a.alpha = alpha; a.resid_gate = resid ? resid_gate : nullptr;
     const int xpre = c->tune.xpre == 1 || c->tune.xpre == 4 ? c->tune.xpre : (k / 4 > 2 * block ? 4 : 1);   // three groups a thread and more
     char name[64];
-    snprintf(name, sizeof name, "jl_matvec_%s_r%d%s%s", pair ? "q8_0p" : ti->tag, rpw, xpre == 4 ? "_x4" : "",
+    snprintf(name, sizeof name, "jl_matvec_%s_r%d%s%s", pair ? "q8_0p" : ti->tag, rpw, !x ? "_pq" : xpre == 4 ? "_x4" : "",
              resid ? "_res" : "");
     void* params[] = {&a};
     unsigned lds = (unsigned)(act_lds_bytes(k) + (pair ? (size_t)k + 16 : 0));
@@ -1414,7 +1414,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     if (e != hipSuccess)
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
-    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_matvec_multi_q4k_res", "jl_matvec_multi_q4k_x4_res", "jl_matvec_multi_q4k_q_res", "jl_matvec_multi_q8_0_res", "jl_matvec_multi_q8_0_x4_res", "jl_matvec_multi_q8_0_q_res", "jl_matvec_multi_q6k_res", "jl_matvec_multi_q6k_x4_res", "jl_matvec_multi_q6k_q_res", "jl_matvec_multi_q8_0p_res", "jl_matvec_multi_q8_0p_x4_res", "jl_matvec_multi_q8_0p_q_res", "jl_matvec_q4k_r1_res", "jl_matvec_q4k_r1_x4_res", "jl_matvec_q8_0_r1_res", "jl_matvec_q8_0_r1_x4_res", "jl_matvec_q6k_r1_res", "jl_matvec_q6k_r1_x4_res", "jl_matvec_q8_0p_r1_res", "jl_matvec_q8_0p_r1_x4_res", "jl_matvec_q8_0p_r1", "jl_matvec_q8_0p_r2", "jl_matvec_q8_0p_r4", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_q4k_k2", "jl_gemm_q4k_k2_planes", "jl_gemm_prep_q4k_planes", "jl_gemm_q4k_r64_planes", "jl_gemm_q4k_wide_planes", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_group2_wide", "jl_moe_quant", "jl_moe_matvec_planes_q4k", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_prep_planes", "jl_moe_gemm_q4k", "jl_moe_g16_prep", "jl_moe_g16_prep_planes", "jl_moe_g16_prep_q6k", "jl_moe_g16_c1", "jl_moe_g16_c2", "jl_moe_g16_c3", "jl_moe_g16_f1", "jl_moe_g16_f2", "jl_moe_g16_f3", "jl_moe_g16_g1", "jl_moe_g16_g2", "jl_moe_g16_g3", "jl_moe_g16_d1", "jl_moe_g16_d2", "jl_moe_g16_d3", "jl_moe_g16p_c1", "jl_moe_g16p_c2", "jl_moe_g16p_c3", "jl_moe_g16p_f1", "jl_moe_g16p_f2", "jl_moe_g16p_f3", "jl_moe_g16p_g1", "jl_moe_g16p_g2", "jl_moe_g16p_g3", "jl_moe_g16p_d1", "jl_moe_g16p_d2", "jl_moe_g16p_d3", "jl_moe_g16q6_c1", "jl_moe_g16q6_c2", "jl_moe_g16q6_c3", "jl_moe_g16q6_f1", "jl_moe_g16q6_f2", "jl_moe_g16q6_f3", "jl_moe_g16q6_g1", "jl_moe_g16q6_g2", "jl_moe_g16q6_g3", "jl_moe_g16q6_d1", "jl_moe_g16q6_d2", "jl_moe_g16q6_d3", "jl_moe_gemm_r64", "jl_moe_gemm_r64_planes", "jl_moe_gemm_q6k_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_mxfp4_matvec1_b1", "jl_mxfp4_matvec1_b2", "jl_mxfp4_matvec1_b3", "jl_mxfp4_scaled_prep", "jl_mxfp4_scaled_gemm", "jl_mxfp4_planes_prep", "jl_mxfp4_planes_gemm", "jl_mxfp4_matvec_planes_r64", "jl_mxfp4_matvec_planes_r32", "jl_mxfp4_matvec_planes_r16", "jl_unpack_mxfp4", "jl_sum_parts", "jl_fill_u32", "jl_probe_read", "jl_probe_empty", "jl_probe_wait", "jl_probe_mfma", "jl_probe_mfma_v5",
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_matvec_q4k_r1_pq", "jl_matvec_q4k_r1_pq_res", "jl_matvec_q8_0_r1_pq", "jl_matvec_q8_0_r1_pq_res", "jl_matvec_q6k_r1_pq", "jl_matvec_q6k_r1_pq_res", "jl_matvec_q8_0p_r1_pq", "jl_matvec_q8_0p_r1_pq_res", "jl_matvec_multi_q4k_res", "jl_matvec_multi_q4k_x4_res", "jl_matvec_multi_q4k_q_res", "jl_matvec_multi_q8_0_res", "jl_matvec_multi_q8_0_x4_res", "jl_matvec_multi_q8_0_q_res", "jl_matvec_multi_q6k_res", "jl_matvec_multi_q6k_x4_res", "jl_matvec_multi_q6k_q_res", "jl_matvec_multi_q8_0p_res", "jl_matvec_multi_q8_0p_x4_res", "jl_matvec_multi_q8_0p_q_res", "jl_matvec_q4k_r1_res", "jl_matvec_q4k_r1_x4_res", "jl_matvec_q8_0_r1_res", "jl_matvec_q8_0_r1_x4_res", "jl_matvec_q6k_r1_res", "jl_matvec_q6k_r1_x4_res", "jl_matvec_q8_0p_r1_res", "jl_matvec_q8_0p_r1_x4_res", "jl_matvec_q8_0p_r1", "jl_matvec_q8_0p_r2", "jl_matvec_q8_0p_r4", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_q4k_k2", "jl_gemm_q4k_k2_planes", "jl_gemm_prep_q4k_planes", "jl_gemm_q4k_r64_planes", "jl_gemm_q4k_wide_planes", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_group2_wide", "jl_moe_quant", "jl_moe_matvec_planes_q4k", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_prep_planes", "jl_moe_gemm_q4k", "jl_moe_g16_prep", "jl_moe_g16_prep_planes", "jl_moe_g16_prep_q6k", "jl_moe_g16_c1", "jl_moe_g16_c2", "jl_moe_g16_c3", "jl_moe_g16_f1", "jl_moe_g16_f2", "jl_moe_g16_f3", "jl_moe_g16_g1", "jl_moe_g16_g2", "jl_moe_g16_g3", "jl_moe_g16_d1", "jl_moe_g16_d2", "jl_moe_g16_d3", "jl_moe_g16p_c1", "jl_moe_g16p_c2", "jl_moe_g16p_c3", "jl_moe_g16p_f1", "jl_moe_g16p_f2", "jl_moe_g16p_f3", "jl_moe_g16p_g1", "jl_moe_g16p_g2", "jl_moe_g16p_g3", "jl_moe_g16p_d1", "jl_moe_g16p_d2", "jl_moe_g16p_d3", "jl_moe_g16q6_c1", "jl_moe_g16q6_c2", "jl_moe_g16q6_c3", "jl_moe_g16q6_f1", "jl_moe_g16q6_f2", "jl_moe_g16q6_f3", "jl_moe_g16q6_g1", "jl_moe_g16q6_g2", "jl_moe_g16q6_g3", "jl_moe_g16q6_d1", "jl_moe_g16q6_d2", "jl_moe_g16q6_d3", "jl_moe_gemm_r64", "jl_moe_gemm_r64_planes", "jl_moe_gemm_q6k_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_mxfp4_matvec1_b1", "jl_mxfp4_matvec1_b2", "jl_mxfp4_matvec1_b3", "jl_mxfp4_scaled_prep", "jl_mxfp4_scaled_gemm", "jl_mxfp4_planes_prep", "jl_mxfp4_planes_gemm", "jl_mxfp4_matvec_planes_r64", "jl_mxfp4_matvec_planes_r32", "jl_mxfp4_matvec_planes_r16", "jl_unpack_mxfp4", "jl_sum_parts", "jl_fill_u32", "jl_probe_read", "jl_probe_empty", "jl_probe_wait", "jl_probe_mfma", "jl_probe_mfma_v5",
                                       "jl_pack_weights", "jl_unpack_q4k", "jl_unpack_q6k", "jl_unpack_q8_0"};
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int rw : {16, 32, 64})

@@ -63,13 +63,20 @@ extern "C" __global__ __launch_bounds__(256) void jl_dequant(
     extern "C" __global__ __launch_bounds__(MAXT) void jl_matvec_##T##_r##RPW##_x4(MatVecArgs p) { \
         matvec_body<TYPE, RPW, 4>(p, jl_smem);                                               \
     }
-// _res: one row a wavefront with resid[r] += weight * out[r] riding on the store (MatVecArgs.resid set)
+// _res: one row a wavefront with resid[r] += weight * out[r] riding on the store (MatVecArgs.resid set);
+// _pq: one row a wavefront over an activation that comes quantized (MatVecArgs.q / as / s16, x null)
 #define JL_MATVEC_RES_KERNEL(T, TYPE)                                                               \
     extern "C" __global__ __launch_bounds__(1024) void jl_matvec_##T##_r1_res(MatVecArgs p) {       \
         matvec_body<TYPE, 1, 1, true>(p, jl_smem);                                                  \
     }                                                                                               \
     extern "C" __global__ __launch_bounds__(1024) void jl_matvec_##T##_r1_x4_res(MatVecArgs p) {    \
         matvec_body<TYPE, 1, 4, true>(p, jl_smem);                                                  \
+    }                                                                                               \
+    extern "C" __global__ __launch_bounds__(1024) void jl_matvec_##T##_r1_pq(MatVecArgs p) {        \
+        matvec_body<TYPE, 1, 1, false, true>(p, jl_smem);                                           \
+    }                                                                                               \
+    extern "C" __global__ __launch_bounds__(1024) void jl_matvec_##T##_r1_pq_res(MatVecArgs p) {    \
+        matvec_body<TYPE, 1, 1, true, true>(p, jl_smem);                                            \
     }
 JL_MATVEC_RES_KERNEL(q4k, JL_Q4_K) JL_MATVEC_RES_KERNEL(q8_0, JL_Q8_0) JL_MATVEC_RES_KERNEL(q6k, JL_Q6_KS)
 JL_MATVEC_RES_KERNEL(q8_0p, JL_Q8_0P)

@@ -589,7 +589,8 @@ __device__ __forceinline__ float resid_weight(float alpha, const float* gate) {
 // RES: the residual add rides on the store (entry points of their own: with the add and its
 // gate's f64 exponential compiled into the plain kernel behind a branch, the plain matvecs ran
 // 10-20 % slower, Q8_0 14336 x 4096 14.2 against 11.8 us).
-template <int TYPE, int RPW, int XP, bool RES>
+// PQ: the activation comes quantized (MatVecArgs.q / as / s16) and is only copied into LDS.
+template <int TYPE, int RPW, int XP, bool RES, bool PQ>
 __device__ __forceinline__ void matvec_body_xp(const MatVecArgs& p, uint8_t* smem) {
     typedef SlotTraits<TYPE> T;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = p.nwaves;
@@ -607,7 +608,7 @@ __device__ __forceinline__ void matvec_body_xp(const MatVecArgs& p, uint8_t* sme
     f32x4 x0[XP];
 #pragma unroll
     for (int i = 0; i < XP; i++) x0[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-    if (p.x) {
+    if constexpr (!PQ) {
         load_x_groups<XP>(p.x, p.k, nwaves * 64, x0);
         __builtin_amdgcn_s_barrier();
     }
@@ -620,7 +621,7 @@ __device__ __forceinline__ void matvec_body_xp(const MatVecArgs& p, uint8_t* sme
             T::load_w(p.w + (size_t)min(r0 + j, p.nrows - 1) * p.row_bytes, s, w[j]);
     }
     constexpr int SH = stage_layout_of(TYPE);
-    if (p.x) stage_act_quantize<SH, XP>(smem, p.x, p.k, p.per, x0, nwaves * 64);
+    if constexpr (!PQ) stage_act_quantize<SH, XP>(smem, p.x, p.k, p.per, x0, nwaves * 64);
     else stage_act_copy<SH>(smem, p.q, p.as, p.s16, p.k, nwaves * 64);
     lds_barrier();   // orders the LDS staging only: the weight loads stay in flight
 
@@ -638,9 +639,9 @@ __device__ __forceinline__ void matvec_body_xp(const MatVecArgs& p, uint8_t* sme
 
 // XP = 1: a vector of at most one float4 group a thread; 4: longer ones (the host picks the
 // entry point; one body compiled for both behind a branch ran the short-vector case 10 % slower).
-template <int TYPE, int RPW, int XP = 1, bool RES = false>
+template <int TYPE, int RPW, int XP = 1, bool RES = false, bool PQ = false>
 __device__ __forceinline__ void matvec_body(const MatVecArgs& p, uint8_t* smem) {
-    matvec_body_xp<TYPE, RPW, XP, RES>(p, smem);
+    matvec_body_xp<TYPE, RPW, XP, RES, PQ>(p, smem);
 }
 
 // Several matvecs of one type in one launch: grid = (row groups, matrices).  Each
