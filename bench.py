@@ -40,7 +40,7 @@ CACHE_BYTES = 256 << 20  # Infinity Cache; rotate through more than twice this
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # script (profiles/), scaled by the same counters over a plain copy of known
 # size (profiles/matvec_q4k_4096_hbm_traffic.md: fetch 4723.0 x 1.9950 KiB + write 16 KiB).
-MEASURED_TRAFFIC = {"c1": 9664922}
+MEASURED_TRAFFIC = {"c1": 9638349}
 
 
 def matvec_bytes(t, nrows, k):
@@ -735,6 +735,10 @@ def ceiling_section(dev, gate_):
     out = {}
     ms = measure(dev, lambda i: dev.probe_dev(0, None, 0, 512, 1024), 200, gate_, warm=50)
     out["empty_kernel"] = {"us_per_launch": round(ms * 1e3, 3), "grid": 512, "block": 1024}
+    # the floor as a function of the grid: workgroups x threads
+    out["empty_kernel_by_grid_us"] = {
+        f"{grid}x{block}": round(measure(dev, lambda i: dev.probe_dev(0, None, 0, grid, block), 200, gate_, warm=20) * 1e3, 3)
+        for grid in (64, 256, 1024, 2048) for block in (64, 256, 1024)}
     # the matrix cores with nothing to wait for: 8 wavefronts a CU, 2000 rounds of four
     # 32x32x16 f16 matrix instructions each; then the same with five vector instructions
     # after each matrix instruction, the prefill GEMM loop's share
@@ -749,16 +753,17 @@ def ceiling_section(dev, gate_):
                          ("48 MB (Q6_K 4096x14336)", 48168960), ("62 MB (Q8_0 14336x4096)", 62390272)]:
         stride = (nbytes + 4095) & ~4095
         ncopies = pool.nbytes // stride
-        best = None
+        best, by_shape = None, {}
         for grid, block in [(256, 1024), (512, 1024), (1024, 512), (2048, 256), (512, 768)]:
             ms = measure(dev, lambda i: dev.probe_dev(1, pool.ptr + (i % ncopies) * stride, nbytes, grid, block),
                          100, gate_, warm=20)
+            by_shape[f"{grid}x{block}"] = round(ms * 1e3, 3)
             if best is None or ms < best[0]:
                 best = (ms, grid, block)
         ms, grid, block = best
         out[name] = {"us_per_launch": round(ms * 1e3, 3), "GB/s": round(nbytes / (ms * 1e-3) / 1e9, 1),
                      "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-                     "grid": grid, "block": block, "copies": ncopies}
+                     "grid": grid, "block": block, "copies": ncopies, "us_by_grid_x_block": by_shape}
     pool.free()
     return out
 
