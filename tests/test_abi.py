@@ -134,3 +134,42 @@ def test_forget_returns_while_another_thread_holds_the_context_lock():
     rc = lib.jl_matvec(ctx, out.ctypes.data, quant.Q4_K, w.ctypes.data, w.nbytes, x.ctypes.data, 1, 256)
     assert rc < 0 and lib.jl_last_error(ctx)
     lib.jl_ctx_destroy(ctx)
+
+
+def test_block_seam_argument_checks_without_a_gpu():
+    """jl_prep_layer / jl_layer_ffn_dev / jl_release_layers / jl_layer_count on a context bound
+    to no device: broken plans are errors, a type without a kernel is a decline (the reference's
+    PrepLayer returns false and the block stays on the CPU, /root/reference/engine/nn/device.go:
+    1096-1131), a good plan fails loudly at the device, and nothing is left prepared."""
+    import ctypes as C
+    lib = _lib.load()
+    ctx = C.c_void_p()
+    opts = _lib.Options(-1, 32, None)
+    assert lib.jl_ctx_create(C.byref(ctx), C.byref(opts)) == _lib.OK and ctx.value
+    E, F = 256, 512
+    gate = np.zeros(F * (E // 32) * 34, np.uint8)
+    down = np.zeros(E * (F // 32) * 34, np.uint8)
+
+    def plan(**kw):
+        p = _lib.LayerPlan(_lib.LAYER_DENSE, quant.Q8_0, quant.Q8_0, E, F, 0, gate.ctypes.data, gate.ctypes.data,
+                           down.ctypes.data, None, 0.0, 0, 0, None)
+        for k, v in kw.items():
+            setattr(p, k, v)
+        return p
+
+    assert lib.jl_layer_count(ctx) == 0
+    assert lib.jl_prep_layer(ctx, 0, None) < 0
+    assert lib.jl_prep_layer(ctx, -1, C.byref(plan())) < 0
+    assert lib.jl_prep_layer(ctx, 0, C.byref(plan(gate=None))) < 0
+    assert lib.jl_prep_layer(ctx, 0, C.byref(plan(kind=7))) < 0
+    assert lib.jl_prep_layer(ctx, 0, C.byref(plan(kind=_lib.LAYER_MOE, n_expert=4, k_used=2))) < 0      # no router
+    assert lib.jl_prep_layer(ctx, 0, C.byref(plan(type=99))) == _lib.DECLINED                            # no kernel
+    assert lib.jl_prep_layer(ctx, 0, C.byref(plan(type=quant.Q4_K, n_embd=96))) == _lib.DECLINED         # k % 256
+    rc = lib.jl_prep_layer(ctx, 0, C.byref(plan()))
+    assert rc < 0 and lib.jl_last_error(ctx)            # a good plan: no device to put it on
+    assert lib.jl_layer_count(ctx) == 0
+    x = np.zeros(E, np.float32)
+    assert lib.jl_layer_ffn_dev(ctx, 0, x.ctypes.data, x.ctypes.data, 1, None) < 0
+    assert b"not prepared" in lib.jl_last_error(ctx)
+    assert lib.jl_release_layers(ctx, 0, 100) == _lib.OK
+    lib.jl_ctx_destroy(ctx)
