@@ -221,3 +221,83 @@ def test_prep_layer_declines_what_has_no_kernel_and_replaces_a_block(dev, devbuf
     assert dev.Layers() == before + 1
     dev.ReleaseLayers(0, 100)
     assert dev.Layers() == 0
+
+
+def test_config2_block_by_handle_at_full_size(dev, devbuf):
+    """The baseline's dense block at its own sizes -- gate and up Q8_0 14336 x 4096, down Q6_K
+    4096 x 14336, RMSNorm in front, activation window 32 -- prepared from host memory and run by
+    handle: the bits of the two pointer-form launches, whose kernels the full-size matvec tests hold
+    to the oracle, and the block's value on a sample of rows recomputed in f64."""
+    E, F, window, eps = 4096, 14336, 32, 1e-5
+    dev.SetActWindow(window)
+    gate, up = synth.quantized_weights(quant.Q8_0, F, E, seed=0), synth.quantized_weights(quant.Q8_0, F, E, seed=1)
+    down = synth.quantized_weights(quant.Q6_K, E, F, seed=2)
+    nw = (1 + 0.1 * np.random.default_rng(3).standard_normal(E)).astype(np.float32)
+    h, resid0 = synth.activations(E, seed=4), synth.activations(E, seed=5)
+    hd, nwd = devbuf(h), devbuf(nw)
+    wg, wu, wd = devbuf(gate), devbuf(up), devbuf(down)
+    g, u, y = (devbuf(shape=(n,), dtype=np.float32, fill=0) for n in (F, F, E))
+    want = devbuf(resid0)
+    assert dev.matvec_group_dev([g.ptr, u.ptr], [quant.Q8_0] * 2, [wg.ptr, wu.ptr], [F, F], hd.ptr, E, norm_w=nwd.ptr,
+                                norm_eps=eps)
+    assert dev.matvec_group_dev([y.ptr], [quant.Q6_K], [wd.ptr], [E], g.ptr, F, act_up=u.ptr, resid=want.ptr, alpha=1.0)
+    dev.synchronize()
+    for b in (wg, wu, wd):
+        b.free()
+    assert dev.PrepLayer(2, _lib.LAYER_DENSE, quant.Q8_0, E, F, gate, up, down, down_type=quant.Q6_K, norm_w=nw,
+                         norm_eps=eps)
+    try:
+        for _ in range(2):
+            got = devbuf(resid0)
+            assert dev.layer_ffn_dev(2, hd.ptr, got.ptr, 1)
+            dev.synchronize()
+            assert np.array_equal(_bits(got.get()), _bits(want.get()))
+    finally:
+        dev.ReleaseLayers(2, 3)
+    # the value itself, on the device's own gate and up (so a moved int8 of the gated activation
+    # cannot hide an error): rows spread over the matrix
+    gg, uu = g.get(), u.get()
+    act = (silu(gg) * uu.astype(np.float64)).astype(np.float32)
+    q, a_s, _ = oracle.quantize_act(act, window)
+    rows = np.unique(np.linspace(0, E - 1, 96).astype(int))
+    nb = F // 256 * 210
+    sample = np.concatenate([down[r * nb:(r + 1) * nb] for r in rows])
+    yy = oracle.matvec_q8act_f64(quant.Q6_K, sample, q, a_s, len(rows), F)
+    assert rel_l2((want.get() - resid0)[rows], yy) <= 2e-3
+
+
+def test_config4_mixture_block_by_handle_at_full_size(dev, devbuf):
+    """The baseline's mixture block at its own sizes -- 128 experts of 768 x 2048 / 2048 x 768 Q4_K,
+    64 rows routed top-8 -- prepared from host memory (340 MB, one allocation) and run by handle:
+    the bits of the pointer-form calls, which the mixture tests hold to the oracle."""
+    t, n_expert, k_used, F, E, rows = quant.Q4_K, 128, 8, 768, 2048, 64
+    dev.SetActWindow(256)
+    gate, up, down = _bank(t, n_expert, F, E, 1000), _bank(t, n_expert, F, E, 2000), _bank(t, n_expert, E, F, 3000)
+    rng = np.random.default_rng(9)
+    router = (rng.standard_normal((n_expert, E)) / np.sqrt(E)).astype(np.float32)
+    h = rng.standard_normal((rows, E)).astype(np.float32)
+    resid0 = rng.standard_normal((rows, E)).astype(np.float32)
+    hd, rd = devbuf(h), devbuf(router)
+    wg, wu, wd = devbuf(gate), devbuf(up), devbuf(down)
+    try:
+        # (a row count of its own each: seven rows are under two columns an expert and run another
+        # kernel form, with another order of f32 sums, than sixty-four)
+        want = {}
+        for n in (rows, 7):
+            want[n] = devbuf(resid0)
+            assert dev.moe_block_dev(want[n].ptr, t, wg.ptr, wu.ptr, wd.ptr, rd.ptr, hd.ptr, n, k_used, n_expert, F, E)
+        dev.synchronize()
+        for b in (wg, wu, wd):
+            b.free()
+        assert dev.PrepLayer(4, _lib.LAYER_MOE, t, E, F, gate, up, down, n_expert=n_expert, k_used=k_used, router=router)
+        for n in (rows, 7):
+            got = devbuf(resid0)
+            assert dev.layer_ffn_dev(4, hd.ptr, got.ptr, n)
+            dev.synchronize()
+            out = got.get()
+            assert np.array_equal(_bits(out), _bits(want[n].get()))
+            assert np.array_equal(_bits(out[n:]), _bits(resid0[n:]))
+            assert not np.array_equal(out[:n], resid0[:n])
+    finally:
+        dev.ReleaseLayers(0, 8)
+        dev.SetActWindow(32)
