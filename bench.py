@@ -273,7 +273,9 @@ def gemm_section(dev, gate, shapes=None, t=None, k=4096, window=256, packed=Fals
     peak (the kernel runs exact integer operands on the f16 matrix cores).
     shapes: {nrows: [ntok, ...]}; default = the baseline's prefill configurations.
     t = Q6_K / Q8_0: the same model's other tensors.  packed: the weights as packed planes
-    (jl_matmul_packed_dev).  Output check: 96 rows spread over the matrix x every token."""
+    (jl_matmul_packed_dev).  Output check: 96 rows spread over the matrix x every token.
+    Q4_K rows also run the opt-in folded-scale form ("gemm.fold" = 1) where it applies, reported
+    beside the exact form with its measured rel-L2 against the exact result."""
     from jitllm_amd import quant, synth
     from jitllm_amd.device import Packed
     from jitllm_amd.hipmem import DeviceArray
@@ -287,6 +289,7 @@ def gemm_section(dev, gate, shapes=None, t=None, k=4096, window=256, packed=Fals
         rows = spread_rows(nrows, 96)
         wrows = dequant_rows(dev, t, w_host, rows, k)
         pl = None
+        folded = t == quant.Q4_K and not packed and dev.fold_admit_dev(t, w.ptr, nrows, k)
         if packed:
             bufs = [DeviceArray(shape=(max(n, 1),), dtype=np.uint32, fill=0) for n in dev.packed_words(t, nrows, k)]
             if not dev.pack_weights_dev(t, w.ptr, nrows, k, bufs[0].ptr, bufs[1].ptr, bufs[2].ptr):
@@ -314,8 +317,31 @@ def gemm_section(dev, gate, shapes=None, t=None, k=4096, window=256, packed=Fals
             out[f"{ntok}x{k}->{nrows}"] = {"us_per_step": round(ms * 1e3, 1), "TFLOP/s": round(tf, 1),
                                           "frac_of_f16_mfma_peak": round(tf / MFMA_F16_PEAK_TFLOPS, 4),
                                           "checked_rel_err": float(f"{err:.2e}")}
+            if folded:
+                # the opt-in folded-scale form beside the exact one: never the line above, and
+                # its time only together with its measured distance from the exact result
+                dev.set_tuning(gemm__fold=1)
+                try:
+                    ms_f = measure(dev, run, 20, gate)
+                    got_f = o.get()
+                finally:
+                    dev.set_tuning(gemm__fold=0)
+                if not np.array_equal(got_f.view(np.uint32), got.view(np.uint32)):   # else: a shape the form does not serve
+                    if not np.all(np.isfinite(got_f)):
+                        raise RuntimeError(f"folded prefill GEMM {ntok}x{k}->{nrows}: non-finite output")
+                    e = got.astype(np.float64)
+                    rel = float(np.sqrt(np.sum((got_f - e) ** 2) / np.sum(e * e)))
+                    if rel > 1e-3:
+                        raise RuntimeError(f"folded prefill GEMM {ntok}x{k}->{nrows}: rel-L2 {rel:.2e} against the exact form")
+                    tf_f = 2.0 * nrows * k * ntok / (ms_f * 1e-3) / 1e12
+                    out[f"{ntok}x{k}->{nrows}"]["folded_opt_in"] = {
+                        "us_per_step": round(ms_f * 1e3, 1), "TFLOP/s": round(tf_f, 1),
+                        "frac_of_f16_mfma_peak": round(tf_f / MFMA_F16_PEAK_TFLOPS, 4),
+                        "rel_l2_vs_exact_form": float(f"{rel:.2e}")}
             x.free()
             o.free()
+        if folded:
+            dev.forget_range(w.ptr, w_host.nbytes)
         w.free()
         if packed:
             for b in bufs:
@@ -726,11 +752,13 @@ def mxfp4_section(dev, gate_):
     return out
 
 
-def ceiling_section(dev, gate_):
+def ceiling_section(dev, gate_, vendor_gemm=False):
     """What a single launch costs on this machine before any arithmetic, beside the kernels it
     bounds: back-to-back empty kernels, and a kernel that only READS n bytes (every thread
     keeps eight 128-bit loads in flight; nothing is stored), over rotating buffers that exceed
-    twice the Infinity Cache, at the sizes of the decode matvecs.  Median of nine windows."""
+    twice the Infinity Cache, at the sizes of the decode matvecs.  Median of nine windows.
+    vendor_gemm (--section ceiling only: it imports torch): the vendor library's plain f16 GEMM
+    at the prefill shapes."""
     from jitllm_amd.hipmem import DeviceArray
     out = {}
     ms = measure(dev, lambda i: dev.probe_dev(0, None, 0, 512, 1024), 200, gate_, warm=50)
@@ -765,6 +793,38 @@ def ceiling_section(dev, gate_):
                      "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                      "grid": grid, "block": block, "copies": ncopies, "us_by_grid_x_block": by_shape}
     pool.free()
+    if vendor_gemm:
+        out["vendor_f16_gemm"] = vendor_gemm_section()
+    return out
+
+
+def vendor_gemm_section():
+    """A yardstick, not a part of the path: the vendor library's plain f16 GEMM (torch.matmul, which
+    runs hipBLASLt) at the prefill GEMM's shapes, its weights ALREADY f16 in memory -- no activation
+    quantizer, no dequantization, none of the exact integer arithmetic.  What a tuned kernel reaches
+    on this machine at these shapes when it has none of that to do."""
+    import torch
+    out = {}
+    for ntok, nrows in ((512, 4096), (2048, 4096), (512, 14336), (2048, 14336)):
+        a = torch.randn(ntok, 4096, device="cuda", dtype=torch.float16)
+        b = torch.randn(nrows, 4096, device="cuda", dtype=torch.float16)
+        for _ in range(5):
+            c = a @ b.t()
+        torch.cuda.synchronize()
+        windows = []
+        for _ in range(9):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(20):
+                c = a @ b.t()
+            e1.record()
+            e1.synchronize()
+            windows.append(e0.elapsed_time(e1) / 20)
+        ms = sorted(windows)[len(windows) // 2]
+        tf = 2.0 * nrows * 4096 * ntok / (ms * 1e-3) / 1e12
+        out[f"{ntok}x4096->{nrows}"] = {"us_per_step": round(ms * 1e3, 1), "TFLOP/s": round(tf, 1),
+                                       "frac_of_f16_mfma_peak": round(tf / MFMA_F16_PEAK_TFLOPS, 4)}
+        del a, b, c
     return out
 
 
@@ -818,7 +878,7 @@ def main():
     if args.section:
         fn = {"mxfp4": mxfp4_section, "moe": moe_section, "moe_packed": lambda d, g: moe_section(d, g, packed=True),
               "moe_decode": moe_decode_section, "ffn": ffn_section,
-              "ffn_packed": ffn_packed_section, "ceiling": ceiling_section,
+              "ffn_packed": ffn_packed_section, "ceiling": lambda d, g: ceiling_section(d, g, vendor_gemm=True),
               "gemm_packed": lambda d, g: gemm_section(d, g, {4096: (512,), 14336: (512,)}, packed=True)}[args.section]
         print(json.dumps({args.section: fn(dev, gate)}), flush=True)
         dev.close()

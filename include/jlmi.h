@@ -110,10 +110,14 @@ int jl_synchronize(jl_ctx *ctx);
  * general decode matvec also for one token), "mxfp4.planes" (packed MXFP4: 2 restores rows
  * first, 3 the plane GEMM whatever the grid, 64 / 32 / 16 rows a workgroup of the plane
  * matvec); value 0 restores the built-in choice.  These change launch shapes and f32 summation
- * order only.  One key changes values: "mxfp4.scaled" = 1 runs jl_matmul_mxfp4_packed_bf16_dev
- * on the block-scaled fp8 x fp4 matrix instruction, which quantizes the activations to MX fp8
- * (rel-L2 about 2.7e-2 against the bf16 activations); it is off unless set.  Mirrors the
- * reference's per-instance tuning knobs (engine/nn/options.go:67-118). */
+ * order only.  Two keys change values, both off unless set: "mxfp4.scaled" = 1 runs
+ * jl_matmul_mxfp4_packed_bf16_dev on the block-scaled fp8 x fp4 matrix instruction, which
+ * quantizes the activations to MX fp8 (rel-L2 about 2.7e-2 against the bf16 activations);
+ * "gemm.fold" = 1 lets the Q4_K prefill GEMM of jl_matmul_dev run its 256 x 128 tiles on
+ * operands that carry the scales (weights d * sc * q - dmin * m and activations d_a * a, each
+ * rounded to f16; rel-L2 about 7e-4 against the exact forms, inside the path's 1e-3), for the
+ * matrices jl_fold_admit_dev has admitted and no others ("gemm.fold_waves": 4 or 8 wavefronts a
+ * workgroup).  Mirrors the reference's per-instance tuning knobs (engine/nn/options.go:67-118). */
 int jl_set_tuning(jl_ctx *ctx, const char *key, int value);
 
 /* Kernels this context has launched so far: how callers and tests check that a grouped
@@ -383,6 +387,17 @@ size_t jl_static_scratch_bytes(void);
  * then undefined.  To learn that, the MXFP4 call alone waits for its kernel. */
 int jl_pack_weights_dev(jl_ctx *ctx, int type, const void *src, int nrows, int k, uint32_t *qs,
                         uint32_t *d, uint32_t *sc, void *stream);
+
+/* Admits a Q4_K matrix in device memory (GGUF rows, 4-byte aligned) to the folded-scale GEMM
+ * form that "gemm.fold" = 1 switches on: checks that no super-block's weights can pass the f16
+ * range (|d| * 945 + |dmin| * 63 <= 65504, finite), waits for that check, and remembers the
+ * matrix by its address, rows and k.  JL_DECLINED for scales outside the range (and for another
+ * type): such a matrix keeps the exact forms whatever the key says.  A call made once after
+ * the weights are in place; jl_forget over the matrix's address range withdraws it, and a
+ * matrix rewritten in place is admitted again by a new call.  Activations beyond the f16
+ * range give non-finite outputs in the folded form, as in any f16 GEMM.  No counterpart in
+ * the reference, whose kernels keep the scales apart (engine/nn/matmul.go:27-189). */
+int jl_fold_admit_dev(jl_ctx *ctx, int type, const void *w, int nrows, int k, void *stream);
 
 /* The inverse permutation for Q4_K, Q6_K, Q8_0 and MXFP4: rows row .. row+nrows of the
  * planes back to GGUF blocks in dst (nrows * k/256 * 144 bytes, 4-byte aligned; Q6_K 210

@@ -92,6 +92,7 @@ SIGNATURES = {
     "jl_matvec_packed": (_int, [_vp, _vp, _int, _vp, _vp, _vp, _int, _int, _vp, _int, _int]),
     "jl_matmul_packed": (_int, [_vp, _vp, _int, _vp, _vp, _vp, _int, _int, _vp, _int, _int, _int]),
     "jl_pack_weights_dev": (_int, [_vp, _int, _vp, _int, _int, _vp, _vp, _vp, _vp]),
+    "jl_fold_admit_dev": (_int, [_vp, _int, _vp, _int, _int, _vp]),
     "jl_unpack_weights_dev": (_int, [_vp, _int, _vp, _vp, _vp, _int, _int, _int, _int, _vp, _vp]),
     "jl_matvec_packed_dev": (_int, [_vp, _vp, _int, _vp, _vp, _vp, _int, _int, _vp, _int, _int, _vp]),
     "jl_matvec_packed_q8_dev": (_int, [_vp, _vp, _int, _vp, _vp, _vp, _int, _int, _vp, _vp, _vp, _int,

@@ -44,6 +44,7 @@ struct Tuning {
     int gemm_planes = 0;
     int moe_form = 0;
     int moe_g16 = 0;
+    int gemm_fold = 0, gemm_fold_waves = 0;
     int moe_chunk = 0;
     int moe_waves = 0;
     int moe_lpr = 0;
@@ -87,6 +88,9 @@ struct jl_ctx {
     // host-pointer calls apply the queue (unlink + hipFree) before their residency lookup
     std::mutex forget_mu;
     std::vector<std::pair<uintptr_t, uintptr_t>> pending_forget;
+    // Q4_K matrices (device address -> rows, k) whose scales jl_fold_admit_dev found inside the
+    // f16 range: the only ones the folded-scale GEMM form is used for (under forget_mu)
+    std::map<uintptr_t, std::pair<int, int>> fold_ok;
     bool no_device = false;   // created with device < 0: host-side bookkeeping only
     // the static device array of scratch.hip on this context's device (null: the lookup
     // failed and static_err says why), and the state of a call that lives on it
@@ -654,6 +658,14 @@ int gemm_q4k_launch(jl_ctx* c, float* out, const void* w, const float* x, int nr
     }
     if (form == 2 && kGemmWideLdsBytes > c->lds_limit) form = 1;
     if (form == 6 && !k2_fits) form = 1;
+    // the opt-in folded-scale form (kernels/gemm_q4k_fold.h): asked for with "gemm.fold" = 1,
+    // and only for a matrix whose scales jl_fold_admit_dev has checked
+    bool fold = false;
+    if (c->tune.gemm_fold == 1 && form == 2 && !pl && 2u * 128u * 136u * 2u <= c->lds_limit) {
+        std::lock_guard<std::mutex> g(c->forget_mu);
+        auto it = c->fold_ok.find((uintptr_t)w);
+        fold = it != c->fold_ok.end() && it->second.first == nrows && it->second.second == k;
+    }
     const int tile = form == 2 ? kGemmWideTok : kGemmTile;
     const int tok_pad = (ntok + tile - 1) / tile * tile;
     const int nsb = k / 256;
@@ -669,8 +681,8 @@ int gemm_q4k_launch(jl_ctx* c, float* out, const void* w, const float* x, int nr
     // 87.1 -> 83.4; "gemm.prep" = 4 asks for four wavefronts)
     const bool prep16 = c->tune.gemm_prep != 4;
     // (the plane kernels take the activations in the planes' K order: their own prep)
-    rc = launch(c, pl ? "jl_gemm_prep_q4k_planes" : prep16 ? "jl_gemm_prep_q4k_w16" : "jl_gemm_prep_q4k", (unsigned)nsb,
-                (unsigned)(tok_pad / 32), pl || prep16 ? 1024 : 256, 0, st, pp);
+    rc = launch(c, fold ? "jl_gemm_prep_q4k_fold" : pl ? "jl_gemm_prep_q4k_planes" : prep16 ? "jl_gemm_prep_q4k_w16" : "jl_gemm_prep_q4k",
+                (unsigned)nsb, (unsigned)(tok_pad / 32), fold || pl || prep16 ? 1024 : 256, 0, st, pp);
     if (rc != JL_OK) return rc;
     if (form == 3) return gemm_q4k_w16_launch(c, out, w, bq, da, nrows, k, ntok, tok_pad, st);
     GemmArgs ga;
@@ -679,6 +691,15 @@ int gemm_q4k_launch(jl_ctx* c, float* out, const void* w, const float* x, int nr
     ga.nrows = nrows; ga.k = k; ga.ntok = ntok; ga.tok_pad = tok_pad; ga.row_bytes = nsb * 144;
     ga.out_stride = nrows; ga.sb_per = 0;
     void* gp[] = {&ga};
+    if (fold) {
+        // four wavefronts a workgroup, two workgroups a CU, from a full round of the chip on;
+        // eight below (measured, us: 2048 tokens x 14336 rows 238 against 251; 1024 x 4096
+        // 59.7 against 55.1; a round or so, 2048 x 4096 and 512 x 14336, the same)
+        const long groups = (long)(tok_pad / kGemmWideTok) * ((nrows + 127) / 128);
+        const bool w8 = c->tune.gemm_fold_waves == 8 || (c->tune.gemm_fold_waves != 4 && groups < (long)c->num_cu);
+        return launch(c, w8 ? "jl_gemm_q4k_fold_wide" : "jl_gemm_q4k_fold_wide4", (unsigned)(tok_pad / kGemmWideTok),
+                      (unsigned)((nrows + 127) / 128), w8 ? 512 : 256, 2u * 128u * 136u * 2u, st, gp);   // JL_GEMM_FOLD_LDS_BYTES
+    }
     if (form == 6)   // 128 x 64 tiles over the whole of K, the K halves on two groups of wavefronts
         return launch(c, pl ? "jl_gemm_q4k_k2_planes" : "jl_gemm_q4k_k2", (unsigned)(tok_pad / kGemmTile), (unsigned)((nrows + 63) / 64), 512,
                       kGemmK2LdsBytes, st, gp);
@@ -1414,7 +1435,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     if (e != hipSuccess)
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
-    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_matvec_q4k_r1_pq", "jl_matvec_q4k_r1_pq_res", "jl_matvec_q8_0_r1_pq", "jl_matvec_q8_0_r1_pq_res", "jl_matvec_q6k_r1_pq", "jl_matvec_q6k_r1_pq_res", "jl_matvec_q8_0p_r1_pq", "jl_matvec_q8_0p_r1_pq_res", "jl_matvec_multi_q4k_res", "jl_matvec_multi_q4k_x4_res", "jl_matvec_multi_q4k_q_res", "jl_matvec_multi_q8_0_res", "jl_matvec_multi_q8_0_x4_res", "jl_matvec_multi_q8_0_q_res", "jl_matvec_multi_q6k_res", "jl_matvec_multi_q6k_x4_res", "jl_matvec_multi_q6k_q_res", "jl_matvec_multi_q8_0p_res", "jl_matvec_multi_q8_0p_x4_res", "jl_matvec_multi_q8_0p_q_res", "jl_matvec_q4k_r1_res", "jl_matvec_q4k_r1_x4_res", "jl_matvec_q8_0_r1_res", "jl_matvec_q8_0_r1_x4_res", "jl_matvec_q6k_r1_res", "jl_matvec_q6k_r1_x4_res", "jl_matvec_q8_0p_r1_res", "jl_matvec_q8_0p_r1_x4_res", "jl_matvec_q8_0p_r1", "jl_matvec_q8_0p_r2", "jl_matvec_q8_0p_r4", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_q4k_k2", "jl_gemm_q4k_k2_planes", "jl_gemm_prep_q4k_planes", "jl_gemm_q4k_r64_planes", "jl_gemm_q4k_wide_planes", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_group2_wide", "jl_moe_quant", "jl_moe_matvec_planes_q4k", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_prep_planes", "jl_moe_gemm_q4k", "jl_moe_g16_prep", "jl_moe_g16_prep_planes", "jl_moe_g16_prep_q6k", "jl_moe_g16_c1", "jl_moe_g16_c2", "jl_moe_g16_c3", "jl_moe_g16_f1", "jl_moe_g16_f2", "jl_moe_g16_f3", "jl_moe_g16_g1", "jl_moe_g16_g2", "jl_moe_g16_g3", "jl_moe_g16_d1", "jl_moe_g16_d2", "jl_moe_g16_d3", "jl_moe_g16p_c1", "jl_moe_g16p_c2", "jl_moe_g16p_c3", "jl_moe_g16p_f1", "jl_moe_g16p_f2", "jl_moe_g16p_f3", "jl_moe_g16p_g1", "jl_moe_g16p_g2", "jl_moe_g16p_g3", "jl_moe_g16p_d1", "jl_moe_g16p_d2", "jl_moe_g16p_d3", "jl_moe_g16q6_c1", "jl_moe_g16q6_c2", "jl_moe_g16q6_c3", "jl_moe_g16q6_f1", "jl_moe_g16q6_f2", "jl_moe_g16q6_f3", "jl_moe_g16q6_g1", "jl_moe_g16q6_g2", "jl_moe_g16q6_g3", "jl_moe_g16q6_d1", "jl_moe_g16q6_d2", "jl_moe_g16q6_d3", "jl_moe_gemm_r64", "jl_moe_gemm_r64_planes", "jl_moe_gemm_q6k_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_mxfp4_matvec1_b1", "jl_mxfp4_matvec1_b2", "jl_mxfp4_matvec1_b3", "jl_mxfp4_scaled_prep", "jl_mxfp4_scaled_gemm", "jl_mxfp4_planes_prep", "jl_mxfp4_planes_gemm", "jl_mxfp4_matvec_planes_r64", "jl_mxfp4_matvec_planes_r32", "jl_mxfp4_matvec_planes_r16", "jl_unpack_mxfp4", "jl_sum_parts", "jl_fill_u32", "jl_probe_read", "jl_probe_empty", "jl_probe_wait", "jl_probe_mfma", "jl_probe_mfma_v5",
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_matvec_q4k_r1_pq", "jl_matvec_q4k_r1_pq_res", "jl_matvec_q8_0_r1_pq", "jl_matvec_q8_0_r1_pq_res", "jl_matvec_q6k_r1_pq", "jl_matvec_q6k_r1_pq_res", "jl_matvec_q8_0p_r1_pq", "jl_matvec_q8_0p_r1_pq_res", "jl_matvec_multi_q4k_res", "jl_matvec_multi_q4k_x4_res", "jl_matvec_multi_q4k_q_res", "jl_matvec_multi_q8_0_res", "jl_matvec_multi_q8_0_x4_res", "jl_matvec_multi_q8_0_q_res", "jl_matvec_multi_q6k_res", "jl_matvec_multi_q6k_x4_res", "jl_matvec_multi_q6k_q_res", "jl_matvec_multi_q8_0p_res", "jl_matvec_multi_q8_0p_x4_res", "jl_matvec_multi_q8_0p_q_res", "jl_matvec_q4k_r1_res", "jl_matvec_q4k_r1_x4_res", "jl_matvec_q8_0_r1_res", "jl_matvec_q8_0_r1_x4_res", "jl_matvec_q6k_r1_res", "jl_matvec_q6k_r1_x4_res", "jl_matvec_q8_0p_r1_res", "jl_matvec_q8_0p_r1_x4_res", "jl_matvec_q8_0p_r1", "jl_matvec_q8_0p_r2", "jl_matvec_q8_0p_r4", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_prep_q4k_fold", "jl_gemm_q4k_fold_wide", "jl_gemm_q4k_fold_wide4", "jl_gemm_q4k_k2", "jl_gemm_q4k_k2_planes", "jl_gemm_prep_q4k_planes", "jl_gemm_q4k_r64_planes", "jl_gemm_q4k_wide_planes", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_group2_wide", "jl_moe_quant", "jl_moe_matvec_planes_q4k", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_prep_planes", "jl_moe_gemm_q4k", "jl_moe_g16_prep", "jl_moe_g16_prep_planes", "jl_moe_g16_prep_q6k", "jl_moe_g16_c1", "jl_moe_g16_c2", "jl_moe_g16_c3", "jl_moe_g16_f1", "jl_moe_g16_f2", "jl_moe_g16_f3", "jl_moe_g16_g1", "jl_moe_g16_g2", "jl_moe_g16_g3", "jl_moe_g16_d1", "jl_moe_g16_d2", "jl_moe_g16_d3", "jl_moe_g16p_c1", "jl_moe_g16p_c2", "jl_moe_g16p_c3", "jl_moe_g16p_f1", "jl_moe_g16p_f2", "jl_moe_g16p_f3", "jl_moe_g16p_g1", "jl_moe_g16p_g2", "jl_moe_g16p_g3", "jl_moe_g16p_d1", "jl_moe_g16p_d2", "jl_moe_g16p_d3", "jl_moe_g16q6_c1", "jl_moe_g16q6_c2", "jl_moe_g16q6_c3", "jl_moe_g16q6_f1", "jl_moe_g16q6_f2", "jl_moe_g16q6_f3", "jl_moe_g16q6_g1", "jl_moe_g16q6_g2", "jl_moe_g16q6_g3", "jl_moe_g16q6_d1", "jl_moe_g16q6_d2", "jl_moe_g16q6_d3", "jl_moe_gemm_r64", "jl_moe_gemm_r64_planes", "jl_moe_gemm_q6k_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_mxfp4_matvec1_b1", "jl_mxfp4_matvec1_b2", "jl_mxfp4_matvec1_b3", "jl_mxfp4_scaled_prep", "jl_mxfp4_scaled_gemm", "jl_mxfp4_planes_prep", "jl_mxfp4_planes_gemm", "jl_mxfp4_matvec_planes_r64", "jl_mxfp4_matvec_planes_r32", "jl_mxfp4_matvec_planes_r16", "jl_unpack_mxfp4", "jl_sum_parts", "jl_fill_u32", "jl_q4k_fold_range", "jl_probe_read", "jl_probe_empty", "jl_probe_wait", "jl_probe_mfma", "jl_probe_mfma_v5",
                                       "jl_pack_weights", "jl_unpack_q4k", "jl_unpack_q6k", "jl_unpack_q8_0"};
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int rw : {16, 32, 64})
@@ -1541,6 +1562,8 @@ int jl_set_tuning(jl_ctx* c, const char* key, int value) {
     else if (!strcmp(key, "matvec.xpre")) c->tune.xpre = value;
     else if (!strcmp(key, "matvec.act_split")) c->tune.act_split = value;
     else if (!strcmp(key, "gemm.form")) c->tune.gemm_form = value;
+    else if (!strcmp(key, "gemm.fold")) c->tune.gemm_fold = value;
+    else if (!strcmp(key, "gemm.fold_waves")) c->tune.gemm_fold_waves = value;
     else if (!strcmp(key, "gemm.split")) c->tune.gemm_split = value;
     else if (!strcmp(key, "gemm.prep")) c->tune.gemm_prep = value;
     else if (!strcmp(key, "gemm.planes")) c->tune.gemm_planes = value;
@@ -1735,6 +1758,34 @@ int jl_pack_weights_dev(jl_ctx* c, int type, const void* src, int nrows, int k, 
     HIP_TRY(c, H->StreamSynchronize(st));
     HIP_TRY(c, H->Memcpy(&flag, c->flag_ws, 4, hipMemcpyDeviceToHost));
     return flag ? JL_DECLINED : JL_OK;
+}
+
+int jl_fold_admit_dev(jl_ctx* c, int type, const void* w, int nrows, int k, void* stream) {
+    if (!c) return JL_ERR_ARG;
+    if (type != JL_TYPE_Q4_K || nrows <= 0 || k <= 0 || k % 256) return JL_DECLINED;
+    if (!w) return fail(c, JL_ERR_ARG, "fold admit: null weights");
+    if ((uintptr_t)w & 3) return JL_DECLINED;
+    {
+        std::lock_guard<std::mutex> g(c->forget_mu);
+        c->fold_ok.erase((uintptr_t)w);   // whatever an earlier matrix at this address was found to be
+    }
+    HIP_TRY(c, H->SetDevice(c->device));
+    hipStream_t st = pick_stream(c, stream);
+    int rc = ws_ensure(c, &c->flag_ws, &c->flag_ws_bytes, 256);
+    if (rc != JL_OK) return rc;
+    uint32_t flag = 0;
+    HIP_TRY(c, H->Memcpy(c->flag_ws, &flag, 4, hipMemcpyHostToDevice));
+    FoldRangeArgs a;
+    a.w = (const uint8_t*)w; a.nblocks = (size_t)nrows * (size_t)(k / 256); a.flag = (uint32_t*)c->flag_ws;
+    void* params[] = {&a};
+    rc = launch(c, "jl_q4k_fold_range", (unsigned)((a.nblocks + 255) / 256), 1, 256, 0, st, params);
+    if (rc != JL_OK) return rc;
+    HIP_TRY(c, H->StreamSynchronize(st));
+    HIP_TRY(c, H->Memcpy(&flag, c->flag_ws, 4, hipMemcpyDeviceToHost));
+    if (flag) return JL_DECLINED;
+    std::lock_guard<std::mutex> g(c->forget_mu);
+    c->fold_ok[(uintptr_t)w] = {nrows, k};
+    return JL_OK;
 }
 
 int jl_unpack_weights_dev(jl_ctx* c, int type, const uint32_t* qs, const uint32_t* d, const uint32_t* sc,
@@ -2510,6 +2561,8 @@ int jl_forget(jl_ctx* c, const void* p, size_t n) {
     {
         std::lock_guard<std::mutex> g(c->forget_mu);
         c->pending_forget.emplace_back((uintptr_t)p, (uintptr_t)p + n);
+        // a device range: the matrices admitted to the folded-scale form inside it
+        c->fold_ok.erase(c->fold_ok.lower_bound((uintptr_t)p), c->fold_ok.lower_bound((uintptr_t)p + n));
     }
     if (c->mu_owner.load() != std::this_thread::get_id() && c->mu.try_lock()) {
         c->mu_owner.store(std::this_thread::get_id());

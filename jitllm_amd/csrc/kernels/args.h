@@ -357,6 +357,13 @@ struct PackArgs {
     uint32_t* flag;       // MXFP4: set to 1 when a block's exponent cannot be stored (else untouched)
 };
 
+// Scale range of a Q4_K matrix for the folded-scale GEMM (kernels/gemm_q4k_fold.h).
+struct FoldRangeArgs {
+    const uint8_t* w;     // GGUF super-blocks, 144 bytes each
+    size_t nblocks;
+    uint32_t* flag;       // set to 1 when a super-block's weights can pass the f16 range (else untouched)
+};
+
 struct UnpackArgs {
     uint8_t* dst;         // [nrows][k/256] Q4_K super-blocks
     const uint32_t* qs;

@@ -78,12 +78,15 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 // in the high nibble, jit/gpu/kernels/pack.go:210-239), so vector v = 2*ks + kg of a stage is
 // word v%4 of the stage's sub-block v/4, and its eight values pair with the activations of
 // elements 4w + (0, 2, 16, 18, 1, 3, 17, 19) of that sub-block.
-template <int NW, bool PL = false, class Load>
+// FOLD: the fragments hold f16(q * d_a), the token's scale folded into the operand (the form of
+// kernels/gemm_q4k_fold.h: one rounding to f16 more than the exact form, no sums fragment).
+template <int NW, bool PL = false, bool FOLD = false, class Load>
 __device__ __forceinline__ void gemm_prep_group(u32* lds, int sb, int grp, int ngrp, uint16_t* bqp, float* dap,
                                                 Load load) {
     constexpr int TPW = 32 / NW, FPW = 16 / NW;   // tokens and fragments per wavefront
     u32* sq = lds;                       // [32 tokens][65]: 64 words of int8 + 1 pad (bank spread)
     i32* sA = (i32*)(lds + 32 * 65);     // [32 tokens][8 sub-block sums]
+    float* sD = (float*)(lds + JL_GEMM_PREP_LDS_WORDS);   // FOLD: [32 tokens] scales
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     f32x4 v[TPW];
 #pragma unroll
@@ -101,10 +104,12 @@ __device__ __forceinline__ void gemm_prep_group(u32* lds, int sb, int grp, int n
         sq[tl * 65 + lane] = q;
         if ((lane & 7) == 0) sA[tl * 8 + (lane >> 3)] = a32;
         if (lane == 0) dap[(size_t)sb * (32 * ngrp) + grp * 32 + tl] = d;
+        if (FOLD && lane == 0) sD[tl] = d;
     }
     __syncthreads();
     const int tl = lane & 31, kg = lane >> 5;
     u32x4* dst = (u32x4*)bqp;
+    const float dtl = FOLD ? sD[tl] : 1.0f;
 #pragma unroll
     for (int i = 0; i < FPW; i++) {
         const int pi = wave * FPW + i, h = pi >> 3, ks = pi & 7;
@@ -120,12 +125,15 @@ __device__ __forceinline__ void gemm_prep_group(u32* lds, int sb, int grp, int n
             lo = sq[tl * 65 + 16 * g + c];
             hi = sq[tl * 65 + 16 * g + 8 + c];
         }
-        auto f = [](u32 w, int b) { return (_Float16)(float)(int8_t)(w >> (8 * b)); };
+        auto f = [&](u32 w, int b) {
+            const float q = (float)(int8_t)(w >> (8 * b));
+            return (_Float16)(FOLD ? q * dtl : q);
+        };
         const f16x8 o = {f(lo, 0), f(lo, 2), f(hi, 0), f(hi, 2), f(lo, 1), f(lo, 3), f(hi, 1), f(hi, 3)};
         dst[(((size_t)(2 * sb + h) * ngrp + grp) * JL_GEMM_ASTAGE_FRAGS + ks) * 64 + lane] =
             __builtin_bit_cast(u32x4, o);
     }
-    if (wave == 0) {
+    if (!FOLD && wave == 0) {
         // A = 64*A_hi + A_lo with 0 <= A_lo < 64 (arithmetic shift: floor); lanes 0-31 carry
         // the low parts, lanes 32-63 the high parts
         f16x8 o;
@@ -139,11 +147,11 @@ __device__ __forceinline__ void gemm_prep_group(u32* lds, int sb, int grp, int n
     }
 }
 
-template <int NW, bool PL = false>
+template <int NW, bool PL = false, bool FOLD = false>
 __device__ __forceinline__ void gemm_prep_q4k_body(const GemmPrepArgs& p, u32* lds) {
     const int lane = threadIdx.x & 63;
     const int sb = blockIdx.x, grp = blockIdx.y;
-    gemm_prep_group<NW, PL>(lds, sb, grp, p.tok_pad >> 5, p.bq, p.da, [&](int tl) {
+    gemm_prep_group<NW, PL, FOLD>(lds, sb, grp, p.tok_pad >> 5, p.bq, p.da, [&](int tl) {
         const int t = grp * 32 + tl;
         f32x4 v = f32x4{0.f, 0.f, 0.f, 0.f};
         if (t < p.ntok) v = ((const f32x4*)(p.x + (size_t)t * p.k + (size_t)sb * 256))[lane];

@@ -6,6 +6,7 @@
 #include "dequant.h"
 #include "gemm_q4k.h"
 #include "gemm_q4k_k2.h"
+#include "gemm_q4k_fold.h"
 #include "gemm_q6k.h"
 #include "gemm_w32.h"
 #include "matvec.h"
@@ -201,6 +202,15 @@ extern "C" __global__ __launch_bounds__(256, 3) void jl_gemm_q4k_w32(GemmArgs p)
 extern "C" __global__ __launch_bounds__(512) void jl_gemm_q4k_r128(GemmArgs p) {
     gemm_q4k_body<2>(p, jl_smem, blockIdx.x * JL_GEMM_TILE, blockIdx.y * 128);
 }
+// the folded-scale form (kernels/gemm_q4k_fold.h): its prep, block = 1024, and its wide tile,
+// grid = (tok_pad/256, ceil(nrows/128)), block = 512, dynamic LDS = JL_GEMM_FOLD_LDS_BYTES
+extern "C" __global__ __launch_bounds__(1024) void jl_gemm_prep_q4k_fold(GemmPrepArgs p) {
+    __shared__ u32 lds[JL_GEMM_PREP_LDS_WORDS + 32];
+    gemm_prep_q4k_body<16, false, true>(p, lds);
+}
+extern "C" __global__ __launch_bounds__(512) void jl_gemm_q4k_fold_wide(GemmArgs p) { gemm_q4k_fold_wide_body<false>(p, jl_smem); }
+// the same tile on four wavefronts of 64 tokens: block = 256, two workgroups a CU
+extern "C" __global__ __launch_bounds__(256, 2) void jl_gemm_q4k_fold_wide4(GemmArgs p) { gemm_q4k_fold_wide4_body(p, jl_smem); }
 extern "C" __global__ __launch_bounds__(512) void jl_gemm_q4k_wide(GemmArgs p) {
     gemm_split_slice(p);
     gemm_q4k_wide_body<false>(p, jl_smem);
@@ -409,6 +419,17 @@ JL_MX_FEW_KERNEL(1) JL_MX_FEW_KERNEL(2) JL_MX_FEW_KERNEL(3) JL_MX_FEW_KERNEL(4)
 
 // n words of `value`: the selection and weight tables of a dense block run as a mixture of one
 // expert (a kernel, not a memset, so that a caller may capture it).  grid = ceil(n / 256), block = 256
+// A Q4_K weight is d * sc * q - dmin * m with sc, m <= 63 and q <= 15: a super-block whose
+// |d| * 945 + |dmin| * 63 passes the largest f16 cannot be folded (a NaN or infinite scale
+// fails the comparison and is flagged too).  grid = ceil(nblocks/256), block = 256.
+extern "C" __global__ __launch_bounds__(256) void jl_q4k_fold_range(FoldRangeArgs a) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= a.nblocks) return;
+    const u32 h = *(const u32*)(a.w + i * 144);
+    const float d = fabsf(half_bits_to_f32((uint16_t)(h & 0xFFFF))), dmin = fabsf(half_bits_to_f32((uint16_t)(h >> 16)));
+    if (!(d * 945.f + dmin * 63.f <= 65504.f)) atomicOr(a.flag, 1u);
+}
+
 extern "C" __global__ __launch_bounds__(256) void jl_fill_u32(u32* __restrict__ dst, size_t n, u32 value) {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (i < n) dst[i] = value;

@@ -212,6 +212,11 @@ class Device:
         return self._served(self._l.jl_pack_weights_dev(self._ctx, t, _ptr(src), nrows, k, _ptr(qs), _ptr(d),
                                                         _opt(sc), stream), "jl_pack_weights_dev")
 
+    def fold_admit_dev(self, t, w, nrows, k, stream=None):
+        """Admits a Q4_K matrix to the folded-scale GEMM form ("gemm.fold" = 1); False when its
+        scales can pass the f16 range."""
+        return self._served(self._l.jl_fold_admit_dev(self._ctx, t, _ptr(w), nrows, k, stream), "jl_fold_admit_dev")
+
     def unpack_weights_dev(self, t, p, nrows, k, dst, stream=None):
         return self._served(self._l.jl_unpack_weights_dev(self._ctx, t, _ptr(p.qs), _ptr(p.d), _opt(p.sc),
                                                           p.row, p.stride, nrows, k, _ptr(dst), stream),

@@ -173,3 +173,21 @@ def test_block_seam_argument_checks_without_a_gpu():
     assert b"not prepared" in lib.jl_last_error(ctx)
     assert lib.jl_release_layers(ctx, 0, 100) == _lib.OK
     lib.jl_ctx_destroy(ctx)
+
+
+def test_fold_admission_argument_checks_without_a_gpu():
+    """jl_fold_admit_dev on a context bound to no device: what the folded-scale GEMM form does
+    not serve is a decline, a null matrix an error, and a good request fails at the device."""
+    import ctypes as C
+    lib = _lib.load()
+    ctx = C.c_void_p()
+    opts = _lib.Options(-1, 32, None)
+    assert lib.jl_ctx_create(C.byref(ctx), C.byref(opts)) == _lib.OK and ctx.value
+    w = np.zeros(4 * 144, np.uint8)
+    assert lib.jl_fold_admit_dev(ctx, quant.Q8_0, w.ctypes.data, 4, 256, None) == _lib.DECLINED
+    assert lib.jl_fold_admit_dev(ctx, quant.Q4_K, w.ctypes.data, 4, 96, None) == _lib.DECLINED
+    assert lib.jl_fold_admit_dev(ctx, quant.Q4_K, w.ctypes.data + 1, 4, 256, None) == _lib.DECLINED
+    assert lib.jl_fold_admit_dev(ctx, quant.Q4_K, None, 4, 256, None) < 0
+    assert lib.jl_fold_admit_dev(ctx, quant.Q4_K, w.ctypes.data, 4, 256, None) < 0
+    assert lib.jl_set_tuning(ctx, b"gemm.fold", 1) == _lib.OK and lib.jl_set_tuning(ctx, b"gemm.fold_waves", 8) == _lib.OK
+    lib.jl_ctx_destroy(ctx)
