@@ -540,7 +540,10 @@ template <> struct SlotTraits<JL_Q6_K> {
 // a second register set -- measured slower for every type but Q4_K, where they tie: more loads
 // in flight per wavefront do not help a kernel that is not waiting on latency.  Kept behind a
 // run-time switch it also cost the plain loop, so it is gone.  So did requesting all four chunks
-// of a long row before the activation is staged: Q6_K 4096 x 14336 13.4 -> 16.3 us.)
+// of a long row before the activation is staged: Q6_K 4096 x 14336 13.4 -> 16.3 us, and 13.3 ->
+// 14.7 with the loads' issue order pinned and the waits checked in the assembly (15, 10, 5, 0
+// loads left in flight before the four dot products): a CU returns its loads in the order they
+// were issued, so the last wavefront's first chunk arrives behind the first wavefront's last.)
 // store(row, total) receives a finished row in lane 63.
 template <int TYPE, int RPW, class Store>
 __device__ __forceinline__ void matvec_rows(const uint8_t* w0, int row_bytes, const ActLds& A, int nrows, int r0,
