@@ -800,14 +800,17 @@ def ceiling_section(dev, gate_, vendor_gemm=False):
 
 def vendor_gemm_section():
     """A yardstick, not a part of the path: the vendor library's plain f16 GEMM (torch.matmul, which
-    runs hipBLASLt) at the prefill GEMM's shapes, its weights ALREADY f16 in memory -- no activation
+    runs hipBLASLt) at the prefill GEMM's shapes and the MXFP4 section's, its weights ALREADY f16 / bf16 in memory -- no activation
     quantizer, no dequantization, none of the exact integer arithmetic.  What a tuned kernel reaches
     on this machine at these shapes when it has none of that to do."""
     import torch
     out = {}
-    for ntok, nrows in ((512, 4096), (2048, 4096), (512, 14336), (2048, 14336)):
-        a = torch.randn(ntok, 4096, device="cuda", dtype=torch.float16)
-        b = torch.randn(nrows, 4096, device="cuda", dtype=torch.float16)
+    # the Q4_K prefill shapes in f16, then the MXFP4 section's 2880 x 2880 in bf16
+    for ntok, k, nrows, dt in ((512, 4096, 4096, torch.float16), (2048, 4096, 4096, torch.float16),
+                               (512, 4096, 14336, torch.float16), (2048, 4096, 14336, torch.float16),
+                               (64, 2880, 2880, torch.bfloat16), (1024, 2880, 2880, torch.bfloat16)):
+        a = torch.randn(ntok, k, device="cuda", dtype=dt)
+        b = torch.randn(nrows, k, device="cuda", dtype=dt)
         for _ in range(5):
             c = a @ b.t()
         torch.cuda.synchronize()
@@ -821,9 +824,10 @@ def vendor_gemm_section():
             e1.synchronize()
             windows.append(e0.elapsed_time(e1) / 20)
         ms = sorted(windows)[len(windows) // 2]
-        tf = 2.0 * nrows * 4096 * ntok / (ms * 1e-3) / 1e12
-        out[f"{ntok}x4096->{nrows}"] = {"us_per_step": round(ms * 1e3, 1), "TFLOP/s": round(tf, 1),
-                                       "frac_of_f16_mfma_peak": round(tf / MFMA_F16_PEAK_TFLOPS, 4)}
+        tf = 2.0 * nrows * k * ntok / (ms * 1e-3) / 1e12
+        out[f"{ntok}x{k}->{nrows} {str(dt).split('.')[-1]}"] = {
+            "us_per_step": round(ms * 1e3, 1), "TFLOP/s": round(tf, 1),
+            "frac_of_f16_mfma_peak": round(tf / MFMA_F16_PEAK_TFLOPS, 4)}
         del a, b, c
     return out
 
