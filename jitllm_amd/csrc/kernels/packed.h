@@ -490,6 +490,10 @@ __device__ __forceinline__ void pk_stage_x(const PackedMatVecArgs& p, int c, int
 // jit/gpu/kernels/elem.go:252-267): every workgroup forms the row's sum of squares itself,
 // in f64, before anything else; k floats from L2 are cheaper than a launch.  The norm's
 // weights ride in the gate partner's registers (p.x2), so NORM implies the two-operand load.
+// (The first chunk's weights requested before the reduction instead of after it measured slower
+// both ways it was tried, us for the gated block over planes: 44.7 -> 54.4 with __syncthreads() in
+// the reduction, whose fence waits for every load in flight; 45.0 -> 46.7 with barriers that order
+// LDS only: the activation's quantization then no longer runs under the weights' way from memory.)
 template <int TYPE, int RW, int XPRE, bool FUSED, bool GATED = false, bool NORM = false>
 __device__ __forceinline__ void packed_matvec_body(const PackedMatVecArgs& p, uint8_t* smem) {
     static_assert(!NORM || (FUSED && GATED), "the norm's weights ride in the second operand");
