@@ -285,6 +285,37 @@ int jl_matvec_packed_multi_dev(jl_ctx *ctx, float *const *outs, int type, const 
                                float alpha, const float *resid_gate, const float *norm_w, float norm_eps,
                                float *norm_out, int nrows, int k, int m, void *stream);
 
+/* JIT.MatVecPackedMulti / MatVecPackedGather / MatVecPackedGatherAct as the reference's callers
+ * have them, over HOST memory (engine/nn/packedmulti.go:24,84,93): m matrices of one type and
+ * shape, matrix j's planes qs[j], d[j], sc[j] (sc, or an entry of it, may be null for Q8_0) read
+ * from row row0[j] of a buffer of `stride` rows, outs[j] receiving nrows floats.  xstride 0 is
+ * Multi (every matrix reads x[0:k]); xstride >= k is Gather (matrix j reads x[j*xstride :
+ * j*xstride+k]); up, when given, is GatherAct with act = JL_ACT_SILU (matrix j reads
+ * silu(x_j) * up_j; another act: JL_DECLINED).  The planes are uploaded on first use and stay
+ * resident, keyed on their qs pointer, until jl_forget over it, as for jl_matvec_packed.  One
+ * launch per sixteen matrices; returns after the results are in outs.  m < 2 is declined, as the
+ * reference declines it ("one matrix is not a batch").  Unlike the reference's GatherAct, which
+ * forms the gated product in place in x, x is left as it was. */
+#define JL_ACT_SILU 0   /* kernels.ActSiLU, jit/gpu/kernels/actkind.go:14 */
+int jl_matvec_packed_multi(jl_ctx *ctx, float *const *outs, int type, const uint32_t *const *qs,
+                           const uint32_t *const *d, const uint32_t *const *sc, const int *row0, int stride,
+                           const float *x, size_t xstride, const float *up, int act, int nrows, int k,
+                           int m);
+
+/* JIT.MatVecPackedGroup over HOST memory (engine/nn/packedgroup.go:18-51, MVGroup): n <=
+ * JL_MAX_GROUP packed matvecs that read one activation x[0:k] -- a block's q, k and v, its gate
+ * and up, or one projection -- matrix i of type types[i] with rows[i] rows from row row[i] of
+ * planes holding stride[i] rows (0: rows[i], as MVGroup's Packed.Stride).  act_up, when given,
+ * makes the activation silu(x) * act_up (act = JL_ACT_SILU; x is left as it was, MVGroup.ActUp);
+ * resid, when given, takes matrix 0's rows as they are made, resid[r] += alpha * outs[0][r]
+ * (MVGroup.Resid / Alpha).  Nothing runs unless every matrix can be served (JL_DECLINED
+ * otherwise), as the reference returns false having run nothing.  Matrices of one type and row
+ * count that follow one another share a launch. */
+int jl_matvec_packed_group(jl_ctx *ctx, int n, float *const *outs, const int *types,
+                           const uint32_t *const *qs, const uint32_t *const *d, const uint32_t *const *sc,
+                           const int *row, const int *stride, const int *rows, const float *x, int k,
+                           const float *act_up, int act, float *resid, float alpha);
+
 /* JIT.MatMulPacked / MatMul semantics on resident operands (engine/nn/packedmm.go:23,
  * matmul.go:27): x [ntok][k] f32 -> out [ntok][nrows], every token quantized on
  * its own.  Q4_K with the 256 window runs the matrix-core GEMM (quantize-and-

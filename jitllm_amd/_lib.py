@@ -18,6 +18,8 @@ class Options(C.Structure):
 
 
 _vp, _sz, _int = C.c_void_p, C.c_size_t, C.c_int
+ACT_SILU = 0   # kernels.ActSiLU
+MAX_GROUP = 4
 
 MAX_GROUP = 4
 
@@ -78,6 +80,11 @@ SIGNATURES = {
     "jl_matvec_multi_dev": (_int, [_vp, C.POINTER(_vp), _int, C.POINTER(_vp), _vp, _int, _int, _int, _vp]),
     "jl_matvec_gather_dev": (_int, [_vp, C.POINTER(_vp), _int, C.POINTER(_vp), _vp, _sz, _vp, _int, _int, _int,
                                     _vp]),
+    "jl_matvec_packed_multi": (_int, [_vp, C.POINTER(_vp), _int, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp),
+                                      C.POINTER(C.c_int), _int, _vp, _sz, _vp, _int, _int, _int, _int]),
+    "jl_matvec_packed_group": (_int, [_vp, _int, C.POINTER(_vp), C.POINTER(C.c_int), C.POINTER(_vp), C.POINTER(_vp),
+                                      C.POINTER(_vp), C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_int), _vp,
+                                      _int, _vp, _int, _vp, C.c_float]),
     "jl_matvec_packed_multi_dev": (_int, [_vp, _vp, _int, _vp, _vp, _vp, C.POINTER(C.c_int), _int, _vp, C.c_size_t,
                                           _vp, _vp, C.c_float, _vp, _vp, C.c_float, _vp, _int, _int, _int, _vp]),
     "jl_matmul_dev": (_int, [_vp, _vp, _int, _vp, _vp, _int, _int, _int, _vp]),

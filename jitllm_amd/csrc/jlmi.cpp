@@ -2493,9 +2493,166 @@ int jl_matmul(jl_ctx* c, float* out, int type, const void* w, size_t wbytes, con
     return JL_OK;
 }
 
+namespace {
+// The three planes of a matrix in host memory as ONE device allocation keyed on the QS pointer
+// (uploaded on first use, jl_forget over the QS pointer releases it).  Called with c->mu held.
+int resident_planes(jl_ctx* c, int type, const PlaneRef& host, int k, PlaneRef* pl) {
+    size_t nq, nd, nsc;
+    if (!packed_words(type, (size_t)host.stride, k, &nq, &nd, &nsc)) return JL_DECLINED;
+    auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
+    const size_t o_d = up(nq * 4), o_sc = o_d + up(nd * 4), total = o_sc + up(nsc * 4);
+    void* dev = nullptr;
+    auto it = c->resident.find(host.qs);
+    if (it != c->resident.end() && it->second.bytes == total) {
+        dev = it->second.dev;
+    } else {
+        if (it != c->resident.end()) {
+            HIP_TRY(c, H->Free(it->second.dev));
+            c->resident.erase(it);
+        }
+        HIP_TRY(c, H->Malloc(&dev, total));
+        hipError_t e = H->Memcpy(dev, host.qs, nq * 4, hipMemcpyHostToDevice);
+        if (e == hipSuccess) e = H->Memcpy((char*)dev + o_d, host.d, nd * 4, hipMemcpyHostToDevice);
+        if (e == hipSuccess && nsc) e = H->Memcpy((char*)dev + o_sc, host.sc, nsc * 4, hipMemcpyHostToDevice);
+        if (e != hipSuccess) {
+            (void)H->Free(dev);
+            return fail(c, JL_ERR_HIP, "plane upload: %s", H->GetErrorString(e));
+        }
+        c->resident[host.qs] = Resident{dev, total};
+    }
+    *pl = PlaneRef{(const uint32_t*)dev, (const uint32_t*)((char*)dev + o_d), (const uint32_t*)((char*)dev + o_sc),
+                   host.row, host.stride};
+    return JL_OK;
+}
+
+// Host floats -> the staging buffer at a float offset (the buffer is already large enough).
+int stage_in(jl_ctx* c, size_t off, const float* src, size_t n) {
+    HIP_TRY(c, H->MemcpyAsync((float*)c->stage_x + off, src, n * 4, hipMemcpyHostToDevice, c->stream));
+    return JL_OK;
+}
+size_t up64(size_t n) { return (n + 63) & ~(size_t)63; }   // floats: keeps every staged vector 256-byte aligned
+}  // namespace
+
 int jl_matvec_packed(jl_ctx* c, float* out, int type, const uint32_t* qs, const uint32_t* d,
                      const uint32_t* sc, int row, int stride, const float* x, int nrows, int k) {
     return jl_matmul_packed(c, out, type, qs, d, sc, row, stride, x, nrows, k, 1);
+}
+
+int jl_matvec_packed_multi(jl_ctx* c, float* const* outs, int type, const uint32_t* const* qs,
+                           const uint32_t* const* d, const uint32_t* const* sc, const int* row0, int stride,
+                           const float* x, size_t xstride, const float* up, int act, int nrows, int k, int m) {
+    if (!c) return JL_ERR_ARG;
+    CtxLock lock(c);
+    drain_forget(c);
+    // one matrix is not a batch (packedmulti.go:31-33, 109): jl_matvec_packed serves it
+    if (m < 2 || nrows <= 0 || k <= 0 || (xstride != 0 && xstride < (size_t)k)) return JL_DECLINED;
+    if (up && act != JL_ACT_SILU) return JL_DECLINED;   // the one gated activation the kernels bake in
+    if (!outs || !qs || !d || !row0 || !x) return fail(c, JL_ERR_ARG, "packed multi: null operand");
+    if (up && xstride == 0) return fail(c, JL_ERR_ARG, "packed multi: a gated activation needs one activation a matrix");
+    if (c->no_device) return fail(c, JL_ERR_HIP, "this context is bound to no device");
+    const TypeInfo* ti = nullptr;
+    for (int j = 0; j < m; j++) {
+        if (!outs[j] || !qs[j] || !d[j]) return fail(c, JL_ERR_ARG, "packed multi: null operand of matrix %d", j);
+        const PlaneRef host = {qs[j], d[j], sc ? sc[j] : nullptr, row0[j], stride};
+        int rc = packed_check(c, type, host, nrows, k, &ti);
+        if (rc != JL_OK) return rc;
+    }
+    HIP_TRY(c, H->SetDevice(c->device));
+    std::vector<PlaneRef> pls((size_t)m);
+    for (int j = 0; j < m; j++) {
+        const PlaneRef host = {qs[j], d[j], sc ? sc[j] : nullptr, row0[j], stride};
+        int rc = resident_planes(c, type, host, k, &pls[(size_t)j]);
+        if (rc != JL_OK) return rc;
+    }
+    const size_t nx = xstride ? (size_t)(m - 1) * xstride + (size_t)k : (size_t)k, o_up = up64(nx);
+    int rc = ensure_stage(c, &c->stage_x, &c->stage_x_bytes, (o_up + (up ? nx : 0)) * 4);
+    if (rc != JL_OK) return rc;
+    const size_t orow = up64((size_t)nrows);
+    if ((rc = ensure_stage(c, &c->stage_out, &c->stage_out_bytes, (size_t)m * orow * 4)) != JL_OK) return rc;
+    if ((rc = stage_in(c, 0, x, nx)) != JL_OK) return rc;
+    if (up && (rc = stage_in(c, o_up, up, nx)) != JL_OK) return rc;
+    const float* xd = (const float*)c->stage_x;
+    const float* ud = up ? xd + o_up : nullptr;
+    for (int j0 = 0; j0 < m; j0 += JL_MAX_MULTI) {   // sixteen matrices a launch
+        const int n = std::min(m - j0, (int)JL_MAX_MULTI);
+        float* od[JL_MAX_MULTI];
+        for (int j = 0; j < n; j++) od[j] = (float*)c->stage_out + (size_t)(j0 + j) * orow;
+        rc = packed_matvec_multi_launch(c, type, n, od, &pls[(size_t)j0], xd + (size_t)j0 * xstride, xstride,
+                                        ud ? ud + (size_t)j0 * xstride : nullptr, nullptr, 0.f, nullptr, nullptr, 0.f,
+                                        nullptr, nrows, k, c->stream);
+        if (rc != JL_OK) {
+            (void)H->StreamSynchronize(c->stream);
+            return rc;
+        }
+    }
+    for (int j = 0; j < m; j++)
+        HIP_TRY(c, H->MemcpyAsync(outs[j], (float*)c->stage_out + (size_t)j * orow, (size_t)nrows * 4,
+                                  hipMemcpyDeviceToHost, c->stream));
+    HIP_TRY(c, H->StreamSynchronize(c->stream));
+    return JL_OK;
+}
+
+int jl_matvec_packed_group(jl_ctx* c, int n, float* const* outs, const int* types, const uint32_t* const* qs,
+                           const uint32_t* const* d, const uint32_t* const* sc, const int* row, const int* stride,
+                           const int* rows, const float* x, int k, const float* act_up, int act, float* resid,
+                           float alpha) {
+    if (!c) return JL_ERR_ARG;
+    CtxLock lock(c);
+    drain_forget(c);
+    if (n < 1 || n > JL_MAX_GROUP || k <= 0) return JL_DECLINED;   // MaxGroup, packedgroup.go:12
+    if (act_up && act != JL_ACT_SILU) return JL_DECLINED;
+    if (!outs || !types || !qs || !d || !row || !stride || !rows || !x) return fail(c, JL_ERR_ARG, "packed group: null operand");
+    if (c->no_device) return fail(c, JL_ERR_HIP, "this context is bound to no device");
+    // nothing runs unless every matrix can (packedgroup.go:47-50)
+    for (int i = 0; i < n; i++) {
+        if (!outs[i] || !qs[i] || !d[i]) return fail(c, JL_ERR_ARG, "packed group: null operand of matrix %d", i);
+        if (rows[i] <= 0) return JL_DECLINED;
+        const TypeInfo* ti = nullptr;
+        const PlaneRef host = {qs[i], d[i], sc ? sc[i] : nullptr, row[i], stride[i] ? stride[i] : rows[i]};
+        int rc = packed_check(c, types[i], host, rows[i], k, &ti);
+        if (rc != JL_OK) return rc;
+    }
+    HIP_TRY(c, H->SetDevice(c->device));
+    PlaneRef pls[JL_MAX_GROUP];
+    for (int i = 0; i < n; i++) {
+        const PlaneRef host = {qs[i], d[i], sc ? sc[i] : nullptr, row[i], stride[i] ? stride[i] : rows[i]};
+        int rc = resident_planes(c, types[i], host, k, &pls[i]);
+        if (rc != JL_OK) return rc;
+    }
+    // staged: x, the gate's partner, the residual (matrix 0's rows)
+    const size_t o_up = up64((size_t)k), o_res = o_up + (act_up ? up64((size_t)k) : 0);
+    int rc = ensure_stage(c, &c->stage_x, &c->stage_x_bytes, (o_res + (resid ? up64((size_t)rows[0]) : 0)) * 4);
+    if (rc != JL_OK) return rc;
+    size_t o_out[JL_MAX_GROUP], total = 0;
+    for (int i = 0; i < n; i++) { o_out[i] = total; total += up64((size_t)rows[i]); }
+    if ((rc = ensure_stage(c, &c->stage_out, &c->stage_out_bytes, total * 4)) != JL_OK) return rc;
+    if ((rc = stage_in(c, 0, x, (size_t)k)) != JL_OK) return rc;
+    if (act_up && (rc = stage_in(c, o_up, act_up, (size_t)k)) != JL_OK) return rc;
+    if (resid && (rc = stage_in(c, o_res, resid, (size_t)rows[0])) != JL_OK) return rc;
+    const float* xd = (const float*)c->stage_x;
+    const float* ud = act_up ? xd + o_up : nullptr;
+    float* rd = resid ? (float*)c->stage_x + o_res : nullptr;
+    // matrices of one type and row count that follow one another share a launch (a block's gate
+    // and up); the residual rides on matrix 0 (MVGroup.Resid, packedgroup.go:32-36)
+    for (int i = 0; i < n;) {
+        int e = i + 1;
+        while (e < n && types[e] == types[i] && rows[e] == rows[i] && pls[e].stride == pls[i].stride) e++;
+        float* od[JL_MAX_GROUP];
+        for (int j = i; j < e; j++) od[j - i] = (float*)c->stage_out + o_out[j];
+        rc = packed_matvec_multi_launch(c, types[i], e - i, od, &pls[i], xd, 0, ud, i == 0 ? rd : nullptr, alpha, nullptr,
+                                        nullptr, 0.f, nullptr, rows[i], k, c->stream);
+        if (rc != JL_OK) {
+            (void)H->StreamSynchronize(c->stream);
+            return rc;
+        }
+        i = e;
+    }
+    for (int i = 0; i < n; i++)
+        HIP_TRY(c, H->MemcpyAsync(outs[i], (float*)c->stage_out + o_out[i], (size_t)rows[i] * 4, hipMemcpyDeviceToHost,
+                                  c->stream));
+    if (resid) HIP_TRY(c, H->MemcpyAsync(resid, rd, (size_t)rows[0] * 4, hipMemcpyDeviceToHost, c->stream));
+    HIP_TRY(c, H->StreamSynchronize(c->stream));
+    return JL_OK;
 }
 
 int jl_matmul_packed(jl_ctx* c, float* out, int type, const uint32_t* qs, const uint32_t* d,
@@ -2509,33 +2666,9 @@ int jl_matmul_packed(jl_ctx* c, float* out, int type, const uint32_t* qs, const 
     int rc = packed_check(c, type, host, nrows, k, &ti);
     if (rc != JL_OK) return rc;
     if (!out || !x || ntok <= 0) return fail(c, JL_ERR_ARG, "packed matmul: bad operand");
-    size_t nq, nd, nsc;
-    if (!packed_words(type, (size_t)stride, k, &nq, &nd, &nsc)) return JL_DECLINED;
     HIP_TRY(c, H->SetDevice(c->device));
-    // the three planes live in one device allocation keyed on the QS pointer
-    auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
-    const size_t o_d = up(nq * 4), o_sc = o_d + up(nd * 4), total = o_sc + up(nsc * 4);
-    void* dev = nullptr;
-    auto it = c->resident.find(qs);
-    if (it != c->resident.end() && it->second.bytes == total) {
-        dev = it->second.dev;
-    } else {
-        if (it != c->resident.end()) {
-            HIP_TRY(c, H->Free(it->second.dev));
-            c->resident.erase(it);
-        }
-        HIP_TRY(c, H->Malloc(&dev, total));
-        hipError_t e = H->Memcpy(dev, qs, nq * 4, hipMemcpyHostToDevice);
-        if (e == hipSuccess) e = H->Memcpy((char*)dev + o_d, d, nd * 4, hipMemcpyHostToDevice);
-        if (e == hipSuccess && nsc) e = H->Memcpy((char*)dev + o_sc, sc, nsc * 4, hipMemcpyHostToDevice);
-        if (e != hipSuccess) {
-            (void)H->Free(dev);
-            return fail(c, JL_ERR_HIP, "plane upload: %s", H->GetErrorString(e));
-        }
-        c->resident[qs] = Resident{dev, total};
-    }
-    const PlaneRef pl = {(const uint32_t*)dev, (const uint32_t*)((char*)dev + o_d),
-                         (const uint32_t*)((char*)dev + o_sc), row, stride};
+    PlaneRef pl;
+    if ((rc = resident_planes(c, type, host, k, &pl)) != JL_OK) return rc;
     size_t xb = (size_t)ntok * k * 4, ob = (size_t)ntok * nrows * 4;
     if ((rc = ensure_stage(c, &c->stage_x, &c->stage_x_bytes, xb)) != JL_OK) return rc;
     if ((rc = ensure_stage(c, &c->stage_out, &c->stage_out_bytes, ob)) != JL_OK) return rc;

@@ -37,6 +37,16 @@ class Packed:
         self.qs, self.d, self.sc, self.row, self.stride = qs, d, sc, row, stride
 
 
+class MVGroup:
+    """nn.MVGroup (/root/reference/engine/nn/packedgroup.go:18-37): up to MAX_GROUP packed matvecs
+    that read one activation X[:K]; Out[i] gets Rows[i] rows of P[i] (type T[i])."""
+
+    def __init__(self, Out, T, P, Rows, X, K, ActUp=None, Act=0, Resid=None, Alpha=0.0):
+        self.N = len(P)
+        self.Out, self.T, self.P, self.Rows, self.X, self.K = list(Out), list(T), list(P), list(Rows), X, K
+        self.ActUp, self.Act, self.Resid, self.Alpha = ActUp, Act, Resid, Alpha
+
+
 class Device:
     def __init__(self, device=0, act_window=32, code_object=None):
         self._l = _lib.load()
@@ -202,6 +212,50 @@ class Device:
         return self._served(self._l.jl_matmul_packed(self._ctx, _ptr(out), t, _ptr(p.qs), _ptr(p.d),
                                                      _opt(p.sc), p.row, p.stride, _ptr(x), nrows, k, ntok),
                             "jl_matmul_packed")
+
+    def _packed_multi(self, outs, t, ps, x, xstride, up, act, nrows, k, what):
+        m = len(ps)
+        assert len(outs) == m and x.dtype == np.float32 and all(o.dtype == np.float32 for o in outs)
+        po = (C.c_void_p * m)(*[_ptr(o) for o in outs])
+        pq = (C.c_void_p * m)(*[_ptr(p.qs) for p in ps])
+        pd = (C.c_void_p * m)(*[_ptr(p.d) for p in ps])
+        psc = (C.c_void_p * m)(*[_opt(p.sc) for p in ps])
+        pr = (C.c_int * m)(*[p.row for p in ps])
+        stride = ps[0].stride if m else 0
+        assert all(p.stride == stride for p in ps)
+        return self._served(self._l.jl_matvec_packed_multi(self._ctx, po, t, pq, pd, psc, pr, stride, _ptr(x), xstride,
+                                                           _opt(up), act, nrows, k, m), what)
+
+    def MatVecPackedMulti(self, outs, t, ps, x, nrows, k):
+        """JIT.MatVecPackedMulti (/root/reference/engine/nn/packedmulti.go:24): several packed matvecs
+        that share one activation; outs and ps are lists (numpy arrays, Packed)."""
+        return self._packed_multi(outs, t, ps, x, 0, None, 0, nrows, k, "jl_matvec_packed_multi")
+
+    def MatVecPackedGather(self, outs, t, ps, x, xstride, nrows, k):
+        """JIT.MatVecPackedGather (/root/reference/engine/nn/packedmulti.go:84): matrix j reads
+        x[j*xstride : j*xstride+k]."""
+        return self._packed_multi(outs, t, ps, x, xstride, None, 0, nrows, k, "jl_matvec_packed_multi")
+
+    def MatVecPackedGatherAct(self, outs, t, ps, x, up, act, xstride, nrows, k):
+        """JIT.MatVecPackedGatherAct (/root/reference/engine/nn/packedmulti.go:93): matrix j reads
+        act(x_j) * up_j; x is left as it was."""
+        assert up.dtype == np.float32
+        return self._packed_multi(outs, t, ps, x, xstride, up, act, nrows, k, "jl_matvec_packed_multi")
+
+    def MatVecPackedGroup(self, g):
+        """JIT.MatVecPackedGroup (/root/reference/engine/nn/packedgroup.go:51); g = MVGroup."""
+        n = g.N
+        po = (C.c_void_p * n)(*[_ptr(o) for o in g.Out[:n]])
+        pt = (C.c_int * n)(*g.T[:n])
+        pq = (C.c_void_p * n)(*[_ptr(p.qs) for p in g.P[:n]])
+        pd = (C.c_void_p * n)(*[_ptr(p.d) for p in g.P[:n]])
+        psc = (C.c_void_p * n)(*[_opt(p.sc) for p in g.P[:n]])
+        pr = (C.c_int * n)(*[p.row for p in g.P[:n]])
+        pst = (C.c_int * n)(*[p.stride for p in g.P[:n]])
+        prw = (C.c_int * n)(*g.Rows[:n])
+        return self._served(self._l.jl_matvec_packed_group(self._ctx, n, po, pt, pq, pd, psc, pr, pst, prw, _ptr(g.X), g.K,
+                                                           _opt(g.ActUp), g.Act, _opt(g.Resid), float(g.Alpha)),
+                            "jl_matvec_packed_group")
 
     def ForgetPacked(self, p):
         self._served(self._l.jl_forget(self._ctx, _ptr(p.qs), 4), "jl_forget")

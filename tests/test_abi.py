@@ -191,3 +191,42 @@ def test_fold_admission_argument_checks_without_a_gpu():
     assert lib.jl_fold_admit_dev(ctx, quant.Q4_K, w.ctypes.data, 4, 256, None) < 0
     assert lib.jl_set_tuning(ctx, b"gemm.fold", 1) == _lib.OK and lib.jl_set_tuning(ctx, b"gemm.fold_waves", 8) == _lib.OK
     lib.jl_ctx_destroy(ctx)
+
+
+def test_grouped_host_forms_argument_checks_without_a_gpu():
+    """jl_matvec_packed_multi / jl_matvec_packed_group on a context bound to no device: the
+    reference's declines are declines (one matrix is not a batch, an activation the kernels do not
+    bake in, more matrices than a group holds), null operands are errors, and a good call fails
+    at the device."""
+    import ctypes as C
+    lib = _lib.load()
+    ctx = C.c_void_p()
+    opts = _lib.Options(-1, 32, None)
+    assert lib.jl_ctx_create(C.byref(ctx), C.byref(opts)) == _lib.OK and ctx.value
+    nrows, k, m = 32, 256, 2
+    qs, d = np.zeros(nrows * k // 4, np.uint32), np.zeros(nrows * k // 32, np.uint32)
+    x = np.zeros(2 * k, np.float32)
+    outs = [np.zeros(nrows, np.float32) for _ in range(m)]
+    po = (C.c_void_p * m)(*[o.ctypes.data for o in outs])
+    pq = (C.c_void_p * m)(*[qs.ctypes.data] * m)
+    pd = (C.c_void_p * m)(*[d.ctypes.data] * m)
+    psc = (C.c_void_p * m)(None, None)
+    pr = (C.c_int * m)(0, 0)
+    call = lambda **kw: lib.jl_matvec_packed_multi(ctx, kw.get("outs", po), quant.Q8_0, pq, pd, psc, pr, nrows, x.ctypes.data,
+                                                   kw.get("xstride", 0), kw.get("up"), kw.get("act", 0), nrows, k, kw.get("m", m))
+    assert call(m=1) == _lib.DECLINED
+    assert call(xstride=k - 1) == _lib.DECLINED
+    assert call(xstride=k, up=x.ctypes.data, act=3) == _lib.DECLINED
+    assert call(outs=None) < 0
+    assert call(up=x.ctypes.data) < 0                      # a gated activation with one shared x
+    assert call() < 0 and b"no device" in lib.jl_last_error(ctx)
+    pt = (C.c_int * m)(quant.Q8_0, quant.Q8_0)
+    pst = (C.c_int * m)(0, 0)
+    prw = (C.c_int * m)(nrows, nrows)
+    grp = lambda n, **kw: lib.jl_matvec_packed_group(ctx, n, po, pt, pq, pd, psc, pr, pst, prw, kw.get("x", x.ctypes.data), k,
+                                                     kw.get("up"), kw.get("act", 0), None, C.c_float(0))
+    assert grp(0) == _lib.DECLINED and grp(_lib.MAX_GROUP + 1) == _lib.DECLINED
+    assert grp(2, up=x.ctypes.data, act=2) == _lib.DECLINED
+    assert grp(2, x=None) < 0
+    assert grp(2) < 0 and b"no device" in lib.jl_last_error(ctx)
+    lib.jl_ctx_destroy(ctx)

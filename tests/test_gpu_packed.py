@@ -383,6 +383,139 @@ def test_packed_host_pointer_seam(dev):
     dev.SetActWindow(32)
 
 
+@pytest.mark.parametrize("t", TYPES)
+def test_grouped_operators_over_host_planes(dev, devbuf, t):
+    """JIT.MatVecPackedMulti / Gather / GatherAct over host memory
+    (/root/reference/engine/nn/packedmulti.go:24,84,93): a bank's sheets as row ranges of one set of
+    planes, twenty matrices (two launches of at most sixteen), against the oracle and, bit for bit,
+    against the device-pointer form; what the reference declines is declined."""
+    from jitllm_amd import _lib
+    n_expert, nrows, k, window = 7, 90, 1024, _window(t)
+    experts = [4, 0, 5, 2, 6, 1, 3, 3, 0, 6, 2, 2, 5, 1, 4, 0, 6, 3, 1, 5]
+    m = len(experts)
+    dev.SetActWindow(window)
+    bank = synth.random_weights(t, n_expert * nrows, k, seed=131)
+    qs, d, sc = oracle.pack_weights(t, bank, n_expert * nrows, k)
+    sc = sc if sc is not None and sc.size else None
+    ps = [Packed(qs, d, sc, e * nrows, n_expert * nrows) for e in experts]
+    xstride = k + 64
+    xs = synth.activations(m * xstride, seed=61).reshape(m, xstride)
+    ups = synth.activations(m * xstride, seed=62).reshape(m, xstride)
+    rb = quant.row_bytes(t, k)
+    sheet = lambda e: bank[e * nrows * rb:(e + 1) * nrows * rb]
+    planes_d = _dev_planes(devbuf, qs, d, sc, stride=n_expert * nrows)
+    xd, ud = devbuf(xs), devbuf(ups)
+
+    def dev_form(js, xstride_, up):
+        outs = [devbuf(shape=(nrows,), dtype=np.float32, fill=np.float32(9e30)) for _ in js]
+        assert dev.matvec_packed_multi_dev([o.ptr for o in outs], t, [(planes_d.qs, planes_d.d, planes_d.sc)] * len(js),
+                                           [experts[j] * nrows for j in js], n_expert * nrows,
+                                           xd.ptr + js[0] * xstride_ * 4, xstride_, (ud.ptr + js[0] * xstride_ * 4) if up else None,
+                                           nrows, k)
+        dev.synchronize()
+        return [o.get() for o in outs]
+
+    x0 = xs[0].copy()
+    # Multi: one shared activation
+    outs = [np.full(nrows + 3, np.float32(7e30)) for _ in range(m)]
+    assert dev.MatVecPackedMulti(outs, t, ps, xs[0], nrows, k) is True
+    same = dev_form(list(range(16)), 0, False)
+    for j, e in enumerate(experts):
+        assert np.all(outs[j][nrows:] == np.float32(7e30)), "wrote past nrows"
+        assert nmse(outs[j][:nrows], _like_for_like(t, sheet(e), xs[0][:k], nrows, k, window)) <= 1e-10
+        if j < 16:
+            assert np.array_equal(outs[j][:nrows].view(np.uint32), same[j].view(np.uint32))
+    # Gather: an activation a matrix, at a stride
+    outs = [np.full(nrows, np.float32(7e30)) for _ in range(m)]
+    assert dev.MatVecPackedGather(outs, t, ps, xs.reshape(-1), xstride, nrows, k) is True
+    same = dev_form(list(range(16)), xstride, False) + dev_form(list(range(16, m)), xstride, False)
+    for j, e in enumerate(experts):
+        assert nmse(outs[j], _like_for_like(t, sheet(e), xs[j][:k], nrows, k, window)) <= 1e-10
+        assert np.array_equal(outs[j].view(np.uint32), same[j].view(np.uint32))
+    # GatherAct: silu(x_j) * up_j, x left as it was
+    keep = xs.copy()
+    outs = [np.full(nrows, np.float32(7e30)) for _ in range(m)]
+    assert dev.MatVecPackedGatherAct(outs, t, ps, xs.reshape(-1), ups.reshape(-1), _lib.ACT_SILU, xstride, nrows, k) is True
+    assert np.array_equal(xs, keep)
+    same = dev_form(list(range(16)), xstride, True) + dev_form(list(range(16, m)), xstride, True)
+    for j, e in enumerate(experts):
+        g = xs[j][:k].astype(np.float64)
+        h = (g / (1 + np.exp(-g)) * ups[j][:k].astype(np.float64)).astype(np.float32)
+        assert rel_l2(outs[j], _like_for_like(t, sheet(e), h, nrows, k, window)) <= 1e-3
+        assert np.array_equal(outs[j].view(np.uint32), same[j].view(np.uint32))
+    # one allocation for the bank: every matrix has the same QS pointer
+    assert dev.resident_count() >= 1
+    # declines, as the reference's: one matrix, another activation, a stride shorter than k, k off the grid
+    one = [np.zeros(nrows, np.float32)]
+    assert dev.MatVecPackedMulti(one, t, ps[:1], x0, nrows, k) is False
+    assert dev.MatVecPackedGatherAct(outs, t, ps, xs.reshape(-1), ups.reshape(-1), 1, xstride, nrows, k) is False
+    assert dev.MatVecPackedGather(outs, t, ps, xs.reshape(-1), k - 32, nrows, k) is False
+    assert dev.MatVecPackedMulti(outs, t, ps, xs[0], nrows, k - 16) is False
+    dev.ForgetPacked(ps[0])
+    dev.SetActWindow(32)
+
+
+def test_group_operator_over_host_planes(dev, devbuf):
+    """JIT.MatVecPackedGroup over host memory (/root/reference/engine/nn/packedgroup.go:18-51): a
+    block's q, k and v of different types and row counts on one activation; its gate and up (one
+    type, one shape: one launch); a down projection on silu(x) * up with the residual riding on
+    it.  Every matrix is the packed matvec of that matrix (TestGroupMatchesMatVec), bit for bit."""
+    from jitllm_amd import _lib
+    from jitllm_amd.device import MVGroup
+    k, window = 2048, 256
+    dev.SetActWindow(window)
+    specs = [(quant.Q4_K, 512), (quant.Q4_K, 128), (quant.Q6_K, 128)]
+    ws = [synth.quantized_weights(t, r, k, seed=70 + i) for i, (t, r) in enumerate(specs)]
+    packs = []
+    for (t, r), w in zip(specs, ws):
+        qs, d, sc = oracle.pack_weights(t, w, r, k)
+        packs.append(Packed(qs, d, sc if sc is not None and sc.size else None, 0, 0))   # stride 0: rows
+    x = synth.activations(k, seed=9)
+    n0 = dev.launch_count()
+    outs = [np.full(r, np.float32(7e30)) for _, r in specs]
+    g = MVGroup(outs, [t for t, _ in specs], packs, [r for _, r in specs], x, k)
+    assert dev.MatVecPackedGroup(g) is True
+    assert dev.launch_count() - n0 == 3       # three types / shapes: three launches
+    for (t, r), w, o, p in zip(specs, ws, outs, packs):
+        assert nmse(o, _like_for_like(t, w, x, r, k, window)) <= 1e-10
+        single = np.zeros(r, np.float32)
+        assert dev.MatVecPacked(single, t, Packed(p.qs, p.d, p.sc, 0, r), x, r, k) is True
+        assert np.array_equal(single.view(np.uint32), o.view(np.uint32))
+    # gate and up: one launch
+    n0 = dev.launch_count()
+    gu = [np.zeros(512, np.float32), np.zeros(512, np.float32)]
+    w2 = synth.quantized_weights(quant.Q4_K, 512, k, seed=90)
+    q2 = oracle.pack_weights(quant.Q4_K, w2, 512, k)
+    p2 = Packed(q2[0], q2[1], q2[2], 0, 512)
+    assert dev.MatVecPackedGroup(MVGroup(gu, [quant.Q4_K] * 2, [packs[0], p2], [512, 512], x, k)) is True
+    assert dev.launch_count() - n0 == 1
+    assert np.array_equal(gu[0].view(np.uint32), outs[0].view(np.uint32))
+    assert nmse(gu[1], _like_for_like(quant.Q4_K, w2, x, 512, k, window)) <= 1e-10
+    # a down projection: silu(x) * up in front, the residual on matrix 0
+    up = synth.activations(k, seed=10)
+    resid0 = synth.activations(512, seed=11)
+    resid = resid0.copy()
+    keep = x.copy()
+    y = [np.zeros(512, np.float32)]
+    assert dev.MatVecPackedGroup(MVGroup(y, [quant.Q4_K], [packs[0]], [512], x, k, ActUp=up, Act=_lib.ACT_SILU,
+                                         Resid=resid, Alpha=0.5)) is True
+    assert np.array_equal(x, keep)
+    gx = x.astype(np.float64)
+    h = (gx / (1 + np.exp(-gx)) * up.astype(np.float64)).astype(np.float32)
+    assert rel_l2(y[0], _like_for_like(quant.Q4_K, ws[0], h, 512, k, window)) <= 1e-3
+    assert np.array_equal(resid, (resid0 + (np.float32(0.5) * y[0]).astype(np.float32)).astype(np.float32))
+    # nothing runs unless every matrix can: the second matrix's type has no planes
+    before = [o.copy() for o in outs]
+    bad = MVGroup(outs, [quant.Q4_K, quant.MXFP4, quant.Q6_K], packs, [r for _, r in specs], x, k)
+    n0 = dev.launch_count()
+    assert dev.MatVecPackedGroup(bad) is False
+    assert dev.launch_count() == n0 and all(np.array_equal(a, b) for a, b in zip(before, outs))
+    assert dev.MatVecPackedGroup(MVGroup(y, [quant.Q4_K], [packs[0]], [512], x, k, ActUp=up, Act=1)) is False
+    for p in packs + [p2]:
+        dev.ForgetPacked(p)
+    dev.SetActWindow(32)
+
+
 @pytest.mark.parametrize("shape", [(130, 300, 1024, 0, 300), (512, 260, 2048, 90, 400), (256, 700, 512, 0, 700),
                                    (96, 150, 2816, 37, 200), (200, 33000, 256, 0, 33000)],
                          ids=lambda s: "x".join(map(str, s)))
