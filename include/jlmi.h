@@ -554,6 +554,14 @@ typedef struct jl_packed_bank {
     int stride;
 } jl_packed_bank;
 
+/* jl_moe_ffn_dev over HOST memory: resid [rows][n_embd] (read, accumulated, written back), the
+ * three banks as GGUF bytes (uploaded on first use and resident, each keyed on its pointer, until
+ * jl_forget over it), x [rows][n_embd], sel [rows][sel_stride] and wt [rows][k_used] as the host
+ * router made them (engine/model/moe.go:697-761).  Returns after resid is back in host memory. */
+int jl_moe_grouped(jl_ctx *ctx, float *resid, int type, const void *gate_bank, const void *up_bank,
+                   const void *down_bank, const float *x, const uint32_t *sel, int sel_stride,
+                   const float *wt, int rows, int k_used, int n_expert, int n_ffn, int n_embd);
+
 /* jl_moe_matvec_dev over banks of packed planes: the per-expert matrix-core tile reads every
  * sheet where it lies (Q4_K with the activation window of 256; anything else JL_DECLINED).
  * bank1 / out1 may be null; both banks must share one layout (sheet_bytes, stride). */

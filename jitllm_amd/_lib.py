@@ -80,6 +80,7 @@ SIGNATURES = {
     "jl_matvec_multi_dev": (_int, [_vp, C.POINTER(_vp), _int, C.POINTER(_vp), _vp, _int, _int, _int, _vp]),
     "jl_matvec_gather_dev": (_int, [_vp, C.POINTER(_vp), _int, C.POINTER(_vp), _vp, _sz, _vp, _int, _int, _int,
                                     _vp]),
+    "jl_moe_grouped": (_int, [_vp, _vp, _int, _vp, _vp, _vp, _vp, _vp, _int, _vp, _int, _int, _int, _int, _int]),
     "jl_matvec_packed_multi": (_int, [_vp, C.POINTER(_vp), _int, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp),
                                       C.POINTER(C.c_int), _int, _vp, _sz, _vp, _int, _int, _int, _int]),
     "jl_matvec_packed_group": (_int, [_vp, _int, C.POINTER(_vp), C.POINTER(C.c_int), C.POINTER(_vp), C.POINTER(_vp),

@@ -2592,6 +2592,48 @@ int jl_matvec_packed_multi(jl_ctx* c, float* const* outs, int type, const uint32
     return JL_OK;
 }
 
+int jl_moe_grouped(jl_ctx* c, float* resid, int type, const void* gate_bank, const void* up_bank,
+                   const void* down_bank, const float* x, const uint32_t* sel, int sel_stride, const float* wt,
+                   int rows, int k_used, int n_expert, int n_ffn, int n_embd) {
+    if (!c) return JL_ERR_ARG;
+    CtxLock lock(c);
+    drain_forget(c);
+    if (rows <= 0 || k_used <= 0 || n_expert <= 0 || n_ffn <= 0 || n_embd <= 0 || sel_stride < k_used)
+        return fail(c, JL_ERR_ARG, "moe grouped: bad shape");
+    if (!resid || !gate_bank || !up_bank || !down_bank || !x || !sel || !wt)
+        return fail(c, JL_ERR_ARG, "moe grouped: null operand");
+    const TypeInfo* ti = type_info(type);
+    if (!ti || n_embd % ti->block_elems || n_ffn % ti->block_elems) return JL_DECLINED;
+    if (n_expert > 1024 || k_used > 16 || n_ffn % 256 != 0 || n_embd % 256 != 0) return JL_DECLINED;
+    if (c->no_device) return fail(c, JL_ERR_HIP, "this context is bound to no device");
+    HIP_TRY(c, H->SetDevice(c->device));
+    // the three banks stay resident, each keyed on its host pointer
+    const size_t bank = (size_t)n_expert * n_ffn * (size_t)(n_embd / ti->block_elems) * ti->block_bytes;
+    void *gd = nullptr, *ud = nullptr, *dd = nullptr;
+    int rc = resident_weight(c, gate_bank, bank, &gd);
+    if (rc == JL_OK) rc = resident_weight(c, up_bank, bank, &ud);
+    if (rc == JL_OK) rc = resident_weight(c, down_bank, bank, &dd);
+    if (rc != JL_OK) return rc;
+    // staged as floats: x, resid, wt, then the selections (32-bit words as well)
+    const size_t nx = (size_t)rows * n_embd, o_res = up64(nx), o_wt = o_res + up64(nx),
+                 o_sel = o_wt + up64((size_t)rows * k_used), total = o_sel + up64((size_t)rows * sel_stride);
+    if ((rc = ensure_stage(c, &c->stage_x, &c->stage_x_bytes, total * 4)) != JL_OK) return rc;
+    if ((rc = stage_in(c, 0, x, nx)) != JL_OK) return rc;
+    if ((rc = stage_in(c, o_res, resid, nx)) != JL_OK) return rc;
+    if ((rc = stage_in(c, o_wt, wt, (size_t)rows * k_used)) != JL_OK) return rc;
+    if ((rc = stage_in(c, o_sel, (const float*)sel, (size_t)rows * sel_stride)) != JL_OK) return rc;
+    float* base = (float*)c->stage_x;
+    rc = moe_ffn(c, base + o_res, type, type, gd, ud, dd, nullptr, nullptr, nullptr, base, (const uint32_t*)(base + o_sel),
+                 sel_stride, base + o_wt, rows, k_used, n_expert, n_ffn, n_embd, c->stream);
+    if (rc != JL_OK) {
+        (void)H->StreamSynchronize(c->stream);
+        return rc;
+    }
+    HIP_TRY(c, H->MemcpyAsync(resid, base + o_res, nx * 4, hipMemcpyDeviceToHost, c->stream));
+    HIP_TRY(c, H->StreamSynchronize(c->stream));
+    return JL_OK;
+}
+
 int jl_matvec_packed_group(jl_ctx* c, int n, float* const* outs, const int* types, const uint32_t* const* qs,
                            const uint32_t* const* d, const uint32_t* const* sc, const int* row, const int* stride,
                            const int* rows, const float* x, int k, const float* act_up, int act, float* resid,

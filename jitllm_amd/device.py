@@ -257,6 +257,14 @@ class Device:
                                                            _opt(g.ActUp), g.Act, _opt(g.Resid), float(g.Alpha)),
                             "jl_matvec_packed_group")
 
+    def MoEGrouped(self, resid, t, gate_bank, up_bank, down_bank, x, sel, wt, rows, k_used, n_expert, n_ffn, n_embd):
+        """One routed feed-forward block over host memory (moeBatchFrom,
+        /root/reference/engine/model/moe.go:510-761): resid [rows][n_embd] accumulated in place."""
+        assert resid.dtype == np.float32 and x.dtype == np.float32 and wt.dtype == np.float32 and sel.dtype == np.uint32
+        return self._served(self._l.jl_moe_grouped(self._ctx, _ptr(resid), t, _ptr(gate_bank), _ptr(up_bank), _ptr(down_bank),
+                                                   _ptr(x), _ptr(sel), sel.shape[1], _ptr(wt), rows, k_used, n_expert,
+                                                   n_ffn, n_embd), "jl_moe_grouped")
+
     def ForgetPacked(self, p):
         self._served(self._l.jl_forget(self._ctx, _ptr(p.qs), 4), "jl_forget")
 

@@ -329,6 +329,36 @@ def test_moe_block_vs_oracle(dev, devbuf, shape):
     dev.SetActWindow(32)
 
 
+def test_moe_block_over_host_memory(dev, devbuf):
+    """jl_moe_grouped: the routed block with every operand in host memory (banks resident per host
+    pointer after the first call, the residual read, accumulated and written back): the oracle's
+    block, and the device-pointer call's bits."""
+    shape = (6, 8, 2, 256, 512)
+    rows, n_expert, k_used, n_ffn, n_embd = shape
+    t, window = quant.Q4_K, 256
+    dev.SetActWindow(window)
+    sel, wt, gate, up, down, x, want = _block_case(shape)
+    r0 = synth.activations(rows * n_embd, seed=41).reshape(rows, n_embd)
+    gd, ud, dd, xd, sd, wd = devbuf(gate), devbuf(up), devbuf(down), devbuf(x), devbuf(sel), devbuf(wt)
+    rd = devbuf(r0)
+    assert dev.moe_ffn_dev(rd.ptr, t, gd.ptr, ud.ptr, dd.ptr, xd.ptr, sd.ptr, k_used + 1, wd.ptr, rows, k_used, n_expert,
+                           n_ffn, n_embd)
+    dev.synchronize()
+    same = rd.get()
+    n_res = dev.resident_count()
+    for call in range(2):
+        resid = r0.copy()
+        assert dev.MoEGrouped(resid, t, gate, up, down, x, sel, wt, rows, k_used, n_expert, n_ffn, n_embd) is True
+        assert np.array_equal(resid.view(np.uint32), same.view(np.uint32))
+        assert rel_l2(resid - r0, want) <= 1e-3
+        assert dev.resident_count() == n_res + 3          # three banks, uploaded once
+    for b in (gate, up, down):
+        dev.Forget(b)
+    assert dev.resident_count() == n_res
+    assert dev.MoEGrouped(r0.copy(), quant.MXFP4, gate, up, down, x, sel, wt, rows, k_used, n_expert, n_ffn, n_embd) is False
+    dev.SetActWindow(32)
+
+
 def test_moe_block_prefill_1024_rows_vs_oracle_on_sampled_rows(dev, devbuf):
     """The Qwen3-30B-A3B block at a prefill batch, the size the benchmark times: 1024 rows routed
     top-8 over 128 experts (64 columns an expert on average: the matrix-core forms with groups of
