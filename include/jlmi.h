@@ -151,14 +151,24 @@ int jl_matvec(jl_ctx *ctx, float *out, int type, const void *w, size_t wbytes,
 
 /* nn.CopyForgetter.Forget (engine/nn/device.go:1570-1581): drop any device copy
  * keyed inside [p, p+n).  Callable from any thread, also from inside a page-in that
- * this context's own upload started: it only queues the range under a lock of its own
- * -- no HIP call, no lock that a launch or an upload holds (the reference queues the
- * range the same way when its device is busy, jit/gpu/tier/forget.go:20-40).  The
- * next host-pointer call on the context unlinks and frees the matching copies before
- * it looks its weight up; jl_ctx_destroy frees what is left. */
+ * this context's own upload started: it queues the range under a lock of its own that no
+ * launch or upload holds, and never blocks.  If the context is free at that moment the
+ * queue is applied at once (the copies are freed now); if another thread's call, or this
+ * thread's own, holds the context, the next host-pointer call applies it before it looks
+ * its weight up (the reference applies or queues the same way, jit/gpu/tier/forget.go:20-49);
+ * jl_ctx_destroy frees what is left.  A range of DEVICE addresses withdraws the matrices
+ * jl_fold_admit_dev admitted inside it. */
 int jl_forget(jl_ctx *ctx, const void *p, size_t n);
 
-/* The lock the host-pointer entry points hold for their whole synchronous run (the
+/* Threads.  The host-pointer entry points (no _dev in the name) may be called from any
+ * thread: each holds the context's lock for its whole synchronous run.  The *_dev entry
+ * points take no lock and share the context's workspaces (activation fragments, K-split
+ * slabs, the mixture block's lists, the flag word of jl_pack_weights_dev and
+ * jl_fold_admit_dev): a context's *_dev calls are made by one thread at a time, on one stream
+ * at a time, as the reference's tier makes its device calls (jit/gpu/tier/tier.go:2831-2843);
+ * give each thread that launches concurrently a context of its own.
+ *
+ * The lock the host-pointer entry points hold for their whole synchronous run (the
  * reference's tier serialises the same way, jit/gpu/tier/tier.go:2831-2843), for a
  * caller that needs several of them to run as one.  Not recursive: a host-pointer call
  * between lock and unlock on the same thread deadlocks; *_dev calls and jl_forget take
