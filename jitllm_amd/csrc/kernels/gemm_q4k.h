@@ -376,21 +376,31 @@ __device__ __forceinline__ void gemm_q4k_body(const GemmArgs& p, uint8_t* smem, 
 
     // prologue: stage 0 of the weights into LDS, stage 1 into registers; the first
     // stage's activation fragments into the ring
+    // The loads go out in the order the loop issues them -- a stage's weights, the next stage's,
+    // the activation fragments in K order, the token scale; the loop's head adds the stage after
+    // that.  The wait the compiler puts before a register's first use in the loop is the smaller
+    // of the counts on the two ways in: with stage 1's weights requested last here, every
+    // first half-stage waited for the weights its own head had just requested.
     GemmWRegs wa, wb;   // stages alternate between the two register sets
-    load_w(0, 0, wa);
+    load_w(0, 0, wb);
+    load_w(0, 1, wa);
+    __builtin_amdgcn_sched_barrier(0);
     f16x8 aring[8], aaug;
 #pragma unroll
-    for (int ks = 0; ks < 8; ks++) aring[ks] = a_frag(0, ks);
-    aaug = aring[0];
-    {
-        GemmWScale k0;
-        w_scale(wa, 0, sW, k0);
-#pragma unroll
-        for (int c = 0; c < 4; c++) gemm_w_word(wa, k0, c);
+    for (int ks = 0; ks < 8; ks++) {
+        aring[ks] = a_frag(0, ks);
+        __builtin_amdgcn_sched_barrier(0);
     }
-    load_w(0, 1, wa);
+    aaug = aring[0];
     const int da_tok = min(t0 + (tid & (JL_GEMM_TILE - 1)), p.tok_pad - 1);
     float da_reg = p.da[da_tok];
+    __builtin_amdgcn_sched_barrier(0);
+    {
+        GemmWScale k0;
+        w_scale(wb, 0, sW, k0);
+#pragma unroll
+        for (int c = 0; c < 4; c++) gemm_w_word(wb, k0, c);
+    }
     lds_barrier();
 
     // One stage.  HALF is the stage's half of its super-block; wcur holds the next
@@ -414,6 +424,10 @@ __device__ __forceinline__ void gemm_q4k_body(const GemmArgs& p, uint8_t* smem, 
         // instructions, so the vector work runs under the matrix core.
         GemmWScale wsc;
         w_scale(wcur, nhalf, wnext, wsc);
+        // (all four header words stay live to here: d and dmin are read only by the stage that
+        // writes the minimum columns, and a word nobody reads is handed out as a temporary while
+        // its load is still in flight -- writing it then waits for the load just requested)
+        asm volatile("" ::"v"(wcur.hdr));
         // matrix work: per K-step one activation fragment (already in the ring) against
         // the two row groups' weight fragments, fetched from LDS a K-step ahead; the ring
         // slot is refilled with the next stage's fragment as soon as it has been used

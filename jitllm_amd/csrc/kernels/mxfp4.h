@@ -105,7 +105,9 @@ __device__ __forceinline__ void mx_load_w(const MxGemmArgs& p, int r0, int wave,
         const uint8_t* blk = p.w + (size_t)row * p.row_bytes + (size_t)min(b, nblk - 1) * 17;
         r.e[i] = blk[0];
         r.q[i] = ld16_a1(blk + 1);
-        if (b >= nblk) r.q[i] = u32x4{0, 0, 0, 0};  // past the end of K: zero codes
+        // (a block past the end of K reads the row's last block again; the decode zeroes its codes.
+        // Zeroing them here is a select on the loaded words, and the wait for the load comes to
+        // stand right behind the load: every stage then began with a whole trip to memory)
     }
 }
 
@@ -154,28 +156,42 @@ __device__ __forceinline__ void mx_gemm_body(const MxGemmArgs& p, uint8_t* smem)
 #pragma unroll
         for (int e = 0; e < 16; e++) acc[j][e] = 0.f;
 
-    auto decode_half = [&](const MxWRegs& r, int i, int h, __bf16* buf) {
+    const int nblk = p.k / 32;
+    auto decode_half = [&](const MxWRegs& r, int i, int h, __bf16* buf, int stg) {
         // block i of the thread's two, words (2h, 2h+1): elements 8h.. and 16+8h..
+        // (stg: the stage r holds; its blocks past the end of K decode as zero codes)
+        const bool past = stg * 8 + (lane & 7) >= nblk;
         u32x4 lo, hi;
-        mx_dequant_half(r.q[i][2 * h], r.q[i][2 * h + 1], mx_scale(r.e[i]), lo, hi);
+        mx_dequant_half(past ? 0u : r.q[i][2 * h], past ? 0u : r.q[i][2 * h + 1], mx_scale(r.e[i]), lo, hi);
         __bf16* dst = buf + wdst + 8 * i * JL_MX_STRIDE + 8 * h;
         *(u32x4*)dst = lo;
         *(u32x4*)(dst + 16) = hi;
     };
 
+    // The loads before the loop go out in the loop's own order (a stage's weights, the next
+    // stage's, then the activation fragments; the loop's head adds the stage after that): the
+    // wait the compiler puts before a register's first use in the loop is the smaller of the
+    // counts on the two ways in, and with the second stage's weights requested last here it made
+    // every other stage wait for the weights its own head had just requested.
     MxWRegs wa, wb;
     bf16x8 aring[8];
     const int last = max(s_hi - 1, s_lo);
-    if (decodes) mx_load_w(p, r0, wave, lane, s_lo, wa);
+    if (decodes) {
+        mx_load_w(p, r0, wave, lane, s_lo, wb);
+        mx_load_w(p, r0, wave, lane, min(s_lo + 1, last), wa);
+    }
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int ks2 = 0; ks2 < 8; ks2++) aring[ks2] = a_frag(s_lo, ks2);
+    for (int ks2 = 0; ks2 < 8; ks2++) {
+        aring[ks2] = a_frag(s_lo, ks2);
+        __builtin_amdgcn_sched_barrier(0);   // in K order, as the loop requests them
+    }
     if (decodes) {
 #pragma unroll
         for (int i = 0; i < 2; i++) {
-            decode_half(wa, i, 0, sW);
-            decode_half(wa, i, 1, sW);
+            decode_half(wb, i, 0, sW, s_lo);
+            decode_half(wb, i, 1, sW, s_lo);
         }
-        mx_load_w(p, r0, wave, lane, min(s_lo + 1, last), wa);
     }
     mx_lds_barrier();
 
@@ -203,7 +219,7 @@ __device__ __forceinline__ void mx_gemm_body(const MxGemmArgs& p, uint8_t* smem)
             if (j == NJ - 1) {
                 aring[ks2] = a_frag(nst, ks2);
                 // half a block of the next stage's weights in every second K-step
-                if (decodes && (ks2 & 1)) decode_half(wcur, ks2 >> 2, (ks2 >> 1) & 1, wnext);
+                if (decodes && (ks2 & 1)) decode_half(wcur, ks2 >> 2, (ks2 >> 1) & 1, wnext, nst);
             }
             __builtin_amdgcn_sched_barrier(0);
         }
