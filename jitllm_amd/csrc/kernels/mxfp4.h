@@ -545,23 +545,25 @@ __device__ __forceinline__ void mx_planes_gemm_body(const MxPlanesGemmArgs& p, f
 #pragma unroll
         for (int s = 0; s < 2; s++) qoff[j][s] = (u32)(2 * s + kg) * (u32)p.stride + row;
     }
-    struct WOps { u32 q[2][4]; u32 d[2][2]; };     // [row tile][matrix K-step], [row tile][block]
+    // [row tile][matrix K-step], [row tile][block]; past: the K-step's second block lies beyond K
+    // (its codes are zeroed where they are used: a select on the loaded words here would put the
+    // wait for the load right behind the load)
+    struct WOps { u32 q[2][4]; u32 d[2][2]; bool past; };
     struct AOps { u32x4 a[2][4]; };                // [token tile][matrix K-step]
     auto load_w = [&](int ks, WOps& o) {
         ks = min(ks, nks - 1);
+        o.past = 2 * ks + 1 >= nblk;       // the second block of a last, half K-step (uniform)
 #pragma unroll
         for (int bi = 0; bi < 2; bi++) {
             const int b = 2 * ks + bi;
-            const bool past = b >= nblk;   // the second block of a last, half K-step (uniform)
-            const size_t bc = (size_t)(past ? nblk - 1 : b);
+            const size_t bc = (size_t)min(b, nblk - 1);
             const u32* qb = p.qs + bc * 4 * n;
             const u32* db = p.d + bc * dwords;
 #pragma unroll
             for (int j = 0; j < 2; j++) {
 #pragma unroll
                 for (int s = 0; s < 2; s++) {
-                    const u32 v = qb[qoff[j][s]];
-                    o.q[j][2 * bi + s] = past ? 0u : v;
+                    o.q[j][2 * bi + s] = qb[qoff[j][s]];
                 }
                 o.d[j][bi] = db[doff[j]];
             }
@@ -590,7 +592,7 @@ __device__ __forceinline__ void mx_planes_gemm_body(const MxPlanesGemmArgs& p, f
 #pragma unroll
             for (int j = 0; j < 2; j++) {
                 const float scale = mx_scale((uint8_t)(((wo.d[j][s4 >> 1] >> sh[j]) & 0xFF) + 1));
-                const u32 q = wo.q[j][s4];
+                const u32 q = (s4 >> 1) && wo.past ? 0u : wo.q[j][s4];
                 u32x4 wb;
                 wb.x = __builtin_bit_cast(u32, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(q, scale, 0));
                 wb.y = __builtin_bit_cast(u32, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(q, scale, 1));
@@ -612,10 +614,14 @@ __device__ __forceinline__ void mx_planes_gemm_body(const MxPlanesGemmArgs& p, f
     load_w(wave, w0);
     load_a(wave, a0);
     load_w(wave + 4, w1);
+    // (the barrier keeps a step's requests in front of its matrix work: left to itself the
+    // scheduler moved fragment loads down to just before their use, a whole trip to memory each)
 #define JL_MXP_STEP(N, WL, AL, WC, AC)                   \
     load_w(wave + 4 * (n + (N) + 2), WL);                \
     load_a(wave + 4 * (n + (N) + 1), AL);                \
-    if (n + (N) < my_steps) compute(WC, AC);
+    __builtin_amdgcn_sched_barrier(0);                   \
+    if (n + (N) < my_steps) compute(WC, AC);             \
+    __builtin_amdgcn_sched_barrier(0);
     const int my_steps = (nks - wave + 3) / 4;   // K-steps wave, wave + 4, ... (uniform)
     for (int n = 0; n < my_steps; n += 6) {
         JL_MXP_STEP(0, w2, a1, w0, a0)
