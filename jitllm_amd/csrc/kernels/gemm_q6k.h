@@ -50,14 +50,19 @@ __device__ __forceinline__ void gemm_q6k_split_slice(GemmArgs& p) {
     p.out += (size_t)blockIdx.z * p.ntok * p.out_stride;
 }
 
-// t0, r0: the tile's first token and row (a grouped launch places tiles per expert; a
-// wavefront whose tokens lie past ntok loads and computes nothing)
+// t0, r0: the tile's first token and row.  SKIP (a grouped launch, which places tiles per expert and
+// leaves many of them ragged): a wavefront whose tokens all lie past ntok loads and computes
+// nothing.  Without it every wavefront walks the same loop (one without tokens works on the last
+// group's fragments and stores nothing): the compiler sets the wait before a register's first use
+// to the smallest count over all ways to get there, and with a branch round the matrix work the
+// wait in front of the dequantization drained the fragment loads at every stage's head.
+template <bool SKIP = false>
 __device__ __forceinline__ void gemm_q6k_body(const GemmArgs& p, uint8_t* smem, int t0, int r0) {
     _Float16* sA = (_Float16*)smem;                 // [64][JL_GEMM_STRIDE]: 2 * (sc >> 1) * (q - 32)
     _Float16* sB = sA + 64 * JL_GEMM_STRIDE;        // (sc & 1) * (q - 32)
     const int tid = threadIdx.x, lane = tid & 63;
     const int tg = __builtin_amdgcn_readfirstlane(tid >> 6);   // this wavefront: tokens 32*tg..
-    const bool live = t0 + 32 * tg < p.ntok;                   // else no token of its 32 exists
+    const bool live = !SKIP || t0 + 32 * tg < p.ntok;          // (SKIP) else no token of its 32 exists
     const int arow = lane & 31, kg = lane >> 5;
     const int nsb = p.k / 256, nsteps = 2 * nsb;
     // this thread's share of a weight stage
@@ -102,7 +107,7 @@ __device__ __forceinline__ void gemm_q6k_body(const GemmArgs& p, uint8_t* smem, 
         }
     };
     // fragment (step, ks) of this wavefront's 32 tokens
-    const size_t ngrp = (size_t)(p.tok_pad >> 5), mygrp = (size_t)(t0 >> 5) + tg;
+    const size_t ngrp = (size_t)(p.tok_pad >> 5), mygrp = min((size_t)(t0 >> 5) + tg, ngrp - 1);
     auto a_frag = [&](int step, int ks) {
         return ((const f16x8*)p.bq)[(((size_t)step * ngrp + mygrp) * JL_GEMM_ASTAGE_FRAGS + ks) * 64 + lane];
     };
@@ -110,7 +115,7 @@ __device__ __forceinline__ void gemm_q6k_body(const GemmArgs& p, uint8_t* smem, 
     const uint8_t* drow[2];
 #pragma unroll
     for (int j = 0; j < 2; j++) drow[j] = p.w + (size_t)min(r0 + 32 * j + arow, p.nrows - 1) * p.row_bytes + 208;
-    const float* dap = p.da + t0 + 32 * tg + 4 * kg;
+    const float* dap = p.da + min(t0 + 32 * tg, p.tok_pad - 32) + 4 * kg;
 
     f32x16 out[2], acc[2];
 #pragma unroll
@@ -118,25 +123,34 @@ __device__ __forceinline__ void gemm_q6k_body(const GemmArgs& p, uint8_t* smem, 
 #pragma unroll
         for (int e = 0; e < 16; e++) out[j][e] = 0.f;
 
+    // Before the loop the loads go out in the loop's order: the weights, then the fragments in K order.
     Gemm6Raw raw;
     load_raw(0, raw);
+    __builtin_amdgcn_sched_barrier(0);
     f16x8 aring[8];
     if (live) {
 #pragma unroll
-        for (int ks = 0; ks < 8; ks++) aring[ks] = a_frag(0, ks);
+        for (int ks = 0; ks < 8; ks++) {
+            aring[ks] = a_frag(0, ks);
+            __builtin_amdgcn_sched_barrier(0);
+        }
     }
-    for (int step = 0; step < nsteps; step++) {
-        const int sb = step >> 1, half = step & 1;
+    // One stage (half a super-block; the half is a compile-time constant, so the loads that
+    // only the second half needs are no branch in the loop).
+    auto stage = [&](auto HALF, int step) {
+        constexpr int half = decltype(HALF)::value;
+        const int sb = step >> 1;
         dequant(raw);
         load_raw(min(step + 1, nsteps - 1), raw);   // a whole stage of matrix work covers the latency
         uint16_t dbits[2] = {0, 0};
         f32x4 dav[4];
-        if (half && live) {
+        if (half == 1 && live) {
 #pragma unroll
             for (int j = 0; j < 2; j++) dbits[j] = ld2(drow[j] + (size_t)sb * 210);
 #pragma unroll
             for (int i = 0; i < 4; i++) dav[i] = *(const f32x4*)(dap + (size_t)sb * p.tok_pad + 8 * i);
         }
+        __builtin_amdgcn_sched_barrier(0);
         lds_barrier();
         if (live) {
             const int nstep = min(step + 1, nsteps - 1);
@@ -158,7 +172,11 @@ __device__ __forceinline__ void gemm_q6k_body(const GemmArgs& p, uint8_t* smem, 
                                                                     (half == 0 && ks == 0) ? czero : acc[j], 0, 0, 0);
                     acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aring[ks], wfb[j], acc[j], 0, 0, 0);
                 }
+                // the next stage's fragment for this slot, requested HERE (left to itself the
+                // scheduler gathers all eight behind the last matrix instruction, a trip to L2
+                // before the next stage can start)
                 aring[ks] = a_frag(nstep, ks);
+                __builtin_amdgcn_sched_barrier(0);
             }
             if (half) {
                 // out += d_a * (d * P) for the super-block
@@ -171,8 +189,12 @@ __device__ __forceinline__ void gemm_q6k_body(const GemmArgs& p, uint8_t* smem, 
             }
         }
         lds_barrier();
+    };
+    for (int step = 0; step < nsteps; step += 2) {
+        stage(GemmIntC<0>{}, step);
+        stage(GemmIntC<1>{}, step + 1);
     }
-    if (!live) return;
+    if (SKIP && !live) return;
     // store: lane = row (contiguous in memory), register = token
 #pragma unroll
     for (int j = 0; j < 2; j++) {

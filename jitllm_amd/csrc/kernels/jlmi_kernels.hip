@@ -361,7 +361,7 @@ __device__ __forceinline__ void moe_gemm_tiles(const MoeGemmArgs& p) {
         g.ntok = 32 * slot0 + ncol;                  // tokens are positions in the workspace
         g.out_stride = p.nrows; g.sb_per = 0;
         g.out = p.out[mat] + ((ptrdiff_t)c_lo - (ptrdiff_t)32 * slot0) * p.nrows;   // workspace position -> column
-        if constexpr (TYPE == JL_Q6_K) gemm_q6k_body(g, jl_smem, 32 * slot0 + 128 * ctile, (int)rt * 64);
+        if constexpr (TYPE == JL_Q6_K) gemm_q6k_body<true>(g, jl_smem, 32 * slot0 + 128 * ctile, (int)rt * 64);
         else gemm_q4k_body<1, true, PL>(g, jl_smem, 32 * slot0 + 128 * ctile, (int)rt * 64);
         __syncthreads();   // the tile's LDS is free for the next one
     }
