@@ -871,12 +871,12 @@ __device__ __forceinline__ void mx_few_body(const MxGemmArgs& p, float* part) {
         const uint8_t* blk = wrow + (size_t)min(b, nblk - 1) * 17;
         w.e = blk[0];
         w.q = ld16_a1(blk + 1);
-        if (b >= nblk) w.q = u32x4{0, 0, 0, 0};   // past the end of K: zero codes
+        // (a block past the end of K reads the row's last block; its codes are zeroed where they
+        // are used.  A select on the loaded words here puts the wait for the load right behind
+        // the load, and so does a copy of one register set into the other at the loop's end: the
+        // loop is unrolled over the two sets instead)
     };
-    W wcur, wnxt;
-    if (wave < ngroups) load_w(wave, wcur);
-    for (int G = wave; G < ngroups; G += 8) {
-        if (G + 8 < ngroups) load_w(G + 8, wnxt);
+    auto group = [&](int G, const W& wcur) {
         // the group's sixteen NT activation operands go out together; left to itself the
         // scheduler sinks each load next to its use and the loop becomes a chain of waits
         bf16x8 af[4 * NT];
@@ -885,9 +885,10 @@ __device__ __forceinline__ void mx_few_body(const MxGemmArgs& p, float* part) {
             af[i] = __builtin_bit_cast(bf16x8, xf[((size_t)G * 4 * NT + i) * 64 + lane]);
         __builtin_amdgcn_sched_barrier(0);
         const float scale = mx_scale((uint8_t)wcur.e);
+        const bool past = 4 * G + kq >= nblk;
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            const u32 q = wcur.q[j];
+            const u32 q = past ? 0u : wcur.q[j];
             const u32x4 wv = {__builtin_bit_cast(u32, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(q, scale, 0)),
                               __builtin_bit_cast(u32, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(q, scale, 1)),
                               __builtin_bit_cast(u32, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(q, scale, 2)),
@@ -897,7 +898,20 @@ __device__ __forceinline__ void mx_few_body(const MxGemmArgs& p, float* part) {
             for (int t = 0; t < NT; t++)
                 out[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[j * NT + t], wf, out[t], 0, 0, 0);
         }
-        wcur = wnxt;
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    // A wavefront's groups are wave, wave + 8, ...: four of them (all of K = 4096) have their weights
+    // requested together before the first group's fragments, so the weights make ONE trip to memory
+    // a wavefront; a group's matrix work is far too short to cover the next group's trip.
+    for (int G0 = wave; G0 < ngroups; G0 += 32) {
+        W w[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            if (G0 + 8 * i < ngroups) load_w(G0 + 8 * i, w[i]);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            if (G0 + 8 * i < ngroups) group(G0 + 8 * i, w[i]);
     }
 
     // the eight K shares, added in wavefront order; part [wave][tile][lane] of four floats
