@@ -844,7 +844,7 @@ def main():
     ap.add_argument("--matvec", metavar="TYPE,NROWS,K[,packed][,w32]", help="only this decode matvec (TYPE q4_k, q6_k or "
                     "q8_0; packed = packed planes; w32 = activation window 32), for profiling one kernel; "
                     "prints its section alone")
-    ap.add_argument("--section", choices=["mxfp4", "moe", "moe_packed", "moe_decode", "ffn", "ffn_packed", "ceiling", "gemm_packed"],
+    ap.add_argument("--section", choices=["mxfp4", "moe", "moe_packed", "moe_prefill", "moe_decode", "ffn", "ffn_packed", "ceiling", "gemm_packed"],
                     help="only this section of the default run, for profiling its kernels; prints the section alone")
     ap.add_argument("--tune", metavar="KEY=VALUE", action="append", default=[],
                     help="a tuning key of the library (include/jlmi.h, jl_set_tuning), e.g. gemm.form=6; repeatable")
@@ -881,6 +881,7 @@ def main():
         return
     if args.section:
         fn = {"mxfp4": mxfp4_section, "moe": moe_section, "moe_packed": lambda d, g: moe_section(d, g, packed=True),
+              "moe_prefill": lambda d, g: moe_section(d, g, 1024),
               "moe_decode": moe_decode_section, "ffn": ffn_section,
               "ffn_packed": ffn_packed_section, "ceiling": lambda d, g: ceiling_section(d, g, vendor_gemm=True),
               "gemm_packed": lambda d, g: gemm_section(d, g, {4096: (512,), 14336: (512,)}, packed=True)}[args.section]
