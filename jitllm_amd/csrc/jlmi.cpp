@@ -1439,7 +1439,7 @@ int jl_ctx_create(jl_ctx** out, const jl_options* opts) {
     if (e != hipSuccess)
         return bail(JL_ERR_HIP, "hipModuleLoad(" + path + "): " + H->GetErrorString(e));
 
-    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_matvec_q4k_r1_pq", "jl_matvec_q4k_r1_pq_res", "jl_matvec_q8_0_r1_pq", "jl_matvec_q8_0_r1_pq_res", "jl_matvec_q6k_r1_pq", "jl_matvec_q6k_r1_pq_res", "jl_matvec_q8_0p_r1_pq", "jl_matvec_q8_0p_r1_pq_res", "jl_matvec_multi_q4k_res", "jl_matvec_multi_q4k_x4_res", "jl_matvec_multi_q4k_q_res", "jl_matvec_multi_q8_0_res", "jl_matvec_multi_q8_0_x4_res", "jl_matvec_multi_q8_0_q_res", "jl_matvec_multi_q6k_res", "jl_matvec_multi_q6k_x4_res", "jl_matvec_multi_q6k_q_res", "jl_matvec_multi_q8_0p_res", "jl_matvec_multi_q8_0p_x4_res", "jl_matvec_multi_q8_0p_q_res", "jl_matvec_q4k_r1_res", "jl_matvec_q4k_r1_x4_res", "jl_matvec_q8_0_r1_res", "jl_matvec_q8_0_r1_x4_res", "jl_matvec_q6k_r1_res", "jl_matvec_q6k_r1_x4_res", "jl_matvec_q8_0p_r1_res", "jl_matvec_q8_0p_r1_x4_res", "jl_matvec_q8_0p_r1", "jl_matvec_q8_0p_r2", "jl_matvec_q8_0p_r4", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_prep_q4k_fold", "jl_gemm_q4k_fold_wide", "jl_gemm_q4k_fold_wide4", "jl_gemm_q4k_k2", "jl_gemm_q4k_k2_planes", "jl_gemm_prep_q4k_planes", "jl_gemm_q4k_r64_planes", "jl_gemm_q4k_wide_planes", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_group2_wide", "jl_moe_quant", "jl_moe_matvec_planes_q4k", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_prep_planes", "jl_moe_gemm_q4k", "jl_moe_g16_prep", "jl_moe_g16_prep_planes", "jl_moe_g16_prep_q6k", "jl_moe_g16_c1", "jl_moe_g16_c2", "jl_moe_g16_c3", "jl_moe_g16_f1", "jl_moe_g16_f2", "jl_moe_g16_f3", "jl_moe_g16_g1", "jl_moe_g16_g2", "jl_moe_g16_g3", "jl_moe_g16_d1", "jl_moe_g16_d2", "jl_moe_g16_d3", "jl_moe_g16p_c1", "jl_moe_g16p_c2", "jl_moe_g16p_c3", "jl_moe_g16p_f1", "jl_moe_g16p_f2", "jl_moe_g16p_f3", "jl_moe_g16p_g1", "jl_moe_g16p_g2", "jl_moe_g16p_g3", "jl_moe_g16p_d1", "jl_moe_g16p_d2", "jl_moe_g16p_d3", "jl_moe_g16q6_c1", "jl_moe_g16q6_c2", "jl_moe_g16q6_c3", "jl_moe_g16q6_f1", "jl_moe_g16q6_f2", "jl_moe_g16q6_f3", "jl_moe_g16q6_g1", "jl_moe_g16q6_g2", "jl_moe_g16q6_g3", "jl_moe_g16q6_d1", "jl_moe_g16q6_d2", "jl_moe_g16q6_d3", "jl_moe_gemm_r64", "jl_moe_gemm_r64_planes", "jl_moe_gemm_q6k_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_mxfp4_matvec1_b1", "jl_mxfp4_matvec1_b2", "jl_mxfp4_matvec1_b3", "jl_mxfp4_scaled_prep", "jl_mxfp4_scaled_gemm", "jl_mxfp4_planes_prep", "jl_mxfp4_planes_gemm", "jl_mxfp4_matvec_planes_r64", "jl_mxfp4_matvec_planes_r32", "jl_mxfp4_matvec_planes_r16", "jl_unpack_mxfp4", "jl_sum_parts", "jl_fill_u32", "jl_q4k_fold_range", "jl_probe_read", "jl_probe_empty", "jl_probe_wait", "jl_probe_mfma", "jl_probe_mfma_v5",
+    std::vector<std::string> names = {"jl_quantize_act", "jl_dequant", "jl_matvec_q4k_r1_pq", "jl_matvec_q4k_r1_pq_res", "jl_matvec_q8_0_r1_pq", "jl_matvec_q8_0_r1_pq_res", "jl_matvec_q6k_r1_pq", "jl_matvec_q6k_r1_pq_res", "jl_matvec_q8_0p_r1_pq", "jl_matvec_q8_0p_r1_pq_res", "jl_matvec_multi_q4k_res", "jl_matvec_multi_q4k_x4_res", "jl_matvec_multi_q4k_q_res", "jl_matvec_multi_q8_0_res", "jl_matvec_multi_q8_0_x4_res", "jl_matvec_multi_q8_0_q_res", "jl_matvec_multi_q6k_res", "jl_matvec_multi_q6k_x4_res", "jl_matvec_multi_q6k_q_res", "jl_matvec_multi_q8_0p_res", "jl_matvec_multi_q8_0p_x4_res", "jl_matvec_multi_q8_0p_q_res", "jl_matvec_q4k_r1_res", "jl_matvec_q4k_r1_x4_res", "jl_matvec_q8_0_r1_res", "jl_matvec_q8_0_r1_x4_res", "jl_matvec_q6k_r1_res", "jl_matvec_q6k_r1_x4_res", "jl_matvec_q8_0p_r1_res", "jl_matvec_q8_0p_r1_x4_res", "jl_matvec_q8_0p_r1", "jl_matvec_q8_0p_r2", "jl_matvec_q8_0p_r4", "jl_gemm_prep_q4k", "jl_gemm_prep_q4k_w16", "jl_gemm_q4k_r64", "jl_gemm_q6k_r64", "jl_gemm_prep_w32", "jl_gemm_q8_0_w32", "jl_gemm_q6k_w32", "jl_gemm_q4k_w32", "jl_gemm_q4k_r128", "jl_gemm_q4k_wide", "jl_gemm_prep_q4k_fold", "jl_gemm_q4k_fold_wide", "jl_gemm_q4k_fold_wide4", "jl_gemm_q4k_k2", "jl_gemm_q4k_k2_planes", "jl_gemm_prep_q4k_planes", "jl_gemm_q4k_r64_planes", "jl_gemm_q4k_wide_planes", "jl_gemm_w16_prep_q4k", "jl_gemm_q4k_w16", "jl_gemm_q4k_few_t1", "jl_gemm_q4k_few_t2", "jl_gemm_q4k_few_t3", "jl_gemm_q4k_few_t4", "jl_gemm_q4k_few32", "jl_moe_route", "jl_moe_route_g2", "jl_moe_route_g4", "jl_moe_logits", "jl_moe_logits_e8", "jl_moe_group", "jl_moe_group2", "jl_moe_group2_wide", "jl_moe_quant", "jl_moe_matvec_planes_q4k", "jl_moe_combine", "jl_moe_worklist", "jl_moe_gemm_prep", "jl_moe_gemm_prep_planes", "jl_moe_gemm_q4k", "jl_moe_g16_prep", "jl_moe_g16_prep_planes", "jl_moe_g16_prep_q6k", "jl_moe_g16_c1", "jl_moe_g16_c2", "jl_moe_g16_c3", "jl_moe_g16_f1", "jl_moe_g16_f2", "jl_moe_g16_f3", "jl_moe_g16_g1", "jl_moe_g16_g2", "jl_moe_g16_g3", "jl_moe_g16_d1", "jl_moe_g16_d2", "jl_moe_g16_d3", "jl_moe_g16p_c1", "jl_moe_g16p_c2", "jl_moe_g16p_c3", "jl_moe_g16p_f1", "jl_moe_g16p_f2", "jl_moe_g16p_f3", "jl_moe_g16p_g1", "jl_moe_g16p_g2", "jl_moe_g16p_g3", "jl_moe_g16p_d1", "jl_moe_g16p_d2", "jl_moe_g16p_d3", "jl_moe_g16q6_c1", "jl_moe_g16q6_c2", "jl_moe_g16q6_c3", "jl_moe_g16q6_f1", "jl_moe_g16q6_f2", "jl_moe_g16q6_f3", "jl_moe_g16q6_g1", "jl_moe_g16q6_g2", "jl_moe_g16q6_g3", "jl_moe_g16q6_d1", "jl_moe_g16q6_d2", "jl_moe_g16q6_d3", "jl_moe_gemm_r64", "jl_moe_gemm_r64_planes", "jl_moe_gemm_q6k_r64", "jl_mxfp4_prep", "jl_mxfp4_prep_few", "jl_mxfp4_few_t1", "jl_mxfp4_few_t2", "jl_mxfp4_few_t3", "jl_mxfp4_few_t4", "jl_mxfp4_gemm", "jl_mxfp4_gemm_r96", "jl_mxfp4_matvec", "jl_mxfp4_matvec1_b1", "jl_mxfp4_matvec1_b2", "jl_mxfp4_matvec1_b3", "jl_mxfp4_scaled_prep", "jl_mxfp4_scaled_gemm", "jl_mxfp4_planes_prep", "jl_mxfp4_planes_gemm", "jl_mxfp4_matvec_planes_r64", "jl_mxfp4_matvec_planes_r32", "jl_mxfp4_matvec_planes_r16", "jl_unpack_mxfp4", "jl_sum_parts", "jl_fill_u32", "jl_q4k_fold_range", "jl_probe_read", "jl_probe_empty", "jl_probe_wait", "jl_probe_mfma", "jl_probe_mfma_v5",
                                       "jl_pack_weights", "jl_unpack_q4k", "jl_unpack_q6k", "jl_unpack_q8_0"};
     for (const char* tag : {"q4k", "q8_0", "q6k"})
         for (int rw : {16, 32, 64})
@@ -1886,7 +1886,9 @@ int jl_moe_route_dev(jl_ctx* c, const float* logits, int rows, int n_expert, int
     MoeRouteArgs a;
     a.logits = logits; a.sel = sel; a.wt = wt; a.n_expert = n_expert; a.k_used = k_used; a.sel_stride = sel_stride;
     void* params[] = {&a};
-    return launch(c, "jl_moe_route", (unsigned)rows, 1, 64, 0, pick_stream(c, stream), params);
+    // the form with the fewest experts a lane that holds them all (less code for a lone wavefront to fetch)
+    const char* name = n_expert <= 128 ? "jl_moe_route_g2" : n_expert <= 256 ? "jl_moe_route_g4" : "jl_moe_route";
+    return launch(c, name, (unsigned)rows, 1, 64, 0, pick_stream(c, stream), params);
 }
 
 int jl_moe_logits_dev(jl_ctx* c, float* logits, int wtype, const void* w, const float* x, int n_expert, int k,

@@ -241,7 +241,9 @@ extern "C" __global__ __launch_bounds__(256, 2) void jl_gemm_q4k_w16(GemmW16Args
 
 // ------------------------------------------------------- mixture of experts
 // grid = rows, block = 64
-extern "C" __global__ __launch_bounds__(64) void jl_moe_route(MoeRouteArgs p) { moe_route_body(p); }
+extern "C" __global__ __launch_bounds__(64) void jl_moe_route(MoeRouteArgs p) { moe_route_body<16>(p); }
+extern "C" __global__ __launch_bounds__(64) void jl_moe_route_g2(MoeRouteArgs p) { moe_route_body<2>(p); }
+extern "C" __global__ __launch_bounds__(64) void jl_moe_route_g4(MoeRouteArgs p) { moe_route_body<4>(p); }
 // grid = (experts, ceil(tokens / JL_LOGITS_TOK)), block = 128
 extern "C" __global__ __launch_bounds__(128) void jl_moe_logits(MoeLogitsArgs p) {
     __shared__ float part[JL_LOGITS_TOK * 128];

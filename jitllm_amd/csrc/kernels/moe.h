@@ -91,23 +91,27 @@ __device__ __forceinline__ void route_wave_argmax(i32& key, i32& idx) {
     idx = __builtin_amdgcn_readlane(idx, 63);
 }
 
+// NG: experts a lane at most (n_expert <= 64 * NG).  The router is one wavefront a row on a CU of
+// its own, so every wavefront fetches the kernel's code itself: the sixteen-a-lane form is 14 KB of
+// straight-line code, mostly skipped, for 128 experts.
+template <int NG = 16>
 __device__ __forceinline__ void moe_route_body(const MoeRouteArgs& p) {
     const int lane = threadIdx.x & 63, n = p.n_expert;
     const size_t row = blockIdx.x;
     const float* lg = p.logits + row * (size_t)n;
-    float v[16];
+    float v[NG];
     float mx = -__builtin_inff();
 #pragma unroll
-    for (int i = 0; i < 16; i++) {
+    for (int i = 0; i < NG; i++) {
         const int e = lane + 64 * i;
         v[i] = e < n ? lg[min(e, n - 1)] : -__builtin_inff();
         if (v[i] > mx) mx = v[i];
     }
     mx = route_wave_max(mx);
     double sum = 0.0;
-    float sc[16];
+    float sc[NG];
 #pragma unroll
-    for (int i = 0; i < 16; i++) {
+    for (int i = 0; i < NG; i++) {
         const int e = lane + 64 * i;
         double ex = 0.0;
         if (64 * i < n) ex = e < n ? exp((double)v[i] - (double)mx) : 0.0;   // (uniform: whole groups of 64 past n are skipped)
@@ -117,7 +121,7 @@ __device__ __forceinline__ void moe_route_body(const MoeRouteArgs& p) {
     sum = route_wave_sum(sum);
     const double inv = 1.0 / sum;
 #pragma unroll
-    for (int i = 0; i < 16; i++) sc[i] = (float)((double)sc[i] * inv);
+    for (int i = 0; i < NG; i++) sc[i] = (float)((double)sc[i] * inv);
 
     // Scores are >= 0, so their bit patterns order as integers; -1 marks "none".
     i32 prev_key = 0, prev_idx = -1;
@@ -129,7 +133,7 @@ __device__ __forceinline__ void moe_route_body(const MoeRouteArgs& p) {
         // of equal values is kept)
         i32 bk = -1, bi = 0x7fffffff;
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
+        for (int i = 0; i < NG; i++) {
             if (64 * i >= n) continue;   // uniform
             const int e = lane + 64 * i;
             const float x = sc[i];
@@ -1067,15 +1071,18 @@ __device__ __forceinline__ void moe_g16_body(const MoeG16Args& p, uint8_t* smem)
         // tasks of this wavefront requested ahead of the weights, which have the longer way and
         // would hold them up (a wavefront's loads return in order)
         constexpr bool X2 = FUSED == 2;           // columns are silu(x) * x2 (the down projection's)
-        constexpr int TB = FUSED == 1 ? 16 : 8;   // tasks of a wavefront in flight: 128 or 64 a workgroup of eight
+        constexpr int TB = 8;   // tasks of a wavefront in flight: 64 a workgroup of eight
         const int ntask = ncg * nsb;
+        // task / nsb for task < 16 * nsb <= 1024 as a multiplication (a division is ~30 instructions,
+        // and this code runs once a workgroup, fetched cold)
+        const u32 nsb_inv = 65536u / (u32)nsb + 1u;
         u32 rowv = 0;
         f32x4 xv[TB], xu[X2 ? TB : 1];
         auto issue = [&](int t0) {
 #pragma unroll
             for (int b = 0; b < TB; b++) {
                 const int task = min(t0 + b * nwaves, ntask - 1);
-                const int i = task / nsb, sb = task - i * nsb;
+                const int i = (int)(((u32)task * nsb_inv) >> 16), sb = task - i * nsb;
                 const size_t row = (size_t)__shfl(rowv, i, 64);
                 xv[b] = ((const f32x4*)(p.x + row * (size_t)p.k + (size_t)sb * 256))[lane];
                 if (X2) xu[X2 ? b : 0] = ((const f32x4*)(p.x2 + row * (size_t)p.k + (size_t)sb * 256))[lane];
@@ -1104,7 +1111,7 @@ __device__ __forceinline__ void moe_g16_body(const MoeG16Args& p, uint8_t* smem)
                 for (int b = 0; b < TB; b++) {
                     const int task = t0 + b * nwaves;
                     if (task < ntask) {   // uniform
-                        const int i = task / nsb, sb = task - i * nsb;
+                        const int i = (int)(((u32)task * nsb_inv) >> 16), sb = task - i * nsb;
                         f32x4 w = xv[b];
                         if (X2) {
                             const f32x4 u = xu[X2 ? b : 0];
@@ -1198,6 +1205,16 @@ __device__ __forceinline__ void moe_g16_body(const MoeG16Args& p, uint8_t* smem)
                         u32 m4 = 0x000F000Fu, m2 = 0x00300030u;
                         asm volatile("" : "+v"(m4), "+v"(m2));
                         const f16x2 off = {(_Float16)-1056.0f, (_Float16)-1056.0f};
+                        // the super-block's fragments and token scales requested from LDS in one go (see below)
+                        u32x4 af[8][NT];
+                        f32x4 dav[NT];
+#pragma unroll
+                        for (int ks = 0; ks < 8; ks++)
+#pragma unroll
+                            for (int r = 0; r < NT; r++) af[ks][r] = sA4[r * RV + sb * V + ks * 65 + lane];
+#pragma unroll
+                        for (int r = 0; r < NT; r++) dav[r] = *(const f32x4*)(sAf + ((size_t)r * RV + sb * V + 552) * 4 + 4 * kg);
+                        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                         for (int ks = 0; ks < 8; ks++) {
                             const int hh = ks >> 2, w = ks & 3;
@@ -1222,20 +1239,18 @@ __device__ __forceinline__ void moe_g16_body(const MoeG16Args& p, uint8_t* smem)
                             const f32x4 czero = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                             for (int r = 0; r < NT; r++) {
-                                const f16x8 af = __builtin_bit_cast(f16x8, sA4[r * RV + sb * V + ks * 65 + lane]);
-                                accP[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, __builtin_bit_cast(f16x8, oa),
+                                const f16x8 a = __builtin_bit_cast(f16x8, af[ks][r]);
+                                accP[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, __builtin_bit_cast(f16x8, oa),
                                                                                  ks == 0 ? czero : accP[r], 0, 0, 0);
-                                accP[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, __builtin_bit_cast(f16x8, ob), accP[r], 0, 0, 0);
+                                accP[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, __builtin_bit_cast(f16x8, ob), accP[r], 0, 0, 0);
                             }
                         }
                         // out += d_a * (d * P) for the super-block
                         const float dd = half_bits_to_f32((uint16_t)(hd[cur][s].z & 0xFFFF));
 #pragma unroll
-                        for (int r = 0; r < NT; r++) {
-                            const f32x4 dav = *(const f32x4*)(sAf + ((size_t)r * RV + sb * V + 552) * 4 + 4 * kg);
+                        for (int r = 0; r < NT; r++)
 #pragma unroll
-                            for (int el = 0; el < 4; el++) out[r][el] = fmaf(dav[el], dd * accP[r][el], out[r][el]);
-                        }
+                            for (int el = 0; el < 4; el++) out[r][el] = fmaf(dav[r][el], dd * accP[r][el], out[r][el]);
                     } else {
                     GemmWideScale sc, sc1;
                     if (PL) {
@@ -1244,15 +1259,29 @@ __device__ __forceinline__ void moe_g16_body(const MoeG16Args& p, uint8_t* smem)
                     } else {
                         gemm_wide_scale(hd[cur][s], kg & 1, kg >> 1, sc);
                     }
+                    // the super-block's fragments, sums and token scales are requested from LDS in one
+                    // go: read one K-step at a time, each matrix instruction waited a full LDS latency
+                    // behind its own read, with two wavefronts a SIMD to hide it
+                    u32x4 af[8][NT], augw[NT];
+                    f32x4 dav[NT];
+#pragma unroll
+                    for (int ks = 0; ks < 8; ks++)
+#pragma unroll
+                        for (int r = 0; r < NT; r++) af[ks][r] = sA4[r * RV + sb * V + ks * 65 + lane];
+#pragma unroll
+                    for (int r = 0; r < NT; r++) {
+                        augw[r] = sA4[r * RV + sb * V + 520 + (lane & 31)];
+                        dav[r] = *(const f32x4*)(sAf + ((size_t)r * RV + sb * V + 552) * 4 + 4 * kg);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                     for (int ks = 0; ks < 8; ks++) {
                         const f16x8 b = moe_g16_word(wq[cur][s][ks >> 2][ks & 3], PL && ks >= 4 ? sc1 : sc, mask_lo, mask_hi, magic);
                         const f32x4 czero = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                        for (int r = 0; r < NT; r++) {
-                            const f16x8 af = __builtin_bit_cast(f16x8, sA4[r * RV + sb * V + ks * 65 + lane]);
-                            accP[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, b, ks == 0 ? czero : accP[r], 0, 0, 0);
-                        }
+                        for (int r = 0; r < NT; r++)
+                            accP[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, af[ks][r]), b,
+                                                                             ks == 0 ? czero : accP[r], 0, 0, 0);
                     }
                     // out += d_a * (d * P - dmin * M) for the super-block
                     const float mul = kg == 0 ? 1.0f : (kg == 1 ? 64.0f : 0.0f);
@@ -1272,16 +1301,14 @@ __device__ __forceinline__ void moe_g16_body(const MoeG16Args& p, uint8_t* smem)
                     const float dmin = half_bits_to_f32((uint16_t)(hd[cur][s].x >> 16));
 #pragma unroll
                     for (int r = 0; r < NT; r++) {
-                        u32x4 augw = u32x4{0u, 0u, 0u, 0u};
-                        if (lane < 32) augw = sA4[r * RV + sb * V + 520 + lane];
-                        const f16x8 aug = __builtin_bit_cast(f16x8, augw);
-                        const f32x4 dav = *(const f32x4*)(sAf + ((size_t)r * RV + sb * V + 552) * 4 + 4 * kg);
+                        // lanes 32-63 (kg 2, 3) meet minimum columns of zero, so what they hold of the sums does not count
+                        const f16x8 aug = __builtin_bit_cast(f16x8, augw[r]);
                         const f32x4 czero = {0.f, 0.f, 0.f, 0.f};
                         const f32x4 accM = __builtin_amdgcn_mfma_f32_16x16x32_f16(aug, mm, czero, 0, 0, 0);
 #pragma unroll
                         for (int el = 0; el < 4; el++) {
                             const float uu = fmaf(dd, accP[r][el], -(dmin * accM[el]));
-                            out[r][el] = fmaf(dav[el], uu, out[r][el]);
+                            out[r][el] = fmaf(dav[r][el], uu, out[r][el]);
                         }
                     }
                     }

@@ -46,12 +46,13 @@ def silu(g):
                                                        ("random", 64, 128, 8), ("random", 300, 60, 6),
                                                        ("random", 1, 1000, 16), ("one_expert", 129, 16, 2),
                                                        ("random", 2048, 128, 8), ("random", 700, 1000, 16),
-                                                       ("one_expert", 2100, 7, 2)])
+                                                       ("one_expert", 2100, 7, 2), ("random", 2600, 128, 8),
+                                                       ("random", 4400, 64, 16)])
 def test_grouping_is_bit_exact(dev, devbuf, mode, rows, n_expert, k_used, form):
     """Both forms of the grouping kernel against the oracle's groupPairs: integer work, exact.
     Runs of 64 pairs that end inside a row, more runs than wavefronts (300 x 6 pairs), more
-    experts than pairs, every pair on a handful of experts and pair lists of many runs a
-    wavefront (16,384 pairs) are among the cases."""
+    experts than pairs, every pair on a handful of experts, pair lists of many runs a wavefront
+    (16,384 and 20,800 pairs) and past 65,535 pairs (70,400: 32-bit counts) are among the cases."""
     dev.set_tuning(moe__group=form)
     sel, _ = route(rows, n_expert, k_used, 3, mode)
     used, perm, col_e, pos = oracle.group_pairs(sel.reshape(-1), rows, k_used, n_expert, 1)
@@ -413,7 +414,7 @@ def test_moe_block_q6k_down_sheets_vs_oracle(dev, devbuf, rows):
     dev.SetActWindow(32)
 
 
-@pytest.mark.parametrize("case", [(64, 128, 8), (7, 16, 1), (33, 1000, 16), (5, 8, 8), (20, 130, 4)],
+@pytest.mark.parametrize("case", [(64, 128, 8), (7, 16, 1), (33, 1000, 16), (5, 8, 8), (20, 130, 4), (9, 256, 8), (11, 257, 6)],
                          ids=lambda c: "x".join(map(str, c)))
 def test_router_vs_oracle(dev, devbuf, case):
     """The device router against oracle.MoERouter's restatement: the selection (integer work)
