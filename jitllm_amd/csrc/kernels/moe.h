@@ -91,9 +91,10 @@ __device__ __forceinline__ void route_wave_argmax(i32& key, i32& idx) {
     idx = __builtin_amdgcn_readlane(idx, 63);
 }
 
-// NG: experts a lane at most (n_expert <= 64 * NG).  The router is one wavefront a row on a CU of
-// its own, so every wavefront fetches the kernel's code itself: the sixteen-a-lane form is 14 KB of
-// straight-line code, mostly skipped, for 128 experts.
+// NG: experts a lane at most (n_expert <= 64 * NG).  The router is one wavefront a row, a dependent
+// chain of f64 arithmetic, and every expert slot a lane does not need still costs a clamped load, its
+// compares and a skipped branch in each loop: 128 experts in the sixteen-a-lane form 8.1 us, in the
+// two-a-lane form 5.6.
 template <int NG = 16>
 __device__ __forceinline__ void moe_route_body(const MoeRouteArgs& p) {
     const int lane = threadIdx.x & 63, n = p.n_expert;
@@ -1071,10 +1072,14 @@ __device__ __forceinline__ void moe_g16_body(const MoeG16Args& p, uint8_t* smem)
         // tasks of this wavefront requested ahead of the weights, which have the longer way and
         // would hold them up (a wavefront's loads return in order)
         constexpr bool X2 = FUSED == 2;           // columns are silu(x) * x2 (the down projection's)
-        constexpr int TB = 8;   // tasks of a wavefront in flight: 64 a workgroup of eight
+        // tasks of a wavefront in flight: 32 (K = 768: ten columns) or 64 a workgroup of eight.  Slots past
+        // the last task repeat its load (a slot that requested nothing would make every wait that follows
+        // count as if none had: 104.5 -> 105.9 us for the 64-row block), and a repeated load still takes
+        // its place in the queue in front of the weights, so there are no more slots than a handful of
+        // columns needs (sixteen and eight: 108.0 us)
+        constexpr int TB = X2 ? 4 : 8;
         const int ntask = ncg * nsb;
-        // task / nsb for task < 16 * nsb <= 1024 as a multiplication (a division is ~30 instructions,
-        // and this code runs once a workgroup, fetched cold)
+        // task / nsb for task < 16 * nsb <= 1024 as a multiplication (a division is ~30 instructions)
         const u32 nsb_inv = 65536u / (u32)nsb + 1u;
         u32 rowv = 0;
         f32x4 xv[TB], xu[X2 ? TB : 1];
