@@ -792,6 +792,14 @@ def ceiling_section(dev, gate_, vendor_gemm=False):
         out[name] = {"us_per_launch": round(ms * 1e3, 3), "GB/s": round(nbytes / (ms * 1e-3) / 1e9, 1),
                      "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                      "grid": grid, "block": block, "copies": ncopies, "us_by_grid_x_block": by_shape}
+    if vendor_gemm:
+        # (--section ceiling only) how many CUs a read needs: the mixture block's bytes, 320 MB, through
+        # 64 to 512 workgroups -- half the CUs read nearly as fast as all of them, a quarter does not
+        nbytes = 320 << 20
+        out["pure_read_320MB_us_by_grid_x_block"] = {
+            f"{grid}x{block}": round(measure(dev, lambda i: dev.probe_dev(1, pool.ptr + (i % 2) * nbytes, nbytes, grid, block),
+                                             20, gate_, warm=4) * 1e3, 1)
+            for grid, block in [(512, 1024), (256, 1024), (256, 512), (128, 1024), (128, 512), (126, 1024), (64, 1024)]}
     pool.free()
     if vendor_gemm:
         out["vendor_f16_gemm"] = vendor_gemm_section()
